@@ -1,0 +1,111 @@
+// Launch interface between the host tile class and the HIP kernels (gfx950).
+#pragma once
+#include "../../include/rpu_amd.h"
+#include "philox.h"
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace rpu_amd {
+
+// IO non-idealities of one pass, absolute steps (see IOPar::initialize).
+struct IoDev {
+  float inp_res, inp_bound, inp_noise, inp_asym;
+  float out_res, out_bound, out_noise, out_asym, out_scale;
+  float nm_thres, nm_assumed_wmax, max_bm_res;
+  int noise_management, bound_management, bm_test_negative_bound, max_bm_factor;
+  int inp_sto_round, out_sto_round;
+  int perfect;
+};
+
+// Per-sample bookkeeping of the noisy MVM, all arrays of length >= m_batch.
+struct MvmState {
+  float *nm;       // noise-management scale
+  float *nm_np;    // AbsMaxNPSum scale (IterativeWorstCase only)
+  float *red;      // bound-management reduction of the current round
+  float *scale;    // input scale of the current round
+  float *fin;      // factor applied to the ADC output (0 = sample short-cut to zero)
+  int *rounds;     // rounds run so far
+  int *hit_up;     // 1 + largest output index that hit the upper bound this round (0 = none)
+  int *hit_lo;     // same for the lower bound
+  int *list[2];    // ping-pong lists of samples that need another round
+  int *count;      // count[r] = number of samples in the list read by round r (r >= 1)
+};
+
+struct MvmArgs {
+  const float *w; // row-major [d_size][x_size]
+  int x_size, d_size;
+  const float *in;
+  long in_sb, in_sk; // input element (b, k) at in[b * in_sb + k * in_sk]
+  float *out;
+  long out_sb, out_so; // output element (b, o) at out[b * out_sb + o * out_so]
+  int m_batch;
+  int K, O;       // contraction length and number of outputs
+  int transposed; // 0: out[o] = sum_k W[o][k] in[k] (forward); 1: out[o] = sum_k W[k][o] in[k] (backward)
+  int round;      // bound-management round, 0-based
+  float alpha, beta; // only used when io.perfect: out = alpha * acc + beta * out
+  IoDev io;
+  MvmState st;
+  PhiloxKey key;
+  uint32_t call;
+};
+
+// noise management + per-sample state for round 0
+void launch_mvm_init(const MvmArgs &a, hipStream_t s);
+// one round of DAC -> MFMA contraction -> ADC
+void launch_mvm_round(const MvmArgs &a, hipStream_t s);
+// after round `a.round`: decide which samples need another round and set up their scales
+void launch_mvm_advance(const MvmArgs &a, hipStream_t s);
+// number of rounds that can ever be needed with these IO settings
+int mvm_max_rounds(const IoDev &io);
+
+// [B][X-1] (or [X-1][B]) -> [B][X] with a trailing column of ones (always batch-first output)
+void launch_make_bias(const float *in, float *out, int m_batch, int x_size, int in_trans, hipStream_t s);
+// [B][X] -> [B][X-1] (or [X-1][B]) dropping the last column
+void launch_drop_bias(const float *in, float *out, int m_batch, int x_size, int out_trans, hipStream_t s);
+
+// ----- pulsed update ---------------------------------------------------------------------------
+
+struct UpdateDev {
+  int pulse_type, desired_bl, fixed_bl, update_management, update_bl_management, sto_round;
+  float um_grad_scale, res, x_res_implicit, d_res_implicit;
+};
+
+struct DeviceDev {
+  int kind;
+  int ls_mult_noise;
+  float dw_min, dw_min_std;
+  const float *w_max, *w_min, *scale_up, *scale_down, *slope_up, *slope_down; // [d_size][x_size]
+};
+
+struct UpdateArgs {
+  float *w; // [d_size][x_size]
+  int x_size, d_size, m_batch;
+  const float *x;
+  long x_sb, x_sj; // x element (b, j) at x[b * x_sb + j * x_sj]
+  const float *d;
+  long d_sb, d_si;
+  float lr;
+  UpdateDev up;
+  DeviceDev dev;
+  // per-call scratch
+  int *bl;       // [B] bit-line length per sample
+  float *prob_a; // [B] probability scale of d
+  float *prob_b; // [B] probability scale of x
+  uint32_t *x_words; // [B][X] packed pulse words
+  uint32_t *d_words; // [B][D]
+  float *x_val;  // [B][X] implicit line values
+  float *d_val;  // [B][D]
+  PhiloxKey key;
+  uint32_t call;
+};
+
+void launch_update_prepare(const UpdateArgs &a, hipStream_t s);       // BL, A, B per sample
+void launch_update_bitlines(const UpdateArgs &a, hipStream_t s);      // stochastic pulse words
+void launch_update_implicit_lines(const UpdateArgs &a, hipStream_t s); // deterministic line values
+void launch_update_pulsed(const UpdateArgs &a, hipStream_t s);        // coincidences + device steps
+void launch_update_implicit(const UpdateArgs &a, hipStream_t s);
+void launch_implicit_counts(const UpdateArgs &a, int32_t *counts, hipStream_t s);
+// clip weights into [w_min, w_max]
+void launch_clip(float *w, const float *w_min, const float *w_max, size_t n, hipStream_t s);
+
+} // namespace rpu_amd

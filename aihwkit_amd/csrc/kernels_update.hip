@@ -1,0 +1,385 @@
+// Pulsed weight update of the analog tile on gfx950.
+//
+// Stages of one update call over a batch (all on one stream, no host round trip):
+//   1. per sample: abs-max of x and d -> bit-line length BL and probability scales A (for d), B (for x)
+//      (src/rpucuda/rpu_pulsed_meta_parameter.cpp:152-236),
+//   2. per line element and sample: one packed 32-bit pulse word, bit 0 = sign, bits 1..BL = pulses
+//      drawn with probability |v| * scale (src/rpucuda/sparse_bit_line_maker.cpp:199-238; word format
+//      src/rpucuda/rpu_weight_updater.cpp:297-324),
+//   3. per cross-point: walk the samples in batch order, n = popcount(x_word & d_word) coincidences of
+//      one sample all have the sign sign(x) * sign(d), apply n device steps
+//      (src/rpucuda/rpu_weight_updater.cpp:263-283, rpu_pulsed_device.h:450-459; device steps
+//      rpu_constantstep_device.cpp:27-55, rpu_linearstep_device.cpp:112-164).
+// The weight matrix and the per-device parameter arrays are row-major [d_size][x_size]; a wavefront
+// covers 64 consecutive x of one d row, so the d word of a sample is wave-uniform (scalar load) and
+// the x words, weights and parameters are read with unit stride.
+#include "kernels.h"
+
+namespace rpu_amd {
+
+namespace {
+
+__device__ __forceinline__ float block_max(float v, float *sh) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off));
+  if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = v;
+  __syncthreads();
+  float r = sh[0];
+  for (int i = 1; i < (int)(blockDim.x >> 6); ++i) r = fmaxf(r, sh[i]);
+  __syncthreads();
+  return r;
+}
+
+// rpu_pulsed_meta_parameter.cpp:152-181
+__device__ __forceinline__ void calc_bl_ab(const UpdateDev &up, int &BL, float &A, float &B, float lr, float dw_min) {
+  if (lr == 0.0f) {
+    A = 0.0f;
+    B = 0.0f;
+    BL = 0;
+    return;
+  }
+  if (up.fixed_bl || up.update_bl_management) {
+    BL = up.desired_bl;
+    A = sqrtf(lr / (dw_min * (float)BL));
+    B = A;
+  } else {
+    if ((dw_min * (float)up.desired_bl) < lr) {
+      A = 1.0f;
+      B = 1.0f;
+      BL = max((int)ceilf(lr / dw_min), 1);
+    } else {
+      BL = up.desired_bl;
+      A = sqrtf(lr / (dw_min * (float)BL));
+      B = A;
+    }
+  }
+}
+
+__global__ __launch_bounds__(256) void k_update_prepare(UpdateArgs a) {
+  __shared__ float sh[8];
+  const int b = blockIdx.x;
+  const float lr = fabsf(a.lr);
+  const float dw_min = a.dev.dw_min;
+  int BL;
+  float A, B;
+  if (a.up.update_management || a.up.update_bl_management) {
+    float xm = 0.0f, dm = 0.0f;
+    for (int j = threadIdx.x; j < a.x_size; j += blockDim.x) xm = fmaxf(xm, fabsf(a.x[(long)b * a.x_sb + (long)j * a.x_sj]));
+    for (int i = threadIdx.x; i < a.d_size; i += blockDim.x) dm = fmaxf(dm, fabsf(a.d[(long)b * a.d_sb + (long)i * a.d_si]));
+    xm = block_max(xm, sh);
+    dm = block_max(dm, sh);
+    if (threadIdx.x != 0) return;
+    // rpu_pulsed_meta_parameter.cpp:183-236
+    calc_bl_ab(a.up, BL, A, B, lr, dw_min);
+    if (lr > 0.0f) {
+      if (dm == 0.0f || xm == 0.0f) {
+        A = 1.0f;
+        B = 1.0f;
+        BL = 0;
+      } else {
+        const float x_val = xm;
+        float d_val = a.up.um_grad_scale * dm;
+        const float k_val = lr * x_val * d_val / dw_min;
+        if (a.up.update_bl_management) {
+          BL = (int)ceilf(k_val);
+          if (BL > a.up.desired_bl) BL = a.up.desired_bl;
+          A = sqrtf(lr / (dw_min * (float)BL));
+          B = A;
+        }
+        if (a.up.update_management) {
+          if (k_val > (float)a.up.desired_bl) d_val *= (float)a.up.desired_bl / k_val;
+          A *= sqrtf(x_val / d_val);
+          B *= sqrtf(d_val / x_val);
+        }
+      }
+    }
+  } else {
+    if (threadIdx.x != 0) return;
+    calc_bl_ab(a.up, BL, A, B, lr, dw_min);
+  }
+  // one 32-bit word holds the sign and at most 31 pulses
+  if (BL > 31) BL = 31;
+  a.bl[b] = BL;
+  a.prob_a[b] = A;
+  a.prob_b[b] = B;
+}
+
+__device__ __forceinline__ float discretize_prob(float pp, float res, int sto_round, uint32_t rnd) {
+  if (res <= 0.0f) return pp;
+  float q = pp / res;
+  if (sto_round) q = q + (u32_to_uniform(rnd) - 0.5f);
+  return rintf(q) * res;
+}
+
+// one thread per (sample, line element); x lines first, then d lines
+__global__ __launch_bounds__(256) void k_update_bitlines(UpdateArgs a) {
+  const long per_sample = (long)a.x_size + a.d_size;
+  const long total = per_sample * a.m_batch;
+  for (long idx = blockIdx.x * (long)blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
+    const int b = (int)(idx / per_sample);
+    const int e = (int)(idx % per_sample);
+    const bool is_x = e < a.x_size;
+    const int j = is_x ? e : e - a.x_size;
+    const float v = is_x ? a.x[(long)b * a.x_sb + (long)j * a.x_sj] : a.d[(long)b * a.d_sb + (long)j * a.d_si];
+    const float P = is_x ? a.prob_b[b] : a.prob_a[b];
+    const int K = a.bl[b];
+    const uint32_t purpose = is_x ? RNG_PULSE_X : RNG_PULSE_D;
+    uint32_t sr = 0;
+    if (a.up.res > 0.0f && a.up.sto_round) {
+      sr = philox4x32_10((uint32_t)j, (uint32_t)b, a.call, RNG_UPDATE_SR | ((uint32_t)is_x << 8), a.key.k0, a.key.k1).v[0];
+    }
+    const float PP = discretize_prob(fabsf(v) * P, a.up.res, a.up.sto_round, sr);
+    uint32_t word = 0;
+    if (PP != 0.0f && K > 0) {
+      for (int k0 = 0; k0 < K; k0 += 4) {
+        const Philox4 r = philox4x32_10((uint32_t)j, (uint32_t)b, a.call, purpose | ((uint32_t)(k0 >> 2) << 8), a.key.k0, a.key.k1);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          if (k0 + q < K && PP > u32_to_uniform(r.v[q])) word |= (2u << (k0 + q));
+        }
+      }
+      word |= (v > 0.0f) ? 0u : 1u;
+    }
+    if (is_x) a.x_words[(long)b * a.x_size + j] = word;
+    else a.d_words[(long)b * a.d_size + j] = word;
+  }
+}
+
+// deterministic implicit line values (src/rpucuda/dense_bit_line_maker.cpp:209-235)
+__global__ __launch_bounds__(256) void k_update_implicit_lines(UpdateArgs a) {
+  const long per_sample = (long)a.x_size + a.d_size;
+  const long total = per_sample * a.m_batch;
+  for (long idx = blockIdx.x * (long)blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
+    const int b = (int)(idx / per_sample);
+    const int e = (int)(idx % per_sample);
+    const bool is_x = e < a.x_size;
+    const int j = is_x ? e : e - a.x_size;
+    float v = is_x ? a.x[(long)b * a.x_sb + (long)j * a.x_sj] : a.d[(long)b * a.d_sb + (long)j * a.d_si];
+    if (a.lr < 0.0f) v = -v;
+    const float P = is_x ? a.prob_b[b] : a.prob_a[b];
+    const float res = is_x ? a.up.x_res_implicit : a.up.d_res_implicit;
+    uint32_t sr = 0;
+    if (res > 0.0f && a.up.sto_round) {
+      sr = philox4x32_10((uint32_t)j, (uint32_t)b, a.call, RNG_UPDATE_SR | ((uint32_t)is_x << 8), a.key.k0, a.key.k1).v[0];
+    }
+    float pp = discretize_prob(fabsf(v) * P, res, a.up.sto_round, sr);
+    pp = fmaxf(fminf(pp, 1.0f), 0.0f);
+    const float val = (v >= 0.0f) ? pp : -pp;
+    if (is_x) a.x_val[(long)b * a.x_size + j] = val;
+    else a.d_val[(long)b * a.d_size + j] = val;
+  }
+}
+
+// ---- device steps ------------------------------------------------------------------------------
+
+struct CtocStream {
+  // four N(0,1) per Philox call, keyed by (cross-point, refill index, call)
+  float n0, n1, n2, n3;
+  int left;
+  uint32_t refill;
+  uint32_t cell;
+  __device__ __forceinline__ float next(PhiloxKey key, uint32_t call) {
+    if (left == 0) {
+      float t[4];
+      philox_normal4(cell, refill, call, RNG_CTOC, key, t);
+      n0 = t[0]; n1 = t[1]; n2 = t[2]; n3 = t[3];
+      left = 4;
+      ++refill;
+    }
+    const float g = n0;
+    n0 = n1; n1 = n2; n2 = n3;
+    --left;
+    return g;
+  }
+};
+
+struct CellParams {
+  float w_max, w_min, scale_up, scale_down, slope_up, slope_down;
+};
+
+template <int KIND, bool MULT>
+__device__ __forceinline__ float device_step(float w, int sign_down, const CellParams &c, float std_, CtocStream &rng,
+                                             PhiloxKey key, uint32_t call) {
+  if (KIND == RPU_DEVICE_CONSTANT_STEP) {
+    if (std_ > 0.0f) {
+      const float f = 1.0f + std_ * rng.next(key, call);
+      if (sign_down) w -= f * c.scale_down;
+      else w += f * c.scale_up;
+    } else {
+      if (sign_down) w -= c.scale_down;
+      else w += c.scale_up;
+    }
+    w = fminf(w, c.w_max);
+    w = fmaxf(w, c.w_min);
+  } else {
+    const float f = (std_ > 0.0f) ? 1.0f + std_ * rng.next(key, call) : 1.0f;
+    if (MULT) {
+      if (sign_down) w -= (c.slope_down * w + c.scale_down) * f;
+      else w += (c.slope_up * w + c.scale_up) * f;
+    } else {
+      if (sign_down) w -= c.slope_down * w + c.scale_down * f;
+      else w += c.slope_up * w + c.scale_up * f;
+    }
+    w = fmaxf(w, c.w_min);
+    w = fminf(w, c.w_max);
+  }
+  return w;
+}
+
+template <int KIND>
+__device__ __forceinline__ CellParams load_cell(const DeviceDev &d, long k) {
+  CellParams c;
+  c.w_max = d.w_max[k];
+  c.w_min = d.w_min[k];
+  c.scale_up = d.scale_up[k];
+  c.scale_down = d.scale_down[k];
+  if (KIND != RPU_DEVICE_CONSTANT_STEP) {
+    c.slope_up = d.slope_up[k];
+    c.slope_down = d.slope_down[k];
+  } else {
+    c.slope_up = 0.0f;
+    c.slope_down = 0.0f;
+  }
+  return c;
+}
+
+// grid: x = ceil(x_size / 256), y = d_size.  One thread per cross-point, samples in batch order.
+template <int KIND, bool MULT>
+__global__ __launch_bounds__(256) void k_update_pulsed(UpdateArgs a) {
+  const int i = blockIdx.y;
+  const int j = blockIdx.x * blockDim.x + threadIdx.x;
+  if (j >= a.x_size) return;
+  const long k = (long)i * a.x_size + j;
+  const CellParams c = load_cell<KIND>(a.dev, k);
+  float w = a.w[k];
+  CtocStream rng;
+  rng.left = 0;
+  rng.refill = 0;
+  rng.cell = (uint32_t)k;
+  rng.n0 = rng.n1 = rng.n2 = rng.n3 = 0.0f;
+  const float std_ = a.dev.dw_min_std;
+  const uint32_t lr_neg = a.lr < 0.0f ? 1u : 0u;
+  const uint32_t *dwp = a.d_words + i;
+  const uint32_t *xwp = a.x_words + j;
+  for (int b = 0; b < a.m_batch; ++b) {
+    const uint32_t dw = dwp[(long)b * a.d_size]; // wave-uniform
+    if ((dw >> 1) == 0) continue;
+    const uint32_t xw = xwp[(long)b * a.x_size];
+    int n = __popc(xw & dw & ~1u);
+    if (n == 0) continue;
+    // sign > 0 (step down) when x and d have the same sign and lr > 0
+    const int sign_down = (((xw ^ dw) & 1u) ^ lr_neg) == 0u;
+    for (; n > 0; --n) w = device_step<KIND, MULT>(w, sign_down, c, std_, rng, a.key, a.call);
+  }
+  a.w[k] = w;
+}
+
+// deterministic implicit: n = (int) rintf((dv * BL) * xv) per sample (dense_bit_line_maker.cpp:237-264),
+// |n| steps, n > 0 steps down (rpu_pulsed_device.h:461-474)
+template <int KIND, bool MULT>
+__global__ __launch_bounds__(256) void k_update_implicit(UpdateArgs a) {
+  const int i = blockIdx.y;
+  const int j = blockIdx.x * blockDim.x + threadIdx.x;
+  if (j >= a.x_size) return;
+  const long k = (long)i * a.x_size + j;
+  const CellParams c = load_cell<KIND>(a.dev, k);
+  float w = a.w[k];
+  CtocStream rng;
+  rng.left = 0;
+  rng.refill = 0;
+  rng.cell = (uint32_t)k;
+  rng.n0 = rng.n1 = rng.n2 = rng.n3 = 0.0f;
+  const float std_ = a.dev.dw_min_std;
+  for (int b = 0; b < a.m_batch; ++b) {
+    float dc = a.d_val[(long)b * a.d_size + i];
+    if (dc == 0.0f) continue;
+    dc *= (float)a.bl[b];
+    const int cn = (int)rintf(dc * a.x_val[(long)b * a.x_size + j]);
+    if (cn == 0) continue;
+    const int sign_down = cn > 0;
+    for (int n = abs(cn); n > 0; --n) w = device_step<KIND, MULT>(w, sign_down, c, std_, rng, a.key, a.call);
+  }
+  a.w[k] = w;
+}
+
+__global__ __launch_bounds__(256) void k_implicit_counts(UpdateArgs a, int32_t *counts) {
+  const long per = (long)a.x_size * a.d_size;
+  const long total = per * a.m_batch;
+  for (long idx = blockIdx.x * (long)blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
+    const int b = (int)(idx / per);
+    const long rem = idx % per;
+    const int i = (int)(rem / a.x_size);
+    const int j = (int)(rem % a.x_size);
+    float dc = a.d_val[(long)b * a.d_size + i];
+    int cn = 0;
+    if (dc != 0.0f) {
+      dc *= (float)a.bl[b];
+      cn = (int)rintf(dc * a.x_val[(long)b * a.x_size + j]);
+    }
+    counts[idx] = cn;
+  }
+}
+
+__global__ void k_clip(float *w, const float *w_min, const float *w_max, size_t n) {
+  for (size_t idx = blockIdx.x * (size_t)blockDim.x + threadIdx.x; idx < n; idx += (size_t)gridDim.x * blockDim.x) {
+    float v = w[idx];
+    v = fminf(v, w_max[idx]);
+    v = fmaxf(v, w_min[idx]);
+    w[idx] = v;
+  }
+}
+
+int grid_for(long total) {
+  long blocks = (total + 255) / 256;
+  if (blocks > 65536) blocks = 65536;
+  if (blocks < 1) blocks = 1;
+  return (int)blocks;
+}
+
+} // namespace
+
+void launch_update_prepare(const UpdateArgs &a, hipStream_t s) {
+  hipLaunchKernelGGL(k_update_prepare, dim3(a.m_batch), dim3(256), 0, s, a);
+}
+
+void launch_update_bitlines(const UpdateArgs &a, hipStream_t s) {
+  const long total = ((long)a.x_size + a.d_size) * a.m_batch;
+  hipLaunchKernelGGL(k_update_bitlines, dim3(grid_for(total)), dim3(256), 0, s, a);
+}
+
+void launch_update_implicit_lines(const UpdateArgs &a, hipStream_t s) {
+  const long total = ((long)a.x_size + a.d_size) * a.m_batch;
+  hipLaunchKernelGGL(k_update_implicit_lines, dim3(grid_for(total)), dim3(256), 0, s, a);
+}
+
+#define RPU_DISPATCH_DEVICE(KERNEL, grid, s, a)                                                     \
+  do {                                                                                              \
+    if ((a).dev.kind == RPU_DEVICE_CONSTANT_STEP) {                                                 \
+      hipLaunchKernelGGL((KERNEL<RPU_DEVICE_CONSTANT_STEP, true>), grid, dim3(256), 0, s, a);       \
+    } else if ((a).dev.ls_mult_noise) {                                                             \
+      hipLaunchKernelGGL((KERNEL<RPU_DEVICE_LINEAR_STEP, true>), grid, dim3(256), 0, s, a);         \
+    } else {                                                                                        \
+      hipLaunchKernelGGL((KERNEL<RPU_DEVICE_LINEAR_STEP, false>), grid, dim3(256), 0, s, a);        \
+    }                                                                                               \
+  } while (0)
+
+void launch_update_pulsed(const UpdateArgs &a, hipStream_t s) {
+  dim3 grid((a.x_size + 255) / 256, a.d_size);
+  RPU_DISPATCH_DEVICE(k_update_pulsed, grid, s, a);
+}
+
+void launch_update_implicit(const UpdateArgs &a, hipStream_t s) {
+  dim3 grid((a.x_size + 255) / 256, a.d_size);
+  RPU_DISPATCH_DEVICE(k_update_implicit, grid, s, a);
+}
+
+void launch_implicit_counts(const UpdateArgs &a, int32_t *counts, hipStream_t s) {
+  const long total = (long)a.x_size * a.d_size * a.m_batch;
+  hipLaunchKernelGGL(k_implicit_counts, dim3(grid_for(total)), dim3(256), 0, s, a, counts);
+}
+
+void launch_clip(float *w, const float *w_min, const float *w_max, size_t n, hipStream_t s) {
+  hipLaunchKernelGGL(k_clip, dim3(grid_for((long)n)), dim3(256), 0, s, w, w_min, w_max, n);
+}
+
+} // namespace rpu_amd

@@ -1,0 +1,669 @@
+// The analog tile object behind the C ABI: host-side state (parameters, sampled device arrays,
+// weights) plus, once moved to a GPU, the HBM-resident weights / per-device parameters and the scratch
+// buffers of the kernels.  It plays the role of the reference's RPUPulsed (src/rpucuda/rpu_pulsed.{h,cpp})
+// and RPUCudaPulsed (src/rpucuda/cuda/rpucuda_pulsed.{h,cu}) pair.
+#include "../../include/rpu_amd.h"
+#include "kernels.h"
+#include "rpu_host.h"
+
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstring>
+#include <memory>
+#include <mutex>
+#include <string>
+#include <vector>
+
+namespace rpu_amd {
+
+#define RPU_HIP_CHECK(expr)                                                                         \
+  do {                                                                                              \
+    hipError_t _e = (expr);                                                                         \
+    if (_e != hipSuccess) {                                                                         \
+      throw RpuError(std::string("HIP error: ") + hipGetErrorString(_e) + " in " #expr);            \
+    }                                                                                               \
+  } while (0)
+
+namespace {
+
+template <typename T> struct DevBuf {
+  T *p = nullptr;
+  size_t n = 0;
+  void ensure(size_t count) {
+    if (count <= n) return;
+    release();
+    RPU_HIP_CHECK(hipMalloc((void **)&p, count * sizeof(T)));
+    n = count;
+  }
+  void release() {
+    if (p) (void)hipFree(p);
+    p = nullptr;
+    n = 0;
+  }
+};
+
+class DeviceGuard {
+public:
+  explicit DeviceGuard(int device) {
+    RPU_HIP_CHECK(hipGetDevice(&prev_));
+    if (device != prev_) {
+      RPU_HIP_CHECK(hipSetDevice(device));
+      changed_ = true;
+    }
+  }
+  ~DeviceGuard() {
+    if (changed_) (void)hipSetDevice(prev_);
+  }
+
+private:
+  int prev_ = 0;
+  bool changed_ = false;
+};
+
+__global__ void k_philox_probe(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint32_t k0, uint32_t k1,
+                               uint32_t *out) {
+  const Philox4 r = philox4x32_10(c0, c1, c2, c3, k0, k1);
+  out[0] = r.v[0];
+  out[1] = r.v[1];
+  out[2] = r.v[2];
+  out[3] = r.v[3];
+}
+
+const char *const kHiddenNames[10] = {"max_bound",       "min_bound",  "dwmin_up", "dwmin_down", "decay_scales",
+                                      "diffusion_rates", "reset_bias", "drift_nu", "slope_up",   "slope_down"};
+
+} // namespace
+
+struct Tile {
+  int X = 0, D = 0;
+  IOPar fio, bio;
+  UpdatePar up;
+  DevicePar dev;
+  DeviceArrays arr;          // host copy of the per-device parameters (never changed by the kernels)
+  std::vector<float> w_host; // weights while the tile is not resident on a GPU
+  float lr = 0.0f;           // as RPUAbstract: zero until set_learning_rate
+  uint64_t seed = 0;
+  uint32_t call = 0;
+  std::mutex mutex;
+
+  // GPU residency
+  int device_id = -1;
+  hipStream_t last_stream = nullptr;
+  DevBuf<float> d_w, d_wmax, d_wmin, d_sup, d_sdown, d_slup, d_sldown;
+  // MVM scratch
+  DevBuf<float> s_nm, s_nmnp, s_red, s_scale, s_fin, s_bias;
+  DevBuf<int> s_rounds, s_hitup, s_hitlo, s_list0, s_list1, s_count;
+  // update scratch
+  DevBuf<int> u_bl;
+  DevBuf<float> u_a, u_b, u_xval, u_dval;
+  DevBuf<uint32_t> u_xw, u_dw;
+  int last_update_batch = 0;
+  int last_update_pulse = -1;
+  int last_forward_batch = 0;
+
+  bool resident() const { return device_id >= 0; }
+  size_t size() const { return (size_t)X * (size_t)D; }
+
+  ~Tile() {
+    if (resident()) {
+      try {
+        DeviceGuard g(device_id);
+        (void)hipDeviceSynchronize();
+        release_all();
+      } catch (...) {
+      }
+    }
+  }
+
+  void release_all() {
+    d_w.release(); d_wmax.release(); d_wmin.release(); d_sup.release(); d_sdown.release();
+    d_slup.release(); d_sldown.release();
+    s_nm.release(); s_nmnp.release(); s_red.release(); s_scale.release(); s_fin.release(); s_bias.release();
+    s_rounds.release(); s_hitup.release(); s_hitlo.release(); s_list0.release(); s_list1.release(); s_count.release();
+    u_bl.release(); u_a.release(); u_b.release(); u_xval.release(); u_dval.release(); u_xw.release(); u_dw.release();
+  }
+
+  PhiloxKey key() const {
+    PhiloxKey k;
+    k.k0 = (uint32_t)(seed & 0xffffffffu);
+    k.k1 = (uint32_t)(seed >> 32);
+    return k;
+  }
+
+  void clip_host(std::vector<float> &w) const {
+    if (!dev.pulsed()) return;
+    for (size_t i = 0; i < w.size(); ++i) {
+      w[i] = std::min(w[i], arr.w_max[i]);
+      w[i] = std::max(w[i], arr.w_min[i]);
+    }
+  }
+
+  void upload_params() {
+    if (!dev.pulsed()) return;
+    const size_t n = size(), bytes = n * sizeof(float);
+    d_wmax.ensure(n); d_wmin.ensure(n); d_sup.ensure(n); d_sdown.ensure(n);
+    RPU_HIP_CHECK(hipMemcpy(d_wmax.p, arr.w_max.data(), bytes, hipMemcpyHostToDevice));
+    RPU_HIP_CHECK(hipMemcpy(d_wmin.p, arr.w_min.data(), bytes, hipMemcpyHostToDevice));
+    RPU_HIP_CHECK(hipMemcpy(d_sup.p, arr.scale_up.data(), bytes, hipMemcpyHostToDevice));
+    RPU_HIP_CHECK(hipMemcpy(d_sdown.p, arr.scale_down.data(), bytes, hipMemcpyHostToDevice));
+    if (dev.linear()) {
+      d_slup.ensure(n); d_sldown.ensure(n);
+      RPU_HIP_CHECK(hipMemcpy(d_slup.p, arr.slope_up.data(), bytes, hipMemcpyHostToDevice));
+      RPU_HIP_CHECK(hipMemcpy(d_sldown.p, arr.slope_down.data(), bytes, hipMemcpyHostToDevice));
+    }
+  }
+
+  void to_device(int dev_id) {
+    if (resident()) throw RpuError("Tile is already resident on a GPU.");
+    int count = 0;
+    if (hipGetDeviceCount(&count) != hipSuccess || count <= 0) {
+      throw RpuError("No HIP device available: this library has no CPU compute path.");
+    }
+    int target = dev_id;
+    if (target < 0) RPU_HIP_CHECK(hipGetDevice(&target));
+    if (target >= count) throw RpuError("Invalid HIP device id.");
+    DeviceGuard g(target);
+    device_id = target;
+    try {
+      d_w.ensure(size());
+      RPU_HIP_CHECK(hipMemcpy(d_w.p, w_host.data(), size() * sizeof(float), hipMemcpyHostToDevice));
+      upload_params();
+      s_count.ensure(64);
+    } catch (...) {
+      release_all();
+      device_id = -1;
+      throw;
+    }
+  }
+
+  void sync_last() {
+    RPU_HIP_CHECK(hipStreamSynchronize(last_stream));
+  }
+
+  void ensure_mvm_scratch(int B) {
+    const size_t n = (size_t)B;
+    s_nm.ensure(n); s_nmnp.ensure(n); s_red.ensure(n); s_scale.ensure(n); s_fin.ensure(n);
+    s_rounds.ensure(n); s_hitup.ensure(n); s_hitlo.ensure(n); s_list0.ensure(n); s_list1.ensure(n);
+    s_count.ensure(64);
+  }
+
+  IoDev io_dev(const IOPar &io) const {
+    IoDev d;
+    d.inp_res = io.p.inp_res; d.inp_bound = io.p.inp_bound; d.inp_noise = io.p.inp_noise; d.inp_asym = io.p.inp_asymmetry;
+    d.out_res = io.p.out_res; d.out_bound = io.p.out_bound; d.out_noise = io.p.out_noise; d.out_asym = io.p.out_asymmetry;
+    d.out_scale = io.p.out_scale; d.nm_thres = io.p.nm_thres; d.nm_assumed_wmax = io.p.nm_assumed_wmax;
+    d.max_bm_res = io.p.max_bm_res; d.noise_management = io.p.noise_management;
+    d.bound_management = io.p.bound_management; d.bm_test_negative_bound = io.p.bm_test_negative_bound;
+    d.max_bm_factor = io.p.max_bm_factor; d.inp_sto_round = io.p.inp_sto_round; d.out_sto_round = io.p.out_sto_round;
+    d.perfect = io.perfect ? 1 : 0;
+    return d;
+  }
+
+  void check_compute(int m_batch, const void *p0, const void *p1) {
+    if (!resident()) throw RpuError("Tile is not resident on a GPU: forward / backward / update need rpu_tile_to_device first.");
+    if (m_batch <= 0) throw RpuError("m_batch must be positive.");
+    if (!p0 || !p1) throw RpuError("Null device pointer.");
+  }
+
+  // shared driver of forward (transposed = 0) and backward (transposed = 1)
+  void mvm(const float *in, float *out, int B, bool bias, bool in_trans, bool out_trans, bool transposed, hipStream_t s) {
+    const IOPar &io = transposed ? bio : fio;
+    const int K = transposed ? D : X;
+    const int O = transposed ? X : D;
+    ensure_mvm_scratch(B);
+    MvmArgs a{};
+    a.w = d_w.p; a.x_size = X; a.d_size = D; a.m_batch = B; a.K = K; a.O = O; a.transposed = transposed ? 1 : 0;
+    a.io = io_dev(io);
+    a.alpha = io.p.out_scale; a.beta = 0.0f;
+    a.key = key(); a.call = call++;
+    a.st.nm = s_nm.p; a.st.nm_np = s_nmnp.p; a.st.red = s_red.p; a.st.scale = s_scale.p; a.st.fin = s_fin.p;
+    a.st.rounds = s_rounds.p; a.st.hit_up = s_hitup.p; a.st.hit_lo = s_hitlo.p;
+    a.st.list[0] = s_list0.p; a.st.list[1] = s_list1.p; a.st.count = s_count.p;
+
+    // the x side carries the optional bias column: input of forward, output of backward
+    float *final_out = out;
+    if (!transposed) {
+      if (bias) {
+        s_bias.ensure((size_t)B * X);
+        launch_make_bias(in, s_bias.p, B, X, in_trans ? 1 : 0, s);
+        a.in = s_bias.p; a.in_sb = X; a.in_sk = 1;
+      } else {
+        a.in = in; a.in_sb = in_trans ? 1 : X; a.in_sk = in_trans ? B : 1;
+      }
+      a.out = out; a.out_sb = out_trans ? 1 : D; a.out_so = out_trans ? B : 1;
+    } else {
+      a.in = in; a.in_sb = in_trans ? 1 : D; a.in_sk = in_trans ? B : 1;
+      if (bias) {
+        s_bias.ensure((size_t)B * X);
+        a.out = s_bias.p; a.out_sb = X; a.out_so = 1;
+      } else {
+        a.out = out; a.out_sb = out_trans ? 1 : X; a.out_so = out_trans ? B : 1;
+      }
+    }
+
+    if (io.perfect) {
+      a.round = 0;
+      launch_mvm_round(a, s);
+    } else {
+      launch_mvm_init(a, s);
+      const int rounds = mvm_max_rounds(a.io);
+      for (int r = 0; r < rounds; ++r) {
+        a.round = r;
+        launch_mvm_round(a, s);
+        if (r + 1 < rounds) launch_mvm_advance(a, s);
+      }
+    }
+    if (transposed && bias) launch_drop_bias(s_bias.p, final_out, B, X, out_trans ? 1 : 0, s);
+    RPU_HIP_CHECK(hipGetLastError());
+    last_stream = s;
+    if (!transposed) last_forward_batch = B;
+  }
+
+  void update(const float *x, const float *d, int B, bool bias, bool x_trans, bool d_trans, hipStream_t s) {
+    if (lr == 0.0f) return;
+    const float *xin = x;
+    long x_sb = x_trans ? 1 : X, x_sj = x_trans ? B : 1;
+    if (bias) {
+      s_bias.ensure((size_t)B * X);
+      launch_make_bias(x, s_bias.p, B, X, x_trans ? 1 : 0, s);
+      xin = s_bias.p; x_sb = X; x_sj = 1;
+    }
+    const long d_sb = d_trans ? 1 : D, d_si = d_trans ? B : 1;
+
+    if (!dev.pulsed() || up.p.pulse_type == RPU_PULSE_NONE) {
+      // W += -lr * d^T x as a contraction over the batch (rpu.cpp:624-634): "weights" = d, K = batch
+      MvmArgs a{};
+      a.w = d; a.transposed = d_trans ? 0 : 1; // element (o = i, k = b): d[b * D + i] or d[i * B + b]
+      a.x_size = d_trans ? B : D; a.d_size = d_trans ? D : B;
+      a.K = B; a.O = D; a.m_batch = X;
+      a.in = xin; a.in_sb = x_sj; a.in_sk = x_sb; // "sample" = column j of x, contraction over b
+      a.out = d_w.p; a.out_sb = 1; a.out_so = X;
+      a.io = io_dev(fio); a.io.perfect = 1;
+      a.alpha = -lr; a.beta = 1.0f; a.round = 0;
+      a.key = key(); a.call = call++;
+      launch_mvm_round(a, s);
+      RPU_HIP_CHECK(hipGetLastError());
+      last_stream = s;
+      last_update_batch = B;
+      last_update_pulse = RPU_PULSE_NONE;
+      return;
+    }
+
+    UpdateArgs a{};
+    a.w = d_w.p; a.x_size = X; a.d_size = D; a.m_batch = B;
+    a.x = xin; a.x_sb = x_sb; a.x_sj = x_sj; a.d = d; a.d_sb = d_sb; a.d_si = d_si;
+    a.lr = lr;
+    a.up.pulse_type = up.p.pulse_type; a.up.desired_bl = up.p.desired_bl; a.up.fixed_bl = up.p.fixed_bl;
+    a.up.update_management = up.p.update_management; a.up.update_bl_management = up.p.update_bl_management;
+    a.up.sto_round = up.p.sto_round; a.up.um_grad_scale = up.p.um_grad_scale; a.up.res = up.p.res;
+    a.up.x_res_implicit = up.p.x_res_implicit; a.up.d_res_implicit = up.p.d_res_implicit;
+    a.dev.kind = dev.p.kind; a.dev.ls_mult_noise = dev.p.ls_mult_noise; a.dev.dw_min = dev.p.dw_min;
+    a.dev.dw_min_std = dev.p.dw_min_std;
+    a.dev.w_max = d_wmax.p; a.dev.w_min = d_wmin.p; a.dev.scale_up = d_sup.p; a.dev.scale_down = d_sdown.p;
+    a.dev.slope_up = d_slup.p; a.dev.slope_down = d_sldown.p;
+    u_bl.ensure(B); u_a.ensure(B); u_b.ensure(B);
+    a.bl = u_bl.p; a.prob_a = u_a.p; a.prob_b = u_b.p;
+    a.key = key(); a.call = call++;
+    launch_update_prepare(a, s);
+    if (up.p.pulse_type == RPU_PULSE_STOCHASTIC_COMPRESSED) {
+      u_xw.ensure((size_t)B * X); u_dw.ensure((size_t)B * D);
+      a.x_words = u_xw.p; a.d_words = u_dw.p;
+      launch_update_bitlines(a, s);
+      launch_update_pulsed(a, s);
+    } else {
+      u_xval.ensure((size_t)B * X); u_dval.ensure((size_t)B * D);
+      a.x_val = u_xval.p; a.d_val = u_dval.p;
+      launch_update_implicit_lines(a, s);
+      launch_update_implicit(a, s);
+    }
+    RPU_HIP_CHECK(hipGetLastError());
+    last_stream = s;
+    last_update_batch = B;
+    last_update_pulse = up.p.pulse_type;
+  }
+};
+
+} // namespace rpu_amd
+
+// ---------------------------------------------------------------------------------------------------
+// C ABI
+
+using namespace rpu_amd;
+
+struct rpu_tile {
+  Tile t;
+};
+
+namespace {
+thread_local std::string g_last_error;
+
+template <typename F> int guarded(F &&f) {
+  try {
+    f();
+    return 0;
+  } catch (const std::exception &e) {
+    g_last_error = e.what();
+    return 1;
+  } catch (...) {
+    g_last_error = "unknown error";
+    return 2;
+  }
+}
+} // namespace
+
+extern "C" {
+
+const char *rpu_last_error(void) { return g_last_error.c_str(); }
+int rpu_abi_version(void) { return RPU_AMD_ABI_VERSION; }
+
+int rpu_tile_config_default(rpu_tile_config *cfg, int device_kind) {
+  return guarded([&] {
+    if (!cfg) throw RpuError("cfg is null");
+    fill_default_config(cfg, device_kind);
+  });
+}
+
+int rpu_tile_create(rpu_tile_t **out, int x_size, int d_size, const rpu_tile_config *cfg) {
+  return guarded([&] {
+    if (!out || !cfg) throw RpuError("null argument");
+    if (x_size <= 0 || d_size <= 0) throw RpuError("x_size and d_size must be positive.");
+    auto h = std::make_unique<rpu_tile>();
+    Tile &t = h->t;
+    t.X = x_size;
+    t.D = d_size;
+    t.fio.p = cfg->f_io;
+    t.bio.p = cfg->b_io;
+    t.up.p = cfg->up;
+    t.dev.p = cfg->device;
+    t.fio.initialize(false);
+    t.bio.initialize(true);
+    t.up.initialize();
+    t.dev.initialize();
+    t.dev.populate(x_size, d_size, t.arr);
+    t.w_host.assign(t.size(), 0.0f);
+    t.clip_host(t.w_host);
+    *out = h.release();
+  });
+}
+
+int rpu_tile_clone(rpu_tile_t **out, const rpu_tile_t *src_c) {
+  return guarded([&] {
+    if (!out || !src_c) throw RpuError("null argument");
+    rpu_tile *src = const_cast<rpu_tile *>(src_c);
+    std::lock_guard<std::mutex> lock(src->t.mutex);
+    auto h = std::make_unique<rpu_tile>();
+    Tile &t = h->t;
+    const Tile &s = src->t;
+    t.X = s.X; t.D = s.D; t.fio = s.fio; t.bio = s.bio; t.up = s.up; t.dev = s.dev; t.arr = s.arr;
+    t.lr = s.lr; t.seed = s.seed; t.call = s.call;
+    t.w_host = s.w_host;
+    if (s.resident()) {
+      DeviceGuard g(s.device_id);
+      RPU_HIP_CHECK(hipStreamSynchronize(s.last_stream));
+      t.w_host.resize(s.size());
+      RPU_HIP_CHECK(hipMemcpy(t.w_host.data(), s.d_w.p, s.size() * sizeof(float), hipMemcpyDeviceToHost));
+      t.to_device(s.device_id);
+    }
+    *out = h.release();
+  });
+}
+
+int rpu_tile_to_device(rpu_tile_t *tile, int device_id) {
+  return guarded([&] {
+    if (!tile) throw RpuError("null tile");
+    std::lock_guard<std::mutex> lock(tile->t.mutex);
+    tile->t.to_device(device_id);
+  });
+}
+
+int rpu_tile_destroy(rpu_tile_t *tile) {
+  return guarded([&] { delete tile; });
+}
+
+int rpu_tile_forward(rpu_tile_t *tile, const float *x_dev, float *y_dev, int m_batch, int bias, int x_trans,
+                     int d_trans, int is_test, void *stream) {
+  (void)is_test; // the analog forward pass is the same in training and evaluation (rpu_forward_backward_pass.cpp:816-818)
+  return guarded([&] {
+    if (!tile) throw RpuError("null tile");
+    Tile &t = tile->t;
+    std::lock_guard<std::mutex> lock(t.mutex);
+    t.check_compute(m_batch, x_dev, y_dev);
+    DeviceGuard g(t.device_id);
+    t.mvm(x_dev, y_dev, m_batch, bias != 0, x_trans != 0, d_trans != 0, false, (hipStream_t)stream);
+  });
+}
+
+int rpu_tile_backward(rpu_tile_t *tile, const float *d_dev, float *x_dev, int m_batch, int bias, int d_trans,
+                      int x_trans, void *stream) {
+  return guarded([&] {
+    if (!tile) throw RpuError("null tile");
+    Tile &t = tile->t;
+    std::lock_guard<std::mutex> lock(t.mutex);
+    t.check_compute(m_batch, d_dev, x_dev);
+    DeviceGuard g(t.device_id);
+    t.mvm(d_dev, x_dev, m_batch, bias != 0, d_trans != 0, x_trans != 0, true, (hipStream_t)stream);
+  });
+}
+
+int rpu_tile_update(rpu_tile_t *tile, const float *x_dev, const float *d_dev, int m_batch, int bias, int x_trans,
+                    int d_trans, void *stream) {
+  return guarded([&] {
+    if (!tile) throw RpuError("null tile");
+    Tile &t = tile->t;
+    std::lock_guard<std::mutex> lock(t.mutex);
+    t.check_compute(m_batch, x_dev, d_dev);
+    DeviceGuard g(t.device_id);
+    t.update(x_dev, d_dev, m_batch, bias != 0, x_trans != 0, d_trans != 0, (hipStream_t)stream);
+  });
+}
+
+int rpu_tile_get_x_size(const rpu_tile_t *tile) { return tile ? tile->t.X : -1; }
+int rpu_tile_get_d_size(const rpu_tile_t *tile) { return tile ? tile->t.D : -1; }
+int rpu_tile_is_on_device(const rpu_tile_t *tile) { return (tile && tile->t.resident()) ? 1 : 0; }
+
+int rpu_tile_set_learning_rate(rpu_tile_t *tile, float lr) {
+  return guarded([&] {
+    if (!tile) throw RpuError("null tile");
+    std::lock_guard<std::mutex> lock(tile->t.mutex);
+    tile->t.lr = lr;
+  });
+}
+float rpu_tile_get_learning_rate(const rpu_tile_t *tile) { return tile ? tile->t.lr : 0.0f; }
+
+int rpu_tile_set_weights(rpu_tile_t *tile, const float *w_host) {
+  return guarded([&] {
+    if (!tile || !w_host) throw RpuError("null argument");
+    Tile &t = tile->t;
+    std::lock_guard<std::mutex> lock(t.mutex);
+    std::vector<float> w(w_host, w_host + t.size());
+    t.clip_host(w);
+    if (t.resident()) {
+      DeviceGuard g(t.device_id);
+      t.sync_last();
+      RPU_HIP_CHECK(hipMemcpy(t.d_w.p, w.data(), t.size() * sizeof(float), hipMemcpyHostToDevice));
+    } else {
+      t.w_host.swap(w);
+    }
+  });
+}
+
+int rpu_tile_get_weights(rpu_tile_t *tile, float *w_host) {
+  return guarded([&] {
+    if (!tile || !w_host) throw RpuError("null argument");
+    Tile &t = tile->t;
+    std::lock_guard<std::mutex> lock(t.mutex);
+    if (t.resident()) {
+      DeviceGuard g(t.device_id);
+      t.sync_last();
+      RPU_HIP_CHECK(hipMemcpy(w_host, t.d_w.p, t.size() * sizeof(float), hipMemcpyDeviceToHost));
+    } else {
+      std::memcpy(w_host, t.w_host.data(), t.size() * sizeof(float));
+    }
+  });
+}
+
+int rpu_tile_weights_device_ptr(rpu_tile_t *tile, float **w_dev) {
+  return guarded([&] {
+    if (!tile || !w_dev) throw RpuError("null argument");
+    *w_dev = tile->t.resident() ? tile->t.d_w.p : nullptr;
+  });
+}
+
+int rpu_tile_hidden_parameter_count(const rpu_tile_t *tile) {
+  if (!tile || !tile->t.dev.pulsed()) return 0;
+  return tile->t.dev.linear() ? 10 : 8;
+}
+
+const char *rpu_tile_hidden_parameter_name(const rpu_tile_t *tile, int idx) {
+  if (idx < 0 || idx >= rpu_tile_hidden_parameter_count(tile)) return nullptr;
+  return kHiddenNames[idx];
+}
+
+static std::vector<float> *hidden_slot(Tile &t, int idx) {
+  switch (idx) {
+  case 0: return &t.arr.w_max;
+  case 1: return &t.arr.w_min;
+  case 2: return &t.arr.scale_up;
+  case 3: return &t.arr.scale_down;
+  case 4: return &t.arr.decay_scale;
+  case 5: return &t.arr.diffusion_rate;
+  case 6: return &t.arr.reset_bias;
+  case 8: return &t.arr.slope_up;
+  case 9: return &t.arr.slope_down;
+  default: return nullptr; // drift_nu: no drifter on this path, reported as zeros
+  }
+}
+
+int rpu_tile_get_hidden_parameters(rpu_tile_t *tile, float *data_host) {
+  return guarded([&] {
+    if (!tile || !data_host) throw RpuError("null argument");
+    Tile &t = tile->t;
+    std::lock_guard<std::mutex> lock(t.mutex);
+    const size_t n = t.size();
+    const int count = rpu_tile_hidden_parameter_count(tile);
+    for (int k = 0; k < count; ++k) {
+      std::vector<float> *a = hidden_slot(t, k);
+      if (a) std::memcpy(data_host + (size_t)k * n, a->data(), n * sizeof(float));
+      else std::memset(data_host + (size_t)k * n, 0, n * sizeof(float));
+    }
+  });
+}
+
+int rpu_tile_set_hidden_parameters(rpu_tile_t *tile, const float *data_host) {
+  return guarded([&] {
+    if (!tile || !data_host) throw RpuError("null argument");
+    Tile &t = tile->t;
+    std::lock_guard<std::mutex> lock(t.mutex);
+    const size_t n = t.size();
+    const int count = rpu_tile_hidden_parameter_count(tile);
+    for (int k = 0; k < count; ++k) {
+      std::vector<float> *a = hidden_slot(t, k);
+      if (a) std::memcpy(a->data(), data_host + (size_t)k * n, n * sizeof(float));
+    }
+    // new bounds apply to the current weights at once (rpu_pulsed_device.cpp setDeviceParameter -> onSetWeights)
+    if (t.resident()) {
+      DeviceGuard g(t.device_id);
+      t.sync_last();
+      t.upload_params();
+      launch_clip(t.d_w.p, t.d_wmin.p, t.d_wmax.p, n, t.last_stream);
+      RPU_HIP_CHECK(hipStreamSynchronize(t.last_stream));
+    } else {
+      t.clip_host(t.w_host);
+    }
+  });
+}
+
+int rpu_tile_set_seed(rpu_tile_t *tile, uint64_t seed) {
+  return guarded([&] {
+    if (!tile) throw RpuError("null tile");
+    std::lock_guard<std::mutex> lock(tile->t.mutex);
+    tile->t.seed = seed;
+    tile->t.call = 0;
+  });
+}
+
+int rpu_tile_get_update_words(rpu_tile_t *tile, uint32_t *x_words_host, uint32_t *d_words_host, int32_t *bl_host,
+                              int m_batch) {
+  return guarded([&] {
+    if (!tile || !x_words_host || !d_words_host || !bl_host) throw RpuError("null argument");
+    Tile &t = tile->t;
+    std::lock_guard<std::mutex> lock(t.mutex);
+    if (!t.resident() || t.last_update_pulse != RPU_PULSE_STOCHASTIC_COMPRESSED || m_batch != t.last_update_batch) {
+      throw RpuError("No stochastic update of this batch size has run on this tile.");
+    }
+    DeviceGuard g(t.device_id);
+    t.sync_last();
+    RPU_HIP_CHECK(hipMemcpy(x_words_host, t.u_xw.p, (size_t)m_batch * t.X * 4, hipMemcpyDeviceToHost));
+    RPU_HIP_CHECK(hipMemcpy(d_words_host, t.u_dw.p, (size_t)m_batch * t.D * 4, hipMemcpyDeviceToHost));
+    RPU_HIP_CHECK(hipMemcpy(bl_host, t.u_bl.p, (size_t)m_batch * 4, hipMemcpyDeviceToHost));
+  });
+}
+
+int rpu_tile_get_implicit_counts(rpu_tile_t *tile, int32_t *counts_host, int m_batch) {
+  return guarded([&] {
+    if (!tile || !counts_host) throw RpuError("null argument");
+    Tile &t = tile->t;
+    std::lock_guard<std::mutex> lock(t.mutex);
+    if (!t.resident() || t.last_update_pulse != RPU_PULSE_DETERMINISTIC_IMPLICIT || m_batch != t.last_update_batch) {
+      throw RpuError("No deterministic implicit update of this batch size has run on this tile.");
+    }
+    DeviceGuard g(t.device_id);
+    t.sync_last();
+    const size_t total = (size_t)m_batch * t.size();
+    DevBuf<int32_t> tmp;
+    tmp.ensure(total);
+    UpdateArgs a{};
+    a.x_size = t.X; a.d_size = t.D; a.m_batch = m_batch;
+    a.bl = t.u_bl.p; a.x_val = t.u_xval.p; a.d_val = t.u_dval.p;
+    try {
+      launch_implicit_counts(a, tmp.p, t.last_stream);
+      RPU_HIP_CHECK(hipStreamSynchronize(t.last_stream));
+      RPU_HIP_CHECK(hipMemcpy(counts_host, tmp.p, total * 4, hipMemcpyDeviceToHost));
+    } catch (...) {
+      tmp.release();
+      throw;
+    }
+    tmp.release();
+  });
+}
+
+int rpu_tile_get_bm_rounds(rpu_tile_t *tile, int32_t *rounds_host, int m_batch) {
+  return guarded([&] {
+    if (!tile || !rounds_host) throw RpuError("null argument");
+    Tile &t = tile->t;
+    std::lock_guard<std::mutex> lock(t.mutex);
+    if (!t.resident() || m_batch != t.last_forward_batch || t.fio.perfect) {
+      throw RpuError("No analog forward pass of this batch size has run on this tile.");
+    }
+    DeviceGuard g(t.device_id);
+    t.sync_last();
+    RPU_HIP_CHECK(hipMemcpy(rounds_host, t.s_rounds.p, (size_t)m_batch * 4, hipMemcpyDeviceToHost));
+  });
+}
+
+int rpu_philox4x32_10(const uint32_t counter[4], const uint32_t key[2], uint32_t out[4]) {
+  return guarded([&] {
+    if (!counter || !key || !out) throw RpuError("null argument");
+    const Philox4 r = philox4x32_10(counter[0], counter[1], counter[2], counter[3], key[0], key[1]);
+    for (int i = 0; i < 4; ++i) out[i] = r.v[i];
+  });
+}
+
+int rpu_philox4x32_10_device(const uint32_t counter[4], const uint32_t key[2], uint32_t out[4], int device_id) {
+  return guarded([&] {
+    if (!counter || !key || !out) throw RpuError("null argument");
+    int target = device_id;
+    if (target < 0) RPU_HIP_CHECK(hipGetDevice(&target));
+    DeviceGuard g(target);
+    DevBuf<uint32_t> buf;
+    buf.ensure(4);
+    hipLaunchKernelGGL(k_philox_probe, dim3(1), dim3(1), 0, nullptr, counter[0], counter[1], counter[2], counter[3],
+                       key[0], key[1], buf.p);
+    hipError_t e = hipMemcpy(out, buf.p, 16, hipMemcpyDeviceToHost);
+    buf.release();
+    if (e != hipSuccess) throw RpuError(std::string("HIP error: ") + hipGetErrorString(e));
+  });
+}
+
+} // extern "C"

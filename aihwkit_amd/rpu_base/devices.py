@@ -1,0 +1,304 @@
+"""Mirror of ``rpu_base.devices``: parameter structs and enums of the analog tile.
+
+Class and field names are those of the reference bindings
+(src/aihwkit/simulator/rpu_base_src/rpu_base_devices.cpp:436-656, rpu_base_utils.cpp:55-91) so that
+``parameters_to_bindings`` style code (src/aihwkit/simulator/parameters/helpers.py:64-123), which copies
+dataclass fields onto these objects by name, works unchanged.  Defaults are the C++ defaults of the
+reference structs (src/rpucuda/rpu_pulsed_meta_parameter.h:50-106,248-323, rpu_pulsed_device.h:52-114,
+rpu_linearstep_device.h:16-80).
+"""
+import enum
+import sys
+
+from .._cabi import DeviceParams, IOParams, TileConfig, UpdateParams
+
+FLT_MAX = 3.4028234663852886e38
+
+
+class BoundManagementType(enum.IntEnum):
+    """rpu_base_utils.cpp:55-58."""
+
+    # pylint: disable=invalid-name
+    NONE = 0
+    Iterative = 1
+    IterativeWorstCase = 2
+
+
+class NoiseManagementType(enum.IntEnum):
+    """rpu_base_utils.cpp:66-72."""
+
+    NONE = 0
+    AbsMax = 1
+    AbsMaxNPSum = 2
+    Max = 3
+    Constant = 4
+    AverageAbsMax = 5
+
+
+class WeightNoiseType(enum.IntEnum):
+    """rpu_base_utils.cpp:74-77."""
+
+    NONE = 0
+    AdditiveConstant = 1
+    PCMRead = 2
+
+
+class PulseType(enum.IntEnum):
+    """rpu_base_utils.cpp:79-85."""
+
+    NONE = 0
+    StochasticCompressed = 1
+    Stochastic = 2
+    NoneWithDevice = 3
+    MeanCount = 4
+    DeterministicImplicit = 5
+
+
+class AnalogMVType(enum.IntEnum):
+    """rpu_base_utils.cpp:87-91."""
+
+    Ideal = 0
+    OnePass = 1
+    PosNegSeparate = 2
+    PosNegSeparateDigitalSum = 3
+
+
+# pybind exposes the member called "None" of each enum; Python's enum cannot define it in the class body.
+for _e in (BoundManagementType, NoiseManagementType, WeightNoiseType, PulseType):
+    setattr(_e, "None", _e.NONE)  # reachable through getattr(Enum, "None") like the reference
+
+
+class _Struct:
+    """Attribute bag with fixed fields: unknown names raise, as on a pybind struct."""
+
+    _defaults = {}
+
+    def __init__(self):
+        for name, value in self._all_defaults().items():
+            object.__setattr__(self, name, value)
+
+    @classmethod
+    def _all_defaults(cls):
+        out = {}
+        for klass in reversed(cls.__mro__):
+            out.update(getattr(klass, "_defaults", {}))
+        return out
+
+    def __setattr__(self, name, value):
+        if name not in self._all_defaults():
+            raise AttributeError(f"{type(self).__name__} has no field {name!r}")
+        object.__setattr__(self, name, value)
+
+    def __str__(self):
+        fields = ", ".join(f"{k}={getattr(self, k)!r}" for k in self._all_defaults())
+        return f"{type(self).__name__}({fields})"
+
+
+class AnalogTileInputOutputParameter(_Struct):
+    """rpu_base_devices.cpp:485-519 over IOMetaParameter (rpu_pulsed_meta_parameter.h:50-106)."""
+
+    _defaults = dict(
+        bm_test_negative_bound=True, bound_management=BoundManagementType.NONE, inp_bound=1.0,
+        inp_noise=0.0, inp_res=1.0 / (2.0**7 - 2.0), inp_sto_round=False, is_perfect=False,
+        max_bm_factor=1000, max_bm_res=0.25, nm_assumed_wmax=0.6, nm_decay=1e-3, nm_thres=0.0,
+        noise_management=NoiseManagementType.AbsMax, out_bound=12.0, out_noise=0.06,
+        out_noise_std=0.0, out_res=1.0 / (2.0**9 - 2.0), out_scale=1.0, out_sto_round=False,
+        w_noise=0.0, w_noise_type=WeightNoiseType.NONE, ir_drop=0.0, ir_drop_g_ratio=5.7143e5,
+        out_nonlinearity=0.0, out_nonlinearity_std=0.0, mv_type=AnalogMVType.OnePass,
+        inp_asymmetry=0.0, out_asymmetry=0.0, slope_calibration=0.5, r_series=0.0, v_offset_std=0.0,
+        v_offset_w_min=0.0, w_read_asymmetry_dtod=0.0,
+    )
+
+    def _to_c(self) -> IOParams:
+        p = IOParams()
+        p.is_perfect = int(bool(self.is_perfect))
+        p.mv_type = int(self.mv_type)
+        p.noise_management = int(self.noise_management)
+        p.bound_management = int(self.bound_management)
+        p.bm_test_negative_bound = int(bool(self.bm_test_negative_bound))
+        p.max_bm_factor = int(self.max_bm_factor)
+        p.inp_sto_round = int(bool(self.inp_sto_round))
+        p.out_sto_round = int(bool(self.out_sto_round))
+        for name in ("inp_bound", "inp_res", "inp_noise", "inp_asymmetry", "out_bound", "out_res",
+                     "out_noise", "out_asymmetry", "out_scale", "nm_thres", "nm_assumed_wmax",
+                     "max_bm_res", "w_noise", "ir_drop", "out_noise_std", "out_nonlinearity",
+                     "out_nonlinearity_std", "v_offset_std", "r_series", "w_read_asymmetry_dtod"):
+            setattr(p, name, float(getattr(self, name)))
+        p.w_noise_type = int(self.w_noise_type)
+        return p
+
+
+class AnalogTileUpdateParameter(_Struct):
+    """rpu_base_devices.cpp:469-483 over PulsedUpdateMetaParameter (rpu_pulsed_meta_parameter.h:248-323)."""
+
+    _defaults = dict(
+        fixed_bl=True, desired_bl=31, d_res_implicit=0.0, pulse_type=PulseType.StochasticCompressed,
+        res=0.0, sto_round=False, um_reg_scale=1.0, um_grad_scale=1.0, d_sparsity=False,
+        update_management=True, update_bl_management=True, x_res_implicit=0.0,
+    )
+
+    def _to_c(self) -> UpdateParams:
+        p = UpdateParams()
+        p.pulse_type = int(self.pulse_type)
+        p.desired_bl = int(self.desired_bl)
+        p.fixed_bl = int(bool(self.fixed_bl))
+        p.update_management = int(bool(self.update_management))
+        p.update_bl_management = int(bool(self.update_bl_management))
+        p.sto_round = int(bool(self.sto_round))
+        p.um_grad_scale = float(self.um_grad_scale)
+        p.res = float(self.res)
+        p.x_res_implicit = float(self.x_res_implicit)
+        p.d_res_implicit = float(self.d_res_implicit)
+        return p
+
+
+class AbstractResistiveDeviceParameter(_Struct):
+    """rpu_base_devices.cpp:536-539 (+ the SimpleMetaParameter fields diffusion / lifetime)."""
+
+    _defaults = dict(construction_seed=0, diffusion=0.0, lifetime=0.0)
+    _kind = None
+
+    def _fill_c(self, p: DeviceParams) -> None:
+        p.construction_seed = int(self.construction_seed)
+        p.diffusion = float(self.diffusion)
+        p.lifetime = float(self.lifetime)
+
+    def _to_c(self) -> DeviceParams:
+        from .._cabi import check, lib
+
+        cfg = TileConfig()
+        check(lib().rpu_tile_config_default(cfg, int(self._kind)))
+        p = cfg.device
+        self._fill_c(p)
+        return p
+
+
+class IdealResistiveDeviceParameter(AbstractResistiveDeviceParameter):
+    """rpu_base_devices.cpp:545-552: no device physics; the update is a plain rank-B outer product."""
+
+    _defaults = dict(reset_std=0.01)
+    _kind = 0
+
+    def _fill_c(self, p):
+        super()._fill_c(p)
+        p.reset_std = float(self.reset_std)
+
+
+class PulsedResistiveDeviceParameter(AbstractResistiveDeviceParameter):
+    """rpu_base_devices.cpp:554-581 over PulsedRPUDeviceMetaParameter (rpu_pulsed_device.h:52-114)."""
+
+    _defaults = dict(
+        corrupt_devices_prob=0.0, corrupt_devices_range=FLT_MAX, diffusion_dtod=0.0, dw_min=0.001,
+        dw_min_dtod=0.3, dw_min_dtod_log_normal=False, dw_min_std=0.3, enforce_consistency=False,
+        lifetime_dtod=0.0, perfect_bias=False, reset=0.0, reset_std=0.01, reset_dtod=0.0, up_down=0.0,
+        up_down_dtod=0.01, w_max=0.6, w_max_dtod=0.3, w_min=-0.6, w_min_dtod=0.3, count_pulses=False,
+    )
+
+    def _fill_c(self, p):
+        super()._fill_c(p)
+        for name in ("corrupt_devices_prob", "corrupt_devices_range", "diffusion_dtod", "dw_min",
+                     "dw_min_dtod", "dw_min_std", "lifetime_dtod", "reset", "reset_std", "reset_dtod",
+                     "up_down", "up_down_dtod", "w_max", "w_max_dtod", "w_min", "w_min_dtod"):
+            setattr(p, name, float(getattr(self, name)))
+        p.dw_min_dtod_log_normal = int(bool(self.dw_min_dtod_log_normal))
+        p.enforce_consistency = int(bool(self.enforce_consistency))
+        p.perfect_bias = int(bool(self.perfect_bias))
+        if self.count_pulses:
+            raise RuntimeError("count_pulses is not implemented on this path.")
+
+    def calc_weight_granularity(self) -> float:
+        """rpu_constantstep_device.h:27, rpu_linearstep_device.h:58: the granularity is dw_min."""
+        return float(self.dw_min)
+
+
+class ConstantStepResistiveDeviceParameter(PulsedResistiveDeviceParameter):
+    """rpu_base_devices.cpp:583-600."""
+
+    _kind = 1
+
+
+class LinearStepResistiveDeviceParameter(PulsedResistiveDeviceParameter):
+    """rpu_base_devices.cpp:602-631 over the LinearStep tail (rpu_linearstep_device.h:16-31)."""
+
+    _defaults = dict(
+        gamma_up=0.0, gamma_down=0.0, gamma_up_dtod=0.05, gamma_down_dtod=0.05, allow_increasing=False,
+        mean_bound_reference=True, write_noise_std=0.0, apply_write_noise_on_set=True, mult_noise=True,
+        reverse_up=False, reverse_down=False, reverse_offset=0.01,
+    )
+    _kind = 2
+
+    def _fill_c(self, p):
+        super()._fill_c(p)
+        p.ls_decrease_up = float(self.gamma_up)
+        p.ls_decrease_down = float(self.gamma_down)
+        p.ls_decrease_up_dtod = float(self.gamma_up_dtod)
+        p.ls_decrease_down_dtod = float(self.gamma_down_dtod)
+        p.ls_allow_increasing_slope = int(bool(self.allow_increasing))
+        p.ls_mean_bound_reference = int(bool(self.mean_bound_reference))
+        p.write_noise_std = float(self.write_noise_std)
+        p.ls_mult_noise = int(bool(self.mult_noise))
+        p.ls_reverse_up = int(bool(self.reverse_up))
+        p.ls_reverse_down = int(bool(self.reverse_down))
+        p.ls_reverse_offset = float(self.reverse_offset)
+
+
+class SoftBoundsResistiveDeviceParameter(LinearStepResistiveDeviceParameter):
+    """rpu_base_devices.cpp:633-656 over SoftBoundsRPUDeviceMetaParameter (rpu_linearstep_device.h:66-80)."""
+
+    _defaults = dict(gamma_up=1.0, gamma_down=1.0, gamma_up_dtod=0.0, gamma_down_dtod=0.0,
+                     mean_bound_reference=False)
+    _kind = 3
+
+    def _fill_c(self, p):
+        if not (self.gamma_up == 1.0 and self.gamma_down == 1.0 and self.gamma_up_dtod == 0.0
+                and self.gamma_down_dtod == 0.0 and not self.allow_increasing
+                and not self.mean_bound_reference):
+            raise RuntimeError("SoftBounds set to wrong values!")  # rpu_linearstep_device.h:81-87
+        super()._fill_c(p)
+
+
+class AnalogTileParameter(_Struct):
+    """rpu_base_devices.cpp:453-467 over PulsedMetaParameter (rpu_pulsed.h:127-151)."""
+
+    _defaults = dict(forward_io=None, backward_io=None, update=None)
+
+    def __init__(self):
+        super().__init__()
+        self.forward_io = AnalogTileInputOutputParameter()
+        self.backward_io = AnalogTileInputOutputParameter()
+        self.update = AnalogTileUpdateParameter()
+
+    def _config(self, device_param) -> TileConfig:
+        cfg = TileConfig()
+        cfg.f_io = self.forward_io._to_c()
+        cfg.b_io = self.backward_io._to_c()
+        cfg.up = self.update._to_c()
+        cfg.device = device_param._to_c()
+        return cfg
+
+    def create_array(self, x_size: int, d_size: int, device_param):
+        """Build the host-side analog tile (device parameters are sampled here, on the CPU)."""
+        from .tiles import AnalogTile
+
+        if not isinstance(device_param, AbstractResistiveDeviceParameter) or device_param._kind is None:
+            raise TypeError("device_param must be one of the *ResistiveDeviceParameter classes")
+        return AnalogTile._create(int(x_size), int(d_size), self._config(device_param))
+
+
+class FloatingPointTileParameter(_Struct):
+    """rpu_base_devices.cpp:436-451: floating-point tile = ideal device with perfect IO and no pulses."""
+
+    _defaults = dict(diffusion=0.0, lifetime=0.0, drift=None)
+
+    def create_array(self, x_size: int, d_size: int):
+        from .tiles import FloatingPointTile
+
+        meta = AnalogTileParameter()
+        meta.forward_io.is_perfect = True
+        meta.backward_io.is_perfect = True
+        meta.update.pulse_type = PulseType.NONE
+        return FloatingPointTile._create(int(x_size), int(d_size), meta._config(IdealResistiveDeviceParameter()))
+
+
+__all__ = [name for name, obj in vars(sys.modules[__name__]).items()
+           if isinstance(obj, type) and not name.startswith("_")]

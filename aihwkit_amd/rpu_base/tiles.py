@@ -1,0 +1,267 @@
+"""Mirror of ``rpu_base.tiles``: tile classes with the call signatures of the reference bindings.
+
+Reference: src/aihwkit/simulator/rpu_base_src/rpu_base_tiles.cpp (CPU tiles ``FloatingPointTile`` /
+``AnalogTile``) and rpu_base_tiles_cuda.cpp (``CudaFloatingPointTile`` / ``CudaAnalogTile``).
+
+The host tiles hold parameters, the sampled per-device arrays and the weights; they can be inspected
+and copied to a GPU (``CudaAnalogTile(cpu_tile)``, as ``.cuda()`` does in the reference,
+src/aihwkit/simulator/tiles/rpucuda.py:145-209) but they do not compute: ``forward`` / ``backward`` /
+``update`` exist only on the GPU tiles and run hand-written HIP kernels through the C ABI.  Positional
+argument order is the reference's; it is what its Python callers rely on
+(src/aihwkit/simulator/tiles/periphery.py:1061,1165,1225).
+"""
+import ctypes as C
+from typing import List
+
+import torch
+
+from .._cabi import check, lib
+
+_DTYPE = torch.float32
+
+
+def _check_input(tensor: torch.Tensor, cuda: bool, name: str) -> torch.Tensor:
+    # CHECK_TORCH_INPUT / CHECK_TORCH_CUDA_INPUT (rpu_base_tiles.cpp:15-22)
+    if not isinstance(tensor, torch.Tensor):
+        raise TypeError(f"{name} must be a torch.Tensor")
+    tensor = tensor.contiguous()
+    if tensor.dtype != _DTYPE:
+        raise RuntimeError(f"{name} must be a float32 tensor")
+    if cuda and not tensor.is_cuda:
+        raise RuntimeError(f"{name} must be a CUDA tensor")
+    if not cuda and tensor.is_cuda:
+        raise RuntimeError(f"{name} must be a CPU tensor")
+    return tensor
+
+
+class _TileBase:
+    """State surface shared by host and GPU tiles."""
+
+    def __init__(self, handle):
+        self._h = C.c_void_p(handle)
+
+    def __del__(self):
+        handle, self._h = getattr(self, "_h", None), None
+        if handle:
+            try:
+                lib().rpu_tile_destroy(handle)
+            except Exception:  # pylint: disable=broad-except
+                pass
+
+    @classmethod
+    def _create(cls, x_size, d_size, config):
+        handle = C.c_void_p()
+        check(lib().rpu_tile_create(C.byref(handle), x_size, d_size, C.byref(config)))
+        return cls(handle.value)
+
+    def _clone_handle(self):
+        handle = C.c_void_p()
+        check(lib().rpu_tile_clone(C.byref(handle), self._h))
+        return handle.value
+
+    def __copy__(self):
+        return type(self)(self._clone_handle())
+
+    def __deepcopy__(self, memo):
+        return type(self)(self._clone_handle())
+
+    # -- sizes / learning rate (rpu_base_tiles.cpp get_x_size, get_d_size, get/set_learning_rate)
+    def get_x_size(self) -> int:
+        return lib().rpu_tile_get_x_size(self._h)
+
+    def get_d_size(self) -> int:
+        return lib().rpu_tile_get_d_size(self._h)
+
+    def get_learning_rate(self) -> float:
+        return float(lib().rpu_tile_get_learning_rate(self._h))
+
+    def set_learning_rate(self, learning_rate: float) -> None:
+        check(lib().rpu_tile_set_learning_rate(self._h, float(learning_rate)))
+
+    # -- weights: [d_size, x_size] CPU tensors (rpu_base_tiles.cpp:161-214)
+    def get_weights(self) -> torch.Tensor:
+        out = torch.empty(self.get_d_size(), self.get_x_size(), dtype=_DTYPE)
+        check(lib().rpu_tile_get_weights(self._h, out.data_ptr()))
+        return out
+
+    def set_weights(self, weights: torch.Tensor) -> None:
+        weights = _check_input(weights.detach().cpu() if weights.is_cuda else weights.detach(), False, "weights")
+        if weights.dim() != 2 or weights.size(0) != self.get_d_size() or weights.size(1) != self.get_x_size():
+            raise RuntimeError(
+                f"Invalid weights dimensions: expected [{self.get_d_size()},{self.get_x_size()}] array")
+        check(lib().rpu_tile_set_weights(self._h, weights.data_ptr()))
+
+    # -- hidden per-device parameters (rpu_base_tiles.cpp:763-825)
+    def get_hidden_parameter_names(self) -> List[str]:
+        count = lib().rpu_tile_hidden_parameter_count(self._h)
+        return [lib().rpu_tile_hidden_parameter_name(self._h, k).decode() for k in range(count)]
+
+    def get_hidden_parameters(self) -> torch.Tensor:
+        count = lib().rpu_tile_hidden_parameter_count(self._h)
+        out = torch.empty(count, self.get_d_size(), self.get_x_size(), dtype=_DTYPE)
+        if count:
+            check(lib().rpu_tile_get_hidden_parameters(self._h, out.data_ptr()))
+        return out
+
+    def set_hidden_parameters(self, params: torch.Tensor) -> None:
+        count = lib().rpu_tile_hidden_parameter_count(self._h)
+        params = _check_input(params.detach(), False, "hidden parameters")
+        if params.dim() != 3 or tuple(params.shape) != (count, self.get_d_size(), self.get_x_size()):
+            raise RuntimeError(
+                f"Invalid parameters dimensions: expected [{count},{self.get_d_size()},{self.get_x_size()}] array")
+        if count:
+            check(lib().rpu_tile_set_hidden_parameters(self._h, params.data_ptr()))
+
+    def set_seed(self, seed: int) -> None:
+        """Seed of the Philox generator behind every random draw of this tile on the GPU."""
+        check(lib().rpu_tile_set_seed(self._h, int(seed) & 0xFFFFFFFFFFFFFFFF))
+
+    def get_brief_info(self) -> str:
+        where = "gfx950" if lib().rpu_tile_is_on_device(self._h) else "host"
+        return f"{type(self).__name__}({self.get_d_size()},{self.get_x_size()}) [{where}]"
+
+    # -- the hot path is not provided on host tiles
+    def forward(self, *args, **kwargs):
+        raise RuntimeError("Host tiles do not compute: build a CudaAnalogTile(tile) / CudaFloatingPointTile(tile).")
+
+    backward = forward
+    update = forward
+
+
+class FloatingPointTile(_TileBase):
+    """Host-side floating point tile (rpu_base_tiles.cpp ``FloatingPointTile``)."""
+
+
+class AnalogTile(_TileBase):
+    """Host-side analog tile (rpu_base_tiles.cpp ``AnalogTile``)."""
+
+
+class _CudaTileMixin:
+    def _init_cuda(self, tile: _TileBase):
+        if not isinstance(tile, _TileBase):
+            raise TypeError("expected a host tile")
+        if not torch.cuda.is_available():
+            raise RuntimeError("No GPU available: the analog tile kernels need a HIP device.")
+        handle = tile._clone_handle()
+        _TileBase.__init__(self, handle)
+        check(lib().rpu_tile_to_device(self._h, torch.cuda.current_device()))
+        self._device = torch.device("cuda", torch.cuda.current_device())
+
+    @staticmethod
+    def _stream_for(tensor: torch.Tensor):
+        return C.c_void_p(torch.cuda.current_stream(tensor.device).cuda_stream)
+
+    def _finish(self, tensor: torch.Tensor, non_blocking: bool):
+        if not non_blocking:
+            torch.cuda.current_stream(tensor.device).synchronize()
+
+    # rpu_base_tiles_cuda.cpp:159-236
+    def forward(self, x_input: torch.Tensor, bias: bool = False, x_trans: bool = False, d_trans: bool = False,
+                is_test: bool = False, non_blocking: bool = False) -> torch.Tensor:
+        x_input = _check_input(x_input, True, "x_input")
+        if x_input.dim() < 1:
+            raise RuntimeError("Invalid x_input dimensions: expected at least 1 dimensional tensor")
+        in_size = x_input.size(0) if x_trans else x_input.size(-1)
+        expected = self.get_x_size() - (1 if bias else 0)
+        if in_size != expected:
+            shape = f"[*, {expected}]" if x_trans else f"[{expected},*]"
+            raise RuntimeError(f"Invalid x_input dimensions: expected {shape} tensor")
+        m_batch = x_input.numel() // in_size
+        dims = list(x_input.shape)
+        dims[0 if d_trans else -1] = self.get_d_size()
+        d_output = torch.empty(dims, dtype=x_input.dtype, device=x_input.device)
+        check(lib().rpu_tile_forward(self._h, x_input.data_ptr(), d_output.data_ptr(), m_batch, int(bias),
+                                     int(x_trans), int(d_trans), int(is_test), self._stream_for(x_input)))
+        self._finish(x_input, non_blocking)
+        return d_output
+
+    # rpu_base_tiles_cuda.cpp:237-309
+    def backward(self, d_input: torch.Tensor, bias: bool = False, d_trans: bool = False, x_trans: bool = False,
+                 non_blocking: bool = False) -> torch.Tensor:
+        d_input = _check_input(d_input, True, "d_input")
+        if d_input.dim() < 1:
+            raise RuntimeError("Invalid d_input dimensions: expected at least 1 dimensional tensor")
+        in_size = d_input.size(0) if d_trans else d_input.size(-1)
+        expected = self.get_d_size()
+        if in_size != expected:
+            shape = f"[*, {expected}]" if d_trans else f"[{expected},*]"
+            raise RuntimeError(f"Invalid d_input dimensions: expected {shape} tensor")
+        m_batch = d_input.numel() // in_size
+        dims = list(d_input.shape)
+        dims[0 if x_trans else -1] = self.get_x_size() - (1 if bias else 0)
+        x_output = torch.empty(dims, dtype=d_input.dtype, device=d_input.device)
+        check(lib().rpu_tile_backward(self._h, d_input.data_ptr(), x_output.data_ptr(), m_batch, int(bias),
+                                      int(d_trans), int(x_trans), self._stream_for(d_input)))
+        self._finish(d_input, non_blocking)
+        return x_output
+
+    # rpu_base_tiles_cuda.cpp:310-397.  The keyword names of the 4th / 5th argument are swapped in the
+    # reference (py::arg("d_trans") precedes py::arg("x_trans")); positions are what callers use.
+    def update(self, x_input: torch.Tensor, d_input: torch.Tensor, bias: bool, x_trans: bool = False,
+               d_trans: bool = False, non_blocking: bool = False) -> None:
+        if self.get_learning_rate() == 0.0:
+            return
+        d_input = _check_input(d_input, True, "d_input")
+        x_input = _check_input(x_input, True, "x_input")
+        if x_input.dim() < 1 or d_input.dim() < 1:
+            raise RuntimeError("Invalid x_input/d_input dimensions: expected at least 1 dimensional tensor")
+        in_size = x_input.size(0) if x_trans else x_input.size(-1)
+        expected_in = self.get_x_size() - (1 if bias else 0)
+        m_batch = x_input.numel() // in_size
+        out_size = d_input.size(0) if d_trans else d_input.size(-1)
+        expected_out = self.get_d_size()
+        m_batch_from_d = d_input.numel() // out_size
+        if in_size != expected_in:
+            shape = f"[*, {expected_in}]" if x_trans else f"[{expected_in}, *]"
+            raise RuntimeError(f"Invalid x_input dimensions: expected {shape} tensor")
+        if out_size != expected_out:
+            shape = f"[*, {expected_out}]" if d_trans else f"[{expected_out}, *]"
+            raise RuntimeError(f"Invalid d_input dimensions: expected {shape} tensor")
+        if m_batch != m_batch_from_d:
+            raise RuntimeError("Invalid x_input or d_input dimensions: batch dimensions mismatch!")
+        check(lib().rpu_tile_update(self._h, x_input.data_ptr(), d_input.data_ptr(), m_batch, int(bias),
+                                    int(x_trans), int(d_trans), self._stream_for(x_input)))
+        self._finish(x_input, non_blocking)
+
+    # -- inspection hooks
+    def get_update_words(self, m_batch: int):
+        """Packed pulse words and per-sample BL of the last stochastic update (CPU tensors)."""
+        x_words = torch.empty(m_batch, self.get_x_size(), dtype=torch.int32)
+        d_words = torch.empty(m_batch, self.get_d_size(), dtype=torch.int32)
+        bl = torch.empty(m_batch, dtype=torch.int32)
+        check(lib().rpu_tile_get_update_words(self._h, x_words.data_ptr(), d_words.data_ptr(), bl.data_ptr(), m_batch))
+        return x_words, d_words, bl
+
+    def get_implicit_counts(self, m_batch: int) -> torch.Tensor:
+        """Signed coincidence counts [m_batch, d_size, x_size] of the last deterministic-implicit update."""
+        counts = torch.empty(m_batch, self.get_d_size(), self.get_x_size(), dtype=torch.int32)
+        check(lib().rpu_tile_get_implicit_counts(self._h, counts.data_ptr(), m_batch))
+        return counts
+
+    def get_bm_rounds(self, m_batch: int) -> torch.Tensor:
+        """Number of bound-management rounds each sample of the last forward pass took."""
+        rounds = torch.empty(m_batch, dtype=torch.int32)
+        check(lib().rpu_tile_get_bm_rounds(self._h, rounds.data_ptr(), m_batch))
+        return rounds
+
+
+class CudaFloatingPointTile(_CudaTileMixin, _TileBase):
+    """GPU floating point tile (rpu_base_tiles_cuda.cpp:45-58)."""
+
+    def __init__(self, tile):  # pylint: disable=super-init-not-called
+        if isinstance(tile, int):
+            _TileBase.__init__(self, tile)
+            self._device = torch.device("cuda", torch.cuda.current_device())
+        else:
+            self._init_cuda(tile)
+
+
+class CudaAnalogTile(_CudaTileMixin, _TileBase):
+    """GPU analog tile (rpu_base_tiles_cuda.cpp:524-543): built from a host tile."""
+
+    def __init__(self, tile):  # pylint: disable=super-init-not-called
+        if isinstance(tile, int):
+            _TileBase.__init__(self, tile)
+            self._device = torch.device("cuda", torch.cuda.current_device())
+        else:
+            self._init_cuda(tile)

@@ -1,0 +1,301 @@
+/*
+ * rpu_amd.h -- C ABI of the MI355X (gfx950) analog-tile library (librpu_amd.so).
+ *
+ * The entry points below are what the `rpu_base` binding layer of IBM/aihwkit
+ * would bind for the analog-tile hot path (noisy forward / backward MVM and the
+ * pulsed update).  Every declaration cites the reference interface it replaces
+ * (paths relative to the reference checkout; R/ = src/rpucuda/,
+ * C/ = src/rpucuda/cuda/, B/ = src/aihwkit/simulator/rpu_base_src/).
+ *
+ * Conventions
+ *  - plain C: opaque handles, plain-old-data parameter structs, raw pointers.
+ *  - every function returns 0 on success and a non-zero code on failure;
+ *    rpu_last_error() returns the message of the last failure on the calling
+ *    thread (the reference throws std::runtime_error, R/utility_functions.h:63-69;
+ *    a binding layer turns the message into its RuntimeError).
+ *  - `*_dev` pointers are device (HBM) pointers of the GPU the tile lives on,
+ *    `*_host` pointers are host pointers.  `stream` is a hipStream_t passed as
+ *    void* (NULL = the default stream).
+ *  - weights are exchanged row-major [d_size][x_size] exactly like the reference
+ *    (R/rpu.h:674, B/rpu_base_tiles.cpp:161-214).
+ *  - compute entry points (forward / backward / update) exist for GPU-resident
+ *    tiles only.  There is no CPU compute path in this library.
+ */
+#ifndef RPU_AMD_H
+#define RPU_AMD_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define RPU_AMD_ABI_VERSION 1
+
+/* ---- enums: integer values equal the reference enum class order ------------ */
+
+/* R/rpu_pulsed_meta_parameter.h:17-27 NoiseManagementType */
+enum rpu_noise_management {
+  RPU_NM_NONE = 0,
+  RPU_NM_ABS_MAX = 1,
+  RPU_NM_ABS_MAX_NP_SUM = 2,
+  RPU_NM_MAX = 3,
+  RPU_NM_CONSTANT = 4,
+  RPU_NM_AVERAGE_ABS_MAX = 5,              /* not provided: creation fails */
+  RPU_NM_AVERAGE_ABS_MAX_SINGLE_VALUE = 6, /* not provided */
+  RPU_NM_ABS_MAX_SINGLE_VALUE = 7          /* not provided */
+};
+
+/* R/rpu_pulsed_meta_parameter.h:29 BoundManagementType */
+enum rpu_bound_management {
+  RPU_BM_NONE = 0,
+  RPU_BM_ITERATIVE = 1,
+  RPU_BM_ITERATIVE_WORST_CASE = 2
+};
+
+/* R/rpu_pulsed_meta_parameter.h:33-40 PulseType */
+enum rpu_pulse_type {
+  RPU_PULSE_NONE = 0,                  /* floating point rank-B update */
+  RPU_PULSE_STOCHASTIC_COMPRESSED = 1,
+  RPU_PULSE_STOCHASTIC = 2,            /* not provided (CPU-only in the reference too) */
+  RPU_PULSE_NONE_WITH_DEVICE = 3,
+  RPU_PULSE_MEAN_COUNT = 4,            /* not provided (CPU-only in the reference too) */
+  RPU_PULSE_DETERMINISTIC_IMPLICIT = 5
+};
+
+/* R/rpu_pulsed_meta_parameter.h:42-49 AnalogMVType */
+enum rpu_mv_type {
+  RPU_MV_IDEAL = 0,
+  RPU_MV_ONE_PASS = 1
+  /* PosNegSeparate(2), PosNegSeparateDigitalSum(3), SplitMode(4), BitWise(5): not provided */
+};
+
+/* device kinds; B/rpu_base_devices.cpp:545-656 */
+enum rpu_device_kind {
+  RPU_DEVICE_IDEAL = 0,         /* IdealResistiveDeviceParameter / FloatingPoint: no device physics */
+  RPU_DEVICE_CONSTANT_STEP = 1, /* ConstantStepResistiveDeviceParameter */
+  RPU_DEVICE_LINEAR_STEP = 2,   /* LinearStepResistiveDeviceParameter */
+  RPU_DEVICE_SOFT_BOUNDS = 3    /* SoftBoundsResistiveDeviceParameter (LinearStep with fixed ls_* values) */
+};
+
+/* ---- parameter structs ------------------------------------------------------ */
+
+/* Replaces IOMetaParameter<float> (R/rpu_pulsed_meta_parameter.h:50-106) as bound by
+ * AnalogTileInputOutputParameter (B/rpu_base_devices.cpp:485-519).  Field names and defaults are
+ * the C++ ones; `inp_res` / `out_res` accept "1/steps" or "steps" and are converted to an absolute
+ * step res * 2 * bound at creation (R/rpu_pulsed_meta_parameter.cpp:26-37,56-57).
+ * Fields in the "not provided" block must be left at their inactive value or creation fails. */
+typedef struct rpu_io_params {
+  int32_t is_perfect;             /* 0 */
+  int32_t mv_type;                /* RPU_MV_ONE_PASS */
+  int32_t noise_management;       /* RPU_NM_ABS_MAX */
+  int32_t bound_management;       /* RPU_BM_NONE (python default ITERATIVE) */
+  int32_t bm_test_negative_bound; /* 1 */
+  int32_t max_bm_factor;          /* 1000 */
+  int32_t inp_sto_round;          /* 0 */
+  int32_t out_sto_round;          /* 0 */
+  float inp_bound;                /* 1 */
+  float inp_res;                  /* 1/126 */
+  float inp_noise;                /* 0 */
+  float inp_asymmetry;            /* 0 */
+  float out_bound;                /* 12 */
+  float out_res;                  /* 1/510 */
+  float out_noise;                /* 0.06 */
+  float out_asymmetry;            /* 0 */
+  float out_scale;                /* 1 */
+  float nm_thres;                 /* 0 */
+  float nm_assumed_wmax;          /* 0.6 */
+  float max_bm_res;               /* 0.25 */
+  /* not provided (must stay inactive): */
+  int32_t w_noise_type;           /* 0 = None */
+  float w_noise;                  /* ignored while w_noise_type == 0 */
+  float ir_drop;                  /* 0 */
+  float out_noise_std;            /* 0 */
+  float out_nonlinearity;         /* 0 */
+  float out_nonlinearity_std;     /* 0 */
+  float v_offset_std;             /* 0 */
+  float r_series;                 /* 0 */
+  float w_read_asymmetry_dtod;    /* 0 */
+} rpu_io_params;
+
+/* Replaces PulsedUpdateMetaParameter<float> (R/rpu_pulsed_meta_parameter.h:248-323) as bound by
+ * AnalogTileUpdateParameter (B/rpu_base_devices.cpp:469-483). */
+typedef struct rpu_update_params {
+  int32_t pulse_type;           /* RPU_PULSE_STOCHASTIC_COMPRESSED */
+  int32_t desired_bl;           /* 31; at most 31 (one 32-bit pulse word per line and sample) */
+  int32_t fixed_bl;             /* 1 */
+  int32_t update_management;    /* 1 */
+  int32_t update_bl_management; /* 1 */
+  int32_t sto_round;            /* 0 */
+  float um_grad_scale;          /* 1 */
+  float res;                    /* 0 : resolution of the pulse probability (0..1) */
+  float x_res_implicit;         /* 0 */
+  float d_res_implicit;         /* 0 */
+} rpu_update_params;
+
+/* Replaces PulsedRPUDeviceMetaParameter<float> (R/rpu_pulsed_device.h:52-114) plus the LinearStep
+ * tail (R/rpu_linearstep_device.h:16-31) and the SimpleRPUDeviceMetaParameter fields that feed
+ * device construction (R/rpu_simple_device.h:54,89).  For RPU_DEVICE_SOFT_BOUNDS the ls_* fields
+ * are overwritten with the SoftBounds constants (R/rpu_linearstep_device.h:68-80). */
+typedef struct rpu_device_params {
+  int32_t kind;                    /* enum rpu_device_kind */
+  uint32_t construction_seed;      /* 0 = time based (as the reference) */
+  int32_t enforce_consistency;     /* 0 in C++, 1 in the python configs */
+  int32_t perfect_bias;            /* 0 */
+  int32_t dw_min_dtod_log_normal;  /* 0 */
+  int32_t adjust_bounds_with_up_down; /* 0 */
+  float dw_min;                    /* 0.001 */
+  float dw_min_dtod;               /* 0.3 */
+  float dw_min_std;                /* 0.3 (cycle-to-cycle) */
+  float w_min;                     /* -0.6 */
+  float w_min_dtod;                /* 0.3 */
+  float w_max;                     /* 0.6 */
+  float w_max_dtod;                /* 0.3 */
+  float up_down;                   /* 0 */
+  float up_down_dtod;              /* 0.01 */
+  float adjust_bounds_with_up_down_dev; /* 0 */
+  float corrupt_devices_prob;      /* 0 */
+  float corrupt_devices_range;     /* FLT_MAX */
+  float lifetime;                  /* 0 */
+  float lifetime_dtod;             /* 0 */
+  float diffusion;                 /* 0 */
+  float diffusion_dtod;            /* 0 */
+  float reset;                     /* 0 */
+  float reset_dtod;                /* 0 */
+  float reset_std;                 /* 0.01 */
+  float write_noise_std;           /* 0 ; > 0 is not provided */
+  /* LinearStep tail */
+  int32_t ls_allow_increasing_slope; /* 0 */
+  int32_t ls_mean_bound_reference;   /* 1 */
+  int32_t ls_mult_noise;             /* 1 */
+  int32_t ls_reverse_up;             /* 0 */
+  int32_t ls_reverse_down;           /* 0 */
+  float ls_decrease_up;              /* 0 */
+  float ls_decrease_down;            /* 0 */
+  float ls_decrease_up_dtod;         /* 0.05 */
+  float ls_decrease_down_dtod;       /* 0.05 */
+  float ls_reverse_offset;           /* 0.01 */
+} rpu_device_params;
+
+/* Replaces PulsedMetaParameter<float> (R/rpu_pulsed.h:127-151): forward IO, backward IO, update. */
+typedef struct rpu_tile_config {
+  rpu_io_params f_io;
+  rpu_io_params b_io;
+  rpu_update_params up;
+  rpu_device_params device;
+} rpu_tile_config;
+
+typedef struct rpu_tile rpu_tile_t; /* opaque */
+
+/* ---- defaults ---------------------------------------------------------------- */
+
+/* Fill `cfg` with the C++ defaults of the reference structs cited above for the given device kind. */
+int rpu_tile_config_default(rpu_tile_config *cfg, int device_kind);
+
+/* ---- construction / residency --------------------------------------------------- */
+
+/* Replaces PulsedMetaParameter::createRPUArray (R/rpu_pulsed.cpp:48-56) reached through
+ * AnalogTileParameter.create_array (B/rpu_base_devices.cpp:453-467): builds the host-side tile,
+ * samples the device-to-device parameters on the CPU with RealWorldRNG(construction_seed)
+ * (R/rpu_pulsed.cpp:460-495, R/rpu_pulsed_device.cpp:593-733).  Touches no GPU. */
+int rpu_tile_create(rpu_tile_t **out, int x_size, int d_size, const rpu_tile_config *cfg);
+
+/* Deep copy (host state and, if resident, device state); B/rpu_base_tiles.cpp __copy__/__deepcopy__. */
+int rpu_tile_clone(rpu_tile_t **out, const rpu_tile_t *src);
+
+/* Replaces the CudaAnalogTile(cpu_tile) constructor (B/rpu_base_tiles_cuda.cpp:45-58,524-543;
+ * C/rpucuda_pulsed.cu:69-88): allocates HBM on HIP device `device_id` (-1 = current) and uploads
+ * weights and per-device parameters. */
+int rpu_tile_to_device(rpu_tile_t *tile, int device_id);
+
+int rpu_tile_destroy(rpu_tile_t *tile);
+
+/* ---- hot path -------------------------------------------------------------------- */
+
+/* Replaces RPUSimple::forward (R/rpu.cpp:508-533; GPU: C/rpucuda_pulsed.cu:646-659) as bound at
+ * B/rpu_base_tiles_cuda.cpp:159-236.  x_dev is [m_batch][x_size - bias] (x_trans: [x_size - bias][m_batch]),
+ * y_dev is [m_batch][d_size] (d_trans: [d_size][m_batch]).  Asynchronous on `stream`. */
+int rpu_tile_forward(rpu_tile_t *tile, const float *x_dev, float *y_dev, int m_batch, int bias,
+                     int x_trans, int d_trans, int is_test, void *stream);
+
+/* Replaces RPUSimple::backward (R/rpu.cpp:535-554) as bound at B/rpu_base_tiles.cpp:475-539. */
+int rpu_tile_backward(rpu_tile_t *tile, const float *d_dev, float *x_dev, int m_batch, int bias,
+                      int d_trans, int x_trans, void *stream);
+
+/* Replaces RPUSimple::update -> RPUPulsed::updateMatrix (R/rpu.cpp:556-575, R/rpu_pulsed.cpp:558-585;
+ * GPU: C/rpucuda_pulsed.cu:897-930, C/pulsed_weight_updater.cu:332-434) as bound at
+ * B/rpu_base_tiles.cpp:541-620.  A zero learning rate makes this a no-op, as in the binding. */
+int rpu_tile_update(rpu_tile_t *tile, const float *x_dev, const float *d_dev, int m_batch, int bias,
+                    int x_trans, int d_trans, void *stream);
+
+/* ---- state ------------------------------------------------------------------------ */
+
+int rpu_tile_get_x_size(const rpu_tile_t *tile); /* R/rpu.h:76 getXSize */
+int rpu_tile_get_d_size(const rpu_tile_t *tile); /* R/rpu.h:77 getDSize */
+int rpu_tile_is_on_device(const rpu_tile_t *tile);
+
+/* RPUAbstract::setLearningRate / getLearningRate (R/rpu.h:85-86, B/rpu_base_tiles.cpp get/set_learning_rate) */
+int rpu_tile_set_learning_rate(rpu_tile_t *tile, float lr);
+float rpu_tile_get_learning_rate(const rpu_tile_t *tile);
+
+/* RPUPulsed::setWeights (clips into the per-device bounds, R/rpu_pulsed.cpp:288-292,
+ * R/rpu_pulsed_device.cpp:545-571) and RPUSimple::getWeights; row-major [d_size][x_size] host buffers.
+ * On a GPU tile these synchronise with the stream of the last compute call. */
+int rpu_tile_set_weights(rpu_tile_t *tile, const float *w_host);
+int rpu_tile_get_weights(rpu_tile_t *tile, float *w_host);
+
+/* Device pointer of the row-major [d_size][x_size] weight matrix in HBM (NULL if not resident).
+ * Stands in for the shared-weights aliasing of RPUCudaSimple::setSharedWeights (C/rpucuda.cu:322-334). */
+int rpu_tile_weights_device_ptr(rpu_tile_t *tile, float **w_dev);
+
+/* Hidden per-device parameters: RPUPulsed::getDeviceParameterNames / getDeviceParameter /
+ * setDeviceParameter (R/rpu_pulsed.cpp:392-410, R/rpu_pulsed_device.cpp:235-330) as bound at
+ * B/rpu_base_tiles.cpp:763-825.  Names in order: max_bound, min_bound, dwmin_up, dwmin_down,
+ * decay_scales, diffusion_rates, reset_bias, drift_nu [, slope_up, slope_down].
+ * `data_host` is [n][d_size][x_size]. */
+int rpu_tile_hidden_parameter_count(const rpu_tile_t *tile);
+const char *rpu_tile_hidden_parameter_name(const rpu_tile_t *tile, int idx);
+int rpu_tile_get_hidden_parameters(rpu_tile_t *tile, float *data_host);
+int rpu_tile_set_hidden_parameters(rpu_tile_t *tile, const float *data_host);
+
+/* Seed of the counter-based Philox4x32-10 generator that drives every random draw on the GPU
+ * (output noise, stochastic rounding, pulse trains, cycle-to-cycle noise).  A draw is a pure
+ * function of (seed, call index, purpose, element index); the call index restarts at 0 here.
+ * Stands in for the per-context cuRAND state of the reference (C/cuda_util.cu:163-176,779-800). */
+int rpu_tile_set_seed(rpu_tile_t *tile, uint64_t seed);
+
+/* ---- inspection hooks (mirror the reference's debug hooks) ------------------------------ */
+
+/* After rpu_tile_update with a stochastic pulse type: copies the packed pulse words of that call
+ * to the host.  Word format (R/rpu_weight_updater.cpp:297-324, C/bit_line_maker.cu:886-927):
+ * bit 0 = sign (1 = negative input), bits 1..BL = pulses.  x_words_host is [m_batch][x_size],
+ * d_words_host is [m_batch][d_size], bl_host is [m_batch] (the per-sample BL chosen by update
+ * management).  Mirrors BitLineMaker::getCountsDebug (C/bit_line_maker.cu:1884). */
+int rpu_tile_get_update_words(rpu_tile_t *tile, uint32_t *x_words_host, uint32_t *d_words_host,
+                              int32_t *bl_host, int m_batch);
+
+/* After rpu_tile_update with RPU_PULSE_DETERMINISTIC_IMPLICIT: signed coincidence counts
+ * n[b][i][j] = (int) rintf((dv_i * BL) * xv_j) (R/dense_bit_line_maker.cpp:237-264) recomputed on the
+ * GPU from the stored line values of that call; counts_host is [m_batch][d_size][x_size]. */
+int rpu_tile_get_implicit_counts(rpu_tile_t *tile, int32_t *counts_host, int m_batch);
+
+/* After rpu_tile_forward with bound management: the number of rounds each sample took;
+ * rounds_host is [m_batch]. */
+int rpu_tile_get_bm_rounds(rpu_tile_t *tile, int32_t *rounds_host, int m_batch);
+
+/* Philox4x32-10 block function (Salmon, Moraes, Dror, Shaw, SC'11) as the kernels evaluate it, on the
+ * host and, through a one-thread kernel, on GPU `device_id` (-1 = current).  For known-answer tests of
+ * the generator; no counterpart in the reference, which uses cuRAND XORWOW (C/cuda_util.cu:163-176). */
+int rpu_philox4x32_10(const uint32_t counter[4], const uint32_t key[2], uint32_t out[4]);
+int rpu_philox4x32_10_device(const uint32_t counter[4], const uint32_t key[2], uint32_t out[4],
+                             int device_id);
+
+/* ---- errors / info ------------------------------------------------------------------------ */
+
+const char *rpu_last_error(void);
+int rpu_abi_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* RPU_AMD_H */

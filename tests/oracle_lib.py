@@ -1,0 +1,148 @@
+"""ctypes wrapper around oracle/librpu_oracle.so -- the CPU restatement used as checker by the tests."""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+from aihwkit_amd._cabi import TileConfig
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+ORACLE_DIR = os.path.join(ROOT, "oracle")
+ORACLE_LIB = os.path.join(ORACLE_DIR, "librpu_oracle.so")
+
+_lib = None
+
+
+def oracle():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(ORACLE_LIB):
+            subprocess.check_call(["make", "-C", ORACLE_DIR])
+        lib = C.CDLL(ORACLE_LIB)
+        P = C.c_void_p
+        lib.orc_create.restype = P
+        lib.orc_create.argtypes = [C.c_int, C.c_int, C.POINTER(TileConfig)]
+        lib.orc_destroy.argtypes = [P]
+        lib.orc_last_error.restype = C.c_char_p
+        lib.orc_set_seed.argtypes = [P, C.c_uint]
+        lib.orc_use_gauss_table.argtypes = [P, C.c_int]
+        lib.orc_set_learning_rate.argtypes = [P, C.c_float]
+        lib.orc_set_weights.argtypes = [P, P]
+        lib.orc_get_weights.argtypes = [P, P]
+        lib.orc_hidden_count.argtypes = [P]
+        lib.orc_get_hidden.argtypes = [P, P]
+        lib.orc_set_hidden.argtypes = [P, P]
+        lib.orc_forward.argtypes = [P, P, P, C.c_int, C.c_int, C.c_int, C.c_int]
+        lib.orc_get_bm_rounds.argtypes = [P, P, C.c_int]
+        lib.orc_backward.argtypes = [P, P, P, C.c_int, C.c_int, C.c_int, C.c_int]
+        lib.orc_update.argtypes = [P, P, P, C.c_int, C.c_int, C.c_int, C.c_int]
+        lib.orc_update_with_words.argtypes = [P, P, P, P, C.c_int]
+        lib.orc_update_bl_ab.argtypes = [P, P, P, C.c_int, P, P, P]
+        lib.orc_implicit_counts.argtypes = [P, P, P, C.c_int, P]
+        _lib = lib
+    return _lib
+
+
+def _f32(a):
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+class OracleTile:
+    """CPU tile with the reference's per-sample semantics (see oracle/rpu_oracle.cpp)."""
+
+    def __init__(self, x_size, d_size, config: TileConfig):
+        self.lib = oracle()
+        self.X, self.D = x_size, d_size
+        self.h = self.lib.orc_create(x_size, d_size, C.byref(config))
+        if not self.h:
+            raise RuntimeError(self.lib.orc_last_error().decode())
+
+    def __del__(self):
+        if getattr(self, "h", None):
+            self.lib.orc_destroy(self.h)
+            self.h = None
+
+    def set_seed(self, seed):
+        self.lib.orc_set_seed(self.h, seed)
+
+    def use_gauss_table(self, on):
+        self.lib.orc_use_gauss_table(self.h, int(on))
+
+    def set_learning_rate(self, lr):
+        self.lib.orc_set_learning_rate(self.h, lr)
+
+    def set_weights(self, w):
+        w = _f32(w)
+        assert w.shape == (self.D, self.X)
+        self.lib.orc_set_weights(self.h, w.ctypes.data)
+
+    def get_weights(self):
+        w = np.empty((self.D, self.X), np.float32)
+        self.lib.orc_get_weights(self.h, w.ctypes.data)
+        return w
+
+    def get_hidden(self):
+        n = self.lib.orc_hidden_count(self.h)
+        out = np.zeros((n, self.D, self.X), np.float32)
+        if n:
+            self.lib.orc_get_hidden(self.h, out.ctypes.data)
+        return out
+
+    def set_hidden(self, data):
+        data = _f32(data)
+        assert data.shape == (self.lib.orc_hidden_count(self.h), self.D, self.X)
+        self.lib.orc_set_hidden(self.h, data.ctypes.data)
+
+    def forward(self, x, bias=False, x_trans=False, d_trans=False):
+        x = _f32(x)
+        m = x.size // (self.X - int(bias))
+        y = np.empty((self.D, m) if d_trans else (m, self.D), np.float32)
+        self.lib.orc_forward(self.h, x.ctypes.data, y.ctypes.data, m, int(bias), int(x_trans), int(d_trans))
+        return y
+
+    def bm_rounds(self, m):
+        r = np.zeros(m, np.int32)
+        self.lib.orc_get_bm_rounds(self.h, r.ctypes.data, m)
+        return r
+
+    def backward(self, d, bias=False, d_trans=False, x_trans=False):
+        d = _f32(d)
+        m = d.size // self.D
+        xs = self.X - int(bias)
+        x = np.empty((xs, m) if x_trans else (m, xs), np.float32)
+        self.lib.orc_backward(self.h, d.ctypes.data, x.ctypes.data, m, int(bias), int(d_trans), int(x_trans))
+        return x
+
+    def update(self, x, d, bias=False, x_trans=False, d_trans=False):
+        x, d = _f32(x), _f32(d)
+        m = d.size // self.D
+        rc = self.lib.orc_update(self.h, x.ctypes.data, d.ctypes.data, m, int(bias), int(x_trans), int(d_trans))
+        if rc:
+            raise RuntimeError(self.lib.orc_last_error().decode())
+
+    def update_with_words(self, x_words, d_words, bl):
+        xw = np.ascontiguousarray(x_words).view(np.uint32)
+        dw = np.ascontiguousarray(d_words).view(np.uint32)
+        bl = np.ascontiguousarray(bl, dtype=np.int32)
+        self.lib.orc_update_with_words(self.h, xw.ctypes.data, dw.ctypes.data, bl.ctypes.data, len(bl))
+
+    def update_bl_ab(self, x, d):
+        x, d = _f32(x), _f32(d)
+        m = d.size // self.D
+        bl = np.zeros(m, np.int32)
+        a = np.zeros(m, np.float32)
+        b = np.zeros(m, np.float32)
+        rc = self.lib.orc_update_bl_ab(self.h, x.ctypes.data, d.ctypes.data, m, bl.ctypes.data, a.ctypes.data, b.ctypes.data)
+        if rc:
+            raise RuntimeError(self.lib.orc_last_error().decode())
+        return bl, a, b
+
+    def implicit_counts(self, x, d):
+        x, d = _f32(x), _f32(d)
+        m = d.size // self.D
+        c = np.zeros((m, self.D, self.X), np.int32)
+        rc = self.lib.orc_implicit_counts(self.h, x.ctypes.data, d.ctypes.data, m, c.ctypes.data)
+        if rc:
+            raise RuntimeError(self.lib.orc_last_error().decode())
+        return c

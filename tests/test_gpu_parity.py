@@ -1,0 +1,248 @@
+"""GPU parity tests: the HIP path (through the C ABI) against the CPU oracle on the same inputs.
+
+Bar: pulse words / coincidence counts / bit-line lengths bit-exact; weights and outputs within 1e-5
+absolute (fp32) when noise is off and pulses are deterministic or shared.
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+import torch
+
+from aihwkit_amd._cabi import lib
+from aihwkit_amd.rpu_base import devices as dv
+from aihwkit_amd.rpu_base import tiles
+from helpers import (build_pair, config1, config1_data, config2, config2_data, constant_step, io_params,
+                     make_meta, noise_free_io, soft_bounds)
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-5
+
+
+def cuda(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def test_philox_known_answers_on_device(gpu_device):
+    # Random123 known-answer vectors for philox4x32-10
+    kat = [
+        ([0, 0, 0, 0], [0, 0], [0x6627E8D5, 0xE169C58D, 0xBC57AC4C, 0x9B00DBD8]),
+        ([0xFFFFFFFF] * 4, [0xFFFFFFFF] * 2, [0x408F276D, 0x41C83B0E, 0xA20BC7C6, 0x6D5451FD]),
+        ([0x243F6A88, 0x85A308D3, 0x13198A2E, 0x03707344], [0xA4093822, 0x299F31D0],
+         [0xD16CFE09, 0x94FDCCEB, 0x5001E420, 0x24126EA1]),
+    ]
+    for ctr, key, want in kat:
+        out = (C.c_uint32 * 4)()
+        assert lib().rpu_philox4x32_10_device((C.c_uint32 * 4)(*ctr), (C.c_uint32 * 2)(*key), out, 0) == 0
+        assert list(out) == want
+
+
+@pytest.mark.parametrize("x_size,d_size,batch", [(64, 32, 32), (100, 70, 33), (512, 512, 100), (1024, 1024, 256)])
+@pytest.mark.parametrize("bm", [dv.BoundManagementType.NONE, dv.BoundManagementType.Iterative])
+def test_forward_exact_arithmetic_is_bit_exact(gpu_device, x_size, d_size, batch, bm):
+    """With a power-of-two DAC step and weights on a 1/64 grid every product and partial sum is exact in
+    fp32, so the summation order cannot matter: GPU and oracle must agree to the last bit."""
+    rng = np.random.default_rng(5)
+    f_io = noise_free_io(inp_res=1 / 128.0, out_res=1 / 512.0, bound_management=bm,
+                         noise_management=dv.NoiseManagementType.AbsMax)
+    meta = make_meta(f_io, noise_free_io(inp_res=1 / 128.0, out_res=1 / 512.0))
+    dev = constant_step(w_max_dtod=0.0, w_min_dtod=0.0, w_max=1.0, w_min=-1.0, construction_seed=7)
+    host, orc, _ = build_pair(meta, dev, x_size, d_size, gpu=False)
+    w = (rng.integers(-38, 39, (d_size, x_size)) / 64.0).astype(np.float32)
+    host.set_weights(torch.from_numpy(w))
+    orc.set_weights(w)
+    gpu = tiles.CudaAnalogTile(host)
+    x = rng.uniform(-1, 1, (batch, x_size)).astype(np.float32)
+    x[0] = 0.0  # the zero short-cut
+    y_gpu = gpu.forward(cuda(x), False, False, False, False, False).cpu().numpy()
+    y_orc = orc.forward(x)
+    assert np.array_equal(y_gpu, y_orc)
+    if bm != dv.BoundManagementType.NONE:
+        assert np.array_equal(gpu.get_bm_rounds(batch).numpy(), orc.bm_rounds(batch))
+        if x_size >= 512:
+            assert orc.bm_rounds(batch).max() > 1  # the case does exercise re-runs
+    # backward, same property
+    d = rng.uniform(-1, 1, (batch, d_size)).astype(np.float32)
+    assert np.array_equal(gpu.backward(cuda(d), False, False, False, False).cpu().numpy(), orc.backward(d))
+
+
+def _compare_with_lsb_flips(y_gpu, y_orc, lsb_per_row, max_flip_fraction):
+    diff = np.abs(y_gpu - y_orc)
+    bad = diff > TOL
+    # a differing entry must be exactly one ADC step (times the sample's output scale) away
+    rows = np.nonzero(bad)[0]
+    if rows.size:
+        steps = diff[bad] / lsb_per_row[rows]
+        assert np.allclose(steps, 1.0, atol=1e-3), steps
+    return bad.mean() <= max_flip_fraction, bad.mean()
+
+
+@pytest.mark.parametrize("cfg,data,shape", [(config1, config1_data, (512, 512, 100)),
+                                            (config2, config2_data, (1024, 1024, 256))])
+def test_forward_backward_benchmark_configs_noise_free(gpu_device, cfg, data, shape):
+    """Real DAC / ADC steps (1/126, 1/510): pre-ADC sums differ in the last bits between summation
+    orders, so an output may land on the other side of an ADC rounding edge.  Everything else must be
+    within 1e-5 and the flips must be exactly one LSB and rare."""
+    x_size, d_size, batch = shape
+    meta, dev = cfg(noise=False)
+    host, orc, _ = build_pair(meta, dev, x_size, d_size, gpu=False)
+    w, x, d = data(x_size, d_size, batch)
+    host.set_weights(torch.from_numpy(w))
+    orc.set_weights(w)
+    gpu = tiles.CudaAnalogTile(host)
+    assert np.array_equal(gpu.get_weights().numpy(), orc.get_weights())
+
+    y_gpu = gpu.forward(cuda(x), False, False, False, False, False).cpu().numpy()
+    y_orc = orc.forward(x)
+    r_gpu, r_orc = gpu.get_bm_rounds(batch).numpy(), orc.bm_rounds(batch)
+    same_rounds = r_gpu == r_orc
+    assert same_rounds.mean() > 0.97  # a flip at the ADC bound can change the round count of a sample
+    out_step = (1.0 / 510.0) * 24.0 if cfg is config2 else (1.0 / 511.0) * 24.0
+    nm = np.abs(x).max(axis=1)
+    lsb = out_step * nm * (2.0 ** (r_orc - 1))
+    ok, frac = _compare_with_lsb_flips(y_gpu[same_rounds], y_orc[same_rounds], lsb[same_rounds], 5e-3)
+    assert ok, frac
+
+    x_gpu = gpu.backward(cuda(d), False, False, False, False).cpu().numpy()
+    x_orc = orc.backward(d)
+    lsb_b = out_step * np.abs(d).max(axis=1)
+    ok, frac = _compare_with_lsb_flips(x_gpu, x_orc, lsb_b, 5e-3)
+    assert ok, frac
+
+
+@pytest.mark.parametrize("x_trans,d_trans,bias", [(False, False, False), (True, False, False), (False, True, False),
+                                                  (True, True, False), (False, False, True), (True, True, True)])
+def test_forward_backward_layouts(gpu_device, x_trans, d_trans, bias):
+    rng = np.random.default_rng(11)
+    x_size, d_size, batch = 72, 40, 19
+    f_io = noise_free_io(inp_res=1 / 128.0, out_res=1 / 512.0, bound_management=dv.BoundManagementType.Iterative)
+    meta = make_meta(f_io, noise_free_io(inp_res=1 / 128.0, out_res=1 / 512.0))
+    dev = constant_step(w_max_dtod=0.0, w_min_dtod=0.0, w_max=1.0, w_min=-1.0, construction_seed=7)
+    host, orc, _ = build_pair(meta, dev, x_size, d_size, gpu=False)
+    w = (rng.integers(-38, 39, (d_size, x_size)) / 64.0).astype(np.float32)
+    host.set_weights(torch.from_numpy(w))
+    orc.set_weights(w)
+    gpu = tiles.CudaAnalogTile(host)
+    xs = x_size - int(bias)
+    x = rng.uniform(-1, 1, (xs, batch) if x_trans else (batch, xs)).astype(np.float32)
+    y_gpu = gpu.forward(cuda(x), bias, x_trans, d_trans, False, False).cpu().numpy()
+    assert y_gpu.shape == ((d_size, batch) if d_trans else (batch, d_size))
+    assert np.array_equal(y_gpu, orc.forward(x, bias, x_trans, d_trans))
+    d = rng.uniform(-1, 1, (d_size, batch) if d_trans else (batch, d_size)).astype(np.float32)
+    x_gpu = gpu.backward(cuda(d), bias, d_trans, x_trans, False).cpu().numpy()
+    assert x_gpu.shape == ((xs, batch) if x_trans else (batch, xs))
+    assert np.array_equal(x_gpu, orc.backward(d, bias, d_trans, x_trans))
+
+
+def test_floating_point_tile(gpu_device):
+    rng = np.random.default_rng(3)
+    x_size, d_size, batch = 200, 150, 64
+    host = dv.FloatingPointTileParameter().create_array(x_size, d_size)
+    w = rng.standard_normal((d_size, x_size)).astype(np.float32)
+    host.set_weights(torch.from_numpy(w))
+    gpu = tiles.CudaFloatingPointTile(host)
+    x = rng.standard_normal((batch, x_size)).astype(np.float32)
+    d = rng.standard_normal((batch, d_size)).astype(np.float32)
+    y = gpu.forward(cuda(x)).cpu().numpy()
+    assert np.allclose(y, x.astype(np.float64) @ w.T.astype(np.float64), atol=1e-4)
+    xb = gpu.backward(cuda(d)).cpu().numpy()
+    assert np.allclose(xb, d.astype(np.float64) @ w.astype(np.float64), atol=1e-4)
+    gpu.set_learning_rate(0.1)
+    gpu.update(cuda(x), cuda(d), False)
+    want = w.astype(np.float64) - 0.1 * d.T.astype(np.float64) @ x.astype(np.float64)
+    assert np.allclose(gpu.get_weights().numpy(), want, atol=1e-4)
+
+
+def _word_invariants(words, values, bl):
+    words = words.astype(np.int64) & 0xFFFFFFFF
+    pulses = words >> 1
+    # no pulse beyond the sample's BL
+    limit = (1 << bl.astype(np.int64)) - 1
+    assert np.all((pulses & ~limit[:, None]) == 0)
+    # sign bit only where the input is not positive, and zero input gives an empty word
+    has = pulses != 0
+    assert np.all(((words & 1) == 1)[has] == (values <= 0)[has])
+    assert np.all(words[values == 0] == 0)
+
+
+@pytest.mark.parametrize("device", ["constant", "soft"])
+@pytest.mark.parametrize("um", [True, False])
+def test_stochastic_update_words_drive_the_oracle_to_the_same_weights(gpu_device, device, um):
+    """Cycle-to-cycle noise off: the GPU's packed pulse words, fed to the oracle's sparse update loop
+    (the reference's updateVectorWithDeviceAndCounts protocol), must give the GPU's weights."""
+    rng = np.random.default_rng(21)
+    x_size, d_size, batch = 96, 80, 40
+    meta = make_meta(desired_bl=31, update_management=um, update_bl_management=um)
+    kw = dict(dw_min=0.001, dw_min_std=0.0, construction_seed=99, enforce_consistency=True)
+    dev = constant_step(**kw) if device == "constant" else soft_bounds(**kw)
+    host, orc, _ = build_pair(meta, dev, x_size, d_size, gpu=False)
+    w = rng.uniform(-0.5, 0.5, (d_size, x_size)).astype(np.float32)
+    host.set_weights(torch.from_numpy(w))
+    orc.set_weights(w)
+    gpu = tiles.CudaAnalogTile(host)
+    gpu.set_seed(4)
+    x = rng.uniform(-1, 1, (batch, x_size)).astype(np.float32)
+    d = (0.3 * rng.standard_normal((batch, d_size))).astype(np.float32)
+    x[3] = 0.0
+    d[5, :7] = 0.0
+    for lr in (0.01, 0.02):
+        gpu.set_learning_rate(lr)
+        orc.set_learning_rate(lr)
+        gpu.update(cuda(x), cuda(d), False, False, False, False)
+        xw, dw, bl = (t.numpy() for t in gpu.get_update_words(batch))
+        bl_orc, _, _ = orc.update_bl_ab(x, d)
+        assert np.array_equal(bl, bl_orc)
+        _word_invariants(xw, x, bl)
+        _word_invariants(dw, d, bl)
+        assert (xw >> 1).any() and (dw >> 1).any()
+        orc.update_with_words(xw, dw, bl)
+        assert np.abs(gpu.get_weights().numpy() - orc.get_weights()).max() <= TOL
+    assert np.abs(orc.get_weights() - np.clip(w, orc.get_hidden()[1], orc.get_hidden()[0])).max() > 1e-3
+
+
+def test_pulse_probabilities_saturate(gpu_device):
+    """|v| * scale >= 1 gives all BL pulses, 0 gives none (the reference's bit-line maker test protocol)."""
+    x_size, d_size, batch = 64, 64, 8
+    meta = make_meta(desired_bl=31, update_management=False, update_bl_management=False)
+    dev = constant_step(dw_min=0.001, dw_min_std=0.0, dw_min_dtod=0.0, construction_seed=1)
+    host, orc, gpu = build_pair(meta, dev, x_size, d_size)
+    lr = 0.031 * 4.0  # A = B = sqrt(lr / (dw_min * BL)) = 2
+    gpu.set_learning_rate(lr)
+    x = np.zeros((batch, x_size), np.float32)
+    d = np.zeros((batch, d_size), np.float32)
+    x[:, ::2] = 0.6
+    x[:, 1::4] = -0.75
+    d[:, ::2] = -1.0
+    gpu.update(cuda(x), cuda(d), False)
+    xw, dw, bl = (t.numpy().astype(np.int64) & 0xFFFFFFFF for t in gpu.get_update_words(batch))
+    assert np.all(bl == 31)
+    full = 0xFFFFFFFE
+    assert np.all(xw[:, ::2] == full) and np.all(xw[:, 1::4] == (full | 1)) and np.all(xw[:, 3::4] == 0)
+    assert np.all(dw[:, ::2] == (full | 1)) and np.all(dw[:, 1::2] == 0)
+
+
+@pytest.mark.parametrize("device", ["constant", "soft"])
+def test_deterministic_implicit_counts_are_bit_exact(gpu_device, device):
+    rng = np.random.default_rng(8)
+    x_size, d_size, batch = 70, 50, 24
+    meta = make_meta(desired_bl=31, pulse_type=dv.PulseType.DeterministicImplicit, x_res_implicit=1 / 20.0,
+                     d_res_implicit=1 / 30.0)
+    kw = dict(dw_min=0.001, dw_min_std=0.0, construction_seed=5, enforce_consistency=True)
+    dev = constant_step(**kw) if device == "constant" else soft_bounds(**kw)
+    host, orc, _ = build_pair(meta, dev, x_size, d_size, gpu=False)
+    w = rng.uniform(-0.4, 0.4, (d_size, x_size)).astype(np.float32)
+    host.set_weights(torch.from_numpy(w))
+    orc.set_weights(w)
+    gpu = tiles.CudaAnalogTile(host)
+    x = rng.uniform(-1, 1, (batch, x_size)).astype(np.float32)
+    d = (0.2 * rng.standard_normal((batch, d_size))).astype(np.float32)
+    gpu.set_learning_rate(0.02)
+    orc.set_learning_rate(0.02)
+    for _ in range(2):
+        gpu.update(cuda(x), cuda(d), False)
+        counts = gpu.get_implicit_counts(batch).numpy()
+        assert np.array_equal(counts, orc.implicit_counts(x, d))
+        assert np.abs(counts).max() >= 2
+        orc.update(x, d)
+        assert np.abs(gpu.get_weights().numpy() - orc.get_weights()).max() <= TOL
