@@ -155,6 +155,17 @@ class _CudaTileMixin:
         if not non_blocking:
             torch.cuda.current_stream(tensor.device).synchronize()
 
+    @staticmethod
+    def _out_dims(inp: torch.Tensor, in_trans: bool, out_trans: bool, m_batch: int, out_size: int):
+        # The reference copies the input dims and replaces the first (transposed) or last entry
+        # (rpu_base_tiles_cuda.cpp:170-189).  That is only a valid shape when both flags agree, which is
+        # how its Python callers use it; with mixed flags the result is the plain 2-D matrix.
+        if in_trans == out_trans:
+            dims = list(inp.shape)
+            dims[0 if out_trans else -1] = out_size
+            return dims
+        return [out_size, m_batch] if out_trans else [m_batch, out_size]
+
     # rpu_base_tiles_cuda.cpp:159-236
     def forward(self, x_input: torch.Tensor, bias: bool = False, x_trans: bool = False, d_trans: bool = False,
                 is_test: bool = False, non_blocking: bool = False) -> torch.Tensor:
@@ -167,9 +178,8 @@ class _CudaTileMixin:
             shape = f"[*, {expected}]" if x_trans else f"[{expected},*]"
             raise RuntimeError(f"Invalid x_input dimensions: expected {shape} tensor")
         m_batch = x_input.numel() // in_size
-        dims = list(x_input.shape)
-        dims[0 if d_trans else -1] = self.get_d_size()
-        d_output = torch.empty(dims, dtype=x_input.dtype, device=x_input.device)
+        d_output = torch.empty(self._out_dims(x_input, x_trans, d_trans, m_batch, self.get_d_size()),
+                               dtype=x_input.dtype, device=x_input.device)
         check(lib().rpu_tile_forward(self._h, x_input.data_ptr(), d_output.data_ptr(), m_batch, int(bias),
                                      int(x_trans), int(d_trans), int(is_test), self._stream_for(x_input)))
         self._finish(x_input, non_blocking)
@@ -187,9 +197,9 @@ class _CudaTileMixin:
             shape = f"[*, {expected}]" if d_trans else f"[{expected},*]"
             raise RuntimeError(f"Invalid d_input dimensions: expected {shape} tensor")
         m_batch = d_input.numel() // in_size
-        dims = list(d_input.shape)
-        dims[0 if x_trans else -1] = self.get_x_size() - (1 if bias else 0)
-        x_output = torch.empty(dims, dtype=d_input.dtype, device=d_input.device)
+        x_output = torch.empty(
+            self._out_dims(d_input, d_trans, x_trans, m_batch, self.get_x_size() - (1 if bias else 0)),
+            dtype=d_input.dtype, device=d_input.device)
         check(lib().rpu_tile_backward(self._h, d_input.data_ptr(), x_output.data_ptr(), m_batch, int(bias),
                                       int(d_trans), int(x_trans), self._stream_for(d_input)))
         self._finish(d_input, non_blocking)
