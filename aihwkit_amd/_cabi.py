@@ -93,6 +93,9 @@ SYMBOLS = {
     "rpu_tile_get_update_words": (C.c_int, [_P, _P, _P, _P, C.c_int]),
     "rpu_tile_get_implicit_counts": (C.c_int, [_P, _P, C.c_int]),
     "rpu_tile_get_bm_rounds": (C.c_int, [_P, _P, C.c_int]),
+    "rpu_tile_set_profiling": (C.c_int, [_P, C.c_int]),
+    "rpu_tile_get_profile": (C.c_int, [_P, _P, C.c_int, C.POINTER(C.c_int)]),
+    "rpu_tile_profile_name": (C.c_char_p, [_P, C.c_int]),
     "rpu_philox4x32_10": (C.c_int, [C.POINTER(C.c_uint32), C.POINTER(C.c_uint32), C.POINTER(C.c_uint32)]),
     "rpu_philox4x32_10_device": (C.c_int, [C.POINTER(C.c_uint32), C.POINTER(C.c_uint32), C.POINTER(C.c_uint32), C.c_int]),
     "rpu_last_error": (C.c_char_p, []),

@@ -102,6 +102,29 @@ struct Tile {
   int last_update_pulse = -1;
   int last_forward_batch = 0;
 
+  // optional per-kernel timing with HIP events on the launch stream
+  bool profiling = false;
+  std::vector<hipEvent_t> prof_events;
+  std::vector<const char *> prof_names;
+  size_t prof_used = 0;
+
+  void prof_begin(hipStream_t s) {
+    if (!profiling) return;
+    prof_used = 0;
+    prof_names.clear();
+    prof_mark(s, nullptr);
+  }
+  void prof_mark(hipStream_t s, const char *name) {
+    if (!profiling) return;
+    if (prof_used == prof_events.size()) {
+      hipEvent_t e;
+      RPU_HIP_CHECK(hipEventCreate(&e));
+      prof_events.push_back(e);
+    }
+    RPU_HIP_CHECK(hipEventRecord(prof_events[prof_used++], s));
+    if (name) prof_names.push_back(name);
+  }
+
   bool resident() const { return device_id >= 0; }
   size_t size() const { return (size_t)X * (size_t)D; }
 
@@ -110,6 +133,7 @@ struct Tile {
       try {
         DeviceGuard g(device_id);
         (void)hipDeviceSynchronize();
+        for (hipEvent_t e : prof_events) (void)hipEventDestroy(e);
         release_all();
       } catch (...) {
       }
@@ -244,14 +268,22 @@ struct Tile {
 
     if (io.perfect) {
       a.round = 0;
+      prof_begin(s);
       launch_mvm_round(a, s);
+      prof_mark(s, "mvm_round");
     } else {
+      prof_begin(s);
       launch_mvm_init(a, s);
+      prof_mark(s, "mvm_init");
       const int rounds = mvm_max_rounds(a.io);
       for (int r = 0; r < rounds; ++r) {
         a.round = r;
         launch_mvm_round(a, s);
-        if (r + 1 < rounds) launch_mvm_advance(a, s);
+        prof_mark(s, "mvm_round");
+        if (r + 1 < rounds) {
+          launch_mvm_advance(a, s);
+          prof_mark(s, "mvm_advance");
+        }
       }
     }
     if (transposed && bias) launch_drop_bias(s_bias.p, final_out, B, X, out_trans ? 1 : 0, s);
@@ -282,7 +314,9 @@ struct Tile {
       a.io = io_dev(fio); a.io.perfect = 1;
       a.alpha = -lr; a.beta = 1.0f; a.round = 0;
       a.key = key(); a.call = call++;
+      prof_begin(s);
       launch_mvm_round(a, s);
+      prof_mark(s, "fp_update");
       RPU_HIP_CHECK(hipGetLastError());
       last_stream = s;
       last_update_batch = B;
@@ -305,17 +339,26 @@ struct Tile {
     u_bl.ensure(B); u_a.ensure(B); u_b.ensure(B);
     a.bl = u_bl.p; a.prob_a = u_a.p; a.prob_b = u_b.p;
     a.key = key(); a.call = call++;
-    launch_update_prepare(a, s);
     if (up.p.pulse_type == RPU_PULSE_STOCHASTIC_COMPRESSED) {
       u_xw.ensure((size_t)B * X); u_dw.ensure((size_t)B * D);
       a.x_words = u_xw.p; a.d_words = u_dw.p;
-      launch_update_bitlines(a, s);
-      launch_update_pulsed(a, s);
     } else {
       u_xval.ensure((size_t)B * X); u_dval.ensure((size_t)B * D);
       a.x_val = u_xval.p; a.d_val = u_dval.p;
+    }
+    prof_begin(s);
+    launch_update_prepare(a, s);
+    prof_mark(s, "update_prepare");
+    if (up.p.pulse_type == RPU_PULSE_STOCHASTIC_COMPRESSED) {
+      launch_update_bitlines(a, s);
+      prof_mark(s, "update_bitlines");
+      launch_update_pulsed(a, s);
+      prof_mark(s, "update_pulsed");
+    } else {
       launch_update_implicit_lines(a, s);
+      prof_mark(s, "update_implicit_lines");
       launch_update_implicit(a, s);
+      prof_mark(s, "update_implicit");
     }
     RPU_HIP_CHECK(hipGetLastError());
     last_stream = s;
@@ -640,6 +683,38 @@ int rpu_tile_get_bm_rounds(rpu_tile_t *tile, int32_t *rounds_host, int m_batch) 
     t.sync_last();
     RPU_HIP_CHECK(hipMemcpy(rounds_host, t.s_rounds.p, (size_t)m_batch * 4, hipMemcpyDeviceToHost));
   });
+}
+
+int rpu_tile_set_profiling(rpu_tile_t *tile, int enable) {
+  return guarded([&] {
+    if (!tile) throw RpuError("null tile");
+    std::lock_guard<std::mutex> lock(tile->t.mutex);
+    tile->t.profiling = enable != 0;
+    tile->t.prof_used = 0;
+    tile->t.prof_names.clear();
+  });
+}
+
+int rpu_tile_get_profile(rpu_tile_t *tile, float *ms_host, int capacity, int *count) {
+  return guarded([&] {
+    if (!tile || !count) throw RpuError("null argument");
+    Tile &t = tile->t;
+    std::lock_guard<std::mutex> lock(t.mutex);
+    const int n = (int)t.prof_names.size();
+    *count = n;
+    if (n == 0 || !ms_host) return;
+    if (capacity < n) throw RpuError("profile buffer too small");
+    DeviceGuard g(t.device_id);
+    t.sync_last();
+    for (int i = 0; i < n; ++i) {
+      RPU_HIP_CHECK(hipEventElapsedTime(&ms_host[i], t.prof_events[i], t.prof_events[i + 1]));
+    }
+  });
+}
+
+const char *rpu_tile_profile_name(const rpu_tile_t *tile, int idx) {
+  if (!tile || idx < 0 || idx >= (int)tile->t.prof_names.size()) return nullptr;
+  return tile->t.prof_names[idx];
 }
 
 int rpu_philox4x32_10(const uint32_t counter[4], const uint32_t key[2], uint32_t out[4]) {

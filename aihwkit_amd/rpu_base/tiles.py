@@ -248,6 +248,17 @@ class _CudaTileMixin:
         check(lib().rpu_tile_get_implicit_counts(self._h, counts.data_ptr(), m_batch))
         return counts
 
+    def set_profiling(self, enable: bool) -> None:
+        """Record HIP events around every kernel of the following compute calls."""
+        check(lib().rpu_tile_set_profiling(self._h, int(enable)))
+
+    def get_profile(self):
+        """[(kernel name, milliseconds)] of the last compute call, in launch order."""
+        count = C.c_int(0)
+        buf = (C.c_float * 128)()
+        check(lib().rpu_tile_get_profile(self._h, buf, 128, C.byref(count)))
+        return [(lib().rpu_tile_profile_name(self._h, k).decode(), float(buf[k])) for k in range(count.value)]
+
     def get_bm_rounds(self, m_batch: int) -> torch.Tensor:
         """Number of bound-management rounds each sample of the last forward pass took."""
         rounds = torch.empty(m_batch, dtype=torch.int32)

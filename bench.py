@@ -1,0 +1,198 @@
+#!/usr/bin/env python3
+"""Benchmark of the analog-tile hot path on one MI355X.
+
+A step is one forward + one backward + one pulsed update of a single analog tile over one batch of
+synthetic inputs that are resident in HBM (benchmark configuration 2: 1024 x 1024 SoftBounds tile with
+device-to-device and cycle-to-cycle variation, batch 256, BL 31, update management and update-BL
+management on, 7-bit DAC / 9-bit ADC, out_noise 0.06, abs-max noise management, iterative bound
+management in the forward pass).
+
+Prints ONE JSON line: `value` is the pulsed-update rate in Gdevice-updates/s (x_size * d_size * batch
+per update call / time of the update call); the noisy forward / backward rates (GFLOP/s counted as
+2 * x * d * batch per call, bound-management re-runs not counted) are in `forward` / `backward`.
+`roofline` covers the dominant kernel of the step (the per-cross-point update kernel) against HBM
+bandwidth, `roofline_forward` the MFMA contraction kernel against the fp32 matrix peak, `cpu_baseline`
+the CPU oracle timed on this host.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, "tests"), os.path.join(ROOT, "oracle")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
+FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU oracle timing")
+    ap.add_argument("--config", type=int, default=2, choices=(1, 2), help="benchmark configuration (2 is graded)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU; an analog tile is an independent unit and the path "
+              "uses no collective, so --gpus must be 1.", file=sys.stderr)
+        return 2
+
+    import numpy as np
+    import torch
+
+    from aihwkit_amd._cabi import lib
+    from aihwkit_amd.rpu_base import tiles
+    from helpers import config1, config1_data, config2, config2_data
+
+    lib()  # fails loudly if the HIP library is not built
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 1
+    torch.cuda.set_device(0)
+
+    if args.config == 2:
+        x_size, d_size, batch = 1024, 1024, 256
+        meta, dev = config2()
+        w, x, d = config2_data(x_size, d_size, batch)
+        workload = "config2: 1024x1024 SoftBounds (dtod + ctoc), batch 256, BL 31, UM+UBLM, 7/9-bit IO, iterative BM"
+        bytes_per_device = 32.0  # w read + w write + 6 parameter arrays
+    else:
+        x_size, d_size, batch = 512, 512, 100
+        meta, dev = config1()
+        w, x, d = config1_data(x_size, d_size, batch)
+        workload = "config1: 512x512 ConstantStep (no variation), batch 100, BL 31, UM+UBLM"
+        bytes_per_device = 24.0
+    lr = 0.01
+    host = meta.create_array(x_size, d_size, dev)
+    host.set_weights(torch.from_numpy(w))
+    tile = tiles.CudaAnalogTile(host)
+    tile.set_learning_rate(lr)
+    tile.set_seed(1234)
+    xg = torch.from_numpy(x).cuda()
+    dg = torch.from_numpy(d).cuda()
+
+    def step():
+        tile.forward(xg, False, False, False, False, True)
+        tile.backward(dg, False, False, False, True)
+        tile.update(xg, dg, False, False, False, True)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    def time_calls(fn, n):
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        fn()
+        torch.cuda.synchronize()
+        start.record()
+        for _ in range(n):
+            fn()
+        end.record()
+        torch.cuda.synchronize()
+        return start.elapsed_time(end) / n
+
+    n = max(args.steps, 10)
+    ms_update = time_calls(lambda: tile.update(xg, dg, False, False, False, True), n)
+    ms_forward = time_calls(lambda: tile.forward(xg, False, False, False, False, True), n)
+    ms_backward = time_calls(lambda: tile.backward(dg, False, False, False, True), n)
+
+    # per-kernel durations from HIP events recorded by the library on the launch stream
+    tile.set_profiling(True)
+
+    def kernel_ms(fn, n_calls):
+        acc = {}
+        for _ in range(n_calls):
+            fn()
+            for name, ms in tile.get_profile():
+                acc.setdefault(name, []).append(ms)
+        return {k: (float(np.sum(v)) / n_calls, len(v) // n_calls) for k, v in acc.items()}
+
+    prof_update = kernel_ms(lambda: tile.update(xg, dg, False, False, False, True), n)
+    prof_forward = kernel_ms(lambda: tile.forward(xg, False, False, False, False, True), n)
+    rounds = tile.get_bm_rounds(batch).numpy()  # of the last forward call, before backward reuses the state
+    prof_backward = kernel_ms(lambda: tile.backward(dg, False, False, False, True), n)
+    tile.set_profiling(False)
+
+    devices_per_call = float(x_size) * d_size * batch
+    flops_per_call = 2.0 * x_size * d_size * batch
+    update_bytes = bytes_per_device * x_size * d_size + 4.0 * (x_size + d_size) * batch
+    k_update_ms = prof_update["update_pulsed"][0]
+    k_fwd_ms = prof_forward["mvm_round"][0]   # all rounds of one forward call
+    k_bwd_ms = prof_backward["mvm_round"][0]
+
+    out = {
+        "metric": "pulsed-update Gdevice-updates/s + noisy fwd GFLOP/s, 1024^2 tile, 1 MI355X",
+        "value": devices_per_call / (ms_update * 1e-3) / 1e9,
+        "unit": "Gdevice-updates/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": workload, "x_size": x_size, "d_size": d_size, "batch": batch, "lr": lr,
+                   "step": "forward + backward + update"},
+        "update": {"ms_per_call": ms_update, "kernels_ms": {k: v[0] for k, v in prof_update.items()}},
+        "forward": {"ms_per_call": ms_forward, "gflops": flops_per_call / (ms_forward * 1e-3) / 1e9,
+                    "mean_bm_rounds": float(rounds.mean()), "kernels_ms": {k: v[0] for k, v in prof_forward.items()}},
+        "backward": {"ms_per_call": ms_backward, "gflops": flops_per_call / (ms_backward * 1e-3) / 1e9,
+                     "kernels_ms": {k: v[0] for k, v in prof_backward.items()}},
+        "roofline": {"kernel": "k_update_pulsed", "bound": "hbm", "achieved": update_bytes / (k_update_ms * 1e-3) / 1e9,
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": update_bytes / (k_update_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None,
+                     "algorithmic_bytes": update_bytes, "kernel_ms": k_update_ms},
+        "roofline_forward": {"kernel": "k_mvm_round (all rounds of a call)", "bound": "mfma",
+                             "achieved": flops_per_call / (k_fwd_ms * 1e-3) / 1e12, "peak": FP32_MFMA_PEAK_TFLOPS,
+                             "unit": "TFLOP/s", "frac": flops_per_call / (k_fwd_ms * 1e-3) / 1e12 / FP32_MFMA_PEAK_TFLOPS,
+                             "traffic": None, "algorithmic_flops": flops_per_call, "kernel_ms": k_fwd_ms},
+        "roofline_backward": {"kernel": "k_mvm_round", "bound": "mfma",
+                              "achieved": flops_per_call / (k_bwd_ms * 1e-3) / 1e12, "peak": FP32_MFMA_PEAK_TFLOPS,
+                              "unit": "TFLOP/s", "frac": flops_per_call / (k_bwd_ms * 1e-3) / 1e12 / FP32_MFMA_PEAK_TFLOPS,
+                              "kernel_ms": k_bwd_ms},
+    }
+
+    if not args.no_cpu_baseline:
+        from oracle_lib import OracleTile
+
+        orc = OracleTile(x_size, d_size, meta._config(dev))
+        orc.set_weights(w)
+        orc.set_learning_rate(lr)
+        orc.set_seed(7)
+        orc.forward(x[:8])
+        t0 = time.perf_counter()
+        orc.forward(x)
+        cpu_fwd = time.perf_counter() - t0
+        t0 = time.perf_counter()
+        orc.backward(d)
+        cpu_bwd = time.perf_counter() - t0
+        n_upd = 3
+        t0 = time.perf_counter()
+        for _ in range(n_upd):
+            orc.update(x, d)
+        cpu_upd = (time.perf_counter() - t0) / n_upd
+        out["cpu_baseline"] = {
+            "value": devices_per_call / cpu_upd / 1e9, "unit": "Gdevice-updates/s", "cores": 1, "kind": "port",
+            "sample": f"{n_upd} full update calls, 1 forward and 1 backward call of the same workload on the CPU oracle (1 thread)",
+            "update_ms": cpu_upd * 1e3, "forward_ms": cpu_fwd * 1e3, "forward_gflops": flops_per_call / cpu_fwd / 1e9,
+            "backward_ms": cpu_bwd * 1e3, "backward_gflops": flops_per_call / cpu_bwd / 1e9,
+            "host_cpus": os.cpu_count(),
+        }
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

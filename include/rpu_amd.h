@@ -283,6 +283,14 @@ int rpu_tile_get_implicit_counts(rpu_tile_t *tile, int32_t *counts_host, int m_b
  * rounds_host is [m_batch]. */
 int rpu_tile_get_bm_rounds(rpu_tile_t *tile, int32_t *rounds_host, int m_batch);
 
+/* Per-kernel timing: while enabled, every compute call records HIP events on its launch stream
+ * around each kernel; rpu_tile_get_profile waits for the last call and returns the kernel durations
+ * in milliseconds in launch order (names through rpu_tile_profile_name).  Takes the place of the
+ * reference's CUDA_TIMING_* event macros (C/cuda_util.h:144-163). */
+int rpu_tile_set_profiling(rpu_tile_t *tile, int enable);
+int rpu_tile_get_profile(rpu_tile_t *tile, float *ms_host, int capacity, int *count);
+const char *rpu_tile_profile_name(const rpu_tile_t *tile, int idx);
+
 /* Philox4x32-10 block function (Salmon, Moraes, Dror, Shaw, SC'11) as the kernels evaluate it, on the
  * host and, through a one-thread kernel, on GPU `device_id` (-1 = current).  For known-answer tests of
  * the generator; no counterpart in the reference, which uses cuRAND XORWOW (C/cuda_util.cu:163-176). */

@@ -1,4 +1,5 @@
-"""ctypes wrapper around oracle/librpu_oracle.so -- the CPU restatement used as checker by the tests."""
+"""TEST INFRASTRUCTURE -- ctypes wrapper around librpu_oracle.so, the CPU restatement that tests, the
+smoke check and the cpu_baseline leg of the benchmark use as checker.  The shipped package never imports it."""
 import ctypes as C
 import os
 import subprocess
@@ -7,8 +8,7 @@ import numpy as np
 
 from aihwkit_amd._cabi import TileConfig
 
-ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-ORACLE_DIR = os.path.join(ROOT, "oracle")
+ORACLE_DIR = os.path.dirname(os.path.abspath(__file__))
 ORACLE_LIB = os.path.join(ORACLE_DIR, "librpu_oracle.so")
 
 _lib = None

@@ -1,0 +1,201 @@
+"""Statistical parity with noise and stochastic pulses on: mean and variance of outputs and of the
+weight change over 64 seeds must agree between the GPU path and the CPU oracle within 3 sigma, plus
+size-independent properties at the full benchmark size (1024 x 1024, batch 256)."""
+import numpy as np
+import pytest
+import torch
+
+from aihwkit_amd.rpu_base import devices as dv
+from aihwkit_amd.rpu_base import tiles
+from helpers import build_pair, config2, config2_data, constant_step, io_params, make_meta, soft_bounds
+
+pytestmark = pytest.mark.gpu
+
+N_SEEDS = 64
+
+
+def cuda(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def compare_moments(a, b, what):
+    """a, b: [seeds, ...] samples of the same quantity from two implementations.
+
+    Per element: z = (mean_a - mean_b) / sqrt((var_a + var_b) / n) must exceed 3 no more often than chance
+    allows; pooled over all elements the mean of z must vanish within 4 standard errors and the summed
+    variances must agree within 3 sigma of the summed-variance estimator."""
+    n = a.shape[0]
+    a = a.reshape(n, -1).astype(np.float64)
+    b = b.reshape(n, -1).astype(np.float64)
+    ma, mb = a.mean(0), b.mean(0)
+    va, vb = a.var(0, ddof=1), b.var(0, ddof=1)
+    live = (va + vb) > 0
+    assert live.mean() > 0.5, what
+    z = (ma[live] - mb[live]) / np.sqrt((va[live] + vb[live]) / n)
+    frac = np.mean(np.abs(z) > 3.0)
+    assert frac < 0.012, (what, "fraction of elements beyond 3 sigma", frac)  # 0.27 % for a Gaussian, t-tails allowed for
+    assert abs(z.mean()) < 4.0 / np.sqrt(z.size) + 0.01, (what, "pooled mean shift (in sigma)", z.mean())
+    # elements whose mean differs although neither implementation shows any variance would be a deterministic bug
+    dead = ~live
+    assert np.allclose(ma[dead], mb[dead], atol=1e-5), what
+    # variance: pooled ratio; the estimator's own spread from the per-element fourth moments
+    sa, sb = va[live].sum(), vb[live].sum()
+    m4a = ((a[:, live] - ma[live]) ** 4).mean(0)
+    m4b = ((b[:, live] - mb[live]) ** 4).mean(0)
+    sd = np.sqrt(((m4a - va[live] ** 2).clip(0) + (m4b - vb[live] ** 2).clip(0)).sum() / n)
+    assert abs(sa - sb) < 3.0 * sd + 0.01 * max(sa, sb), (what, "pooled variance", sa, sb, sd)
+    ratio = np.log(va[live & (va > 0) & (vb > 0)] / vb[live & (va > 0) & (vb > 0)])
+    assert np.mean(np.abs(ratio) > 1.5) < 0.02, (what, "per-element variance ratio tails")
+
+
+def test_forward_backward_output_moments_over_64_seeds(gpu_device):
+    rng = np.random.default_rng(0)
+    x_size, d_size, batch = 768, 128, 32
+    f_io = io_params(out_noise=0.06, noise_management=dv.NoiseManagementType.AbsMax,
+                     bound_management=dv.BoundManagementType.Iterative)
+    b_io = io_params(out_noise=0.06, noise_management=dv.NoiseManagementType.AbsMax)
+    meta = make_meta(f_io, b_io)
+    dev = soft_bounds(construction_seed=123, enforce_consistency=True)
+    host, orc, _ = build_pair(meta, dev, x_size, d_size, gpu=False)
+    w = rng.uniform(-0.6, 0.6, (d_size, x_size)).astype(np.float32)
+    host.set_weights(torch.from_numpy(w))
+    orc.set_weights(w)
+    gpu = tiles.CudaAnalogTile(host)
+    x = rng.uniform(-1, 1, (batch, x_size)).astype(np.float32)
+    d = (0.05 * rng.standard_normal((batch, d_size))).astype(np.float32)
+    xg, dg = cuda(x), cuda(d)
+    yg, yo, bg, bo, rg, ro = [], [], [], [], [], []
+    for s in range(N_SEEDS):
+        gpu.set_seed(1000 + s)
+        orc.set_seed(1 + s)
+        yg.append(gpu.forward(xg, False, False, False, False, False).cpu().numpy())
+        rg.append(gpu.get_bm_rounds(batch).numpy())
+        yo.append(orc.forward(x))
+        ro.append(orc.bm_rounds(batch))
+        bg.append(gpu.backward(dg, False, False, False, False).cpu().numpy())
+        bo.append(orc.backward(d))
+    assert np.mean(ro) > 1.5  # bound management is exercised
+    assert abs(np.mean(rg) - np.mean(ro)) < 0.05
+    compare_moments(np.stack(yg), np.stack(yo), "forward outputs")
+    compare_moments(np.stack(bg), np.stack(bo), "backward outputs")
+    # two GPU calls with the same seed give the same numbers, another seed does not
+    gpu.set_seed(5)
+    y1 = gpu.forward(xg, False, False, False, False, False).cpu().numpy()
+    gpu.set_seed(5)
+    y2 = gpu.forward(xg, False, False, False, False, False).cpu().numpy()
+    gpu.set_seed(6)
+    y3 = gpu.forward(xg, False, False, False, False, False).cpu().numpy()
+    assert np.array_equal(y1, y2) and not np.array_equal(y1, y3)
+
+
+@pytest.mark.parametrize("device,um", [("soft", True), ("constant", False), ("constant", True)])
+def test_update_weight_change_moments_over_64_seeds(gpu_device, device, um):
+    rng = np.random.default_rng(1)
+    x_size, d_size, batch = 128, 96, 24
+    meta = make_meta(desired_bl=31, update_management=um, update_bl_management=um)
+    kw = dict(dw_min=0.001, dw_min_dtod=0.3, dw_min_std=0.3, up_down_dtod=0.01, w_max_dtod=0.3, w_min_dtod=0.3,
+              construction_seed=123, enforce_consistency=True)
+    dev = soft_bounds(**kw) if device == "soft" else constant_step(**kw)
+    host, orc, _ = build_pair(meta, dev, x_size, d_size, gpu=False)
+    w = rng.uniform(-0.6, 0.6, (d_size, x_size)).astype(np.float32)
+    host.set_weights(torch.from_numpy(w))
+    orc.set_weights(w)
+    w0 = orc.get_weights()
+    x = rng.uniform(-1, 1, (batch, x_size)).astype(np.float32)
+    d = (0.05 * rng.standard_normal((batch, d_size))).astype(np.float32)
+    xg, dg = cuda(x), cuda(d)
+    dwg, dwo = [], []
+    for s in range(N_SEEDS):
+        gpu = tiles.CudaAnalogTile(host)
+        gpu.set_seed(77 + s)
+        gpu.set_learning_rate(0.01)
+        gpu.update(xg, dg, False, False, False, False)
+        dwg.append(gpu.get_weights().numpy() - w0)
+        orc.set_weights(w)
+        orc.set_seed(1 + s)
+        orc.set_learning_rate(0.01)
+        orc.update(x, d)
+        dwo.append(orc.get_weights() - w0)
+    dwg, dwo = np.stack(dwg), np.stack(dwo)
+    assert np.abs(dwo).mean() > 5e-4
+    compare_moments(dwg, dwo, f"weight change {device} um={um}")
+    # the mean step follows -lr * d^T x (scaled by the device's own step sizes): strongly correlated with it
+    sgd = -(d.T @ x)
+    assert np.corrcoef(dwg.mean(0).ravel(), sgd.ravel())[0, 1] > 0.9
+
+
+def test_full_size_update_noise_free_matches_oracle_through_the_pulse_words(gpu_device):
+    """Benchmark configuration 2 at full size, cycle-to-cycle noise off: the GPU's pulse words drive the
+    oracle's device model to the same 1M weights (1e-5)."""
+    meta, dev = config2(ctoc=False)
+    host, orc, _ = build_pair(meta, dev, 1024, 1024, gpu=False)
+    w, x, d = config2_data()
+    host.set_weights(torch.from_numpy(w))
+    orc.set_weights(w)
+    gpu = tiles.CudaAnalogTile(host)
+    gpu.set_seed(3)
+    gpu.set_learning_rate(0.01)
+    orc.set_learning_rate(0.01)
+    gpu.update(cuda(x), cuda(d), False, False, False, False)
+    xw, dw, bl = (t.numpy() for t in gpu.get_update_words(256))
+    assert np.array_equal(bl, orc.update_bl_ab(x, d)[0])
+    orc.update_with_words(xw, dw, bl)
+    wg = gpu.get_weights().numpy()
+    assert np.abs(wg - orc.get_weights()).max() <= 1e-5
+    # expected number of coincidences per cross-point and call: lr * E|x| * E|d| * B / dw_min = 51 (+- statistics)
+    pulses_x = np.zeros((256, 1024), np.int64)
+    xs = (xw.astype(np.int64) & 0xFFFFFFFF) >> 1
+    ds = (dw.astype(np.int64) & 0xFFFFFFFF) >> 1
+    coinc = 0.0
+    for k in range(31):
+        coinc += (((xs >> k) & 1).sum(1) * ((ds >> k) & 1).sum(1)).sum()
+    del pulses_x
+    assert coinc / (1024 * 1024) == pytest.approx(0.01 * np.abs(x).mean() * np.abs(d).mean() * 256 / 0.001, rel=0.05)
+
+
+def test_full_size_update_cycle_noise_is_zero_mean_with_the_expected_spread(gpu_device):
+    """Same call with cycle-to-cycle noise on (std 0.3): against the noise-free result for the *same* pulse
+    words the difference must be zero-mean, and its variance must be the sum over the applied pulses of
+    (0.3 * step)^2 with step = scale * (1 - w / bound), evaluated at the start weights (+- 10 %)."""
+    meta, dev = config2(ctoc=True)
+    meta0, dev0 = config2(ctoc=False)
+    host, _, _ = build_pair(meta, dev, 1024, 1024, gpu=False)
+    _, orc0, _ = build_pair(meta0, dev0, 1024, 1024, gpu=False)
+    w, x, d = config2_data()
+    host.set_weights(torch.from_numpy(w))
+    orc0.set_weights(w)
+    w0 = orc0.get_weights()
+    gpu = tiles.CudaAnalogTile(host)
+    gpu.set_seed(11)
+    gpu.set_learning_rate(0.01)
+    orc0.set_learning_rate(0.01)
+    gpu.update(cuda(x), cuda(d), False, False, False, False)
+    xw, dw, bl = (t.numpy() for t in gpu.get_update_words(256))
+    orc0.update_with_words(xw, dw, bl)
+    e = (gpu.get_weights().numpy() - orc0.get_weights()).astype(np.float64)
+    hid = orc0.get_hidden().astype(np.float64)
+    w_max, w_min, up, down = hid[0], hid[1], hid[2], hid[3]
+    # up / down pulse counts per cross-point from the words
+    xs = xw.astype(np.int64) & 0xFFFFFFFF
+    ds = dw.astype(np.int64) & 0xFFFFFFFF
+    n_up = np.zeros((1024, 1024))
+    n_down = np.zeros((1024, 1024))
+    for b in range(256):
+        xb, db = xs[b], ds[b]
+        sx, sd = (xb & 1), (db & 1)
+        cnt = np.zeros((1024, 1024))
+        for k in range(1, int(bl[b]) + 1):
+            cnt += np.outer((db >> k) & 1, (xb >> k) & 1)
+        same = np.equal.outer(sd, sx)
+        n_down += np.where(same, cnt, 0)
+        n_up += np.where(same, 0, cnt)
+    step_up = up * (1 - w0 / w_max)
+    step_down = down * (1 - w0 / w_min)
+    var_pred = 0.09 * (n_up * step_up**2 + n_down * step_down**2)
+    inner = (w0 > w_min + 0.05) & (w0 < w_max - 0.05) & (var_pred > 0)
+    assert inner.mean() > 0.7
+    assert abs(e[inner].mean()) < 4 * e[inner].std() / np.sqrt(inner.sum())
+    assert e[inner].var() == pytest.approx(var_pred[inner].mean(), rel=0.1)
+    zz = e[inner] / np.sqrt(var_pred[inner])
+    assert zz.std() == pytest.approx(1.0, rel=0.1)
+    assert np.mean(np.abs(zz) > 3) < 0.01
