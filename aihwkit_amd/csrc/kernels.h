@@ -93,6 +93,14 @@ struct UpdateArgs {
   float *prob_b; // [B] probability scale of x
   uint32_t *x_words; // [B][X] packed pulse words
   uint32_t *d_words; // [B][D]
+  // sample-transposed pulse bits: plane (chunk c, slot k) of line element e is the 32-bit word whose bit q
+  // is pulse slot k of sample 32 c + q; element (c, k, e) at planes[(c * plane_slots + k) * size + e]
+  uint32_t *x_planes;
+  uint32_t *d_planes;
+  int plane_slots; // slots per chunk the plane buffers are laid out for
+  int n_chunks;    // ceil(m_batch / 32)
+  int *kmax;       // kmax[0..1]: largest BL of a batch (ping-pong by call), kmax[2]: constant 31
+  int kmax_slot;   // which entry this call uses
   float *x_val;  // [B][X] implicit line values
   float *d_val;  // [B][D]
   PhiloxKey key;
@@ -102,6 +110,7 @@ struct UpdateArgs {
 void launch_update_prepare(const UpdateArgs &a, hipStream_t s);       // BL, A, B per sample
 void launch_update_bitlines(const UpdateArgs &a, hipStream_t s);      // stochastic pulse words
 void launch_update_implicit_lines(const UpdateArgs &a, hipStream_t s); // deterministic line values
+void launch_update_planes(const UpdateArgs &a, hipStream_t s);        // pulse words -> sample-transposed bit planes
 void launch_update_pulsed(const UpdateArgs &a, hipStream_t s);        // coincidences + device steps
 void launch_update_implicit(const UpdateArgs &a, hipStream_t s);
 void launch_implicit_counts(const UpdateArgs &a, int32_t *counts, hipStream_t s);

@@ -100,6 +100,11 @@ __global__ __launch_bounds__(256) void k_update_prepare(UpdateArgs a) {
   // one 32-bit word holds the sign and at most 31 pulses
   if (BL > 31) BL = 31;
   a.bl[b] = BL;
+  // largest BL of the batch: this call's slot was zeroed by the previous call, which used the other one
+  if (a.kmax) {
+    if (BL > 0) atomicMax(&a.kmax[a.kmax_slot], BL);
+    if (b == 0) a.kmax[a.kmax_slot ^ 1] = 0;
+  }
   a.prob_a[b] = A;
   a.prob_b[b] = B;
 }
@@ -226,6 +231,35 @@ __device__ __forceinline__ float device_step(float w, int sign_down, const CellP
   return w;
 }
 
+// one device pulse with the normal already drawn
+template <int KIND, bool MULT>
+__device__ __forceinline__ float device_step_g(float w, int sign_down, const CellParams &c, float std_, float g) {
+  if (KIND == RPU_DEVICE_CONSTANT_STEP) {
+    if (std_ > 0.0f) {
+      const float f = 1.0f + std_ * g;
+      if (sign_down) w -= f * c.scale_down;
+      else w += f * c.scale_up;
+    } else {
+      if (sign_down) w -= c.scale_down;
+      else w += c.scale_up;
+    }
+    w = fminf(w, c.w_max);
+    w = fmaxf(w, c.w_min);
+  } else {
+    const float f = (std_ > 0.0f) ? 1.0f + std_ * g : 1.0f;
+    if (MULT) {
+      if (sign_down) w -= (c.slope_down * w + c.scale_down) * f;
+      else w += (c.slope_up * w + c.scale_up) * f;
+    } else {
+      if (sign_down) w -= c.slope_down * w + c.scale_down * f;
+      else w += c.slope_up * w + c.scale_up * f;
+    }
+    w = fmaxf(w, c.w_min);
+    w = fminf(w, c.w_max);
+  }
+  return w;
+}
+
 template <int KIND>
 __device__ __forceinline__ CellParams load_cell(const DeviceDev &d, long k) {
   CellParams c;
@@ -243,35 +277,148 @@ __device__ __forceinline__ CellParams load_cell(const DeviceDev &d, long k) {
   return c;
 }
 
-// grid: x = ceil(x_size / 256), y = d_size.  One thread per cross-point, samples in batch order.
+// Pulse words -> bit planes.  One wave per (line element, block of 64 samples): lane q holds the word of
+// sample 64 sb + q, a 64-bit ballot per pulse slot is the plane word of two 32-sample chunks.
+__global__ __launch_bounds__(256) void k_update_planes(UpdateArgs a) {
+  const int lane = threadIdx.x & 63;
+  const int e = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int sb = blockIdx.y;
+  const int total = a.x_size + a.d_size;
+  if (e >= total) return;
+  const bool is_x = e < a.x_size;
+  const int el = is_x ? e : e - a.x_size;
+  const int size = is_x ? a.x_size : a.d_size;
+  const uint32_t *words = is_x ? a.x_words : a.d_words;
+  uint32_t *planes = is_x ? a.x_planes : a.d_planes;
+  const int b = sb * 64 + lane;
+  const uint32_t word = (b < a.m_batch) ? words[(long)b * size + el] : 0u;
+  const int kmax = a.kmax[a.kmax_slot];
+  const int c0 = 2 * sb;
+  for (int k = 0; k < kmax; ++k) {
+    const unsigned long long m = __ballot((word >> (k + 1)) & 1u);
+    if (lane == 0) {
+      planes[((long)c0 * a.plane_slots + k) * size + el] = (uint32_t)m;
+      if (c0 + 1 < a.n_chunks) planes[((long)(c0 + 1) * a.plane_slots + k) * size + el] = (uint32_t)(m >> 32);
+    }
+  }
+}
+
+// grid: x = ceil(x_size / 256), y = d_size.  One thread per cross-point; a wave covers 64 consecutive x of
+// one d row.  The batch is walked in blocks of 128 samples.  For a block every lane first builds the 128-bit
+// set of samples in which its cross-point has a coincidence: OR over the pulse slots of
+// (x_plane & d_plane), with the d planes wave-uniform and the x planes read with unit stride.  Then every
+// lane walks its own set in batch order; the count and direction of an event come from the two packed
+// words of that sample.  The wave loop applies at most one pulse per lane and pass and ends when the lane
+// with the most pulses is done; the eight noise factors of eight passes come from one Philox call per
+// lane, keyed by (cross-point, refill index).
 template <int KIND, bool MULT>
 __global__ __launch_bounds__(256) void k_update_pulsed(UpdateArgs a) {
   const int i = blockIdx.y;
-  const int j = blockIdx.x * blockDim.x + threadIdx.x;
-  if (j >= a.x_size) return;
-  const long k = (long)i * a.x_size + j;
-  const CellParams c = load_cell<KIND>(a.dev, k);
-  float w = a.w[k];
-  CtocStream rng;
-  rng.left = 0;
-  rng.refill = 0;
-  rng.cell = (uint32_t)k;
-  rng.n0 = rng.n1 = rng.n2 = rng.n3 = 0.0f;
+  const int jt = blockIdx.x * blockDim.x + threadIdx.x;
+  const bool valid = jt < a.x_size;
+  const int j = valid ? jt : a.x_size - 1;
+  const unsigned cell = (unsigned)i * (unsigned)a.x_size + (unsigned)j;
+  const CellParams cp = load_cell<KIND>(a.dev, cell);
+  float w = a.w[cell];
   const float std_ = a.dev.dw_min_std;
   const uint32_t lr_neg = a.lr < 0.0f ? 1u : 0u;
-  const uint32_t *dwp = a.d_words + i;
+  const int kmax = a.kmax[a.kmax_slot];
+  const int n_chunks = a.n_chunks;
+  const uint32_t *xpl = a.x_planes + j;
+  const uint32_t *dpl = a.d_planes + i;
   const uint32_t *xwp = a.x_words + j;
-  for (int b = 0; b < a.m_batch; ++b) {
-    const uint32_t dw = dwp[(long)b * a.d_size]; // wave-uniform
-    if ((dw >> 1) == 0) continue;
-    const uint32_t xw = xwp[(long)b * a.x_size];
-    int n = __popc(xw & dw & ~1u);
-    if (n == 0) continue;
-    // sign > 0 (step down) when x and d have the same sign and lr > 0
-    const int sign_down = (((xw ^ dw) & 1u) ^ lr_neg) == 0u;
-    for (; n > 0; --n) w = device_step<KIND, MULT>(w, sign_down, c, std_, rng, a.key, a.call);
+  const uint32_t *dwp = a.d_words + i;
+  const unsigned xs = (unsigned)a.x_size, ds = (unsigned)a.d_size;
+  const int slots = a.plane_slots;
+
+  uint32_t refill = 0;
+  for (int c0 = 0; c0 < n_chunks; c0 += 4) {
+    // event sets of the next 128 samples
+    uint32_t ev[4];
+#pragma unroll
+    for (int cc = 0; cc < 4; ++cc) {
+      const int c = c0 + cc;
+      uint32_t e = 0u;
+      if (c < n_chunks) {
+        const unsigned base = (unsigned)c * (unsigned)slots;
+        for (int k = 0; k < kmax; ++k) {
+          const uint32_t dk = dpl[(base + k) * ds]; // wave-uniform
+          if (dk) e |= dk & xpl[(base + k) * xs];
+        }
+      }
+      ev[cc] = valid ? e : 0u;
+    }
+    unsigned long long cur = ((unsigned long long)ev[1] << 32) | ev[0];
+    unsigned long long nxt = ((unsigned long long)ev[3] << 32) | ev[2];
+    unsigned sample0 = (unsigned)c0 * 32u; // sample index of bit 0 of cur
+    int left = 0;                          // pulses left in the current event
+    // parameters of the current event's direction
+    float slope = 0.0f, scale = 0.0f;
+    uint32_t flip = 0u; // sign bit to apply to the step: down = subtract
+    bool block_done = !__any((cur | nxt) != 0ull);
+    while (!block_done) {
+      float f[8];
+      if (std_ > 0.0f) {
+        float g[8];
+        philox_normal8(cell, refill, a.call, RNG_CTOC, a.key, g);
+#pragma unroll
+        for (int q = 0; q < 8; ++q) f[q] = 1.0f + std_ * g[q];
+      } else {
+#pragma unroll
+        for (int q = 0; q < 8; ++q) f[q] = 1.0f;
+      }
+      ++refill;
+#pragma unroll
+      for (int q = 0; q < 8; ++q) {
+        if (left == 0) {
+          if (cur == 0ull) {
+            cur = nxt;
+            nxt = 0ull;
+            sample0 += 64u;
+          }
+          if (cur != 0ull) {
+            const int bit = __ffsll((long long)cur) - 1;
+            cur &= cur - 1ull;
+            const unsigned b = sample0 + (unsigned)bit;
+            const uint32_t xw = xwp[__umul24(b, xs)];
+            const uint32_t dw = dwp[__umul24(b, ds)];
+            left = __popc(xw & dw & ~1u);
+            // step down when x and d have the same sign and lr > 0
+            const bool down = (((xw ^ dw) & 1u) ^ lr_neg) == 0u;
+            slope = down ? cp.slope_down : cp.slope_up;
+            scale = down ? cp.scale_down : cp.scale_up;
+            flip = down ? 0x80000000u : 0u;
+          }
+        }
+        if (!__any(left > 0)) {
+          block_done = true;
+          break;
+        }
+        if (left > 0) {
+          // one pulse: ConstantStep  w +- scale * f ; LinearStep  w +- (slope * w + scale) * f  (mult noise)
+          // or w +- (slope * w + scale * f) (additive noise); "-" as the addition of the negated step
+          float step;
+          if (KIND == RPU_DEVICE_CONSTANT_STEP) {
+            step = (std_ > 0.0f) ? f[q] * scale : scale;
+          } else if (MULT) {
+            step = (slope * w + scale) * f[q];
+          } else {
+            step = slope * w + scale * f[q];
+          }
+          w = w + __uint_as_float(__float_as_uint(step) ^ flip);
+          if (KIND == RPU_DEVICE_CONSTANT_STEP) {
+            w = fminf(w, cp.w_max);
+            w = fmaxf(w, cp.w_min);
+          } else {
+            w = fmaxf(w, cp.w_min);
+            w = fminf(w, cp.w_max);
+          }
+          --left;
+        }
+      }
+    }
   }
-  a.w[k] = w;
+  if (valid) a.w[cell] = w;
 }
 
 // deterministic implicit: n = (int) rintf((dv * BL) * xv) per sample (dense_bit_line_maker.cpp:237-264),
@@ -362,6 +509,11 @@ void launch_update_implicit_lines(const UpdateArgs &a, hipStream_t s) {
       hipLaunchKernelGGL((KERNEL<RPU_DEVICE_LINEAR_STEP, false>), grid, dim3(256), 0, s, a);        \
     }                                                                                               \
   } while (0)
+
+void launch_update_planes(const UpdateArgs &a, hipStream_t s) {
+  dim3 grid((a.x_size + a.d_size + 3) / 4, (a.m_batch + 63) / 64);
+  hipLaunchKernelGGL(k_update_planes, grid, dim3(256), 0, s, a);
+}
 
 void launch_update_pulsed(const UpdateArgs &a, hipStream_t s) {
   dim3 grid((a.x_size + 255) / 256, a.d_size);

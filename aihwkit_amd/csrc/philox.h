@@ -23,21 +23,16 @@ struct Philox4 {
   uint32_t v[4];
 };
 
-RPU_HD uint32_t philox_mulhi(uint32_t a, uint32_t b) {
-#if defined(__HIP_DEVICE_COMPILE__)
-  return __umulhi(a, b);
-#else
-  return (uint32_t)(((uint64_t)a * (uint64_t)b) >> 32);
-#endif
-}
-
 RPU_HD Philox4 philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint32_t k0,
                              uint32_t k1) {
   const uint32_t M0 = 0xD2511F53u, M1 = 0xCD9E8D57u, W0 = 0x9E3779B9u, W1 = 0xBB67AE85u;
 #pragma unroll
   for (int r = 0; r < 10; ++r) {
-    const uint32_t hi0 = philox_mulhi(M0, c0), lo0 = M0 * c0;
-    const uint32_t hi1 = philox_mulhi(M1, c2), lo1 = M1 * c2;
+    // one 32 x 32 -> 64 bit product per multiplier (v_mad_u64_u32 on gfx950)
+    const uint64_t p0 = (uint64_t)M0 * (uint64_t)c0;
+    const uint64_t p1 = (uint64_t)M1 * (uint64_t)c2;
+    const uint32_t hi0 = (uint32_t)(p0 >> 32), lo0 = (uint32_t)p0;
+    const uint32_t hi1 = (uint32_t)(p1 >> 32), lo1 = (uint32_t)p1;
     const uint32_t n0 = hi1 ^ c1 ^ k0;
     const uint32_t n2 = hi0 ^ c3 ^ k1;
     c0 = n0;
@@ -81,6 +76,29 @@ __device__ __forceinline__ void box_muller(uint32_t r0, uint32_t r1, float &n0, 
   __sincosf(6.283185307179586f * t, &s, &c);
   n0 = rad * c;
   n1 = rad * s;
+}
+
+// Box-Muller on one 32-bit word: radius from the high 16 bits (mid-point rule, so the discrete
+// radius distribution keeps E[r^2] = 2 to O(2^-32)), angle from the low 16 bits.  Two N(0,1) whose
+// resolution (2^-16 of the radius range, 2^16 angles) is finer than the fp32 rounding of a weight update
+// that adds step * (1 + std * n) to a weight; |n| <= 4.9.
+__device__ __forceinline__ void box_muller16(uint32_t r, float &n0, float &n1) {
+  const float u = ((float)(r >> 16) + 0.5f) * (1.0f / 65536.0f);
+  const float t = (float)(r & 0xffffu) * (1.0f / 65536.0f); // turns
+  // -2 ln(u) = -2 ln(2) log2(u)
+  const float rad = __builtin_amdgcn_sqrtf(-1.3862943611198906f * __builtin_amdgcn_logf(u));
+  n0 = rad * __builtin_amdgcn_cosf(t);
+  n1 = rad * __builtin_amdgcn_sinf(t);
+}
+
+// eight N(0,1) from one Philox call
+__device__ __forceinline__ void philox_normal8(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3,
+                                               PhiloxKey key, float out[8]) {
+  const Philox4 r = philox4x32_10(c0, c1, c2, c3, key.k0, key.k1);
+  box_muller16(r.v[0], out[0], out[1]);
+  box_muller16(r.v[1], out[2], out[3]);
+  box_muller16(r.v[2], out[4], out[5]);
+  box_muller16(r.v[3], out[6], out[7]);
 }
 
 __device__ __forceinline__ void philox_normal4(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3,

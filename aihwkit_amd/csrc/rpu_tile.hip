@@ -97,7 +97,9 @@ struct Tile {
   // update scratch
   DevBuf<int> u_bl;
   DevBuf<float> u_a, u_b, u_xval, u_dval;
-  DevBuf<uint32_t> u_xw, u_dw;
+  DevBuf<uint32_t> u_xw, u_dw, u_xpl, u_dpl;
+  DevBuf<int> u_kmax;
+  uint32_t update_calls = 0;
   int last_update_batch = 0;
   int last_update_pulse = -1;
   int last_forward_batch = 0;
@@ -146,6 +148,7 @@ struct Tile {
     s_nm.release(); s_nmnp.release(); s_red.release(); s_scale.release(); s_fin.release(); s_bias.release();
     s_rounds.release(); s_hitup.release(); s_hitlo.release(); s_list0.release(); s_list1.release(); s_count.release();
     u_bl.release(); u_a.release(); u_b.release(); u_xval.release(); u_dval.release(); u_xw.release(); u_dw.release();
+    u_xpl.release(); u_dpl.release(); u_kmax.release();
   }
 
   PhiloxKey key() const {
@@ -292,6 +295,20 @@ struct Tile {
     if (!transposed) last_forward_batch = B;
   }
 
+  void set_plane_args(UpdateArgs &a, int B) {
+    const int slots = 31;
+    const int chunks = (B + 31) / 32;
+    u_xpl.ensure((size_t)chunks * slots * X);
+    u_dpl.ensure((size_t)chunks * slots * D);
+    if (!u_kmax.p) {
+      u_kmax.ensure(4);
+      const int init[4] = {0, 0, 31, 0};
+      RPU_HIP_CHECK(hipMemcpy(u_kmax.p, init, sizeof(init), hipMemcpyHostToDevice));
+    }
+    a.x_planes = u_xpl.p; a.d_planes = u_dpl.p; a.plane_slots = slots; a.n_chunks = chunks;
+    a.kmax = u_kmax.p;
+  }
+
   // device steps for pulse words made elsewhere (the reference's updateVectorWithCounts debug protocol)
   void update_with_words(const uint32_t *x_words, const uint32_t *d_words, int B, hipStream_t s) {
     if (lr == 0.0f) return;
@@ -304,7 +321,11 @@ struct Tile {
     a.dev.slope_up = d_slup.p; a.dev.slope_down = d_sldown.p;
     a.x_words = const_cast<uint32_t *>(x_words); a.d_words = const_cast<uint32_t *>(d_words);
     a.key = key(); a.call = call++;
+    set_plane_args(a, B);
+    a.kmax_slot = 2; // words from outside: all 31 slots may be in use
     prof_begin(s);
+    launch_update_planes(a, s);
+    prof_mark(s, "update_planes");
     launch_update_pulsed(a, s);
     prof_mark(s, "update_pulsed");
     RPU_HIP_CHECK(hipGetLastError());
@@ -361,6 +382,8 @@ struct Tile {
     if (up.p.pulse_type == RPU_PULSE_STOCHASTIC_COMPRESSED) {
       u_xw.ensure((size_t)B * X); u_dw.ensure((size_t)B * D);
       a.x_words = u_xw.p; a.d_words = u_dw.p;
+      set_plane_args(a, B);
+      a.kmax_slot = (int)(update_calls++ & 1u);
     } else {
       u_xval.ensure((size_t)B * X); u_dval.ensure((size_t)B * D);
       a.x_val = u_xval.p; a.d_val = u_dval.p;
@@ -371,6 +394,8 @@ struct Tile {
     if (up.p.pulse_type == RPU_PULSE_STOCHASTIC_COMPRESSED) {
       launch_update_bitlines(a, s);
       prof_mark(s, "update_bitlines");
+      launch_update_planes(a, s);
+      prof_mark(s, "update_planes");
       launch_update_pulsed(a, s);
       prof_mark(s, "update_pulsed");
     } else {
