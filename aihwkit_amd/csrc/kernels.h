@@ -40,6 +40,8 @@ struct MvmArgs {
   long out_sb, out_so; // output element (b, o) at out[b * out_sb + o * out_so]
   int m_batch;
   int K, O;       // contraction length and number of outputs
+  int k_pad;      // K rounded up to the step of the contraction kernel (mvm_k_pad)
+  float *xq[2];   // ping-pong scratch [samples of the round][k_pad]: DAC-quantized inputs, zero padded
   int transposed; // 0: out[o] = sum_k W[o][k] in[k] (forward); 1: out[o] = sum_k W[k][o] in[k] (backward)
   int round;      // bound-management round, 0-based
   float alpha, beta; // only used when io.perfect: out = alpha * acc + beta * out
@@ -57,6 +59,8 @@ void launch_mvm_round(const MvmArgs &a, hipStream_t s);
 void launch_mvm_advance(const MvmArgs &a, hipStream_t s);
 // number of rounds that can ever be needed with these IO settings
 int mvm_max_rounds(const IoDev &io);
+// row length of the quantized-input scratch for a contraction length K
+int mvm_k_pad(int K);
 
 // [B][X-1] (or [X-1][B]) -> [B][X] with a trailing column of ones (always batch-first output)
 void launch_make_bias(const float *in, float *out, int m_batch, int x_size, int in_trans, hipStream_t s);

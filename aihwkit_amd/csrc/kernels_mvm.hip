@@ -6,13 +6,19 @@
 // Iterative bound management re-runs only the samples whose ADC saturated, with a halved input
 // range, through per-sample state kept in HBM; the host never waits for a round.
 //
-// Work decomposition of a round: one workgroup (4 waves) owns a 32 (outputs) x 32 (samples) tile of
-// the result.  The 4 waves split the contraction length K in four contiguous quarters, each wave
-// runs v_mfma_f32_32x32x2_f32 over its quarter straight from global memory (operands are read as
-// one float4 per lane and 8 k-values, quantized in registers), the four partial tiles are summed in
-// a fixed order through LDS and each wave finishes 8 output rows: noise, quantize, clip, bound
-// bookkeeping, rescale, store.  A 1024 x 1024 tile at batch 256 gives 256 workgroups = 1024 waves,
-// one per SIMD of the chip.
+// Kernels of a call:
+//   k_mvm_init     one workgroup per sample: noise-management scale, per-sample state of round 0 and the
+//                  DAC-quantized input row, written k-contiguous and zero padded into a scratch matrix.
+//   k_mvm_round    the contraction + ADC epilogue.  One workgroup (4 waves) owns a 32 (outputs) x 32
+//                  (samples) tile; the 4 waves split the contraction length in four contiguous parts, each
+//                  runs v_mfma_f32_32x32x2_f32 over its part with both operands read straight from global
+//                  memory one full 128-byte line per row and step (16 k-values per half-wave), the four
+//                  partial tiles are summed in a fixed order through LDS and each wave finishes 8 output
+//                  rows: noise, quantize, clip, bound bookkeeping, rescale, store.  Workgroups are numbered
+//                  so that the 8 XCDs each work on a contiguous band of output rows (own L2 slice of W).
+//   k_mvm_advance  after a round, one workgroup per sample of that round: decide whether the sample needs
+//                  another round and, if so, append it to the next round's list and re-quantize its row
+//                  with the halved input range into the other scratch matrix.
 #include "kernels.h"
 
 namespace rpu_amd {
@@ -23,6 +29,7 @@ namespace {
 
 constexpr int TILE = 32;
 constexpr int WAVES = 4;
+constexpr int KSTEP = 32; // k-values per wave step: 128 bytes per operand row
 
 __device__ __forceinline__ float dac_value(float x, float scale, const IoDev &io, PhiloxKey key,
                                            uint32_t call, int round, int b, int k) {
@@ -49,15 +56,44 @@ __device__ __forceinline__ float dac_value(float x, float scale, const IoDev &io
   return v;
 }
 
+// quantized copy of sample b's input row into row `slot` of a scratch matrix (whole workgroup)
+__device__ __forceinline__ void write_dac_row(const MvmArgs &a, int b, int slot, float scale, int round, float *dst) {
+  const float *row = a.in + (long)b * a.in_sb;
+  float *out = dst + (long)slot * a.k_pad;
+  for (int k = threadIdx.x; k < a.k_pad; k += blockDim.x) {
+    float v = 0.0f;
+    if (k < a.K) {
+      v = row[(long)k * a.in_sk];
+      if (!a.io.perfect) v = dac_value(v, scale, a.io, a.key, a.call, round, b, k);
+    }
+    out[k] = v;
+  }
+}
+
+// PD = number of contraction steps whose operand loads are in flight per wave (prefetch depth); the scratch
+// row length k_pad is a multiple of KSTEP * WAVES * PD so every wave runs whole groups of PD steps.
+// WMODE = how the weight operand is addressed:
+//   0  contraction index contiguous (forward), rows 16-byte aligned, K a multiple of 16: float4 loads
+//   1  output index contiguous (backward): scalar loads, 32 consecutive outputs per half-wave and k
+//   2  any strides, every element guarded
+// Modes 0 and 1 load without predicates: out-of-range rows / k are clamped to valid addresses, their
+// products are either multiplied by the zero padding of the quantized inputs or never stored.
+template <int PD, int WMODE>
 __global__ __launch_bounds__(256) void k_mvm_round(MvmArgs a) {
   __shared__ float red[WAVES][16][64];
 
   const int n_act = (a.round > 0) ? a.st.count[a.round] : a.m_batch;
-  const int tile_b = blockIdx.y;
-  if (tile_b * TILE >= n_act) {
+  // workgroup n runs on XCD n % 8; XCD x owns the output-row tiles [x * per, (x + 1) * per)
+  const int tiles_o = (a.O + TILE - 1) / TILE;
+  const int per = (tiles_o + 7) / 8;
+  const int n = blockIdx.x;
+  const int xcd = n & 7;
+  const int m = n >> 3;
+  const int tile_o = xcd * per + (m % per);
+  const int tile_b = m / per;
+  if (tile_o >= tiles_o || tile_b * TILE >= n_act) {
     return; // whole workgroup leaves: no barrier is reached by anyone
   }
-  const int tile_o = blockIdx.x;
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int r = lane & 31;
@@ -68,80 +104,67 @@ __global__ __launch_bounds__(256) void k_mvm_round(MvmArgs a) {
   const bool o_ok = o_in < a.O;
   const int slot_in = tile_b * TILE + r;
   const bool b_ok = slot_in < n_act;
-  int b_in = 0;
-  if (b_ok) {
-    b_in = (a.round > 0) ? a.st.list[a.round & 1][slot_in] : slot_in;
-  }
-  const float scale_in = (b_ok && !a.io.perfect) ? a.st.scale[b_in] : 1.0f;
 
   const long w_so = a.transposed ? 1 : a.x_size;
   const long w_sk = a.transposed ? a.x_size : 1;
-  const float *w_row = a.w + (long)(o_ok ? o_in : 0) * w_so;
-  const float *in_row = a.in + (long)b_in * a.in_sb;
+  const int o_clamped = o_ok ? o_in : a.O - 1;
+  const float *w_row = a.w + (long)o_clamped * w_so;
+  const float *x_row = a.xq[a.round & 1] + (long)(b_ok ? slot_in : n_act - 1) * a.k_pad;
 
   const int K = a.K;
-  const int kq = ((K + 31) / 32) * 8; // per-wave share, a multiple of 8
-  const int k_begin = wave * kq;
-  const int k_end = min(K, k_begin + kq);
-
-  const bool full8 = (K % 8) == 0;
-  const bool vec_w = full8 && (w_sk == 1) && ((a.x_size & 3) == 0) && ((((uintptr_t)a.w) & 15) == 0);
-  const bool vec_in = full8 && (a.in_sk == 1) && ((a.in_sb & 3) == 0) && ((((uintptr_t)a.in) & 15) == 0);
-  const bool plain_dac = a.io.perfect || (!a.io.inp_sto_round && !(a.io.inp_noise > 0.0f) && a.io.inp_asym == 0.0f);
-  const float inp_res = a.io.inp_res;
-  const float inp_bound = a.io.inp_bound;
+  const int per_wave = a.k_pad / (KSTEP * WAVES); // a multiple of PD
+  const int s_begin = wave * per_wave;
+  const int s_end = s_begin + per_wave;
 
   floatx16 acc;
 #pragma unroll
   for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
 
-#pragma unroll 2
-  for (int k = k_begin; k < k_end; k += 8) {
-    const int kk = k + h * 4;
-    float wv[4], xv[4];
-    if (vec_w) {
-      const float4 t = o_ok ? *reinterpret_cast<const float4 *>(w_row + kk) : make_float4(0.f, 0.f, 0.f, 0.f);
-      wv[0] = t.x; wv[1] = t.y; wv[2] = t.z; wv[3] = t.w;
+  auto load_step = [&](int s, float (&wd)[16], float (&xd)[16]) {
+    const int k0 = s * KSTEP + h * 16;
+#pragma unroll
+    for (int v4 = 0; v4 < 4; ++v4) {
+      const float4 t = *reinterpret_cast<const float4 *>(x_row + k0 + v4 * 4);
+      xd[v4 * 4 + 0] = t.x; xd[v4 * 4 + 1] = t.y; xd[v4 * 4 + 2] = t.z; xd[v4 * 4 + 3] = t.w;
+    }
+    if (WMODE == 0) {
+      const int kc = min(k0, K - 16); // K % 16 == 0: a group is either whole or entirely zero padding
+#pragma unroll
+      for (int v4 = 0; v4 < 4; ++v4) {
+        const float4 t = *reinterpret_cast<const float4 *>(w_row + kc + v4 * 4);
+        wd[v4 * 4 + 0] = t.x; wd[v4 * 4 + 1] = t.y; wd[v4 * 4 + 2] = t.z; wd[v4 * 4 + 3] = t.w;
+      }
+    } else if (WMODE == 1) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int kc = min(k0 + i, K - 1);
+        wd[i] = w_row[(long)kc * w_sk];
+      }
     } else {
 #pragma unroll
-      for (int m = 0; m < 4; ++m) {
-        wv[m] = (o_ok && (kk + m) < k_end) ? w_row[(long)(kk + m) * w_sk] : 0.0f;
+      for (int i = 0; i < 16; ++i) {
+        wd[i] = (o_ok && (k0 + i) < K) ? a.w[(long)o_in * w_so + (long)(k0 + i) * w_sk] : 0.0f;
       }
     }
-    if (vec_in) {
-      const float4 t = b_ok ? *reinterpret_cast<const float4 *>(in_row + kk) : make_float4(0.f, 0.f, 0.f, 0.f);
-      xv[0] = t.x; xv[1] = t.y; xv[2] = t.z; xv[3] = t.w;
-    } else {
+  };
+
+  // steps s_begin .. s_end-1 in groups of PD; the loads of the next PD steps are always in flight
+  float wb[PD][16], xb[PD][16];
 #pragma unroll
-      for (int m = 0; m < 4; ++m) {
-        xv[m] = (b_ok && (kk + m) < k_end) ? in_row[(long)(kk + m) * a.in_sk] : 0.0f;
+  for (int p = 0; p < PD; ++p) load_step(s_begin + p, wb[p], xb[p]);
+  for (int s = s_begin; s < s_end; s += PD) {
+#pragma unroll
+    for (int p = 0; p < PD; ++p) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(wb[p][i], xb[p][i], acc, 0, 0, 0);
       }
-    }
-    if (!a.io.perfect) {
-      if (plain_dac) {
-#pragma unroll
-        for (int m = 0; m < 4; ++m) {
-          float v = xv[m] * scale_in;
-          if (inp_res > 0.0f) v = rintf(v / inp_res) * inp_res;
-          v = (v > inp_bound) ? inp_bound : v;
-          v = (v < -inp_bound) ? -inp_bound : v;
-          xv[m] = v;
-        }
-      } else {
-#pragma unroll
-        for (int m = 0; m < 4; ++m) {
-          const bool ok = b_ok && (kk + m) < k_end;
-          xv[m] = ok ? dac_value(xv[m], scale_in, a.io, a.key, a.call, a.round, b_in, kk + m) : 0.0f;
-        }
-      }
-    }
-#pragma unroll
-    for (int m = 0; m < 4; ++m) {
-      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(wv[m], xv[m], acc, 0, 0, 0);
+      // refill this buffer with the step PD ahead; past the end the last step is re-read and never used
+      load_step(min(s + PD + p, s_end - 1), wb[p], xb[p]);
     }
   }
 
-  // sum the four K-quarters in a fixed order
+  // sum the four parts of the contraction in a fixed order
 #pragma unroll
   for (int i = 0; i < 16; ++i) red[wave][i][lane] = acc[i];
   __syncthreads();
@@ -149,23 +172,23 @@ __global__ __launch_bounds__(256) void k_mvm_round(MvmArgs a) {
   // this wave finishes accumulator group `wave`: rows wave*8 + h*4 + m, column r
   float v[4];
 #pragma unroll
-  for (int m = 0; m < 4; ++m) {
-    const int i = wave * 4 + m;
-    v[m] = ((red[0][i][lane] + red[1][i][lane]) + red[2][i][lane]) + red[3][i][lane];
+  for (int q = 0; q < 4; ++q) {
+    const int i = wave * 4 + q;
+    v[q] = ((red[0][i][lane] + red[1][i][lane]) + red[2][i][lane]) + red[3][i][lane];
   }
   if (!b_ok) return;
-  const int b = b_in;
+  const int b = (a.round > 0) ? a.st.list[a.round & 1][slot_in] : slot_in;
   const int o0 = tile_o * TILE + wave * 8 + h * 4;
   if (o0 >= a.O) return;
 
   float *out_p = a.out + (long)b * a.out_sb + (long)o0 * a.out_so;
   if (a.io.perfect) {
 #pragma unroll
-    for (int m = 0; m < 4; ++m) {
-      if (o0 + m < a.O) {
-        float res = a.alpha * v[m];
-        if (a.beta != 0.0f) res += a.beta * out_p[(long)m * a.out_so];
-        out_p[(long)m * a.out_so] = res;
+    for (int q = 0; q < 4; ++q) {
+      if (o0 + q < a.O) {
+        float res = a.alpha * v[q];
+        if (a.beta != 0.0f) res += a.beta * out_p[(long)q * a.out_so];
+        out_p[(long)q * a.out_so] = res;
       }
     }
     return;
@@ -174,8 +197,8 @@ __global__ __launch_bounds__(256) void k_mvm_round(MvmArgs a) {
   const float fin = a.st.fin[b];
   if (fin == 0.0f) { // zero input: the reference short-cuts to a zero output
 #pragma unroll
-    for (int m = 0; m < 4; ++m) {
-      if (o0 + m < a.O) out_p[(long)m * a.out_so] = 0.0f;
+    for (int q = 0; q < 4; ++q) {
+      if (o0 + q < a.O) out_p[(long)q * a.out_so] = 0.0f;
     }
     return;
   }
@@ -188,26 +211,26 @@ __global__ __launch_bounds__(256) void k_mvm_round(MvmArgs a) {
   const float bound = a.io.out_bound;
   int up = 0, lo = 0;
 #pragma unroll
-  for (int m = 0; m < 4; ++m) {
-    float y = v[m];
+  for (int q = 0; q < 4; ++q) {
+    float y = v[q];
     if (a.io.out_asym > 0.0f) y = y < 0.0f ? y * (1.0f - a.io.out_asym) : y;
-    if (a.io.out_noise > 0.0f) y += a.io.out_noise * nz[m];
+    if (a.io.out_noise > 0.0f) y += a.io.out_noise * nz[q];
     if (a.io.out_res > 0.0f) {
-      float q = y / a.io.out_res;
+      float qq = y / a.io.out_res;
       if (a.io.out_sto_round) {
-        const Philox4 rr = philox4x32_10((uint32_t)(o0 + m), (uint32_t)b, a.call, RNG_OUT_SR | ((uint32_t)a.round << 8), a.key.k0, a.key.k1);
-        q = q + (u32_to_uniform(rr.v[0]) - 0.5f);
+        const Philox4 rr = philox4x32_10((uint32_t)(o0 + q), (uint32_t)b, a.call, RNG_OUT_SR | ((uint32_t)a.round << 8), a.key.k0, a.key.k1);
+        qq = qq + (u32_to_uniform(rr.v[0]) - 0.5f);
       }
-      y = rintf(q) * a.io.out_res;
+      y = rintf(qq) * a.io.out_res;
     }
     if (y > bound) {
       y = bound;
-      if (o0 + m < a.O) up = o0 + m + 1;
+      if (o0 + q < a.O) up = o0 + q + 1;
     } else if (y < -bound) {
       y = -bound;
-      if (o0 + m < a.O) lo = o0 + m + 1;
+      if (o0 + q < a.O) lo = o0 + q + 1;
     }
-    v[m] = y * fin;
+    v[q] = y * fin;
   }
   if (with_bm) {
     if (up) atomicMax(&a.st.hit_up[b], up);
@@ -217,8 +240,8 @@ __global__ __launch_bounds__(256) void k_mvm_round(MvmArgs a) {
     *reinterpret_cast<float4 *>(out_p) = make_float4(v[0], v[1], v[2], v[3]);
   } else {
 #pragma unroll
-    for (int m = 0; m < 4; ++m) {
-      if (o0 + m < a.O) out_p[(long)m * a.out_so] = v[m];
+    for (int q = 0; q < 4; ++q) {
+      if (o0 + q < a.O) out_p[(long)q * a.out_so] = v[q];
     }
   }
 }
@@ -249,37 +272,44 @@ __device__ __forceinline__ float block_reduce_sum(float v, float *sh) {
   return r;
 }
 
-__device__ __forceinline__ void set_round_scales(const MvmArgs &a, int b, float nm, float red) {
+// input scale and output factor of a round; returns the input scale
+__device__ __forceinline__ float set_round_scales(const MvmArgs &a, int b, float nm, float red) {
   const IoDev &io = a.io;
   const bool use_nm = io.noise_management != RPU_NM_NONE;
   const bool bm = io.bound_management != RPU_BM_NONE;
+  float scale, fin;
   if (a.transposed) {
     // backward: scale = 1 / nm ; result *= out_scale * nm
     if (use_nm && nm <= 0.0f) {
-      a.st.scale[b] = 0.0f;
-      a.st.fin[b] = 0.0f;
-      return;
+      scale = 0.0f;
+      fin = 0.0f;
+    } else {
+      scale = use_nm ? 1.0f / nm : 1.0f;
+      fin = use_nm ? io.out_scale * nm : io.out_scale;
     }
-    a.st.scale[b] = use_nm ? 1.0f / nm : 1.0f;
-    a.st.fin[b] = use_nm ? io.out_scale * nm : io.out_scale;
-    return;
+  } else if (use_nm && nm <= 0.0f && io.inp_noise <= 0.0f) {
+    scale = 0.0f;
+    fin = 0.0f;
+  } else {
+    scale = 1.0f;
+    if (use_nm && nm > 0.0f) scale /= nm;
+    if (bm) scale /= red;
+    fin = io.out_scale / scale;
   }
-  if (use_nm && nm <= 0.0f && io.inp_noise <= 0.0f) {
-    a.st.scale[b] = 0.0f;
-    a.st.fin[b] = 0.0f;
-    return;
-  }
-  float scale = 1.0f;
-  if (use_nm && nm > 0.0f) scale /= nm;
-  if (bm) scale /= red;
   a.st.scale[b] = scale;
-  a.st.fin[b] = io.out_scale / scale;
+  a.st.fin[b] = fin;
+  return scale;
 }
 
 __global__ __launch_bounds__(256) void k_mvm_init(MvmArgs a) {
   __shared__ float sh[8];
+  __shared__ float sh_scale;
   const int b = blockIdx.x;
   const IoDev &io = a.io;
+  if (io.perfect) { // plain copy into the k-contiguous scratch
+    write_dac_row(a, b, b, 1.0f, 0, a.xq[0]);
+    return;
+  }
   const float *row = a.in + (long)b * a.in_sb;
   float nm = 1.0f;
   if (io.noise_management == RPU_NM_ABS_MAX || io.noise_management == RPU_NM_ABS_MAX_NP_SUM ||
@@ -319,44 +349,56 @@ __global__ __launch_bounds__(256) void k_mvm_init(MvmArgs a) {
     a.st.red[b] = 1.0f;
     a.st.hit_up[b] = 0;
     a.st.hit_lo[b] = 0;
-    set_round_scales(a, b, nm, 1.0f);
+    sh_scale = set_round_scales(a, b, nm, 1.0f);
     a.st.rounds[b] = (a.st.fin[b] == 0.0f) ? 0 : 1;
   }
   if (b == 0 && threadIdx.x < 40) a.st.count[threadIdx.x] = 0;
+  __syncthreads();
+  write_dac_row(a, b, b, sh_scale, 0, a.xq[0]);
 }
 
-// After round a.round: samples whose ADC saturated get another round unless the reduction limit is
-// reached (rpu_forward_backward_pass.cpp:944-983).
+// After round a.round, one workgroup per sample of that round: samples whose ADC saturated get another
+// round unless the reduction limit is reached (rpu_forward_backward_pass.cpp:944-983).
 __global__ __launch_bounds__(256) void k_mvm_advance(MvmArgs a) {
+  __shared__ int sh_pos;
+  __shared__ float sh_scale;
   const int n_act = (a.round > 0) ? a.st.count[a.round] : a.m_batch;
-  const int slot = blockIdx.x * blockDim.x + threadIdx.x;
+  const int slot = blockIdx.x;
   if (slot >= n_act) return;
   const int b = (a.round > 0) ? a.st.list[a.round & 1][slot] : slot;
-  const IoDev &io = a.io;
-  const int up = a.st.hit_up[b], lo = a.st.hit_lo[b];
-  a.st.hit_up[b] = 0;
-  a.st.hit_lo[b] = 0;
-  if (a.st.fin[b] == 0.0f) return;
-  // the CPU loop sets "failed" on an upper hit and *assigns* !bm_test_negative_bound on a lower hit,
-  // walking the outputs in index order: the last hit decides
-  const bool failed = io.bm_test_negative_bound ? (up > 0 || lo > 0) : (up > lo);
-  if (!failed) return;
-  float red = a.st.red[b];
-  const bool stop = ((int)red > io.max_bm_factor) || ((io.inp_res > 0.0f) && (red > io.max_bm_res / io.inp_res));
-  if (stop) return;
-  red *= 2.0f;
-  float nm = a.st.nm[b];
-  if (a.round == 0 && io.bound_management == RPU_BM_ITERATIVE_WORST_CASE &&
-      io.noise_management != RPU_NM_ABS_MAX_NP_SUM) {
-    nm = a.st.nm_np[b];
-    a.st.nm[b] = nm;
-    red = 1.0f;
+  if (threadIdx.x == 0) {
+    const IoDev &io = a.io;
+    int pos = -1;
+    const int up = a.st.hit_up[b], lo = a.st.hit_lo[b];
+    a.st.hit_up[b] = 0;
+    a.st.hit_lo[b] = 0;
+    // the CPU loop sets "failed" on an upper hit and *assigns* !bm_test_negative_bound on a lower hit,
+    // walking the outputs in index order: the last hit decides
+    const bool failed = io.bm_test_negative_bound ? (up > 0 || lo > 0) : (up > lo);
+    if (failed && a.st.fin[b] != 0.0f) {
+      float red = a.st.red[b];
+      const bool stop = ((int)red > io.max_bm_factor) || ((io.inp_res > 0.0f) && (red > io.max_bm_res / io.inp_res));
+      if (!stop) {
+        red *= 2.0f;
+        float nm = a.st.nm[b];
+        if (a.round == 0 && io.bound_management == RPU_BM_ITERATIVE_WORST_CASE &&
+            io.noise_management != RPU_NM_ABS_MAX_NP_SUM) {
+          nm = a.st.nm_np[b];
+          a.st.nm[b] = nm;
+          red = 1.0f;
+        }
+        a.st.red[b] = red;
+        a.st.rounds[b] += 1;
+        sh_scale = set_round_scales(a, b, nm, red);
+        pos = atomicAdd(&a.st.count[a.round + 1], 1);
+        a.st.list[(a.round + 1) & 1][pos] = b;
+      }
+    }
+    sh_pos = pos;
   }
-  a.st.red[b] = red;
-  a.st.rounds[b] += 1;
-  set_round_scales(a, b, nm, red);
-  const int pos = atomicAdd(&a.st.count[a.round + 1], 1);
-  a.st.list[(a.round + 1) & 1][pos] = b;
+  __syncthreads();
+  if (sh_pos < 0) return;
+  write_dac_row(a, b, sh_pos, sh_scale, a.round + 1, a.xq[(a.round + 1) & 1]);
 }
 
 __global__ void k_make_bias(const float *in, float *out, int m_batch, int x_size, int in_trans) {
@@ -399,17 +441,45 @@ int mvm_max_rounds(const IoDev &io) {
   return rounds > 32 ? 32 : rounds;
 }
 
+// prefetch depth used for a contraction length: deep for long contractions, where each of the few
+// resident waves must cover the memory latency alone
+static int mvm_prefetch_depth(int K) { return K >= 512 ? 4 : 1; }
+
+int mvm_k_pad(int K) {
+  const int unit = KSTEP * WAVES * mvm_prefetch_depth(K);
+  return ((K + unit - 1) / unit) * unit;
+}
+
 void launch_mvm_init(const MvmArgs &a, hipStream_t s) {
   hipLaunchKernelGGL(k_mvm_init, dim3(a.m_batch), dim3(256), 0, s, a);
 }
 
 void launch_mvm_round(const MvmArgs &a, hipStream_t s) {
-  dim3 grid((a.O + TILE - 1) / TILE, (a.m_batch + TILE - 1) / TILE);
-  hipLaunchKernelGGL(k_mvm_round, grid, dim3(256), 0, s, a);
+  const int tiles_o = (a.O + TILE - 1) / TILE;
+  const int per = (tiles_o + 7) / 8;
+  const int tiles_b = (a.m_batch + TILE - 1) / TILE;
+  const dim3 grid(8 * per * tiles_b);
+  const bool deep = mvm_prefetch_depth(a.K) == 4;
+  int mode = 2;
+  if (!a.transposed && (a.x_size & 3) == 0 && (a.K & 15) == 0 && a.K >= 16 && ((((uintptr_t)a.w) & 15) == 0)) {
+    mode = 0;
+  } else if (a.transposed) {
+    mode = 1;
+  }
+  if (mode == 0) {
+    if (deep) hipLaunchKernelGGL((k_mvm_round<4, 0>), grid, dim3(256), 0, s, a);
+    else hipLaunchKernelGGL((k_mvm_round<1, 0>), grid, dim3(256), 0, s, a);
+  } else if (mode == 1) {
+    if (deep) hipLaunchKernelGGL((k_mvm_round<4, 1>), grid, dim3(256), 0, s, a);
+    else hipLaunchKernelGGL((k_mvm_round<1, 1>), grid, dim3(256), 0, s, a);
+  } else {
+    if (deep) hipLaunchKernelGGL((k_mvm_round<4, 2>), grid, dim3(256), 0, s, a);
+    else hipLaunchKernelGGL((k_mvm_round<1, 2>), grid, dim3(256), 0, s, a);
+  }
 }
 
 void launch_mvm_advance(const MvmArgs &a, hipStream_t s) {
-  hipLaunchKernelGGL(k_mvm_advance, dim3((a.m_batch + 255) / 256), dim3(256), 0, s, a);
+  hipLaunchKernelGGL(k_mvm_advance, dim3(a.m_batch), dim3(256), 0, s, a);
 }
 
 void launch_make_bias(const float *in, float *out, int m_batch, int x_size, int in_trans, hipStream_t s) {

@@ -92,7 +92,7 @@ struct Tile {
   hipStream_t last_stream = nullptr;
   DevBuf<float> d_w, d_wmax, d_wmin, d_sup, d_sdown, d_slup, d_sldown;
   // MVM scratch
-  DevBuf<float> s_nm, s_nmnp, s_red, s_scale, s_fin, s_bias;
+  DevBuf<float> s_nm, s_nmnp, s_red, s_scale, s_fin, s_bias, s_xq0, s_xq1;
   DevBuf<int> s_rounds, s_hitup, s_hitlo, s_list0, s_list1, s_count;
   // update scratch
   DevBuf<int> u_bl;
@@ -145,7 +145,7 @@ struct Tile {
   void release_all() {
     d_w.release(); d_wmax.release(); d_wmin.release(); d_sup.release(); d_sdown.release();
     d_slup.release(); d_sldown.release();
-    s_nm.release(); s_nmnp.release(); s_red.release(); s_scale.release(); s_fin.release(); s_bias.release();
+    s_nm.release(); s_nmnp.release(); s_red.release(); s_scale.release(); s_fin.release(); s_bias.release(); s_xq0.release(); s_xq1.release();
     s_rounds.release(); s_hitup.release(); s_hitlo.release(); s_list0.release(); s_list1.release(); s_count.release();
     u_bl.release(); u_a.release(); u_b.release(); u_xval.release(); u_dval.release(); u_xw.release(); u_dw.release();
     u_xpl.release(); u_dpl.release(); u_kmax.release();
@@ -247,6 +247,10 @@ struct Tile {
     a.st.nm = s_nm.p; a.st.nm_np = s_nmnp.p; a.st.red = s_red.p; a.st.scale = s_scale.p; a.st.fin = s_fin.p;
     a.st.rounds = s_rounds.p; a.st.hit_up = s_hitup.p; a.st.hit_lo = s_hitlo.p;
     a.st.list[0] = s_list0.p; a.st.list[1] = s_list1.p; a.st.count = s_count.p;
+    a.k_pad = mvm_k_pad(K);
+    s_xq0.ensure((size_t)B * a.k_pad);
+    if (!io.perfect && io.p.bound_management != RPU_BM_NONE) s_xq1.ensure((size_t)B * a.k_pad);
+    a.xq[0] = s_xq0.p; a.xq[1] = s_xq1.p;
 
     // the x side carries the optional bias column: input of forward, output of backward
     float *final_out = out;
@@ -272,6 +276,8 @@ struct Tile {
     if (io.perfect) {
       a.round = 0;
       prof_begin(s);
+      launch_mvm_init(a, s);
+      prof_mark(s, "mvm_init");
       launch_mvm_round(a, s);
       prof_mark(s, "mvm_round");
     } else {
@@ -354,7 +360,12 @@ struct Tile {
       a.io = io_dev(fio); a.io.perfect = 1;
       a.alpha = -lr; a.beta = 1.0f; a.round = 0;
       a.key = key(); a.call = call++;
+      a.k_pad = mvm_k_pad(B);
+      s_xq0.ensure((size_t)X * a.k_pad);
+      a.xq[0] = s_xq0.p; a.xq[1] = nullptr;
       prof_begin(s);
+      launch_mvm_init(a, s);
+      prof_mark(s, "fp_update_gather");
       launch_mvm_round(a, s);
       prof_mark(s, "fp_update");
       RPU_HIP_CHECK(hipGetLastError());
