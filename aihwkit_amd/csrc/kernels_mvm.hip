@@ -78,22 +78,22 @@ __device__ __forceinline__ void write_dac_row(const MvmArgs &a, int b, int slot,
 //   2  any strides, every element guarded
 // Modes 0 and 1 load without predicates: out-of-range rows / k are clamped to valid addresses, their
 // products are either multiplied by the zero padding of the quantized inputs or never stored.
-template <int PD, int WMODE>
-__global__ __launch_bounds__(256) void k_mvm_round(MvmArgs a) {
-  __shared__ float red[WAVES][16][64];
-
-  const int n_act = (a.round > 0) ? a.st.count[a.round] : a.m_batch;
-  // workgroup n runs on XCD n % 8; XCD x owns the output-row tiles [x * per, (x + 1) * per)
+// tile number n -> (output tile, sample tile): workgroup n runs on XCD n % 8 and XCD x owns the
+// output-row tiles [x * per, (x + 1) * per)
+__device__ __forceinline__ bool tile_of(const MvmArgs &a, int n, int n_act, int &tile_o, int &tile_b) {
   const int tiles_o = (a.O + TILE - 1) / TILE;
   const int per = (tiles_o + 7) / 8;
-  const int n = blockIdx.x;
   const int xcd = n & 7;
   const int m = n >> 3;
-  const int tile_o = xcd * per + (m % per);
-  const int tile_b = m / per;
-  if (tile_o >= tiles_o || tile_b * TILE >= n_act) {
-    return; // whole workgroup leaves: no barrier is reached by anyone
-  }
+  tile_o = xcd * per + (m % per);
+  tile_b = m / per;
+  return tile_o < tiles_o && tile_b * TILE < n_act;
+}
+
+// one 32 x 32 output tile of round `round`; called by a whole workgroup (contains one workgroup barrier)
+template <int PD, int WMODE>
+__device__ __forceinline__ void mvm_round_tile(const MvmArgs &a, int round, int tile_o, int tile_b, int n_act,
+                                               float (*red)[16][64]) {
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int r = lane & 31;
@@ -109,7 +109,7 @@ __global__ __launch_bounds__(256) void k_mvm_round(MvmArgs a) {
   const long w_sk = a.transposed ? a.x_size : 1;
   const int o_clamped = o_ok ? o_in : a.O - 1;
   const float *w_row = a.w + (long)o_clamped * w_so;
-  const float *x_row = a.xq[a.round & 1] + (long)(b_ok ? slot_in : n_act - 1) * a.k_pad;
+  const float *x_row = a.xq[round & 1] + (long)(b_ok ? slot_in : n_act - 1) * a.k_pad;
 
   const int K = a.K;
   const int per_wave = a.k_pad / (KSTEP * WAVES); // a multiple of PD
@@ -177,7 +177,7 @@ __global__ __launch_bounds__(256) void k_mvm_round(MvmArgs a) {
     v[q] = ((red[0][i][lane] + red[1][i][lane]) + red[2][i][lane]) + red[3][i][lane];
   }
   if (!b_ok) return;
-  const int b = (a.round > 0) ? a.st.list[a.round & 1][slot_in] : slot_in;
+  const int b = (round > 0) ? a.st.list[round & 1][slot_in] : slot_in;
   const int o0 = tile_o * TILE + wave * 8 + h * 4;
   if (o0 >= a.O) return;
 
@@ -205,7 +205,7 @@ __global__ __launch_bounds__(256) void k_mvm_round(MvmArgs a) {
 
   float nz[4] = {0.f, 0.f, 0.f, 0.f};
   if (a.io.out_noise > 0.0f) {
-    philox_normal4((uint32_t)(o0 >> 2), (uint32_t)b, a.call, RNG_OUT_NOISE | ((uint32_t)a.round << 8), a.key, nz);
+    philox_normal4((uint32_t)(o0 >> 2), (uint32_t)b, a.call, RNG_OUT_NOISE | ((uint32_t)round << 8), a.key, nz);
   }
   const bool with_bm = a.io.bound_management != RPU_BM_NONE;
   const float bound = a.io.out_bound;
@@ -218,7 +218,7 @@ __global__ __launch_bounds__(256) void k_mvm_round(MvmArgs a) {
     if (a.io.out_res > 0.0f) {
       float qq = y / a.io.out_res;
       if (a.io.out_sto_round) {
-        const Philox4 rr = philox4x32_10((uint32_t)(o0 + q), (uint32_t)b, a.call, RNG_OUT_SR | ((uint32_t)a.round << 8), a.key.k0, a.key.k1);
+        const Philox4 rr = philox4x32_10((uint32_t)(o0 + q), (uint32_t)b, a.call, RNG_OUT_SR | ((uint32_t)round << 8), a.key.k0, a.key.k1);
         qq = qq + (u32_to_uniform(rr.v[0]) - 0.5f);
       }
       y = rintf(qq) * a.io.out_res;
@@ -301,10 +301,9 @@ __device__ __forceinline__ float set_round_scales(const MvmArgs &a, int b, float
   return scale;
 }
 
-__global__ __launch_bounds__(256) void k_mvm_init(MvmArgs a) {
-  __shared__ float sh[8];
-  __shared__ float sh_scale;
-  const int b = blockIdx.x;
+// state of round 0 and quantized input row of sample b; called by a whole workgroup
+__device__ __forceinline__ void mvm_init_sample(const MvmArgs &a, int b, float *sh, float *sh_scale_p) {
+  float &sh_scale = *sh_scale_p;
   const IoDev &io = a.io;
   if (io.perfect) { // plain copy into the k-contiguous scratch
     write_dac_row(a, b, b, 1.0f, 0, a.xq[0]);
@@ -312,8 +311,9 @@ __global__ __launch_bounds__(256) void k_mvm_init(MvmArgs a) {
   }
   const float *row = a.in + (long)b * a.in_sb;
   float nm = 1.0f;
-  if (io.noise_management == RPU_NM_ABS_MAX || io.noise_management == RPU_NM_ABS_MAX_NP_SUM ||
-      io.bound_management == RPU_BM_ITERATIVE_WORST_CASE || io.noise_management == RPU_NM_MAX) {
+  const bool worst_case = io.bound_management == RPU_BM_ITERATIVE_WORST_CASE;
+  const bool need_np = io.noise_management == RPU_NM_ABS_MAX_NP_SUM || worst_case;
+  if (io.noise_management == RPU_NM_ABS_MAX || io.noise_management == RPU_NM_MAX || need_np) {
     float amax = 0.0f, vmax = -INFINITY, ps = 0.0f, ns = 0.0f;
     for (int k = threadIdx.x; k < a.K; k += blockDim.x) {
       const float x = row[(long)k * a.in_sk];
@@ -326,10 +326,10 @@ __global__ __launch_bounds__(256) void k_mvm_init(MvmArgs a) {
     if (io.noise_management == RPU_NM_MAX) {
       vmax = block_reduce_max(vmax, sh);
       nm = io.nm_thres > 0.0f ? fminf(vmax, io.nm_thres) : vmax;
-    } else {
+    } else if (io.noise_management == RPU_NM_ABS_MAX) {
       nm = io.nm_thres > 0.0f ? fminf(amax, io.nm_thres) : amax;
     }
-    if (io.noise_management == RPU_NM_ABS_MAX_NP_SUM || io.bound_management == RPU_BM_ITERATIVE_WORST_CASE) {
+    if (need_np) {
       ps = block_reduce_sum(ps, sh);
       ns = block_reduce_sum(ns, sh);
       const float bound = isinf(io.out_bound) ? 1.0f : io.out_bound;
@@ -341,7 +341,8 @@ __global__ __launch_bounds__(256) void k_mvm_init(MvmArgs a) {
       if (io.noise_management == RPU_NM_ABS_MAX_NP_SUM) nm = np;
       if (threadIdx.x == 0) a.st.nm_np[b] = np;
     }
-  } else if (io.noise_management == RPU_NM_CONSTANT) {
+  }
+  if (io.noise_management == RPU_NM_CONSTANT) {
     nm = io.nm_thres > 0.0f ? io.nm_thres : 1.0f;
   }
   if (threadIdx.x == 0) {
@@ -355,17 +356,22 @@ __global__ __launch_bounds__(256) void k_mvm_init(MvmArgs a) {
   if (b == 0 && threadIdx.x < 40) a.st.count[threadIdx.x] = 0;
   __syncthreads();
   write_dac_row(a, b, b, sh_scale, 0, a.xq[0]);
+  __syncthreads(); // sh / sh_scale are reused by the caller's next sample
 }
 
-// After round a.round, one workgroup per sample of that round: samples whose ADC saturated get another
-// round unless the reduction limit is reached (rpu_forward_backward_pass.cpp:944-983).
-__global__ __launch_bounds__(256) void k_mvm_advance(MvmArgs a) {
-  __shared__ int sh_pos;
+__global__ __launch_bounds__(256) void k_mvm_init(MvmArgs a) {
+  __shared__ float sh[8];
   __shared__ float sh_scale;
-  const int n_act = (a.round > 0) ? a.st.count[a.round] : a.m_batch;
-  const int slot = blockIdx.x;
-  if (slot >= n_act) return;
-  const int b = (a.round > 0) ? a.st.list[a.round & 1][slot] : slot;
+  mvm_init_sample(a, blockIdx.x, sh, &sh_scale);
+}
+
+// After round `round`, for the sample in `slot` of that round's list: samples whose ADC saturated get
+// another round unless the reduction limit is reached (rpu_forward_backward_pass.cpp:944-983).  Called by a
+// whole workgroup.
+__device__ __forceinline__ void mvm_advance_slot(const MvmArgs &a, int round, int slot, int *sh_pos_p, float *sh_scale_p) {
+  int &sh_pos = *sh_pos_p;
+  float &sh_scale = *sh_scale_p;
+  const int b = (round > 0) ? a.st.list[round & 1][slot] : slot;
   if (threadIdx.x == 0) {
     const IoDev &io = a.io;
     int pos = -1;
@@ -381,7 +387,7 @@ __global__ __launch_bounds__(256) void k_mvm_advance(MvmArgs a) {
       if (!stop) {
         red *= 2.0f;
         float nm = a.st.nm[b];
-        if (a.round == 0 && io.bound_management == RPU_BM_ITERATIVE_WORST_CASE &&
+        if (round == 0 && io.bound_management == RPU_BM_ITERATIVE_WORST_CASE &&
             io.noise_management != RPU_NM_ABS_MAX_NP_SUM) {
           nm = a.st.nm_np[b];
           a.st.nm[b] = nm;
@@ -390,15 +396,32 @@ __global__ __launch_bounds__(256) void k_mvm_advance(MvmArgs a) {
         a.st.red[b] = red;
         a.st.rounds[b] += 1;
         sh_scale = set_round_scales(a, b, nm, red);
-        pos = atomicAdd(&a.st.count[a.round + 1], 1);
-        a.st.list[(a.round + 1) & 1][pos] = b;
+        pos = atomicAdd(&a.st.count[round + 1], 1);
+        a.st.list[(round + 1) & 1][pos] = b;
       }
     }
     sh_pos = pos;
   }
   __syncthreads();
-  if (sh_pos < 0) return;
-  write_dac_row(a, b, sh_pos, sh_scale, a.round + 1, a.xq[(a.round + 1) & 1]);
+  if (sh_pos >= 0) write_dac_row(a, b, sh_pos, sh_scale, round + 1, a.xq[(round + 1) & 1]);
+  __syncthreads();
+}
+
+__global__ __launch_bounds__(256) void k_mvm_advance(MvmArgs a) {
+  __shared__ int sh_pos;
+  __shared__ float sh_scale;
+  const int n_act = (a.round > 0) ? a.st.count[a.round] : a.m_batch;
+  if ((int)blockIdx.x >= n_act) return;
+  mvm_advance_slot(a, a.round, blockIdx.x, &sh_pos, &sh_scale);
+}
+
+template <int PD, int WMODE>
+__global__ __launch_bounds__(256) void k_mvm_round(MvmArgs a) {
+  __shared__ float red[WAVES][16][64];
+  const int n_act = (a.round > 0) ? a.st.count[a.round] : a.m_batch;
+  int tile_o, tile_b;
+  if (!tile_of(a, blockIdx.x, n_act, tile_o, tile_b)) return;
+  mvm_round_tile<PD, WMODE>(a, a.round, tile_o, tile_b, n_act, red);
 }
 
 __global__ void k_make_bias(const float *in, float *out, int m_batch, int x_size, int in_trans) {
@@ -450,6 +473,13 @@ int mvm_k_pad(int K) {
   return ((K + unit - 1) / unit) * unit;
 }
 
+// addressing mode of the weight operand (see k_mvm_round)
+static int weight_mode(const MvmArgs &a) {
+  if (!a.transposed && (a.x_size & 3) == 0 && (a.K & 15) == 0 && a.K >= 16 && ((((uintptr_t)a.w) & 15) == 0)) return 0;
+  if (a.transposed) return 1;
+  return 2;
+}
+
 void launch_mvm_init(const MvmArgs &a, hipStream_t s) {
   hipLaunchKernelGGL(k_mvm_init, dim3(a.m_batch), dim3(256), 0, s, a);
 }
@@ -460,12 +490,7 @@ void launch_mvm_round(const MvmArgs &a, hipStream_t s) {
   const int tiles_b = (a.m_batch + TILE - 1) / TILE;
   const dim3 grid(8 * per * tiles_b);
   const bool deep = mvm_prefetch_depth(a.K) == 4;
-  int mode = 2;
-  if (!a.transposed && (a.x_size & 3) == 0 && (a.K & 15) == 0 && a.K >= 16 && ((((uintptr_t)a.w) & 15) == 0)) {
-    mode = 0;
-  } else if (a.transposed) {
-    mode = 1;
-  }
+  const int mode = weight_mode(a);
   if (mode == 0) {
     if (deep) hipLaunchKernelGGL((k_mvm_round<4, 0>), grid, dim3(256), 0, s, a);
     else hipLaunchKernelGGL((k_mvm_round<1, 0>), grid, dim3(256), 0, s, a);

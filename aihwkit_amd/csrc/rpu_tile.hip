@@ -273,15 +273,14 @@ struct Tile {
       }
     }
 
+    prof_begin(s);
     if (io.perfect) {
       a.round = 0;
-      prof_begin(s);
       launch_mvm_init(a, s);
       prof_mark(s, "mvm_init");
       launch_mvm_round(a, s);
       prof_mark(s, "mvm_round");
     } else {
-      prof_begin(s);
       launch_mvm_init(a, s);
       prof_mark(s, "mvm_init");
       const int rounds = mvm_max_rounds(a.io);

@@ -132,7 +132,7 @@ def main() -> int:
     flops_per_call = 2.0 * x_size * d_size * batch
     update_bytes = bytes_per_device * x_size * d_size + 4.0 * (x_size + d_size) * batch
     k_update_ms = prof_update["update_pulsed"][0]
-    k_fwd_ms = prof_forward["mvm_round"][0]   # all rounds of one forward call
+    k_fwd_ms = prof_forward["mvm_round"][0]   # all round launches of one forward call
     k_bwd_ms = prof_backward["mvm_round"][0]
 
     out = {

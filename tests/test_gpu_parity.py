@@ -246,3 +246,90 @@ def test_deterministic_implicit_counts_are_bit_exact(gpu_device, device):
         assert np.abs(counts).max() >= 2
         orc.update(x, d)
         assert np.abs(gpu.get_weights().numpy() - orc.get_weights()).max() <= TOL
+
+
+NM, BM = dv.NoiseManagementType, dv.BoundManagementType
+
+
+@pytest.mark.parametrize("nm,nm_thres", [(NM.NONE, 0.0), (NM.AbsMax, 0.0), (NM.AbsMax, 0.5), (NM.Max, 0.0),
+                                         (NM.Constant, 2.0), (NM.AbsMaxNPSum, 0.0)])
+@pytest.mark.parametrize("bm", [BM.NONE, BM.Iterative, BM.IterativeWorstCase])
+def test_forward_noise_and_bound_management_modes_bit_exact(gpu_device, nm, nm_thres, bm):
+    """Every noise / bound management mode, with input / output asymmetry, an output scale and the
+    negative-bound test switched off, in the exact-arithmetic setting (inputs and weights on binary grids)."""
+    rng = np.random.default_rng(17)
+    x_size, d_size, batch = 256, 96, 40
+    f_io = noise_free_io(inp_res=1 / 128.0, out_res=1 / 512.0, bound_management=bm, noise_management=nm,
+                         nm_thres=nm_thres, inp_asymmetry=0.25, out_asymmetry=0.5, out_scale=2.0, out_bound=4.0,
+                         bm_test_negative_bound=False)
+    b_io = noise_free_io(inp_res=1 / 128.0, out_res=1 / 512.0, noise_management=nm, nm_thres=nm_thres,
+                         inp_asymmetry=0.25, out_scale=0.5)
+    meta = make_meta(f_io, b_io)
+    dev = constant_step(w_max_dtod=0.0, w_min_dtod=0.0, w_max=1.0, w_min=-1.0, construction_seed=7)
+    host, orc, _ = build_pair(meta, dev, x_size, d_size, gpu=False)
+    w = (rng.integers(-38, 39, (d_size, x_size)) / 64.0).astype(np.float32)
+    host.set_weights(torch.from_numpy(w))
+    orc.set_weights(w)
+    gpu = tiles.CudaAnalogTile(host)
+    x = (rng.integers(-64, 65, (batch, x_size)) / 64.0).astype(np.float32)
+    x[1] = 0.0
+    x[2] = -np.abs(x[2])  # Max noise management sees no positive entry
+    y_gpu = gpu.forward(cuda(x), False, False, False, False, False).cpu().numpy()
+    assert np.array_equal(y_gpu, orc.forward(x))
+    if bm != BM.NONE:
+        assert np.array_equal(gpu.get_bm_rounds(batch).numpy(), orc.bm_rounds(batch))
+        if nm != NM.AbsMaxNPSum:  # the NP-sum scale is made so that the first round fits
+            assert orc.bm_rounds(batch).max() >= 2
+    d = (rng.integers(-64, 65, (batch, d_size)) / 64.0).astype(np.float32)
+    assert np.array_equal(gpu.backward(cuda(d), False, False, False, False).cpu().numpy(), orc.backward(d))
+
+
+def test_linear_step_additive_noise_device_and_negative_learning_rate(gpu_device):
+    """LinearStep (not SoftBounds) with additive-noise form and mean-bound reference slopes, positive and
+    negative learning rate: GPU words -> oracle device loop, 1e-5."""
+    rng = np.random.default_rng(31)
+    x_size, d_size, batch = 80, 48, 20
+    dev = dv.LinearStepResistiveDeviceParameter()
+    for k, v in dict(gamma_up=0.4, gamma_down=0.2, gamma_up_dtod=0.05, gamma_down_dtod=0.05, mult_noise=False,
+                     dw_min=0.002, dw_min_std=0.0, construction_seed=9, enforce_consistency=True).items():
+        setattr(dev, k, v)
+    meta = make_meta(desired_bl=20)
+    host, orc, _ = build_pair(meta, dev, x_size, d_size, gpu=False)
+    w = rng.uniform(-0.4, 0.4, (d_size, x_size)).astype(np.float32)
+    host.set_weights(torch.from_numpy(w))
+    orc.set_weights(w)
+    gpu = tiles.CudaAnalogTile(host)
+    x = rng.uniform(-1, 1, (batch, x_size)).astype(np.float32)
+    d = (0.2 * rng.standard_normal((batch, d_size))).astype(np.float32)
+    before = orc.get_weights()
+    for lr in (0.02, -0.02):
+        gpu.set_learning_rate(lr)
+        orc.set_learning_rate(lr)
+        gpu.update(cuda(x), cuda(d), False, False, False, False)
+        xw, dw, bl = (t.numpy() for t in gpu.get_update_words(batch))
+        assert bl.max() <= 20
+        orc.update_with_words(xw, dw, bl)
+        assert np.abs(gpu.get_weights().numpy() - orc.get_weights()).max() <= TOL
+    # the two calls push in opposite directions
+    assert np.abs(orc.get_weights() - before).mean() < 0.5 * 0.002 * 20
+
+
+@pytest.mark.parametrize("x_trans,d_trans,bias", [(True, True, False), (False, False, True), (True, False, True)])
+def test_update_layouts_and_bias_column(gpu_device, x_trans, d_trans, bias):
+    rng = np.random.default_rng(13)
+    x_size, d_size, batch = 65, 33, 17
+    meta = make_meta(desired_bl=31, pulse_type=dv.PulseType.DeterministicImplicit)
+    dev = constant_step(dw_min=0.001, dw_min_std=0.0, construction_seed=5, enforce_consistency=True)
+    host, orc, _ = build_pair(meta, dev, x_size, d_size, gpu=False)
+    gpu = tiles.CudaAnalogTile(host)
+    xs = x_size - int(bias)
+    x = rng.uniform(-1, 1, (xs, batch) if x_trans else (batch, xs)).astype(np.float32)
+    d = (0.3 * rng.standard_normal((d_size, batch) if d_trans else (batch, d_size))).astype(np.float32)
+    gpu.set_learning_rate(0.05)
+    orc.set_learning_rate(0.05)
+    gpu.update(cuda(x), cuda(d), bias, x_trans, d_trans, False)
+    orc.update(x, d, bias, x_trans, d_trans)
+    assert np.abs(gpu.get_weights().numpy() - orc.get_weights()).max() <= TOL
+    assert np.abs(orc.get_weights()).max() > 5e-3
+    if bias:  # the bias column saw a constant input of one
+        assert np.abs(orc.get_weights()[:, -1]).mean() > np.abs(orc.get_weights()[:, :-1]).mean()

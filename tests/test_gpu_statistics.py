@@ -239,3 +239,59 @@ def test_cycle_to_cycle_noise_alone_matches_the_oracle_for_fixed_pulse_words(gpu
     wg, wo = np.stack(wg), np.stack(wo)
     assert wo.std(0).mean() > 1e-3
     compare_moments(wg, wo, f"cycle-to-cycle noise {device}")
+
+
+def test_stochastic_rounding_and_input_noise_moments(gpu_device):
+    """DAC / ADC stochastic rounding and input noise are random per element: moments over 64 seeds."""
+    rng = np.random.default_rng(7)
+    x_size, d_size, batch = 128, 64, 16
+    f_io = io_params(out_noise=0.02, inp_noise=0.05, inp_sto_round=True, out_sto_round=True, inp_res=1 / 16.0,
+                     out_res=1 / 32.0, noise_management=dv.NoiseManagementType.AbsMax)
+    meta = make_meta(f_io, io_params(out_noise=0.0))
+    dev = soft_bounds(construction_seed=3, enforce_consistency=True)
+    host, orc, _ = build_pair(meta, dev, x_size, d_size, gpu=False)
+    orc.use_gauss_table(False)
+    w = rng.uniform(-0.3, 0.3, (d_size, x_size)).astype(np.float32)
+    host.set_weights(torch.from_numpy(w))
+    orc.set_weights(w)
+    gpu = tiles.CudaAnalogTile(host)
+    x = rng.uniform(-1, 1, (batch, x_size)).astype(np.float32)
+    xg = cuda(x)
+    yg, yo = [], []
+    for s in range(N_SEEDS):
+        gpu.set_seed(300 + s)
+        orc.set_seed(1 + s)
+        yg.append(gpu.forward(xg, False, False, False, False, False).cpu().numpy())
+        yo.append(orc.forward(x))
+    yg, yo = np.stack(yg), np.stack(yo)
+    assert yo.std(0).mean() > 0.1  # coarse ADC: the rounding noise dominates
+    compare_moments(yg, yo, "stochastic rounding + input noise")
+    # unbiasedness of stochastic rounding: the seed-mean approaches the unquantized product
+    ideal = x @ w.T
+    assert np.abs(yg.mean(0) - ideal).mean() < 0.12
+
+
+def test_discretized_pulse_probabilities_moments(gpu_device):
+    """update.res > 0 with stochastic rounding of the pulse probabilities."""
+    rng = np.random.default_rng(9)
+    x_size, d_size, batch = 64, 48, 16
+    meta = make_meta(desired_bl=31, update_management=False, update_bl_management=False, res=1 / 8.0, sto_round=True)
+    dev = constant_step(dw_min=0.001, dw_min_dtod=0.1, dw_min_std=0.0, construction_seed=2, enforce_consistency=True)
+    host, orc, _ = build_pair(meta, dev, x_size, d_size, gpu=False)
+    w0 = orc.get_weights()
+    x = rng.uniform(-1, 1, (batch, x_size)).astype(np.float32)
+    d = (0.5 * rng.standard_normal((batch, d_size))).astype(np.float32)
+    xg, dg = cuda(x), cuda(d)
+    dwg, dwo = [], []
+    for s in range(N_SEEDS):
+        gpu = tiles.CudaAnalogTile(host)
+        gpu.set_seed(40 + s)
+        gpu.set_learning_rate(0.01)
+        gpu.update(xg, dg, False, False, False, False)
+        dwg.append(gpu.get_weights().numpy() - w0)
+        orc.set_weights(w0)
+        orc.set_seed(1 + s)
+        orc.set_learning_rate(0.01)
+        orc.update(x, d)
+        dwo.append(orc.get_weights() - w0)
+    compare_moments(np.stack(dwg), np.stack(dwo), "discretized pulse probabilities")
