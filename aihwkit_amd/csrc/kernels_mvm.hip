@@ -11,8 +11,8 @@
 //                  DAC-quantized input row, written k-contiguous and zero padded into a scratch matrix.
 //   k_mvm_round    the contraction + ADC epilogue.  One workgroup (4 waves) owns a 32 (outputs) x 32
 //                  (samples) tile; the 4 waves split the contraction length in four contiguous parts, each
-//                  runs v_mfma_f32_32x32x2_f32 over its part with both operands read straight from global
-//                  memory one full 128-byte line per row and step (16 k-values per half-wave), the four
+//                  runs v_mfma_f32_32x32x2_f32 over its part in steps of 32 k-values: unit-stride global
+//                  loads -> wave-private LDS tile -> MFMA operand registers, software pipelined.  The four
 //                  partial tiles are summed in a fixed order through LDS and each wave finishes 8 output
 //                  rows: noise, quantize, clip, bound bookkeeping, rescale, store.  Workgroups are numbered
 //                  so that the 8 XCDs each work on a contiguous band of output rows (own L2 slice of W).
@@ -70,14 +70,8 @@ __device__ __forceinline__ void write_dac_row(const MvmArgs &a, int b, int slot,
   }
 }
 
-// PD = number of contraction steps whose operand loads are in flight per wave (prefetch depth); the scratch
-// row length k_pad is a multiple of KSTEP * WAVES * PD so every wave runs whole groups of PD steps.
-// WMODE = how the weight operand is addressed:
-//   0  contraction index contiguous (forward), rows 16-byte aligned, K a multiple of 16: float4 loads
-//   1  output index contiguous (backward): scalar loads, 32 consecutive outputs per half-wave and k
-//   2  any strides, every element guarded
-// Modes 0 and 1 load without predicates: out-of-range rows / k are clamped to valid addresses, their
-// products are either multiplied by the zero padding of the quantized inputs or never stored.
+constexpr int LDS_ROW = KSTEP + 4; // floats per staged row: 16-byte aligned, conflict-free 128-bit reads
+
 // tile number n -> (output tile, sample tile): workgroup n runs on XCD n % 8 and XCD x owns the
 // output-row tiles [x * per, (x + 1) * per)
 __device__ __forceinline__ bool tile_of(const MvmArgs &a, int n, int n_act, int &tile_o, int &tile_b) {
@@ -90,16 +84,28 @@ __device__ __forceinline__ bool tile_of(const MvmArgs &a, int n, int n_act, int 
   return tile_o < tiles_o && tile_b * TILE < n_act;
 }
 
-// one 32 x 32 output tile of round `round`; called by a whole workgroup (contains one workgroup barrier)
+// WMODE = how the weight operand is addressed:
+//   0  contraction index contiguous (forward), rows 16-byte aligned, K a multiple of 16
+//   1  output index contiguous (backward: W is read transposed in place)
+//   2  any strides, every element guarded
+// Operand tiles with a contiguous contraction index (the quantized inputs always, the weights in mode 0) are
+// fetched with unit-stride 16-byte loads, 8 lanes per 128-byte row segment, staged in a wave-private LDS
+// tile and read back in the MFMA operand layout (lane (r, h) holds row r, k = 16 h .. 16 h + 15).  Reading
+// them straight into that layout would make every lane of a load touch a different cache line, which is
+// address-bound in the vector L1.  Mode 1 reads the weights directly: 32 consecutive outputs per half-wave
+// and k are one line.  Out-of-range rows / k are clamped to valid addresses: their products meet the zero
+// padding of the quantized inputs or are never stored.
+// PD = 2: software pipeline over two register sets (steps s + 1 and s + 2 in flight while step s is in
+// LDS), k_pad a multiple of 2 * KSTEP * WAVES; PD = 1: one register set, for short contractions.
 template <int PD, int WMODE>
 __device__ __forceinline__ void mvm_round_tile(const MvmArgs &a, int round, int tile_o, int tile_b, int n_act,
-                                               float (*red)[16][64]) {
+                                               float (*red)[16][64], float *stage) {
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int r = lane & 31;
   const int h = lane >> 5;
 
-  // operand rows owned by this lane
+  // operand rows owned by this lane in the MFMA layout
   const int o_in = tile_o * TILE + r;
   const bool o_ok = o_in < a.O;
   const int slot_in = tile_b * TILE + r;
@@ -107,60 +113,121 @@ __device__ __forceinline__ void mvm_round_tile(const MvmArgs &a, int round, int 
 
   const long w_so = a.transposed ? 1 : a.x_size;
   const long w_sk = a.transposed ? a.x_size : 1;
-  const int o_clamped = o_ok ? o_in : a.O - 1;
-  const float *w_row = a.w + (long)o_clamped * w_so;
-  const float *x_row = a.xq[round & 1] + (long)(b_ok ? slot_in : n_act - 1) * a.k_pad;
-
   const int K = a.K;
   const int per_wave = a.k_pad / (KSTEP * WAVES); // a multiple of PD
   const int s_begin = wave * per_wave;
   const int s_end = s_begin + per_wave;
 
+  float *stage_x = stage + wave * (2 * TILE * LDS_ROW);
+  float *stage_w = stage_x + TILE * LDS_ROW;
+
+  // staging layout of this lane: pass t covers rows 8 t .. 8 t + 7, lane = (row in pass) * 8 + 16-byte chunk
+  const int st_row = lane >> 3;
+  const int st_chunk = (lane & 7) * 4;
+  const float *xq = a.xq[round & 1];
+  const float *x_src[4];
+  const float *w_src[4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    const int row = t * 8 + st_row;
+    const int slot = min(tile_b * TILE + row, n_act - 1);
+    x_src[t] = xq + (long)slot * a.k_pad + st_chunk;
+    const int o = min(tile_o * TILE + row, a.O - 1);
+    w_src[t] = a.w + (long)o * a.x_size;
+  }
+  const float *w_col = a.w + (long)(o_ok ? o_in : a.O - 1) * w_so; // mode 1: this lane's output column
+
   floatx16 acc;
 #pragma unroll
   for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
 
-  auto load_step = [&](int s, float (&wd)[16], float (&xd)[16]) {
-    const int k0 = s * KSTEP + h * 16;
+  auto gload = [&](int s, float4 (&gx)[4], float4 (&gw)[4], float (&wd)[16]) {
+    const int k0 = s * KSTEP;
 #pragma unroll
-    for (int v4 = 0; v4 < 4; ++v4) {
-      const float4 t = *reinterpret_cast<const float4 *>(x_row + k0 + v4 * 4);
-      xd[v4 * 4 + 0] = t.x; xd[v4 * 4 + 1] = t.y; xd[v4 * 4 + 2] = t.z; xd[v4 * 4 + 3] = t.w;
-    }
+    for (int t = 0; t < 4; ++t) gx[t] = *reinterpret_cast<const float4 *>(x_src[t] + k0);
     if (WMODE == 0) {
-      const int kc = min(k0, K - 16); // K % 16 == 0: a group is either whole or entirely zero padding
+      const int kc = min(k0 + st_chunk, K - 4); // K % 16 == 0: past K the inputs are zero padding
 #pragma unroll
-      for (int v4 = 0; v4 < 4; ++v4) {
-        const float4 t = *reinterpret_cast<const float4 *>(w_row + kc + v4 * 4);
-        wd[v4 * 4 + 0] = t.x; wd[v4 * 4 + 1] = t.y; wd[v4 * 4 + 2] = t.z; wd[v4 * 4 + 3] = t.w;
-      }
+      for (int t = 0; t < 4; ++t) gw[t] = *reinterpret_cast<const float4 *>(w_src[t] + kc);
     } else if (WMODE == 1) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
-        const int kc = min(k0 + i, K - 1);
-        wd[i] = w_row[(long)kc * w_sk];
+        const int kc = min(k0 + h * 16 + i, K - 1);
+        wd[i] = w_col[(long)kc * w_sk];
       }
     } else {
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
-        wd[i] = (o_ok && (k0 + i) < K) ? a.w[(long)o_in * w_so + (long)(k0 + i) * w_sk] : 0.0f;
+        const int k = k0 + h * 16 + i;
+        wd[i] = (o_ok && k < K) ? a.w[(long)o_in * w_so + (long)k * w_sk] : 0.0f;
       }
     }
   };
-
-  // steps s_begin .. s_end-1 in groups of PD; the loads of the next PD steps are always in flight
-  float wb[PD][16], xb[PD][16];
+  auto lds_store = [&](const float4 (&gx)[4], const float4 (&gw)[4]) {
 #pragma unroll
-  for (int p = 0; p < PD; ++p) load_step(s_begin + p, wb[p], xb[p]);
-  for (int s = s_begin; s < s_end; s += PD) {
+    for (int t = 0; t < 4; ++t) {
+      const int off = (t * 8 + st_row) * LDS_ROW + st_chunk;
+      *reinterpret_cast<float4 *>(stage_x + off) = gx[t];
+      if (WMODE == 0) *reinterpret_cast<float4 *>(stage_w + off) = gw[t];
+    }
+  };
+  auto lds_read = [&](float (&xd)[16], float (&wd)[16]) {
 #pragma unroll
-    for (int p = 0; p < PD; ++p) {
-#pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(wb[p][i], xb[p][i], acc, 0, 0, 0);
+    for (int v4 = 0; v4 < 4; ++v4) {
+      const int off = r * LDS_ROW + h * 16 + v4 * 4;
+      const float4 tx = *reinterpret_cast<const float4 *>(stage_x + off);
+      xd[v4 * 4 + 0] = tx.x; xd[v4 * 4 + 1] = tx.y; xd[v4 * 4 + 2] = tx.z; xd[v4 * 4 + 3] = tx.w;
+      if (WMODE == 0) {
+        const float4 tw = *reinterpret_cast<const float4 *>(stage_w + off);
+        wd[v4 * 4 + 0] = tw.x; wd[v4 * 4 + 1] = tw.y; wd[v4 * 4 + 2] = tw.z; wd[v4 * 4 + 3] = tw.w;
       }
-      // refill this buffer with the step PD ahead; past the end the last step is re-read and never used
-      load_step(min(s + PD + p, s_end - 1), wb[p], xb[p]);
+    }
+  };
+  auto mfma16 = [&](const float (&wd)[16], const float (&xd)[16]) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(wd[i], xd[i], acc, 0, 0, 0);
+  };
+
+  if (PD == 2) {
+    // register sets A and B alternate; the weights of mode 1 / 2 live in wa / wb until their step runs
+    float4 gxa[4], gwa[4], gxb[4], gwb[4];
+    float wa[16], wb[16], xc[16], wc[16];
+    gload(s_begin, gxa, gwa, wa);
+    gload(s_begin + 1, gxb, gwb, wb);
+    lds_store(gxa, gwa);
+    for (int s = s_begin; s < s_end; s += 2) {
+      // step s (set A is in LDS)
+      lds_read(xc, wc);
+      if (WMODE != 0) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) wc[i] = wa[i];
+      }
+      gload(min(s + 2, s_end - 1), gxa, gwa, wa);
+      mfma16(wc, xc);
+      lds_store(gxb, gwb);
+      // step s + 1 (set B is in LDS)
+      lds_read(xc, wc);
+      if (WMODE != 0) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) wc[i] = wb[i];
+      }
+      gload(min(s + 3, s_end - 1), gxb, gwb, wb);
+      mfma16(wc, xc);
+      lds_store(gxa, gwa);
+    }
+  } else {
+    float4 gx[4], gw[4];
+    float wn[16], xc[16], wc[16];
+    gload(s_begin, gx, gw, wn);
+    for (int s = s_begin; s < s_end; ++s) {
+      lds_store(gx, gw);
+      lds_read(xc, wc);
+      if (WMODE != 0) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) wc[i] = wn[i];
+      }
+      gload(min(s + 1, s_end - 1), gx, gw, wn);
+      mfma16(wc, xc);
     }
   }
 
@@ -418,10 +485,11 @@ __global__ __launch_bounds__(256) void k_mvm_advance(MvmArgs a) {
 template <int PD, int WMODE>
 __global__ __launch_bounds__(256) void k_mvm_round(MvmArgs a) {
   __shared__ float red[WAVES][16][64];
+  __shared__ __attribute__((aligned(16))) float stage[WAVES * 2 * TILE * LDS_ROW];
   const int n_act = (a.round > 0) ? a.st.count[a.round] : a.m_batch;
   int tile_o, tile_b;
   if (!tile_of(a, blockIdx.x, n_act, tile_o, tile_b)) return;
-  mvm_round_tile<PD, WMODE>(a, a.round, tile_o, tile_b, n_act, red);
+  mvm_round_tile<PD, WMODE>(a, a.round, tile_o, tile_b, n_act, red, stage);
 }
 
 __global__ void k_make_bias(const float *in, float *out, int m_batch, int x_size, int in_trans) {
@@ -466,7 +534,7 @@ int mvm_max_rounds(const IoDev &io) {
 
 // prefetch depth used for a contraction length: deep for long contractions, where each of the few
 // resident waves must cover the memory latency alone
-static int mvm_prefetch_depth(int K) { return K >= 512 ? 4 : 1; }
+static int mvm_prefetch_depth(int K) { return K >= 256 ? 2 : 1; }
 
 int mvm_k_pad(int K) {
   const int unit = KSTEP * WAVES * mvm_prefetch_depth(K);
@@ -489,16 +557,16 @@ void launch_mvm_round(const MvmArgs &a, hipStream_t s) {
   const int per = (tiles_o + 7) / 8;
   const int tiles_b = (a.m_batch + TILE - 1) / TILE;
   const dim3 grid(8 * per * tiles_b);
-  const bool deep = mvm_prefetch_depth(a.K) == 4;
+  const bool deep = mvm_prefetch_depth(a.K) == 2;
   const int mode = weight_mode(a);
   if (mode == 0) {
-    if (deep) hipLaunchKernelGGL((k_mvm_round<4, 0>), grid, dim3(256), 0, s, a);
+    if (deep) hipLaunchKernelGGL((k_mvm_round<2, 0>), grid, dim3(256), 0, s, a);
     else hipLaunchKernelGGL((k_mvm_round<1, 0>), grid, dim3(256), 0, s, a);
   } else if (mode == 1) {
-    if (deep) hipLaunchKernelGGL((k_mvm_round<4, 1>), grid, dim3(256), 0, s, a);
+    if (deep) hipLaunchKernelGGL((k_mvm_round<2, 1>), grid, dim3(256), 0, s, a);
     else hipLaunchKernelGGL((k_mvm_round<1, 1>), grid, dim3(256), 0, s, a);
   } else {
-    if (deep) hipLaunchKernelGGL((k_mvm_round<4, 2>), grid, dim3(256), 0, s, a);
+    if (deep) hipLaunchKernelGGL((k_mvm_round<2, 2>), grid, dim3(256), 0, s, a);
     else hipLaunchKernelGGL((k_mvm_round<1, 2>), grid, dim3(256), 0, s, a);
   }
 }
