@@ -98,7 +98,8 @@ struct UpdateArgs {
   uint32_t *x_words; // [B][X] packed pulse words
   uint32_t *d_words; // [B][D]
   // sample-transposed pulse bits: plane (chunk c, slot k) of line element e is the 32-bit word whose bit q
-  // is pulse slot k of sample 32 c + q; element (c, k, e) at planes[(c * plane_slots + k) * size + e]
+  // is pulse slot k of sample 32 c + q; element (c, k, e) at planes[(c * plane_slots + k) * size + e];
+  // slot plane_slots - 1 holds the sign bits (bit 0 of the packed words)
   uint32_t *x_planes;
   uint32_t *d_planes;
   int plane_slots; // slots per chunk the plane buffers are laid out for

@@ -301,28 +301,157 @@ __global__ __launch_bounds__(256) void k_update_planes(UpdateArgs a) {
       if (c0 + 1 < a.n_chunks) planes[((long)(c0 + 1) * a.plane_slots + k) * size + el] = (uint32_t)(m >> 32);
     }
   }
+  // the last slot of a chunk holds the sign bits of its samples
+  const unsigned long long sg = __ballot(word & 1u);
+  if (lane == 0) {
+    const int ks = a.plane_slots - 1;
+    planes[((long)c0 * a.plane_slots + ks) * size + el] = (uint32_t)sg;
+    if (c0 + 1 < a.n_chunks) planes[((long)(c0 + 1) * a.plane_slots + ks) * size + el] = (uint32_t)(sg >> 32);
+  }
 }
 
-// grid: x = ceil(x_size / 256), y = d_size.  One thread per cross-point; a wave covers 64 consecutive x of
-// one d row.  The batch is walked in blocks of 128 samples.  For a block every lane first builds the 128-bit
-// set of samples in which its cross-point has a coincidence: OR over the pulse slots of
-// (x_plane & d_plane), with the d planes wave-uniform and the x planes read with unit stride.  Then every
-// lane walks its own set in batch order; the count and direction of an event come from the two packed
-// words of that sample.  The wave loop applies at most one pulse per lane and pass and ends when the lane
-// with the most pulses is done; the eight noise factors of eight passes come from one Philox call per
-// lane, keyed by (cross-point, refill index).
+// Cross-point parameters of the pulse loop.  A step down subtracts (slope_down * w + scale_down) * f; with
+// the down parameters negated every pulse is the same "w += (slope * w + scale) * f", and negation is
+// exact in floating point.  The two clips of the reference (rpu_constantstep_device.cpp:48-53:
+// min(w_max) then max(w_min); rpu_linearstep_device.cpp:155-160: max(w_min) then min(w_max)) are a
+// median of three for bounds chosen so that crossed bounds give what the reference's order gives.
+template <int KIND>
+struct PulseCell {
+  float scale_up, scale_dn, slope_up, slope_dn, lo, hi;
+  __device__ __forceinline__ void load(const DeviceDev &d, unsigned cell) {
+    const float w_max = d.w_max[cell], w_min = d.w_min[cell];
+    scale_up = d.scale_up[cell];
+    scale_dn = -d.scale_down[cell];
+    if (KIND != RPU_DEVICE_CONSTANT_STEP) {
+      slope_up = d.slope_up[cell];
+      slope_dn = -d.slope_down[cell];
+      lo = fminf(w_min, w_max); // crossed bounds: always w_max
+      hi = w_max;
+    } else {
+      slope_up = slope_dn = 0.0f;
+      lo = w_min;
+      hi = fmaxf(w_min, w_max); // crossed bounds: always w_min
+    }
+  }
+};
+
+// one pulse with the noise factor f = 1 + std * N(0,1) (1 without cycle-to-cycle noise)
 template <int KIND, bool MULT>
-__global__ __launch_bounds__(256) void k_update_pulsed(UpdateArgs a) {
-  const int i = blockIdx.y;
-  const int jt = blockIdx.x * blockDim.x + threadIdx.x;
-  const bool valid = jt < a.x_size;
-  const int j = valid ? jt : a.x_size - 1;
-  const unsigned cell = (unsigned)i * (unsigned)a.x_size + (unsigned)j;
-  const CellParams cp = load_cell<KIND>(a.dev, cell);
-  float w = a.w[cell];
+__device__ __forceinline__ float pulse(float w, float slope, float scale, float f, float lo, float hi) {
+  float step;
+  if (KIND == RPU_DEVICE_CONSTANT_STEP) step = scale * f;
+  else if (MULT) step = (slope * w + scale) * f;
+  else step = slope * w + scale * f;
+  return __builtin_amdgcn_fmed3f(w + step, lo, hi);
+}
+
+// eight noise factors of one cross-point, keyed by (cross-point, refill index)
+__device__ __forceinline__ void noise_factors(float (&f)[8], float std_, unsigned cell, uint32_t refill,
+                                              const UpdateArgs &a) {
+  if (std_ > 0.0f) {
+    float g[8];
+    philox_normal8(cell, refill, a.call, RNG_CTOC, a.key, g);
+#pragma unroll
+    for (int q = 0; q < 8; ++q) f[q] = 1.0f + std_ * g[q];
+  } else {
+#pragma unroll
+    for (int q = 0; q < 8; ++q) f[q] = 1.0f;
+  }
+}
+
+// Pulse loop for short bit lines (at most 2^NB - 1 pulse slots in use).  The batch is walked in chunks of
+// 32 samples.  For a chunk every lane builds, from the bit planes alone, the coincidence count of each
+// of its 32 samples as NB bit-sliced words (a ripple-carry add of x_plane & d_plane per slot; the d
+// planes are wave-uniform) and the direction word sign(x) ^ sign(d).  The lanes then walk their samples
+// in batch order: lowest set bit of the pending set, count and direction by bit extraction, one pulse
+// per lane and pass.  The wave moves to the next chunk when no lane has a pulse left; the noise
+// factors of eight passes come from one Philox call per lane and carry over chunk ends.
+template <int KIND, bool MULT, int NB>
+__device__ __forceinline__ float pulsed_counted(const UpdateArgs &a, float w, const PulseCell<KIND> &cp, unsigned cell,
+                                                int i, int j, bool valid, int kmax) {
+  const float std_ = a.dev.dw_min_std;
+  const uint32_t lr_mask = a.lr < 0.0f ? 0xffffffffu : 0u;
+  const int n_chunks = a.n_chunks;
+  const unsigned xs = (unsigned)a.x_size, ds = (unsigned)a.d_size;
+  const unsigned slots = (unsigned)a.plane_slots;
+  const uint32_t *xpl = a.x_planes + j;
+  const uint32_t *dpl = a.d_planes + i;
+
+  uint32_t cnt[NB];
+#pragma unroll
+  for (int n = 0; n < NB; ++n) cnt[n] = 0u;
+  uint32_t cur = 0u, same = 0u; // pending samples of the chunk; bit set: x and d have the same sign
+  int left = 0;
+  float slope = 0.0f, scale = 0.0f;
+  int c = -1;
+  uint32_t refill = 0;
+  bool finished = false;
+  while (!finished) {
+    float f[8];
+    noise_factors(f, std_, cell, refill, a);
+    ++refill;
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      while (!__any((cur | (uint32_t)left) != 0u)) {
+        if (++c >= n_chunks) {
+          finished = true;
+          break;
+        }
+        const unsigned base = (unsigned)c * slots;
+#pragma unroll
+        for (int n = 0; n < NB; ++n) cnt[n] = 0u;
+#pragma unroll
+        for (int k = 0; k < (1 << NB) - 1; ++k) {
+          if (k < kmax) {
+            const uint32_t dk = dpl[(base + k) * ds]; // wave-uniform
+            if (dk) {
+              uint32_t carry = dk & xpl[(base + k) * xs];
+#pragma unroll
+              for (int n = 0; n < NB; ++n) {
+                const uint32_t t = cnt[n] & carry;
+                cnt[n] ^= carry;
+                carry = t;
+              }
+            }
+          }
+        }
+        cur = cnt[0];
+#pragma unroll
+        for (int n = 1; n < NB; ++n) cur |= cnt[n];
+        if (!valid) cur = 0u;
+        same = ~(xpl[(base + slots - 1) * xs] ^ dpl[(base + slots - 1) * ds]) ^ lr_mask;
+      }
+      if (finished) break;
+      if (left == 0 && cur != 0u) {
+        const int bit = __ffs((int)cur) - 1;
+        cur &= cur - 1u;
+        left = (int)((cnt[0] >> bit) & 1u);
+#pragma unroll
+        for (int n = 1; n < NB; ++n) left += (int)(((cnt[n] >> bit) & 1u) << n);
+        // step down when x and d have the same sign and lr > 0
+        const bool down = ((same >> bit) & 1u) != 0u;
+        slope = down ? cp.slope_dn : cp.slope_up;
+        scale = down ? cp.scale_dn : cp.scale_up;
+      }
+      if (left > 0) {
+        w = pulse<KIND, MULT>(w, slope, scale, f[q], cp.lo, cp.hi);
+        --left;
+      }
+    }
+  }
+  return w;
+}
+
+// Pulse loop for any bit-line length.  The batch is walked in blocks of 128 samples.  For a block every lane
+// first builds the 128-bit set of samples in which its cross-point has a coincidence: OR over the pulse
+// slots of (x_plane & d_plane).  Then every lane walks its own set in batch order; the count and
+// direction of an event come from the two packed words of that sample.  The wave loop applies at most
+// one pulse per lane and pass and ends when the lane with the most pulses is done.
+template <int KIND, bool MULT>
+__device__ __forceinline__ float pulsed_gather(const UpdateArgs &a, float w, const PulseCell<KIND> &cp, unsigned cell,
+                                               int i, int j, bool valid, int kmax) {
   const float std_ = a.dev.dw_min_std;
   const uint32_t lr_neg = a.lr < 0.0f ? 1u : 0u;
-  const int kmax = a.kmax[a.kmax_slot];
   const int n_chunks = a.n_chunks;
   const uint32_t *xpl = a.x_planes + j;
   const uint32_t *dpl = a.d_planes + i;
@@ -352,21 +481,11 @@ __global__ __launch_bounds__(256) void k_update_pulsed(UpdateArgs a) {
     unsigned long long nxt = ((unsigned long long)ev[3] << 32) | ev[2];
     unsigned sample0 = (unsigned)c0 * 32u; // sample index of bit 0 of cur
     int left = 0;                          // pulses left in the current event
-    // parameters of the current event's direction
     float slope = 0.0f, scale = 0.0f;
-    uint32_t flip = 0u; // sign bit to apply to the step: down = subtract
     bool block_done = !__any((cur | nxt) != 0ull);
     while (!block_done) {
       float f[8];
-      if (std_ > 0.0f) {
-        float g[8];
-        philox_normal8(cell, refill, a.call, RNG_CTOC, a.key, g);
-#pragma unroll
-        for (int q = 0; q < 8; ++q) f[q] = 1.0f + std_ * g[q];
-      } else {
-#pragma unroll
-        for (int q = 0; q < 8; ++q) f[q] = 1.0f;
-      }
+      noise_factors(f, std_, cell, refill, a);
       ++refill;
 #pragma unroll
       for (int q = 0; q < 8; ++q) {
@@ -385,9 +504,8 @@ __global__ __launch_bounds__(256) void k_update_pulsed(UpdateArgs a) {
             left = __popc(xw & dw & ~1u);
             // step down when x and d have the same sign and lr > 0
             const bool down = (((xw ^ dw) & 1u) ^ lr_neg) == 0u;
-            slope = down ? cp.slope_down : cp.slope_up;
-            scale = down ? cp.scale_down : cp.scale_up;
-            flip = down ? 0x80000000u : 0u;
+            slope = down ? cp.slope_dn : cp.slope_up;
+            scale = down ? cp.scale_dn : cp.scale_up;
           }
         }
         if (!__any(left > 0)) {
@@ -395,29 +513,32 @@ __global__ __launch_bounds__(256) void k_update_pulsed(UpdateArgs a) {
           break;
         }
         if (left > 0) {
-          // one pulse: ConstantStep  w +- scale * f ; LinearStep  w +- (slope * w + scale) * f  (mult noise)
-          // or w +- (slope * w + scale * f) (additive noise); "-" as the addition of the negated step
-          float step;
-          if (KIND == RPU_DEVICE_CONSTANT_STEP) {
-            step = (std_ > 0.0f) ? f[q] * scale : scale;
-          } else if (MULT) {
-            step = (slope * w + scale) * f[q];
-          } else {
-            step = slope * w + scale * f[q];
-          }
-          w = w + __uint_as_float(__float_as_uint(step) ^ flip);
-          if (KIND == RPU_DEVICE_CONSTANT_STEP) {
-            w = fminf(w, cp.w_max);
-            w = fmaxf(w, cp.w_min);
-          } else {
-            w = fmaxf(w, cp.w_min);
-            w = fminf(w, cp.w_max);
-          }
+          w = pulse<KIND, MULT>(w, slope, scale, f[q], cp.lo, cp.hi);
           --left;
         }
       }
     }
   }
+  return w;
+}
+
+// grid: x = ceil(x_size / 256), y = d_size.  One thread per cross-point; a wave covers 64 consecutive x of
+// one d row, so everything that belongs to the d line is wave-uniform and the x planes, weights and
+// parameters are read with unit stride.  The pulse loop is chosen by the longest bit line of the batch.
+template <int KIND, bool MULT>
+__global__ __launch_bounds__(256) void k_update_pulsed(UpdateArgs a) {
+  const int i = blockIdx.y;
+  const int jt = blockIdx.x * blockDim.x + threadIdx.x;
+  const bool valid = jt < a.x_size;
+  const int j = valid ? jt : a.x_size - 1;
+  const unsigned cell = (unsigned)i * (unsigned)a.x_size + (unsigned)j;
+  PulseCell<KIND> cp;
+  cp.load(a.dev, cell);
+  float w = a.w[cell];
+  const int kmax = a.kmax[a.kmax_slot];
+  if (kmax <= 3) w = pulsed_counted<KIND, MULT, 2>(a, w, cp, cell, i, j, valid, kmax);
+  else if (kmax <= 7) w = pulsed_counted<KIND, MULT, 3>(a, w, cp, cell, i, j, valid, kmax);
+  else w = pulsed_gather<KIND, MULT>(a, w, cp, cell, i, j, valid, kmax);
   if (valid) a.w[cell] = w;
 }
 

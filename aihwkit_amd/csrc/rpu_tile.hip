@@ -301,7 +301,7 @@ struct Tile {
   }
 
   void set_plane_args(UpdateArgs &a, int B) {
-    const int slots = 31;
+    const int slots = 32; // 31 pulse slots and the sign plane
     const int chunks = (B + 31) / 32;
     u_xpl.ensure((size_t)chunks * slots * X);
     u_dpl.ensure((size_t)chunks * slots * D);
