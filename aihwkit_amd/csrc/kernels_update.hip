@@ -349,10 +349,7 @@ __device__ __forceinline__ float pulse(float w, float slope, float scale, float 
 __device__ __forceinline__ void noise_factors(float (&f)[8], float std_, unsigned cell, uint32_t refill,
                                               const UpdateArgs &a) {
   if (std_ > 0.0f) {
-    float g[8];
-    philox_normal8(cell, refill, a.call, RNG_CTOC, a.key, g);
-#pragma unroll
-    for (int q = 0; q < 8; ++q) f[q] = 1.0f + std_ * g[q];
+    philox_factor8(cell, refill, a.call, RNG_CTOC, a.key, std_, f);
   } else {
 #pragma unroll
     for (int q = 0; q < 8; ++q) f[q] = 1.0f;
@@ -363,9 +360,10 @@ __device__ __forceinline__ void noise_factors(float (&f)[8], float std_, unsigne
 // 32 samples.  For a chunk every lane builds, from the bit planes alone, the coincidence count of each
 // of its 32 samples as NB bit-sliced words (a ripple-carry add of x_plane & d_plane per slot; the d
 // planes are wave-uniform) and the direction word sign(x) ^ sign(d).  The lanes then walk their samples
-// in batch order: lowest set bit of the pending set, count and direction by bit extraction, one pulse
-// per lane and pass.  The wave moves to the next chunk when no lane has a pulse left; the noise
-// factors of eight passes come from one Philox call per lane and carry over chunk ends.
+// in batch order, one pulse per lane and pass: the lowest sample with a count left gives the direction,
+// its count is decremented in the bit slices (ripple borrow).  The wave moves to the next chunk when no
+// lane has a pulse left; the noise factors of eight passes come from one Philox call per lane and carry
+// over chunk ends.
 template <int KIND, bool MULT, int NB>
 __device__ __forceinline__ float pulsed_counted(const UpdateArgs &a, float w, const PulseCell<KIND> &cp, unsigned cell,
                                                 int i, int j, bool valid, int kmax) {
@@ -377,67 +375,82 @@ __device__ __forceinline__ float pulsed_counted(const UpdateArgs &a, float w, co
   const uint32_t *xpl = a.x_planes + j;
   const uint32_t *dpl = a.d_planes + i;
 
-  uint32_t cnt[NB];
+  float f[8];
 #pragma unroll
-  for (int n = 0; n < NB; ++n) cnt[n] = 0u;
-  uint32_t cur = 0u, same = 0u; // pending samples of the chunk; bit set: x and d have the same sign
-  int left = 0;
-  float slope = 0.0f, scale = 0.0f;
-  int c = -1;
-  uint32_t refill = 0;
-  bool finished = false;
-  while (!finished) {
-    float f[8];
-    noise_factors(f, std_, cell, refill, a);
-    ++refill;
+  for (int q = 0; q < 8; ++q) f[q] = 1.0f;
+  uint32_t pass = 0;
+  for (int c = 0; c < n_chunks; ++c) {
+    const unsigned base = (unsigned)c * slots;
+    uint32_t cnt[NB];
 #pragma unroll
-    for (int q = 0; q < 8; ++q) {
-      while (!__any((cur | (uint32_t)left) != 0u)) {
-        if (++c >= n_chunks) {
-          finished = true;
-          break;
-        }
-        const unsigned base = (unsigned)c * slots;
+    for (int n = 0; n < NB; ++n) cnt[n] = 0u;
 #pragma unroll
-        for (int n = 0; n < NB; ++n) cnt[n] = 0u;
+    for (int k = 0; k < (1 << NB) - 1; ++k) {
+      if (k < kmax) {
+        const uint32_t dk = dpl[(base + k) * ds]; // wave-uniform
+        if (dk) {
+          uint32_t carry = valid ? (dk & xpl[(base + k) * xs]) : 0u;
 #pragma unroll
-        for (int k = 0; k < (1 << NB) - 1; ++k) {
-          if (k < kmax) {
-            const uint32_t dk = dpl[(base + k) * ds]; // wave-uniform
-            if (dk) {
-              uint32_t carry = dk & xpl[(base + k) * xs];
-#pragma unroll
-              for (int n = 0; n < NB; ++n) {
-                const uint32_t t = cnt[n] & carry;
-                cnt[n] ^= carry;
-                carry = t;
-              }
-            }
+          for (int n = 0; n < NB; ++n) {
+            const uint32_t t = cnt[n] & carry;
+            cnt[n] ^= carry;
+            carry = t;
           }
         }
-        cur = cnt[0];
-#pragma unroll
-        for (int n = 1; n < NB; ++n) cur |= cnt[n];
-        if (!valid) cur = 0u;
-        same = ~(xpl[(base + slots - 1) * xs] ^ dpl[(base + slots - 1) * ds]) ^ lr_mask;
-      }
-      if (finished) break;
-      if (left == 0 && cur != 0u) {
-        const int bit = __ffs((int)cur) - 1;
-        cur &= cur - 1u;
-        left = (int)((cnt[0] >> bit) & 1u);
-#pragma unroll
-        for (int n = 1; n < NB; ++n) left += (int)(((cnt[n] >> bit) & 1u) << n);
-        // step down when x and d have the same sign and lr > 0
-        const bool down = ((same >> bit) & 1u) != 0u;
-        slope = down ? cp.slope_dn : cp.slope_up;
-        scale = down ? cp.scale_dn : cp.scale_up;
-      }
-      if (left > 0) {
-        w = pulse<KIND, MULT>(w, slope, scale, f[q], cp.lo, cp.hi);
-        --left;
       }
     }
+    uint32_t cur = cnt[0];
+#pragma unroll
+    for (int n = 1; n < NB; ++n) cur |= cnt[n];
+    if (!__any(cur != 0u)) continue;
+    // bit set: x and d have the same sign, which steps down when lr > 0
+    const uint32_t same = ~(xpl[(base + slots - 1) * xs] ^ dpl[(base + slots - 1) * ds]) ^ lr_mask;
+    // One pass: the lowest sample with a count left gives the direction, its count is decremented (ripple
+    // borrow), one pulse.  The passes are unrolled by eight so that each uses a fixed noise register; a
+    // chunk enters the unrolled loop where the previous one left it.
+#define RPU_PULSE_PASS(Q)                                                                       \
+  {                                                                                             \
+    const bool active = cur != 0u;                                                              \
+    const uint32_t m = cur & (0u - cur);                                                        \
+    uint32_t borrow = m;                                                                        \
+    _Pragma("unroll") for (int n = 0; n < NB; ++n) {                                            \
+      const uint32_t t = ~cnt[n] & borrow;                                                      \
+      cnt[n] ^= borrow;                                                                         \
+      borrow = t;                                                                               \
+    }                                                                                           \
+    cur = cnt[0];                                                                               \
+    _Pragma("unroll") for (int n = 1; n < NB; ++n) cur |= cnt[n];                               \
+    const bool down = (same & m) != 0u;                                                         \
+    const float slope = down ? cp.slope_dn : cp.slope_up;                                       \
+    const float scale = down ? cp.scale_dn : cp.scale_up;                                       \
+    const float wn = pulse<KIND, MULT>(w, slope, scale, f[Q], cp.lo, cp.hi);                    \
+    w = active ? wn : w;                                                                        \
+    ++pass;                                                                                     \
+    if (!__any(cur != 0u)) goto chunk_done;                                                     \
+  }
+    switch (pass & 7u) {
+      do {
+      case 0:
+        noise_factors(f, std_, cell, pass >> 3, a);
+        RPU_PULSE_PASS(0)
+      case 1:
+        RPU_PULSE_PASS(1)
+      case 2:
+        RPU_PULSE_PASS(2)
+      case 3:
+        RPU_PULSE_PASS(3)
+      case 4:
+        RPU_PULSE_PASS(4)
+      case 5:
+        RPU_PULSE_PASS(5)
+      case 6:
+        RPU_PULSE_PASS(6)
+      case 7:
+        RPU_PULSE_PASS(7)
+      } while (true);
+    }
+#undef RPU_PULSE_PASS
+  chunk_done:;
   }
   return w;
 }

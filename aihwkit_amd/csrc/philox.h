@@ -101,6 +101,22 @@ __device__ __forceinline__ void philox_normal8(uint32_t c0, uint32_t c1, uint32_
   box_muller16(r.v[3], out[6], out[7]);
 }
 
+// eight factors 1 + std * N(0,1) from one Philox call: box_muller16 with std folded into the radius
+// (std * sqrt(-2 ln u) = sqrt(-2 ln2 std^2 log2 u)) and the final multiply-add fused
+__device__ __forceinline__ void philox_factor8(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3,
+                                               PhiloxKey key, float std_, float out[8]) {
+  const Philox4 r = philox4x32_10(c0, c1, c2, c3, key.k0, key.k1);
+  const float m = -1.3862943611198906f * std_ * std_;
+#pragma unroll
+  for (int p = 0; p < 4; ++p) {
+    const float u = __builtin_fmaf((float)(r.v[p] >> 16), 1.0f / 65536.0f, 0.5f / 65536.0f);
+    const float t = (float)(r.v[p] & 0xffffu) * (1.0f / 65536.0f); // turns
+    const float rad = __builtin_amdgcn_sqrtf(m * __builtin_amdgcn_logf(u));
+    out[2 * p] = __builtin_fmaf(rad, __builtin_amdgcn_cosf(t), 1.0f);
+    out[2 * p + 1] = __builtin_fmaf(rad, __builtin_amdgcn_sinf(t), 1.0f);
+  }
+}
+
 __device__ __forceinline__ void philox_normal4(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3,
                                                PhiloxKey key, float out[4]) {
   const Philox4 r = philox4x32_10(c0, c1, c2, c3, key.k0, key.k1);
