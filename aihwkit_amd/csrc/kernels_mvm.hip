@@ -24,6 +24,7 @@
 namespace rpu_amd {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 namespace {
 
@@ -95,8 +96,8 @@ __device__ __forceinline__ bool tile_of(const MvmArgs &a, int n, int n_act, int 
 // address-bound in the vector L1.  Mode 1 reads the weights directly: 32 consecutive outputs per half-wave
 // and k are one line.  Out-of-range rows / k are clamped to valid addresses: their products meet the zero
 // padding of the quantized inputs or are never stored.
-// PD = 2: software pipeline over two register sets (steps s + 1 and s + 2 in flight while step s is in
-// LDS), k_pad a multiple of 2 * KSTEP * WAVES; PD = 1: one register set, for short contractions.
+// PD = 2, 4: software pipeline with the global loads of PD steps in flight, k_pad a multiple of
+// PD * KSTEP * WAVES; PD = 1: one register set, for short contractions.
 template <int PD, int WMODE>
 __device__ __forceinline__ void mvm_round_tile(const MvmArgs &a, int round, int tile_o, int tile_b, int n_act,
                                                float (*red)[16][64], float *stage) {
@@ -141,14 +142,14 @@ __device__ __forceinline__ void mvm_round_tile(const MvmArgs &a, int round, int 
 #pragma unroll
   for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
 
-  auto gload = [&](int s, float4 (&gx)[4], float4 (&gw)[4], float (&wd)[16]) {
+  auto gload = [&](int s, f32x4 (&gx)[4], f32x4 (&gw)[4], float (&wd)[16]) {
     const int k0 = s * KSTEP;
 #pragma unroll
-    for (int t = 0; t < 4; ++t) gx[t] = *reinterpret_cast<const float4 *>(x_src[t] + k0);
+    for (int t = 0; t < 4; ++t) gx[t] = *reinterpret_cast<const f32x4 *>(x_src[t] + k0);
     if (WMODE == 0) {
       const int kc = min(k0 + st_chunk, K - 4); // K % 16 == 0: past K the inputs are zero padding
 #pragma unroll
-      for (int t = 0; t < 4; ++t) gw[t] = *reinterpret_cast<const float4 *>(w_src[t] + kc);
+      for (int t = 0; t < 4; ++t) gw[t] = *reinterpret_cast<const f32x4 *>(w_src[t] + kc);
     } else if (WMODE == 1) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
@@ -163,22 +164,22 @@ __device__ __forceinline__ void mvm_round_tile(const MvmArgs &a, int round, int 
       }
     }
   };
-  auto lds_store = [&](const float4 (&gx)[4], const float4 (&gw)[4]) {
+  auto lds_store = [&](const f32x4 (&gx)[4], const f32x4 (&gw)[4]) {
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
       const int off = (t * 8 + st_row) * LDS_ROW + st_chunk;
-      *reinterpret_cast<float4 *>(stage_x + off) = gx[t];
-      if (WMODE == 0) *reinterpret_cast<float4 *>(stage_w + off) = gw[t];
+      *reinterpret_cast<f32x4 *>(stage_x + off) = gx[t];
+      if (WMODE == 0) *reinterpret_cast<f32x4 *>(stage_w + off) = gw[t];
     }
   };
   auto lds_read = [&](float (&xd)[16], float (&wd)[16]) {
 #pragma unroll
     for (int v4 = 0; v4 < 4; ++v4) {
       const int off = r * LDS_ROW + h * 16 + v4 * 4;
-      const float4 tx = *reinterpret_cast<const float4 *>(stage_x + off);
+      const f32x4 tx = *reinterpret_cast<const f32x4 *>(stage_x + off);
       xd[v4 * 4 + 0] = tx.x; xd[v4 * 4 + 1] = tx.y; xd[v4 * 4 + 2] = tx.z; xd[v4 * 4 + 3] = tx.w;
       if (WMODE == 0) {
-        const float4 tw = *reinterpret_cast<const float4 *>(stage_w + off);
+        const f32x4 tw = *reinterpret_cast<const f32x4 *>(stage_w + off);
         wd[v4 * 4 + 0] = tw.x; wd[v4 * 4 + 1] = tw.y; wd[v4 * 4 + 2] = tw.z; wd[v4 * 4 + 3] = tw.w;
       }
     }
@@ -188,35 +189,54 @@ __device__ __forceinline__ void mvm_round_tile(const MvmArgs &a, int round, int 
     for (int i = 0; i < 16; ++i) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(wd[i], xd[i], acc, 0, 0, 0);
   };
 
-  if (PD == 2) {
-    // register sets A and B alternate; the weights of mode 1 / 2 live in wa / wb until their step runs
-    float4 gxa[4], gwa[4], gxb[4], gwb[4];
-    float wa[16], wb[16], xc[16], wc[16];
-    gload(s_begin, gxa, gwa, wa);
-    gload(s_begin + 1, gxb, gwb, wb);
-    lds_store(gxa, gwa);
-    for (int s = s_begin; s < s_end; s += 2) {
-      // step s (set A is in LDS)
-      lds_read(xc, wc);
-      if (WMODE != 0) {
-#pragma unroll
-        for (int i = 0; i < 16; ++i) wc[i] = wa[i];
-      }
-      gload(min(s + 2, s_end - 1), gxa, gwa, wa);
-      mfma16(wc, xc);
-      lds_store(gxb, gwb);
-      // step s + 1 (set B is in LDS)
-      lds_read(xc, wc);
-      if (WMODE != 0) {
-#pragma unroll
-        for (int i = 0; i < 16; ++i) wc[i] = wb[i];
-      }
-      gload(min(s + 3, s_end - 1), gxb, gwb, wb);
-      mfma16(wc, xc);
-      lds_store(gxa, gwa);
+  if constexpr (PD >= 2) {
+    // PD register sets hold the global loads of the next PD steps; the operand registers are double
+    // buffered, so the LDS round trip of step t + 1 and the loads of step t + 1 + PD are issued ahead
+    // of the 16 MFMAs of step t and complete underneath them.
+    f32x4 gx0[4], gw0[4], gx1[4], gw1[4], gx2[4], gw2[4], gx3[4], gw3[4];
+    float wr0[16], wr1[16], wr2[16], wr3[16];
+    float xc0[16], wc0[16], xc1[16], wc1[16];
+    // step T runs from the operand registers (XC, WC); step T + 1 moves from register set (GX, GW, WR)
+    // through LDS into (XN, WN) and the set is refilled with step T + 1 + PD
+#define RPU_MVM_STEP(T, GX, GW, WR, XC, WC, XN, WN)                      \
+  {                                                                      \
+    lds_store(GX, GW);                                                   \
+    if (WMODE != 0) {                                                    \
+      _Pragma("unroll") for (int i = 0; i < 16; ++i) WN[i] = WR[i];      \
+    }                                                                    \
+    gload(min((T) + 1 + PD, s_end - 1), GX, GW, WR);                     \
+    lds_read(XN, WN);                                                    \
+    __builtin_amdgcn_sched_barrier(0);                                   \
+    mfma16(WC, XC);                                                      \
+    __builtin_amdgcn_sched_barrier(0);                                   \
+  }
+    gload(s_begin, gx0, gw0, wr0);
+    gload(min(s_begin + 1, s_end - 1), gx1, gw1, wr1);
+    if constexpr (PD == 4) {
+      gload(min(s_begin + 2, s_end - 1), gx2, gw2, wr2);
+      gload(min(s_begin + 3, s_end - 1), gx3, gw3, wr3);
     }
+    lds_store(gx0, gw0);
+    lds_read(xc0, wc0);
+    if (WMODE != 0) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) wc0[i] = wr0[i];
+    }
+    gload(min(s_begin + PD, s_end - 1), gx0, gw0, wr0);
+    for (int s = s_begin; s < s_end; s += PD) {
+      if constexpr (PD == 4) {
+        RPU_MVM_STEP(s, gx1, gw1, wr1, xc0, wc0, xc1, wc1)
+        RPU_MVM_STEP(s + 1, gx2, gw2, wr2, xc1, wc1, xc0, wc0)
+        RPU_MVM_STEP(s + 2, gx3, gw3, wr3, xc0, wc0, xc1, wc1)
+        RPU_MVM_STEP(s + 3, gx0, gw0, wr0, xc1, wc1, xc0, wc0)
+      } else {
+        RPU_MVM_STEP(s, gx1, gw1, wr1, xc0, wc0, xc1, wc1)
+        RPU_MVM_STEP(s + 1, gx0, gw0, wr0, xc1, wc1, xc0, wc0)
+      }
+    }
+#undef RPU_MVM_STEP
   } else {
-    float4 gx[4], gw[4];
+    f32x4 gx[4], gw[4];
     float wn[16], xc[16], wc[16];
     gload(s_begin, gx, gw, wn);
     for (int s = s_begin; s < s_end; ++s) {
@@ -534,7 +554,7 @@ int mvm_max_rounds(const IoDev &io) {
 
 // prefetch depth used for a contraction length: deep for long contractions, where each of the few
 // resident waves must cover the memory latency alone
-static int mvm_prefetch_depth(int K) { return K >= 256 ? 2 : 1; }
+static int mvm_prefetch_depth(int K) { return K >= 512 ? 4 : (K >= 256 ? 2 : 1); }
 
 int mvm_k_pad(int K) {
   const int unit = KSTEP * WAVES * mvm_prefetch_depth(K);
@@ -557,18 +577,23 @@ void launch_mvm_round(const MvmArgs &a, hipStream_t s) {
   const int per = (tiles_o + 7) / 8;
   const int tiles_b = (a.m_batch + TILE - 1) / TILE;
   const dim3 grid(8 * per * tiles_b);
-  const bool deep = mvm_prefetch_depth(a.K) == 2;
+  const int depth = mvm_prefetch_depth(a.K);
   const int mode = weight_mode(a);
+#define RPU_LAUNCH_ROUND(PD, WMODE) hipLaunchKernelGGL((k_mvm_round<PD, WMODE>), grid, dim3(256), 0, s, a)
   if (mode == 0) {
-    if (deep) hipLaunchKernelGGL((k_mvm_round<2, 0>), grid, dim3(256), 0, s, a);
-    else hipLaunchKernelGGL((k_mvm_round<1, 0>), grid, dim3(256), 0, s, a);
+    if (depth == 4) RPU_LAUNCH_ROUND(4, 0);
+    else if (depth == 2) RPU_LAUNCH_ROUND(2, 0);
+    else RPU_LAUNCH_ROUND(1, 0);
   } else if (mode == 1) {
-    if (deep) hipLaunchKernelGGL((k_mvm_round<2, 1>), grid, dim3(256), 0, s, a);
-    else hipLaunchKernelGGL((k_mvm_round<1, 1>), grid, dim3(256), 0, s, a);
+    if (depth == 4) RPU_LAUNCH_ROUND(4, 1);
+    else if (depth == 2) RPU_LAUNCH_ROUND(2, 1);
+    else RPU_LAUNCH_ROUND(1, 1);
   } else {
-    if (deep) hipLaunchKernelGGL((k_mvm_round<2, 2>), grid, dim3(256), 0, s, a);
-    else hipLaunchKernelGGL((k_mvm_round<1, 2>), grid, dim3(256), 0, s, a);
+    if (depth == 4) RPU_LAUNCH_ROUND(4, 2);
+    else if (depth == 2) RPU_LAUNCH_ROUND(2, 2);
+    else RPU_LAUNCH_ROUND(1, 2);
   }
+#undef RPU_LAUNCH_ROUND
 }
 
 void launch_mvm_advance(const MvmArgs &a, hipStream_t s) {
