@@ -28,7 +28,10 @@ struct MvmState {
   int *hit_up;     // 1 + largest output index that hit the upper bound this round (0 = none)
   int *hit_lo;     // same for the lower bound
   int *list[2];    // ping-pong lists of samples that need another round
+  int *row[2];     // row[i][pos]: row of xq[i] that holds the quantized input of the sample at list[i][pos]
+  float *next_scale[2]; // next_scale[i][pos]: input scale that sample would use one round later (0: no such round)
   int *count;      // count[r] = number of samples in the list read by round r (r >= 1)
+  int *tile_done;  // tile_done[r * tiles_b + t] = workgroups of round r that have finished sample tile t
 };
 
 struct MvmArgs {
@@ -41,9 +44,10 @@ struct MvmArgs {
   int m_batch;
   int K, O;       // contraction length and number of outputs
   int k_pad;      // K rounded up to the step of the contraction kernel (mvm_k_pad)
-  float *xq[2];   // ping-pong scratch [samples of the round][k_pad]: DAC-quantized inputs, zero padded
+  float *xq[2];   // ping-pong scratch [rows][k_pad]: DAC-quantized inputs, zero padded (rows: see MvmState::row)
   int transposed; // 0: out[o] = sum_k W[o][k] in[k] (forward); 1: out[o] = sum_k W[k][o] in[k] (backward)
   int round;      // bound-management round, 0-based
+  int max_rounds; // rounds launched for this call (mvm_max_rounds)
   float alpha, beta; // only used when io.perfect: out = alpha * acc + beta * out
   IoDev io;
   MvmState st;
@@ -55,8 +59,6 @@ struct MvmArgs {
 void launch_mvm_init(const MvmArgs &a, hipStream_t s);
 // one round of DAC -> MFMA contraction -> ADC
 void launch_mvm_round(const MvmArgs &a, hipStream_t s);
-// after round `a.round`: decide which samples need another round and set up their scales
-void launch_mvm_advance(const MvmArgs &a, hipStream_t s);
 // number of rounds that can ever be needed with these IO settings
 int mvm_max_rounds(const IoDev &io);
 // row length of the quantized-input scratch for a contraction length K

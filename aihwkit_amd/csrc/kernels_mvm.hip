@@ -16,9 +16,11 @@
 //                  partial tiles are summed in a fixed order through LDS and each wave finishes 8 output
 //                  rows: noise, quantize, clip, bound bookkeeping, rescale, store.  Workgroups are numbered
 //                  so that the 8 XCDs each work on a contiguous band of output rows (own L2 slice of W).
-//   k_mvm_advance  after a round, one workgroup per sample of that round: decide whether the sample needs
-//                  another round and, if so, append it to the next round's list and re-quantize its row
-//                  with the halved input range into the other scratch matrix.
+//                  With bound management a workgroup first writes its share of the tile's input rows as the
+//                  next round would quantize them (halved input range) into the other scratch matrix, and the
+//                  last workgroup to finish a sample tile (a device-scope counter per tile and round) decides
+//                  which of its 32 samples need that round and appends them to its list; no kernel sits
+//                  between two rounds.
 #include "kernels.h"
 
 namespace rpu_amd {
@@ -85,6 +87,119 @@ __device__ __forceinline__ bool tile_of(const MvmArgs &a, int n, int n_act, int 
   return tile_o < tiles_o && tile_b * TILE < n_act;
 }
 
+// ADC stage for outputs o0 .. o0 + 3 of sample b: v holds the analog sums (rpu_forward_backward_pass.cpp:666-719)
+// up / lo return 1 + the largest output index that hit the upper / lower ADC bound (0: none).
+__device__ __forceinline__ void mvm_finish_outputs(const MvmArgs &a, int round, int b, float fin, int o0, float (&v)[4],
+                                                   int &up, int &lo) {
+  up = 0;
+  lo = 0;
+  float *out_p = a.out + (long)b * a.out_sb + (long)o0 * a.out_so;
+  if (a.io.perfect) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      if (o0 + q < a.O) {
+        float res = a.alpha * v[q];
+        if (a.beta != 0.0f) res += a.beta * out_p[(long)q * a.out_so];
+        out_p[(long)q * a.out_so] = res;
+      }
+    }
+    return;
+  }
+
+  if (fin == 0.0f) { // zero input: the reference short-cuts to a zero output
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      if (o0 + q < a.O) out_p[(long)q * a.out_so] = 0.0f;
+    }
+    return;
+  }
+
+  float nz[4] = {0.f, 0.f, 0.f, 0.f};
+  if (a.io.out_noise > 0.0f) {
+    philox_normal4((uint32_t)(o0 >> 2), (uint32_t)b, a.call, RNG_OUT_NOISE | ((uint32_t)round << 8), a.key, nz);
+  }
+  const float bound = a.io.out_bound;
+  int hit_u = 0, hit_l = 0;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    float y = v[q];
+    if (a.io.out_asym > 0.0f) y = y < 0.0f ? y * (1.0f - a.io.out_asym) : y;
+    if (a.io.out_noise > 0.0f) y += a.io.out_noise * nz[q];
+    if (a.io.out_res > 0.0f) {
+      float qq = y / a.io.out_res;
+      if (a.io.out_sto_round) {
+        const Philox4 rr = philox4x32_10((uint32_t)(o0 + q), (uint32_t)b, a.call, RNG_OUT_SR | ((uint32_t)round << 8), a.key.k0, a.key.k1);
+        qq = qq + (u32_to_uniform(rr.v[0]) - 0.5f);
+      }
+      y = rintf(qq) * a.io.out_res;
+    }
+    const bool over = y > bound, under = y < -bound;
+    y = over ? bound : (under ? -bound : y);
+    const bool counts = o0 + q < a.O;
+    hit_u = (over && counts) ? o0 + q + 1 : hit_u;
+    hit_l = (under && counts) ? o0 + q + 1 : hit_l;
+    v[q] = y * fin;
+  }
+  up = hit_u;
+  lo = hit_l;
+  if (a.out_so == 1 && (o0 + 3) < a.O && ((((uintptr_t)out_p) & 15) == 0)) {
+    *reinterpret_cast<float4 *>(out_p) = make_float4(v[0], v[1], v[2], v[3]);
+  } else {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      if (o0 + q < a.O) out_p[(long)q * a.out_so] = v[q];
+    }
+  }
+}
+
+// Instruction order of one pipelined step (a hint to the scheduler): the 16 MFMAs are spread over the step with
+// the LDS writes of the next step's tiles between the first ones and its global loads and LDS reads
+// between the others, so that the LDS and memory pipes work underneath the matrix pipe of the same wave.
+template <int WMODE>
+__device__ __forceinline__ void mvm_step_schedule() {
+#define RPU_SG(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)
+#define RPU_SG_MFMA 0x008
+#define RPU_SG_VMEM 0x020
+#define RPU_SG_DSR 0x100
+#define RPU_SG_DSW 0x200
+  if (WMODE == 0) { // per step: 8 LDS writes, 8 global loads, 8 LDS reads
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      RPU_SG(RPU_SG_MFMA, 1);
+      RPU_SG(RPU_SG_DSW, 1);
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      RPU_SG(RPU_SG_MFMA, 1);
+      RPU_SG(RPU_SG_VMEM, 1);
+      RPU_SG(RPU_SG_DSR, 1);
+    }
+  } else { // per step: 4 LDS writes, 20 global loads, 4 LDS reads
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      RPU_SG(RPU_SG_MFMA, 1);
+      RPU_SG(RPU_SG_DSW, 1);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      RPU_SG(RPU_SG_MFMA, 1);
+      RPU_SG(RPU_SG_VMEM, 2);
+      RPU_SG(RPU_SG_DSR, 1);
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      RPU_SG(RPU_SG_MFMA, 1);
+      RPU_SG(RPU_SG_VMEM, 2);
+    }
+  }
+#undef RPU_SG
+#undef RPU_SG_MFMA
+#undef RPU_SG_VMEM
+#undef RPU_SG_DSR
+#undef RPU_SG_DSW
+  __builtin_amdgcn_sched_barrier(0);
+}
+
 // WMODE = how the weight operand is addressed:
 //   0  contraction index contiguous (forward), rows 16-byte aligned, K a multiple of 16
 //   1  output index contiguous (backward: W is read transposed in place)
@@ -132,7 +247,8 @@ __device__ __forceinline__ void mvm_round_tile(const MvmArgs &a, int round, int 
   for (int t = 0; t < 4; ++t) {
     const int row = t * 8 + st_row;
     const int slot = min(tile_b * TILE + row, n_act - 1);
-    x_src[t] = xq + (long)slot * a.k_pad + st_chunk;
+    const int xrow = (round > 0) ? a.st.row[round & 1][slot] : slot;
+    x_src[t] = xq + (long)xrow * a.k_pad + st_chunk;
     const int o = min(tile_o * TILE + row, a.O - 1);
     w_src[t] = a.w + (long)o * a.x_size;
   }
@@ -141,6 +257,14 @@ __device__ __forceinline__ void mvm_round_tile(const MvmArgs &a, int round, int 
   floatx16 acc;
 #pragma unroll
   for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
+
+  // sample of this lane's output column and its output factor: fetched now, used by the ADC stage
+  int b_out = slot_in;
+  float fin_out = 1.0f;
+  if (!a.io.perfect && b_ok) {
+    if (round > 0) b_out = a.st.list[round & 1][slot_in];
+    fin_out = a.st.fin[b_out];
+  }
 
   auto gload = [&](int s, f32x4 (&gx)[4], f32x4 (&gw)[4], float (&wd)[16]) {
     const int k0 = s * KSTEP;
@@ -206,9 +330,8 @@ __device__ __forceinline__ void mvm_round_tile(const MvmArgs &a, int round, int 
     }                                                                    \
     gload(min((T) + 1 + PD, s_end - 1), GX, GW, WR);                     \
     lds_read(XN, WN);                                                    \
-    __builtin_amdgcn_sched_barrier(0);                                   \
     mfma16(WC, XC);                                                      \
-    __builtin_amdgcn_sched_barrier(0);                                   \
+    mvm_step_schedule<WMODE>();                                          \
   }
     gload(s_begin, gx0, gw0, wr0);
     gload(min(s_begin + 1, s_end - 1), gx1, gw1, wr1);
@@ -263,72 +386,29 @@ __device__ __forceinline__ void mvm_round_tile(const MvmArgs &a, int round, int 
     const int i = wave * 4 + q;
     v[q] = ((red[0][i][lane] + red[1][i][lane]) + red[2][i][lane]) + red[3][i][lane];
   }
-  if (!b_ok) return;
-  const int b = (round > 0) ? a.st.list[round & 1][slot_in] : slot_in;
   const int o0 = tile_o * TILE + wave * 8 + h * 4;
-  if (o0 >= a.O) return;
-
-  float *out_p = a.out + (long)b * a.out_sb + (long)o0 * a.out_so;
-  if (a.io.perfect) {
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      if (o0 + q < a.O) {
-        float res = a.alpha * v[q];
-        if (a.beta != 0.0f) res += a.beta * out_p[(long)q * a.out_so];
-        out_p[(long)q * a.out_so] = res;
-      }
-    }
-    return;
-  }
-
-  const float fin = a.st.fin[b];
-  if (fin == 0.0f) { // zero input: the reference short-cuts to a zero output
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      if (o0 + q < a.O) out_p[(long)q * a.out_so] = 0.0f;
-    }
-    return;
-  }
-
-  float nz[4] = {0.f, 0.f, 0.f, 0.f};
-  if (a.io.out_noise > 0.0f) {
-    philox_normal4((uint32_t)(o0 >> 2), (uint32_t)b, a.call, RNG_OUT_NOISE | ((uint32_t)round << 8), a.key, nz);
-  }
-  const bool with_bm = a.io.bound_management != RPU_BM_NONE;
-  const float bound = a.io.out_bound;
   int up = 0, lo = 0;
-#pragma unroll
-  for (int q = 0; q < 4; ++q) {
-    float y = v[q];
-    if (a.io.out_asym > 0.0f) y = y < 0.0f ? y * (1.0f - a.io.out_asym) : y;
-    if (a.io.out_noise > 0.0f) y += a.io.out_noise * nz[q];
-    if (a.io.out_res > 0.0f) {
-      float qq = y / a.io.out_res;
-      if (a.io.out_sto_round) {
-        const Philox4 rr = philox4x32_10((uint32_t)(o0 + q), (uint32_t)b, a.call, RNG_OUT_SR | ((uint32_t)round << 8), a.key.k0, a.key.k1);
-        qq = qq + (u32_to_uniform(rr.v[0]) - 0.5f);
+  if (b_ok && o0 < a.O) mvm_finish_outputs(a, round, b_out, fin_out, o0, v, up, lo);
+  if (!a.io.perfect && a.io.bound_management != RPU_BM_NONE) {
+    // saturation flags of the tile's 32 samples: combined in LDS, then one device-scope atomic per sample
+    // and bound.  The returned values are consumed so that the wave waits until the atomics have been
+    // performed before the workgroup signals its tile as finished (mvm_tile_finished).
+    int *hits = reinterpret_cast<int *>(&red[0][0][0]); // the partial sums have been consumed ...
+    __syncthreads();                                      // ... by every wave
+    if (threadIdx.x < 2 * TILE) hits[threadIdx.x] = 0;
+    __syncthreads();
+    if (up) atomicMax(&hits[r], up);
+    if (lo) atomicMax(&hits[TILE + r], lo);
+    __syncthreads();
+    if (threadIdx.x < 2 * TILE) {
+      const int t = threadIdx.x & (TILE - 1);
+      const int hit = hits[threadIdx.x];
+      const int slot = tile_b * TILE + t;
+      if (hit && slot < n_act) {
+        const int bs = (round > 0) ? a.st.list[round & 1][slot] : slot;
+        const int old = atomicMax(threadIdx.x < TILE ? &a.st.hit_up[bs] : &a.st.hit_lo[bs], hit);
+        asm volatile("" ::"v"(old));
       }
-      y = rintf(qq) * a.io.out_res;
-    }
-    if (y > bound) {
-      y = bound;
-      if (o0 + q < a.O) up = o0 + q + 1;
-    } else if (y < -bound) {
-      y = -bound;
-      if (o0 + q < a.O) lo = o0 + q + 1;
-    }
-    v[q] = y * fin;
-  }
-  if (with_bm) {
-    if (up) atomicMax(&a.st.hit_up[b], up);
-    if (lo) atomicMax(&a.st.hit_lo[b], lo);
-  }
-  if (a.out_so == 1 && (o0 + 3) < a.O && ((((uintptr_t)out_p) & 15) == 0)) {
-    *reinterpret_cast<float4 *>(out_p) = make_float4(v[0], v[1], v[2], v[3]);
-  } else {
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      if (o0 + q < a.O) out_p[(long)q * a.out_so] = v[q];
     }
   }
 }
@@ -359,12 +439,12 @@ __device__ __forceinline__ float block_reduce_sum(float v, float *sh) {
   return r;
 }
 
-// input scale and output factor of a round; returns the input scale
-__device__ __forceinline__ float set_round_scales(const MvmArgs &a, int b, float nm, float red) {
+// input scale of a round and the factor applied to its ADC output
+__device__ __forceinline__ float round_scales(const MvmArgs &a, float nm, float red, float &fin) {
   const IoDev &io = a.io;
   const bool use_nm = io.noise_management != RPU_NM_NONE;
   const bool bm = io.bound_management != RPU_BM_NONE;
-  float scale, fin;
+  float scale;
   if (a.transposed) {
     // backward: scale = 1 / nm ; result *= out_scale * nm
     if (use_nm && nm <= 0.0f) {
@@ -383,9 +463,38 @@ __device__ __forceinline__ float set_round_scales(const MvmArgs &a, int b, float
     if (bm) scale /= red;
     fin = io.out_scale / scale;
   }
+  return scale;
+}
+
+__device__ __forceinline__ float set_round_scales(const MvmArgs &a, int b, float nm, float red) {
+  float fin;
+  const float scale = round_scales(a, nm, red, fin);
   a.st.scale[b] = scale;
   a.st.fin[b] = fin;
   return scale;
+}
+
+// Noise-management value and reduction that sample b, now at (nm, red) with output factor fin, would use in
+// the round after `round`; false when the reduction limit is reached or the sample is short-cut to zero
+// (rpu_forward_backward_pass.cpp:944-983).
+__device__ __forceinline__ bool next_round_params(const MvmArgs &a, int round, int b, float fin, float &nm, float &red) {
+  const IoDev &io = a.io;
+  if (fin == 0.0f) return false;
+  const bool stop = ((int)red > io.max_bm_factor) || ((io.inp_res > 0.0f) && (red > io.max_bm_res / io.inp_res));
+  if (stop) return false;
+  red *= 2.0f;
+  if (round == 0 && io.bound_management == RPU_BM_ITERATIVE_WORST_CASE && io.noise_management != RPU_NM_ABS_MAX_NP_SUM) {
+    nm = a.st.nm_np[b];
+    red = 1.0f;
+  }
+  return true;
+}
+
+// input scale of the round after `round` for such a sample, 0 when there is none
+__device__ __forceinline__ float next_round_scale(const MvmArgs &a, int round, int b, float fin, float nm, float red) {
+  if (!next_round_params(a, round, b, fin, nm, red)) return 0.0f;
+  float fin_next;
+  return round_scales(a, nm, red, fin_next);
 }
 
 // state of round 0 and quantized input row of sample b; called by a whole workgroup
@@ -438,9 +547,15 @@ __device__ __forceinline__ void mvm_init_sample(const MvmArgs &a, int b, float *
     a.st.hit_up[b] = 0;
     a.st.hit_lo[b] = 0;
     sh_scale = set_round_scales(a, b, nm, 1.0f);
-    a.st.rounds[b] = (a.st.fin[b] == 0.0f) ? 0 : 1;
+    const float fin = a.st.fin[b];
+    a.st.rounds[b] = (fin == 0.0f) ? 0 : 1;
+    if (io.bound_management != RPU_BM_NONE) a.st.next_scale[0][b] = next_round_scale(a, 0, b, fin, nm, 1.0f);
   }
   if (b == 0 && threadIdx.x < 40) a.st.count[threadIdx.x] = 0;
+  {
+    const int n_done = 32 * ((a.m_batch + TILE - 1) / TILE);
+    for (int idx = b * blockDim.x + threadIdx.x; idx < n_done; idx += gridDim.x * blockDim.x) a.st.tile_done[idx] = 0;
+  }
   __syncthreads();
   write_dac_row(a, b, b, sh_scale, 0, a.xq[0]);
   __syncthreads(); // sh / sh_scale are reused by the caller's next sample
@@ -452,54 +567,97 @@ __global__ __launch_bounds__(256) void k_mvm_init(MvmArgs a) {
   mvm_init_sample(a, blockIdx.x, sh, &sh_scale);
 }
 
-// After round `round`, for the sample in `slot` of that round's list: samples whose ADC saturated get
-// another round unless the reduction limit is reached (rpu_forward_backward_pass.cpp:944-983).  Called by a
-// whole workgroup.
-__device__ __forceinline__ void mvm_advance_slot(const MvmArgs &a, int round, int slot, int *sh_pos_p, float *sh_scale_p) {
-  int &sh_pos = *sh_pos_p;
-  float &sh_scale = *sh_scale_p;
-  const int b = (round > 0) ? a.st.list[round & 1][slot] : slot;
-  if (threadIdx.x == 0) {
-    const IoDev &io = a.io;
-    int pos = -1;
-    const int up = a.st.hit_up[b], lo = a.st.hit_lo[b];
-    a.st.hit_up[b] = 0;
-    a.st.hit_lo[b] = 0;
-    // the CPU loop sets "failed" on an upper hit and *assigns* !bm_test_negative_bound on a lower hit,
-    // walking the outputs in index order: the last hit decides
-    const bool failed = io.bm_test_negative_bound ? (up > 0 || lo > 0) : (up > lo);
-    if (failed && a.st.fin[b] != 0.0f) {
-      float red = a.st.red[b];
-      const bool stop = ((int)red > io.max_bm_factor) || ((io.inp_res > 0.0f) && (red > io.max_bm_res / io.inp_res));
-      if (!stop) {
-        red *= 2.0f;
-        float nm = a.st.nm[b];
-        if (round == 0 && io.bound_management == RPU_BM_ITERATIVE_WORST_CASE &&
-            io.noise_management != RPU_NM_ABS_MAX_NP_SUM) {
-          nm = a.st.nm_np[b];
-          a.st.nm[b] = nm;
-          red = 1.0f;
-        }
-        a.st.red[b] = red;
-        a.st.rounds[b] += 1;
-        sh_scale = set_round_scales(a, b, nm, red);
-        pos = atomicAdd(&a.st.count[round + 1], 1);
-        a.st.list[(round + 1) & 1][pos] = b;
-      }
+// At the start of round `round`, the workgroups of a sample tile (one per output tile) each quantize a
+// 1 / tiles_o share of the tile's input rows with the input range the *next* round would use (next_scale),
+// into the other scratch matrix at the rows of this round's list positions.  Whether a sample needs that
+// round is only known when all of its outputs are done; writing the rows ahead costs a few elements per
+// thread and takes the re-quantization off the path between two rounds.
+__device__ __forceinline__ void mvm_prepare_next_rows(const MvmArgs &a, int round, int tile_o, int tile_b, int n_act) {
+  __shared__ float sh_next_scale[TILE];
+  __shared__ int sh_next_b[TILE];
+  if (threadIdx.x < TILE) {
+    const int slot = tile_b * TILE + threadIdx.x;
+    int b = 0;
+    float scale = 0.0f; // 0: the sample can have no further round
+    if (slot < n_act) {
+      b = (round > 0) ? a.st.list[round & 1][slot] : slot;
+      scale = a.st.next_scale[round & 1][slot];
     }
-    sh_pos = pos;
+    sh_next_b[threadIdx.x] = b;
+    sh_next_scale[threadIdx.x] = scale;
   }
   __syncthreads();
-  if (sh_pos >= 0) write_dac_row(a, b, sh_pos, sh_scale, round + 1, a.xq[(round + 1) & 1]);
-  __syncthreads();
+  const int tiles_o = (a.O + TILE - 1) / TILE;
+  const int chunk = (a.k_pad + tiles_o - 1) / tiles_o;
+  const int k_lo = tile_o * chunk;
+  const int k_hi = min(k_lo + chunk, a.k_pad);
+  float *dst = a.xq[(round + 1) & 1];
+  // a trip covers 32 k-values of all 32 rows: 8 threads-rows x 4 rows each
+  const int kq = threadIdx.x & 31, rq = threadIdx.x >> 5;
+  for (int k0 = k_lo; k0 < k_hi; k0 += 32) {
+    const int k = k0 + kq;
+    const bool k_ok = k < k_hi;
+    float xv[4], sc[4];
+    int bt[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      bt[i] = sh_next_b[4 * rq + i];
+      sc[i] = sh_next_scale[4 * rq + i];
+      xv[i] = (k_ok && sc[i] != 0.0f && k < a.K) ? a.in[(long)bt[i] * a.in_sb + (long)k * a.in_sk] : 0.0f;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if (k_ok && sc[i] != 0.0f) {
+        const float v = (k < a.K) ? dac_value(xv[i], sc[i], a.io, a.key, a.call, round + 1, bt[i], k) : 0.0f;
+        dst[(long)(tile_b * TILE + 4 * rq + i) * a.k_pad + k] = v;
+      }
+    }
+  }
 }
 
-__global__ __launch_bounds__(256) void k_mvm_advance(MvmArgs a) {
-  __shared__ int sh_pos;
-  __shared__ float sh_scale;
-  const int n_act = (a.round > 0) ? a.st.count[a.round] : a.m_batch;
-  if ((int)blockIdx.x >= n_act) return;
-  mvm_advance_slot(a, a.round, blockIdx.x, &sh_pos, &sh_scale);
+// After round `round`, for sample b at position `slot` of that round's list: a sample whose ADC saturated
+// gets another round unless the reduction limit is reached (rpu_forward_backward_pass.cpp:944-983); its
+// quantized row for that round was written by mvm_prepare_next_rows.  One thread per sample.
+__device__ __forceinline__ void mvm_advance_sample(const MvmArgs &a, int round, int b, int slot) {
+  const IoDev &io = a.io;
+  // the flags were raised with device-scope atomics by workgroups on any XCD: read and clear them the same way
+  const int up = atomicExch(&a.st.hit_up[b], 0);
+  const int lo = atomicExch(&a.st.hit_lo[b], 0);
+  // the CPU loop sets "failed" on an upper hit and *assigns* !bm_test_negative_bound on a lower hit,
+  // walking the outputs in index order: the last hit decides
+  const bool failed = io.bm_test_negative_bound ? (up > 0 || lo > 0) : (up > lo);
+  if (!failed) return;
+  float nm = a.st.nm[b], red = a.st.red[b];
+  if (!next_round_params(a, round, b, a.st.fin[b], nm, red)) return;
+  a.st.nm[b] = nm;
+  a.st.red[b] = red;
+  a.st.rounds[b] += 1;
+  set_round_scales(a, b, nm, red);
+  const int pos = atomicAdd(&a.st.count[round + 1], 1);
+  a.st.list[(round + 1) & 1][pos] = b;
+  a.st.row[(round + 1) & 1][pos] = slot;
+  a.st.next_scale[(round + 1) & 1][pos] = next_round_scale(a, round + 1, b, a.st.fin[b], nm, red);
+}
+
+// Called by every workgroup of a round once its outputs are stored and its saturation flags are raised.  The
+// workgroups of a sample tile (one per output tile, spread over the XCDs) count themselves off; the last one
+// decides for the 32 samples of the tile whether they need another round, so that the next round's kernel
+// can follow directly.
+__device__ __forceinline__ void mvm_tile_finished(const MvmArgs &a, int round, int tile_b, int n_act) {
+  __shared__ int sh_last;
+  const int tiles_o = (a.O + TILE - 1) / TILE;
+  const int tiles_b = (a.m_batch + TILE - 1) / TILE;
+  __syncthreads(); // all flag atomics of this workgroup have been performed
+  if (threadIdx.x == 0) {
+    const int prev = atomicAdd(&a.st.tile_done[round * tiles_b + tile_b], 1);
+    sh_last = (prev == tiles_o - 1) ? 1 : 0;
+  }
+  __syncthreads();
+  if (!sh_last) return;
+  if (threadIdx.x < TILE) {
+    const int slot = tile_b * TILE + threadIdx.x;
+    if (slot < n_act) mvm_advance_sample(a, round, (round > 0) ? a.st.list[round & 1][slot] : slot, slot);
+  }
 }
 
 template <int PD, int WMODE>
@@ -509,7 +667,10 @@ __global__ __launch_bounds__(256) void k_mvm_round(MvmArgs a) {
   const int n_act = (a.round > 0) ? a.st.count[a.round] : a.m_batch;
   int tile_o, tile_b;
   if (!tile_of(a, blockIdx.x, n_act, tile_o, tile_b)) return;
+  const bool more_rounds = a.round + 1 < a.max_rounds;
+  if (more_rounds) mvm_prepare_next_rows(a, a.round, tile_o, tile_b, n_act);
   mvm_round_tile<PD, WMODE>(a, a.round, tile_o, tile_b, n_act, red, stage);
+  if (more_rounds) mvm_tile_finished(a, a.round, tile_b, n_act);
 }
 
 __global__ void k_make_bias(const float *in, float *out, int m_batch, int x_size, int in_trans) {
@@ -594,10 +755,6 @@ void launch_mvm_round(const MvmArgs &a, hipStream_t s) {
     else RPU_LAUNCH_ROUND(1, 2);
   }
 #undef RPU_LAUNCH_ROUND
-}
-
-void launch_mvm_advance(const MvmArgs &a, hipStream_t s) {
-  hipLaunchKernelGGL(k_mvm_advance, dim3(a.m_batch), dim3(256), 0, s, a);
 }
 
 void launch_make_bias(const float *in, float *out, int m_batch, int x_size, int in_trans, hipStream_t s) {

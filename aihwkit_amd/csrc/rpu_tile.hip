@@ -92,8 +92,8 @@ struct Tile {
   hipStream_t last_stream = nullptr;
   DevBuf<float> d_w, d_wmax, d_wmin, d_sup, d_sdown, d_slup, d_sldown;
   // MVM scratch
-  DevBuf<float> s_nm, s_nmnp, s_red, s_scale, s_fin, s_bias, s_xq0, s_xq1;
-  DevBuf<int> s_rounds, s_hitup, s_hitlo, s_list0, s_list1, s_count;
+  DevBuf<float> s_nsc0, s_nsc1, s_nm, s_nmnp, s_red, s_scale, s_fin, s_bias, s_xq0, s_xq1;
+  DevBuf<int> s_rounds, s_hitup, s_hitlo, s_list0, s_list1, s_row0, s_row1, s_count, s_tiledone;
   // update scratch
   DevBuf<int> u_bl;
   DevBuf<float> u_a, u_b, u_xval, u_dval;
@@ -145,8 +145,8 @@ struct Tile {
   void release_all() {
     d_w.release(); d_wmax.release(); d_wmin.release(); d_sup.release(); d_sdown.release();
     d_slup.release(); d_sldown.release();
-    s_nm.release(); s_nmnp.release(); s_red.release(); s_scale.release(); s_fin.release(); s_bias.release(); s_xq0.release(); s_xq1.release();
-    s_rounds.release(); s_hitup.release(); s_hitlo.release(); s_list0.release(); s_list1.release(); s_count.release();
+    s_nsc0.release(); s_nsc1.release(); s_nm.release(); s_nmnp.release(); s_red.release(); s_scale.release(); s_fin.release(); s_bias.release(); s_xq0.release(); s_xq1.release();
+    s_rounds.release(); s_hitup.release(); s_hitlo.release(); s_list0.release(); s_list1.release(); s_row0.release(); s_row1.release(); s_count.release(); s_tiledone.release();
     u_bl.release(); u_a.release(); u_b.release(); u_xval.release(); u_dval.release(); u_xw.release(); u_dw.release();
     u_xpl.release(); u_dpl.release(); u_kmax.release();
   }
@@ -210,9 +210,10 @@ struct Tile {
 
   void ensure_mvm_scratch(int B) {
     const size_t n = (size_t)B;
-    s_nm.ensure(n); s_nmnp.ensure(n); s_red.ensure(n); s_scale.ensure(n); s_fin.ensure(n);
-    s_rounds.ensure(n); s_hitup.ensure(n); s_hitlo.ensure(n); s_list0.ensure(n); s_list1.ensure(n);
+    s_nsc0.ensure(n); s_nsc1.ensure(n); s_nm.ensure(n); s_nmnp.ensure(n); s_red.ensure(n); s_scale.ensure(n); s_fin.ensure(n);
+    s_rounds.ensure(n); s_hitup.ensure(n); s_hitlo.ensure(n); s_list0.ensure(n); s_list1.ensure(n); s_row0.ensure(n); s_row1.ensure(n);
     s_count.ensure(64);
+    s_tiledone.ensure((size_t)32 * ((n + 31) / 32));
   }
 
   IoDev io_dev(const IOPar &io) const {
@@ -244,9 +245,12 @@ struct Tile {
     a.io = io_dev(io);
     a.alpha = io.p.out_scale; a.beta = 0.0f;
     a.key = key(); a.call = call++;
+    a.st.next_scale[0] = s_nsc0.p; a.st.next_scale[1] = s_nsc1.p;
     a.st.nm = s_nm.p; a.st.nm_np = s_nmnp.p; a.st.red = s_red.p; a.st.scale = s_scale.p; a.st.fin = s_fin.p;
     a.st.rounds = s_rounds.p; a.st.hit_up = s_hitup.p; a.st.hit_lo = s_hitlo.p;
-    a.st.list[0] = s_list0.p; a.st.list[1] = s_list1.p; a.st.count = s_count.p;
+    a.st.list[0] = s_list0.p; a.st.list[1] = s_list1.p; a.st.row[0] = s_row0.p; a.st.row[1] = s_row1.p;
+    a.st.count = s_count.p;
+    a.st.tile_done = s_tiledone.p;
     a.k_pad = mvm_k_pad(K);
     s_xq0.ensure((size_t)B * a.k_pad);
     if (!io.perfect && io.p.bound_management != RPU_BM_NONE) s_xq1.ensure((size_t)B * a.k_pad);
@@ -283,15 +287,13 @@ struct Tile {
     } else {
       launch_mvm_init(a, s);
       prof_mark(s, "mvm_init");
-      const int rounds = mvm_max_rounds(a.io);
-      for (int r = 0; r < rounds; ++r) {
+      // every round after the first works on the samples whose ADC saturated in the one before; the
+      // last workgroup to finish a sample tile sets up the next round for that tile
+      a.max_rounds = mvm_max_rounds(a.io);
+      for (int r = 0; r < a.max_rounds; ++r) {
         a.round = r;
         launch_mvm_round(a, s);
         prof_mark(s, "mvm_round");
-        if (r + 1 < rounds) {
-          launch_mvm_advance(a, s);
-          prof_mark(s, "mvm_advance");
-        }
       }
     }
     if (transposed && bias) launch_drop_bias(s_bias.p, final_out, B, X, out_trans ? 1 : 0, s);
