@@ -366,7 +366,7 @@ __device__ __forceinline__ void noise_factors(float (&f)[8], float std_, unsigne
 // over chunk ends.
 template <int KIND, bool MULT, int NB>
 __device__ __forceinline__ float pulsed_counted(const UpdateArgs &a, float w, const PulseCell<KIND> &cp, unsigned cell,
-                                                int i, int j, bool valid, int kmax) {
+                                                int i, int j, bool valid, int kmax, float *noise_lds) {
   const float std_ = a.dev.dw_min_std;
   const uint32_t lr_mask = a.lr < 0.0f ? 0xffffffffu : 0u;
   const int n_chunks = a.n_chunks;
@@ -375,9 +375,6 @@ __device__ __forceinline__ float pulsed_counted(const UpdateArgs &a, float w, co
   const uint32_t *xpl = a.x_planes + j;
   const uint32_t *dpl = a.d_planes + i;
 
-  float f[8];
-#pragma unroll
-  for (int q = 0; q < 8; ++q) f[q] = 1.0f;
   uint32_t pass = 0;
   for (int c = 0; c < n_chunks; ++c) {
     const unsigned base = (unsigned)c * slots;
@@ -406,51 +403,35 @@ __device__ __forceinline__ float pulsed_counted(const UpdateArgs &a, float w, co
     // bit set: x and d have the same sign, which steps down when lr > 0
     const uint32_t same = ~(xpl[(base + slots - 1) * xs] ^ dpl[(base + slots - 1) * ds]) ^ lr_mask;
     // One pass: the lowest sample with a count left gives the direction, its count is decremented (ripple
-    // borrow), one pulse.  The passes are unrolled by eight so that each uses a fixed noise register; a
-    // chunk enters the unrolled loop where the previous one left it.
-#define RPU_PULSE_PASS(Q)                                                                       \
-  {                                                                                             \
-    const bool active = cur != 0u;                                                              \
-    const uint32_t m = cur & (0u - cur);                                                        \
-    uint32_t borrow = m;                                                                        \
-    _Pragma("unroll") for (int n = 0; n < NB; ++n) {                                            \
-      const uint32_t t = ~cnt[n] & borrow;                                                      \
-      cnt[n] ^= borrow;                                                                         \
-      borrow = t;                                                                               \
-    }                                                                                           \
-    cur = cnt[0];                                                                               \
-    _Pragma("unroll") for (int n = 1; n < NB; ++n) cur |= cnt[n];                               \
-    const bool down = (same & m) != 0u;                                                         \
-    const float slope = down ? cp.slope_dn : cp.slope_up;                                       \
-    const float scale = down ? cp.scale_dn : cp.scale_up;                                       \
-    const float wn = pulse<KIND, MULT>(w, slope, scale, f[Q], cp.lo, cp.hi);                    \
-    w = active ? wn : w;                                                                        \
-    ++pass;                                                                                     \
-    if (!__any(cur != 0u)) goto chunk_done;                                                     \
-  }
-    switch (pass & 7u) {
-      do {
-      case 0:
+    // borrow), one pulse.  The noise factors of eight passes are parked in LDS (one column per thread), so
+    // that a pass picks its factor by the wave-uniform pass number without unrolling across chunk ends.
+    do {
+      if ((pass & 7u) == 0u) {
+        float f[8];
         noise_factors(f, std_, cell, pass >> 3, a);
-        RPU_PULSE_PASS(0)
-      case 1:
-        RPU_PULSE_PASS(1)
-      case 2:
-        RPU_PULSE_PASS(2)
-      case 3:
-        RPU_PULSE_PASS(3)
-      case 4:
-        RPU_PULSE_PASS(4)
-      case 5:
-        RPU_PULSE_PASS(5)
-      case 6:
-        RPU_PULSE_PASS(6)
-      case 7:
-        RPU_PULSE_PASS(7)
-      } while (true);
-    }
-#undef RPU_PULSE_PASS
-  chunk_done:;
+#pragma unroll
+        for (int q = 0; q < 8; ++q) noise_lds[q * 256] = f[q];
+      }
+      const float fq = noise_lds[(pass & 7u) * 256];
+      ++pass;
+      const bool active = cur != 0u;
+      const uint32_t m = cur & (0u - cur);
+      uint32_t borrow = m;
+#pragma unroll
+      for (int n = 0; n < NB; ++n) {
+        const uint32_t t = ~cnt[n] & borrow;
+        cnt[n] ^= borrow;
+        borrow = t;
+      }
+      cur = cnt[0];
+#pragma unroll
+      for (int n = 1; n < NB; ++n) cur |= cnt[n];
+      const bool down = (same & m) != 0u;
+      const float slope = down ? cp.slope_dn : cp.slope_up;
+      const float scale = down ? cp.scale_dn : cp.scale_up;
+      const float wn = pulse<KIND, MULT>(w, slope, scale, fq, cp.lo, cp.hi);
+      w = active ? wn : w;
+    } while (__any(cur != 0u));
   }
   return w;
 }
@@ -549,8 +530,9 @@ __global__ __launch_bounds__(256) void k_update_pulsed(UpdateArgs a) {
   cp.load(a.dev, cell);
   float w = a.w[cell];
   const int kmax = a.kmax[a.kmax_slot];
-  if (kmax <= 3) w = pulsed_counted<KIND, MULT, 2>(a, w, cp, cell, i, j, valid, kmax);
-  else if (kmax <= 7) w = pulsed_counted<KIND, MULT, 3>(a, w, cp, cell, i, j, valid, kmax);
+  __shared__ float noise[8 * 256]; // noise[q][thread]: a thread only ever touches its own column
+  if (kmax <= 3) w = pulsed_counted<KIND, MULT, 2>(a, w, cp, cell, i, j, valid, kmax, noise + threadIdx.x);
+  else if (kmax <= 7) w = pulsed_counted<KIND, MULT, 3>(a, w, cp, cell, i, j, valid, kmax, noise + threadIdx.x);
   else w = pulsed_gather<KIND, MULT>(a, w, cp, cell, i, j, valid, kmax);
   if (valid) a.w[cell] = w;
 }
