@@ -33,8 +33,14 @@ RPU_HD Philox4 philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3,
     const uint64_t p1 = (uint64_t)M1 * (uint64_t)c2;
     const uint32_t hi0 = (uint32_t)(p0 >> 32), lo0 = (uint32_t)p0;
     const uint32_t hi1 = (uint32_t)(p1 >> 32), lo1 = (uint32_t)p1;
+#if defined(__HIP_DEVICE_COMPILE__)
+    // three-input xor in one instruction (v_bitop3_b32, truth table 0x96)
+    const uint32_t n0 = __builtin_amdgcn_bitop3_b32(hi1, c1, k0, 0x96);
+    const uint32_t n2 = __builtin_amdgcn_bitop3_b32(hi0, c3, k1, 0x96);
+#else
     const uint32_t n0 = hi1 ^ c1 ^ k0;
     const uint32_t n2 = hi0 ^ c3 ^ k1;
+#endif
     c0 = n0;
     c1 = lo1;
     c2 = n2;

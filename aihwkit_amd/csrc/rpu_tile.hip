@@ -115,6 +115,9 @@ struct Tile {
     prof_used = 0;
     prof_names.clear();
     prof_mark(s, nullptr);
+    // an empty bracket first: what two consecutive event records cost on this stream, for callers that want
+    // to take the bracket's own time out of the kernel figures
+    prof_mark(s, "_bracket");
   }
   void prof_mark(hipStream_t s, const char *name) {
     if (!profiling) return;

@@ -28,6 +28,14 @@ for _p in (ROOT, os.path.join(ROOT, "tests"), os.path.join(ROOT, "oracle")):
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
 FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix
 
+# HBM bytes per launch at configuration 2 from rocprofv3 counter runs of `bench.py --pmc` (FETCH_SIZE and
+# WRITE_SIZE in KiB per dispatch, one run each; the summaries are under profiles/).  A copy of 64 MiB in the
+# same runs reads FETCH_SIZE = 32784 and WRITE_SIZE = 65536, so FETCH_SIZE is scaled by 2.0 and WRITE_SIZE by 1.0.
+PMC_TRAFFIC_BYTES = {
+    "k_update_pulsed": (15532 * 2.0 + 4096 * 1.0) * 1024,
+    "k_mvm_round": (6800 * 2.0 + 2115 * 1.0) * 1024,  # a round over all 256 samples
+}
+
 
 def main() -> int:
     ap = argparse.ArgumentParser()
@@ -112,13 +120,18 @@ def main() -> int:
         return start.elapsed_time(end) / n
 
     def kernel_ms(fn, n_calls):
-        # per-kernel durations from HIP events recorded by the library on the launch stream
+        # Per-kernel durations from HIP events that the library records on the launch stream around each
+        # kernel.  The first bracket of a call is empty ("_bracket"): the time between two consecutive event
+        # records with nothing in between, taken out of every kernel's bracket.
         acc = {}
         for _ in range(n_calls):
             fn()
             for name, ms in tile.get_profile():
                 acc.setdefault(name, []).append(ms)
-        return {k: (float(np.sum(v)) / n_calls, len(v) // n_calls) for k, v in acc.items()}
+        bracket = float(np.mean(acc.pop("_bracket")))
+        out = {k: (float(np.sum(v)) / n_calls - bracket * (len(v) // n_calls), len(v) // n_calls) for k, v in acc.items()}
+        out["_bracket"] = (bracket, 1)
+        return out
 
     n = max(args.steps, 10)
     # forward / backward alone, on the initial weights (they do not change the tile)
@@ -175,12 +188,14 @@ def main() -> int:
                      "kernels_ms": {k: v[0] for k, v in prof_backward.items()}},
         "roofline": {"kernel": "k_update_pulsed", "bound": "hbm", "achieved": update_bytes / (k_update_ms * 1e-3) / 1e9,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": update_bytes / (k_update_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None,
+                     "frac": update_bytes / (k_update_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                     "traffic": PMC_TRAFFIC_BYTES["k_update_pulsed"] if args.config == 2 else None,
                      "algorithmic_bytes": update_bytes, "kernel_ms": k_update_ms},
         "roofline_forward": {"kernel": "k_mvm_round (all rounds of a call)", "bound": "mfma",
                              "achieved": flops_per_call / (k_fwd_ms * 1e-3) / 1e12, "peak": FP32_MFMA_PEAK_TFLOPS,
                              "unit": "TFLOP/s", "frac": flops_per_call / (k_fwd_ms * 1e-3) / 1e12 / FP32_MFMA_PEAK_TFLOPS,
-                             "traffic": None, "algorithmic_flops": flops_per_call, "kernel_ms": k_fwd_ms},
+                             "traffic": PMC_TRAFFIC_BYTES["k_mvm_round"] if args.config == 2 else None,
+                             "algorithmic_flops": flops_per_call, "kernel_ms": k_fwd_ms},
         "roofline_backward": {"kernel": "k_mvm_round", "bound": "mfma",
                               "achieved": flops_per_call / (k_bwd_ms * 1e-3) / 1e12, "peak": FP32_MFMA_PEAK_TFLOPS,
                               "unit": "TFLOP/s", "frac": flops_per_call / (k_bwd_ms * 1e-3) / 1e12 / FP32_MFMA_PEAK_TFLOPS,
