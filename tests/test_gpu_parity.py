@@ -201,6 +201,75 @@ def test_stochastic_update_words_drive_the_oracle_to_the_same_weights(gpu_device
     assert np.abs(orc.get_weights() - np.clip(w, orc.get_hidden()[1], orc.get_hidden()[0])).max() > 1e-3
 
 
+@pytest.mark.parametrize("desired_bl", [1, 2, 3, 4, 7, 8, 13])
+@pytest.mark.parametrize("device", ["constant", "soft"])
+def test_short_bit_lines_words_drive_the_oracle_to_the_same_weights(gpu_device, device, desired_bl):
+    """Fixed bit-line lengths around the limits of the update kernel's pulse loops (counts kept in 2 or 3
+    bit slices up to 3 / 7 slots, packed-word gathers beyond), with pulse probabilities high enough that a
+    sample often has several coincidences; odd sizes leave idle lanes and a ragged last chunk."""
+    rng = np.random.default_rng(100 + desired_bl)
+    x_size, d_size, batch = 70, 37, 45
+    meta = make_meta(desired_bl=desired_bl, update_management=False, update_bl_management=False)
+    kw = dict(dw_min=0.002, dw_min_std=0.0, construction_seed=5, enforce_consistency=True)
+    dev = constant_step(**kw) if device == "constant" else soft_bounds(**kw)
+    host, orc, _ = build_pair(meta, dev, x_size, d_size, gpu=False)
+    w = rng.uniform(-0.5, 0.5, (d_size, x_size)).astype(np.float32)
+    host.set_weights(torch.from_numpy(w))
+    orc.set_weights(w)
+    gpu = tiles.CudaAnalogTile(host)
+    gpu.set_seed(11)
+    x = rng.uniform(-1, 1, (batch, x_size)).astype(np.float32)
+    d = rng.uniform(-1, 1, (batch, d_size)).astype(np.float32)
+    lr = 0.002 * desired_bl * 0.64  # A = B = sqrt(lr / (dw_min BL)) = 0.8
+    counts_seen = set()
+    for sign in (1.0, -1.0):
+        gpu.set_learning_rate(sign * lr)
+        orc.set_learning_rate(sign * lr)
+        gpu.update(cuda(x), cuda(d), False, False, False, False)
+        xw, dw, bl = (t.numpy() for t in gpu.get_update_words(batch))
+        assert np.all(bl == desired_bl)
+        n = np.bitwise_count((xw[:, None, :].view(np.uint32) & dw[:, :, None].view(np.uint32)) >> 1)
+        counts_seen |= set(np.unique(n).tolist())
+        orc.update_with_words(xw, dw, bl)
+        assert np.abs(gpu.get_weights().numpy() - orc.get_weights()).max() <= TOL
+    assert max(counts_seen) >= min(desired_bl, 3)  # samples with several coincidences did occur
+
+
+@pytest.mark.parametrize("device", ["constant", "soft"])
+def test_crossed_and_tight_bounds_clip_like_the_reference_order(gpu_device, device):
+    """ConstantStep clips min(w_max) then max(w_min), LinearStep max(w_min) then min(w_max): with hidden
+    parameters whose bounds are crossed (w_min > w_max) or equal, the order decides the result."""
+    rng = np.random.default_rng(77)
+    x_size, d_size, batch = 64, 32, 24
+    meta = make_meta(desired_bl=5, update_management=False, update_bl_management=False)
+    kw = dict(dw_min=0.01, dw_min_std=0.0, construction_seed=3, enforce_consistency=True)
+    dev = constant_step(**kw) if device == "constant" else soft_bounds(**kw)
+    host, orc, _ = build_pair(meta, dev, x_size, d_size, gpu=False)
+    hidden = host.get_hidden_parameters()
+    hi, lo = hidden[0].clone(), hidden[1].clone()
+    hidden[0][:, ::3] = lo[:, ::3] * 0.5   # upper bound below zero ...
+    hidden[1][:, ::3] = hi[:, ::3] * 0.5   # ... lower bound above zero: crossed
+    hidden[1][:, 1::3] = hidden[0][:, 1::3]  # equal bounds
+    host.set_hidden_parameters(hidden)
+    orc.set_hidden(hidden.numpy())
+    w = rng.uniform(-0.1, 0.1, (d_size, x_size)).astype(np.float32)
+    host.set_weights(torch.from_numpy(w))
+    gpu = tiles.CudaAnalogTile(host)
+    gpu.set_seed(2)
+    orc.set_weights(gpu.get_weights().numpy())  # both start from what the library's set_weights made of w
+    lr = 0.01 * 5 * 0.81
+    gpu.set_learning_rate(lr)
+    orc.set_learning_rate(lr)
+    x = rng.uniform(-1, 1, (batch, x_size)).astype(np.float32)
+    d = rng.uniform(-1, 1, (batch, d_size)).astype(np.float32)
+    gpu.update(cuda(x), cuda(d), False, False, False, False)
+    xw, dw, bl = (t.numpy() for t in gpu.get_update_words(batch))
+    orc.update_with_words(xw, dw, bl)
+    got, want = gpu.get_weights().numpy(), orc.get_weights()
+    assert np.abs(got - want).max() <= TOL
+    assert np.abs(want - w).max() > 1e-3
+
+
 def test_pulse_probabilities_saturate(gpu_device):
     """|v| * scale >= 1 gives all BL pulses, 0 gives none (the reference's bit-line maker test protocol)."""
     x_size, d_size, batch = 64, 64, 8
