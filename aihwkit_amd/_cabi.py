@@ -65,12 +65,35 @@ class TileConfig(C.Structure):
     _fields_ = [("f_io", IOParams), ("b_io", IOParams), ("up", UpdateParams), ("device", DeviceParams)]
 
 
+MAX_VECTOR_DEVICES = 4
+
+
+class TransferParams(C.Structure):
+    """``rpu_transfer_params``."""
+
+    _fields_ = [
+        ("n_devices", i32), ("construction_seed", u32), ("units_in_mbatch", i32), ("n_reads_per_transfer", i32),
+        ("no_self_transfer", i32), ("random_selection", i32), ("scale_transfer_lr", i32), ("scale_fast_lr", i32),
+        ("transfer_columns", i32),
+        ("gamma", f32), ("transfer_every", f32), ("with_reset_prob", f32), ("fast_lr", f32), ("transfer_lr", f32),
+        ("n_gamma_vec", i32), ("n_transfer_lr_vec", i32), ("n_transfer_every_vec", i32),
+        ("gamma_vec", f32 * MAX_VECTOR_DEVICES), ("transfer_lr_vec", f32 * MAX_VECTOR_DEVICES),
+        ("transfer_every_vec", f32 * MAX_VECTOR_DEVICES),
+        ("transfer_io", IOParams), ("transfer_up", UpdateParams),
+        ("fast_device", DeviceParams), ("rest_device", DeviceParams),
+    ]
+
+
 # every symbol include/rpu_amd.h declares: name -> (restype, argtypes)
 _P = C.c_void_p
 _FP = C.POINTER(C.c_float)
 SYMBOLS = {
     "rpu_tile_config_default": (C.c_int, [C.POINTER(TileConfig), C.c_int]),
     "rpu_tile_create": (C.c_int, [C.POINTER(_P), C.c_int, C.c_int, C.POINTER(TileConfig)]),
+    "rpu_transfer_params_default": (C.c_int, [C.POINTER(TransferParams), C.c_int]),
+    "rpu_tile_create_transfer": (C.c_int, [C.POINTER(_P), C.c_int, C.c_int, C.POINTER(TileConfig),
+                                           C.POINTER(TransferParams)]),
+    "rpu_tile_get_transfer_state": (C.c_int, [_P, C.POINTER(C.c_uint64), C.POINTER(C.c_int32)]),
     "rpu_tile_clone": (C.c_int, [C.POINTER(_P), _P]),
     "rpu_tile_to_device": (C.c_int, [_P, C.c_int]),
     "rpu_tile_destroy": (C.c_int, [_P]),

@@ -124,4 +124,15 @@ void launch_implicit_counts(const UpdateArgs &a, int32_t *counts, hipStream_t s)
 // clip weights into [w_min, w_max]
 void launch_clip(float *w, const float *w_min, const float *w_max, size_t n, hipStream_t s);
 
+// n_vec unit vectors of length `size`: row v is e_((start + v) % size)
+void launch_unit_vectors(float *out, int n_vec, int size, int start, hipStream_t s);
+
+// out = sum_k gamma[k] * w[k], k < n (VectorRPUDevice::reduceToWeights, rpu_vector_device.cpp:530-536)
+struct ReduceArgs {
+  const float *w[4];
+  float gamma[4];
+  int n;
+};
+void launch_reduce_weights(float *out, const ReduceArgs &r, size_t size, hipStream_t s);
+
 } // namespace rpu_amd

@@ -592,6 +592,23 @@ __global__ void k_clip(float *w, const float *w_min, const float *w_max, size_t 
   }
 }
 
+__global__ void k_unit_vectors(float *out, int n_vec, int size, int start) {
+  const long n = (long)n_vec * size;
+  for (long idx = blockIdx.x * (long)blockDim.x + threadIdx.x; idx < n; idx += (long)gridDim.x * blockDim.x) {
+    const int v = (int)(idx / size);
+    const int j = (int)(idx % size);
+    out[idx] = (j == (start + v) % size) ? 1.0f : 0.0f;
+  }
+}
+
+__global__ void k_reduce_weights(float *out, ReduceArgs r, size_t n) {
+  for (size_t idx = blockIdx.x * (size_t)blockDim.x + threadIdx.x; idx < n; idx += (size_t)gridDim.x * blockDim.x) {
+    float acc = 0.0f;
+    for (int k = 0; k < r.n; ++k) acc += r.gamma[k] * r.w[k][idx];
+    out[idx] = acc;
+  }
+}
+
 int grid_for(long total) {
   long blocks = (total + 255) / 256;
   if (blocks > 65536) blocks = 65536;
@@ -644,6 +661,14 @@ void launch_update_implicit(const UpdateArgs &a, hipStream_t s) {
 void launch_implicit_counts(const UpdateArgs &a, int32_t *counts, hipStream_t s) {
   const long total = (long)a.x_size * a.d_size * a.m_batch;
   hipLaunchKernelGGL(k_implicit_counts, dim3(grid_for(total)), dim3(256), 0, s, a, counts);
+}
+
+void launch_unit_vectors(float *out, int n_vec, int size, int start, hipStream_t s) {
+  hipLaunchKernelGGL(k_unit_vectors, dim3(grid_for((long)n_vec * size)), dim3(256), 0, s, out, n_vec, size, start);
+}
+
+void launch_reduce_weights(float *out, const ReduceArgs &r, size_t size, hipStream_t s) {
+  hipLaunchKernelGGL(k_reduce_weights, dim3(grid_for((long)size)), dim3(256), 0, s, out, r, size);
 }
 
 void launch_clip(float *w, const float *w_min, const float *w_max, size_t n, hipStream_t s) {

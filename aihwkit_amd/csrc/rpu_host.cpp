@@ -124,7 +124,7 @@ void UpdatePar::initialize() {
 
 void DevicePar::initialize() {
   if (p.kind < RPU_DEVICE_IDEAL || p.kind > RPU_DEVICE_SOFT_BOUNDS) {
-    throw RpuError("Unknown device kind.");
+    throw RpuError("Unknown device kind (a transfer compound is created with rpu_tile_create_transfer).");
   }
   if (p.kind == RPU_DEVICE_SOFT_BOUNDS) {
     // SoftBounds is LinearStep with zero step at the (actual) bounds (rpu_linearstep_device.h:68-80)
@@ -152,7 +152,27 @@ void DevicePar::initialize() {
   }
 }
 
+namespace {
+void populate_from(const DevicePar &dev, ConstructionRng &rng, int x_size, int d_size, DeviceArrays &a);
+}
+
 void DevicePar::populate(int x_size, int d_size, DeviceArrays &a) const {
+  ConstructionRng rng(p.construction_seed);
+  populate_from(*this, rng, x_size, d_size, a);
+}
+
+void populate_chain(const std::vector<DevicePar> &pars, unsigned int seed, int x_size, int d_size,
+                    std::vector<DeviceArrays> &out) {
+  ConstructionRng rng(seed);
+  out.assign(pars.size(), DeviceArrays());
+  for (size_t k = 0; k < pars.size(); ++k) populate_from(pars[k], rng, x_size, d_size, out[k]);
+}
+
+namespace {
+void populate_from(const DevicePar &dev, ConstructionRng &rng, int x_size, int d_size, DeviceArrays &a) {
+  const rpu_device_params &p = dev.p;
+  const auto pulsed = [&] { return dev.pulsed(); };
+  const auto linear = [&] { return dev.linear(); };
   const size_t n = (size_t)x_size * (size_t)d_size;
   a = DeviceArrays();
   if (!pulsed()) {
@@ -165,8 +185,6 @@ void DevicePar::populate(int x_size, int d_size, DeviceArrays &a) const {
   a.decay_scale.resize(n);
   a.diffusion_rate.resize(n);
   a.reset_bias.resize(n);
-
-  ConstructionRng rng(p.construction_seed);
 
   const float bias_up = p.up_down > 0.0f ? 0.0f : p.up_down;
   const float bias_down = p.up_down > 0.0f ? -p.up_down : 0.0f;
@@ -281,6 +299,81 @@ void DevicePar::populate(int x_size, int d_size, DeviceArrays &a) const {
     }
   }
 }
+} // namespace
+
+void TransferPar::initialize(int x_size, int d_size) {
+  const int n_dev = p.n_devices;
+  if (n_dev < 2) throw RpuError("Need at least 2 devices");
+  if (n_dev > RPU_MAX_VECTOR_DEVICES) throw RpuError("At most 4 devices in a transfer chain.");
+  if (p.random_selection) throw RpuError("random_selection is not provided.");
+  if (p.with_reset_prob > 0.0f) throw RpuError("with_reset_prob > 0 is not provided.");
+  devs.clear();
+  for (int k = 0; k < n_dev; ++k) {
+    DevicePar d;
+    d.p = k == 0 ? p.fast_device : p.rest_device;
+    d.initialize();
+    if (!d.pulsed()) throw RpuError("The devices of a transfer chain must be pulsed devices.");
+    devs.push_back(d);
+  }
+  in_size = p.transfer_columns ? x_size : d_size;
+  out_size = p.transfer_columns ? d_size : x_size;
+
+  // weightening of the devices (rpu_transfer_device.cpp:146-168)
+  gamma_vec.clear();
+  if (p.n_gamma_vec > 0) {
+    if (p.n_gamma_vec != n_dev) throw RpuError("If gamma_vec is set manually expect the same size as number of devices.");
+    float g = 0.0f;
+    for (int i = 0; i < n_dev; ++i) gamma_vec.push_back(p.gamma_vec[i]);
+    for (int i = 0; i < n_dev - 1; ++i) g += gamma_vec[i];
+    if (gamma_vec[n_dev - 1] == 0.0f) {
+      throw RpuError("Expect that last device has some constribution to the network weights. [otherwise why transfer?]");
+    }
+    p.gamma = g;
+  } else {
+    gamma_vec.resize(n_dev);
+    for (int i = 0; i < n_dev; ++i) gamma_vec[n_dev - i - 1] = powf(p.gamma, (float)i);
+  }
+  lr_vec.clear();
+  if (p.n_transfer_lr_vec > 0) {
+    if (p.n_transfer_lr_vec != n_dev) throw RpuError("Expect transfer_lr_vec of size n_devices.");
+    for (int i = 0; i < n_dev; ++i) lr_vec.push_back(p.transfer_lr_vec[i]);
+  } else {
+    lr_vec.assign(n_dev, p.transfer_lr);
+  }
+  if (p.n_reads_per_transfer > in_size) p.n_reads_per_transfer = in_size;
+  if (p.n_reads_per_transfer < 1) throw RpuError("n_reads_per_transfer must be positive.");
+  every_vec.clear();
+  if (p.n_transfer_every_vec > 0) {
+    if (p.n_transfer_every_vec != n_dev) throw RpuError("Expect transfer_every_vec to be of length n_devices");
+    for (int i = 0; i < n_dev; ++i) every_vec.push_back(p.transfer_every_vec[i]);
+  } else {
+    float every = p.transfer_every;
+    for (int i = 0; i < n_dev; ++i) {
+      every_vec.push_back(every);
+      every *= (float)out_size / (float)p.n_reads_per_transfer;
+    }
+    if (p.no_self_transfer) every_vec[n_dev - 1] = 0.0f;
+  }
+  // IO of the read: management off (rpu_transfer_device.cpp:198-213)
+  io.p = p.transfer_io;
+  io.p.bound_management = RPU_BM_NONE;
+  io.p.noise_management = RPU_NM_NONE;
+  io.initialize(!p.transfer_columns);
+  up.p = p.transfer_up;
+  up.initialize();
+  fully_hidden = (p.gamma == 0.0f) && (gamma_vec.back() == 1.0f);
+}
+
+int TransferPar::transfer_every(int from_idx, int m_batch) const {
+  if (p.units_in_mbatch) return std::max((int)ceilf(every_vec[from_idx] * (float)m_batch), 0);
+  return std::max((int)roundf(every_vec[from_idx]), 0);
+}
+
+float TransferPar::granularity() const {
+  float g = 0.0f;
+  for (const DevicePar &d : devs) g += d.weight_granularity();
+  return g / (float)devs.size();
+}
 
 void fill_default_config(rpu_tile_config *cfg, int device_kind) {
   rpu_io_params io{};
@@ -365,6 +458,31 @@ void fill_default_config(rpu_tile_config *cfg, int device_kind) {
     d.ls_mean_bound_reference = 0;
   }
   cfg->device = d;
+}
+
+void fill_default_transfer(rpu_transfer_params *tp, int device_kind) {
+  rpu_tile_config cfg;
+  fill_default_config(&cfg, device_kind);
+  rpu_transfer_params t{};
+  t.n_devices = 2;
+  t.construction_seed = 0;
+  t.units_in_mbatch = 0;
+  t.n_reads_per_transfer = 1;
+  t.no_self_transfer = 1;
+  t.random_selection = 0;
+  t.scale_transfer_lr = 1;
+  t.scale_fast_lr = 1;
+  t.transfer_columns = 1;
+  t.gamma = 0.0f;
+  t.transfer_every = 1.0f;
+  t.with_reset_prob = 0.0f;
+  t.fast_lr = 0.0f;
+  t.transfer_lr = 1.0f;
+  t.transfer_io = cfg.f_io;
+  t.transfer_up = cfg.up;
+  t.fast_device = cfg.device;
+  t.rest_device = cfg.device;
+  *tp = t;
 }
 
 } // namespace rpu_amd

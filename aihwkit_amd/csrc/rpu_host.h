@@ -44,6 +44,39 @@ struct DevicePar {
   void populate(int x_size, int d_size, DeviceArrays &out) const;
 };
 
+// Samples several devices one after the other from one stream seeded once, as VectorRPUDevice::populate
+// hands the same RealWorldRNG to every sub-device (rpu_vector_device.cpp:397-431).
+void populate_chain(const std::vector<DevicePar> &pars, unsigned int seed, int x_size, int d_size,
+                    std::vector<DeviceArrays> &out);
+
+// Validated parameters of the transfer compound (TransferRPUDeviceMetaParameter::initializeWithSize,
+// rpu_transfer_device.cpp:119-217).
+struct TransferPar {
+  rpu_transfer_params p{};
+  IOPar io;      // transfer_io, noise and bound management forced off
+  UpdatePar up;  // transfer_up
+  std::vector<DevicePar> devs;
+  std::vector<float> gamma_vec, lr_vec, every_vec;
+  bool fully_hidden = false; // gamma == 0 and the last gamma_vec entry is 1: the last device IS the tile's weights
+  int in_size = 0, out_size = 0;
+  void initialize(int x_size, int d_size);
+  int n() const { return (int)devs.size(); }
+  // rpu_transfer_device.cpp:219-230
+  float transfer_lr(int from_idx, float current_lr) const {
+    return p.scale_transfer_lr ? lr_vec[from_idx] * current_lr : lr_vec[from_idx];
+  }
+  // rpu_transfer_device.cpp:394-403
+  int transfer_every(int from_idx, int m_batch) const;
+  // rpu_transfer_device.cpp:366-383
+  float fast_lr(float learning_rate) const {
+    if (p.fast_lr > 0.0f) return p.scale_fast_lr ? p.fast_lr * learning_rate : p.fast_lr;
+    return learning_rate;
+  }
+  // average over the devices (rpu_vector_device.cpp:411-421)
+  float granularity() const;
+};
+
 void fill_default_config(rpu_tile_config *cfg, int device_kind);
+void fill_default_transfer(rpu_transfer_params *tp, int device_kind);
 
 } // namespace rpu_amd

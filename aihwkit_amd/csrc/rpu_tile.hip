@@ -75,6 +75,49 @@ const char *const kHiddenNames[10] = {"max_bound",       "min_bound",  "dwmin_up
 
 } // namespace
 
+// One physical device matrix of a compound: its parameters, sampled arrays and weights.
+struct DeviceSlot {
+  DevicePar par;
+  DeviceArrays arr;
+  std::vector<float> w_host; // weights while the tile is not resident on a GPU
+  DevBuf<float> d_w, d_wmax, d_wmin, d_sup, d_sdown, d_slup, d_sldown;
+  void release() {
+    d_w.release(); d_wmax.release(); d_wmin.release(); d_sup.release(); d_sdown.release();
+    d_slup.release(); d_sldown.release();
+  }
+  void clip_host() {
+    for (size_t i = 0; i < w_host.size(); ++i) {
+      w_host[i] = std::min(w_host[i], arr.w_max[i]);
+      w_host[i] = std::max(w_host[i], arr.w_min[i]);
+    }
+  }
+  void upload(size_t n, bool with_weights) {
+    const size_t bytes = n * sizeof(float);
+    d_wmax.ensure(n); d_wmin.ensure(n); d_sup.ensure(n); d_sdown.ensure(n);
+    RPU_HIP_CHECK(hipMemcpy(d_wmax.p, arr.w_max.data(), bytes, hipMemcpyHostToDevice));
+    RPU_HIP_CHECK(hipMemcpy(d_wmin.p, arr.w_min.data(), bytes, hipMemcpyHostToDevice));
+    RPU_HIP_CHECK(hipMemcpy(d_sup.p, arr.scale_up.data(), bytes, hipMemcpyHostToDevice));
+    RPU_HIP_CHECK(hipMemcpy(d_sdown.p, arr.scale_down.data(), bytes, hipMemcpyHostToDevice));
+    if (par.linear()) {
+      d_slup.ensure(n); d_sldown.ensure(n);
+      RPU_HIP_CHECK(hipMemcpy(d_slup.p, arr.slope_up.data(), bytes, hipMemcpyHostToDevice));
+      RPU_HIP_CHECK(hipMemcpy(d_sldown.p, arr.slope_down.data(), bytes, hipMemcpyHostToDevice));
+    }
+    if (with_weights) {
+      d_w.ensure(n);
+      RPU_HIP_CHECK(hipMemcpy(d_w.p, w_host.data(), bytes, hipMemcpyHostToDevice));
+    }
+  }
+};
+
+// what the update kernels need to know about the device matrix they write
+struct DeviceView {
+  float *w;
+  const float *w_max, *w_min, *scale_up, *scale_down, *slope_up, *slope_down;
+  const DevicePar *par;
+  float granularity; // dw_min used for BL and the pulse probabilities
+};
+
 struct Tile {
   int X = 0, D = 0;
   IOPar fio, bio;
@@ -100,6 +143,14 @@ struct Tile {
   DevBuf<uint32_t> u_xw, u_dw, u_xpl, u_dpl;
   DevBuf<int> u_kmax;
   uint32_t update_calls = 0;
+  // transfer compound (rpu_transfer_device.{h,cpp}): device 0 takes the gradient update, device j is read
+  // column by column and written onto device j + 1; the tile's weights d_w are the weighted sum, or the
+  // last device itself when that one alone is visible
+  std::unique_ptr<TransferPar> tr;
+  std::vector<std::unique_ptr<DeviceSlot>> slots;
+  uint64_t update_idx = 0;
+  std::vector<int> slice_idx;
+  DevBuf<float> t_unit, t_read;
   int last_update_batch = 0;
   int last_update_pulse = -1;
   int last_forward_batch = 0;
@@ -131,6 +182,9 @@ struct Tile {
   }
 
   bool resident() const { return device_id >= 0; }
+  bool is_transfer() const { return tr != nullptr; }
+  // the matrix forward / backward contract with
+  float *wdev() { return (tr && tr->fully_hidden) ? slots.back()->d_w.p : d_w.p; }
   size_t size() const { return (size_t)X * (size_t)D; }
 
   ~Tile() {
@@ -152,6 +206,8 @@ struct Tile {
     s_rounds.release(); s_hitup.release(); s_hitlo.release(); s_list0.release(); s_list1.release(); s_row0.release(); s_row1.release(); s_count.release(); s_tiledone.release();
     u_bl.release(); u_a.release(); u_b.release(); u_xval.release(); u_dval.release(); u_xw.release(); u_dw.release();
     u_xpl.release(); u_dpl.release(); u_kmax.release();
+    t_unit.release(); t_read.release();
+    for (auto &sl : slots) sl->release();
   }
 
   PhiloxKey key() const {
@@ -196,9 +252,17 @@ struct Tile {
     DeviceGuard g(target);
     device_id = target;
     try {
-      d_w.ensure(size());
-      RPU_HIP_CHECK(hipMemcpy(d_w.p, w_host.data(), size() * sizeof(float), hipMemcpyHostToDevice));
-      upload_params();
+      if (is_transfer()) {
+        for (auto &sl : slots) sl->upload(size(), true);
+        if (!tr->fully_hidden) {
+          d_w.ensure(size());
+          RPU_HIP_CHECK(hipMemcpy(d_w.p, w_host.data(), size() * sizeof(float), hipMemcpyHostToDevice));
+        }
+      } else {
+        d_w.ensure(size());
+        RPU_HIP_CHECK(hipMemcpy(d_w.p, w_host.data(), size() * sizeof(float), hipMemcpyHostToDevice));
+        upload_params();
+      }
       s_count.ensure(64);
     } catch (...) {
       release_all();
@@ -238,13 +302,15 @@ struct Tile {
   }
 
   // shared driver of forward (transposed = 0) and backward (transposed = 1)
-  void mvm(const float *in, float *out, int B, bool bias, bool in_trans, bool out_trans, bool transposed, hipStream_t s) {
-    const IOPar &io = transposed ? bio : fio;
+  void mvm(const float *in, float *out, int B, bool bias, bool in_trans, bool out_trans, bool transposed, hipStream_t s,
+           const float *w_other = nullptr, const IOPar *io_other = nullptr) {
+    const IOPar &io = io_other ? *io_other : (transposed ? bio : fio);
     const int K = transposed ? D : X;
     const int O = transposed ? X : D;
     ensure_mvm_scratch(B);
     MvmArgs a{};
-    a.w = d_w.p; a.x_size = X; a.d_size = D; a.m_batch = B; a.K = K; a.O = O; a.transposed = transposed ? 1 : 0;
+    a.w = w_other ? w_other : wdev(); a.x_size = X; a.d_size = D; a.m_batch = B; a.K = K; a.O = O;
+    a.transposed = transposed ? 1 : 0;
     a.io = io_dev(io);
     a.alpha = io.p.out_scale; a.beta = 0.0f;
     a.key = key(); a.call = call++;
@@ -302,7 +368,7 @@ struct Tile {
     if (transposed && bias) launch_drop_bias(s_bias.p, final_out, B, X, out_trans ? 1 : 0, s);
     RPU_HIP_CHECK(hipGetLastError());
     last_stream = s;
-    if (!transposed) last_forward_batch = B;
+    if (!transposed && !w_other) last_forward_batch = B;
   }
 
   void set_plane_args(UpdateArgs &a, int B) {
@@ -322,6 +388,7 @@ struct Tile {
   // device steps for pulse words made elsewhere (the reference's updateVectorWithCounts debug protocol)
   void update_with_words(const uint32_t *x_words, const uint32_t *d_words, int B, hipStream_t s) {
     if (lr == 0.0f) return;
+    if (is_transfer()) throw RpuError("update_with_words is not provided for a transfer compound.");
     if (!dev.pulsed()) throw RpuError("update_with_words needs a pulsed device.");
     UpdateArgs a{};
     a.w = d_w.p; a.x_size = X; a.d_size = D; a.m_batch = B; a.lr = lr;
@@ -379,18 +446,37 @@ struct Tile {
       return;
     }
 
+    if (is_transfer()) {
+      transfer_update(xin, x_sb, x_sj, d, d_sb, d_si, B, s);
+      return;
+    }
+    DeviceView dv{d_w.p, d_wmax.p, d_wmin.p, d_sup.p, d_sdown.p, d_slup.p, d_sldown.p, &dev, dev.p.dw_min};
+    pulsed_update_on(dv, up, lr, xin, x_sb, x_sj, d, d_sb, d_si, B, s);
+  }
+
+  DeviceView view_of(DeviceSlot &sl, float granularity) {
+    return DeviceView{sl.d_w.p, sl.d_wmax.p, sl.d_wmin.p, sl.d_sup.p, sl.d_sdown.p, sl.d_slup.p, sl.d_sldown.p,
+                      &sl.par, granularity};
+  }
+
+  // pulsed update of one device matrix (rpu_weight_updater.cpp:197-294)
+  void pulsed_update_on(const DeviceView &dv, const UpdatePar &up, float lr, const float *xin, long x_sb, long x_sj,
+                        const float *d, long d_sb, long d_si, int B, hipStream_t s) {
+    if (lr == 0.0f) return;
+    const DevicePar &dev = *dv.par;
     UpdateArgs a{};
-    a.w = d_w.p; a.x_size = X; a.d_size = D; a.m_batch = B;
+    a.w = dv.w; a.x_size = X; a.d_size = D; a.m_batch = B;
     a.x = xin; a.x_sb = x_sb; a.x_sj = x_sj; a.d = d; a.d_sb = d_sb; a.d_si = d_si;
     a.lr = lr;
     a.up.pulse_type = up.p.pulse_type; a.up.desired_bl = up.p.desired_bl; a.up.fixed_bl = up.p.fixed_bl;
     a.up.update_management = up.p.update_management; a.up.update_bl_management = up.p.update_bl_management;
     a.up.sto_round = up.p.sto_round; a.up.um_grad_scale = up.p.um_grad_scale; a.up.res = up.p.res;
     a.up.x_res_implicit = up.p.x_res_implicit; a.up.d_res_implicit = up.p.d_res_implicit;
-    a.dev.kind = dev.p.kind; a.dev.ls_mult_noise = dev.p.ls_mult_noise; a.dev.dw_min = dev.p.dw_min;
+    a.dev.kind = dev.p.kind; a.dev.ls_mult_noise = dev.p.ls_mult_noise; a.dev.dw_min = dv.granularity;
     a.dev.dw_min_std = dev.p.dw_min_std;
-    a.dev.w_max = d_wmax.p; a.dev.w_min = d_wmin.p; a.dev.scale_up = d_sup.p; a.dev.scale_down = d_sdown.p;
-    a.dev.slope_up = d_slup.p; a.dev.slope_down = d_sldown.p;
+    a.dev.w_max = const_cast<float *>(dv.w_max); a.dev.w_min = const_cast<float *>(dv.w_min);
+    a.dev.scale_up = const_cast<float *>(dv.scale_up); a.dev.scale_down = const_cast<float *>(dv.scale_down);
+    a.dev.slope_up = const_cast<float *>(dv.slope_up); a.dev.slope_down = const_cast<float *>(dv.slope_down);
     u_bl.ensure(B); u_a.ensure(B); u_b.ensure(B);
     a.bl = u_bl.p; a.prob_a = u_a.p; a.prob_b = u_b.p;
     a.key = key(); a.call = call++;
@@ -423,6 +509,116 @@ struct Tile {
     last_stream = s;
     last_update_batch = B;
     last_update_pulse = up.p.pulse_type;
+  }
+
+  // ---- transfer compound ----------------------------------------------------------------------
+
+  // tile weights = sum_k gamma_k w_k, unless the last device alone is visible (rpu_transfer_device.cpp:596-602)
+  void reduce_to_weights(hipStream_t s) {
+    if (tr->fully_hidden) return;
+    ReduceArgs r{};
+    r.n = tr->n();
+    for (int k = 0; k < r.n; ++k) {
+      r.w[k] = slots[k]->d_w.p;
+      r.gamma[k] = tr->gamma_vec[k];
+    }
+    launch_reduce_weights(d_w.p, r, size(), s);
+  }
+
+  // TransferRPUDevice::transfer / readAndUpdate (rpu_transfer_device.cpp:428-516): the next
+  // n_reads_per_transfer columns (rows) of device `from` are read through transfer_io with unit vectors
+  // (scaled by -1 so that the write adds) and written onto device `to` with a pulsed update under
+  // transfer_up.  Reading all of them before writing is the same as one by one: `from` is not written.
+  void do_transfer(int to, int from, float current_lr, hipStream_t s) {
+    const TransferPar &tp = *tr;
+    const int in_size = tp.in_size, out_size = tp.out_size;
+    const int start = slice_idx[from];
+    const int n_vec = std::min(tp.p.n_reads_per_transfer, in_size);
+    slice_idx[from] = (start + n_vec) % in_size;
+    const float lr_t = tp.transfer_lr(from, current_lr);
+    if (lr_t == 0.0f || to == from) return;
+    t_unit.ensure((size_t)n_vec * in_size);
+    t_read.ensure((size_t)n_vec * out_size);
+    launch_unit_vectors(t_unit.p, n_vec, in_size, start, s);
+    IOPar io = tp.io;
+    io.p.out_scale = -io.p.out_scale;
+    const bool cols = tp.p.transfer_columns != 0;
+    mvm(t_unit.p, t_read.p, n_vec, false, false, false, !cols, s, slots[from]->d_w.p, &io);
+    DeviceView dv = view_of(*slots[to], slots[to]->par.weight_granularity());
+    if (cols) pulsed_update_on(dv, tp.up, lr_t, t_unit.p, X, 1, t_read.p, D, 1, n_vec, s);
+    else pulsed_update_on(dv, tp.up, lr_t, t_read.p, X, 1, t_unit.p, D, 1, n_vec, s);
+  }
+
+  // TransferRPUDevice::doSparseUpdate / finishUpdateCycle per update vector (rpu_transfer_device.cpp:520-557):
+  // the gradient goes onto device 0; after every vector the update counter advances and each device whose
+  // period divides it transfers.  The batch is cut at those points (C/rpucuda_transfer_device.cu:393-510).
+  void transfer_update(const float *xin, long x_sb, long x_sj, const float *d, long d_sb, long d_si, int B, hipStream_t s) {
+    const TransferPar &tp = *tr;
+    const float lr_fast = tp.fast_lr(lr);
+    const int n_dev = tp.n();
+    std::vector<int> every(n_dev);
+    for (int j = 0; j < n_dev; ++j) every[j] = tp.transfer_every(j, B);
+    DeviceView dv0 = view_of(*slots[0], tp.granularity());
+    int b0 = 0;
+    while (b0 < B) {
+      // vectors until the next transfer of any device
+      uint64_t chunk = (uint64_t)(B - b0);
+      for (int j = 0; j < n_dev; ++j) {
+        if (every[j] > 0) chunk = std::min<uint64_t>(chunk, (uint64_t)every[j] - update_idx % (uint64_t)every[j]);
+      }
+      pulsed_update_on(dv0, up, lr_fast, xin + (long)b0 * x_sb, x_sb, x_sj, d + (long)b0 * d_sb, d_sb, d_si, (int)chunk, s);
+      update_idx += chunk;
+      b0 += (int)chunk;
+      for (int j = 0; j < n_dev; ++j) {
+        if (every[j] > 0 && update_idx % (uint64_t)every[j] == 0) do_transfer(std::min(j + 1, n_dev - 1), j, lr, s);
+      }
+    }
+    reduce_to_weights(s);
+    last_stream = s;
+    last_update_batch = B;
+  }
+
+  // TransferRPUDevice::onSetWeights (rpu_transfer_device.cpp:559-594): every device to zero, the last one gets
+  // the weights over its significance, each is clipped into its own bounds, counters restart
+  void transfer_set_weights_host(const float *w) {
+    const int last = tr->n() - 1;
+    const size_t n = size();
+    for (auto &sl : slots) sl->w_host.assign(n, 0.0f);
+    const float g = tr->fully_hidden ? 1.0f : tr->gamma_vec[last];
+    for (size_t i = 0; i < n; ++i) slots[last]->w_host[i] = tr->fully_hidden ? w[i] : w[i] / g;
+    for (auto &sl : slots) sl->clip_host();
+    update_idx = 0;
+    std::fill(slice_idx.begin(), slice_idx.end(), 0);
+    transfer_reduce_host();
+  }
+
+  void transfer_reduce_host() {
+    const size_t n = size();
+    w_host.assign(n, 0.0f);
+    if (tr->fully_hidden) {
+      w_host = slots.back()->w_host;
+      return;
+    }
+    for (int k = 0; k < tr->n(); ++k) {
+      for (size_t i = 0; i < n; ++i) w_host[i] += tr->gamma_vec[k] * slots[k]->w_host[i];
+    }
+  }
+
+  // device -> host copies of all matrices of the compound
+  void transfer_download() {
+    const size_t bytes = size() * sizeof(float);
+    for (auto &sl : slots) {
+      sl->w_host.resize(size());
+      RPU_HIP_CHECK(hipMemcpy(sl->w_host.data(), sl->d_w.p, bytes, hipMemcpyDeviceToHost));
+    }
+    w_host.resize(size());
+    RPU_HIP_CHECK(hipMemcpy(w_host.data(), wdev(), bytes, hipMemcpyDeviceToHost));
+  }
+
+  void transfer_upload_weights() {
+    const size_t bytes = size() * sizeof(float);
+    for (auto &sl : slots) RPU_HIP_CHECK(hipMemcpy(sl->d_w.p, sl->w_host.data(), bytes, hipMemcpyHostToDevice));
+    if (!tr->fully_hidden) RPU_HIP_CHECK(hipMemcpy(d_w.p, w_host.data(), bytes, hipMemcpyHostToDevice));
   }
 };
 
@@ -489,6 +685,63 @@ int rpu_tile_create(rpu_tile_t **out, int x_size, int d_size, const rpu_tile_con
   });
 }
 
+int rpu_transfer_params_default(rpu_transfer_params *tp, int device_kind) {
+  return guarded([&] {
+    if (!tp) throw RpuError("tp is null");
+    fill_default_transfer(tp, device_kind);
+  });
+}
+
+int rpu_tile_create_transfer(rpu_tile_t **out, int x_size, int d_size, const rpu_tile_config *cfg,
+                             const rpu_transfer_params *tp) {
+  return guarded([&] {
+    if (!out || !cfg || !tp) throw RpuError("null argument");
+    if (x_size <= 0 || d_size <= 0) throw RpuError("Tile sizes must be positive.");
+    auto h = std::make_unique<rpu_tile>();
+    Tile &t = h->t;
+    t.X = x_size;
+    t.D = d_size;
+    t.fio.p = cfg->f_io;
+    t.bio.p = cfg->b_io;
+    t.up.p = cfg->up;
+    t.fio.initialize(false);
+    t.bio.initialize(true);
+    t.up.initialize();
+    if (t.up.p.pulse_type == RPU_PULSE_NONE || t.up.p.pulse_type == RPU_PULSE_NONE_WITH_DEVICE) {
+      throw RpuError("A transfer compound needs a pulsed update (pulse_type None is not provided).");
+    }
+    t.tr = std::make_unique<TransferPar>();
+    t.tr->p = *tp;
+    t.tr->initialize(x_size, d_size);
+    t.dev = t.tr->devs[0]; // the device the gradient update sees
+    std::vector<DeviceArrays> arrays;
+    populate_chain(t.tr->devs, tp->construction_seed, x_size, d_size, arrays);
+    for (int k = 0; k < t.tr->n(); ++k) {
+      auto sl = std::make_unique<DeviceSlot>();
+      sl->par = t.tr->devs[k];
+      sl->arr = std::move(arrays[k]);
+      t.slots.push_back(std::move(sl));
+    }
+    t.slice_idx.assign(t.tr->n(), 0);
+    std::vector<float> zeros(t.size(), 0.0f);
+    t.transfer_set_weights_host(zeros.data());
+    *out = h.release();
+  });
+}
+
+int rpu_tile_get_transfer_state(rpu_tile_t *tile, uint64_t *update_idx, int32_t *slice_indices_host) {
+  return guarded([&] {
+    if (!tile) throw RpuError("null tile");
+    Tile &t = tile->t;
+    std::lock_guard<std::mutex> lock(t.mutex);
+    if (!t.is_transfer()) throw RpuError("Not a transfer compound.");
+    if (update_idx) *update_idx = t.update_idx;
+    if (slice_indices_host) {
+      for (int k = 0; k < t.tr->n(); ++k) slice_indices_host[k] = t.slice_idx[k];
+    }
+  });
+}
+
 int rpu_tile_clone(rpu_tile_t **out, const rpu_tile_t *src_c) {
   return guarded([&] {
     if (!out || !src_c) throw RpuError("null argument");
@@ -500,7 +753,25 @@ int rpu_tile_clone(rpu_tile_t **out, const rpu_tile_t *src_c) {
     t.X = s.X; t.D = s.D; t.fio = s.fio; t.bio = s.bio; t.up = s.up; t.dev = s.dev; t.arr = s.arr;
     t.lr = s.lr; t.seed = s.seed; t.call = s.call;
     t.w_host = s.w_host;
-    if (s.resident()) {
+    if (s.is_transfer()) {
+      t.tr = std::make_unique<TransferPar>(*s.tr);
+      t.update_idx = s.update_idx;
+      t.slice_idx = s.slice_idx;
+      if (s.resident()) {
+        DeviceGuard g(s.device_id);
+        RPU_HIP_CHECK(hipStreamSynchronize(s.last_stream));
+        const_cast<Tile &>(s).transfer_download();
+        t.w_host = s.w_host;
+      }
+      for (const auto &sl : s.slots) {
+        auto c = std::make_unique<DeviceSlot>();
+        c->par = sl->par;
+        c->arr = sl->arr;
+        c->w_host = sl->w_host;
+        t.slots.push_back(std::move(c));
+      }
+      if (s.resident()) t.to_device(s.device_id);
+    } else if (s.resident()) {
       DeviceGuard g(s.device_id);
       RPU_HIP_CHECK(hipStreamSynchronize(s.last_stream));
       t.w_host.resize(s.size());
@@ -590,6 +861,17 @@ int rpu_tile_set_weights(rpu_tile_t *tile, const float *w_host) {
     if (!tile || !w_host) throw RpuError("null argument");
     Tile &t = tile->t;
     std::lock_guard<std::mutex> lock(t.mutex);
+    if (t.is_transfer()) {
+      if (t.resident()) {
+        DeviceGuard g(t.device_id);
+        t.sync_last();
+        t.transfer_set_weights_host(w_host);
+        t.transfer_upload_weights();
+      } else {
+        t.transfer_set_weights_host(w_host);
+      }
+      return;
+    }
     std::vector<float> w(w_host, w_host + t.size());
     t.clip_host(w);
     if (t.resident()) {
@@ -610,7 +892,7 @@ int rpu_tile_get_weights(rpu_tile_t *tile, float *w_host) {
     if (t.resident()) {
       DeviceGuard g(t.device_id);
       t.sync_last();
-      RPU_HIP_CHECK(hipMemcpy(w_host, t.d_w.p, t.size() * sizeof(float), hipMemcpyDeviceToHost));
+      RPU_HIP_CHECK(hipMemcpy(w_host, t.wdev(), t.size() * sizeof(float), hipMemcpyDeviceToHost));
     } else {
       std::memcpy(w_host, t.w_host.data(), t.size() * sizeof(float));
     }
@@ -620,34 +902,65 @@ int rpu_tile_get_weights(rpu_tile_t *tile, float *w_host) {
 int rpu_tile_weights_device_ptr(rpu_tile_t *tile, float **w_dev) {
   return guarded([&] {
     if (!tile || !w_dev) throw RpuError("null argument");
-    *w_dev = tile->t.resident() ? tile->t.d_w.p : nullptr;
+    *w_dev = tile->t.resident() ? tile->t.wdev() : nullptr;
   });
 }
 
+// entry idx of a transfer compound's hidden parameters: (device, index within the device); the index one
+// past the device's own arrays is its weight matrix "hidden_weights_k" (rpu_vector_device.cpp:188-203)
+static void compound_entry(const Tile &t, int idx, int &device, int &local, int &n_local) {
+  device = 0;
+  for (const auto &sl : t.slots) {
+    n_local = sl->par.linear() ? 10 : 8;
+    if (idx <= n_local) {
+      local = idx;
+      return;
+    }
+    idx -= n_local + 1;
+    ++device;
+  }
+  device = -1;
+}
+
 int rpu_tile_hidden_parameter_count(const rpu_tile_t *tile) {
-  if (!tile || !tile->t.dev.pulsed()) return 0;
+  if (!tile) return 0;
+  if (tile->t.is_transfer()) {
+    int n = 0;
+    for (const auto &sl : tile->t.slots) n += (sl->par.linear() ? 10 : 8) + 1;
+    return n;
+  }
+  if (!tile->t.dev.pulsed()) return 0;
   return tile->t.dev.linear() ? 10 : 8;
 }
 
 const char *rpu_tile_hidden_parameter_name(const rpu_tile_t *tile, int idx) {
   if (idx < 0 || idx >= rpu_tile_hidden_parameter_count(tile)) return nullptr;
+  if (tile->t.is_transfer()) {
+    static thread_local std::string name;
+    int device, local, n_local;
+    compound_entry(tile->t, idx, device, local, n_local);
+    name = std::string(local < n_local ? kHiddenNames[local] : "hidden_weights") + "_" + std::to_string(device);
+    return name.c_str();
+  }
   return kHiddenNames[idx];
 }
 
-static std::vector<float> *hidden_slot(Tile &t, int idx) {
+static std::vector<float> *hidden_array(DeviceArrays &arr, int idx) {
   switch (idx) {
-  case 0: return &t.arr.w_max;
-  case 1: return &t.arr.w_min;
-  case 2: return &t.arr.scale_up;
-  case 3: return &t.arr.scale_down;
-  case 4: return &t.arr.decay_scale;
-  case 5: return &t.arr.diffusion_rate;
-  case 6: return &t.arr.reset_bias;
-  case 8: return &t.arr.slope_up;
-  case 9: return &t.arr.slope_down;
+  case 0: return &arr.w_max;
+  case 1: return &arr.w_min;
+  case 2: return &arr.scale_up;
+  case 3: return &arr.scale_down;
+  case 4: return &arr.decay_scale;
+  case 5: return &arr.diffusion_rate;
+  case 6: return &arr.reset_bias;
+  case 8: return &arr.slope_up;
+  case 9: return &arr.slope_down;
   default: return nullptr; // drift_nu: no drifter on this path, reported as zeros
   }
 }
+
+static std::vector<float> *hidden_slot(Tile &t, int idx) { return hidden_array(t.arr, idx); }
 
 int rpu_tile_get_hidden_parameters(rpu_tile_t *tile, float *data_host) {
   return guarded([&] {
@@ -656,6 +969,22 @@ int rpu_tile_get_hidden_parameters(rpu_tile_t *tile, float *data_host) {
     std::lock_guard<std::mutex> lock(t.mutex);
     const size_t n = t.size();
     const int count = rpu_tile_hidden_parameter_count(tile);
+    if (t.is_transfer()) {
+      if (t.resident()) {
+        DeviceGuard g(t.device_id);
+        t.sync_last();
+        t.transfer_download();
+      }
+      for (int k = 0; k < count; ++k) {
+        int device, local, n_local;
+        compound_entry(t, k, device, local, n_local);
+        DeviceSlot &sl = *t.slots[device];
+        std::vector<float> *a = local < n_local ? hidden_array(sl.arr, local) : &sl.w_host;
+        if (a) std::memcpy(data_host + (size_t)k * n, a->data(), n * sizeof(float));
+        else std::memset(data_host + (size_t)k * n, 0, n * sizeof(float));
+      }
+      return;
+    }
     for (int k = 0; k < count; ++k) {
       std::vector<float> *a = hidden_slot(t, k);
       if (a) std::memcpy(data_host + (size_t)k * n, a->data(), n * sizeof(float));
@@ -671,6 +1000,32 @@ int rpu_tile_set_hidden_parameters(rpu_tile_t *tile, const float *data_host) {
     std::lock_guard<std::mutex> lock(t.mutex);
     const size_t n = t.size();
     const int count = rpu_tile_hidden_parameter_count(tile);
+    if (t.is_transfer()) {
+      // VectorRPUDevice::setDeviceParameter (rpu_vector_device.cpp:286-325): per device its weights, then its
+      // arrays (which clip those weights), then the tile weights are reduced again
+      if (t.resident()) {
+        DeviceGuard g(t.device_id);
+        t.sync_last();
+      }
+      for (int k = 0; k < count; ++k) {
+        int device, local, n_local;
+        compound_entry(t, k, device, local, n_local);
+        DeviceSlot &sl = *t.slots[device];
+        std::vector<float> *a = local < n_local ? hidden_array(sl.arr, local) : &sl.w_host;
+        if (a) {
+          a->resize(n);
+          std::memcpy(a->data(), data_host + (size_t)k * n, n * sizeof(float));
+        }
+      }
+      for (auto &sl : t.slots) sl->clip_host();
+      t.transfer_reduce_host();
+      if (t.resident()) {
+        DeviceGuard g(t.device_id);
+        for (auto &sl : t.slots) sl->upload(n, true);
+        t.transfer_upload_weights();
+      }
+      return;
+    }
     for (int k = 0; k < count; ++k) {
       std::vector<float> *a = hidden_slot(t, k);
       if (a) std::memcpy(a->data(), data_host + (size_t)k * n, n * sizeof(float));

@@ -10,7 +10,7 @@ rpu_linearstep_device.h:16-80).
 import enum
 import sys
 
-from .._cabi import DeviceParams, IOParams, TileConfig, UpdateParams
+from .._cabi import MAX_VECTOR_DEVICES, DeviceParams, IOParams, TileConfig, TransferParams, UpdateParams
 
 FLT_MAX = 3.4028234663852886e38
 
@@ -88,6 +88,9 @@ class _Struct:
         if name not in self._all_defaults():
             raise AttributeError(f"{type(self).__name__} has no field {name!r}")
         object.__setattr__(self, name, value)
+
+    def _all_values(self):
+        return {k: getattr(self, k) for k in self._all_defaults()}
 
     def __str__(self):
         fields = ", ".join(f"{k}={getattr(self, k)!r}" for k in self._all_defaults())
@@ -257,6 +260,79 @@ class SoftBoundsResistiveDeviceParameter(LinearStepResistiveDeviceParameter):
         super()._fill_c(p)
 
 
+class VectorResistiveDeviceParameter(AbstractResistiveDeviceParameter):
+    """rpu_base_devices.cpp:686-714 over VectorRPUDeviceMetaParameter: a list of device parameters.
+    Only its transfer subclass can be turned into a tile on this path."""
+
+    _defaults = dict(gamma_vec=None, update_policy=0, first_update_idx=0)
+
+    def __init__(self):
+        super().__init__()
+        object.__setattr__(self, "gamma_vec", [])
+        object.__setattr__(self, "_vec_par", [])
+
+    def append_parameter(self, parameter) -> bool:
+        """VectorRPUDeviceMetaParameter::appendVecPar (rpu_vector_device.cpp:74-91): pulsed devices only."""
+        if not isinstance(parameter, PulsedResistiveDeviceParameter):
+            return False
+        self._vec_par.append(parameter)
+        return True
+
+    def calc_weight_granularity(self) -> float:
+        return float(self._vec_par[0].calc_weight_granularity()) if self._vec_par else 0.0
+
+
+class TransferResistiveDeviceParameter(VectorResistiveDeviceParameter):
+    """rpu_base_devices.cpp:742-777 over TransferRPUDeviceMetaParameter (rpu_transfer_device.h:52-127)."""
+
+    _defaults = dict(
+        gamma=0.0, transfer_every=1.0, no_self_transfer=True, transfer_every_vec=None, units_in_mbatch=False,
+        n_reads_per_transfer=1, with_reset_prob=0.0, random_selection=False, transfer_columns=True,
+        transfer_lr=1.0, fast_lr=0.0, transfer_lr_vec=None, scale_transfer_lr=True, scale_fast_lr=True,
+        transfer_forward=None, transfer_update=None,
+    )
+    _kind = 4
+
+    def __init__(self):
+        super().__init__()
+        object.__setattr__(self, "transfer_every_vec", [])
+        object.__setattr__(self, "transfer_lr_vec", [])
+        object.__setattr__(self, "transfer_forward", AnalogTileInputOutputParameter())
+        object.__setattr__(self, "transfer_update", AnalogTileUpdateParameter())
+
+    def _to_transfer_c(self) -> TransferParams:
+        n_dev = len(self._vec_par)
+        if n_dev < 2:
+            raise RuntimeError("Need at least 2 devices")
+        if n_dev > MAX_VECTOR_DEVICES:
+            raise RuntimeError(f"At most {MAX_VECTOR_DEVICES} devices in a transfer chain.")
+        rest = self._vec_par[1]
+        for other in self._vec_par[2:]:
+            if type(other) is not type(rest) or other._all_values() != rest._all_values():
+                raise RuntimeError("Only the first device can be a different RPU device. ")
+        p = TransferParams()
+        p.n_devices = n_dev
+        p.construction_seed = int(self.construction_seed)
+        for name in ("units_in_mbatch", "no_self_transfer", "random_selection", "scale_transfer_lr",
+                     "scale_fast_lr", "transfer_columns"):
+            setattr(p, name, int(bool(getattr(self, name))))
+        p.n_reads_per_transfer = int(self.n_reads_per_transfer)
+        for name in ("gamma", "transfer_every", "with_reset_prob", "fast_lr", "transfer_lr"):
+            setattr(p, name, float(getattr(self, name)))
+        for name in ("gamma_vec", "transfer_lr_vec", "transfer_every_vec"):
+            values = list(getattr(self, name) or [])
+            if len(values) > MAX_VECTOR_DEVICES:
+                raise RuntimeError(f"{name} is longer than {MAX_VECTOR_DEVICES}")
+            setattr(p, "n_" + name, len(values))
+            for k, v in enumerate(values):
+                getattr(p, name)[k] = float(v)
+        p.transfer_io = self.transfer_forward._to_c()
+        p.transfer_up = self.transfer_update._to_c()
+        p.fast_device = self._vec_par[0]._to_c()
+        p.rest_device = rest._to_c()
+        return p
+
+
 class AnalogTileParameter(_Struct):
     """rpu_base_devices.cpp:453-467 over PulsedMetaParameter (rpu_pulsed.h:127-151)."""
 
@@ -282,6 +358,10 @@ class AnalogTileParameter(_Struct):
 
         if not isinstance(device_param, AbstractResistiveDeviceParameter) or device_param._kind is None:
             raise TypeError("device_param must be one of the *ResistiveDeviceParameter classes")
+        if isinstance(device_param, TransferResistiveDeviceParameter):
+            transfer = device_param._to_transfer_c()
+            config = self._config(device_param._vec_par[0])
+            return AnalogTile._create_transfer(int(x_size), int(d_size), config, transfer)
         return AnalogTile._create(int(x_size), int(d_size), self._config(device_param))
 
 

@@ -54,6 +54,19 @@ class _TileBase:
         check(lib().rpu_tile_create(C.byref(handle), x_size, d_size, C.byref(config)))
         return cls(handle.value)
 
+    @classmethod
+    def _create_transfer(cls, x_size, d_size, config, transfer):
+        handle = C.c_void_p()
+        check(lib().rpu_tile_create_transfer(C.byref(handle), x_size, d_size, C.byref(config), C.byref(transfer)))
+        return cls(handle.value)
+
+    def get_transfer_state(self):
+        """(number of update vectors since the weights were set, next column per device) of a transfer compound."""
+        count = C.c_uint64(0)
+        slices = (C.c_int32 * 4)()
+        check(lib().rpu_tile_get_transfer_state(self._h, C.byref(count), slices))
+        return int(count.value), list(slices)
+
     def _clone_handle(self):
         handle = C.c_void_p()
         check(lib().rpu_tile_clone(C.byref(handle), self._h))

@@ -75,7 +75,8 @@ enum rpu_device_kind {
   RPU_DEVICE_IDEAL = 0,         /* IdealResistiveDeviceParameter / FloatingPoint: no device physics */
   RPU_DEVICE_CONSTANT_STEP = 1, /* ConstantStepResistiveDeviceParameter */
   RPU_DEVICE_LINEAR_STEP = 2,   /* LinearStepResistiveDeviceParameter */
-  RPU_DEVICE_SOFT_BOUNDS = 3    /* SoftBoundsResistiveDeviceParameter (LinearStep with fixed ls_* values) */
+  RPU_DEVICE_SOFT_BOUNDS = 3,   /* SoftBoundsResistiveDeviceParameter (LinearStep with fixed ls_* values) */
+  RPU_DEVICE_TRANSFER = 4       /* TransferResistiveDeviceParameter: a chain of the kinds above (rpu_transfer_params) */
 };
 
 /* ---- parameter structs ------------------------------------------------------ */
@@ -185,6 +186,43 @@ typedef struct rpu_tile_config {
   rpu_device_params device;
 } rpu_tile_config;
 
+/* Replaces TransferRPUDeviceMetaParameter<float> (R/rpu_transfer_device.h:52-127, with the gamma_vec of
+ * VectorRPUDeviceMetaParameter, R/rpu_vector_device.h) as bound by TransferResistiveDeviceParameter
+ * (B/rpu_base_devices.cpp:742-777; transfer_forward = transfer_io, transfer_update = transfer_up).  The
+ * compound holds n_devices weight matrices: device 0 takes the gradient update, every transfer_every
+ * updates n_reads_per_transfer columns (rows) of device j are read through transfer_io and written
+ * onto device j + 1 with a pulsed update under transfer_up; the tile's weights are
+ * sum_k gamma_vec[k] * w_k.  Device 0 is fast_device, all others rest_device (the reference allows only
+ * the first to differ, R/rpu_transfer_device.cpp:136-144).  Empty vectors (n_* = 0) are filled as the
+ * reference does (R/rpu_transfer_device.cpp:146-196). */
+#define RPU_MAX_VECTOR_DEVICES 4
+typedef struct rpu_transfer_params {
+  int32_t n_devices;            /* 2 */
+  uint32_t construction_seed;   /* 0 = time based; one stream samples all devices in order */
+  int32_t units_in_mbatch;      /* 0 */
+  int32_t n_reads_per_transfer; /* 1 */
+  int32_t no_self_transfer;     /* 1 */
+  int32_t random_selection;     /* 0 ; 1 is not provided */
+  int32_t scale_transfer_lr;    /* 1 */
+  int32_t scale_fast_lr;        /* 1 */
+  int32_t transfer_columns;     /* 1 ; 0 = rows (read with the backward pass) */
+  float gamma;                  /* 0 */
+  float transfer_every;         /* 1 */
+  float with_reset_prob;        /* 0 ; > 0 is not provided */
+  float fast_lr;                /* 0 */
+  float transfer_lr;            /* 1 */
+  int32_t n_gamma_vec;          /* 0 or n_devices */
+  int32_t n_transfer_lr_vec;    /* 0 or n_devices */
+  int32_t n_transfer_every_vec; /* 0 or n_devices */
+  float gamma_vec[RPU_MAX_VECTOR_DEVICES];
+  float transfer_lr_vec[RPU_MAX_VECTOR_DEVICES];
+  float transfer_every_vec[RPU_MAX_VECTOR_DEVICES];
+  rpu_io_params transfer_io;
+  rpu_update_params transfer_up;
+  rpu_device_params fast_device;
+  rpu_device_params rest_device;
+} rpu_transfer_params;
+
 typedef struct rpu_tile rpu_tile_t; /* opaque */
 
 /* ---- defaults ---------------------------------------------------------------- */
@@ -199,6 +237,25 @@ int rpu_tile_config_default(rpu_tile_config *cfg, int device_kind);
  * samples the device-to-device parameters on the CPU with RealWorldRNG(construction_seed)
  * (R/rpu_pulsed.cpp:460-495, R/rpu_pulsed_device.cpp:593-733).  Touches no GPU. */
 int rpu_tile_create(rpu_tile_t **out, int x_size, int d_size, const rpu_tile_config *cfg);
+
+/* C++ defaults of TransferRPUDeviceMetaParameter with two devices of `device_kind`. */
+int rpu_transfer_params_default(rpu_transfer_params *tp, int device_kind);
+
+/* As rpu_tile_create with a transfer compound as the tile's device (cfg->device is ignored):
+ * TransferRPUDeviceMetaParameter::createDevice -> TransferRPUDevice::populate
+ * (R/rpu_transfer_device.cpp:333-358, R/rpu_vector_device.cpp:397-431).  Forward / backward act on the
+ * reduced weights; rpu_tile_update follows TransferRPUDevice::doSparseUpdate / finishUpdateCycle
+ * (R/rpu_transfer_device.cpp:520-557): the batch is cut where a transfer is due, as the reference's GPU
+ * path does (C/rpucuda_transfer_device.cu:393-510).  Hidden parameters: per device k its arrays with
+ * the suffix _k, then hidden_weights_k (R/rpu_vector_device.cpp:188-203). */
+int rpu_tile_create_transfer(rpu_tile_t **out, int x_size, int d_size, const rpu_tile_config *cfg,
+                             const rpu_transfer_params *tp);
+
+/* Counters of a transfer tile: number of update vectors seen since the weights were set and the next
+ * column (row) each device transfers (TransferRPUDevice::current_update_idx_, current_slice_indices_;
+ * the reference exposes them through dumpExtra, R/rpu_transfer_device.cpp:672-688).
+ * slice_indices_host is [n_devices]. */
+int rpu_tile_get_transfer_state(rpu_tile_t *tile, uint64_t *update_idx, int32_t *slice_indices_host);
 
 /* Deep copy (host state and, if resident, device state); B/rpu_base_tiles.cpp __copy__/__deepcopy__. */
 int rpu_tile_clone(rpu_tile_t **out, const rpu_tile_t *src);

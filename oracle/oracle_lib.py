@@ -28,6 +28,7 @@ def oracle():
         lib.orc_set_seed.argtypes = [P, C.c_uint]
         lib.orc_use_gauss_table.argtypes = [P, C.c_int]
         lib.orc_set_learning_rate.argtypes = [P, C.c_float]
+        lib.orc_set_weight_granularity.argtypes = [P, C.c_float]
         lib.orc_set_weights.argtypes = [P, P]
         lib.orc_get_weights.argtypes = [P, P]
         lib.orc_hidden_count.argtypes = [P]
@@ -68,6 +69,9 @@ class OracleTile:
 
     def use_gauss_table(self, on):
         self.lib.orc_use_gauss_table(self.h, int(on))
+
+    def set_weight_granularity(self, g):
+        self.lib.orc_set_weight_granularity(self.h, float(g))
 
     def set_learning_rate(self, lr):
         self.lib.orc_set_learning_rate(self.h, lr)

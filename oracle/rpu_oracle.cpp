@@ -183,6 +183,7 @@ struct OrcTile {
   rpu_update_params up;
   rpu_device_params dev;
   float lr = 0.01f; // R/rpu.h:186 default learning rate is set by the caller; 0.01 here
+  float granularity = 0.0f; // 0: the device's dw_min
   OrcRng rng;
   std::vector<float> w;
   // R/rpu_pulsed_device.h:296-312 per-device arrays
@@ -639,7 +640,9 @@ float find_abs_max(const float *v, int n, int inc) {
 // BL / A / B of one sample as R/sparse_bit_line_maker.cpp:299-314 and R/dense_bit_line_maker.cpp:285-300
 bool sample_bl_ab(OrcTile &t, const float *x, int x_inc, const float *d, int d_inc, float lr_abs,
                   int &BL, float &A, float &B) {
-  const float dw_min = t.dev.dw_min; // weight granularity (R/rpu_constantstep_device.h:27, R/rpu_linearstep_device.h:58)
+  // weight granularity (R/rpu_constantstep_device.h:27, R/rpu_linearstep_device.h:58); a compound device gives
+  // its own (R/rpu_vector_device.cpp:411-421), set through orc_set_weight_granularity
+  const float dw_min = t.granularity > 0.0f ? t.granularity : t.dev.dw_min;
   A = 0;
   B = 0;
   BL = 0;
@@ -894,6 +897,7 @@ void orc_destroy(void *h) { delete static_cast<OrcTile *>(h); }
 void orc_set_seed(void *h, unsigned int seed) { static_cast<OrcTile *>(h)->rng.seed(seed); }
 void orc_use_gauss_table(void *h, int on) { static_cast<OrcTile *>(h)->rng.use_table = on != 0; }
 void orc_set_learning_rate(void *h, float lr) { static_cast<OrcTile *>(h)->lr = lr; }
+void orc_set_weight_granularity(void *h, float g) { static_cast<OrcTile *>(h)->granularity = g; }
 
 void orc_set_weights(void *h, const float *w) { // R/rpu_pulsed.cpp:288-292
   auto *t = static_cast<OrcTile *>(h);
