@@ -69,6 +69,26 @@ def config2(noise=True, ctoc=True):
     return meta, dev
 
 
+def config3(noise=True):
+    """Tiki-Taka transfer compound of two SoftBounds devices (A fast, C slow): one column transferred every two
+    mini-batches (configuration 3; settings of examples/08_simple_layer_with_tiki_taka.py:29-45 of the reference)."""
+    on = 0.06 if noise else 0.0
+    f_io = io_params(out_noise=on, noise_management=dv.NoiseManagementType.AbsMax,
+                     bound_management=dv.BoundManagementType.Iterative)
+    b_io = io_params(out_noise=on, noise_management=dv.NoiseManagementType.AbsMax)
+    meta = make_meta(f_io, b_io, desired_bl=31, update_management=True, update_bl_management=True)
+    fast = soft_bounds(w_min=-0.3, w_max=0.3, enforce_consistency=True)
+    slow = soft_bounds(w_min=-0.6, w_max=0.6, enforce_consistency=True)
+    tr = transfer_param([fast, slow], construction_seed=123, units_in_mbatch=True, transfer_every=2.0,
+                        n_reads_per_transfer=1, gamma=0.0, scale_transfer_lr=True, transfer_lr=1.0, fast_lr=0.1,
+                        transfer_columns=True)
+    tr.transfer_forward = io_params(out_noise=on)
+    return meta, tr
+
+
+CONFIG3_SHAPES = ((785, 256), (257, 128), (129, 10))  # (x_size with bias column, d_size) of the MLP 784-256-128-10
+
+
 def config2_data(x_size=1024, d_size=1024, batch=256):
     w = np.random.default_rng(0).uniform(-0.6, 0.6, (d_size, x_size)).astype(np.float32)
     x = np.random.default_rng(1).uniform(-1, 1, (batch, x_size)).astype(np.float32)

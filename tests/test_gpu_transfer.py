@@ -9,8 +9,8 @@ import torch
 
 from aihwkit_amd.rpu_base import devices as dv
 from aihwkit_amd.rpu_base import tiles
-from helpers import (build_transfer_pair, constant_step, device_weights, io_params, make_meta, noise_free_io,
-                     soft_bounds, transfer_param)
+from helpers import (CONFIG3_SHAPES, build_transfer_pair, config3, constant_step, device_weights, io_params,
+                     make_meta, noise_free_io, soft_bounds, transfer_param)
 from test_gpu_statistics import compare_moments
 
 pytestmark = pytest.mark.gpu
@@ -76,6 +76,37 @@ def test_deterministic_trajectories_match_the_oracle(gpu_device, device, kw):
         y = gpu.forward(cuda(x), False, False, False, False, False).cpu().numpy()
         assert np.abs(y - orc.forward(x)).max() <= 1e-4, step  # one ADC step is 0.047: no flipped code
     assert moved > 1e-3 and np.abs(orc.device_weights(0)).max() > 1e-2  # transfers and gradient steps did happen
+
+
+@pytest.mark.parametrize("shape", CONFIG3_SHAPES)
+def test_configuration_3_tiles_noise_free(gpu_device, shape):
+    """The tile shapes and transfer settings of benchmark configuration 3 (batch 64, one column every two
+    mini-batches), with deterministic pulses and noise-free IO so that the trajectory is comparable."""
+    rng = np.random.default_rng(12)
+    x_size, d_size = shape
+    batch = 64
+    meta, tr = config3(noise=False)
+    meta.update.pulse_type = PT.DeterministicImplicit
+    tr.transfer_update.pulse_type = PT.DeterministicImplicit
+    for dev in tr._vec_par:
+        dev.dw_min_std = 0.0
+    host, orc, gpu = build_transfer_pair(meta, tr, x_size, d_size)
+    w = rng.uniform(-0.3, 0.3, (d_size, x_size)).astype(np.float32)
+    gpu.set_weights(torch.from_numpy(w))
+    orc.set_weights(w)
+    gpu.set_learning_rate(0.1)
+    orc.set_learning_rate(0.1)
+    for step in range(4):
+        x = rng.uniform(0, 1, (batch, x_size)).astype(np.float32)
+        d = (0.2 * rng.standard_normal((batch, d_size))).astype(np.float32)
+        gpu.update(cuda(x), cuda(d), False, False, False, False)
+        orc.update(x, d)
+        check_state(gpu, orc, 2, f"step {step}")
+    assert gpu.get_transfer_state() == (256, [2, 0, 0, 0])
+    assert np.abs(orc.device_weights(0)).max() > 1e-3   # the gradient reached the fast device
+    if d_size > 10:  # with ten outputs the first two columns of A are still below one ADC step when they are read
+        hidden = orc.devices[1].get_hidden()
+        assert np.abs(orc.device_weights(1) - np.clip(w, hidden[1], hidden[0])).max() > 1e-4
 
 
 def test_three_device_chain_with_layouts_and_bias(gpu_device):
