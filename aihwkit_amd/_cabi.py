@@ -84,6 +84,16 @@ class TransferParams(C.Structure):
     ]
 
 
+class PcmNoiseParams(C.Structure):
+    """``rpu_pcm_noise_params``."""
+
+    _fields_ = [
+        ("g_max", f32), ("g_min", f32), ("t_read", f32), ("t_0", f32), ("prog_noise_scale", f32),
+        ("read_noise_scale", f32), ("drift_scale", f32), ("prog_coeff", f32 * 3),
+        ("prog_coeff_g_max_reference", f32),
+    ]
+
+
 # every symbol include/rpu_amd.h declares: name -> (restype, argtypes)
 _P = C.c_void_p
 _FP = C.POINTER(C.c_float)
@@ -94,6 +104,11 @@ SYMBOLS = {
     "rpu_tile_create_transfer": (C.c_int, [C.POINTER(_P), C.c_int, C.c_int, C.POINTER(TileConfig),
                                            C.POINTER(TransferParams)]),
     "rpu_tile_get_transfer_state": (C.c_int, [_P, C.POINTER(C.c_uint64), C.POINTER(C.c_int32)]),
+    "rpu_pcm_noise_params_default": (C.c_int, [C.POINTER(PcmNoiseParams)]),
+    "rpu_tile_program_weights": (C.c_int, [_P, C.POINTER(PcmNoiseParams), C.c_int, _P]),
+    "rpu_tile_drift_weights": (C.c_int, [_P, C.POINTER(PcmNoiseParams), C.c_float, _P]),
+    "rpu_tile_get_drift_state": (C.c_int, [_P, _P, _P, _P]),
+    "rpu_tile_drift_readout": (C.c_int, [_P, C.POINTER(C.c_float), _P]),
     "rpu_tile_clone": (C.c_int, [C.POINTER(_P), _P]),
     "rpu_tile_to_device": (C.c_int, [_P, C.c_int]),
     "rpu_tile_destroy": (C.c_int, [_P]),

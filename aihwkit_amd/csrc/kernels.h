@@ -124,6 +124,22 @@ void launch_implicit_counts(const UpdateArgs &a, int32_t *counts, hipStream_t s)
 // clip weights into [w_min, w_max]
 void launch_clip(float *w, const float *w_min, const float *w_max, size_t n, hipStream_t s);
 
+// ---- inference weight pipeline (kernels_inference.hip) ------------------------------------------
+struct PcmDev {
+  float g_max, g_min, prog_noise_scale, read_noise_scale, drift_scale;
+  float c0, c1, c2, sig_scale; // programming-noise polynomial and g_max / prog_coeff_g_max_reference
+  float drift_base_log2;       // log2(t / t_0) when t > t_0, else 0 (no drift)
+  float read_sigma;            // sqrt(ln((t + t_read) / (2 t_read))) when t > 0, else < 0 (no read noise)
+};
+// abs_max_bits[0] = bits of max |w| (non-negative floats order like their bit patterns)
+void launch_abs_max(const float *w, size_t n, uint32_t *abs_max_bits, hipStream_t s);
+void launch_pcm_program(const float *w_ref, float *w_prog, float *nu_plus, float *nu_minus, size_t n,
+                        const uint32_t *abs_max_bits, const PcmDev &p, PhiloxKey key, uint32_t call, hipStream_t s);
+void launch_pcm_drift(const float *w_prog, const float *nu_plus, const float *nu_minus, float *w_out, size_t n,
+                      const uint32_t *abs_max_bits, const PcmDev &p, PhiloxKey key, uint32_t call, hipStream_t s);
+// out[0] = mean |v| over n values, one workgroup, fixed summation order
+void launch_mean_abs(const float *v, size_t n, float *out, hipStream_t s);
+
 // n_vec unit vectors of length `size`: row v is e_((start + v) % size)
 void launch_unit_vectors(float *out, int n_vec, int size, int start, hipStream_t s);
 

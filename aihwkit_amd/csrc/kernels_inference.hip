@@ -1,0 +1,147 @@
+// Inference weight pipeline on gfx950: statistical PCM programming noise, conductance drift and accumulated
+// 1/f read noise applied to the HBM-resident weight matrix (the reference does this in torch on the host side
+// of its bindings: src/aihwkit/inference/noise/pcm.py:100-158 over
+// src/aihwkit/inference/converter/conductance.py:51-82).  Element-wise kernels, one read and one write of each
+// array: HBM-bound.  Every normal is a Philox draw keyed by (element, call), so a seed reproduces a run.
+#include "kernels.h"
+
+namespace rpu_amd {
+
+namespace {
+
+constexpr float ZERO_CLIP = 1e-7f;
+
+__global__ __launch_bounds__(256) void k_abs_max(const float *w, size_t n, uint32_t *out_bits) {
+  __shared__ float sh[4];
+  float m = 0.0f;
+  for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+    m = fmaxf(m, fabsf(w[i]));
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off));
+  if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = m;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    m = fmaxf(fmaxf(sh[0], sh[1]), fmaxf(sh[2], sh[3]));
+    atomicMax(out_bits, __float_as_uint(m));
+  }
+}
+
+__global__ void k_zero_u32(uint32_t *p) { p[0] = 0u; }
+
+// weights -> (g_plus, g_minus): conductance.py:51-63
+__device__ __forceinline__ void to_conductances(float w, float ratio, const PcmDev &p, float &gp, float &gm) {
+  const float sw = w * ratio;
+  gp = fminf(fmaxf(sw, 0.0f), p.g_max) + p.g_min;
+  gm = fminf(fmaxf(-sw, 0.0f), p.g_max) + p.g_min;
+}
+
+// pcm.py:100-117
+__device__ __forceinline__ float program_conductance(float g, const PcmDev &p, float normal) {
+  const float rel = g / p.g_max;
+  float mat = rel;
+  float sig = p.c0 + mat * p.c1;
+  mat *= rel;
+  sig += mat * p.c2;
+  sig *= p.sig_scale;
+  return fmaxf(g + p.prog_noise_scale * sig * normal, 0.0f);
+}
+
+// pcm.py:119-131
+__device__ __forceinline__ float drift_coefficient(float g, const PcmDev &p, float normal) {
+  const float rel = fmaxf(fabsf(g / p.g_max), ZERO_CLIP);
+  const float lg = logf(rel);
+  const float mu = fminf(fmaxf(-0.0155f * lg + 0.0244f, 0.049f), 0.1f);
+  const float sd = fminf(fmaxf(-0.0125f * lg - 0.0059f, 0.008f), 0.045f);
+  return fmaxf(fabsf(mu + sd * normal), 0.0f) * p.drift_scale;
+}
+
+__global__ __launch_bounds__(256) void k_pcm_program(const float *w_ref, float *w_prog, float *nu_plus, float *nu_minus,
+                                                      size_t n, const uint32_t *abs_max_bits, PcmDev p, PhiloxKey key,
+                                                      uint32_t call) {
+  const float abs_max = __uint_as_float(abs_max_bits[0]);
+  const float ratio = (p.g_max - p.g_min) / fmaxf(abs_max, ZERO_CLIP);
+  for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+    float gp, gm;
+    to_conductances(w_ref[i], ratio, p, gp, gm);
+    float nz[4];
+    philox_normal4((uint32_t)i, (uint32_t)(i >> 32), call, RNG_PCM_PROGRAM, key, nz);
+    const float gp_prog = program_conductance(gp, p, nz[0]);
+    const float gm_prog = program_conductance(gm, p, nz[1]);
+    nu_plus[i] = drift_coefficient(gp, p, nz[2]);
+    nu_minus[i] = drift_coefficient(gm, p, nz[3]);
+    w_prog[i] = ((gp_prog - p.g_min) - (gm_prog - p.g_min)) / ratio; // conductance.py:65-82
+  }
+}
+
+// pcm.py:133-158
+__device__ __forceinline__ float drift_conductance(float g, float nu, const PcmDev &p, float normal) {
+  const float g_drift = p.drift_base_log2 > 0.0f ? g * exp2f(-nu * p.drift_base_log2) : g;
+  if (p.read_sigma < 0.0f) return fmaxf(g, 0.0f);
+  const float q = fminf(0.0088f / fmaxf(powf(fabsf(g) / p.g_max, 0.65f), 1e-3f), 0.2f);
+  const float sig = q * p.read_sigma;
+  return fmaxf(g_drift + fabsf(g_drift) * p.read_noise_scale * sig * normal, 0.0f);
+}
+
+__global__ __launch_bounds__(256) void k_pcm_drift(const float *w_prog, const float *nu_plus, const float *nu_minus,
+                                                    float *w_out, size_t n, const uint32_t *abs_max_bits, PcmDev p,
+                                                    PhiloxKey key, uint32_t call) {
+  const float abs_max = __uint_as_float(abs_max_bits[0]);
+  const float ratio = (p.g_max - p.g_min) / fmaxf(abs_max, ZERO_CLIP);
+  for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+    float gp, gm;
+    to_conductances(w_prog[i], ratio, p, gp, gm);
+    float nz[4];
+    philox_normal4((uint32_t)i, (uint32_t)(i >> 32), call, RNG_PCM_DRIFT, key, nz);
+    const float gp_f = drift_conductance(gp, nu_plus[i], p, nz[0]);
+    const float gm_f = drift_conductance(gm, nu_minus[i], p, nz[1]);
+    w_out[i] = ((gp_f - p.g_min) - (gm_f - p.g_min)) / ratio;
+  }
+}
+
+__global__ __launch_bounds__(1024) void k_mean_abs(const float *v, size_t n, float *out) {
+  __shared__ float sh[16];
+  float acc = 0.0f;
+  for (size_t i = threadIdx.x; i < n; i += blockDim.x) acc += fabsf(v[i]);
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off);
+  if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = acc;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float total = 0.0f;
+    for (int k = 0; k < 16; ++k) total += sh[k];
+    out[0] = total / (float)n;
+  }
+}
+
+int grid_of(size_t n) {
+  size_t blocks = (n + 255) / 256;
+  if (blocks > 4096) blocks = 4096;
+  if (blocks < 1) blocks = 1;
+  return (int)blocks;
+}
+
+} // namespace
+
+void launch_abs_max(const float *w, size_t n, uint32_t *abs_max_bits, hipStream_t s) {
+  hipLaunchKernelGGL(k_zero_u32, dim3(1), dim3(1), 0, s, abs_max_bits);
+  hipLaunchKernelGGL(k_abs_max, dim3(grid_of(n)), dim3(256), 0, s, w, n, abs_max_bits);
+}
+
+void launch_pcm_program(const float *w_ref, float *w_prog, float *nu_plus, float *nu_minus, size_t n,
+                        const uint32_t *abs_max_bits, const PcmDev &p, PhiloxKey key, uint32_t call, hipStream_t s) {
+  hipLaunchKernelGGL(k_pcm_program, dim3(grid_of(n)), dim3(256), 0, s, w_ref, w_prog, nu_plus, nu_minus, n, abs_max_bits,
+                     p, key, call);
+}
+
+void launch_pcm_drift(const float *w_prog, const float *nu_plus, const float *nu_minus, float *w_out, size_t n,
+                      const uint32_t *abs_max_bits, const PcmDev &p, PhiloxKey key, uint32_t call, hipStream_t s) {
+  hipLaunchKernelGGL(k_pcm_drift, dim3(grid_of(n)), dim3(256), 0, s, w_prog, nu_plus, nu_minus, w_out, n, abs_max_bits, p,
+                     key, call);
+}
+
+void launch_mean_abs(const float *v, size_t n, float *out, hipStream_t s) {
+  hipLaunchKernelGGL(k_mean_abs, dim3(1), dim3(1024), 0, s, v, n, out);
+}
+
+} // namespace rpu_amd

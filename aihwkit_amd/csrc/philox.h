@@ -65,7 +65,9 @@ enum RngPurpose : uint32_t {
   RNG_PULSE_X = 5,    // x bit lines
   RNG_PULSE_D = 6,    // d bit lines
   RNG_CTOC = 7,       // cycle-to-cycle update noise
-  RNG_UPDATE_SR = 8   // stochastic rounding of pulse probabilities
+  RNG_UPDATE_SR = 8,  // stochastic rounding of pulse probabilities
+  RNG_PCM_PROGRAM = 9, // programming noise and drift coefficients of the inference weight pipeline
+  RNG_PCM_DRIFT = 10   // accumulated read noise at inference time
 };
 
 // uniform in [0, 1) with 24 bits

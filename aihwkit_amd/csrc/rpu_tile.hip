@@ -9,6 +9,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <cmath>
 #include <cstring>
 #include <memory>
 #include <mutex>
@@ -151,6 +152,10 @@ struct Tile {
   uint64_t update_idx = 0;
   std::vector<int> slice_idx;
   DevBuf<float> t_unit, t_read;
+  // inference weight pipeline: reference and programmed weights, drift coefficients of both conductances
+  DevBuf<float> i_ref, i_prog, i_nu_plus, i_nu_minus, i_scalar;
+  DevBuf<uint32_t> i_absmax;
+  bool has_reference = false, programmed = false;
   int last_update_batch = 0;
   int last_update_pulse = -1;
   int last_forward_batch = 0;
@@ -207,6 +212,8 @@ struct Tile {
     u_bl.release(); u_a.release(); u_b.release(); u_xval.release(); u_dval.release(); u_xw.release(); u_dw.release();
     u_xpl.release(); u_dpl.release(); u_kmax.release();
     t_unit.release(); t_read.release();
+    i_ref.release(); i_prog.release(); i_nu_plus.release(); i_nu_minus.release(); i_scalar.release(); i_absmax.release();
+    has_reference = programmed = false;
     for (auto &sl : slots) sl->release();
   }
 
@@ -511,6 +518,71 @@ struct Tile {
     last_update_pulse = up.p.pulse_type;
   }
 
+  // ---- inference weight pipeline ------------------------------------------------------------------
+
+  static PcmDev pcm_dev(const rpu_pcm_noise_params &q, float t_inference) {
+    if (!(q.g_max > 0.0f) || q.g_min < 0.0f || q.g_min >= q.g_max) throw RpuError("g_min should be smaller than g_max");
+    PcmDev p{};
+    p.g_max = q.g_max; p.g_min = q.g_min;
+    p.prog_noise_scale = q.prog_noise_scale; p.read_noise_scale = q.read_noise_scale; p.drift_scale = q.drift_scale;
+    p.c0 = q.prog_coeff[0]; p.c1 = q.prog_coeff[1]; p.c2 = q.prog_coeff[2];
+    p.sig_scale = q.g_max / q.prog_coeff_g_max_reference;
+    const double t = (double)t_inference + (double)q.t_0; // pcm.py:138-152
+    p.drift_base_log2 = t > (double)q.t_0 ? (float)std::log2(t / (double)q.t_0) : 0.0f;
+    p.read_sigma = t > 0.0 ? (float)std::sqrt(std::log((t + (double)q.t_read) / (2.0 * (double)q.t_read))) : -1.0f;
+    return p;
+  }
+
+  void check_inference_tile() {
+    if (!resident()) throw RpuError("Tile is not resident on a GPU.");
+    if (is_transfer() || dev.pulsed()) {
+      throw RpuError("The inference weight pipeline needs a tile with an ideal device (as InferenceRPUConfig has).");
+    }
+  }
+
+  void program_weights(const rpu_pcm_noise_params &q, bool from_reference, hipStream_t s) {
+    check_inference_tile();
+    const size_t n = size();
+    i_ref.ensure(n); i_prog.ensure(n); i_nu_plus.ensure(n); i_nu_minus.ensure(n); i_absmax.ensure(1);
+    if (!from_reference || !has_reference) {
+      RPU_HIP_CHECK(hipMemcpyAsync(i_ref.p, d_w.p, n * sizeof(float), hipMemcpyDeviceToDevice, s));
+      has_reference = true;
+    }
+    const PcmDev p = pcm_dev(q, 0.0f);
+    launch_abs_max(i_ref.p, n, i_absmax.p, s);
+    launch_pcm_program(i_ref.p, i_prog.p, i_nu_plus.p, i_nu_minus.p, n, i_absmax.p, p, key(), call++, s);
+    RPU_HIP_CHECK(hipMemcpyAsync(d_w.p, i_prog.p, n * sizeof(float), hipMemcpyDeviceToDevice, s));
+    RPU_HIP_CHECK(hipGetLastError());
+    programmed = true;
+    last_stream = s;
+  }
+
+  void drift_weights(const rpu_pcm_noise_params &q, float t_inference, hipStream_t s) {
+    check_inference_tile();
+    if (!programmed) program_weights(q, true, s);
+    const size_t n = size();
+    const PcmDev p = pcm_dev(q, t_inference);
+    launch_abs_max(i_prog.p, n, i_absmax.p, s);
+    launch_pcm_drift(i_prog.p, i_nu_plus.p, i_nu_minus.p, d_w.p, n, i_absmax.p, p, key(), call++, s);
+    RPU_HIP_CHECK(hipGetLastError());
+    last_stream = s;
+  }
+
+  float drift_readout(hipStream_t s) {
+    check_inference_tile();
+    t_unit.ensure((size_t)X * X);
+    t_read.ensure((size_t)X * D);
+    i_scalar.ensure(1);
+    launch_unit_vectors(t_unit.p, X, X, 0, s);
+    mvm(t_unit.p, t_read.p, X, false, false, false, false, s);
+    launch_mean_abs(t_read.p, (size_t)X * D, i_scalar.p, s);
+    float value = 0.0f;
+    RPU_HIP_CHECK(hipMemcpyAsync(&value, i_scalar.p, sizeof(float), hipMemcpyDeviceToHost, s));
+    RPU_HIP_CHECK(hipStreamSynchronize(s));
+    last_stream = s;
+    return std::max(value, 0.0001f);
+  }
+
   // ---- transfer compound ----------------------------------------------------------------------
 
   // tile weights = sum_k gamma_k w_k, unless the last device alone is visible (rpu_transfer_device.cpp:596-602)
@@ -726,6 +798,66 @@ int rpu_tile_create_transfer(rpu_tile_t **out, int x_size, int d_size, const rpu
     std::vector<float> zeros(t.size(), 0.0f);
     t.transfer_set_weights_host(zeros.data());
     *out = h.release();
+  });
+}
+
+int rpu_pcm_noise_params_default(rpu_pcm_noise_params *p) {
+  return guarded([&] {
+    if (!p) throw RpuError("null argument");
+    rpu_pcm_noise_params q{};
+    q.g_max = 25.0f; q.g_min = 0.0f; q.t_read = 250.0e-9f; q.t_0 = 20.0f;
+    q.prog_noise_scale = 1.0f; q.read_noise_scale = 1.0f; q.drift_scale = 1.0f;
+    q.prog_coeff[0] = 0.26348f; q.prog_coeff[1] = 1.9650f; q.prog_coeff[2] = -1.1731f;
+    q.prog_coeff_g_max_reference = 25.0f;
+    *p = q;
+  });
+}
+
+int rpu_tile_program_weights(rpu_tile_t *tile, const rpu_pcm_noise_params *p, int from_reference, void *stream) {
+  return guarded([&] {
+    if (!tile || !p) throw RpuError("null argument");
+    Tile &t = tile->t;
+    std::lock_guard<std::mutex> lock(t.mutex);
+    if (!t.resident()) throw RpuError("Tile is not resident on a GPU.");
+    DeviceGuard g(t.device_id);
+    t.program_weights(*p, from_reference != 0, (hipStream_t)stream);
+  });
+}
+
+int rpu_tile_drift_weights(rpu_tile_t *tile, const rpu_pcm_noise_params *p, float t_inference, void *stream) {
+  return guarded([&] {
+    if (!tile || !p) throw RpuError("null argument");
+    Tile &t = tile->t;
+    std::lock_guard<std::mutex> lock(t.mutex);
+    if (!t.resident()) throw RpuError("Tile is not resident on a GPU.");
+    DeviceGuard g(t.device_id);
+    t.drift_weights(*p, t_inference, (hipStream_t)stream);
+  });
+}
+
+int rpu_tile_get_drift_state(rpu_tile_t *tile, float *programmed_host, float *nu_plus_host, float *nu_minus_host) {
+  return guarded([&] {
+    if (!tile) throw RpuError("null tile");
+    Tile &t = tile->t;
+    std::lock_guard<std::mutex> lock(t.mutex);
+    if (!t.resident() || !t.programmed) throw RpuError("The weights have not been programmed.");
+    DeviceGuard g(t.device_id);
+    t.sync_last();
+    const size_t bytes = t.size() * sizeof(float);
+    if (programmed_host) RPU_HIP_CHECK(hipMemcpy(programmed_host, t.i_prog.p, bytes, hipMemcpyDeviceToHost));
+    if (nu_plus_host) RPU_HIP_CHECK(hipMemcpy(nu_plus_host, t.i_nu_plus.p, bytes, hipMemcpyDeviceToHost));
+    if (nu_minus_host) RPU_HIP_CHECK(hipMemcpy(nu_minus_host, t.i_nu_minus.p, bytes, hipMemcpyDeviceToHost));
+  });
+}
+
+int rpu_tile_drift_readout(rpu_tile_t *tile, float *mean_abs_host, void *stream) {
+  return guarded([&] {
+    if (!tile || !mean_abs_host) throw RpuError("null argument");
+    Tile &t = tile->t;
+    std::lock_guard<std::mutex> lock(t.mutex);
+    if (!t.resident()) throw RpuError("Tile is not resident on a GPU.");
+    DeviceGuard g(t.device_id);
+    *mean_abs_host = t.drift_readout((hipStream_t)stream);
   });
 }
 

@@ -223,6 +223,22 @@ typedef struct rpu_transfer_params {
   rpu_device_params rest_device;
 } rpu_transfer_params;
 
+/* Replaces PCMLikeNoiseModel (src/aihwkit/inference/noise/pcm.py:27-158) over the
+ * SinglePairConductanceConverter (src/aihwkit/inference/converter/conductance.py:24-82): statistical
+ * programming noise, conductance drift and accumulated 1/f read noise of PCM devices, applied to the
+ * weight matrix of an inference tile.  Defaults are the Python defaults. */
+typedef struct rpu_pcm_noise_params {
+  float g_max;                      /* 25 (uS) */
+  float g_min;                      /* 0 */
+  float t_read;                     /* 250e-9 (s) */
+  float t_0;                        /* 20 (s) */
+  float prog_noise_scale;           /* 1 */
+  float read_noise_scale;           /* 1 */
+  float drift_scale;                /* 1 */
+  float prog_coeff[3];              /* 0.26348, 1.9650, -1.1731 */
+  float prog_coeff_g_max_reference; /* 25 */
+} rpu_pcm_noise_params;
+
 typedef struct rpu_tile rpu_tile_t; /* opaque */
 
 /* ---- defaults ---------------------------------------------------------------- */
@@ -320,6 +336,32 @@ int rpu_tile_set_hidden_parameters(rpu_tile_t *tile, const float *data_host);
  * function of (seed, call index, purpose, element index); the call index restarts at 0 here.
  * Stands in for the per-context cuRAND state of the reference (C/cuda_util.cu:163-176,779-800). */
 int rpu_tile_set_seed(rpu_tile_t *tile, uint64_t seed);
+
+/* ---- inference weight pipeline ------------------------------------------------------------- */
+
+int rpu_pcm_noise_params_default(rpu_pcm_noise_params *p);
+
+/* Replaces InferenceTileWithPeriphery.program_weights (src/aihwkit/simulator/tiles/inference.py:161-213) with
+ * BaseNoiseModel.apply_programming_noise (src/aihwkit/inference/noise/base.py:82-103): the reference weights
+ * (the current weights, taken anew unless from_reference != 0 and a reference exists) are mapped to a pair of
+ * conductances per cross-point, programming noise is added and the drift coefficients of both conductances
+ * are drawn (pcm.py:100-131); the tile's weights become the programmed weights.  All on the GPU: the
+ * reference moves the matrix to the host and back.  GPU tiles with an ideal device only. */
+int rpu_tile_program_weights(rpu_tile_t *tile, const rpu_pcm_noise_params *p, int from_reference, void *stream);
+
+/* Replaces InferenceTileWithPeriphery.drift_weights (inference.py:215-262) with BaseNoiseModel.apply_drift_noise
+ * (base.py:105-131, pcm.py:133-158): the tile's weights become the programmed weights drifted to t_inference
+ * seconds after programming with accumulated read noise.  Programs first if that has not happened. */
+int rpu_tile_drift_weights(rpu_tile_t *tile, const rpu_pcm_noise_params *p, float t_inference, void *stream);
+
+/* Host copies [d_size][x_size] of the programmed weights and of the drift coefficients of the positive and
+ * the negative conductance (InferenceTile.programmed_weights, drift_noise_parameters); NULL pointers are skipped. */
+int rpu_tile_get_drift_state(rpu_tile_t *tile, float *programmed_host, float *nu_plus_host, float *nu_minus_host);
+
+/* Read-out of GlobalDriftCompensation (src/aihwkit/inference/compensation/drift.py:21-41, base.py:25-62):
+ * the unit vectors are forwarded through the tile and max(mean |output|, 1e-4) is returned; the ratio of the
+ * value after programming to the value after drift is the output scale alpha. */
+int rpu_tile_drift_readout(rpu_tile_t *tile, float *mean_abs_host, void *stream);
 
 /* ---- inspection hooks (mirror the reference's debug hooks) ------------------------------ */
 

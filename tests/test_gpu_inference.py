@@ -1,0 +1,163 @@
+"""GPU parity of the inference weight pipeline (PCM programming noise, drift, read noise, global drift
+compensation) against the numpy PCM oracle: exact where the model is deterministic, by moments where it draws."""
+import numpy as np
+import pytest
+import torch
+
+from aihwkit_amd.inference import InferenceTile, PCMLikeNoiseModel
+from aihwkit_amd.rpu_base import devices as dv
+from helpers import io_params, make_meta, noise_free_io
+from oracle_lib import OracleTile
+from pcm_oracle import PcmOracle
+
+pytestmark = pytest.mark.gpu
+
+DAY = 86400.0
+
+
+def make_tile(out_size, in_size, w, **model):
+    tile = InferenceTile(out_size, in_size, forward_io=noise_free_io(inp_res=1 / 254.0, out_res=1 / 254.0),
+                         noise_model=PCMLikeNoiseModel(**model))
+    tile.set_weights(torch.from_numpy(w))
+    return tile.cuda()
+
+
+def test_deterministic_parts_match_the_oracle(gpu_device):
+    rng = np.random.default_rng(0)
+    w = rng.normal(0, 0.3, (96, 130)).astype(np.float32)
+    tile = make_tile(96, 130, w, prog_noise_scale=0.0, read_noise_scale=0.0, g_min=1.0)
+    tile.tile.set_seed(5)
+    tile.program_weights()
+    prog, nu_p, nu_m = (t.numpy() for t in tile.drift_state())
+    assert np.abs(prog - w).max() <= 1e-6 and np.abs(tile.get_weights().numpy() - w).max() <= 1e-6
+    orc = PcmOracle(prog_noise_scale=0.0, read_noise_scale=0.0, g_min=1.0)
+    for t_inf in (0.0, 3600.0, DAY, 365 * DAY):
+        tile.drift_weights(t_inf)
+        want = orc.apply_drift_noise(prog, [nu_p, nu_m], t_inf)
+        assert np.abs(tile.get_weights().numpy() - want).max() <= 1e-5, t_inf
+    # drifting starts from the programmed weights every time, not from the drifted ones
+    tile.drift_weights(0.0)
+    assert np.abs(tile.get_weights().numpy() - prog).max() <= 1e-6
+    # from_reference: programming again starts from the stored reference, not from the current weights
+    tile.drift_weights(DAY)
+    tile.program_weights(from_reference=True)
+    assert np.abs(tile.get_weights().numpy() - w).max() <= 1e-6
+    tile.set_weights(torch.from_numpy(2 * w))
+    tile.program_weights(from_reference=False)
+    assert np.abs(tile.get_weights().numpy() - 2 * w).max() <= 2e-6
+
+
+def binned_moments(g_rel, values, edges):
+    out = []
+    for lo, hi in zip(edges[:-1], edges[1:]):
+        sel = (g_rel >= lo) & (g_rel < hi)
+        out.append((values[sel].mean(), values[sel].std(), int(sel.sum())))
+    return out
+
+
+def test_programming_noise_and_drift_coefficients_by_conductance_bin(gpu_device):
+    rng = np.random.default_rng(1)
+    w = rng.uniform(-1, 1, (512, 512)).astype(np.float32)
+    w.flat[0] = 1.0
+    tile = make_tile(512, 512, w)
+    tile.tile.set_seed(7)
+    tile.program_weights()
+    prog, nu_p, nu_m = (t.numpy() for t in tile.drift_state())
+    orc = PcmOracle(seed=11)
+    want_prog, (want_nu_p, want_nu_m) = orc.apply_programming_noise(w)
+    edges = np.linspace(0.0, 1.0, 9)
+    g_rel = np.abs(w)
+    for got, want, what in [(prog - w, want_prog - w, "programming error"), (np.where(w > 0, nu_p, nu_m),
+                                                                             np.where(w > 0, want_nu_p, want_nu_m), "nu")]:
+        for (m_g, s_g, n), (m_w, s_w, _) in zip(binned_moments(g_rel, got, edges), binned_moments(g_rel, want, edges)):
+            assert abs(m_g - m_w) < 4.5 * np.hypot(s_g, s_w) / np.sqrt(n), what
+            assert abs(s_g - s_w) < 4.5 * s_w / np.sqrt(2 * n) + 1e-9, what
+    # the device that is not used sits at g_min = 0: half-normal programming noise, drift coefficient at the upper clips
+    idle = np.where(w > 0, nu_m, nu_p)
+    assert idle.mean() == pytest.approx(0.1, rel=0.02) and idle.std() == pytest.approx(0.045, rel=0.05)
+    # the two conductances of a cross-point draw independently
+    strong = w > 0.5
+    assert abs(np.corrcoef(nu_p[strong], nu_m[strong])[0, 1]) < 0.03
+    # a second programming run draws new noise, a re-seeded one repeats
+    tile.program_weights()
+    again = tile.drift_state()[0].numpy()
+    assert np.abs(again - prog).max() > 1e-3
+    tile.tile.set_seed(7)
+    tile.program_weights()
+    assert np.array_equal(tile.drift_state()[0].numpy(), prog)
+
+
+def test_drift_with_read_noise_by_conductance_bin(gpu_device):
+    rng = np.random.default_rng(2)
+    w = rng.uniform(-1, 1, (512, 512)).astype(np.float32)
+    w.flat[0] = -1.0
+    tile = make_tile(512, 512, w, prog_noise_scale=0.0)
+    tile.tile.set_seed(9)
+    tile.program_weights()
+    prog, nu_p, nu_m = (t.numpy() for t in tile.drift_state())
+    tile.drift_weights(DAY)
+    got = tile.get_weights().numpy()
+    want = PcmOracle(prog_noise_scale=0.0, seed=21).apply_drift_noise(prog, [nu_p, nu_m], DAY)
+    clean = PcmOracle(prog_noise_scale=0.0, read_noise_scale=0.0).apply_drift_noise(prog, [nu_p, nu_m], DAY)
+    edges = np.linspace(0.0, 1.0, 9)
+    for (m_g, s_g, n), (m_w, s_w, _) in zip(binned_moments(np.abs(w), got - clean, edges),
+                                            binned_moments(np.abs(w), want - clean, edges)):
+        assert abs(m_g - m_w) < 4.5 * np.hypot(s_g, s_w) / np.sqrt(n)
+        assert abs(s_g - s_w) < 4.5 * s_w / np.sqrt(2 * n)
+
+
+def test_global_drift_compensation_restores_the_output_level(gpu_device):
+    rng = np.random.default_rng(3)
+    w = rng.normal(0, 0.25, (256, 384)).astype(np.float32)
+    tile = make_tile(256, 384, w)
+    tile.tile.set_seed(3)
+    tile.program_weights()
+    assert tile.alpha == 1.0 and tile.drift_baseline > 0
+    # the read-out is the mean |output| of the unit vectors = mean |programmed weight| up to the ADC
+    assert tile.drift_baseline == pytest.approx(np.abs(tile.get_weights().numpy()).mean(), rel=0.05)
+    x = torch.from_numpy(rng.normal(0, 1, (64, 384)).astype(np.float32)).cuda()
+    fresh = tile.forward(x, is_test=True).cpu().numpy()
+    tile.drift_weights(30 * DAY)
+    assert tile.alpha == pytest.approx((30 * DAY / 20.0) ** 0.06, rel=0.15)      # typical nu ~ 0.06
+    raw = tile.forward(x, is_test=False).cpu().numpy()
+    compensated = tile.forward(x, is_test=True).cpu().numpy()
+    assert np.abs(raw).mean() < 0.7 * np.abs(fresh).mean()
+    assert np.abs(compensated).mean() == pytest.approx(np.abs(fresh).mean(), rel=0.05)
+    assert np.corrcoef(compensated.ravel(), fresh.ravel())[0, 1] > 0.97
+
+
+def test_inference_forward_after_drift_matches_the_oracle_tile(gpu_device):
+    """Transformer-width tile (512 x 512, 1024 tokens, 8-bit converters) with drifted weights: the analog
+    forward pass on those weights against the CPU oracle tile holding the same weights."""
+    rng = np.random.default_rng(4)
+    w = rng.normal(0, 0.02, (512, 512)).astype(np.float32)
+    io = noise_free_io(inp_res=1 / 254.0, out_res=1 / 254.0, noise_management=dv.NoiseManagementType.AbsMax)
+    tile = InferenceTile(512, 512, forward_io=io)
+    tile.set_weights(torch.from_numpy(w))
+    tile.cuda()
+    tile.tile.set_seed(1)
+    tile.drift_weights(DAY)                      # programs first
+    drifted = tile.get_weights().numpy()
+    assert 0.4 < np.abs(drifted).mean() / np.abs(w).mean() < 0.9
+    meta = make_meta(io, noise_free_io())
+    meta.backward_io.is_perfect = True
+    meta.update.pulse_type = dv.PulseType.NONE
+    orc = OracleTile(512, 512, meta._config(dv.IdealResistiveDeviceParameter()))
+    orc.set_weights(drifted)
+    x = rng.normal(0, 1, (1024, 512)).astype(np.float32)
+    got = tile.forward(torch.from_numpy(x).cuda(), is_test=False).cpu().numpy()
+    want = orc.forward(x)
+    step = np.abs(x).max(1, keepdims=True) * 24.0 / 254.0        # one ADC code after noise management
+    off = np.abs(got - want) > 1e-5
+    assert off.mean() < 0.005 and np.all(np.abs(got - want)[off] <= 1.001 * np.broadcast_to(step, got.shape)[off])
+
+
+def test_pipeline_needs_an_ideal_device_gpu_tile(gpu_device):
+    from helpers import build_pair, constant_step
+    _, _, gpu = build_pair(make_meta(), constant_step(), 8, 8)
+    from aihwkit_amd._cabi import PcmNoiseParams, lib
+    import ctypes as C
+    p = PcmNoiseParams()
+    assert lib().rpu_pcm_noise_params_default(C.byref(p)) == 0 and p.g_max == 25.0
+    assert lib().rpu_tile_program_weights(gpu._h, C.byref(p), 1, None) != 0
+    assert b"ideal device" in lib().rpu_last_error()
