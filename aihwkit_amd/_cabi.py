@@ -104,6 +104,9 @@ SYMBOLS = {
     "rpu_tile_create_transfer": (C.c_int, [C.POINTER(_P), C.c_int, C.c_int, C.POINTER(TileConfig),
                                            C.POINTER(TransferParams)]),
     "rpu_tile_get_transfer_state": (C.c_int, [_P, C.POINTER(C.c_uint64), C.POINTER(C.c_int32)]),
+    "rpu_group_create": (C.c_int, [C.POINTER(_P), C.POINTER(_P), C.c_int]),
+    "rpu_group_forward": (C.c_int, [_P, C.POINTER(_P), C.POINTER(_P), C.c_int, C.c_int, _P]),
+    "rpu_group_destroy": (C.c_int, [_P]),
     "rpu_pcm_noise_params_default": (C.c_int, [C.POINTER(PcmNoiseParams)]),
     "rpu_tile_program_weights": (C.c_int, [_P, C.POINTER(PcmNoiseParams), C.c_int, _P]),
     "rpu_tile_drift_weights": (C.c_int, [_P, C.POINTER(PcmNoiseParams), C.c_float, _P]),

@@ -59,6 +59,20 @@ struct MvmArgs {
 void launch_mvm_init(const MvmArgs &a, hipStream_t s);
 // one round of DAC -> MFMA contraction -> ADC
 void launch_mvm_round(const MvmArgs &a, hipStream_t s);
+// Several tiles in one launch: args[t] are the tiles' arguments in HBM, start[t] .. start[t + 1] the workgroups of
+// tile t in a round launch (all tiles share m_batch).  The tiles of one round launch share a kernel variant.
+struct MvmGroup {
+  const MvmArgs *args;
+  const int *start; // [n + 1]
+  int n;
+  int m_batch;
+};
+void launch_mvm_init_group(const MvmGroup &g, hipStream_t s);
+void launch_mvm_round_group(const MvmGroup &g, int prefetch_depth, int weight_mode, int total_workgroups, int round,
+                            hipStream_t s);
+int mvm_round_workgroups(const MvmArgs &a);            // workgroups of a round launch for this tile
+void mvm_round_variant(const MvmArgs &a, int &prefetch_depth, int &weight_mode);
+
 // number of rounds that can ever be needed with these IO settings
 int mvm_max_rounds(const IoDev &io);
 // row length of the quantized-input scratch for a contraction length K

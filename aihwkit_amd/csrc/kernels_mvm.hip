@@ -660,17 +660,44 @@ __device__ __forceinline__ void mvm_tile_finished(const MvmArgs &a, int round, i
   }
 }
 
+// work of workgroup number n of a round launch of one tile
+template <int PD, int WMODE>
+__device__ __forceinline__ void mvm_round_workgroup(const MvmArgs &a, int round, int n, float (*red)[16][64],
+                                                    float *stage) {
+  const int n_act = (round > 0) ? a.st.count[round] : a.m_batch;
+  int tile_o, tile_b;
+  if (!tile_of(a, n, n_act, tile_o, tile_b)) return;
+  const bool more_rounds = round + 1 < a.max_rounds;
+  if (more_rounds) mvm_prepare_next_rows(a, round, tile_o, tile_b, n_act);
+  mvm_round_tile<PD, WMODE>(a, round, tile_o, tile_b, n_act, red, stage);
+  if (more_rounds) mvm_tile_finished(a, round, tile_b, n_act);
+}
+
 template <int PD, int WMODE>
 __global__ __launch_bounds__(256) void k_mvm_round(MvmArgs a) {
   __shared__ float red[WAVES][16][64];
   __shared__ __attribute__((aligned(16))) float stage[WAVES * 2 * TILE * LDS_ROW];
-  const int n_act = (a.round > 0) ? a.st.count[a.round] : a.m_batch;
-  int tile_o, tile_b;
-  if (!tile_of(a, blockIdx.x, n_act, tile_o, tile_b)) return;
-  const bool more_rounds = a.round + 1 < a.max_rounds;
-  if (more_rounds) mvm_prepare_next_rows(a, a.round, tile_o, tile_b, n_act);
-  mvm_round_tile<PD, WMODE>(a, a.round, tile_o, tile_b, n_act, red, stage);
-  if (more_rounds) mvm_tile_finished(a, a.round, tile_b, n_act);
+  mvm_round_workgroup<PD, WMODE>(a, a.round, blockIdx.x, red, stage);
+}
+
+// The same for several tiles in one launch: a workgroup finds its tile in the table of first workgroup numbers
+// (a multiple of 8 per tile, so the XCD of a workgroup is the one its tile-local number implies).
+template <int PD, int WMODE>
+__global__ __launch_bounds__(256) void k_mvm_round_group(MvmGroup g, int round) {
+  __shared__ float red[WAVES][16][64];
+  __shared__ __attribute__((aligned(16))) float stage[WAVES * 2 * TILE * LDS_ROW];
+  int t = 0;
+  while (t + 1 < g.n && (int)blockIdx.x >= g.start[t + 1]) ++t;
+  const MvmArgs &a = g.args[t];
+  if (round > 0 && round >= a.max_rounds) return;
+  mvm_round_workgroup<PD, WMODE>(a, round, (int)blockIdx.x - g.start[t], red, stage);
+}
+
+__global__ __launch_bounds__(256) void k_mvm_init_group(MvmGroup g) {
+  __shared__ float sh[8];
+  __shared__ float sh_scale;
+  const int t = blockIdx.x / g.m_batch;
+  mvm_init_sample(g.args[t], blockIdx.x - t * g.m_batch, sh, &sh_scale);
 }
 
 __global__ void k_make_bias(const float *in, float *out, int m_batch, int x_size, int in_trans) {
@@ -733,11 +760,43 @@ void launch_mvm_init(const MvmArgs &a, hipStream_t s) {
   hipLaunchKernelGGL(k_mvm_init, dim3(a.m_batch), dim3(256), 0, s, a);
 }
 
-void launch_mvm_round(const MvmArgs &a, hipStream_t s) {
+int mvm_round_workgroups(const MvmArgs &a) {
   const int tiles_o = (a.O + TILE - 1) / TILE;
   const int per = (tiles_o + 7) / 8;
   const int tiles_b = (a.m_batch + TILE - 1) / TILE;
-  const dim3 grid(8 * per * tiles_b);
+  return 8 * per * tiles_b;
+}
+
+void mvm_round_variant(const MvmArgs &a, int &prefetch_depth, int &mode) {
+  prefetch_depth = mvm_prefetch_depth(a.K);
+  mode = weight_mode(a);
+}
+
+void launch_mvm_init_group(const MvmGroup &g, hipStream_t s) {
+  hipLaunchKernelGGL(k_mvm_init_group, dim3(g.n * g.m_batch), dim3(256), 0, s, g);
+}
+
+void launch_mvm_round_group(const MvmGroup &g, int depth, int mode, int total_workgroups, int round, hipStream_t s) {
+  const dim3 grid(total_workgroups);
+#define RPU_LAUNCH_ROUND(PD, WMODE) hipLaunchKernelGGL((k_mvm_round_group<PD, WMODE>), grid, dim3(256), 0, s, g, round)
+  if (mode == 0) {
+    if (depth == 4) RPU_LAUNCH_ROUND(4, 0);
+    else if (depth == 2) RPU_LAUNCH_ROUND(2, 0);
+    else RPU_LAUNCH_ROUND(1, 0);
+  } else if (mode == 1) {
+    if (depth == 4) RPU_LAUNCH_ROUND(4, 1);
+    else if (depth == 2) RPU_LAUNCH_ROUND(2, 1);
+    else RPU_LAUNCH_ROUND(1, 1);
+  } else {
+    if (depth == 4) RPU_LAUNCH_ROUND(4, 2);
+    else if (depth == 2) RPU_LAUNCH_ROUND(2, 2);
+    else RPU_LAUNCH_ROUND(1, 2);
+  }
+#undef RPU_LAUNCH_ROUND
+}
+
+void launch_mvm_round(const MvmArgs &a, hipStream_t s) {
+  const dim3 grid(mvm_round_workgroups(a));
   const int depth = mvm_prefetch_depth(a.K);
   const int mode = weight_mode(a);
 #define RPU_LAUNCH_ROUND(PD, WMODE) hipLaunchKernelGGL((k_mvm_round<PD, WMODE>), grid, dim3(256), 0, s, a)

@@ -309,9 +309,8 @@ struct Tile {
   }
 
   // shared driver of forward (transposed = 0) and backward (transposed = 1)
-  void mvm(const float *in, float *out, int B, bool bias, bool in_trans, bool out_trans, bool transposed, hipStream_t s,
-           const float *w_other = nullptr, const IOPar *io_other = nullptr) {
-    const IOPar &io = io_other ? *io_other : (transposed ? bio : fio);
+  // arguments of the MVM kernels for one call, scratch sized for B samples; the caller sets in / out
+  MvmArgs mvm_args(int B, bool transposed, const float *w_other, const IOPar &io) {
     const int K = transposed ? D : X;
     const int O = transposed ? X : D;
     ensure_mvm_scratch(B);
@@ -331,6 +330,14 @@ struct Tile {
     s_xq0.ensure((size_t)B * a.k_pad);
     if (!io.perfect && io.p.bound_management != RPU_BM_NONE) s_xq1.ensure((size_t)B * a.k_pad);
     a.xq[0] = s_xq0.p; a.xq[1] = s_xq1.p;
+    a.max_rounds = io.perfect ? 0 : mvm_max_rounds(a.io);
+    return a;
+  }
+
+  void mvm(const float *in, float *out, int B, bool bias, bool in_trans, bool out_trans, bool transposed, hipStream_t s,
+           const float *w_other = nullptr, const IOPar *io_other = nullptr) {
+    const IOPar &io = io_other ? *io_other : (transposed ? bio : fio);
+    MvmArgs a = mvm_args(B, transposed, w_other, io);
 
     // the x side carries the optional bias column: input of forward, output of backward
     float *final_out = out;
@@ -365,7 +372,6 @@ struct Tile {
       prof_mark(s, "mvm_init");
       // every round after the first works on the samples whose ADC saturated in the one before; the
       // last workgroup to finish a sample tile sets up the next round for that tile
-      a.max_rounds = mvm_max_rounds(a.io);
       for (int r = 0; r < a.max_rounds; ++r) {
         a.round = r;
         launch_mvm_round(a, s);
@@ -798,6 +804,134 @@ int rpu_tile_create_transfer(rpu_tile_t **out, int x_size, int d_size, const rpu
     std::vector<float> zeros(t.size(), 0.0f);
     t.transfer_set_weights_host(zeros.data());
     *out = h.release();
+  });
+}
+
+// ---- grouped forward over several tiles ------------------------------------------------------------
+
+struct rpu_group {
+  std::vector<rpu_tile *> tiles;
+  int device_id = -1;
+  DevBuf<MvmArgs> d_args;
+  DevBuf<int> d_start;
+  MvmArgs *h_args = nullptr; // pinned staging
+  int *h_start = nullptr;
+  hipEvent_t copied = nullptr;
+  std::mutex mutex;
+  ~rpu_group() {
+    if (device_id >= 0) {
+      try {
+        DeviceGuard g(device_id);
+        if (copied) {
+          (void)hipEventSynchronize(copied);
+          (void)hipEventDestroy(copied);
+        }
+        if (h_args) (void)hipHostFree(h_args);
+        if (h_start) (void)hipHostFree(h_start);
+        d_args.release();
+        d_start.release();
+      } catch (...) {
+      }
+    }
+  }
+};
+
+int rpu_group_create(rpu_group_t **out, rpu_tile_t *const *tiles, int n_tiles) {
+  return guarded([&] {
+    if (!out || !tiles || n_tiles <= 0) throw RpuError("null or empty tile list");
+    auto g = std::make_unique<rpu_group>();
+    for (int i = 0; i < n_tiles; ++i) {
+      if (!tiles[i]) throw RpuError("null tile in the list");
+      for (int j = 0; j < i; ++j) {
+        if (tiles[j] == tiles[i]) throw RpuError("A tile may be in a group only once.");
+      }
+      Tile &t = tiles[i]->t;
+      if (!t.resident()) throw RpuError("All tiles of a group must be resident on a GPU.");
+      if (g->device_id < 0) g->device_id = t.device_id;
+      if (t.device_id != g->device_id) throw RpuError("All tiles of a group must be on the same GPU.");
+      g->tiles.push_back(tiles[i]);
+    }
+    DeviceGuard dg(g->device_id);
+    const size_t n = (size_t)n_tiles;
+    g->d_args.ensure(n);
+    g->d_start.ensure(2 * n + 2);
+    RPU_HIP_CHECK(hipHostMalloc((void **)&g->h_args, n * sizeof(MvmArgs), hipHostMallocDefault));
+    RPU_HIP_CHECK(hipHostMalloc((void **)&g->h_start, (2 * n + 2) * sizeof(int), hipHostMallocDefault));
+    RPU_HIP_CHECK(hipEventCreateWithFlags(&g->copied, hipEventDisableTiming));
+    *out = g.release();
+  });
+}
+
+int rpu_group_destroy(rpu_group_t *group) {
+  return guarded([&] { delete group; });
+}
+
+int rpu_group_forward(rpu_group_t *group, const float *const *x_dev, float *const *y_dev, int m_batch, int is_test,
+                      void *stream) {
+  (void)is_test;
+  return guarded([&] {
+    if (!group || !x_dev || !y_dev) throw RpuError("null argument");
+    if (m_batch <= 0) throw RpuError("m_batch must be positive.");
+    std::lock_guard<std::mutex> glock(group->mutex);
+    DeviceGuard dg(group->device_id);
+    hipStream_t s = (hipStream_t)stream;
+    const int n = (int)group->tiles.size();
+    // the staging buffers may still feed the copy of the previous call
+    RPU_HIP_CHECK(hipEventSynchronize(group->copied));
+
+    // per tile: arguments of a plain forward call (row-major x [m_batch][x_size], y [m_batch][d_size])
+    std::vector<MvmArgs> args(n);
+    std::vector<int> depth(n), mode(n);
+    int rounds = 1;
+    for (int i = 0; i < n; ++i) {
+      Tile &t = group->tiles[i]->t;
+      std::lock_guard<std::mutex> lock(t.mutex);
+      t.check_compute(m_batch, x_dev[i], y_dev[i]);
+      MvmArgs a = t.mvm_args(m_batch, false, nullptr, t.fio);
+      a.in = x_dev[i]; a.in_sb = t.X; a.in_sk = 1;
+      a.out = y_dev[i]; a.out_sb = t.D; a.out_so = 1;
+      mvm_round_variant(a, depth[i], mode[i]);
+      rounds = std::max(rounds, a.max_rounds);
+      args[i] = a;
+      t.last_stream = s;
+      t.last_forward_batch = m_batch;
+    }
+    // tiles that share a kernel variant sit next to each other
+    std::vector<int> order(n);
+    for (int i = 0; i < n; ++i) order[i] = i;
+    std::stable_sort(order.begin(), order.end(),
+                     [&](int a, int b) { return depth[a] * 4 + mode[a] < depth[b] * 4 + mode[b]; });
+    struct Segment { int first, count, depth, mode, start_offset, workgroups; };
+    std::vector<Segment> segments;
+    int cursor = 0; // position in h_start
+    for (int i = 0; i < n;) {
+      Segment seg{i, 0, depth[order[i]], mode[order[i]], cursor, 0};
+      int wg = 0;
+      int j = i;
+      for (; j < n && depth[order[j]] == seg.depth && mode[order[j]] == seg.mode; ++j) {
+        group->h_start[cursor++] = wg;
+        wg += mvm_round_workgroups(args[order[j]]);
+      }
+      group->h_start[cursor++] = wg;
+      seg.count = j - i;
+      seg.workgroups = wg;
+      segments.push_back(seg);
+      i = j;
+    }
+    for (int i = 0; i < n; ++i) group->h_args[i] = args[order[i]];
+    RPU_HIP_CHECK(hipMemcpyAsync(group->d_args.p, group->h_args, (size_t)n * sizeof(MvmArgs), hipMemcpyHostToDevice, s));
+    RPU_HIP_CHECK(hipMemcpyAsync(group->d_start.p, group->h_start, (size_t)cursor * sizeof(int), hipMemcpyHostToDevice, s));
+    RPU_HIP_CHECK(hipEventRecord(group->copied, s));
+
+    MvmGroup all{group->d_args.p, nullptr, n, m_batch};
+    launch_mvm_init_group(all, s);
+    for (int r = 0; r < rounds; ++r) {
+      for (const Segment &seg : segments) {
+        MvmGroup g{group->d_args.p + seg.first, group->d_start.p + seg.start_offset, seg.count, m_batch};
+        launch_mvm_round_group(g, seg.depth, seg.mode, seg.workgroups, r, s);
+      }
+    }
+    RPU_HIP_CHECK(hipGetLastError());
   });
 }
 

@@ -311,3 +311,47 @@ class CudaAnalogTile(_CudaTileMixin, _TileBase):
             self._device = torch.device("cuda", torch.cuda.current_device())
         else:
             self._init_cuda(tile)
+
+
+class TileGroup:
+    """Forward pass of several GPU tiles in a few kernel launches.
+
+    The reference runs the tiles of a tile array one after the other (TileModuleArray.forward,
+    src/aihwkit/simulator/tiles/array.py:155-182); a group gives every tile the same result as its own
+    ``forward(x, False, False, False, is_test)`` would, with one launch per kernel variant and round for all of them.
+    """
+
+    def __init__(self, tile_list):
+        self._tiles = list(tile_list)
+        if not self._tiles:
+            raise RuntimeError("empty tile list")
+        handles = (C.c_void_p * len(self._tiles))(*[t._h for t in self._tiles])
+        self._g = C.c_void_p()
+        check(lib().rpu_group_create(C.byref(self._g), handles, len(self._tiles)))
+
+    def __del__(self):
+        handle, self._g = getattr(self, "_g", None), None
+        if handle:
+            try:
+                lib().rpu_group_destroy(handle)
+            except Exception:  # pylint: disable=broad-except
+                pass
+
+    def forward(self, x_inputs, is_test: bool = False, non_blocking: bool = False):
+        """x_inputs[i]: CUDA tensor [m_batch, x_size_i]; returns the list of outputs [m_batch, d_size_i]."""
+        if len(x_inputs) != len(self._tiles):
+            raise RuntimeError("one input per tile expected")
+        xs = [_check_input(x, True, "x_input") for x in x_inputs]
+        m_batch = xs[0].shape[0]
+        for x, tile in zip(xs, self._tiles):
+            if x.dim() != 2 or x.shape[0] != m_batch or x.shape[1] != tile.get_x_size():
+                raise RuntimeError("Invalid x_input dimensions")
+        ys = [torch.empty(m_batch, tile.get_d_size(), dtype=_DTYPE, device=xs[0].device) for tile in self._tiles]
+        x_ptrs = (C.c_void_p * len(xs))(*[x.data_ptr() for x in xs])
+        y_ptrs = (C.c_void_p * len(ys))(*[y.data_ptr() for y in ys])
+        stream = torch.cuda.current_stream(xs[0].device)
+        check(lib().rpu_group_forward(self._g, x_ptrs, y_ptrs, m_batch, int(is_test), C.c_void_p(stream.cuda_stream)))
+        if not non_blocking:
+            stream.synchronize()
+        return ys
+

@@ -46,8 +46,9 @@ def main() -> int:
     ap.add_argument("--pmc", action="store_true",
                     help="counter-collection mode for rocprofv3 --pmc: one 64 MiB calibration copy, then 3 update, "
                          "3 forward and 3 backward calls; no timing, no JSON line")
-    ap.add_argument("--config", type=int, default=2, choices=(1, 2, 3),
-                    help="benchmark configuration: 2 is the graded one; 3 is the Tiki-Taka MLP of transfer tiles")
+    ap.add_argument("--config", type=int, default=2, choices=(1, 2, 3, 5),
+                    help="benchmark configuration: 2 is the graded one; 3 is the Tiki-Taka MLP of transfer tiles; "
+                         "5 is the forward pass of the GPT-2-small linear layers as PCM inference tiles")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; an analog tile is an independent unit and the path "
@@ -69,6 +70,8 @@ def main() -> int:
 
     if args.config == 3:
         return bench_config3(args)
+    if args.config == 5:
+        return bench_config5(args)
 
     if args.config == 2:
         x_size, d_size, batch = 1024, 1024, 256
@@ -306,6 +309,115 @@ def bench_config3(args) -> int:
         out["cpu_baseline"] = {"value": 1e3 / cpu_ms, "unit": "steps/s", "cores": 1, "kind": "port",
                                "sample": "2 steps of the same three tiles on the CPU transfer oracle (1 thread)",
                                "ms_per_step": cpu_ms, "host_cpus": os.cpu_count()}
+    print(json.dumps(out))
+    return 0
+
+
+# GPT-2-small linear layers split into tiles of at most 512 x 512 the way the reference's tile array does
+# (src/aihwkit/simulator/tiles/array.py:82-97): (in, out) -> input splits x output splits
+CONFIG5_LAYERS = (
+    (768, 2304, (384, 384), (461, 461, 461, 461, 460)),
+    (768, 768, (384, 384), (384, 384)),
+    (768, 3072, (384, 384), (512,) * 6),
+    (3072, 768, (512,) * 6, (384, 384)),
+)
+
+
+def bench_config5(args) -> int:
+    """Configuration 5: forward pass of the four GPT-2-small linear shapes for 1024 tokens through PCM inference
+    tiles (weights N(0, 0.02) programmed with PCM noise and drifted to one day, global drift compensation, 8-bit
+    DAC / ADC, out_noise 0.04, abs-max noise management); the partial outputs of the input splits are summed
+    digitally.  A step = the forward pass of all 38 tiles."""
+    import numpy as np
+    import torch
+
+    from aihwkit_amd.inference import InferenceTile
+    from aihwkit_amd.rpu_base import devices as dv
+    from helpers import io_params
+
+    torch.cuda.set_device(0)
+    tokens = 1024
+    rng = np.random.default_rng(0)
+    io = io_params(inp_res=1 / 254.0, out_res=1 / 254.0, out_noise=0.04, noise_management=dv.NoiseManagementType.AbsMax,
+                   bound_management=dv.BoundManagementType.Iterative)
+    layers, flops, n_tiles = [], 0.0, 0
+    for in_size, out_size, in_split, out_split in CONFIG5_LAYERS:
+        x = torch.from_numpy(rng.standard_normal((tokens, in_size)).astype(np.float32)).cuda()
+        grid, i0 = [], 0
+        for n_in in in_split:
+            row = []
+            for n_out in out_split:
+                tile = InferenceTile(n_out, n_in, forward_io=io)
+                tile.set_weights(torch.from_numpy((0.02 * rng.standard_normal((n_out, n_in))).astype(np.float32)))
+                tile.cuda()
+                tile.tile.set_seed(1000 + n_tiles)
+                tile.drift_weights(86400.0)
+                row.append(tile)
+                n_tiles += 1
+            grid.append((x[:, i0:i0 + n_in].contiguous(), row))
+            i0 += n_in
+        layers.append(grid)
+        flops += 2.0 * tokens * in_size * out_size
+
+    from aihwkit_amd.rpu_base.tiles import TileGroup
+
+    # one group per layer: all tiles of the layer in a few launches; partial outputs of the input splits are summed
+    groups = []
+    for grid in layers:
+        flat_tiles = [tile for _, row in grid for tile in row]
+        flat_x = [x_part for x_part, row in grid for _ in row]
+        groups.append((TileGroup([t.tile for t in flat_tiles]), flat_tiles, flat_x, len(grid), len(grid[0][1])))
+
+    def step():
+        outs = []
+        for group, flat_tiles, flat_x, n_in, n_out in groups:
+            ys = group.forward(flat_x, is_test=True, non_blocking=True)
+            ys = [y * t.alpha for y, t in zip(ys, flat_tiles)]            # global drift compensation per tile
+            total = None
+            for i in range(n_in):
+                y = torch.cat(ys[i * n_out:(i + 1) * n_out], dim=1)
+                total = y if total is None else total + y
+            outs.append(total)
+        return outs
+
+    def step_per_tile():
+        outs = []
+        for grid in layers:
+            total = None
+            for x_part, row in grid:
+                y = torch.cat([tile.forward(x_part, is_test=True) for tile in row], dim=1)
+                total = y if total is None else total + y
+            outs.append(total)
+        return outs
+
+    for _ in range(3):
+        step_per_tile()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(max(args.steps // 4, 3)):
+        step_per_tile()
+    torch.cuda.synchronize()
+    ms_per_tile_loop = (time.perf_counter() - t0) * 1e3 / max(args.steps // 4, 3)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    out = {
+        "metric": "noisy inference forward of the GPT-2-small linear shapes as 38 PCM tiles, tokens/s, 1 MI355X",
+        "value": tokens / (ms_per_step * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "config5: 768->2304, 768->768, 768->3072, 3072->768 split into 38 tiles of at most 512 x 512, "
+                               "1024 tokens, PCM programming noise + drift to 1 day + global drift compensation, 8-bit IO, "
+                               "out_noise 0.04, abs-max noise management", "tokens": tokens, "tiles": n_tiles},
+        "useful_tflops": flops / (ms_per_step * 1e-3) / 1e12,
+        "ms_per_step_one_call_per_tile": ms_per_tile_loop,
+    }
     print(json.dumps(out))
     return 0
 

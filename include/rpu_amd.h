@@ -337,6 +337,21 @@ int rpu_tile_set_hidden_parameters(rpu_tile_t *tile, const float *data_host);
  * Stands in for the per-context cuRAND state of the reference (C/cuda_util.cu:163-176,779-800). */
 int rpu_tile_set_seed(rpu_tile_t *tile, uint64_t seed);
 
+/* ---- several tiles in one launch ------------------------------------------------------------ */
+
+/* A layer larger than one tile is an array of tiles whose forward passes the reference runs one after the other
+ * from Python (TileModuleArray.forward, src/aihwkit/simulator/tiles/array.py:155-182).  A group runs the forward
+ * pass of all its tiles in a few launches (one per kernel variant and bound-management round) instead of
+ * several per tile.  The tiles must be resident on the same GPU; each keeps its own state, seed and call
+ * counter, and a grouped call gives every tile exactly what rpu_tile_forward with the same arguments would.
+ * x_dev[i] is [m_batch][x_size_i], y_dev[i] is [m_batch][d_size_i] (no bias column, no transposed layouts).
+ * The tiles must outlive the group. */
+typedef struct rpu_group rpu_group_t; /* opaque */
+int rpu_group_create(rpu_group_t **out, rpu_tile_t *const *tiles, int n_tiles);
+int rpu_group_forward(rpu_group_t *group, const float *const *x_dev, float *const *y_dev, int m_batch,
+                      int is_test, void *stream);
+int rpu_group_destroy(rpu_group_t *group);
+
 /* ---- inference weight pipeline ------------------------------------------------------------- */
 
 int rpu_pcm_noise_params_default(rpu_pcm_noise_params *p);

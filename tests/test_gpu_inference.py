@@ -161,3 +161,41 @@ def test_pipeline_needs_an_ideal_device_gpu_tile(gpu_device):
     assert lib().rpu_pcm_noise_params_default(C.byref(p)) == 0 and p.g_max == 25.0
     assert lib().rpu_tile_program_weights(gpu._h, C.byref(p), 1, None) != 0
     assert b"ideal device" in lib().rpu_last_error()
+
+
+def test_grouped_forward_equals_the_tiles_own_forward(gpu_device):
+    """Tiles of different shapes and kernel variants, noise on: a group call must give every tile bit for bit
+    what its own forward call gives for the same seed and call counter."""
+    import copy
+
+    from aihwkit_amd.rpu_base import tiles as tl
+    from helpers import build_pair, constant_step
+
+    rng = np.random.default_rng(6)
+    shapes = [(384, 461), (512, 384), (384, 460), (100, 70), (128, 64), (512, 512)]   # (x_size, d_size)
+    batch = 96
+    f_io = io_params(inp_res=1 / 254.0, out_res=1 / 254.0, out_noise=0.04, noise_management=dv.NoiseManagementType.AbsMax,
+                     bound_management=dv.BoundManagementType.Iterative)
+    singles, grouped, xs = [], [], []
+    for k, (x_size, d_size) in enumerate(shapes):
+        io = f_io if k != 4 else noise_free_io(is_perfect=True)       # one tile with a perfect forward pass
+        _, _, gpu = build_pair(make_meta(io, noise_free_io()), constant_step(construction_seed=k + 1), x_size, d_size)
+        scale = 0.5 if k == 1 else 0.05                                # one tile saturates: several rounds
+        gpu.set_weights(torch.from_numpy(rng.normal(0, scale, (d_size, x_size)).astype(np.float32)))
+        gpu.set_seed(40 + k)
+        singles.append(gpu)
+        grouped.append(copy.deepcopy(gpu))
+        grouped[-1].set_seed(40 + k)
+        xs.append(torch.from_numpy(rng.normal(0, 1, (batch, x_size)).astype(np.float32)).cuda())
+    group = tl.TileGroup(grouped)
+    for _ in range(3):                                                 # the call counters advance together
+        want = [t.forward(x, False, False, False, False, False) for t, x in zip(singles, xs)]
+        got = group.forward(xs)
+        for k, (a, b) in enumerate(zip(got, want)):
+            assert torch.equal(a, b), k
+    assert singles[1].get_bm_rounds(batch).max() > 1
+    assert torch.equal(grouped[1].get_bm_rounds(batch), singles[1].get_bm_rounds(batch))
+    with pytest.raises(RuntimeError):
+        tl.TileGroup([grouped[0], grouped[0]])
+    with pytest.raises(RuntimeError):
+        group.forward(xs[:-1])
