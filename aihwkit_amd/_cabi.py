@@ -104,6 +104,11 @@ SYMBOLS = {
     "rpu_tile_create_transfer": (C.c_int, [C.POINTER(_P), C.c_int, C.c_int, C.POINTER(TileConfig),
                                            C.POINTER(TransferParams)]),
     "rpu_tile_get_transfer_state": (C.c_int, [_P, C.POINTER(C.c_uint64), C.POINTER(C.c_int32)]),
+    "rpu_tile_set_matrix_indices": (C.c_int, [_P, _P, C.c_int, C.c_int]),
+    "rpu_tile_has_matrix_indices": (C.c_int, [_P]),
+    "rpu_tile_forward_indexed": (C.c_int, [_P, _P, _P, C.c_int, C.c_long, C.c_int, _P]),
+    "rpu_tile_backward_indexed": (C.c_int, [_P, _P, _P, C.c_int, C.c_long, _P]),
+    "rpu_tile_update_indexed": (C.c_int, [_P, _P, _P, C.c_int, C.c_long, _P]),
     "rpu_group_create": (C.c_int, [C.POINTER(_P), C.POINTER(_P), C.c_int]),
     "rpu_group_forward": (C.c_int, [_P, C.POINTER(_P), C.POINTER(_P), C.c_int, C.c_int, _P]),
     "rpu_group_destroy": (C.c_int, [_P]),

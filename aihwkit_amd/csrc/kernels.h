@@ -154,6 +154,20 @@ void launch_pcm_drift(const float *w_prog, const float *nu_plus, const float *nu
 // out[0] = mean |v| over n values, one workgroup, fixed summation order
 void launch_mean_abs(const float *v, size_t n, float *out, hipStream_t s);
 
+// ---- indexed (convolution) interface: RPUSimple::copyIndexedInput / copyIndexedOutput / permute132 with
+// trans = true (rpu.cpp:1017-1115, math_util.cpp:319-346).  indices is [x_size][patches]: 0 = padding zero,
+// 1 = bias one, j >= 2 = element j - 2 of the image; images are `image_size` apart.
+// x_mat[(n * patches + p) * x_size + k] = value of patch p of image n
+void launch_gather_indexed(float *x_mat, const float *images, const int *indices, int x_size, int patches, int n_images,
+                           long image_size, hipStream_t s);
+// images[(j - 2) + n * image_size] += x_mat[...] (images must be zeroed before)
+void launch_scatter_indexed(float *images, const float *x_mat, const int *indices, int x_size, int patches, int n_images,
+                            long image_size, hipStream_t s);
+// [n][d][p] <-> [(n, p)][d]
+void launch_ndp_to_bd(float *bd, const float *ndp, int n_images, int d_size, int patches, hipStream_t s);
+void launch_bd_to_ndp(float *ndp, const float *bd, int n_images, int d_size, int patches, hipStream_t s);
+void launch_fill(float *p, float value, size_t n, hipStream_t s);
+
 // n_vec unit vectors of length `size`: row v is e_((start + v) % size)
 void launch_unit_vectors(float *out, int n_vec, int size, int start, hipStream_t s);
 

@@ -3,6 +3,7 @@
 // of its bindings: src/aihwkit/inference/noise/pcm.py:100-158 over
 // src/aihwkit/inference/converter/conductance.py:51-82).  Element-wise kernels, one read and one write of each
 // array: HBM-bound.  Every normal is a Philox draw keyed by (element, call), so a seed reproduces a run.
+// The file also holds the gather / scatter / permute kernels of the indexed (convolution) interface.
 #include "kernels.h"
 
 namespace rpu_amd {
@@ -114,6 +115,58 @@ __global__ __launch_bounds__(1024) void k_mean_abs(const float *v, size_t n, flo
   }
 }
 
+__global__ __launch_bounds__(256) void k_gather_indexed(float *x_mat, const float *images, const int *indices, int x_size,
+                                                         int patches, int n_images, long image_size) {
+  const size_t total = (size_t)n_images * patches * x_size;
+  for (size_t idx = blockIdx.x * (size_t)blockDim.x + threadIdx.x; idx < total; idx += (size_t)gridDim.x * blockDim.x) {
+    const int k = (int)(idx % x_size);
+    const size_t b = idx / x_size;
+    const int p = (int)(b % patches);
+    const size_t n = b / patches;
+    const int j = indices[(size_t)k * patches + p];
+    x_mat[idx] = (j <= 1) ? (float)j : images[(size_t)(j - 2) + n * image_size];
+  }
+}
+
+__global__ __launch_bounds__(256) void k_scatter_indexed(float *images, const float *x_mat, const int *indices, int x_size,
+                                                          int patches, int n_images, long image_size) {
+  const size_t total = (size_t)n_images * patches * x_size;
+  for (size_t idx = blockIdx.x * (size_t)blockDim.x + threadIdx.x; idx < total; idx += (size_t)gridDim.x * blockDim.x) {
+    const int k = (int)(idx % x_size);
+    const size_t b = idx / x_size;
+    const int p = (int)(b % patches);
+    const size_t n = b / patches;
+    const int j = indices[(size_t)k * patches + p];
+    if (j > 1) atomicAdd(&images[(size_t)(j - 2) + n * image_size], x_mat[idx]);
+  }
+}
+
+// ndp index (n, d, p) <-> bd index ((n, p), d)
+__global__ __launch_bounds__(256) void k_ndp_bd(float *dst, const float *src, int n_images, int d_size, int patches,
+                                                 int to_bd) {
+  const size_t total = (size_t)n_images * d_size * patches;
+  for (size_t idx = blockIdx.x * (size_t)blockDim.x + threadIdx.x; idx < total; idx += (size_t)gridDim.x * blockDim.x) {
+    // idx walks the destination with unit stride
+    if (to_bd) {
+      const int d = (int)(idx % d_size);
+      const size_t b = idx / d_size;
+      const int p = (int)(b % patches);
+      const size_t n = b / patches;
+      dst[idx] = src[(n * d_size + d) * patches + p];
+    } else {
+      const int p = (int)(idx % patches);
+      const size_t nd = idx / patches;
+      const int d = (int)(nd % d_size);
+      const size_t n = nd / d_size;
+      dst[idx] = src[(n * patches + p) * d_size + d];
+    }
+  }
+}
+
+__global__ void k_fill(float *p, float value, size_t n) {
+  for (size_t idx = blockIdx.x * (size_t)blockDim.x + threadIdx.x; idx < n; idx += (size_t)gridDim.x * blockDim.x) p[idx] = value;
+}
+
 int grid_of(size_t n) {
   size_t blocks = (n + 255) / 256;
   if (blocks > 4096) blocks = 4096;
@@ -138,6 +191,34 @@ void launch_pcm_drift(const float *w_prog, const float *nu_plus, const float *nu
                       const uint32_t *abs_max_bits, const PcmDev &p, PhiloxKey key, uint32_t call, hipStream_t s) {
   hipLaunchKernelGGL(k_pcm_drift, dim3(grid_of(n)), dim3(256), 0, s, w_prog, nu_plus, nu_minus, w_out, n, abs_max_bits, p,
                      key, call);
+}
+
+void launch_gather_indexed(float *x_mat, const float *images, const int *indices, int x_size, int patches, int n_images,
+                           long image_size, hipStream_t s) {
+  const size_t total = (size_t)n_images * patches * x_size;
+  hipLaunchKernelGGL(k_gather_indexed, dim3(grid_of(total)), dim3(256), 0, s, x_mat, images, indices, x_size, patches,
+                     n_images, image_size);
+}
+
+void launch_scatter_indexed(float *images, const float *x_mat, const int *indices, int x_size, int patches, int n_images,
+                            long image_size, hipStream_t s) {
+  const size_t total = (size_t)n_images * patches * x_size;
+  hipLaunchKernelGGL(k_scatter_indexed, dim3(grid_of(total)), dim3(256), 0, s, images, x_mat, indices, x_size, patches,
+                     n_images, image_size);
+}
+
+void launch_ndp_to_bd(float *bd, const float *ndp, int n_images, int d_size, int patches, hipStream_t s) {
+  const size_t total = (size_t)n_images * d_size * patches;
+  hipLaunchKernelGGL(k_ndp_bd, dim3(grid_of(total)), dim3(256), 0, s, bd, ndp, n_images, d_size, patches, 1);
+}
+
+void launch_bd_to_ndp(float *ndp, const float *bd, int n_images, int d_size, int patches, hipStream_t s) {
+  const size_t total = (size_t)n_images * d_size * patches;
+  hipLaunchKernelGGL(k_ndp_bd, dim3(grid_of(total)), dim3(256), 0, s, ndp, bd, n_images, d_size, patches, 0);
+}
+
+void launch_fill(float *p, float value, size_t n, hipStream_t s) {
+  hipLaunchKernelGGL(k_fill, dim3(grid_of(n)), dim3(256), 0, s, p, value, n);
 }
 
 void launch_mean_abs(const float *v, size_t n, float *out, hipStream_t s) {

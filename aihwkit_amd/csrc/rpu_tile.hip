@@ -156,6 +156,11 @@ struct Tile {
   DevBuf<float> i_ref, i_prog, i_nu_plus, i_nu_minus, i_scalar;
   DevBuf<uint32_t> i_absmax;
   bool has_reference = false, programmed = false;
+  // indexed (convolution) interface: index matrix [X][patches] and the unfolded matrices
+  std::vector<int32_t> idx_host;
+  int idx_patches = 0;
+  DevBuf<int> x_idx;
+  DevBuf<float> x_mat, d_mat;
   int last_update_batch = 0;
   int last_update_pulse = -1;
   int last_forward_batch = 0;
@@ -214,6 +219,7 @@ struct Tile {
     t_unit.release(); t_read.release();
     i_ref.release(); i_prog.release(); i_nu_plus.release(); i_nu_minus.release(); i_scalar.release(); i_absmax.release();
     has_reference = programmed = false;
+    x_idx.release(); x_mat.release(); d_mat.release();
     for (auto &sl : slots) sl->release();
   }
 
@@ -524,6 +530,48 @@ struct Tile {
     last_update_pulse = up.p.pulse_type;
   }
 
+  // ---- indexed (convolution) interface ---------------------------------------------------------------
+
+  void ensure_indexed(int n_images) {
+    if (idx_patches <= 0) throw RpuError("The index matrix has not been set (set_matrix_indices).");
+    if (n_images <= 0) throw RpuError("n_images must be positive.");
+    if (!x_idx.p) {
+      x_idx.ensure(idx_host.size());
+      RPU_HIP_CHECK(hipMemcpy(x_idx.p, idx_host.data(), idx_host.size() * sizeof(int32_t), hipMemcpyHostToDevice));
+    }
+    const size_t B = (size_t)n_images * idx_patches;
+    x_mat.ensure(B * X);
+    d_mat.ensure(B * D);
+  }
+
+  void forward_indexed(const float *x, float *d, int n_images, long image_size, hipStream_t s) {
+    ensure_indexed(n_images);
+    const int B = n_images * idx_patches;
+    launch_gather_indexed(x_mat.p, x, x_idx.p, X, idx_patches, n_images, image_size, s);
+    mvm(x_mat.p, d_mat.p, B, false, false, false, false, s);
+    launch_bd_to_ndp(d, d_mat.p, n_images, D, idx_patches, s);
+    RPU_HIP_CHECK(hipGetLastError());
+  }
+
+  void backward_indexed(const float *d, float *x, int n_images, long image_size, hipStream_t s) {
+    ensure_indexed(n_images);
+    const int B = n_images * idx_patches;
+    launch_ndp_to_bd(d_mat.p, d, n_images, D, idx_patches, s);
+    mvm(d_mat.p, x_mat.p, B, false, false, false, true, s);
+    launch_fill(x, 0.0f, (size_t)n_images * image_size, s);
+    launch_scatter_indexed(x, x_mat.p, x_idx.p, X, idx_patches, n_images, image_size, s);
+    RPU_HIP_CHECK(hipGetLastError());
+  }
+
+  void update_indexed(const float *x, const float *d, int n_images, long image_size, hipStream_t s) {
+    ensure_indexed(n_images);
+    const int B = n_images * idx_patches;
+    launch_gather_indexed(x_mat.p, x, x_idx.p, X, idx_patches, n_images, image_size, s);
+    launch_ndp_to_bd(d_mat.p, d, n_images, D, idx_patches, s);
+    update(x_mat.p, d_mat.p, B, false, false, false, s);
+    RPU_HIP_CHECK(hipGetLastError());
+  }
+
   // ---- inference weight pipeline ------------------------------------------------------------------
 
   static PcmDev pcm_dev(const rpu_pcm_noise_params &q, float t_inference) {
@@ -807,6 +855,59 @@ int rpu_tile_create_transfer(rpu_tile_t **out, int x_size, int d_size, const rpu
   });
 }
 
+int rpu_tile_set_matrix_indices(rpu_tile_t *tile, const int32_t *indices_host, int x_size, int patches) {
+  return guarded([&] {
+    if (!tile || !indices_host) throw RpuError("null argument");
+    Tile &t = tile->t;
+    std::lock_guard<std::mutex> lock(t.mutex);
+    if (x_size != t.X) throw RpuError("The index matrix must have x_size rows.");
+    if (patches <= 0) throw RpuError("patches must be positive.");
+    if (t.resident()) {
+      DeviceGuard g(t.device_id);
+      t.sync_last();
+      t.x_idx.release();
+    }
+    t.idx_host.assign(indices_host, indices_host + (size_t)x_size * patches);
+    for (int32_t j : t.idx_host) {
+      if (j < 0) throw RpuError("Negative entry in the index matrix.");
+    }
+    t.idx_patches = patches;
+  });
+}
+
+int rpu_tile_has_matrix_indices(const rpu_tile_t *tile) { return tile ? tile->t.idx_patches : 0; }
+
+#define RPU_INDEXED_ENTRY(NAME, CALL)                                                          \
+  return guarded([&] {                                                                         \
+    if (!tile) throw RpuError("null tile");                                                    \
+    Tile &t = tile->t;                                                                         \
+    std::lock_guard<std::mutex> lock(t.mutex);                                                 \
+    t.check_compute(n_images, x_dev, d_dev);                                                   \
+    if (image_size <= 0) throw RpuError("image_size must be positive.");                       \
+    for (int32_t j : t.idx_host) {                                                             \
+      if ((long)j - 2 >= image_size) throw RpuError("Index matrix entry beyond the image size."); \
+    }                                                                                          \
+    DeviceGuard g(t.device_id);                                                                \
+    CALL;                                                                                      \
+  })
+
+int rpu_tile_forward_indexed(rpu_tile_t *tile, const float *x_dev, float *d_dev, int n_images, long image_size,
+                             int is_test, void *stream) {
+  (void)is_test;
+  RPU_INDEXED_ENTRY(forward, t.forward_indexed(x_dev, d_dev, n_images, image_size, (hipStream_t)stream));
+}
+
+int rpu_tile_backward_indexed(rpu_tile_t *tile, const float *d_dev, float *x_dev, int n_images, long image_size,
+                              void *stream) {
+  RPU_INDEXED_ENTRY(backward, t.backward_indexed(d_dev, x_dev, n_images, image_size, (hipStream_t)stream));
+}
+
+int rpu_tile_update_indexed(rpu_tile_t *tile, const float *x_dev, const float *d_dev, int n_images, long image_size,
+                            void *stream) {
+  RPU_INDEXED_ENTRY(update, t.update_indexed(x_dev, d_dev, n_images, image_size, (hipStream_t)stream));
+}
+#undef RPU_INDEXED_ENTRY
+
 // ---- grouped forward over several tiles ------------------------------------------------------------
 
 struct rpu_group {
@@ -1019,6 +1120,8 @@ int rpu_tile_clone(rpu_tile_t **out, const rpu_tile_t *src_c) {
     t.X = s.X; t.D = s.D; t.fio = s.fio; t.bio = s.bio; t.up = s.up; t.dev = s.dev; t.arr = s.arr;
     t.lr = s.lr; t.seed = s.seed; t.call = s.call;
     t.w_host = s.w_host;
+    t.idx_host = s.idx_host;
+    t.idx_patches = s.idx_patches;
     if (s.is_transfer()) {
       t.tr = std::make_unique<TransferPar>(*s.tr);
       t.update_idx = s.update_idx;

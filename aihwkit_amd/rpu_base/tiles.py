@@ -104,6 +104,21 @@ class _TileBase:
                 f"Invalid weights dimensions: expected [{self.get_d_size()},{self.get_x_size()}] array")
         check(lib().rpu_tile_set_weights(self._h, weights.data_ptr()))
 
+    # -- index matrix of the *_indexed methods (rpu_base_tiles.cpp:721-760)
+    def set_matrix_indices(self, indices: torch.Tensor) -> None:
+        """int32 tensor with x_size * patches entries, patch index fastest (what the conv layers produce)."""
+        if indices.dtype != torch.int32:
+            raise RuntimeError("indices must be an int32 tensor")
+        indices = indices.detach().cpu().contiguous()
+        x_size = self.get_x_size()
+        if indices.numel() == 0 or indices.numel() % x_size != 0:
+            raise RuntimeError("The number of indices must be a multiple of x_size")
+        patches = indices.numel() // x_size
+        check(lib().rpu_tile_set_matrix_indices(self._h, indices.data_ptr(), x_size, patches))
+
+    def has_matrix_indices(self) -> bool:
+        return lib().rpu_tile_has_matrix_indices(self._h) > 0
+
     # -- hidden per-device parameters (rpu_base_tiles.cpp:763-825)
     def get_hidden_parameter_names(self) -> List[str]:
         count = lib().rpu_tile_hidden_parameter_count(self._h)
@@ -247,6 +262,52 @@ class _CudaTileMixin:
         self._finish(x_input, non_blocking)
 
     # -- inspection hooks
+    # -- indexed (convolution) interface (rpu_base_tiles.cpp:621-737)
+    def _patches(self) -> int:
+        patches = lib().rpu_tile_has_matrix_indices(self._h)
+        if patches <= 0:
+            raise RuntimeError("The index matrix has not been set (set_matrix_indices).")
+        return patches
+
+    def forward_indexed(self, x_input: torch.Tensor, d_tensor: torch.Tensor, is_test: bool = False,
+                        non_blocking: bool = False) -> torch.Tensor:
+        """x_input: N, C, (D), H, W images; d_tensor: the output tensor N, C_out, (d_depth,) d_height, d_width."""
+        x_input = _check_input(x_input, True, "x_input")
+        d_tensor = _check_input(d_tensor, True, "d_tensor")
+        n_images = x_input.size(0)
+        patches = d_tensor.numel() // d_tensor.size(0) // d_tensor.size(1)
+        if patches != self._patches() or d_tensor.size(1) != self.get_d_size() or d_tensor.size(0) != n_images:
+            raise RuntimeError("Invalid d_tensor dimensions for the index matrix that is set")
+        check(lib().rpu_tile_forward_indexed(self._h, x_input.data_ptr(), d_tensor.data_ptr(), n_images,
+                                             x_input.numel() // n_images, int(is_test), self._stream_for(x_input)))
+        self._finish(x_input, non_blocking)
+        return d_tensor
+
+    def backward_indexed(self, d_input: torch.Tensor, x_tensor: torch.Tensor, non_blocking: bool = False) -> torch.Tensor:
+        d_input = _check_input(d_input, True, "d_input")
+        x_tensor = _check_input(x_tensor, True, "x_tensor")
+        n_images = d_input.size(0)
+        patches = d_input.numel() // d_input.size(0) // d_input.size(1)
+        if patches != self._patches() or d_input.size(1) != self.get_d_size() or x_tensor.size(0) != n_images:
+            raise RuntimeError("Invalid d_input dimensions for the index matrix that is set")
+        check(lib().rpu_tile_backward_indexed(self._h, d_input.data_ptr(), x_tensor.data_ptr(), n_images,
+                                              x_tensor.numel() // n_images, self._stream_for(d_input)))
+        self._finish(d_input, non_blocking)
+        return x_tensor
+
+    def update_indexed(self, x_input: torch.Tensor, d_input: torch.Tensor, non_blocking: bool = False) -> None:
+        if self.get_learning_rate() == 0.0:
+            return
+        x_input = _check_input(x_input, True, "x_input")
+        d_input = _check_input(d_input, True, "d_input")
+        n_images = d_input.size(0)
+        patches = d_input.numel() // d_input.size(0) // d_input.size(1)
+        if patches != self._patches() or d_input.size(1) != self.get_d_size() or x_input.size(0) != n_images:
+            raise RuntimeError("Invalid x_input or d_input dimensions for the index matrix that is set")
+        check(lib().rpu_tile_update_indexed(self._h, x_input.data_ptr(), d_input.data_ptr(), n_images,
+                                            x_input.numel() // n_images, self._stream_for(x_input)))
+        self._finish(x_input, non_blocking)
+
     def get_update_words(self, m_batch: int):
         """Packed pulse words and per-sample BL of the last stochastic update (CPU tensors)."""
         x_words = torch.empty(m_batch, self.get_x_size(), dtype=torch.int32)

@@ -337,6 +337,27 @@ int rpu_tile_set_hidden_parameters(rpu_tile_t *tile, const float *data_host);
  * Stands in for the per-context cuRAND state of the reference (C/cuda_util.cu:163-176,779-800). */
 int rpu_tile_set_seed(rpu_tile_t *tile, uint64_t seed);
 
+/* ---- indexed (convolution) interface ----------------------------------------------------------- */
+
+/* Replaces RPUSimple::setMatrixIndices (R/rpu.h:397-402) as bound at B/rpu_base_tiles.cpp:721-737: the index
+ * matrix of an unfolded convolution, [x_size][patches] int32 on the host: 0 = zero padding, 1 = bias one,
+ * j >= 2 = element j - 2 of one input image (src/aihwkit/nn/modules/conv.py:534-575). */
+int rpu_tile_set_matrix_indices(rpu_tile_t *tile, const int32_t *indices_host, int x_size, int patches);
+int rpu_tile_has_matrix_indices(const rpu_tile_t *tile); /* patches per image of the index matrix, 0 if none is set */
+
+/* Replace RPUSimple::forwardIndexed / backwardIndexed / updateIndexed (R/rpu.cpp:1117-1239) as bound at
+ * B/rpu_base_tiles.cpp:621-720 (always with trans = true, dim3 = images, m_batch = patches per image):
+ * x_dev holds n_images input images of image_size floats (N, C, H, W), d_dev is [n_images][d_size][patches]
+ * (N, C_out, H_out * W_out).  Forward gathers the patches through the index matrix and runs the tile's forward
+ * pass over n_images * patches samples; backward runs the tile's backward pass and adds the patch gradients
+ * into the (zeroed) images; update gathers the patches and runs the tile's update. */
+int rpu_tile_forward_indexed(rpu_tile_t *tile, const float *x_dev, float *d_dev, int n_images, long image_size,
+                             int is_test, void *stream);
+int rpu_tile_backward_indexed(rpu_tile_t *tile, const float *d_dev, float *x_dev, int n_images, long image_size,
+                              void *stream);
+int rpu_tile_update_indexed(rpu_tile_t *tile, const float *x_dev, const float *d_dev, int n_images, long image_size,
+                            void *stream);
+
 /* ---- several tiles in one launch ------------------------------------------------------------ */
 
 /* A layer larger than one tile is an array of tiles whose forward passes the reference runs one after the other

@@ -1,0 +1,91 @@
+"""GPU parity of the indexed (convolution) interface against the indexed oracle, and against torch's convolution
+for a perfect tile."""
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from aihwkit_amd.rpu_base import devices as dv
+from aihwkit_amd.rpu_base import tiles
+from helpers import build_pair, constant_step, make_meta, noise_free_io
+from indexed_oracle import IndexedOracle
+from test_oracle_indexed_pins import conv_indices
+
+pytestmark = pytest.mark.gpu
+
+
+def cuda(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def test_perfect_tile_is_a_convolution(gpu_device):
+    rng = np.random.default_rng(0)
+    c_in, c_out, height, width, n, kernel = 16, 32, 12, 12, 8, (5, 5)      # the second LeNet convolution
+    indices, patches = conv_indices((c_in, height, width), kernel, (1, 1), (0, 0), (1, 1), True)
+    x_size = c_in * 25 + 1
+    meta = dv.FloatingPointTileParameter()
+    host = meta.create_array(x_size, c_out)
+    w = rng.normal(0, 0.1, (c_out, x_size)).astype(np.float32)
+    host.set_weights(torch.from_numpy(w))
+    gpu = tiles.CudaFloatingPointTile(host)
+    assert not gpu.has_matrix_indices()
+    with pytest.raises(RuntimeError):
+        gpu.forward_indexed(torch.zeros(n, c_in, height, width).cuda(), torch.zeros(n, c_out, 8, 8).cuda())
+    gpu.set_matrix_indices(indices)
+    assert gpu.has_matrix_indices()
+    x = rng.normal(0, 1, (n, c_in, height, width)).astype(np.float32)
+    y = gpu.forward_indexed(cuda(x), torch.empty(n, c_out, 8, 8).cuda()).cpu()
+    weight = torch.from_numpy(w[:, :-1].reshape(c_out, c_in, 5, 5).copy())
+    want = F.conv2d(torch.from_numpy(x), weight, torch.from_numpy(w[:, -1].copy()))
+    assert torch.allclose(y, want, atol=1e-4)
+    grad = rng.normal(0, 1, (n, c_out, 8, 8)).astype(np.float32)
+    dx = gpu.backward_indexed(cuda(grad), torch.empty(n, c_in, height, width).cuda()).cpu()
+    want_dx = F.conv_transpose2d(torch.from_numpy(grad), weight)
+    assert torch.allclose(dx, want_dx, atol=1e-4)
+    gpu.set_learning_rate(0.01)
+    gpu.update_indexed(cuda(x), cuda(grad))
+    xt = torch.from_numpy(x).requires_grad_(False)
+    wg = weight.clone().requires_grad_(True)
+    bg = torch.from_numpy(w[:, -1].copy()).requires_grad_(True)
+    (F.conv2d(xt, wg, bg) * torch.from_numpy(grad)).sum().backward()
+    want_w = w.copy()
+    want_w[:, :-1] -= 0.01 * wg.grad.numpy().reshape(c_out, -1)
+    want_w[:, -1] -= 0.01 * bg.grad.numpy()
+    assert np.abs(gpu.get_weights().numpy() - want_w).max() <= 2e-4
+
+
+@pytest.mark.parametrize("kernel,stride,padding", [((3, 3), (1, 1), (1, 1)), ((5, 5), (2, 2), (0, 0))])
+def test_analog_tile_matches_the_indexed_oracle(gpu_device, kernel, stride, padding):
+    rng = np.random.default_rng(1)
+    c_in, c_out, height, width, n = 3, 20, 11, 10, 5
+    indices, patches = conv_indices((c_in, height, width), kernel, stride, padding, (1, 1), True)
+    x_size = c_in * kernel[0] * kernel[1] + 1
+    f_io = noise_free_io(noise_management=dv.NoiseManagementType.AbsMax, bound_management=dv.BoundManagementType.Iterative)
+    b_io = noise_free_io(noise_management=dv.NoiseManagementType.AbsMax)
+    meta = make_meta(f_io, b_io, pulse_type=dv.PulseType.DeterministicImplicit, desired_bl=31)
+    dev = constant_step(dw_min=0.002, dw_min_std=0.0, construction_seed=4)
+    host, orc_tile, gpu = build_pair(meta, dev, x_size, c_out)
+    w = rng.normal(0, 0.2, (c_out, x_size)).astype(np.float32)
+    gpu.set_weights(torch.from_numpy(w))
+    orc_tile.set_weights(w)
+    gpu.set_matrix_indices(indices)
+    twin = tiles.CudaAnalogTile(host)                       # a copy made before the indices were set has none
+    assert not twin.has_matrix_indices()
+    orc = IndexedOracle(orc_tile, indices.numpy(), patches)
+    x = rng.normal(0, 1, (n, c_in, height, width)).astype(np.float32)
+    out_hw = (int(np.sqrt(patches)), patches // int(np.sqrt(patches))) if int(np.sqrt(patches)) ** 2 == patches else (1, patches)
+    y = gpu.forward_indexed(cuda(x), torch.empty(n, c_out, *out_hw).cuda()).cpu().numpy().reshape(n, c_out, patches)
+    want = orc.forward(x)
+    off = np.abs(y - want) > 1e-5
+    assert off.mean() < 0.005 and np.abs(y - want).max() < 0.2      # an ADC code may flip at a rounding edge
+    grad = (0.3 * rng.normal(0, 1, (n, c_out, patches))).astype(np.float32)
+    dx = gpu.backward_indexed(cuda(grad.reshape(n, c_out, *out_hw)), torch.empty(n, c_in, height, width).cuda())
+    want_dx = orc.backward(grad, c_in * height * width)
+    diff = np.abs(dx.cpu().numpy().reshape(n, -1) - want_dx)
+    assert (diff > 1e-4).mean() < 0.01 and diff.max() < 0.5
+    gpu.set_learning_rate(0.05)
+    orc_tile.set_learning_rate(0.05)
+    gpu.update_indexed(cuda(x), cuda(grad.reshape(n, c_out, *out_hw)))
+    orc.update(x, grad)
+    assert np.abs(gpu.get_weights().numpy() - orc_tile.get_weights()).max() <= 1e-5
+    assert np.abs(orc_tile.get_weights() - np.clip(w, orc_tile.get_hidden()[1], orc_tile.get_hidden()[0])).max() > 1e-3
