@@ -48,6 +48,8 @@ struct MvmArgs {
   int transposed; // 0: out[o] = sum_k W[o][k] in[k] (forward); 1: out[o] = sum_k W[k][o] in[k] (backward)
   int round;      // bound-management round, 0-based
   int max_rounds; // rounds launched for this call (mvm_max_rounds)
+  int speculate;  // 1: each round also quantizes every row for the round after it (short path between rounds, for
+                  // small batches); 0: only the rows of samples that saturated are quantized, once that is known
   float alpha, beta; // only used when io.perfect: out = alpha * acc + beta * out
   IoDev io;
   MvmState st;

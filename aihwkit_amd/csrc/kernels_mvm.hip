@@ -27,6 +27,7 @@ namespace rpu_amd {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4_unaligned __attribute__((ext_vector_type(4), aligned(4))); // a 16-byte load from any float address
 
 namespace {
 
@@ -59,11 +60,13 @@ __device__ __forceinline__ float dac_value(float x, float scale, const IoDev &io
   return v;
 }
 
-// quantized copy of sample b's input row into row `slot` of a scratch matrix (whole workgroup)
-__device__ __forceinline__ void write_dac_row(const MvmArgs &a, int b, int slot, float scale, int round, float *dst) {
+// quantized copy of sample b's input row into row `slot` of a scratch matrix, by `width` threads of which
+// this one is number t
+__device__ __forceinline__ void write_dac_row(const MvmArgs &a, int b, int slot, float scale, int round, float *dst,
+                                              int t, int width) {
   const float *row = a.in + (long)b * a.in_sb;
   float *out = dst + (long)slot * a.k_pad;
-  for (int k = threadIdx.x; k < a.k_pad; k += blockDim.x) {
+  for (int k = t; k < a.k_pad; k += width) {
     float v = 0.0f;
     if (k < a.K) {
       v = row[(long)k * a.in_sk];
@@ -75,16 +78,30 @@ __device__ __forceinline__ void write_dac_row(const MvmArgs &a, int b, int slot,
 
 constexpr int LDS_ROW = KSTEP + 4; // floats per staged row: 16-byte aligned, conflict-free 128-bit reads
 
-// tile number n -> (output tile, sample tile): workgroup n runs on XCD n % 8 and XCD x owns the
-// output-row tiles [x * per, (x + 1) * per)
+// workgroup number n -> (output tile, sample tile).  With 8 or more output tiles workgroup n runs on XCD n % 8 and
+// XCD x owns the output-row tiles [x * per, (x + 1) * per): each L2 holds a band of W.  A matrix of fewer output
+// tiles fits every L2, and consecutive workgroups (hence all XCDs) simply walk the tiles in order.
 __device__ __forceinline__ bool tile_of(const MvmArgs &a, int n, int n_act, int &tile_o, int &tile_b) {
   const int tiles_o = (a.O + TILE - 1) / TILE;
+  if (tiles_o < 8) {
+    tile_o = n % tiles_o;
+    tile_b = n / tiles_o;
+    return tile_b * TILE < n_act;
+  }
   const int per = (tiles_o + 7) / 8;
   const int xcd = n & 7;
   const int m = n >> 3;
   tile_o = xcd * per + (m % per);
   tile_b = m / per;
   return tile_o < tiles_o && tile_b * TILE < n_act;
+}
+
+// workgroups that cover n_act samples (a multiple of 8)
+__host__ __device__ __forceinline__ int workgroups_for(int O, int n_act) {
+  const int tiles_o = (O + TILE - 1) / TILE;
+  const int tiles_b = (n_act + TILE - 1) / TILE;
+  if (tiles_o < 8) return (tiles_o * tiles_b + 7) & ~7;
+  return 8 * ((tiles_o + 7) / 8) * tiles_b;
 }
 
 // ADC stage for outputs o0 .. o0 + 3 of sample b: v holds the analog sums (rpu_forward_backward_pass.cpp:666-719)
@@ -162,7 +179,7 @@ __device__ __forceinline__ void mvm_step_schedule() {
 #define RPU_SG_VMEM 0x020
 #define RPU_SG_DSR 0x100
 #define RPU_SG_DSW 0x200
-  if (WMODE == 0) { // per step: 8 LDS writes, 8 global loads, 8 LDS reads
+  if (WMODE != 1) { // per step: 8 LDS writes, 8 global loads, 8 LDS reads
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       RPU_SG(RPU_SG_MFMA, 1);
@@ -203,8 +220,9 @@ __device__ __forceinline__ void mvm_step_schedule() {
 // WMODE = how the weight operand is addressed:
 //   0  contraction index contiguous (forward), rows 16-byte aligned, K a multiple of 16
 //   1  output index contiguous (backward: W is read transposed in place)
-//   2  any strides, every element guarded
-// Operand tiles with a contiguous contraction index (the quantized inputs always, the weights in mode 0) are
+//   2  contraction index contiguous, any row length and alignment (a tile with a bias column has an odd row
+//      length): 16-byte loads from 4-byte aligned addresses, the last 1 .. 3 elements of a row one by one
+// Operand tiles with a contiguous contraction index (the quantized inputs always, the weights in modes 0, 2) are
 // fetched with unit-stride 16-byte loads, 8 lanes per 128-byte row segment, staged in a wave-private LDS
 // tile and read back in the MFMA operand layout (lane (r, h) holds row r, k = 16 h .. 16 h + 15).  Reading
 // them straight into that layout would make every lane of a load touch a different cache line, which is
@@ -212,7 +230,7 @@ __device__ __forceinline__ void mvm_step_schedule() {
 // and k are one line.  Out-of-range rows / k are clamped to valid addresses: their products meet the zero
 // padding of the quantized inputs or are never stored.
 // PD = 2, 4: software pipeline with the global loads of PD steps in flight, k_pad a multiple of
-// PD * KSTEP * WAVES; PD = 1: one register set, for short contractions.
+// PD * KSTEP * WAVES; PD = 1: one register set, for short contractions, k_pad a multiple of KSTEP.
 template <int PD, int WMODE>
 __device__ __forceinline__ void mvm_round_tile(const MvmArgs &a, int round, int tile_o, int tile_b, int n_act,
                                                float (*red)[16][64], float *stage) {
@@ -230,9 +248,12 @@ __device__ __forceinline__ void mvm_round_tile(const MvmArgs &a, int round, int 
   const long w_so = a.transposed ? 1 : a.x_size;
   const long w_sk = a.transposed ? a.x_size : 1;
   const int K = a.K;
-  const int per_wave = a.k_pad / (KSTEP * WAVES); // a multiple of PD
-  const int s_begin = wave * per_wave;
-  const int s_end = s_begin + per_wave;
+  // steps of 32 k-values, dealt to the waves in contiguous parts (equal parts, a multiple of PD, when PD >= 2;
+  // a short contraction may leave the last waves without a step)
+  const int steps = a.k_pad / KSTEP;
+  const int per_wave = (steps + WAVES - 1) / WAVES;
+  const int s_begin = min(wave * per_wave, steps);
+  const int s_end = min(s_begin + per_wave, steps);
 
   float *stage_x = stage + wave * (2 * TILE * LDS_ROW);
   float *stage_w = stage_x + TILE * LDS_ROW;
@@ -281,10 +302,20 @@ __device__ __forceinline__ void mvm_round_tile(const MvmArgs &a, int round, int 
         wd[i] = w_col[(long)kc * w_sk];
       }
     } else {
+      const int kc = k0 + st_chunk;
+      if (kc + 4 <= K) {
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const int k = k0 + h * 16 + i;
-        wd[i] = (o_ok && k < K) ? a.w[(long)o_in * w_so + (long)k * w_sk] : 0.0f;
+        for (int t = 0; t < 4; ++t) gw[t] = *reinterpret_cast<const f32x4_unaligned *>(w_src[t] + kc);
+      } else { // the end of a row: nothing is read past it
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          f32x4 z;
+          z.x = (kc < K) ? w_src[t][kc] : 0.0f;
+          z.y = (kc + 1 < K) ? w_src[t][kc + 1] : 0.0f;
+          z.z = (kc + 2 < K) ? w_src[t][kc + 2] : 0.0f;
+          z.w = 0.0f;
+          gw[t] = z;
+        }
       }
     }
   };
@@ -293,7 +324,7 @@ __device__ __forceinline__ void mvm_round_tile(const MvmArgs &a, int round, int 
     for (int t = 0; t < 4; ++t) {
       const int off = (t * 8 + st_row) * LDS_ROW + st_chunk;
       *reinterpret_cast<f32x4 *>(stage_x + off) = gx[t];
-      if (WMODE == 0) *reinterpret_cast<f32x4 *>(stage_w + off) = gw[t];
+      if (WMODE != 1) *reinterpret_cast<f32x4 *>(stage_w + off) = gw[t];
     }
   };
   auto lds_read = [&](float (&xd)[16], float (&wd)[16]) {
@@ -302,7 +333,7 @@ __device__ __forceinline__ void mvm_round_tile(const MvmArgs &a, int round, int 
       const int off = r * LDS_ROW + h * 16 + v4 * 4;
       const f32x4 tx = *reinterpret_cast<const f32x4 *>(stage_x + off);
       xd[v4 * 4 + 0] = tx.x; xd[v4 * 4 + 1] = tx.y; xd[v4 * 4 + 2] = tx.z; xd[v4 * 4 + 3] = tx.w;
-      if (WMODE == 0) {
+      if (WMODE != 1) {
         const f32x4 tw = *reinterpret_cast<const f32x4 *>(stage_w + off);
         wd[v4 * 4 + 0] = tw.x; wd[v4 * 4 + 1] = tw.y; wd[v4 * 4 + 2] = tw.z; wd[v4 * 4 + 3] = tw.w;
       }
@@ -325,7 +356,7 @@ __device__ __forceinline__ void mvm_round_tile(const MvmArgs &a, int round, int 
 #define RPU_MVM_STEP(T, GX, GW, WR, XC, WC, XN, WN)                      \
   {                                                                      \
     lds_store(GX, GW);                                                   \
-    if (WMODE != 0) {                                                    \
+    if (WMODE == 1) {                                                    \
       _Pragma("unroll") for (int i = 0; i < 16; ++i) WN[i] = WR[i];      \
     }                                                                    \
     gload(min((T) + 1 + PD, s_end - 1), GX, GW, WR);                     \
@@ -341,7 +372,7 @@ __device__ __forceinline__ void mvm_round_tile(const MvmArgs &a, int round, int 
     }
     lds_store(gx0, gw0);
     lds_read(xc0, wc0);
-    if (WMODE != 0) {
+    if (WMODE == 1) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) wc0[i] = wr0[i];
     }
@@ -361,11 +392,11 @@ __device__ __forceinline__ void mvm_round_tile(const MvmArgs &a, int round, int 
   } else {
     f32x4 gx[4], gw[4];
     float wn[16], xc[16], wc[16];
-    gload(s_begin, gx, gw, wn);
+    if (s_begin < s_end) gload(s_begin, gx, gw, wn);
     for (int s = s_begin; s < s_end; ++s) {
       lds_store(gx, gw);
       lds_read(xc, wc);
-      if (WMODE != 0) {
+      if (WMODE == 1) {
 #pragma unroll
         for (int i = 0; i < 16; ++i) wc[i] = wn[i];
       }
@@ -417,26 +448,40 @@ __device__ __forceinline__ void mvm_round_tile(const MvmArgs &a, int round, int 
 // per-sample noise management and state of round 0.  One workgroup per sample.
 // rpu_forward_backward_pass.cpp:112-178 (scales), :919-969 (forward), :1003-1022 (backward)
 
-__device__ __forceinline__ float block_reduce_max(float v, float *sh) {
+// Reductions over the SUB threads that share a sample: SUB = 256 is the whole workgroup (through LDS), smaller
+// values are aligned lane groups of a wave (shuffles).  Every thread of the group gets the result.
+template <int SUB>
+__device__ __forceinline__ float group_max(float v, float *sh) {
+  if constexpr (SUB == 256) {
 #pragma unroll
-  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off));
-  if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = v;
-  __syncthreads();
-  float r = sh[0];
-  for (int i = 1; i < (int)(blockDim.x >> 6); ++i) r = fmaxf(r, sh[i]);
-  __syncthreads();
-  return r;
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off));
+    if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = v;
+    __syncthreads();
+    const float r = fmaxf(fmaxf(sh[0], sh[1]), fmaxf(sh[2], sh[3]));
+    __syncthreads();
+    return r;
+  } else {
+#pragma unroll
+    for (int off = SUB / 2; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off));
+    return v;
+  }
 }
 
-__device__ __forceinline__ float block_reduce_sum(float v, float *sh) {
+template <int SUB>
+__device__ __forceinline__ float group_sum(float v, float *sh) {
+  if constexpr (SUB == 256) {
 #pragma unroll
-  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
-  if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = v;
-  __syncthreads();
-  float r = sh[0];
-  for (int i = 1; i < (int)(blockDim.x >> 6); ++i) r += sh[i];
-  __syncthreads();
-  return r;
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
+    if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = v;
+    __syncthreads();
+    const float r = ((sh[0] + sh[1]) + sh[2]) + sh[3];
+    __syncthreads();
+    return r;
+  } else {
+#pragma unroll
+    for (int off = SUB / 2; off > 0; off >>= 1) v += __shfl_xor(v, off);
+    return v;
+  }
 }
 
 // input scale of a round and the factor applied to its ADC output
@@ -497,12 +542,13 @@ __device__ __forceinline__ float next_round_scale(const MvmArgs &a, int round, i
   return round_scales(a, nm, red, fin_next);
 }
 
-// state of round 0 and quantized input row of sample b; called by a whole workgroup
-__device__ __forceinline__ void mvm_init_sample(const MvmArgs &a, int b, float *sh, float *sh_scale_p) {
-  float &sh_scale = *sh_scale_p;
+// State of round 0 and quantized input row of sample b, by the SUB threads that share the sample (this one is
+// number t of them); gid / gstride number the threads that work on this tile's call, for clearing its counters.
+template <int SUB>
+__device__ __forceinline__ void mvm_init_sample(const MvmArgs &a, int b, int t, long gid, long gstride, float *sh) {
   const IoDev &io = a.io;
   if (io.perfect) { // plain copy into the k-contiguous scratch
-    write_dac_row(a, b, b, 1.0f, 0, a.xq[0]);
+    write_dac_row(a, b, b, 1.0f, 0, a.xq[0], t, SUB);
     return;
   }
   const float *row = a.in + (long)b * a.in_sb;
@@ -511,23 +557,23 @@ __device__ __forceinline__ void mvm_init_sample(const MvmArgs &a, int b, float *
   const bool need_np = io.noise_management == RPU_NM_ABS_MAX_NP_SUM || worst_case;
   if (io.noise_management == RPU_NM_ABS_MAX || io.noise_management == RPU_NM_MAX || need_np) {
     float amax = 0.0f, vmax = -INFINITY, ps = 0.0f, ns = 0.0f;
-    for (int k = threadIdx.x; k < a.K; k += blockDim.x) {
+    for (int k = t; k < a.K; k += SUB) {
       const float x = row[(long)k * a.in_sk];
       amax = fmaxf(amax, fabsf(x));
       vmax = fmaxf(vmax, x);
       ps += x > 0.0f ? x : 0.0f;
       ns += x < 0.0f ? x : 0.0f;
     }
-    amax = block_reduce_max(amax, sh);
+    amax = group_max<SUB>(amax, sh);
     if (io.noise_management == RPU_NM_MAX) {
-      vmax = block_reduce_max(vmax, sh);
+      vmax = group_max<SUB>(vmax, sh);
       nm = io.nm_thres > 0.0f ? fminf(vmax, io.nm_thres) : vmax;
     } else if (io.noise_management == RPU_NM_ABS_MAX) {
       nm = io.nm_thres > 0.0f ? fminf(amax, io.nm_thres) : amax;
     }
     if (need_np) {
-      ps = block_reduce_sum(ps, sh);
-      ns = block_reduce_sum(ns, sh);
+      ps = group_sum<SUB>(ps, sh);
+      ns = group_sum<SUB>(ns, sh);
       const float bound = isinf(io.out_bound) ? 1.0f : io.out_bound;
       const float sum = fmaxf(ps, -ns);
       const float am = io.nm_thres > 0.0f ? fminf(amax, io.nm_thres) : amax;
@@ -535,36 +581,40 @@ __device__ __forceinline__ void mvm_init_sample(const MvmArgs &a, int b, float *
       if (io.inp_res > 0.0f) np = fminf(am / io.inp_res * io.max_bm_res, np);
       np = fmaxf(am, np);
       if (io.noise_management == RPU_NM_ABS_MAX_NP_SUM) nm = np;
-      if (threadIdx.x == 0) a.st.nm_np[b] = np;
+      if (t == 0) a.st.nm_np[b] = np;
     }
   }
   if (io.noise_management == RPU_NM_CONSTANT) {
     nm = io.nm_thres > 0.0f ? io.nm_thres : 1.0f;
   }
-  if (threadIdx.x == 0) {
+  // every thread of the group knows nm: the scales need no exchange
+  float fin;
+  const float scale = round_scales(a, nm, 1.0f, fin);
+  if (t == 0) {
     a.st.nm[b] = nm;
     a.st.red[b] = 1.0f;
     a.st.hit_up[b] = 0;
     a.st.hit_lo[b] = 0;
-    sh_scale = set_round_scales(a, b, nm, 1.0f);
-    const float fin = a.st.fin[b];
+    a.st.scale[b] = scale;
+    a.st.fin[b] = fin;
     a.st.rounds[b] = (fin == 0.0f) ? 0 : 1;
     if (io.bound_management != RPU_BM_NONE) a.st.next_scale[0][b] = next_round_scale(a, 0, b, fin, nm, 1.0f);
   }
-  if (b == 0 && threadIdx.x < 40) a.st.count[threadIdx.x] = 0;
+  if (gid < 40) a.st.count[gid] = 0;
   {
-    const int n_done = 32 * ((a.m_batch + TILE - 1) / TILE);
-    for (int idx = b * blockDim.x + threadIdx.x; idx < n_done; idx += gridDim.x * blockDim.x) a.st.tile_done[idx] = 0;
+    const long n_done = 32L * ((a.m_batch + TILE - 1) / TILE);
+    for (long idx = gid; idx < n_done; idx += gstride) a.st.tile_done[idx] = 0;
   }
-  __syncthreads();
-  write_dac_row(a, b, b, sh_scale, 0, a.xq[0]);
-  __syncthreads(); // sh / sh_scale are reused by the caller's next sample
+  write_dac_row(a, b, b, scale, 0, a.xq[0], t, SUB);
 }
 
+// SUB threads per sample: a workgroup holds 256 / SUB samples
+template <int SUB>
 __global__ __launch_bounds__(256) void k_mvm_init(MvmArgs a) {
   __shared__ float sh[8];
-  __shared__ float sh_scale;
-  mvm_init_sample(a, blockIdx.x, sh, &sh_scale);
+  const int b = blockIdx.x * (256 / SUB) + threadIdx.x / SUB;
+  if (b >= a.m_batch) return; // a whole group of SUB threads leaves together
+  mvm_init_sample<SUB>(a, b, threadIdx.x % SUB, blockIdx.x * 256L + threadIdx.x, gridDim.x * 256L, sh);
 }
 
 // At the start of round `round`, the workgroups of a sample tile (one per output tile) each quantize a
@@ -617,8 +667,10 @@ __device__ __forceinline__ void mvm_prepare_next_rows(const MvmArgs &a, int roun
 
 // After round `round`, for sample b at position `slot` of that round's list: a sample whose ADC saturated
 // gets another round unless the reduction limit is reached (rpu_forward_backward_pass.cpp:944-983); its
-// quantized row for that round was written by mvm_prepare_next_rows.  One thread per sample.
-__device__ __forceinline__ void mvm_advance_sample(const MvmArgs &a, int round, int b, int slot) {
+// quantized row for that round was written by mvm_prepare_next_rows, or (a.speculate == 0) is written by the
+// caller into row `pos` of the other scratch matrix.  One thread per sample; returns the sample's position in
+// the next round's list, -1 when it has no further round.
+__device__ __forceinline__ int mvm_advance_sample(const MvmArgs &a, int round, int b, int slot, float &scale) {
   const IoDev &io = a.io;
   // the flags were raised with device-scope atomics by workgroups on any XCD: read and clear them the same way
   const int up = atomicExch(&a.st.hit_up[b], 0);
@@ -626,17 +678,18 @@ __device__ __forceinline__ void mvm_advance_sample(const MvmArgs &a, int round, 
   // the CPU loop sets "failed" on an upper hit and *assigns* !bm_test_negative_bound on a lower hit,
   // walking the outputs in index order: the last hit decides
   const bool failed = io.bm_test_negative_bound ? (up > 0 || lo > 0) : (up > lo);
-  if (!failed) return;
+  if (!failed) return -1;
   float nm = a.st.nm[b], red = a.st.red[b];
-  if (!next_round_params(a, round, b, a.st.fin[b], nm, red)) return;
+  if (!next_round_params(a, round, b, a.st.fin[b], nm, red)) return -1;
   a.st.nm[b] = nm;
   a.st.red[b] = red;
   a.st.rounds[b] += 1;
-  set_round_scales(a, b, nm, red);
+  scale = set_round_scales(a, b, nm, red);
   const int pos = atomicAdd(&a.st.count[round + 1], 1);
   a.st.list[(round + 1) & 1][pos] = b;
-  a.st.row[(round + 1) & 1][pos] = slot;
+  a.st.row[(round + 1) & 1][pos] = a.speculate ? slot : pos;
   a.st.next_scale[(round + 1) & 1][pos] = next_round_scale(a, round + 1, b, a.st.fin[b], nm, red);
+  return pos;
 }
 
 // Called by every workgroup of a round once its outputs are stored and its saturation flags are raised.  The
@@ -654,21 +707,41 @@ __device__ __forceinline__ void mvm_tile_finished(const MvmArgs &a, int round, i
   }
   __syncthreads();
   if (!sh_last) return;
+  __shared__ int sh_more, sh_more_b[TILE], sh_more_pos[TILE];
+  __shared__ float sh_more_scale[TILE];
+  if (threadIdx.x == 0) sh_more = 0;
+  __syncthreads();
   if (threadIdx.x < TILE) {
     const int slot = tile_b * TILE + threadIdx.x;
-    if (slot < n_act) mvm_advance_sample(a, round, (round > 0) ? a.st.list[round & 1][slot] : slot, slot);
+    if (slot < n_act) {
+      const int b = (round > 0) ? a.st.list[round & 1][slot] : slot;
+      float scale = 0.0f;
+      const int pos = mvm_advance_sample(a, round, b, slot, scale);
+      if (pos >= 0 && !a.speculate) {
+        const int i = atomicAdd(&sh_more, 1);
+        sh_more_b[i] = b;
+        sh_more_pos[i] = pos;
+        sh_more_scale[i] = scale;
+      }
+    }
+  }
+  if (a.speculate) return;
+  // a large batch does not quantize rows ahead (few samples go on, and twice the input traffic would be paid for
+  // them): the rows of the samples that do go on are written now
+  __syncthreads();
+  for (int i = 0; i < sh_more; ++i) {
+    write_dac_row(a, sh_more_b[i], sh_more_pos[i], sh_more_scale[i], round + 1, a.xq[(round + 1) & 1], threadIdx.x, 256);
   }
 }
 
 // work of workgroup number n of a round launch of one tile
 template <int PD, int WMODE>
-__device__ __forceinline__ void mvm_round_workgroup(const MvmArgs &a, int round, int n, float (*red)[16][64],
+__device__ __forceinline__ void mvm_round_workgroup(const MvmArgs &a, int round, int n, int n_act, float (*red)[16][64],
                                                     float *stage) {
-  const int n_act = (round > 0) ? a.st.count[round] : a.m_batch;
   int tile_o, tile_b;
   if (!tile_of(a, n, n_act, tile_o, tile_b)) return;
   const bool more_rounds = round + 1 < a.max_rounds;
-  if (more_rounds) mvm_prepare_next_rows(a, round, tile_o, tile_b, n_act);
+  if (more_rounds && a.speculate) mvm_prepare_next_rows(a, round, tile_o, tile_b, n_act);
   mvm_round_tile<PD, WMODE>(a, round, tile_o, tile_b, n_act, red, stage);
   if (more_rounds) mvm_tile_finished(a, round, tile_b, n_act);
 }
@@ -677,7 +750,8 @@ template <int PD, int WMODE>
 __global__ __launch_bounds__(256) void k_mvm_round(MvmArgs a) {
   __shared__ float red[WAVES][16][64];
   __shared__ __attribute__((aligned(16))) float stage[WAVES * 2 * TILE * LDS_ROW];
-  mvm_round_workgroup<PD, WMODE>(a, a.round, blockIdx.x, red, stage);
+  const int n_act = (a.round > 0) ? a.st.count[a.round] : a.m_batch;
+  mvm_round_workgroup<PD, WMODE>(a, a.round, blockIdx.x, n_act, red, stage);
 }
 
 // The same for several tiles in one launch: a workgroup finds its tile in the table of first workgroup numbers
@@ -690,14 +764,15 @@ __global__ __launch_bounds__(256) void k_mvm_round_group(MvmGroup g, int round) 
   while (t + 1 < g.n && (int)blockIdx.x >= g.start[t + 1]) ++t;
   const MvmArgs &a = g.args[t];
   if (round > 0 && round >= a.max_rounds) return;
-  mvm_round_workgroup<PD, WMODE>(a, round, (int)blockIdx.x - g.start[t], red, stage);
+  const int n_act = (round > 0) ? a.st.count[round] : a.m_batch;
+  mvm_round_workgroup<PD, WMODE>(a, round, (int)blockIdx.x - g.start[t], n_act, red, stage);
 }
 
 __global__ __launch_bounds__(256) void k_mvm_init_group(MvmGroup g) {
   __shared__ float sh[8];
-  __shared__ float sh_scale;
   const int t = blockIdx.x / g.m_batch;
-  mvm_init_sample(g.args[t], blockIdx.x - t * g.m_batch, sh, &sh_scale);
+  const int b = blockIdx.x - t * g.m_batch;
+  mvm_init_sample<256>(g.args[t], b, threadIdx.x, b * 256L + threadIdx.x, g.m_batch * 256L, sh);
 }
 
 __global__ void k_make_bias(const float *in, float *out, int m_batch, int x_size, int in_trans) {
@@ -745,7 +820,8 @@ int mvm_max_rounds(const IoDev &io) {
 static int mvm_prefetch_depth(int K) { return K >= 512 ? 4 : (K >= 256 ? 2 : 1); }
 
 int mvm_k_pad(int K) {
-  const int unit = KSTEP * WAVES * mvm_prefetch_depth(K);
+  const int depth = mvm_prefetch_depth(K);
+  const int unit = depth == 1 ? KSTEP : KSTEP * WAVES * depth;
   return ((K + unit - 1) / unit) * unit;
 }
 
@@ -756,16 +832,19 @@ static int weight_mode(const MvmArgs &a) {
   return 2;
 }
 
+// A small batch gets a workgroup per sample (most workgroups in flight, shortest latency); a large one gets as
+// many threads per sample as its rows can keep busy.
 void launch_mvm_init(const MvmArgs &a, hipStream_t s) {
-  hipLaunchKernelGGL(k_mvm_init, dim3(a.m_batch), dim3(256), 0, s, a);
+  if (a.m_batch <= 1024 || a.K > 512) {
+    hipLaunchKernelGGL(k_mvm_init<256>, dim3(a.m_batch), dim3(256), 0, s, a);
+  } else if (a.K > 64) {
+    hipLaunchKernelGGL(k_mvm_init<64>, dim3((a.m_batch + 3) / 4), dim3(256), 0, s, a);
+  } else {
+    hipLaunchKernelGGL(k_mvm_init<16>, dim3((a.m_batch + 15) / 16), dim3(256), 0, s, a);
+  }
 }
 
-int mvm_round_workgroups(const MvmArgs &a) {
-  const int tiles_o = (a.O + TILE - 1) / TILE;
-  const int per = (tiles_o + 7) / 8;
-  const int tiles_b = (a.m_batch + TILE - 1) / TILE;
-  return 8 * per * tiles_b;
-}
+int mvm_round_workgroups(const MvmArgs &a) { return workgroups_for(a.O, a.m_batch); }
 
 void mvm_round_variant(const MvmArgs &a, int &prefetch_depth, int &mode) {
   prefetch_depth = mvm_prefetch_depth(a.K);

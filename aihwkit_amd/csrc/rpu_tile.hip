@@ -337,6 +337,7 @@ struct Tile {
     if (!io.perfect && io.p.bound_management != RPU_BM_NONE) s_xq1.ensure((size_t)B * a.k_pad);
     a.xq[0] = s_xq0.p; a.xq[1] = s_xq1.p;
     a.max_rounds = io.perfect ? 0 : mvm_max_rounds(a.io);
+    a.speculate = B <= 1024 ? 1 : 0;
     return a;
   }
 

@@ -137,6 +137,17 @@ class InferenceTile:
         check(lib().rpu_tile_get_drift_state(tile._h, out[0].data_ptr(), out[1].data_ptr(), out[2].data_ptr()))
         return tuple(out)
 
+    def set_matrix_indices(self, indices: torch.Tensor) -> None:
+        """Index matrix of a convolution layer (what ``AnalogConvNd`` computes once per input shape)."""
+        self._gpu().set_matrix_indices(indices)
+
+    def forward_indexed(self, x_input: torch.Tensor, d_tensor: torch.Tensor, is_test: bool = False) -> torch.Tensor:
+        """Analog forward of a convolution through the index matrix, drift compensation as in ``forward``."""
+        out = self._gpu().forward_indexed(x_input, d_tensor, is_test)
+        if is_test and self.drift_compensation is not None and self.alpha != 1.0:
+            out.mul_(self.alpha)
+        return out
+
     def forward(self, x_input: torch.Tensor, is_test: bool = False) -> torch.Tensor:
         """Analog forward; in evaluation mode the output is scaled by the drift compensation (inference.py:264-282)."""
         out = self._gpu().forward(x_input, False, False, False, is_test, False)

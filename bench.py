@@ -46,7 +46,7 @@ def main() -> int:
     ap.add_argument("--pmc", action="store_true",
                     help="counter-collection mode for rocprofv3 --pmc: one 64 MiB calibration copy, then 3 update, "
                          "3 forward and 3 backward calls; no timing, no JSON line")
-    ap.add_argument("--config", type=int, default=2, choices=(1, 2, 3, 5),
+    ap.add_argument("--config", type=int, default=2, choices=(1, 2, 3, 4, 5),
                     help="benchmark configuration: 2 is the graded one; 3 is the Tiki-Taka MLP of transfer tiles; "
                          "5 is the forward pass of the GPT-2-small linear layers as PCM inference tiles")
     args = ap.parse_args()
@@ -70,6 +70,8 @@ def main() -> int:
 
     if args.config == 3:
         return bench_config3(args)
+    if args.config == 4:
+        return bench_config4(args)
     if args.config == 5:
         return bench_config5(args)
 
@@ -417,6 +419,126 @@ def bench_config5(args) -> int:
                                "out_noise 0.04, abs-max noise management", "tokens": tokens, "tiles": n_tiles},
         "useful_tflops": flops / (ms_per_step * 1e-3) / 1e12,
         "ms_per_step_one_call_per_tile": ms_per_tile_loop,
+    }
+    print(json.dumps(out))
+    return 0
+
+
+def conv_index_matrix(image_shape, kernel, with_bias=True):
+    """Index matrix of an unpadded stride-1 2-d convolution: entry [k, p] names the image element (offset by 2) that
+    patch p reads at kernel position k; 1 marks the bias row.  Returns (int32 indices [x_size * patches], patches)."""
+    import torch
+    import torch.nn.functional as F
+
+    size = int(torch.tensor(image_shape).prod())
+    numbered = torch.arange(2, size + 2, dtype=torch.float32).reshape(1, *image_shape)
+    unfolded = F.unfold(numbered, kernel_size=kernel)[0]                       # [C k k, patches]
+    if with_bias:
+        unfolded = torch.cat([unfolded, torch.ones(1, unfolded.shape[1])], dim=0)
+    return unfolded.to(torch.int32).contiguous().reshape(-1), unfolded.shape[1]
+
+
+def bench_config4(args) -> int:
+    """Configuration 4: forward pass of a LeNet5-shaped stack for 512 images of 28 x 28: two 5 x 5 convolutions
+    (1 -> 16, 16 -> 32) as indexed analog tiles, tanh and 2 x 2 max pooling in torch between them, then 512 -> 128 -> 10
+    fully connected tiles.  Weights are programmed with PCM noise and drifted to one day with global drift
+    compensation; 8-bit DAC / ADC.  A step = the forward pass of the 512 images."""
+    import numpy as np
+    import torch
+    import torch.nn.functional as F
+
+    from aihwkit_amd.inference import InferenceTile
+    from aihwkit_amd.rpu_base import devices as dv
+    from helpers import io_params
+
+    torch.cuda.set_device(0)
+    batch = 512
+    rng = np.random.default_rng(0)
+    io = io_params(inp_res=1 / 254.0, out_res=1 / 254.0, out_noise=0.06, noise_management=dv.NoiseManagementType.AbsMax,
+                   bound_management=dv.BoundManagementType.Iterative)
+    shapes = (("conv", (1, 28, 28), 16), ("conv", (16, 12, 12), 32), ("fc", 512, 128), ("fc", 128, 10))
+    stack, flops, host_weights = [], 0.0, []
+    for k, (kind, in_shape, out_size) in enumerate(shapes):
+        if kind == "conv":
+            indices, patches = conv_index_matrix(in_shape, (5, 5))
+            in_size = in_shape[0] * 25 + 1
+        else:
+            indices, patches, in_size = None, 1, in_shape + 1
+        w = (rng.uniform(-1, 1, (out_size, in_size)) / np.sqrt(in_size)).astype(np.float32)
+        tile = InferenceTile(out_size, in_size, forward_io=io)
+        tile.set_weights(torch.from_numpy(w))
+        tile.cuda()
+        tile.tile.set_seed(2000 + k)
+        if indices is not None:
+            tile.set_matrix_indices(indices)
+        tile.drift_weights(86400.0)
+        stack.append((kind, tile, patches, out_size))
+        host_weights.append(w)
+        flops += 2.0 * batch * patches * in_size * out_size
+    x = torch.from_numpy(rng.uniform(0, 1, (batch, 1, 28, 28)).astype(np.float32)).cuda()
+    ones = torch.ones(batch, 1, device="cuda")
+
+    def step():
+        h = x
+        for kind, tile, patches, out_size in stack:
+            if kind == "conv":
+                side = int(round(patches ** 0.5))
+                y = tile.forward_indexed(h, torch.empty(h.size(0), out_size, side, side, device="cuda"), is_test=True)
+                h = F.max_pool2d(torch.tanh(y), 2)
+            else:
+                h = tile.forward(torch.cat([h.reshape(h.size(0), -1), ones], dim=1), is_test=True)
+                if out_size != 10:
+                    h = torch.tanh(h)
+        return h
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    cpu = None
+    if not args.no_cpu_baseline:
+        from indexed_oracle import IndexedOracle
+        from oracle_lib import OracleTile
+
+        sample = 16
+        meta = dv.AnalogTileParameter()
+        meta.forward_io = io
+        t0 = time.perf_counter()
+        h = x[:sample].cpu().numpy()
+        for (kind, tile, patches, out_size), w in zip(stack, host_weights):
+            orc = OracleTile(w.shape[1], w.shape[0], meta._config(dv.IdealResistiveDeviceParameter()))
+            orc.set_weights(w)
+            if kind == "conv":
+                side = int(round(patches ** 0.5))
+                in_shape = h.shape[1:]
+                idx, _ = conv_index_matrix(in_shape, (5, 5))
+                y = IndexedOracle(orc, idx.numpy(), patches).forward(h).reshape(sample, out_size, side, side)
+                h = F.max_pool2d(torch.tanh(torch.from_numpy(y)), 2).numpy()
+            else:
+                flat = np.concatenate([h.reshape(sample, -1), np.ones((sample, 1), np.float32)], axis=1)
+                h = orc.forward(np.ascontiguousarray(flat))
+                if out_size != 10:
+                    h = np.tanh(h)
+        dt = time.perf_counter() - t0
+        cpu = {"value": sample / dt, "unit": "images/s", "cores": 1, "kind": "port",
+               "sample": "forward of %d images through the oracle tiles and the numpy index gather "
+                         "(weights as set, without the PCM perturbation)" % sample}
+    out = {
+        "metric": "noisy inference forward of a LeNet5-shaped stack of PCM tiles, images/s, 1 MI355X",
+        "value": batch / (ms_per_step * 1e-3), "unit": "images/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "config4: conv 1->16 5x5 (tile 26 x 16, 576 patches), conv 16->32 5x5 (tile 401 x 32, 64 "
+                               "patches), fc 513 x 128, fc 129 x 10, batch 512 images 28 x 28, PCM programming noise + "
+                               "drift to 1 day + global drift compensation, 8-bit IO, abs-max noise management",
+                   "batch": batch},
+        "useful_tflops": flops / (ms_per_step * 1e-3) / 1e12,
+        "cpu_baseline": cpu,
     }
     print(json.dumps(out))
     return 0
