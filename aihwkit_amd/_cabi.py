@@ -109,6 +109,17 @@ SYMBOLS = {
     "rpu_tile_forward_indexed": (C.c_int, [_P, _P, _P, C.c_int, C.c_long, C.c_int, _P]),
     "rpu_tile_backward_indexed": (C.c_int, [_P, _P, _P, C.c_int, C.c_long, _P]),
     "rpu_tile_update_indexed": (C.c_int, [_P, _P, _P, C.c_int, C.c_long, _P]),
+    "rpu_tile_decay_weights": (C.c_int, [_P, C.c_float, C.c_int, _P]),
+    "rpu_tile_diffuse_weights": (C.c_int, [_P, _P]),
+    "rpu_tile_clip_weights": (C.c_int, [_P, C.c_int, C.c_float, C.c_float, _P]),
+    "rpu_tile_reset_columns": (C.c_int, [_P, C.c_int, C.c_int, C.c_float, _P]),
+    "rpu_tile_set_shared_weights": (C.c_int, [_P, _P]),
+    "rpu_tile_get_shared_weights_if": (C.c_int, [_P]),
+    "rpu_tile_set_delta_weights": (C.c_int, [_P, _P]),
+    "rpu_tile_extra_count": (C.c_int, [_P]),
+    "rpu_tile_extra_name": (C.c_char_p, [_P, C.c_int]),
+    "rpu_tile_get_extra": (C.c_int, [_P, C.POINTER(C.c_int64)]),
+    "rpu_tile_set_extra": (C.c_int, [_P, C.POINTER(C.c_int64), C.c_int]),
     "rpu_group_create": (C.c_int, [C.POINTER(_P), C.POINTER(_P), C.c_int]),
     "rpu_group_forward": (C.c_int, [_P, C.POINTER(_P), C.POINTER(_P), C.c_int, C.c_int, _P]),
     "rpu_group_destroy": (C.c_int, [_P]),

@@ -137,6 +137,26 @@ void launch_update_planes(const UpdateArgs &a, hipStream_t s);        // pulse w
 void launch_update_pulsed(const UpdateArgs &a, hipStream_t s);        // coincidences + device steps
 void launch_update_implicit(const UpdateArgs &a, hipStream_t s);
 void launch_implicit_counts(const UpdateArgs &a, int32_t *counts, hipStream_t s);
+// ----- weight maintenance between steps (kernels_state.hip); w_min / w_max may be null (no device bounds)
+void launch_decay_device(float *w, const float *decay_scale, const float *reset_bias, const float *w_min,
+                         const float *w_max, float alpha, int bias_no_decay, int x_size, size_t n, hipStream_t s);
+void launch_decay_scalar(float *w, float scale, int bias_no_decay, int x_size, size_t n, hipStream_t s);
+// rates == null: the same rate for every element
+void launch_diffuse(float *w, const float *rates, float rate, const float *w_min, const float *w_max, PhiloxKey key,
+                    uint32_t call, size_t n, hipStream_t s);
+// clip to +- clip (clip < 0: bounds only); clip_dev != null: the value is read from device memory and a value
+// that is not positive leaves the weights alone
+void launch_clip_value(float *w, const float *w_min, const float *w_max, float clip, const float *clip_dev, size_t n,
+                       hipStream_t s);
+void launch_clip_value_gaussian(const float *w, size_t n, float sigma, float fixed_value, float *clip_out, hipStream_t s);
+void launch_clip_value_channel(const float *w, int x_size, int d_size, float fixed_value, float *row_max, float *clip_out,
+                               hipStream_t s);
+void launch_reset_cols(float *w, const float *reset_bias, const float *w_min, const float *w_max, float reset_std,
+                       int start_col, int n_cols, float reset_prob, int x_size, int d_size, PhiloxKey key, uint32_t call,
+                       hipStream_t s);
+// prev_w_and_delta holds the weights from before an update: it becomes scale * (w - previous), w gets them back
+void launch_delta_finish(float *w, float *prev_w_and_delta, float scale, size_t n, hipStream_t s);
+
 // clip weights into [w_min, w_max]
 void launch_clip(float *w, const float *w_min, const float *w_max, size_t n, hipStream_t s);
 

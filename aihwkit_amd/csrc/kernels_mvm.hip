@@ -641,25 +641,37 @@ __device__ __forceinline__ void mvm_prepare_next_rows(const MvmArgs &a, int roun
   const int chunk = (a.k_pad + tiles_o - 1) / tiles_o;
   const int k_lo = tile_o * chunk;
   const int k_hi = min(k_lo + chunk, a.k_pad);
-  float *dst = a.xq[(round + 1) & 1];
-  // a trip covers 32 k-values of all 32 rows: 8 threads-rows x 4 rows each
+  float *__restrict__ dst = a.xq[(round + 1) & 1];
+  const float *__restrict__ in = a.in;
+  // a trip covers 32 k-values of all 32 rows: 8 thread-rows x 4 rows each.  The loads of four trips are issued
+  // together: a narrow tile has few workgroups per sample tile and each walks a long piece of the rows.
   const int kq = threadIdx.x & 31, rq = threadIdx.x >> 5;
-  for (int k0 = k_lo; k0 < k_hi; k0 += 32) {
-    const int k = k0 + kq;
-    const bool k_ok = k < k_hi;
-    float xv[4], sc[4];
-    int bt[4];
+  float sc[4];
+  int bt[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      bt[i] = sh_next_b[4 * rq + i];
-      sc[i] = sh_next_scale[4 * rq + i];
-      xv[i] = (k_ok && sc[i] != 0.0f && k < a.K) ? a.in[(long)bt[i] * a.in_sb + (long)k * a.in_sk] : 0.0f;
+  for (int i = 0; i < 4; ++i) {
+    bt[i] = sh_next_b[4 * rq + i];
+    sc[i] = sh_next_scale[4 * rq + i];
+  }
+  for (int k0 = k_lo; k0 < k_hi; k0 += 128) {
+    float xv[4][4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int k = k0 + 32 * u + kq;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        xv[u][i] = (k < k_hi && sc[i] != 0.0f && k < a.K) ? in[(long)bt[i] * a.in_sb + (long)k * a.in_sk] : 0.0f;
+      }
     }
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      if (k_ok && sc[i] != 0.0f) {
-        const float v = (k < a.K) ? dac_value(xv[i], sc[i], a.io, a.key, a.call, round + 1, bt[i], k) : 0.0f;
-        dst[(long)(tile_b * TILE + 4 * rq + i) * a.k_pad + k] = v;
+    for (int u = 0; u < 4; ++u) {
+      const int k = k0 + 32 * u + kq;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        if (k < k_hi && sc[i] != 0.0f) {
+          const float v = (k < a.K) ? dac_value(xv[u][i], sc[i], a.io, a.key, a.call, round + 1, bt[i], k) : 0.0f;
+          dst[(long)(tile_b * TILE + 4 * rq + i) * a.k_pad + k] = v;
+        }
       }
     }
   }

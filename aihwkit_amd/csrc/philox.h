@@ -67,7 +67,9 @@ enum RngPurpose : uint32_t {
   RNG_CTOC = 7,       // cycle-to-cycle update noise
   RNG_UPDATE_SR = 8,  // stochastic rounding of pulse probabilities
   RNG_PCM_PROGRAM = 9, // programming noise and drift coefficients of the inference weight pipeline
-  RNG_PCM_DRIFT = 10   // accumulated read noise at inference time
+  RNG_PCM_DRIFT = 10,  // accumulated read noise at inference time
+  RNG_DIFFUSE = 11,    // weight diffusion
+  RNG_RESET = 12       // column reset (noise, and with round 1 the reset lottery)
 };
 
 // uniform in [0, 1) with 24 bits

@@ -31,16 +31,26 @@ namespace {
 template <typename T> struct DevBuf {
   T *p = nullptr;
   size_t n = 0;
+  bool owned = true;
   void ensure(size_t count) {
     if (count <= n) return;
+    if (!owned) throw RpuError("A buffer that belongs to the caller cannot grow.");
     release();
     RPU_HIP_CHECK(hipMalloc((void **)&p, count * sizeof(T)));
     n = count;
   }
+  // use memory of the caller from now on (never freed here)
+  void adopt(T *external, size_t count) {
+    release();
+    p = external;
+    n = count;
+    owned = false;
+  }
   void release() {
-    if (p) (void)hipFree(p);
+    if (p && owned) (void)hipFree(p);
     p = nullptr;
     n = 0;
+    owned = true;
   }
 };
 
@@ -159,11 +169,17 @@ struct Tile {
   // indexed (convolution) interface: index matrix [X][patches] and the unfolded matrices
   std::vector<int32_t> idx_host;
   int idx_patches = 0;
+  int32_t idx_max = 0; // largest entry of the index matrix
   DevBuf<int> x_idx;
   DevBuf<float> x_mat, d_mat;
   int last_update_batch = 0;
   int last_update_pulse = -1;
   int last_forward_batch = 0;
+  // weight maintenance: per-device decay scales, diffusion rates and reset biases (uploaded at first use),
+  // clip value computed on the device, and the caller's buffer that takes the updates instead of the weights
+  DevBuf<float> d_decay, d_diff, d_rbias, s_clip;
+  bool state_params_valid = false;
+  float *delta_w = nullptr;
 
   // optional per-kernel timing with HIP events on the launch stream
   bool profiling = false;
@@ -220,6 +236,9 @@ struct Tile {
     i_ref.release(); i_prog.release(); i_nu_plus.release(); i_nu_minus.release(); i_scalar.release(); i_absmax.release();
     has_reference = programmed = false;
     x_idx.release(); x_mat.release(); d_mat.release();
+    d_decay.release(); d_diff.release(); d_rbias.release(); s_clip.release();
+    state_params_valid = false;
+    delta_w = nullptr;
     for (auto &sl : slots) sl->release();
   }
 
@@ -239,6 +258,7 @@ struct Tile {
   }
 
   void upload_params() {
+    state_params_valid = false;
     if (!dev.pulsed()) return;
     const size_t n = size(), bytes = n * sizeof(float);
     d_wmax.ensure(n); d_wmin.ensure(n); d_sup.ensure(n); d_sdown.ensure(n);
@@ -429,8 +449,28 @@ struct Tile {
     last_stream = s;
   }
 
+  // With delta weights set the update lands in the caller's buffer as the gradient-like quantity dW with
+  // W_new = W - lr * dW and the weights stay as they are (RPUPulsed::updateMatrix, rpu_pulsed.cpp:560-585;
+  // RPUSimple::updateMatrix with getUpWeights / getUpBeta, rpu.cpp:624-634, 1489-1510).
   void update(const float *x, const float *d, int B, bool bias, bool x_trans, bool d_trans, hipStream_t s) {
-    if (lr == 0.0f) return;
+    const bool fp_update = !dev.pulsed() || up.p.pulse_type == RPU_PULSE_NONE;
+    if (delta_w && !fp_update) {
+      if (lr == 0.0f) throw RpuError("Delta weights of a pulsed update need a learning rate.");
+      RPU_HIP_CHECK(hipMemcpyAsync(delta_w, d_w.p, size() * sizeof(float), hipMemcpyDeviceToDevice, s));
+      float *delta = delta_w;
+      delta_w = nullptr;
+      try {
+        update(x, d, B, bias, x_trans, d_trans, s);
+      } catch (...) {
+        delta_w = delta;
+        throw;
+      }
+      delta_w = delta;
+      launch_delta_finish(d_w.p, delta_w, -1.0f / lr, size(), s);
+      RPU_HIP_CHECK(hipGetLastError());
+      return;
+    }
+    if (lr == 0.0f && !delta_w) return;
     const float *xin = x;
     long x_sb = x_trans ? 1 : X, x_sj = x_trans ? B : 1;
     if (bias) {
@@ -440,16 +480,16 @@ struct Tile {
     }
     const long d_sb = d_trans ? 1 : D, d_si = d_trans ? B : 1;
 
-    if (!dev.pulsed() || up.p.pulse_type == RPU_PULSE_NONE) {
+    if (fp_update) {
       // W += -lr * d^T x as a contraction over the batch (rpu.cpp:624-634): "weights" = d, K = batch
       MvmArgs a{};
       a.w = d; a.transposed = d_trans ? 0 : 1; // element (o = i, k = b): d[b * D + i] or d[i * B + b]
       a.x_size = d_trans ? B : D; a.d_size = d_trans ? D : B;
       a.K = B; a.O = D; a.m_batch = X;
       a.in = xin; a.in_sb = x_sj; a.in_sk = x_sb; // "sample" = column j of x, contraction over b
-      a.out = d_w.p; a.out_sb = 1; a.out_so = X;
+      a.out = delta_w ? delta_w : d_w.p; a.out_sb = 1; a.out_so = X;
       a.io = io_dev(fio); a.io.perfect = 1;
-      a.alpha = -lr; a.beta = 1.0f; a.round = 0;
+      a.alpha = delta_w ? 1.0f : -lr; a.beta = delta_w ? 0.0f : 1.0f; a.round = 0;
       a.key = key(); a.call = call++;
       a.k_pad = mvm_k_pad(B);
       s_xq0.ensure((size_t)X * a.k_pad);
@@ -472,6 +512,107 @@ struct Tile {
     }
     DeviceView dv{d_w.p, d_wmax.p, d_wmin.p, d_sup.p, d_sdown.p, d_slup.p, d_sldown.p, &dev, dev.p.dw_min};
     pulsed_update_on(dv, up, lr, xin, x_sb, x_sj, d, d_sb, d_si, B, s);
+  }
+
+  // ----- weight maintenance between steps (decay, diffusion, clipping, column reset) ------------------------------
+
+  void ensure_state_params() {
+    if (!dev.pulsed() || state_params_valid) return;
+    const size_t n = size(), bytes = n * sizeof(float);
+    d_decay.ensure(n); d_diff.ensure(n); d_rbias.ensure(n);
+    RPU_HIP_CHECK(hipMemcpy(d_decay.p, arr.decay_scale.data(), bytes, hipMemcpyHostToDevice));
+    RPU_HIP_CHECK(hipMemcpy(d_diff.p, arr.diffusion_rate.data(), bytes, hipMemcpyHostToDevice));
+    RPU_HIP_CHECK(hipMemcpy(d_rbias.p, arr.reset_bias.data(), bytes, hipMemcpyHostToDevice));
+    state_params_valid = true;
+  }
+
+  void check_maintenance(const char *what) {
+    if (!resident()) throw RpuError(std::string(what) + " needs the tile on a GPU (rpu_tile_to_device).");
+    if (is_transfer()) throw RpuError(std::string(what) + " is not provided for a transfer compound.");
+  }
+
+  // RPUPulsed::decayWeights -> PulsedRPUDevice::decayWeights (rpu_pulsed_device.cpp:392-420) for a pulsed device,
+  // SimpleRPUDevice::decayWeights (rpu_simple_device.cpp:96-115) otherwise
+  void decay_weights(float alpha, bool bias_no_decay, hipStream_t s) {
+    check_maintenance("decay_weights");
+    if (dev.pulsed()) {
+      ensure_state_params();
+      launch_decay_device(d_w.p, d_decay.p, d_rbias.p, d_wmin.p, d_wmax.p, alpha, bias_no_decay ? 1 : 0, X, size(), s);
+    } else {
+      const float rate = dev.p.lifetime > 1.0f ? 1.0f / dev.p.lifetime : 0.0f;
+      const float scale = 1.0f - alpha * rate;
+      if (scale > 0.0f && scale < 1.0f) launch_decay_scalar(d_w.p, scale, bias_no_decay ? 1 : 0, X, size(), s);
+    }
+    RPU_HIP_CHECK(hipGetLastError());
+    last_stream = s;
+  }
+
+  // rpu_pulsed_device.cpp:432-446, rpu_simple_device.cpp:124-134
+  void diffuse_weights(hipStream_t s) {
+    check_maintenance("diffuse_weights");
+    if (dev.pulsed()) {
+      ensure_state_params();
+      launch_diffuse(d_w.p, d_diff.p, 0.0f, d_wmin.p, d_wmax.p, key(), call++, size(), s);
+    } else if (dev.p.diffusion > 0.0f) {
+      launch_diffuse(d_w.p, nullptr, dev.p.diffusion, nullptr, nullptr, key(), call++, size(), s);
+    }
+    RPU_HIP_CHECK(hipGetLastError());
+    last_stream = s;
+  }
+
+  // RPUPulsed::clipWeights (rpu_pulsed.cpp:263-278), WeightClipper::apply (weight_clipper.cpp:30-106)
+  void clip_weights(int type, float fixed_value, float sigma, hipStream_t s) {
+    check_maintenance("clip_weights");
+    if (type == RPU_CLIP_FIXED_VALUE) {
+      if (dev.pulsed()) launch_clip_value(d_w.p, d_wmin.p, d_wmax.p, fixed_value, nullptr, size(), s);
+      else if (fixed_value >= 0.0f) launch_clip_value(d_w.p, nullptr, nullptr, fixed_value, nullptr, size(), s);
+    } else if (type == RPU_CLIP_NONE) {
+      if (dev.pulsed()) throw RpuError("Sophisticated clipping is NOT implemented for most training devices");
+    } else if (type == RPU_CLIP_LAYER_GAUSSIAN || type == RPU_CLIP_AVERAGE_CHANNEL_MAX) {
+      if (dev.pulsed()) throw RpuError("Sophisticated clipping is NOT implemented for most training devices");
+      s_clip.ensure(1 + (size_t)D);
+      if (type == RPU_CLIP_LAYER_GAUSSIAN) launch_clip_value_gaussian(d_w.p, size(), sigma, fixed_value, s_clip.p, s);
+      else launch_clip_value_channel(d_w.p, X, D, fixed_value, s_clip.p + 1, s_clip.p, s);
+      launch_clip_value(d_w.p, nullptr, nullptr, 0.0f, s_clip.p, size(), s);
+    } else {
+      throw RpuError("Clipping type not implemented.");
+    }
+    RPU_HIP_CHECK(hipGetLastError());
+    last_stream = s;
+  }
+
+  // RPUPulsed::resetCols -> rpu_pulsed_device.cpp:469-494 / rpu_simple_device.cpp:148-168
+  void reset_columns(int start_col, int n_cols, float reset_prob, hipStream_t s) {
+    check_maintenance("reset_columns");
+    if (start_col < 0 || start_col >= X) throw RpuError("start_column_idx out of range.");
+    int n = n_cols >= 0 ? n_cols : X;
+    if (n > X) n = X; // the wrapped range covers every column once
+    if (n == 0) return;
+    if (dev.pulsed()) {
+      ensure_state_params();
+      launch_reset_cols(d_w.p, d_rbias.p, d_wmin.p, d_wmax.p, dev.p.reset_std, start_col, n, reset_prob, X, D, key(),
+                        call++, s);
+    } else {
+      launch_reset_cols(d_w.p, nullptr, nullptr, nullptr, dev.p.reset_std, start_col, n, reset_prob, X, D, key(), call++, s);
+    }
+    RPU_HIP_CHECK(hipGetLastError());
+    last_stream = s;
+  }
+
+  // RPUSimple::setSharedWeights (rpu.cpp:1384-1398): the caller's memory becomes the weight matrix
+  void set_shared_weights(float *w_dev) {
+    check_maintenance("set_shared_weights");
+    if (!w_dev) throw RpuError("Null device pointer.");
+    if (w_dev == d_w.p) return;
+    sync_last();
+    RPU_HIP_CHECK(hipMemcpy(w_dev, d_w.p, size() * sizeof(float), hipMemcpyDeviceToDevice));
+    d_w.adopt(w_dev, size());
+  }
+
+  // RPUSimple::setDeltaWeights (rpu.cpp:1459-1481): null ends the mode
+  void set_delta_weights(float *dw_dev) {
+    if (dw_dev) check_maintenance("set_delta_weights");
+    delta_w = dw_dev;
   }
 
   DeviceView view_of(DeviceSlot &sl, float granularity) {
@@ -869,8 +1010,10 @@ int rpu_tile_set_matrix_indices(rpu_tile_t *tile, const int32_t *indices_host, i
       t.x_idx.release();
     }
     t.idx_host.assign(indices_host, indices_host + (size_t)x_size * patches);
+    t.idx_max = 0;
     for (int32_t j : t.idx_host) {
       if (j < 0) throw RpuError("Negative entry in the index matrix.");
+      t.idx_max = std::max(t.idx_max, j);
     }
     t.idx_patches = patches;
   });
@@ -885,9 +1028,7 @@ int rpu_tile_has_matrix_indices(const rpu_tile_t *tile) { return tile ? tile->t.
     std::lock_guard<std::mutex> lock(t.mutex);                                                 \
     t.check_compute(n_images, x_dev, d_dev);                                                   \
     if (image_size <= 0) throw RpuError("image_size must be positive.");                       \
-    for (int32_t j : t.idx_host) {                                                             \
-      if ((long)j - 2 >= image_size) throw RpuError("Index matrix entry beyond the image size."); \
-    }                                                                                          \
+    if ((long)t.idx_max - 2 >= image_size) throw RpuError("Index matrix entry beyond the image size."); \
     DeviceGuard g(t.device_id);                                                                \
     CALL;                                                                                      \
   })
@@ -908,6 +1049,97 @@ int rpu_tile_update_indexed(rpu_tile_t *tile, const float *x_dev, const float *d
   RPU_INDEXED_ENTRY(update, t.update_indexed(x_dev, d_dev, n_images, image_size, (hipStream_t)stream));
 }
 #undef RPU_INDEXED_ENTRY
+
+// ---- weight maintenance between steps, shared and delta weights, extra state --------------------------
+
+#define RPU_MAINTENANCE_ENTRY(CALL)                                \
+  return guarded([&] {                                             \
+    if (!tile) throw RpuError("null tile");                        \
+    Tile &t = tile->t;                                             \
+    std::lock_guard<std::mutex> lock(t.mutex);                     \
+    if (!t.resident()) {                                           \
+      CALL;                                                        \
+      return;                                                      \
+    }                                                              \
+    DeviceGuard g(t.device_id);                                    \
+    CALL;                                                          \
+  })
+
+int rpu_tile_decay_weights(rpu_tile_t *tile, float alpha, int bias_no_decay, void *stream) {
+  RPU_MAINTENANCE_ENTRY(t.decay_weights(alpha, bias_no_decay != 0, (hipStream_t)stream));
+}
+
+int rpu_tile_diffuse_weights(rpu_tile_t *tile, void *stream) {
+  RPU_MAINTENANCE_ENTRY(t.diffuse_weights((hipStream_t)stream));
+}
+
+int rpu_tile_clip_weights(rpu_tile_t *tile, int clip_type, float fixed_value, float sigma, void *stream) {
+  RPU_MAINTENANCE_ENTRY(t.clip_weights(clip_type, fixed_value, sigma, (hipStream_t)stream));
+}
+
+int rpu_tile_reset_columns(rpu_tile_t *tile, int start_column_idx, int num_columns, float reset_prob, void *stream) {
+  RPU_MAINTENANCE_ENTRY(t.reset_columns(start_column_idx, num_columns, reset_prob, (hipStream_t)stream));
+}
+
+int rpu_tile_set_shared_weights(rpu_tile_t *tile, float *weights_dev) {
+  RPU_MAINTENANCE_ENTRY(t.set_shared_weights(weights_dev));
+}
+
+int rpu_tile_get_shared_weights_if(const rpu_tile_t *tile) { return (tile && !tile->t.d_w.owned) ? 1 : 0; }
+
+int rpu_tile_set_delta_weights(rpu_tile_t *tile, float *delta_weights_dev) {
+  RPU_MAINTENANCE_ENTRY(t.set_delta_weights(delta_weights_dev));
+}
+#undef RPU_MAINTENANCE_ENTRY
+
+// The state beyond weights and device parameters that decides what the next calls compute: the seed and the
+// call counter of the random streams, the update counters and, for a transfer compound, its transfer counters.
+static void extra_fields(const Tile &t, std::vector<std::string> &names, std::vector<int64_t> &values) {
+  names = {"seed", "call", "update_calls", "transfer.update_idx"};
+  values = {(int64_t)t.seed, (int64_t)t.call, (int64_t)t.update_calls, (int64_t)t.update_idx};
+  for (size_t k = 0; k < t.slice_idx.size(); ++k) {
+    names.push_back("transfer.slice_idx_" + std::to_string(k));
+    values.push_back(t.slice_idx[k]);
+  }
+}
+static thread_local std::string g_extra_name;
+
+int rpu_tile_extra_count(const rpu_tile_t *tile) { return tile ? 4 + (int)tile->t.slice_idx.size() : 0; }
+
+const char *rpu_tile_extra_name(const rpu_tile_t *tile, int idx) {
+  if (!tile || idx < 0 || idx >= rpu_tile_extra_count(tile)) return nullptr;
+  std::vector<std::string> names;
+  std::vector<int64_t> values;
+  extra_fields(tile->t, names, values);
+  g_extra_name = names[idx];
+  return g_extra_name.c_str();
+}
+
+int rpu_tile_get_extra(rpu_tile_t *tile, int64_t *values_host) {
+  return guarded([&] {
+    if (!tile || !values_host) throw RpuError("null argument");
+    Tile &t = tile->t;
+    std::lock_guard<std::mutex> lock(t.mutex);
+    std::vector<std::string> names;
+    std::vector<int64_t> values;
+    extra_fields(t, names, values);
+    std::memcpy(values_host, values.data(), values.size() * sizeof(int64_t));
+  });
+}
+
+int rpu_tile_set_extra(rpu_tile_t *tile, const int64_t *values_host, int count) {
+  return guarded([&] {
+    if (!tile || !values_host) throw RpuError("null argument");
+    Tile &t = tile->t;
+    std::lock_guard<std::mutex> lock(t.mutex);
+    if (count != rpu_tile_extra_count(tile)) throw RpuError("Extra state of a different tile layout.");
+    t.seed = (uint64_t)values_host[0];
+    t.call = (uint32_t)values_host[1];
+    t.update_calls = (uint32_t)values_host[2];
+    t.update_idx = (uint64_t)values_host[3];
+    for (size_t k = 0; k < t.slice_idx.size(); ++k) t.slice_idx[k] = (int)values_host[4 + k];
+  });
+}
 
 // ---- grouped forward over several tiles ------------------------------------------------------------
 
@@ -1123,6 +1355,8 @@ int rpu_tile_clone(rpu_tile_t **out, const rpu_tile_t *src_c) {
     t.w_host = s.w_host;
     t.idx_host = s.idx_host;
     t.idx_patches = s.idx_patches;
+    t.idx_max = s.idx_max;
+    t.update_calls = s.update_calls;
     if (s.is_transfer()) {
       t.tr = std::make_unique<TransferPar>(*s.tr);
       t.update_idx = s.update_idx;

@@ -54,6 +54,24 @@ class PulseType(enum.IntEnum):
     DeterministicImplicit = 5
 
 
+class WeightClipType(enum.IntEnum):
+    """src/rpucuda/weight_clipper.h:14-19."""
+
+    NONE = 0
+    FIXED_VALUE = 1
+    LAYER_GAUSSIAN = 2
+    AVERAGE_CHANNEL_MAX = 3
+
+
+class WeightClipParameter:
+    """src/rpucuda/weight_clipper.h:22-27 (``rpu_base.tiles.WeightClipParameter`` in the reference bindings)."""
+
+    def __init__(self, type=WeightClipType.NONE, fixed_value: float = -1.0, sigma: float = 2.5):  # pylint: disable=redefined-builtin
+        self.type = WeightClipType(type)
+        self.fixed_value = float(fixed_value)
+        self.sigma = float(sigma)
+
+
 class AnalogMVType(enum.IntEnum):
     """rpu_base_utils.cpp:87-91."""
 
@@ -377,7 +395,10 @@ class FloatingPointTileParameter(_Struct):
         meta.forward_io.is_perfect = True
         meta.backward_io.is_perfect = True
         meta.update.pulse_type = PulseType.NONE
-        return FloatingPointTile._create(int(x_size), int(d_size), meta._config(IdealResistiveDeviceParameter()))
+        device = IdealResistiveDeviceParameter()
+        device.diffusion = float(self.diffusion)
+        device.lifetime = float(self.lifetime)
+        return FloatingPointTile._create(int(x_size), int(d_size), meta._config(device))
 
 
 __all__ = [name for name, obj in vars(sys.modules[__name__]).items()

@@ -144,6 +144,26 @@ class _TileBase:
         """Seed of the Philox generator behind every random draw of this tile on the GPU."""
         check(lib().rpu_tile_set_seed(self._h, int(seed) & 0xFFFFFFFFFFFFFFFF))
 
+    # -- state beyond weights and hidden parameters (rpu_base_tiles.cpp:89-113)
+    def dump_extra(self) -> dict:
+        count = lib().rpu_tile_extra_count(self._h)
+        values = (C.c_int64 * count)()
+        check(lib().rpu_tile_get_extra(self._h, values))
+        return {"rpu." + lib().rpu_tile_extra_name(self._h, k).decode(): int(values[k]) for k in range(count)}
+
+    def load_extra(self, state: dict, strict: bool) -> None:
+        current = self.dump_extra()
+        for name in current:
+            if name in state:
+                current[name] = int(state[name])
+            elif strict:
+                raise RuntimeError("Cannot find the key: '" + name + "' in state.")
+        values = (C.c_int64 * len(current))(*current.values())
+        check(lib().rpu_tile_set_extra(self._h, values, len(current)))
+
+    def get_shared_weights_if(self) -> bool:
+        return bool(lib().rpu_tile_get_shared_weights_if(self._h))
+
     def get_brief_info(self) -> str:
         where = "gfx950" if lib().rpu_tile_is_on_device(self._h) else "host"
         return f"{type(self).__name__}({self.get_d_size()},{self.get_x_size()}) [{where}]"
@@ -263,6 +283,49 @@ class _CudaTileMixin:
 
     # -- inspection hooks
     # -- indexed (convolution) interface (rpu_base_tiles.cpp:621-737)
+    # -- weight maintenance between steps (rpu_base_tiles.cpp:276-404); the matrix in HBM is changed in place
+    def _current_stream(self):
+        return C.c_void_p(torch.cuda.current_stream(self._device).cuda_stream)
+
+    def decay_weights(self, alpha: float = 1.0) -> None:
+        check(lib().rpu_tile_decay_weights(self._h, float(alpha), 0, self._current_stream()))
+
+    def diffuse_weights(self) -> None:
+        check(lib().rpu_tile_diffuse_weights(self._h, self._current_stream()))
+
+    def clip_weights(self, weight_clipper_params) -> None:
+        par = weight_clipper_params
+        check(lib().rpu_tile_clip_weights(self._h, int(par.type), float(par.fixed_value), float(par.sigma),
+                                          self._current_stream()))
+
+    def reset_columns(self, start_column_idx: int = 0, num_columns: int = 1, reset_prob: float = 1.0) -> None:
+        check(lib().rpu_tile_reset_columns(self._h, int(start_column_idx), int(num_columns), float(reset_prob),
+                                           self._current_stream()))
+
+    # -- shared and delta weights (rpu_base_tiles.cpp:215-251)
+    def _check_matrix(self, tensor: torch.Tensor, what: str) -> torch.Tensor:
+        if isinstance(tensor, torch.Tensor) and not tensor.is_contiguous():
+            raise RuntimeError(what + " must be contiguous")
+        tensor = _check_input(tensor, True, what)
+        if tensor.dim() != 2 or tensor.size(0) != self.get_d_size() or tensor.size(1) != self.get_x_size():
+            raise RuntimeError("Invalid %s dimensions: expected [%d,%d] tensor" % (what, self.get_d_size(), self.get_x_size()))
+        return tensor
+
+    def set_shared_weights(self, weights: torch.Tensor) -> None:
+        """``weights`` (a CUDA tensor) becomes the weight matrix of the tile and must outlive it."""
+        weights = self._check_matrix(weights, "weights")
+        check(lib().rpu_tile_set_shared_weights(self._h, weights.data_ptr()))
+        self._shared_weights = weights
+
+    def set_delta_weights(self, delta_weights: torch.Tensor) -> None:
+        delta_weights = self._check_matrix(delta_weights, "delta weights")
+        check(lib().rpu_tile_set_delta_weights(self._h, delta_weights.data_ptr()))
+        self._delta_weights = delta_weights
+
+    def reset_delta_weights(self) -> None:
+        check(lib().rpu_tile_set_delta_weights(self._h, None))
+        self._delta_weights = None
+
     def _patches(self) -> int:
         patches = lib().rpu_tile_has_matrix_indices(self._h)
         if patches <= 0:

@@ -399,6 +399,56 @@ int rpu_tile_get_drift_state(rpu_tile_t *tile, float *programmed_host, float *nu
  * value after programming to the value after drift is the output scale alpha. */
 int rpu_tile_drift_readout(rpu_tile_t *tile, float *mean_abs_host, void *stream);
 
+/* ---- weight maintenance between training steps ------------------------------------------- */
+/* All of these work on the matrix in HBM of a resident tile, on `stream`; a transfer compound refuses them. */
+
+/* decay_weights (src/aihwkit/simulator/rpu_base_src/rpu_base_tiles.cpp:276-291): a pulsed device decays each
+ * weight towards its reset bias with its own decay scale and clips to its bounds,
+ * w = (w - b) * (1 + alpha * (scale - 1)) + b   (src/rpucuda/rpu_pulsed_device.cpp:392-420);
+ * other tiles scale by 1 - alpha / lifetime (src/rpucuda/rpu_simple_device.cpp:96-115).  bias_no_decay
+ * leaves the last column alone. */
+int rpu_tile_decay_weights(rpu_tile_t *tile, float alpha, int bias_no_decay, void *stream);
+
+/* diffuse_weights (rpu_base_tiles.cpp:372-386): w += diffusion_rate * N(0, 1), then the bounds
+ * (rpu_pulsed_device.cpp:432-446, rpu_simple_device.cpp:124-134). */
+int rpu_tile_diffuse_weights(rpu_tile_t *tile, void *stream);
+
+/* clip_weights (rpu_base_tiles.cpp:315-329) with the fields of WeightClipParameter
+ * (src/rpucuda/weight_clipper.h:14-27).  Fixed value: +- fixed_value and, on a pulsed device, its bounds
+ * (rpu_pulsed_device.cpp:448-467).  Layer Gaussian and average channel max (weight_clipper.cpp:38-93) are for
+ * floating-point / ideal devices only, as in the reference (src/rpucuda/rpu_pulsed.cpp:269-278). */
+enum rpu_clip_type {
+  RPU_CLIP_NONE = 0,
+  RPU_CLIP_FIXED_VALUE = 1,
+  RPU_CLIP_LAYER_GAUSSIAN = 2,
+  RPU_CLIP_AVERAGE_CHANNEL_MAX = 3
+};
+int rpu_tile_clip_weights(rpu_tile_t *tile, int clip_type, float fixed_value, float sigma, void *stream);
+
+/* reset_columns (rpu_base_tiles.cpp:387-404): columns start .. start + num - 1 (wrapping; num < 0: all) are set
+ * to reset_bias + reset_std * N(0, 1) and clipped, each element with probability reset_prob
+ * (rpu_pulsed_device.cpp:469-494; without bias and bounds on other tiles, rpu_simple_device.cpp:148-168). */
+int rpu_tile_reset_columns(rpu_tile_t *tile, int start_column_idx, int num_columns, float reset_prob, void *stream);
+
+/* set_shared_weights (rpu_base_tiles.cpp:215-229, src/rpucuda/rpu.cpp:1384-1398): the tile's weights are copied
+ * into the caller's device buffer [d_size][x_size], which is the weight matrix from then on (never freed by
+ * the library; it must outlive the tile or its move off the GPU). */
+int rpu_tile_set_shared_weights(rpu_tile_t *tile, float *weights_dev);
+int rpu_tile_get_shared_weights_if(const rpu_tile_t *tile);
+
+/* set_delta_weights / reset_delta_weights (rpu_base_tiles.cpp:230-251): while a device buffer [d_size][x_size]
+ * is set, an update leaves the weights as they are and writes dW with W_new = W - lr * dW into the buffer
+ * (rpu.cpp:1459-1510, rpu_pulsed.cpp:560-585); null ends the mode. */
+int rpu_tile_set_delta_weights(rpu_tile_t *tile, float *delta_weights_dev);
+
+/* dump_extra / load_extra (rpu_base_tiles.cpp:89-113): the state beyond weights and hidden parameters that
+ * decides what the next calls compute, as named 64-bit integers: seed and call counter of the random streams,
+ * update counter, transfer counters of a compound. */
+int rpu_tile_extra_count(const rpu_tile_t *tile);
+const char *rpu_tile_extra_name(const rpu_tile_t *tile, int idx);
+int rpu_tile_get_extra(rpu_tile_t *tile, int64_t *values_host);
+int rpu_tile_set_extra(rpu_tile_t *tile, const int64_t *values_host, int count);
+
 /* ---- inspection hooks (mirror the reference's debug hooks) ------------------------------ */
 
 /* After rpu_tile_update with a stochastic pulse type: copies the packed pulse words of that call

@@ -1,0 +1,237 @@
+"""GPU parity of the weight maintenance between steps (decay, diffusion, clipping, column reset), of shared and
+delta weights and of the extra state, against the numpy restatement and against the tile's own update path."""
+import numpy as np
+import pytest
+import torch
+
+import state_oracle as so
+from aihwkit_amd.rpu_base import devices as dv
+from aihwkit_amd.rpu_base import tiles
+from helpers import make_meta, noise_free_io, soft_bounds
+
+pytestmark = pytest.mark.gpu
+F = np.float32
+
+
+def hidden(tile):
+    names = tile.get_hidden_parameter_names()
+    values = tile.get_hidden_parameters().numpy()
+    return {name: values[k] for k, name in enumerate(names)}
+
+
+def pulsed_tile(x_size=37, d_size=23, **device):
+    meta = make_meta(noise_free_io(), noise_free_io(), pulse_type=dv.PulseType.StochasticCompressed, desired_bl=31)
+    dev = soft_bounds(construction_seed=5, **device)
+    host = meta.create_array(x_size, d_size, dev)
+    rng = np.random.default_rng(0)
+    host.set_weights(torch.from_numpy(rng.uniform(-0.5, 0.5, (d_size, x_size)).astype(F)))
+    return tiles.CudaAnalogTile(host)
+
+
+def fp_tile(x_size=37, d_size=23, scale=0.3, **par):
+    meta = dv.FloatingPointTileParameter()
+    for name, value in par.items():
+        setattr(meta, name, value)
+    host = meta.create_array(x_size, d_size)
+    rng = np.random.default_rng(0)
+    host.set_weights(torch.from_numpy(rng.normal(0.01, scale, (d_size, x_size)).astype(F)))
+    return tiles.CudaFloatingPointTile(host)
+
+
+def test_decay_of_a_pulsed_device(gpu_device):
+    tile = pulsed_tile(lifetime=50.0, lifetime_dtod=0.2, reset=0.02, reset_dtod=0.5)
+    par = hidden(tile)
+    assert par["decay_scales"].std() > 1e-4 and par["reset_bias"].std() > 1e-3
+    w = tile.get_weights().numpy()
+    for alpha in (1.0, 0.3):
+        tile.decay_weights(alpha)
+        w = so.decay_device(w, par["decay_scales"], par["reset_bias"], par["min_bound"], par["max_bound"], alpha)
+        assert np.abs(tile.get_weights().numpy() - w).max() <= 1e-6
+    assert np.abs(w - tile.get_weights().numpy()).max() <= 1e-6
+
+
+def test_decay_of_a_floating_point_tile(gpu_device):
+    tile = fp_tile(lifetime=20.0)
+    w = tile.get_weights().numpy()
+    tile.decay_weights(2.0)
+    assert np.abs(tile.get_weights().numpy() - so.decay_simple(w, 20.0, 2.0)).max() <= 1e-7
+    still = fp_tile()                                    # no lifetime: nothing happens
+    w = still.get_weights().numpy()
+    still.decay_weights()
+    assert np.array_equal(still.get_weights().numpy(), w)
+
+
+def test_diffusion_statistics_and_replay(gpu_device):
+    tile = pulsed_tile(x_size=512, d_size=256, diffusion=0.004, diffusion_dtod=0.3, w_max=2.0, w_min=-2.0)
+    par = hidden(tile)
+    w0 = tile.get_weights().numpy()
+    tile.set_seed(11)
+    tile.diffuse_weights()
+    w1 = tile.get_weights().numpy()
+    z = (w1 - w0) / par["diffusion_rates"]
+    n = z.size
+    assert abs(z.mean()) < 4 / np.sqrt(n) and abs(z.var() - 1) < 4 * np.sqrt(2 / n) + 1e-3    # fp32 rounding of w1 - w0
+    assert abs((z ** 4).mean() - 3) < 0.1
+    tile.diffuse_weights()                                # the next call draws new numbers
+    z2 = (tile.get_weights().numpy() - w1) / par["diffusion_rates"]
+    assert abs(np.corrcoef(z.ravel(), z2.ravel())[0, 1]) < 0.01
+    tile.set_weights(torch.from_numpy(w0))                # the same seed replays the same draws
+    tile.set_seed(11)
+    tile.diffuse_weights()
+    assert np.array_equal(tile.get_weights().numpy(), w1)
+    # bounds hold: a device with tight bounds stays inside
+    tight = pulsed_tile(diffusion=0.5)
+    tight.diffuse_weights()
+    tp = hidden(tight)
+    wt = tight.get_weights().numpy()
+    assert (wt <= tp["max_bound"]).all() and (wt >= tp["min_bound"]).all()
+    assert ((wt == tp["max_bound"]) | (wt == tp["min_bound"])).mean() > 0.2
+    # floating point tile: one rate, no bounds
+    fp = fp_tile(x_size=300, d_size=200, diffusion=0.05)
+    w0 = fp.get_weights().numpy()
+    fp.diffuse_weights()
+    z = (fp.get_weights().numpy() - w0) / 0.05
+    assert abs(z.mean()) < 0.02 and abs(z.std() - 1) < 0.02
+
+
+def test_clip_weights(gpu_device):
+    tile = pulsed_tile()
+    par = hidden(tile)
+    w = tile.get_weights().numpy()
+    tile.clip_weights(dv.WeightClipParameter(dv.WeightClipType.FIXED_VALUE, fixed_value=0.2))
+    assert np.array_equal(tile.get_weights().numpy(), so.clip_fixed(w, 0.2, par["min_bound"], par["max_bound"]))
+    with pytest.raises(RuntimeError):
+        tile.clip_weights(dv.WeightClipParameter(dv.WeightClipType.LAYER_GAUSSIAN))
+    for clip_type, value in ((dv.WeightClipType.LAYER_GAUSSIAN, lambda w: so.clip_value_layer_gaussian(w, 1.5)),
+                             (dv.WeightClipType.AVERAGE_CHANNEL_MAX, so.clip_value_average_channel_max),
+                             (dv.WeightClipType.FIXED_VALUE, lambda w: 0.25)):
+        fp = fp_tile(x_size=130, d_size=70)
+        w = fp.get_weights().numpy()
+        fp.clip_weights(dv.WeightClipParameter(clip_type, fixed_value=0.25 if clip_type == dv.WeightClipType.FIXED_VALUE
+                                               else -1.0, sigma=1.5))
+        want = so.clip_with_value(w, value(w))
+        got = fp.get_weights().numpy()
+        assert np.abs(got - want).max() <= 1e-6 and (got != w).mean() > 0.003, clip_type
+    fp = fp_tile()
+    w = fp.get_weights().numpy()
+    fp.clip_weights(dv.WeightClipParameter(dv.WeightClipType.LAYER_GAUSSIAN, fixed_value=0.1, sigma=2.5))
+    assert np.array_equal(fp.get_weights().numpy(), np.clip(w, -0.1, 0.1))       # the fixed value caps the clip value
+    fp.clip_weights(dv.WeightClipParameter())                                     # type None: unchanged
+    assert np.array_equal(fp.get_weights().numpy(), np.clip(w, -0.1, 0.1))
+
+
+def test_reset_columns(gpu_device):
+    tile = pulsed_tile(x_size=40, d_size=300, reset=0.05, reset_dtod=0.4, reset_std=0.02, w_max=2.0, w_min=-2.0)
+    par = hidden(tile)
+    w0 = tile.get_weights().numpy()
+    tile.reset_columns(36, 7, 1.0)                        # columns 36 .. 39 and 0 .. 2
+    w1 = tile.get_weights().numpy()
+    cols = so.reset_column_mask(40, 36, 7)
+    assert cols.sum() == 7 and np.array_equal(w1[:, ~cols], w0[:, ~cols])
+    # away from the device bounds the new value is the bias plus N(0, reset_std); at a bound it is the bound
+    inside = (par["reset_bias"] + 0.1 < par["max_bound"]) & (par["reset_bias"] - 0.1 > par["min_bound"])
+    assert inside.mean() > 0.9 and (w1 <= par["max_bound"]).all() and (w1 >= par["min_bound"]).all()
+    z = ((w1 - par["reset_bias"]) / 0.02)[:, cols][inside[:, cols]]
+    assert abs(z.mean()) < 4 / np.sqrt(z.size) and abs(z.std() - 1) < 0.06
+    tile.reset_columns(0, -1, 0.3)                        # every column, 30 % of the elements
+    w2 = tile.get_weights().numpy()
+    changed = w2 != w1
+    assert abs(changed.mean() - 0.3) < 0.02
+    z = ((w2 - par["reset_bias"]) / 0.02)[changed & inside]
+    assert abs(z.mean()) < 0.05 and abs(z.std() - 1) < 0.05
+    with pytest.raises(RuntimeError):
+        tile.reset_columns(40, 1, 1.0)
+    # no noise: exactly the (clipped) reset bias; floating point tile: zero
+    exact = pulsed_tile(reset=0.3, reset_dtod=1.0, reset_std=0.0)
+    ep = hidden(exact)
+    exact.reset_columns(3, 2, 1.0)
+    want = np.clip(ep["reset_bias"], ep["min_bound"], ep["max_bound"])
+    assert np.array_equal(exact.get_weights().numpy()[:, 3:5], want[:, 3:5])
+    assert (want != ep["reset_bias"]).any()
+    fp = fp_tile()
+    fp.reset_columns(1, 3, 1.0)
+    got = fp.get_weights().numpy()
+    assert np.abs(got[:, 1:4]).max() < 0.06 and abs(got[:, 1:4].std() - 0.01) < 0.002     # reset_std 0.01, no bias
+
+
+def test_shared_weights(gpu_device):
+    tile = pulsed_tile()
+    w = tile.get_weights()
+    shared = torch.zeros(23, 37, device="cuda")
+    assert not tile.get_shared_weights_if()
+    tile.set_shared_weights(shared)
+    assert tile.get_shared_weights_if()
+    assert torch.equal(shared.cpu(), w)                   # the tile's weights moved into the tensor
+    rng = np.random.default_rng(3)
+    x = torch.from_numpy(rng.uniform(-1, 1, (8, 37)).astype(F)).cuda()
+    d = torch.from_numpy(rng.normal(0, 0.3, (8, 23)).astype(F)).cuda()
+    tile.set_learning_rate(0.1)
+    tile.update(x, d, False)
+    assert not torch.equal(shared.cpu(), w)               # the update wrote into the tensor
+    assert torch.equal(shared.cpu(), tile.get_weights())
+    shared.mul_(0.5)                                       # and the tile computes with what the tensor holds
+    y = tile.forward(x, False, False, False, True)
+    assert torch.allclose(y, x @ shared.t(), atol=0.06)   # DAC / ADC steps of the analog forward
+    assert (y - 2.0 * (x @ shared.t())).abs().max() > 0.3
+    with pytest.raises(RuntimeError):
+        tile.set_shared_weights(torch.zeros(37, 23, device="cuda"))
+    with pytest.raises(RuntimeError):
+        tile.set_shared_weights(torch.zeros(23, 37))
+
+
+def test_delta_weights(gpu_device):
+    rng = np.random.default_rng(4)
+    x = torch.from_numpy(rng.uniform(-1, 1, (16, 37)).astype(F)).cuda()
+    d = torch.from_numpy(rng.normal(0, 0.3, (16, 23)).astype(F)).cuda()
+    # floating point tile: the buffer receives d^T x, the weights stay
+    fp = fp_tile()
+    fp.set_learning_rate(0.1)
+    w0 = fp.get_weights()
+    delta = torch.full((23, 37), 7.0, device="cuda")
+    fp.set_delta_weights(delta)
+    fp.update(x, d, False)
+    assert torch.equal(fp.get_weights(), w0)
+    assert torch.allclose(delta, d.t() @ x, atol=1e-4)
+    fp.reset_delta_weights()
+    fp.update(x, d, False)
+    assert torch.allclose(fp.get_weights(), w0 - 0.1 * (d.t() @ x).cpu(), atol=1e-5)
+    # pulsed tile: W - lr * delta is what the same update writes on a twin with the same random streams
+    tile, twin = pulsed_tile(), pulsed_tile()
+    for t in (tile, twin):
+        t.set_learning_rate(0.05)
+        t.set_seed(9)
+    w0 = tile.get_weights()
+    delta = torch.zeros(23, 37, device="cuda")
+    tile.set_delta_weights(delta)
+    tile.update(x, d, False)
+    twin.update(x, d, False)
+    assert torch.equal(tile.get_weights(), w0)
+    assert (twin.get_weights() - w0).abs().max() > 1e-3
+    assert torch.allclose(w0 - 0.05 * delta.cpu(), twin.get_weights(), atol=1e-6)
+
+
+def test_extra_state_replays_the_random_streams(gpu_device):
+    rng = np.random.default_rng(5)
+    x = torch.from_numpy(rng.uniform(-1, 1, (16, 37)).astype(F)).cuda()
+    d = torch.from_numpy(rng.normal(0, 0.3, (16, 23)).astype(F)).cuda()
+    tile = pulsed_tile()
+    tile.set_learning_rate(0.05)
+    tile.set_seed(21)
+    tile.update(x, d, False)
+    state = tile.dump_extra()
+    assert state["rpu.seed"] == 21 and state["rpu.call"] > 0
+    w_mid = tile.get_weights()
+    tile.update(x, d, False)
+    w_end = tile.get_weights()
+    other = pulsed_tile()
+    other.set_learning_rate(0.05)
+    other.set_weights(w_mid)
+    other.load_extra(state, True)
+    other.update(x, d, False)
+    assert torch.equal(other.get_weights(), w_end)
+    with pytest.raises(RuntimeError):
+        other.load_extra({"rpu.seed": 1}, True)
+    before = other.dump_extra()
+    other.load_extra({"rpu.seed": 1}, False)                # not strict: the keys that are missing keep their values
+    after = other.dump_extra()
+    assert after["rpu.seed"] == 1 and after["rpu.call"] == before["rpu.call"]
