@@ -81,25 +81,26 @@ constexpr int LDS_ROW = KSTEP + 4; // floats per staged row: 16-byte aligned, co
 // workgroup number n -> (output tile, sample tile).  With 8 or more output tiles workgroup n runs on XCD n % 8 and
 // XCD x owns the output-row tiles [x * per, (x + 1) * per): each L2 holds a band of W.  A matrix of fewer output
 // tiles fits every L2, and consecutive workgroups (hence all XCDs) simply walk the tiles in order.
+template <int EDGE = 32>
 __device__ __forceinline__ bool tile_of(const MvmArgs &a, int n, int n_act, int &tile_o, int &tile_b) {
-  const int tiles_o = (a.O + TILE - 1) / TILE;
+  const int tiles_o = (a.O + EDGE - 1) / EDGE;
   if (tiles_o < 8) {
     tile_o = n % tiles_o;
     tile_b = n / tiles_o;
-    return tile_b * TILE < n_act;
+    return tile_b * EDGE < n_act;
   }
   const int per = (tiles_o + 7) / 8;
   const int xcd = n & 7;
   const int m = n >> 3;
   tile_o = xcd * per + (m % per);
   tile_b = m / per;
-  return tile_o < tiles_o && tile_b * TILE < n_act;
+  return tile_o < tiles_o && tile_b * EDGE < n_act;
 }
 
-// workgroups that cover n_act samples (a multiple of 8)
-__host__ __device__ __forceinline__ int workgroups_for(int O, int n_act) {
-  const int tiles_o = (O + TILE - 1) / TILE;
-  const int tiles_b = (n_act + TILE - 1) / TILE;
+// workgroups that cover n_act samples with tiles of edge x edge (a multiple of 8)
+__host__ __device__ __forceinline__ int workgroups_for(int O, int n_act, int edge = 32) {
+  const int tiles_o = (O + edge - 1) / edge;
+  const int tiles_b = (n_act + edge - 1) / edge;
   if (tiles_o < 8) return (tiles_o * tiles_b + 7) & ~7;
   return 8 * ((tiles_o + 7) / 8) * tiles_b;
 }
@@ -679,10 +680,11 @@ __device__ __forceinline__ void mvm_prepare_next_rows(const MvmArgs &a, int roun
 
 // After round `round`, for sample b at position `slot` of that round's list: a sample whose ADC saturated
 // gets another round unless the reduction limit is reached (rpu_forward_backward_pass.cpp:944-983); its
-// quantized row for that round was written by mvm_prepare_next_rows, or (a.speculate == 0) is written by the
-// caller into row `pos` of the other scratch matrix.  One thread per sample; returns the sample's position in
+// quantized row for that round was written ahead at the row of its list position (rows_ahead), or is written by
+// the caller into row `pos` of the other scratch matrix.  One thread per sample; returns the sample's position in
 // the next round's list, -1 when it has no further round.
-__device__ __forceinline__ int mvm_advance_sample(const MvmArgs &a, int round, int b, int slot, float &scale) {
+__device__ __forceinline__ int mvm_advance_sample(const MvmArgs &a, int round, int b, int slot, bool rows_ahead,
+                                                  float &scale) {
   const IoDev &io = a.io;
   // the flags were raised with device-scope atomics by workgroups on any XCD: read and clear them the same way
   const int up = atomicExch(&a.st.hit_up[b], 0);
@@ -699,7 +701,7 @@ __device__ __forceinline__ int mvm_advance_sample(const MvmArgs &a, int round, i
   scale = set_round_scales(a, b, nm, red);
   const int pos = atomicAdd(&a.st.count[round + 1], 1);
   a.st.list[(round + 1) & 1][pos] = b;
-  a.st.row[(round + 1) & 1][pos] = a.speculate ? slot : pos;
+  a.st.row[(round + 1) & 1][pos] = rows_ahead ? slot : pos;
   a.st.next_scale[(round + 1) & 1][pos] = next_round_scale(a, round + 1, b, a.st.fin[b], nm, red);
   return pos;
 }
@@ -728,7 +730,7 @@ __device__ __forceinline__ void mvm_tile_finished(const MvmArgs &a, int round, i
     if (slot < n_act) {
       const int b = (round > 0) ? a.st.list[round & 1][slot] : slot;
       float scale = 0.0f;
-      const int pos = mvm_advance_sample(a, round, b, slot, scale);
+      const int pos = mvm_advance_sample(a, round, b, slot, a.speculate != 0, scale);
       if (pos >= 0 && !a.speculate) {
         const int i = atomicAdd(&sh_more, 1);
         sh_more_b[i] = b;
@@ -763,7 +765,278 @@ __global__ __launch_bounds__(256) void k_mvm_round(MvmArgs a) {
   __shared__ float red[WAVES][16][64];
   __shared__ __attribute__((aligned(16))) float stage[WAVES * 2 * TILE * LDS_ROW];
   const int n_act = (a.round > 0) ? a.st.count[a.round] : a.m_batch;
+  if (a.big_from > 0 && n_act >= a.big_from) return; // this round is run by k_mvm_big
   mvm_round_workgroup<PD, WMODE>(a, a.round, blockIdx.x, n_act, red, stage);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Large-batch round: one workgroup (4 waves as 2 x 2) owns 128 outputs x 128 samples, each wave a 64 x 64 block as
+// 2 x 2 MFMA tiles.  Both operands go through LDS stages of 32 k-values shared by the four waves (a stage is
+// fetched into registers while the previous one is multiplied, then written to the other LDS buffer: one barrier
+// per stage), so a byte fetched from L2 feeds 64 multiply-adds instead of 16 and the matrix pipe, not the memory
+// path, sets the pace.  Same per-sample state, lists, epilogue and random streams as the 32 x 32 kernel: a round
+// may be run by either (the launcher picks by the number of samples in the round).
+// WT = 0: weights contiguous along k (forward), 1: contiguous along the outputs (backward, W read in place).
+
+constexpr int BT = 128;        // tile edge
+constexpr int BKS = 32;        // k-values per stage
+constexpr int BPITCH = 36;     // floats per staged row of a k-contiguous operand
+constexpr int BPITCH_T = 132;  // floats per staged k-row of an output-contiguous weight tile
+
+__device__ __forceinline__ void big_prepare_next_rows(const MvmArgs &a, int round, int tile_o, int tile_b, int n_act,
+                                                      int *sh_b, float *sh_scale) {
+  if (threadIdx.x < BT) {
+    const int slot = tile_b * BT + threadIdx.x;
+    int b = 0;
+    float scale = 0.0f;
+    if (slot < n_act) {
+      b = (round > 0) ? a.st.list[round & 1][slot] : slot;
+      scale = a.st.next_scale[round & 1][slot];
+    }
+    sh_b[threadIdx.x] = b;
+    sh_scale[threadIdx.x] = scale;
+  }
+  __syncthreads();
+  const int tiles_o = (a.O + BT - 1) / BT;
+  const int chunk = (((a.k_pad + tiles_o - 1) / tiles_o) + 31) & ~31;
+  const int k_lo = tile_o * chunk;
+  const int k_hi = min(k_lo + chunk, a.k_pad);
+  float *__restrict__ dst = a.xq[(round + 1) & 1];
+  const float *__restrict__ in = a.in;
+  const int kq = threadIdx.x & 31, rq = threadIdx.x >> 5; // 8 thread-rows, 16 rows each, 4 at a time
+  for (int k0 = k_lo; k0 < k_hi; k0 += 32) {
+    const int k = k0 + kq;
+    for (int jb = 0; jb < 4; ++jb) {
+      float xv[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int row = rq * 16 + jb * 4 + i;
+        xv[i] = (sh_scale[row] != 0.0f && k < a.K) ? in[(long)sh_b[row] * a.in_sb + (long)k * a.in_sk] : 0.0f;
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int row = rq * 16 + jb * 4 + i;
+        const float sc = sh_scale[row];
+        if (sc != 0.0f) {
+          const float v = (k < a.K) ? dac_value(xv[i], sc, a.io, a.key, a.call, round + 1, sh_b[row], k) : 0.0f;
+          dst[(long)(tile_b * BT + row) * a.k_pad + k] = v;
+        }
+      }
+    }
+  }
+}
+
+template <int WT>
+__global__ __launch_bounds__(256, 2) void k_mvm_big(MvmArgs a, int min_active) {
+  __shared__ __attribute__((aligned(16))) float lds_x[2][BT * BPITCH];
+  __shared__ __attribute__((aligned(16))) float lds_w[2][WT ? BKS * BPITCH_T : BT * BPITCH];
+  __shared__ int sh_hits[2 * BT];
+  __shared__ int sh_b[BT];
+  __shared__ float sh_scale[BT];
+  __shared__ int sh_last;
+
+  const int round = a.round;
+  const int n_act = (round > 0) ? a.st.count[round] : a.m_batch;
+  if (n_act < min_active) return; // this round is run by the 32 x 32 kernel
+  int tile_o, tile_b;
+  if (!tile_of<BT>(a, blockIdx.x, n_act, tile_o, tile_b)) return;
+  const bool more_rounds = round + 1 < a.max_rounds;
+  if (more_rounds) big_prepare_next_rows(a, round, tile_o, tile_b, n_act, sh_b, sh_scale);
+
+  const int t = threadIdx.x;
+  const int lane = t & 63, wave = t >> 6;
+  const int r = lane & 31, h = lane >> 5;
+  const int wy = wave >> 1, wx = wave & 1;
+  const int K = a.K;
+
+  // global -> LDS assignment.  k-contiguous operand: chunk c = t + 256 j covers row c / 8, floats 4 (c % 8) ..;
+  // output-contiguous weights: chunk c covers k-row c / 32, outputs 4 (c % 32) ..
+  const float *xq = a.xq[round & 1];
+  const float *x_src[4];
+  const float *w_src[4];
+  const int st_col = (t & 7) * 4;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int row = (t >> 3) + 32 * j;
+    const int slot = min(tile_b * BT + row, n_act - 1);
+    const int xrow = (round > 0) ? a.st.row[round & 1][slot] : slot;
+    x_src[j] = xq + (long)xrow * a.k_pad + st_col;
+    if (WT == 0) w_src[j] = a.w + (long)min(tile_o * BT + row, a.O - 1) * a.x_size;
+  }
+  const int wt_o = tile_o * BT + (t & 31) * 4; // WT = 1: first of this thread's four outputs
+
+  auto gload = [&](int s, f32x4 (&gx)[4], f32x4 (&gw)[4]) {
+    const int k0 = s * BKS;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) gx[j] = *reinterpret_cast<const f32x4 *>(x_src[j] + k0);
+    if (WT == 0) {
+      const int kc = k0 + st_col;
+      if (kc + 4 <= K) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) gw[j] = *reinterpret_cast<const f32x4_unaligned *>(w_src[j] + kc);
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          f32x4 z;
+          z.x = (kc < K) ? w_src[j][kc] : 0.0f;
+          z.y = (kc + 1 < K) ? w_src[j][kc + 1] : 0.0f;
+          z.z = (kc + 2 < K) ? w_src[j][kc + 2] : 0.0f;
+          z.w = 0.0f;
+          gw[j] = z;
+        }
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int k = min(k0 + (t >> 5) + 8 * j, K - 1); // rows past K meet the zero padding of the inputs
+        const float *row = a.w + (long)k * a.x_size;
+        if (wt_o + 4 <= a.O) {
+          gw[j] = *reinterpret_cast<const f32x4_unaligned *>(row + wt_o);
+        } else {
+          f32x4 z;
+          z.x = (wt_o < a.O) ? row[wt_o] : 0.0f;
+          z.y = (wt_o + 1 < a.O) ? row[wt_o + 1] : 0.0f;
+          z.z = (wt_o + 2 < a.O) ? row[wt_o + 2] : 0.0f;
+          z.w = 0.0f;
+          gw[j] = z;
+        }
+      }
+    }
+  };
+  auto lds_store = [&](int buf, const f32x4 (&gx)[4], const f32x4 (&gw)[4]) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int row = (t >> 3) + 32 * j;
+      *reinterpret_cast<f32x4 *>(&lds_x[buf][row * BPITCH + st_col]) = gx[j];
+      if (WT == 0) {
+        *reinterpret_cast<f32x4 *>(&lds_w[buf][row * BPITCH + st_col]) = gw[j];
+      } else {
+        const int krow = (t >> 5) + 8 * j;
+        *reinterpret_cast<f32x4 *>(&lds_w[buf][krow * BPITCH_T + (t & 31) * 4]) = gw[j];
+      }
+    }
+  };
+
+  floatx16 acc[2][2];
+#pragma unroll
+  for (int oi = 0; oi < 2; ++oi)
+#pragma unroll
+    for (int bi = 0; bi < 2; ++bi)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[oi][bi][i] = 0.0f;
+
+  // lane (r, h) multiplies k = 16 h .. 16 h + 15 of a stage, four values at a time
+  auto compute = [&](int buf) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      f32x4 wa[2], xb[2];
+      const int kk = h * 16 + q * 4;
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        xb[i] = *reinterpret_cast<const f32x4 *>(&lds_x[buf][(wx * 64 + i * 32 + r) * BPITCH + kk]);
+        if (WT == 0) {
+          wa[i] = *reinterpret_cast<const f32x4 *>(&lds_w[buf][(wy * 64 + i * 32 + r) * BPITCH + kk]);
+        } else {
+          const float *col = &lds_w[buf][kk * BPITCH_T + wy * 64 + i * 32 + r];
+          wa[i].x = col[0];
+          wa[i].y = col[BPITCH_T];
+          wa[i].z = col[2 * BPITCH_T];
+          wa[i].w = col[3 * BPITCH_T];
+        }
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+#pragma unroll
+        for (int oi = 0; oi < 2; ++oi)
+#pragma unroll
+          for (int bi = 0; bi < 2; ++bi)
+            acc[oi][bi] = __builtin_amdgcn_mfma_f32_32x32x2f32(wa[oi][e], xb[bi][e], acc[oi][bi], 0, 0, 0);
+      }
+    }
+  };
+
+  const int stages = a.k_pad / BKS;
+  {
+    f32x4 gx[4], gw[4];
+    gload(0, gx, gw);
+    lds_store(0, gx, gw);
+    __syncthreads();
+    for (int s = 0; s < stages; ++s) {
+      const bool next = s + 1 < stages;
+      if (next) gload(s + 1, gx, gw);
+      compute(s & 1);
+      if (next) lds_store((s + 1) & 1, gx, gw);
+      __syncthreads();
+    }
+  }
+
+  // ADC stage: lane (r, h) of wave (wy, wx) holds, for its 2 x 2 tiles, sample column r and output rows
+  // g * 8 + h * 4 + q of each tile
+  if (t < 2 * BT) sh_hits[t] = 0;
+  __syncthreads();
+  const bool flags = !a.io.perfect && a.io.bound_management != RPU_BM_NONE;
+#pragma unroll
+  for (int bi = 0; bi < 2; ++bi) {
+    const int local_b = wx * 64 + bi * 32 + r;
+    const int slot = tile_b * BT + local_b;
+    if (slot >= n_act) continue;
+    int b_out = slot;
+    float fin_out = 1.0f;
+    if (!a.io.perfect) {
+      if (round > 0) b_out = a.st.list[round & 1][slot];
+      fin_out = a.st.fin[b_out];
+    }
+    int up_max = 0, lo_max = 0;
+#pragma unroll
+    for (int oi = 0; oi < 2; ++oi) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int o0 = tile_o * BT + wy * 64 + oi * 32 + g * 8 + h * 4;
+        if (o0 >= a.O) continue;
+        float v[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) v[q] = acc[oi][bi][4 * g + q];
+        int up, lo;
+        mvm_finish_outputs(a, round, b_out, fin_out, o0, v, up, lo);
+        up_max = max(up_max, up);
+        lo_max = max(lo_max, lo);
+      }
+    }
+    if (flags) {
+      if (up_max) atomicMax(&sh_hits[local_b], up_max);
+      if (lo_max) atomicMax(&sh_hits[BT + local_b], lo_max);
+    }
+  }
+  if (!flags) return;
+  __syncthreads();
+  {
+    const int local_b = t & (BT - 1);
+    const int hit = sh_hits[t];
+    const int slot = tile_b * BT + local_b;
+    if (hit && slot < n_act) {
+      const int bs = (round > 0) ? a.st.list[round & 1][slot] : slot;
+      const int old = atomicMax(t < BT ? &a.st.hit_up[bs] : &a.st.hit_lo[bs], hit);
+      asm volatile("" ::"v"(old));
+    }
+  }
+  if (!more_rounds) return;
+  // the last workgroup of this sample tile decides which of its samples go on (see mvm_tile_finished)
+  __syncthreads();
+  if (t == 0) {
+    const int tiles_o = (a.O + BT - 1) / BT;
+    const int tiles_b = (a.m_batch + BT - 1) / BT;
+    const int prev = atomicAdd(&a.st.tile_done[round * tiles_b + tile_b], 1);
+    sh_last = (prev == tiles_o - 1) ? 1 : 0;
+  }
+  __syncthreads();
+  if (!sh_last) return;
+  if (t < BT) {
+    const int slot = tile_b * BT + t;
+    if (slot < n_act) {
+      float scale;
+      mvm_advance_sample(a, round, (round > 0) ? a.st.list[round & 1][slot] : slot, slot, true, scale);
+    }
+  }
 }
 
 // The same for several tiles in one launch: a workgroup finds its tile in the table of first workgroup numbers
@@ -886,7 +1159,24 @@ void launch_mvm_round_group(const MvmGroup &g, int depth, int mode, int total_wo
 #undef RPU_LAUNCH_ROUND
 }
 
-void launch_mvm_round(const MvmArgs &a, hipStream_t s) {
+// samples of a round from which the large-tile kernel takes over, 0 when this call never uses it: it needs
+// outputs for a whole 128-wide tile and enough tiles to fill half the chip
+static int big_threshold(const MvmArgs &a) {
+  if (a.m_batch < 2048 || a.O < 128) return 0;
+  if (workgroups_for(a.O, a.m_batch, 128) < 128) return 0;
+  return 2048;
+}
+
+void launch_mvm_round(const MvmArgs &a_in, hipStream_t s) {
+  MvmArgs a = a_in;
+  a.big_from = big_threshold(a);
+  if (a.big_from > 0) {
+    const dim3 big_grid(workgroups_for(a.O, a.m_batch, 128));
+    const int min_active = a.round > 0 ? a.big_from : 0;
+    if (a.transposed) hipLaunchKernelGGL(k_mvm_big<1>, big_grid, dim3(256), 0, s, a, min_active);
+    else hipLaunchKernelGGL(k_mvm_big<0>, big_grid, dim3(256), 0, s, a, min_active);
+    if (a.round == 0) return; // later rounds: whichever kernel the number of listed samples calls for
+  }
   const dim3 grid(mvm_round_workgroups(a));
   const int depth = mvm_prefetch_depth(a.K);
   const int mode = weight_mode(a);

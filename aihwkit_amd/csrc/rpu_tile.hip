@@ -357,7 +357,10 @@ struct Tile {
     if (!io.perfect && io.p.bound_management != RPU_BM_NONE) s_xq1.ensure((size_t)B * a.k_pad);
     a.xq[0] = s_xq0.p; a.xq[1] = s_xq1.p;
     a.max_rounds = io.perfect ? 0 : mvm_max_rounds(a.io);
-    a.speculate = B <= 1024 ? 1 : 0;
+    // rows for the next bound-management round are quantized ahead when the batch is small (shortest path between
+    // rounds) or when at least four workgroups per sample tile share that work; a large batch on a narrow tile
+    // quantizes only the rows of the samples that saturated
+    a.speculate = (B <= 1024 || O > 96) ? 1 : 0;
     return a;
   }
 

@@ -38,7 +38,8 @@ def test_philox_known_answers_on_device(gpu_device):
         assert list(out) == want
 
 
-@pytest.mark.parametrize("x_size,d_size,batch", [(64, 32, 32), (100, 70, 33), (512, 512, 100), (1024, 1024, 256)])
+@pytest.mark.parametrize("x_size,d_size,batch", [(64, 32, 32), (100, 70, 33), (512, 512, 100), (1024, 1024, 256),
+                                                 (1024, 1024, 4096), (777, 1000, 4700)])   # the last two: 128 x 128 tiles
 @pytest.mark.parametrize("bm", [dv.BoundManagementType.NONE, dv.BoundManagementType.Iterative])
 def test_forward_exact_arithmetic_is_bit_exact(gpu_device, x_size, d_size, batch, bm):
     """With a power-of-two DAC step and weights on a 1/64 grid every product and partial sum is exact in
