@@ -50,7 +50,7 @@ struct MvmArgs {
   int max_rounds; // rounds launched for this call (mvm_max_rounds)
   int speculate;  // 1: each round also quantizes every row for the round after it (short path between rounds, for
                   // small batches); 0: only the rows of samples that saturated are quantized, once that is known
-  int big_from;   // > 0: rounds with at least this many samples are run by the large-tile kernel (set by the launcher)
+  int big_from;   // > 0: rounds with at least this many samples are run by the large-tile kernel; < 0: round 0 is
   float alpha, beta; // only used when io.perfect: out = alpha * acc + beta * out
   IoDev io;
   MvmState st;
@@ -70,16 +70,22 @@ struct MvmGroup {
   int n;
   int m_batch;
 };
-void launch_mvm_init_group(const MvmGroup &g, hipStream_t s);
+void launch_mvm_init_group(const MvmGroup &g, int max_k, hipStream_t s);
 void launch_mvm_round_group(const MvmGroup &g, int prefetch_depth, int weight_mode, int total_workgroups, int round,
                             hipStream_t s);
 int mvm_round_workgroups(const MvmArgs &a);            // workgroups of a round launch for this tile
+// Large-tile (128 x 128) variant for round 0 of a group: args[t].big_from < 0 marks the tiles it runs, start[]
+// counts its workgroups (mvm_big_workgroups; 0 for the other tiles).
+int mvm_big_workgroups(const MvmArgs &a);
+void launch_mvm_big_group(const MvmGroup &g, int total_workgroups, hipStream_t s);
 void mvm_round_variant(const MvmArgs &a, int &prefetch_depth, int &weight_mode);
 
 // number of rounds that can ever be needed with these IO settings
 int mvm_max_rounds(const IoDev &io);
 // row length of the quantized-input scratch for a contraction length K
-int mvm_k_pad(int K);
+int mvm_k_pad(int K, bool tight = false);
+// whether a call of this shape has rounds run by the large-tile kernel (then the padding can be tight)
+bool mvm_uses_large_tiles(int m_batch, int O);
 
 // [B][X-1] (or [X-1][B]) -> [B][X] with a trailing column of ones (always batch-first output)
 void launch_make_bias(const float *in, float *out, int m_batch, int x_size, int in_trans, hipStream_t s);

@@ -31,6 +31,14 @@ typedef float f32x4_unaligned __attribute__((ext_vector_type(4), aligned(4))); /
 
 namespace {
 
+// Element i (0 or 1) of a two-pointer array of the argument block.  Both pointers are read with constant indices and
+// the choice is made on their bits: an index computed at run time (which is also what a plain conditional is
+// folded to) would force a kernel's copy of the whole block into indexed (scratch) memory.
+template <typename T> __device__ __forceinline__ T *pick2(T *const (&p)[2], int i) {
+  const uintptr_t p0 = (uintptr_t)p[0], p1 = (uintptr_t)p[1];
+  return (T *)(p0 ^ ((p0 ^ p1) & (uintptr_t)(-(intptr_t)(i & 1))));
+}
+
 constexpr int TILE = 32;
 constexpr int WAVES = 4;
 constexpr int KSTEP = 32; // k-values per wave step: 128 bytes per operand row
@@ -262,14 +270,14 @@ __device__ __forceinline__ void mvm_round_tile(const MvmArgs &a, int round, int 
   // staging layout of this lane: pass t covers rows 8 t .. 8 t + 7, lane = (row in pass) * 8 + 16-byte chunk
   const int st_row = lane >> 3;
   const int st_chunk = (lane & 7) * 4;
-  const float *xq = a.xq[round & 1];
+  const float *xq = pick2(a.xq, round & 1);
   const float *x_src[4];
   const float *w_src[4];
 #pragma unroll
   for (int t = 0; t < 4; ++t) {
     const int row = t * 8 + st_row;
     const int slot = min(tile_b * TILE + row, n_act - 1);
-    const int xrow = (round > 0) ? a.st.row[round & 1][slot] : slot;
+    const int xrow = (round > 0) ? pick2(a.st.row, round & 1)[slot] : slot;
     x_src[t] = xq + (long)xrow * a.k_pad + st_chunk;
     const int o = min(tile_o * TILE + row, a.O - 1);
     w_src[t] = a.w + (long)o * a.x_size;
@@ -284,7 +292,7 @@ __device__ __forceinline__ void mvm_round_tile(const MvmArgs &a, int round, int 
   int b_out = slot_in;
   float fin_out = 1.0f;
   if (!a.io.perfect && b_ok) {
-    if (round > 0) b_out = a.st.list[round & 1][slot_in];
+    if (round > 0) b_out = pick2(a.st.list, round & 1)[slot_in];
     fin_out = a.st.fin[b_out];
   }
 
@@ -437,7 +445,7 @@ __device__ __forceinline__ void mvm_round_tile(const MvmArgs &a, int round, int 
       const int hit = hits[threadIdx.x];
       const int slot = tile_b * TILE + t;
       if (hit && slot < n_act) {
-        const int bs = (round > 0) ? a.st.list[round & 1][slot] : slot;
+        const int bs = (round > 0) ? pick2(a.st.list, round & 1)[slot] : slot;
         const int old = atomicMax(threadIdx.x < TILE ? &a.st.hit_up[bs] : &a.st.hit_lo[bs], hit);
         asm volatile("" ::"v"(old));
       }
@@ -631,8 +639,8 @@ __device__ __forceinline__ void mvm_prepare_next_rows(const MvmArgs &a, int roun
     int b = 0;
     float scale = 0.0f; // 0: the sample can have no further round
     if (slot < n_act) {
-      b = (round > 0) ? a.st.list[round & 1][slot] : slot;
-      scale = a.st.next_scale[round & 1][slot];
+      b = (round > 0) ? pick2(a.st.list, round & 1)[slot] : slot;
+      scale = pick2(a.st.next_scale, round & 1)[slot];
     }
     sh_next_b[threadIdx.x] = b;
     sh_next_scale[threadIdx.x] = scale;
@@ -642,7 +650,7 @@ __device__ __forceinline__ void mvm_prepare_next_rows(const MvmArgs &a, int roun
   const int chunk = (a.k_pad + tiles_o - 1) / tiles_o;
   const int k_lo = tile_o * chunk;
   const int k_hi = min(k_lo + chunk, a.k_pad);
-  float *__restrict__ dst = a.xq[(round + 1) & 1];
+  float *__restrict__ dst = pick2(a.xq, (round + 1) & 1);
   const float *__restrict__ in = a.in;
   // a trip covers 32 k-values of all 32 rows: 8 thread-rows x 4 rows each.  The loads of four trips are issued
   // together: a narrow tile has few workgroups per sample tile and each walks a long piece of the rows.
@@ -700,9 +708,9 @@ __device__ __forceinline__ int mvm_advance_sample(const MvmArgs &a, int round, i
   a.st.rounds[b] += 1;
   scale = set_round_scales(a, b, nm, red);
   const int pos = atomicAdd(&a.st.count[round + 1], 1);
-  a.st.list[(round + 1) & 1][pos] = b;
-  a.st.row[(round + 1) & 1][pos] = rows_ahead ? slot : pos;
-  a.st.next_scale[(round + 1) & 1][pos] = next_round_scale(a, round + 1, b, a.st.fin[b], nm, red);
+  pick2(a.st.list, (round + 1) & 1)[pos] = b;
+  pick2(a.st.row, (round + 1) & 1)[pos] = rows_ahead ? slot : pos;
+  pick2(a.st.next_scale, (round + 1) & 1)[pos] = next_round_scale(a, round + 1, b, a.st.fin[b], nm, red);
   return pos;
 }
 
@@ -728,7 +736,7 @@ __device__ __forceinline__ void mvm_tile_finished(const MvmArgs &a, int round, i
   if (threadIdx.x < TILE) {
     const int slot = tile_b * TILE + threadIdx.x;
     if (slot < n_act) {
-      const int b = (round > 0) ? a.st.list[round & 1][slot] : slot;
+      const int b = (round > 0) ? pick2(a.st.list, round & 1)[slot] : slot;
       float scale = 0.0f;
       const int pos = mvm_advance_sample(a, round, b, slot, a.speculate != 0, scale);
       if (pos >= 0 && !a.speculate) {
@@ -744,7 +752,7 @@ __device__ __forceinline__ void mvm_tile_finished(const MvmArgs &a, int round, i
   // them): the rows of the samples that do go on are written now
   __syncthreads();
   for (int i = 0; i < sh_more; ++i) {
-    write_dac_row(a, sh_more_b[i], sh_more_pos[i], sh_more_scale[i], round + 1, a.xq[(round + 1) & 1], threadIdx.x, 256);
+    write_dac_row(a, sh_more_b[i], sh_more_pos[i], sh_more_scale[i], round + 1, pick2(a.xq, (round + 1) & 1), threadIdx.x, 256);
   }
 }
 
@@ -760,12 +768,73 @@ __device__ __forceinline__ void mvm_round_workgroup(const MvmArgs &a, int round,
   if (more_rounds) mvm_tile_finished(a, round, tile_b, n_act);
 }
 
+// big_from > 0: the large-tile kernel runs the rounds that list at least that many samples; < 0: it runs round 0
+__device__ __forceinline__ bool runs_on_large_tiles(const MvmArgs &a, int round, int n_act) {
+  return (a.big_from > 0 && n_act >= a.big_from) || (a.big_from < 0 && round == 0);
+}
+
+// Rounds after the first usually list few samples, but their launch is sized before that is known.  When the
+// full grid would be large, this variant runs them instead: a fixed number of workgroups walk the tiles of the
+// listed samples, with one register set (k_pad only needs to be a multiple of 32).
+template <int WMODE>
+__global__ __launch_bounds__(256) void k_mvm_round_tail(MvmArgs a) {
+  __shared__ float red[WAVES][16][64];
+  __shared__ __attribute__((aligned(16))) float stage[WAVES * 2 * TILE * LDS_ROW];
+  const int n_act = (a.round > 0) ? a.st.count[a.round] : a.m_batch;
+  if (runs_on_large_tiles(a, a.round, n_act)) return;
+  const int total = workgroups_for(a.O, n_act);
+  for (int n = blockIdx.x; n < total; n += gridDim.x) {
+    mvm_round_workgroup<1, WMODE>(a, a.round, n, n_act, red, stage);
+    __syncthreads(); // LDS is reused by the next tile
+  }
+}
+
+// The same for a group: the workgroups first find out, one thread per tile, how many 32 x 32 tiles each member has
+// listed for this round (usually none), then walk the concatenation of those.  tile_first .. tile_first + n_tiles
+// are the group members of this launch's kernel variant.
+constexpr int MAX_GROUP = 1024;
+
+template <int WMODE>
+__global__ __launch_bounds__(256) void k_mvm_round_tail_group(MvmGroup g, int round) {
+  __shared__ float red[WAVES][16][64];
+  __shared__ __attribute__((aligned(16))) float stage[WAVES * 2 * TILE * LDS_ROW];
+  __shared__ int sh_first[MAX_GROUP + 1]; // first workgroup number of member t; [g.n] = total
+  for (int t = threadIdx.x; t < g.n; t += blockDim.x) {
+    const MvmArgs &a = g.args[t];
+    int wg = 0;
+    if (round < a.max_rounds) {
+      const int n_act = (round > 0) ? a.st.count[round] : a.m_batch;
+      if (!runs_on_large_tiles(a, round, n_act) && n_act > 0) wg = workgroups_for(a.O, n_act);
+    }
+    sh_first[t + 1] = wg;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int sum = 0;
+    sh_first[0] = 0;
+    for (int t = 0; t < g.n; ++t) {
+      sum += sh_first[t + 1];
+      sh_first[t + 1] = sum;
+    }
+  }
+  __syncthreads();
+  const int total = sh_first[g.n];
+  int t = 0;
+  for (int n = blockIdx.x; n < total; n += gridDim.x) {
+    while (n >= sh_first[t + 1]) ++t;
+    const MvmArgs &a = g.args[t];
+    const int n_act = (round > 0) ? a.st.count[round] : a.m_batch;
+    mvm_round_workgroup<1, WMODE>(a, round, n - sh_first[t], n_act, red, stage);
+    __syncthreads();
+  }
+}
+
 template <int PD, int WMODE>
 __global__ __launch_bounds__(256) void k_mvm_round(MvmArgs a) {
   __shared__ float red[WAVES][16][64];
   __shared__ __attribute__((aligned(16))) float stage[WAVES * 2 * TILE * LDS_ROW];
   const int n_act = (a.round > 0) ? a.st.count[a.round] : a.m_batch;
-  if (a.big_from > 0 && n_act >= a.big_from) return; // this round is run by k_mvm_big
+  if (runs_on_large_tiles(a, a.round, n_act)) return;
   mvm_round_workgroup<PD, WMODE>(a, a.round, blockIdx.x, n_act, red, stage);
 }
 
@@ -790,8 +859,8 @@ __device__ __forceinline__ void big_prepare_next_rows(const MvmArgs &a, int roun
     int b = 0;
     float scale = 0.0f;
     if (slot < n_act) {
-      b = (round > 0) ? a.st.list[round & 1][slot] : slot;
-      scale = a.st.next_scale[round & 1][slot];
+      b = (round > 0) ? pick2(a.st.list, round & 1)[slot] : slot;
+      scale = pick2(a.st.next_scale, round & 1)[slot];
     }
     sh_b[threadIdx.x] = b;
     sh_scale[threadIdx.x] = scale;
@@ -801,33 +870,32 @@ __device__ __forceinline__ void big_prepare_next_rows(const MvmArgs &a, int roun
   const int chunk = (((a.k_pad + tiles_o - 1) / tiles_o) + 31) & ~31;
   const int k_lo = tile_o * chunk;
   const int k_hi = min(k_lo + chunk, a.k_pad);
-  float *__restrict__ dst = a.xq[(round + 1) & 1];
+  float *__restrict__ dst = pick2(a.xq, (round + 1) & 1);
   const float *__restrict__ in = a.in;
-  const int kq = threadIdx.x & 31, rq = threadIdx.x >> 5; // 8 thread-rows, 16 rows each, 4 at a time
+  const int kq = threadIdx.x & 31, rq = threadIdx.x >> 5; // 8 thread-rows of 16 rows each
   for (int k0 = k_lo; k0 < k_hi; k0 += 32) {
     const int k = k0 + kq;
-    for (int jb = 0; jb < 4; ++jb) {
-      float xv[4];
+    float xv[16]; // all 16 loads of a trip are in flight together
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int row = rq * 16 + jb * 4 + i;
-        xv[i] = (sh_scale[row] != 0.0f && k < a.K) ? in[(long)sh_b[row] * a.in_sb + (long)k * a.in_sk] : 0.0f;
-      }
+    for (int i = 0; i < 16; ++i) {
+      const int row = rq * 16 + i;
+      xv[i] = (sh_scale[row] != 0.0f && k < a.K) ? in[(long)sh_b[row] * a.in_sb + (long)k * a.in_sk] : 0.0f;
+    }
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int row = rq * 16 + jb * 4 + i;
-        const float sc = sh_scale[row];
-        if (sc != 0.0f) {
-          const float v = (k < a.K) ? dac_value(xv[i], sc, a.io, a.key, a.call, round + 1, sh_b[row], k) : 0.0f;
-          dst[(long)(tile_b * BT + row) * a.k_pad + k] = v;
-        }
+    for (int i = 0; i < 16; ++i) {
+      const int row = rq * 16 + i;
+      const float sc = sh_scale[row];
+      if (sc != 0.0f) {
+        const float v = (k < a.K) ? dac_value(xv[i], sc, a.io, a.key, a.call, round + 1, sh_b[row], k) : 0.0f;
+        dst[(long)(tile_b * BT + row) * a.k_pad + k] = v;
       }
     }
   }
 }
 
+// work of workgroup number n of a large-tile round launch of one tile
 template <int WT>
-__global__ __launch_bounds__(256, 2) void k_mvm_big(MvmArgs a, int min_active) {
+__device__ __forceinline__ void mvm_big_workgroup(const MvmArgs &a, const int round, const int n, const int min_active) {
   __shared__ __attribute__((aligned(16))) float lds_x[2][BT * BPITCH];
   __shared__ __attribute__((aligned(16))) float lds_w[2][WT ? BKS * BPITCH_T : BT * BPITCH];
   __shared__ int sh_hits[2 * BT];
@@ -835,11 +903,13 @@ __global__ __launch_bounds__(256, 2) void k_mvm_big(MvmArgs a, int min_active) {
   __shared__ float sh_scale[BT];
   __shared__ int sh_last;
 
-  const int round = a.round;
   const int n_act = (round > 0) ? a.st.count[round] : a.m_batch;
   if (n_act < min_active) return; // this round is run by the 32 x 32 kernel
-  int tile_o, tile_b;
-  if (!tile_of<BT>(a, blockIdx.x, n_act, tile_o, tile_b)) return;
+  // workgroup n runs on XCD n % 8: an XCD walks the output tiles of one sample tile after the other, so a tile of
+  // quantized inputs (the large operand) enters one L2 only and the small weight matrix is what every XCD streams
+  const int tile_o = (n >> 3) % ((a.O + BT - 1) / BT);
+  const int tile_b = ((n >> 3) / ((a.O + BT - 1) / BT)) * 8 + (n & 7);
+  if (tile_b * BT >= n_act) return;
   const bool more_rounds = round + 1 < a.max_rounds;
   if (more_rounds) big_prepare_next_rows(a, round, tile_o, tile_b, n_act, sh_b, sh_scale);
 
@@ -851,7 +921,7 @@ __global__ __launch_bounds__(256, 2) void k_mvm_big(MvmArgs a, int min_active) {
 
   // global -> LDS assignment.  k-contiguous operand: chunk c = t + 256 j covers row c / 8, floats 4 (c % 8) ..;
   // output-contiguous weights: chunk c covers k-row c / 32, outputs 4 (c % 32) ..
-  const float *xq = a.xq[round & 1];
+  const float *xq = pick2(a.xq, round & 1);
   const float *x_src[4];
   const float *w_src[4];
   const int st_col = (t & 7) * 4;
@@ -859,7 +929,7 @@ __global__ __launch_bounds__(256, 2) void k_mvm_big(MvmArgs a, int min_active) {
   for (int j = 0; j < 4; ++j) {
     const int row = (t >> 3) + 32 * j;
     const int slot = min(tile_b * BT + row, n_act - 1);
-    const int xrow = (round > 0) ? a.st.row[round & 1][slot] : slot;
+    const int xrow = (round > 0) ? pick2(a.st.row, round & 1)[slot] : slot;
     x_src[j] = xq + (long)xrow * a.k_pad + st_col;
     if (WT == 0) w_src[j] = a.w + (long)min(tile_o * BT + row, a.O - 1) * a.x_size;
   }
@@ -917,40 +987,45 @@ __global__ __launch_bounds__(256, 2) void k_mvm_big(MvmArgs a, int min_active) {
     }
   };
 
-  floatx16 acc[2][2];
+  // accumulators of the 2 x 2 MFMA tiles (output block, sample block), named one by one so that they stay in
+  // registers whatever the inlining order
+  floatx16 acc00, acc01, acc10, acc11;
 #pragma unroll
-  for (int oi = 0; oi < 2; ++oi)
-#pragma unroll
-    for (int bi = 0; bi < 2; ++bi)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) acc[oi][bi][i] = 0.0f;
+  for (int i = 0; i < 16; ++i) {
+    acc00[i] = 0.0f;
+    acc01[i] = 0.0f;
+    acc10[i] = 0.0f;
+    acc11[i] = 0.0f;
+  }
 
   // lane (r, h) multiplies k = 16 h .. 16 h + 15 of a stage, four values at a time
-  auto compute = [&](int buf) {
+  auto compute = [&](int buf) __attribute__((always_inline)) {
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
-      f32x4 wa[2], xb[2];
       const int kk = h * 16 + q * 4;
-#pragma unroll
-      for (int i = 0; i < 2; ++i) {
-        xb[i] = *reinterpret_cast<const f32x4 *>(&lds_x[buf][(wx * 64 + i * 32 + r) * BPITCH + kk]);
-        if (WT == 0) {
-          wa[i] = *reinterpret_cast<const f32x4 *>(&lds_w[buf][(wy * 64 + i * 32 + r) * BPITCH + kk]);
-        } else {
-          const float *col = &lds_w[buf][kk * BPITCH_T + wy * 64 + i * 32 + r];
-          wa[i].x = col[0];
-          wa[i].y = col[BPITCH_T];
-          wa[i].z = col[2 * BPITCH_T];
-          wa[i].w = col[3 * BPITCH_T];
-        }
+      const f32x4 xb0 = *reinterpret_cast<const f32x4 *>(&lds_x[buf][(wx * 64 + r) * BPITCH + kk]);
+      const f32x4 xb1 = *reinterpret_cast<const f32x4 *>(&lds_x[buf][(wx * 64 + 32 + r) * BPITCH + kk]);
+      f32x4 wa0, wa1;
+      if (WT == 0) {
+        wa0 = *reinterpret_cast<const f32x4 *>(&lds_w[buf][(wy * 64 + r) * BPITCH + kk]);
+        wa1 = *reinterpret_cast<const f32x4 *>(&lds_w[buf][(wy * 64 + 32 + r) * BPITCH + kk]);
+      } else {
+        const float *col = &lds_w[buf][kk * BPITCH_T + wy * 64 + r];
+        wa0.x = col[0];
+        wa0.y = col[BPITCH_T];
+        wa0.z = col[2 * BPITCH_T];
+        wa0.w = col[3 * BPITCH_T];
+        wa1.x = col[32];
+        wa1.y = col[BPITCH_T + 32];
+        wa1.z = col[2 * BPITCH_T + 32];
+        wa1.w = col[3 * BPITCH_T + 32];
       }
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-#pragma unroll
-        for (int oi = 0; oi < 2; ++oi)
-#pragma unroll
-          for (int bi = 0; bi < 2; ++bi)
-            acc[oi][bi] = __builtin_amdgcn_mfma_f32_32x32x2f32(wa[oi][e], xb[bi][e], acc[oi][bi], 0, 0, 0);
+        acc00 = __builtin_amdgcn_mfma_f32_32x32x2f32(wa0[e], xb0[e], acc00, 0, 0, 0);
+        acc01 = __builtin_amdgcn_mfma_f32_32x32x2f32(wa0[e], xb1[e], acc01, 0, 0, 0);
+        acc10 = __builtin_amdgcn_mfma_f32_32x32x2f32(wa1[e], xb0[e], acc10, 0, 0, 0);
+        acc11 = __builtin_amdgcn_mfma_f32_32x32x2f32(wa1[e], xb1[e], acc11, 0, 0, 0);
       }
     }
   };
@@ -975,15 +1050,15 @@ __global__ __launch_bounds__(256, 2) void k_mvm_big(MvmArgs a, int min_active) {
   if (t < 2 * BT) sh_hits[t] = 0;
   __syncthreads();
   const bool flags = !a.io.perfect && a.io.bound_management != RPU_BM_NONE;
-#pragma unroll
-  for (int bi = 0; bi < 2; ++bi) {
+  // sample block bi of this wave: its two output blocks
+  auto finish_block = [&](const int bi, const floatx16 &acc_o0, const floatx16 &acc_o1) __attribute__((always_inline)) {
     const int local_b = wx * 64 + bi * 32 + r;
     const int slot = tile_b * BT + local_b;
-    if (slot >= n_act) continue;
+    if (slot >= n_act) return;
     int b_out = slot;
     float fin_out = 1.0f;
     if (!a.io.perfect) {
-      if (round > 0) b_out = a.st.list[round & 1][slot];
+      if (round > 0) b_out = pick2(a.st.list, round & 1)[slot];
       fin_out = a.st.fin[b_out];
     }
     int up_max = 0, lo_max = 0;
@@ -992,12 +1067,11 @@ __global__ __launch_bounds__(256, 2) void k_mvm_big(MvmArgs a, int min_active) {
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         const int o0 = tile_o * BT + wy * 64 + oi * 32 + g * 8 + h * 4;
-        if (o0 >= a.O) continue;
         float v[4];
 #pragma unroll
-        for (int q = 0; q < 4; ++q) v[q] = acc[oi][bi][4 * g + q];
-        int up, lo;
-        mvm_finish_outputs(a, round, b_out, fin_out, o0, v, up, lo);
+        for (int q = 0; q < 4; ++q) v[q] = oi ? acc_o1[4 * g + q] : acc_o0[4 * g + q];
+        int up = 0, lo = 0;
+        if (o0 < a.O) mvm_finish_outputs(a, round, b_out, fin_out, o0, v, up, lo);
         up_max = max(up_max, up);
         lo_max = max(lo_max, lo);
       }
@@ -1006,7 +1080,9 @@ __global__ __launch_bounds__(256, 2) void k_mvm_big(MvmArgs a, int min_active) {
       if (up_max) atomicMax(&sh_hits[local_b], up_max);
       if (lo_max) atomicMax(&sh_hits[BT + local_b], lo_max);
     }
-  }
+  };
+  finish_block(0, acc00, acc10);
+  finish_block(1, acc01, acc11);
   if (!flags) return;
   __syncthreads();
   {
@@ -1014,7 +1090,7 @@ __global__ __launch_bounds__(256, 2) void k_mvm_big(MvmArgs a, int min_active) {
     const int hit = sh_hits[t];
     const int slot = tile_b * BT + local_b;
     if (hit && slot < n_act) {
-      const int bs = (round > 0) ? a.st.list[round & 1][slot] : slot;
+      const int bs = (round > 0) ? pick2(a.st.list, round & 1)[slot] : slot;
       const int old = atomicMax(t < BT ? &a.st.hit_up[bs] : &a.st.hit_lo[bs], hit);
       asm volatile("" ::"v"(old));
     }
@@ -1034,9 +1110,23 @@ __global__ __launch_bounds__(256, 2) void k_mvm_big(MvmArgs a, int min_active) {
     const int slot = tile_b * BT + t;
     if (slot < n_act) {
       float scale;
-      mvm_advance_sample(a, round, (round > 0) ? a.st.list[round & 1][slot] : slot, slot, true, scale);
+      mvm_advance_sample(a, round, (round > 0) ? pick2(a.st.list, round & 1)[slot] : slot, slot, true, scale);
     }
   }
+}
+
+template <int WT>
+__global__ __launch_bounds__(256, 2) void k_mvm_big(MvmArgs a, int min_active) {
+  mvm_big_workgroup<WT>(a, a.round, (int)blockIdx.x, min_active);
+}
+
+// several tiles in one launch (forward, round 0): a tile that is not run by this kernel has no workgroups in the table
+__global__ __launch_bounds__(256, 2) void k_mvm_big_group(MvmGroup g, int round) {
+  int t = 0;
+  while (t + 1 < g.n && (int)blockIdx.x >= g.start[t + 1]) ++t;
+  const MvmArgs &a = g.args[t];
+  if (round > 0 && round >= a.max_rounds) return;
+  mvm_big_workgroup<0>(a, round, (int)blockIdx.x - g.start[t], 0);
 }
 
 // The same for several tiles in one launch: a workgroup finds its tile in the table of first workgroup numbers
@@ -1050,14 +1140,19 @@ __global__ __launch_bounds__(256) void k_mvm_round_group(MvmGroup g, int round) 
   const MvmArgs &a = g.args[t];
   if (round > 0 && round >= a.max_rounds) return;
   const int n_act = (round > 0) ? a.st.count[round] : a.m_batch;
+  if (runs_on_large_tiles(a, round, n_act)) return;
   mvm_round_workgroup<PD, WMODE>(a, round, (int)blockIdx.x - g.start[t], n_act, red, stage);
 }
 
+template <int SUB>
 __global__ __launch_bounds__(256) void k_mvm_init_group(MvmGroup g) {
   __shared__ float sh[8];
-  const int t = blockIdx.x / g.m_batch;
-  const int b = blockIdx.x - t * g.m_batch;
-  mvm_init_sample<256>(g.args[t], b, threadIdx.x, b * 256L + threadIdx.x, g.m_batch * 256L, sh);
+  const long sample = blockIdx.x * (long)(256 / SUB) + threadIdx.x / SUB; // m_batch is a multiple of 256 / SUB
+  const int t = (int)(sample / g.m_batch);
+  if (t >= g.n) return;
+  const int b = (int)(sample - (long)t * g.m_batch);
+  const int lane = threadIdx.x % SUB;
+  mvm_init_sample<SUB>(g.args[t], b, lane, (long)b * SUB + lane, (long)g.m_batch * SUB, sh);
 }
 
 __global__ void k_make_bias(const float *in, float *out, int m_batch, int x_size, int in_trans) {
@@ -1102,10 +1197,16 @@ int mvm_max_rounds(const IoDev &io) {
 
 // prefetch depth used for a contraction length: deep for long contractions, where each of the few
 // resident waves must cover the memory latency alone
-static int mvm_prefetch_depth(int K) { return K >= 512 ? 4 : (K >= 256 ? 2 : 1); }
+static int mvm_prefetch_depth(int K, int k_pad) {
+  if (K >= 512 && k_pad % (KSTEP * WAVES * 4) == 0) return 4;
+  if (K >= 256 && k_pad % (KSTEP * WAVES * 2) == 0) return 2;
+  return 1;
+}
 
-int mvm_k_pad(int K) {
-  const int depth = mvm_prefetch_depth(K);
+// tight: a multiple of 32 (what the large-tile kernel and the single-register-set variants need); otherwise K is
+// rounded up so that the prefetch depth that suits its length can be used
+int mvm_k_pad(int K, bool tight) {
+  const int depth = tight ? 1 : (K >= 512 ? 4 : (K >= 256 ? 2 : 1));
   const int unit = depth == 1 ? KSTEP : KSTEP * WAVES * depth;
   return ((K + unit - 1) / unit) * unit;
 }
@@ -1132,15 +1233,52 @@ void launch_mvm_init(const MvmArgs &a, hipStream_t s) {
 int mvm_round_workgroups(const MvmArgs &a) { return workgroups_for(a.O, a.m_batch); }
 
 void mvm_round_variant(const MvmArgs &a, int &prefetch_depth, int &mode) {
-  prefetch_depth = mvm_prefetch_depth(a.K);
+  prefetch_depth = mvm_prefetch_depth(a.K, a.k_pad);
   mode = weight_mode(a);
 }
 
-void launch_mvm_init_group(const MvmGroup &g, hipStream_t s) {
-  hipLaunchKernelGGL(k_mvm_init_group, dim3(g.n * g.m_batch), dim3(256), 0, s, g);
+// max_k: the longest input row of the group
+void launch_mvm_init_group(const MvmGroup &g, int max_k, hipStream_t s) {
+  const long samples = (long)g.n * g.m_batch;
+  if (samples > 2048 && max_k <= 512 && g.m_batch % 4 == 0) {
+    hipLaunchKernelGGL(k_mvm_init_group<64>, dim3((unsigned)(samples / 4)), dim3(256), 0, s, g);
+  } else {
+    hipLaunchKernelGGL(k_mvm_init_group<256>, dim3((unsigned)samples), dim3(256), 0, s, g);
+  }
 }
 
+constexpr int TAIL_GRID = 1024; // workgroups of a later-round launch when the full grid would be larger
+
+static int big_workgroups(const MvmArgs &a) {
+  const int tiles_o = (a.O + 127) / 128, tiles_b = (a.m_batch + 127) / 128;
+  return 8 * tiles_o * ((tiles_b + 7) / 8);
+}
+
+int mvm_big_workgroups(const MvmArgs &a) { return a.O >= 128 ? big_workgroups(a) : 0; }
+
+void launch_mvm_big_group(const MvmGroup &g, int total_workgroups, hipStream_t s) {
+  hipLaunchKernelGGL(k_mvm_big_group, dim3(total_workgroups), dim3(256), 0, s, g, 0);
+}
+
+// samples of a round from which the large-tile kernel takes over, 0 when a call of this shape never uses it: it
+// needs outputs for a whole 128-wide tile and enough tiles to fill half the chip
+static int big_threshold(int m_batch, int O) {
+  if (m_batch < 2048 || O < 128) return 0;
+  const int tiles_o = (O + 127) / 128, tiles_b = (m_batch + 127) / 128;
+  if (8 * tiles_o * ((tiles_b + 7) / 8) < 128) return 0;
+  return 2048;
+}
+
+bool mvm_uses_large_tiles(int m_batch, int O) { return big_threshold(m_batch, O) > 0; }
+
 void launch_mvm_round_group(const MvmGroup &g, int depth, int mode, int total_workgroups, int round, hipStream_t s) {
+  if (round > 0 && total_workgroups > TAIL_GRID && g.n <= MAX_GROUP) {
+    const dim3 tail(TAIL_GRID);
+    if (mode == 0) hipLaunchKernelGGL(k_mvm_round_tail_group<0>, tail, dim3(256), 0, s, g, round);
+    else if (mode == 1) hipLaunchKernelGGL(k_mvm_round_tail_group<1>, tail, dim3(256), 0, s, g, round);
+    else hipLaunchKernelGGL(k_mvm_round_tail_group<2>, tail, dim3(256), 0, s, g, round);
+    return;
+  }
   const dim3 grid(total_workgroups);
 #define RPU_LAUNCH_ROUND(PD, WMODE) hipLaunchKernelGGL((k_mvm_round_group<PD, WMODE>), grid, dim3(256), 0, s, g, round)
   if (mode == 0) {
@@ -1159,27 +1297,27 @@ void launch_mvm_round_group(const MvmGroup &g, int depth, int mode, int total_wo
 #undef RPU_LAUNCH_ROUND
 }
 
-// samples of a round from which the large-tile kernel takes over, 0 when this call never uses it: it needs
-// outputs for a whole 128-wide tile and enough tiles to fill half the chip
-static int big_threshold(const MvmArgs &a) {
-  if (a.m_batch < 2048 || a.O < 128) return 0;
-  if (workgroups_for(a.O, a.m_batch, 128) < 128) return 0;
-  return 2048;
-}
-
 void launch_mvm_round(const MvmArgs &a_in, hipStream_t s) {
   MvmArgs a = a_in;
-  a.big_from = big_threshold(a);
+  a.big_from = big_threshold(a.m_batch, a.O);
   if (a.big_from > 0) {
-    const dim3 big_grid(workgroups_for(a.O, a.m_batch, 128));
+    const dim3 big_grid(big_workgroups(a));
     const int min_active = a.round > 0 ? a.big_from : 0;
     if (a.transposed) hipLaunchKernelGGL(k_mvm_big<1>, big_grid, dim3(256), 0, s, a, min_active);
     else hipLaunchKernelGGL(k_mvm_big<0>, big_grid, dim3(256), 0, s, a, min_active);
     if (a.round == 0) return; // later rounds: whichever kernel the number of listed samples calls for
   }
-  const dim3 grid(mvm_round_workgroups(a));
-  const int depth = mvm_prefetch_depth(a.K);
+  const int all = mvm_round_workgroups(a);
   const int mode = weight_mode(a);
+  if (a.round > 0 && all > TAIL_GRID) {
+    const dim3 grid(TAIL_GRID);
+    if (mode == 0) hipLaunchKernelGGL(k_mvm_round_tail<0>, grid, dim3(256), 0, s, a);
+    else if (mode == 1) hipLaunchKernelGGL(k_mvm_round_tail<1>, grid, dim3(256), 0, s, a);
+    else hipLaunchKernelGGL(k_mvm_round_tail<2>, grid, dim3(256), 0, s, a);
+    return;
+  }
+  const dim3 grid(all);
+  const int depth = mvm_prefetch_depth(a.K, a.k_pad);
 #define RPU_LAUNCH_ROUND(PD, WMODE) hipLaunchKernelGGL((k_mvm_round<PD, WMODE>), grid, dim3(256), 0, s, a)
   if (mode == 0) {
     if (depth == 4) RPU_LAUNCH_ROUND(4, 0);

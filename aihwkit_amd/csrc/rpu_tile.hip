@@ -336,7 +336,7 @@ struct Tile {
 
   // shared driver of forward (transposed = 0) and backward (transposed = 1)
   // arguments of the MVM kernels for one call, scratch sized for B samples; the caller sets in / out
-  MvmArgs mvm_args(int B, bool transposed, const float *w_other, const IOPar &io) {
+  MvmArgs mvm_args(int B, bool transposed, const float *w_other, const IOPar &io, int large_tiles = -1) {
     const int K = transposed ? D : X;
     const int O = transposed ? X : D;
     ensure_mvm_scratch(B);
@@ -352,7 +352,9 @@ struct Tile {
     a.st.list[0] = s_list0.p; a.st.list[1] = s_list1.p; a.st.row[0] = s_row0.p; a.st.row[1] = s_row1.p;
     a.st.count = s_count.p;
     a.st.tile_done = s_tiledone.p;
-    a.k_pad = mvm_k_pad(K);
+    // large_tiles: whether rounds of this call run on the large-tile kernel (-1: what the shape alone decides)
+    const bool tight = large_tiles < 0 ? mvm_uses_large_tiles(B, O) : large_tiles != 0;
+    a.k_pad = mvm_k_pad(K, tight);
     s_xq0.ensure((size_t)B * a.k_pad);
     if (!io.perfect && io.p.bound_management != RPU_BM_NONE) s_xq1.ensure((size_t)B * a.k_pad);
     a.xq[0] = s_xq0.p; a.xq[1] = s_xq1.p;
@@ -1191,9 +1193,9 @@ int rpu_group_create(rpu_group_t **out, rpu_tile_t *const *tiles, int n_tiles) {
     DeviceGuard dg(g->device_id);
     const size_t n = (size_t)n_tiles;
     g->d_args.ensure(n);
-    g->d_start.ensure(2 * n + 2);
+    g->d_start.ensure(3 * n + 4);
     RPU_HIP_CHECK(hipHostMalloc((void **)&g->h_args, n * sizeof(MvmArgs), hipHostMallocDefault));
-    RPU_HIP_CHECK(hipHostMalloc((void **)&g->h_start, (2 * n + 2) * sizeof(int), hipHostMallocDefault));
+    RPU_HIP_CHECK(hipHostMalloc((void **)&g->h_start, (3 * n + 4) * sizeof(int), hipHostMallocDefault));
     RPU_HIP_CHECK(hipEventCreateWithFlags(&g->copied, hipEventDisableTiming));
     *out = g.release();
   });
@@ -1216,6 +1218,19 @@ int rpu_group_forward(rpu_group_t *group, const float *const *x_dev, float *cons
     // the staging buffers may still feed the copy of the previous call
     RPU_HIP_CHECK(hipEventSynchronize(group->copied));
 
+    // a batch of 1024 or more on tiles at least 128 outputs wide: the large-tile kernel runs round 0 of those tiles,
+    // if the group has enough of its workgroups to fill the chip
+    int big_total = 0;
+    if (m_batch >= 1024) {
+      for (int i = 0; i < n; ++i) {
+        MvmArgs shape{};
+        shape.O = group->tiles[i]->t.D;
+        shape.m_batch = m_batch;
+        big_total += mvm_big_workgroups(shape);
+      }
+    }
+    const bool use_big = big_total >= 256;
+    bool all_big = use_big;
     // per tile: arguments of a plain forward call (row-major x [m_batch][x_size], y [m_batch][d_size])
     std::vector<MvmArgs> args(n);
     std::vector<int> depth(n), mode(n);
@@ -1224,9 +1239,12 @@ int rpu_group_forward(rpu_group_t *group, const float *const *x_dev, float *cons
       Tile &t = group->tiles[i]->t;
       std::lock_guard<std::mutex> lock(t.mutex);
       t.check_compute(m_batch, x_dev[i], y_dev[i]);
-      MvmArgs a = t.mvm_args(m_batch, false, nullptr, t.fio);
+      const bool big = use_big && t.D >= 128;
+      MvmArgs a = t.mvm_args(m_batch, false, nullptr, t.fio, big ? 1 : 0);
       a.in = x_dev[i]; a.in_sb = t.X; a.in_sk = 1;
       a.out = y_dev[i]; a.out_sb = t.D; a.out_so = 1;
+      a.big_from = big ? -1 : 0;
+      if (!big) all_big = false;
       mvm_round_variant(a, depth[i], mode[i]);
       rounds = std::max(rounds, a.max_rounds);
       args[i] = a;
@@ -1255,14 +1273,30 @@ int rpu_group_forward(rpu_group_t *group, const float *const *x_dev, float *cons
       segments.push_back(seg);
       i = j;
     }
+    const int big_offset = cursor; // table of the large-tile launch over all tiles, in the order of d_args
+    if (use_big) {
+      int wg = 0;
+      for (int i = 0; i < n; ++i) {
+        group->h_start[cursor++] = wg;
+        if (args[order[i]].big_from != 0) wg += mvm_big_workgroups(args[order[i]]);
+      }
+      group->h_start[cursor++] = wg;
+    }
     for (int i = 0; i < n; ++i) group->h_args[i] = args[order[i]];
     RPU_HIP_CHECK(hipMemcpyAsync(group->d_args.p, group->h_args, (size_t)n * sizeof(MvmArgs), hipMemcpyHostToDevice, s));
     RPU_HIP_CHECK(hipMemcpyAsync(group->d_start.p, group->h_start, (size_t)cursor * sizeof(int), hipMemcpyHostToDevice, s));
     RPU_HIP_CHECK(hipEventRecord(group->copied, s));
 
     MvmGroup all{group->d_args.p, nullptr, n, m_batch};
-    launch_mvm_init_group(all, s);
+    int max_k = 0;
+    for (int i = 0; i < n; ++i) max_k = std::max(max_k, args[i].K);
+    launch_mvm_init_group(all, max_k, s);
     for (int r = 0; r < rounds; ++r) {
+      if (use_big && r == 0) {
+        MvmGroup g{group->d_args.p, group->d_start.p + big_offset, n, m_batch};
+        launch_mvm_big_group(g, big_total, s);
+        if (all_big) continue;
+      }
       for (const Segment &seg : segments) {
         MvmGroup g{group->d_args.p + seg.first, group->d_start.p + seg.start_offset, seg.count, m_batch};
         launch_mvm_round_group(g, seg.depth, seg.mode, seg.workgroups, r, s);

@@ -199,3 +199,34 @@ def test_grouped_forward_equals_the_tiles_own_forward(gpu_device):
         tl.TileGroup([grouped[0], grouped[0]])
     with pytest.raises(RuntimeError):
         group.forward(xs[:-1])
+
+
+def test_grouped_forward_at_a_token_batch_is_exact_in_exact_arithmetic(gpu_device):
+    """At a batch of 1024 the group runs round 0 on 128 x 128 workgroup tiles (another summation order than a tile's
+    own forward).  With a power-of-two DAC step and weights on a 1/64 grid every partial sum is exact, so group,
+    single-tile call and oracle must still agree to the last bit; one narrow tile stays on the 32 x 32 kernel."""
+    from aihwkit_amd.rpu_base import tiles as tl
+    from helpers import build_pair, constant_step
+
+    rng = np.random.default_rng(8)
+    batch = 1024
+    shapes = [(70, 512), (96, 512), (130, 512), (64, 500), (33, 512), (70, 512), (96, 512), (130, 512), (64, 512),
+              (50, 40)]
+    f_io = noise_free_io(inp_res=1 / 128.0, out_res=1 / 512.0, noise_management=dv.NoiseManagementType.AbsMax,
+                         bound_management=dv.BoundManagementType.Iterative)
+    grouped, oracles, xs = [], [], []
+    for k, (x_size, d_size) in enumerate(shapes):
+        dev = constant_step(w_max_dtod=0.0, w_min_dtod=0.0, w_max=1.0, w_min=-1.0, construction_seed=k + 1)
+        host, orc, _ = build_pair(make_meta(f_io, noise_free_io()), dev, x_size, d_size, gpu=False)
+        w = (rng.integers(-60, 61, (d_size, x_size)) / 64.0).astype(np.float32)
+        host.set_weights(torch.from_numpy(w))
+        orc.set_weights(w)
+        grouped.append(tl.CudaAnalogTile(host))
+        oracles.append(orc)
+        xs.append(rng.uniform(-1, 1, (batch, x_size)).astype(np.float32))
+    group = tl.TileGroup(grouped)
+    got = group.forward([torch.from_numpy(x).cuda() for x in xs])
+    for k, (y, orc, x) in enumerate(zip(got, oracles, xs)):
+        assert np.array_equal(y.cpu().numpy(), orc.forward(x)), k
+        assert np.array_equal(grouped[k].get_bm_rounds(batch).numpy(), orc.bm_rounds(batch)), k
+    assert oracles[2].bm_rounds(batch).max() > 1                       # the later rounds were exercised
