@@ -138,9 +138,9 @@ struct UpdateArgs {
 };
 
 void launch_update_prepare(const UpdateArgs &a, hipStream_t s);       // BL, A, B per sample
-void launch_update_bitlines(const UpdateArgs &a, hipStream_t s);      // stochastic pulse words
+void launch_update_lines(const UpdateArgs &a, hipStream_t s);         // stochastic pulse words and their bit planes
 void launch_update_implicit_lines(const UpdateArgs &a, hipStream_t s); // deterministic line values
-void launch_update_planes(const UpdateArgs &a, hipStream_t s);        // pulse words -> sample-transposed bit planes
+void launch_update_planes(const UpdateArgs &a, hipStream_t s);        // bit planes of pulse words made elsewhere
 void launch_update_pulsed(const UpdateArgs &a, hipStream_t s);        // coincidences + device steps
 void launch_update_implicit(const UpdateArgs &a, hipStream_t s);
 void launch_implicit_counts(const UpdateArgs &a, int32_t *counts, hipStream_t s);

@@ -116,37 +116,78 @@ __device__ __forceinline__ float discretize_prob(float pp, float res, int sto_ro
   return rintf(q) * res;
 }
 
-// one thread per (sample, line element); x lines first, then d lines
-__global__ __launch_bounds__(256) void k_update_bitlines(UpdateArgs a) {
-  const long per_sample = (long)a.x_size + a.d_size;
-  const long total = per_sample * a.m_batch;
-  for (long idx = blockIdx.x * (long)blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
-    const int b = (int)(idx / per_sample);
-    const int e = (int)(idx % per_sample);
-    const bool is_x = e < a.x_size;
-    const int j = is_x ? e : e - a.x_size;
-    const float v = is_x ? a.x[(long)b * a.x_sb + (long)j * a.x_sj] : a.d[(long)b * a.d_sb + (long)j * a.d_si];
-    const float P = is_x ? a.prob_b[b] : a.prob_a[b];
-    const int K = a.bl[b];
-    const uint32_t purpose = is_x ? RNG_PULSE_X : RNG_PULSE_D;
-    uint32_t sr = 0;
-    if (a.up.res > 0.0f && a.up.sto_round) {
-      sr = philox4x32_10((uint32_t)j, (uint32_t)b, a.call, RNG_UPDATE_SR | ((uint32_t)is_x << 8), a.key.k0, a.key.k1).v[0];
-    }
-    const float PP = discretize_prob(fabsf(v) * P, a.up.res, a.up.sto_round, sr);
-    uint32_t word = 0;
-    if (PP != 0.0f && K > 0) {
-      for (int k0 = 0; k0 < K; k0 += 4) {
-        const Philox4 r = philox4x32_10((uint32_t)j, (uint32_t)b, a.call, purpose | ((uint32_t)(k0 >> 2) << 8), a.key.k0, a.key.k1);
+// packed pulse word of line element j (an x line or a d line) for sample b: bit 0 = sign, bits 1..K = pulses
+__device__ __forceinline__ uint32_t pulse_word(const UpdateArgs &a, bool is_x, int j, int b, float v, float P, int K) {
+  uint32_t sr = 0;
+  if (a.up.res > 0.0f && a.up.sto_round) {
+    sr = philox4x32_10((uint32_t)j, (uint32_t)b, a.call, RNG_UPDATE_SR | ((uint32_t)is_x << 8), a.key.k0, a.key.k1).v[0];
+  }
+  const float PP = discretize_prob(fabsf(v) * P, a.up.res, a.up.sto_round, sr);
+  const uint32_t purpose = is_x ? RNG_PULSE_X : RNG_PULSE_D;
+  uint32_t word = 0;
+  if (PP != 0.0f && K > 0) {
+    for (int k0 = 0; k0 < K; k0 += 4) {
+      const Philox4 r = philox4x32_10((uint32_t)j, (uint32_t)b, a.call, purpose | ((uint32_t)(k0 >> 2) << 8), a.key.k0, a.key.k1);
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          if (k0 + q < K && PP > u32_to_uniform(r.v[q])) word |= (2u << (k0 + q));
-        }
+      for (int q = 0; q < 4; ++q) {
+        if (k0 + q < K && PP > u32_to_uniform(r.v[q])) word |= (2u << (k0 + q));
       }
-      word |= (v > 0.0f) ? 0u : 1u;
     }
-    if (is_x) a.x_words[(long)b * a.x_size + j] = word;
-    else a.d_words[(long)b * a.d_size + j] = word;
+    word |= (v > 0.0f) ? 0u : 1u;
+  }
+  return word;
+}
+
+// Pulse words and their sample-transposed bit planes in one pass.  A workgroup owns 64 samples x 4 line elements
+// (x lines first, then d lines), one element per wave with its lanes on the 64 samples, so that a ballot over the
+// wave is a plane word.  Values and packed words pass through LDS to be read and written 16 bytes per sample row.
+__global__ __launch_bounds__(256) void k_update_lines(UpdateArgs a) {
+  __shared__ float vals[64][5];
+  __shared__ uint32_t wt[64][5];
+  const int tiles_x = (a.x_size + 3) / 4;
+  const bool is_x = (int)blockIdx.x < tiles_x;
+  const int e0 = (is_x ? (int)blockIdx.x : (int)blockIdx.x - tiles_x) * 4;
+  const int size = is_x ? a.x_size : a.d_size;
+  const int b0 = blockIdx.y * 64;
+  const float *src = is_x ? a.x : a.d;
+  const long s_b = is_x ? a.x_sb : a.d_sb, s_e = is_x ? a.x_sj : a.d_si;
+  const int rb = threadIdx.x >> 2, ce = threadIdx.x & 3;
+  {
+    const int b = b0 + rb, e = e0 + ce;
+    vals[rb][ce] = (b < a.m_batch && e < size) ? src[(long)b * s_b + (long)e * s_e] : 0.0f;
+  }
+  __syncthreads();
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int b = b0 + lane;
+  const int e = e0 + wave;
+  if (e < size) {
+    const bool b_ok = b < a.m_batch;
+    const float P = b_ok ? (is_x ? a.prob_b[b] : a.prob_a[b]) : 0.0f;
+    const int K = b_ok ? a.bl[b] : 0;
+    const int kmax = a.kmax[a.kmax_slot];
+    uint32_t *planes = is_x ? a.x_planes : a.d_planes;
+    const int c0 = 2 * blockIdx.y;
+    const uint32_t word = b_ok ? pulse_word(a, is_x, e, b, vals[lane][wave], P, K) : 0u;
+    wt[lane][wave] = word;
+    for (int k = 0; k < kmax; ++k) {
+      const unsigned long long m = __ballot((word >> (k + 1)) & 1u);
+      if (lane == 0) {
+        planes[((long)c0 * a.plane_slots + k) * size + e] = (uint32_t)m;
+        if (c0 + 1 < a.n_chunks) planes[((long)(c0 + 1) * a.plane_slots + k) * size + e] = (uint32_t)(m >> 32);
+      }
+    }
+    const unsigned long long sg = __ballot(word & 1u); // the last slot of a chunk holds the sign bits
+    if (lane == 0) {
+      const int ks = a.plane_slots - 1;
+      planes[((long)c0 * a.plane_slots + ks) * size + e] = (uint32_t)sg;
+      if (c0 + 1 < a.n_chunks) planes[((long)(c0 + 1) * a.plane_slots + ks) * size + e] = (uint32_t)(sg >> 32);
+    }
+  }
+  __syncthreads();
+  {
+    uint32_t *words = is_x ? a.x_words : a.d_words;
+    const int bb = b0 + rb, ee = e0 + ce;
+    if (bb < a.m_batch && ee < size) words[(long)bb * size + ee] = wt[rb][ce];
   }
 }
 
@@ -338,11 +379,13 @@ struct PulseCell {
 // one pulse with the noise factor f = 1 + std * N(0,1) (1 without cycle-to-cycle noise)
 template <int KIND, bool MULT>
 __device__ __forceinline__ float pulse(float w, float slope, float scale, float f, float lo, float hi) {
-  float step;
-  if (KIND == RPU_DEVICE_CONSTANT_STEP) step = scale * f;
-  else if (MULT) step = (slope * w + scale) * f;
-  else step = slope * w + scale * f;
-  return __builtin_amdgcn_fmed3f(w + step, lo, hi);
+  // fused multiply-adds: one rounding less per operation than the reference's separate multiply and add, a
+  // difference of at most half an ulp of w per pulse
+  float wn;
+  if (KIND == RPU_DEVICE_CONSTANT_STEP) wn = __builtin_fmaf(scale, f, w);
+  else if (MULT) wn = __builtin_fmaf(__builtin_fmaf(slope, w, scale), f, w);
+  else wn = __builtin_fmaf(scale, f, __builtin_fmaf(slope, w, w));
+  return __builtin_amdgcn_fmed3f(wn, lo, hi);
 }
 
 // eight noise factors of one cross-point, keyed by (cross-point, refill index)
@@ -622,9 +665,9 @@ void launch_update_prepare(const UpdateArgs &a, hipStream_t s) {
   hipLaunchKernelGGL(k_update_prepare, dim3(a.m_batch), dim3(256), 0, s, a);
 }
 
-void launch_update_bitlines(const UpdateArgs &a, hipStream_t s) {
-  const long total = ((long)a.x_size + a.d_size) * a.m_batch;
-  hipLaunchKernelGGL(k_update_bitlines, dim3(grid_for(total)), dim3(256), 0, s, a);
+void launch_update_lines(const UpdateArgs &a, hipStream_t s) {
+  const dim3 grid((a.x_size + 3) / 4 + (a.d_size + 3) / 4, (a.m_batch + 63) / 64);
+  hipLaunchKernelGGL(k_update_lines, grid, dim3(256), 0, s, a);
 }
 
 void launch_update_implicit_lines(const UpdateArgs &a, hipStream_t s) {

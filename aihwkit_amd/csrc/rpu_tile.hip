@@ -659,10 +659,8 @@ struct Tile {
     launch_update_prepare(a, s);
     prof_mark(s, "update_prepare");
     if (up.p.pulse_type == RPU_PULSE_STOCHASTIC_COMPRESSED) {
-      launch_update_bitlines(a, s);
-      prof_mark(s, "update_bitlines");
-      launch_update_planes(a, s);
-      prof_mark(s, "update_planes");
+      launch_update_lines(a, s);
+      prof_mark(s, "update_lines");
       launch_update_pulsed(a, s);
       prof_mark(s, "update_pulsed");
     } else {
