@@ -80,6 +80,19 @@ int mvm_big_workgroups(const MvmArgs &a);
 void launch_mvm_big_group(const MvmGroup &g, int total_workgroups, hipStream_t s);
 void mvm_round_variant(const MvmArgs &a, int &prefetch_depth, int &weight_mode);
 
+// Fused convolution forward (unfold + noisy MVM with its bound-management rounds) for tiles of at most 32 outputs:
+// images [n_images][image_size], idx_t the transposed index matrix [patches][x_size], out [n_images][d_size][patches].
+// MvmArgs carries the tile (w, sizes, io, key, call, max_rounds, st.rounds, alpha); in / out / xq are not used.
+struct ConvArgs {
+  const float *images;
+  const int *idx_t;
+  float *out;
+  int patches, n_images;
+  long image_size;
+};
+bool conv_forward_supported(const MvmArgs &a);
+void launch_conv_forward(const MvmArgs &a, const ConvArgs &c, hipStream_t s);
+
 // number of rounds that can ever be needed with these IO settings
 int mvm_max_rounds(const IoDev &io);
 // row length of the quantized-input scratch for a contraction length K

@@ -113,33 +113,10 @@ __host__ __device__ __forceinline__ int workgroups_for(int O, int n_act, int edg
   return 8 * ((tiles_o + 7) / 8) * tiles_b;
 }
 
-// ADC stage for outputs o0 .. o0 + 3 of sample b: v holds the analog sums (rpu_forward_backward_pass.cpp:666-719)
-// up / lo return 1 + the largest output index that hit the upper / lower ADC bound (0: none).
-__device__ __forceinline__ void mvm_finish_outputs(const MvmArgs &a, int round, int b, float fin, int o0, float (&v)[4],
-                                                   int &up, int &lo) {
-  up = 0;
-  lo = 0;
-  float *out_p = a.out + (long)b * a.out_sb + (long)o0 * a.out_so;
-  if (a.io.perfect) {
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      if (o0 + q < a.O) {
-        float res = a.alpha * v[q];
-        if (a.beta != 0.0f) res += a.beta * out_p[(long)q * a.out_so];
-        out_p[(long)q * a.out_so] = res;
-      }
-    }
-    return;
-  }
-
-  if (fin == 0.0f) { // zero input: the reference short-cuts to a zero output
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      if (o0 + q < a.O) out_p[(long)q * a.out_so] = 0.0f;
-    }
-    return;
-  }
-
+// ADC of the four analog sums v of outputs o0 .. o0 + 3 of sample b: asymmetry, noise, quantization, clipping, output
+// factor; up / lo return 1 + the largest output index that hit the upper / lower bound (0: none)
+__device__ __forceinline__ void mvm_adc_values(const MvmArgs &a, int round, int b, float fin, int o0, float (&v)[4],
+                                               int &up, int &lo) {
   float nz[4] = {0.f, 0.f, 0.f, 0.f};
   if (a.io.out_noise > 0.0f) {
     philox_normal4((uint32_t)(o0 >> 2), (uint32_t)b, a.call, RNG_OUT_NOISE | ((uint32_t)round << 8), a.key, nz);
@@ -168,6 +145,36 @@ __device__ __forceinline__ void mvm_finish_outputs(const MvmArgs &a, int round, 
   }
   up = hit_u;
   lo = hit_l;
+}
+
+// ADC stage for outputs o0 .. o0 + 3 of sample b: v holds the analog sums (rpu_forward_backward_pass.cpp:666-719)
+// up / lo return 1 + the largest output index that hit the upper / lower ADC bound (0: none).
+__device__ __forceinline__ void mvm_finish_outputs(const MvmArgs &a, int round, int b, float fin, int o0, float (&v)[4],
+                                                   int &up, int &lo) {
+  up = 0;
+  lo = 0;
+  float *out_p = a.out + (long)b * a.out_sb + (long)o0 * a.out_so;
+  if (a.io.perfect) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      if (o0 + q < a.O) {
+        float res = a.alpha * v[q];
+        if (a.beta != 0.0f) res += a.beta * out_p[(long)q * a.out_so];
+        out_p[(long)q * a.out_so] = res;
+      }
+    }
+    return;
+  }
+
+  if (fin == 0.0f) { // zero input: the reference short-cuts to a zero output
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      if (o0 + q < a.O) out_p[(long)q * a.out_so] = 0.0f;
+    }
+    return;
+  }
+
+  mvm_adc_values(a, round, b, fin, o0, v, up, lo);
   if (a.out_so == 1 && (o0 + 3) < a.O && ((((uintptr_t)out_p) & 15) == 0)) {
     *reinterpret_cast<float4 *>(out_p) = make_float4(v[0], v[1], v[2], v[3]);
   } else {
@@ -1129,6 +1136,177 @@ __global__ __launch_bounds__(256, 2) void k_mvm_big_group(MvmGroup g, int round)
   mvm_big_workgroup<0>(a, round, (int)blockIdx.x - g.start[t], 0);
 }
 
+// ---------------------------------------------------------------------------------------------
+// Convolution forward for a tile of at most 32 outputs, fused: unfold by the index matrix, noise management, DAC,
+// contraction, ADC and the bound-management rounds in one kernel, the result written in the image layout
+// [n][output][patch].  A wave owns 32 consecutive patches; it has all outputs of its patches, so whether a patch
+// needs another round (and that round) stays inside the wave: no lists, no scratch matrices, no further launch.
+// The unfolded matrix is never written: element k of patch (n, p) is gathered from the image through the
+// transposed index matrix idx_t[p][k] (0: padding, 1: the bias input, j >= 2: image element j - 2) where it is needed.
+// Random streams, per-patch state and results are those of the unfolded path (same counters: element k, patch number).
+
+typedef int i32x4_unaligned __attribute__((ext_vector_type(4), aligned(4)));
+
+// ONE_STEP: the patch row fits one contraction step (K <= 32, a first convolution layer): the gathered values stay
+// in registers between noise management and the rounds.
+template <bool ONE_STEP>
+__global__ __launch_bounds__(256, 3) void k_conv_forward(MvmArgs a, ConvArgs c) {
+  const int lane = threadIdx.x & 63;
+  const int r = lane & 31, h = lane >> 5;
+  const long tile = blockIdx.x * 4L + (threadIdx.x >> 6);
+  const long total = (long)c.n_images * c.patches;
+  if (tile * 32 >= total) return;
+  const long s_raw = tile * 32 + r;
+  const bool s_ok = s_raw < total;
+  const long sample = s_ok ? s_raw : total - 1;
+  const int n = (int)(sample / c.patches);
+  const int p = (int)(sample - (long)n * c.patches);
+  const float *image = c.images + (long)n * c.image_size;
+  const int *idx_row = c.idx_t + (long)p * a.K;
+  const float *w_row = a.w + (long)min(r, a.O - 1) * a.x_size;
+  const int K = a.K, O = a.O;
+  const int steps = ONE_STEP ? 1 : (K + 31) / 32;
+  const IoDev &io = a.io;
+  const int b = (int)sample; // the patch number keys the random streams
+
+  // the 16 elements k0 .. k0 + 15 of this lane's patch row (zero past K)
+  auto gather16 = [&](int k0, float (&x)[16]) __attribute__((always_inline)) {
+#pragma unroll
+    for (int v4 = 0; v4 < 4; ++v4) {
+      const int k = k0 + 4 * v4;
+      int j[4];
+      if (k + 4 <= K) {
+        const i32x4_unaligned t = *reinterpret_cast<const i32x4_unaligned *>(idx_row + k);
+        j[0] = t.x; j[1] = t.y; j[2] = t.z; j[3] = t.w;
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) j[e] = (k + e < K) ? idx_row[k + e] : 0;
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) x[4 * v4 + e] = (j[e] <= 1) ? (float)j[e] : image[j[e] - 2];
+    }
+  };
+  auto weights16 = [&](int k0, float (&w)[16]) __attribute__((always_inline)) {
+#pragma unroll
+    for (int v4 = 0; v4 < 4; ++v4) {
+      const int k = k0 + 4 * v4;
+      if (k + 4 <= K) {
+        const f32x4_unaligned t = *reinterpret_cast<const f32x4_unaligned *>(w_row + k);
+        w[4 * v4] = t.x; w[4 * v4 + 1] = t.y; w[4 * v4 + 2] = t.z; w[4 * v4 + 3] = t.w;
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) w[4 * v4 + e] = (k + e < K) ? w_row[k + e] : 0.0f;
+      }
+    }
+    if (r >= O) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) w[i] = 0.0f;
+    }
+  };
+
+  float x_keep[16];
+  if (ONE_STEP) gather16(h * 16, x_keep);
+
+  // noise management over the patch row (rpu_forward_backward_pass.cpp:112-178)
+  float nm = 1.0f;
+  if (!io.perfect && (io.noise_management == RPU_NM_ABS_MAX || io.noise_management == RPU_NM_MAX)) {
+    float amax = 0.0f, vmax = -INFINITY;
+    for (int st = 0; st < steps; ++st) {
+      float x[16];
+      if (!ONE_STEP) gather16(st * 32 + h * 16, x);
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const float xv = ONE_STEP ? x_keep[i] : x[i];
+        if (st * 32 + h * 16 + i < K) {
+          amax = fmaxf(amax, fabsf(xv));
+          vmax = fmaxf(vmax, xv);
+        }
+      }
+    }
+    amax = fmaxf(amax, __shfl_xor(amax, 32));
+    vmax = fmaxf(vmax, __shfl_xor(vmax, 32));
+    const float m = io.noise_management == RPU_NM_MAX ? vmax : amax;
+    nm = io.nm_thres > 0.0f ? fminf(m, io.nm_thres) : m;
+  } else if (!io.perfect && io.noise_management == RPU_NM_CONSTANT) {
+    nm = io.nm_thres > 0.0f ? io.nm_thres : 1.0f;
+  }
+  float red = 1.0f, fin = 1.0f, scale = 1.0f;
+  if (!io.perfect) scale = round_scales(a, nm, red, fin);
+  bool active = s_ok;
+  int rounds_run = 0;
+  float *out = c.out + (long)n * O * c.patches + p;
+
+  const int max_rounds = io.perfect ? 1 : a.max_rounds;
+  for (int round = 0; round < max_rounds; ++round) {
+    floatx16 acc;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
+    if (fin != 0.0f || io.perfect) {
+      for (int st = 0; st < steps; ++st) {
+        const int k0 = st * 32 + h * 16;
+        float xd[16], wd[16];
+        if (!ONE_STEP) gather16(k0, xd);
+        weights16(k0, wd);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          float x = ONE_STEP ? x_keep[i] : xd[i];
+          if (!io.perfect && k0 + i < K) x = dac_value(x, scale, io, a.key, a.call, round, b, k0 + i);
+          xd[i] = x;
+        }
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(wd[i], xd[i], acc, 0, 0, 0);
+      }
+    }
+    // ADC: lane (r, h) holds, of patch r, the outputs g * 8 + h * 4 + q
+    int up_max = 0, lo_max = 0;
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const int o0 = g * 8 + h * 4;
+      if (o0 >= O) continue;
+      float v[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) v[q] = acc[4 * g + q];
+      int up = 0, lo = 0;
+      if (io.perfect) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) v[q] *= a.alpha;
+      } else if (fin == 0.0f) { // zero input: the reference short-cuts to a zero output
+#pragma unroll
+        for (int q = 0; q < 4; ++q) v[q] = 0.0f;
+      } else {
+        mvm_adc_values(a, round, b, fin, o0, v, up, lo);
+      }
+      if (active) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          if (o0 + q < O) out[(long)(o0 + q) * c.patches] = v[q];
+        }
+      }
+      up_max = max(up_max, up);
+      lo_max = max(lo_max, lo);
+    }
+    if (active && (io.perfect || fin != 0.0f)) rounds_run = round + 1;
+    if (io.perfect || io.bound_management == RPU_BM_NONE) break;
+    // both halves of the wave hold outputs of patch r
+    up_max = max(up_max, __shfl_xor(up_max, 32));
+    lo_max = max(lo_max, __shfl_xor(lo_max, 32));
+    const bool failed = io.bm_test_negative_bound ? (up_max > 0 || lo_max > 0) : (up_max > lo_max);
+    bool more = false;
+    if (active && failed) {
+      float nm_next = nm, red_next = red;
+      if (next_round_params(a, round, b, fin, nm_next, red_next)) {
+        nm = nm_next;
+        red = red_next;
+        scale = round_scales(a, nm, red, fin);
+        more = true;
+      }
+    }
+    active = more;
+    if (!__any(active)) break;
+  }
+  if (s_ok && !io.perfect && h == 0) a.st.rounds[b] = rounds_run;
+}
+
 // The same for several tiles in one launch: a workgroup finds its tile in the table of first workgroup numbers
 // (a multiple of 8 per tile, so the XCD of a workgroup is the one its tile-local number implies).
 template <int PD, int WMODE>
@@ -1333,6 +1511,21 @@ void launch_mvm_round(const MvmArgs &a_in, hipStream_t s) {
     else RPU_LAUNCH_ROUND(1, 2);
   }
 #undef RPU_LAUNCH_ROUND
+}
+
+bool conv_forward_supported(const MvmArgs &a) {
+  if (a.O > 32 || a.transposed) return false;
+  if (a.io.perfect) return true;
+  const int nm = a.io.noise_management, bm = a.io.bound_management;
+  return (nm == RPU_NM_NONE || nm == RPU_NM_ABS_MAX || nm == RPU_NM_MAX || nm == RPU_NM_CONSTANT) &&
+         (bm == RPU_BM_NONE || bm == RPU_BM_ITERATIVE);
+}
+
+void launch_conv_forward(const MvmArgs &a, const ConvArgs &c, hipStream_t s) {
+  const long tiles = ((long)c.n_images * c.patches + 31) / 32;
+  const dim3 grid((unsigned)((tiles + 3) / 4));
+  if (a.K <= 32) hipLaunchKernelGGL(k_conv_forward<true>, grid, dim3(256), 0, s, a, c);
+  else hipLaunchKernelGGL(k_conv_forward<false>, grid, dim3(256), 0, s, a, c);
 }
 
 void launch_make_bias(const float *in, float *out, int m_batch, int x_size, int in_trans, hipStream_t s) {

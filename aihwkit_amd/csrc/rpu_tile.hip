@@ -170,7 +170,7 @@ struct Tile {
   std::vector<int32_t> idx_host;
   int idx_patches = 0;
   int32_t idx_max = 0; // largest entry of the index matrix
-  DevBuf<int> x_idx;
+  DevBuf<int> x_idx, x_idx_t; // [X][patches] as set, and its transpose [patches][X] for the fused forward
   DevBuf<float> x_mat, d_mat;
   int last_update_batch = 0;
   int last_update_pulse = -1;
@@ -235,7 +235,7 @@ struct Tile {
     t_unit.release(); t_read.release();
     i_ref.release(); i_prog.release(); i_nu_plus.release(); i_nu_minus.release(); i_scalar.release(); i_absmax.release();
     has_reference = programmed = false;
-    x_idx.release(); x_mat.release(); d_mat.release();
+    x_idx.release(); x_idx_t.release(); x_mat.release(); d_mat.release();
     d_decay.release(); d_diff.release(); d_rbias.release(); s_clip.release();
     state_params_valid = false;
     delta_w = nullptr;
@@ -690,6 +690,37 @@ struct Tile {
   }
 
   void forward_indexed(const float *x, float *d, int n_images, long image_size, hipStream_t s) {
+    if (idx_patches <= 0) throw RpuError("The index matrix has not been set (set_matrix_indices).");
+    if (n_images <= 0) throw RpuError("n_images must be positive.");
+    if (D <= 32 && (long)n_images * idx_patches < (1L << 31)) {
+      // narrow tile: unfold, contraction and bound management fused in one kernel, nothing materialized
+      const int B = n_images * idx_patches;
+      ensure_mvm_scratch(B);
+      MvmArgs a{};
+      a.w = wdev(); a.x_size = X; a.d_size = D; a.m_batch = B; a.K = X; a.O = D;
+      a.io = io_dev(fio);
+      a.alpha = fio.p.out_scale;
+      a.max_rounds = fio.perfect ? 0 : mvm_max_rounds(a.io);
+      a.st.rounds = s_rounds.p; a.st.nm_np = s_nmnp.p;
+      if (conv_forward_supported(a)) {
+        if (!x_idx_t.p) {
+          std::vector<int32_t> tr((size_t)X * idx_patches);
+          for (int k = 0; k < X; ++k)
+            for (int p = 0; p < idx_patches; ++p) tr[(size_t)p * X + k] = idx_host[(size_t)k * idx_patches + p];
+          x_idx_t.ensure(tr.size());
+          RPU_HIP_CHECK(hipMemcpy(x_idx_t.p, tr.data(), tr.size() * sizeof(int32_t), hipMemcpyHostToDevice));
+        }
+        a.key = key(); a.call = call++;
+        ConvArgs c{x, x_idx_t.p, d, idx_patches, n_images, image_size};
+        prof_begin(s);
+        launch_conv_forward(a, c, s);
+        prof_mark(s, "conv_forward");
+        RPU_HIP_CHECK(hipGetLastError());
+        last_stream = s;
+        last_forward_batch = B;
+        return;
+      }
+    }
     ensure_indexed(n_images);
     const int B = n_images * idx_patches;
     launch_gather_indexed(x_mat.p, x, x_idx.p, X, idx_patches, n_images, image_size, s);
@@ -1011,6 +1042,7 @@ int rpu_tile_set_matrix_indices(rpu_tile_t *tile, const int32_t *indices_host, i
       DeviceGuard g(t.device_id);
       t.sync_last();
       t.x_idx.release();
+      t.x_idx_t.release();
     }
     t.idx_host.assign(indices_host, indices_host + (size_t)x_size * patches);
     t.idx_max = 0;
