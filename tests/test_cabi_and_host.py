@@ -167,3 +167,39 @@ def test_product_does_not_touch_the_oracle():
         for name in files:
             if name.endswith((".py", ".cpp", ".hip", ".h", "Makefile")):
                 assert "oracle" not in open(os.path.join(base, name), errors="ignore").read().lower(), name
+
+
+def test_extra_state_and_maintenance_calls_on_a_host_tile():
+    """dump_extra / load_extra work without a GPU; the weight maintenance calls compute on the GPU only and say so."""
+    import ctypes as C
+
+    from aihwkit_amd._cabi import lib
+    from aihwkit_amd.rpu_base import devices as dv
+
+    meta = dv.AnalogTileParameter()
+    tile = meta.create_array(6, 4, dv.ConstantStepResistiveDeviceParameter())
+    tile.set_seed(77)
+    state = tile.dump_extra()
+    assert state["rpu.seed"] == 77 and state["rpu.call"] == 0 and set(state) >= {"rpu.update_calls", "rpu.transfer.update_idx"}
+    other = meta.create_array(6, 4, dv.ConstantStepResistiveDeviceParameter())
+    other.load_extra({"rpu.seed": 5, "rpu.call": 9}, False)
+    assert other.dump_extra()["rpu.seed"] == 5 and other.dump_extra()["rpu.call"] == 9
+    with pytest.raises(RuntimeError, match="Cannot find the key"):
+        other.load_extra({"rpu.seed": 5}, True)
+    other.load_extra(state, True)
+    assert other.dump_extra() == state
+    # a transfer compound carries its counters
+    tr = dv.TransferResistiveDeviceParameter()
+    tr.append_parameter(dv.SoftBoundsResistiveDeviceParameter())
+    tr.append_parameter(dv.SoftBoundsResistiveDeviceParameter())
+    compound = meta.create_array(6, 4, tr)
+    assert any(name.startswith("rpu.transfer.slice_idx_") for name in compound.dump_extra())
+    with pytest.raises(RuntimeError):
+        compound.load_extra(state, True)                       # another layout: the slice counters are missing
+    # no CPU compute path: maintenance needs the tile on a GPU
+    for call in (lambda: lib().rpu_tile_decay_weights(tile._h, C.c_float(1.0), 0, None),
+                 lambda: lib().rpu_tile_diffuse_weights(tile._h, None),
+                 lambda: lib().rpu_tile_clip_weights(tile._h, 1, C.c_float(0.1), C.c_float(2.5), None),
+                 lambda: lib().rpu_tile_reset_columns(tile._h, 0, 1, C.c_float(1.0), None)):
+        assert call() != 0 and b"GPU" in lib().rpu_last_error()
+    assert not tile.get_shared_weights_if()
