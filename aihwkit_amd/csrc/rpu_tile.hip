@@ -1116,6 +1116,14 @@ int rpu_tile_reset_columns(rpu_tile_t *tile, int start_column_idx, int num_colum
   RPU_MAINTENANCE_ENTRY(t.reset_columns(start_column_idx, num_columns, reset_prob, (hipStream_t)stream));
 }
 
+int rpu_tile_set_forward_out_scale(rpu_tile_t *tile, float out_scale) {
+  return guarded([&] {
+    if (!tile) throw RpuError("null tile");
+    std::lock_guard<std::mutex> lock(tile->t.mutex);
+    tile->t.fio.p.out_scale = out_scale;
+  });
+}
+
 int rpu_tile_set_shared_weights(rpu_tile_t *tile, float *weights_dev) {
   RPU_MAINTENANCE_ENTRY(t.set_shared_weights(weights_dev));
 }
@@ -1237,6 +1245,11 @@ int rpu_group_destroy(rpu_group_t *group) {
 
 int rpu_group_forward(rpu_group_t *group, const float *const *x_dev, float *const *y_dev, int m_batch, int is_test,
                       void *stream) {
+  return rpu_group_forward_strided(group, x_dev, nullptr, y_dev, nullptr, m_batch, is_test, stream);
+}
+
+int rpu_group_forward_strided(rpu_group_t *group, const float *const *x_dev, const long *x_ld, float *const *y_dev,
+                              const long *y_ld, int m_batch, int is_test, void *stream) {
   (void)is_test;
   return guarded([&] {
     if (!group || !x_dev || !y_dev) throw RpuError("null argument");
@@ -1271,8 +1284,9 @@ int rpu_group_forward(rpu_group_t *group, const float *const *x_dev, float *cons
       t.check_compute(m_batch, x_dev[i], y_dev[i]);
       const bool big = use_big && t.D >= 128;
       MvmArgs a = t.mvm_args(m_batch, false, nullptr, t.fio, big ? 1 : 0);
-      a.in = x_dev[i]; a.in_sb = t.X; a.in_sk = 1;
-      a.out = y_dev[i]; a.out_sb = t.D; a.out_so = 1;
+      a.in = x_dev[i]; a.in_sb = x_ld ? x_ld[i] : t.X; a.in_sk = 1;
+      a.out = y_dev[i]; a.out_sb = y_ld ? y_ld[i] : t.D; a.out_so = 1;
+      if (a.in_sb < t.X || a.out_sb < t.D) throw RpuError("A row stride is shorter than the row.");
       a.big_from = big ? -1 : 0;
       if (!big) all_big = false;
       mvm_round_variant(a, depth[i], mode[i]);

@@ -85,6 +85,8 @@ class InferenceTile:
         self.drift_compensation = drift_compensation
         self.drift_baseline: Optional[float] = None
         self.alpha = 1.0
+        self._out_scale = float(meta.forward_io.out_scale)
+        self._alpha_in_tile = False
 
     def set_weights(self, weights: torch.Tensor) -> None:
         (self.tile or self.host).set_weights(weights)
@@ -106,6 +108,8 @@ class InferenceTile:
         return C.c_void_p(torch.cuda.current_stream().cuda_stream)
 
     def _readout(self) -> float:
+        if self._alpha_in_tile:   # the read-out is of the uncompensated tile
+            check(lib().rpu_tile_set_forward_out_scale(self._gpu()._h, float(self._out_scale)))
         value = C.c_float(0.0)
         check(lib().rpu_tile_drift_readout(self._gpu()._h, C.byref(value), self._stream()))
         return float(value.value)
@@ -119,6 +123,8 @@ class InferenceTile:
         if self.drift_compensation is not None:
             self.drift_baseline = self._readout()
         self.alpha = 1.0
+        if self._alpha_in_tile:
+            self.compensate_in_tile(True)
 
     def drift_weights(self, t_inference: float = 0.0) -> None:
         """inference.py:215-262."""
@@ -128,6 +134,16 @@ class InferenceTile:
                                            self._stream()))
         if self.drift_compensation is not None:
             self.alpha = self.drift_compensation.apply(self._readout(), self.drift_baseline)
+        if self._alpha_in_tile:
+            self.compensate_in_tile(True)
+
+    def compensate_in_tile(self, enable: bool = True) -> None:
+        """Let the drift-compensation factor ride on the tile's ADC stage (its forward ``out_scale``) instead of
+        multiplying the output tensor afterwards; for callers that forward in evaluation mode only, e.g. through a
+        ``TileGroup``.  Call again after ``drift_weights`` / ``program_weights`` changed the factor."""
+        self._alpha_in_tile = bool(enable)
+        scale = self._out_scale * (self.alpha if enable else 1.0)
+        check(lib().rpu_tile_set_forward_out_scale(self._gpu()._h, float(scale)))
 
     def drift_state(self):
         """(programmed weights, drift coefficients of the positive and of the negative conductance), CPU tensors."""
@@ -144,13 +160,13 @@ class InferenceTile:
     def forward_indexed(self, x_input: torch.Tensor, d_tensor: torch.Tensor, is_test: bool = False) -> torch.Tensor:
         """Analog forward of a convolution through the index matrix, drift compensation as in ``forward``."""
         out = self._gpu().forward_indexed(x_input, d_tensor, is_test)
-        if is_test and self.drift_compensation is not None and self.alpha != 1.0:
+        if is_test and self.drift_compensation is not None and self.alpha != 1.0 and not self._alpha_in_tile:
             out.mul_(self.alpha)
         return out
 
     def forward(self, x_input: torch.Tensor, is_test: bool = False) -> torch.Tensor:
         """Analog forward; in evaluation mode the output is scaled by the drift compensation (inference.py:264-282)."""
         out = self._gpu().forward(x_input, False, False, False, is_test, False)
-        if is_test and self.drift_compensation is not None and self.alpha != 1.0:
+        if is_test and self.drift_compensation is not None and self.alpha != 1.0 and not self._alpha_in_tile:
             out = out * self.alpha
         return out

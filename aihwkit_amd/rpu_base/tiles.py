@@ -461,21 +461,43 @@ class TileGroup:
             except Exception:  # pylint: disable=broad-except
                 pass
 
-    def forward(self, x_inputs, is_test: bool = False, non_blocking: bool = False):
-        """x_inputs[i]: CUDA tensor [m_batch, x_size_i]; returns the list of outputs [m_batch, d_size_i]."""
+    @staticmethod
+    def _rows(tensor: torch.Tensor, what: str) -> torch.Tensor:
+        # dense rows or a column slice of a larger row-major matrix
+        if not isinstance(tensor, torch.Tensor) or tensor.dtype != _DTYPE or not tensor.is_cuda:
+            raise RuntimeError(what + " must be a float32 CUDA tensor")
+        if tensor.dim() != 2 or (tensor.shape[1] > 1 and tensor.stride(1) != 1):
+            raise RuntimeError(what + " must be a matrix with unit column stride")
+        return tensor
+
+    def forward(self, x_inputs, is_test: bool = False, non_blocking: bool = False, outs=None):
+        """x_inputs[i]: CUDA tensor [m_batch, x_size_i] (column slices of one matrix are read in place); returns the
+        list of outputs [m_batch, d_size_i].  ``outs`` may give the output tensors, e.g. column slices of one
+        [m_batch, out_total] matrix, which the tiles then fill in place."""
         if len(x_inputs) != len(self._tiles):
             raise RuntimeError("one input per tile expected")
-        xs = [_check_input(x, True, "x_input") for x in x_inputs]
+        xs = [self._rows(x, "x_input") for x in x_inputs]
         m_batch = xs[0].shape[0]
         for x, tile in zip(xs, self._tiles):
-            if x.dim() != 2 or x.shape[0] != m_batch or x.shape[1] != tile.get_x_size():
+            if x.shape[0] != m_batch or x.shape[1] != tile.get_x_size():
                 raise RuntimeError("Invalid x_input dimensions")
-        ys = [torch.empty(m_batch, tile.get_d_size(), dtype=_DTYPE, device=xs[0].device) for tile in self._tiles]
-        x_ptrs = (C.c_void_p * len(xs))(*[x.data_ptr() for x in xs])
-        y_ptrs = (C.c_void_p * len(ys))(*[y.data_ptr() for y in ys])
+        if outs is None:
+            ys = [torch.empty(m_batch, tile.get_d_size(), dtype=_DTYPE, device=xs[0].device) for tile in self._tiles]
+        else:
+            if len(outs) != len(self._tiles):
+                raise RuntimeError("one output per tile expected")
+            ys = [self._rows(y, "output") for y in outs]
+            for y, tile in zip(ys, self._tiles):
+                if y.shape[0] != m_batch or y.shape[1] != tile.get_d_size():
+                    raise RuntimeError("Invalid output dimensions")
+        n = len(xs)
+        x_ptrs = (C.c_void_p * n)(*[x.data_ptr() for x in xs])
+        y_ptrs = (C.c_void_p * n)(*[y.data_ptr() for y in ys])
+        x_ld = (C.c_long * n)(*[x.stride(0) if x.shape[0] > 1 else x.shape[1] for x in xs])
+        y_ld = (C.c_long * n)(*[y.stride(0) if y.shape[0] > 1 else y.shape[1] for y in ys])
         stream = torch.cuda.current_stream(xs[0].device)
-        check(lib().rpu_group_forward(self._g, x_ptrs, y_ptrs, m_batch, int(is_test), C.c_void_p(stream.cuda_stream)))
+        check(lib().rpu_group_forward_strided(self._g, x_ptrs, x_ld, y_ptrs, y_ld, m_batch, int(is_test),
+                                              C.c_void_p(stream.cuda_stream)))
         if not non_blocking:
             stream.synchronize()
         return ys
-

@@ -386,6 +386,7 @@ def bench_config5(args) -> int:
 
     from aihwkit_amd.inference import InferenceTile
     from aihwkit_amd.rpu_base import devices as dv
+    from aihwkit_amd.rpu_base.tiles import TileGroup
     from helpers import io_params
 
     torch.cuda.set_device(0)
@@ -412,27 +413,6 @@ def bench_config5(args) -> int:
         layers.append(grid)
         flops += 2.0 * tokens * in_size * out_size
 
-    from aihwkit_amd.rpu_base.tiles import TileGroup
-
-    # one group per layer: all tiles of the layer in a few launches; partial outputs of the input splits are summed
-    groups = []
-    for grid in layers:
-        flat_tiles = [tile for _, row in grid for tile in row]
-        flat_x = [x_part for x_part, row in grid for _ in row]
-        groups.append((TileGroup([t.tile for t in flat_tiles]), flat_tiles, flat_x, len(grid), len(grid[0][1])))
-
-    def step():
-        outs = []
-        for group, flat_tiles, flat_x, n_in, n_out in groups:
-            ys = group.forward(flat_x, is_test=True, non_blocking=True)
-            ys = [y * t.alpha for y, t in zip(ys, flat_tiles)]            # global drift compensation per tile
-            total = None
-            for i in range(n_in):
-                y = torch.cat(ys[i * n_out:(i + 1) * n_out], dim=1)
-                total = y if total is None else total + y
-            outs.append(total)
-        return outs
-
     def step_per_tile():
         outs = []
         for grid in layers:
@@ -451,6 +431,33 @@ def bench_config5(args) -> int:
         step_per_tile()
     torch.cuda.synchronize()
     ms_per_tile_loop = (time.perf_counter() - t0) * 1e3 / max(args.steps // 4, 3)
+
+    # one group per layer: all tiles of the layer in a few launches.  The tiles read column slices of the layer input
+    # and write column slices of one partial-output matrix per input split in place; the drift-compensation factor of
+    # a tile rides on its ADC stage; the partial outputs of the input splits are summed digitally.
+    groups = []
+    for li, grid in enumerate(layers):
+        in_size, out_size, in_split, out_split = CONFIG5_LAYERS[li]
+        x_layer = torch.cat([x_part for x_part, _ in grid], dim=1)                       # [tokens, in_size]
+        partial = torch.empty(len(in_split), tokens, out_size, device="cuda")
+        flat_tiles, flat_x, flat_y, i0 = [], [], [], 0
+        for i, (n_in, (_, row)) in enumerate(zip(in_split, grid)):
+            o0 = 0
+            for tile, n_out in zip(row, out_split):
+                tile.compensate_in_tile(True)
+                flat_tiles.append(tile)
+                flat_x.append(x_layer[:, i0:i0 + n_in])
+                flat_y.append(partial[i][:, o0:o0 + n_out])
+                o0 += n_out
+            i0 += n_in
+        groups.append((TileGroup([t.tile for t in flat_tiles]), flat_x, flat_y, partial))
+
+    def step():
+        outs = []
+        for group, flat_x, flat_y, partial in groups:
+            group.forward(flat_x, is_test=True, non_blocking=True, outs=flat_y)
+            outs.append(partial.sum(dim=0) if partial.shape[0] > 1 else partial[0])
+        return outs
 
     for _ in range(args.warmup):
         step()

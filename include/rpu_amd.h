@@ -371,6 +371,11 @@ typedef struct rpu_group rpu_group_t; /* opaque */
 int rpu_group_create(rpu_group_t **out, rpu_tile_t *const *tiles, int n_tiles);
 int rpu_group_forward(rpu_group_t *group, const float *const *x_dev, float *const *y_dev, int m_batch,
                       int is_test, void *stream);
+/* The same with a row stride (in floats) per input and output, so that the tiles of a layer read column slices of
+ * the layer's input [m_batch][in_total] and write column slices of one output [m_batch][out_total] in place
+ * (what array.py:155-182 does with torch.split / torch.cat); null strides mean dense rows. */
+int rpu_group_forward_strided(rpu_group_t *group, const float *const *x_dev, const long *x_ld, float *const *y_dev,
+                              const long *y_ld, int m_batch, int is_test, void *stream);
 int rpu_group_destroy(rpu_group_t *group);
 
 /* ---- inference weight pipeline ------------------------------------------------------------- */
@@ -429,6 +434,11 @@ int rpu_tile_clip_weights(rpu_tile_t *tile, int clip_type, float fixed_value, fl
  * to reset_bias + reset_std * N(0, 1) and clipped, each element with probability reset_prob
  * (rpu_pulsed_device.cpp:469-494; without bias and bounds on other tiles, rpu_simple_device.cpp:148-168). */
 int rpu_tile_reset_columns(rpu_tile_t *tile, int start_column_idx, int num_columns, float reset_prob, void *stream);
+
+/* Replaces the out_scale of the forward IO parameters (rpu_io_params.out_scale) from now on.  No counterpart in the
+ * reference, which applies run-time output factors such as the drift-compensation alpha to the output tensor in
+ * Python (src/aihwkit/simulator/tiles/inference.py:264-282); here the factor rides on the ADC stage. */
+int rpu_tile_set_forward_out_scale(rpu_tile_t *tile, float out_scale);
 
 /* set_shared_weights (rpu_base_tiles.cpp:215-229, src/rpucuda/rpu.cpp:1384-1398): the tile's weights are copied
  * into the caller's device buffer [d_size][x_size], which is the weight matrix from then on (never freed by

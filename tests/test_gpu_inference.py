@@ -230,3 +230,68 @@ def test_grouped_forward_at_a_token_batch_is_exact_in_exact_arithmetic(gpu_devic
         assert np.array_equal(y.cpu().numpy(), orc.forward(x)), k
         assert np.array_equal(grouped[k].get_bm_rounds(batch).numpy(), orc.bm_rounds(batch)), k
     assert oracles[2].bm_rounds(batch).max() > 1                       # the later rounds were exercised
+
+
+def test_group_reads_and_writes_column_slices_and_compensation_in_the_tile(gpu_device):
+    """Strided group call: inputs as column slices of the layer input, outputs as column slices of one matrix, must
+    give bit for bit what the dense call gives; the drift-compensation factor on the ADC stage equals the multiply."""
+    from aihwkit_amd.rpu_base import tiles as tl
+
+    rng = np.random.default_rng(9)
+    batch, in_sizes, out_sizes = 40, (24, 36), (17, 30, 9)
+    f_io = io_params(inp_res=1 / 254.0, out_res=1 / 254.0, out_noise=0.04, noise_management=dv.NoiseManagementType.AbsMax,
+                     bound_management=dv.BoundManagementType.Iterative)
+    inf_tiles = []
+    for n_in in in_sizes:
+        for n_out in out_sizes:
+            t = InferenceTile(n_out, n_in, forward_io=f_io)
+            t.set_weights(torch.from_numpy(rng.normal(0, 0.1, (n_out, n_in)).astype(np.float32)))
+            t.cuda()
+            t.tile.set_seed(100 + len(inf_tiles))
+            t.drift_weights(1000.0)
+            inf_tiles.append(t)
+    assert all(abs(t.alpha - 1.0) > 1e-3 for t in inf_tiles)
+    x = torch.from_numpy(rng.normal(0, 1, (batch, sum(in_sizes))).astype(np.float32)).cuda()
+    x_slices, i0 = [], 0
+    for n_in in in_sizes:
+        x_slices += [x[:, i0:i0 + n_in]] * len(out_sizes)
+        i0 += n_in
+    group = tl.TileGroup([t.tile for t in inf_tiles])
+    for t in inf_tiles:
+        t.tile.set_seed(5)
+    dense = group.forward([s.contiguous() for s in x_slices], is_test=True)
+    partial = torch.full((len(in_sizes), batch, sum(out_sizes)), 7.0, device="cuda")
+    outs = []
+    for i in range(len(in_sizes)):
+        o0 = 0
+        for n_out in out_sizes:
+            outs.append(partial[i][:, o0:o0 + n_out])
+            o0 += n_out
+    for t in inf_tiles:
+        t.tile.set_seed(5)
+    got = group.forward(x_slices, is_test=True, outs=outs)
+    for k, (a, b) in enumerate(zip(got, dense)):
+        assert torch.equal(a, b), k
+    assert torch.equal(partial[1][:, :out_sizes[0]], dense[len(out_sizes)])
+    # the compensation factor in the tile
+    for t in inf_tiles:
+        t.tile.set_seed(5)
+        t.compensate_in_tile(True)
+    folded = group.forward(x_slices, is_test=True)
+    for t, a, b in zip(inf_tiles, folded, dense):
+        assert torch.allclose(a, b * t.alpha, rtol=1e-6, atol=1e-7)
+    # a later drift step measures the uncompensated tile and renews the factor in the tile
+    t = inf_tiles[0]
+    before = t.alpha
+    t.drift_weights(1.0e6)
+    assert t.alpha > before * 1.01
+    t.tile.set_seed(5)
+    y_tile = t.forward(x_slices[0].contiguous(), is_test=True)
+    t.compensate_in_tile(False)
+    t.tile.set_seed(5)
+    y_mul = t.forward(x_slices[0].contiguous(), is_test=True)
+    assert torch.allclose(y_tile, y_mul, rtol=1e-6, atol=1e-7)
+    with pytest.raises(RuntimeError):
+        group.forward(x_slices, outs=outs[:-1])
+    with pytest.raises(RuntimeError):
+        group.forward([s.t() for s in x_slices])
