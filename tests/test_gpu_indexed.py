@@ -89,3 +89,31 @@ def test_analog_tile_matches_the_indexed_oracle(gpu_device, kernel, stride, padd
     orc.update(x, grad)
     assert np.abs(gpu.get_weights().numpy() - orc_tile.get_weights()).max() <= 1e-5
     assert np.abs(orc_tile.get_weights() - np.clip(w, orc_tile.get_hidden()[1], orc_tile.get_hidden()[0])).max() > 1e-3
+
+
+@pytest.mark.parametrize("c_in", [2, 8])          # patch rows of 19 (one contraction step) and 73 elements (three)
+def test_fused_convolution_forward_is_bit_exact_with_bound_management_rounds(gpu_device, c_in):
+    """Exact arithmetic (power-of-two DAC step, weights on a 1/64 grid) with weights large enough to saturate the ADC:
+    outputs and rounds per patch of the fused kernel must equal the oracle's to the last bit."""
+    rng = np.random.default_rng(2)
+    c_out, height, width, n = 20, 9, 8, 13
+    indices, patches = conv_indices((c_in, height, width), (3, 3), (1, 1), (1, 1), (1, 1), True)
+    x_size = c_in * 9 + 1
+    f_io = noise_free_io(inp_res=1 / 128.0, out_res=1 / 512.0, out_bound=4.0, noise_management=dv.NoiseManagementType.AbsMax,
+                         bound_management=dv.BoundManagementType.Iterative)
+    meta = make_meta(f_io, noise_free_io())
+    dev = constant_step(w_max_dtod=0.0, w_min_dtod=0.0, w_max=1.0, w_min=-1.0, construction_seed=3)
+    host, orc_tile, _ = build_pair(meta, dev, x_size, c_out, gpu=False)
+    w = (rng.integers(-60, 61, (c_out, x_size)) / 64.0).astype(np.float32)
+    host.set_weights(torch.from_numpy(w))
+    orc_tile.set_weights(w)
+    gpu = tiles.CudaAnalogTile(host)
+    gpu.set_matrix_indices(indices)
+    x = rng.uniform(-1, 1, (n, c_in, height, width)).astype(np.float32)
+    x[0] = 0.0                                                          # patches of zeros: the zero short-cut
+    y = gpu.forward_indexed(cuda(x), torch.empty(n, c_out, height, width).cuda()).cpu().numpy().reshape(n, c_out, patches)
+    want = IndexedOracle(orc_tile, indices.numpy(), patches).forward(x)
+    assert np.array_equal(y, want)
+    rounds = orc_tile.bm_rounds(n * patches)
+    assert rounds.max() > 1 and rounds.min() >= 1
+    assert np.array_equal(gpu.get_bm_rounds(n * patches).numpy(), rounds)
