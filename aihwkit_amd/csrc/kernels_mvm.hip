@@ -21,6 +21,14 @@
 //                  last workgroup to finish a sample tile (a device-scope counter per tile and round) decides
 //                  which of its 32 samples need that round and appends them to its list; no kernel sits
 //                  between two rounds.
+//   k_mvm_round_tail   later rounds of a launch whose full grid would be large: a fixed number of workgroups walk
+//                  the tiles of the samples that are listed (usually few).
+//   k_mvm_big      large batches on wide tiles: 128 x 128 workgroup tiles, both operands staged through LDS and
+//                  shared by the four waves (64 x 64 per wave), same state / epilogue / random streams; a round is
+//                  run by this or by the 32 x 32 kernel, by the number of samples it lists.
+//   k_conv_forward convolution forward of a narrow tile (at most 32 outputs): unfold by the index matrix, noise
+//                  management, DAC, contraction, ADC and the bound-management rounds in one kernel.
+//   *_group        the same kernels over the tiles of a group in one launch.
 #include "kernels.h"
 
 namespace rpu_amd {
@@ -797,8 +805,7 @@ __global__ __launch_bounds__(256) void k_mvm_round_tail(MvmArgs a) {
 }
 
 // The same for a group: the workgroups first find out, one thread per tile, how many 32 x 32 tiles each member has
-// listed for this round (usually none), then walk the concatenation of those.  tile_first .. tile_first + n_tiles
-// are the group members of this launch's kernel variant.
+// listed for this round (usually none), then walk the concatenation of those.
 constexpr int MAX_GROUP = 1024;
 
 template <int WMODE>
