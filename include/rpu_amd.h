@@ -20,6 +20,10 @@
  *    (R/rpu.h:674, B/rpu_base_tiles.cpp:161-214).
  *  - compute entry points (forward / backward / update) exist for GPU-resident
  *    tiles only.  There is no CPU compute path in this library.
+ *  - a tile owns its scratch memory (per-sample state, quantized inputs, pulse words): calls on one tile
+ *    must be ordered on the device, i.e. issued on one stream or on streams the caller orders with events.
+ *    Calls on different tiles are independent.  The library allocates device memory when a tile first meets
+ *    a larger batch; after that, calls with the same or smaller shapes allocate nothing.
  */
 #ifndef RPU_AMD_H
 #define RPU_AMD_H
