@@ -1314,6 +1314,172 @@ __global__ __launch_bounds__(256, 3) void k_conv_forward(MvmArgs a, ConvArgs c) 
   if (s_ok && !io.perfect && h == 0) a.st.rounds[b] = rounds_run;
 }
 
+// Long patch rows (more than two contraction steps): one workgroup per 32 patches, its four waves share the patches
+// and deal the contraction steps among themselves (partial sums added through LDS in a fixed order, each wave then
+// finishes 8 of the 32 output rows).  Every wave keeps the per-patch state, so the round loop is workgroup-uniform.
+__global__ __launch_bounds__(256) void k_conv_forward_split(MvmArgs a, ConvArgs c) {
+  __shared__ float red[WAVES][16][64];
+  __shared__ float sh_max[2][WAVES][32];
+  __shared__ int sh_hits[2][32];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 31, h = lane >> 5;
+  const long tile = blockIdx.x;
+  const long total = (long)c.n_images * c.patches;
+  const long s_raw = tile * 32 + r;
+  const bool s_ok = s_raw < total;
+  const long sample = s_ok ? s_raw : total - 1;
+  const int n = (int)(sample / c.patches);
+  const int p = (int)(sample - (long)n * c.patches);
+  const float *image = c.images + (long)n * c.image_size;
+  const int *idx_row = c.idx_t + (long)p * a.K;
+  const float *w_row = a.w + (long)min(r, a.O - 1) * a.x_size;
+  const int K = a.K, O = a.O;
+  const int steps = (K + 31) / 32;
+  const IoDev &io = a.io;
+  const int b = (int)sample;
+
+  auto gather16 = [&](int k0, float (&x)[16]) __attribute__((always_inline)) {
+#pragma unroll
+    for (int v4 = 0; v4 < 4; ++v4) {
+      const int k = k0 + 4 * v4;
+      int j[4];
+      if (k + 4 <= K) {
+        const i32x4_unaligned t = *reinterpret_cast<const i32x4_unaligned *>(idx_row + k);
+        j[0] = t.x; j[1] = t.y; j[2] = t.z; j[3] = t.w;
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) j[e] = (k + e < K) ? idx_row[k + e] : 0;
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) x[4 * v4 + e] = (j[e] <= 1) ? (float)j[e] : image[j[e] - 2];
+    }
+  };
+  auto weights16 = [&](int k0, float (&w)[16]) __attribute__((always_inline)) {
+#pragma unroll
+    for (int v4 = 0; v4 < 4; ++v4) {
+      const int k = k0 + 4 * v4;
+      if (k + 4 <= K) {
+        const f32x4_unaligned t = *reinterpret_cast<const f32x4_unaligned *>(w_row + k);
+        w[4 * v4] = t.x; w[4 * v4 + 1] = t.y; w[4 * v4 + 2] = t.z; w[4 * v4 + 3] = t.w;
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) w[4 * v4 + e] = (k + e < K) ? w_row[k + e] : 0.0f;
+      }
+    }
+    if (r >= O) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) w[i] = 0.0f;
+    }
+  };
+
+  float nm = 1.0f;
+  if (!io.perfect && (io.noise_management == RPU_NM_ABS_MAX || io.noise_management == RPU_NM_MAX)) {
+    float amax = 0.0f, vmax = -INFINITY;
+    for (int st = wave; st < steps; st += WAVES) {
+      float x[16];
+      gather16(st * 32 + h * 16, x);
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        if (st * 32 + h * 16 + i < K) {
+          amax = fmaxf(amax, fabsf(x[i]));
+          vmax = fmaxf(vmax, x[i]);
+        }
+      }
+    }
+    amax = fmaxf(amax, __shfl_xor(amax, 32));
+    vmax = fmaxf(vmax, __shfl_xor(vmax, 32));
+    if (h == 0) {
+      sh_max[0][wave][r] = amax;
+      sh_max[1][wave][r] = vmax;
+    }
+    __syncthreads();
+    amax = fmaxf(fmaxf(sh_max[0][0][r], sh_max[0][1][r]), fmaxf(sh_max[0][2][r], sh_max[0][3][r]));
+    vmax = fmaxf(fmaxf(sh_max[1][0][r], sh_max[1][1][r]), fmaxf(sh_max[1][2][r], sh_max[1][3][r]));
+    const float m = io.noise_management == RPU_NM_MAX ? vmax : amax;
+    nm = io.nm_thres > 0.0f ? fminf(m, io.nm_thres) : m;
+  } else if (!io.perfect && io.noise_management == RPU_NM_CONSTANT) {
+    nm = io.nm_thres > 0.0f ? io.nm_thres : 1.0f;
+  }
+  float red_f = 1.0f, fin = 1.0f, scale = 1.0f;
+  if (!io.perfect) scale = round_scales(a, nm, red_f, fin);
+  bool active = s_ok;
+  int rounds_run = 0;
+  float *out = c.out + (long)n * O * c.patches + p;
+
+  const int max_rounds = io.perfect ? 1 : a.max_rounds;
+  for (int round = 0; round < max_rounds; ++round) {
+    floatx16 acc;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
+    if (fin != 0.0f || io.perfect) {
+      for (int st = wave; st < steps; st += WAVES) {
+        const int k0 = st * 32 + h * 16;
+        float xd[16], wd[16];
+        gather16(k0, xd);
+        weights16(k0, wd);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          if (!io.perfect && k0 + i < K) xd[i] = dac_value(xd[i], scale, io, a.key, a.call, round, b, k0 + i);
+        }
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(wd[i], xd[i], acc, 0, 0, 0);
+      }
+    }
+    if (threadIdx.x < 64) sh_hits[threadIdx.x >> 5][threadIdx.x & 31] = 0;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) red[wave][i][lane] = acc[i];
+    __syncthreads();
+    // this wave finishes the output rows wave * 8 + h * 4 + q of patch r
+    {
+      const int o0 = wave * 8 + h * 4;
+      float v[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int i = wave * 4 + q;
+        v[q] = ((red[0][i][lane] + red[1][i][lane]) + red[2][i][lane]) + red[3][i][lane];
+      }
+      int up = 0, lo = 0;
+      if (o0 < O) {
+        if (io.perfect) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) v[q] *= a.alpha;
+        } else if (fin == 0.0f) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) v[q] = 0.0f;
+        } else {
+          mvm_adc_values(a, round, b, fin, o0, v, up, lo);
+        }
+        if (active) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            if (o0 + q < O) out[(long)(o0 + q) * c.patches] = v[q];
+          }
+        }
+      }
+      if (up) atomicMax(&sh_hits[0][r], up);
+      if (lo) atomicMax(&sh_hits[1][r], lo);
+    }
+    if (active && (io.perfect || fin != 0.0f)) rounds_run = round + 1;
+    if (io.perfect || io.bound_management == RPU_BM_NONE) break;
+    __syncthreads();
+    const int up_max = sh_hits[0][r], lo_max = sh_hits[1][r];
+    const bool failed = io.bm_test_negative_bound ? (up_max > 0 || lo_max > 0) : (up_max > lo_max);
+    bool more = false;
+    if (active && failed) {
+      float nm_next = nm, red_next = red_f;
+      if (next_round_params(a, round, b, fin, nm_next, red_next)) {
+        nm = nm_next;
+        red_f = red_next;
+        scale = round_scales(a, nm, red_f, fin);
+        more = true;
+      }
+    }
+    active = more;
+    if (!__syncthreads_or(active ? 1 : 0)) break; // also keeps red / sh_hits until every wave has read them
+  }
+  if (s_ok && !io.perfect && wave == 0 && h == 0) a.st.rounds[b] = rounds_run;
+}
+
 // The same for several tiles in one launch: a workgroup finds its tile in the table of first workgroup numbers
 // (a multiple of 8 per tile, so the XCD of a workgroup is the one its tile-local number implies).
 template <int PD, int WMODE>
@@ -1532,7 +1698,8 @@ void launch_conv_forward(const MvmArgs &a, const ConvArgs &c, hipStream_t s) {
   const long tiles = ((long)c.n_images * c.patches + 31) / 32;
   const dim3 grid((unsigned)((tiles + 3) / 4));
   if (a.K <= 32) hipLaunchKernelGGL(k_conv_forward<true>, grid, dim3(256), 0, s, a, c);
-  else hipLaunchKernelGGL(k_conv_forward<false>, grid, dim3(256), 0, s, a, c);
+  else if (a.K <= 64) hipLaunchKernelGGL(k_conv_forward<false>, grid, dim3(256), 0, s, a, c);
+  else hipLaunchKernelGGL(k_conv_forward_split, dim3((unsigned)tiles), dim3(256), 0, s, a, c);
 }
 
 void launch_make_bias(const float *in, float *out, int m_batch, int x_size, int in_trans, hipStream_t s) {
