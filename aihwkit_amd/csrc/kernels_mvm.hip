@@ -1134,13 +1134,14 @@ __global__ __launch_bounds__(256, 2) void k_mvm_big(MvmArgs a, int min_active) {
   mvm_big_workgroup<WT>(a, a.round, (int)blockIdx.x, min_active);
 }
 
-// several tiles in one launch (forward, round 0): a tile that is not run by this kernel has no workgroups in the table
+// several tiles in one launch (round 0): a tile that is not run by this kernel has no workgroups in the table
+template <int WT>
 __global__ __launch_bounds__(256, 2) void k_mvm_big_group(MvmGroup g, int round) {
   int t = 0;
   while (t + 1 < g.n && (int)blockIdx.x >= g.start[t + 1]) ++t;
   const MvmArgs &a = g.args[t];
   if (round > 0 && round >= a.max_rounds) return;
-  mvm_big_workgroup<0>(a, round, (int)blockIdx.x - g.start[t], 0);
+  mvm_big_workgroup<WT>(a, round, (int)blockIdx.x - g.start[t], 0);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -1607,8 +1608,9 @@ static int big_workgroups(const MvmArgs &a) {
 
 int mvm_big_workgroups(const MvmArgs &a) { return a.O >= 128 ? big_workgroups(a) : 0; }
 
-void launch_mvm_big_group(const MvmGroup &g, int total_workgroups, hipStream_t s) {
-  hipLaunchKernelGGL(k_mvm_big_group, dim3(total_workgroups), dim3(256), 0, s, g, 0);
+void launch_mvm_big_group(const MvmGroup &g, int total_workgroups, bool transposed, hipStream_t s) {
+  if (transposed) hipLaunchKernelGGL(k_mvm_big_group<1>, dim3(total_workgroups), dim3(256), 0, s, g, 0);
+  else hipLaunchKernelGGL(k_mvm_big_group<0>, dim3(total_workgroups), dim3(256), 0, s, g, 0);
 }
 
 // samples of a round from which the large-tile kernel takes over, 0 when a call of this shape never uses it: it

@@ -1243,6 +1243,9 @@ int rpu_group_destroy(rpu_group_t *group) {
   return guarded([&] { delete group; });
 }
 
+static int group_mvm(rpu_group_t *group, const float *const *x_dev, const long *x_ld, float *const *y_dev,
+                     const long *y_ld, int m_batch, bool transposed, void *stream);
+
 int rpu_group_forward(rpu_group_t *group, const float *const *x_dev, float *const *y_dev, int m_batch, int is_test,
                       void *stream) {
   return rpu_group_forward_strided(group, x_dev, nullptr, y_dev, nullptr, m_batch, is_test, stream);
@@ -1251,6 +1254,17 @@ int rpu_group_forward(rpu_group_t *group, const float *const *x_dev, float *cons
 int rpu_group_forward_strided(rpu_group_t *group, const float *const *x_dev, const long *x_ld, float *const *y_dev,
                               const long *y_ld, int m_batch, int is_test, void *stream) {
   (void)is_test;
+  return group_mvm(group, x_dev, x_ld, y_dev, y_ld, m_batch, false, stream);
+}
+
+int rpu_group_backward_strided(rpu_group_t *group, const float *const *d_dev, const long *d_ld, float *const *x_dev,
+                               const long *x_ld, int m_batch, void *stream) {
+  return group_mvm(group, d_dev, d_ld, x_dev, x_ld, m_batch, true, stream);
+}
+
+// forward (inputs x, outputs y) or backward (inputs d, outputs x) of all tiles of a group
+static int group_mvm(rpu_group_t *group, const float *const *x_dev, const long *x_ld, float *const *y_dev,
+                     const long *y_ld, int m_batch, bool transposed, void *stream) {
   return guarded([&] {
     if (!group || !x_dev || !y_dev) throw RpuError("null argument");
     if (m_batch <= 0) throw RpuError("m_batch must be positive.");
@@ -1267,7 +1281,7 @@ int rpu_group_forward_strided(rpu_group_t *group, const float *const *x_dev, con
     if (m_batch >= 1024) {
       for (int i = 0; i < n; ++i) {
         MvmArgs shape{};
-        shape.O = group->tiles[i]->t.D;
+        shape.O = transposed ? group->tiles[i]->t.X : group->tiles[i]->t.D;
         shape.m_batch = m_batch;
         big_total += mvm_big_workgroups(shape);
       }
@@ -1282,18 +1296,19 @@ int rpu_group_forward_strided(rpu_group_t *group, const float *const *x_dev, con
       Tile &t = group->tiles[i]->t;
       std::lock_guard<std::mutex> lock(t.mutex);
       t.check_compute(m_batch, x_dev[i], y_dev[i]);
-      const bool big = use_big && t.D >= 128;
-      MvmArgs a = t.mvm_args(m_batch, false, nullptr, t.fio, big ? 1 : 0);
-      a.in = x_dev[i]; a.in_sb = x_ld ? x_ld[i] : t.X; a.in_sk = 1;
-      a.out = y_dev[i]; a.out_sb = y_ld ? y_ld[i] : t.D; a.out_so = 1;
-      if (a.in_sb < t.X || a.out_sb < t.D) throw RpuError("A row stride is shorter than the row.");
+      const int in_size = transposed ? t.D : t.X, out_size = transposed ? t.X : t.D;
+      const bool big = use_big && out_size >= 128;
+      MvmArgs a = t.mvm_args(m_batch, transposed, nullptr, transposed ? t.bio : t.fio, big ? 1 : 0);
+      a.in = x_dev[i]; a.in_sb = x_ld ? x_ld[i] : in_size; a.in_sk = 1;
+      a.out = y_dev[i]; a.out_sb = y_ld ? y_ld[i] : out_size; a.out_so = 1;
+      if (a.in_sb < in_size || a.out_sb < out_size) throw RpuError("A row stride is shorter than the row.");
       a.big_from = big ? -1 : 0;
       if (!big) all_big = false;
       mvm_round_variant(a, depth[i], mode[i]);
       rounds = std::max(rounds, a.max_rounds);
       args[i] = a;
       t.last_stream = s;
-      t.last_forward_batch = m_batch;
+      if (!transposed) t.last_forward_batch = m_batch;
     }
     // tiles that share a kernel variant sit next to each other
     std::vector<int> order(n);
@@ -1338,7 +1353,7 @@ int rpu_group_forward_strided(rpu_group_t *group, const float *const *x_dev, con
     for (int r = 0; r < rounds; ++r) {
       if (use_big && r == 0) {
         MvmGroup g{group->d_args.p, group->d_start.p + big_offset, n, m_batch};
-        launch_mvm_big_group(g, big_total, s);
+        launch_mvm_big_group(g, big_total, transposed, s);
         if (all_big) continue;
       }
       for (const Segment &seg : segments) {

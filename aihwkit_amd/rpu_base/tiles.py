@@ -470,6 +470,36 @@ class TileGroup:
             raise RuntimeError(what + " must be a matrix with unit column stride")
         return tensor
 
+    def backward(self, d_inputs, non_blocking: bool = False, outs=None):
+        """d_inputs[i]: CUDA tensor [m_batch, d_size_i]; returns the input gradients [m_batch, x_size_i] of every tile
+        (``outs``: tensors to fill, e.g. column slices), each what the tile's own ``backward`` gives."""
+        if len(d_inputs) != len(self._tiles):
+            raise RuntimeError("one input per tile expected")
+        ds = [self._rows(d, "d_input") for d in d_inputs]
+        m_batch = ds[0].shape[0]
+        for d, tile in zip(ds, self._tiles):
+            if d.shape[0] != m_batch or d.shape[1] != tile.get_d_size():
+                raise RuntimeError("Invalid d_input dimensions")
+        if outs is None:
+            xs = [torch.empty(m_batch, tile.get_x_size(), dtype=_DTYPE, device=ds[0].device) for tile in self._tiles]
+        else:
+            if len(outs) != len(self._tiles):
+                raise RuntimeError("one output per tile expected")
+            xs = [self._rows(x, "output") for x in outs]
+            for x, tile in zip(xs, self._tiles):
+                if x.shape[0] != m_batch or x.shape[1] != tile.get_x_size():
+                    raise RuntimeError("Invalid output dimensions")
+        n = len(ds)
+        d_ptrs = (C.c_void_p * n)(*[d.data_ptr() for d in ds])
+        x_ptrs = (C.c_void_p * n)(*[x.data_ptr() for x in xs])
+        d_ld = (C.c_long * n)(*[d.stride(0) if d.shape[0] > 1 else d.shape[1] for d in ds])
+        x_ld = (C.c_long * n)(*[x.stride(0) if x.shape[0] > 1 else x.shape[1] for x in xs])
+        stream = torch.cuda.current_stream(ds[0].device)
+        check(lib().rpu_group_backward_strided(self._g, d_ptrs, d_ld, x_ptrs, x_ld, m_batch, C.c_void_p(stream.cuda_stream)))
+        if not non_blocking:
+            stream.synchronize()
+        return xs
+
     def forward(self, x_inputs, is_test: bool = False, non_blocking: bool = False, outs=None):
         """x_inputs[i]: CUDA tensor [m_batch, x_size_i] (column slices of one matrix are read in place); returns the
         list of outputs [m_batch, d_size_i].  ``outs`` may give the output tensors, e.g. column slices of one

@@ -380,6 +380,11 @@ int rpu_group_forward(rpu_group_t *group, const float *const *x_dev, float *cons
  * (what array.py:155-182 does with torch.split / torch.cat); null strides mean dense rows. */
 int rpu_group_forward_strided(rpu_group_t *group, const float *const *x_dev, const long *x_ld, float *const *y_dev,
                               const long *y_ld, int m_batch, int is_test, void *stream);
+/* Backward pass of all tiles of the group: d_dev[i] is [m_batch][d_size_i] with row stride d_ld[i], x_dev[i] receives
+ * [m_batch][x_size_i] with row stride x_ld[i] (null strides: dense rows); every tile gets what rpu_tile_backward
+ * gives it. */
+int rpu_group_backward_strided(rpu_group_t *group, const float *const *d_dev, const long *d_ld, float *const *x_dev,
+                               const long *x_ld, int m_batch, void *stream);
 int rpu_group_destroy(rpu_group_t *group);
 
 /* ---- inference weight pipeline ------------------------------------------------------------- */

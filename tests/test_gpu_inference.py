@@ -295,3 +295,39 @@ def test_group_reads_and_writes_column_slices_and_compensation_in_the_tile(gpu_d
         group.forward(x_slices, outs=outs[:-1])
     with pytest.raises(RuntimeError):
         group.forward([s.t() for s in x_slices])
+
+
+def test_grouped_backward_equals_the_tiles_own_backward(gpu_device):
+    """Noisy backward pass (abs-max noise management) of tiles of different shapes: the group call gives every tile bit
+    for bit what its own backward call gives for the same seed and call counter; strided gradients are filled in place."""
+    import copy
+
+    from aihwkit_amd.rpu_base import tiles as tl
+    from helpers import build_pair, constant_step
+
+    rng = np.random.default_rng(12)
+    shapes = [(384, 461), (512, 384), (100, 70), (129, 10)]            # (x_size, d_size)
+    batch = 80
+    b_io = io_params(inp_res=1 / 254.0, out_res=1 / 254.0, out_noise=0.04, noise_management=dv.NoiseManagementType.AbsMax)
+    singles, grouped, ds = [], [], []
+    for k, (x_size, d_size) in enumerate(shapes):
+        _, _, gpu = build_pair(make_meta(noise_free_io(), b_io), constant_step(construction_seed=k + 1), x_size, d_size)
+        gpu.set_weights(torch.from_numpy(rng.normal(0, 0.1, (d_size, x_size)).astype(np.float32)))
+        gpu.set_seed(60 + k)
+        singles.append(gpu)
+        grouped.append(copy.deepcopy(gpu))
+        grouped[-1].set_seed(60 + k)
+        ds.append(torch.from_numpy(rng.normal(0, 0.3, (batch, d_size)).astype(np.float32)).cuda())
+    group = tl.TileGroup(grouped)
+    all_x = torch.zeros(batch, sum(x for x, _ in shapes), device="cuda")
+    outs, i0 = [], 0
+    for x_size, _ in shapes:
+        outs.append(all_x[:, i0:i0 + x_size])
+        i0 += x_size
+    for rep in range(2):
+        want = [t.backward(d, False, False, False, False) for t, d in zip(singles, ds)]
+        got = group.backward(ds, outs=outs if rep else None)
+        for k, (a, b) in enumerate(zip(got, want)):
+            assert torch.equal(a, b), (rep, k)
+    assert torch.equal(all_x[:, :shapes[0][0]], want[0])
+    assert want[0].abs().max() > 0.1
