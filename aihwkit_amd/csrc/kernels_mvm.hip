@@ -907,6 +907,19 @@ __device__ __forceinline__ void big_prepare_next_rows(const MvmArgs &a, int roun
   }
 }
 
+// Instruction order of 16 MFMAs and the LDS reads of the operands that follow them (a hint to the scheduler): the
+// reads are spread behind the first MFMAs so that they complete underneath the rest.
+template <int WT>
+__device__ __forceinline__ void mvm_big_schedule() {
+  // WT = 0: 4 wide LDS reads; WT = 1: 2 wide reads and the 8 single reads of the transposed weight tile
+#pragma unroll
+  for (int i = 0; i < (WT == 0 ? 4 : 6); ++i) {
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); // one MFMA
+    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); // one LDS read
+  }
+  __builtin_amdgcn_sched_group_barrier(0x008, WT == 0 ? 12 : 10, 0);
+}
+
 // work of workgroup number n of a large-tile round launch of one tile
 template <int WT>
 __device__ __forceinline__ void mvm_big_workgroup(const MvmArgs &a, const int round, const int n, const int min_active) {
@@ -1012,36 +1025,52 @@ __device__ __forceinline__ void mvm_big_workgroup(const MvmArgs &a, const int ro
     acc11[i] = 0.0f;
   }
 
-  // lane (r, h) multiplies k = 16 h .. 16 h + 15 of a stage, four values at a time
-  auto compute = [&](int buf) __attribute__((always_inline)) {
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const int kk = h * 16 + q * 4;
-      const f32x4 xb0 = *reinterpret_cast<const f32x4 *>(&lds_x[buf][(wx * 64 + r) * BPITCH + kk]);
-      const f32x4 xb1 = *reinterpret_cast<const f32x4 *>(&lds_x[buf][(wx * 64 + 32 + r) * BPITCH + kk]);
-      f32x4 wa0, wa1;
-      if (WT == 0) {
-        wa0 = *reinterpret_cast<const f32x4 *>(&lds_w[buf][(wy * 64 + r) * BPITCH + kk]);
-        wa1 = *reinterpret_cast<const f32x4 *>(&lds_w[buf][(wy * 64 + 32 + r) * BPITCH + kk]);
-      } else {
-        const float *col = &lds_w[buf][kk * BPITCH_T + wy * 64 + r];
-        wa0.x = col[0];
-        wa0.y = col[BPITCH_T];
-        wa0.z = col[2 * BPITCH_T];
-        wa0.w = col[3 * BPITCH_T];
-        wa1.x = col[32];
-        wa1.y = col[BPITCH_T + 32];
-        wa1.z = col[2 * BPITCH_T + 32];
-        wa1.w = col[3 * BPITCH_T + 32];
-      }
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        acc00 = __builtin_amdgcn_mfma_f32_32x32x2f32(wa0[e], xb0[e], acc00, 0, 0, 0);
-        acc01 = __builtin_amdgcn_mfma_f32_32x32x2f32(wa0[e], xb1[e], acc01, 0, 0, 0);
-        acc10 = __builtin_amdgcn_mfma_f32_32x32x2f32(wa1[e], xb0[e], acc10, 0, 0, 0);
-        acc11 = __builtin_amdgcn_mfma_f32_32x32x2f32(wa1[e], xb1[e], acc11, 0, 0, 0);
-      }
+  // lane (r, h) multiplies k = 16 h .. 16 h + 15 of a stage, four values at a time; the operands of the next four
+  // are read from LDS before the 16 MFMAs of the current four are issued, so that the reads complete underneath them
+  struct Operands {
+    f32x4 xb0, xb1, wa0, wa1;
+  };
+  auto read_operands = [&](int buf, int q, Operands &o) __attribute__((always_inline)) {
+    const int kk = h * 16 + q * 4;
+    o.xb0 = *reinterpret_cast<const f32x4 *>(&lds_x[buf][(wx * 64 + r) * BPITCH + kk]);
+    o.xb1 = *reinterpret_cast<const f32x4 *>(&lds_x[buf][(wx * 64 + 32 + r) * BPITCH + kk]);
+    if (WT == 0) {
+      o.wa0 = *reinterpret_cast<const f32x4 *>(&lds_w[buf][(wy * 64 + r) * BPITCH + kk]);
+      o.wa1 = *reinterpret_cast<const f32x4 *>(&lds_w[buf][(wy * 64 + 32 + r) * BPITCH + kk]);
+    } else {
+      const float *col = &lds_w[buf][kk * BPITCH_T + wy * 64 + r];
+      o.wa0.x = col[0];
+      o.wa0.y = col[BPITCH_T];
+      o.wa0.z = col[2 * BPITCH_T];
+      o.wa0.w = col[3 * BPITCH_T];
+      o.wa1.x = col[32];
+      o.wa1.y = col[BPITCH_T + 32];
+      o.wa1.z = col[2 * BPITCH_T + 32];
+      o.wa1.w = col[3 * BPITCH_T + 32];
     }
+  };
+  auto multiply = [&](const Operands &o) __attribute__((always_inline)) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      acc00 = __builtin_amdgcn_mfma_f32_32x32x2f32(o.wa0[e], o.xb0[e], acc00, 0, 0, 0);
+      acc01 = __builtin_amdgcn_mfma_f32_32x32x2f32(o.wa0[e], o.xb1[e], acc01, 0, 0, 0);
+      acc10 = __builtin_amdgcn_mfma_f32_32x32x2f32(o.wa1[e], o.xb0[e], acc10, 0, 0, 0);
+      acc11 = __builtin_amdgcn_mfma_f32_32x32x2f32(o.wa1[e], o.xb1[e], acc11, 0, 0, 0);
+    }
+  };
+  auto compute = [&](int buf) __attribute__((always_inline)) {
+    Operands even, odd;
+    read_operands(buf, 0, even);
+    read_operands(buf, 1, odd);
+    multiply(even);
+    mvm_big_schedule<WT>();
+    read_operands(buf, 2, even);
+    multiply(odd);
+    mvm_big_schedule<WT>();
+    read_operands(buf, 3, odd);
+    multiply(even);
+    mvm_big_schedule<WT>();
+    multiply(odd);
   };
 
   const int stages = a.k_pad / BKS;
