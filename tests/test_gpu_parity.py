@@ -403,3 +403,41 @@ def test_update_layouts_and_bias_column(gpu_device, x_trans, d_trans, bias):
     assert np.abs(orc.get_weights()).max() > 5e-3
     if bias:  # the bias column saw a constant input of one
         assert np.abs(orc.get_weights()[:, -1]).mean() > np.abs(orc.get_weights()[:, :-1]).mean()
+
+
+@pytest.mark.parametrize("direction", ["forward", "backward"])
+def test_output_noise_of_the_large_tile_kernel_is_standard_normal_and_unshared(gpu_device, direction):
+    """Batch 4096 on a 1024 x 1024 tile runs on the 128 x 128 workgroup tiles.  With no ADC quantization and no bound
+    management the difference to the same pass without output noise, divided by out_noise times the per-sample
+    output factor (the abs-max of the input), must be standard normal and uncorrelated between samples, outputs
+    and workgroup tiles."""
+    rng = np.random.default_rng(21)
+    size, batch, sigma = 1024, 4096, 0.06
+
+    def tile(noise):
+        io = noise_free_io(inp_res=1 / 126.0, out_res=-1.0, out_bound=1e6, out_noise=noise,
+                           noise_management=dv.NoiseManagementType.AbsMax)
+        meta = make_meta(io, io)
+        dev = constant_step(w_max_dtod=0.0, w_min_dtod=0.0, w_max=1.0, w_min=-1.0, construction_seed=3)
+        host = meta.create_array(size, size, dev)
+        host.set_weights(torch.from_numpy(w))
+        gpu = tiles.CudaAnalogTile(host)
+        gpu.set_seed(77)
+        return gpu
+
+    w = rng.uniform(-0.3, 0.3, (size, size)).astype(np.float32)
+    v = cuda(rng.uniform(-1, 1, (batch, size)).astype(np.float32))
+    noisy, clean = tile(sigma), tile(0.0)
+    if direction == "forward":
+        y, y0 = noisy.forward(v, False, False, False, False, False), clean.forward(v, False, False, False, False, False)
+    else:
+        y, y0 = noisy.backward(v, False, False, False, False), clean.backward(v, False, False, False, False)
+    z = ((y - y0) / (sigma * v.abs().amax(dim=1, keepdim=True))).double()
+    n = z.numel()
+    assert abs(z.mean().item()) < 4 / np.sqrt(n)
+    assert abs(z.var().item() - 1) < 5 * np.sqrt(2 / n) + 2e-3          # fp32 rounding of y - y0 adds a little
+    assert abs((z ** 4).mean().item() - 3) < 0.05
+    zc = z - z.mean()
+    for a, b in ((zc[:, :-1], zc[:, 1:]), (zc[:-1], zc[1:]), (zc[:, :128], zc[:, 128:256]), (zc[:128], zc[128:256]),
+                 (zc[:, :512], zc[:, 512:])):
+        assert abs((a * b).mean().item()) < 5 / np.sqrt(a.numel())
