@@ -695,13 +695,13 @@ struct Tile {
     if (D <= 32 && (long)n_images * idx_patches < (1L << 31)) {
       // narrow tile: unfold, contraction and bound management fused in one kernel, nothing materialized
       const int B = n_images * idx_patches;
-      ensure_mvm_scratch(B);
+      s_rounds.ensure((size_t)B); // the only per-patch state that leaves the kernel: rounds run (get_bm_rounds)
       MvmArgs a{};
       a.w = wdev(); a.x_size = X; a.d_size = D; a.m_batch = B; a.K = X; a.O = D;
       a.io = io_dev(fio);
       a.alpha = fio.p.out_scale;
       a.max_rounds = fio.perfect ? 0 : mvm_max_rounds(a.io);
-      a.st.rounds = s_rounds.p; a.st.nm_np = s_nmnp.p;
+      a.st.rounds = s_rounds.p;
       if (conv_forward_supported(a)) {
         if (!x_idx_t.p) {
           std::vector<int32_t> tr((size_t)X * idx_patches);
