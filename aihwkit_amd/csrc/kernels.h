@@ -50,6 +50,7 @@ struct MvmArgs {
   int max_rounds; // rounds launched for this call (mvm_max_rounds)
   int speculate;  // 1: each round also quantizes every row for the round after it (short path between rounds, for
                   // small batches); 0: only the rows of samples that saturated are quantized, once that is known
+  int rows_ahead_in_init; // 1: the init kernel also writes the rows of round 1 (round 0 then prepares nothing)
   int big_from;   // > 0: rounds with at least this many samples are run by the large-tile kernel; < 0: round 0 is
   float alpha, beta; // only used when io.perfect: out = alpha * acc + beta * out
   IoDev io;

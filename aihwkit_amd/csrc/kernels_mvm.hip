@@ -576,17 +576,41 @@ __device__ __forceinline__ void mvm_init_sample(const MvmArgs &a, int b, int t, 
     return;
   }
   const float *row = a.in + (long)b * a.in_sb;
+  // a row of up to 8 elements per thread is read once and kept for the statistics and the quantized rows
+  constexpr int KEEP = 8;
+  const bool kept = a.k_pad <= KEEP * SUB;
+  float xk[KEEP];
+  if (kept) {
+#pragma unroll
+    for (int i = 0; i < KEEP; ++i) {
+      const int k = t + i * SUB;
+      xk[i] = (k < a.K) ? row[(long)k * a.in_sk] : 0.0f;
+    }
+  }
   float nm = 1.0f;
   const bool worst_case = io.bound_management == RPU_BM_ITERATIVE_WORST_CASE;
   const bool need_np = io.noise_management == RPU_NM_ABS_MAX_NP_SUM || worst_case;
   if (io.noise_management == RPU_NM_ABS_MAX || io.noise_management == RPU_NM_MAX || need_np) {
     float amax = 0.0f, vmax = -INFINITY, ps = 0.0f, ns = 0.0f;
-    for (int k = t; k < a.K; k += SUB) {
-      const float x = row[(long)k * a.in_sk];
-      amax = fmaxf(amax, fabsf(x));
-      vmax = fmaxf(vmax, x);
-      ps += x > 0.0f ? x : 0.0f;
-      ns += x < 0.0f ? x : 0.0f;
+    if (kept) {
+#pragma unroll
+      for (int i = 0; i < KEEP; ++i) {
+        if (t + i * SUB < a.K) {
+          const float x = xk[i];
+          amax = fmaxf(amax, fabsf(x));
+          vmax = fmaxf(vmax, x);
+          ps += x > 0.0f ? x : 0.0f;
+          ns += x < 0.0f ? x : 0.0f;
+        }
+      }
+    } else {
+      for (int k = t; k < a.K; k += SUB) {
+        const float x = row[(long)k * a.in_sk];
+        amax = fmaxf(amax, fabsf(x));
+        vmax = fmaxf(vmax, x);
+        ps += x > 0.0f ? x : 0.0f;
+        ns += x < 0.0f ? x : 0.0f;
+      }
     }
     amax = group_max<SUB>(amax, sh);
     if (io.noise_management == RPU_NM_MAX) {
@@ -629,7 +653,25 @@ __device__ __forceinline__ void mvm_init_sample(const MvmArgs &a, int b, int t, 
     const long n_done = 32L * ((a.m_batch + TILE - 1) / TILE);
     for (long idx = gid; idx < n_done; idx += gstride) a.st.tile_done[idx] = 0;
   }
-  write_dac_row(a, b, b, scale, 0, a.xq[0], t, SUB);
+  // the input range of a second round is known as well: its row is quantized now, while the input is at hand,
+  // so that the first round has nothing to prepare
+  float next = 0.0f;
+  if (a.rows_ahead_in_init && io.bound_management != RPU_BM_NONE) next = next_round_scale(a, 0, b, fin, nm, 1.0f);
+  if (kept) {
+    float *out0 = a.xq[0] + (long)b * a.k_pad;
+    float *out1 = a.xq[1] + (long)b * a.k_pad;
+#pragma unroll
+    for (int i = 0; i < KEEP; ++i) {
+      const int k = t + i * SUB;
+      if (k < a.k_pad) {
+        out0[k] = (k < a.K) ? dac_value(xk[i], scale, io, a.key, a.call, 0, b, k) : 0.0f;
+        if (next != 0.0f) out1[k] = (k < a.K) ? dac_value(xk[i], next, io, a.key, a.call, 1, b, k) : 0.0f;
+      }
+    }
+  } else {
+    write_dac_row(a, b, b, scale, 0, a.xq[0], t, SUB);
+    if (next != 0.0f) write_dac_row(a, b, b, next, 1, a.xq[1], t, SUB);
+  }
 }
 
 // SUB threads per sample: a workgroup holds 256 / SUB samples
@@ -778,7 +820,9 @@ __device__ __forceinline__ void mvm_round_workgroup(const MvmArgs &a, int round,
   int tile_o, tile_b;
   if (!tile_of(a, n, n_act, tile_o, tile_b)) return;
   const bool more_rounds = round + 1 < a.max_rounds;
-  if (more_rounds && a.speculate) mvm_prepare_next_rows(a, round, tile_o, tile_b, n_act);
+  if (more_rounds && a.speculate && !(round == 0 && a.rows_ahead_in_init)) {
+    mvm_prepare_next_rows(a, round, tile_o, tile_b, n_act);
+  }
   mvm_round_tile<PD, WMODE>(a, round, tile_o, tile_b, n_act, red, stage);
   if (more_rounds) mvm_tile_finished(a, round, tile_b, n_act);
 }
@@ -938,7 +982,9 @@ __device__ __forceinline__ void mvm_big_workgroup(const MvmArgs &a, const int ro
   const int tile_b = ((n >> 3) / ((a.O + BT - 1) / BT)) * 8 + (n & 7);
   if (tile_b * BT >= n_act) return;
   const bool more_rounds = round + 1 < a.max_rounds;
-  if (more_rounds) big_prepare_next_rows(a, round, tile_o, tile_b, n_act, sh_b, sh_scale);
+  if (more_rounds && !(round == 0 && a.rows_ahead_in_init)) {
+    big_prepare_next_rows(a, round, tile_o, tile_b, n_act, sh_b, sh_scale);
+  }
 
   const int t = threadIdx.x;
   const int lane = t & 63, wave = t >> 6;

@@ -363,6 +363,7 @@ struct Tile {
     // rounds) or when at least four workgroups per sample tile share that work; a large batch on a narrow tile
     // quantizes only the rows of the samples that saturated
     a.speculate = (B <= 1024 || O > 96) ? 1 : 0;
+    a.rows_ahead_in_init = (a.speculate || tight) ? 1 : 0;
     return a;
   }
 
