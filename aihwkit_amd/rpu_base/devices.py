@@ -376,11 +376,16 @@ class AnalogTileParameter(_Struct):
 
         if not isinstance(device_param, AbstractResistiveDeviceParameter) or device_param._kind is None:
             raise TypeError("device_param must be one of the *ResistiveDeviceParameter classes")
+        import copy
+
         if isinstance(device_param, TransferResistiveDeviceParameter):
             transfer = device_param._to_transfer_c()
             config = self._config(device_param._vec_par[0])
-            return AnalogTile._create_transfer(int(x_size), int(d_size), config, transfer)
-        return AnalogTile._create(int(x_size), int(d_size), self._config(device_param))
+            tile = AnalogTile._create_transfer(int(x_size), int(d_size), config, transfer)
+        else:
+            tile = AnalogTile._create(int(x_size), int(d_size), self._config(device_param))
+        tile._meta_parameters, tile._parameters = copy.deepcopy(self), copy.deepcopy(device_param)
+        return tile
 
 
 class FloatingPointTileParameter(_Struct):
@@ -389,6 +394,8 @@ class FloatingPointTileParameter(_Struct):
     _defaults = dict(diffusion=0.0, lifetime=0.0, drift=None)
 
     def create_array(self, x_size: int, d_size: int):
+        import copy
+
         from .tiles import FloatingPointTile
 
         meta = AnalogTileParameter()
@@ -398,7 +405,9 @@ class FloatingPointTileParameter(_Struct):
         device = IdealResistiveDeviceParameter()
         device.diffusion = float(self.diffusion)
         device.lifetime = float(self.lifetime)
-        return FloatingPointTile._create(int(x_size), int(d_size), meta._config(device))
+        tile = FloatingPointTile._create(int(x_size), int(d_size), meta._config(device))
+        tile._meta_parameters, tile._parameters = copy.deepcopy(self), copy.deepcopy(self)
+        return tile
 
 
 __all__ = [name for name, obj in vars(sys.modules[__name__]).items()

@@ -72,11 +72,40 @@ class _TileBase:
         check(lib().rpu_tile_clone(C.byref(handle), self._h))
         return handle.value
 
+    def _copy_parameters_to(self, other):
+        other._meta_parameters = getattr(self, "_meta_parameters", None)
+        other._parameters = getattr(self, "_parameters", None)
+        return other
+
     def __copy__(self):
-        return type(self)(self._clone_handle())
+        return self._copy_parameters_to(type(self)(self._clone_handle()))
 
     def __deepcopy__(self, memo):
-        return type(self)(self._clone_handle())
+        return self._copy_parameters_to(type(self)(self._clone_handle()))
+
+    # -- parameter structs the tile was built from (rpu_base_tiles.cpp get_parameters / get_meta_parameters)
+    def get_meta_parameters(self):
+        return self._meta_parameters
+
+    def get_parameters(self):
+        return self._parameters
+
+    def set_weights_uniform_random(self, min_value: float, max_value: float) -> None:
+        """Uniform random weights in [min_value, max_value], clipped into the device bounds like ``set_weights``
+        (RPUPulsed::setWeightsUniformRandom, src/rpucuda/rpu_pulsed.cpp:280-284); the draw uses torch's generator."""
+        shape = (self.get_d_size(), self.get_x_size())
+        self.set_weights(torch.rand(shape, dtype=_DTYPE) * (float(max_value) - float(min_value)) + float(min_value))
+
+    # -- hardware-aware-training utilities and device-level drift of the reference bindings that this library does
+    #    not provide (rpu_base_tiles.cpp:292-371, 845-868)
+    def _not_provided(self, *args, **kwargs):
+        raise RuntimeError("Not provided by this library: drift_weights (device-level power-law drift), "
+                           "remap_weights, modify_weights and get_pulse_counters.")
+
+    drift_weights = _not_provided
+    remap_weights = _not_provided
+    modify_weights = _not_provided
+    get_pulse_counters = _not_provided
 
     # -- sizes / learning rate (rpu_base_tiles.cpp get_x_size, get_d_size, get/set_learning_rate)
     def get_x_size(self) -> int:
@@ -192,6 +221,7 @@ class _CudaTileMixin:
             raise RuntimeError("No GPU available: the analog tile kernels need a HIP device.")
         handle = tile._clone_handle()
         _TileBase.__init__(self, handle)
+        tile._copy_parameters_to(self)
         check(lib().rpu_tile_to_device(self._h, torch.cuda.current_device()))
         self._device = torch.device("cuda", torch.cuda.current_device())
 

@@ -203,3 +203,32 @@ def test_extra_state_and_maintenance_calls_on_a_host_tile():
                  lambda: lib().rpu_tile_reset_columns(tile._h, 0, 1, C.c_float(1.0), None)):
         assert call() != 0 and b"GPU" in lib().rpu_last_error()
     assert not tile.get_shared_weights_if()
+
+
+def test_parameter_accessors_and_random_weights_on_a_host_tile():
+    import copy
+
+    import torch
+
+    from aihwkit_amd.rpu_base import devices as dv
+
+    meta = dv.AnalogTileParameter()
+    meta.forward_io.out_noise = 0.01
+    dev = dv.SoftBoundsResistiveDeviceParameter()
+    dev.dw_min = 0.002
+    tile = meta.create_array(7, 5, dev)
+    assert tile.get_meta_parameters().forward_io.out_noise == 0.01 and tile.get_parameters().dw_min == 0.002
+    meta.forward_io.out_noise = 0.5                                     # the tile keeps what it was built from
+    assert tile.get_meta_parameters().forward_io.out_noise == 0.01
+    assert copy.deepcopy(tile).get_parameters().dw_min == 0.002
+    torch.manual_seed(0)
+    tile.set_weights_uniform_random(-0.2, 0.1)
+    w = tile.get_weights()
+    assert w.min() >= -0.2 and w.max() <= 0.1 and w.std() > 0.03
+    hidden = dict(zip(tile.get_hidden_parameter_names(), tile.get_hidden_parameters()))
+    assert (w <= hidden["max_bound"]).all() and (w >= hidden["min_bound"]).all()
+    for name in ("drift_weights", "remap_weights", "modify_weights", "get_pulse_counters"):
+        with pytest.raises(RuntimeError, match="Not provided"):
+            getattr(tile, name)()
+    fp = dv.FloatingPointTileParameter().create_array(3, 2)
+    assert fp.get_meta_parameters().lifetime == 0.0
