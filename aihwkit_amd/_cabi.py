@@ -56,6 +56,32 @@ class DeviceParams(C.Structure):
         ("ls_reverse_up", i32), ("ls_reverse_down", i32),
         ("ls_decrease_up", f32), ("ls_decrease_down", f32), ("ls_decrease_up_dtod", f32),
         ("ls_decrease_down_dtod", f32), ("ls_reverse_offset", f32),
+        ("drift_nu", f32), ("drift_nu_dtod", f32), ("drift_nu_std", f32), ("drift_wg_ratio", f32),
+        ("drift_g_offset", f32), ("drift_w_offset", f32), ("drift_nu_k", f32), ("drift_log_g0", f32),
+        ("drift_t0", f32), ("drift_reset_tol", f32), ("drift_w_read_std", f32), ("count_pulses", i32),
+    ]
+
+
+class RemapParams(C.Structure):
+    """``rpu_remap_params``."""
+
+    _fields_ = [
+        ("type", i32), ("clip_if", i32), ("max_scale_range", f32), ("max_scale_ref", f32),
+        ("row_norm", f32), ("remapped_wmax", f32),
+    ]
+
+
+MAX_MODIFIER_COEFFS = 8
+
+
+class ModifierParams(C.Structure):
+    """``rpu_modifier_params``."""
+
+    _fields_ = [
+        ("type", i32), ("per_batch_sample", i32), ("sto_round", i32), ("enable_during_test", i32),
+        ("copy_last_column", i32), ("rel_to_actual_wmax", i32), ("n_coeffs", i32),
+        ("std_dev", f32), ("res", f32), ("dorefa_clip", f32), ("pdrop", f32), ("assumed_wmax", f32),
+        ("g_max", f32), ("coeffs", f32 * MAX_MODIFIER_COEFFS),
     ]
 
 
@@ -113,6 +139,12 @@ SYMBOLS = {
     "rpu_tile_diffuse_weights": (C.c_int, [_P, _P]),
     "rpu_tile_clip_weights": (C.c_int, [_P, C.c_int, C.c_float, C.c_float, _P]),
     "rpu_tile_reset_columns": (C.c_int, [_P, C.c_int, C.c_int, C.c_float, _P]),
+    "rpu_tile_drift_device_weights": (C.c_int, [_P, C.c_float, _P]),
+    "rpu_tile_remap_weights": (C.c_int, [_P, C.POINTER(RemapParams), _P, _P]),
+    "rpu_tile_modify_weights": (C.c_int, [_P, C.POINTER(ModifierParams), _P]),
+    "rpu_tile_get_modified_weights": (C.c_int, [_P, _P]),
+    "rpu_tile_pulse_counter_count": (C.c_int, [_P]),
+    "rpu_tile_get_pulse_counters": (C.c_int, [_P, _P]),
     "rpu_tile_set_shared_weights": (C.c_int, [_P, _P]),
     "rpu_tile_get_shared_weights_if": (C.c_int, [_P]),
     "rpu_tile_set_delta_weights": (C.c_int, [_P, _P]),

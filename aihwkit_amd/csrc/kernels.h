@@ -178,6 +178,43 @@ void launch_reset_cols(float *w, const float *reset_bias, const float *w_min, co
 // prev_w_and_delta holds the weights from before an update: it becomes scale * (w - previous), w gets them back
 void launch_delta_finish(float *w, float *prev_w_and_delta, float scale, size_t n, hipStream_t s);
 
+// power-law drift of every weight that has stayed within reset_tol of its value after the last call
+// (WeightDrifter::apply, weight_drifter.cpp:108-150); nu == null: the same nu0 for every element
+struct DriftDev {
+  float nu0, nu_std, wg_ratio, g_offset, w_offset, nu_k, log_g0, reset_tol, w_read_std;
+  float a; // g_offset * wg_ratio + w_offset, zero when within reset_tol of zero
+};
+void launch_device_drift(float *w, float *prev, float *w0, float *t, const float *nu, const float *w_min,
+                         const float *w_max, const DriftDev &p, float current_t, PhiloxKey key, uint32_t call, size_t n,
+                         hipStream_t s);
+
+// per-row statistic of the first n_cols columns: largest absolute value, or sum of squares
+void launch_row_stat(const float *w, int x_size, int d_size, int n_cols, int sum_squares, float *row_out, hipStream_t s);
+// out[0] = largest of v[0..n-1] when positive, else 1
+void launch_max_or_one(const float *v, int n, float *out, hipStream_t s);
+// WeightRemapper::apply (weight_remapper.cpp:19-190): from the row statistic in row_stat the per-row factors
+// mul / div and the new scales; then w[i][j] = w[i][j] * mul[i] / div[i]
+struct RemapDev {
+  int type, clip_if;
+  float max_scale_range, max_scale_ref, row_norm, remapped_wmax;
+};
+void launch_remap(float *w, float *scales, float *row_stat, float *mul, float *div, int x_size, int d_size,
+                  const RemapDev &p, hipStream_t s);
+
+// WeightModifier::apply (weight_modifier.cpp:28-224): out = modified copy of w; amax_dev == null: assumed_wmax
+struct ModifierDev {
+  int type, sto_round, copy_last_column, n_coeffs;
+  float std_dev, res, dorefa_clip, pdrop, g_max, assumed_wmax;
+  float coeffs[8];
+};
+void launch_modify(float *out, const float *w, const ModifierDev &p, const float *amax_dev, PhiloxKey key, uint32_t call,
+                   int x_size, size_t n, hipStream_t s);
+
+// adds the coincidences of the batch to the per-cross-point counters: pos where the signs of x and d agree,
+// neg where they differ (kernelPulseCounter, cuda/pwu_kernel.h:1523-1627); implicit: from the line values
+void launch_count_pulses(const UpdateArgs &a, unsigned long long *pos, unsigned long long *neg, bool implicit,
+                         hipStream_t s);
+
 // clip weights into [w_min, w_max]
 void launch_clip(float *w, const float *w_min, const float *w_max, size_t n, hipStream_t s);
 

@@ -161,6 +161,205 @@ __global__ __launch_bounds__(256) void k_delta_finish(float *w, float *prev_w_an
   }
 }
 
+// WeightDrifter::apply (weight_drifter.cpp:108-150) with the saturation of a pulsed device
+// (weight_drifter.cpp:98-106) folded in; z[0] varies nu, z[1] is the read noise
+__global__ __launch_bounds__(256) void k_device_drift(float *w, float *prev, float *w0, float *t, const float *nu,
+                                                       const float *w_min, const float *w_max, DriftDev p,
+                                                       float current_t, PhiloxKey key, uint32_t call, size_t n) {
+  const bool random = p.nu_std > 0.0f || p.w_read_std > 0.0f;
+  for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+    float z[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (random) philox_normal4((uint32_t)i, (uint32_t)(i >> 32), call, RNG_DEVICE_DRIFT, key, z);
+    float v = w[i];
+    if (fabsf(prev[i] - v) > p.reset_tol) {
+      // the weight has changed: its drift starts again from here
+      t[i] = current_t;
+      w0[i] = v;
+    } else {
+      float nu_i = nu ? nu[i] : p.nu0;
+      if (p.nu_std > 0.0f) nu_i = nu_i + p.nu_std * nu_i * z[0];
+      if (p.nu_k != 0.0f) nu_i = nu_i - p.nu_k * logf((v - p.w_offset) / p.wg_ratio + p.g_offset) + p.nu_k * p.log_g0;
+      const float delta_t = fmaxf(current_t - t[i], 1.0f);
+      const float nu_scale = powf(delta_t, -nu_i);
+      v = w0[i] * nu_scale;
+      if (p.a != 0.0f) v = v + p.a * (nu_scale - 1.0f);
+    }
+    if (p.w_read_std > 0.0f) v += p.w_read_std * z[1];
+    v = clip_to(v, w_min, w_max, i);
+    prev[i] = v;
+    w[i] = v;
+  }
+}
+
+// one workgroup per row: largest absolute value or sum of squares of the first n_cols columns
+__global__ __launch_bounds__(256) void k_row_stat(const float *w, int x_size, int n_cols, int sum_squares,
+                                                   float *row_out) {
+  __shared__ float sh[4];
+  const float *row = w + (size_t)blockIdx.x * x_size;
+  float m = 0.0f;
+  if (sum_squares) {
+    for (int j = threadIdx.x; j < n_cols; j += blockDim.x) m = __builtin_fmaf(row[j], row[j], m);
+    m = block_sum(m, sh);
+  } else {
+    for (int j = threadIdx.x; j < n_cols; j += blockDim.x) m = fmaxf(m, fabsf(row[j]));
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off));
+    if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = m;
+    __syncthreads();
+    m = fmaxf(fmaxf(sh[0], sh[1]), fmaxf(sh[2], sh[3]));
+  }
+  if (threadIdx.x == 0) row_out[blockIdx.x] = m;
+}
+
+__device__ __forceinline__ float block_max(float v, float *sh) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off));
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = v;
+  __syncthreads();
+  float r = sh[0];
+  for (int i = 1; i < (int)(blockDim.x >> 6); ++i) r = fmaxf(r, sh[i]);
+  return r;
+}
+
+__global__ __launch_bounds__(256) void k_max_or_one(const float *v, int n, float *out) {
+  __shared__ float sh[4];
+  float m = 0.0f;
+  for (int i = threadIdx.x; i < n; i += blockDim.x) m = fmaxf(m, v[i]);
+  m = block_max(m, sh);
+  if (threadIdx.x == 0) *out = m > 0.0f ? m : 1.0f;
+}
+
+// One workgroup: the per-row factors of a remap and the new scales.  The weights then become w * mul / div, which
+// is the reference's w / f with mul = 1, and its w * old_scale / new_scale under a bounded scale range.
+__global__ __launch_bounds__(256) void k_remap_factors(float *scales, const float *row_stat, float *mul, float *div,
+                                                        int d_size, RemapDev p) {
+  __shared__ float sh[4];
+  if (p.type == RPU_REMAP_LAYERWISE_SYMMETRIC) {
+    float m = 0.0f;
+    for (int i = threadIdx.x; i < d_size; i += blockDim.x) m = fmaxf(m, row_stat[i]);
+    float amax = block_max(m, sh) / p.remapped_wmax;
+    if (!(amax > 0.0f)) amax = 1.0f;
+    for (int i = threadIdx.x; i < d_size; i += blockDim.x) {
+      if (amax != 1.0f) scales[i] *= amax;
+      mul[i] = 1.0f;
+      div[i] = amax;
+    }
+  } else if (p.type == RPU_REMAP_CHANNELWISE_SYMMETRIC && !(p.max_scale_range > 0.0f)) {
+    for (int i = threadIdx.x; i < d_size; i += blockDim.x) {
+      float amax = row_stat[i];
+      if (p.remapped_wmax != 1.0f) amax /= p.remapped_wmax;
+      const float f = amax > 0.0f ? amax : 1.0f;
+      scales[i] *= f;
+      mul[i] = 1.0f;
+      div[i] = f;
+    }
+  } else if (p.type == RPU_REMAP_CHANNELWISE_SYMMETRIC) {
+    // bounded spread of the scales: no scale may exceed max_scale_range times the smallest one
+    float mn = 3.4028234664e38f;
+    for (int i = threadIdx.x; i < d_size; i += blockDim.x) mn = fminf(mn, scales[i]);
+    float min_scale = fmaxf(-block_max(-mn, sh), 0.0f);
+    if (min_scale > 0.0f && p.max_scale_ref != 0.0f) min_scale = fmaxf(min_scale, p.max_scale_ref);
+    for (int i = threadIdx.x; i < d_size; i += blockDim.x) {
+      const float amax = row_stat[i];
+      const float old_scale = scales[i];
+      float new_scale = amax > 0.0f ? amax * old_scale : old_scale;
+      if (min_scale > 0.0f && new_scale / min_scale > p.max_scale_range) new_scale = min_scale * p.max_scale_range;
+      scales[i] = new_scale;
+      mul[i] = old_scale;
+      div[i] = new_scale;
+    }
+  } else { // RPU_REMAP_CHANNELWISE_NORM: row_stat holds the sums of squares
+    for (int i = threadIdx.x; i < d_size; i += blockDim.x) {
+      float nm = sqrtf(row_stat[i]);
+      nm = nm > 0.0f ? nm : 1.0f;
+      nm /= p.row_norm;
+      nm = nm > 1.0f ? nm : 1.0f;
+      if (!p.clip_if) scales[i] *= nm;
+      mul[i] = 1.0f;
+      div[i] = nm;
+    }
+  }
+}
+
+__global__ __launch_bounds__(256) void k_remap_apply(float *w, const float *mul, const float *div, int x_size, size_t n) {
+  for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+    const size_t r = i / x_size;
+    w[i] = w[i] * mul[r] / div[r];
+  }
+}
+
+// getDiscretizedValueRound (utility_functions.h:195-202)
+__device__ __forceinline__ float discretize(float v, float res, int sto_round, float u) {
+  if (res <= 0.0f) return v;
+  return sto_round ? roundf(v / res + (u - 0.5f)) * res : roundf(v / res) * res;
+}
+
+// WeightModifier::apply (weight_modifier.cpp:28-224).  One Philox call per element: words 0, 1 give the normal
+// draw, word 2 the stochastic rounding, word 3 the dropped connections.
+__global__ __launch_bounds__(256) void k_modify(float *out, const float *w, ModifierDev p, const float *amax_dev,
+                                                 PhiloxKey key, uint32_t call, int x_size, size_t n) {
+  const float amax = amax_dev ? *amax_dev : p.assumed_wmax;
+  for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+    float v = w[i];
+    if (p.copy_last_column && (int)(i % x_size) == x_size - 1) {
+      out[i] = v;
+      continue;
+    }
+    const Philox4 r = philox4x32_10((uint32_t)i, (uint32_t)(i >> 32), call, RNG_MODIFIER, key.k0, key.k1);
+    float z, z_unused;
+    box_muller(r.v[0], r.v[1], z, z_unused);
+    const float u = u32_to_uniform(r.v[2]);
+    switch (p.type) {
+    case RPU_MODIFIER_DISCRETIZE:
+      if (p.res > 0.0f) v = amax * discretize(v / amax, p.res, p.sto_round, u);
+      break;
+    case RPU_MODIFIER_MULT_NORMAL:
+      if (p.std_dev > 0.0f) v += v * (p.std_dev * amax) * z;
+      break;
+    case RPU_MODIFIER_ADD_NORMAL:
+      if (p.std_dev > 0.0f) v += (p.std_dev * amax) * z;
+      break;
+    case RPU_MODIFIER_DISCRETIZE_ADD_NORMAL:
+      if (p.res > 0.0f || p.std_dev * amax > 0.0f) {
+        v = amax * discretize(v / amax, p.res, p.sto_round, u);
+        v = v + (p.std_dev * amax) * z;
+      }
+      break;
+    case RPU_MODIFIER_DOREFA:
+      if (p.res > 0.0f) {
+        const float scale = fabsf(p.dorefa_clip / tanhf(amax));
+        v = discretize(tanhf(v) * scale, p.res, p.sto_round, u);
+      }
+      break;
+    case RPU_MODIFIER_POLY:
+    case RPU_MODIFIER_PROG_NOISE:
+      if (p.std_dev > 0.0f && p.n_coeffs > 0) {
+        const float aw = fabsf(v) / amax;
+        float paw = 1.0f, sig = p.coeffs[0];
+        for (int c = 1; c < p.n_coeffs; ++c) {
+          paw *= aw;
+          sig += p.coeffs[c] * paw;
+        }
+        if (p.type == RPU_MODIFIER_POLY) {
+          sig *= p.std_dev;
+          v += amax * sig * z;
+        } else {
+          // the noise never changes the sign of a weight
+          sig *= p.std_dev / p.g_max;
+          const float noisy = fabsf(v + amax * sig * z);
+          v = v < 0.0f ? -noisy : noisy;
+        }
+      }
+      break;
+    default: // copy, drop connect
+      break;
+    }
+    if (p.pdrop > 0.0f && u32_to_uniform(r.v[3]) < p.pdrop) v = 0.0f;
+    out[i] = v;
+  }
+}
+
 int grid_for(size_t n) {
   const size_t blocks = (n + 255) / 256;
   return (int)(blocks > 8192 ? 8192 : (blocks ? blocks : 1));
@@ -203,6 +402,34 @@ void launch_reset_cols(float *w, const float *reset_bias, const float *w_min, co
                        hipStream_t s) {
   hipLaunchKernelGGL(k_reset_cols, dim3(grid_for((size_t)d_size * n_cols)), dim3(256), 0, s, w, reset_bias, w_min, w_max,
                      reset_std, start_col, n_cols, reset_prob, x_size, d_size, key, call);
+}
+
+void launch_device_drift(float *w, float *prev, float *w0, float *t, const float *nu, const float *w_min,
+                         const float *w_max, const DriftDev &p, float current_t, PhiloxKey key, uint32_t call, size_t n,
+                         hipStream_t s) {
+  hipLaunchKernelGGL(k_device_drift, dim3(grid_for(n)), dim3(256), 0, s, w, prev, w0, t, nu, w_min, w_max, p, current_t,
+                     key, call, n);
+}
+
+void launch_row_stat(const float *w, int x_size, int d_size, int n_cols, int sum_squares, float *row_out, hipStream_t s) {
+  hipLaunchKernelGGL(k_row_stat, dim3(d_size), dim3(256), 0, s, w, x_size, n_cols, sum_squares, row_out);
+}
+
+void launch_max_or_one(const float *v, int n, float *out, hipStream_t s) {
+  hipLaunchKernelGGL(k_max_or_one, dim3(1), dim3(256), 0, s, v, n, out);
+}
+
+void launch_remap(float *w, float *scales, float *row_stat, float *mul, float *div, int x_size, int d_size,
+                  const RemapDev &p, hipStream_t s) {
+  launch_row_stat(w, x_size, d_size, x_size, p.type == RPU_REMAP_CHANNELWISE_NORM ? 1 : 0, row_stat, s);
+  hipLaunchKernelGGL(k_remap_factors, dim3(1), dim3(256), 0, s, scales, row_stat, mul, div, d_size, p);
+  const size_t n = (size_t)x_size * d_size;
+  hipLaunchKernelGGL(k_remap_apply, dim3(grid_for(n)), dim3(256), 0, s, w, mul, div, x_size, n);
+}
+
+void launch_modify(float *out, const float *w, const ModifierDev &p, const float *amax_dev, PhiloxKey key, uint32_t call,
+                   int x_size, size_t n, hipStream_t s) {
+  hipLaunchKernelGGL(k_modify, dim3(grid_for(n)), dim3(256), 0, s, out, w, p, amax_dev, key, call, x_size, n);
 }
 
 void launch_delta_finish(float *w, float *prev_w_and_delta, float scale, size_t n, hipStream_t s) {

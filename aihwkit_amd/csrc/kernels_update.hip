@@ -626,6 +626,52 @@ __global__ __launch_bounds__(256) void k_implicit_counts(UpdateArgs a, int32_t *
   }
 }
 
+// kernelPulseCounter (cuda/pwu_kernel.h:1523-1627) on the bit planes: one thread per cross-point
+__global__ __launch_bounds__(256) void k_count_pulses(UpdateArgs a, unsigned long long *pos, unsigned long long *neg) {
+  const int i = blockIdx.y;
+  const int j = blockIdx.x * blockDim.x + threadIdx.x;
+  if (j >= a.x_size) return;
+  const int kmax = a.kmax[a.kmax_slot];
+  const unsigned xs = (unsigned)a.x_size, ds = (unsigned)a.d_size, slots = (unsigned)a.plane_slots;
+  const uint32_t *xpl = a.x_planes + j;
+  const uint32_t *dpl = a.d_planes + i;
+  unsigned n_same = 0, n_diff = 0;
+  for (int c = 0; c < a.n_chunks; ++c) {
+    const unsigned base = (unsigned)c * slots;
+    const uint32_t same = ~(xpl[(base + slots - 1) * xs] ^ dpl[(base + slots - 1) * ds]);
+    for (int k = 0; k < kmax; ++k) {
+      const uint32_t dk = dpl[(base + k) * ds]; // wave-uniform
+      if (!dk) continue;
+      const uint32_t m = dk & xpl[(base + k) * xs];
+      n_same += __popc(m & same);
+      n_diff += __popc(m & ~same);
+    }
+  }
+  const size_t cell = (size_t)i * a.x_size + j;
+  pos[cell] += n_same;
+  neg[cell] += n_diff;
+}
+
+// the same for the deterministic implicit pulses: n > 0 are coincidences of equal sign
+__global__ __launch_bounds__(256) void k_count_pulses_implicit(UpdateArgs a, unsigned long long *pos,
+                                                                unsigned long long *neg) {
+  const int i = blockIdx.y;
+  const int j = blockIdx.x * blockDim.x + threadIdx.x;
+  if (j >= a.x_size) return;
+  unsigned long long n_same = 0, n_diff = 0;
+  for (int b = 0; b < a.m_batch; ++b) {
+    float dc = a.d_val[(long)b * a.d_size + i];
+    if (dc == 0.0f) continue;
+    dc *= (float)a.bl[b];
+    const int cn = (int)rintf(dc * a.x_val[(long)b * a.x_size + j]);
+    if (cn > 0) n_same += (unsigned)cn;
+    else n_diff += (unsigned)(-cn);
+  }
+  const size_t cell = (size_t)i * a.x_size + j;
+  pos[cell] += n_same;
+  neg[cell] += n_diff;
+}
+
 __global__ void k_clip(float *w, const float *w_min, const float *w_max, size_t n) {
   for (size_t idx = blockIdx.x * (size_t)blockDim.x + threadIdx.x; idx < n; idx += (size_t)gridDim.x * blockDim.x) {
     float v = w[idx];
@@ -699,6 +745,13 @@ void launch_update_pulsed(const UpdateArgs &a, hipStream_t s) {
 void launch_update_implicit(const UpdateArgs &a, hipStream_t s) {
   dim3 grid((a.x_size + 255) / 256, a.d_size);
   RPU_DISPATCH_DEVICE(k_update_implicit, grid, s, a);
+}
+
+void launch_count_pulses(const UpdateArgs &a, unsigned long long *pos, unsigned long long *neg, bool implicit,
+                         hipStream_t s) {
+  dim3 grid((a.x_size + 255) / 256, a.d_size);
+  if (implicit) hipLaunchKernelGGL(k_count_pulses_implicit, grid, dim3(256), 0, s, a, pos, neg);
+  else hipLaunchKernelGGL(k_count_pulses, grid, dim3(256), 0, s, a, pos, neg);
 }
 
 void launch_implicit_counts(const UpdateArgs &a, int32_t *counts, hipStream_t s) {

@@ -69,7 +69,9 @@ enum RngPurpose : uint32_t {
   RNG_PCM_PROGRAM = 9, // programming noise and drift coefficients of the inference weight pipeline
   RNG_PCM_DRIFT = 10,  // accumulated read noise at inference time
   RNG_DIFFUSE = 11,    // weight diffusion
-  RNG_RESET = 12       // column reset (noise, and with round 1 the reset lottery)
+  RNG_RESET = 12,      // column reset (noise, and with round 1 the reset lottery)
+  RNG_DEVICE_DRIFT = 13, // power-law drift of a training tile: nu variation and read noise
+  RNG_MODIFIER = 14      // weight modifier: noise, stochastic rounding, drop connections
 };
 
 // uniform in [0, 1) with 24 bits

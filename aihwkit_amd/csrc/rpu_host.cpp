@@ -175,6 +175,12 @@ void populate_from(const DevicePar &dev, ConstructionRng &rng, int x_size, int d
   const auto linear = [&] { return dev.linear(); };
   const size_t n = (size_t)x_size * (size_t)d_size;
   a = DeviceArrays();
+  // the drift coefficients are drawn first, in memory order (SimpleRPUDevice::populate,
+  // rpu_simple_device.cpp:171-182; WeightDrifter::populate, weight_drifter.cpp:57-65)
+  if (p.drift_nu > 0.0f) {
+    a.drift_nu.resize(n);
+    for (size_t k = 0; k < n; ++k) a.drift_nu[k] = p.drift_nu + p.drift_nu_dtod * p.drift_nu * rng.normal();
+  }
   if (!pulsed()) {
     return;
   }
@@ -450,6 +456,19 @@ void fill_default_config(rpu_tile_config *cfg, int device_kind) {
   d.ls_decrease_up_dtod = 0.05f;
   d.ls_decrease_down_dtod = 0.05f;
   d.ls_reverse_offset = 0.01f;
+  // DriftParameter (weight_drifter.h:14-60)
+  d.drift_nu = 0.0f;
+  d.drift_nu_dtod = 0.0f;
+  d.drift_nu_std = 0.0f;
+  d.drift_wg_ratio = 1.0f;
+  d.drift_g_offset = 0.0f;
+  d.drift_w_offset = 0.0f;
+  d.drift_nu_k = 0.0f;
+  d.drift_log_g0 = 0.0f;
+  d.drift_t0 = 1.0f;
+  d.drift_reset_tol = 1e-7f;
+  d.drift_w_read_std = 0.0f;
+  d.count_pulses = 0;
   if (device_kind == RPU_DEVICE_SOFT_BOUNDS) {
     d.ls_decrease_up = 1.0f;
     d.ls_decrease_down = 1.0f;

@@ -32,6 +32,7 @@ struct UpdatePar {
 struct DeviceArrays {
   std::vector<float> w_max, w_min, scale_up, scale_down, decay_scale, diffusion_rate, reset_bias;
   std::vector<float> slope_up, slope_down; // LinearStep / SoftBounds only
+  std::vector<float> drift_nu;             // only with drift_nu > 0 in the parameters
 };
 
 struct DevicePar {

@@ -180,6 +180,15 @@ struct Tile {
   DevBuf<float> d_decay, d_diff, d_rbias, s_clip;
   bool state_params_valid = false;
   float *delta_w = nullptr;
+  // hardware-aware training: the modified copy of the weights that forward / backward contract with, scratch of
+  // the remapper ([3 D + 1]: row statistic, multiplier, divisor, one scalar), the drift clock per weight and the
+  // pulse counters [2][size]
+  DevBuf<float> d_fbw, s_rowstat;
+  bool fb_during_test = false;
+  DevBuf<float> dr_prev, dr_w0, dr_t, d_nu;
+  float drift_t = 0.0f;
+  bool nu_valid = false;
+  DevBuf<unsigned long long> d_cnt;
 
   // optional per-kernel timing with HIP events on the launch stream
   bool profiling = false;
@@ -211,6 +220,11 @@ struct Tile {
   bool is_transfer() const { return tr != nullptr; }
   // the matrix forward / backward contract with
   float *wdev() { return (tr && tr->fully_hidden) ? slots.back()->d_w.p : d_w.p; }
+  // RPUSimple::getFBWeights (rpu.cpp:1483-1487): once modified weights exist, forward and backward use them,
+  // during evaluation only if the modifier asked for it
+  const float *mvm_weights(bool is_test) {
+    return (d_fbw.p && (!is_test || fb_during_test)) ? d_fbw.p : wdev();
+  }
   size_t size() const { return (size_t)X * (size_t)D; }
 
   ~Tile() {
@@ -239,6 +253,11 @@ struct Tile {
     d_decay.release(); d_diff.release(); d_rbias.release(); s_clip.release();
     state_params_valid = false;
     delta_w = nullptr;
+    d_fbw.release(); s_rowstat.release(); dr_prev.release(); dr_w0.release(); dr_t.release(); d_nu.release();
+    d_cnt.release();
+    fb_during_test = false;
+    drift_t = 0.0f;
+    nu_valid = false;
     for (auto &sl : slots) sl->release();
   }
 
@@ -259,6 +278,7 @@ struct Tile {
 
   void upload_params() {
     state_params_valid = false;
+    nu_valid = false;
     if (!dev.pulsed()) return;
     const size_t n = size(), bytes = n * sizeof(float);
     d_wmax.ensure(n); d_wmin.ensure(n); d_sup.ensure(n); d_sdown.ensure(n);
@@ -368,9 +388,9 @@ struct Tile {
   }
 
   void mvm(const float *in, float *out, int B, bool bias, bool in_trans, bool out_trans, bool transposed, hipStream_t s,
-           const float *w_other = nullptr, const IOPar *io_other = nullptr) {
+           const float *w_other = nullptr, const IOPar *io_other = nullptr, bool is_test = false) {
     const IOPar &io = io_other ? *io_other : (transposed ? bio : fio);
-    MvmArgs a = mvm_args(B, transposed, w_other, io);
+    MvmArgs a = mvm_args(B, transposed, w_other ? w_other : mvm_weights(is_test), io);
 
     // the x side carries the optional bias column: input of forward, output of backward
     float *final_out = out;
@@ -449,6 +469,7 @@ struct Tile {
     prof_begin(s);
     launch_update_planes(a, s);
     prof_mark(s, "update_planes");
+    if (dev.p.count_pulses) count_pulses(a, false, s);
     launch_update_pulsed(a, s);
     prof_mark(s, "update_pulsed");
     RPU_HIP_CHECK(hipGetLastError());
@@ -605,6 +626,111 @@ struct Tile {
     last_stream = s;
   }
 
+  // RPUPulsed::driftWeights -> PulsedRPUDevice::driftWeights (rpu_pulsed_device.cpp:422-430) for a pulsed device,
+  // which drifts only when its parameters ask for it; RPUSimple::driftWeights (rpu.cpp:1581-1587) otherwise, with
+  // the one nu of the parameters.  WeightDrifter::apply (weight_drifter.cpp:108-150) starts the clocks at its
+  // first call.
+  void drift_device_weights(float time_since_last_call, hipStream_t s) {
+    check_maintenance("drift_weights");
+    const rpu_device_params &q = dev.p;
+    if (dev.pulsed() && !(q.drift_nu > 0.0f)) return;
+    const size_t n = size();
+    const bool per_device = arr.drift_nu.size() == n;
+    if (per_device && !nu_valid) {
+      d_nu.ensure(n);
+      RPU_HIP_CHECK(hipMemcpy(d_nu.p, arr.drift_nu.data(), n * sizeof(float), hipMemcpyHostToDevice));
+      nu_valid = true;
+    }
+    if (!dr_prev.p) {
+      dr_prev.ensure(n); dr_w0.ensure(n); dr_t.ensure(n);
+      RPU_HIP_CHECK(hipMemcpyAsync(dr_prev.p, d_w.p, n * sizeof(float), hipMemcpyDeviceToDevice, s));
+      RPU_HIP_CHECK(hipMemcpyAsync(dr_w0.p, d_w.p, n * sizeof(float), hipMemcpyDeviceToDevice, s));
+      launch_fill(dr_t.p, 0.0f, n, s);
+      drift_t = 0.0f;
+    }
+    drift_t += time_since_last_call / q.drift_t0;
+    DriftDev p{};
+    p.nu0 = q.drift_nu; p.nu_std = q.drift_nu_std; p.wg_ratio = q.drift_wg_ratio; p.g_offset = q.drift_g_offset;
+    p.w_offset = q.drift_w_offset; p.nu_k = q.drift_nu_k; p.log_g0 = q.drift_log_g0; p.reset_tol = q.drift_reset_tol;
+    p.w_read_std = q.drift_w_read_std;
+    p.a = q.drift_g_offset * q.drift_wg_ratio + q.drift_w_offset;
+    if (std::fabs(p.a) < p.reset_tol) p.a = 0.0f;
+    const bool random = p.nu_std > 0.0f || p.w_read_std > 0.0f;
+    launch_device_drift(d_w.p, dr_prev.p, dr_w0.p, dr_t.p, per_device ? d_nu.p : nullptr,
+                        dev.pulsed() ? d_wmin.p : nullptr, dev.pulsed() ? d_wmax.p : nullptr, p, drift_t, key(),
+                        random ? call++ : call, n, s);
+    RPU_HIP_CHECK(hipGetLastError());
+    last_stream = s;
+  }
+
+  // RPUSimple::remapWeights (rpu.cpp:1740-1747), WeightRemapper::apply (weight_remapper.cpp:19-190)
+  void remap_weights(const rpu_remap_params &q, float *scales_dev, hipStream_t s) {
+    check_maintenance("remap_weights");
+    switch (q.type) {
+    case RPU_REMAP_NONE:
+      return;
+    case RPU_REMAP_LAYERWISE_SYMMETRIC:
+    case RPU_REMAP_CHANNELWISE_SYMMETRIC:
+    case RPU_REMAP_CHANNELWISE_NORM:
+      break;
+    case RPU_REMAP_CHANNELWISE_ASYMMETRIC:
+      throw RpuError("Expect scales and biases given.");
+    default:
+      throw RpuError("Remapping type not implemented.");
+    }
+    if (!scales_dev) throw RpuError("Expect scales given.");
+    if (q.type == RPU_REMAP_CHANNELWISE_NORM && !(q.row_norm > 0.0f)) throw RpuError("Expect row_norm >0.");
+    if (q.type == RPU_REMAP_CHANNELWISE_SYMMETRIC && q.max_scale_range > 0.0f && q.remapped_wmax != 1.0f) {
+      throw RpuError("For max_scales set, expect wrmpar.remapped_wmax to be 1.");
+    }
+    s_rowstat.ensure(3 * (size_t)D + 1);
+    RemapDev p{};
+    p.type = q.type; p.clip_if = q.clip_if; p.max_scale_range = q.max_scale_range; p.max_scale_ref = q.max_scale_ref;
+    p.row_norm = q.row_norm; p.remapped_wmax = q.remapped_wmax;
+    launch_remap(d_w.p, scales_dev, s_rowstat.p, s_rowstat.p + D, s_rowstat.p + 2 * (size_t)D, X, D, p, s);
+    RPU_HIP_CHECK(hipGetLastError());
+    last_stream = s;
+  }
+
+  // RPUSimple::modifyFBWeights (rpu.cpp:1749-1758), WeightModifier::apply (weight_modifier.cpp:28-224)
+  void modify_weights(const rpu_modifier_params &q, hipStream_t s) {
+    check_maintenance("modify_weights");
+    if (q.type < RPU_MODIFIER_COPY || q.type > RPU_MODIFIER_PROG_NOISE) {
+      throw RpuError("Requested WeightModifierType not implemented.");
+    }
+    if (q.type == RPU_MODIFIER_PCM_NOISE) throw RpuError("Requested WeightModifierType not implemented in CPU version.");
+    if (q.type != RPU_MODIFIER_COPY && q.per_batch_sample) throw RpuError("Per batch sample is not implemented in RPUCuda");
+    if (q.n_coeffs < 0 || q.n_coeffs > RPU_MAX_MODIFIER_COEFFS) throw RpuError("Too many modifier coefficients.");
+    const size_t n = size();
+    d_fbw.ensure(n);
+    fb_during_test = q.enable_during_test != 0;
+    ModifierDev p{};
+    p.type = q.type; p.sto_round = q.sto_round; p.copy_last_column = q.copy_last_column; p.n_coeffs = q.n_coeffs;
+    p.std_dev = q.std_dev; p.res = q.res; p.dorefa_clip = q.dorefa_clip; p.pdrop = q.pdrop; p.g_max = q.g_max;
+    p.assumed_wmax = q.assumed_wmax;
+    for (int c = 0; c < q.n_coeffs; ++c) p.coeffs[c] = q.coeffs[c];
+    const float *amax_dev = nullptr;
+    if (q.rel_to_actual_wmax && q.type != RPU_MODIFIER_COPY) {
+      s_rowstat.ensure(3 * (size_t)D + 1);
+      launch_row_stat(d_w.p, X, D, q.copy_last_column ? X - 1 : X, 0, s_rowstat.p, s);
+      launch_max_or_one(s_rowstat.p, D, s_rowstat.p + 3 * (size_t)D, s);
+      amax_dev = s_rowstat.p + 3 * (size_t)D;
+    }
+    launch_modify(d_fbw.p, d_w.p, p, amax_dev, key(), call++, X, n, s);
+    RPU_HIP_CHECK(hipGetLastError());
+    last_stream = s;
+  }
+
+  // two 64-bit counters per cross-point, made at the first counted update
+  void count_pulses(const UpdateArgs &a, bool implicit, hipStream_t s) {
+    if (!d_cnt.p) {
+      d_cnt.ensure(2 * size());
+      launch_fill(reinterpret_cast<float *>(d_cnt.p), 0.0f, 4 * size(), s); // all-zero bits
+    }
+    launch_count_pulses(a, d_cnt.p, d_cnt.p + size(), implicit, s);
+    prof_mark(s, "count_pulses");
+  }
+
   // RPUSimple::setSharedWeights (rpu.cpp:1384-1398): the caller's memory becomes the weight matrix
   void set_shared_weights(float *w_dev) {
     check_maintenance("set_shared_weights");
@@ -659,14 +785,17 @@ struct Tile {
     prof_begin(s);
     launch_update_prepare(a, s);
     prof_mark(s, "update_prepare");
+    const bool counting = dev.p.count_pulses && !is_transfer();
     if (up.p.pulse_type == RPU_PULSE_STOCHASTIC_COMPRESSED) {
       launch_update_lines(a, s);
       prof_mark(s, "update_lines");
+      if (counting) count_pulses(a, false, s);
       launch_update_pulsed(a, s);
       prof_mark(s, "update_pulsed");
     } else {
       launch_update_implicit_lines(a, s);
       prof_mark(s, "update_implicit_lines");
+      if (counting) count_pulses(a, true, s);
       launch_update_implicit(a, s);
       prof_mark(s, "update_implicit");
     }
@@ -690,7 +819,7 @@ struct Tile {
     d_mat.ensure(B * D);
   }
 
-  void forward_indexed(const float *x, float *d, int n_images, long image_size, hipStream_t s) {
+  void forward_indexed(const float *x, float *d, int n_images, long image_size, bool is_test, hipStream_t s) {
     if (idx_patches <= 0) throw RpuError("The index matrix has not been set (set_matrix_indices).");
     if (n_images <= 0) throw RpuError("n_images must be positive.");
     if (D <= 32 && (long)n_images * idx_patches < (1L << 31)) {
@@ -698,7 +827,7 @@ struct Tile {
       const int B = n_images * idx_patches;
       s_rounds.ensure((size_t)B); // the only per-patch state that leaves the kernel: rounds run (get_bm_rounds)
       MvmArgs a{};
-      a.w = wdev(); a.x_size = X; a.d_size = D; a.m_batch = B; a.K = X; a.O = D;
+      a.w = mvm_weights(is_test); a.x_size = X; a.d_size = D; a.m_batch = B; a.K = X; a.O = D;
       a.io = io_dev(fio);
       a.alpha = fio.p.out_scale;
       a.max_rounds = fio.perfect ? 0 : mvm_max_rounds(a.io);
@@ -725,7 +854,7 @@ struct Tile {
     ensure_indexed(n_images);
     const int B = n_images * idx_patches;
     launch_gather_indexed(x_mat.p, x, x_idx.p, X, idx_patches, n_images, image_size, s);
-    mvm(x_mat.p, d_mat.p, B, false, false, false, false, s);
+    mvm(x_mat.p, d_mat.p, B, false, false, false, false, s, nullptr, nullptr, is_test);
     launch_bd_to_ndp(d, d_mat.p, n_images, D, idx_patches, s);
     RPU_HIP_CHECK(hipGetLastError());
   }
@@ -1071,8 +1200,7 @@ int rpu_tile_has_matrix_indices(const rpu_tile_t *tile) { return tile ? tile->t.
 
 int rpu_tile_forward_indexed(rpu_tile_t *tile, const float *x_dev, float *d_dev, int n_images, long image_size,
                              int is_test, void *stream) {
-  (void)is_test;
-  RPU_INDEXED_ENTRY(forward, t.forward_indexed(x_dev, d_dev, n_images, image_size, (hipStream_t)stream));
+  RPU_INDEXED_ENTRY(forward, t.forward_indexed(x_dev, d_dev, n_images, image_size, is_test != 0, (hipStream_t)stream));
 }
 
 int rpu_tile_backward_indexed(rpu_tile_t *tile, const float *d_dev, float *x_dev, int n_images, long image_size,
@@ -1115,6 +1243,53 @@ int rpu_tile_clip_weights(rpu_tile_t *tile, int clip_type, float fixed_value, fl
 
 int rpu_tile_reset_columns(rpu_tile_t *tile, int start_column_idx, int num_columns, float reset_prob, void *stream) {
   RPU_MAINTENANCE_ENTRY(t.reset_columns(start_column_idx, num_columns, reset_prob, (hipStream_t)stream));
+}
+
+int rpu_tile_drift_device_weights(rpu_tile_t *tile, float time_since_last_call, void *stream) {
+  RPU_MAINTENANCE_ENTRY(t.drift_device_weights(time_since_last_call, (hipStream_t)stream));
+}
+
+int rpu_tile_remap_weights(rpu_tile_t *tile, const rpu_remap_params *p, float *scales_dev, void *stream) {
+  if (!p) return guarded([] { throw RpuError("null parameters"); });
+  RPU_MAINTENANCE_ENTRY(t.remap_weights(*p, scales_dev, (hipStream_t)stream));
+}
+
+int rpu_tile_modify_weights(rpu_tile_t *tile, const rpu_modifier_params *p, void *stream) {
+  if (!p) return guarded([] { throw RpuError("null parameters"); });
+  RPU_MAINTENANCE_ENTRY(t.modify_weights(*p, (hipStream_t)stream));
+}
+
+int rpu_tile_get_modified_weights(rpu_tile_t *tile, float *w_host) {
+  return guarded([&] {
+    if (!tile || !w_host) throw RpuError("null argument");
+    Tile &t = tile->t;
+    std::lock_guard<std::mutex> lock(t.mutex);
+    if (!t.resident() || !t.d_fbw.p) throw RpuError("No modified weights: modify_weights has not been called.");
+    DeviceGuard g(t.device_id);
+    t.sync_last();
+    RPU_HIP_CHECK(hipMemcpy(w_host, t.d_fbw.p, t.size() * sizeof(float), hipMemcpyDeviceToHost));
+  });
+}
+
+int rpu_tile_pulse_counter_count(const rpu_tile_t *tile) {
+  return (tile && !tile->t.is_transfer() && tile->t.dev.pulsed() && tile->t.dev.p.count_pulses) ? 2 : 0;
+}
+
+int rpu_tile_get_pulse_counters(rpu_tile_t *tile, uint64_t *counters_host) {
+  return guarded([&] {
+    if (!tile || !counters_host) throw RpuError("null argument");
+    Tile &t = tile->t;
+    std::lock_guard<std::mutex> lock(t.mutex);
+    if (!rpu_tile_pulse_counter_count(tile)) throw RpuError("The tile does not count pulses (count_pulses).");
+    const size_t bytes = 2 * t.size() * sizeof(uint64_t);
+    if (!t.resident() || !t.d_cnt.p) {
+      std::memset(counters_host, 0, bytes); // nothing counted yet
+      return;
+    }
+    DeviceGuard g(t.device_id);
+    t.sync_last();
+    RPU_HIP_CHECK(hipMemcpy(counters_host, t.d_cnt.p, bytes, hipMemcpyDeviceToHost));
+  });
 }
 
 int rpu_tile_set_forward_out_scale(rpu_tile_t *tile, float out_scale) {
@@ -1245,7 +1420,7 @@ int rpu_group_destroy(rpu_group_t *group) {
 }
 
 static int group_mvm(rpu_group_t *group, const float *const *x_dev, const long *x_ld, float *const *y_dev,
-                     const long *y_ld, int m_batch, bool transposed, void *stream);
+                     const long *y_ld, int m_batch, bool transposed, bool is_test, void *stream);
 
 int rpu_group_forward(rpu_group_t *group, const float *const *x_dev, float *const *y_dev, int m_batch, int is_test,
                       void *stream) {
@@ -1254,18 +1429,17 @@ int rpu_group_forward(rpu_group_t *group, const float *const *x_dev, float *cons
 
 int rpu_group_forward_strided(rpu_group_t *group, const float *const *x_dev, const long *x_ld, float *const *y_dev,
                               const long *y_ld, int m_batch, int is_test, void *stream) {
-  (void)is_test;
-  return group_mvm(group, x_dev, x_ld, y_dev, y_ld, m_batch, false, stream);
+  return group_mvm(group, x_dev, x_ld, y_dev, y_ld, m_batch, false, is_test != 0, stream);
 }
 
 int rpu_group_backward_strided(rpu_group_t *group, const float *const *d_dev, const long *d_ld, float *const *x_dev,
                                const long *x_ld, int m_batch, void *stream) {
-  return group_mvm(group, d_dev, d_ld, x_dev, x_ld, m_batch, true, stream);
+  return group_mvm(group, d_dev, d_ld, x_dev, x_ld, m_batch, true, false, stream);
 }
 
 // forward (inputs x, outputs y) or backward (inputs d, outputs x) of all tiles of a group
 static int group_mvm(rpu_group_t *group, const float *const *x_dev, const long *x_ld, float *const *y_dev,
-                     const long *y_ld, int m_batch, bool transposed, void *stream) {
+                     const long *y_ld, int m_batch, bool transposed, bool is_test, void *stream) {
   return guarded([&] {
     if (!group || !x_dev || !y_dev) throw RpuError("null argument");
     if (m_batch <= 0) throw RpuError("m_batch must be positive.");
@@ -1299,7 +1473,7 @@ static int group_mvm(rpu_group_t *group, const float *const *x_dev, const long *
       t.check_compute(m_batch, x_dev[i], y_dev[i]);
       const int in_size = transposed ? t.D : t.X, out_size = transposed ? t.X : t.D;
       const bool big = use_big && out_size >= 128;
-      MvmArgs a = t.mvm_args(m_batch, transposed, nullptr, transposed ? t.bio : t.fio, big ? 1 : 0);
+      MvmArgs a = t.mvm_args(m_batch, transposed, t.mvm_weights(is_test), transposed ? t.bio : t.fio, big ? 1 : 0);
       a.in = x_dev[i]; a.in_sb = x_ld ? x_ld[i] : in_size; a.in_sk = 1;
       a.out = y_dev[i]; a.out_sb = y_ld ? y_ld[i] : out_size; a.out_so = 1;
       if (a.in_sb < in_size || a.out_sb < out_size) throw RpuError("A row stride is shorter than the row.");
@@ -1478,6 +1652,23 @@ int rpu_tile_clone(rpu_tile_t **out, const rpu_tile_t *src_c) {
       t.w_host.resize(s.size());
       RPU_HIP_CHECK(hipMemcpy(t.w_host.data(), s.d_w.p, s.size() * sizeof(float), hipMemcpyDeviceToHost));
       t.to_device(s.device_id);
+      // modified weights, drift clocks and pulse counters travel with the copy
+      const size_t n = s.size();
+      const auto dup = [&](DevBuf<float> &dst, const DevBuf<float> &from) {
+        if (!from.p) return;
+        dst.ensure(n);
+        RPU_HIP_CHECK(hipMemcpy(dst.p, from.p, n * sizeof(float), hipMemcpyDeviceToDevice));
+      };
+      dup(t.d_fbw, s.d_fbw);
+      t.fb_during_test = s.fb_during_test;
+      dup(t.dr_prev, s.dr_prev);
+      dup(t.dr_w0, s.dr_w0);
+      dup(t.dr_t, s.dr_t);
+      t.drift_t = s.drift_t;
+      if (s.d_cnt.p) {
+        t.d_cnt.ensure(2 * n);
+        RPU_HIP_CHECK(hipMemcpy(t.d_cnt.p, s.d_cnt.p, 2 * n * sizeof(unsigned long long), hipMemcpyDeviceToDevice));
+      }
     }
     *out = h.release();
   });
@@ -1497,14 +1688,16 @@ int rpu_tile_destroy(rpu_tile_t *tile) {
 
 int rpu_tile_forward(rpu_tile_t *tile, const float *x_dev, float *y_dev, int m_batch, int bias, int x_trans,
                      int d_trans, int is_test, void *stream) {
-  (void)is_test; // the analog forward pass is the same in training and evaluation (rpu_forward_backward_pass.cpp:816-818)
+  // the analog forward pass is the same in training and evaluation (rpu_forward_backward_pass.cpp:816-818); is_test
+  // only decides whether modified weights are used
   return guarded([&] {
     if (!tile) throw RpuError("null tile");
     Tile &t = tile->t;
     std::lock_guard<std::mutex> lock(t.mutex);
     t.check_compute(m_batch, x_dev, y_dev);
     DeviceGuard g(t.device_id);
-    t.mvm(x_dev, y_dev, m_batch, bias != 0, x_trans != 0, d_trans != 0, false, (hipStream_t)stream);
+    t.mvm(x_dev, y_dev, m_batch, bias != 0, x_trans != 0, d_trans != 0, false, (hipStream_t)stream, nullptr, nullptr,
+          is_test != 0);
   });
 }
 
@@ -1655,9 +1848,10 @@ static std::vector<float> *hidden_array(DeviceArrays &arr, int idx) {
   case 4: return &arr.decay_scale;
   case 5: return &arr.diffusion_rate;
   case 6: return &arr.reset_bias;
+  case 7: return arr.drift_nu.empty() ? nullptr : &arr.drift_nu; // without a drifter reported as zeros
   case 8: return &arr.slope_up;
   case 9: return &arr.slope_down;
-  default: return nullptr; // drift_nu: no drifter on this path, reported as zeros
+  default: return nullptr;
   }
 }
 

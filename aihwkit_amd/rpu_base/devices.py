@@ -72,6 +72,71 @@ class WeightClipParameter:
         self.sigma = float(sigma)
 
 
+class WeightRemapType(enum.IntEnum):
+    """src/rpucuda/weight_remapper.h:14-22 (the bindings expose the first three, rpu_base_utils.cpp:44-47)."""
+
+    NONE = 0
+    LayerwiseSymmetric = 1
+    ChannelwiseSymmetric = 2
+    ChannelwiseNorm = 3
+    ChannelwiseExceeded = 4
+    LayerwiseAsymmetric = 5
+    ChannelwiseAsymmetric = 6
+
+
+class WeightRemapParameter:
+    """src/rpucuda/weight_remapper.h:25-38 (``rpu_base.tiles.WeightRemapParameter``, rpu_base_utils.cpp:24-29)."""
+
+    def __init__(self):
+        self.type = WeightRemapType.NONE
+        self.max_scale_range = 0.0
+        self.max_scale_ref = 0.0
+        self.row_norm = 1.0
+        self.remapped_wmax = 1.0
+        self.clip_if = True
+
+
+class WeightModifierType(enum.IntEnum):
+    """src/rpucuda/weight_modifier.h:14-25 (rpu_base_utils.cpp:31-42)."""
+
+    Copy = 0
+    Discretize = 1
+    MultNormal = 2
+    AddNormal = 3
+    DiscretizeAddNormal = 4
+    DoReFa = 5
+    Poly = 6
+    PCMNoise = 7
+    DropConnect = 8
+    ProgNoise = 9
+
+
+class WeightModifierParameter:
+    """src/rpucuda/weight_modifier.h:27-50 (``rpu_base.tiles.WeightModifierParameter``, rpu_base_tiles.cpp:30-51).
+    The pcm_* fields belong to the PCMNoise type, which only the reference's CUDA code has."""
+
+    def __init__(self):
+        self.type = WeightModifierType.Copy
+        self.std_dev = 0.0
+        self.per_batch_sample = False
+        self.res = 0.1
+        self.sto_round = False
+        self.dorefa_clip = 0.6
+        self.pdrop = 0.0
+        self.enable_during_test = False
+        self.copy_last_column = False
+        self.rel_to_actual_wmax = True
+        self.assumed_wmax = 1.0
+        self.g_max = 25.0
+        self.coeffs = [0.26348 / 25.0, 0.0768, -0.001877 * 25.0]
+        self.pcm_zero_thres = 0.0
+        self.pcm_t_inference = 0.0
+        self.pcm_prob_at_reset = 0.0
+        self.pcm_prob_at_gmax = 0.0
+        self.pcm_prob_at_random = 0.0
+        self.pcm_t0 = 20.0
+
+
 class AnalogMVType(enum.IntEnum):
     """rpu_base_utils.cpp:87-91."""
 
@@ -82,8 +147,9 @@ class AnalogMVType(enum.IntEnum):
 
 
 # pybind exposes the member called "None" of each enum; Python's enum cannot define it in the class body.
-for _e in (BoundManagementType, NoiseManagementType, WeightNoiseType, PulseType):
+for _e in (BoundManagementType, NoiseManagementType, WeightNoiseType, PulseType, WeightClipType, WeightRemapType):
     setattr(_e, "None", _e.NONE)  # reachable through getattr(Enum, "None") like the reference
+setattr(WeightModifierType, "None", WeightModifierType.Copy)  # rpu_base_utils.cpp:42
 
 
 class _Struct:
@@ -92,8 +158,11 @@ class _Struct:
     _defaults = {}
 
     def __init__(self):
+        import copy
+
         for name, value in self._all_defaults().items():
-            object.__setattr__(self, name, value)
+            # a nested struct is this object's own
+            object.__setattr__(self, name, copy.deepcopy(value) if isinstance(value, _Struct) else value)
 
     @classmethod
     def _all_defaults(cls):
@@ -109,6 +178,11 @@ class _Struct:
 
     def _all_values(self):
         return {k: getattr(self, k) for k in self._all_defaults()}
+
+    def __eq__(self, other):
+        return type(other) is type(self) and other._all_values() == self._all_values()
+
+    __hash__ = None
 
     def __str__(self):
         fields = ", ".join(f"{k}={getattr(self, k)!r}" for k in self._all_defaults())
@@ -173,16 +247,37 @@ class AnalogTileUpdateParameter(_Struct):
         return p
 
 
-class AbstractResistiveDeviceParameter(_Struct):
-    """rpu_base_devices.cpp:536-539 (+ the SimpleMetaParameter fields diffusion / lifetime)."""
+class DriftParameter(_Struct):
+    """rpu_base_devices.cpp:521-533 over DriftParameter (src/rpucuda/weight_drifter.h:14-60): power-law drift
+    w = w0 (delta_t / t_0)^(-nu) of a training tile; active on a pulsed device when nu > 0."""
 
-    _defaults = dict(construction_seed=0, diffusion=0.0, lifetime=0.0)
+    _defaults = dict(nu=0.0, nu_dtod=0.0, nu_std=0.0, wg_ratio=1.0, g_offset=0.0, w_offset=0.0, nu_k=0.0,
+                     log_g0=0.0, t_0=1.0, reset_tol=1e-7, w_noise_std=0.0)
+
+    _C_NAMES = dict(nu="drift_nu", nu_dtod="drift_nu_dtod", nu_std="drift_nu_std", wg_ratio="drift_wg_ratio",
+                    g_offset="drift_g_offset", w_offset="drift_w_offset", nu_k="drift_nu_k",
+                    log_g0="drift_log_g0", t_0="drift_t0", reset_tol="drift_reset_tol",
+                    w_noise_std="drift_w_read_std")
+
+    def _fill_c(self, p: DeviceParams, simple: bool = False) -> None:
+        for name, c_name in self._C_NAMES.items():
+            setattr(p, c_name, float(getattr(self, name)))
+        if simple:
+            p.drift_nu_dtod = 0.0  # DriftParameter::setSimpleDrift (weight_drifter.h:46-49)
+
+
+class AbstractResistiveDeviceParameter(_Struct):
+    """rpu_base_devices.cpp:536-539 (+ the SimpleMetaParameter fields diffusion / lifetime / drift)."""
+
+    _defaults = dict(construction_seed=0, diffusion=0.0, lifetime=0.0, drift=DriftParameter())
     _kind = None
 
     def _fill_c(self, p: DeviceParams) -> None:
         p.construction_seed = int(self.construction_seed)
         p.diffusion = float(self.diffusion)
         p.lifetime = float(self.lifetime)
+        if self.drift is not None:
+            self.drift._fill_c(p)
 
     def _to_c(self) -> DeviceParams:
         from .._cabi import check, lib
@@ -224,8 +319,7 @@ class PulsedResistiveDeviceParameter(AbstractResistiveDeviceParameter):
         p.dw_min_dtod_log_normal = int(bool(self.dw_min_dtod_log_normal))
         p.enforce_consistency = int(bool(self.enforce_consistency))
         p.perfect_bias = int(bool(self.perfect_bias))
-        if self.count_pulses:
-            raise RuntimeError("count_pulses is not implemented on this path.")
+        p.count_pulses = int(bool(self.count_pulses))
 
     def calc_weight_granularity(self) -> float:
         """rpu_constantstep_device.h:27, rpu_linearstep_device.h:58: the granularity is dw_min."""
@@ -391,7 +485,7 @@ class AnalogTileParameter(_Struct):
 class FloatingPointTileParameter(_Struct):
     """rpu_base_devices.cpp:436-451: floating-point tile = ideal device with perfect IO and no pulses."""
 
-    _defaults = dict(diffusion=0.0, lifetime=0.0, drift=None)
+    _defaults = dict(diffusion=0.0, lifetime=0.0, drift=DriftParameter())
 
     def create_array(self, x_size: int, d_size: int):
         import copy
@@ -405,7 +499,10 @@ class FloatingPointTileParameter(_Struct):
         device = IdealResistiveDeviceParameter()
         device.diffusion = float(self.diffusion)
         device.lifetime = float(self.lifetime)
-        tile = FloatingPointTile._create(int(x_size), int(d_size), meta._config(device))
+        config = meta._config(device)
+        if self.drift is not None:
+            self.drift._fill_c(config.device, simple=True)  # RPUSimple::driftWeights (rpu.cpp:1581-1587)
+        tile = FloatingPointTile._create(int(x_size), int(d_size), config)
         tile._meta_parameters, tile._parameters = copy.deepcopy(self), copy.deepcopy(self)
         return tile
 

@@ -15,7 +15,10 @@ from typing import List
 
 import torch
 
-from .._cabi import check, lib
+from .._cabi import MAX_MODIFIER_COEFFS, ModifierParams, RemapParams, check, lib
+# the reference binds these parameter structs in its tiles module (rpu_base_utils.cpp:17-58)
+from .devices import (WeightClipParameter, WeightClipType, WeightModifierParameter,  # noqa: F401
+                      WeightModifierType, WeightRemapParameter, WeightRemapType)
 
 _DTYPE = torch.float32
 
@@ -96,16 +99,23 @@ class _TileBase:
         shape = (self.get_d_size(), self.get_x_size())
         self.set_weights(torch.rand(shape, dtype=_DTYPE) * (float(max_value) - float(min_value)) + float(min_value))
 
-    # -- hardware-aware-training utilities and device-level drift of the reference bindings that this library does
-    #    not provide (rpu_base_tiles.cpp:292-371, 845-868)
-    def _not_provided(self, *args, **kwargs):
-        raise RuntimeError("Not provided by this library: drift_weights (device-level power-law drift), "
-                           "remap_weights, modify_weights and get_pulse_counters.")
+    # -- hardware-aware-training utilities of the reference bindings (rpu_base_tiles.cpp:292-371, 845-868): they work
+    #    on the matrix in HBM and are methods of the GPU tiles
+    def _needs_gpu(self, *args, **kwargs):
+        raise RuntimeError("Host tiles do not compute: build a CudaAnalogTile(tile) / CudaFloatingPointTile(tile).")
 
-    drift_weights = _not_provided
-    remap_weights = _not_provided
-    modify_weights = _not_provided
-    get_pulse_counters = _not_provided
+    drift_weights = _needs_gpu
+    remap_weights = _needs_gpu
+    modify_weights = _needs_gpu
+
+    def get_pulse_counters(self) -> torch.Tensor:
+        """int64 [2, d_size, x_size] (up-counting pulses where the signs of x and d agree, then where they differ)
+        of a tile whose device has ``count_pulses`` set, else an empty tensor (rpu_base_tiles.cpp:845-868)."""
+        if not lib().rpu_tile_pulse_counter_count(self._h):
+            return torch.empty(0, dtype=torch.int64)
+        out = torch.empty(2, self.get_d_size(), self.get_x_size(), dtype=torch.int64)
+        check(lib().rpu_tile_get_pulse_counters(self._h, out.data_ptr()))
+        return out
 
     # -- sizes / learning rate (rpu_base_tiles.cpp get_x_size, get_d_size, get/set_learning_rate)
     def get_x_size(self) -> int:
@@ -331,6 +341,48 @@ class _CudaTileMixin:
     def reset_columns(self, start_column_idx: int = 0, num_columns: int = 1, reset_prob: float = 1.0) -> None:
         check(lib().rpu_tile_reset_columns(self._h, int(start_column_idx), int(num_columns), float(reset_prob),
                                            self._current_stream()))
+
+    def drift_weights(self, time_since_last_call: float) -> None:
+        """Power-law drift of the weights that have not changed since the last call (rpu_base_tiles.cpp:293-313)."""
+        check(lib().rpu_tile_drift_device_weights(self._h, float(time_since_last_call), self._current_stream()))
+
+    def remap_weights(self, weight_remap_params, scales: torch.Tensor) -> torch.Tensor:
+        """Rescales the rows of the weights, ``scales`` ([d_size], on the tile's GPU) takes the factors up in place
+        and is returned (rpu_base_tiles.cpp:330-356)."""
+        if isinstance(scales, torch.Tensor) and not scales.is_contiguous():
+            raise RuntimeError("scales must be contiguous")
+        scales = _check_input(scales, True, "scales")
+        if scales.numel() != self.get_d_size() or scales.dim() != 1:
+            raise RuntimeError("Invalid scales dimensions: expected [%d] tensor" % self.get_d_size())
+        par = weight_remap_params
+        c_par = RemapParams(int(par.type), int(bool(getattr(par, "clip_if", True))), float(par.max_scale_range),
+                            float(par.max_scale_ref), float(getattr(par, "row_norm", 1.0)), float(par.remapped_wmax))
+        check(lib().rpu_tile_remap_weights(self._h, C.byref(c_par), scales.data_ptr(), self._current_stream()))
+        return scales
+
+    def modify_weights(self, weight_modifier_params) -> None:
+        """Makes the modified copy of the weights that forward and backward use from now on
+        (rpu_base_tiles.cpp:357-371)."""
+        par = weight_modifier_params
+        coeffs = [float(c) for c in par.coeffs]
+        if len(coeffs) > MAX_MODIFIER_COEFFS:
+            raise RuntimeError("At most %d modifier coefficients." % MAX_MODIFIER_COEFFS)
+        c_par = ModifierParams()
+        c_par.type = int(par.type)
+        for name in ("per_batch_sample", "sto_round", "enable_during_test", "copy_last_column", "rel_to_actual_wmax"):
+            setattr(c_par, name, int(bool(getattr(par, name))))
+        for name in ("std_dev", "res", "dorefa_clip", "pdrop", "assumed_wmax", "g_max"):
+            setattr(c_par, name, float(getattr(par, name)))
+        c_par.n_coeffs = len(coeffs)
+        for k, c in enumerate(coeffs):
+            c_par.coeffs[k] = c
+        check(lib().rpu_tile_modify_weights(self._h, C.byref(c_par), self._current_stream()))
+
+    def get_modified_weights(self) -> torch.Tensor:
+        """[d_size, x_size] CPU tensor of the weights forward and backward contract with after ``modify_weights``."""
+        out = torch.empty(self.get_d_size(), self.get_x_size(), dtype=_DTYPE)
+        check(lib().rpu_tile_get_modified_weights(self._h, out.data_ptr()))
+        return out
 
     # -- shared and delta weights (rpu_base_tiles.cpp:215-251)
     def _check_matrix(self, tensor: torch.Tensor, what: str) -> torch.Tensor:

@@ -180,6 +180,19 @@ typedef struct rpu_device_params {
   float ls_decrease_up_dtod;         /* 0.05 */
   float ls_decrease_down_dtod;       /* 0.05 */
   float ls_reverse_offset;           /* 0.01 */
+  /* Power-law drift of the device (DriftParameter, R/weight_drifter.h:14-60); active when drift_nu > 0. */
+  float drift_nu;                    /* 0 */
+  float drift_nu_dtod;               /* 0 */
+  float drift_nu_std;                /* 0 (redrawn at every call) */
+  float drift_wg_ratio;              /* 1 */
+  float drift_g_offset;              /* 0 */
+  float drift_w_offset;              /* 0 */
+  float drift_nu_k;                  /* 0 */
+  float drift_log_g0;                /* 0 */
+  float drift_t0;                    /* 1 */
+  float drift_reset_tol;             /* 1e-7 */
+  float drift_w_read_std;            /* 0 */
+  int32_t count_pulses;              /* 0 ; 1: every update also counts the pulses of each cross-point */
 } rpu_device_params;
 
 /* Replaces PulsedMetaParameter<float> (R/rpu_pulsed.h:127-151): forward IO, backward IO, update. */
@@ -443,6 +456,89 @@ int rpu_tile_clip_weights(rpu_tile_t *tile, int clip_type, float fixed_value, fl
  * to reset_bias + reset_std * N(0, 1) and clipped, each element with probability reset_prob
  * (rpu_pulsed_device.cpp:469-494; without bias and bounds on other tiles, rpu_simple_device.cpp:148-168). */
 int rpu_tile_reset_columns(rpu_tile_t *tile, int start_column_idx, int num_columns, float reset_prob, void *stream);
+
+/* drift_weights of a training tile (rpu_base_tiles.cpp:293-313): power-law conductance drift
+ * w = w0 * (delta_t / t0)^(-nu) of every weight that has not changed by more than reset_tol since the last call;
+ * a changed weight restarts its drift clock (src/rpucuda/weight_drifter.cpp:108-150).  A pulsed device has its own
+ * nu per cross-point (hidden parameter drift_nu) and saturates at its bounds (rpu_pulsed_device.cpp:422-430); other
+ * tiles drift with the one nu of their parameters (src/rpucuda/rpu.cpp:1581-1587).  The drift fields of
+ * rpu_device_params configure it; with drift_nu <= 0 on a pulsed device the call does nothing, as in the reference.
+ * Not to be confused with rpu_tile_drift_weights, the PCM inference drift above. */
+int rpu_tile_drift_device_weights(rpu_tile_t *tile, float time_since_last_call, void *stream);
+
+/* remap_weights (rpu_base_tiles.cpp:330-356) with the fields of WeightRemapParameter
+ * (src/rpucuda/weight_remapper.h:25-38): the rows of the weight matrix are divided by a factor that the per-row
+ * output scales scales_dev[d_size] (device memory, updated in place) take up, so that scales[i] * W[i][:] stays
+ * what it was (src/rpucuda/weight_remapper.cpp:19-190).  Layerwise symmetric: the largest absolute weight maps to
+ * remapped_wmax; channelwise symmetric: that of each row does, optionally with the spread of the scales bounded
+ * by max_scale_range; channelwise norm: rows whose norm exceeds row_norm are scaled down to it (the scales take the
+ * factor unless clip_if).  The asymmetric types need biases, which the reference's binding does not pass, and
+ * ChannelwiseExceeded needs the signal-channel bound management: both are refused. */
+enum rpu_remap_type {
+  RPU_REMAP_NONE = 0,
+  RPU_REMAP_LAYERWISE_SYMMETRIC = 1,
+  RPU_REMAP_CHANNELWISE_SYMMETRIC = 2,
+  RPU_REMAP_CHANNELWISE_NORM = 3,
+  RPU_REMAP_CHANNELWISE_EXCEEDED = 4,
+  RPU_REMAP_LAYERWISE_ASYMMETRIC = 5,
+  RPU_REMAP_CHANNELWISE_ASYMMETRIC = 6
+};
+typedef struct rpu_remap_params {
+  int32_t type;          /* enum rpu_remap_type, NONE */
+  int32_t clip_if;       /* 1 */
+  float max_scale_range; /* 0 */
+  float max_scale_ref;   /* 0 */
+  float row_norm;        /* 1 */
+  float remapped_wmax;   /* 1 */
+} rpu_remap_params;
+int rpu_tile_remap_weights(rpu_tile_t *tile, const rpu_remap_params *p, float *scales_dev, void *stream);
+
+/* modify_weights (rpu_base_tiles.cpp:357-371) with the fields of WeightModifierParameter
+ * (src/rpucuda/weight_modifier.h:27-50): makes a modified copy of the weights that forward and backward (not the
+ * update) contract with from then on; during evaluation (is_test) only if enable_during_test
+ * (src/rpucuda/rpu.cpp:1483-1487, 1749-1758; src/rpucuda/weight_modifier.cpp:28-224).  The reference value amax is
+ * the largest absolute weight (rel_to_actual_wmax; without the last column under copy_last_column) or
+ * assumed_wmax.  PCMNoise exists only in the reference's CUDA code and is refused; per_batch_sample is refused as
+ * in the reference. */
+enum rpu_modifier_type {
+  RPU_MODIFIER_COPY = 0,
+  RPU_MODIFIER_DISCRETIZE = 1,
+  RPU_MODIFIER_MULT_NORMAL = 2,
+  RPU_MODIFIER_ADD_NORMAL = 3,
+  RPU_MODIFIER_DISCRETIZE_ADD_NORMAL = 4,
+  RPU_MODIFIER_DOREFA = 5,
+  RPU_MODIFIER_POLY = 6,
+  RPU_MODIFIER_PCM_NOISE = 7,
+  RPU_MODIFIER_DROP_CONNECT = 8,
+  RPU_MODIFIER_PROG_NOISE = 9
+};
+#define RPU_MAX_MODIFIER_COEFFS 8
+typedef struct rpu_modifier_params {
+  int32_t type;               /* enum rpu_modifier_type, COPY */
+  int32_t per_batch_sample;   /* 0 */
+  int32_t sto_round;          /* 0 */
+  int32_t enable_during_test; /* 0 */
+  int32_t copy_last_column;   /* 0 */
+  int32_t rel_to_actual_wmax; /* 1 */
+  int32_t n_coeffs;           /* 3 */
+  float std_dev;              /* 0 */
+  float res;                  /* 0.1 */
+  float dorefa_clip;          /* 0.6 */
+  float pdrop;                /* 0 */
+  float assumed_wmax;         /* 1 */
+  float g_max;                /* 25 */
+  float coeffs[RPU_MAX_MODIFIER_COEFFS]; /* 0.26348 / 25, 0.0768, -0.001877 * 25 */
+} rpu_modifier_params;
+int rpu_tile_modify_weights(rpu_tile_t *tile, const rpu_modifier_params *p, void *stream);
+/* Host copy [d_size][x_size] of the modified weights; returns an error if none have been made. */
+int rpu_tile_get_modified_weights(rpu_tile_t *tile, float *w_host);
+
+/* get_pulse_counters (rpu_base_tiles.cpp:845-868, src/rpucuda/cuda/rpucuda_pulsed_device.cu:316-343): with
+ * count_pulses set in the device parameters every pulsed update adds, per cross-point, the number of up and of
+ * down pulses it applies to two 64-bit counters.  counters_host is [2][d_size][x_size], positive first; the
+ * return value of rpu_tile_pulse_counter_count is 2 when the tile counts and 0 otherwise. */
+int rpu_tile_pulse_counter_count(const rpu_tile_t *tile);
+int rpu_tile_get_pulse_counters(rpu_tile_t *tile, uint64_t *counters_host);
 
 /* Replaces the out_scale of the forward IO parameters (rpu_io_params.out_scale) from now on.  No counterpart in the
  * reference, which applies run-time output factors such as the drift-compensation alpha to the output tensor in

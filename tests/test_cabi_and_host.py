@@ -227,8 +227,18 @@ def test_parameter_accessors_and_random_weights_on_a_host_tile():
     assert w.min() >= -0.2 and w.max() <= 0.1 and w.std() > 0.03
     hidden = dict(zip(tile.get_hidden_parameter_names(), tile.get_hidden_parameters()))
     assert (w <= hidden["max_bound"]).all() and (w >= hidden["min_bound"]).all()
-    for name in ("drift_weights", "remap_weights", "modify_weights", "get_pulse_counters"):
-        with pytest.raises(RuntimeError, match="Not provided"):
+    for name in ("drift_weights", "remap_weights", "modify_weights"):       # they work on the matrix in HBM
+        with pytest.raises(RuntimeError, match="Host tiles do not compute"):
             getattr(tile, name)()
+    assert tile.get_pulse_counters().numel() == 0                           # count_pulses is off
+    dev.count_pulses = True
+    dev.drift.nu = 0.05
+    dev.drift.nu_dtod = 0.1
+    counting = meta.create_array(7, 5, dev)
+    assert counting.get_pulse_counters().shape == (2, 5, 7) and counting.get_pulse_counters().sum() == 0
+    nu = dict(zip(counting.get_hidden_parameter_names(), counting.get_hidden_parameters()))["drift_nu"]
+    assert abs(float(nu.mean()) - 0.05) < 0.005 and 0.002 < float(nu.std()) < 0.01   # nu (1 + nu_dtod N(0, 1))
+    assert float(hidden["drift_nu"].abs().max()) == 0.0                     # no drifter: zeros, as the reference
+    assert dv.SoftBoundsResistiveDeviceParameter().drift.nu == 0.0          # a struct of its own per object
     fp = dv.FloatingPointTileParameter().create_array(3, 2)
     assert fp.get_meta_parameters().lifetime == 0.0
