@@ -57,6 +57,12 @@ struct MvmArgs {
   MvmState st;
   PhiloxKey key;
   uint32_t call;
+  // Analog non-idealities that add to the sums before the ADC stage (output-referred weight noise, IR drop):
+  // pre_add[row * O + o] for the output o of the sample whose quantized input is row `row` of xq[round & 1];
+  // null: none.  Only the 32 x 32 round kernels read it.
+  const float *pre_add;
+  int small_tiles_only;     // 1: never the large-tile kernel (its row padding differs)
+  const int *skip_if_zero;  // non-null: a round launch does nothing when this device value is zero
 };
 
 // noise management + per-sample state for round 0
@@ -93,6 +99,20 @@ struct ConvArgs {
 };
 bool conv_forward_supported(const MvmArgs &a);
 void launch_conv_forward(const MvmArgs &a, const ConvArgs &c, hipStream_t s);
+
+// ---- analog non-idealities before the ADC (kernels_nonideal.hip), rpu_forward_backward_pass.cpp:325-433, 535-560
+// transformed copy of the quantized input rows [rows][k_pad]: mode 0 x^2, 1 |x|, 2 x (1 - (1 - j / K)^2)
+void launch_side_rows(const float *xq, float *out, int rows, int k_pad, int K, int mode, const int *skip_if_zero,
+                      hipStream_t s);
+void launch_abs_copy(const float *w, float *out, size_t n, hipStream_t s);
+struct SideDev {
+  int w_noise_type; // 0 none, 1 additive constant (row_sumsq), 2 PCM read (s_noise)
+  float w_noise, ir_drop, a_scale; // a_scale = in_size / ir_drop_g_ratio
+};
+// pre[row][o] = w_noise term * N(0, 1) - IR-drop term; s_cur / s_ir are null without IR drop
+void launch_side_combine(float *pre, const float *s_noise, const float *row_sumsq, const float *s_cur, const float *s_ir,
+                         const SideDev &p, int rows, int O, PhiloxKey key, uint32_t call, int round,
+                         const int *skip_if_zero, hipStream_t s);
 
 // number of rounds that can ever be needed with these IO settings
 int mvm_max_rounds(const IoDev &io);

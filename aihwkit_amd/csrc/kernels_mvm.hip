@@ -124,7 +124,7 @@ __host__ __device__ __forceinline__ int workgroups_for(int O, int n_act, int edg
 // ADC of the four analog sums v of outputs o0 .. o0 + 3 of sample b: asymmetry, noise, quantization, clipping, output
 // factor; up / lo return 1 + the largest output index that hit the upper / lower bound (0: none)
 __device__ __forceinline__ void mvm_adc_values(const MvmArgs &a, int round, int b, float fin, int o0, float (&v)[4],
-                                               int &up, int &lo) {
+                                               int &up, int &lo, const float *pre = nullptr) {
   float nz[4] = {0.f, 0.f, 0.f, 0.f};
   if (a.io.out_noise > 0.0f) {
     philox_normal4((uint32_t)(o0 >> 2), (uint32_t)b, a.call, RNG_OUT_NOISE | ((uint32_t)round << 8), a.key, nz);
@@ -134,6 +134,7 @@ __device__ __forceinline__ void mvm_adc_values(const MvmArgs &a, int round, int 
 #pragma unroll
   for (int q = 0; q < 4; ++q) {
     float y = v[q];
+    if (pre && o0 + q < a.O) y += pre[o0 + q]; // weight noise, IR drop (rpu_forward_backward_pass.cpp:535-560)
     if (a.io.out_asym > 0.0f) y = y < 0.0f ? y * (1.0f - a.io.out_asym) : y;
     if (a.io.out_noise > 0.0f) y += a.io.out_noise * nz[q];
     if (a.io.out_res > 0.0f) {
@@ -158,7 +159,7 @@ __device__ __forceinline__ void mvm_adc_values(const MvmArgs &a, int round, int 
 // ADC stage for outputs o0 .. o0 + 3 of sample b: v holds the analog sums (rpu_forward_backward_pass.cpp:666-719)
 // up / lo return 1 + the largest output index that hit the upper / lower ADC bound (0: none).
 __device__ __forceinline__ void mvm_finish_outputs(const MvmArgs &a, int round, int b, float fin, int o0, float (&v)[4],
-                                                   int &up, int &lo) {
+                                                   int &up, int &lo, const float *pre = nullptr) {
   up = 0;
   lo = 0;
   float *out_p = a.out + (long)b * a.out_sb + (long)o0 * a.out_so;
@@ -182,7 +183,7 @@ __device__ __forceinline__ void mvm_finish_outputs(const MvmArgs &a, int round, 
     return;
   }
 
-  mvm_adc_values(a, round, b, fin, o0, v, up, lo);
+  mvm_adc_values(a, round, b, fin, o0, v, up, lo, pre);
   if (a.out_so == 1 && (o0 + 3) < a.O && ((((uintptr_t)out_p) & 15) == 0)) {
     *reinterpret_cast<float4 *>(out_p) = make_float4(v[0], v[1], v[2], v[3]);
   } else {
@@ -443,7 +444,14 @@ __device__ __forceinline__ void mvm_round_tile(const MvmArgs &a, int round, int 
   }
   const int o0 = tile_o * TILE + wave * 8 + h * 4;
   int up = 0, lo = 0;
-  if (b_ok && o0 < a.O) mvm_finish_outputs(a, round, b_out, fin_out, o0, v, up, lo);
+  if (b_ok && o0 < a.O) {
+    const float *pre = nullptr;
+    if (a.pre_add) {
+      const int xrow = (round > 0) ? pick2(a.st.row, round & 1)[slot_in] : slot_in;
+      pre = a.pre_add + (long)xrow * a.O;
+    }
+    mvm_finish_outputs(a, round, b_out, fin_out, o0, v, up, lo, pre);
+  }
   if (!a.io.perfect && a.io.bound_management != RPU_BM_NONE) {
     // saturation flags of the tile's 32 samples: combined in LDS, then one device-scope atomic per sample
     // and bound.  The returned values are consumed so that the wave waits until the atomics have been
@@ -891,6 +899,7 @@ template <int PD, int WMODE>
 __global__ __launch_bounds__(256) void k_mvm_round(MvmArgs a) {
   __shared__ float red[WAVES][16][64];
   __shared__ __attribute__((aligned(16))) float stage[WAVES * 2 * TILE * LDS_ROW];
+  if (a.skip_if_zero && *a.skip_if_zero == 0) return;
   const int n_act = (a.round > 0) ? a.st.count[a.round] : a.m_batch;
   if (runs_on_large_tiles(a, a.round, n_act)) return;
   mvm_round_workgroup<PD, WMODE>(a, a.round, blockIdx.x, n_act, red, stage);
@@ -1727,7 +1736,7 @@ void launch_mvm_round_group(const MvmGroup &g, int depth, int mode, int total_wo
 
 void launch_mvm_round(const MvmArgs &a_in, hipStream_t s) {
   MvmArgs a = a_in;
-  a.big_from = big_threshold(a.m_batch, a.O);
+  a.big_from = a.small_tiles_only ? 0 : big_threshold(a.m_batch, a.O);
   if (a.big_from > 0) {
     const dim3 big_grid(big_workgroups(a));
     const int min_active = a.round > 0 ? a.big_from : 0;

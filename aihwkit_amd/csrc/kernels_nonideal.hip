@@ -1,0 +1,99 @@
+// Analog non-idealities of the MVM that act on the sums before the ADC stage: output-referred weight noise
+// (ForwardBackwardPassIOManaged::applyOutputWeightNoise, rpu_forward_backward_pass.cpp:325-385) and IR drop
+// (applyIrDrop, :387-433, with computeTotalCurrent, :508-530).  Each of them needs one or two more contractions of
+// the same shape as the MVM itself, over transformed operands (|W| with x^2 or |x|, W with position-weighted x);
+// those run on the MFMA round kernel.  The kernels here make the transformed operands and combine the results
+// into the one addend per output that the ADC stage of the round kernel reads.
+#include "kernels.h"
+
+namespace rpu_amd {
+
+namespace {
+
+int grid_for(size_t n) {
+  const size_t blocks = (n + 255) / 256;
+  return (int)(blocks > 8192 ? 8192 : (blocks ? blocks : 1));
+}
+
+__global__ __launch_bounds__(256) void k_side_rows(const float *xq, float *out, size_t total, int k_pad, int K, int mode,
+                                                    const int *skip_if_zero) {
+  if (skip_if_zero && *skip_if_zero == 0) return;
+  for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+    const int j = (int)(i % k_pad);
+    const float x = xq[i];
+    float v;
+    if (mode == 0) {
+      v = x * x;
+    } else if (mode == 1) {
+      v = fabsf(x);
+    } else {
+      // lines far from the output see the largest drop: x_j (1 - (1 - j / n)^2)
+      const float p = 1.0f - (float)j / (float)K;
+      v = x * (1.0f - p * p);
+    }
+    out[i] = j < K ? v : 0.0f;
+  }
+}
+
+__global__ __launch_bounds__(256) void k_abs_copy(const float *w, float *out, size_t n) {
+  for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+    out[i] = fabsf(w[i]);
+  }
+}
+
+// four outputs per thread (one Philox call)
+__global__ __launch_bounds__(256) void k_side_combine(float *pre, const float *s_noise, const float *row_sumsq,
+                                                       const float *s_cur, const float *s_ir, SideDev p, int rows, int O,
+                                                       PhiloxKey key, uint32_t call, int round, const int *skip_if_zero) {
+  if (skip_if_zero && *skip_if_zero == 0) return;
+  const int quads = (O + 3) / 4;
+  const size_t total = (size_t)rows * quads;
+  for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+    const int row = (int)(i / quads);
+    const int o0 = (int)(i % quads) * 4;
+    float z[4] = {0.f, 0.f, 0.f, 0.f};
+    const bool noisy = p.w_noise_type != 0 && p.w_noise > 0.0f;
+    if (noisy) philox_normal4((uint32_t)(o0 >> 2), (uint32_t)row, call, RNG_W_NOISE | ((uint32_t)round << 8), key, z);
+    const float x_norm = (noisy && p.w_noise_type == 1) ? sqrtf(row_sumsq[row]) : 0.0f;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int o = o0 + q;
+      if (o >= O) break;
+      const size_t k = (size_t)row * O + o;
+      float v = 0.0f;
+      if (p.ir_drop > 0.0f) {
+        // a_i = sum_j |w_ij| |x_j| n / (Gw / g_max); c_i = a_i (a_i (0.05 a_i - 0.2) + 0.5)
+        const float a = p.a_scale * s_cur[k];
+        const float c = a * (a * (0.05f * a - 0.2f) + 0.5f);
+        v -= c * (p.ir_drop * s_ir[k]);
+      }
+      if (noisy) {
+        if (p.w_noise_type == 1) v += (p.w_noise * x_norm) * z[q];
+        else v += p.w_noise * sqrtf(s_noise[k]) * z[q];
+      }
+      pre[k] = v;
+    }
+  }
+}
+
+} // namespace
+
+void launch_side_rows(const float *xq, float *out, int rows, int k_pad, int K, int mode, const int *skip_if_zero,
+                      hipStream_t s) {
+  const size_t total = (size_t)rows * k_pad;
+  hipLaunchKernelGGL(k_side_rows, dim3(grid_for(total)), dim3(256), 0, s, xq, out, total, k_pad, K, mode, skip_if_zero);
+}
+
+void launch_abs_copy(const float *w, float *out, size_t n, hipStream_t s) {
+  hipLaunchKernelGGL(k_abs_copy, dim3(grid_for(n)), dim3(256), 0, s, w, out, n);
+}
+
+void launch_side_combine(float *pre, const float *s_noise, const float *row_sumsq, const float *s_cur, const float *s_ir,
+                         const SideDev &p, int rows, int O, PhiloxKey key, uint32_t call, int round,
+                         const int *skip_if_zero, hipStream_t s) {
+  const size_t total = (size_t)rows * ((O + 3) / 4);
+  hipLaunchKernelGGL(k_side_combine, dim3(grid_for(total)), dim3(256), 0, s, pre, s_noise, row_sumsq, s_cur, s_ir, p,
+                     rows, O, key, call, round, skip_if_zero);
+}
+
+} // namespace rpu_amd

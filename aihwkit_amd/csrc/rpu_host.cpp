@@ -52,11 +52,8 @@ void IOPar::initialize(bool backward) {
   if (p.mv_type != RPU_MV_ONE_PASS) {
     throw RpuError("AnalogMVType not implemented on this path (only Ideal and OnePass).");
   }
-  if (p.w_noise_type != 0) {
-    throw RpuError("Output weight noise (w_noise_type) is not implemented on this path.");
-  }
-  if (p.ir_drop > 0.0f) {
-    throw RpuError("IR drop is not implemented on this path.");
+  if (p.w_noise_type < 0 || p.w_noise_type > 2) {
+    throw RpuError("Output noise type not implemented");
   }
   if (p.out_noise_std > 0.0f) {
     throw RpuError("out_noise_std is not implemented on this path.");
@@ -403,6 +400,7 @@ void fill_default_config(rpu_tile_config *cfg, int device_kind) {
   io.nm_thres = 0.0f;
   io.nm_assumed_wmax = 0.6f;
   io.max_bm_res = 0.25f;
+  io.ir_drop_g_ratio = 5.7143e5f;
   cfg->f_io = io;
   cfg->b_io = io;
 

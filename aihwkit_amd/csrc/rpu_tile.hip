@@ -185,6 +185,9 @@ struct Tile {
   // pulse counters [2][size]
   DevBuf<float> d_fbw, s_rowstat;
   bool fb_during_test = false;
+  // analog non-idealities before the ADC: the addend per output, up to three side contractions, the transformed
+  // input rows, |W| and the squared row norms
+  DevBuf<float> n_pre, n_s1, n_s2, n_s3, n_rows, n_absw, n_sumsq;
   DevBuf<float> dr_prev, dr_w0, dr_t, d_nu;
   float drift_t = 0.0f;
   bool nu_valid = false;
@@ -253,6 +256,8 @@ struct Tile {
     d_decay.release(); d_diff.release(); d_rbias.release(); s_clip.release();
     state_params_valid = false;
     delta_w = nullptr;
+    n_pre.release(); n_s1.release(); n_s2.release(); n_s3.release(); n_rows.release(); n_absw.release();
+    n_sumsq.release();
     d_fbw.release(); s_rowstat.release(); dr_prev.release(); dr_w0.release(); dr_t.release(); d_nu.release();
     d_cnt.release();
     fb_during_test = false;
@@ -387,10 +392,69 @@ struct Tile {
     return a;
   }
 
+  // whether a pass with these IO parameters has non-idealities that add to the sums before the ADC
+  static bool has_pre_adc_terms(const IOPar &io) {
+    return !io.perfect && ((io.p.w_noise_type != 0 && io.p.w_noise > 0.0f) || io.p.ir_drop > 0.0f);
+  }
+
+  // The addend of every output of round a.round from the quantized inputs of that round: weight noise and IR drop
+  // (ForwardBackwardPassIOManaged::applyNonIdealities, rpu_forward_backward_pass.cpp:535-560).  The extra
+  // contractions run on the round kernel without its ADC stage; rounds that list no sample do nothing.
+  void pre_adc_terms(MvmArgs &a, const IOPar &io, hipStream_t s) {
+    const int B = a.m_batch, r = a.round;
+    const size_t out_n = (size_t)B * a.O, row_n = (size_t)B * a.k_pad;
+    const int *skip = r > 0 ? a.st.count + r : nullptr;
+    const float *xq = a.xq[r & 1];
+    const bool noisy = io.p.w_noise_type != 0 && io.p.w_noise > 0.0f;
+    const bool ir = io.p.ir_drop > 0.0f;
+    const bool need_abs = ir || (noisy && io.p.w_noise_type == 2);
+    n_pre.ensure(out_n);
+    n_rows.ensure(row_n);
+    if (need_abs && r == 0) {
+      n_absw.ensure(size());
+      launch_abs_copy(a.w, n_absw.p, size(), s);
+    }
+    const auto contract = [&](const float *w, int mode, float *dst) {
+      launch_side_rows(xq, n_rows.p, B, a.k_pad, a.K, mode, skip, s);
+      MvmArgs g{};
+      g.w = w; g.x_size = X; g.d_size = D; g.m_batch = B; g.K = a.K; g.O = a.O; g.k_pad = a.k_pad;
+      g.transposed = a.transposed;
+      g.xq[0] = n_rows.p; g.xq[1] = nullptr;
+      g.out = dst; g.out_sb = a.O; g.out_so = 1;
+      g.io = a.io; g.io.perfect = 1;
+      g.alpha = 1.0f; g.beta = 0.0f; g.round = 0;
+      g.key = a.key; g.call = a.call;
+      g.small_tiles_only = 1;
+      g.skip_if_zero = skip;
+      launch_mvm_round(g, s);
+    };
+    if (noisy && io.p.w_noise_type == 1) {
+      n_sumsq.ensure((size_t)B);
+      launch_row_stat(xq, a.k_pad, B, a.K, 1, n_sumsq.p, s);
+    } else if (noisy) {
+      n_s1.ensure(out_n);
+      contract(n_absw.p, 0, n_s1.p);
+    }
+    if (ir) {
+      n_s2.ensure(out_n); n_s3.ensure(out_n);
+      contract(n_absw.p, 1, n_s2.p);
+      contract(a.w, 2, n_s3.p);
+    }
+    SideDev p{};
+    p.w_noise_type = noisy ? io.p.w_noise_type : 0;
+    p.w_noise = io.p.w_noise; p.ir_drop = ir ? io.p.ir_drop : 0.0f;
+    p.a_scale = (float)a.K / io.p.ir_drop_g_ratio;
+    launch_side_combine(n_pre.p, n_s1.p, n_sumsq.p, n_s2.p, n_s3.p, p, B, a.O, a.key, a.call, r, skip, s);
+    a.pre_add = n_pre.p;
+    prof_mark(s, "pre_adc_terms");
+  }
+
   void mvm(const float *in, float *out, int B, bool bias, bool in_trans, bool out_trans, bool transposed, hipStream_t s,
            const float *w_other = nullptr, const IOPar *io_other = nullptr, bool is_test = false) {
     const IOPar &io = io_other ? *io_other : (transposed ? bio : fio);
-    MvmArgs a = mvm_args(B, transposed, w_other ? w_other : mvm_weights(is_test), io);
+    const bool side = has_pre_adc_terms(io);
+    MvmArgs a = mvm_args(B, transposed, w_other ? w_other : mvm_weights(is_test), io, side ? 0 : -1);
+    a.small_tiles_only = side ? 1 : 0;
 
     // the x side carries the optional bias column: input of forward, output of backward
     float *final_out = out;
@@ -427,6 +491,7 @@ struct Tile {
       // last workgroup to finish a sample tile sets up the next round for that tile
       for (int r = 0; r < a.max_rounds; ++r) {
         a.round = r;
+        if (side) pre_adc_terms(a, io, s);
         launch_mvm_round(a, s);
         prof_mark(s, "mvm_round");
       }
@@ -822,7 +887,7 @@ struct Tile {
   void forward_indexed(const float *x, float *d, int n_images, long image_size, bool is_test, hipStream_t s) {
     if (idx_patches <= 0) throw RpuError("The index matrix has not been set (set_matrix_indices).");
     if (n_images <= 0) throw RpuError("n_images must be positive.");
-    if (D <= 32 && (long)n_images * idx_patches < (1L << 31)) {
+    if (D <= 32 && (long)n_images * idx_patches < (1L << 31) && !has_pre_adc_terms(fio)) {
       // narrow tile: unfold, contraction and bound management fused in one kernel, nothing materialized
       const int B = n_images * idx_patches;
       s_rounds.ensure((size_t)B); // the only per-patch state that leaves the kernel: rounds run (get_bm_rounds)
@@ -1471,6 +1536,9 @@ static int group_mvm(rpu_group_t *group, const float *const *x_dev, const long *
       Tile &t = group->tiles[i]->t;
       std::lock_guard<std::mutex> lock(t.mutex);
       t.check_compute(m_batch, x_dev[i], y_dev[i]);
+      if (Tile::has_pre_adc_terms(transposed ? t.bio : t.fio)) {
+        throw RpuError("Output-referred weight noise and IR drop are not provided for a group: call the tiles one by one.");
+      }
       const int in_size = transposed ? t.D : t.X, out_size = transposed ? t.X : t.D;
       const bool big = use_big && out_size >= 128;
       MvmArgs a = t.mvm_args(m_batch, transposed, t.mvm_weights(is_test), transposed ? t.bio : t.fio, big ? 1 : 0);

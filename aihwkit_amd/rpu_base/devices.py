@@ -217,7 +217,8 @@ class AnalogTileInputOutputParameter(_Struct):
         for name in ("inp_bound", "inp_res", "inp_noise", "inp_asymmetry", "out_bound", "out_res",
                      "out_noise", "out_asymmetry", "out_scale", "nm_thres", "nm_assumed_wmax",
                      "max_bm_res", "w_noise", "ir_drop", "out_noise_std", "out_nonlinearity",
-                     "out_nonlinearity_std", "v_offset_std", "r_series", "w_read_asymmetry_dtod"):
+                     "out_nonlinearity_std", "v_offset_std", "r_series", "w_read_asymmetry_dtod",
+                     "ir_drop_g_ratio"):
             setattr(p, name, float(getattr(self, name)))
         p.w_noise_type = int(self.w_noise_type)
         return p

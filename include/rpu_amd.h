@@ -111,16 +111,18 @@ typedef struct rpu_io_params {
   float nm_thres;                 /* 0 */
   float nm_assumed_wmax;          /* 0.6 */
   float max_bm_res;               /* 0.25 */
-  /* not provided (must stay inactive): */
-  int32_t w_noise_type;           /* 0 = None */
+  /* output-referred weight noise (R/rpu_forward_backward_pass.cpp:325-385) and IR drop (:387-433) */
+  int32_t w_noise_type;           /* 0 = None, 1 = AdditiveConstant, 2 = PCMRead */
   float w_noise;                  /* ignored while w_noise_type == 0 */
   float ir_drop;                  /* 0 */
+  /* not provided (must stay inactive): */
   float out_noise_std;            /* 0 */
   float out_nonlinearity;         /* 0 */
   float out_nonlinearity_std;     /* 0 */
   float v_offset_std;             /* 0 */
   float r_series;                 /* 0 */
   float w_read_asymmetry_dtod;    /* 0 */
+  float ir_drop_g_ratio;          /* 5.7143e5: wire conductance over g_max (ir_drop_Gw_div_gmax) */
 } rpu_io_params;
 
 /* Replaces PulsedUpdateMetaParameter<float> (R/rpu_pulsed_meta_parameter.h:248-323) as bound by

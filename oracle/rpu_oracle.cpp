@@ -169,9 +169,12 @@ bool init_io(OrcIO &io, bool backward) {
   if (p.out_bound <= 0.0f) p.out_bound = std::numeric_limits<float>::infinity();
   if (p.inp_bound <= 0.0f) p.inp_bound = std::numeric_limits<float>::infinity();
   if (backward) p.bound_management = RPU_BM_NONE;
-  if (p.w_noise_type != 0 || p.ir_drop > 0.f || p.out_noise_std > 0.f || p.out_nonlinearity > 0.f ||
-      p.v_offset_std > 0.f || p.r_series > 0.f) {
-    g_err = "oracle: w_noise / ir_drop / out_noise_std / out_nonlinearity / v_offset / r_series not restated";
+  if (p.w_noise_type < 0 || p.w_noise_type > 2) {
+    g_err = "Output noise type not implemented";
+    return false;
+  }
+  if (p.out_noise_std > 0.f || p.out_nonlinearity > 0.f || p.v_offset_std > 0.f || p.r_series > 0.f) {
+    g_err = "oracle: out_noise_std / out_nonlinearity / v_offset / r_series not restated";
     return false;
   }
   return true;
@@ -467,12 +470,72 @@ bool finalize_output(OrcTile &t, float *out, int out_size, int out_inc, const rp
   return bound_test_passed;
 }
 
+// R/rpu_forward_backward_pass.cpp:508-530 computeTotalCurrent and :387-433 applyIrDrop
+void apply_ir_drop(OrcTile &t, float *out, int out_size, int out_inc, const float *in, int in_size,
+                   const rpu_io_params &io, bool transposed) {
+  if (io.ir_drop <= 0.0f) return;
+  const int X = t.X;
+  const float *w = t.w.data();
+  std::vector<float> current((size_t)out_size), c_values((size_t)out_size), pos_in((size_t)in_size);
+  for (int i = 0; i < out_size; ++i) {
+    float accum = 0.0f;
+    for (int j = 0; j < in_size; ++j) {
+      const float wij = transposed ? w[(size_t)j * X + i] : w[(size_t)i * X + j];
+      accum += std::fabs(wij) * std::fabs(in[j]);
+    }
+    current[i] = accum;
+  }
+  const float a_scale = (float)in_size / io.ir_drop_g_ratio;
+  for (int i = 0; i < out_size; ++i) {
+    const float a = a_scale * current[i];
+    c_values[i] = a * (a * (0.05f * a - 0.2f) + 0.5f);
+  }
+  for (int j = 0; j < in_size; ++j) {
+    const float p = (1.0f - (float)j / (float)in_size);
+    pos_in[j] = in[j] * (1.0f - p * p);
+  }
+  for (int i = 0; i < out_size; ++i) {
+    float accum = 0.0f;
+    for (int j = 0; j < in_size; ++j) {
+      const float wij = transposed ? w[(size_t)j * X + i] : w[(size_t)i * X + j];
+      accum += wij * pos_in[j];
+    }
+    out[(size_t)i * out_inc] -= c_values[i] * (io.ir_drop * accum);
+  }
+}
+
+// R/rpu_forward_backward_pass.cpp:325-385 applyOutputWeightNoise
+void apply_output_weight_noise(OrcTile &t, float *out, int out_size, int out_inc, const float *in, int in_size,
+                               const rpu_io_params &io, bool transposed) {
+  if (io.w_noise_type == 0 || !(io.w_noise > 0.0f)) return;
+  const int X = t.X;
+  const float *w = t.w.data();
+  if (io.w_noise_type == 1) { // AdditiveConstant
+    float sq = 0.0f;
+    for (int j = 0; j < in_size; ++j) sq += in[j] * in[j];
+    const float w_std = io.w_noise * std::sqrt(sq);
+    for (int i = 0; i < out_size; ++i) out[(size_t)i * out_inc] += w_std * t.rng.gauss();
+    return;
+  }
+  for (int i = 0; i < out_size; ++i) { // PCMRead
+    float accum = 0.0f;
+    for (int j = 0; j < in_size; ++j) {
+      const float wij = transposed ? w[(size_t)j * X + i] : w[(size_t)i * X + j];
+      accum += std::fabs(wij) * (in[j] * in[j]);
+    }
+    out[(size_t)i * out_inc] += io.w_noise * std::sqrt(accum) * t.rng.gauss();
+  }
+}
+
 // R/rpu_forward_backward_pass.cpp:800-829 computeAnalogMV, OnePass
 bool analog_mv(OrcTile &t, const float *in, int in_size, int in_inc, float *out, int out_size,
                int out_inc, float scale, bool scaling, const rpu_io_params &io, bool transposed) {
   t.in_buf.resize(in_size);
   prepare_input(t, t.in_buf.data(), in, in_size, in_inc, scale, scaling, io);
   gemv(t, t.in_buf.data(), out, out_inc, transposed);
+  // applyNonIdealities (:535-560): IR drop, then the weight-dependent noise
+  apply_ir_drop(t, out, out_size, out_inc, t.in_buf.data(), in_size, io, transposed);
+  apply_output_weight_noise(t, out, out_size, out_inc, t.in_buf.data(), in_size, io, transposed);
   return finalize_output(t, out, out_size, out_inc, io);
 }
 

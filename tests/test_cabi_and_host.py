@@ -110,9 +110,10 @@ def test_unsupported_parameters_fail_loudly():
     with pytest.raises(RuntimeError, match="expects bound==1"):
         make_meta(io_params(inp_bound=2.0)).create_array(4, 4, dev)
     with pytest.raises(RuntimeError, match="not implemented"):
-        make_meta(io_params(ir_drop=1.0)).create_array(4, 4, dev)
+        make_meta(io_params(out_noise_std=0.1)).create_array(4, 4, dev)
     with pytest.raises(RuntimeError, match="not implemented"):
-        make_meta(io_params(w_noise_type=dv.WeightNoiseType.PCMRead, w_noise=0.1)).create_array(4, 4, dev)
+        make_meta(io_params(v_offset_std=0.1)).create_array(4, 4, dev)
+    make_meta(io_params(ir_drop=1.0, w_noise_type=dv.WeightNoiseType.PCMRead, w_noise=0.1)).create_array(4, 4, dev)
     with pytest.raises(RuntimeError, match="desired_bl"):
         make_meta(desired_bl=255).create_array(4, 4, dev)
     with pytest.raises(RuntimeError, match="not supported"):

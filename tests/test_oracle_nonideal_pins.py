@@ -1,0 +1,90 @@
+"""Pins of the IR-drop and output-referred weight-noise restatement in oracle/rpu_oracle.cpp: closed forms on tiles
+whose sums can be written down, the position dependence of the drop, and the variance laws of the two noise types."""
+import numpy as np
+
+from aihwkit_amd.rpu_base import devices as dv
+from helpers import constant_step, io_params, make_meta
+from oracle_lib import OracleTile
+
+F = np.float32
+
+
+def oracle_tile(x_size, d_size, w, **io):
+    # no quantization, no clipping, no scaling: the inputs reach the array as they are
+    base = dict(out_noise=0.0, inp_noise=0.0, inp_res=-1.0, out_res=-1.0, out_bound=1e6,
+                noise_management=dv.NoiseManagementType.NONE, bound_management=dv.BoundManagementType.NONE)
+    base.update(io)
+    meta = make_meta(io_params(**base), io_params(**base))
+    dev = constant_step(w_max=10.0, w_min=-10.0, w_max_dtod=0.0, w_min_dtod=0.0, construction_seed=1)
+    tile = OracleTile(x_size, d_size, meta._config(dev))
+    tile.set_weights(np.asarray(w, dtype=F))
+    return tile
+
+
+def drop_factor(a):
+    return a * (a * (0.05 * a - 0.2) + 0.5)
+
+
+def test_ir_drop_closed_form_on_a_constant_tile():
+    for n, d, w, v, ratio, scale in ((8, 3, 0.5, 0.7, 40.0, 1.0), (20, 2, -0.3, 0.9, 150.0, 2.5), (5, 4, 0.4, -1.0, 10.0, 0.5)):
+        tile = oracle_tile(n, d, np.full((d, n), w), ir_drop=scale, ir_drop_g_ratio=ratio)
+        y = tile.forward(np.full((1, n), v, dtype=F))[0]
+        a = n / ratio * (n * abs(w) * abs(v))                    # total current, scaled by n / (Gw / g_max)
+        s = sum(1.0 - (1.0 - j / n) ** 2 for j in range(n))      # sum of the position weights
+        want = n * w * v - scale * drop_factor(a) * w * v * s
+        np.testing.assert_allclose(y, np.full(d, want), rtol=2e-6)
+        assert abs(want - n * w * v) > 1e-3 * abs(n * w * v)     # the drop is visible in this setting
+
+
+def test_ir_drop_depends_on_the_position_of_the_input_line():
+    n, ratio = 10, 8.0
+    w = np.linspace(0.2, 0.9, 3 * n).reshape(3, n).astype(F) * np.array([[1], [-1], [1]], dtype=F)
+    tile = oracle_tile(n, 3, w, ir_drop=1.0, ir_drop_g_ratio=ratio)
+    for j in (0, 1, 5, 9):
+        x = np.zeros((1, n), dtype=F)
+        x[0, j] = -0.8
+        y = tile.forward(x)[0].astype(np.float64)
+        a = n / ratio * np.abs(w[:, j].astype(np.float64)) * 0.8
+        want = w[:, j] * -0.8 * (1.0 - drop_factor(a) * (1.0 - (1.0 - j / n) ** 2))
+        np.testing.assert_allclose(y, want, rtol=3e-6)
+    x = np.zeros((1, n), dtype=F)
+    x[0, 0] = 1.0                                                # the line next to the output sees no drop at all
+    np.testing.assert_array_equal(tile.forward(x)[0], w[:, 0])
+    # backward: the same law on the transposed matrix (n = d_size input lines)
+    dvec = np.zeros((1, 3), dtype=F)
+    dvec[0, 2] = 0.5
+    got = tile.backward(dvec)[0].astype(np.float64)
+    a = 3 / ratio * np.abs(w[2].astype(np.float64)) * 0.5
+    want = w[2] * 0.5 * (1.0 - drop_factor(a) * (1.0 - (1.0 - 2 / 3) ** 2))
+    np.testing.assert_allclose(got, want, rtol=3e-6)
+
+
+def test_weight_noise_variance_laws():
+    rng = np.random.default_rng(0)
+    n, d, m = 16, 400, 50
+    x = rng.uniform(-1, 1, (m, n)).astype(F)
+    # additive constant: sigma = w_noise |x|_2 for every output, whatever the weights
+    tile = oracle_tile(n, d, np.zeros((d, n)), w_noise=0.05, w_noise_type=dv.WeightNoiseType.AdditiveConstant)
+    tile.set_seed(3)
+    y = tile.forward(x).astype(np.float64)
+    z = y / (0.05 * np.linalg.norm(x.astype(np.float64), axis=1))[:, None]
+    assert abs(z.mean()) < 4 / np.sqrt(z.size) and abs(z.std() - 1) < 4 / np.sqrt(2 * z.size)
+    assert abs(np.corrcoef(z[:, :-1].ravel(), z[:, 1:].ravel())[0, 1]) < 4 / np.sqrt(z.size)
+    # PCM read noise: sigma_i^2 = w_noise^2 sum_j |w_ij| x_j^2
+    w = rng.uniform(-0.6, 0.6, (d, n)).astype(F)
+    w[:50] *= 0.01                                               # rows of small conductance are quiet
+    tile = oracle_tile(n, d, w, w_noise=0.1, w_noise_type=dv.WeightNoiseType.PCMRead)
+    tile.set_seed(4)
+    y = tile.forward(x).astype(np.float64)
+    clean = x.astype(np.float64) @ w.T.astype(np.float64)
+    sigma = 0.1 * np.sqrt((x.astype(np.float64) ** 2) @ np.abs(w.T.astype(np.float64)))
+    z = (y - clean) / sigma
+    assert abs(z.mean()) < 4 / np.sqrt(z.size) and abs(z.std() - 1) < 4 / np.sqrt(2 * z.size)
+    assert abs(z[:, :50].std() - 1) < 4 / np.sqrt(2 * 50 * m)    # the law holds on the quiet rows as well
+    assert (y - clean)[:, :50].std() < 0.2 * (y - clean)[:, 50:].std()
+    # backward uses the transposed matrix: sigma_j^2 = w_noise^2 sum_i |w_ij| d_i^2
+    dm = rng.uniform(-1, 1, (m, d)).astype(F)
+    got = tile.backward(dm).astype(np.float64)
+    sigma = 0.1 * np.sqrt((dm.astype(np.float64) ** 2) @ np.abs(w.astype(np.float64)))
+    z = (got - dm.astype(np.float64) @ w.astype(np.float64)) / sigma
+    assert abs(z.mean()) < 4 / np.sqrt(z.size) and abs(z.std() - 1) < 4 / np.sqrt(2 * z.size)
