@@ -1333,7 +1333,9 @@ __global__ __launch_bounds__(256, 3) void k_conv_forward(MvmArgs a, ConvArgs c) 
     floatx16 acc;
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
-    if (fin != 0.0f || io.perfect) {
+    // wave-uniform: the lanes also carry the weight rows of the contraction, whatever their own patch holds (a zero
+    // patch has scale 0 and contributes zeros)
+    if (__any(fin != 0.0f) || io.perfect) {
       for (int st = 0; st < steps; ++st) {
         const int k0 = st * 32 + h * 16;
         float xd[16], wd[16];
@@ -1496,7 +1498,9 @@ __global__ __launch_bounds__(256) void k_conv_forward_split(MvmArgs a, ConvArgs 
     floatx16 acc;
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
-    if (fin != 0.0f || io.perfect) {
+    // wave-uniform: the lanes also carry the weight rows of the contraction, whatever their own patch holds (a zero
+    // patch has scale 0 and contributes zeros)
+    if (__any(fin != 0.0f) || io.perfect) {
       for (int st = wave; st < steps; st += WAVES) {
         const int k0 = st * 32 + h * 16;
         float xd[16], wd[16];

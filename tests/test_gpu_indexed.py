@@ -117,3 +117,32 @@ def test_fused_convolution_forward_is_bit_exact_with_bound_management_rounds(gpu
     rounds = orc_tile.bm_rounds(n * patches)
     assert rounds.max() > 1 and rounds.min() >= 1
     assert np.array_equal(gpu.get_bm_rounds(n * patches).numpy(), rounds)
+
+
+@pytest.mark.parametrize("c_in,kernel", [(3, 3), (16, 5)])       # the per-wave kernel and the one that splits long rows
+def test_zero_patches_beside_others_without_a_bias_column(gpu_device, c_in, kernel):
+    """Without a bias column a patch of zeros short-cuts to zero outputs (its noise-management scale is zero); the
+    other patches of the same 32-patch tile must not notice."""
+    rng = np.random.default_rng(8)
+    c_out, height, width, n = 20, 9, 10, 3
+    indices, patches = conv_indices((c_in, height, width), (kernel, kernel), (1, 1), (0, 0), (1, 1), False)
+    x_size = c_in * kernel * kernel
+    f_io = noise_free_io(inp_res=1 / 128.0, out_res=1 / 512.0, out_bound=4.0, noise_management=dv.NoiseManagementType.AbsMax,
+                         bound_management=dv.BoundManagementType.Iterative)
+    meta = make_meta(f_io, noise_free_io())
+    dev = constant_step(w_max_dtod=0.0, w_min_dtod=0.0, w_max=1.0, w_min=-1.0, construction_seed=3)
+    host, orc_tile, _ = build_pair(meta, dev, x_size, c_out, gpu=False)
+    w = (rng.integers(-60, 61, (c_out, x_size)) / 64.0).astype(np.float32)
+    host.set_weights(torch.from_numpy(w))
+    orc_tile.set_weights(w)
+    gpu = tiles.CudaAnalogTile(host)
+    gpu.set_matrix_indices(indices)
+    x = (rng.integers(-64, 65, (n, c_in, height, width)) / 64.0).astype(np.float32)
+    x[0, :, :, : width // 2 + 1] = 0.0                              # zero and non-zero patches alternate along a row
+    x[2] = 0.0
+    y = gpu.forward_indexed(cuda(x), torch.empty(n, c_out, 1, patches).cuda()).cpu().numpy().reshape(n, c_out, patches)
+    want = IndexedOracle(orc_tile, indices.numpy(), patches).forward(x)
+    rounds = orc_tile.bm_rounds(n * patches)
+    assert (rounds == 0).sum() >= patches and (rounds[:patches] == 0).any() and (rounds[:patches] > 0).any()
+    assert np.array_equal(y, want)
+    assert np.array_equal(gpu.get_bm_rounds(n * patches).numpy(), rounds)
