@@ -160,3 +160,215 @@ def test_random_convolution_forward_cases_are_bit_exact(gpu_device):
         if not ok:
             failures.append(desc)
     assert not failures, failures[:3]
+
+
+SIZES = [1, 2, 3, 31, 32, 33, 63, 64, 65, 100, 255, 256, 257, 300]
+
+def one_implicit(seed):
+    rng = np.random.default_rng(seed)
+    x_size = int(rng.choice(SIZES))
+    d_size = int(rng.choice([1, 2, 3, 5, 16, 17, 33, 64, 65, 96, 128, 129]))
+    batch = int(rng.choice([1, 2, 7, 31, 32, 33, 64, 65, 100, 129]))
+    bias = bool(rng.integers(2)) and x_size > 1
+    x_trans, d_trans = bool(rng.integers(2)), bool(rng.integers(2))
+    bl = int(rng.choice([1, 5, 31]))
+    um = bool(rng.integers(2))
+    kind = int(rng.integers(3))
+    kw = dict(dw_min=0.002, dw_min_std=0.0, construction_seed=int(rng.integers(1, 99)), enforce_consistency=True)
+    if kind == 0:
+        dev = constant_step(**kw)
+    elif kind == 1:
+        dev = soft_bounds(**kw)
+    else:
+        dev = dv.LinearStepResistiveDeviceParameter()
+        for k, v in dict(gamma_up=0.4, gamma_down=0.2, gamma_up_dtod=0.05, gamma_down_dtod=0.05,
+                         mult_noise=bool(rng.integers(2)), **kw).items():
+            setattr(dev, k, v)
+    meta = make_meta(desired_bl=bl, pulse_type=dv.PulseType.DeterministicImplicit, update_management=um,
+                     update_bl_management=um,
+                     x_res_implicit=float(rng.choice([0.0, 1 / 20.0])), d_res_implicit=float(rng.choice([0.0, 1 / 30.0])))
+    host, orc, _ = build_pair(meta, dev, x_size, d_size, gpu=False)
+    w = rng.uniform(-0.4, 0.4, (d_size, x_size)).astype(np.float32)
+    host.set_weights(torch.from_numpy(w))
+    orc.set_weights(host.get_weights().numpy())
+    gpu = tiles.CudaAnalogTile(host)
+    lr = float(rng.choice([0.02, 0.1, -0.05]))
+    gpu.set_learning_rate(lr)
+    orc.set_learning_rate(lr)
+    xs = x_size - int(bias)
+    x = rng.uniform(-1, 1, (xs, batch) if x_trans else (batch, xs)).astype(np.float32)
+    d = (0.3 * rng.standard_normal((d_size, batch) if d_trans else (batch, d_size))).astype(np.float32)
+    gpu.update(cuda(x), cuda(d), bias, x_trans, d_trans, False)
+    orc.update(x, d, bias, x_trans, d_trans)
+    diff = np.abs(gpu.get_weights().numpy() - orc.get_weights()).max()
+    return diff <= 2e-5, dict(seed=seed, X=x_size, D=d_size, B=batch, bias=bias, xt=x_trans, dt=d_trans, bl=bl, um=um,
+                              kind=kind, lr=lr, diff=float(diff))
+
+def one_fp(seed):
+    rng = np.random.default_rng(seed)
+    x_size = int(rng.choice(SIZES))
+    d_size = int(rng.choice(SIZES))
+    batch = int(rng.choice([1, 2, 7, 31, 33, 64, 100, 257, 1025, 2049]))
+    bias = bool(rng.integers(2)) and x_size > 1
+    x_trans, d_trans = bool(rng.integers(2)), bool(rng.integers(2))
+    meta = dv.FloatingPointTileParameter()
+    host = meta.create_array(x_size, d_size)
+    w = (rng.integers(-38, 39, (d_size, x_size)) / 64.0).astype(np.float32)
+    host.set_weights(torch.from_numpy(w))
+    gpu = tiles.CudaFloatingPointTile(host)
+    xs = x_size - int(bias)
+    x = (rng.integers(-64, 65, (batch, xs)) / 64.0).astype(np.float32)
+    d = (rng.integers(-64, 65, (batch, d_size)) / 64.0).astype(np.float32)
+    xb = np.concatenate([x, np.ones((batch, 1), np.float32)], 1) if bias else x
+    y = gpu.forward(cuda(x.T if x_trans else x), bias, x_trans, d_trans).cpu().numpy()
+    y = y.T if d_trans else y
+    ok = np.array_equal(y, xb @ w.T)
+    g = gpu.backward(cuda(d.T if d_trans else d), bias, d_trans, x_trans).cpu().numpy()
+    g = g.T if x_trans else g
+    want_g = d @ w
+    ok2 = np.array_equal(g, want_g[:, :xs])
+    gpu.set_learning_rate(0.25)
+    gpu.update(cuda(x.T if x_trans else x), cuda(d.T if d_trans else d), bias, x_trans, d_trans)
+    ok3 = np.array_equal(gpu.get_weights().numpy(), (w - 0.25 * (d.T @ xb)).astype(np.float32))
+    return ok and ok2 and ok3, dict(seed=seed, X=x_size, D=d_size, B=batch, bias=bias, xt=x_trans, dt=d_trans, f=ok,
+                                    b=ok2, u=ok3)
+
+
+def test_random_implicit_update_cases_follow_the_oracle(gpu_device):
+    """Deterministic implicit pulses over layouts, bias column, three devices, update management, learning-rate sign."""
+    failures = [desc for ok, desc in (one_implicit(seed) for seed in range(20000, 20150)) if not ok]
+    assert not failures, failures[:3]
+
+
+def test_random_floating_point_tile_cases_are_exact(gpu_device):
+    """Perfect forward / backward and the outer-product update on binary grids: exact against numpy."""
+    failures = [desc for ok, desc in (one_fp(seed) for seed in range(30000, 30150)) if not ok]
+    assert not failures, failures[:3]
+
+
+def one_group(seed):
+    rng = np.random.default_rng(seed)
+    n_tiles = int(rng.choice([1, 2, 3, 5, 9, 17]))
+    batch = int(rng.choice([1, 7, 33, 96, 257, 1024, 1100, 2048]))
+    strided = bool(rng.integers(2))
+    grouped, oracles, xs, ds, shapes = [], [], [], [], []
+    budget = 40_000_000
+    for k in range(n_tiles):
+        x_size = int(rng.choice([1, 3, 31, 33, 64, 70, 96, 129, 130, 257]))
+        d_size = int(rng.choice([1, 5, 32, 40, 127, 128, 129, 256, 300, 512]))
+        if x_size * d_size * batch > budget // n_tiles:
+            d_size = max(1, (budget // n_tiles) // (x_size * batch))
+        nm = [NM.NONE, NM.AbsMax, NM.Max][rng.integers(3)]
+        bm = [BM.NONE, BM.Iterative][rng.integers(2)]
+        perfect = rng.integers(8) == 0
+        f_io = noise_free_io(is_perfect=True) if perfect else noise_free_io(
+            inp_res=1 / 128.0, out_res=1 / 512.0, noise_management=nm, bound_management=bm,
+            out_bound=float(rng.choice([2.0, 12.0])))
+        b_io = noise_free_io(inp_res=1 / 128.0, out_res=1 / 512.0, noise_management=nm)
+        dev = constant_step(w_max_dtod=0.0, w_min_dtod=0.0, w_max=1.0, w_min=-1.0, construction_seed=k + 1)
+        host, orc, _ = build_pair(make_meta(f_io, b_io), dev, x_size, d_size, gpu=False)
+        w = (rng.integers(-60, 61, (d_size, x_size)) / 64.0).astype(np.float32)
+        host.set_weights(torch.from_numpy(w))
+        orc.set_weights(w)
+        grouped.append(tiles.CudaAnalogTile(host))
+        oracles.append(orc)
+        shapes.append((x_size, d_size))
+        xs.append((rng.integers(-64, 65, (batch, x_size)) / 64.0).astype(np.float32))
+        ds.append((rng.integers(-64, 65, (batch, d_size)) / 64.0).astype(np.float32))
+    group = tiles.TileGroup(grouped)
+    desc = dict(seed=seed, n=n_tiles, B=batch, strided=strided, shapes=shapes)
+    if strided:
+        all_x = torch.cat([cuda(x) for x in xs], dim=1)
+        x_in, i0 = [], 0
+        for x_size, _ in shapes:
+            x_in.append(all_x[:, i0:i0 + x_size])
+            i0 += x_size
+        all_y = torch.full((batch, sum(d for _, d in shapes)), 7.0, device="cuda")
+        outs, i0 = [], 0
+        for _, d_size in shapes:
+            outs.append(all_y[:, i0:i0 + d_size])
+            i0 += d_size
+        got = group.forward(x_in, outs=outs)
+    else:
+        got = group.forward([cuda(x) for x in xs])
+    ok = True
+    for k, (y, orc, x) in enumerate(zip(got, oracles, xs)):
+        if not np.array_equal(y.cpu().numpy(), orc.forward(x)):
+            ok = False
+            desc.setdefault("fwd_bad", []).append(k)
+    gb = group.backward([cuda(d) for d in ds])
+    for k, (g, orc, d) in enumerate(zip(gb, oracles, ds)):
+        if not np.array_equal(g.cpu().numpy(), orc.backward(d)):
+            ok = False
+            desc.setdefault("bwd_bad", []).append(k)
+    return ok, desc
+
+
+def test_random_groups_are_bit_exact(gpu_device):
+    """Groups of 1 to 17 tiles of mixed shapes and IO modes (one in eight with a perfect forward), batches on both sides
+    of the large-tile threshold, dense tensors or column slices of one matrix: every tile's outputs and input
+    gradients equal the oracle's in the exact-arithmetic setting."""
+    failures = [desc for ok, desc in (one_group(seed) for seed in range(40000, 40100)) if not ok]
+    assert not failures, failures[:3]
+
+
+def one_transfer(seed):
+    from helpers import build_transfer_pair, device_weights, transfer_param
+
+    rng = np.random.default_rng(seed)
+    x_size = int(rng.choice([2, 5, 31, 33, 37, 64, 65, 130]))
+    d_size = int(rng.choice([1, 3, 21, 32, 33, 64, 70]))
+    batch = int(rng.choice([1, 3, 8, 33]))
+    n_devices = int(rng.choice([2, 2, 3, 4]))
+    soft = bool(rng.integers(2))
+    kw = dict(transfer_every=float(rng.choice([1.0, 2.0, 3.0, 5.0])), n_reads_per_transfer=int(rng.choice([1, 2, 3, 40])),
+              units_in_mbatch=bool(rng.integers(2)), transfer_columns=bool(rng.integers(2)))
+    if rng.integers(2):
+        kw["gamma"] = float(rng.choice([0.0, 0.3]))
+    if rng.integers(2):
+        kw["transfer_lr"] = float(rng.choice([0.5, 1.0, 2.0]))
+    if rng.integers(3) == 0:
+        kw.update(fast_lr=0.02, scale_fast_lr=bool(rng.integers(2)))
+    if rng.integers(3) == 0:
+        kw["scale_transfer_lr"] = bool(rng.integers(2))
+    f_io = noise_free_io(noise_management=NM.AbsMax, bound_management=BM.Iterative)
+    b_io = noise_free_io(noise_management=NM.AbsMax)
+    meta = make_meta(f_io, b_io, pulse_type=dv.PulseType.DeterministicImplicit, desired_bl=31)
+    make = soft_bounds if soft else constant_step
+    devs = [make(dw_min=0.002, dw_min_std=0.0, enforce_consistency=True) for _ in range(n_devices)]
+    devs[0].dw_min = 0.004
+    tr = transfer_param(devs, construction_seed=int(rng.integers(1, 99)), **kw)
+    tr.transfer_forward = noise_free_io()
+    tr.transfer_update.pulse_type = dv.PulseType.DeterministicImplicit
+    tr.transfer_update.desired_bl = 31
+    host, orc, gpu = build_transfer_pair(meta, tr, x_size, d_size)
+    w = rng.uniform(-0.4, 0.4, (d_size, x_size)).astype(np.float32)
+    gpu.set_weights(torch.from_numpy(w))
+    orc.set_weights(w)
+    gpu.set_learning_rate(0.05)
+    orc.set_learning_rate(0.05)
+    desc = dict(seed=seed, X=x_size, D=d_size, B=batch, n=n_devices, soft=soft, kw=kw)
+    for step in range(5):
+        x = rng.uniform(-1, 1, (batch, x_size)).astype(np.float32)
+        d = (0.5 * rng.standard_normal((batch, d_size))).astype(np.float32)
+        gpu.update(cuda(x), cuda(d), False, False, False, False)
+        orc.update(x, d)
+        for k in range(n_devices):
+            diff = np.abs(device_weights(gpu, k) - orc.device_weights(k)).max()
+            if diff > 2e-5:
+                return False, dict(desc, step=step, device=k, diff=float(diff))
+        diff = np.abs(gpu.get_weights().numpy() - orc.get_weights()).max()
+        if diff > 2e-5:
+            return False, dict(desc, step=step, what="weights", diff=float(diff))
+        count, slices = gpu.get_transfer_state()
+        if count != orc.update_idx or slices[:n_devices] != orc.slice_idx:
+            return False, dict(desc, step=step, what="state", got=(count, slices), want=(orc.update_idx, orc.slice_idx))
+    return True, desc
+
+
+def test_random_transfer_compounds_follow_the_oracle(gpu_device):
+    """Two to four devices, columns or rows, transfer periods in vectors or mini-batches, more reads than columns,
+    learning-rate scalings, visible fast device or fully hidden chain: five update calls each, all device matrices,
+    the reduced weights and the transfer counters against the oracle."""
+    failures = [desc for ok, desc in (one_transfer(seed) for seed in range(50000, 50080)) if not ok]
+    assert not failures, failures[:3]
