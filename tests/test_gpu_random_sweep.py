@@ -8,7 +8,7 @@ import torch
 
 from aihwkit_amd.rpu_base import devices as dv
 from aihwkit_amd.rpu_base import tiles
-from helpers import build_pair, constant_step, make_meta, noise_free_io, soft_bounds
+from helpers import build_pair, constant_step, io_params, make_meta, noise_free_io, soft_bounds
 
 pytestmark = pytest.mark.gpu
 NM, BM = dv.NoiseManagementType, dv.BoundManagementType
@@ -372,3 +372,148 @@ def test_random_transfer_compounds_follow_the_oracle(gpu_device):
     the reduced weights and the transfer counters against the oracle."""
     failures = [desc for ok, desc in (one_transfer(seed) for seed in range(50000, 50080)) if not ok]
     assert not failures, failures[:3]
+
+
+def one_conv_backward_update(seed):
+    from indexed_oracle import IndexedOracle
+    from test_oracle_indexed_pins import conv_indices
+
+    rng = np.random.default_rng(seed)
+    c_in = int(rng.choice([1, 2, 3, 7, 8]))
+    c_out = int(rng.choice([1, 3, 16, 20, 33]))
+    k = int(rng.choice([1, 3, 5]))
+    stride = int(rng.choice([1, 2]))
+    pad = int(rng.choice([0, 1, 2]))
+    height, width = int(rng.integers(5, 13)), int(rng.integers(5, 13))
+    n = int(rng.choice([1, 3, 6]))
+    bias = bool(rng.integers(2))
+    indices, patches = conv_indices((c_in, height, width), (k, k), (stride, stride), (pad, pad), (1, 1), bias)
+    x_size = c_in * k * k + int(bias)
+    b_io = noise_free_io(inp_res=1 / 128.0, out_res=1 / 512.0, noise_management=[NM.NONE, NM.AbsMax][rng.integers(2)])
+    meta = make_meta(noise_free_io(), b_io, pulse_type=dv.PulseType.DeterministicImplicit, desired_bl=31)
+    dev = constant_step(dw_min=0.002, dw_min_std=0.0, construction_seed=4, w_max_dtod=0.0, w_min_dtod=0.0, w_max=1.0,
+                        w_min=-1.0)
+    host, orc_tile, _ = build_pair(meta, dev, x_size, c_out, gpu=False)
+    w = (rng.integers(-38, 39, (c_out, x_size)) / 64.0).astype(np.float32)
+    host.set_weights(torch.from_numpy(w))
+    orc_tile.set_weights(w)
+    gpu = tiles.CudaAnalogTile(host)
+    gpu.set_matrix_indices(indices)
+    orc = IndexedOracle(orc_tile, indices.numpy(), patches)
+    x = (rng.integers(-64, 65, (n, c_in, height, width)) / 64.0).astype(np.float32)
+    grad = (rng.integers(-64, 65, (n, c_out, patches)) / 64.0).astype(np.float32)
+    desc = dict(seed=seed, c_in=c_in, c_out=c_out, k=k, stride=stride, pad=pad, hw=(height, width), n=n, bias=bias,
+                patches=patches)
+    dx = gpu.backward_indexed(cuda(grad.reshape(n, c_out, 1, patches)), torch.full((n, c_in, height, width), 3.0).cuda())
+    want_dx = orc.backward(grad, c_in * height * width)
+    diff = np.abs(dx.cpu().numpy().reshape(n, -1) - want_dx).max()
+    if diff > 1e-5 * max(1.0, np.abs(want_dx).max()):
+        return False, dict(desc, what="backward", diff=float(diff))
+    gpu.set_learning_rate(0.05)
+    orc_tile.set_learning_rate(0.05)
+    gpu.update_indexed(cuda(x), cuda(grad.reshape(n, c_out, 1, patches)))
+    orc.update(x, grad)
+    diff = np.abs(gpu.get_weights().numpy() - orc_tile.get_weights()).max()
+    if diff > 2e-5:
+        return False, dict(desc, what="update", diff=float(diff))
+    return True, desc
+
+
+def test_random_convolution_backward_and_update_cases_follow_the_oracle(gpu_device):
+    """Fold (scatter-add into the image gradient, which is overwritten, not accumulated into) and the pulsed update on
+    the unfolded matrices, over kernel sizes, strides, paddings and the bias row."""
+    failures = [desc for ok, desc in (one_conv_backward_update(seed) for seed in range(60000, 60100)) if not ok]
+    assert not failures, failures[:3]
+
+
+def noise_check(z, desc):
+    n = z.size
+    if n < 400:
+        return True, desc
+    z = z.astype(np.float64)
+    probs = []
+    if abs(z.mean()) > 4.5 / np.sqrt(n):
+        probs.append(("mean", z.mean()))
+    if abs(z.std() - 1) > 4.5 / np.sqrt(2 * n):
+        probs.append(("std", z.std()))
+    if z.shape[1] > 1:
+        c = np.corrcoef(z[:, :-1].ravel(), z[:, 1:].ravel())[0, 1]
+        if abs(c) > 4.5 / np.sqrt(n):
+            probs.append(("corr_out", c))
+    if z.shape[0] > 1:
+        c = np.corrcoef(z[:-1].ravel(), z[1:].ravel())[0, 1]
+        if abs(c) > 4.5 / np.sqrt(n):
+            probs.append(("corr_sample", c))
+    # shared streams show up as repeated values
+    r = np.round(z.ravel() * 2 ** 12).astype(np.int64)
+    dup = n - np.unique(r).size
+    expected = n * n / 2 / (2 ** 12 * 8)   # birthday estimate over ~8 sigma span
+    if dup > 5 * expected + 20:
+        probs.append(("dups", dup, expected))
+    return not probs, dict(desc, probs=probs)
+
+def one_noisy_mvm(seed):
+    rng = np.random.default_rng(seed)
+    x_size = int(rng.choice([3, 31, 33, 64, 100, 257]))
+    d_size = int(rng.choice([1, 5, 32, 33, 127, 128, 129, 300]))
+    batch = int(rng.choice([7, 33, 257, 1025, 2049, 4100]))
+    if x_size * d_size * batch > 80_000_000:
+        batch = 2049 if d_size >= 128 else 257
+    transposed = bool(rng.integers(2))
+    io = io_params(inp_res=-1.0, out_res=-1.0, out_bound=1e6, out_noise=0.5, inp_noise=0.0, noise_management=NM.NONE,
+                   bound_management=BM.NONE)
+    meta = make_meta(io, io)
+    dev = constant_step(w_max_dtod=0.0, w_min_dtod=0.0, w_max=1.0, w_min=-1.0, construction_seed=1)
+    host, _orc, _ = build_pair(meta, dev, x_size, d_size, gpu=False)
+    w = (rng.integers(-38, 39, (d_size, x_size)) / 64.0).astype(np.float32)
+    host.set_weights(torch.from_numpy(w))
+    gpu = tiles.CudaAnalogTile(host)
+    gpu.set_seed(seed)
+    desc = dict(seed=seed, X=x_size, D=d_size, B=batch, transposed=transposed)
+    if not transposed:
+        x = (rng.integers(-64, 65, (batch, x_size)) / 64.0).astype(np.float32)
+        y = gpu.forward(cuda(x)).cpu().numpy()
+        z = (y - x @ w.T) / 0.5
+    else:
+        d = (rng.integers(-64, 65, (batch, d_size)) / 64.0).astype(np.float32)
+        y = gpu.backward(cuda(d)).cpu().numpy()
+        z = (y - d @ w) / 0.5
+    return noise_check(z, desc)
+
+def one_noisy_conv(seed):
+    from test_oracle_indexed_pins import conv_indices
+
+    rng = np.random.default_rng(seed)
+    c_in = int(rng.choice([1, 3, 8, 16]))
+    c_out = int(rng.choice([3, 16, 32]))
+    k = int(rng.choice([1, 3, 5]))
+    height, width = int(rng.integers(8, 15)), int(rng.integers(8, 15))
+    n = int(rng.choice([3, 13]))
+    indices, patches = conv_indices((c_in, height, width), (k, k), (1, 1), (1, 1), (1, 1), True)
+    x_size = c_in * k * k + 1
+    io = io_params(inp_res=-1.0, out_res=-1.0, out_bound=1e6, out_noise=0.5, inp_noise=0.0, noise_management=NM.NONE,
+                   bound_management=BM.NONE)
+    meta = make_meta(io, io)
+    dev = constant_step(w_max_dtod=0.0, w_min_dtod=0.0, w_max=1.0, w_min=-1.0, construction_seed=1)
+    host, _orc, _ = build_pair(meta, dev, x_size, c_out, gpu=False)
+    w = (rng.integers(-38, 39, (c_out, x_size)) / 64.0).astype(np.float32)
+    host.set_weights(torch.from_numpy(w))
+    gpu = tiles.CudaAnalogTile(host)
+    gpu.set_matrix_indices(indices)
+    gpu.set_seed(seed)
+    x = (rng.integers(-64, 65, (n, c_in, height, width)) / 64.0).astype(np.float32)
+    y = gpu.forward_indexed(cuda(x), torch.empty(n, c_out, 1, patches).cuda()).cpu().numpy().reshape(n, c_out, patches)
+    weight = torch.from_numpy(w[:, :-1].reshape(c_out, c_in, k, k).copy())
+    clean = torch.nn.functional.conv2d(torch.from_numpy(x), weight, torch.from_numpy(w[:, -1].copy()),
+                                       padding=1).numpy().reshape(n, c_out, -1)
+    z = ((y - clean) / 0.5).transpose(0, 2, 1).reshape(-1, c_out)     # [patch, out]
+    return noise_check(z, dict(seed=seed, conv=(c_in, c_out, k, height, width, n)))
+
+
+def test_output_noise_is_standard_normal_and_unshared_over_random_shapes(gpu_device):
+    """Output noise of forward, backward and the fused convolution over shapes that reach every kernel variant: the
+    standardized residuals have zero mean and unit variance (4.5 sigma), no correlation between neighbouring outputs
+    or samples, and no more repeated values than chance gives (shared streams would repeat)."""
+    suspects = [desc for ok, desc in (one_noisy_mvm(seed) for seed in range(70000, 70080)) if not ok]
+    suspects += [desc for ok, desc in (one_noisy_conv(seed) for seed in range(71000, 71060)) if not ok]
+    assert not suspects, suspects[:3]
