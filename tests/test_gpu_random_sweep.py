@@ -90,10 +90,17 @@ def one_update(seed):
         d[2] = 0.0
     gpu.update(cuda(x), cuda(d), False)
     xw, dw, blv = gpu.get_update_words(batch)
+    bl_orc, _, _ = orc.update_bl_ab(x, d)
+    words_ok = np.array_equal(blv.numpy(), bl_orc) and int(blv.max()) <= bl
+    for words, values in ((xw.numpy().view(np.uint32), x), (dw.numpy().view(np.uint32), d)):
+        # no pulse beyond a sample's bit line, none on a zero value, the sign bit where the value is negative
+        words_ok = words_ok and not (words >> (blv.numpy().astype(np.uint32)[:, None] + 1)).any()
+        words_ok = words_ok and not (words[values == 0] >> 1).any()
+        words_ok = words_ok and np.array_equal((words & 1)[(words >> 1) != 0] == 1, (values < 0)[(words >> 1) != 0])
     orc.update_with_words(xw.numpy(), dw.numpy(), blv.numpy())
     diff = np.abs(gpu.get_weights().numpy() - orc.get_weights()).max()
-    desc = dict(seed=seed, X=x_size, D=d_size, B=batch, bl=bl, um=um, soft=soft, lr=lr, diff=float(diff))
-    return diff <= 2e-5, desc
+    desc = dict(seed=seed, X=x_size, D=d_size, B=batch, bl=bl, um=um, soft=soft, lr=lr, diff=float(diff), words_ok=words_ok)
+    return diff <= 2e-5 and words_ok, desc
 
 
 def test_random_mvm_cases_are_bit_exact(gpu_device):
