@@ -61,6 +61,8 @@ struct MvmArgs {
   // pre_add[row * O + o] for the output o of the sample whose quantized input is row `row` of xq[round & 1];
   // null: none.  Only the 32 x 32 round kernels read it.
   const float *pre_add;
+  int nm_phase;             // running-average noise management: 1 = the init kernel only stores every sample's
+                            // largest absolute input in st.nm, 2 = it takes the scales from st.nm; 0 otherwise
   int small_tiles_only;     // 1: never the large-tile kernel (its row padding differs)
   const int *skip_if_zero;  // non-null: a round launch does nothing when this device value is zero
 };
@@ -69,6 +71,10 @@ struct MvmArgs {
 void launch_mvm_init(const MvmArgs &a, hipStream_t s);
 // one round of DAC -> MFMA contraction -> ADC
 void launch_mvm_round(const MvmArgs &a, hipStream_t s);
+// AverageAbsMax noise management (rpu_forward_backward_pass.cpp:138-149): nm[b] holds the largest absolute input of
+// sample b and becomes the running average after that sample, in batch order; aux carries the value between calls
+// (negative: not started)
+void launch_nm_running_average(float *nm, int m_batch, float decay, float *aux, hipStream_t s);
 // Several tiles in one launch: args[t] are the tiles' arguments in HBM, start[t] .. start[t + 1] the workgroups of
 // tile t in a round launch (all tiles share m_batch).  The tiles of one round launch share a kernel variant.
 struct MvmGroup {

@@ -598,7 +598,9 @@ __device__ __forceinline__ void mvm_init_sample(const MvmArgs &a, int b, int t, 
   float nm = 1.0f;
   const bool worst_case = io.bound_management == RPU_BM_ITERATIVE_WORST_CASE;
   const bool need_np = io.noise_management == RPU_NM_ABS_MAX_NP_SUM || worst_case;
-  if (io.noise_management == RPU_NM_ABS_MAX || io.noise_management == RPU_NM_MAX || need_np) {
+  const bool running = io.noise_management == RPU_NM_AVERAGE_ABS_MAX ||
+                       io.noise_management == RPU_NM_AVERAGE_ABS_MAX_SINGLE_VALUE;
+  if (io.noise_management == RPU_NM_ABS_MAX || io.noise_management == RPU_NM_MAX || need_np || (running && a.nm_phase == 1)) {
     float amax = 0.0f, vmax = -INFINITY, ps = 0.0f, ns = 0.0f;
     if (kept) {
 #pragma unroll
@@ -621,6 +623,10 @@ __device__ __forceinline__ void mvm_init_sample(const MvmArgs &a, int b, int t, 
       }
     }
     amax = group_max<SUB>(amax, sh);
+    if (running && a.nm_phase == 1) { // first pass of the running average: the scan over the batch comes next
+      if (t == 0) a.st.nm[b] = amax;
+      return;
+    }
     if (io.noise_management == RPU_NM_MAX) {
       vmax = group_max<SUB>(vmax, sh);
       nm = io.nm_thres > 0.0f ? fminf(vmax, io.nm_thres) : vmax;
@@ -643,6 +649,7 @@ __device__ __forceinline__ void mvm_init_sample(const MvmArgs &a, int b, int t, 
   if (io.noise_management == RPU_NM_CONSTANT) {
     nm = io.nm_thres > 0.0f ? io.nm_thres : 1.0f;
   }
+  if (running) nm = a.st.nm[b]; // second pass: the averaged scale of this sample
   // every thread of the group knows nm: the scales need no exchange
   float fin;
   const float scale = round_scales(a, nm, 1.0f, fin);
@@ -1668,6 +1675,22 @@ void launch_mvm_init(const MvmArgs &a, hipStream_t s) {
   } else {
     hipLaunchKernelGGL(k_mvm_init<16>, dim3((a.m_batch + 15) / 16), dim3(256), 0, s, a);
   }
+}
+
+// a linear recurrence over the batch, evaluated in the reference's order and rounding by one thread
+__global__ void k_nm_running_average(float *nm, int m_batch, float decay, float *aux) {
+  if (blockIdx.x != 0 || threadIdx.x != 0) return;
+  float v = *aux;
+  for (int b = 0; b < m_batch; ++b) {
+    const float amax = nm[b];
+    v = v < 0.0f ? amax : v * (1.0f - decay) + decay * amax;
+    nm[b] = v;
+  }
+  *aux = v;
+}
+
+void launch_nm_running_average(float *nm, int m_batch, float decay, float *aux, hipStream_t s) {
+  hipLaunchKernelGGL(k_nm_running_average, dim3(1), dim3(64), 0, s, nm, m_batch, decay, aux);
 }
 
 int mvm_round_workgroups(const MvmArgs &a) { return workgroups_for(a.O, a.m_batch); }

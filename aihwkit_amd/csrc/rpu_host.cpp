@@ -70,6 +70,8 @@ void IOPar::initialize(bool backward) {
   case RPU_NM_ABS_MAX_NP_SUM:
   case RPU_NM_MAX:
   case RPU_NM_CONSTANT:
+  case RPU_NM_AVERAGE_ABS_MAX:
+  case RPU_NM_AVERAGE_ABS_MAX_SINGLE_VALUE:
     break;
   default:
     throw RpuError("Noise Management type not implemented!");
@@ -401,6 +403,7 @@ void fill_default_config(rpu_tile_config *cfg, int device_kind) {
   io.nm_assumed_wmax = 0.6f;
   io.max_bm_res = 0.25f;
   io.ir_drop_g_ratio = 5.7143e5f;
+  io.nm_decay = 1e-3f;
   cfg->f_io = io;
   cfg->b_io = io;
 

@@ -188,6 +188,10 @@ struct Tile {
   // analog non-idealities before the ADC: the addend per output, up to three side contractions, the transformed
   // input rows, |W| and the squared row norms
   DevBuf<float> n_pre, n_s1, n_s2, n_s3, n_rows, n_absw, n_sumsq;
+  // running AverageAbsMax noise-management scale, one value shared by forward and backward as in the reference
+  // (rpu_forward_backward_pass.h:241); negative: not started
+  DevBuf<float> nm_aux;
+  float nm_aux_host = -1.0f; // its value while no device copy exists, and what extra state reads / writes
   DevBuf<float> dr_prev, dr_w0, dr_t, d_nu;
   float drift_t = 0.0f;
   bool nu_valid = false;
@@ -258,12 +262,25 @@ struct Tile {
     delta_w = nullptr;
     n_pre.release(); n_s1.release(); n_s2.release(); n_s3.release(); n_rows.release(); n_absw.release();
     n_sumsq.release();
+    nm_aux.release();
     d_fbw.release(); s_rowstat.release(); dr_prev.release(); dr_w0.release(); dr_t.release(); d_nu.release();
     d_cnt.release();
     fb_during_test = false;
     drift_t = 0.0f;
     nu_valid = false;
     for (auto &sl : slots) sl->release();
+  }
+
+  // brings nm_aux_host and the device copy in line (to_host: before the value is read on the host)
+  void sync_nm_aux(bool to_host) {
+    if (!resident() || !nm_aux.p) return;
+    if (to_host) {
+      sync_last();
+      RPU_HIP_CHECK(hipMemcpy(&nm_aux_host, nm_aux.p, sizeof(float), hipMemcpyDeviceToHost));
+    } else {
+      sync_last();
+      RPU_HIP_CHECK(hipMemcpy(nm_aux.p, &nm_aux_host, sizeof(float), hipMemcpyHostToDevice));
+    }
   }
 
   PhiloxKey key() const {
@@ -485,6 +502,17 @@ struct Tile {
       launch_mvm_round(a, s);
       prof_mark(s, "mvm_round");
     } else {
+      if (io.p.noise_management == RPU_NM_AVERAGE_ABS_MAX || io.p.noise_management == RPU_NM_AVERAGE_ABS_MAX_SINGLE_VALUE) {
+        // per-sample maxima, the recurrence over the batch in its order, then the usual set-up with those scales
+        if (!nm_aux.p) {
+          nm_aux.ensure(1);
+          launch_fill(nm_aux.p, nm_aux_host, 1, s);
+        }
+        a.nm_phase = 1;
+        launch_mvm_init(a, s);
+        launch_nm_running_average(a.st.nm, B, io.p.nm_decay, nm_aux.p, s);
+        a.nm_phase = 2;
+      }
       launch_mvm_init(a, s);
       prof_mark(s, "mvm_init");
       // every round after the first works on the samples whose ADC saturated in the one before; the
@@ -1378,9 +1406,24 @@ int rpu_tile_set_delta_weights(rpu_tile_t *tile, float *delta_weights_dev) {
 
 // The state beyond weights and device parameters that decides what the next calls compute: the seed and the
 // call counter of the random streams, the update counters and, for a transfer compound, its transfer counters.
+static int64_t float_bits(float v) {
+  uint32_t u;
+  std::memcpy(&u, &v, sizeof(u));
+  return (int64_t)u;
+}
+static float bits_float(int64_t b) {
+  const uint32_t u = (uint32_t)b;
+  float v;
+  std::memcpy(&v, &u, sizeof(v));
+  return v;
+}
+constexpr int kFixedExtras = 6;
+
+// floats travel as their bit patterns
 static void extra_fields(const Tile &t, std::vector<std::string> &names, std::vector<int64_t> &values) {
-  names = {"seed", "call", "update_calls", "transfer.update_idx"};
-  values = {(int64_t)t.seed, (int64_t)t.call, (int64_t)t.update_calls, (int64_t)t.update_idx};
+  names = {"seed", "call", "update_calls", "transfer.update_idx", "nm_running_average.bits", "drift_time.bits"};
+  values = {(int64_t)t.seed, (int64_t)t.call, (int64_t)t.update_calls, (int64_t)t.update_idx, float_bits(t.nm_aux_host),
+            float_bits(t.drift_t)};
   for (size_t k = 0; k < t.slice_idx.size(); ++k) {
     names.push_back("transfer.slice_idx_" + std::to_string(k));
     values.push_back(t.slice_idx[k]);
@@ -1388,7 +1431,7 @@ static void extra_fields(const Tile &t, std::vector<std::string> &names, std::ve
 }
 static thread_local std::string g_extra_name;
 
-int rpu_tile_extra_count(const rpu_tile_t *tile) { return tile ? 4 + (int)tile->t.slice_idx.size() : 0; }
+int rpu_tile_extra_count(const rpu_tile_t *tile) { return tile ? kFixedExtras + (int)tile->t.slice_idx.size() : 0; }
 
 const char *rpu_tile_extra_name(const rpu_tile_t *tile, int idx) {
   if (!tile || idx < 0 || idx >= rpu_tile_extra_count(tile)) return nullptr;
@@ -1406,6 +1449,10 @@ int rpu_tile_get_extra(rpu_tile_t *tile, int64_t *values_host) {
     std::lock_guard<std::mutex> lock(t.mutex);
     std::vector<std::string> names;
     std::vector<int64_t> values;
+    if (t.resident()) {
+      DeviceGuard g(t.device_id);
+      t.sync_nm_aux(true);
+    }
     extra_fields(t, names, values);
     std::memcpy(values_host, values.data(), values.size() * sizeof(int64_t));
   });
@@ -1421,7 +1468,13 @@ int rpu_tile_set_extra(rpu_tile_t *tile, const int64_t *values_host, int count) 
     t.call = (uint32_t)values_host[1];
     t.update_calls = (uint32_t)values_host[2];
     t.update_idx = (uint64_t)values_host[3];
-    for (size_t k = 0; k < t.slice_idx.size(); ++k) t.slice_idx[k] = (int)values_host[4 + k];
+    t.nm_aux_host = bits_float(values_host[4]);
+    t.drift_t = bits_float(values_host[5]);
+    if (t.resident()) {
+      DeviceGuard g(t.device_id);
+      t.sync_nm_aux(false);
+    }
+    for (size_t k = 0; k < t.slice_idx.size(); ++k) t.slice_idx[k] = (int)values_host[kFixedExtras + k];
   });
 }
 
@@ -1538,6 +1591,13 @@ static int group_mvm(rpu_group_t *group, const float *const *x_dev, const long *
       t.check_compute(m_batch, x_dev[i], y_dev[i]);
       if (Tile::has_pre_adc_terms(transposed ? t.bio : t.fio)) {
         throw RpuError("Output-referred weight noise and IR drop are not provided for a group: call the tiles one by one.");
+      }
+      {
+        const IOPar &gio = transposed ? t.bio : t.fio;
+        if (!gio.perfect && (gio.p.noise_management == RPU_NM_AVERAGE_ABS_MAX ||
+                             gio.p.noise_management == RPU_NM_AVERAGE_ABS_MAX_SINGLE_VALUE)) {
+          throw RpuError("Running-average noise management is not provided for a group: call the tiles one by one.");
+        }
       }
       const int in_size = transposed ? t.D : t.X, out_size = transposed ? t.X : t.D;
       const bool big = use_big && out_size >= 128;
@@ -1691,6 +1751,11 @@ int rpu_tile_clone(rpu_tile_t **out, const rpu_tile_t *src_c) {
     const Tile &s = src->t;
     t.X = s.X; t.D = s.D; t.fio = s.fio; t.bio = s.bio; t.up = s.up; t.dev = s.dev; t.arr = s.arr;
     t.lr = s.lr; t.seed = s.seed; t.call = s.call;
+    if (s.resident()) {
+      DeviceGuard g(s.device_id);
+      const_cast<Tile &>(s).sync_nm_aux(true);
+    }
+    t.nm_aux_host = s.nm_aux_host;
     t.w_host = s.w_host;
     t.idx_host = s.idx_host;
     t.idx_patches = s.idx_patches;

@@ -218,7 +218,7 @@ class AnalogTileInputOutputParameter(_Struct):
                      "out_noise", "out_asymmetry", "out_scale", "nm_thres", "nm_assumed_wmax",
                      "max_bm_res", "w_noise", "ir_drop", "out_noise_std", "out_nonlinearity",
                      "out_nonlinearity_std", "v_offset_std", "r_series", "w_read_asymmetry_dtod",
-                     "ir_drop_g_ratio"):
+                     "ir_drop_g_ratio", "nm_decay"):
             setattr(p, name, float(getattr(self, name)))
         p.w_noise_type = int(self.w_noise_type)
         return p

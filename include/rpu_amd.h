@@ -45,8 +45,8 @@ enum rpu_noise_management {
   RPU_NM_ABS_MAX_NP_SUM = 2,
   RPU_NM_MAX = 3,
   RPU_NM_CONSTANT = 4,
-  RPU_NM_AVERAGE_ABS_MAX = 5,              /* not provided: creation fails */
-  RPU_NM_AVERAGE_ABS_MAX_SINGLE_VALUE = 6, /* not provided */
+  RPU_NM_AVERAGE_ABS_MAX = 5,              /* running average over the samples seen so far (nm_decay) */
+  RPU_NM_AVERAGE_ABS_MAX_SINGLE_VALUE = 6, /* the same on this path, as in the reference's CPU code */
   RPU_NM_ABS_MAX_SINGLE_VALUE = 7          /* not provided */
 };
 
@@ -123,6 +123,7 @@ typedef struct rpu_io_params {
   float r_series;                 /* 0 */
   float w_read_asymmetry_dtod;    /* 0 */
   float ir_drop_g_ratio;          /* 5.7143e5: wire conductance over g_max (ir_drop_Gw_div_gmax) */
+  float nm_decay;                 /* 1e-3: weight of a new sample in the AverageAbsMax running average */
 } rpu_io_params;
 
 /* Replaces PulsedUpdateMetaParameter<float> (R/rpu_pulsed_meta_parameter.h:248-323) as bound by

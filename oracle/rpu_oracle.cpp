@@ -194,6 +194,7 @@ struct OrcTile {
   // R/rpu_linearstep_device.h:199-200
   std::vector<float> slope_up, slope_down;
   std::vector<int32_t> last_rounds;
+  float aux_nm = -1.0f; // running AverageAbsMax scale (R/rpu_forward_backward_pass.h:241), negative: not started
   // scratch
   std::vector<float> in_buf, bias_buf;
   std::vector<std::vector<int>> x_idx, d_idx;
@@ -355,8 +356,19 @@ void clip_to_bounds(OrcTile &t) {
 // forward / backward
 
 // R/rpu_forward_backward_pass.cpp:112-178 computeNoiseManagement
-float noise_management(const float *in, int size, int inc, int nm_type, const rpu_io_params &io) {
+float noise_management(const float *in, int size, int inc, int nm_type, const rpu_io_params &io, float &aux) {
   switch (nm_type) {
+  case RPU_NM_AVERAGE_ABS_MAX:
+  case RPU_NM_AVERAGE_ABS_MAX_SINGLE_VALUE: { // :138-149, one running value shared by forward and backward
+    float amax = 0.f;
+    for (int j = 0; j < size; ++j) amax = std::max(amax, fabsf(in[(size_t)j * inc]));
+    if (aux < 0.0f) {
+      aux = amax;
+    } else {
+      aux = aux * (1.0f - io.nm_decay) + io.nm_decay * amax;
+    }
+    return aux;
+  }
   case RPU_NM_NONE:
     return 1.0f;
   case RPU_NM_ABS_MAX: {
@@ -543,7 +555,7 @@ bool analog_mv(OrcTile &t, const float *in, int in_size, int in_inc, float *out,
 int forward_vector(OrcTile &t, const float *x, int x_inc, float *y, int d_inc) {
   const rpu_io_params &io = t.fio.p;
   const int X = t.X, D = t.D;
-  float nm_scale = noise_management(x, X, x_inc, io.noise_management, io);
+  float nm_scale = noise_management(x, X, x_inc, io.noise_management, io, t.aux_nm);
   const bool nm = io.noise_management != RPU_NM_NONE;
   const bool bm = io.bound_management != RPU_BM_NONE;
   if (nm && (nm_scale <= 0.0f) && (io.inp_noise <= 0.0f)) {
@@ -561,7 +573,7 @@ int forward_vector(OrcTile &t, const float *x, int x_inc, float *y, int d_inc) {
     reduction *= 2.0f;
     if (bm_round == 1 && io.bound_management == RPU_BM_ITERATIVE_WORST_CASE &&
         io.noise_management != RPU_NM_ABS_MAX_NP_SUM) {
-      nm_scale = noise_management(x, X, x_inc, RPU_NM_ABS_MAX_NP_SUM, io);
+      nm_scale = noise_management(x, X, x_inc, RPU_NM_ABS_MAX_NP_SUM, io, t.aux_nm);
       reduction = 1.0f;
     }
     bm_round++;
@@ -594,7 +606,7 @@ int forward_vector(OrcTile &t, const float *x, int x_inc, float *y, int d_inc) {
 void backward_vector(OrcTile &t, const float *d, int d_inc, float *x, int x_inc) {
   const rpu_io_params &io = t.bio.p;
   const int X = t.X, D = t.D;
-  float nm_scale = noise_management(d, D, d_inc, io.noise_management, io);
+  float nm_scale = noise_management(d, D, d_inc, io.noise_management, io, t.aux_nm);
   const bool nm = io.noise_management != RPU_NM_NONE;
   const float out_scale = io.out_scale * 1.0f;
   const bool scaling = nm && nm_scale > 0.0f;

@@ -143,3 +143,48 @@ def test_weight_noise_under_bound_management_and_other_paths(gpu_device):
     group = tiles.TileGroup([gpu, quiet_gpu])
     with pytest.raises(RuntimeError, match="not provided for a group"):
         group.forward([torch.from_numpy(x).cuda(), torch.from_numpy(x).cuda()])
+
+
+@pytest.mark.parametrize("bm", [dv.BoundManagementType.NONE, dv.BoundManagementType.Iterative,
+                                dv.BoundManagementType.IterativeWorstCase])
+def test_running_average_noise_management_is_bit_exact_and_shared(gpu_device, bm):
+    """AverageAbsMax in the exact-arithmetic setting: the scale of a sample depends on every sample before it, in this
+    call and in earlier forward and backward calls; outputs, rounds and the continuation must equal the oracle's."""
+    rng = np.random.default_rng(11)
+    x_size, d_size = 100, 70
+    io = dict(inp_res=1 / 128.0, out_res=1 / 512.0, out_noise=0.0, inp_noise=0.0, out_bound=4.0, nm_decay=0.25,
+              noise_management=dv.NoiseManagementType.AverageAbsMax)
+    meta = make_meta(io_params(bound_management=bm, **io), io_params(**io))
+    dev = constant_step(w_max=1.0, w_min=-1.0, w_max_dtod=0.0, w_min_dtod=0.0, construction_seed=1)
+    host, orc, _ = build_pair(meta, dev, x_size, d_size, gpu=False)
+    w = (rng.integers(-38, 39, (d_size, x_size)) / 64.0).astype(F)
+    host.set_weights(torch.from_numpy(w))
+    orc.set_weights(w)
+    gpu = tiles.CudaAnalogTile(host)
+    for batch in (1, 37, 300):
+        x = ((rng.integers(-64, 65, (batch, x_size)) / 64.0) * rng.uniform(0.05, 1.0, (batch, 1))).astype(F)
+        x = (np.round(x * 64) / 64).astype(F)
+        if batch > 2:
+            x[1] = 0.0
+        assert np.array_equal(gpu.forward(torch.from_numpy(x).cuda()).cpu().numpy(), orc.forward(x)), batch
+        if bm != dv.BoundManagementType.NONE:
+            assert np.array_equal(gpu.get_bm_rounds(batch).numpy(), orc.bm_rounds(batch))
+        d = (rng.integers(-64, 65, (batch, d_size)) / 64.0).astype(F)
+        assert np.array_equal(gpu.backward(torch.from_numpy(d).cuda()).cpu().numpy(), orc.backward(d)), batch
+    # the running value is part of the extra state: a copy that loads it continues identically
+    state = gpu.dump_extra()
+    assert "rpu.nm_running_average.bits" in state
+    other = tiles.CudaAnalogTile(host)
+    other.load_extra(state, True)
+    x = (rng.integers(-64, 65, (9, x_size)) / 256.0).astype(F)
+    want = orc.forward(x)
+    assert np.array_equal(other.forward(torch.from_numpy(x).cuda()).cpu().numpy(), want)
+    assert np.array_equal(gpu.forward(torch.from_numpy(x).cuda()).cpu().numpy(), want)
+    fresh = tiles.CudaAnalogTile(host)                            # without the state the average starts anew
+    assert not np.array_equal(fresh.forward(torch.from_numpy(x).cuda()).cpu().numpy(), want)
+    import copy
+    twin = copy.deepcopy(gpu)                                     # a copy carries the value
+    x2 = (rng.integers(-64, 65, (5, x_size)) / 128.0).astype(F)
+    assert np.array_equal(twin.forward(torch.from_numpy(x2).cuda()).cpu().numpy(), orc.forward(x2))
+    with pytest.raises(RuntimeError, match="not provided for a group"):
+        tiles.TileGroup([gpu, twin]).forward([torch.from_numpy(x2).cuda(), torch.from_numpy(x2).cuda()])

@@ -88,3 +88,33 @@ def test_weight_noise_variance_laws():
     sigma = 0.1 * np.sqrt((dm.astype(np.float64) ** 2) @ np.abs(w.astype(np.float64)))
     z = (got - dm.astype(np.float64) @ w.astype(np.float64)) / sigma
     assert abs(z.mean()) < 4 / np.sqrt(z.size) and abs(z.std() - 1) < 4 / np.sqrt(2 * z.size)
+
+
+def test_running_average_noise_management_closed_form():
+    """AverageAbsMax: the first sample sets the scale, every further one moves it by nm_decay towards its own largest
+    absolute input; forward and backward share the one value and it lives on between calls.  With an identity tile and
+    the DAC clipping at 1 the largest output of a sample whose input exceeds the scale is the scale itself.  Maxima
+    1, 2, 2, 2, ... with nm_decay = 0.5 give 2 - 2^-b."""
+    n = 6
+    io = dict(noise_management=dv.NoiseManagementType.AverageAbsMax, nm_decay=0.5, inp_bound=1.0)
+    tile = oracle_tile(n, n, np.eye(n), **io)
+    x = np.zeros((5, n), dtype=F)
+    x[:, 0] = [1.0, 2.0, 2.0, 2.0, 2.0]
+    x[:, 1] = [0.5, -0.25, 0.125, 1.0, -2.0]                     # smaller entries pass through unchanged
+    y = tile.forward(x)
+    want = 2.0 - 0.5 ** np.arange(5)
+    np.testing.assert_allclose(y[:, 0], want, rtol=1e-6)
+    np.testing.assert_allclose(y[:3, 1], x[:3, 1], rtol=1e-6)
+    np.testing.assert_allclose(y[4, 1], -want[4], rtol=1e-6)      # clipped on the negative side as well
+    d = np.zeros((2, n), dtype=F)
+    d[:, 3] = [-2.0, 2.0]                                         # the backward pass continues the same average
+    g = tile.backward(d)
+    np.testing.assert_allclose(np.abs(g[:, 3]), 2.0 - 0.5 ** np.arange(5, 7), rtol=1e-6)
+    y = tile.forward(x[1:2])                                      # and the next forward call goes on from there
+    np.testing.assert_allclose(y[0, 0], 2.0 - 0.5 ** 7, rtol=1e-6)
+    fresh = oracle_tile(n, n, np.eye(n), **io)                    # another tile starts from its own first sample
+    np.testing.assert_allclose(fresh.forward(x[1:3])[:, 0], [2.0, 2.0], rtol=1e-6)
+    # a sample below the average is scaled by the average, not by its own maximum: nothing clips, the value survives
+    low = np.zeros((1, n), dtype=F)
+    low[0, 2] = 0.01
+    np.testing.assert_allclose(fresh.forward(low)[0, 2], 0.01, rtol=1e-5)
