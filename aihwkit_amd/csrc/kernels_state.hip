@@ -56,8 +56,16 @@ __global__ __launch_bounds__(256) void k_clip_value(float *w, const float *w_min
   if (clip_dev && !(clip > 0.0f)) return;
   for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
     float v = w[i];
-    if (symmetric) v = fminf(fmaxf(v, -clip), clip);
-    w[i] = clip_to(v, w_min, w_max, i);
+    if (symmetric) {
+      // the reference's order: upper limits first, then the lower ones win (it matters for a device whose sampled
+      // bounds lie beyond the clip value on the wrong side)
+      const float hi = w_max ? fminf(w_max[i], clip) : clip;
+      const float lo = w_min ? fmaxf(w_min[i], -clip) : -clip;
+      v = fmaxf(fminf(v, hi), lo);
+    } else {
+      v = clip_to(v, w_min, w_max, i);
+    }
+    w[i] = v;
   }
 }
 
@@ -185,7 +193,9 @@ __global__ __launch_bounds__(256) void k_device_drift(float *w, float *prev, flo
       if (p.a != 0.0f) v = v + p.a * (nu_scale - 1.0f);
     }
     if (p.w_read_std > 0.0f) v += p.w_read_std * z[1];
-    v = clip_to(v, w_min, w_max, i);
+    // saturate (weight_drifter.cpp:98-106): the lower bound first, the upper one wins
+    if (w_min) v = fmaxf(v, w_min[i]);
+    if (w_max) v = fminf(v, w_max[i]);
     prev[i] = v;
     w[i] = v;
   }

@@ -163,8 +163,8 @@ class Drifter:
         out = np.where(changed, w, drifted).astype(F)
         if self.w_read_std > 0:
             out = (out + self.w_read_std * read_normals.astype(F)).astype(F)
-        if w_min is not None:
-            out = np.maximum(np.minimum(out, w_max), w_min)
+        if w_min is not None:                                   # saturate, :98-106: MIN(MAX(min, w), max)
+            out = np.minimum(np.maximum(out, w_min), w_max)
         self.prev = out.copy()
         return out
 

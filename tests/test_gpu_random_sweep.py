@@ -524,3 +524,102 @@ def test_output_noise_is_standard_normal_and_unshared_over_random_shapes(gpu_dev
     suspects = [desc for ok, desc in (one_noisy_mvm(seed) for seed in range(70000, 70080)) if not ok]
     suspects += [desc for ok, desc in (one_noisy_conv(seed) for seed in range(71000, 71060)) if not ok]
     assert not suspects, suspects[:3]
+
+
+def one_state(seed):
+    """Weight maintenance and hardware-aware-training helpers on random shapes against the numpy restatements.  The
+    large pulsed tiles hold devices whose sampled bounds cross or lie beyond a clip value on the wrong side, where the
+    order of the two limits decides the result."""
+    import hwa_oracle as ho
+    import state_oracle as so
+
+    F = np.float32
+    rng = np.random.default_rng(seed)
+    x = int(rng.choice([1, 2, 3, 31, 33, 63, 64, 65, 255, 256, 257, 1000, 1025]))
+    d = int(rng.choice([1, 2, 5, 33, 64, 255, 257, 300]))
+    bad = []
+
+    def fp_tile():
+        host = dv.FloatingPointTileParameter().create_array(x, d)
+        host.set_weights(torch.from_numpy(rng.normal(0.01, 0.3, (d, x)).astype(F)))
+        return tiles.CudaFloatingPointTile(host)
+
+    def hidden(tile):
+        values = tile.get_hidden_parameters().numpy()
+        return {name: values[k] for k, name in enumerate(tile.get_hidden_parameter_names())}
+
+    # remap
+    tile = fp_tile()
+    w = tile.get_weights().numpy()
+    s0 = rng.uniform(0.5, 2.0, d).astype(F)
+    kind = [1, 2, 3][rng.integers(3)]
+    kw = {1: dict(remapped_wmax=float(rng.choice([1.0, 0.7]))),
+          2: [dict(), dict(max_scale_range=1.4), dict(remapped_wmax=0.8)][rng.integers(3)],
+          3: dict(row_norm=float(rng.choice([0.5, 3.0])), clip_if=bool(rng.integers(2)))}[kind]
+    par = tiles.WeightRemapParameter()
+    par.type = kind
+    for name, value in kw.items():
+        setattr(par, name, value)
+    scales = torch.from_numpy(s0).cuda()
+    tile.remap_weights(par, scales)
+    want_w, want_s = ho.remap(w, s0, kind, **kw)
+    if not (np.allclose(scales.cpu().numpy(), want_s, rtol=3e-6)
+            and np.allclose(tile.get_weights().numpy(), want_w, rtol=3e-6, atol=1e-9)):
+        bad.append(("remap", kind, kw))
+    # deterministic modifiers (a value on a rounding edge may fall to either side)
+    tile = fp_tile()
+    w = tile.get_weights().numpy()
+    mod_kind = [1, 5][rng.integers(2)]
+    mod_kw = dict(res=float(rng.choice([0.05, 0.132])), copy_last_column=bool(rng.integers(2)) and x > 1,
+                  rel_to_actual_wmax=bool(rng.integers(2)), assumed_wmax=0.9)
+    mod = tiles.WeightModifierParameter()
+    mod.type = mod_kind
+    for name, value in mod_kw.items():
+        setattr(mod, name, value)
+    tile.modify_weights(mod)
+    off = np.abs(tile.get_modified_weights().numpy() - ho.modify(w, mod_kind, **mod_kw)) > 1e-6
+    if off.mean() > 2e-3 + 2.0 / off.size:
+        bad.append(("modify", mod_kind, mod_kw, float(off.mean())))
+    # decay, clip and drift of a pulsed tile
+    meta = make_meta(noise_free_io(), noise_free_io())
+    dev = soft_bounds(construction_seed=int(rng.integers(1, 99)), lifetime=50.0, lifetime_dtod=0.2, reset=0.02,
+                      reset_dtod=0.5)
+    dev.drift.nu = 0.07
+    dev.drift.nu_dtod = 0.2
+    host = meta.create_array(x, d, dev)
+    host.set_weights(torch.from_numpy(rng.uniform(-0.5, 0.5, (d, x)).astype(F)))
+    tile = tiles.CudaAnalogTile(host)
+    par_h = hidden(tile)
+    w = tile.get_weights().numpy()
+    tile.decay_weights(0.7)
+    w = so.decay_device(w, par_h["decay_scales"], par_h["reset_bias"], par_h["min_bound"], par_h["max_bound"], 0.7)
+    if np.abs(tile.get_weights().numpy() - w).max() > 1e-6:
+        bad.append(("decay",))
+    w = tile.get_weights().numpy()
+    tile.clip_weights(tiles.WeightClipParameter(type=tiles.WeightClipType.FIXED_VALUE, fixed_value=0.3))
+    if np.abs(tile.get_weights().numpy() - so.clip_fixed(w, 0.3, par_h["min_bound"], par_h["max_bound"])).max() > 0:
+        bad.append(("clip",))
+    w = tile.get_weights().numpy()
+    drifter = ho.Drifter(par_h["drift_nu"])
+    tile.drift_weights(5.0)
+    want = drifter.apply(w, 5.0, w_min=par_h["min_bound"], w_max=par_h["max_bound"])
+    if not np.allclose(tile.get_weights().numpy(), want, rtol=3e-6, atol=1e-7):
+        bad.append(("drift",))
+    # clip types of a floating-point tile
+    if x * d > 1:
+        tile = fp_tile()
+        w = tile.get_weights().numpy()
+        tile.clip_weights(tiles.WeightClipParameter(type=tiles.WeightClipType.LAYER_GAUSSIAN, sigma=1.5))
+        if np.abs(tile.get_weights().numpy() - so.clip_with_value(w, so.clip_value_layer_gaussian(w, 1.5))).max() > 2e-6:
+            bad.append(("clip_gauss",))
+    tile = fp_tile()
+    w = tile.get_weights().numpy()
+    tile.clip_weights(tiles.WeightClipParameter(type=tiles.WeightClipType.AVERAGE_CHANNEL_MAX))
+    if np.abs(tile.get_weights().numpy() - so.clip_with_value(w, so.clip_value_average_channel_max(w))).max() > 2e-6:
+        bad.append(("clip_channel",))
+    return not bad, dict(seed=seed, X=x, D=d, bad=bad)
+
+
+def test_random_state_and_training_helper_cases_follow_the_oracles(gpu_device):
+    failures = [desc for ok, desc in (one_state(seed) for seed in range(80000, 80120)) if not ok]
+    assert not failures, failures[:3]

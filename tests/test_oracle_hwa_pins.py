@@ -149,6 +149,11 @@ def test_drift_golden_vector_and_clock():
     want = np.clip(w * 2.0 ** (-(0.1 + 0.03 * z.astype(np.float64))) - 0.01 * z, -0.2, 0.2)
     np.testing.assert_allclose(out, want, rtol=1e-5, atol=1e-7)
     np.testing.assert_array_equal(d.prev, out)
+    # a device whose sampled bounds cross (min above max): the saturation applies the lower bound first, the upper wins
+    d = ho.Drifter(0.1)
+    out = d.apply(np.array([[0.3, 0.3]], dtype=F), 2.0, w_min=np.array([[0.5, -1.0]], dtype=F),
+                  w_max=np.array([[0.1, 1.0]], dtype=F))
+    np.testing.assert_allclose(out, [[0.1, 0.3 * 2.0 ** (-0.1)]], rtol=1e-6)
 
 
 def test_pulse_counts_against_brute_force():
