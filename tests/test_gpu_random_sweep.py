@@ -623,3 +623,88 @@ def one_state(seed):
 def test_random_state_and_training_helper_cases_follow_the_oracles(gpu_device):
     failures = [desc for ok, desc in (one_state(seed) for seed in range(80000, 80120)) if not ok]
     assert not failures, failures[:3]
+
+
+def one_pcm(seed):
+    from aihwkit_amd.inference.pcm import InferenceTile, PCMLikeNoiseModel
+    from pcm_oracle import PcmOracle
+
+    F = np.float32
+    rng = np.random.default_rng(seed)
+    out_size = int(rng.choice([1, 3, 33, 96, 257]))
+    in_size = int(rng.choice([1, 2, 31, 130, 513]))
+    model = dict(prog_noise_scale=0.0, read_noise_scale=0.0, g_min=float(rng.choice([0.0, 1.0, 3.0])),
+                 g_max=float(rng.choice([25.0, 40.0])), drift_scale=float(rng.choice([1.0, 0.5])),
+                 t_0=float(rng.choice([20.0, 50.0])))
+    w = rng.normal(0, 0.3, (out_size, in_size)).astype(F)
+    tile = InferenceTile(out_size, in_size, forward_io=noise_free_io(inp_res=1 / 254.0, out_res=1 / 254.0),
+                         noise_model=PCMLikeNoiseModel(**model))
+    tile.set_weights(torch.from_numpy(w))
+    tile = tile.cuda()
+    tile.tile.set_seed(seed)
+    tile.program_weights()
+    prog, nu_p, nu_m = (t.numpy() for t in tile.drift_state())
+    bad = []
+    if np.abs(prog - w).max() > 2e-6:
+        bad.append(("program", float(np.abs(prog - w).max())))
+    orc = PcmOracle(**model)
+    for t_inf in (0.0, float(rng.choice([10.0, 3600.0])), 86400.0 * 365):
+        tile.drift_weights(t_inf)
+        want = orc.apply_drift_noise(prog, [nu_p, nu_m], t_inf)
+        diff = np.abs(tile.get_weights().numpy() - want).max()
+        if diff > 1e-5:
+            bad.append(("drift", t_inf, float(diff)))
+    return not bad, dict(seed=seed, shape=(out_size, in_size), model=model, bad=bad)
+
+def one_irdrop(seed):
+    F = np.float32
+    rng = np.random.default_rng(seed)
+    x_size = int(rng.choice([2, 31, 33, 64, 65, 129, 300]))
+    d_size = int(rng.choice([1, 3, 32, 33, 97, 200]))
+    batch = int(rng.choice([1, 7, 33, 100, 300]))
+    bias = bool(rng.integers(2))
+    x_trans = bool(rng.integers(2))
+    d_trans = x_trans
+    nm = [NM.NONE, NM.AbsMax][rng.integers(2)]
+    bm = [BM.NONE, BM.Iterative][rng.integers(2)]
+    lines = max(x_size, d_size)                                   # the longer of the two directions sets the scale
+    mean_current = 0.3 * 0.5 * lines
+    io = dict(out_noise=0.0, inp_noise=0.0, out_res=-1.0, ir_drop=float(rng.choice([0.5, 1.0, 2.0])),
+              ir_drop_g_ratio=lines * mean_current / 0.4, out_bound=float(rng.choice([1.0, 3.0, 12.0])),
+              noise_management=nm)
+    meta = make_meta(io_params(bound_management=bm, **io), io_params(**io))
+    dev = constant_step(w_max=1.0, w_min=-1.0, w_max_dtod=0.0, w_min_dtod=0.0, construction_seed=1)
+    host, orc, _ = build_pair(meta, dev, x_size, d_size, gpu=False)
+    w = rng.uniform(-0.6, 0.6, (d_size, x_size)).astype(F)
+    host.set_weights(torch.from_numpy(w))
+    orc.set_weights(w)
+    gpu = tiles.CudaAnalogTile(host)
+    xs = x_size - int(bias)
+    x = rng.uniform(-1, 1, (batch, xs)).astype(F)
+    xin = np.ascontiguousarray(x.T) if x_trans else x
+    want = orc.forward(xin, bias, x_trans, d_trans)
+    got = gpu.forward(torch.from_numpy(xin).cuda(), bias, x_trans, d_trans).cpu().numpy()
+    bad = []
+    scale = max(np.abs(want).max(), 1e-3)
+    if np.abs(got - want).max() > 2e-5 * scale:
+        bad.append(("fwd", float(np.abs(got - want).max() / scale)))
+    if bm != BM.NONE and not np.array_equal(gpu.get_bm_rounds(batch).numpy(), orc.bm_rounds(batch)):
+        bad.append(("rounds",))
+    d = rng.normal(0, 0.5, (batch, d_size)).astype(F)
+    din = np.ascontiguousarray(d.T) if d_trans else d
+    want_b = orc.backward(din, bias, d_trans, x_trans)
+    got_b = gpu.backward(torch.from_numpy(din).cuda(), bias, d_trans, x_trans).cpu().numpy()
+    sb = max(np.abs(want_b).max(), 1e-3)
+    if np.abs(got_b - want_b).max() > 2e-5 * sb:
+        bad.append(("bwd", float(np.abs(got_b - want_b).max() / sb)))
+    return not bad, dict(seed=seed, X=x_size, D=d_size, B=batch, bias=bias, trans=x_trans, nm=str(nm), bm=str(bm), io=io,
+                         bad=bad)
+
+
+def test_random_inference_pipeline_and_ir_drop_cases_follow_the_oracles(gpu_device):
+    """Programming and drift of the PCM pipeline with the noise scales at zero (conductance mapping, drift exponents,
+    g_min / g_max / t_0 variants) to 1e-5; IR drop over shapes, layouts, bias column and bound management to 2e-5 of
+    the output range with identical round counts."""
+    failures = [desc for ok, desc in (one_pcm(seed) for seed in range(90000, 90100)) if not ok]
+    failures += [desc for ok, desc in (one_irdrop(seed) for seed in range(91000, 91150)) if not ok]
+    assert not failures, failures[:3]
