@@ -441,3 +441,69 @@ def test_output_noise_of_the_large_tile_kernel_is_standard_normal_and_unshared(g
     for a, b in ((zc[:, :-1], zc[:, 1:]), (zc[:-1], zc[1:]), (zc[:, :128], zc[:, 128:256]), (zc[:128], zc[128:256]),
                  (zc[:, :512], zc[:, 512:])):
         assert abs((a * b).mean().item()) < 5 / np.sqrt(a.numel())
+
+
+@pytest.mark.parametrize("x_size,d_size,bm", [(800, 64, BM.Iterative), (64, 800, BM.NONE)])
+def test_operands_beyond_two_to_the_31_elements(gpu_device, x_size, d_size, bm):
+    """Three million samples: the input (or output) matrix and the quantized-input scratch hold more than 2^31
+    elements, so every row offset needs 64-bit arithmetic.  Exact-arithmetic setting; the oracle checks the first, middle
+    and last rows and 200 random ones (rows are independent)."""
+    batch = 3_000_000
+    rng = np.random.default_rng(1)
+    f_io = noise_free_io(inp_res=1 / 128.0, out_res=1 / 512.0, noise_management=NM.AbsMax, bound_management=bm, out_bound=4.0)
+    b_io = noise_free_io(inp_res=1 / 128.0, out_res=1 / 512.0, noise_management=NM.AbsMax)
+    dev = constant_step(w_max_dtod=0.0, w_min_dtod=0.0, w_max=1.0, w_min=-1.0, construction_seed=7)
+    host, orc, _ = build_pair(make_meta(f_io, b_io), dev, x_size, d_size, gpu=False)
+    w = (rng.integers(-38, 39, (d_size, x_size)) / 64.0).astype(np.float32)
+    host.set_weights(torch.from_numpy(w))
+    orc.set_weights(w)
+    gpu = tiles.CudaAnalogTile(host)
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(3)
+    rows = np.concatenate([np.arange(0, 40), np.arange(batch // 2 - 20, batch // 2 + 20), np.arange(batch - 40, batch),
+                           rng.integers(0, batch, 200)])
+    pick = torch.from_numpy(rows).cuda()
+    x = torch.randint(-64, 65, (batch, x_size), device="cuda", generator=gen).float() / 64.0
+    assert max(x.numel(), batch * d_size) > 2 ** 31
+    y = gpu.forward(x)
+    assert np.array_equal(y[pick].cpu().numpy(), orc.forward(x[pick].cpu().numpy()))
+    if bm != BM.NONE:
+        rounds = gpu.get_bm_rounds(batch).numpy()
+        assert np.array_equal(rounds[rows], orc.bm_rounds(len(rows))) and rounds.max() > 1
+    del x, y
+    d = torch.randint(-64, 65, (batch, d_size), device="cuda", generator=gen).float() / 64.0
+    gx = gpu.backward(d)
+    assert np.array_equal(gx[pick].cpu().numpy(), orc.backward(d[pick].cpu().numpy()))
+
+
+@pytest.mark.parametrize("x_size,d_size,batch", [(33, 70000, 3), (70000, 33, 3), (5000, 5000, 2), (1, 1, 1), (1, 70000, 1),
+                                                 (70000, 1, 5)])
+def test_extreme_tile_shapes(gpu_device, x_size, d_size, batch):
+    """One-line tiles, a single cross-point, more than 65535 rows or columns, 25 million cross-points: forward and
+    backward bit-exact (exact-arithmetic setting), the stochastic update through the GPU's words to 1e-5, and the
+    elementwise maintenance kernels run."""
+    rng = np.random.default_rng(1)
+    f_io = noise_free_io(inp_res=1 / 128.0, out_res=1 / 512.0, noise_management=NM.AbsMax, bound_management=BM.Iterative,
+                         out_bound=4.0)
+    b_io = noise_free_io(inp_res=1 / 128.0, out_res=1 / 512.0, noise_management=NM.AbsMax)
+    dev = constant_step(w_max_dtod=0.0, w_min_dtod=0.0, w_max=1.0, w_min=-1.0, dw_min_std=0.0, construction_seed=7)
+    host, orc, _ = build_pair(make_meta(f_io, b_io, desired_bl=31), dev, x_size, d_size, gpu=False)
+    w = (rng.integers(-38, 39, (d_size, x_size)) / 64.0).astype(np.float32)
+    host.set_weights(torch.from_numpy(w))
+    orc.set_weights(w)
+    gpu = tiles.CudaAnalogTile(host)
+    x = (rng.integers(-64, 65, (batch, x_size)) / 64.0).astype(np.float32)
+    d = (rng.integers(-64, 65, (batch, d_size)) / 64.0).astype(np.float32)
+    assert np.array_equal(gpu.forward(cuda(x)).cpu().numpy(), orc.forward(x))
+    assert np.array_equal(gpu.get_bm_rounds(batch).numpy(), orc.bm_rounds(batch))
+    assert np.array_equal(gpu.backward(cuda(d)).cpu().numpy(), orc.backward(d))
+    gpu.set_learning_rate(0.05)
+    orc.set_learning_rate(0.05)
+    gpu.update(cuda(x), cuda(0.2 * d), False)
+    xw, dw, bl = (t.numpy() for t in gpu.get_update_words(batch))
+    orc.update_with_words(xw, dw, bl)
+    assert np.abs(gpu.get_weights().numpy() - orc.get_weights()).max() <= TOL
+    if x_size * d_size > 1:
+        assert np.abs(orc.get_weights() - w).max() > 0
+    gpu.clip_weights(tiles.WeightClipParameter(type=tiles.WeightClipType.FIXED_VALUE, fixed_value=0.25))
+    assert float(gpu.get_weights().abs().max()) <= 0.25
