@@ -370,10 +370,14 @@ struct Tile {
     return d;
   }
 
-  void check_compute(int m_batch, const void *p0, const void *p1) {
+  // false: an empty batch, nothing to do (the reference's loops over the samples run zero times; pointers of an empty
+  // tensor may be null)
+  bool check_compute(int m_batch, const void *p0, const void *p1) {
     if (!resident()) throw RpuError("Tile is not resident on a GPU: forward / backward / update need rpu_tile_to_device first.");
-    if (m_batch <= 0) throw RpuError("m_batch must be positive.");
+    if (m_batch < 0) throw RpuError("m_batch must not be negative.");
+    if (m_batch == 0) return false;
     if (!p0 || !p1) throw RpuError("Null device pointer.");
+    return true;
   }
 
   // shared driver of forward (transposed = 0) and backward (transposed = 1)
@@ -1284,7 +1288,7 @@ int rpu_tile_has_matrix_indices(const rpu_tile_t *tile) { return tile ? tile->t.
     if (!tile) throw RpuError("null tile");                                                    \
     Tile &t = tile->t;                                                                         \
     std::lock_guard<std::mutex> lock(t.mutex);                                                 \
-    t.check_compute(n_images, x_dev, d_dev);                                                   \
+    if (!t.check_compute(n_images, x_dev, d_dev)) return;                                      \
     if (image_size <= 0) throw RpuError("image_size must be positive.");                       \
     if ((long)t.idx_max - 2 >= image_size) throw RpuError("Index matrix entry beyond the image size."); \
     DeviceGuard g(t.device_id);                                                                \
@@ -1560,7 +1564,8 @@ static int group_mvm(rpu_group_t *group, const float *const *x_dev, const long *
                      const long *y_ld, int m_batch, bool transposed, bool is_test, void *stream) {
   return guarded([&] {
     if (!group || !x_dev || !y_dev) throw RpuError("null argument");
-    if (m_batch <= 0) throw RpuError("m_batch must be positive.");
+    if (m_batch < 0) throw RpuError("m_batch must not be negative.");
+    if (m_batch == 0) return;
     std::lock_guard<std::mutex> glock(group->mutex);
     DeviceGuard dg(group->device_id);
     hipStream_t s = (hipStream_t)stream;
@@ -1588,7 +1593,7 @@ static int group_mvm(rpu_group_t *group, const float *const *x_dev, const long *
     for (int i = 0; i < n; ++i) {
       Tile &t = group->tiles[i]->t;
       std::lock_guard<std::mutex> lock(t.mutex);
-      t.check_compute(m_batch, x_dev[i], y_dev[i]);
+      (void)t.check_compute(m_batch, x_dev[i], y_dev[i]);
       if (Tile::has_pre_adc_terms(transposed ? t.bio : t.fio)) {
         throw RpuError("Output-referred weight noise and IR drop are not provided for a group: call the tiles one by one.");
       }
@@ -1827,7 +1832,7 @@ int rpu_tile_forward(rpu_tile_t *tile, const float *x_dev, float *y_dev, int m_b
     if (!tile) throw RpuError("null tile");
     Tile &t = tile->t;
     std::lock_guard<std::mutex> lock(t.mutex);
-    t.check_compute(m_batch, x_dev, y_dev);
+    if (!t.check_compute(m_batch, x_dev, y_dev)) return;
     DeviceGuard g(t.device_id);
     t.mvm(x_dev, y_dev, m_batch, bias != 0, x_trans != 0, d_trans != 0, false, (hipStream_t)stream, nullptr, nullptr,
           is_test != 0);
@@ -1840,7 +1845,7 @@ int rpu_tile_backward(rpu_tile_t *tile, const float *d_dev, float *x_dev, int m_
     if (!tile) throw RpuError("null tile");
     Tile &t = tile->t;
     std::lock_guard<std::mutex> lock(t.mutex);
-    t.check_compute(m_batch, d_dev, x_dev);
+    if (!t.check_compute(m_batch, d_dev, x_dev)) return;
     DeviceGuard g(t.device_id);
     t.mvm(d_dev, x_dev, m_batch, bias != 0, d_trans != 0, x_trans != 0, true, (hipStream_t)stream);
   });
@@ -1852,7 +1857,7 @@ int rpu_tile_update(rpu_tile_t *tile, const float *x_dev, const float *d_dev, in
     if (!tile) throw RpuError("null tile");
     Tile &t = tile->t;
     std::lock_guard<std::mutex> lock(t.mutex);
-    t.check_compute(m_batch, x_dev, d_dev);
+    if (!t.check_compute(m_batch, x_dev, d_dev)) return;
     DeviceGuard g(t.device_id);
     t.update(x_dev, d_dev, m_batch, bias != 0, x_trans != 0, d_trans != 0, (hipStream_t)stream);
   });
@@ -1864,7 +1869,7 @@ int rpu_tile_update_with_words(rpu_tile_t *tile, const uint32_t *x_words_dev, co
     if (!tile) throw RpuError("null tile");
     Tile &t = tile->t;
     std::lock_guard<std::mutex> lock(t.mutex);
-    t.check_compute(m_batch, x_words_dev, d_words_dev);
+    if (!t.check_compute(m_batch, x_words_dev, d_words_dev)) return;
     DeviceGuard g(t.device_id);
     t.update_with_words(x_words_dev, d_words_dev, m_batch, (hipStream_t)stream);
   });

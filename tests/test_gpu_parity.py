@@ -507,3 +507,20 @@ def test_extreme_tile_shapes(gpu_device, x_size, d_size, batch):
         assert np.abs(orc.get_weights() - w).max() > 0
     gpu.clip_weights(tiles.WeightClipParameter(type=tiles.WeightClipType.FIXED_VALUE, fixed_value=0.25))
     assert float(gpu.get_weights().abs().max()) <= 0.25
+
+
+def test_empty_batches_do_nothing(gpu_device):
+    """A batch of zero samples: empty outputs, untouched weights and random streams (the reference's loops over the
+    samples run zero times)."""
+    meta, dev = config1(noise=False)
+    host, _orc, gpu = build_pair(meta, dev, 40, 24)
+    gpu.set_learning_rate(0.05)
+    w = gpu.get_weights()
+    state = gpu.dump_extra()
+    assert tuple(gpu.forward(torch.empty(0, 40, device="cuda")).shape) == (0, 24)
+    assert tuple(gpu.backward(torch.empty(0, 24, device="cuda")).shape) == (0, 40)
+    assert tuple(gpu.forward(torch.empty(40, 0, device="cuda"), False, True, True).shape) == (24, 0)
+    gpu.update(torch.empty(0, 40, device="cuda"), torch.empty(0, 24, device="cuda"), False)
+    assert torch.equal(gpu.get_weights(), w) and gpu.dump_extra() == state
+    x = torch.rand(3, 40, device="cuda")
+    assert tuple(gpu.forward(x).shape) == (3, 24)                 # and the tile works on as before
