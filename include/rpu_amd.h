@@ -307,7 +307,8 @@ int rpu_tile_destroy(rpu_tile_t *tile);
 
 /* Replaces RPUSimple::forward (R/rpu.cpp:508-533; GPU: C/rpucuda_pulsed.cu:646-659) as bound at
  * B/rpu_base_tiles_cuda.cpp:159-236.  x_dev is [m_batch][x_size - bias] (x_trans: [x_size - bias][m_batch]),
- * y_dev is [m_batch][d_size] (d_trans: [d_size][m_batch]).  Asynchronous on `stream`. */
+ * y_dev is [m_batch][d_size] (d_trans: [d_size][m_batch]).  Asynchronous on `stream`.  m_batch == 0 does nothing
+ * and succeeds (here and in backward, update and the indexed and grouped calls); a negative value is an error. */
 int rpu_tile_forward(rpu_tile_t *tile, const float *x_dev, float *y_dev, int m_batch, int bias,
                      int x_trans, int d_trans, int is_test, void *stream);
 
