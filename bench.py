@@ -37,6 +37,41 @@ PMC_TRAFFIC_BYTES = {
 }
 
 
+def batch_sweep() -> int:
+    """Call time against the batch on the configuration-2 tile: shows where a second workgroup per CU starts to cost
+    its full time (the per-CU operand fetch rate bounds the 32 x 32 round kernel)."""
+    import numpy as np
+    import torch
+
+    from aihwkit_amd.rpu_base import tiles
+    from helpers import config2
+
+    meta, dev = config2()
+    host = meta.create_array(1024, 1024, dev)
+    host.set_weights(torch.from_numpy(np.random.default_rng(0).uniform(-0.6, 0.6, (1024, 1024)).astype(np.float32)))
+    tile = tiles.CudaAnalogTile(host)
+    out = {"workload": "config2 tile, forward / backward call time against the batch", "unit": "us", "calls": 200,
+           "batches": {}}
+    for batch in (32, 64, 128, 256, 512, 1024, 2000):
+        x = torch.rand(batch, 1024, device="cuda") * 2 - 1
+        d = torch.randn(batch, 1024, device="cuda") * 0.1
+        entry = {}
+        for name, fn, arg in (("forward", tile.forward, x), ("backward", tile.backward, d)):
+            for _ in range(10):
+                fn(arg, non_blocking=True)
+            torch.cuda.synchronize()
+            start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            start.record()
+            for _ in range(200):
+                fn(arg, non_blocking=True)
+            stop.record()
+            torch.cuda.synchronize()
+            entry[name] = round(start.elapsed_time(stop) / 200 * 1000, 1)
+        out["batches"][str(batch)] = entry
+    print(json.dumps(out))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -48,6 +83,9 @@ def main() -> int:
     ap.add_argument("--pmc", action="store_true",
                     help="counter-collection mode for rocprofv3 --pmc: one 64 MiB calibration copy, then 3 update, "
                          "3 forward and 3 backward calls; no timing, no JSON line")
+    ap.add_argument("--batch-sweep", action="store_true",
+                    help="instead of the benchmark line: forward and backward call times of the configuration-2 tile "
+                         "at batches 32 .. 2000 (HIP events over 200 calls each), one JSON line")
     ap.add_argument("--config", type=int, default=2, choices=(1, 2, 3, 4, 5),
                     help="benchmark configuration: 2 is the graded one; 3 is the Tiki-Taka MLP of transfer tiles; "
                          "5 is the forward pass of the GPT-2-small linear layers as PCM inference tiles")
@@ -70,6 +108,8 @@ def main() -> int:
         return 1
     torch.cuda.set_device(0)
 
+    if args.batch_sweep:
+        return batch_sweep()
     if args.config == 3:
         return bench_config3(args)
     if args.config == 4:
