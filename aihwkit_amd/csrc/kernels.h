@@ -184,6 +184,8 @@ void launch_update_planes(const UpdateArgs &a, hipStream_t s);        // bit pla
 void launch_update_pulsed(const UpdateArgs &a, hipStream_t s);        // coincidences + device steps
 void launch_update_implicit(const UpdateArgs &a, hipStream_t s);
 void launch_implicit_counts(const UpdateArgs &a, int32_t *counts, hipStream_t s);
+// floating-point update with the device bounds applied after every sample (x, d, strides, lr, w, dev.w_min / w_max)
+void launch_update_fp_clipped(const UpdateArgs &a, hipStream_t s);
 // ----- weight maintenance between steps (kernels_state.hip); w_min / w_max may be null (no device bounds)
 void launch_decay_device(float *w, const float *decay_scale, const float *reset_bias, const float *w_min,
                          const float *w_max, float alpha, int bias_no_decay, int x_size, size_t n, hipStream_t s);

@@ -203,17 +203,38 @@ __global__ __launch_bounds__(256) void k_update_implicit_lines(UpdateArgs a) {
     float v = is_x ? a.x[(long)b * a.x_sb + (long)j * a.x_sj] : a.d[(long)b * a.d_sb + (long)j * a.d_si];
     if (a.lr < 0.0f) v = -v;
     const float P = is_x ? a.prob_b[b] : a.prob_a[b];
-    const float res = is_x ? a.up.x_res_implicit : a.up.d_res_implicit;
+    const bool mean_count = a.up.pulse_type == RPU_PULSE_MEAN_COUNT;
+    const float res = mean_count ? a.up.res : (is_x ? a.up.x_res_implicit : a.up.d_res_implicit);
     uint32_t sr = 0;
     if (res > 0.0f && a.up.sto_round) {
       sr = philox4x32_10((uint32_t)j, (uint32_t)b, a.call, RNG_UPDATE_SR | ((uint32_t)is_x << 8), a.key.k0, a.key.k1).v[0];
     }
     float pp = discretize_prob(fabsf(v) * P, res, a.up.sto_round, sr);
-    pp = fmaxf(fminf(pp, 1.0f), 0.0f);
-    const float val = (v >= 0.0f) ? pp : -pp;
+    float val;
+    if (mean_count) {
+      // generateCountsMean (dense_bit_line_maker.cpp:140-170): the expected number of pulses, no fluctuation; the d line
+      // stores its count over BL as generateCoincidences (:176-201) divides it
+      const int BL = a.bl[b];
+      const int ntimes = pp == 0.0f ? 0 : max(min((int)rintf((float)BL * pp), BL), 0);
+      const float count = (v >= 0.0f) ? (float)ntimes : -(float)ntimes;
+      val = (is_x || ntimes == 0) ? count : count / (float)BL;
+    } else {
+      pp = fmaxf(fminf(pp, 1.0f), 0.0f);
+      val = (v >= 0.0f) ? pp : -pp;
+    }
     if (is_x) a.x_val[(long)b * a.x_size + j] = val;
     else a.d_val[(long)b * a.d_size + j] = val;
   }
+}
+
+// signed coincidence count of cross-point (i, j) for sample b from the stored line values:
+// rintf((dv * BL) * xv) (generateCoincidencesDetI, dense_bit_line_maker.cpp:237-264), or with mean counts
+// rintf((d_count / BL) * x_count) (generateCoincidences, :176-201)
+__device__ __forceinline__ int implicit_count(const UpdateArgs &a, int b, int i, int j) {
+  float dc = a.d_val[(long)b * a.d_size + i];
+  if (dc == 0.0f) return 0;
+  if (a.up.pulse_type != RPU_PULSE_MEAN_COUNT) dc *= (float)a.bl[b];
+  return (int)rintf(dc * a.x_val[(long)b * a.x_size + j]);
 }
 
 // ---- device steps ------------------------------------------------------------------------------
@@ -597,10 +618,7 @@ __global__ __launch_bounds__(256) void k_update_implicit(UpdateArgs a) {
   rng.n0 = rng.n1 = rng.n2 = rng.n3 = 0.0f;
   const float std_ = a.dev.dw_min_std;
   for (int b = 0; b < a.m_batch; ++b) {
-    float dc = a.d_val[(long)b * a.d_size + i];
-    if (dc == 0.0f) continue;
-    dc *= (float)a.bl[b];
-    const int cn = (int)rintf(dc * a.x_val[(long)b * a.x_size + j]);
+    const int cn = implicit_count(a, b, i, j);
     if (cn == 0) continue;
     const int sign_down = cn > 0;
     for (int n = abs(cn); n > 0; --n) w = device_step<KIND, MULT>(w, sign_down, c, std_, rng, a.key, a.call);
@@ -616,13 +634,7 @@ __global__ __launch_bounds__(256) void k_implicit_counts(UpdateArgs a, int32_t *
     const long rem = idx % per;
     const int i = (int)(rem / a.x_size);
     const int j = (int)(rem % a.x_size);
-    float dc = a.d_val[(long)b * a.d_size + i];
-    int cn = 0;
-    if (dc != 0.0f) {
-      dc *= (float)a.bl[b];
-      cn = (int)rintf(dc * a.x_val[(long)b * a.x_size + j]);
-    }
-    counts[idx] = cn;
+    counts[idx] = implicit_count(a, b, i, j);
   }
 }
 
@@ -660,16 +672,31 @@ __global__ __launch_bounds__(256) void k_count_pulses_implicit(UpdateArgs a, uns
   if (j >= a.x_size) return;
   unsigned long long n_same = 0, n_diff = 0;
   for (int b = 0; b < a.m_batch; ++b) {
-    float dc = a.d_val[(long)b * a.d_size + i];
-    if (dc == 0.0f) continue;
-    dc *= (float)a.bl[b];
-    const int cn = (int)rintf(dc * a.x_val[(long)b * a.x_size + j]);
+    const int cn = implicit_count(a, b, i, j);
     if (cn > 0) n_same += (unsigned)cn;
     else n_diff += (unsigned)(-cn);
   }
   const size_t cell = (size_t)i * a.x_size + j;
   pos[cell] += n_same;
   neg[cell] += n_diff;
+}
+
+// PulseType NoneWithDevice (rpu_weight_updater.cpp:216-224): per sample the floating-point outer product
+// w_ij += (-lr d_i) x_j, then the device bounds; the clipping makes the samples a sequence, one thread per cross-point
+// walks it
+__global__ __launch_bounds__(256) void k_update_fp_clipped(UpdateArgs a) {
+  const int i = blockIdx.y;
+  const int j = blockIdx.x * blockDim.x + threadIdx.x;
+  if (j >= a.x_size) return;
+  const size_t cell = (size_t)i * a.x_size + j;
+  float w = a.w[cell];
+  const float lo = a.dev.w_min[cell], hi = a.dev.w_max[cell];
+  for (int b = 0; b < a.m_batch; ++b) {
+    const float di = -a.lr * a.d[(long)b * a.d_sb + (long)i * a.d_si]; // wave-uniform
+    w = w + di * a.x[(long)b * a.x_sb + (long)j * a.x_sj];
+    w = fmaxf(fminf(w, hi), lo);
+  }
+  a.w[cell] = w;
 }
 
 __global__ void k_clip(float *w, const float *w_min, const float *w_max, size_t n) {
@@ -752,6 +779,11 @@ void launch_count_pulses(const UpdateArgs &a, unsigned long long *pos, unsigned 
   dim3 grid((a.x_size + 255) / 256, a.d_size);
   if (implicit) hipLaunchKernelGGL(k_count_pulses_implicit, grid, dim3(256), 0, s, a, pos, neg);
   else hipLaunchKernelGGL(k_count_pulses, grid, dim3(256), 0, s, a, pos, neg);
+}
+
+void launch_update_fp_clipped(const UpdateArgs &a, hipStream_t s) {
+  dim3 grid((a.x_size + 255) / 256, a.d_size);
+  hipLaunchKernelGGL(k_update_fp_clipped, grid, dim3(256), 0, s, a);
 }
 
 void launch_implicit_counts(const UpdateArgs &a, int32_t *counts, hipStream_t s) {

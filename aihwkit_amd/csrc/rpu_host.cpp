@@ -108,15 +108,15 @@ void UpdatePar::initialize() {
   p.update_management = (p.update_management || p.update_bl_management) ? 1 : 0;
   switch (p.pulse_type) {
   case RPU_PULSE_NONE:
+  case RPU_PULSE_NONE_WITH_DEVICE:
   case RPU_PULSE_STOCHASTIC_COMPRESSED:
+  case RPU_PULSE_MEAN_COUNT:
   case RPU_PULSE_DETERMINISTIC_IMPLICIT:
     break;
-  case RPU_PULSE_NONE_WITH_DEVICE:
-    throw RpuError("PulseType NoneWithDevice is not implemented on this path.");
   default:
     throw RpuError("PulseType not supported");
   }
-  if (p.pulse_type != RPU_PULSE_NONE && (p.desired_bl < 1 || p.desired_bl > 31)) {
+  if (p.pulse_type != RPU_PULSE_NONE && p.pulse_type != RPU_PULSE_NONE_WITH_DEVICE && (p.desired_bl < 1 || p.desired_bl > 31)) {
     throw RpuError("desired_bl must be within 1..31 (one 32-bit pulse word per line).");
   }
 }

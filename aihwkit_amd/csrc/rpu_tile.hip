@@ -577,7 +577,9 @@ struct Tile {
   // W_new = W - lr * dW and the weights stay as they are (RPUPulsed::updateMatrix, rpu_pulsed.cpp:560-585;
   // RPUSimple::updateMatrix with getUpWeights / getUpBeta, rpu.cpp:624-634, 1489-1510).
   void update(const float *x, const float *d, int B, bool bias, bool x_trans, bool d_trans, hipStream_t s) {
-    const bool fp_update = !dev.pulsed() || up.p.pulse_type == RPU_PULSE_NONE;
+    // NoneWithDevice: the floating-point update, then the device bounds (rpu_weight_updater.cpp:216-224)
+    const bool with_device = up.p.pulse_type == RPU_PULSE_NONE_WITH_DEVICE;
+    const bool fp_update = !dev.pulsed() || up.p.pulse_type == RPU_PULSE_NONE || with_device;
     if (delta_w && !fp_update) {
       if (lr == 0.0f) throw RpuError("Delta weights of a pulsed update need a learning rate.");
       RPU_HIP_CHECK(hipMemcpyAsync(delta_w, d_w.p, size() * sizeof(float), hipMemcpyDeviceToDevice, s));
@@ -604,6 +606,21 @@ struct Tile {
     }
     const long d_sb = d_trans ? 1 : D, d_si = d_trans ? B : 1;
 
+    if (with_device && dev.pulsed() && !delta_w && !is_transfer()) {
+      // the bounds after every sample make the batch a sequence per cross-point
+      UpdateArgs a{};
+      a.w = d_w.p; a.x_size = X; a.d_size = D; a.m_batch = B; a.lr = lr;
+      a.x = xin; a.x_sb = x_sb; a.x_sj = x_sj; a.d = d; a.d_sb = d_sb; a.d_si = d_si;
+      a.dev.w_max = d_wmax.p; a.dev.w_min = d_wmin.p;
+      prof_begin(s);
+      launch_update_fp_clipped(a, s);
+      prof_mark(s, "update_fp_clipped");
+      RPU_HIP_CHECK(hipGetLastError());
+      last_stream = s;
+      last_update_batch = B;
+      last_update_pulse = RPU_PULSE_NONE_WITH_DEVICE;
+      return;
+    }
     if (fp_update) {
       // W += -lr * d^T x as a contraction over the batch (rpu.cpp:624-634): "weights" = d, K = batch
       MvmArgs a{};
@@ -2107,7 +2124,8 @@ int rpu_tile_get_implicit_counts(rpu_tile_t *tile, int32_t *counts_host, int m_b
     if (!tile || !counts_host) throw RpuError("null argument");
     Tile &t = tile->t;
     std::lock_guard<std::mutex> lock(t.mutex);
-    if (!t.resident() || t.last_update_pulse != RPU_PULSE_DETERMINISTIC_IMPLICIT || m_batch != t.last_update_batch) {
+    if (!t.resident() || m_batch != t.last_update_batch ||
+        (t.last_update_pulse != RPU_PULSE_DETERMINISTIC_IMPLICIT && t.last_update_pulse != RPU_PULSE_MEAN_COUNT)) {
       throw RpuError("No deterministic implicit update of this batch size has run on this tile.");
     }
     DeviceGuard g(t.device_id);
@@ -2118,6 +2136,7 @@ int rpu_tile_get_implicit_counts(rpu_tile_t *tile, int32_t *counts_host, int m_b
     UpdateArgs a{};
     a.x_size = t.X; a.d_size = t.D; a.m_batch = m_batch;
     a.bl = t.u_bl.p; a.x_val = t.u_xval.p; a.d_val = t.u_dval.p;
+    a.up.pulse_type = t.last_update_pulse;
     try {
       launch_implicit_counts(a, tmp.p, t.last_stream);
       RPU_HIP_CHECK(hipStreamSynchronize(t.last_stream));

@@ -839,6 +839,56 @@ void generate_coincidences_det(int *coinc, const float *xv, int X, const float *
   }
 }
 
+// R/dense_bit_line_maker.cpp:140-170 generateCountsMean: the expected number of pulses of a line, signed
+void generate_counts_mean(OrcTile &t, int *counts, const float *v, int v_inc, int v_size, float p, int BL, float lr) {
+  for (int j = 0; j < v_size; ++j) {
+    const float value = lr < 0.0f ? -v[(size_t)j * v_inc] : v[(size_t)j * v_inc];
+    const float pp = discretize(fabsf(value) * p, t.up.res, t.up.sto_round != 0, t.rng);
+    if (pp == 0.0f) {
+      counts[j] = 0;
+      continue;
+    }
+    const int ntimes = std::max(std::min((int)rintf((float)BL * pp), BL), 0);
+    counts[j] = (value >= 0.0f) ? ntimes : -ntimes;
+  }
+}
+
+// R/dense_bit_line_maker.cpp:176-201 generateCoincidences
+void generate_coincidences_mean(int *coinc, const int *xc, int X, const int *dcnt, int D, int BL) {
+  const float bl = (float)BL;
+  size_t idx = 0;
+  for (int i = 0; i < D; ++i) {
+    float dc = (float)dcnt[i];
+    if (dc != 0.0f) {
+      dc /= bl;
+      for (int j = 0; j < X; ++j) coinc[idx++] = (int)rintf(dc * (float)xc[j]);
+    } else {
+      for (int j = 0; j < X; ++j) coinc[idx++] = 0;
+    }
+  }
+}
+
+// the coincidences of one sample for either dense scheme (makeCoincidences, R/dense_bit_line_maker.cpp:267-331)
+bool dense_coincidences(OrcTile &t, const float *x, int x_inc, const float *d, int d_inc, float lr, int *coinc) {
+  const int X = t.X, D = t.D;
+  int BL;
+  float A, B;
+  if (!sample_bl_ab(t, x, x_inc, d, d_inc, fabsf(lr), BL, A, B)) return false;
+  if (t.up.pulse_type == RPU_PULSE_MEAN_COUNT) {
+    std::vector<int> xc((size_t)X), dcnt((size_t)D);
+    generate_counts_mean(t, xc.data(), x, x_inc, X, B, BL, lr);
+    generate_counts_mean(t, dcnt.data(), d, d_inc, D, A, BL, lr);
+    generate_coincidences_mean(coinc, xc.data(), X, dcnt.data(), D, BL);
+    return true;
+  }
+  t.xv.resize(X);
+  t.dv.resize(D);
+  generate_det_implicit(t, t.xv.data(), x, x_inc, X, B, t.up.x_res_implicit, lr);
+  generate_det_implicit(t, t.dv.data(), d, d_inc, D, A, t.up.d_res_implicit, lr);
+  generate_coincidences_det(coinc, t.xv.data(), X, t.dv.data(), D, BL);
+  return true;
+}
+
 // R/rpu_pulsed_device.h:461-474 PULSED_UPDATE_W_LOOP_DENSE
 void dense_update(OrcTile &t, const int *coinc) {
   const size_t total = (size_t)t.X * t.D;
@@ -856,12 +906,19 @@ bool update_vector(OrcTile &t, const float *x, int x_inc, const float *d, int d_
   const float lr = t.lr; // R/rpu.cpp:1400-1403 getAlphaLearningRate with bwd_alpha = 1
   if (!lr) return true;
   const int X = t.X, D = t.D;
-  if (!is_pulsed_device(t) || t.up.pulse_type == RPU_PULSE_NONE) {
+  if (!is_pulsed_device(t) || t.up.pulse_type == RPU_PULSE_NONE || t.up.pulse_type == RPU_PULSE_NONE_WITH_DEVICE) {
     // R/rpu.cpp:706-714 RPUSimple::updateVector: W += -lr * d x^T
     for (int i = 0; i < D; ++i) {
       const float di = -lr * d[(size_t)i * d_inc];
       float *row = t.w.data() + (size_t)i * X;
       for (int j = 0; j < X; ++j) row[j] += di * x[(size_t)j * x_inc];
+    }
+    if (is_pulsed_device(t) && t.up.pulse_type == RPU_PULSE_NONE_WITH_DEVICE) {
+      // R/rpu_weight_updater.cpp:220-222 clipWeights(weights, -1): the device bounds only
+      for (size_t k = 0; k < t.w.size(); ++k) {
+        t.w[k] = std::min(t.w[k], t.w_max[k]);
+        t.w[k] = std::max(t.w[k], t.w_min[k]);
+      }
     }
     return true;
   }
@@ -876,14 +933,9 @@ bool update_vector(OrcTile &t, const float *x, int x_inc, const float *d, int d_
     sparse_update(t, BL, lr < 0.0f ? -1 : 1);
     return true;
   }
-  if (t.up.pulse_type == RPU_PULSE_DETERMINISTIC_IMPLICIT) {
-    if (!sample_bl_ab(t, x, x_inc, d, d_inc, fabsf(lr), BL, A, B)) return false;
-    t.xv.resize(X);
-    t.dv.resize(D);
+  if (t.up.pulse_type == RPU_PULSE_DETERMINISTIC_IMPLICIT || t.up.pulse_type == RPU_PULSE_MEAN_COUNT) {
     t.coinc.resize((size_t)X * D);
-    generate_det_implicit(t, t.xv.data(), x, x_inc, X, B, t.up.x_res_implicit, lr);
-    generate_det_implicit(t, t.dv.data(), d, d_inc, D, A, t.up.d_res_implicit, lr);
-    generate_coincidences_det(t.coinc.data(), t.xv.data(), X, t.dv.data(), D, BL);
+    if (!dense_coincidences(t, x, x_inc, d, d_inc, lr, t.coinc.data())) return false;
     dense_update(t, t.coinc.data());
     return true;
   }
@@ -1123,15 +1175,8 @@ int orc_update_bl_ab(void *h, const float *x, const float *d, int m_batch, int32
 int orc_implicit_counts(void *h, const float *x, const float *d, int m_batch, int32_t *counts) {
   auto *t = static_cast<OrcTile *>(h);
   const int X = t->X, D = t->D;
-  t->xv.resize(X);
-  t->dv.resize(D);
   for (int b = 0; b < m_batch; ++b) {
-    int BL;
-    float A, B;
-    if (!sample_bl_ab(*t, x + (size_t)b * X, 1, d + (size_t)b * D, 1, fabsf(t->lr), BL, A, B)) return 1;
-    generate_det_implicit(*t, t->xv.data(), x + (size_t)b * X, 1, X, B, t->up.x_res_implicit, t->lr);
-    generate_det_implicit(*t, t->dv.data(), d + (size_t)b * D, 1, D, A, t->up.d_res_implicit, t->lr);
-    generate_coincidences_det(counts + (size_t)b * X * D, t->xv.data(), X, t->dv.data(), D, BL);
+    if (!dense_coincidences(*t, x + (size_t)b * X, 1, d + (size_t)b * D, 1, t->lr, counts + (size_t)b * X * D)) return 1;
   }
   return 0;
 }

@@ -524,3 +524,37 @@ def test_empty_batches_do_nothing(gpu_device):
     assert torch.equal(gpu.get_weights(), w) and gpu.dump_extra() == state
     x = torch.rand(3, 40, device="cuda")
     assert tuple(gpu.forward(x).shape) == (3, 24)                 # and the tile works on as before
+
+
+def test_none_with_device_update_is_the_outer_product_inside_the_bounds(gpu_device):
+    """PulseType NoneWithDevice: per sample the floating-point outer product, then the device bounds (no pulses, no step
+    sizes).  The clipping after every sample makes the result depend on the order of the batch."""
+    rng = np.random.default_rng(21)
+    for x_size, d_size, batch, bias, trans in ((70, 45, 9, False, False), (257, 33, 40, True, True), (1, 1, 3, False, False)):
+        meta = make_meta(noise_free_io(), noise_free_io(), pulse_type=dv.PulseType.NoneWithDevice)
+        dev = soft_bounds(construction_seed=3)
+        host, orc, _ = build_pair(meta, dev, x_size, d_size, gpu=False)
+        w = rng.uniform(-0.3, 0.3, (d_size, x_size)).astype(np.float32)
+        host.set_weights(torch.from_numpy(w))
+        orc.set_weights(host.get_weights().numpy())
+        gpu = tiles.CudaAnalogTile(host)
+        xs = x_size - int(bias)
+        x = rng.uniform(-1, 1, (xs, batch) if trans else (batch, xs)).astype(np.float32)
+        d = rng.normal(0, 0.5, (d_size, batch) if trans else (batch, d_size)).astype(np.float32)
+        hidden = gpu.get_hidden_parameters().numpy()
+        for lr in (1.0, -0.5):
+            gpu.set_learning_rate(lr)
+            orc.set_learning_rate(lr)
+            before = gpu.get_weights().numpy()
+            gpu.update(cuda(x), cuda(d), bias, trans, trans)
+            orc.update(x, d, bias, trans, trans)
+            got = gpu.get_weights().numpy()
+            assert np.array_equal(got, orc.get_weights())            # the same float operations in the same order
+            assert (got <= hidden[0]).all() and (got >= hidden[1]).all()
+            if x_size > 1:
+                at_bound = (got == hidden[0]) | (got == hidden[1])
+                assert 0.01 < at_bound.mean() < 0.9
+                xb = (x.T if trans else x)
+                xb = np.concatenate([xb, np.ones((batch, 1), np.float32)], 1) if bias else xb
+                once = np.clip(before - lr * (d if trans else d.T) @ xb, hidden[1], hidden[0])
+                assert np.abs(got - once).max() > 1e-3                # clipping once at the end is not the same thing

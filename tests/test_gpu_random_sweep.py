@@ -191,8 +191,9 @@ def one_implicit(seed):
         for k, v in dict(gamma_up=0.4, gamma_down=0.2, gamma_up_dtod=0.05, gamma_down_dtod=0.05,
                          mult_noise=bool(rng.integers(2)), **kw).items():
             setattr(dev, k, v)
-    meta = make_meta(desired_bl=bl, pulse_type=dv.PulseType.DeterministicImplicit, update_management=um,
-                     update_bl_management=um,
+    pulse_type = [dv.PulseType.DeterministicImplicit, dv.PulseType.MeanCount][rng.integers(2)]
+    meta = make_meta(desired_bl=bl, pulse_type=pulse_type, update_management=um,
+                     update_bl_management=um, res=float(rng.choice([0.0, 1 / 16.0])),
                      x_res_implicit=float(rng.choice([0.0, 1 / 20.0])), d_res_implicit=float(rng.choice([0.0, 1 / 30.0])))
     host, orc, _ = build_pair(meta, dev, x_size, d_size, gpu=False)
     w = rng.uniform(-0.4, 0.4, (d_size, x_size)).astype(np.float32)
@@ -206,10 +207,14 @@ def one_implicit(seed):
     x = rng.uniform(-1, 1, (xs, batch) if x_trans else (batch, xs)).astype(np.float32)
     d = (0.3 * rng.standard_normal((d_size, batch) if d_trans else (batch, d_size))).astype(np.float32)
     gpu.update(cuda(x), cuda(d), bias, x_trans, d_trans, False)
+    counts_ok = True
+    if not bias and not x_trans and not d_trans:
+        counts_ok = np.array_equal(gpu.get_implicit_counts(batch).numpy(), orc.implicit_counts(x, d))
     orc.update(x, d, bias, x_trans, d_trans)
     diff = np.abs(gpu.get_weights().numpy() - orc.get_weights()).max()
-    return diff <= 2e-5, dict(seed=seed, X=x_size, D=d_size, B=batch, bias=bias, xt=x_trans, dt=d_trans, bl=bl, um=um,
-                              kind=kind, lr=lr, diff=float(diff))
+    return diff <= 2e-5 and counts_ok, dict(seed=seed, X=x_size, D=d_size, B=batch, bias=bias, xt=x_trans, dt=d_trans, bl=bl,
+                                            um=um, kind=kind, lr=lr, pulse=str(pulse_type), diff=float(diff),
+                                            counts_ok=counts_ok)
 
 def one_fp(seed):
     rng = np.random.default_rng(seed)
@@ -242,7 +247,8 @@ def one_fp(seed):
 
 
 def test_random_implicit_update_cases_follow_the_oracle(gpu_device):
-    """Deterministic implicit pulses over layouts, bias column, three devices, update management, learning-rate sign."""
+    """Deterministic implicit pulses and mean counts over layouts, bias column, three devices, update management,
+    learning-rate sign: coincidence counts bit-exact, weights to 2e-5."""
     failures = [desc for ok, desc in (one_implicit(seed) for seed in range(20000, 20150)) if not ok]
     assert not failures, failures[:3]
 

@@ -118,3 +118,39 @@ def test_running_average_noise_management_closed_form():
     low = np.zeros((1, n), dtype=F)
     low[0, 2] = 0.01
     np.testing.assert_allclose(fresh.forward(low)[0, 2], 0.01, rtol=1e-5)
+
+
+def test_mean_count_and_none_with_device_updates_closed_form():
+    """MeanCount: every line gets round(BL p) pulses, a cross-point round(d_count / BL * x_count) steps of dw_min (no
+    variation here); NoneWithDevice: the floating-point outer product, then the device bounds."""
+    from oracle_lib import OracleTile
+
+    dev = constant_step(dw_min=0.01, dw_min_dtod=0.0, dw_min_std=0.0, up_down_dtod=0.0, w_max=0.3, w_min=-0.3, w_max_dtod=0.0,
+                        w_min_dtod=0.0, construction_seed=1)
+    meta = make_meta(pulse_type=dv.PulseType.MeanCount, desired_bl=10, update_management=False, update_bl_management=False,
+                     fixed_bl=True)
+    tile = OracleTile(3, 2, meta._config(dev))
+    tile.set_weights(np.zeros((2, 3), dtype=F))
+    tile.set_learning_rate(0.1)
+    # lr / (dw_min BL) = 1: A = B = 1, so p = |value|; counts round(10 p): x -> 10, 5, 0(-), d -> 8, -4 (round half even)
+    x = np.array([[1.0, 0.5, -0.04]], dtype=F)
+    d = np.array([[0.8, -0.35]], dtype=F)
+    counts = tile.implicit_counts(x, d)[0]
+    # rintf(d_count / 10 * x_count): [8, 4, 0] and [-4, -2, 0]
+    np.testing.assert_array_equal(counts, [[8, 4, 0], [-4, -2, 0]])
+    tile.update(x, d)
+    np.testing.assert_allclose(tile.get_weights(), [[-0.08, -0.04, 0.0], [0.04, 0.02, 0.0]], atol=1e-7)   # w -= lr d x^T
+    x2 = np.array([[0.25, -1.0, 0.0]], dtype=F)                   # 2.5 rounds to 2 (half to even), negative input
+    np.testing.assert_array_equal(tile.implicit_counts(x2, d)[0], [[2, -8, 0], [-1, 4, 0]])
+    # NoneWithDevice
+    meta = make_meta(pulse_type=dv.PulseType.NoneWithDevice)
+    tile = OracleTile(3, 2, meta._config(dev))
+    w0 = np.array([[0.25, 0.0, -0.29], [0.0, 0.1, 0.2]], dtype=F)
+    tile.set_weights(w0)
+    tile.set_learning_rate(0.5)
+    xs = np.array([[1.0, 0.5, -1.0], [0.5, 0.0, 1.0]], dtype=F)
+    ds = np.array([[-0.4, 0.2], [0.1, -0.3]], dtype=F)
+    tile.update(xs, ds)
+    want = np.clip(np.clip(w0 - 0.5 * np.outer(ds[0], xs[0]), -0.3, 0.3) - 0.5 * np.outer(ds[1], xs[1]), -0.3, 0.3)
+    np.testing.assert_allclose(tile.get_weights(), want, atol=1e-6)
+    assert (np.abs(w0 - 0.5 * ds.T @ xs) > 0.3).any()             # the example does reach the bounds
