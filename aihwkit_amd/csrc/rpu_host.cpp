@@ -106,6 +106,10 @@ void IOPar::initialize(bool backward) {
 
 void UpdatePar::initialize() {
   p.update_management = (p.update_management || p.update_bl_management) ? 1 : 0;
+  // Stochastic keeps the pulse trains of positive and negative inputs in separate lists
+  // (sparse_bit_line_maker.cpp:145-196, 323-333); every cross-point sees the same pulses in the same order as with the
+  // compressed lists, so the two types are one on this path
+  if (p.pulse_type == RPU_PULSE_STOCHASTIC) p.pulse_type = RPU_PULSE_STOCHASTIC_COMPRESSED;
   switch (p.pulse_type) {
   case RPU_PULSE_NONE:
   case RPU_PULSE_NONE_WITH_DEVICE:

@@ -61,7 +61,7 @@ enum rpu_bound_management {
 enum rpu_pulse_type {
   RPU_PULSE_NONE = 0,                  /* floating point rank-B update */
   RPU_PULSE_STOCHASTIC_COMPRESSED = 1,
-  RPU_PULSE_STOCHASTIC = 2,            /* not provided (CPU-only in the reference too) */
+  RPU_PULSE_STOCHASTIC = 2,            /* treated as STOCHASTIC_COMPRESSED: the same pulses per cross-point */
   RPU_PULSE_NONE_WITH_DEVICE = 3,      /* floating point update, device bounds after every sample */
   RPU_PULSE_MEAN_COUNT = 4,            /* deterministic counts round(BL p) per line (R/dense_bit_line_maker.cpp:140-208) */
   RPU_PULSE_DETERMINISTIC_IMPLICIT = 5

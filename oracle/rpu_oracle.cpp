@@ -924,7 +924,9 @@ bool update_vector(OrcTile &t, const float *x, int x_inc, const float *d, int d_
   }
   int BL;
   float A, B;
-  if (t.up.pulse_type == RPU_PULSE_STOCHASTIC_COMPRESSED) {
+  // Stochastic differs from StochasticCompressed only in keeping positive and negative x in separate lists
+  // (R/sparse_bit_line_maker.cpp:145-196): per cross-point the same pulses in the same order
+  if (t.up.pulse_type == RPU_PULSE_STOCHASTIC_COMPRESSED || t.up.pulse_type == RPU_PULSE_STOCHASTIC) {
     if (!sample_bl_ab(t, x, x_inc, d, d_inc, lr < 0.0f ? -lr : lr, BL, A, B)) return false;
     if (BL == 0) return true;
     ensure_sparse_containers(t);

@@ -117,7 +117,8 @@ def test_unsupported_parameters_fail_loudly():
     with pytest.raises(RuntimeError, match="desired_bl"):
         make_meta(desired_bl=255).create_array(4, 4, dev)
     with pytest.raises(RuntimeError, match="not supported"):
-        make_meta(pulse_type=dv.PulseType.Stochastic).create_array(4, 4, dev)
+        make_meta(pulse_type=17).create_array(4, 4, dev)
+    make_meta(pulse_type=dv.PulseType.Stochastic).create_array(4, 4, dev)
     make_meta(pulse_type=dv.PulseType.MeanCount).create_array(4, 4, dev)
     make_meta(pulse_type=dv.PulseType.NoneWithDevice).create_array(4, 4, dev)
     bad = soft_bounds()

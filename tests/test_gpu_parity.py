@@ -558,3 +558,20 @@ def test_none_with_device_update_is_the_outer_product_inside_the_bounds(gpu_devi
                 xb = np.concatenate([xb, np.ones((batch, 1), np.float32)], 1) if bias else xb
                 once = np.clip(before - lr * (d if trans else d.T) @ xb, hidden[1], hidden[0])
                 assert np.abs(got - once).max() > 1e-3                # clipping once at the end is not the same thing
+
+
+def test_stochastic_pulse_type_is_the_compressed_one(gpu_device):
+    """PulseType Stochastic (separate lists for positive and negative inputs in the reference's CPU code) gives every
+    cross-point the pulses of StochasticCompressed: same seed, same weights."""
+    rng = np.random.default_rng(4)
+    x = rng.uniform(-1, 1, (20, 50)).astype(np.float32)
+    d = rng.normal(0, 0.3, (20, 30)).astype(np.float32)
+    results = []
+    for pulse_type in (dv.PulseType.Stochastic, dv.PulseType.StochasticCompressed):
+        meta = make_meta(noise_free_io(), noise_free_io(), pulse_type=pulse_type, desired_bl=31)
+        host, _orc, gpu = build_pair(meta, soft_bounds(construction_seed=2), 50, 30)
+        gpu.set_learning_rate(0.05)
+        gpu.set_seed(77)
+        gpu.update(cuda(x), cuda(d), False)
+        results.append(gpu.get_weights())
+    assert torch.equal(results[0], results[1]) and not torch.equal(results[0], torch.zeros_like(results[0]))
