@@ -60,6 +60,7 @@ class DeviceParams(C.Structure):
         ("drift_nu", f32), ("drift_nu_dtod", f32), ("drift_nu_std", f32), ("drift_wg_ratio", f32),
         ("drift_g_offset", f32), ("drift_w_offset", f32), ("drift_nu_k", f32), ("drift_log_g0", f32),
         ("drift_t0", f32), ("drift_reset_tol", f32), ("drift_w_read_std", f32), ("count_pulses", i32),
+        ("apply_write_noise_on_set", i32),
     ]
 
 

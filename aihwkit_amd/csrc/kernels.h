@@ -184,6 +184,13 @@ void launch_update_planes(const UpdateArgs &a, hipStream_t s);        // bit pla
 void launch_update_pulsed(const UpdateArgs &a, hipStream_t s);        // coincidences + device steps
 void launch_update_implicit(const UpdateArgs &a, hipStream_t s);
 void launch_implicit_counts(const UpdateArgs &a, int32_t *counts, hipStream_t s);
+// after an update of the persistent weights: w_apparent = w_persistent + noise_std * N(0, 1) at every cross-point that
+// took a pulse (from the planes / line values of that update)
+void launch_write_noise_touched(const UpdateArgs &a, float *w_apparent, const float *w_persistent, float noise_std,
+                                bool implicit, hipStream_t s);
+// the same at every cross-point (after weight maintenance and set_weights)
+void launch_write_noise_all(float *w_apparent, const float *w_persistent, float noise_std, PhiloxKey key, uint32_t call,
+                            size_t n, hipStream_t s);
 // floating-point update with the device bounds applied after every sample (x, d, strides, lr, w, dev.w_min / w_max)
 void launch_update_fp_clipped(const UpdateArgs &a, hipStream_t s);
 // ----- weight maintenance between steps (kernels_state.hip); w_min / w_max may be null (no device bounds)

@@ -160,6 +160,22 @@ __global__ __launch_bounds__(256) void k_reset_cols(float *w, const float *reset
   }
 }
 
+// PulsedRPUDevice::applyUpdateWriteNoise (rpu_pulsed_device.cpp:573-588): every shown weight is its persistent one
+// plus fresh noise; four elements per thread
+__global__ __launch_bounds__(256) void k_write_noise_all(float *w_apparent, const float *w_persistent, float noise_std,
+                                                          PhiloxKey key, uint32_t call, size_t n) {
+  const size_t quads = (n + 3) / 4;
+  for (size_t q = blockIdx.x * (size_t)blockDim.x + threadIdx.x; q < quads; q += (size_t)gridDim.x * blockDim.x) {
+    float z[4];
+    philox_normal4((uint32_t)q, (uint32_t)(q >> 32), call, RNG_WRITE_NOISE | (1u << 8), key, z);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const size_t i = 4 * q + e;
+      if (i < n) w_apparent[i] = w_persistent[i] + noise_std * z[e];
+    }
+  }
+}
+
 // RPUSimple::getAndResetWeightUpdate (rpu.cpp:1432-1442)
 __global__ __launch_bounds__(256) void k_delta_finish(float *w, float *prev_w_and_delta, float scale, size_t n) {
   for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
@@ -440,6 +456,12 @@ void launch_remap(float *w, float *scales, float *row_stat, float *mul, float *d
 void launch_modify(float *out, const float *w, const ModifierDev &p, const float *amax_dev, PhiloxKey key, uint32_t call,
                    int x_size, size_t n, hipStream_t s) {
   hipLaunchKernelGGL(k_modify, dim3(grid_for(n)), dim3(256), 0, s, out, w, p, amax_dev, key, call, x_size, n);
+}
+
+void launch_write_noise_all(float *w_apparent, const float *w_persistent, float noise_std, PhiloxKey key, uint32_t call,
+                            size_t n, hipStream_t s) {
+  hipLaunchKernelGGL(k_write_noise_all, dim3(grid_for((n + 3) / 4)), dim3(256), 0, s, w_apparent, w_persistent, noise_std,
+                     key, call, n);
 }
 
 void launch_delta_finish(float *w, float *prev_w_and_delta, float scale, size_t n, hipStream_t s) {

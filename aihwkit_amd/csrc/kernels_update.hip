@@ -681,6 +681,39 @@ __global__ __launch_bounds__(256) void k_count_pulses_implicit(UpdateArgs a, uns
   neg[cell] += n_diff;
 }
 
+// Write noise (rpu_linearstep_device.cpp:112-164): the pulses act on the persistent weights; a cross-point that took at
+// least one pulse in this update shows its persistent weight plus fresh noise, the others keep what they showed.
+// Runs after the update kernel, on the same bit planes (or line values): one thread per cross-point.
+__global__ __launch_bounds__(256) void k_write_noise_touched(UpdateArgs a, float *w_apparent, const float *w_persistent,
+                                                              float noise_std, int implicit) {
+  const int i = blockIdx.y;
+  const int j = blockIdx.x * blockDim.x + threadIdx.x;
+  if (j >= a.x_size) return;
+  bool touched = false;
+  if (implicit) {
+    for (int b = 0; b < a.m_batch && !touched; ++b) touched = implicit_count(a, b, i, j) != 0;
+  } else {
+    const int kmax = a.kmax[a.kmax_slot];
+    const unsigned xs = (unsigned)a.x_size, ds = (unsigned)a.d_size, slots = (unsigned)a.plane_slots;
+    const uint32_t *xpl = a.x_planes + j;
+    const uint32_t *dpl = a.d_planes + i;
+    uint32_t any = 0u;
+    for (int c = 0; c < a.n_chunks; ++c) {
+      const unsigned base = (unsigned)c * slots;
+      for (int k = 0; k < kmax; ++k) {
+        const uint32_t dk = dpl[(base + k) * ds]; // wave-uniform
+        if (dk) any |= dk & xpl[(base + k) * xs];
+      }
+    }
+    touched = any != 0u;
+  }
+  if (!touched) return;
+  const size_t cell = (size_t)i * a.x_size + j;
+  float z[4];
+  philox_normal4((uint32_t)cell, (uint32_t)(cell >> 32), a.call, RNG_WRITE_NOISE, a.key, z);
+  w_apparent[cell] = w_persistent[cell] + noise_std * z[0];
+}
+
 // PulseType NoneWithDevice (rpu_weight_updater.cpp:216-224): per sample the floating-point outer product
 // w_ij += (-lr d_i) x_j, then the device bounds; the clipping makes the samples a sequence, one thread per cross-point
 // walks it
@@ -779,6 +812,12 @@ void launch_count_pulses(const UpdateArgs &a, unsigned long long *pos, unsigned 
   dim3 grid((a.x_size + 255) / 256, a.d_size);
   if (implicit) hipLaunchKernelGGL(k_count_pulses_implicit, grid, dim3(256), 0, s, a, pos, neg);
   else hipLaunchKernelGGL(k_count_pulses, grid, dim3(256), 0, s, a, pos, neg);
+}
+
+void launch_write_noise_touched(const UpdateArgs &a, float *w_apparent, const float *w_persistent, float noise_std,
+                                bool implicit, hipStream_t s) {
+  dim3 grid((a.x_size + 255) / 256, a.d_size);
+  hipLaunchKernelGGL(k_write_noise_touched, grid, dim3(256), 0, s, a, w_apparent, w_persistent, noise_std, implicit ? 1 : 0);
 }
 
 void launch_update_fp_clipped(const UpdateArgs &a, hipStream_t s) {

@@ -72,7 +72,8 @@ enum RngPurpose : uint32_t {
   RNG_RESET = 12,      // column reset (noise, and with round 1 the reset lottery)
   RNG_DEVICE_DRIFT = 13, // power-law drift of a training tile: nu variation and read noise
   RNG_MODIFIER = 14,     // weight modifier: noise, stochastic rounding, drop connections
-  RNG_W_NOISE = 15       // output-referred weight noise of the analog MVM
+  RNG_W_NOISE = 15,      // output-referred weight noise of the analog MVM
+  RNG_WRITE_NOISE = 16   // write noise on the shown weights (round 0: after an update, 1: refresh of all)
 };
 
 // uniform in [0, 1) with 24 bits

@@ -139,8 +139,8 @@ void DevicePar::initialize() {
     p.ls_mean_bound_reference = 0;
   }
   if (pulsed()) {
-    if (p.write_noise_std > 0.0f) {
-      throw RpuError("write_noise_std > 0 (persistent weights) is not implemented on this path.");
+    if (p.write_noise_std > 0.0f && !linear()) {
+      throw RpuError("Device does not support write noise"); // rpu_pulsed_device.h:107-111
     }
     if (p.w_min > 0.0f || p.w_max < 0.0f) {
       throw RpuError("The closed interval [w_min,w_max] needs to contain 0.");
@@ -322,6 +322,7 @@ void TransferPar::initialize(int x_size, int d_size) {
     d.p = k == 0 ? p.fast_device : p.rest_device;
     d.initialize();
     if (!d.pulsed()) throw RpuError("The devices of a transfer chain must be pulsed devices.");
+    if (d.persistent_weights()) throw RpuError("write_noise_std > 0 is not provided for the devices of a transfer chain.");
     devs.push_back(d);
   }
   in_size = p.transfer_columns ? x_size : d_size;
@@ -451,6 +452,7 @@ void fill_default_config(rpu_tile_config *cfg, int device_kind) {
   d.reset_dtod = 0.0f;
   d.reset_std = 0.01f;
   d.write_noise_std = 0.0f;
+  d.apply_write_noise_on_set = 1;
   d.ls_allow_increasing_slope = 0;
   d.ls_mean_bound_reference = 1;
   d.ls_mult_noise = 1;

@@ -33,6 +33,7 @@ struct DeviceArrays {
   std::vector<float> w_max, w_min, scale_up, scale_down, decay_scale, diffusion_rate, reset_bias;
   std::vector<float> slope_up, slope_down; // LinearStep / SoftBounds only
   std::vector<float> drift_nu;             // only with drift_nu > 0 in the parameters
+  std::vector<float> persistent;           // persistent weights, only with write_noise_std > 0
 };
 
 struct DevicePar {
@@ -40,6 +41,8 @@ struct DevicePar {
   void initialize();
   bool pulsed() const { return p.kind != RPU_DEVICE_IDEAL; }
   bool linear() const { return p.kind == RPU_DEVICE_LINEAR_STEP || p.kind == RPU_DEVICE_SOFT_BOUNDS; }
+  bool persistent_weights() const { return linear() && p.write_noise_std > 0.0f; } // usesPersistentWeight
+  float scaled_write_noise() const { return p.write_noise_std * p.dw_min; }        // getScaledWriteNoise
   float weight_granularity() const { return p.dw_min; }
   // rpu_pulsed_device.cpp:593-733 and rpu_linearstep_device.cpp:20-74
   void populate(int x_size, int d_size, DeviceArrays &out) const;

@@ -13,6 +13,7 @@
 #include <cstring>
 #include <memory>
 #include <mutex>
+#include <random>
 #include <string>
 #include <vector>
 
@@ -185,6 +186,8 @@ struct Tile {
   // pulse counters [2][size]
   DevBuf<float> d_fbw, s_rowstat;
   bool fb_during_test = false;
+  // write noise: the persistent weights the pulses and the maintenance act on; d_w then holds the shown weights
+  DevBuf<float> d_wp;
   // analog non-idealities before the ADC: the addend per output, up to three side contractions, the transformed
   // input rows, |W| and the squared row norms
   DevBuf<float> n_pre, n_s1, n_s2, n_s3, n_rows, n_absw, n_sumsq;
@@ -227,6 +230,15 @@ struct Tile {
   bool is_transfer() const { return tr != nullptr; }
   // the matrix forward / backward contract with
   float *wdev() { return (tr && tr->fully_hidden) ? slots.back()->d_w.p : d_w.p; }
+  bool persistent() const { return !tr && dev.persistent_weights(); }
+  // the matrix that pulses and weight maintenance change
+  float *wp_dev() { return persistent() ? d_wp.p : d_w.p; }
+  // PulsedRPUDevice::applyUpdateWriteNoise (rpu_pulsed_device.cpp:573-588): all shown weights are redrawn
+  void refresh_shown_weights(hipStream_t s) {
+    if (!persistent()) return;
+    launch_write_noise_all(d_w.p, d_wp.p, dev.scaled_write_noise(), key(), call++, size(), s);
+  }
+
   // RPUSimple::getFBWeights (rpu.cpp:1483-1487): once modified weights exist, forward and backward use them,
   // during evaluation only if the modifier asked for it
   const float *mvm_weights(bool is_test) {
@@ -263,6 +275,7 @@ struct Tile {
     n_pre.release(); n_s1.release(); n_s2.release(); n_s3.release(); n_rows.release(); n_absw.release();
     n_sumsq.release();
     nm_aux.release();
+    d_wp.release();
     d_fbw.release(); s_rowstat.release(); dr_prev.release(); dr_w0.release(); dr_t.release(); d_nu.release();
     d_cnt.release();
     fb_during_test = false;
@@ -336,6 +349,11 @@ struct Tile {
       } else {
         d_w.ensure(size());
         RPU_HIP_CHECK(hipMemcpy(d_w.p, w_host.data(), size() * sizeof(float), hipMemcpyHostToDevice));
+        if (persistent()) {
+          if (arr.persistent.size() != size()) arr.persistent = w_host;
+          d_wp.ensure(size());
+          RPU_HIP_CHECK(hipMemcpy(d_wp.p, arr.persistent.data(), size() * sizeof(float), hipMemcpyHostToDevice));
+        }
         upload_params();
       }
       s_count.ensure(64);
@@ -554,7 +572,7 @@ struct Tile {
     if (is_transfer()) throw RpuError("update_with_words is not provided for a transfer compound.");
     if (!dev.pulsed()) throw RpuError("update_with_words needs a pulsed device.");
     UpdateArgs a{};
-    a.w = d_w.p; a.x_size = X; a.d_size = D; a.m_batch = B; a.lr = lr;
+    a.w = wp_dev(); a.x_size = X; a.d_size = D; a.m_batch = B; a.lr = lr;
     a.dev.kind = dev.p.kind; a.dev.ls_mult_noise = dev.p.ls_mult_noise; a.dev.dw_min = dev.p.dw_min;
     a.dev.dw_min_std = dev.p.dw_min_std;
     a.dev.w_max = d_wmax.p; a.dev.w_min = d_wmin.p; a.dev.scale_up = d_sup.p; a.dev.scale_down = d_sdown.p;
@@ -569,6 +587,7 @@ struct Tile {
     if (dev.p.count_pulses) count_pulses(a, false, s);
     launch_update_pulsed(a, s);
     prof_mark(s, "update_pulsed");
+    if (persistent()) launch_write_noise_touched(a, d_w.p, d_wp.p, dev.scaled_write_noise(), false, s);
     RPU_HIP_CHECK(hipGetLastError());
     last_stream = s;
   }
@@ -609,12 +628,13 @@ struct Tile {
     if (with_device && dev.pulsed() && !delta_w && !is_transfer()) {
       // the bounds after every sample make the batch a sequence per cross-point
       UpdateArgs a{};
-      a.w = d_w.p; a.x_size = X; a.d_size = D; a.m_batch = B; a.lr = lr;
+      a.w = wp_dev(); a.x_size = X; a.d_size = D; a.m_batch = B; a.lr = lr;
       a.x = xin; a.x_sb = x_sb; a.x_sj = x_sj; a.d = d; a.d_sb = d_sb; a.d_si = d_si;
       a.dev.w_max = d_wmax.p; a.dev.w_min = d_wmin.p;
       prof_begin(s);
       launch_update_fp_clipped(a, s);
       prof_mark(s, "update_fp_clipped");
+      refresh_shown_weights(s); // clipWeights ends with applyUpdateWriteNoise (rpu_pulsed_device.cpp:448-467)
       RPU_HIP_CHECK(hipGetLastError());
       last_stream = s;
       last_update_batch = B;
@@ -651,7 +671,8 @@ struct Tile {
       transfer_update(xin, x_sb, x_sj, d, d_sb, d_si, B, s);
       return;
     }
-    DeviceView dv{d_w.p, d_wmax.p, d_wmin.p, d_sup.p, d_sdown.p, d_slup.p, d_sldown.p, &dev, dev.p.dw_min};
+    if (persistent() && delta_w) throw RpuError("Delta weights are not provided for a device with write noise.");
+    DeviceView dv{wp_dev(), d_wmax.p, d_wmin.p, d_sup.p, d_sdown.p, d_slup.p, d_sldown.p, &dev, dev.p.dw_min};
     pulsed_update_on(dv, up, lr, xin, x_sb, x_sj, d, d_sb, d_si, B, s);
   }
 
@@ -678,7 +699,8 @@ struct Tile {
     check_maintenance("decay_weights");
     if (dev.pulsed()) {
       ensure_state_params();
-      launch_decay_device(d_w.p, d_decay.p, d_rbias.p, d_wmin.p, d_wmax.p, alpha, bias_no_decay ? 1 : 0, X, size(), s);
+      launch_decay_device(wp_dev(), d_decay.p, d_rbias.p, d_wmin.p, d_wmax.p, alpha, bias_no_decay ? 1 : 0, X, size(), s);
+      refresh_shown_weights(s);
     } else {
       const float rate = dev.p.lifetime > 1.0f ? 1.0f / dev.p.lifetime : 0.0f;
       const float scale = 1.0f - alpha * rate;
@@ -693,7 +715,8 @@ struct Tile {
     check_maintenance("diffuse_weights");
     if (dev.pulsed()) {
       ensure_state_params();
-      launch_diffuse(d_w.p, d_diff.p, 0.0f, d_wmin.p, d_wmax.p, key(), call++, size(), s);
+      launch_diffuse(wp_dev(), d_diff.p, 0.0f, d_wmin.p, d_wmax.p, key(), call++, size(), s);
+      refresh_shown_weights(s);
     } else if (dev.p.diffusion > 0.0f) {
       launch_diffuse(d_w.p, nullptr, dev.p.diffusion, nullptr, nullptr, key(), call++, size(), s);
     }
@@ -705,8 +728,10 @@ struct Tile {
   void clip_weights(int type, float fixed_value, float sigma, hipStream_t s) {
     check_maintenance("clip_weights");
     if (type == RPU_CLIP_FIXED_VALUE) {
-      if (dev.pulsed()) launch_clip_value(d_w.p, d_wmin.p, d_wmax.p, fixed_value, nullptr, size(), s);
-      else if (fixed_value >= 0.0f) launch_clip_value(d_w.p, nullptr, nullptr, fixed_value, nullptr, size(), s);
+      if (dev.pulsed()) {
+        launch_clip_value(wp_dev(), d_wmin.p, d_wmax.p, fixed_value, nullptr, size(), s);
+        refresh_shown_weights(s);
+      } else if (fixed_value >= 0.0f) launch_clip_value(d_w.p, nullptr, nullptr, fixed_value, nullptr, size(), s);
     } else if (type == RPU_CLIP_NONE) {
       if (dev.pulsed()) throw RpuError("Sophisticated clipping is NOT implemented for most training devices");
     } else if (type == RPU_CLIP_LAYER_GAUSSIAN || type == RPU_CLIP_AVERAGE_CHANNEL_MAX) {
@@ -731,8 +756,9 @@ struct Tile {
     if (n == 0) return;
     if (dev.pulsed()) {
       ensure_state_params();
-      launch_reset_cols(d_w.p, d_rbias.p, d_wmin.p, d_wmax.p, dev.p.reset_std, start_col, n, reset_prob, X, D, key(),
+      launch_reset_cols(wp_dev(), d_rbias.p, d_wmin.p, d_wmax.p, dev.p.reset_std, start_col, n, reset_prob, X, D, key(),
                         call++, s);
+      refresh_shown_weights(s);
     } else {
       launch_reset_cols(d_w.p, nullptr, nullptr, nullptr, dev.p.reset_std, start_col, n, reset_prob, X, D, key(), call++, s);
     }
@@ -757,8 +783,8 @@ struct Tile {
     }
     if (!dr_prev.p) {
       dr_prev.ensure(n); dr_w0.ensure(n); dr_t.ensure(n);
-      RPU_HIP_CHECK(hipMemcpyAsync(dr_prev.p, d_w.p, n * sizeof(float), hipMemcpyDeviceToDevice, s));
-      RPU_HIP_CHECK(hipMemcpyAsync(dr_w0.p, d_w.p, n * sizeof(float), hipMemcpyDeviceToDevice, s));
+      RPU_HIP_CHECK(hipMemcpyAsync(dr_prev.p, wp_dev(), n * sizeof(float), hipMemcpyDeviceToDevice, s));
+      RPU_HIP_CHECK(hipMemcpyAsync(dr_w0.p, wp_dev(), n * sizeof(float), hipMemcpyDeviceToDevice, s));
       launch_fill(dr_t.p, 0.0f, n, s);
       drift_t = 0.0f;
     }
@@ -770,9 +796,10 @@ struct Tile {
     p.a = q.drift_g_offset * q.drift_wg_ratio + q.drift_w_offset;
     if (std::fabs(p.a) < p.reset_tol) p.a = 0.0f;
     const bool random = p.nu_std > 0.0f || p.w_read_std > 0.0f;
-    launch_device_drift(d_w.p, dr_prev.p, dr_w0.p, dr_t.p, per_device ? d_nu.p : nullptr,
+    launch_device_drift(wp_dev(), dr_prev.p, dr_w0.p, dr_t.p, per_device ? d_nu.p : nullptr,
                         dev.pulsed() ? d_wmin.p : nullptr, dev.pulsed() ? d_wmax.p : nullptr, p, drift_t, key(),
                         random ? call++ : call, n, s);
+    refresh_shown_weights(s);
     RPU_HIP_CHECK(hipGetLastError());
     last_stream = s;
   }
@@ -912,6 +939,12 @@ struct Tile {
       if (counting) count_pulses(a, true, s);
       launch_update_implicit(a, s);
       prof_mark(s, "update_implicit");
+    }
+    // write noise: cross-points that took a pulse show their new persistent weight with fresh noise
+    if (dv.w == d_wp.p && persistent()) {
+      launch_write_noise_touched(a, d_w.p, d_wp.p, dev.scaled_write_noise(),
+                                 up.p.pulse_type != RPU_PULSE_STOCHASTIC_COMPRESSED, s);
+      prof_mark(s, "write_noise");
     }
     RPU_HIP_CHECK(hipGetLastError());
     last_stream = s;
@@ -1815,6 +1848,7 @@ int rpu_tile_clone(rpu_tile_t **out, const rpu_tile_t *src_c) {
         RPU_HIP_CHECK(hipMemcpy(dst.p, from.p, n * sizeof(float), hipMemcpyDeviceToDevice));
       };
       dup(t.d_fbw, s.d_fbw);
+      dup(t.d_wp, s.d_wp);
       t.fb_during_test = s.fb_during_test;
       dup(t.dr_prev, s.dr_prev);
       dup(t.dr_w0, s.dr_w0);
@@ -1923,11 +1957,30 @@ int rpu_tile_set_weights(rpu_tile_t *tile, const float *w_host) {
     }
     std::vector<float> w(w_host, w_host + t.size());
     t.clip_host(w);
+    // onSetWeights (rpu_pulsed_device.cpp:545-571): with write noise the given weights become the persistent ones and
+    // the shown ones are those, with fresh noise if apply_write_noise_on_set
     if (t.resident()) {
       DeviceGuard g(t.device_id);
       t.sync_last();
       RPU_HIP_CHECK(hipMemcpy(t.d_w.p, w.data(), t.size() * sizeof(float), hipMemcpyHostToDevice));
+      if (t.persistent()) {
+        RPU_HIP_CHECK(hipMemcpy(t.d_wp.p, w.data(), t.size() * sizeof(float), hipMemcpyHostToDevice));
+        if (t.dev.p.apply_write_noise_on_set) {
+          t.refresh_shown_weights(t.last_stream);
+          RPU_HIP_CHECK(hipStreamSynchronize(t.last_stream));
+        }
+      }
     } else {
+      if (t.persistent()) {
+        t.arr.persistent = w;
+        if (t.dev.p.apply_write_noise_on_set) {
+          // a host tile draws its noise on the CPU, from the tile's seed and call counter
+          std::mt19937 engine((uint32_t)(t.seed ^ (t.seed >> 32)) + 0x9e3779b9u * (++t.call));
+          std::normal_distribution<float> normal(0.0f, 1.0f);
+          const float std_ = t.dev.scaled_write_noise();
+          for (float &v : w) v += std_ * normal(engine);
+        }
+      }
       t.w_host.swap(w);
     }
   });
@@ -1979,7 +2032,14 @@ int rpu_tile_hidden_parameter_count(const rpu_tile_t *tile) {
     return n;
   }
   if (!tile->t.dev.pulsed()) return 0;
-  return tile->t.dev.linear() ? 10 : 8;
+  return (tile->t.dev.linear() ? 10 : 8) + (tile->t.persistent() ? 1 : 0);
+}
+
+// index into kHiddenNames of entry idx of a single tile, or -1 for the persistent weights, which sit between the
+// base entries and the slopes (PulsedRPUDevice::getDPNames then LinearStepRPUDevice's, rpu_pulsed_device.cpp:235-253)
+static int single_hidden_code(const Tile &t, int idx) {
+  if (!t.persistent() || idx < 8) return idx;
+  return idx == 8 ? -1 : idx - 1;
 }
 
 const char *rpu_tile_hidden_parameter_name(const rpu_tile_t *tile, int idx) {
@@ -1991,7 +2051,8 @@ const char *rpu_tile_hidden_parameter_name(const rpu_tile_t *tile, int idx) {
     name = std::string(local < n_local ? kHiddenNames[local] : "hidden_weights") + "_" + std::to_string(device);
     return name.c_str();
   }
-  return kHiddenNames[idx];
+  const int code = single_hidden_code(tile->t, idx);
+  return code < 0 ? "persistent_weights" : kHiddenNames[code];
 }
 
 static std::vector<float> *hidden_array(DeviceArrays &arr, int idx) {
@@ -2010,7 +2071,10 @@ static std::vector<float> *hidden_array(DeviceArrays &arr, int idx) {
   }
 }
 
-static std::vector<float> *hidden_slot(Tile &t, int idx) { return hidden_array(t.arr, idx); }
+static std::vector<float> *hidden_slot(Tile &t, int idx) {
+  const int code = single_hidden_code(t, idx);
+  return code < 0 ? &t.arr.persistent : hidden_array(t.arr, code);
+}
 
 int rpu_tile_get_hidden_parameters(rpu_tile_t *tile, float *data_host) {
   return guarded([&] {
@@ -2035,9 +2099,20 @@ int rpu_tile_get_hidden_parameters(rpu_tile_t *tile, float *data_host) {
       }
       return;
     }
+    if (t.persistent()) {
+      // the persistent weights live on the GPU while the tile is resident
+      t.arr.persistent.resize(n);
+      if (t.resident()) {
+        DeviceGuard g(t.device_id);
+        t.sync_last();
+        RPU_HIP_CHECK(hipMemcpy(t.arr.persistent.data(), t.d_wp.p, n * sizeof(float), hipMemcpyDeviceToHost));
+      } else if (t.arr.persistent.empty()) {
+        t.arr.persistent = t.w_host;
+      }
+    }
     for (int k = 0; k < count; ++k) {
       std::vector<float> *a = hidden_slot(t, k);
-      if (a) std::memcpy(data_host + (size_t)k * n, a->data(), n * sizeof(float));
+      if (a && a->size() == n) std::memcpy(data_host + (size_t)k * n, a->data(), n * sizeof(float));
       else std::memset(data_host + (size_t)k * n, 0, n * sizeof(float));
     }
   });
@@ -2078,17 +2153,26 @@ int rpu_tile_set_hidden_parameters(rpu_tile_t *tile, const float *data_host) {
     }
     for (int k = 0; k < count; ++k) {
       std::vector<float> *a = hidden_slot(t, k);
-      if (a) std::memcpy(a->data(), data_host + (size_t)k * n, n * sizeof(float));
+      if (a) {
+        a->resize(n);
+        std::memcpy(a->data(), data_host + (size_t)k * n, n * sizeof(float));
+      }
     }
-    // new bounds apply to the current weights at once (rpu_pulsed_device.cpp setDeviceParameter -> onSetWeights)
+    // new bounds apply to the current weights at once (rpu_pulsed_device.cpp setDeviceParameter -> onSetWeights);
+    // with write noise onSetWeights then takes the clipped shown weights as the persistent ones, whatever was given
     if (t.resident()) {
       DeviceGuard g(t.device_id);
       t.sync_last();
       t.upload_params();
       launch_clip(t.d_w.p, t.d_wmin.p, t.d_wmax.p, n, t.last_stream);
+      if (t.persistent()) {
+        RPU_HIP_CHECK(hipMemcpyAsync(t.d_wp.p, t.d_w.p, n * sizeof(float), hipMemcpyDeviceToDevice, t.last_stream));
+        if (t.dev.p.apply_write_noise_on_set) t.refresh_shown_weights(t.last_stream);
+      }
       RPU_HIP_CHECK(hipStreamSynchronize(t.last_stream));
     } else {
       t.clip_host(t.w_host);
+      if (t.persistent()) t.arr.persistent = t.w_host;
     }
   });
 }

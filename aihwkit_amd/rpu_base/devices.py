@@ -352,6 +352,7 @@ class LinearStepResistiveDeviceParameter(PulsedResistiveDeviceParameter):
         p.ls_allow_increasing_slope = int(bool(self.allow_increasing))
         p.ls_mean_bound_reference = int(bool(self.mean_bound_reference))
         p.write_noise_std = float(self.write_noise_std)
+        p.apply_write_noise_on_set = int(bool(self.apply_write_noise_on_set))
         p.ls_mult_noise = int(bool(self.mult_noise))
         p.ls_reverse_up = int(bool(self.reverse_up))
         p.ls_reverse_down = int(bool(self.reverse_down))

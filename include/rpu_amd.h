@@ -171,7 +171,7 @@ typedef struct rpu_device_params {
   float reset;                     /* 0 */
   float reset_dtod;                /* 0 */
   float reset_std;                 /* 0.01 */
-  float write_noise_std;           /* 0 ; > 0 is not provided */
+  float write_noise_std;           /* 0 ; > 0 (LinearStep / SoftBounds): persistent weights, see apply_write_noise_on_set */
   /* LinearStep tail */
   int32_t ls_allow_increasing_slope; /* 0 */
   int32_t ls_mean_bound_reference;   /* 1 */
@@ -196,6 +196,11 @@ typedef struct rpu_device_params {
   float drift_reset_tol;             /* 1e-7 */
   float drift_w_read_std;            /* 0 */
   int32_t count_pulses;              /* 0 ; 1: every update also counts the pulses of each cross-point */
+  /* Write noise (R/rpu_linearstep_device.cpp:112-164, R/rpu_pulsed_device.cpp:545-588): with write_noise_std > 0 the
+   * pulses act on hidden persistent weights and the weights that forward / backward and get_weights see are those
+   * plus write_noise_std * dw_min * N(0, 1), redrawn for a cross-point whenever it takes a pulse and for all after
+   * weight maintenance; set_weights redraws it when this flag is set. */
+  int32_t apply_write_noise_on_set;  /* 1 */
 } rpu_device_params;
 
 /* Replaces PulsedMetaParameter<float> (R/rpu_pulsed.h:127-151): forward IO, backward IO, update. */

@@ -31,6 +31,7 @@ def oracle():
         lib.orc_set_weight_granularity.argtypes = [P, C.c_float]
         lib.orc_set_weights.argtypes = [P, P]
         lib.orc_get_weights.argtypes = [P, P]
+        lib.orc_get_persistent.argtypes = [P, P]
         lib.orc_hidden_count.argtypes = [P]
         lib.orc_get_hidden.argtypes = [P, P]
         lib.orc_set_hidden.argtypes = [P, P]
@@ -58,6 +59,8 @@ class OracleTile:
         self.h = self.lib.orc_create(x_size, d_size, C.byref(config))
         if not self.h:
             raise RuntimeError(self.lib.orc_last_error().decode())
+        # the C side seeds from the clock, as the reference does for seed 0; tests want the same draws on every run
+        self.lib.orc_set_seed(self.h, 20250131)
 
     def __del__(self):
         if getattr(self, "h", None):
@@ -84,6 +87,12 @@ class OracleTile:
     def get_weights(self):
         w = np.empty((self.D, self.X), np.float32)
         self.lib.orc_get_weights(self.h, w.ctypes.data)
+        return w
+
+    def get_persistent(self):
+        """The weights the pulses act on (the shown ones without write noise)."""
+        w = np.empty((self.D, self.X), np.float32)
+        self.lib.orc_get_persistent(self.h, w.ctypes.data)
         return w
 
     def get_hidden(self):

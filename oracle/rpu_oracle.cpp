@@ -194,6 +194,8 @@ struct OrcTile {
   // R/rpu_linearstep_device.h:199-200
   std::vector<float> slope_up, slope_down;
   std::vector<int32_t> last_rounds;
+  // write noise (R/rpu_pulsed_device.h:89-104): the weights the pulses act on; w then holds the shown weights
+  std::vector<float> w_persistent;
   float aux_nm = -1.0f; // running AverageAbsMax scale (R/rpu_forward_backward_pass.h:241), negative: not started
   // scratch
   std::vector<float> in_buf, bias_buf;
@@ -204,6 +206,9 @@ struct OrcTile {
 };
 
 bool is_pulsed_device(const OrcTile &t) { return t.dev.kind != RPU_DEVICE_IDEAL; }
+bool uses_persistent(const OrcTile &t) {
+  return (t.dev.kind == RPU_DEVICE_LINEAR_STEP || t.dev.kind == RPU_DEVICE_SOFT_BOUNDS) && t.dev.write_noise_std > 0.0f;
+}
 bool is_linear_device(const OrcTile &t) {
   return t.dev.kind == RPU_DEVICE_LINEAR_STEP || t.dev.kind == RPU_DEVICE_SOFT_BOUNDS;
 }
@@ -748,7 +753,8 @@ void generate_counts(OrcTile &t, std::vector<int> &counts, std::vector<std::vect
 // ConstantStep: R/rpu_constantstep_device.cpp:27-55 ; LinearStep: R/rpu_linearstep_device.cpp:112-164
 inline void device_step(OrcTile &t, size_t k, int sign, bool dense_form) {
   const rpu_device_params &par = t.dev;
-  float &w = t.w[k];
+  const bool persist = uses_persistent(t);
+  float &w = persist ? t.w_persistent[k] : t.w[k];
   const float std_ = par.dw_min_std;
   if (par.kind == RPU_DEVICE_CONSTANT_STEP) {
     if (std_ > 0.0f || dense_form) {
@@ -784,6 +790,8 @@ inline void device_step(OrcTile &t, size_t k, int sign, bool dense_form) {
     }
     w = std::max(w, t.w_min[k]);
     w = std::min(w, t.w_max[k]);
+    // update_once_mult / update_once_add (R/rpu_linearstep_device.cpp:112-164): the shown weight is redrawn
+    if (persist) t.w[k] = w + par.write_noise_std * par.dw_min * t.rng.gauss();
   }
 }
 
@@ -1007,10 +1015,11 @@ void *orc_create(int x_size, int d_size, const rpu_tile_config *cfg) {
     t->dev.ls_mean_bound_reference = 0;
   }
   t->w.assign((size_t)x_size * d_size, 0.f);
+  t->w_persistent.assign((size_t)x_size * d_size, 0.f);
   t->rng.seed(0);
   if (is_pulsed_device(*t)) {
-    if (t->dev.write_noise_std > 0.f) {
-      g_err = "oracle: write noise not restated";
+    if (t->dev.write_noise_std > 0.f && !is_linear_device(*t)) { // R/rpu_pulsed_device.h:106-111
+      g_err = "oracle: Device does not support write noise";
       return nullptr;
     }
     OrcRealWorldRng rw(t->dev.construction_seed);
@@ -1028,10 +1037,26 @@ void orc_use_gauss_table(void *h, int on) { static_cast<OrcTile *>(h)->rng.use_t
 void orc_set_learning_rate(void *h, float lr) { static_cast<OrcTile *>(h)->lr = lr; }
 void orc_set_weight_granularity(void *h, float g) { static_cast<OrcTile *>(h)->granularity = g; }
 
+// onSetWeights (R/rpu_pulsed_device.cpp:545-571) after the bounds: the given weights are the persistent ones, the shown
+// ones get fresh noise if asked for
+static void on_set_weights(OrcTile &t) {
+  if (!uses_persistent(t)) return;
+  t.w_persistent = t.w;
+  if (t.dev.apply_write_noise_on_set) {
+    const float std_ = t.dev.write_noise_std * t.dev.dw_min;
+    for (size_t k = 0; k < t.w.size(); ++k) t.w[k] = t.w_persistent[k] + std_ * t.rng.gauss();
+  }
+}
 void orc_set_weights(void *h, const float *w) { // R/rpu_pulsed.cpp:288-292
   auto *t = static_cast<OrcTile *>(h);
   memcpy(t->w.data(), w, sizeof(float) * t->w.size());
   clip_to_bounds(*t);
+  on_set_weights(*t);
+}
+void orc_get_persistent(void *h, float *w) {
+  auto *t = static_cast<OrcTile *>(h);
+  const std::vector<float> &src = uses_persistent(*t) ? t->w_persistent : t->w;
+  memcpy(w, src.data(), sizeof(float) * src.size());
 }
 void orc_get_weights(void *h, float *w) {
   auto *t = static_cast<OrcTile *>(h);
@@ -1075,6 +1100,7 @@ void orc_set_hidden(void *h, const float *data) { // R/rpu_pulsed_device.cpp:290
     if (a) memcpy(a->data(), data + k * n, sizeof(float) * n);
   }
   clip_to_bounds(*t);
+  on_set_weights(*t);
 }
 
 // R/rpu.cpp:508-533 forward + R/rpu.cpp:42-57 forwardMatrix loop

@@ -129,8 +129,13 @@ def test_unsupported_parameters_fail_loudly():
         make_meta().create_array(4, 4, constant_step(w_min=0.1))
     with pytest.raises(AttributeError):
         dev.no_such_field = 1
-    with pytest.raises(RuntimeError, match="write_noise_std"):
-        make_meta().create_array(4, 4, soft_bounds(write_noise_std=0.1))
+    make_meta().create_array(4, 4, soft_bounds(write_noise_std=0.1))    # LinearStep / SoftBounds implement write noise
+    cfg = make_meta()._config(constant_step())                          # ConstantStep does not (through the C ABI)
+    cfg.device.write_noise_std = 0.1
+    import ctypes
+    handle = ctypes.c_void_p()
+    assert _cabi.lib().rpu_tile_create(ctypes.byref(handle), 4, 4, ctypes.byref(cfg)) != 0
+    assert b"write noise" in _cabi.lib().rpu_last_error()
 
 
 def test_enums_have_the_reference_values():

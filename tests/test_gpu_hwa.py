@@ -382,3 +382,72 @@ def test_pulse_counters_of_implicit_updates(gpu_device):
     want = np.stack([np.where(n > 0, n, 0).sum(axis=0), np.where(n < 0, -n, 0).sum(axis=0)])
     assert want[0].sum() > 100 and want[1].sum() > 100
     assert np.array_equal(tile.get_pulse_counters().numpy(), want)
+
+
+# ---- write noise (persistent weights) -------------------------------------------------------------------------------
+
+def test_write_noise_persistent_weights(gpu_device):
+    """SoftBounds with write_noise_std: the pulses and the maintenance act on the persistent weights, which follow the
+    trajectory of the same device without write noise (oracle and GPU, deterministic pulses); the shown weights are those
+    plus N(0, (write_noise_std dw_min)^2), redrawn where a pulse landed, for all after maintenance and set_weights."""
+    from helpers import build_pair
+
+    rng = np.random.default_rng(5)
+    x_size, d_size, batch = 70, 45, 8
+    sigma = 5.0 * 0.002
+    for pulse_type in (dv.PulseType.DeterministicImplicit, dv.PulseType.StochasticCompressed):
+        meta = make_meta(noise_free_io(), noise_free_io(), pulse_type=pulse_type, desired_bl=31)
+        kw = dict(dw_min=0.002, dw_min_std=0.0, construction_seed=3, lifetime=40.0)
+        host, orc, noisy = build_pair(meta, soft_bounds(write_noise_std=5.0, **kw), x_size, d_size)
+        _h, _o, plain = build_pair(meta, soft_bounds(**kw), x_size, d_size)
+        names = noisy.get_hidden_parameter_names()
+        assert names.index("persistent_weights") == 8 and names[-2:] == ["slope_up", "slope_down"] and len(names) == 11
+        persistent = lambda: noisy.get_hidden_parameters()[8].numpy()       # noqa: E731
+        w = rng.uniform(-0.3, 0.3, (d_size, x_size)).astype(F)
+        for t in (noisy, plain):
+            t.set_weights(torch.from_numpy(w))
+            t.set_learning_rate(0.05)
+            t.set_seed(31)
+        shown0 = noisy.get_weights().numpy()
+        assert np.array_equal(persistent(), plain.get_weights().numpy())
+        z = (shown0 - persistent()) / sigma
+        assert abs(z.mean()) < 4 / np.sqrt(z.size) and abs(z.std() - 1) < 4 / np.sqrt(2 * z.size)
+        x = rng.uniform(-1, 1, (batch, x_size)).astype(F)
+        x[:, :12] = 0.0                                           # columns that see no pulse
+        d = rng.normal(0, 0.3, (batch, d_size)).astype(F)
+        xg, dg = torch.from_numpy(x).cuda(), torch.from_numpy(d).cuda()
+        noisy.update(xg, dg, False)
+        plain.update(xg, dg, False)
+        assert np.array_equal(persistent(), plain.get_weights().numpy())    # same seed, same pulses, same steps
+        touched = plain.get_weights().numpy() != np.clip(w, hidden(plain)["min_bound"], hidden(plain)["max_bound"])
+        assert not touched[:, :12].any() and 0.2 < touched.mean() < 0.95
+        shown1 = noisy.get_weights().numpy()
+        assert np.array_equal(shown1[:, :12], shown0[:, :12])    # no pulse, no new noise
+        z1 = ((shown1 - persistent()) / sigma)[touched]
+        assert abs(z1.mean()) < 4 / np.sqrt(z1.size) and abs(z1.std() - 1) < 4 / np.sqrt(2 * z1.size)
+        assert abs(np.corrcoef(z1, z[touched])[0, 1]) < 4 / np.sqrt(z1.size)   # redrawn
+        if pulse_type == dv.PulseType.DeterministicImplicit:     # the oracle walks the same deterministic pulses
+            orc.set_weights(w)
+            orc.set_learning_rate(0.05)
+            orc.update(x, d)
+            assert np.abs(orc.get_persistent() - persistent()).max() <= 1e-5
+        # forward contracts with the shown weights
+        y = noisy.forward(xg).cpu().numpy()
+        assert np.abs(y - plain.forward(xg).cpu().numpy()).max() > 1e-3
+        # maintenance acts on the persistent weights and redraws every shown one
+        noisy.decay_weights(1.0)
+        plain.decay_weights(1.0)
+        assert np.abs(persistent() - plain.get_weights().numpy()).max() <= 1e-7
+        shown2 = noisy.get_weights().numpy()
+        z2 = (shown2 - persistent()) / sigma
+        assert abs(z2.std() - 1) < 4 / np.sqrt(2 * z2.size) and abs(np.corrcoef(z2.ravel(), z.ravel())[0, 1]) < 4 / np.sqrt(z2.size)
+        assert not np.array_equal(shown2[:, :12], shown1[:, :12])
+        # a copy carries both matrices
+        import copy
+        twin = copy.deepcopy(noisy)
+        assert np.array_equal(twin.get_hidden_parameters()[8].numpy(), persistent())
+        assert np.array_equal(twin.get_weights().numpy(), shown2)
+    # without apply_write_noise_on_set the given weights are shown as they are
+    _h, _o, quiet = build_pair(meta, soft_bounds(write_noise_std=5.0, apply_write_noise_on_set=False, **kw), x_size, d_size)
+    quiet.set_weights(torch.from_numpy(w))
+    assert np.array_equal(quiet.get_weights().numpy(), quiet.get_hidden_parameters()[8].numpy())

@@ -154,3 +154,40 @@ def test_mean_count_and_none_with_device_updates_closed_form():
     want = np.clip(np.clip(w0 - 0.5 * np.outer(ds[0], xs[0]), -0.3, 0.3) - 0.5 * np.outer(ds[1], xs[1]), -0.3, 0.3)
     np.testing.assert_allclose(tile.get_weights(), want, atol=1e-6)
     assert (np.abs(w0 - 0.5 * ds.T @ xs) > 0.3).any()             # the example does reach the bounds
+
+
+def test_write_noise_persistent_weights_in_the_oracle():
+    """With write noise the pulses act on persistent weights, which follow exactly the trajectory of a device without
+    it; the shown weights are those plus N(0, (write_noise_std dw_min)^2), redrawn only where a pulse landed."""
+    from oracle_lib import OracleTile
+
+    rng = np.random.default_rng(5)
+    x_size, d_size, batch = 40, 30, 6
+    meta = make_meta(pulse_type=dv.PulseType.DeterministicImplicit, desired_bl=31)
+    kw = dict(dw_min=0.002, dw_min_std=0.0, construction_seed=3)
+    from helpers import soft_bounds
+    noisy = OracleTile(x_size, d_size, meta._config(soft_bounds(write_noise_std=5.0, **kw)))
+    plain = OracleTile(x_size, d_size, meta._config(soft_bounds(**kw)))
+    w = rng.uniform(-0.3, 0.3, (d_size, x_size)).astype(F)
+    noisy.set_seed(11)
+    noisy.set_weights(w)
+    plain.set_weights(w)
+    shown0 = noisy.get_weights()
+    np.testing.assert_array_equal(noisy.get_persistent(), plain.get_weights())
+    z = (shown0 - noisy.get_persistent()) / (5.0 * 0.002)       # apply_write_noise_on_set: all redrawn
+    assert abs(z.mean()) < 4 / np.sqrt(z.size) and abs(z.std() - 1) < 4 / np.sqrt(2 * z.size)
+    x = rng.uniform(-1, 1, (batch, x_size)).astype(F)
+    x[:, :10] = 0.0                                              # columns that see no pulse
+    d = rng.normal(0, 0.3, (batch, d_size)).astype(F)
+    for t in (noisy, plain):
+        t.set_learning_rate(0.05)
+        t.update(x, d)
+    np.testing.assert_array_equal(noisy.get_persistent(), plain.get_weights())
+    counts = np.abs(plain.implicit_counts(x, d)).sum(axis=0)
+    shown1 = noisy.get_weights()
+    untouched = counts == 0
+    assert untouched[:, :10].all() and 0.2 < (~untouched).mean() < 0.9
+    np.testing.assert_array_equal(shown1[untouched], shown0[untouched])
+    z = ((shown1 - noisy.get_persistent()) / (5.0 * 0.002))[~untouched]
+    assert abs(z.mean()) < 4 / np.sqrt(z.size) and abs(z.std() - 1) < 4 / np.sqrt(2 * z.size)
+    assert abs(np.corrcoef(z, ((shown0 - plain.get_weights()) / 0.01)[~untouched])[0, 1]) < 0.3   # redrawn, not shifted
