@@ -27,7 +27,7 @@ class IOParams(C.Structure):
         ("w_noise_type", i32), ("w_noise", f32), ("ir_drop", f32), ("out_noise_std", f32),
         ("out_nonlinearity", f32), ("out_nonlinearity_std", f32), ("v_offset_std", f32),
         ("r_series", f32), ("w_read_asymmetry_dtod", f32), ("ir_drop_g_ratio", f32),
-        ("nm_decay", f32),
+        ("nm_decay", f32), ("slope_calibration", f32), ("v_offset_w_min", f32), ("r_series_max_total", f32),
     ]
 
 

@@ -61,6 +61,7 @@ struct MvmArgs {
   // pre_add[row * O + o] for the output o of the sample whose quantized input is row `row` of xq[round & 1];
   // null: none.  Only the 32 x 32 round kernels read it.
   const float *pre_add;
+  int pre_is_total;         // 1: pre_add holds the whole analog value before quantization (the kernel's own sums are unused)
   int nm_phase;             // running-average noise management: 1 = the init kernel only stores every sample's
                             // largest absolute input in st.nm, 2 = it takes the scales from st.nm; 0 otherwise
   int small_tiles_only;     // 1: never the large-tile kernel (its row padding differs)
@@ -107,15 +108,24 @@ bool conv_forward_supported(const MvmArgs &a);
 void launch_conv_forward(const MvmArgs &a, const ConvArgs &c, hipStream_t s);
 
 // ---- analog non-idealities before the ADC (kernels_nonideal.hip), rpu_forward_backward_pass.cpp:325-433, 535-560
-// transformed copy of the quantized input rows [rows][k_pad]: mode 0 x^2, 1 |x|, 2 x (1 - (1 - j / K)^2)
+// transformed copy of the quantized input rows [rows][k_pad]: mode 0 x^2, 1 |x|, 2 x (1 - (1 - j / K)^2), 3 x
 void launch_side_rows(const float *xq, float *out, int rows, int k_pad, int K, int mode, const int *skip_if_zero,
                       hipStream_t s);
 void launch_abs_copy(const float *w, float *out, size_t n, hipStream_t s);
 struct SideDev {
   int w_noise_type; // 0 none, 1 additive constant (row_sumsq), 2 PCM read (s_noise)
   float w_noise, ir_drop, a_scale; // a_scale = in_size / ir_drop_g_ratio
+  // total mode (s_y non-null): the analog value itself is made here, with the per-line terms of the periphery
+  // (applyVoltageOffsets and finalizeOutput up to the output noise, rpu_forward_backward_pass.cpp:436-506, 679-698)
+  const float *s_y;        // W x_q per row and output
+  const float *x_accum;    // sum of x_q per row (only read with v_offset_w_min != 0)
+  const float *v_offset;   // per output, null: no voltage offsets / series resistance
+  const float *out_nl;     // per output, null: no non-linearity
+  const float *out_noise;  // per output, null: out_noise_all for every output
+  float r_series, r_series_max_total, v_offset_w_min, nl_factor, out_noise_all, out_asym;
 };
-// pre[row][o] = w_noise term * N(0, 1) - IR-drop term; s_cur / s_ir are null without IR drop
+// addend mode: pre[row][o] = w_noise term * N(0, 1) - IR-drop term; s_cur / s_ir are null without IR drop.
+// total mode: pre[row][o] = asymmetry(nonlinearity(offsets(s_y - IR drop) + w_noise term)) + output noise
 void launch_side_combine(float *pre, const float *s_noise, const float *row_sumsq, const float *s_cur, const float *s_ir,
                          const SideDev &p, int rows, int O, PhiloxKey key, uint32_t call, int round,
                          const int *skip_if_zero, hipStream_t s);

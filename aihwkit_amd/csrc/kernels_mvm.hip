@@ -134,7 +134,8 @@ __device__ __forceinline__ void mvm_adc_values(const MvmArgs &a, int round, int 
 #pragma unroll
   for (int q = 0; q < 4; ++q) {
     float y = v[q];
-    if (pre && o0 + q < a.O) y += pre[o0 + q]; // weight noise, IR drop (rpu_forward_backward_pass.cpp:535-560)
+    // weight noise, IR drop (rpu_forward_backward_pass.cpp:535-560); with the per-line terms the whole value
+    if (pre && o0 + q < a.O) y = a.pre_is_total ? pre[o0 + q] : y + pre[o0 + q];
     if (a.io.out_asym > 0.0f) y = y < 0.0f ? y * (1.0f - a.io.out_asym) : y;
     if (a.io.out_noise > 0.0f) y += a.io.out_noise * nz[q];
     if (a.io.out_res > 0.0f) {

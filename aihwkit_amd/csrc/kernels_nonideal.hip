@@ -26,10 +26,12 @@ __global__ __launch_bounds__(256) void k_side_rows(const float *xq, float *out, 
       v = x * x;
     } else if (mode == 1) {
       v = fabsf(x);
-    } else {
+    } else if (mode == 2) {
       // lines far from the output see the largest drop: x_j (1 - (1 - j / n)^2)
       const float p = 1.0f - (float)j / (float)K;
       v = x * (1.0f - p * p);
+    } else {
+      v = x;
     }
     out[i] = j < K ? v : 0.0f;
   }
@@ -51,25 +53,49 @@ __global__ __launch_bounds__(256) void k_side_combine(float *pre, const float *s
   for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
     const int row = (int)(i / quads);
     const int o0 = (int)(i % quads) * 4;
-    float z[4] = {0.f, 0.f, 0.f, 0.f};
+    float z[4] = {0.f, 0.f, 0.f, 0.f}, zo[4] = {0.f, 0.f, 0.f, 0.f};
     const bool noisy = p.w_noise_type != 0 && p.w_noise > 0.0f;
     if (noisy) philox_normal4((uint32_t)(o0 >> 2), (uint32_t)row, call, RNG_W_NOISE | ((uint32_t)round << 8), key, z);
+    const bool total = p.s_y != nullptr;
+    const bool out_noisy = total && (p.out_noise != nullptr || p.out_noise_all > 0.0f);
+    if (out_noisy) philox_normal4((uint32_t)(o0 >> 2), (uint32_t)row, call, RNG_OUT_NOISE | ((uint32_t)round << 8), key, zo);
     const float x_norm = (noisy && p.w_noise_type == 1) ? sqrtf(row_sumsq[row]) : 0.0f;
+    const float y_ref = (total && p.v_offset && p.v_offset_w_min != 0.0f) ? -p.v_offset_w_min * p.x_accum[row] : 0.0f;
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
       const int o = o0 + q;
       if (o >= O) break;
       const size_t k = (size_t)row * O + o;
-      float v = 0.0f;
+      float v = total ? p.s_y[k] : 0.0f;
       if (p.ir_drop > 0.0f) {
         // a_i = sum_j |w_ij| |x_j| n / (Gw / g_max); c_i = a_i (a_i (0.05 a_i - 0.2) + 0.5)
         const float a = p.a_scale * s_cur[k];
         const float c = a * (a * (0.05f * a - 0.2f) + 0.5f);
         v -= c * (p.ir_drop * s_ir[k]);
       }
+      if (total && p.v_offset) {
+        const float vo = p.v_offset[o];
+        const float rs = fmaxf(p.r_series, 0.0f);
+        if (p.v_offset_w_min == 0.0f) {
+          v = rs <= 0.0f ? v * (1.0f - vo) : (1.0f - vo) * v / (1.0f + fminf(rs * fabsf(v), p.r_series_max_total));
+        } else if (rs <= 0.0f) {
+          v = v * (1.0f - vo) - vo * (y_ref * 2.0f);
+        } else {
+          // the positive and the reference line see their own series resistance
+          const float y_pos = v + y_ref;
+          const float p_nom = 1.0f + fminf(rs * fabsf(y_pos), p.r_series_max_total);
+          const float n_nom = 1.0f + fminf(rs * fabsf(y_ref), p.r_series_max_total);
+          v = (1.0f - vo) * y_pos / p_nom - (1.0f + vo) * y_ref / n_nom;
+        }
+      }
       if (noisy) {
         if (p.w_noise_type == 1) v += (p.w_noise * x_norm) * z[q];
         else v += p.w_noise * sqrtf(s_noise[k]) * z[q];
+      }
+      if (total) {
+        if (p.out_nl) v = p.nl_factor * v / (1.0f + fabsf(p.out_nl[o] * v));
+        if (p.out_asym > 0.0f) v = v < 0.0f ? v * (1.0f - p.out_asym) : v;
+        if (out_noisy) v += (p.out_noise ? p.out_noise[o] : p.out_noise_all) * zo[q];
       }
       pre[k] = v;
     }

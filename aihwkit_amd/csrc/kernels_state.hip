@@ -217,13 +217,16 @@ __global__ __launch_bounds__(256) void k_device_drift(float *w, float *prev, flo
   }
 }
 
-// one workgroup per row: largest absolute value or sum of squares of the first n_cols columns
+// one workgroup per row: largest absolute value (0), sum of squares (1) or sum (2) of the first n_cols columns
 __global__ __launch_bounds__(256) void k_row_stat(const float *w, int x_size, int n_cols, int sum_squares,
                                                    float *row_out) {
   __shared__ float sh[4];
   const float *row = w + (size_t)blockIdx.x * x_size;
   float m = 0.0f;
-  if (sum_squares) {
+  if (sum_squares == 2) {
+    for (int j = threadIdx.x; j < n_cols; j += blockDim.x) m += row[j];
+    m = block_sum(m, sh);
+  } else if (sum_squares) {
     for (int j = threadIdx.x; j < n_cols; j += blockDim.x) m = __builtin_fmaf(row[j], row[j], m);
     m = block_sum(m, sh);
   } else {

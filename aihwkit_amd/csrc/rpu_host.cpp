@@ -55,14 +55,8 @@ void IOPar::initialize(bool backward) {
   if (p.w_noise_type < 0 || p.w_noise_type > 2) {
     throw RpuError("Output noise type not implemented");
   }
-  if (p.out_noise_std > 0.0f) {
-    throw RpuError("out_noise_std is not implemented on this path.");
-  }
-  if (p.out_nonlinearity > 0.0f || p.out_nonlinearity_std > 0.0f || p.r_series > 0.0f) {
-    throw RpuError("Output non-linearity / r_series are not implemented on this path.");
-  }
-  if (p.v_offset_std > 0.0f) {
-    throw RpuError("Voltage offsets are not implemented on this path.");
+  if (p.w_read_asymmetry_dtod > 0.0f) {
+    throw RpuError("w_read_asymmetry_dtod is only read by the PosNegSeparate MV types, which are not implemented on this path.");
   }
   switch (p.noise_management) {
   case RPU_NM_NONE:
@@ -102,6 +96,47 @@ void IOPar::initialize(bool backward) {
   if (backward) {
     p.bound_management = RPU_BM_NONE; // the backward pass never iterates (rpu_forward_backward_pass.cpp:1002)
   }
+}
+
+// Per-line values of the periphery (ForwardBackwardPassIOManaged::populateFBParameter,
+// rpu_forward_backward_pass.cpp:254-318): voltage offsets, non-linearity coefficients with the slope calibration
+// factor, and output noise levels.  The reference draws them from the tile's run-time generator; any stream will do.
+void IOPar::populate_lines(int out_size, unsigned int seed) {
+  v_offset.clear();
+  out_nl.clear();
+  out_noise_values.clear();
+  nl_factor = 1.0f;
+  if (perfect) return;
+  ConstructionRng rng(seed); // 0: from the clock
+  if (has_voltage_offsets()) {
+    v_offset.resize(out_size);
+    for (float &v : v_offset) v = std::max(p.v_offset_std * rng.normal(), 0.0f);
+  }
+  const float out_bound = (p.out_bound > 0.0f && p.out_bound < std::numeric_limits<float>::infinity()) ? p.out_bound : 1.0f;
+  if (has_nl_calibration()) {
+    out_nl.resize(out_size);
+    for (float &v : out_nl) {
+      v = fabsf(p.out_nonlinearity / out_bound * (1.0f + std::max(p.out_nonlinearity_std, 0.0f) * rng.normal()));
+    }
+  }
+  set_nl_factor();
+  if (p.out_noise_std > 0.0f) {
+    out_noise_values.resize(out_size);
+    for (float &v : out_noise_values) v = fabsf(p.out_noise * (1.0f + p.out_noise_std * rng.normal()));
+  }
+}
+
+void IOPar::set_nl_factor() {
+  nl_factor = 1.0f;
+  if (perfect || p.slope_calibration <= 0.0f) return;
+  const float out_bound = (p.out_bound > 0.0f && p.out_bound < std::numeric_limits<float>::infinity()) ? p.out_bound : 1.0f;
+  float sum_nl = 0.0f;
+  if (p.out_nonlinearity > 0.0f) {
+    for (float v : out_nl) sum_nl += fabsf(v);
+  }
+  const float n = out_nl.empty() ? 1.0f : (float)out_nl.size();
+  const float f = 1.0f + (sum_nl / n + p.r_series) * p.slope_calibration * out_bound;
+  nl_factor = f * f;
 }
 
 void UpdatePar::initialize() {
@@ -369,6 +404,10 @@ void TransferPar::initialize(int x_size, int d_size) {
   io.p.bound_management = RPU_BM_NONE;
   io.p.noise_management = RPU_NM_NONE;
   io.initialize(!p.transfer_columns);
+  if (io.has_line_terms()) {
+    throw RpuError("Per-line terms (voltage offsets, series resistance, output non-linearity, out_noise_std) are not "
+                   "provided for the read of a transfer.");
+  }
   up.p = p.transfer_up;
   up.initialize();
   fully_hidden = (p.gamma == 0.0f) && (gamma_vec.back() == 1.0f);
@@ -409,6 +448,9 @@ void fill_default_config(rpu_tile_config *cfg, int device_kind) {
   io.max_bm_res = 0.25f;
   io.ir_drop_g_ratio = 5.7143e5f;
   io.nm_decay = 1e-3f;
+  io.slope_calibration = 0.5f;
+  io.v_offset_w_min = 0.0f;
+  io.r_series_max_total = std::numeric_limits<float>::max();
   cfg->f_io = io;
   cfg->b_io = io;
 

@@ -21,6 +21,14 @@ struct IOPar {
   rpu_io_params p{};
   bool perfect = false;
   void initialize(bool backward); // rpu_pulsed_meta_parameter.cpp:39-128
+  // per-output-line values of the periphery (MVParameter, rpu_forward_backward_pass.h:17-26); empty when off
+  std::vector<float> v_offset, out_nl, out_noise_values;
+  float nl_factor = 1.0f;
+  bool has_voltage_offsets() const { return !perfect && (p.v_offset_std > 0.0f || p.r_series > 0.0f); }
+  bool has_nl_calibration() const { return !perfect && (p.out_nonlinearity > 0.0f || p.r_series > 0.0f); }
+  bool has_line_terms() const { return has_voltage_offsets() || has_nl_calibration() || (!perfect && p.out_noise_std > 0.0f); }
+  void populate_lines(int out_size, unsigned int seed);
+  void set_nl_factor(); // from out_nl: after sampling and after the values were set from outside
 };
 
 struct UpdatePar {

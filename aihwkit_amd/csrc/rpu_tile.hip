@@ -190,7 +190,9 @@ struct Tile {
   DevBuf<float> d_wp;
   // analog non-idealities before the ADC: the addend per output, up to three side contractions, the transformed
   // input rows, |W| and the squared row norms
-  DevBuf<float> n_pre, n_s1, n_s2, n_s3, n_rows, n_absw, n_sumsq;
+  DevBuf<float> n_pre, n_s1, n_s2, n_s3, n_s4, n_rows, n_absw, n_sumsq, n_xsum;
+  DevBuf<float> d_line[2][3]; // per direction: voltage offsets, non-linearity coefficients, output noise levels
+  bool line_valid[2][3] = {{false, false, false}, {false, false, false}};
   // running AverageAbsMax noise-management scale, one value shared by forward and backward as in the reference
   // (rpu_forward_backward_pass.h:241); negative: not started
   DevBuf<float> nm_aux;
@@ -274,6 +276,10 @@ struct Tile {
     delta_w = nullptr;
     n_pre.release(); n_s1.release(); n_s2.release(); n_s3.release(); n_rows.release(); n_absw.release();
     n_sumsq.release();
+    n_s4.release();
+    n_xsum.release();
+    for (auto &dir : d_line) for (auto &b : dir) b.release();
+    for (auto &dir : line_valid) for (bool &v : dir) v = false;
     nm_aux.release();
     d_wp.release();
     d_fbw.release(); s_rowstat.release(); dr_prev.release(); dr_w0.release(); dr_t.release(); d_nu.release();
@@ -433,7 +439,25 @@ struct Tile {
 
   // whether a pass with these IO parameters has non-idealities that add to the sums before the ADC
   static bool has_pre_adc_terms(const IOPar &io) {
-    return !io.perfect && ((io.p.w_noise_type != 0 && io.p.w_noise > 0.0f) || io.p.ir_drop > 0.0f);
+    return !io.perfect && ((io.p.w_noise_type != 0 && io.p.w_noise > 0.0f) || io.p.ir_drop > 0.0f || io.has_line_terms());
+  }
+
+  // per-line values of both directions; a fixed construction seed fixes them too
+  void populate_lines(unsigned int construction_seed) {
+    fio.populate_lines(D, construction_seed ? construction_seed * 2654435761u + 1u : 0u);
+    bio.populate_lines(X, construction_seed ? construction_seed * 2654435761u + 2u : 0u);
+  }
+
+  // device copies of the per-line values of a direction (0 forward, 1 backward)
+  const float *line_values(int dir, int which, const std::vector<float> &host) {
+    if (host.empty()) return nullptr;
+    DevBuf<float> &buf = d_line[dir][which];
+    if (!line_valid[dir][which]) {
+      buf.ensure(host.size());
+      RPU_HIP_CHECK(hipMemcpy(buf.p, host.data(), host.size() * sizeof(float), hipMemcpyHostToDevice));
+      line_valid[dir][which] = true;
+    }
+    return buf.p;
   }
 
   // The addend of every output of round a.round from the quantized inputs of that round: weight noise and IR drop
@@ -447,6 +471,7 @@ struct Tile {
     const bool noisy = io.p.w_noise_type != 0 && io.p.w_noise > 0.0f;
     const bool ir = io.p.ir_drop > 0.0f;
     const bool need_abs = ir || (noisy && io.p.w_noise_type == 2);
+    const bool total = io.has_line_terms();
     n_pre.ensure(out_n);
     n_rows.ensure(row_n);
     if (need_abs && r == 0) {
@@ -454,11 +479,11 @@ struct Tile {
       launch_abs_copy(a.w, n_absw.p, size(), s);
     }
     const auto contract = [&](const float *w, int mode, float *dst) {
-      launch_side_rows(xq, n_rows.p, B, a.k_pad, a.K, mode, skip, s);
+      if (mode != 3) launch_side_rows(xq, n_rows.p, B, a.k_pad, a.K, mode, skip, s);
       MvmArgs g{};
       g.w = w; g.x_size = X; g.d_size = D; g.m_batch = B; g.K = a.K; g.O = a.O; g.k_pad = a.k_pad;
       g.transposed = a.transposed;
-      g.xq[0] = n_rows.p; g.xq[1] = nullptr;
+      g.xq[0] = mode != 3 ? n_rows.p : const_cast<float *>(xq); g.xq[1] = nullptr;
       g.out = dst; g.out_sb = a.O; g.out_so = 1;
       g.io = a.io; g.io.perfect = 1;
       g.alpha = 1.0f; g.beta = 0.0f; g.round = 0;
@@ -483,6 +508,29 @@ struct Tile {
     p.w_noise_type = noisy ? io.p.w_noise_type : 0;
     p.w_noise = io.p.w_noise; p.ir_drop = ir ? io.p.ir_drop : 0.0f;
     p.a_scale = (float)a.K / io.p.ir_drop_g_ratio;
+    if (total) {
+      // the value itself is made beside the round kernel, whose ADC stage then only quantizes and clips
+      const int dir = a.transposed ? 1 : 0;
+      n_s4.ensure(out_n);
+      contract(a.w, 3, n_s4.p);
+      p.s_y = n_s4.p;
+      if (io.has_voltage_offsets()) {
+        p.v_offset = line_values(dir, 0, io.v_offset);
+        if (io.p.v_offset_w_min != 0.0f) {
+          n_xsum.ensure((size_t)B);
+          launch_row_stat(xq, a.k_pad, B, a.K, 2, n_xsum.p, s);
+          p.x_accum = n_xsum.p;
+        }
+      }
+      if (io.has_nl_calibration()) p.out_nl = line_values(dir, 1, io.out_nl);
+      p.out_noise = line_values(dir, 2, io.out_noise_values);
+      p.r_series = io.p.r_series; p.r_series_max_total = io.p.r_series_max_total;
+      p.v_offset_w_min = io.p.v_offset_w_min; p.nl_factor = io.nl_factor;
+      p.out_noise_all = io.p.out_noise; p.out_asym = io.p.out_asymmetry;
+      a.pre_is_total = 1;
+      a.io.out_noise = 0.0f;
+      a.io.out_asym = 0.0f;
+    }
     launch_side_combine(n_pre.p, n_s1.p, n_sumsq.p, n_s2.p, n_s3.p, p, B, a.O, a.key, a.call, r, skip, s);
     a.pre_add = n_pre.p;
     prof_mark(s, "pre_adc_terms");
@@ -1255,6 +1303,7 @@ int rpu_tile_create(rpu_tile_t **out, int x_size, int d_size, const rpu_tile_con
     t.dev.p = cfg->device;
     t.fio.initialize(false);
     t.bio.initialize(true);
+    t.populate_lines(cfg->device.construction_seed);
     t.up.initialize();
     t.dev.initialize();
     t.dev.populate(x_size, d_size, t.arr);
@@ -1285,6 +1334,7 @@ int rpu_tile_create_transfer(rpu_tile_t **out, int x_size, int d_size, const rpu
     t.up.p = cfg->up;
     t.fio.initialize(false);
     t.bio.initialize(true);
+    t.populate_lines(tp->construction_seed);
     t.up.initialize();
     if (t.up.p.pulse_type == RPU_PULSE_NONE || t.up.p.pulse_type == RPU_PULSE_NONE_WITH_DEVICE) {
       throw RpuError("A transfer compound needs a pulsed update (pulse_type None is not provided).");
@@ -1482,10 +1532,31 @@ static void extra_fields(const Tile &t, std::vector<std::string> &names, std::ve
     names.push_back("transfer.slice_idx_" + std::to_string(k));
     values.push_back(t.slice_idx[k]);
   }
+  // per-line values of the periphery (the reference's "fwd.v_offset", "fwd.out_nonlinearity", ... entries,
+  // rpu_forward_backward_pass.cpp:62-80), one entry per line
+  const auto lines = [&](const char *prefix, const char *what, const std::vector<float> &v) {
+    for (size_t k = 0; k < v.size(); ++k) {
+      names.push_back(std::string(prefix) + what + "_" + std::to_string(k) + ".bits");
+      values.push_back(float_bits(v[k]));
+    }
+  };
+  const IOPar *ios[2] = {&t.fio, &t.bio};
+  for (int dir = 0; dir < 2; ++dir) {
+    const char *prefix = dir ? "bwd." : "fwd.";
+    lines(prefix, "v_offset", ios[dir]->v_offset);
+    lines(prefix, "out_nonlinearity", ios[dir]->out_nl);
+    lines(prefix, "out_noise_values", ios[dir]->out_noise_values);
+  }
+}
+static size_t line_entries(const Tile &t) {
+  return t.fio.v_offset.size() + t.fio.out_nl.size() + t.fio.out_noise_values.size() + t.bio.v_offset.size() +
+         t.bio.out_nl.size() + t.bio.out_noise_values.size();
 }
 static thread_local std::string g_extra_name;
 
-int rpu_tile_extra_count(const rpu_tile_t *tile) { return tile ? kFixedExtras + (int)tile->t.slice_idx.size() : 0; }
+int rpu_tile_extra_count(const rpu_tile_t *tile) {
+  return tile ? kFixedExtras + (int)tile->t.slice_idx.size() + (int)line_entries(tile->t) : 0;
+}
 
 const char *rpu_tile_extra_name(const rpu_tile_t *tile, int idx) {
   if (!tile || idx < 0 || idx >= rpu_tile_extra_count(tile)) return nullptr;
@@ -1529,6 +1600,15 @@ int rpu_tile_set_extra(rpu_tile_t *tile, const int64_t *values_host, int count) 
       t.sync_nm_aux(false);
     }
     for (size_t k = 0; k < t.slice_idx.size(); ++k) t.slice_idx[k] = (int)values_host[kFixedExtras + k];
+    size_t at = kFixedExtras + t.slice_idx.size();
+    IOPar *ios[2] = {&t.fio, &t.bio};
+    for (int dir = 0; dir < 2; ++dir) {
+      for (std::vector<float> *v : {&ios[dir]->v_offset, &ios[dir]->out_nl, &ios[dir]->out_noise_values}) {
+        for (float &x : *v) x = bits_float(values_host[at++]);
+      }
+      ios[dir]->set_nl_factor();
+      for (bool &valid : t.line_valid[dir]) valid = false;
+    }
   });
 }
 

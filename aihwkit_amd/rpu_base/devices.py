@@ -202,6 +202,7 @@ class AnalogTileInputOutputParameter(_Struct):
         out_nonlinearity=0.0, out_nonlinearity_std=0.0, mv_type=AnalogMVType.OnePass,
         inp_asymmetry=0.0, out_asymmetry=0.0, slope_calibration=0.5, r_series=0.0, v_offset_std=0.0,
         v_offset_w_min=0.0, w_read_asymmetry_dtod=0.0,
+        r_series_max_total=3.4028234663852886e38,   # IOMetaParameter field that the reference's binding leaves out
     )
 
     def _to_c(self) -> IOParams:
@@ -218,7 +219,7 @@ class AnalogTileInputOutputParameter(_Struct):
                      "out_noise", "out_asymmetry", "out_scale", "nm_thres", "nm_assumed_wmax",
                      "max_bm_res", "w_noise", "ir_drop", "out_noise_std", "out_nonlinearity",
                      "out_nonlinearity_std", "v_offset_std", "r_series", "w_read_asymmetry_dtod",
-                     "ir_drop_g_ratio", "nm_decay"):
+                     "ir_drop_g_ratio", "nm_decay", "slope_calibration", "v_offset_w_min", "r_series_max_total"):
             setattr(p, name, float(getattr(self, name)))
         p.w_noise_type = int(self.w_noise_type)
         return p

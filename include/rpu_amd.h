@@ -89,7 +89,7 @@ enum rpu_device_kind {
  * AnalogTileInputOutputParameter (B/rpu_base_devices.cpp:485-519).  Field names and defaults are
  * the C++ ones; `inp_res` / `out_res` accept "1/steps" or "steps" and are converted to an absolute
  * step res * 2 * bound at creation (R/rpu_pulsed_meta_parameter.cpp:26-37,56-57).
- * Fields in the "not provided" block must be left at their inactive value or creation fails. */
+ * A field marked "not provided" must be left at its inactive value or creation fails. */
 typedef struct rpu_io_params {
   int32_t is_perfect;             /* 0 */
   int32_t mv_type;                /* RPU_MV_ONE_PASS */
@@ -115,15 +115,19 @@ typedef struct rpu_io_params {
   int32_t w_noise_type;           /* 0 = None, 1 = AdditiveConstant, 2 = PCMRead */
   float w_noise;                  /* ignored while w_noise_type == 0 */
   float ir_drop;                  /* 0 */
-  /* not provided (must stay inactive): */
-  float out_noise_std;            /* 0 */
-  float out_nonlinearity;         /* 0 */
+  /* per-line variations of the periphery, sampled once per tile and direction (R/rpu_forward_backward_pass.cpp:244-318):
+   * they are part of the extra state (rpu_tile_get_extra), "fwd.*" / "bwd.*" */
+  float out_noise_std;            /* 0: relative spread of out_noise from output line to output line */
+  float out_nonlinearity;         /* 0: y -> f y / (1 + nl_i |y|), nl_i = |out_nonlinearity / out_bound (1 + std xi)| */
   float out_nonlinearity_std;     /* 0 */
-  float v_offset_std;             /* 0 */
-  float r_series;                 /* 0 */
-  float w_read_asymmetry_dtod;    /* 0 */
+  float v_offset_std;             /* 0: voltage offset per output line, max(v_offset_std xi, 0) (:436-506) */
+  float r_series;                 /* 0: series resistance, y -> y / (1 + min(r_series |y|, r_series_max_total)) */
+  float w_read_asymmetry_dtod;    /* 0; not provided (only read by the PosNegSeparate MV types) */
   float ir_drop_g_ratio;          /* 5.7143e5: wire conductance over g_max (ir_drop_Gw_div_gmax) */
   float nm_decay;                 /* 1e-3: weight of a new sample in the AverageAbsMax running average */
+  float slope_calibration;        /* 0.5: y / out_bound at which the non-linearity has slope 1 on average (:283-295) */
+  float v_offset_w_min;           /* 0: reference conductance of the offset, typically -1 */
+  float r_series_max_total;       /* FLT_MAX */
 } rpu_io_params;
 
 /* Replaces PulsedUpdateMetaParameter<float> (R/rpu_pulsed_meta_parameter.h:248-323) as bound by

@@ -42,6 +42,11 @@ def oracle():
         lib.orc_update_with_words.argtypes = [P, P, P, P, C.c_int]
         lib.orc_update_bl_ab.argtypes = [P, P, P, C.c_int, P, P, P]
         lib.orc_implicit_counts.argtypes = [P, P, P, C.c_int, P]
+        lib.orc_get_lines.argtypes = [P, C.c_int, C.c_int, P]
+        lib.orc_set_lines.argtypes = [P, C.c_int, C.c_int, P, C.c_int]
+        lib.orc_get_nl_factor.argtypes = [P, C.c_int]
+        lib.orc_repopulate_lines.argtypes = [P]
+        lib.orc_get_nl_factor.restype = C.c_float
         _lib = lib
     return _lib
 
@@ -61,11 +66,29 @@ class OracleTile:
             raise RuntimeError(self.lib.orc_last_error().decode())
         # the C side seeds from the clock, as the reference does for seed 0; tests want the same draws on every run
         self.lib.orc_set_seed(self.h, 20250131)
+        self.lib.orc_repopulate_lines(self.h)
 
     def __del__(self):
         if getattr(self, "h", None):
             self.lib.orc_destroy(self.h)
             self.h = None
+
+    def get_lines(self, direction, which):
+        """Per-line values of the periphery: direction 0 forward / 1 backward; which 0 voltage offsets,
+        1 non-linearity coefficients, 2 output noise levels."""
+        n = self.lib.orc_get_lines(self.h, direction, which, None)
+        out = np.zeros(n, dtype=np.float32)
+        if n:
+            self.lib.orc_get_lines(self.h, direction, which, out.ctypes.data_as(C.c_void_p))
+        return out
+
+    def set_lines(self, direction, which, values):
+        v = _f32(values)
+        if self.lib.orc_set_lines(self.h, direction, which, v.ctypes.data_as(C.c_void_p), v.size):
+            raise RuntimeError("length of the per-line values differs")
+
+    def nl_factor(self, direction):
+        return float(self.lib.orc_get_nl_factor(self.h, direction))
 
     def set_seed(self, seed):
         self.lib.orc_set_seed(self.h, seed)

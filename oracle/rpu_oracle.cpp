@@ -173,12 +173,18 @@ bool init_io(OrcIO &io, bool backward) {
     g_err = "Output noise type not implemented";
     return false;
   }
-  if (p.out_noise_std > 0.f || p.out_nonlinearity > 0.f || p.v_offset_std > 0.f || p.r_series > 0.f) {
-    g_err = "oracle: out_noise_std / out_nonlinearity / v_offset / r_series not restated";
+  if (p.w_read_asymmetry_dtod > 0.f) {
+    g_err = "oracle: w_read_asymmetry_dtod (PosNegSeparate MV types) not restated";
     return false;
   }
   return true;
 }
+
+// R/rpu_pulsed_meta_parameter.h:112-119
+bool io_perfect(const rpu_io_params &p) { return p.is_perfect || p.mv_type == RPU_MV_IDEAL; }
+bool has_voltage_offsets(const rpu_io_params &p) { return p.v_offset_std > 0.0f || p.r_series > 0.0f; }
+bool has_out_nonlinearity(const rpu_io_params &p) { return p.out_nonlinearity > 0.0f && !io_perfect(p); }
+bool has_nl_calibration(const rpu_io_params &p) { return has_out_nonlinearity(p) || p.r_series > 0.0f; }
 
 struct OrcTile {
   int X = 0, D = 0;
@@ -196,6 +202,11 @@ struct OrcTile {
   std::vector<int32_t> last_rounds;
   // write noise (R/rpu_pulsed_device.h:89-104): the weights the pulses act on; w then holds the shown weights
   std::vector<float> w_persistent;
+  // R/rpu_forward_backward_pass.h:17-26 MVParameter of the forward [0] and backward [1] pass
+  struct Lines {
+    std::vector<float> v_offset, out_nl, out_noise;
+    float nl_factor = 1.0f;
+  } lines[2];
   float aux_nm = -1.0f; // running AverageAbsMax scale (R/rpu_forward_backward_pass.h:241), negative: not started
   // scratch
   std::vector<float> in_buf, bias_buf;
@@ -458,8 +469,11 @@ void gemv(const OrcTile &t, const float *in, float *out, int out_inc, bool trans
 
 // R/rpu_forward_backward_pass.cpp:666-719 finalizeOutputImplStage5 (the ADC).  A Gaussian is drawn
 // for every output even when out_noise == 0 (:750-756 instantiate with_noise = true in both branches).
-bool finalize_output(OrcTile &t, float *out, int out_size, int out_inc, const rpu_io_params &io) {
+bool finalize_output(OrcTile &t, float *out, int out_size, int out_inc, const rpu_io_params &io,
+                     const OrcTile::Lines &mv) {
   bool bound_test_passed = true;
+  const bool with_nl = has_nl_calibration(io); // :738-745
+  const float nlf = mv.nl_factor;
   const float bound = io.out_bound > 0.0f ? io.out_bound : std::numeric_limits<float>::infinity();
   const float asymmetry_scale = (1.0f - io.out_asymmetry);
   const float res = io.out_res;
@@ -467,8 +481,10 @@ bool finalize_output(OrcTile &t, float *out, int out_size, int out_inc, const rp
   const bool sr = io.out_sto_round != 0;
   for (int i = 0; i < out_size; ++i) {
     float value = out[(size_t)i * out_inc];
+    if (with_nl) value = nlf * value / (1.0f + std::fabs(mv.out_nl[i] * value)); // :686-688
     if (io.out_asymmetry > 0.0f) value = value < 0.0f ? value * asymmetry_scale : value;
-    value += io.out_noise * t.rng.gauss();
+    const float noise_std = io.out_noise_std > 0.0f ? mv.out_noise[i] : io.out_noise; // :696
+    value += noise_std * t.rng.gauss();
     value = discretize(value, res, sr, t.rng);
     if (with_bm) {
       if (value > bound) {
@@ -485,6 +501,86 @@ bool finalize_output(OrcTile &t, float *out, int out_size, int out_inc, const rp
     out[(size_t)i * out_inc] = value;
   }
   return bound_test_passed;
+}
+
+// R/rpu_forward_backward_pass.cpp:283-295: the slope calibration factor of the non-linearity
+void set_nl_factor(const rpu_io_params &io, OrcTile::Lines &mv, int out_size) {
+  mv.nl_factor = 1.0f;
+  const float out_bound = io.out_bound > 0.0f && io.out_bound < std::numeric_limits<float>::infinity() ? io.out_bound : 1.0f;
+  if (io.slope_calibration > 0.0f) {
+    float sum_nonlinearity = 0.0f;
+    if (has_out_nonlinearity(io)) {
+      for (int i = 0; i < out_size; ++i) sum_nonlinearity += std::fabs(mv.out_nl[i]);
+    }
+    const float r_correction = io.r_series;
+    const float f = 1.0f + (sum_nonlinearity / (float)out_size + r_correction) * io.slope_calibration * out_bound;
+    mv.nl_factor = f * f;
+  }
+}
+
+// R/rpu_forward_backward_pass.cpp:254-318 the populate lambda of populateFBParameter (values drawn from the tile's
+// run-time generator)
+void populate_lines(OrcTile &t, const rpu_io_params &io, OrcTile::Lines &mv, int out_size) {
+  mv = OrcTile::Lines();
+  if (io_perfect(io)) return;
+  if (has_voltage_offsets(io)) {
+    mv.v_offset.resize(out_size);
+    for (int i = 0; i < out_size; ++i) mv.v_offset[i] = std::max(io.v_offset_std * t.rng.gauss(), 0.0f);
+  }
+  const float out_bound = io.out_bound > 0.0f && io.out_bound < std::numeric_limits<float>::infinity() ? io.out_bound : 1.0f;
+  if (has_nl_calibration(io)) {
+    mv.out_nl.resize(out_size);
+    for (int i = 0; i < out_size; ++i) {
+      mv.out_nl[i] =
+          std::fabs(io.out_nonlinearity / out_bound * (1.0f + std::max(io.out_nonlinearity_std, 0.0f) * t.rng.gauss()));
+    }
+  }
+  set_nl_factor(io, mv, out_size);
+  if (io.out_noise_std > 0.0f) {
+    mv.out_noise.resize(out_size);
+    for (int i = 0; i < out_size; ++i) mv.out_noise[i] = std::fabs(io.out_noise * (1.0f + io.out_noise_std * t.rng.gauss()));
+  }
+}
+
+// R/rpu_forward_backward_pass.cpp:436-506 applyVoltageOffsets
+void apply_voltage_offsets(float *out, int out_size, int out_inc, const float *in, int in_size,
+                           const rpu_io_params &io, const OrcTile::Lines &mv) {
+  if (!has_voltage_offsets(io)) return;
+  const float rs = std::max(io.r_series, 0.0f);
+  const float rs_max_total = io.r_series_max_total;
+  if (io.v_offset_w_min == 0.0f) {
+    for (int i = 0; i < out_size; ++i) {
+      float &y = out[(size_t)i * out_inc];
+      const float v_offs = mv.v_offset[i];
+      if (rs <= 0.0f) {
+        y = y * (1.0f - v_offs);
+      } else {
+        const float nom = 1.0f + std::min(rs * std::fabs(y), rs_max_total);
+        y = (1.0f - v_offs) * y / nom;
+      }
+    }
+    return;
+  }
+  float x_accum = 0.0f;
+  for (int j = 0; j < in_size; ++j) x_accum += in[j];
+  if (rs <= 0.0f) {
+    const float y_ref2 = (-io.v_offset_w_min) * x_accum * 2.0f;
+    for (int i = 0; i < out_size; ++i) {
+      float &y = out[(size_t)i * out_inc];
+      const float v_offs = mv.v_offset[i];
+      y = y * (1.0f - v_offs) - v_offs * y_ref2;
+    }
+  } else {
+    const float y_ref = (-io.v_offset_w_min) * x_accum;
+    for (int i = 0; i < out_size; ++i) {
+      float &y = out[(size_t)i * out_inc];
+      const float v_offs = mv.v_offset[i];
+      const float y_pos = y + y_ref;
+      const float p_nom = 1.0f + std::min(rs * std::fabs(y_pos), rs_max_total);
+      const float n_nom = 1.0f + std::min(rs * std::fabs(y_ref), rs_max_total);
+      y = (1.0f - v_offs) * y_pos / p_nom - (1.0f + v_offs) * y_ref / n_nom;
+    }
+  }
 }
 
 // R/rpu_forward_backward_pass.cpp:508-530 computeTotalCurrent and :387-433 applyIrDrop
@@ -550,10 +646,12 @@ bool analog_mv(OrcTile &t, const float *in, int in_size, int in_inc, float *out,
   t.in_buf.resize(in_size);
   prepare_input(t, t.in_buf.data(), in, in_size, in_inc, scale, scaling, io);
   gemv(t, t.in_buf.data(), out, out_inc, transposed);
-  // applyNonIdealities (:535-560): IR drop, then the weight-dependent noise
+  // applyNonIdealities (:535-560): IR drop, voltage offsets, then the weight-dependent noise
+  const OrcTile::Lines &mv = t.lines[transposed ? 1 : 0];
   apply_ir_drop(t, out, out_size, out_inc, t.in_buf.data(), in_size, io, transposed);
+  apply_voltage_offsets(out, out_size, out_inc, t.in_buf.data(), in_size, io, mv);
   apply_output_weight_noise(t, out, out_size, out_inc, t.in_buf.data(), in_size, io, transposed);
-  return finalize_output(t, out, out_size, out_inc, io);
+  return finalize_output(t, out, out_size, out_inc, io, mv);
 }
 
 // R/rpu_forward_backward_pass.cpp:900-988 ForwardBackwardPassIOManaged::forwardVector
@@ -1017,6 +1115,8 @@ void *orc_create(int x_size, int d_size, const rpu_tile_config *cfg) {
   t->w.assign((size_t)x_size * d_size, 0.f);
   t->w_persistent.assign((size_t)x_size * d_size, 0.f);
   t->rng.seed(0);
+  populate_lines(*t, t->fio.p, t->lines[0], d_size);
+  populate_lines(*t, t->bio.p, t->lines[1], x_size);
   if (is_pulsed_device(*t)) {
     if (t->dev.write_noise_std > 0.f && !is_linear_device(*t)) { // R/rpu_pulsed_device.h:106-111
       g_err = "oracle: Device does not support write noise";
@@ -1053,6 +1153,33 @@ void orc_set_weights(void *h, const float *w) { // R/rpu_pulsed.cpp:288-292
   clip_to_bounds(*t);
   on_set_weights(*t);
 }
+// per-line values of the periphery: dir 0 forward / 1 backward; which 0 v_offset, 1 out_nonlinearity, 2 out_noise_values
+// (the entries of the reference's state, R/rpu_forward_backward_pass.cpp:62-100).  Returns the length.
+static std::vector<float> &line_vector(OrcTile &t, int dir, int which) {
+  OrcTile::Lines &mv = t.lines[dir ? 1 : 0];
+  return which == 0 ? mv.v_offset : (which == 1 ? mv.out_nl : mv.out_noise);
+}
+int orc_get_lines(void *h, int dir, int which, float *out) {
+  auto *t = static_cast<OrcTile *>(h);
+  const std::vector<float> &v = line_vector(*t, dir, which);
+  if (out) memcpy(out, v.data(), sizeof(float) * v.size());
+  return (int)v.size();
+}
+int orc_set_lines(void *h, int dir, int which, const float *in, int n) {
+  auto *t = static_cast<OrcTile *>(h);
+  std::vector<float> &v = line_vector(*t, dir, which);
+  if ((int)v.size() != n) return 1;
+  memcpy(v.data(), in, sizeof(float) * v.size());
+  set_nl_factor(dir ? t->bio.p : t->fio.p, t->lines[dir ? 1 : 0], dir ? t->X : t->D);
+  return 0;
+}
+void orc_repopulate_lines(void *h) { // with the generator as it is now seeded
+  auto *t = static_cast<OrcTile *>(h);
+  populate_lines(*t, t->fio.p, t->lines[0], t->D);
+  populate_lines(*t, t->bio.p, t->lines[1], t->X);
+}
+float orc_get_nl_factor(void *h, int dir) { return static_cast<OrcTile *>(h)->lines[dir ? 1 : 0].nl_factor; }
+
 void orc_get_persistent(void *h, float *w) {
   auto *t = static_cast<OrcTile *>(h);
   const std::vector<float> &src = uses_persistent(*t) ? t->w_persistent : t->w;

@@ -110,9 +110,14 @@ def test_unsupported_parameters_fail_loudly():
     with pytest.raises(RuntimeError, match="expects bound==1"):
         make_meta(io_params(inp_bound=2.0)).create_array(4, 4, dev)
     with pytest.raises(RuntimeError, match="not implemented"):
-        make_meta(io_params(out_noise_std=0.1)).create_array(4, 4, dev)
+        make_meta(io_params(w_read_asymmetry_dtod=0.1)).create_array(4, 4, dev)
     with pytest.raises(RuntimeError, match="not implemented"):
-        make_meta(io_params(v_offset_std=0.1)).create_array(4, 4, dev)
+        make_meta(io_params(mv_type=dv.AnalogMVType.PosNegSeparate)).create_array(4, 4, dev)
+    # per-line periphery values are drawn at creation and are part of the extra state of a host tile too
+    host = make_meta(io_params(out_noise_std=0.1, v_offset_std=0.1, r_series=0.01, out_nonlinearity=0.3)).create_array(4, 6, dev)
+    names = [k for k in host.dump_extra() if k.startswith("rpu.fwd.")]
+    assert len(names) == 3 * 6 and "rpu.fwd.v_offset_5.bits" in names and "rpu.fwd.out_noise_values_0.bits" in names
+    assert not any(k.startswith("rpu.bwd.") for k in host.dump_extra())
     make_meta(io_params(ir_drop=1.0, w_noise_type=dv.WeightNoiseType.PCMRead, w_noise=0.1)).create_array(4, 4, dev)
     with pytest.raises(RuntimeError, match="desired_bl"):
         make_meta(desired_bl=255).create_array(4, 4, dev)
