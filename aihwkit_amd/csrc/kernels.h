@@ -109,7 +109,8 @@ void launch_conv_forward(const MvmArgs &a, const ConvArgs &c, hipStream_t s);
 
 // ---- analog non-idealities before the ADC (kernels_nonideal.hip), rpu_forward_backward_pass.cpp:325-433, 535-560
 // transformed copy of the quantized input rows [rows][k_pad]: mode 0 x^2, 1 |x|, 2 x (1 - (1 - j / K)^2), 3 x
-void launch_side_rows(const float *xq, float *out, int rows, int k_pad, int K, int mode, const int *skip_if_zero,
+// part -1 / +1: only the negative / positive inputs (the others read as zero), before the transformation
+void launch_side_rows(const float *xq, float *out, int rows, int k_pad, int K, int mode, int part, const int *skip_if_zero,
                       hipStream_t s);
 void launch_abs_copy(const float *w, float *out, size_t n, hipStream_t s);
 struct SideDev {
@@ -123,6 +124,10 @@ struct SideDev {
   const float *out_nl;     // per output, null: no non-linearity
   const float *out_noise;  // per output, null: out_noise_all for every output
   float r_series, r_series_max_total, v_offset_w_min, nl_factor, out_noise_all, out_asym;
+  // two passes (PosNegSeparate): the first stops after the weight noise (ni_only), the second adds that result
+  // (add_ni) before the non-linearity
+  int ni_only;
+  const float *add_ni;
 };
 // addend mode: pre[row][o] = w_noise term * N(0, 1) - IR-drop term; s_cur / s_ir are null without IR drop.
 // total mode: pre[row][o] = asymmetry(nonlinearity(offsets(s_y - IR drop) + w_noise term)) + output noise

@@ -16,11 +16,13 @@ int grid_for(size_t n) {
 }
 
 __global__ __launch_bounds__(256) void k_side_rows(const float *xq, float *out, size_t total, int k_pad, int K, int mode,
-                                                    const int *skip_if_zero) {
+                                                    int part, const int *skip_if_zero) {
   if (skip_if_zero && *skip_if_zero == 0) return;
   for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
     const int j = (int)(i % k_pad);
-    const float x = xq[i];
+    float x = xq[i];
+    if (part < 0) x = fminf(x, 0.0f);
+    if (part > 0) x = fmaxf(x, 0.0f);
     float v;
     if (mode == 0) {
       v = x * x;
@@ -92,7 +94,8 @@ __global__ __launch_bounds__(256) void k_side_combine(float *pre, const float *s
         if (p.w_noise_type == 1) v += (p.w_noise * x_norm) * z[q];
         else v += p.w_noise * sqrtf(s_noise[k]) * z[q];
       }
-      if (total) {
+      if (p.add_ni) v += p.add_ni[k];
+      if (total && !p.ni_only) {
         if (p.out_nl) v = p.nl_factor * v / (1.0f + fabsf(p.out_nl[o] * v));
         if (p.out_asym > 0.0f) v = v < 0.0f ? v * (1.0f - p.out_asym) : v;
         if (out_noisy) v += (p.out_noise ? p.out_noise[o] : p.out_noise_all) * zo[q];
@@ -104,10 +107,11 @@ __global__ __launch_bounds__(256) void k_side_combine(float *pre, const float *s
 
 } // namespace
 
-void launch_side_rows(const float *xq, float *out, int rows, int k_pad, int K, int mode, const int *skip_if_zero,
+void launch_side_rows(const float *xq, float *out, int rows, int k_pad, int K, int mode, int part, const int *skip_if_zero,
                       hipStream_t s) {
   const size_t total = (size_t)rows * k_pad;
-  hipLaunchKernelGGL(k_side_rows, dim3(grid_for(total)), dim3(256), 0, s, xq, out, total, k_pad, K, mode, skip_if_zero);
+  hipLaunchKernelGGL(k_side_rows, dim3(grid_for(total)), dim3(256), 0, s, xq, out, total, k_pad, K, mode, part,
+                     skip_if_zero);
 }
 
 void launch_abs_copy(const float *w, float *out, size_t n, hipStream_t s) {

@@ -49,14 +49,14 @@ void IOPar::initialize(bool backward) {
     return;
   }
   perfect = false;
-  if (p.mv_type != RPU_MV_ONE_PASS) {
-    throw RpuError("AnalogMVType not implemented on this path (only Ideal and OnePass).");
+  if (p.mv_type != RPU_MV_ONE_PASS && p.mv_type != RPU_MV_POS_NEG_SEPARATE) {
+    throw RpuError("AnalogMVType not implemented on this path (only Ideal, OnePass and PosNegSeparate).");
   }
   if (p.w_noise_type < 0 || p.w_noise_type > 2) {
     throw RpuError("Output noise type not implemented");
   }
   if (p.w_read_asymmetry_dtod > 0.0f) {
-    throw RpuError("w_read_asymmetry_dtod is only read by the PosNegSeparate MV types, which are not implemented on this path.");
+    throw RpuError("w_read_asymmetry_dtod (weights of the negative pass of PosNegSeparate) is not implemented on this path.");
   }
   switch (p.noise_management) {
   case RPU_NM_NONE:
@@ -405,8 +405,8 @@ void TransferPar::initialize(int x_size, int d_size) {
   io.p.noise_management = RPU_NM_NONE;
   io.initialize(!p.transfer_columns);
   if (io.has_line_terms()) {
-    throw RpuError("Per-line terms (voltage offsets, series resistance, output non-linearity, out_noise_std) are not "
-                   "provided for the read of a transfer.");
+    throw RpuError("Per-line terms (voltage offsets, series resistance, output non-linearity, out_noise_std) and "
+                   "PosNegSeparate are not provided for the read of a transfer.");
   }
   up.p = p.transfer_up;
   up.initialize();

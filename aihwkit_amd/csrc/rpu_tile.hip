@@ -190,7 +190,7 @@ struct Tile {
   DevBuf<float> d_wp;
   // analog non-idealities before the ADC: the addend per output, up to three side contractions, the transformed
   // input rows, |W| and the squared row norms
-  DevBuf<float> n_pre, n_s1, n_s2, n_s3, n_s4, n_rows, n_absw, n_sumsq, n_xsum;
+  DevBuf<float> n_pre, n_s1, n_s2, n_s3, n_s4, n_rows, n_absw, n_sumsq, n_xsum, n_part, n_neg;
   DevBuf<float> d_line[2][3]; // per direction: voltage offsets, non-linearity coefficients, output noise levels
   bool line_valid[2][3] = {{false, false, false}, {false, false, false}};
   // running AverageAbsMax noise-management scale, one value shared by forward and backward as in the reference
@@ -278,6 +278,8 @@ struct Tile {
     n_sumsq.release();
     n_s4.release();
     n_xsum.release();
+    n_part.release();
+    n_neg.release();
     for (auto &dir : d_line) for (auto &b : dir) b.release();
     for (auto &dir : line_valid) for (bool &v : dir) v = false;
     nm_aux.release();
@@ -478,60 +480,81 @@ struct Tile {
       n_absw.ensure(size());
       launch_abs_copy(a.w, n_absw.p, size(), s);
     }
-    const auto contract = [&](const float *w, int mode, float *dst) {
-      if (mode != 3) launch_side_rows(xq, n_rows.p, B, a.k_pad, a.K, mode, skip, s);
-      MvmArgs g{};
-      g.w = w; g.x_size = X; g.d_size = D; g.m_batch = B; g.K = a.K; g.O = a.O; g.k_pad = a.k_pad;
-      g.transposed = a.transposed;
-      g.xq[0] = mode != 3 ? n_rows.p : const_cast<float *>(xq); g.xq[1] = nullptr;
-      g.out = dst; g.out_sb = a.O; g.out_so = 1;
-      g.io = a.io; g.io.perfect = 1;
-      g.alpha = 1.0f; g.beta = 0.0f; g.round = 0;
-      g.key = a.key; g.call = a.call;
-      g.small_tiles_only = 1;
-      g.skip_if_zero = skip;
-      launch_mvm_round(g, s);
-    };
-    if (noisy && io.p.w_noise_type == 1) {
-      n_sumsq.ensure((size_t)B);
-      launch_row_stat(xq, a.k_pad, B, a.K, 1, n_sumsq.p, s);
-    } else if (noisy) {
-      n_s1.ensure(out_n);
-      contract(n_absw.p, 0, n_s1.p);
-    }
-    if (ir) {
-      n_s2.ensure(out_n); n_s3.ensure(out_n);
-      contract(n_absw.p, 1, n_s2.p);
-      contract(a.w, 2, n_s3.p);
-    }
-    SideDev p{};
-    p.w_noise_type = noisy ? io.p.w_noise_type : 0;
-    p.w_noise = io.p.w_noise; p.ir_drop = ir ? io.p.ir_drop : 0.0f;
-    p.a_scale = (float)a.K / io.p.ir_drop_g_ratio;
-    if (total) {
-      // the value itself is made beside the round kernel, whose ADC stage then only quantizes and clips
-      const int dir = a.transposed ? 1 : 0;
-      n_s4.ensure(out_n);
-      contract(a.w, 3, n_s4.p);
-      p.s_y = n_s4.p;
-      if (io.has_voltage_offsets()) {
-        p.v_offset = line_values(dir, 0, io.v_offset);
-        if (io.p.v_offset_w_min != 0.0f) {
-          n_xsum.ensure((size_t)B);
-          launch_row_stat(xq, a.k_pad, B, a.K, 2, n_xsum.p, s);
-          p.x_accum = n_xsum.p;
-        }
+    // PosNegSeparate: the negative and the positive inputs see the array one after the other, each pass with its
+    // own IR drop, offsets and weight noise; the sums of both go through the ADC (rpu_forward_backward_pass.cpp:832-893)
+    const bool separate = io.separate_passes();
+    for (int pass = 0; pass < (separate ? 2 : 1); ++pass) {
+      const int part = separate ? (pass == 0 ? -1 : 1) : 0;
+      const float *xin = xq;
+      if (part) {
+        n_part.ensure(row_n);
+        launch_side_rows(xq, n_part.p, B, a.k_pad, a.K, 3, part, skip, s);
+        xin = n_part.p;
       }
-      if (io.has_nl_calibration()) p.out_nl = line_values(dir, 1, io.out_nl);
-      p.out_noise = line_values(dir, 2, io.out_noise_values);
-      p.r_series = io.p.r_series; p.r_series_max_total = io.p.r_series_max_total;
-      p.v_offset_w_min = io.p.v_offset_w_min; p.nl_factor = io.nl_factor;
-      p.out_noise_all = io.p.out_noise; p.out_asym = io.p.out_asymmetry;
-      a.pre_is_total = 1;
-      a.io.out_noise = 0.0f;
-      a.io.out_asym = 0.0f;
+      const auto contract = [&](const float *w, int mode, float *dst) {
+        if (mode != 3) launch_side_rows(xin, n_rows.p, B, a.k_pad, a.K, mode, 0, skip, s);
+        MvmArgs g{};
+        g.w = w; g.x_size = X; g.d_size = D; g.m_batch = B; g.K = a.K; g.O = a.O; g.k_pad = a.k_pad;
+        g.transposed = a.transposed;
+        g.xq[0] = mode != 3 ? n_rows.p : const_cast<float *>(xin); g.xq[1] = nullptr;
+        g.out = dst; g.out_sb = a.O; g.out_so = 1;
+        g.io = a.io; g.io.perfect = 1;
+        g.alpha = 1.0f; g.beta = 0.0f; g.round = 0;
+        g.key = a.key; g.call = a.call;
+        g.small_tiles_only = 1;
+        g.skip_if_zero = skip;
+        launch_mvm_round(g, s);
+      };
+      if (noisy && io.p.w_noise_type == 1) {
+        n_sumsq.ensure((size_t)B);
+        launch_row_stat(xin, a.k_pad, B, a.K, 1, n_sumsq.p, s);
+      } else if (noisy) {
+        n_s1.ensure(out_n);
+        contract(n_absw.p, 0, n_s1.p);
+      }
+      if (ir) {
+        n_s2.ensure(out_n); n_s3.ensure(out_n);
+        contract(n_absw.p, 1, n_s2.p);
+        contract(a.w, 2, n_s3.p);
+      }
+      SideDev p{};
+      p.w_noise_type = noisy ? io.p.w_noise_type : 0;
+      p.w_noise = io.p.w_noise; p.ir_drop = ir ? io.p.ir_drop : 0.0f;
+      p.a_scale = (float)a.K / io.p.ir_drop_g_ratio;
+      if (total) {
+        // the value itself is made beside the round kernel, whose ADC stage then only quantizes and clips
+        const int dir = a.transposed ? 1 : 0;
+        n_s4.ensure(out_n);
+        contract(a.w, 3, n_s4.p);
+        p.s_y = n_s4.p;
+        if (io.has_voltage_offsets()) {
+          p.v_offset = line_values(dir, 0, io.v_offset);
+          if (io.p.v_offset_w_min != 0.0f) {
+            n_xsum.ensure((size_t)B);
+            launch_row_stat(xin, a.k_pad, B, a.K, 2, n_xsum.p, s);
+            p.x_accum = n_xsum.p;
+          }
+        }
+        if (io.has_nl_calibration()) p.out_nl = line_values(dir, 1, io.out_nl);
+        p.out_noise = line_values(dir, 2, io.out_noise_values);
+        p.r_series = io.p.r_series; p.r_series_max_total = io.p.r_series_max_total;
+        p.v_offset_w_min = io.p.v_offset_w_min; p.nl_factor = io.nl_factor;
+        p.out_noise_all = io.p.out_noise; p.out_asym = io.p.out_asymmetry;
+        a.pre_is_total = 1;
+        a.io.out_noise = 0.0f;
+        a.io.out_asym = 0.0f;
+      }
+      float *dst = n_pre.p;
+      if (separate && pass == 0) {
+        n_neg.ensure(out_n);
+        dst = n_neg.p;
+        p.ni_only = 1;
+      } else if (separate) {
+        p.add_ni = n_neg.p;
+      }
+      // the second pass draws its own noise
+      launch_side_combine(dst, n_s1.p, n_sumsq.p, n_s2.p, n_s3.p, p, B, a.O, a.key, a.call, r + 64 * pass, skip, s);
     }
-    launch_side_combine(n_pre.p, n_s1.p, n_sumsq.p, n_s2.p, n_s3.p, p, B, a.O, a.key, a.call, r, skip, s);
     a.pre_add = n_pre.p;
     prof_mark(s, "pre_adc_terms");
   }

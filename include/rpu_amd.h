@@ -70,8 +70,10 @@ enum rpu_pulse_type {
 /* R/rpu_pulsed_meta_parameter.h:42-49 AnalogMVType */
 enum rpu_mv_type {
   RPU_MV_IDEAL = 0,
-  RPU_MV_ONE_PASS = 1
-  /* PosNegSeparate(2), PosNegSeparateDigitalSum(3), SplitMode(4), BitWise(5): not provided */
+  RPU_MV_ONE_PASS = 1,
+  RPU_MV_POS_NEG_SEPARATE = 2 /* negative and positive inputs in two passes, summed before the ADC
+                                 (R/rpu_forward_backward_pass.cpp:832-893) */
+  /* PosNegSeparateDigitalSum(3), SplitMode(4), BitWise(5): not provided */
 };
 
 /* device kinds; B/rpu_base_devices.cpp:545-656 */
@@ -122,7 +124,7 @@ typedef struct rpu_io_params {
   float out_nonlinearity_std;     /* 0 */
   float v_offset_std;             /* 0: voltage offset per output line, max(v_offset_std xi, 0) (:436-506) */
   float r_series;                 /* 0: series resistance, y -> y / (1 + min(r_series |y|, r_series_max_total)) */
-  float w_read_asymmetry_dtod;    /* 0; not provided (only read by the PosNegSeparate MV types) */
+  float w_read_asymmetry_dtod;    /* 0; not provided (weights of the negative pass of the PosNegSeparate types) */
   float ir_drop_g_ratio;          /* 5.7143e5: wire conductance over g_max (ir_drop_Gw_div_gmax) */
   float nm_decay;                 /* 1e-3: weight of a new sample in the AverageAbsMax running average */
   float slope_calibration;        /* 0.5: y / out_bound at which the non-linearity has slope 1 on average (:283-295) */

@@ -151,8 +151,8 @@ bool init_io(OrcIO &io, bool backward) {
     io.perfect = true;
     return true;
   }
-  if (p.mv_type != RPU_MV_ONE_PASS) {
-    g_err = "oracle: only mv_type Ideal / OnePass restated";
+  if (p.mv_type != RPU_MV_ONE_PASS && p.mv_type != RPU_MV_POS_NEG_SEPARATE) {
+    g_err = "oracle: only mv_type Ideal / OnePass / PosNegSeparate restated";
     return false;
   }
   p.out_res = check_res(p.out_res) * (2.0f * p.out_bound);
@@ -640,17 +640,34 @@ void apply_output_weight_noise(OrcTile &t, float *out, int out_size, int out_inc
   }
 }
 
-// R/rpu_forward_backward_pass.cpp:800-829 computeAnalogMV, OnePass
+// R/rpu_forward_backward_pass.cpp:779-797 computeAnalogMVSinglePass: the contraction, then applyNonIdealities
+// (:535-560): IR drop, voltage offsets, then the weight-dependent noise
+void analog_mv_single_pass(OrcTile &t, const float *in, int in_size, float *out, int out_size, int out_inc,
+                           const rpu_io_params &io, bool transposed) {
+  const OrcTile::Lines &mv = t.lines[transposed ? 1 : 0];
+  gemv(t, in, out, out_inc, transposed);
+  apply_ir_drop(t, out, out_size, out_inc, in, in_size, io, transposed);
+  apply_voltage_offsets(out, out_size, out_inc, in, in_size, io, mv);
+  apply_output_weight_noise(t, out, out_size, out_inc, in, in_size, io, transposed);
+}
+
+// R/rpu_forward_backward_pass.cpp:800-897 computeAnalogMV: OnePass and PosNegSeparate
 bool analog_mv(OrcTile &t, const float *in, int in_size, int in_inc, float *out, int out_size,
                int out_inc, float scale, bool scaling, const rpu_io_params &io, bool transposed) {
   t.in_buf.resize(in_size);
   prepare_input(t, t.in_buf.data(), in, in_size, in_inc, scale, scaling, io);
-  gemv(t, t.in_buf.data(), out, out_inc, transposed);
-  // applyNonIdealities (:535-560): IR drop, voltage offsets, then the weight-dependent noise
   const OrcTile::Lines &mv = t.lines[transposed ? 1 : 0];
-  apply_ir_drop(t, out, out_size, out_inc, t.in_buf.data(), in_size, io, transposed);
-  apply_voltage_offsets(out, out_size, out_inc, t.in_buf.data(), in_size, io, mv);
-  apply_output_weight_noise(t, out, out_size, out_inc, t.in_buf.data(), in_size, io, transposed);
+  if (io.mv_type == RPU_MV_POS_NEG_SEPARATE) {
+    // first the negative inputs, then the positive ones; the sums of both passes go through the ADC (:832-893)
+    std::vector<float> part((size_t)in_size), neg_out((size_t)out_size);
+    for (int i = 0; i < in_size; ++i) part[i] = t.in_buf[i] < 0.0f ? t.in_buf[i] : 0.0f;
+    analog_mv_single_pass(t, part.data(), in_size, neg_out.data(), out_size, 1, io, transposed);
+    for (int i = 0; i < in_size; ++i) part[i] = t.in_buf[i] > 0.0f ? t.in_buf[i] : 0.0f;
+    analog_mv_single_pass(t, part.data(), in_size, out, out_size, out_inc, io, transposed);
+    for (int j = 0; j < out_size; ++j) out[(size_t)j * out_inc] += neg_out[j];
+    return finalize_output(t, out, out_size, out_inc, io, mv);
+  }
+  analog_mv_single_pass(t, t.in_buf.data(), in_size, out, out_size, out_inc, io, transposed);
   return finalize_output(t, out, out_size, out_inc, io, mv);
 }
 

@@ -137,3 +137,54 @@ def test_laws_of_the_drawn_line_values():
     assert abs(tile.nl_factor(0) / f ** 2 - 1.0) < 1e-4
     assert len({tuple(np.round(v[:50], 7)) for v in (vo, nl, noise)}) == 3      # separate draws
     assert tile.get_lines(1, 0).shape == (2,)
+
+
+def test_pos_neg_separate_passes():
+    """Negative and positive inputs see the array one after the other; what is not linear in the inputs differs."""
+    pns = dv.AnalogMVType.PosNegSeparate
+    rng = np.random.default_rng(7)
+    # everything linear: the two passes add up to the one pass
+    w = rng.uniform(-0.6, 0.6, (5, 9)).astype(F)
+    x = rng.uniform(-1, 1, (6, 9)).astype(F)
+    one, two = oracle_tile(9, 5, w), oracle_tile(9, 5, w, mv_type=pns)
+    np.testing.assert_allclose(two.forward(x), one.forward(x), rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(two.forward(x), x @ w.T, rtol=1e-5, atol=1e-6)
+    # series resistance acts on the current of each pass: w = [1, 1], x = [0.8, -0.3]
+    kw = dict(r_series=0.5, slope_calibration=0.0)
+    xs = np.array([[0.8, -0.3]], dtype=F)
+    assert abs(oracle_tile(2, 1, [[1.0, 1.0]], **kw).forward(xs)[0, 0] - 0.5 / 1.25) < 1e-6
+    want = 0.8 / 1.4 - 0.3 / 1.15
+    assert abs(oracle_tile(2, 1, [[1.0, 1.0]], mv_type=pns, **kw).forward(xs)[0, 0] - want) < 1e-6
+    # IR drop of a constant tile with the first h lines at +v and the others at -v: each pass has its own total current
+    n, h, wv, v, ratio = 10, 4, 0.5, 0.8, 30.0
+    xs = np.full((1, n), -v, dtype=F)
+    xs[0, :h] = v
+    pos_w = np.array([1.0 - (1.0 - j / n) ** 2 for j in range(n)])
+
+    def drop(a):
+        return a * (a * (0.05 * a - 0.2) + 0.5)
+
+    a_pos, a_neg = n / ratio * wv * v * h, n / ratio * wv * v * (n - h)
+    want = (wv * v * h - drop(a_pos) * wv * v * pos_w[:h].sum()) + (-wv * v * (n - h) + drop(a_neg) * wv * v * pos_w[h:].sum())
+    got = oracle_tile(n, 2, np.full((2, n), wv), mv_type=pns, ir_drop=1.0, ir_drop_g_ratio=ratio).forward(xs)[0]
+    np.testing.assert_allclose(got, [want, want], rtol=3e-6)
+    a_all = n / ratio * wv * v * n
+    want_one = wv * v * (2 * h - n) - drop(a_all) * wv * v * (pos_w[:h].sum() - pos_w[h:].sum())
+    got_one = oracle_tile(n, 2, np.full((2, n), wv), ir_drop=1.0, ir_drop_g_ratio=ratio).forward(xs)[0]
+    np.testing.assert_allclose(got_one, [want_one, want_one], rtol=3e-6)
+    assert abs(want - want_one) > 1e-2
+    # one ADC for the sum: clipping and the non-linearity see both passes together
+    t = oracle_tile(2, 1, [[1.0, 1.0]], mv_type=pns, out_bound=0.4, out_nonlinearity=0.4, slope_calibration=0.0)
+    np.testing.assert_allclose(t.forward(np.array([[0.9, -0.7]], dtype=F))[0, 0], 0.2 / 1.2, rtol=1e-6)   # nl = 1
+    t = oracle_tile(2, 1, [[1.0, 1.0]], mv_type=pns, out_bound=0.4)
+    assert abs(t.forward(np.array([[0.9, -0.7]], dtype=F))[0, 0] - 0.2) < 1e-6   # each pass alone is beyond the bound
+    assert t.forward(np.array([[0.9, -0.1]], dtype=F))[0, 0] == F(0.4)
+    # weight noise is drawn for each pass: the variances of the passes add to the one-pass law
+    d = 4000
+    t = oracle_tile(3, d, np.zeros((d, 3)), mv_type=pns, w_noise=0.1, w_noise_type=dv.WeightNoiseType.AdditiveConstant)
+    t.use_gauss_table(False)
+    y = t.forward(np.array([[0.6, -0.8, 0.0]] * 10, dtype=F)).astype(np.float64) / 0.1
+    assert abs(y.mean()) < 4 / np.sqrt(y.size) and abs(y.std() - 1) < 4 / np.sqrt(2 * y.size)
+    # backward takes the same path
+    t = oracle_tile(1, 2, [[1.0], [1.0]], mv_type=pns, **kw)
+    assert abs(t.backward(np.array([[0.8, -0.3]], dtype=F))[0, 0] - (0.8 / 1.4 - 0.3 / 1.15)) < 1e-6
