@@ -714,3 +714,84 @@ def test_random_inference_pipeline_and_ir_drop_cases_follow_the_oracles(gpu_devi
     failures = [desc for ok, desc in (one_pcm(seed) for seed in range(90000, 90100)) if not ok]
     failures += [desc for ok, desc in (one_irdrop(seed) for seed in range(91000, 91150)) if not ok]
     assert not failures, failures[:3]
+
+
+def extra_lines(tile, direction, kind):
+    state = tile.dump_extra()
+    prefix = f"rpu.{direction}.{kind}_"
+    n = sum(1 for k in state if k.startswith(prefix))
+    return np.array([state[f"{prefix}{i}.bits"] for i in range(n)], dtype=np.uint32).view(np.float32)
+
+
+def one_periphery(seed):
+    """Random mix of voltage offsets, series resistance, non-linearity, asymmetry, IR drop and separate passes."""
+    F = np.float32
+    rng = np.random.default_rng(seed)
+    x_size = int(rng.choice([2, 31, 33, 64, 65, 129, 300]))
+    d_size = int(rng.choice([1, 3, 32, 33, 97, 200]))
+    batch = int(rng.choice([1, 7, 33, 100, 300]))
+    bias = bool(rng.integers(2))
+    x_trans = bool(rng.integers(2))
+    d_trans = x_trans
+    nm = [NM.NONE, NM.AbsMax][rng.integers(2)]   # scales that do not depend on the order of a sum: no DAC edge flips
+    bm = [BM.NONE, BM.Iterative, BM.IterativeWorstCase][rng.integers(3)]
+    lines = max(x_size, d_size)
+    io = dict(out_noise=0.0, inp_noise=0.0, out_res=-1.0, out_bound=float(rng.choice([1.0, 3.0, 12.0])),
+              noise_management=nm, inp_asymmetry=float(rng.choice([0.0, 0.2])), out_asymmetry=float(rng.choice([0.0, 0.3])),
+              out_scale=float(rng.choice([1.0, 2.0])))
+    if rng.integers(2):
+        io.update(v_offset_std=float(rng.choice([0.05, 0.3])), v_offset_w_min=float(rng.choice([0.0, -1.0, -0.5])))
+    if rng.integers(2):
+        io.update(r_series=float(rng.choice([0.005, 0.05])), r_series_max_total=float(rng.choice([0.3, 3.4028234e38])))
+    if rng.integers(2):
+        io.update(out_nonlinearity=float(rng.choice([0.3, 1.5])), out_nonlinearity_std=float(rng.choice([0.0, 0.3])))
+    io["slope_calibration"] = float(rng.choice([0.0, 0.5, 0.8]))
+    if rng.integers(3) == 0:
+        io.update(ir_drop=float(rng.choice([0.5, 1.0])), ir_drop_g_ratio=lines * (0.3 * 0.5 * lines) / 0.4)
+    if rng.integers(2):
+        io["mv_type"] = dv.AnalogMVType.PosNegSeparate
+    if not any(k in io for k in ("v_offset_std", "r_series", "out_nonlinearity", "mv_type")):
+        io["v_offset_std"] = 0.1
+    meta = make_meta(io_params(bound_management=bm, **io), io_params(**io))
+    dev = constant_step(w_max=1.0, w_min=-1.0, w_max_dtod=0.0, w_min_dtod=0.0, construction_seed=int(rng.integers(1, 1000)))
+    host, orc, _ = build_pair(meta, dev, x_size, d_size, gpu=False)
+    w = rng.uniform(-0.6, 0.6, (d_size, x_size)).astype(F)
+    host.set_weights(torch.from_numpy(w))
+    orc.set_weights(w)
+    gpu = tiles.CudaAnalogTile(host)
+    for di, direction in enumerate(("fwd", "bwd")):
+        for k, kind in enumerate(("v_offset", "out_nonlinearity", "out_noise_values")):
+            v = extra_lines(gpu, direction, kind)
+            if v.size:
+                orc.set_lines(di, k, v)
+    xs = x_size - int(bias)
+    x = rng.uniform(-1, 1, (batch, xs)).astype(F)
+    if batch > 2:
+        x[1] = 0.0
+    xin = np.ascontiguousarray(x.T) if x_trans else x
+    want = orc.forward(xin, bias, x_trans, d_trans)
+    got = gpu.forward(torch.from_numpy(xin).cuda(), bias, x_trans, d_trans).cpu().numpy()
+    bad = []
+    scale = max(np.abs(want).max(), 1e-3)
+    if not np.isfinite(got).all() or np.abs(got - want).max() > 5e-5 * scale:
+        bad.append(("fwd", float(np.abs(got - want).max() / scale)))
+    if bm != BM.NONE and not np.array_equal(gpu.get_bm_rounds(batch).numpy(), orc.bm_rounds(batch)):
+        bad.append(("rounds",))
+    d = rng.normal(0, 0.5, (batch, d_size)).astype(F)
+    din = np.ascontiguousarray(d.T) if d_trans else d
+    want_b = orc.backward(din, bias, d_trans, x_trans)
+    got_b = gpu.backward(torch.from_numpy(din).cuda(), bias, d_trans, x_trans).cpu().numpy()
+    sb = max(np.abs(want_b).max(), 1e-3)
+    if not np.isfinite(got_b).all() or np.abs(got_b - want_b).max() > 5e-5 * sb:
+        bad.append(("bwd", float(np.abs(got_b - want_b).max() / sb)))
+    return not bad, dict(seed=seed, X=x_size, D=d_size, B=batch, bias=bias, trans=x_trans, nm=str(nm), bm=str(bm), io=io,
+                         bad=bad)
+
+
+def test_random_periphery_cases_follow_the_oracle(gpu_device):
+    """Voltage offsets (with and without a reference line), series resistance (capped or not), output non-linearity
+    with its calibration, asymmetries, IR drop and PosNegSeparate in random combinations over shapes, layouts, bias
+    column, noise and bound management: 5e-5 of the output range (the calibration factor of the non-linearity
+    amplifies the rounding of the sums several times before the compression) and identical round counts."""
+    failures = [desc for ok, desc in (one_periphery(seed) for seed in range(92000, 92200)) if not ok]
+    assert not failures, failures[:3]
