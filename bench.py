@@ -169,7 +169,7 @@ def main() -> int:
 
     def time_calls(fn, n):
         start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        for _ in range(3):
+        for _ in range(max(3, n)):   # as many untimed calls as timed ones: the clocks of an idle GPU take a while to rise
             fn()
         torch.cuda.synchronize()
         start.record()
