@@ -224,7 +224,7 @@ def main() -> int:
     # tile with the initial weights like the forward / backward figures above, and the update at a batch of 8, where
     # few pulses per cross-point leave it to the memory system.  They come after the graded measurements: in the
     # first GPU process of a freshly started machine the update call measured 8 % slower (0.099 against 0.090 ms)
-    # whenever the large operands of this part had been allocated before the update's own scratch memory.
+    # whenever this part had run before it (cause unknown; later processes on the same machine were not affected).
     other = None
     if args.config == 2 and not args.no_other_batches:
         tile_b = tiles.CudaAnalogTile(host)
