@@ -795,3 +795,62 @@ def test_random_periphery_cases_follow_the_oracle(gpu_device):
     amplifies the rounding of the sums several times before the compression) and identical round counts."""
     failures = [desc for ok, desc in (one_periphery(seed) for seed in range(92000, 92200)) if not ok]
     assert not failures, failures[:3]
+
+
+def one_write_noise(seed):
+    """Persistent weights follow the device without write noise; the shown ones change exactly where a pulse landed."""
+    F = np.float32
+    rng = np.random.default_rng(seed)
+    x_size = int(rng.choice([1, 3, 31, 33, 64, 65, 129, 300]))
+    d_size = int(rng.choice([1, 2, 32, 33, 97, 200]))
+    batch = int(rng.choice([1, 8, 32, 33, 100, 257]))
+    pulse_type = [dv.PulseType.DeterministicImplicit, dv.PulseType.StochasticCompressed, dv.PulseType.MeanCount][rng.integers(3)]
+    bl = int(rng.choice([1, 7, 31]))
+    meta = make_meta(noise_free_io(), noise_free_io(), pulse_type=pulse_type, desired_bl=bl,
+                     update_bl_management=bool(rng.integers(2)), update_management=bool(rng.integers(2)))
+    kw = dict(dw_min=0.002, dw_min_std=float(rng.choice([0.0, 0.3])), construction_seed=int(rng.integers(1, 100)))
+    std = float(rng.choice([1.0, 5.0]))
+    _h, _o, noisy = build_pair(meta, soft_bounds(write_noise_std=std, **kw), x_size, d_size)
+    _h, _o, plain = build_pair(meta, soft_bounds(**kw), x_size, d_size)
+    w = rng.uniform(-0.3, 0.3, (d_size, x_size)).astype(F)
+    for t in (noisy, plain):
+        t.set_weights(torch.from_numpy(w))
+        t.set_learning_rate(0.05)
+        t.set_seed(seed)
+    x = rng.uniform(-1, 1, (batch, x_size)).astype(F)
+    x[:, rng.integers(x_size)] = 0.0                              # a column without pulses
+    x[rng.random((batch, x_size)) < 0.5] = 0.0
+    d = rng.normal(0, 0.3, (batch, d_size)).astype(F)
+    d[rng.random((batch, d_size)) < 0.5] = 0.0
+    bad = []
+    index = noisy.get_hidden_parameter_names().index("persistent_weights")
+    for call in range(2):
+        before_plain = plain.get_weights().numpy()
+        before_shown = noisy.get_weights().numpy()
+        noisy.update(cuda(x), cuda(d), False)
+        plain.update(cuda(x), cuda(d), False)
+        persistent = noisy.get_hidden_parameters()[index].numpy()
+        after_plain = plain.get_weights().numpy()
+        if not np.array_equal(persistent, after_plain):
+            bad.append(("persistent", call, float(np.abs(persistent - after_plain).max())))
+        shown = noisy.get_weights().numpy()
+        changed = shown != before_shown
+        stepped = after_plain != before_plain                      # a step was taken (hard bounds are far away)
+        if (stepped & ~changed).any():
+            bad.append(("not redrawn", call, int((stepped & ~changed).sum())))
+        # a cross-point that saw pulses which cancelled is redrawn too, one that saw none never is
+        silent = (np.abs(x).sum(axis=0) == 0)[None, :] | (np.abs(d).sum(axis=0) == 0)[:, None]
+        if (changed & silent).any():
+            bad.append(("redrawn without pulses", call, int((changed & silent).sum())))
+        z = (shown - persistent)[changed] / (std * 0.002)
+        if z.size > 400 and (abs(z.mean()) > 5 / np.sqrt(z.size) or abs(z.std() - 1) > 5 / np.sqrt(2 * z.size)):
+            bad.append(("moments", call, float(z.mean()), float(z.std()), int(z.size)))
+    return not bad, dict(seed=seed, X=x_size, D=d_size, B=batch, pulse=str(pulse_type), bl=bl, bad=bad)
+
+
+def test_random_write_noise_cases(gpu_device):
+    """Write noise over shapes that straddle the tile edges, batches of one to nine 32-sample chunks and three pulse
+    types: the persistent weights equal the weights of the same device without write noise bit for bit (same seed),
+    every cross-point that stepped shows a new value, none without pulses does, residuals are N(0, (std dw_min)^2)."""
+    failures = [desc for ok, desc in (one_write_noise(seed) for seed in range(93000, 93080)) if not ok]
+    assert not failures, failures[:3]
