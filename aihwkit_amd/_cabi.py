@@ -145,6 +145,8 @@ SYMBOLS = {
     "rpu_tile_remap_weights": (C.c_int, [_P, C.POINTER(RemapParams), _P, _P]),
     "rpu_tile_modify_weights": (C.c_int, [_P, C.POINTER(ModifierParams), _P]),
     "rpu_tile_get_modified_weights": (C.c_int, [_P, _P]),
+    "rpu_tile_get_read_asymmetry": (C.c_int, [_P, C.c_int, _P]),
+    "rpu_tile_set_read_asymmetry": (C.c_int, [_P, C.c_int, _P]),
     "rpu_tile_pulse_counter_count": (C.c_int, [_P]),
     "rpu_tile_get_pulse_counters": (C.c_int, [_P, _P]),
     "rpu_tile_set_shared_weights": (C.c_int, [_P, _P]),

@@ -113,6 +113,7 @@ void launch_conv_forward(const MvmArgs &a, const ConvArgs &c, hipStream_t s);
 void launch_side_rows(const float *xq, float *out, int rows, int k_pad, int K, int mode, int part, const int *skip_if_zero,
                       hipStream_t s);
 void launch_abs_copy(const float *w, float *out, size_t n, hipStream_t s);
+void launch_mul_copy(const float *w, const float *factors, float *out, size_t n, hipStream_t s); // out = w * factors
 struct SideDev {
   int w_noise_type; // 0 none, 1 additive constant (row_sumsq), 2 PCM read (s_noise)
   float w_noise, ir_drop, a_scale; // a_scale = in_size / ir_drop_g_ratio

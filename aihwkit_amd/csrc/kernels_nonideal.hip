@@ -45,6 +45,12 @@ __global__ __launch_bounds__(256) void k_abs_copy(const float *w, float *out, si
   }
 }
 
+__global__ __launch_bounds__(256) void k_mul_copy(const float *w, const float *f, float *out, size_t n) {
+  for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+    out[i] = w[i] * f[i];
+  }
+}
+
 // four outputs per thread (one Philox call)
 __global__ __launch_bounds__(256) void k_side_combine(float *pre, const float *s_noise, const float *row_sumsq,
                                                        const float *s_cur, const float *s_ir, SideDev p, int rows, int O,
@@ -116,6 +122,10 @@ void launch_side_rows(const float *xq, float *out, int rows, int k_pad, int K, i
 
 void launch_abs_copy(const float *w, float *out, size_t n, hipStream_t s) {
   hipLaunchKernelGGL(k_abs_copy, dim3(grid_for(n)), dim3(256), 0, s, w, out, n);
+}
+
+void launch_mul_copy(const float *w, const float *factors, float *out, size_t n, hipStream_t s) {
+  hipLaunchKernelGGL(k_mul_copy, dim3(grid_for(n)), dim3(256), 0, s, w, factors, out, n);
 }
 
 void launch_side_combine(float *pre, const float *s_noise, const float *row_sumsq, const float *s_cur, const float *s_ir,

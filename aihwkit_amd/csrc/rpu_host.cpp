@@ -55,9 +55,6 @@ void IOPar::initialize(bool backward) {
   if (p.w_noise_type < 0 || p.w_noise_type > 2) {
     throw RpuError("Output noise type not implemented");
   }
-  if (p.w_read_asymmetry_dtod > 0.0f) {
-    throw RpuError("w_read_asymmetry_dtod (weights of the negative pass of PosNegSeparate) is not implemented on this path.");
-  }
   switch (p.noise_management) {
   case RPU_NM_NONE:
   case RPU_NM_ABS_MAX:
@@ -101,10 +98,11 @@ void IOPar::initialize(bool backward) {
 // Per-line values of the periphery (ForwardBackwardPassIOManaged::populateFBParameter,
 // rpu_forward_backward_pass.cpp:254-318): voltage offsets, non-linearity coefficients with the slope calibration
 // factor, and output noise levels.  The reference draws them from the tile's run-time generator; any stream will do.
-void IOPar::populate_lines(int out_size, unsigned int seed) {
+void IOPar::populate_lines(int out_size, unsigned int seed, size_t n_weights) {
   v_offset.clear();
   out_nl.clear();
   out_noise_values.clear();
+  w_asymmetry.clear();
   nl_factor = 1.0f;
   if (perfect) return;
   ConstructionRng rng(seed); // 0: from the clock
@@ -120,6 +118,10 @@ void IOPar::populate_lines(int out_size, unsigned int seed) {
     }
   }
   set_nl_factor();
+  if (p.w_read_asymmetry_dtod != 0.0f) {
+    w_asymmetry.resize(n_weights);
+    for (float &v : w_asymmetry) v = 1.0f + p.w_read_asymmetry_dtod * rng.normal();
+  }
   if (p.out_noise_std > 0.0f) {
     out_noise_values.resize(out_size);
     for (float &v : out_noise_values) v = fabsf(p.out_noise * (1.0f + p.out_noise_std * rng.normal()));

@@ -23,6 +23,7 @@ struct IOPar {
   void initialize(bool backward); // rpu_pulsed_meta_parameter.cpp:39-128
   // per-output-line values of the periphery (MVParameter, rpu_forward_backward_pass.h:17-26); empty when off
   std::vector<float> v_offset, out_nl, out_noise_values;
+  std::vector<float> w_asymmetry; // [d_size][x_size] factors of the negative pass (PosNegSeparate), empty when off
   float nl_factor = 1.0f;
   bool has_voltage_offsets() const { return !perfect && (p.v_offset_std > 0.0f || p.r_series > 0.0f); }
   bool has_nl_calibration() const { return !perfect && (p.out_nonlinearity > 0.0f || p.r_series > 0.0f); }
@@ -31,7 +32,7 @@ struct IOPar {
   bool has_line_terms() const {
     return has_voltage_offsets() || has_nl_calibration() || (!perfect && p.out_noise_std > 0.0f) || separate_passes();
   }
-  void populate_lines(int out_size, unsigned int seed);
+  void populate_lines(int out_size, unsigned int seed, size_t n_weights = 0);
   void set_nl_factor(); // from out_nl: after sampling and after the values were set from outside
 };
 

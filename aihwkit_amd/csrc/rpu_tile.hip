@@ -191,8 +191,10 @@ struct Tile {
   // analog non-idealities before the ADC: the addend per output, up to three side contractions, the transformed
   // input rows, |W| and the squared row norms
   DevBuf<float> n_pre, n_s1, n_s2, n_s3, n_s4, n_rows, n_absw, n_sumsq, n_xsum, n_part, n_neg;
-  DevBuf<float> d_line[2][3]; // per direction: voltage offsets, non-linearity coefficients, output noise levels
-  bool line_valid[2][3] = {{false, false, false}, {false, false, false}};
+  // per direction: voltage offsets, non-linearity coefficients, output noise levels, read-asymmetry factors
+  DevBuf<float> d_line[2][4];
+  bool line_valid[2][4] = {{false, false, false, false}, {false, false, false, false}};
+  DevBuf<float> n_wneg, n_absneg; // weights of the negative pass with read asymmetry, and their absolute values
   // running AverageAbsMax noise-management scale, one value shared by forward and backward as in the reference
   // (rpu_forward_backward_pass.h:241); negative: not started
   DevBuf<float> nm_aux;
@@ -280,6 +282,8 @@ struct Tile {
     n_xsum.release();
     n_part.release();
     n_neg.release();
+    n_wneg.release();
+    n_absneg.release();
     for (auto &dir : d_line) for (auto &b : dir) b.release();
     for (auto &dir : line_valid) for (bool &v : dir) v = false;
     nm_aux.release();
@@ -446,8 +450,8 @@ struct Tile {
 
   // per-line values of both directions; a fixed construction seed fixes them too
   void populate_lines(unsigned int construction_seed) {
-    fio.populate_lines(D, construction_seed ? construction_seed * 2654435761u + 1u : 0u);
-    bio.populate_lines(X, construction_seed ? construction_seed * 2654435761u + 2u : 0u);
+    fio.populate_lines(D, construction_seed ? construction_seed * 2654435761u + 1u : 0u, size());
+    bio.populate_lines(X, construction_seed ? construction_seed * 2654435761u + 2u : 0u, size());
   }
 
   // device copies of the per-line values of a direction (0 forward, 1 backward)
@@ -485,6 +489,20 @@ struct Tile {
     const bool separate = io.separate_passes();
     for (int pass = 0; pass < (separate ? 2 : 1); ++pass) {
       const int part = separate ? (pass == 0 ? -1 : 1) : 0;
+      // the negative pass reads every weight through its own asymmetry factor (rpu_forward_backward_pass.cpp:845-856)
+      const float *w_pass = a.w, *absw_pass = n_absw.p;
+      if (part < 0 && io.p.w_read_asymmetry_dtod > 0.0f && !io.w_asymmetry.empty()) {
+        if (r == 0) {
+          n_wneg.ensure(size());
+          launch_mul_copy(a.w, line_values(a.transposed ? 1 : 0, 3, io.w_asymmetry), n_wneg.p, size(), s);
+          if (need_abs) {
+            n_absneg.ensure(size());
+            launch_abs_copy(n_wneg.p, n_absneg.p, size(), s);
+          }
+        }
+        w_pass = n_wneg.p;
+        absw_pass = n_absneg.p;
+      }
       const float *xin = xq;
       if (part) {
         n_part.ensure(row_n);
@@ -510,12 +528,12 @@ struct Tile {
         launch_row_stat(xin, a.k_pad, B, a.K, 1, n_sumsq.p, s);
       } else if (noisy) {
         n_s1.ensure(out_n);
-        contract(n_absw.p, 0, n_s1.p);
+        contract(absw_pass, 0, n_s1.p);
       }
       if (ir) {
         n_s2.ensure(out_n); n_s3.ensure(out_n);
-        contract(n_absw.p, 1, n_s2.p);
-        contract(a.w, 2, n_s3.p);
+        contract(absw_pass, 1, n_s2.p);
+        contract(w_pass, 2, n_s3.p);
       }
       SideDev p{};
       p.w_noise_type = noisy ? io.p.w_noise_type : 0;
@@ -525,7 +543,7 @@ struct Tile {
         // the value itself is made beside the round kernel, whose ADC stage then only quantizes and clips
         const int dir = a.transposed ? 1 : 0;
         n_s4.ensure(out_n);
-        contract(a.w, 3, n_s4.p);
+        contract(w_pass, 3, n_s4.p);
         p.s_y = n_s4.p;
         if (io.has_voltage_offsets()) {
           p.v_offset = line_values(dir, 0, io.v_offset);
@@ -1488,6 +1506,37 @@ int rpu_tile_get_modified_weights(rpu_tile_t *tile, float *w_host) {
     DeviceGuard g(t.device_id);
     t.sync_last();
     RPU_HIP_CHECK(hipMemcpy(w_host, t.d_fbw.p, t.size() * sizeof(float), hipMemcpyDeviceToHost));
+  });
+}
+
+static std::vector<float> &read_asymmetry_of(Tile &t, int backward) {
+  IOPar &io = backward ? t.bio : t.fio;
+  if (io.w_asymmetry.empty()) throw RpuError("No read asymmetry factors: w_read_asymmetry_dtod of this direction is 0.");
+  return io.w_asymmetry;
+}
+
+int rpu_tile_get_read_asymmetry(rpu_tile_t *tile, int backward, float *factors_host) {
+  return guarded([&] {
+    if (!tile || !factors_host) throw RpuError("null argument");
+    Tile &t = tile->t;
+    std::lock_guard<std::mutex> lock(t.mutex);
+    const std::vector<float> &v = read_asymmetry_of(t, backward);
+    std::memcpy(factors_host, v.data(), v.size() * sizeof(float));
+  });
+}
+
+int rpu_tile_set_read_asymmetry(rpu_tile_t *tile, int backward, const float *factors_host) {
+  return guarded([&] {
+    if (!tile || !factors_host) throw RpuError("null argument");
+    Tile &t = tile->t;
+    std::lock_guard<std::mutex> lock(t.mutex);
+    std::vector<float> &v = read_asymmetry_of(t, backward);
+    if (t.resident()) {
+      DeviceGuard g(t.device_id);
+      t.sync_last(); // a call in flight may still read the device copy that the next call replaces
+    }
+    std::memcpy(v.data(), factors_host, v.size() * sizeof(float));
+    t.line_valid[backward ? 1 : 0][3] = false;
   });
 }
 

@@ -108,6 +108,19 @@ class _TileBase:
     remap_weights = _needs_gpu
     modify_weights = _needs_gpu
 
+    def get_read_asymmetry(self, backward: bool = False) -> torch.Tensor:
+        """[d_size, x_size] factors of the negative pass of PosNegSeparate (the reference's ``fwd.w_asymmetry`` /
+        ``bwd.w_asymmetry`` state entries, rpu_forward_backward_pass.cpp:62-100)."""
+        out = torch.empty(self.get_d_size(), self.get_x_size(), dtype=_DTYPE)
+        check(lib().rpu_tile_get_read_asymmetry(self._h, int(bool(backward)), out.data_ptr()))
+        return out
+
+    def set_read_asymmetry(self, factors: torch.Tensor, backward: bool = False) -> None:
+        factors = _check_input(factors, False, "factors")
+        if tuple(factors.shape) != (self.get_d_size(), self.get_x_size()):
+            raise RuntimeError("Invalid dimensions of the read asymmetry factors")
+        check(lib().rpu_tile_set_read_asymmetry(self._h, int(bool(backward)), factors.data_ptr()))
+
     def get_pulse_counters(self) -> torch.Tensor:
         """int64 [2, d_size, x_size] (up-counting pulses where the signs of x and d agree, then where they differ)
         of a tile whose device has ``count_pulses`` set, else an empty tensor (rpu_base_tiles.cpp:845-868)."""

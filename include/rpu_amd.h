@@ -124,7 +124,7 @@ typedef struct rpu_io_params {
   float out_nonlinearity_std;     /* 0 */
   float v_offset_std;             /* 0: voltage offset per output line, max(v_offset_std xi, 0) (:436-506) */
   float r_series;                 /* 0: series resistance, y -> y / (1 + min(r_series |y|, r_series_max_total)) */
-  float w_read_asymmetry_dtod;    /* 0; not provided (weights of the negative pass of the PosNegSeparate types) */
+  float w_read_asymmetry_dtod;    /* 0: the negative pass of PosNegSeparate reads w_ij (1 + dtod xi_ij) (:845-856) */
   float ir_drop_g_ratio;          /* 5.7143e5: wire conductance over g_max (ir_drop_Gw_div_gmax) */
   float nm_decay;                 /* 1e-3: weight of a new sample in the AverageAbsMax running average */
   float slope_calibration;        /* 0.5: y / out_bound at which the non-linearity has slope 1 on average (:283-295) */
@@ -547,6 +547,13 @@ typedef struct rpu_modifier_params {
 int rpu_tile_modify_weights(rpu_tile_t *tile, const rpu_modifier_params *p, void *stream);
 /* Host copy [d_size][x_size] of the modified weights; returns an error if none have been made. */
 int rpu_tile_get_modified_weights(rpu_tile_t *tile, float *w_host);
+
+/* The per-cross-point factors (1 + w_read_asymmetry_dtod xi) of the negative pass of PosNegSeparate, drawn at creation:
+ * the "fwd.w_asymmetry" / "bwd.w_asymmetry" entries of the reference's state (R/rpu_forward_backward_pass.cpp:62-100,
+ * :297-304).  backward = 0 / 1 selects the direction; [d_size][x_size] host floats, the layout of the weights.
+ * Fails when w_read_asymmetry_dtod of that direction is 0 (there are no factors). */
+int rpu_tile_get_read_asymmetry(rpu_tile_t *tile, int backward, float *factors_host);
+int rpu_tile_set_read_asymmetry(rpu_tile_t *tile, int backward, const float *factors_host);
 
 /* get_pulse_counters (rpu_base_tiles.cpp:845-868, src/rpucuda/cuda/rpucuda_pulsed_device.cu:316-343): with
  * count_pulses set in the device parameters every pulsed update adds, per cross-point, the number of up and of

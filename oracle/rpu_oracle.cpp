@@ -173,10 +173,6 @@ bool init_io(OrcIO &io, bool backward) {
     g_err = "Output noise type not implemented";
     return false;
   }
-  if (p.w_read_asymmetry_dtod > 0.f) {
-    g_err = "oracle: w_read_asymmetry_dtod (PosNegSeparate MV types) not restated";
-    return false;
-  }
   return true;
 }
 
@@ -205,6 +201,7 @@ struct OrcTile {
   // R/rpu_forward_backward_pass.h:17-26 MVParameter of the forward [0] and backward [1] pass
   struct Lines {
     std::vector<float> v_offset, out_nl, out_noise;
+    std::vector<float> w_asymmetry; // [D][X] factors of the negative pass of PosNegSeparate
     float nl_factor = 1.0f;
   } lines[2];
   float aux_nm = -1.0f; // running AverageAbsMax scale (R/rpu_forward_backward_pass.h:241), negative: not started
@@ -536,6 +533,10 @@ void populate_lines(OrcTile &t, const rpu_io_params &io, OrcTile::Lines &mv, int
     }
   }
   set_nl_factor(io, mv, out_size);
+  if (io.w_read_asymmetry_dtod != 0.0f) { // :297-304
+    mv.w_asymmetry.resize((size_t)t.X * t.D);
+    for (float &v : mv.w_asymmetry) v = 1.0f + io.w_read_asymmetry_dtod * t.rng.gauss();
+  }
   if (io.out_noise_std > 0.0f) {
     mv.out_noise.resize(out_size);
     for (int i = 0; i < out_size; ++i) mv.out_noise[i] = std::fabs(io.out_noise * (1.0f + io.out_noise_std * t.rng.gauss()));
@@ -661,7 +662,16 @@ bool analog_mv(OrcTile &t, const float *in, int in_size, int in_inc, float *out,
     // first the negative inputs, then the positive ones; the sums of both passes go through the ADC (:832-893)
     std::vector<float> part((size_t)in_size), neg_out((size_t)out_size);
     for (int i = 0; i < in_size; ++i) part[i] = t.in_buf[i] < 0.0f ? t.in_buf[i] : 0.0f;
-    analog_mv_single_pass(t, part.data(), in_size, neg_out.data(), out_size, 1, io, transposed);
+    if (io.w_read_asymmetry_dtod > 0.0f) {
+      // the negative pass reads w_ij * asymmetry_ij, contraction and non-idealities alike (:845-860)
+      std::vector<float> neg_w(t.w.size());
+      for (size_t i = 0; i < neg_w.size(); ++i) neg_w[i] = t.w[i] * mv.w_asymmetry[i];
+      t.w.swap(neg_w);
+      analog_mv_single_pass(t, part.data(), in_size, neg_out.data(), out_size, 1, io, transposed);
+      t.w.swap(neg_w);
+    } else {
+      analog_mv_single_pass(t, part.data(), in_size, neg_out.data(), out_size, 1, io, transposed);
+    }
     for (int i = 0; i < in_size; ++i) part[i] = t.in_buf[i] > 0.0f ? t.in_buf[i] : 0.0f;
     analog_mv_single_pass(t, part.data(), in_size, out, out_size, out_inc, io, transposed);
     for (int j = 0; j < out_size; ++j) out[(size_t)j * out_inc] += neg_out[j];
@@ -1170,11 +1180,12 @@ void orc_set_weights(void *h, const float *w) { // R/rpu_pulsed.cpp:288-292
   clip_to_bounds(*t);
   on_set_weights(*t);
 }
-// per-line values of the periphery: dir 0 forward / 1 backward; which 0 v_offset, 1 out_nonlinearity, 2 out_noise_values
+// per-line values of the periphery: dir 0 forward / 1 backward; which 0 v_offset, 1 out_nonlinearity, 2 out_noise_values,
+// 3 w_asymmetry ([D][X])
 // (the entries of the reference's state, R/rpu_forward_backward_pass.cpp:62-100).  Returns the length.
 static std::vector<float> &line_vector(OrcTile &t, int dir, int which) {
   OrcTile::Lines &mv = t.lines[dir ? 1 : 0];
-  return which == 0 ? mv.v_offset : (which == 1 ? mv.out_nl : mv.out_noise);
+  return which == 0 ? mv.v_offset : (which == 1 ? mv.out_nl : (which == 2 ? mv.out_noise : mv.w_asymmetry));
 }
 int orc_get_lines(void *h, int dir, int which, float *out) {
   auto *t = static_cast<OrcTile *>(h);

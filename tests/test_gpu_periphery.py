@@ -192,6 +192,41 @@ def test_separate_passes_without_nonlinear_terms_and_their_noise(gpu_device):
     assert moments_ok((y - x64 @ w64.T) / 0.2)
 
 
+def test_read_asymmetry_of_the_negative_pass(gpu_device):
+    rng = np.random.default_rng(6)
+    for x_size, d_size, batch in ((37, 23, 50), (300, 200, 96)):
+        x = rng.uniform(-1, 1, (batch, x_size)).astype(F)
+        d = rng.normal(0, 0.5, (batch, d_size)).astype(F)
+        io = dict(mv_type=PNS, w_read_asymmetry_dtod=0.3, ir_drop=1.0, ir_drop_g_ratio=x_size * (0.3 * 0.5 * x_size) / 0.5,
+                  out_bound=float(0.2 * np.sqrt(x_size)), noise_management=dv.NoiseManagementType.AbsMax,
+                  bound_management=dv.BoundManagementType.Iterative)
+        orc, gpu, w = pair(x_size, d_size, **io)
+        plain, _g, _w = pair(x_size, d_size, **dict(io, w_read_asymmetry_dtod=0.0))
+        for direction in (0, 1):
+            factors = gpu.get_read_asymmetry(bool(direction)).numpy()
+            assert factors.shape == (d_size, x_size) and abs(factors.std() / 0.3 - 1) < 0.1
+            orc.set_lines(direction, 3, factors.ravel())
+        assert not np.array_equal(gpu.get_read_asymmetry(False).numpy(), gpu.get_read_asymmetry(True).numpy())
+        want = orc.forward(x)
+        got = gpu.forward(torch.from_numpy(x).cuda()).cpu().numpy()
+        assert np.abs(got - want).max() <= 1e-5 * np.abs(want).max()
+        assert np.array_equal(gpu.get_bm_rounds(batch).numpy(), orc.bm_rounds(batch))
+        assert np.abs(want - plain.forward(x)).max() > 1e-2 * np.abs(want).max()
+        want_b = orc.backward(d)
+        got_b = gpu.backward(torch.from_numpy(d).cuda()).cpu().numpy()
+        assert np.abs(got_b - want_b).max() <= 1e-5 * np.abs(want_b).max()
+        # factors set from outside: all ones is the tile without asymmetry
+        ones = torch.ones(d_size, x_size)
+        gpu.set_read_asymmetry(ones, False)
+        got1 = gpu.forward(torch.from_numpy(x).cuda()).cpu().numpy()
+        assert np.abs(got1 - plain.forward(x)).max() <= 1e-5 * np.abs(got1).max()
+        twin = copy.deepcopy(gpu)
+        assert np.array_equal(twin.get_read_asymmetry(True).numpy(), gpu.get_read_asymmetry(True).numpy())
+    _o, off, _w = pair(8, 8, mv_type=PNS)
+    with pytest.raises(RuntimeError, match="No read asymmetry factors"):
+        off.get_read_asymmetry(False)
+
+
 def test_line_values_are_state(gpu_device):
     """They are fixed by the construction seed, travel with copies and the extra state, and can be set."""
     io = dict(v_offset_std=0.2, out_nonlinearity=0.6, out_nonlinearity_std=0.25, out_noise_std=0.5, out_noise=0.0,
@@ -228,7 +263,5 @@ def test_line_terms_are_refused_where_they_are_not_provided(gpu_device):
     tr.transfer_forward.v_offset_std = 0.1
     with pytest.raises(Exception, match="not provided for the read of a transfer"):
         make_meta().create_array(8, 8, tr)
-    with pytest.raises(Exception, match="PosNegSeparate"):
-        pair(8, 8, w_read_asymmetry_dtod=0.1)
     with pytest.raises(Exception, match="AnalogMVType not implemented"):
         pair(8, 8, mv_type=dv.AnalogMVType.PosNegSeparateDigitalSum)

@@ -188,3 +188,33 @@ def test_pos_neg_separate_passes():
     # backward takes the same path
     t = oracle_tile(1, 2, [[1.0], [1.0]], mv_type=pns, **kw)
     assert abs(t.backward(np.array([[0.8, -0.3]], dtype=F))[0, 0] - (0.8 / 1.4 - 0.3 / 1.15)) < 1e-6
+
+
+def test_read_asymmetry_of_the_negative_pass():
+    pns = dv.AnalogMVType.PosNegSeparate
+    # w = [1, 1], factors [2, 3], x = [0.8, -0.3]: only the negative input reads its weight through the factor
+    t = oracle_tile(2, 1, [[1.0, 1.0]], mv_type=pns, w_read_asymmetry_dtod=0.1)
+    assert t.get_lines(0, 3).shape == (2,) and t.get_lines(1, 3).shape == (2,)
+    t.set_lines(0, 3, [2.0, 3.0])
+    assert abs(t.forward(np.array([[0.8, -0.3]], dtype=F))[0, 0] - (0.8 - 0.9)) < 1e-6
+    assert abs(t.forward(np.array([[-0.8, 0.3]], dtype=F))[0, 0] - (-1.6 + 0.3)) < 1e-6
+    # the IR drop of the negative pass sees the scaled conductances too: one line, closed form with w -> 2 w
+    n, ratio = 4, 10.0
+    t = oracle_tile(n, 1, np.full((1, n), 0.5), mv_type=pns, w_read_asymmetry_dtod=0.1, ir_drop=1.0, ir_drop_g_ratio=ratio)
+    t.set_lines(0, 3, np.full(n, 2.0))
+    x = np.zeros((1, n), dtype=F)
+    x[0, 2] = -0.6
+    a = n / ratio * 1.0 * 0.6
+    want = -0.6 * (1.0 - a * (a * (0.05 * a - 0.2) + 0.5) * (1.0 - (1.0 - 2 / n) ** 2))
+    assert abs(t.forward(x)[0, 0] - want) < 1e-6
+    # one pass does not read the factors; the drawn ones are 1 + dtod xi, both directions their own
+    t = oracle_tile(2, 1, [[1.0, 1.0]], w_read_asymmetry_dtod=0.1)
+    t.set_lines(0, 3, [2.0, 3.0])
+    assert abs(t.forward(np.array([[0.8, -0.3]], dtype=F))[0, 0] - 0.5) < 1e-6
+    t = oracle_tile(100, 100, np.zeros((100, 100)), mv_type=pns, w_read_asymmetry_dtod=0.2)
+    f, b = t.get_lines(0, 3).astype(np.float64), t.get_lines(1, 3).astype(np.float64)
+    assert abs(f.mean() - 1) < 4 * 0.2 / 100 + 0.2 * 0.03 and abs(f.std() / 0.2 - 1) < 0.05 and not np.array_equal(f, b)
+    # backward: the factors keep the layout of the weights
+    t = oracle_tile(1, 2, [[1.0], [1.0]], mv_type=pns, w_read_asymmetry_dtod=0.1)
+    t.set_lines(1, 3, [2.0, 3.0])
+    assert abs(t.backward(np.array([[0.8, -0.3]], dtype=F))[0, 0] - (0.8 - 0.9)) < 1e-6
