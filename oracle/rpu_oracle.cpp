@@ -11,10 +11,9 @@
 // R/math_util.h, which needs a cblas.h or mkl.h header that the image does not have, so this file is
 // pinned by closed forms, brute force on small cases and invariants (see tests/test_oracle_*.py).
 //
-// parity unpinned: populate_pulsed() / populate_linear_step() -- the exact draw order of the
-// device-to-device parameters (R/rpu_pulsed_device.cpp:593-733, R/rpu_linearstep_device.cpp:20-74)
-// can only be pinned bit-for-bit by running the reference; here it is checked through its
-// distributional properties and through the relations between the drawn arrays only.
+// The draw order of the device-to-device parameters in populate_pulsed() / populate_linear_step()
+// (R/rpu_pulsed_device.cpp:593-733, R/rpu_linearstep_device.cpp:20-74) is pinned against the raw libstdc++
+// stream (tests/rawstream.cpp, tests/test_draw_order_pins.py), cross-point by cross-point.
 //
 // Layout: weights and all per-device arrays are row-major [d_size][x_size] (R/rpu.h:674).
 // Built with -O2 -ffp-contract=off so that every expression is evaluated with the reference's

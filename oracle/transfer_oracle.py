@@ -13,8 +13,9 @@ TransferRPUDevice::doSparseUpdate / finishUpdateCycle):
   device j + 1 with learning rate transfer_lr (x current lr) (rpu_transfer_device.cpp:428-516,536-557);
 * tile weights = sum_k gamma_k w_k, or the last device alone when gamma = 0 (rpu_transfer_device.cpp:596-602).
 
-parity unpinned: like the single-device oracle, the draw order of the sampled device arrays is not pinned;
-tests copy the arrays from the library through the hidden-parameter interface.
+This oracle samples nothing itself: tests copy the device arrays from the library through the hidden-parameter
+interface, and the library's draw order for a chain (one generator walked device by device,
+rpu_vector_device.cpp:398-418) is pinned against the raw libstdc++ stream in tests/test_draw_order_pins.py.
 """
 import copy
 import math

@@ -366,7 +366,7 @@ def test_floating_point_update_is_rank_b_sgd():
 
 
 # ------------------------------------------------------------------------------------------------
-# device construction (draw order itself is "parity unpinned"; these pin everything around it)
+# device construction (the draw order is pinned in test_draw_order_pins.py; these pin distributions and relations)
 
 
 def test_populated_arrays_have_the_configured_distributions_and_relations():
