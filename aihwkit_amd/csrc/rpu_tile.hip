@@ -17,6 +17,11 @@
 #include <string>
 #include <vector>
 
+// Scratch of rpu_tile_update_noalloc, the entry point for callers that cannot allocate: one array per GPU the
+// library runs on, held until the process ends.  Host code never uses the array's name as an address: the device
+// address is looked up once per device (noalloc_scratch) and only that pointer is passed on.
+static __device__ __align__(256) unsigned char scratch[RPU_NOALLOC_MAX_SCRATCH_BYTES];
+
 namespace rpu_amd {
 
 #define RPU_HIP_CHECK(expr)                                                                         \
@@ -80,6 +85,25 @@ __global__ void k_philox_probe(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c
   out[1] = r.v[1];
   out[2] = r.v[2];
   out[3] = r.v[3];
+}
+
+__global__ void k_init_kmax(int *kmax) {
+  if (threadIdx.x < 4) kmax[threadIdx.x] = threadIdx.x == 2 ? 31 : 0;
+}
+
+// device address of the static scratch array on the current device, looked up at the first call per device
+unsigned char *noalloc_scratch(int device) {
+  static std::mutex m;
+  static unsigned char *ptr[64] = {};
+  if (device < 0 || device >= 64) throw RpuError("Device number out of range for the static scratch array.");
+  std::lock_guard<std::mutex> lock(m);
+  if (!ptr[device]) {
+    unsigned char *p = nullptr;
+    RPU_HIP_CHECK(hipGetSymbolAddress((void **)&p, HIP_SYMBOL(scratch)));
+    if (!p) throw RpuError("The static scratch array has no device address.");
+    ptr[device] = p;
+  }
+  return ptr[device];
 }
 
 const char *const kHiddenNames[10] = {"max_bound",       "min_bound",  "dwmin_up", "dwmin_down", "decay_scales",
@@ -155,6 +179,10 @@ struct Tile {
   DevBuf<uint32_t> u_xw, u_dw, u_xpl, u_dpl;
   DevBuf<int> u_kmax;
   uint32_t update_calls = 0;
+  // where the last pulsed update left its per-sample values and packed words (own buffers or the static scratch)
+  int *last_bl = nullptr;
+  float *last_a = nullptr, *last_b = nullptr;
+  uint32_t *last_xw = nullptr, *last_dw = nullptr;
   // transfer compound (rpu_transfer_device.{h,cpp}): device 0 takes the gradient update, device j is read
   // column by column and written onto device j + 1; the tile's weights d_w are the weighted sum, or the
   // last device itself when that one alone is visible
@@ -269,6 +297,7 @@ struct Tile {
     s_rounds.release(); s_hitup.release(); s_hitlo.release(); s_list0.release(); s_list1.release(); s_row0.release(); s_row1.release(); s_count.release(); s_tiledone.release();
     u_bl.release(); u_a.release(); u_b.release(); u_xval.release(); u_dval.release(); u_xw.release(); u_dw.release();
     u_xpl.release(); u_dpl.release(); u_kmax.release();
+    last_bl = nullptr; last_a = last_b = nullptr; last_xw = last_dw = nullptr;
     t_unit.release(); t_read.release();
     i_ref.release(); i_prog.release(); i_nu_plus.release(); i_nu_minus.release(); i_scalar.release(); i_absmax.release();
     has_reference = programmed = false;
@@ -641,6 +670,30 @@ struct Tile {
     if (!transposed && !w_other) last_forward_batch = B;
   }
 
+  // Carves the scratch of a stochastic pulsed update out of a caller-provided block (256-byte aligned parts) and
+  // returns the bytes used; with base == nullptr only the size is computed.
+  static size_t carve_update_scratch(unsigned char *base, int X, int D, int B, bool bias, UpdateArgs *a, float **bias_rows) {
+    size_t off = 0;
+    auto take = [&](size_t bytes) {
+      unsigned char *p = base ? base + off : nullptr;
+      off += (bytes + 255) & ~(size_t)255;
+      return p;
+    };
+    const size_t chunks = ((size_t)B + 31) / 32, slots = 32;
+    int *kmax = (int *)take(4 * sizeof(int));
+    int *bl = (int *)take((size_t)B * 4);
+    float *pa = (float *)take((size_t)B * 4), *pb = (float *)take((size_t)B * 4);
+    uint32_t *xw = (uint32_t *)take((size_t)B * X * 4), *dw = (uint32_t *)take((size_t)B * D * 4);
+    uint32_t *xpl = (uint32_t *)take(chunks * slots * X * 4), *dpl = (uint32_t *)take(chunks * slots * D * 4);
+    float *rows = bias ? (float *)take((size_t)B * X * 4) : nullptr;
+    if (a) {
+      a->kmax = kmax; a->bl = bl; a->prob_a = pa; a->prob_b = pb; a->x_words = xw; a->d_words = dw;
+      a->x_planes = xpl; a->d_planes = dpl; a->plane_slots = (int)slots; a->n_chunks = (int)chunks;
+    }
+    if (bias_rows) *bias_rows = rows;
+    return off;
+  }
+
   void set_plane_args(UpdateArgs &a, int B) {
     const int slots = 32; // 31 pulse slots and the sign plane
     const int chunks = (B + 31) / 32;
@@ -983,8 +1036,9 @@ struct Tile {
   }
 
   // pulsed update of one device matrix (rpu_weight_updater.cpp:197-294)
+  // ws != nullptr: the per-call scratch is carved out of that block and nothing is allocated (stochastic pulses only)
   void pulsed_update_on(const DeviceView &dv, const UpdatePar &up, float lr, const float *xin, long x_sb, long x_sj,
-                        const float *d, long d_sb, long d_si, int B, hipStream_t s) {
+                        const float *d, long d_sb, long d_si, int B, hipStream_t s, unsigned char *ws = nullptr) {
     if (lr == 0.0f) return;
     const DevicePar &dev = *dv.par;
     UpdateArgs a{};
@@ -1000,17 +1054,24 @@ struct Tile {
     a.dev.w_max = const_cast<float *>(dv.w_max); a.dev.w_min = const_cast<float *>(dv.w_min);
     a.dev.scale_up = const_cast<float *>(dv.scale_up); a.dev.scale_down = const_cast<float *>(dv.scale_down);
     a.dev.slope_up = const_cast<float *>(dv.slope_up); a.dev.slope_down = const_cast<float *>(dv.slope_down);
-    u_bl.ensure(B); u_a.ensure(B); u_b.ensure(B);
-    a.bl = u_bl.p; a.prob_a = u_a.p; a.prob_b = u_b.p;
     a.key = key(); a.call = call++;
-    if (up.p.pulse_type == RPU_PULSE_STOCHASTIC_COMPRESSED) {
-      u_xw.ensure((size_t)B * X); u_dw.ensure((size_t)B * D);
-      a.x_words = u_xw.p; a.d_words = u_dw.p;
-      set_plane_args(a, B);
-      a.kmax_slot = (int)(update_calls++ & 1u);
+    if (ws) {
+      carve_update_scratch(ws, X, D, B, false, &a, nullptr);
+      // the array keeps the last call's contents: the largest-BL slots start from zero again
+      hipLaunchKernelGGL(k_init_kmax, dim3(1), dim3(64), 0, s, a.kmax);
+      a.kmax_slot = 0;
     } else {
-      u_xval.ensure((size_t)B * X); u_dval.ensure((size_t)B * D);
-      a.x_val = u_xval.p; a.d_val = u_dval.p;
+      u_bl.ensure(B); u_a.ensure(B); u_b.ensure(B);
+      a.bl = u_bl.p; a.prob_a = u_a.p; a.prob_b = u_b.p;
+      if (up.p.pulse_type == RPU_PULSE_STOCHASTIC_COMPRESSED) {
+        u_xw.ensure((size_t)B * X); u_dw.ensure((size_t)B * D);
+        a.x_words = u_xw.p; a.d_words = u_dw.p;
+        set_plane_args(a, B);
+        a.kmax_slot = (int)(update_calls++ & 1u);
+      } else {
+        u_xval.ensure((size_t)B * X); u_dval.ensure((size_t)B * D);
+        a.x_val = u_xval.p; a.d_val = u_dval.p;
+      }
     }
     prof_begin(s);
     launch_update_prepare(a, s);
@@ -1039,6 +1100,44 @@ struct Tile {
     last_stream = s;
     last_update_batch = B;
     last_update_pulse = up.p.pulse_type;
+    last_bl = a.bl; last_a = a.prob_a; last_b = a.prob_b; last_xw = a.x_words; last_dw = a.d_words;
+  }
+
+  // The stochastic pulsed update without any allocation: every buffer beyond inputs and weights lives in the
+  // static scratch array of this GPU.  Same kernels, same random streams and therefore the same weights as update().
+  void update_noalloc(const float *x, const float *d, int B, bool bias, bool x_trans, bool d_trans, hipStream_t s) {
+    if (!dev.pulsed() || up.p.pulse_type != RPU_PULSE_STOCHASTIC_COMPRESSED) {
+      throw RpuError("update_noalloc is provided for stochastic pulses on a pulsed device only.");
+    }
+    if (is_transfer() || persistent() || delta_w || dev.p.count_pulses) {
+      throw RpuError("update_noalloc is not provided for transfer compounds, write noise, delta weights or pulse counters.");
+    }
+    float *rows = nullptr;
+    const size_t need = carve_update_scratch(nullptr, X, D, B, bias, nullptr, nullptr);
+    if (need > (size_t)RPU_NOALLOC_MAX_SCRATCH_BYTES) {
+      throw RpuError("update_noalloc: this call needs " + std::to_string(need) + " bytes of scratch, the static array holds " +
+                     std::to_string((size_t)RPU_NOALLOC_MAX_SCRATCH_BYTES) + ".");
+    }
+    if (lr == 0.0f) return;
+    unsigned char *ws = noalloc_scratch(device_id);
+    carve_update_scratch(ws, X, D, B, bias, nullptr, &rows);
+    const float *xin = x;
+    long x_sb = x_trans ? 1 : X, x_sj = x_trans ? B : 1;
+    if (bias) {
+      launch_make_bias(x, rows, B, X, x_trans ? 1 : 0, s);
+      xin = rows; x_sb = X; x_sj = 1;
+    }
+    const long d_sb = d_trans ? 1 : D, d_si = d_trans ? B : 1;
+    DeviceView dv{wp_dev(), d_wmax.p, d_wmin.p, d_sup.p, d_sdown.p, d_slup.p, d_sldown.p, &dev, dev.p.dw_min};
+    const bool was_profiling = profiling;
+    profiling = false; // event creation allocates
+    try {
+      pulsed_update_on(dv, up, lr, xin, x_sb, x_sj, d, d_sb, d_si, B, s, ws);
+    } catch (...) {
+      profiling = was_profiling;
+      throw;
+    }
+    profiling = was_profiling;
   }
 
   // ---- indexed (convolution) interface ---------------------------------------------------------------
@@ -2066,6 +2165,18 @@ int rpu_tile_update(rpu_tile_t *tile, const float *x_dev, const float *d_dev, in
   });
 }
 
+int rpu_tile_update_noalloc(rpu_tile_t *tile, const float *x_dev, const float *d_dev, int m_batch, int bias, int x_trans,
+                            int d_trans, void *stream) {
+  return guarded([&] {
+    if (!tile) throw RpuError("null tile");
+    Tile &t = tile->t;
+    std::lock_guard<std::mutex> lock(t.mutex);
+    if (!t.check_compute(m_batch, x_dev, d_dev)) return;
+    DeviceGuard g(t.device_id);
+    t.update_noalloc(x_dev, d_dev, m_batch, bias != 0, x_trans != 0, d_trans != 0, (hipStream_t)stream);
+  });
+}
+
 int rpu_tile_update_with_words(rpu_tile_t *tile, const uint32_t *x_words_dev, const uint32_t *d_words_dev, int m_batch,
                                void *stream) {
   return guarded([&] {
@@ -2349,9 +2460,9 @@ int rpu_tile_get_update_words(rpu_tile_t *tile, uint32_t *x_words_host, uint32_t
     }
     DeviceGuard g(t.device_id);
     t.sync_last();
-    RPU_HIP_CHECK(hipMemcpy(x_words_host, t.u_xw.p, (size_t)m_batch * t.X * 4, hipMemcpyDeviceToHost));
-    RPU_HIP_CHECK(hipMemcpy(d_words_host, t.u_dw.p, (size_t)m_batch * t.D * 4, hipMemcpyDeviceToHost));
-    RPU_HIP_CHECK(hipMemcpy(bl_host, t.u_bl.p, (size_t)m_batch * 4, hipMemcpyDeviceToHost));
+    RPU_HIP_CHECK(hipMemcpy(x_words_host, t.last_xw, (size_t)m_batch * t.X * 4, hipMemcpyDeviceToHost));
+    RPU_HIP_CHECK(hipMemcpy(d_words_host, t.last_dw, (size_t)m_batch * t.D * 4, hipMemcpyDeviceToHost));
+    RPU_HIP_CHECK(hipMemcpy(bl_host, t.last_bl, (size_t)m_batch * 4, hipMemcpyDeviceToHost));
   });
 }
 

@@ -330,9 +330,17 @@ class _CudaTileMixin:
             raise RuntimeError(f"Invalid d_input dimensions: expected {shape} tensor")
         if m_batch != m_batch_from_d:
             raise RuntimeError("Invalid x_input or d_input dimensions: batch dimensions mismatch!")
-        check(lib().rpu_tile_update(self._h, x_input.data_ptr(), d_input.data_ptr(), m_batch, int(bias),
-                                    int(x_trans), int(d_trans), self._stream_for(x_input)))
+        entry = lib().rpu_tile_update_noalloc if self._update_without_allocation else lib().rpu_tile_update
+        check(entry(self._h, x_input.data_ptr(), d_input.data_ptr(), m_batch, int(bias),
+                    int(x_trans), int(d_trans), self._stream_for(x_input)))
         self._finish(x_input, non_blocking)
+
+    _update_without_allocation = False
+
+    def set_update_without_allocation(self, enable: bool) -> None:
+        """Not in the reference: route `update` through the entry point that allocates nothing (scratch in a static
+        device array of limited size, shared by all tiles of the GPU)."""
+        self._update_without_allocation = bool(enable)
 
     # -- inspection hooks
     # -- indexed (convolution) interface (rpu_base_tiles.cpp:621-737)

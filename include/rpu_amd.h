@@ -333,6 +333,22 @@ int rpu_tile_backward(rpu_tile_t *tile, const float *d_dev, float *x_dev, int m_
 int rpu_tile_update(rpu_tile_t *tile, const float *x_dev, const float *d_dev, int m_batch, int bias,
                     int x_trans, int d_trans, void *stream);
 
+/* No counterpart in the reference.  For callers that cannot allocate device memory while they run -- code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc: the same update as rpu_tile_update for
+ * RPU_PULSE_STOCHASTIC_COMPRESSED on a ConstantStep / LinearStep / SoftBounds tile (same kernels, same random
+ * streams, bit-identical weights), but every buffer beyond the inputs and the tile's own matrices (per-sample BL and
+ * probability scales, packed pulse words, bit planes, the rows with the bias column) lives in one static device
+ * array of RPU_NOALLOC_MAX_SCRATCH_BYTES per GPU, which the library holds until the process ends.  The call makes
+ * no hipMalloc / hipFree and records no events; a call whose scratch would not fit
+ * (about 8 * m_batch * (x_size + d_size) bytes, + 4 * m_batch * x_size with bias) fails with a message that names both
+ * sizes and changes nothing.  All tiles on a GPU share that GPU's array: calls that overlap in time on one GPU (other
+ * streams, other threads) race, calls on one stream do not.  Not provided for transfer compounds, write noise, delta
+ * weights and pulse counters (error).  rpu_tile_get_update_words / get_update_ab read this call's words until the
+ * next no-allocation call on the same GPU overwrites them. */
+#define RPU_NOALLOC_MAX_SCRATCH_BYTES (6u << 20)
+int rpu_tile_update_noalloc(rpu_tile_t *tile, const float *x_dev, const float *d_dev, int m_batch, int bias,
+                            int x_trans, int d_trans, void *stream);
+
 /* ---- state ------------------------------------------------------------------------ */
 
 int rpu_tile_get_x_size(const rpu_tile_t *tile); /* R/rpu.h:76 getXSize */
