@@ -97,8 +97,9 @@ __global__ __launch_bounds__(256) void k_update_prepare(UpdateArgs a) {
     if (threadIdx.x != 0) return;
     calc_bl_ab(a.up, BL, A, B, lr, dw_min);
   }
-  // one 32-bit word holds the sign and at most 31 pulses
-  if (BL > 31) BL = 31;
+  // one 32-bit word holds the sign and at most 31 pulses; the host refuses calls whose BL could exceed that, so
+  // this never changes a value -- the implicit pulse types keep no words and take any BL
+  if (a.up.pulse_type == RPU_PULSE_STOCHASTIC_COMPRESSED && BL > 31) BL = 31;
   a.bl[b] = BL;
   // largest BL of the batch: this call's slot was zeroed by the previous call, which used the other one
   if (a.kmax) {

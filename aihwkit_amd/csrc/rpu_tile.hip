@@ -1041,6 +1041,13 @@ struct Tile {
                         const float *d, long d_sb, long d_si, int B, hipStream_t s, unsigned char *ws = nullptr) {
     if (lr == 0.0f) return;
     const DevicePar &dev = *dv.par;
+    // calculateBlAB (rpu_pulsed_meta_parameter.cpp:152-181): without a fixed BL and without BL management a learning
+    // rate beyond dw_min * desired_BL lengthens the bit line to ceil(lr / dw_min); a packed word holds 31 pulses
+    if (up.p.pulse_type == RPU_PULSE_STOCHASTIC_COMPRESSED && !up.p.fixed_bl && !up.p.update_bl_management &&
+        dv.granularity * (float)up.p.desired_bl < fabsf(lr) && ceilf(fabsf(lr) / dv.granularity) > 31.0f) {
+      throw RpuError("This learning rate needs a bit line of " + std::to_string((long)ceilf(fabsf(lr) / dv.granularity)) +
+                     " pulses (fixed_BL and update_bl_management are off); stochastic pulse trains hold at most 31.");
+    }
     UpdateArgs a{};
     a.w = dv.w; a.x_size = X; a.d_size = D; a.m_batch = B;
     a.x = xin; a.x_sb = x_sb; a.x_sj = x_sj; a.d = d; a.d_sb = d_sb; a.d_si = d_si;
@@ -2463,6 +2470,22 @@ int rpu_tile_get_update_words(rpu_tile_t *tile, uint32_t *x_words_host, uint32_t
     RPU_HIP_CHECK(hipMemcpy(x_words_host, t.last_xw, (size_t)m_batch * t.X * 4, hipMemcpyDeviceToHost));
     RPU_HIP_CHECK(hipMemcpy(d_words_host, t.last_dw, (size_t)m_batch * t.D * 4, hipMemcpyDeviceToHost));
     RPU_HIP_CHECK(hipMemcpy(bl_host, t.last_bl, (size_t)m_batch * 4, hipMemcpyDeviceToHost));
+  });
+}
+
+int rpu_tile_get_update_ab(rpu_tile_t *tile, float *a_host, float *b_host, int m_batch) {
+  return guarded([&] {
+    if (!tile || !a_host || !b_host) throw RpuError("null argument");
+    Tile &t = tile->t;
+    std::lock_guard<std::mutex> lock(t.mutex);
+    if (!t.resident() || !t.last_a || m_batch != t.last_update_batch || t.last_update_pulse == RPU_PULSE_NONE ||
+        t.last_update_pulse == RPU_PULSE_NONE_WITH_DEVICE) {
+      throw RpuError("No pulsed update of this batch size has run on this tile.");
+    }
+    DeviceGuard g(t.device_id);
+    t.sync_last();
+    RPU_HIP_CHECK(hipMemcpy(a_host, t.last_a, (size_t)m_batch * 4, hipMemcpyDeviceToHost));
+    RPU_HIP_CHECK(hipMemcpy(b_host, t.last_b, (size_t)m_batch * 4, hipMemcpyDeviceToHost));
   });
 }
 

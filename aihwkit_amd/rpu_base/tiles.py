@@ -482,6 +482,13 @@ class _CudaTileMixin:
         check(lib().rpu_tile_get_update_words(self._h, x_words.data_ptr(), d_words.data_ptr(), bl.data_ptr(), m_batch))
         return x_words, d_words, bl
 
+    def get_update_ab(self, m_batch: int):
+        """Per-sample probability scales (A for d, B for x) of the last pulsed update (CPU tensors)."""
+        a = torch.empty(m_batch, dtype=torch.float32)
+        b = torch.empty(m_batch, dtype=torch.float32)
+        check(lib().rpu_tile_get_update_ab(self._h, a.data_ptr(), b.data_ptr(), m_batch))
+        return a, b
+
     def update_with_words(self, x_words: torch.Tensor, d_words: torch.Tensor, non_blocking: bool = False) -> None:
         """Apply the device steps for given packed pulse words (int32 CUDA tensors [m, x_size], [m, d_size])."""
         if x_words.dtype != torch.int32 or d_words.dtype != torch.int32 or not x_words.is_cuda or not d_words.is_cuda:

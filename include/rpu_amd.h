@@ -612,6 +612,11 @@ int rpu_tile_set_extra(rpu_tile_t *tile, const int64_t *values_host, int count);
 int rpu_tile_get_update_words(rpu_tile_t *tile, uint32_t *x_words_host, uint32_t *d_words_host,
                               int32_t *bl_host, int m_batch);
 
+/* After a pulsed rpu_tile_update: the per-sample probability scales of that call, A for the d line and B for the x
+ * line (PulsedUpdateMetaParameter::calculateBlAB / performUpdateManagement, R/rpu_pulsed_meta_parameter.cpp:152-236),
+ * each [m_batch]. */
+int rpu_tile_get_update_ab(rpu_tile_t *tile, float *a_host, float *b_host, int m_batch);
+
 /* After rpu_tile_update with RPU_PULSE_DETERMINISTIC_IMPLICIT: signed coincidence counts
  * n[b][i][j] = (int) rintf((dv_i * BL) * xv_j) (R/dense_bit_line_maker.cpp:237-264) recomputed on the
  * GPU from the stored line values of that call; counts_host is [m_batch][d_size][x_size]. */

@@ -192,8 +192,10 @@ def test_stochastic_update_words_drive_the_oracle_to_the_same_weights(gpu_device
         orc.set_learning_rate(lr)
         gpu.update(cuda(x), cuda(d), False, False, False, False)
         xw, dw, bl = (t.numpy() for t in gpu.get_update_words(batch))
-        bl_orc, _, _ = orc.update_bl_ab(x, d)
+        bl_orc, a_orc, b_orc = orc.update_bl_ab(x, d)
         assert np.array_equal(bl, bl_orc)
+        a_gpu, b_gpu = (t.numpy() for t in gpu.get_update_ab(batch))
+        assert np.array_equal(a_gpu, a_orc) and np.array_equal(b_gpu, b_orc)  # probability scales, bit for bit
         _word_invariants(xw, x, bl)
         _word_invariants(dw, d, bl)
         assert (xw >> 1).any() and (dw >> 1).any()

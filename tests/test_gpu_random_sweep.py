@@ -90,8 +90,10 @@ def one_update(seed):
         d[2] = 0.0
     gpu.update(cuda(x), cuda(d), False)
     xw, dw, blv = gpu.get_update_words(batch)
-    bl_orc, _, _ = orc.update_bl_ab(x, d)
+    bl_orc, a_orc, b_orc = orc.update_bl_ab(x, d)
     words_ok = np.array_equal(blv.numpy(), bl_orc) and int(blv.max()) <= bl
+    a_gpu, b_gpu = (t.numpy() for t in gpu.get_update_ab(batch))
+    words_ok = words_ok and np.array_equal(a_gpu, a_orc) and np.array_equal(b_gpu, b_orc)
     for words, values in ((xw.numpy().view(np.uint32), x), (dw.numpy().view(np.uint32), d)):
         # no pulse beyond a sample's bit line, none on a zero value, the sign bit where the value is negative
         words_ok = words_ok and not (words >> (blv.numpy().astype(np.uint32)[:, None] + 1)).any()

@@ -140,7 +140,10 @@ def test_full_size_update_noise_free_matches_oracle_through_the_pulse_words(gpu_
     orc.set_learning_rate(0.01)
     gpu.update(cuda(x), cuda(d), False, False, False, False)
     xw, dw, bl = (t.numpy() for t in gpu.get_update_words(256))
-    assert np.array_equal(bl, orc.update_bl_ab(x, d)[0])
+    bl_orc, a_orc, b_orc = orc.update_bl_ab(x, d)
+    assert np.array_equal(bl, bl_orc)
+    a_gpu, b_gpu = (t.numpy() for t in gpu.get_update_ab(256))
+    assert np.array_equal(a_gpu, a_orc) and np.array_equal(b_gpu, b_orc)
     orc.update_with_words(xw, dw, bl)
     wg = gpu.get_weights().numpy()
     assert np.abs(wg - orc.get_weights()).max() <= 1e-5

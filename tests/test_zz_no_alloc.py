@@ -44,6 +44,8 @@ def test_update_without_allocation_equals_update(bias, layout):
         assert np.abs(w_noa - before).max() > 1e-4
         for u, v in zip(ref.get_update_words(batch), noa.get_update_words(batch)):
             assert torch.equal(u, v)
+        for u, v in zip(ref.get_update_ab(batch), noa.get_update_ab(batch)):
+            assert torch.equal(u, v)
 
 
 def test_update_without_allocation_on_another_device_kind_and_long_bit_lines():
