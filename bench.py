@@ -21,7 +21,7 @@ import sys
 import time
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
-for _p in (ROOT, os.path.join(ROOT, "tests"), os.path.join(ROOT, "oracle")):
+for _p in (ROOT, os.path.join(ROOT, "oracle")):  # oracle/: only the cpu_baseline legs import from it
     if _p not in sys.path:
         sys.path.insert(0, _p)
 
@@ -44,7 +44,7 @@ def batch_sweep() -> int:
     import torch
 
     from aihwkit_amd.rpu_base import tiles
-    from helpers import config2
+    from aihwkit_amd.benchmark_configs import config2
 
     meta, dev = config2()
     host = meta.create_array(1024, 1024, dev)
@@ -100,7 +100,7 @@ def main() -> int:
 
     from aihwkit_amd._cabi import lib
     from aihwkit_amd.rpu_base import tiles
-    from helpers import config1, config1_data, config2, config2_data
+    from aihwkit_amd.benchmark_configs import config1, config1_data, config2, config2_data
 
     lib()  # fails loudly if the HIP library is not built
     if not torch.cuda.is_available():
@@ -344,7 +344,7 @@ def bench_config3(args) -> int:
     import torch
 
     from aihwkit_amd.rpu_base import tiles
-    from helpers import CONFIG3_SHAPES, config3
+    from aihwkit_amd.benchmark_configs import CONFIG3_SHAPES, config3
 
     torch.cuda.set_device(0)
     batch, lr = 64, 0.1
@@ -389,12 +389,19 @@ def bench_config3(args) -> int:
         "gdevice_updates_per_s": devices / (ms_per_step * 1e-3) / 1e9,
     }
     if not args.no_cpu_baseline:
-        from helpers import build_transfer_pair
+        from transfer_oracle import TransferOracle
 
         cpu_ms = 0.0
         for (x_size, d_size), (_, x, d) in zip(CONFIG3_SHAPES, layer):
             meta, tr = config3()
-            _, orc, _ = build_transfer_pair(meta, tr, x_size, d_size, gpu=False)
+            # the oracle samples nothing itself: it takes the device arrays of a host tile of the library
+            host = meta.create_array(x_size, d_size, tr)
+            orc = TransferOracle(x_size, d_size, meta._config(tr._vec_par[0]), tr._to_transfer_c())
+            names, hidden, start = host.get_hidden_parameter_names(), host.get_hidden_parameters().numpy(), 0
+            for k in range(len(tr._vec_par)):
+                stop = names.index(f"hidden_weights_{k}")
+                orc.set_device_hidden(k, hidden[start:stop].copy())
+                start = stop + 1
             orc.set_learning_rate(lr)
             xh, dh = x.cpu().numpy(), d.cpu().numpy()
             t0 = time.perf_counter()
@@ -431,7 +438,7 @@ def bench_config5(args) -> int:
     from aihwkit_amd.inference import InferenceTile
     from aihwkit_amd.rpu_base import devices as dv
     from aihwkit_amd.rpu_base.tiles import TileGroup
-    from helpers import io_params
+    from aihwkit_amd.benchmark_configs import io_params
 
     torch.cuda.set_device(0)
     tokens = 1024
@@ -526,20 +533,6 @@ def bench_config5(args) -> int:
     return 0
 
 
-def conv_index_matrix(image_shape, kernel, with_bias=True):
-    """Index matrix of an unpadded stride-1 2-d convolution: entry [k, p] names the image element (offset by 2) that
-    patch p reads at kernel position k; 1 marks the bias row.  Returns (int32 indices [x_size * patches], patches)."""
-    import torch
-    import torch.nn.functional as F
-
-    size = int(torch.tensor(image_shape).prod())
-    numbered = torch.arange(2, size + 2, dtype=torch.float32).reshape(1, *image_shape)
-    unfolded = F.unfold(numbered, kernel_size=kernel)[0]                       # [C k k, patches]
-    if with_bias:
-        unfolded = torch.cat([unfolded, torch.ones(1, unfolded.shape[1])], dim=0)
-    return unfolded.to(torch.int32).contiguous().reshape(-1), unfolded.shape[1]
-
-
 def bench_config4(args) -> int:
     """Configuration 4: forward pass of a LeNet5-shaped stack for 512 images of 28 x 28: two 5 x 5 convolutions
     (1 -> 16, 16 -> 32) as indexed analog tiles, tanh and 2 x 2 max pooling in torch between them, then 512 -> 128 -> 10
@@ -550,8 +543,8 @@ def bench_config4(args) -> int:
     import torch.nn.functional as F
 
     from aihwkit_amd.inference import InferenceTile
+    from aihwkit_amd.benchmark_configs import conv_index_matrix, io_params
     from aihwkit_amd.rpu_base import devices as dv
-    from helpers import io_params
 
     torch.cuda.set_device(0)
     batch = 512

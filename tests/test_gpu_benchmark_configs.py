@@ -1,0 +1,339 @@
+"""The benchmark configurations at their full shapes: what the smaller parity cases leave open.
+
+* configurations 1 and 2, real 1/126 (1/127) DAC steps, values BEFORE the ADC on all rows against the oracle and
+  against the exact (float64) contraction of the same quantized inputs;
+* rows whose bound-management round count differs between GPU and oracle sit on the ADC's saturation edge;
+* the 64-seed mean / variance protocol (src/rpucuda/cuda/rpucuda_pulsed_test.cpp:1048-1131) at 1024 x 1024 x 256 for
+  forward, backward and the weight change;
+* a full-size configuration-1 update through the pulse words;
+* configuration 4: the four LeNet5 tiles at their real shapes, 8-bit converters, batch 512.
+"""
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from aihwkit_amd.inference import InferenceTile, PCMLikeNoiseModel
+from aihwkit_amd.rpu_base import devices as dv
+from aihwkit_amd.rpu_base import tiles
+from helpers import (build_pair, config1, config1_data, config2, config2_data, constant_step, conv_index_matrix,
+                     io_params, make_meta, noise_free_io, soft_bounds)
+from indexed_oracle import IndexedOracle
+from oracle_lib import OracleTile
+from test_gpu_statistics import compare_moments
+
+pytestmark = pytest.mark.gpu
+
+F32 = np.float32
+NM, BM = dv.NoiseManagementType, dv.BoundManagementType
+
+
+def cuda(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def dac(x, inp_step, reduction=1.0):
+    """Quantized input rows of the forward pass in the reference's fp32 operation order
+    (rpu_forward_backward_pass.cpp:583-602, 944-969): scale = 1 / nm / reduction, rint(x * scale / step) * step, clip."""
+    nm = np.abs(x).max(axis=1, keepdims=True).astype(F32)
+    scale = (F32(1.0) / nm / F32(reduction)).astype(F32)
+    v = (x * scale).astype(F32)
+    q = (np.rint((v / F32(inp_step)).astype(F32)) * F32(inp_step)).astype(F32)
+    return np.clip(q, F32(-1.0), F32(1.0)), nm, scale
+
+
+@pytest.mark.parametrize("cfg,data,shape", [(config1, config1_data, (512, 512, 100)),
+                                            (config2, config2_data, (1024, 1024, 256))])
+@pytest.mark.parametrize("bm", [BM.NONE, BM.Iterative])
+def test_values_before_the_adc_on_all_rows(gpu_device, cfg, data, shape, bm):
+    """ADC quantization off (out_res <= 0) and the output bound out of reach: what the contraction hands to the ADC.
+    Every element is compared; the tolerance is 1e-5 of the ADC's input range (+-12), and both implementations must
+    be equally close to the exact sum of the same quantized inputs."""
+    x_size, d_size, batch = shape
+    meta, dev = cfg(noise=False)
+    inp_res = meta.forward_io.inp_res
+    for io in (meta.forward_io, meta.backward_io):
+        io.out_res = -1.0
+        io.out_bound = 1.0e4
+    meta.forward_io.bound_management = bm
+    host, orc, _ = build_pair(meta, dev, x_size, d_size, gpu=False)
+    w, x, d = data(x_size, d_size, batch)
+    host.set_weights(torch.from_numpy(w))
+    orc.set_weights(w)
+    wc = orc.get_weights()
+    gpu = tiles.CudaAnalogTile(host)
+    y_gpu = gpu.forward(cuda(x), False, False, False, False, False).cpu().numpy()
+    y_orc = orc.forward(x)
+    xq, nm, _ = dac(x, inp_res * 2.0)
+    exact = (xq.astype(np.float64) @ wc.T.astype(np.float64)) * nm
+    tol = 1e-5 * 12.0
+    assert np.abs(y_gpu - y_orc).max() <= tol
+    err_gpu, err_orc = np.abs(y_gpu - exact), np.abs(y_orc - exact)
+    assert err_gpu.max() <= tol and err_orc.max() <= tol
+    assert np.sqrt((err_gpu ** 2).mean()) <= 1.5 * np.sqrt((err_orc ** 2).mean()) + 1e-7  # no less accurate than the CPU's sum
+    assert (np.abs(y_gpu - y_orc) <= 1e-5).mean() > 0.97                                    # most elements within 1e-5 absolute
+    # backward
+    b_gpu = gpu.backward(cuda(d), False, False, False, False).cpu().numpy()
+    b_orc = orc.backward(d)
+    dq, nmd, _ = dac(d, meta.backward_io.inp_res * 2.0)
+    exact_b = (dq.astype(np.float64) @ wc.astype(np.float64)) * nmd
+    assert np.abs(b_gpu - b_orc).max() <= 1e-5
+    assert np.abs(b_gpu - exact_b).max() <= 1e-5 and np.abs(b_orc - exact_b).max() <= 1e-5
+
+
+def test_rows_with_another_round_count_sit_on_the_saturation_edge(gpu_device):
+    """Configuration 2, noise off, real converter steps.  A sample needs another bound-management round when an ADC
+    code passes +-255 (12 / step): rint(y / step) > 255, i.e. |y| > 255.5 steps.  Where GPU and oracle disagree about
+    the number of rounds, the largest |y| of the deciding round (exact sum of that round's quantized inputs) must lie
+    within rounding distance of that edge; everywhere else outputs agree to 1e-5 up to single-code flips."""
+    meta, dev = config2(noise=False)
+    host, orc, _ = build_pair(meta, dev, 1024, 1024, gpu=False)
+    rng = np.random.default_rng(0)
+    batch = 1024                                      # more samples than the benchmark batch: more near-edge cases
+    w = rng.uniform(-0.6, 0.6, (1024, 1024)).astype(F32)
+    x = rng.uniform(-1, 1, (batch, 1024)).astype(F32)
+    host.set_weights(torch.from_numpy(w))
+    orc.set_weights(w)
+    wc = orc.get_weights().astype(np.float64)
+    gpu = tiles.CudaAnalogTile(host)
+    y_gpu = gpu.forward(cuda(x), False, False, False, False, False).cpu().numpy()
+    y_orc = orc.forward(x)
+    r_gpu, r_orc = gpu.get_bm_rounds(batch).numpy(), orc.bm_rounds(batch)
+    inp_step, out_step = F32(2.0 / 126.0), F32(24.0 / 510.0)
+    edge = 255.5 * float(out_step)
+    differ = np.nonzero(r_gpu != r_orc)[0]
+    assert differ.size < 0.03 * batch
+    for b in differ:
+        r = min(r_gpu[b], r_orc[b])                   # the round one of them passed and the other failed
+        xq, _, _ = dac(x[b:b + 1], inp_step, reduction=2.0 ** (r - 1))
+        peak = np.abs(xq.astype(np.float64) @ wc.T).max()
+        assert abs(peak - edge) <= 2e-5, (b, r_gpu[b], r_orc[b], peak, edge)
+    same = r_gpu == r_orc
+    nm = np.abs(x).max(axis=1)
+    lsb = float(out_step) * nm * (2.0 ** (r_orc - 1))
+    diff = np.abs(y_gpu - y_orc)[same]
+    off = diff > 1e-5
+    assert off.mean() < 5e-3
+    steps = diff[off] / np.broadcast_to(lsb[same][:, None], diff.shape)[off]
+    assert np.allclose(steps, 1.0, atol=1e-3)
+
+
+def test_moments_over_64_seeds_at_the_graded_shape(gpu_device):
+    """Configuration 2 as graded (1024 x 1024, batch 256, output noise 0.06, cycle-to-cycle 0.3, stochastic pulses with
+    update management): mean and variance over 64 seeds of forward outputs, backward outputs and the weight change,
+    GPU against oracle, per element and pooled."""
+    n_seeds = 64
+    meta, dev = config2()
+    host, orc, _ = build_pair(meta, dev, 1024, 1024, gpu=False)
+    w, x, d = config2_data()
+    host.set_weights(torch.from_numpy(w))
+    orc.set_weights(w)
+    w0 = orc.get_weights().copy()
+    xg, dg = cuda(x), cuda(d)
+    gpu = tiles.CudaAnalogTile(host)
+    yg, yo, bg, bo, rg, ro = [], [], [], [], [], []
+    for s in range(n_seeds):
+        gpu.set_seed(500 + s)
+        orc.set_seed(1 + s)
+        yg.append(gpu.forward(xg, False, False, False, False, False).cpu().numpy())
+        rg.append(gpu.get_bm_rounds(256).numpy())
+        yo.append(orc.forward(x))
+        ro.append(orc.bm_rounds(256))
+        bg.append(gpu.backward(dg, False, False, False, False).cpu().numpy())
+        bo.append(orc.backward(d))
+    assert abs(np.mean(rg) - np.mean(ro)) < 0.02 and np.mean(ro) > 1.5
+    compare_moments(np.stack(yg), np.stack(yo), "forward outputs at the graded shape")
+    compare_moments(np.stack(bg), np.stack(bo), "backward outputs at the graded shape")
+    del yg, yo, bg, bo
+    dwg = np.empty((n_seeds, 1024, 1024), F32)
+    dwo = np.empty((n_seeds, 1024, 1024), F32)
+    for s in range(n_seeds):
+        gpu.set_weights(torch.from_numpy(w))
+        gpu.set_seed(900 + s)
+        gpu.set_learning_rate(0.01)
+        gpu.update(xg, dg, False, False, False, False)
+        dwg[s] = gpu.get_weights().numpy() - w0
+        orc.set_weights(w)
+        orc.set_seed(101 + s)
+        orc.set_learning_rate(0.01)
+        orc.update(x, d)
+        dwo[s] = orc.get_weights() - w0
+    assert np.abs(dwo).mean() > 2e-3
+    # per element and pooled on a quarter of the matrix at a time (memory), all four quarters
+    for q in range(4):
+        rows = slice(256 * q, 256 * (q + 1))
+        compare_moments(dwg[:, rows], dwo[:, rows], f"weight change at the graded shape, rows {256 * q}..")
+
+
+def test_full_size_configuration_1_update_through_the_pulse_words(gpu_device):
+    """512 x 512 ConstantStep, batch 100, BL 31, with update management on (default) and off: the GPU's packed words
+    drive the oracle's device loop to the same weights; BL, A and B bit-equal."""
+    for um in (True, False):
+        meta, dev = config1(noise=False)
+        meta.update.update_management = um
+        meta.update.update_bl_management = um
+        host, orc, _ = build_pair(meta, dev, 512, 512, gpu=False)
+        w, x, d = config1_data()
+        host.set_weights(torch.from_numpy(w))
+        orc.set_weights(w)
+        gpu = tiles.CudaAnalogTile(host)
+        gpu.set_seed(8)
+        for lr in (0.01, -0.01):
+            gpu.set_learning_rate(lr)
+            orc.set_learning_rate(lr)
+            gpu.update(cuda(x), cuda(d), False, False, False, False)
+            xw, dw, bl = (t.numpy() for t in gpu.get_update_words(100))
+            bl_o, a_o, b_o = orc.update_bl_ab(x, d)
+            a_g, b_g = (t.numpy() for t in gpu.get_update_ab(100))
+            assert np.array_equal(bl, bl_o) and np.array_equal(a_g, a_o) and np.array_equal(b_g, b_o)
+            assert bl.max() == 31 if not um else bl.max() >= 2
+            orc.update_with_words(xw, dw, bl)
+            assert np.abs(gpu.get_weights().numpy() - orc.get_weights()).max() <= 1e-5
+        assert np.abs(orc.get_weights() - w).max() > 1e-3
+
+
+def test_learning_rate_beyond_the_pulse_word_is_refused_or_exact(gpu_device):
+    """Without a fixed BL and BL management, lr > dw_min * desired_BL stretches the bit line to ceil(lr / dw_min)
+    (rpu_pulsed_meta_parameter.cpp:166-171).  Stochastic words hold 31 pulses: refused.  The implicit pulse types keep
+    no words: they follow the oracle with the long bit line."""
+    rng = np.random.default_rng(4)
+    x = rng.uniform(-1, 1, (9, 40)).astype(F32)
+    d = rng.uniform(-1, 1, (9, 30)).astype(F32)
+    w = rng.uniform(-0.3, 0.3, (30, 40)).astype(F32)
+    kw = dict(dw_min=0.001, dw_min_std=0.0, construction_seed=2, enforce_consistency=True)
+    meta = make_meta(desired_bl=31, fixed_bl=False, update_management=False, update_bl_management=False)
+    _, _, gpu = build_pair(meta, constant_step(**kw), 40, 30)
+    gpu.set_weights(torch.from_numpy(w))
+    before = gpu.get_weights().numpy().copy()
+    gpu.set_learning_rate(0.05)                       # ceil(0.05 / 0.001) = 50 pulses
+    with pytest.raises(RuntimeError, match="bit line of 50 pulses"):
+        gpu.update(cuda(x), cuda(d), False, False, False, False)
+    assert np.array_equal(gpu.get_weights().numpy(), before)
+    gpu.set_learning_rate(0.031)                      # exactly 31: allowed
+    gpu.update(cuda(x), cuda(d), False, False, False, False)
+    assert gpu.get_update_words(9)[2].max() == 31
+    meta = make_meta(desired_bl=31, fixed_bl=False, update_management=False, update_bl_management=False,
+                     pulse_type=dv.PulseType.DeterministicImplicit)
+    _, orc, gpu = build_pair(meta, soft_bounds(**kw), 40, 30)
+    gpu.set_weights(torch.from_numpy(w))
+    orc.set_weights(w)
+    gpu.set_learning_rate(0.05)
+    orc.set_learning_rate(0.05)
+    gpu.update(cuda(x), cuda(d), False, False, False, False)
+    counts = gpu.get_implicit_counts(9).numpy()
+    assert np.array_equal(counts, orc.implicit_counts(x, d)) and np.abs(counts).max() > 31
+    orc.update(x, d)
+    assert np.abs(gpu.get_weights().numpy() - orc.get_weights()).max() <= 1e-5
+
+
+# ---- configuration 4: LeNet5-shaped stack as im2col tiles -------------------------------------------------------
+
+LENET = (("conv", (1, 28, 28), 16), ("conv", (16, 12, 12), 32), ("fc", 512, 128), ("fc", 128, 10))
+
+
+def lenet_stack(io, noise_model, seed=0, w_range=None):
+    rng = np.random.default_rng(seed)
+    stack = []
+    for k, (kind, in_shape, out_size) in enumerate(LENET):
+        if kind == "conv":
+            indices, patches = conv_index_matrix(in_shape, (5, 5))
+            in_size = in_shape[0] * 25 + 1
+        else:
+            indices, patches, in_size = None, 1, in_shape + 1
+        w = rng.uniform(-1, 1, (out_size, in_size))
+        w = (w / np.sqrt(in_size) if w_range is None else w * w_range).astype(F32)   # the benchmark's weights, or mapped to a range
+        tile = InferenceTile(out_size, in_size, forward_io=io, noise_model=noise_model)
+        tile.set_weights(torch.from_numpy(w))
+        tile.cuda()
+        tile.tile.set_seed(2000 + k)
+        if indices is not None:
+            tile.set_matrix_indices(indices)
+        stack.append((kind, tile, indices, patches, out_size, in_size, w))
+    return stack
+
+
+def lenet_layer(kind, tile, patches, out_size, h, is_test=True):
+    if kind == "conv":
+        side = int(round(patches ** 0.5))
+        return tile.forward_indexed(h, torch.empty(h.size(0), out_size, side, side, device="cuda"), is_test=is_test)
+    ones = torch.ones(h.size(0), 1, device="cuda")
+    return tile.forward(torch.cat([h.reshape(h.size(0), -1), ones], dim=1), is_test=is_test)
+
+
+def test_configuration_4_tiles_without_noise_match_the_oracle(gpu_device):
+    """The four tiles at their real shapes (26 -> 16 with 576 patches per image, 401 -> 32 with 64, 513 -> 128,
+    129 -> 10), 8-bit DAC / ADC, abs-max noise management, iterative bound management, all noise scales zero:
+    every layer of 16 images against the indexed oracle around the oracle tile that holds the same (programmed and
+    drifted, here unchanged) weights.  Each layer is fed the GPU's previous activations on both sides."""
+    io = noise_free_io(inp_res=1 / 254.0, out_res=1 / 254.0, noise_management=NM.AbsMax, bound_management=BM.Iterative)
+    quiet = PCMLikeNoiseModel(prog_noise_scale=0.0, read_noise_scale=0.0, drift_scale=0.0)
+    stack = lenet_stack(io, quiet)
+    n = 16
+    h = torch.from_numpy(np.random.default_rng(1).uniform(0, 1, (n, 1, 28, 28)).astype(F32)).cuda()
+    meta = make_meta(io, noise_free_io())
+    meta.backward_io.is_perfect = True
+    meta.update.pulse_type = dv.PulseType.NONE
+    for kind, tile, indices, patches, out_size, in_size, w in stack:
+        tile.drift_weights(86400.0)
+        wt = tile.get_weights().numpy()
+        assert np.abs(wt - w).max() <= 2e-6           # the pipeline with all scales at zero keeps the weights
+        orc = OracleTile(in_size, out_size, meta._config(dv.IdealResistiveDeviceParameter()))
+        orc.set_weights(wt)
+        y = lenet_layer(kind, tile, patches, out_size, h, is_test=False)
+        if kind == "conv":
+            want = IndexedOracle(orc, indices.numpy(), patches).forward(h.cpu().numpy()).reshape(y.shape)
+            nm = None
+        else:
+            flat = np.concatenate([h.reshape(n, -1).cpu().numpy(), np.ones((n, 1), F32)], axis=1)
+            want = orc.forward(np.ascontiguousarray(flat))
+        got = y.cpu().numpy()
+        diff = np.abs(got - want)
+        off = diff > 1e-5
+        # a flip is one ADC code of that sample: at most (24 / 254) * largest input of the patch * 2^(rounds - 1)
+        assert off.mean() < 5e-3, (kind, in_size, off.mean())
+        assert diff.max() <= 24.0 / 254.0 * float(h.abs().max()) * 16.0 * 1.001 + 1e-5
+        h = F.max_pool2d(torch.tanh(y), 2) if kind == "conv" else torch.tanh(y)
+
+
+def test_configuration_4_full_batch_with_pcm_noise_drift_and_compensation(gpu_device):
+    """Batch 512 through the stack with PCM programming noise, drift to one day, read noise, global drift
+    compensation and output noise on: size-independent properties per layer -- the compensated output level is the
+    level before drift, the raw one has shrunk like the weights, outputs correlate with the noise-free ones, stay
+    within the ADC range, and a re-seeded run repeats bit for bit."""
+    io = io_params(inp_res=1 / 254.0, out_res=1 / 254.0, out_noise=0.06, noise_management=NM.AbsMax,
+                   bound_management=BM.Iterative)
+    stack = lenet_stack(io, PCMLikeNoiseModel(), w_range=0.6)       # weights mapped to +-0.6 of the conductance range, as the reference's mapping does
+    clean = lenet_stack(noise_free_io(inp_res=1 / 254.0, out_res=1 / 254.0, noise_management=NM.AbsMax,
+                                      bound_management=BM.Iterative),
+                        PCMLikeNoiseModel(prog_noise_scale=0.0, read_noise_scale=0.0, drift_scale=0.0), w_range=0.6)
+    batch = 512
+    x = torch.from_numpy(np.random.default_rng(2).uniform(0, 1, (batch, 1, 28, 28)).astype(F32)).cuda()
+    h = x
+    for (kind, tile, _, patches, out_size, in_size, w), (_, ref, *_rest) in zip(stack, clean):
+        tile.program_weights()
+        programmed = tile.get_weights().numpy()
+        assert 0.01 < np.abs(programmed - w).std() < 0.05         # programming noise of a few percent of the range
+        fresh = lenet_layer(kind, tile, patches, out_size, h)
+        tile.drift_weights(86400.0)
+        drifted = tile.get_weights().numpy()
+        shrink = np.abs(drifted).mean() / np.abs(programmed).mean()
+        assert 0.4 < shrink < 0.9
+        assert tile.alpha == pytest.approx(1.0 / shrink, rel=0.15)
+        raw = lenet_layer(kind, tile, patches, out_size, h, is_test=False)
+        tile.tile.set_seed(77)
+        comp = lenet_layer(kind, tile, patches, out_size, h)
+        tile.tile.set_seed(77)
+        again = lenet_layer(kind, tile, patches, out_size, h)
+        assert torch.equal(comp, again)
+        assert torch.isfinite(comp).all()
+        level = lambda t: float(t.abs().mean())
+        assert level(raw) == pytest.approx(shrink * level(fresh), rel=0.15)
+        assert level(comp) == pytest.approx(level(fresh), rel=0.12)
+        noise_free = lenet_layer(kind, ref, patches, out_size, h)
+        c = np.corrcoef(comp.cpu().numpy().ravel(), noise_free.cpu().numpy().ravel())[0, 1]
+        assert c > (0.8 if out_size > 10 else 0.7), (in_size, c)
+        # the ADC range after noise management and compensation: |y| <= 12 * max|x| * 2^4 * alpha
+        bound = 12.0 * float(h.abs().max()) * 16.0 * tile.alpha
+        assert float(comp.abs().max()) <= bound * 1.001
+        h = F.max_pool2d(torch.tanh(comp), 2) if kind == "conv" else torch.tanh(comp)
+    assert h.shape == (batch, 10)
