@@ -193,6 +193,8 @@ struct UpdateArgs {
   uint32_t call;
 };
 
+// tables of the update kernels on the current device (once per GPU; blocking copy, no allocation)
+void ensure_update_tables();
 void launch_update_prepare(const UpdateArgs &a, hipStream_t s);       // BL, A, B per sample
 void launch_update_lines(const UpdateArgs &a, hipStream_t s);         // stochastic pulse words and their bit planes
 void launch_update_implicit_lines(const UpdateArgs &a, hipStream_t s); // deterministic line values

@@ -14,6 +14,11 @@
 // covers 64 consecutive x of one d row, so the d word of a sample is wave-uniform (scalar load) and
 // the x words, weights and parameters are read with unit stride.
 #include "kernels.h"
+#include "rpu_host.h"
+
+#include <cmath>
+#include <mutex>
+#include <vector>
 
 namespace rpu_amd {
 
@@ -421,85 +426,146 @@ __device__ __forceinline__ void noise_factors(float (&f)[8], float std_, unsigne
   }
 }
 
-// Pulse loop for short bit lines (at most 2^NB - 1 pulse slots in use).  The batch is walked in chunks of
-// 32 samples.  For a chunk every lane builds, from the bit planes alone, the coincidence count of each
-// of its 32 samples as NB bit-sliced words (a ripple-carry add of x_plane & d_plane per slot; the d
-// planes are wave-uniform) and the direction word sign(x) ^ sign(d).  The lanes then walk their samples
-// in batch order, one pulse per lane and pass: the lowest sample with a count left gives the direction,
-// its count is decremented in the bit slices (ripple borrow).  The wave moves to the next chunk when no
-// lane has a pulse left; the noise factors of eight passes come from one Philox call per lane and carry
-// over chunk ends.
-template <int KIND, bool MULT, int NB>
-__device__ __forceinline__ float pulsed_counted(const UpdateArgs &a, float w, const PulseCell<KIND> &cp, unsigned cell,
-                                                int i, int j, bool valid, int kmax, float *noise_lds) {
-  const float std_ = a.dev.dw_min_std;
-  const uint32_t lr_mask = a.lr < 0.0f ? 0xffffffffu : 0u;
-  const int n_chunks = a.n_chunks;
-  const unsigned xs = (unsigned)a.x_size, ds = (unsigned)a.d_size;
-  const unsigned slots = (unsigned)a.plane_slots;
-  const uint32_t *xpl = a.x_planes + j;
-  const uint32_t *dpl = a.d_planes + i;
+// Normal quantiles of the cycle-to-cycle noise: xi[q] = Phi^-1((q + 0.5) / CTOC_LEVELS) scaled to unit variance,
+// exactly antisymmetric (zero mean).  Filled once per GPU by ensure_update_tables(); the update kernel turns it into
+// the factors 1 + std * xi in LDS.
+constexpr int CTOC_LEVELS = 256;
+__device__ float g_ctoc_xi[CTOC_LEVELS];
 
-  uint32_t pass = 0;
-  for (int c = 0; c < n_chunks; ++c) {
-    const unsigned base = (unsigned)c * slots;
-    uint32_t cnt[NB];
+// bitwise m ? a : b for a mask of all ones or all zeros (v_bfi_b32)
+__device__ __forceinline__ float select_bits(uint32_t m, float a, float b) {
+  return __uint_as_float((__float_as_uint(a) & m) | (__float_as_uint(b) & ~m));
+}
+
+// x bit planes of one 32-sample chunk for the C columns of a lane: NK pulse slots and the sign plane
+template <int NK, int C> struct ChunkPlanes {
+  uint32_t k[C][NK], sg[C];
+  __device__ __forceinline__ void load(const UpdateArgs &a, const int (&j)[C], unsigned chunk) {
+    const unsigned xs = (unsigned)a.x_size, slots = (unsigned)a.plane_slots;
+    const unsigned base = chunk * slots;
 #pragma unroll
-    for (int n = 0; n < NB; ++n) cnt[n] = 0u;
+    for (int c = 0; c < C; ++c) {
+      const uint32_t *xpl = a.x_planes + j[c];
 #pragma unroll
-    for (int k = 0; k < (1 << NB) - 1; ++k) {
-      if (k < kmax) {
-        const uint32_t dk = dpl[(base + k) * ds]; // wave-uniform
-        if (dk) {
-          uint32_t carry = valid ? (dk & xpl[(base + k) * xs]) : 0u;
+      for (int s = 0; s < NK; ++s) k[c][s] = xpl[(base + (unsigned)s) * xs]; // slots beyond the batch's longest line are never tested
+      sg[c] = xpl[(base + slots - 1u) * xs];
+    }
+  }
+};
+
+// Pulse loop for short bit lines (at most NK pulse slots in use).  The lanes of a wave hold cross-points of one d
+// row (C columns per lane, 256 apart), so the d pulses are wave-uniform: the wave walks the 32 samples of a chunk in
+// batch order and, per sample, the pulse slots in which its d line fired -- scalar bit tests and branches, nothing
+// for samples without a d pulse -- and in such a (sample, slot) pass every cross-point whose x line fired in that
+// slot takes one device step.  All coincidences of a sample have one direction per cross-point, sign(x) * sign(d),
+// picked once per sample.  Several columns per lane share the scalar work of a pass and give the vector pipeline
+// independent chains.  The x planes of the next chunk are fetched while the current one is walked (two register
+// sets in turn).  Lanes beyond the row end compute on the last column's data and never store.
+// Cycle-to-cycle noise: a step takes its factor 1 + std * xi from a table of 256 normal quantiles in LDS (unit
+// variance, kurtosis 2.92, |xi| <= 2.9), indexed by one byte of a per-lane xoroshiro64 stream (four factors per 32-bit
+// output, fetched one pass ahead) whose state is one Philox4x32-10 output keyed by (first cross-point of the lane,
+// call): reproducible from the tile seed.
+template <int KIND, bool MULT, int NK, bool NOISE, int C> struct PulsedRows {
+  const UpdateArgs &a;
+  float (&w)[C];
+  const PulseCell<KIND> (&cp)[C];
+  const float *tbl;
+  uint32_t s0 = 1u, s1 = 0u;
+  float fnext[C];
+
+  __device__ __forceinline__ PulsedRows(const UpdateArgs &a_, float (&w_)[C], const PulseCell<KIND> (&cp_)[C], const float *tbl_)
+      : a(a_), w(w_), cp(cp_), tbl(tbl_) {}
+
+  __device__ __forceinline__ void draw() {
+    if (!NOISE) return;
 #pragma unroll
-          for (int n = 0; n < NB; ++n) {
-            const uint32_t t = cnt[n] & carry;
-            cnt[n] ^= carry;
-            carry = t;
+    for (int c = 0; c < C; c += 4) {
+      const uint32_t r = s0 + s1;
+      s1 ^= s0;
+      s0 = __builtin_amdgcn_bitop3_b32(__builtin_rotateleft32(s0, 26), s1, s1 << 9, 0x96); // three-input xor
+      s1 = __builtin_rotateleft32(s1, 13);
+      // one byte of the output per factor: the table offset is the byte times four
+      fnext[c] = *(const float *)((const char *)tbl + ((r & 0xffu) << 2));
+      if (c + 1 < C) fnext[c + 1] = *(const float *)((const char *)tbl + (((r >> 8) & 0xffu) << 2));
+      if (c + 2 < C) fnext[c + 2] = *(const float *)((const char *)tbl + (((r >> 16) & 0xffu) << 2));
+      if (c + 3 < C) fnext[c + 3] = *(const float *)((const char *)tbl + ((r >> 24) << 2));
+    }
+  }
+
+  __device__ __forceinline__ void chunk(const ChunkPlanes<NK, C> &x, unsigned ch, int i, int kmax, uint32_t lr_mask) {
+    const unsigned ds = (unsigned)a.d_size, slots = (unsigned)a.plane_slots;
+    const uint32_t *dpl = a.d_planes + i;
+    const unsigned base = ch * slots;
+    uint32_t dk[NK], any = 0u; // wave-uniform
+#pragma unroll
+    for (int k = 0; k < NK; ++k) {
+      dk[k] = (k < kmax) ? dpl[(base + (unsigned)k) * ds] : 0u;
+      any |= dk[k];
+    }
+    if (!any) return;
+    // bit set: x and d have the same sign, which steps down when lr > 0
+    const uint32_t dflip = ~dpl[(base + slots - 1u) * ds] ^ lr_mask;
+    uint32_t same[C];
+#pragma unroll
+    for (int c = 0; c < C; ++c) same[c] = x.sg[c] ^ dflip;
+    while (any) {
+      const int q = __builtin_ctz(any);
+      any &= any - 1u;
+      float slope[C], scale[C];
+#pragma unroll
+      for (int c = 0; c < C; ++c) {
+        const uint32_t dm = (uint32_t)__builtin_amdgcn_sbfe((int)same[c], (uint32_t)q, 1u);
+        slope[c] = select_bits(dm, cp[c].slope_dn, cp[c].slope_up);
+        scale[c] = select_bits(dm, cp[c].scale_dn, cp[c].scale_up);
+      }
+#pragma unroll
+      for (int k = 0; k < NK; ++k) {
+        if ((dk[k] >> q) & 1u) {
+          float f[C];
+#pragma unroll
+          for (int c = 0; c < C; ++c) f[c] = NOISE ? fnext[c] : 1.0f;
+          draw(); // the factors of the next pass are on their way while this one computes
+#pragma unroll
+          for (int c = 0; c < C; ++c) {
+            const uint32_t pm = (uint32_t)__builtin_amdgcn_sbfe((int)x.k[c][k], (uint32_t)q, 1u);
+            const float wn = pulse<KIND, MULT>(w[c], slope[c], scale[c], f[c], cp[c].lo, cp[c].hi);
+            w[c] = select_bits(pm, wn, w[c]);
           }
         }
       }
     }
-    uint32_t cur = cnt[0];
-#pragma unroll
-    for (int n = 1; n < NB; ++n) cur |= cnt[n];
-    if (!__any(cur != 0u)) continue;
-    // bit set: x and d have the same sign, which steps down when lr > 0
-    const uint32_t same = ~(xpl[(base + slots - 1) * xs] ^ dpl[(base + slots - 1) * ds]) ^ lr_mask;
-    // One pass: the lowest sample with a count left gives the direction, its count is decremented (ripple
-    // borrow), one pulse.  The noise factors of eight passes are parked in LDS (one column per thread), so
-    // that a pass picks its factor by the wave-uniform pass number without unrolling across chunk ends.
-    do {
-      if ((pass & 7u) == 0u) {
-        float f[8];
-        noise_factors(f, std_, cell, pass >> 3, a);
-#pragma unroll
-        for (int q = 0; q < 8; ++q) noise_lds[q * 256] = f[q];
-      }
-      const float fq = noise_lds[(pass & 7u) * 256];
-      ++pass;
-      const bool active = cur != 0u;
-      const uint32_t m = cur & (0u - cur);
-      uint32_t borrow = m;
-#pragma unroll
-      for (int n = 0; n < NB; ++n) {
-        const uint32_t t = ~cnt[n] & borrow;
-        cnt[n] ^= borrow;
-        borrow = t;
-      }
-      cur = cnt[0];
-#pragma unroll
-      for (int n = 1; n < NB; ++n) cur |= cnt[n];
-      const bool down = (same & m) != 0u;
-      const float slope = down ? cp.slope_dn : cp.slope_up;
-      const float scale = down ? cp.scale_dn : cp.scale_up;
-      const float wn = pulse<KIND, MULT>(w, slope, scale, fq, cp.lo, cp.hi);
-      w = active ? wn : w;
-    } while (__any(cur != 0u));
   }
-  return w;
-}
+
+  __device__ __forceinline__ void run(unsigned cell, int i, const int (&j)[C], int kmax) {
+    const uint32_t lr_mask = a.lr < 0.0f ? 0xffffffffu : 0u;
+    const unsigned n_chunks = (unsigned)a.n_chunks;
+    if (NOISE) {
+      const Philox4 r = philox4x32_10(cell, 0u, a.call, RNG_CTOC, a.key.k0, a.key.k1);
+      s0 = r.v[0] | 1u; // the all-zero state is the one fixed point of the generator
+      s1 = r.v[1];
+      draw();
+    }
+    if (NK > 3) { // one register set: the longer lines are the rarer case, and two sets would not fit
+      ChunkPlanes<NK, C> p;
+      for (unsigned ch = 0; ch < n_chunks; ++ch) {
+        p.load(a, j, ch);
+        chunk(p, ch, i, kmax, lr_mask);
+      }
+      return;
+    }
+    ChunkPlanes<NK, C> pa, pb;
+    pa.load(a, j, 0u);
+    for (unsigned ch = 0; ch < n_chunks; ch += 2u) {
+      const bool second = ch + 1u < n_chunks;
+      if (second) pb.load(a, j, ch + 1u);
+      chunk(pa, ch, i, kmax, lr_mask);
+      if (second) {
+        if (ch + 2u < n_chunks) pa.load(a, j, ch + 2u);
+        chunk(pb, ch + 1u, i, kmax, lr_mask);
+      }
+    }
+  }
+};
 
 // Pulse loop for any bit-line length.  The batch is walked in blocks of 128 samples.  For a block every lane
 // first builds the 128-bit set of samples in which its cross-point has a coincidence: OR over the pulse
@@ -581,25 +647,46 @@ __device__ __forceinline__ float pulsed_gather(const UpdateArgs &a, float w, con
   return w;
 }
 
-// grid: x = ceil(x_size / 256), y = d_size.  One thread per cross-point; a wave covers 64 consecutive x of
-// one d row, so everything that belongs to the d line is wave-uniform and the x planes, weights and
-// parameters are read with unit stride.  The pulse loop is chosen by the longest bit line of the batch.
-template <int KIND, bool MULT>
-__global__ __launch_bounds__(256) void k_update_pulsed(UpdateArgs a) {
+// grid: x = ceil(x_size / (256 C)), y = d_size.  A thread holds C cross-points of one d row, 256 columns apart; a
+// wave covers 64 consecutive x per column group, so everything that belongs to the d line is wave-uniform and the x
+// planes, weights and parameters are read with unit stride.  The pulse loop is chosen by the longest bit line of
+// the batch.
+template <int KIND, bool MULT, bool NOISE, int C>
+__global__ __launch_bounds__(256, (C > 1 ? 4 : 8)) void k_update_pulsed(UpdateArgs a) {
+  __shared__ float tbl[CTOC_LEVELS]; // noise factors 1 + std * quantile
+  if (NOISE) {
+    static_assert(CTOC_LEVELS == 256, "one table entry per thread");
+    tbl[threadIdx.x] = __builtin_fmaf(a.dev.dw_min_std, g_ctoc_xi[threadIdx.x], 1.0f);
+    __syncthreads();
+  }
   const int i = blockIdx.y;
-  const int jt = blockIdx.x * blockDim.x + threadIdx.x;
-  const bool valid = jt < a.x_size;
-  const int j = valid ? jt : a.x_size - 1;
-  const unsigned cell = (unsigned)i * (unsigned)a.x_size + (unsigned)j;
-  PulseCell<KIND> cp;
-  cp.load(a.dev, cell);
-  float w = a.w[cell];
+  int j[C];
+  bool valid[C];
+  unsigned cell[C];
+  PulseCell<KIND> cp[C];
+  float w[C];
+#pragma unroll
+  for (int c = 0; c < C; ++c) {
+    const int jt = (blockIdx.x * C + c) * 256 + threadIdx.x;
+    valid[c] = jt < a.x_size;
+    j[c] = valid[c] ? jt : a.x_size - 1;
+    cell[c] = (unsigned)i * (unsigned)a.x_size + (unsigned)j[c];
+    cp[c].load(a.dev, cell[c]);
+    w[c] = a.w[cell[c]];
+  }
   const int kmax = a.kmax[a.kmax_slot];
-  __shared__ float noise[8 * 256]; // noise[q][thread]: a thread only ever touches its own column
-  if (kmax <= 3) w = pulsed_counted<KIND, MULT, 2>(a, w, cp, cell, i, j, valid, kmax, noise + threadIdx.x);
-  else if (kmax <= 7) w = pulsed_counted<KIND, MULT, 3>(a, w, cp, cell, i, j, valid, kmax, noise + threadIdx.x);
-  else w = pulsed_gather<KIND, MULT>(a, w, cp, cell, i, j, valid, kmax);
-  if (valid) a.w[cell] = w;
+  if (kmax <= 3) {
+    PulsedRows<KIND, MULT, 3, NOISE, C>(a, w, cp, tbl).run(cell[0], i, j, kmax);
+  } else if (kmax <= 7) {
+    PulsedRows<KIND, MULT, 7, NOISE, C>(a, w, cp, tbl).run(cell[0], i, j, kmax);
+  } else {
+#pragma unroll
+    for (int c = 0; c < C; ++c) w[c] = pulsed_gather<KIND, MULT>(a, w[c], cp[c], cell[c], i, j[c], valid[c], kmax);
+  }
+#pragma unroll
+  for (int c = 0; c < C; ++c) {
+    if (valid[c]) a.w[cell[c]] = w[c];
+  }
 }
 
 // deterministic implicit: n = (int) rintf((dv * BL) * xv) per sample (dense_bit_line_maker.cpp:237-264),
@@ -798,9 +885,59 @@ void launch_update_planes(const UpdateArgs &a, hipStream_t s) {
   hipLaunchKernelGGL(k_update_planes, grid, dim3(256), 0, s, a);
 }
 
+template <bool NOISE, int C> static void launch_update_pulsed_t(const UpdateArgs &a, hipStream_t s) {
+  dim3 grid((a.x_size + 256 * C - 1) / (256 * C), a.d_size);
+  if (a.dev.kind == RPU_DEVICE_CONSTANT_STEP) {
+    hipLaunchKernelGGL((k_update_pulsed<RPU_DEVICE_CONSTANT_STEP, true, NOISE, C>), grid, dim3(256), 0, s, a);
+  } else if (a.dev.ls_mult_noise) {
+    hipLaunchKernelGGL((k_update_pulsed<RPU_DEVICE_LINEAR_STEP, true, NOISE, C>), grid, dim3(256), 0, s, a);
+  } else {
+    hipLaunchKernelGGL((k_update_pulsed<RPU_DEVICE_LINEAR_STEP, false, NOISE, C>), grid, dim3(256), 0, s, a);
+  }
+}
+
 void launch_update_pulsed(const UpdateArgs &a, hipStream_t s) {
-  dim3 grid((a.x_size + 255) / 256, a.d_size);
-  RPU_DISPATCH_DEVICE(k_update_pulsed, grid, s, a);
+  // several columns per thread once a row is long enough to keep every lane busy with them
+  const bool wide = a.x_size >= 1024 && (long)a.x_size * a.d_size >= (1L << 19);
+  if (a.dev.dw_min_std > 0.0f) {
+    if (wide) launch_update_pulsed_t<true, 4>(a, s);
+    else launch_update_pulsed_t<true, 1>(a, s);
+  } else {
+    if (wide) launch_update_pulsed_t<false, 4>(a, s);
+    else launch_update_pulsed_t<false, 1>(a, s);
+  }
+}
+
+void ensure_update_tables() {
+  static std::mutex m;
+  static bool done[64] = {};
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) throw RpuError("No current HIP device.");
+  std::lock_guard<std::mutex> lock(m);
+  if (done[device]) return;
+  // quantile mid-points of the standard normal by bisection on erfc, lower half mirrored, scaled to unit variance
+  const int n = CTOC_LEVELS;
+  std::vector<double> xi(n);
+  double sum2 = 0.0;
+  for (int q = 0; q < n / 2; ++q) {
+    const double p = (q + 0.5) / n;
+    double lo = -10.0, hi = 0.0;
+    for (int it = 0; it < 80; ++it) {
+      const double mid = 0.5 * (lo + hi);
+      if (0.5 * std::erfc(-mid / std::sqrt(2.0)) < p) lo = mid;
+      else hi = mid;
+    }
+    xi[q] = 0.5 * (lo + hi);
+    xi[n - 1 - q] = -xi[q];
+    sum2 += 2.0 * xi[q] * xi[q];
+  }
+  const double norm = std::sqrt((double)n / sum2);
+  std::vector<float> table(n);
+  for (int q = 0; q < n; ++q) table[q] = (float)(xi[q] * norm);
+  if (hipMemcpyToSymbol(HIP_SYMBOL(g_ctoc_xi), table.data(), sizeof(float) * n) != hipSuccess) {
+    throw RpuError("Upload of the noise quantile table failed.");
+  }
+  done[device] = true;
 }
 
 void launch_update_implicit(const UpdateArgs &a, hipStream_t s) {

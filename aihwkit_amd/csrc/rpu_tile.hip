@@ -398,6 +398,7 @@ struct Tile {
         upload_params();
       }
       s_count.ensure(64);
+      ensure_update_tables();
     } catch (...) {
       release_all();
       device_id = -1;
