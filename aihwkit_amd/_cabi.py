@@ -188,6 +188,7 @@ SYMBOLS = {
     "rpu_tile_get_hidden_parameters": (C.c_int, [_P, _P]),
     "rpu_tile_set_hidden_parameters": (C.c_int, [_P, _P]),
     "rpu_tile_set_seed": (C.c_int, [_P, C.c_uint64]),
+    "rpu_tile_set_update_variant": (C.c_int, [_P, C.c_int, C.c_int]),
     "rpu_tile_update_noalloc": (C.c_int, [_P, _P, _P, C.c_int, C.c_int, C.c_int, C.c_int, _P]),
     "rpu_tile_get_update_words": (C.c_int, [_P, _P, _P, _P, C.c_int]),
     "rpu_tile_get_update_ab": (C.c_int, [_P, _P, _P, C.c_int]),

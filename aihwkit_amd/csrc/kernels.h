@@ -200,6 +200,9 @@ void launch_update_lines(const UpdateArgs &a, hipStream_t s);         // stochas
 void launch_update_implicit_lines(const UpdateArgs &a, hipStream_t s); // deterministic line values
 void launch_update_planes(const UpdateArgs &a, hipStream_t s);        // bit planes of pulse words made elsewhere
 void launch_update_pulsed(const UpdateArgs &a, hipStream_t s);        // coincidences + device steps
+// opt-in variant for LinearStep devices with multiplicative noise: per group of samples_per_step samples the
+// coincidences are counted and applied in closed form with one normal draw for their summed noise
+void launch_update_aggregated(const UpdateArgs &a, int samples_per_step, hipStream_t s);
 void launch_update_implicit(const UpdateArgs &a, hipStream_t s);
 void launch_implicit_counts(const UpdateArgs &a, int32_t *counts, hipStream_t s);
 // after an update of the persistent weights: w_apparent = w_persistent + noise_std * N(0, 1) at every cross-point that

@@ -16,6 +16,7 @@
 #include "kernels.h"
 #include "rpu_host.h"
 
+#include <algorithm>
 #include <cmath>
 #include <mutex>
 #include <vector>
@@ -689,6 +690,227 @@ __global__ __launch_bounds__(256, (C > 1 ? 4 : 8)) void k_update_pulsed(UpdateAr
   }
 }
 
+// ---- opt-in variant: aggregated steps -----------------------------------------------------------------------
+// NOT the reference's per-pulse arithmetic: a statistically equivalent short-cut for LinearStep / SoftBounds devices
+// with multiplicative cycle-to-cycle noise, chosen per tile (rpu_tile_set_update_variant).  The batch is cut into
+// groups of `agg_chunks` 32-sample chunks.  Per group a cross-point only counts its coincidences by direction
+// (population counts on the bit planes) and then takes n_up up-steps and n_dn down-steps in closed form: n noise-free
+// steps w <- w + (slope w + scale) move w to w + (slope w + scale) (a^n - 1) / slope with a = 1 + slope (n steps of
+// the geometric approach to -scale / slope; n (slope w + scale) when slope is zero), the up-steps split in two halves
+// around the down-steps (symmetric splitting: the error of ignoring the order inside a group is third order in
+// n * slope).  The cycle-to-cycle noise of the group's pulses is added as ONE normal draw per group with the summed
+// variance std^2 (n_up step_up^2 + n_dn step_dn^2), step sizes taken at the end of the group, then the device bounds are
+// applied once.  Mean and variance of
+// the weight change agree with the per-pulse update to first order in n * slope (about 1 % of the change per 32
+// samples at benchmark configuration 2); the pulse trains, their counts and their directions are exactly the same.
+struct AggCell {
+  float slope_up, scale_up, slope_dn, scale_dn, lo, hi;
+  float log_up, inv_up, lin_up, log_dn, inv_dn, lin_dn;
+  __device__ __forceinline__ void load(const DeviceDev &d, unsigned cell) {
+    PulseCell<RPU_DEVICE_LINEAR_STEP> p;
+    p.load(d, cell);
+    slope_up = p.slope_up; scale_up = p.scale_up; slope_dn = p.slope_dn; scale_dn = p.scale_dn; lo = p.lo; hi = p.hi;
+    prepare(slope_up, log_up, inv_up, lin_up);
+    prepare(slope_dn, log_dn, inv_dn, lin_dn);
+  }
+  // (a^n - 1) / slope = (exp2(n log2 a) - 1) * inv + n * lin, with lin = 1 and inv = 0 where the slope vanishes (or
+  // where 1 + slope is not positive, which no sensible device has: such a cross-point then takes linear steps)
+  static __device__ __forceinline__ void prepare(float slope, float &lg, float &inv, float &lin) {
+    const bool geometric = fabsf(slope) > 1e-7f;
+    // 1 + slope <= 0 (a bound closer than one step): the first step overshoots the fixed point and is cut back by the
+    // bounds, the following ones do not move: a^n is taken as 0 for every n >= 1
+    lg = !geometric ? 0.0f : (slope > -1.0f ? __builtin_amdgcn_logf(1.0f + slope) : -126.0f);
+    inv = geometric ? 1.0f / slope : 0.0f;
+    lin = geometric ? 0.0f : 1.0f;
+  }
+};
+
+__device__ __forceinline__ float agg_steps(float w, float n, float slope, float scale, float lg, float inv, float lin) {
+  const float first_step = __builtin_fmaf(slope, w, scale);
+  const float e = __builtin_amdgcn_exp2f(n * lg);
+  const float g = __builtin_fmaf(e - 1.0f, inv, n * lin);
+  return __builtin_fmaf(first_step, g, w);
+}
+
+// A lane holds R cross-points of one column (rows i0 .. i0 + R - 1): the x planes of a chunk are fetched once (the
+// next chunk's while this one is counted) and serve R rows, whose d planes are scalar loads.
+template <bool NOISE, int R> struct AggregatedRows {
+  const UpdateArgs &a;
+  const float *tbl;
+  AggCell cp[R];
+  float w[R];
+  unsigned n_all[R], n_dn[R];
+  int i0, rows; // rows: how many of the R rows exist
+  uint32_t s0 = 1u, s1 = 0u, lr_mask;
+
+  __device__ __forceinline__ AggregatedRows(const UpdateArgs &a_, const float *tbl_) : a(a_), tbl(tbl_) {}
+
+  // d planes of four chunks for the R rows, one word per lane: lane ((chunk & 3) * R + row) * 4 + kk holds pulse slot
+  // kk < 3, or the sign plane for kk = 3.  One gather per four chunks instead of a scalar load (and its latency) per
+  // row, chunk and slot; the counting loop reads the words back with v_readlane.
+  __device__ __forceinline__ uint32_t gather_d(unsigned block, int kmax) const {
+    static_assert(R == 4, "lane layout of the d-plane gather");
+    const unsigned lane = threadIdx.x & 63u;
+    const unsigned ch = 4u * block + (lane >> 4), r = (lane >> 2) & 3u, kk = lane & 3u;
+    const unsigned slots = (unsigned)a.plane_slots;
+    const unsigned slot = kk < 3u ? kk : slots - 1u;
+    const unsigned row = min((unsigned)i0 + r, (unsigned)a.d_size - 1u);
+    const bool wanted = ch < (unsigned)a.n_chunks && (kk == 3u || (int)kk < kmax);
+    const unsigned chc = min(ch, (unsigned)a.n_chunks - 1u);
+    const uint32_t v = a.d_planes[(size_t)(chc * slots + slot) * (unsigned)a.d_size + row];
+    return wanted ? v : 0u;
+  }
+
+  // counts of one chunk (q = chunk & 3) from its x planes and the gathered d planes
+  __device__ __forceinline__ void count(const ChunkPlanes<3, 1> &x, uint32_t dvec, int q) {
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      if (r >= rows) continue; // wave-uniform
+      uint32_t dk[3], any = 0u;
+#pragma unroll
+      for (int k = 0; k < 3; ++k) {
+        dk[k] = (uint32_t)__builtin_amdgcn_readlane((int)dvec, (q * R + r) * 4 + k);
+        any |= dk[k];
+      }
+      if (!any) continue;
+      const uint32_t dsg = (uint32_t)__builtin_amdgcn_readlane((int)dvec, (q * R + r) * 4 + 3);
+      const uint32_t same = x.sg[0] ^ (~dsg ^ lr_mask); // bit set: step down
+#pragma unroll
+      for (int k = 0; k < 3; ++k) {
+        if (!dk[k]) continue;
+        const uint32_t hit = dk[k] & x.k[0][k];
+        n_all[r] += __popc(hit);
+        n_dn[r] += __popc(hit & same);
+      }
+    }
+  }
+
+  // any bit-line length: planes read where they are used
+  __device__ __forceinline__ void count_generic(int j, unsigned ch, int kmax) {
+    const unsigned xs = (unsigned)a.x_size, ds = (unsigned)a.d_size, slots = (unsigned)a.plane_slots, base = ch * slots;
+    const uint32_t *xpl = a.x_planes + j;
+    const uint32_t xsg = xpl[(base + slots - 1u) * xs];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      if (r >= rows) continue;
+      const uint32_t *dpl = a.d_planes + (i0 + r);
+      const uint32_t same = xsg ^ (~dpl[(base + slots - 1u) * ds] ^ lr_mask);
+      for (int k = 0; k < kmax; ++k) {
+        const uint32_t dk = dpl[(base + (unsigned)k) * ds];
+        if (!dk) continue;
+        const uint32_t hit = dk & xpl[(base + (unsigned)k) * xs];
+        n_all[r] += __popc(hit);
+        n_dn[r] += __popc(hit & same);
+      }
+    }
+  }
+
+  __device__ __forceinline__ void apply() {
+    uint32_t rnd = 0u;
+    if (NOISE) {
+      rnd = s0 + s1;
+      s1 ^= s0;
+      s0 = __builtin_amdgcn_bitop3_b32(__builtin_rotateleft32(s0, 26), s1, s1 << 9, 0x96);
+      s1 = __builtin_rotateleft32(s1, 13);
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const float nd = (float)n_dn[r], nu = (float)(n_all[r] - n_dn[r]);
+      n_all[r] = n_dn[r] = 0u;
+      // half of the up-steps, all down-steps, the other half of the up-steps (symmetric splitting)
+      float wn = w[r];
+      wn = agg_steps(wn, 0.5f * nu, cp[r].slope_up, cp[r].scale_up, cp[r].log_up, cp[r].inv_up, cp[r].lin_up);
+      wn = agg_steps(wn, nd, cp[r].slope_dn, cp[r].scale_dn, cp[r].log_dn, cp[r].inv_dn, cp[r].lin_dn);
+      wn = agg_steps(wn, 0.5f * nu, cp[r].slope_up, cp[r].scale_up, cp[r].log_up, cp[r].inv_up, cp[r].lin_up);
+      if (NOISE) {
+        // The noise of a pulse is scaled by every later step of the group: n steps of one direction leave
+        // n * (last step)^2 * std^2, so the step sizes are taken where the group ends.
+        const float su = __builtin_fmaf(cp[r].slope_up, wn, cp[r].scale_up);
+        const float sd = __builtin_fmaf(cp[r].slope_dn, wn, cp[r].scale_dn);
+        const float var = __builtin_fmaf(nu * su, su, (nd * sd) * sd);
+        const float xi = *(const float *)((const char *)tbl + (((rnd >> (8 * (r & 3))) & 0xffu) << 2));
+        wn = __builtin_fmaf(__builtin_amdgcn_sqrtf(var), xi, wn);
+      }
+      w[r] = __builtin_amdgcn_fmed3f(wn, cp[r].lo, cp[r].hi);
+    }
+  }
+
+  __device__ __forceinline__ void run(int j, int kmax, int agg_chunks) {
+    const int n_chunks = a.n_chunks;
+    int in_group = 0;
+#pragma unroll
+    for (int r = 0; r < R; ++r) n_all[r] = n_dn[r] = 0u;
+    if (kmax <= 3) {
+      // blocks of four chunks: the x planes and the d-plane gather of the next block are in flight while this one
+      // is counted
+      const int jj[1] = {j};
+      const int n_blocks = (n_chunks + 3) / 4;
+      ChunkPlanes<3, 1> cur[4], nxt[4];
+      uint32_t dcur = gather_d(0u, kmax), dnxt = 0u;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) cur[q].load(a, jj, (unsigned)min(q, n_chunks - 1));
+      for (int b = 0; b < n_blocks; ++b) {
+        if (b + 1 < n_blocks) {
+          dnxt = gather_d((unsigned)b + 1u, kmax);
+#pragma unroll
+          for (int q = 0; q < 4; ++q) nxt[q].load(a, jj, (unsigned)min(4 * b + 4 + q, n_chunks - 1));
+        }
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int ch = 4 * b + q;
+          if (ch < n_chunks) {
+            count(cur[q], dcur, q);
+            if (++in_group == agg_chunks || ch + 1 == n_chunks) { apply(); in_group = 0; }
+          }
+        }
+#pragma unroll
+        for (int q = 0; q < 4; ++q) cur[q] = nxt[q];
+        dcur = dnxt;
+      }
+    } else {
+      for (int ch = 0; ch < n_chunks; ++ch) {
+        count_generic(j, (unsigned)ch, kmax);
+        if (++in_group == agg_chunks || ch + 1 == n_chunks) { apply(); in_group = 0; }
+      }
+    }
+  }
+};
+
+// grid: x = ceil(x_size / 256), y = ceil(d_size / R)
+template <bool NOISE, int R>
+__global__ __launch_bounds__(256) void k_update_aggregated(UpdateArgs a, int agg_chunks) {
+  __shared__ float tbl[CTOC_LEVELS]; // std * quantile
+  if (NOISE) {
+    tbl[threadIdx.x] = a.dev.dw_min_std * g_ctoc_xi[threadIdx.x];
+    __syncthreads();
+  }
+  AggregatedRows<NOISE, R> rows(a, tbl);
+  rows.i0 = blockIdx.y * R;
+  rows.rows = min(R, a.d_size - rows.i0);
+  rows.lr_mask = a.lr < 0.0f ? 0xffffffffu : 0u;
+  const int jt = blockIdx.x * 256 + threadIdx.x;
+  const bool valid = jt < a.x_size;
+  const int j = valid ? jt : a.x_size - 1;
+  unsigned cell[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const int i = min(rows.i0 + r, a.d_size - 1);
+    cell[r] = (unsigned)i * (unsigned)a.x_size + (unsigned)j;
+    rows.cp[r].load(a.dev, cell[r]);
+    rows.w[r] = a.w[cell[r]];
+  }
+  if (NOISE) {
+    const Philox4 p = philox4x32_10(cell[0], 1u, a.call, RNG_CTOC, a.key.k0, a.key.k1);
+    rows.s0 = p.v[0] | 1u;
+    rows.s1 = p.v[1];
+  }
+  rows.run(j, a.kmax[a.kmax_slot], agg_chunks);
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    if (valid && r < rows.rows) a.w[cell[r]] = rows.w[r];
+  }
+}
+
 // deterministic implicit: n = (int) rintf((dv * BL) * xv) per sample (dense_bit_line_maker.cpp:237-264),
 // |n| steps, n > 0 steps down (rpu_pulsed_device.h:461-474)
 template <int KIND, bool MULT>
@@ -906,6 +1128,14 @@ void launch_update_pulsed(const UpdateArgs &a, hipStream_t s) {
     if (wide) launch_update_pulsed_t<false, 4>(a, s);
     else launch_update_pulsed_t<false, 1>(a, s);
   }
+}
+
+void launch_update_aggregated(const UpdateArgs &a, int samples_per_step, hipStream_t s) {
+  const int agg_chunks = std::max(1, samples_per_step / 32);
+  constexpr int R = 4;
+  const dim3 grid((a.x_size + 255) / 256, (a.d_size + R - 1) / R);
+  if (a.dev.dw_min_std > 0.0f) hipLaunchKernelGGL((k_update_aggregated<true, R>), grid, dim3(256), 0, s, a, agg_chunks);
+  else hipLaunchKernelGGL((k_update_aggregated<false, R>), grid, dim3(256), 0, s, a, agg_chunks);
 }
 
 void ensure_update_tables() {

@@ -179,6 +179,7 @@ struct Tile {
   DevBuf<uint32_t> u_xw, u_dw, u_xpl, u_dpl;
   DevBuf<int> u_kmax;
   uint32_t update_calls = 0;
+  int update_variant = RPU_UPDATE_VARIANT_EXACT, update_variant_samples = 32;
   // where the last pulsed update left its per-sample values and packed words (own buffers or the static scratch)
   int *last_bl = nullptr;
   float *last_a = nullptr, *last_b = nullptr;
@@ -1089,8 +1090,13 @@ struct Tile {
       launch_update_lines(a, s);
       prof_mark(s, "update_lines");
       if (counting) count_pulses(a, false, s);
-      launch_update_pulsed(a, s);
-      prof_mark(s, "update_pulsed");
+      if (update_variant == RPU_UPDATE_VARIANT_AGGREGATED && dev.linear() && dev.p.ls_mult_noise && !is_transfer()) {
+        launch_update_aggregated(a, update_variant_samples, s);
+        prof_mark(s, "update_aggregated");
+      } else {
+        launch_update_pulsed(a, s);
+        prof_mark(s, "update_pulsed");
+      }
     } else {
       launch_update_implicit_lines(a, s);
       prof_mark(s, "update_implicit_lines");
@@ -2075,6 +2081,8 @@ int rpu_tile_clone(rpu_tile_t **out, const rpu_tile_t *src_c) {
     t.idx_patches = s.idx_patches;
     t.idx_max = s.idx_max;
     t.update_calls = s.update_calls;
+    t.update_variant = s.update_variant;
+    t.update_variant_samples = s.update_variant_samples;
     if (s.is_transfer()) {
       t.tr = std::make_unique<TransferPar>(*s.tr);
       t.update_idx = s.update_idx;
@@ -2445,6 +2453,24 @@ int rpu_tile_set_hidden_parameters(rpu_tile_t *tile, const float *data_host) {
       t.clip_host(t.w_host);
       if (t.persistent()) t.arr.persistent = t.w_host;
     }
+  });
+}
+
+int rpu_tile_set_update_variant(rpu_tile_t *tile, int variant, int samples_per_step) {
+  return guarded([&] {
+    if (!tile) throw RpuError("null tile");
+    Tile &t = tile->t;
+    std::lock_guard<std::mutex> lock(t.mutex);
+    if (variant != RPU_UPDATE_VARIANT_EXACT && variant != RPU_UPDATE_VARIANT_AGGREGATED) throw RpuError("Unknown update variant.");
+    if (variant == RPU_UPDATE_VARIANT_AGGREGATED) {
+      if (t.is_transfer() || !t.dev.linear() || !t.dev.p.ls_mult_noise || t.persistent()) {
+        throw RpuError("The aggregated update variant is provided for LinearStep / SoftBounds devices with multiplicative "
+                       "noise only (no transfer compound, no write noise).");
+      }
+      if (samples_per_step < 32 || samples_per_step % 32 != 0) throw RpuError("samples_per_step must be a positive multiple of 32.");
+    }
+    t.update_variant = variant;
+    t.update_variant_samples = samples_per_step;
   });
 }
 

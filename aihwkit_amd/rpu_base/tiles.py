@@ -196,6 +196,15 @@ class _TileBase:
         """Seed of the Philox generator behind every random draw of this tile on the GPU."""
         check(lib().rpu_tile_set_seed(self._h, int(seed) & 0xFFFFFFFFFFFFFFFF))
 
+    def set_update_variant(self, variant: str = "exact", samples_per_step: int = 32) -> None:
+        """Not in the reference: "exact" (default) applies the coincidences pulse by pulse like the reference;
+        "aggregated" (opt-in, LinearStep / SoftBounds with multiplicative noise) counts them per group of
+        `samples_per_step` samples and applies them in closed form with one noise draw per group."""
+        codes = {"exact": 0, "aggregated": 1}
+        if variant not in codes:
+            raise RuntimeError("Unknown update variant: " + str(variant))
+        check(lib().rpu_tile_set_update_variant(self._h, codes[variant], int(samples_per_step)))
+
     # -- state beyond weights and hidden parameters (rpu_base_tiles.cpp:89-113)
     def dump_extra(self) -> dict:
         count = lib().rpu_tile_extra_count(self._h)

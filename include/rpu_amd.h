@@ -385,6 +385,18 @@ int rpu_tile_set_hidden_parameters(rpu_tile_t *tile, const float *data_host);
  * Stands in for the per-context cuRAND state of the reference (C/cuda_util.cu:163-176,779-800). */
 int rpu_tile_set_seed(rpu_tile_t *tile, uint64_t seed);
 
+/* No counterpart in the reference.  Chooses how the stochastic pulsed update applies the coincidences of a batch:
+ * RPU_UPDATE_VARIANT_EXACT (default): pulse by pulse in batch order with a normal draw per pulse, as
+ * PulsedRPUWeightUpdater::updateVectorWithDevice (R/rpu_weight_updater.cpp:197-294) does.
+ * RPU_UPDATE_VARIANT_AGGREGATED (opt-in; LinearStep / SoftBounds with multiplicative noise only): per group of
+ * samples_per_step samples (a multiple of 32) a cross-point counts its coincidences by direction and takes them in
+ * closed form (geometric approach to the soft bound) with one normal draw carrying the summed cycle-to-cycle
+ * variance; same pulse trains, same counts, mean and variance of the weight change equal to first order in
+ * n * slope.  A statistical equivalent, not the reference's arithmetic: labelled wherever it is measured. */
+#define RPU_UPDATE_VARIANT_EXACT 0
+#define RPU_UPDATE_VARIANT_AGGREGATED 1
+int rpu_tile_set_update_variant(rpu_tile_t *tile, int variant, int samples_per_step);
+
 /* ---- indexed (convolution) interface ----------------------------------------------------------- */
 
 /* Replaces RPUSimple::setMatrixIndices (R/rpu.h:397-402) as bound at B/rpu_base_tiles.cpp:721-737: the index

@@ -120,15 +120,14 @@ def test_rows_with_another_round_count_sit_on_the_saturation_edge(gpu_device):
 
 def test_moments_over_64_seeds_at_the_graded_shape(gpu_device):
     """Configuration 2 as graded (1024 x 1024, batch 256, output noise 0.06, cycle-to-cycle 0.3, stochastic pulses with
-    update management): mean and variance over 64 seeds of forward outputs, backward outputs and the weight change,
-    GPU against oracle, per element and pooled."""
+    update management): mean and variance over 64 seeds of forward and backward outputs, GPU against oracle, per
+    element and pooled (the weight change: next test)."""
     n_seeds = 64
     meta, dev = config2()
     host, orc, _ = build_pair(meta, dev, 1024, 1024, gpu=False)
     w, x, d = config2_data()
     host.set_weights(torch.from_numpy(w))
     orc.set_weights(w)
-    w0 = orc.get_weights().copy()
     xg, dg = cuda(x), cuda(d)
     gpu = tiles.CudaAnalogTile(host)
     yg, yo, bg, bo, rg, ro = [], [], [], [], [], []
@@ -144,25 +143,109 @@ def test_moments_over_64_seeds_at_the_graded_shape(gpu_device):
     assert abs(np.mean(rg) - np.mean(ro)) < 0.02 and np.mean(ro) > 1.5
     compare_moments(np.stack(yg), np.stack(yo), "forward outputs at the graded shape")
     compare_moments(np.stack(bg), np.stack(bo), "backward outputs at the graded shape")
-    del yg, yo, bg, bo
-    dwg = np.empty((n_seeds, 1024, 1024), F32)
+
+
+@pytest.fixture(scope="module")
+def oracle_weight_changes():
+    """Weight change of the oracle over 64 seeds at the graded shape (shared by the exact kernel and the variants)."""
+    n_seeds = 64
+    meta, dev = config2()
+    host, orc, _ = build_pair(meta, dev, 1024, 1024, gpu=False)
+    w, x, d = config2_data()
+    orc.set_weights(w)
+    w0 = orc.get_weights().copy()
     dwo = np.empty((n_seeds, 1024, 1024), F32)
     for s in range(n_seeds):
-        gpu.set_weights(torch.from_numpy(w))
-        gpu.set_seed(900 + s)
-        gpu.set_learning_rate(0.01)
-        gpu.update(xg, dg, False, False, False, False)
-        dwg[s] = gpu.get_weights().numpy() - w0
         orc.set_weights(w)
         orc.set_seed(101 + s)
         orc.set_learning_rate(0.01)
         orc.update(x, d)
         dwo[s] = orc.get_weights() - w0
     assert np.abs(dwo).mean() > 2e-3
+    return dwo, w0
+
+
+@pytest.mark.parametrize("variant,samples", [("exact", 32), ("aggregated", 32), ("aggregated", 64)])
+def test_weight_change_moments_over_64_seeds_at_the_graded_shape(gpu_device, oracle_weight_changes, variant, samples):
+    """The same protocol for the weight change of one update call, for the per-pulse kernel and for the opt-in
+    aggregated variant with groups of 32 and of 64 samples: a variant is offered only because this unchanged test
+    passes with it (groups of the whole batch, 256 samples, do not pass: 8 % too much noise variance)."""
+    dwo, w0 = oracle_weight_changes
+    meta, dev = config2()
+    host = meta.create_array(1024, 1024, dev)
+    w, x, d = config2_data()
+    host.set_weights(torch.from_numpy(w))
+    gpu = tiles.CudaAnalogTile(host)
+    gpu.set_update_variant(variant, samples)
+    xg, dg = cuda(x), cuda(d)
+    dwg = np.empty_like(dwo)
+    for s in range(dwo.shape[0]):
+        gpu.set_weights(torch.from_numpy(w))
+        gpu.set_seed(900 + s)
+        gpu.set_learning_rate(0.01)
+        gpu.update(xg, dg, False, False, False, False)
+        dwg[s] = gpu.get_weights().numpy() - w0
     # per element and pooled on a quarter of the matrix at a time (memory), all four quarters
     for q in range(4):
         rows = slice(256 * q, 256 * (q + 1))
-        compare_moments(dwg[:, rows], dwo[:, rows], f"weight change at the graded shape, rows {256 * q}..")
+        compare_moments(dwg[:, rows], dwo[:, rows], f"weight change ({variant} {samples}) at the graded shape, rows {256 * q}..")
+
+
+def test_aggregated_variant_closed_form_and_first_order_agreement(gpu_device):
+    """Pins the closed form of the aggregated variant without statistics (cycle-to-cycle noise off):
+    (1) one direction only (x > 0, d > 0): n steps down are exactly the geometric sequence, so the variant must equal
+        the oracle's pulse-by-pulse result to rounding;
+    (2) mixed directions: it may differ from the pulse-by-pulse result only by the ordering error, second order in
+        n * slope -- far below one step;
+    (3) it is refused where it does not apply."""
+    rng = np.random.default_rng(5)
+    x_size, d_size, batch = 200, 90, 96
+    meta = make_meta(desired_bl=31, update_management=True, update_bl_management=True)
+    kw = dict(dw_min=0.001, dw_min_dtod=0.3, dw_min_std=0.0, up_down_dtod=0.01, w_max_dtod=0.3, w_min_dtod=0.3,
+              construction_seed=77, enforce_consistency=True)
+    for one_sided in (True, False):
+        host, orc, _ = build_pair(meta, soft_bounds(**kw), x_size, d_size, gpu=False)
+        w = rng.uniform(-0.4, 0.4, (d_size, x_size)).astype(F32)
+        host.set_weights(torch.from_numpy(w))
+        orc.set_weights(w)
+        x = rng.uniform(-1, 1, (batch, x_size)).astype(F32)
+        d = (0.05 * rng.standard_normal((batch, d_size))).astype(F32)
+        if one_sided:
+            x, d = np.abs(x), np.abs(d)
+        for samples in (32, 96):
+            gpu = tiles.CudaAnalogTile(host)
+            gpu.set_seed(3)
+            gpu.set_learning_rate(0.01)
+            gpu.set_update_variant("aggregated", samples)
+            gpu.update(cuda(x), cuda(d), False, False, False, False)
+            xw, dw, bl = (t.numpy() for t in gpu.get_update_words(batch))
+            twin = OracleTile(x_size, d_size, meta._config(soft_bounds(**kw)))
+            twin.set_hidden(orc.get_hidden())
+            twin.set_weights(w)
+            twin.set_learning_rate(0.01)
+            twin.update_with_words(xw, dw, bl)
+            got, want = gpu.get_weights().numpy(), twin.get_weights()
+            moved = np.abs(want - orc.get_weights())
+            assert moved.mean() > 3e-3                                  # some twenty pulses per cross-point
+            hidden = orc.get_hidden()
+            regular = (np.abs(hidden[8]) < 0.005) & (np.abs(hidden[9]) < 0.005)   # bounds at least 200 steps away from zero
+            assert regular.mean() > 0.95
+            err = np.abs(got - want)
+            if one_sided:
+                assert err[regular].max() <= 3e-6
+            else:
+                # the order of up and down steps inside a group is not kept: each swapped pair costs
+                # scale_up * scale_down * (1 / w_max + 1 / |w_min|), about 4e-6; zero on average
+                # (a step is 1e-3; the larger the group, the more pairs)
+                assert err[regular].max() <= (4e-4 if samples == 32 else 2e-3)
+                assert err[regular].mean() <= (2e-5 if samples == 32 else 2e-4)
+                assert abs((got - want)[regular].mean()) <= 1e-5
+            assert np.all(got <= hidden[0] + 1e-7) and np.all(got >= hidden[1] - 1e-7)
+    with pytest.raises(RuntimeError, match="aggregated update variant"):
+        _, _, cs = build_pair(meta, constant_step(dw_min=0.001), 8, 8)
+        cs.set_update_variant("aggregated", 32)
+    with pytest.raises(RuntimeError, match="multiple of 32"):
+        gpu.set_update_variant("aggregated", 48)
 
 
 def test_full_size_configuration_1_update_through_the_pulse_words(gpu_device):
