@@ -150,6 +150,8 @@ SYMBOLS = {
     "rpu_tile_pulse_counter_count": (C.c_int, [_P]),
     "rpu_tile_get_pulse_counters": (C.c_int, [_P, _P]),
     "rpu_tile_set_shared_weights": (C.c_int, [_P, _P]),
+    "rpu_tile_set_shared_weights_xd": (C.c_int, [_P, _P]),
+    "rpu_tile_set_delta_weights_xd": (C.c_int, [_P, _P]),
     "rpu_tile_get_shared_weights_if": (C.c_int, [_P]),
     "rpu_tile_set_delta_weights": (C.c_int, [_P, _P]),
     "rpu_tile_extra_count": (C.c_int, [_P]),

@@ -233,6 +233,8 @@ void launch_reset_cols(float *w, const float *reset_bias, const float *w_min, co
                        hipStream_t s);
 // prev_w_and_delta holds the weights from before an update: it becomes scale * (w - previous), w gets them back
 void launch_delta_finish(float *w, float *prev_w_and_delta, float scale, size_t n, hipStream_t s);
+// out[c][r] = in[r][c] for a row-major [rows][cols] matrix
+void launch_transpose(const float *in, float *out, int rows, int cols, hipStream_t s);
 
 // power-law drift of every weight that has stayed within reset_tol of its value after the last call
 // (WeightDrifter::apply, weight_drifter.cpp:108-150); nu == null: the same nu0 for every element

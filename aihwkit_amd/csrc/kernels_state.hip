@@ -467,6 +467,26 @@ void launch_write_noise_all(float *w_apparent, const float *w_persistent, float 
                      key, call, n);
 }
 
+// out[c][r] = in[r][c] for a row-major [rows][cols] matrix, 32 x 32 tiles through LDS
+__global__ __launch_bounds__(256) void k_transpose(const float *__restrict__ in, float *__restrict__ out, int rows, int cols) {
+  __shared__ float tile[32][33];
+  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+  const int c0 = blockIdx.x * 32, r0 = blockIdx.y * 32;
+  for (int i = ty; i < 32; i += 8) {
+    const int r = r0 + i, c = c0 + tx;
+    if (r < rows && c < cols) tile[i][tx] = in[(size_t)r * cols + c];
+  }
+  __syncthreads();
+  for (int i = ty; i < 32; i += 8) {
+    const int c = c0 + i, r = r0 + tx;
+    if (r < rows && c < cols) out[(size_t)c * rows + r] = tile[tx][i];
+  }
+}
+
+void launch_transpose(const float *in, float *out, int rows, int cols, hipStream_t s) {
+  hipLaunchKernelGGL(k_transpose, dim3((cols + 31) / 32, (rows + 31) / 32), dim3(256), 0, s, in, out, rows, cols);
+}
+
 void launch_delta_finish(float *w, float *prev_w_and_delta, float scale, size_t n, hipStream_t s) {
   hipLaunchKernelGGL(k_delta_finish, dim3(grid_for(n)), dim3(256), 0, s, w, prev_w_and_delta, scale, n);
 }

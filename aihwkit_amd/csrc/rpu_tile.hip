@@ -210,6 +210,13 @@ struct Tile {
   DevBuf<float> d_decay, d_diff, d_rbias, s_clip;
   bool state_params_valid = false;
   float *delta_w = nullptr;
+  // the reference's CUDA tiles exchange shared and delta weights as [x_size][d_size] (column-major) tensors
+  // (rpu_base_tiles_cuda.cpp:88-130).  The matrices of this library stay row-major [d_size][x_size]; a caller's
+  // column-major tensor is kept in step by transposition: read into the tile before a call that uses the weights,
+  // written back after a call that changes them.
+  float *shared_xd = nullptr;
+  float *delta_xd = nullptr;
+  DevBuf<float> d_delta_own;
   // hardware-aware training: the modified copy of the weights that forward / backward contract with, scratch of
   // the remapper ([3 D + 1]: row statistic, multiplier, divisor, one scalar), the drift clock per weight and the
   // pulse counters [2][size]
@@ -306,6 +313,9 @@ struct Tile {
     d_decay.release(); d_diff.release(); d_rbias.release(); s_clip.release();
     state_params_valid = false;
     delta_w = nullptr;
+    shared_xd = nullptr;
+    delta_xd = nullptr;
+    d_delta_own.release();
     n_pre.release(); n_s1.release(); n_s2.release(); n_s3.release(); n_rows.release(); n_absw.release();
     n_sumsq.release();
     n_s4.release();
@@ -1030,6 +1040,38 @@ struct Tile {
   void set_delta_weights(float *dw_dev) {
     if (dw_dev) check_maintenance("set_delta_weights");
     delta_w = dw_dev;
+    delta_xd = nullptr;
+  }
+
+  // RPUCudaSimple::setSharedWeights (cuda/rpucuda.cu:322-334) with the CUDA tiles' [x_size][d_size] layout: the
+  // tile's weights are copied into the tensor, which mirrors them from then on
+  void set_shared_weights_xd(float *w_xd_dev) {
+    check_maintenance("set_shared_weights");
+    if (!w_xd_dev) throw RpuError("Null device pointer.");
+    if (!d_w.owned) throw RpuError("The tile already uses a row-major shared weight buffer.");
+    sync_last();
+    launch_transpose(d_w.p, w_xd_dev, D, X, last_stream);
+    RPU_HIP_CHECK(hipGetLastError());
+    RPU_HIP_CHECK(hipStreamSynchronize(last_stream));
+    shared_xd = w_xd_dev;
+  }
+  void set_delta_weights_xd(float *dw_xd_dev) {
+    if (!dw_xd_dev) {
+      set_delta_weights(nullptr);
+      return;
+    }
+    check_maintenance("set_delta_weights");
+    d_delta_own.ensure(size());
+    delta_w = d_delta_own.p;
+    delta_xd = dw_xd_dev;
+  }
+  // before a call that reads the weights / after a call that may have changed them (or the delta buffer)
+  void shared_in(hipStream_t s) {
+    if (shared_xd) launch_transpose(shared_xd, d_w.p, X, D, s);
+  }
+  void shared_out(hipStream_t s) {
+    if (shared_xd) launch_transpose(d_w.p, shared_xd, D, X, s);
+    if (delta_xd) launch_transpose(d_delta_own.p, delta_xd, D, X, s);
   }
 
   DeviceView view_of(DeviceSlot &sl, float granularity) {
@@ -1546,7 +1588,9 @@ int rpu_tile_has_matrix_indices(const rpu_tile_t *tile) { return tile ? tile->t.
     if (image_size <= 0) throw RpuError("image_size must be positive.");                       \
     if ((long)t.idx_max - 2 >= image_size) throw RpuError("Index matrix entry beyond the image size."); \
     DeviceGuard g(t.device_id);                                                                \
+    t.shared_in((hipStream_t)stream);                                                          \
     CALL;                                                                                      \
+    t.shared_out((hipStream_t)stream);                                                         \
   })
 
 int rpu_tile_forward_indexed(rpu_tile_t *tile, const float *x_dev, float *d_dev, int n_images, long image_size,
@@ -1568,6 +1612,21 @@ int rpu_tile_update_indexed(rpu_tile_t *tile, const float *x_dev, const float *d
 // ---- weight maintenance between steps, shared and delta weights, extra state --------------------------
 
 #define RPU_MAINTENANCE_ENTRY(CALL)                                \
+  return guarded([&] {                                             \
+    if (!tile) throw RpuError("null tile");                        \
+    Tile &t = tile->t;                                             \
+    std::lock_guard<std::mutex> lock(t.mutex);                     \
+    if (!t.resident()) {                                           \
+      CALL;                                                        \
+      return;                                                      \
+    }                                                              \
+    DeviceGuard g(t.device_id);                                    \
+    t.shared_in((hipStream_t)stream);                              \
+    CALL;                                                          \
+    t.shared_out((hipStream_t)stream);                             \
+  })
+
+#define RPU_MAINTENANCE_ENTRY_NOSYNC(CALL)                         \
   return guarded([&] {                                             \
     if (!tile) throw RpuError("null tile");                        \
     Tile &t = tile->t;                                             \
@@ -1683,13 +1742,23 @@ int rpu_tile_set_forward_out_scale(rpu_tile_t *tile, float out_scale) {
 }
 
 int rpu_tile_set_shared_weights(rpu_tile_t *tile, float *weights_dev) {
-  RPU_MAINTENANCE_ENTRY(t.set_shared_weights(weights_dev));
+  RPU_MAINTENANCE_ENTRY_NOSYNC(t.set_shared_weights(weights_dev));
 }
 
-int rpu_tile_get_shared_weights_if(const rpu_tile_t *tile) { return (tile && !tile->t.d_w.owned) ? 1 : 0; }
+int rpu_tile_get_shared_weights_if(const rpu_tile_t *tile) {
+  return (tile && (!tile->t.d_w.owned || tile->t.shared_xd)) ? 1 : 0;
+}
+
+int rpu_tile_set_shared_weights_xd(rpu_tile_t *tile, float *weights_xd_dev) {
+  RPU_MAINTENANCE_ENTRY_NOSYNC(t.set_shared_weights_xd(weights_xd_dev));
+}
+
+int rpu_tile_set_delta_weights_xd(rpu_tile_t *tile, float *delta_weights_xd_dev) {
+  RPU_MAINTENANCE_ENTRY_NOSYNC(t.set_delta_weights_xd(delta_weights_xd_dev));
+}
 
 int rpu_tile_set_delta_weights(rpu_tile_t *tile, float *delta_weights_dev) {
-  RPU_MAINTENANCE_ENTRY(t.set_delta_weights(delta_weights_dev));
+  RPU_MAINTENANCE_ENTRY_NOSYNC(t.set_delta_weights(delta_weights_dev));
 }
 #undef RPU_MAINTENANCE_ENTRY
 
@@ -1837,6 +1906,7 @@ int rpu_group_create(rpu_group_t **out, rpu_tile_t *const *tiles, int n_tiles) {
       }
       Tile &t = tiles[i]->t;
       if (!t.resident()) throw RpuError("All tiles of a group must be resident on a GPU.");
+      if (t.shared_xd) throw RpuError("A tile with column-major shared weights cannot be in a group.");
       if (g->device_id < 0) g->device_id = t.device_id;
       if (t.device_id != g->device_id) throw RpuError("All tiles of a group must be on the same GPU.");
       g->tiles.push_back(tiles[i]);
@@ -2007,7 +2077,9 @@ int rpu_tile_program_weights(rpu_tile_t *tile, const rpu_pcm_noise_params *p, in
     std::lock_guard<std::mutex> lock(t.mutex);
     if (!t.resident()) throw RpuError("Tile is not resident on a GPU.");
     DeviceGuard g(t.device_id);
+    t.shared_in((hipStream_t)stream);
     t.program_weights(*p, from_reference != 0, (hipStream_t)stream);
+    t.shared_out((hipStream_t)stream);
   });
 }
 
@@ -2018,7 +2090,9 @@ int rpu_tile_drift_weights(rpu_tile_t *tile, const rpu_pcm_noise_params *p, floa
     std::lock_guard<std::mutex> lock(t.mutex);
     if (!t.resident()) throw RpuError("Tile is not resident on a GPU.");
     DeviceGuard g(t.device_id);
+    t.shared_in((hipStream_t)stream);
     t.drift_weights(*p, t_inference, (hipStream_t)stream);
+    t.shared_out((hipStream_t)stream);
   });
 }
 
@@ -2044,6 +2118,7 @@ int rpu_tile_drift_readout(rpu_tile_t *tile, float *mean_abs_host, void *stream)
     std::lock_guard<std::mutex> lock(t.mutex);
     if (!t.resident()) throw RpuError("Tile is not resident on a GPU.");
     DeviceGuard g(t.device_id);
+    t.shared_in((hipStream_t)stream);
     *mean_abs_host = t.drift_readout((hipStream_t)stream);
   });
 }
@@ -2152,6 +2227,7 @@ int rpu_tile_forward(rpu_tile_t *tile, const float *x_dev, float *y_dev, int m_b
     std::lock_guard<std::mutex> lock(t.mutex);
     if (!t.check_compute(m_batch, x_dev, y_dev)) return;
     DeviceGuard g(t.device_id);
+    t.shared_in((hipStream_t)stream);
     t.mvm(x_dev, y_dev, m_batch, bias != 0, x_trans != 0, d_trans != 0, false, (hipStream_t)stream, nullptr, nullptr,
           is_test != 0);
   });
@@ -2165,6 +2241,7 @@ int rpu_tile_backward(rpu_tile_t *tile, const float *d_dev, float *x_dev, int m_
     std::lock_guard<std::mutex> lock(t.mutex);
     if (!t.check_compute(m_batch, d_dev, x_dev)) return;
     DeviceGuard g(t.device_id);
+    t.shared_in((hipStream_t)stream);
     t.mvm(d_dev, x_dev, m_batch, bias != 0, d_trans != 0, x_trans != 0, true, (hipStream_t)stream);
   });
 }
@@ -2177,7 +2254,9 @@ int rpu_tile_update(rpu_tile_t *tile, const float *x_dev, const float *d_dev, in
     std::lock_guard<std::mutex> lock(t.mutex);
     if (!t.check_compute(m_batch, x_dev, d_dev)) return;
     DeviceGuard g(t.device_id);
+    t.shared_in((hipStream_t)stream);
     t.update(x_dev, d_dev, m_batch, bias != 0, x_trans != 0, d_trans != 0, (hipStream_t)stream);
+    t.shared_out((hipStream_t)stream);
   });
 }
 
@@ -2189,7 +2268,9 @@ int rpu_tile_update_noalloc(rpu_tile_t *tile, const float *x_dev, const float *d
     std::lock_guard<std::mutex> lock(t.mutex);
     if (!t.check_compute(m_batch, x_dev, d_dev)) return;
     DeviceGuard g(t.device_id);
+    t.shared_in((hipStream_t)stream);
     t.update_noalloc(x_dev, d_dev, m_batch, bias != 0, x_trans != 0, d_trans != 0, (hipStream_t)stream);
+    t.shared_out((hipStream_t)stream);
   });
 }
 
@@ -2201,7 +2282,9 @@ int rpu_tile_update_with_words(rpu_tile_t *tile, const uint32_t *x_words_dev, co
     std::lock_guard<std::mutex> lock(t.mutex);
     if (!t.check_compute(m_batch, x_words_dev, d_words_dev)) return;
     DeviceGuard g(t.device_id);
+    t.shared_in((hipStream_t)stream);
     t.update_with_words(x_words_dev, d_words_dev, m_batch, (hipStream_t)stream);
+    t.shared_out((hipStream_t)stream);
   });
 }
 
@@ -2249,6 +2332,10 @@ int rpu_tile_set_weights(rpu_tile_t *tile, const float *w_host) {
           RPU_HIP_CHECK(hipStreamSynchronize(t.last_stream));
         }
       }
+      if (t.shared_xd) {
+        t.shared_out(t.last_stream);
+        RPU_HIP_CHECK(hipStreamSynchronize(t.last_stream));
+      }
     } else {
       if (t.persistent()) {
         t.arr.persistent = w;
@@ -2272,6 +2359,7 @@ int rpu_tile_get_weights(rpu_tile_t *tile, float *w_host) {
     std::lock_guard<std::mutex> lock(t.mutex);
     if (t.resident()) {
       DeviceGuard g(t.device_id);
+      t.shared_in(t.last_stream);
       t.sync_last();
       RPU_HIP_CHECK(hipMemcpy(w_host, t.wdev(), t.size() * sizeof(float), hipMemcpyDeviceToHost));
     } else {
@@ -2443,11 +2531,13 @@ int rpu_tile_set_hidden_parameters(rpu_tile_t *tile, const float *data_host) {
       DeviceGuard g(t.device_id);
       t.sync_last();
       t.upload_params();
+      t.shared_in(t.last_stream);
       launch_clip(t.d_w.p, t.d_wmin.p, t.d_wmax.p, n, t.last_stream);
       if (t.persistent()) {
         RPU_HIP_CHECK(hipMemcpyAsync(t.d_wp.p, t.d_w.p, n * sizeof(float), hipMemcpyDeviceToDevice, t.last_stream));
         if (t.dev.p.apply_write_noise_on_set) t.refresh_shown_weights(t.last_stream);
       }
+      t.shared_out(t.last_stream);
       RPU_HIP_CHECK(hipStreamSynchronize(t.last_stream));
     } else {
       t.clip_host(t.w_host);

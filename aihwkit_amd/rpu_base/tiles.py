@@ -414,28 +414,43 @@ class _CudaTileMixin:
         check(lib().rpu_tile_get_modified_weights(self._h, out.data_ptr()))
         return out
 
-    # -- shared and delta weights (rpu_base_tiles.cpp:215-251)
+    # -- shared and delta weights as the reference's CUDA tiles bind them (rpu_base_tiles_cuda.cpp:88-130): the
+    # tensors are [x_size, d_size] ("weight is d major for CUDA"), which is what the reference's Python allocates for
+    # a tile whose class name contains "Cuda" and reads back through .t() (simulator/tiles/base.py:392-446)
     def _check_matrix(self, tensor: torch.Tensor, what: str) -> torch.Tensor:
         if isinstance(tensor, torch.Tensor) and not tensor.is_contiguous():
             raise RuntimeError(what + " must be contiguous")
         tensor = _check_input(tensor, True, what)
-        if tensor.dim() != 2 or tensor.size(0) != self.get_d_size() or tensor.size(1) != self.get_x_size():
-            raise RuntimeError("Invalid %s dimensions: expected [%d,%d] tensor" % (what, self.get_d_size(), self.get_x_size()))
+        if tensor.dim() != 2 or tensor.size(0) != self.get_x_size() or tensor.size(1) != self.get_d_size():
+            raise RuntimeError("Invalid %s dimensions: expected [%d,%d] array" % (what, self.get_x_size(), self.get_d_size()))
+        if tensor.device.index != self._device.index:
+            raise RuntimeError("%s need to be on the same cuda device: expected %d, got %d"
+                               % (what.capitalize(), self._device.index, tensor.device.index))
         return tensor
 
     def set_shared_weights(self, weights: torch.Tensor) -> None:
-        """``weights`` (a CUDA tensor) becomes the weight matrix of the tile and must outlive it."""
+        """``weights``, a CUDA tensor ``[x_size, d_size]``, mirrors the weight matrix of the tile from now on (the
+        tile's weights are copied into it; it is re-read before and re-written after every call) and must outlive it."""
         weights = self._check_matrix(weights, "weights")
-        check(lib().rpu_tile_set_shared_weights(self._h, weights.data_ptr()))
+        check(lib().rpu_tile_set_shared_weights_xd(self._h, weights.data_ptr()))
         self._shared_weights = weights
 
     def set_delta_weights(self, delta_weights: torch.Tensor) -> None:
         delta_weights = self._check_matrix(delta_weights, "delta weights")
-        check(lib().rpu_tile_set_delta_weights(self._h, delta_weights.data_ptr()))
+        check(lib().rpu_tile_set_delta_weights_xd(self._h, delta_weights.data_ptr()))
         self._delta_weights = delta_weights
 
+    def set_shared_weights_row_major(self, weights: torch.Tensor) -> None:
+        """Not in the reference: the tile adopts a ``[d_size, x_size]`` CUDA tensor as its weight matrix itself (no
+        copies between calls), for callers written against this library."""
+        if not (isinstance(weights, torch.Tensor) and weights.is_cuda and weights.is_contiguous()
+                and tuple(weights.shape) == (self.get_d_size(), self.get_x_size()) and weights.dtype == _DTYPE):
+            raise RuntimeError("Invalid weights: expected a contiguous [%d,%d] CUDA tensor" % (self.get_d_size(), self.get_x_size()))
+        check(lib().rpu_tile_set_shared_weights(self._h, weights.data_ptr()))
+        self._shared_weights = weights
+
     def reset_delta_weights(self) -> None:
-        check(lib().rpu_tile_set_delta_weights(self._h, None))
+        check(lib().rpu_tile_set_delta_weights_xd(self._h, None))
         self._delta_weights = None
 
     def _patches(self) -> int:

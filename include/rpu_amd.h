@@ -601,6 +601,19 @@ int rpu_tile_set_forward_out_scale(rpu_tile_t *tile, float out_scale);
 int rpu_tile_set_shared_weights(rpu_tile_t *tile, float *weights_dev);
 int rpu_tile_get_shared_weights_if(const rpu_tile_t *tile);
 
+/* set_shared_weights / set_delta_weights as the reference's CUDA tiles bind them (rpu_base_tiles_cuda.cpp:88-130,
+ * RPUCudaSimple::setSharedWeights, C/rpucuda.cu:322-334): the device tensor is [x_size][d_size] (column-major W), which
+ * is what the reference's Python allocates for a tile whose class name contains "Cuda" and reads back through .t()
+ * (src/aihwkit/simulator/tiles/base.py:392-446).  The matrices of this library stay row-major, so the tensor is kept
+ * in step by a transposition kernel: it takes the tile's weights when it is set, is read into the tile before every
+ * call that uses the weights (the caller may have written to it) and written back after every call that may change
+ * them -- one or two passes over the matrix per call (about 3 us each for 1024 x 1024) on top of the call itself;
+ * the row-major entry points above have no such cost.  With delta weights the update lands in a buffer of the tile
+ * and is transposed into the caller's tensor after the call; null ends the mode.  Not provided for transfer compounds
+ * and for members of a group. */
+int rpu_tile_set_shared_weights_xd(rpu_tile_t *tile, float *weights_xd_dev);
+int rpu_tile_set_delta_weights_xd(rpu_tile_t *tile, float *delta_weights_xd_dev);
+
 /* set_delta_weights / reset_delta_weights (rpu_base_tiles.cpp:230-251): while a device buffer [d_size][x_size]
  * is set, an update leaves the weights as they are and writes dW with W_new = W - lr * dW into the buffer
  * (rpu.cpp:1459-1510, rpu_pulsed.cpp:560-585); null ends the mode. */

@@ -155,31 +155,92 @@ def test_reset_columns(gpu_device):
 
 
 def test_shared_weights(gpu_device):
+    """The reference's CUDA tiles take a [x_size, d_size] tensor (rpu_base_tiles_cuda.cpp:88-109)."""
     tile = pulsed_tile()
     w = tile.get_weights()
-    shared = torch.zeros(23, 37, device="cuda")
+    shared = torch.zeros(37, 23, device="cuda")
     assert not tile.get_shared_weights_if()
     tile.set_shared_weights(shared)
     assert tile.get_shared_weights_if()
-    assert torch.equal(shared.cpu(), w)                   # the tile's weights moved into the tensor
+    assert torch.equal(shared.t().cpu(), w)               # the tile's weights moved into the tensor
     rng = np.random.default_rng(3)
     x = torch.from_numpy(rng.uniform(-1, 1, (8, 37)).astype(F)).cuda()
     d = torch.from_numpy(rng.normal(0, 0.3, (8, 23)).astype(F)).cuda()
     tile.set_learning_rate(0.1)
     tile.update(x, d, False)
-    assert not torch.equal(shared.cpu(), w)               # the update wrote into the tensor
-    assert torch.equal(shared.cpu(), tile.get_weights())
+    assert not torch.equal(shared.t().cpu(), w)           # the update wrote into the tensor
+    assert torch.equal(shared.t().cpu(), tile.get_weights())
     shared.mul_(0.5)                                       # and the tile computes with what the tensor holds
     y = tile.forward(x, False, False, False, True)
-    assert torch.allclose(y, x @ shared.t(), atol=0.06)   # DAC / ADC steps of the analog forward
-    assert (y - 2.0 * (x @ shared.t())).abs().max() > 0.3
+    assert torch.allclose(y, x @ shared, atol=0.06)       # DAC / ADC steps of the analog forward
+    assert (y - 2.0 * (x @ shared)).abs().max() > 0.3
+    assert torch.equal(tile.get_weights(), shared.t().cpu())
+    tile.decay_weights(1.0)                                # maintenance reads and writes the tensor as well
+    assert torch.equal(tile.get_weights(), shared.t().cpu())
+    with pytest.raises(RuntimeError, match=r"expected \[37,23\] array"):
+        tile.set_shared_weights(torch.zeros(23, 37, device="cuda"))
     with pytest.raises(RuntimeError):
-        tile.set_shared_weights(torch.zeros(37, 23, device="cuda"))
+        tile.set_shared_weights(torch.zeros(37, 23))
+
+
+@pytest.mark.parametrize("x_size,d_size", [(96, 64), (64, 64)])
+def test_shared_weights_binding_sequence_of_the_reference(gpu_device, x_size, d_size):
+    """The calls the reference's Python makes when it binds shared weights to a CUDA tile and reads them back
+    (src/aihwkit/simulator/tiles/base.py:386-446): get_weights -> zeros(x_size, d_size) on the GPU ->
+    set_shared_weights -> copy w.t() into it -> weights are read as shared.t().  A square tile must not come out
+    transposed, a non-square one must not be refused; after an update the view equals get_weights()."""
+    rng = np.random.default_rng(8)
+    meta = make_meta(desired_bl=31)
+    host = meta.create_array(x_size, d_size, soft_bounds(construction_seed=3, enforce_consistency=True, dw_min_std=0.0))
+    w = rng.uniform(-0.3, 0.3, (d_size, x_size)).astype(F)
+    host.set_weights(torch.from_numpy(w))
+    tile = tiles.CudaAnalogTile(host)
+    assert "Cuda" in type(tile).__name__
+    w_cpu = tile.get_weights()                                          # (d_size, x_size) on CPU
+    shared = torch.zeros(tile.get_x_size(), tile.get_d_size(), dtype=torch.float32, device="cuda")
+    tile.set_shared_weights(shared)
+    shared.copy_(w_cpu.t().to("cuda"))
+    view = shared.t()                                                   # what _get_tile_weights_ref returns
+    assert torch.equal(view.cpu(), w_cpu)
+    x = torch.from_numpy(rng.uniform(-1, 1, (16, x_size)).astype(F)).cuda()
+    d = torch.from_numpy(rng.normal(0, 0.2, (16, d_size)).astype(F)).cuda()
+    twin = tiles.CudaAnalogTile(host)
+    for t in (tile, twin):
+        t.set_learning_rate(0.05)
+        t.set_seed(4)
+    y, y_twin = tile.forward(x, False, False, False, False), twin.forward(x, False, False, False, False)
+    assert torch.equal(y, y_twin)                                       # not transposed, also when square
+    tile.update(x, d, False)
+    twin.update(x, d, False)
+    assert torch.equal(view.cpu(), tile.get_weights()) and torch.equal(tile.get_weights(), twin.get_weights())
+    assert (tile.get_weights() - w_cpu).abs().max() > 1e-3
+    view.mul_(0.5)                                                      # a write through the context's reference
+    assert torch.equal(tile.get_weights(), 0.5 * twin.get_weights())
+    tile.set_weights(w_cpu)                                             # and set_weights shows in the tensor
+    assert torch.equal(view.cpu(), w_cpu)
+
+
+def test_shared_weights_row_major(gpu_device):
+    """The library's own zero-copy form: a [d_size, x_size] tensor becomes the weight matrix itself."""
+    tile = pulsed_tile()
+    w = tile.get_weights()
+    shared = torch.zeros(23, 37, device="cuda")
+    tile.set_shared_weights_row_major(shared)
+    assert tile.get_shared_weights_if() and torch.equal(shared.cpu(), w)
+    rng = np.random.default_rng(3)
+    x = torch.from_numpy(rng.uniform(-1, 1, (8, 37)).astype(F)).cuda()
+    d = torch.from_numpy(rng.normal(0, 0.3, (8, 23)).astype(F)).cuda()
+    tile.set_learning_rate(0.1)
+    tile.update(x, d, False)
+    assert not torch.equal(shared.cpu(), w) and torch.equal(shared.cpu(), tile.get_weights())
+    shared.mul_(0.5)
+    assert torch.allclose(tile.forward(x, False, False, False, True), x @ shared.t(), atol=0.06)
     with pytest.raises(RuntimeError):
-        tile.set_shared_weights(torch.zeros(23, 37))
+        tile.set_shared_weights_row_major(torch.zeros(37, 23, device="cuda"))
 
 
 def test_delta_weights(gpu_device):
+    """[x_size, d_size] as on the reference's CUDA tiles (rpu_base_tiles_cuda.cpp:110-130)."""
     rng = np.random.default_rng(4)
     x = torch.from_numpy(rng.uniform(-1, 1, (16, 37)).astype(F)).cuda()
     d = torch.from_numpy(rng.normal(0, 0.3, (16, 23)).astype(F)).cuda()
@@ -187,11 +248,11 @@ def test_delta_weights(gpu_device):
     fp = fp_tile()
     fp.set_learning_rate(0.1)
     w0 = fp.get_weights()
-    delta = torch.full((23, 37), 7.0, device="cuda")
+    delta = torch.full((37, 23), 7.0, device="cuda")
     fp.set_delta_weights(delta)
     fp.update(x, d, False)
     assert torch.equal(fp.get_weights(), w0)
-    assert torch.allclose(delta, d.t() @ x, atol=1e-4)
+    assert torch.allclose(delta.t(), d.t() @ x, atol=1e-4)
     fp.reset_delta_weights()
     fp.update(x, d, False)
     assert torch.allclose(fp.get_weights(), w0 - 0.1 * (d.t() @ x).cpu(), atol=1e-5)
@@ -201,13 +262,15 @@ def test_delta_weights(gpu_device):
         t.set_learning_rate(0.05)
         t.set_seed(9)
     w0 = tile.get_weights()
-    delta = torch.zeros(23, 37, device="cuda")
+    delta = torch.zeros(37, 23, device="cuda")
     tile.set_delta_weights(delta)
     tile.update(x, d, False)
     twin.update(x, d, False)
     assert torch.equal(tile.get_weights(), w0)
     assert (twin.get_weights() - w0).abs().max() > 1e-3
-    assert torch.allclose(w0 - 0.05 * delta.cpu(), twin.get_weights(), atol=1e-6)
+    assert torch.allclose(w0 - 0.05 * delta.t().cpu(), twin.get_weights(), atol=1e-6)
+    with pytest.raises(RuntimeError, match=r"expected \[37,23\] array"):
+        tile.set_delta_weights(torch.zeros(23, 37, device="cuda"))
 
 
 def test_extra_state_replays_the_random_streams(gpu_device):
