@@ -25,17 +25,6 @@ namespace rpu_amd {
 
 namespace {
 
-__device__ __forceinline__ float block_max(float v, float *sh) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off));
-  if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = v;
-  __syncthreads();
-  float r = sh[0];
-  for (int i = 1; i < (int)(blockDim.x >> 6); ++i) r = fmaxf(r, sh[i]);
-  __syncthreads();
-  return r;
-}
-
 // rpu_pulsed_meta_parameter.cpp:152-181
 __device__ __forceinline__ void calc_bl_ab(const UpdateDev &up, int &BL, float &A, float &B, float lr, float dw_min) {
   if (lr == 0.0f) {
@@ -61,20 +50,40 @@ __device__ __forceinline__ void calc_bl_ab(const UpdateDev &up, int &BL, float &
   }
 }
 
+// largest absolute value of a line of n elements (element j at v[j * stride]) over the lanes of a wave; rows that are
+// contiguous and 16-byte aligned are read four elements at a time
+__device__ __forceinline__ float wave_abs_max(const float *v, int n, long stride) {
+  const int lane = threadIdx.x & 63;
+  float m = 0.0f;
+  if (stride == 1 && ((((uintptr_t)v) & 15) == 0)) {
+    const int n4 = n >> 2;
+    const float4 *v4 = reinterpret_cast<const float4 *>(v);
+    for (int q = lane; q < n4; q += 64) {
+      const float4 t = v4[q];
+      m = fmaxf(fmaxf(m, fmaxf(fabsf(t.x), fabsf(t.y))), fmaxf(fabsf(t.z), fabsf(t.w)));
+    }
+    for (int j = 4 * n4 + lane; j < n; j += 64) m = fmaxf(m, fabsf(v[j]));
+  } else {
+    for (int j = lane; j < n; j += 64) m = fmaxf(m, fabsf(v[(long)j * stride]));
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off));
+  return m;
+}
+
+// one wave per sample: no barrier between the two line maxima and the sample's BL, A, B
 __global__ __launch_bounds__(256) void k_update_prepare(UpdateArgs a) {
-  __shared__ float sh[8];
-  const int b = blockIdx.x;
+  const int b = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (b >= a.m_batch) return;
+  const bool leader = (threadIdx.x & 63) == 0;
   const float lr = fabsf(a.lr);
   const float dw_min = a.dev.dw_min;
   int BL;
   float A, B;
   if (a.up.update_management || a.up.update_bl_management) {
-    float xm = 0.0f, dm = 0.0f;
-    for (int j = threadIdx.x; j < a.x_size; j += blockDim.x) xm = fmaxf(xm, fabsf(a.x[(long)b * a.x_sb + (long)j * a.x_sj]));
-    for (int i = threadIdx.x; i < a.d_size; i += blockDim.x) dm = fmaxf(dm, fabsf(a.d[(long)b * a.d_sb + (long)i * a.d_si]));
-    xm = block_max(xm, sh);
-    dm = block_max(dm, sh);
-    if (threadIdx.x != 0) return;
+    const float xm = wave_abs_max(a.x + (long)b * a.x_sb, a.x_size, a.x_sj);
+    const float dm = wave_abs_max(a.d + (long)b * a.d_sb, a.d_size, a.d_si);
+    if (!leader) return;
     // rpu_pulsed_meta_parameter.cpp:183-236
     calc_bl_ab(a.up, BL, A, B, lr, dw_min);
     if (lr > 0.0f) {
@@ -100,7 +109,7 @@ __global__ __launch_bounds__(256) void k_update_prepare(UpdateArgs a) {
       }
     }
   } else {
-    if (threadIdx.x != 0) return;
+    if (!leader) return;
     calc_bl_ab(a.up, BL, A, B, lr, dw_min);
   }
   // one 32-bit word holds the sign and at most 31 pulses; the host refuses calls whose BL could exceed that, so
@@ -145,37 +154,44 @@ __device__ __forceinline__ uint32_t pulse_word(const UpdateArgs &a, bool is_x, i
   return word;
 }
 
-// Pulse words and their sample-transposed bit planes in one pass.  A workgroup owns 64 samples x 4 line elements
-// (x lines first, then d lines), one element per wave with its lanes on the 64 samples, so that a ballot over the
-// wave is a plane word.  Values and packed words pass through LDS to be read and written 16 bytes per sample row.
+// Pulse words and their sample-transposed bit planes in one pass.  A workgroup owns 64 samples x 16 line elements
+// (x lines first, then d lines): the values are read 64 bytes per sample row into LDS, then each wave takes every
+// fourth element with its lanes on the 64 samples, so that a ballot over the wave is a plane word; the packed words
+// go back through LDS and are written 64 bytes per sample row.
+constexpr int LINES_E = 16;
+
 __global__ __launch_bounds__(256) void k_update_lines(UpdateArgs a) {
-  __shared__ float vals[64][5];
-  __shared__ uint32_t wt[64][5];
-  const int tiles_x = (a.x_size + 3) / 4;
+  __shared__ float vals[64][LINES_E + 1];
+  __shared__ uint32_t wt[64][LINES_E + 1];
+  const int tiles_x = (a.x_size + LINES_E - 1) / LINES_E;
   const bool is_x = (int)blockIdx.x < tiles_x;
-  const int e0 = (is_x ? (int)blockIdx.x : (int)blockIdx.x - tiles_x) * 4;
+  const int e0 = (is_x ? (int)blockIdx.x : (int)blockIdx.x - tiles_x) * LINES_E;
   const int size = is_x ? a.x_size : a.d_size;
   const int b0 = blockIdx.y * 64;
   const float *src = is_x ? a.x : a.d;
   const long s_b = is_x ? a.x_sb : a.d_sb, s_e = is_x ? a.x_sj : a.d_si;
-  const int rb = threadIdx.x >> 2, ce = threadIdx.x & 3;
-  {
-    const int b = b0 + rb, e = e0 + ce;
-    vals[rb][ce] = (b < a.m_batch && e < size) ? src[(long)b * s_b + (long)e * s_e] : 0.0f;
+  constexpr int ROWS_PER_PASS = 256 / LINES_E;
+  const int col = threadIdx.x % LINES_E, row0 = threadIdx.x / LINES_E;
+#pragma unroll
+  for (int i = 0; i < 64 / ROWS_PER_PASS; ++i) {
+    const int rb = row0 + ROWS_PER_PASS * i;
+    const int b = b0 + rb, e = e0 + col;
+    vals[rb][col] = (b < a.m_batch && e < size) ? src[(long)b * s_b + (long)e * s_e] : 0.0f;
   }
   __syncthreads();
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int b = b0 + lane;
-  const int e = e0 + wave;
-  if (e < size) {
-    const bool b_ok = b < a.m_batch;
-    const float P = b_ok ? (is_x ? a.prob_b[b] : a.prob_a[b]) : 0.0f;
-    const int K = b_ok ? a.bl[b] : 0;
-    const int kmax = a.kmax[a.kmax_slot];
-    uint32_t *planes = is_x ? a.x_planes : a.d_planes;
-    const int c0 = 2 * blockIdx.y;
-    const uint32_t word = b_ok ? pulse_word(a, is_x, e, b, vals[lane][wave], P, K) : 0u;
-    wt[lane][wave] = word;
+  const bool b_ok = b < a.m_batch;
+  const float P = b_ok ? (is_x ? a.prob_b[b] : a.prob_a[b]) : 0.0f;
+  const int K = b_ok ? a.bl[b] : 0;
+  const int kmax = a.kmax[a.kmax_slot];
+  uint32_t *planes = is_x ? a.x_planes : a.d_planes;
+  const int c0 = 2 * blockIdx.y;
+  for (int el = wave; el < LINES_E; el += 4) {
+    const int e = e0 + el;
+    if (e >= size) break; // wave-uniform
+    const uint32_t word = b_ok ? pulse_word(a, is_x, e, b, vals[lane][el], P, K) : 0u;
+    wt[lane][el] = word;
     for (int k = 0; k < kmax; ++k) {
       const unsigned long long m = __ballot((word >> (k + 1)) & 1u);
       if (lane == 0) {
@@ -191,10 +207,12 @@ __global__ __launch_bounds__(256) void k_update_lines(UpdateArgs a) {
     }
   }
   __syncthreads();
-  {
-    uint32_t *words = is_x ? a.x_words : a.d_words;
-    const int bb = b0 + rb, ee = e0 + ce;
-    if (bb < a.m_batch && ee < size) words[(long)bb * size + ee] = wt[rb][ce];
+  uint32_t *words = is_x ? a.x_words : a.d_words;
+#pragma unroll
+  for (int i = 0; i < 64 / ROWS_PER_PASS; ++i) {
+    const int rb = row0 + ROWS_PER_PASS * i;
+    const int bb = b0 + rb, ee = e0 + col;
+    if (bb < a.m_batch && ee < size) words[(long)bb * size + ee] = wt[rb][col];
   }
 }
 
@@ -1078,11 +1096,11 @@ int grid_for(long total) {
 } // namespace
 
 void launch_update_prepare(const UpdateArgs &a, hipStream_t s) {
-  hipLaunchKernelGGL(k_update_prepare, dim3(a.m_batch), dim3(256), 0, s, a);
+  hipLaunchKernelGGL(k_update_prepare, dim3((a.m_batch + 3) / 4), dim3(256), 0, s, a);
 }
 
 void launch_update_lines(const UpdateArgs &a, hipStream_t s) {
-  const dim3 grid((a.x_size + 3) / 4 + (a.d_size + 3) / 4, (a.m_batch + 63) / 64);
+  const dim3 grid((a.x_size + LINES_E - 1) / LINES_E + (a.d_size + LINES_E - 1) / LINES_E, (a.m_batch + 63) / 64);
   hipLaunchKernelGGL(k_update_lines, grid, dim3(256), 0, s, a);
 }
 

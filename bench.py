@@ -28,13 +28,19 @@ for _p in (ROOT, os.path.join(ROOT, "oracle")):  # oracle/: only the cpu_baselin
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
 FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix
 
-# HBM bytes per launch at configuration 2 from rocprofv3 counter runs of `bench.py --pmc` (FETCH_SIZE and
-# WRITE_SIZE in KiB per dispatch, one run each; the summaries are under profiles/).  A copy of 64 MiB in the
-# same runs reads FETCH_SIZE = 32784 and WRITE_SIZE = 65536, so FETCH_SIZE is scaled by 2.0 and WRITE_SIZE by 1.0.
+# Counter values at configuration 2 from rocprofv3 runs of `bench.py --pmc` (one run per counter group; the summaries,
+# with the commands, are under profiles/).  They are constants of this file, not measured in a benchmark run, and
+# the JSON line says so ("traffic_source", "instructions_source").
+# FETCH_SIZE / WRITE_SIZE are KiB per dispatch; a device copy of 64 MiB in the same runs reads FETCH_SIZE = 32784 and
+# WRITE_SIZE = 65536, so FETCH_SIZE is scaled by 2.0 and WRITE_SIZE by 1.0.
 PMC_TRAFFIC_BYTES = {
-    "k_update_pulsed": (15532 * 2.0 + 4096 * 1.0) * 1024,
+    "k_update_pulsed": (15547 * 2.0 + 4096 * 1.0) * 1024,
     "k_mvm_round": (6851 * 2.0 + 2115 * 1.0) * 1024,  # a round over all 256 samples
 }
+PMC_SOURCE = {"k_update_pulsed": "profiles/k_update_pulsed_config2.txt", "k_mvm_round": "profiles/k_mvm_round_config2.txt"}
+# vector-ALU instructions of one k_update_pulsed launch at configuration 2 (SQ_INSTS_VALU summed over its 4096 waves)
+PMC_VALU_INSTS = {"k_update_pulsed": 21947648}
+VALU_PEAK_GINST = 256 * 4 * 2.4 / 4.0  # wave-instructions per ns: 1024 SIMDs, one wave64 instruction per 4 cycles at 2.4 GHz
 
 
 def batch_sweep() -> int:
@@ -219,6 +225,34 @@ def main() -> int:
     prof_update = kernel_ms(lambda: tile.update(xg, dg, False, False, False, True), n)
     tile.set_profiling(False)
 
+    # coincidences (device pulses) of one update call, from the packed words of the last call: the pulses of sample b
+    # in slot k are (x lines that fired) x (d lines that fired)
+    xw, dw, _ = tile.get_update_words(batch)
+    xb_, db_ = xw.numpy().view(np.uint32) >> 1, dw.numpy().view(np.uint32) >> 1
+    pulses = float(sum((((xb_ >> k) & 1).sum(1, dtype=np.float64) * ((db_ >> k) & 1).sum(1, dtype=np.float64)).sum() for k in range(31)))
+
+    # opt-in variant of the update, by name (never the headline value): groups of 32 samples in closed form
+    variants = None
+    if args.config == 2:
+        tile_v = tiles.CudaAnalogTile(host)
+        tile_v.set_learning_rate(lr)
+        tile_v.set_seed(1234)
+        tile_v.set_update_variant("aggregated", 32)
+        ms_v = time_calls(lambda: tile_v.update(xg, dg, False, False, False, True), n)
+        tile_v.set_profiling(True)
+        prof_v = kernel_ms(lambda: tile_v.update(xg, dg, False, False, False, True), n, tile_v)
+        tile_v.set_profiling(False)
+        kv = prof_v["update_aggregated"][0]
+        ub = bytes_per_device * x_size * d_size + 4.0 * (x_size + d_size) * batch
+        variants = {"aggregated_32": {
+            "what": "NOT the reference's per-pulse arithmetic: coincidences counted per 32 samples and applied in closed "
+                    "form with one moment-matched noise draw (rpu_tile_set_update_variant); passes the unchanged 64-seed "
+                    "test of the weight change at this configuration",
+            "ms_per_call": ms_v, "gdevice_updates_per_s": float(x_size) * d_size * batch / (ms_v * 1e-3) / 1e9,
+            "kernel": "k_update_aggregated", "kernel_ms": kv, "hbm_gbs": ub / (kv * 1e-3) / 1e9,
+            "frac_of_hbm_peak": ub / (kv * 1e-3) / 1e9 / HBM_PEAK_GBS}}
+        del tile_v
+
     # The same tile at other batch sizes (supplementary; the graded figures are at the configuration's batch): the
     # contraction at a token-scale batch, where the matrix pipe and not launch latency sets the time, on a second
     # tile with the initial weights like the forward / backward figures above, and the update at a batch of 8, where
@@ -292,17 +326,33 @@ def main() -> int:
                      "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": update_bytes / (k_update_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
                      "traffic": PMC_TRAFFIC_BYTES["k_update_pulsed"] if args.config == 2 else None,
+                     "traffic_source": ("constant from " + PMC_SOURCE["k_update_pulsed"] + " (rocprofv3 --pmc FETCH_SIZE / "
+                                        "WRITE_SIZE), not measured in this run") if args.config == 2 else None,
                      "algorithmic_bytes": update_bytes, "kernel_ms": k_update_ms},
         "roofline_forward": {"kernel": "k_mvm_round (all rounds of a call)", "bound": "mfma",
                              "achieved": flops_per_call / (k_fwd_ms * 1e-3) / 1e12, "peak": FP32_MFMA_PEAK_TFLOPS,
                              "unit": "TFLOP/s", "frac": flops_per_call / (k_fwd_ms * 1e-3) / 1e12 / FP32_MFMA_PEAK_TFLOPS,
                              "traffic": PMC_TRAFFIC_BYTES["k_mvm_round"] if args.config == 2 else None,
+                             "traffic_source": ("constant from " + PMC_SOURCE["k_mvm_round"] + ", not measured in this run")
+                             if args.config == 2 else None,
                              "algorithmic_flops": flops_per_call, "kernel_ms": k_fwd_ms},
         "roofline_backward": {"kernel": "k_mvm_round", "bound": "mfma",
                               "achieved": flops_per_call / (k_bwd_ms * 1e-3) / 1e12, "peak": FP32_MFMA_PEAK_TFLOPS,
                               "unit": "TFLOP/s", "frac": flops_per_call / (k_bwd_ms * 1e-3) / 1e12 / FP32_MFMA_PEAK_TFLOPS,
                               "kernel_ms": k_bwd_ms},
     }
+    if args.config == 2:
+        # what actually bounds the per-pulse kernel: vector-ALU issue (one wave64 instruction per SIMD and 4 cycles)
+        insts = float(PMC_VALU_INSTS["k_update_pulsed"])
+        out["roofline_valu"] = {
+            "kernel": "k_update_pulsed", "bound": "valu issue", "achieved": insts / (k_update_ms * 1e6), "peak": VALU_PEAK_GINST,
+            "unit": "wave-instructions/ns", "frac": insts / (k_update_ms * 1e6) / VALU_PEAK_GINST,
+            "instructions": insts, "instructions_source": "constant from " + PMC_SOURCE["k_update_pulsed"] +
+            " (rocprofv3 --pmc SQ_INSTS_VALU), not measured in this run",
+            "pulses_per_call": pulses, "pulses_per_cross_point": pulses / (x_size * d_size),
+            "wave_instructions_per_pulse": insts / pulses, "lane_instructions_per_pulse": 64.0 * insts / pulses}
+    if variants is not None:
+        out["update_variants"] = variants
     if other is not None:
         out["same_tile_other_batches"] = other
 
@@ -325,12 +375,38 @@ def main() -> int:
         for _ in range(n_upd):
             orc.update(x, d)
         cpu_upd = (time.perf_counter() - t0) / n_upd
+        # all host cores: the update of one tile is a sequence per cross-point and the oracle (like the reference's CPU
+        # path) runs it on one thread, so the cores are used the way a model uses them: one independent tile per core
+        import threading
+
+        cores = int(os.environ.get("OMP_NUM_THREADS", "0")) or os.cpu_count() or 1
+        cores = max(1, min(cores, os.cpu_count() or 1))
+        many = []
+        for k in range(cores):
+            o = OracleTile(x_size, d_size, meta._config(dev))
+            o.set_weights(w)
+            o.set_learning_rate(lr)
+            o.set_seed(100 + k)
+            many.append(o)
+        threads = [threading.Thread(target=lambda o=o: o.update(x, d)) for o in many]   # ctypes releases the GIL
+        t0 = time.perf_counter()
+        for th in threads:
+            th.start()
+        for th in threads:
+            th.join()
+        cpu_all = time.perf_counter() - t0
         out["cpu_baseline"] = {
             "value": devices_per_call / cpu_upd / 1e9, "unit": "Gdevice-updates/s", "cores": 1, "kind": "port",
-            "sample": f"{n_upd} full update calls, 1 forward and 1 backward call of the same workload on the CPU oracle (1 thread)",
+            "sample": f"{n_upd} full update calls, 1 forward and 1 backward call of the same workload on the CPU oracle "
+                      "(1 thread).  The oracle draws its random numbers faster than the reference's CPU path: it takes about "
+                      "0.23 s per update call where the compiled reference took 1.2 s on the survey machine (BASELINE.md), "
+                      "so this baseline is about five times faster than the reference itself would be",
             "update_ms": cpu_upd * 1e3, "forward_ms": cpu_fwd * 1e3, "forward_gflops": flops_per_call / cpu_fwd / 1e9,
             "backward_ms": cpu_bwd * 1e3, "backward_gflops": flops_per_call / cpu_bwd / 1e9,
             "host_cpus": os.cpu_count(),
+            "all_cores": {"value": cores * devices_per_call / cpu_all / 1e9, "unit": "Gdevice-updates/s", "cores": cores,
+                          "sample": f"one full update call on each of {cores} independent tiles at once, one thread per tile "
+                                    "(a tile's update does not split over threads)", "wall_ms": cpu_all * 1e3},
         }
     print(json.dumps(out))
     return 0
