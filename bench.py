@@ -31,10 +31,10 @@ FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix
 # Counter values at configuration 2 from rocprofv3 runs of `bench.py --pmc` (one run per counter group; the summaries,
 # with the commands, are under profiles/).  They are constants of this file, not measured in a benchmark run, and
 # the JSON line says so ("traffic_source", "instructions_source").
-# FETCH_SIZE / WRITE_SIZE are KiB per dispatch; a device copy of 64 MiB in the same runs reads FETCH_SIZE = 32784 and
+# FETCH_SIZE / WRITE_SIZE are KiB per dispatch; a device copy of 64 MiB in the same runs reads FETCH_SIZE = 32782 and
 # WRITE_SIZE = 65536, so FETCH_SIZE is scaled by 2.0 and WRITE_SIZE by 1.0.
 PMC_TRAFFIC_BYTES = {
-    "k_update_pulsed": (15547 * 2.0 + 4096 * 1.0) * 1024,
+    "k_update_pulsed": (15936 * 2.0 + 4096 * 1.0) * 1024,
     "k_mvm_round": (6851 * 2.0 + 2115 * 1.0) * 1024,  # a round over all 256 samples
 }
 PMC_SOURCE = {"k_update_pulsed": "profiles/k_update_pulsed_config2.txt", "k_mvm_round": "profiles/k_mvm_round_config2.txt"}
@@ -88,7 +88,8 @@ def main() -> int:
                     help="skip the supplementary runs of the same tile at batch 16384 (contraction) and 8 (update)")
     ap.add_argument("--pmc", action="store_true",
                     help="counter-collection mode for rocprofv3 --pmc: one 64 MiB calibration copy, then 3 update, "
-                         "3 forward and 3 backward calls; no timing, no JSON line")
+                         "3 forward, 3 backward calls and 3 update calls of the aggregated variant; no timing, "
+                         "no JSON line")
     ap.add_argument("--batch-sweep", action="store_true",
                     help="instead of the benchmark line: forward and backward call times of the configuration-2 tile "
                          "at batches 32 .. 2000 (HIP events over 200 calls each), one JSON line")
@@ -157,6 +158,14 @@ def main() -> int:
         for _ in range(3):
             tile.backward(dg, False, False, False, False)
         if args.config == 2:
+            tile_v = tiles.CudaAnalogTile(host)
+            tile_v.set_learning_rate(lr)
+            tile_v.set_seed(1234)
+            tile_v.set_update_variant("aggregated", 32)
+            for _ in range(3):
+                tile_v.update(xg, dg, False, False, False, False)
+            del tile_v
+        if args.config == 2 and not args.no_other_batches:
             rng = np.random.default_rng(3)
             xb = torch.from_numpy(rng.uniform(-1, 1, (16384, x_size)).astype(np.float32)).cuda()
             db = torch.from_numpy(rng.normal(0, 0.05, (16384, d_size)).astype(np.float32)).cuda()
@@ -164,8 +173,8 @@ def main() -> int:
                 tile.forward(xb, False, False, False, False, False)
             for _ in range(2):
                 tile.backward(db, False, False, False, False)
-        print("pmc run done: 1 copy of 64 MiB, 3 update, 3 forward, 3 backward calls, then 2 forward and 2 backward "
-              "calls at batch 16384", file=sys.stderr)
+        print("pmc run done: 1 copy of 64 MiB, 3 update, 3 forward, 3 backward calls, 3 update calls of the aggregated "
+              "variant, then (unless --no-other-batches) 2 forward and 2 backward calls at batch 16384", file=sys.stderr)
         return 0
 
     def step():
