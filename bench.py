@@ -45,7 +45,7 @@ VALU_PEAK_GINST = 256 * 4 * 2.4 / 4.0  # wave-instructions per ns: 1024 SIMDs, o
 
 def batch_sweep() -> int:
     """Call time against the batch on the configuration-2 tile: shows where a second workgroup per CU starts to cost
-    its full time (the per-CU operand fetch rate bounds the 32 x 32 round kernel)."""
+    its full time."""
     import numpy as np
     import torch
 
