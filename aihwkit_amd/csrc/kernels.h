@@ -62,6 +62,12 @@ struct MvmArgs {
   // null: none.  Only the 32 x 32 round kernels read it.
   const float *pre_add;
   int pre_is_total;         // 1: pre_add holds the whole analog value before quantization (the kernel's own sums are unused)
+  // PosNegSeparateDigitalSum (rpu_forward_backward_pass.cpp:861-877): post_add[row * O + o] is the finished ADC value
+  // of the negative pass, added after this pass's own quantization and clipping; post_hit_up / post_hit_lo[row] hold
+  // that pass's saturation marks (1 + largest output index that hit the bound), read and cleared when the sample is
+  // advanced.  All null otherwise.
+  const float *post_add;
+  int *post_hit_up, *post_hit_lo;
   int nm_phase;             // running-average noise management: 1 = the init kernel only stores every sample's
                             // largest absolute input in st.nm, 2 = it takes the scales from st.nm; 0 otherwise
   int small_tiles_only;     // 1: never the large-tile kernel (its row padding differs)
@@ -129,6 +135,10 @@ struct SideDev {
   // (add_ni) before the non-linearity
   int ni_only;
   const float *add_ni;
+  // PosNegSeparateDigitalSum: the pass ends with its own ADC here (quantization, clipping, saturation marks per row)
+  int adc_here, adc_sto_round;
+  float adc_res, adc_bound;
+  int *hit_up, *hit_lo; // [rows], null: no bound management
 };
 // addend mode: pre[row][o] = w_noise term * N(0, 1) - IR-drop term; s_cur / s_ir are null without IR drop.
 // total mode: pre[row][o] = asymmetry(nonlinearity(offsets(s_y - IR drop) + w_noise term)) + output noise

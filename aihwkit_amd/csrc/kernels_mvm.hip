@@ -124,7 +124,7 @@ __host__ __device__ __forceinline__ int workgroups_for(int O, int n_act, int edg
 // ADC of the four analog sums v of outputs o0 .. o0 + 3 of sample b: asymmetry, noise, quantization, clipping, output
 // factor; up / lo return 1 + the largest output index that hit the upper / lower bound (0: none)
 __device__ __forceinline__ void mvm_adc_values(const MvmArgs &a, int round, int b, float fin, int o0, float (&v)[4],
-                                               int &up, int &lo, const float *pre = nullptr) {
+                                               int &up, int &lo, const float *pre = nullptr, const float *post = nullptr) {
   float nz[4] = {0.f, 0.f, 0.f, 0.f};
   if (a.io.out_noise > 0.0f) {
     philox_normal4((uint32_t)(o0 >> 2), (uint32_t)b, a.call, RNG_OUT_NOISE | ((uint32_t)round << 8), a.key, nz);
@@ -151,6 +151,7 @@ __device__ __forceinline__ void mvm_adc_values(const MvmArgs &a, int round, int 
     const bool counts = o0 + q < a.O;
     hit_u = (over && counts) ? o0 + q + 1 : hit_u;
     hit_l = (under && counts) ? o0 + q + 1 : hit_l;
+    if (post && counts) y += post[o0 + q]; // the other pass, through its own ADC already
     v[q] = y * fin;
   }
   up = hit_u;
@@ -160,7 +161,8 @@ __device__ __forceinline__ void mvm_adc_values(const MvmArgs &a, int round, int 
 // ADC stage for outputs o0 .. o0 + 3 of sample b: v holds the analog sums (rpu_forward_backward_pass.cpp:666-719)
 // up / lo return 1 + the largest output index that hit the upper / lower ADC bound (0: none).
 __device__ __forceinline__ void mvm_finish_outputs(const MvmArgs &a, int round, int b, float fin, int o0, float (&v)[4],
-                                                   int &up, int &lo, const float *pre = nullptr) {
+                                                   int &up, int &lo, const float *pre = nullptr,
+                                                   const float *post = nullptr) {
   up = 0;
   lo = 0;
   float *out_p = a.out + (long)b * a.out_sb + (long)o0 * a.out_so;
@@ -184,7 +186,7 @@ __device__ __forceinline__ void mvm_finish_outputs(const MvmArgs &a, int round, 
     return;
   }
 
-  mvm_adc_values(a, round, b, fin, o0, v, up, lo, pre);
+  mvm_adc_values(a, round, b, fin, o0, v, up, lo, pre, post);
   if (a.out_so == 1 && (o0 + 3) < a.O && ((((uintptr_t)out_p) & 15) == 0)) {
     *reinterpret_cast<float4 *>(out_p) = make_float4(v[0], v[1], v[2], v[3]);
   } else {
@@ -446,12 +448,13 @@ __device__ __forceinline__ void mvm_round_tile(const MvmArgs &a, int round, int 
   const int o0 = tile_o * TILE + wave * 8 + h * 4;
   int up = 0, lo = 0;
   if (b_ok && o0 < a.O) {
-    const float *pre = nullptr;
+    const float *pre = nullptr, *post = nullptr;
     if (a.pre_add) {
       const int xrow = (round > 0) ? pick2(a.st.row, round & 1)[slot_in] : slot_in;
       pre = a.pre_add + (long)xrow * a.O;
+      if (a.post_add) post = a.post_add + (long)xrow * a.O;
     }
-    mvm_finish_outputs(a, round, b_out, fin_out, o0, v, up, lo, pre);
+    mvm_finish_outputs(a, round, b_out, fin_out, o0, v, up, lo, pre, post);
   }
   if (!a.io.perfect && a.io.bound_management != RPU_BM_NONE) {
     // saturation flags of the tile's 32 samples: combined in LDS, then one device-scope atomic per sample
@@ -772,7 +775,15 @@ __device__ __forceinline__ int mvm_advance_sample(const MvmArgs &a, int round, i
   const int lo = atomicExch(&a.st.hit_lo[b], 0);
   // the CPU loop sets "failed" on an upper hit and *assigns* !bm_test_negative_bound on a lower hit,
   // walking the outputs in index order: the last hit decides
-  const bool failed = io.bm_test_negative_bound ? (up > 0 || lo > 0) : (up > lo);
+  bool failed = io.bm_test_negative_bound ? (up > 0 || lo > 0) : (up > lo);
+  if (a.post_hit_up) {
+    // the negative pass went through the ADC stage on its own: either pass can fail the bound test
+    // (rpu_forward_backward_pass.cpp:861-877); a sample short-cut to zero has no passes
+    const int xrow = (round > 0) ? pick2(a.st.row, round & 1)[slot] : slot;
+    const int nu = atomicExch(&a.post_hit_up[xrow], 0);
+    const int nl = atomicExch(&a.post_hit_lo[xrow], 0);
+    if (a.st.fin[b] != 0.0f) failed = failed || (io.bm_test_negative_bound ? (nu > 0 || nl > 0) : (nu > nl));
+  }
   if (!failed) return -1;
   float nm = a.st.nm[b], red = a.st.red[b];
   if (!next_round_params(a, round, b, a.st.fin[b], nm, red)) return -1;

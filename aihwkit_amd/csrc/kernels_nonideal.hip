@@ -62,6 +62,7 @@ __global__ __launch_bounds__(256) void k_side_combine(float *pre, const float *s
     const int row = (int)(i / quads);
     const int o0 = (int)(i % quads) * 4;
     float z[4] = {0.f, 0.f, 0.f, 0.f}, zo[4] = {0.f, 0.f, 0.f, 0.f};
+    int hit_u = 0, hit_l = 0;
     const bool noisy = p.w_noise_type != 0 && p.w_noise > 0.0f;
     if (noisy) philox_normal4((uint32_t)(o0 >> 2), (uint32_t)row, call, RNG_W_NOISE | ((uint32_t)round << 8), key, z);
     const bool total = p.s_y != nullptr;
@@ -106,7 +107,26 @@ __global__ __launch_bounds__(256) void k_side_combine(float *pre, const float *s
         if (p.out_asym > 0.0f) v = v < 0.0f ? v * (1.0f - p.out_asym) : v;
         if (out_noisy) v += (p.out_noise ? p.out_noise[o] : p.out_noise_all) * zo[q];
       }
+      if (p.adc_here) {
+        // this pass's own ADC (finalizeOutput, rpu_forward_backward_pass.cpp:666-719)
+        if (p.adc_res > 0.0f) {
+          float qq = v / p.adc_res;
+          if (p.adc_sto_round) {
+            const Philox4 rr = philox4x32_10((uint32_t)o, (uint32_t)row, call, RNG_OUT_SR | ((uint32_t)round << 8), key.k0, key.k1);
+            qq = qq + (u32_to_uniform(rr.v[0]) - 0.5f);
+          }
+          v = rintf(qq) * p.adc_res;
+        }
+        const bool over = v > p.adc_bound, under = v < -p.adc_bound;
+        v = over ? p.adc_bound : (under ? -p.adc_bound : v);
+        if (over) hit_u = o + 1;
+        if (under) hit_l = o + 1;
+      }
       pre[k] = v;
+    }
+    if (p.hit_up) {
+      if (hit_u) atomicMax(&p.hit_up[row], hit_u);
+      if (hit_l) atomicMax(&p.hit_lo[row], hit_l);
     }
   }
 }

@@ -49,8 +49,10 @@ void IOPar::initialize(bool backward) {
     return;
   }
   perfect = false;
-  if (p.mv_type != RPU_MV_ONE_PASS && p.mv_type != RPU_MV_POS_NEG_SEPARATE) {
-    throw RpuError("AnalogMVType not implemented on this path (only Ideal, OnePass and PosNegSeparate).");
+  if (p.mv_type != RPU_MV_ONE_PASS && p.mv_type != RPU_MV_POS_NEG_SEPARATE &&
+      p.mv_type != RPU_MV_POS_NEG_SEPARATE_DIGITAL_SUM) {
+    throw RpuError("AnalogMVType not implemented on this path (only Ideal, OnePass, PosNegSeparate and "
+                   "PosNegSeparateDigitalSum).");
   }
   if (p.w_noise_type < 0 || p.w_noise_type > 2) {
     throw RpuError("Output noise type not implemented");

@@ -27,7 +27,10 @@ struct IOPar {
   float nl_factor = 1.0f;
   bool has_voltage_offsets() const { return !perfect && (p.v_offset_std > 0.0f || p.r_series > 0.0f); }
   bool has_nl_calibration() const { return !perfect && (p.out_nonlinearity > 0.0f || p.r_series > 0.0f); }
-  bool separate_passes() const { return !perfect && p.mv_type == RPU_MV_POS_NEG_SEPARATE; }
+  bool separate_passes() const {
+    return !perfect && (p.mv_type == RPU_MV_POS_NEG_SEPARATE || p.mv_type == RPU_MV_POS_NEG_SEPARATE_DIGITAL_SUM);
+  }
+  bool digital_sum() const { return !perfect && p.mv_type == RPU_MV_POS_NEG_SEPARATE_DIGITAL_SUM; }
   // whether the analog value has to be built outside the contraction kernel
   bool has_line_terms() const {
     return has_voltage_offsets() || has_nl_calibration() || (!perfect && p.out_noise_std > 0.0f) || separate_passes();

@@ -227,6 +227,7 @@ struct Tile {
   // analog non-idealities before the ADC: the addend per output, up to three side contractions, the transformed
   // input rows, |W| and the squared row norms
   DevBuf<float> n_pre, n_s1, n_s2, n_s3, n_s4, n_rows, n_absw, n_sumsq, n_xsum, n_part, n_neg;
+  DevBuf<int> n_neghit; // [2][B] saturation marks of the negative pass (PosNegSeparateDigitalSum)
   // per direction: voltage offsets, non-linearity coefficients, output noise levels, read-asymmetry factors
   DevBuf<float> d_line[2][4];
   bool line_valid[2][4] = {{false, false, false, false}, {false, false, false, false}};
@@ -322,6 +323,7 @@ struct Tile {
     n_xsum.release();
     n_part.release();
     n_neg.release();
+    n_neghit.release();
     n_wneg.release();
     n_absneg.release();
     for (auto &dir : d_line) for (auto &b : dir) b.release();
@@ -604,10 +606,30 @@ struct Tile {
         a.io.out_asym = 0.0f;
       }
       float *dst = n_pre.p;
+      const bool digital = io.digital_sum();
       if (separate && pass == 0) {
         n_neg.ensure(out_n);
         dst = n_neg.p;
-        p.ni_only = 1;
+        if (digital) {
+          // the pass goes through the ADC stage on its own (rpu_forward_backward_pass.cpp:861-863)
+          p.adc_here = 1;
+          p.adc_res = a.io.out_res; p.adc_bound = a.io.out_bound; p.adc_sto_round = a.io.out_sto_round;
+          if (io.p.bound_management != RPU_BM_NONE) {
+            n_neghit.ensure(2 * (size_t)B);
+            // every round: the pass also converts rows that no sample of this round uses, whose marks nobody clears
+            launch_fill(reinterpret_cast<float *>(n_neghit.p), 0.0f, 2 * (size_t)B, s); // all-zero bits
+            p.hit_up = n_neghit.p;
+            p.hit_lo = n_neghit.p + B;
+          }
+        } else {
+          p.ni_only = 1;
+        }
+      } else if (separate && digital) {
+        a.post_add = n_neg.p;
+        if (io.p.bound_management != RPU_BM_NONE) {
+          a.post_hit_up = n_neghit.p;
+          a.post_hit_lo = n_neghit.p + B;
+        }
       } else if (separate) {
         p.add_ni = n_neg.p;
       }

@@ -71,9 +71,11 @@ enum rpu_pulse_type {
 enum rpu_mv_type {
   RPU_MV_IDEAL = 0,
   RPU_MV_ONE_PASS = 1,
-  RPU_MV_POS_NEG_SEPARATE = 2 /* negative and positive inputs in two passes, summed before the ADC
-                                 (R/rpu_forward_backward_pass.cpp:832-893) */
-  /* PosNegSeparateDigitalSum(3), SplitMode(4), BitWise(5): not provided */
+  RPU_MV_POS_NEG_SEPARATE = 2, /* negative and positive inputs in two passes, summed before the ADC
+                                  (R/rpu_forward_backward_pass.cpp:832-893) */
+  RPU_MV_POS_NEG_SEPARATE_DIGITAL_SUM = 3 /* the two passes each through the ADC stage, the results added
+                                             (R/rpu_forward_backward_pass.cpp:861-877) */
+  /* SplitMode(4), BitWise(5): not provided */
 };
 
 /* device kinds; B/rpu_base_devices.cpp:545-656 */

@@ -150,8 +150,9 @@ bool init_io(OrcIO &io, bool backward) {
     io.perfect = true;
     return true;
   }
-  if (p.mv_type != RPU_MV_ONE_PASS && p.mv_type != RPU_MV_POS_NEG_SEPARATE) {
-    g_err = "oracle: only mv_type Ideal / OnePass / PosNegSeparate restated";
+  if (p.mv_type != RPU_MV_ONE_PASS && p.mv_type != RPU_MV_POS_NEG_SEPARATE &&
+      p.mv_type != RPU_MV_POS_NEG_SEPARATE_DIGITAL_SUM) {
+    g_err = "oracle: only mv_type Ideal / OnePass / PosNegSeparate / PosNegSeparateDigitalSum restated";
     return false;
   }
   p.out_res = check_res(p.out_res) * (2.0f * p.out_bound);
@@ -651,14 +652,17 @@ void analog_mv_single_pass(OrcTile &t, const float *in, int in_size, float *out,
   apply_output_weight_noise(t, out, out_size, out_inc, in, in_size, io, transposed);
 }
 
-// R/rpu_forward_backward_pass.cpp:800-897 computeAnalogMV: OnePass and PosNegSeparate
+// R/rpu_forward_backward_pass.cpp:800-897 computeAnalogMV: OnePass, PosNegSeparate and PosNegSeparateDigitalSum
 bool analog_mv(OrcTile &t, const float *in, int in_size, int in_inc, float *out, int out_size,
                int out_inc, float scale, bool scaling, const rpu_io_params &io, bool transposed) {
   t.in_buf.resize(in_size);
   prepare_input(t, t.in_buf.data(), in, in_size, in_inc, scale, scaling, io);
   const OrcTile::Lines &mv = t.lines[transposed ? 1 : 0];
-  if (io.mv_type == RPU_MV_POS_NEG_SEPARATE) {
-    // first the negative inputs, then the positive ones; the sums of both passes go through the ADC (:832-893)
+  if (io.mv_type == RPU_MV_POS_NEG_SEPARATE || io.mv_type == RPU_MV_POS_NEG_SEPARATE_DIGITAL_SUM) {
+    // first the negative inputs, then the positive ones; the sums of both passes go through the ADC (:832-893),
+    // or, with the digital sum, each pass through the ADC stage on its own (:861-877) and the codes are added
+    const bool digital = io.mv_type == RPU_MV_POS_NEG_SEPARATE_DIGITAL_SUM;
+    bool passed = false;
     std::vector<float> part((size_t)in_size), neg_out((size_t)out_size);
     for (int i = 0; i < in_size; ++i) part[i] = t.in_buf[i] < 0.0f ? t.in_buf[i] : 0.0f;
     if (io.w_read_asymmetry_dtod > 0.0f) {
@@ -671,9 +675,12 @@ bool analog_mv(OrcTile &t, const float *in, int in_size, int in_inc, float *out,
     } else {
       analog_mv_single_pass(t, part.data(), in_size, neg_out.data(), out_size, 1, io, transposed);
     }
+    if (digital) passed = finalize_output(t, neg_out.data(), out_size, 1, io, mv);
     for (int i = 0; i < in_size; ++i) part[i] = t.in_buf[i] > 0.0f ? t.in_buf[i] : 0.0f;
     analog_mv_single_pass(t, part.data(), in_size, out, out_size, out_inc, io, transposed);
+    if (digital) passed = finalize_output(t, out, out_size, out_inc, io, mv) && passed;
     for (int j = 0; j < out_size; ++j) out[(size_t)j * out_inc] += neg_out[j];
+    if (digital) return passed;
     return finalize_output(t, out, out_size, out_inc, io, mv);
   }
   analog_mv_single_pass(t, t.in_buf.data(), in_size, out, out_size, out_inc, io, transposed);

@@ -110,7 +110,7 @@ def test_unsupported_parameters_fail_loudly():
     with pytest.raises(RuntimeError, match="expects bound==1"):
         make_meta(io_params(inp_bound=2.0)).create_array(4, 4, dev)
     with pytest.raises(RuntimeError, match="not implemented"):
-        make_meta(io_params(mv_type=dv.AnalogMVType.PosNegSeparateDigitalSum)).create_array(4, 4, dev)
+        make_meta(io_params(mv_type=4)).create_array(4, 4, dev)                   # SplitMode
     # per-line periphery values are drawn at creation and are part of the extra state of a host tile too
     host = make_meta(io_params(out_noise_std=0.1, v_offset_std=0.1, r_series=0.01, out_nonlinearity=0.3)).create_array(4, 6, dev)
     names = [k for k in host.dump_extra() if k.startswith("rpu.fwd.")]

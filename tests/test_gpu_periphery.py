@@ -44,8 +44,13 @@ def pair(x_size, d_size, seed=0, construction_seed=7, **io):
 
 
 PNS = dv.AnalogMVType.PosNegSeparate
+PNSD = dv.AnalogMVType.PosNegSeparateDigitalSum
 
 CASES = {
+    "digital_sum_ir_drop": dict(mv_type=PNSD, ir_drop=1.0),
+    "digital_sum_series_resistance": dict(mv_type=PNSD, r_series=0.03, v_offset_std=0.1, v_offset_w_min=-1.0),
+    "digital_sum_everything": dict(mv_type=PNSD, v_offset_std=0.1, r_series=0.01, out_nonlinearity=0.5,
+                                   out_nonlinearity_std=0.2, ir_drop=1.0, out_asymmetry=0.05),
     "separate_passes_ir_drop": dict(mv_type=PNS, ir_drop=1.0),
     "separate_passes_series_resistance": dict(mv_type=PNS, r_series=0.03, v_offset_std=0.1, v_offset_w_min=-1.0),
     "separate_passes_everything": dict(mv_type=PNS, v_offset_std=0.1, r_series=0.01, out_nonlinearity=0.5,
@@ -86,7 +91,7 @@ def test_line_terms_with_quantized_inputs_and_bound_management(gpu_device, shape
     rounds = orc.bm_rounds(batch)
     # an uncalibrated non-linearity, or a series resistance on the large current of a pass, compresses the sums below
     # the bound; every other case needs a second round for some samples
-    need = 1 if ("uncalibrated" in case or case == "separate_passes_series_resistance") else 2
+    need = 1 if ("uncalibrated" in case or case.endswith("passes_series_resistance")) else 2
     assert rounds.max() >= need and len(set(rounds[rounds > 0])) >= need
     assert np.array_equal(gpu.get_bm_rounds(batch).numpy(), rounds)
     scale = np.abs(want).max()
@@ -192,6 +197,54 @@ def test_separate_passes_without_nonlinear_terms_and_their_noise(gpu_device):
     assert moments_ok((y - x64 @ w64.T) / 0.2)
 
 
+def test_digital_sum_of_separately_converted_passes(gpu_device):
+    """PosNegSeparateDigitalSum: each pass goes through the ADC stage on its own (noise, quantization, clipping, bound
+    test) and the converted values are added.  (1) With a wide ADC and no quantization it is the analog sum, i.e. the
+    one-pass tile.  (2) With the real ADC step every output is the sum of two codes: a multiple of the step, within the
+    flips of a rounding edge of the oracle's; the bound test is per pass (the round counts equal the oracle's; with
+    random signs a pass carries half the inputs, so samples whose analog sum saturates get by with fewer rounds).
+    (3) Output noise is drawn per pass: its variance is twice the one-pass variance."""
+    rng = np.random.default_rng(8)
+    x_size, d_size, batch = 96, 160, 64
+    x = rng.uniform(-1, 1, (batch, x_size)).astype(F)
+    d = rng.uniform(-1, 1, (batch, d_size)).astype(F)
+    io = dict(out_bound=1e6, noise_management=dv.NoiseManagementType.AbsMax, bound_management=dv.BoundManagementType.Iterative)
+    orc, gpu, w = pair(x_size, d_size, mv_type=PNSD, **io)
+    _o, one, _w = pair(x_size, d_size, **io)
+    got = gpu.forward(torch.from_numpy(x).cuda()).cpu().numpy()
+    assert np.abs(got - orc.forward(x)).max() <= 1e-5 * np.abs(got).max()
+    assert np.abs(got - one.forward(torch.from_numpy(x).cuda()).cpu().numpy()).max() <= 1e-5 * np.abs(got).max()
+    # (2)
+    step = 2 * 2.0 / 510
+    io = dict(out_bound=2.0, out_res=1.0 / 510, noise_management=dv.NoiseManagementType.AbsMax,
+              bound_management=dv.BoundManagementType.Iterative)
+    orc, gpu, w = pair(x_size, d_size, mv_type=PNSD, **io)
+    _o, analog, _w = pair(x_size, d_size, mv_type=PNS, **io)
+    want = orc.forward(x)
+    got = gpu.forward(torch.from_numpy(x).cuda()).cpu().numpy()
+    rounds = gpu.get_bm_rounds(batch).numpy()
+    assert np.array_equal(rounds, orc.bm_rounds(batch))
+    analog.forward(torch.from_numpy(x).cuda())
+    assert (rounds <= analog.get_bm_rounds(batch).numpy()).all() and rounds.sum() < analog.get_bm_rounds(batch).numpy().sum()
+    scale = np.abs(x).max(axis=1, keepdims=True) * 2.0 ** (rounds[:, None] - 1)   # output factor of the last round
+    codes = got / (step * scale)
+    assert np.abs(codes - np.rint(codes)).max() < 2e-3
+    diff = np.abs(got - want) / (step * scale)
+    off = diff > 1e-3
+    assert off.mean() < 5e-3 and np.allclose(diff[off], 1.0, atol=1e-2)
+    want_b = orc.backward(d)
+    got_b = gpu.backward(torch.from_numpy(d).cuda()).cpu().numpy()
+    diff = np.abs(got_b - want_b) / (step * np.abs(d).max(axis=1, keepdims=True))
+    off = diff > 1e-3
+    assert off.mean() < 5e-3 and np.allclose(diff[off], 1.0, atol=1e-2)
+    # (3)
+    base = dict(inp_res=-1.0, out_bound=1e6, noise_management=dv.NoiseManagementType.NONE,
+                bound_management=dv.BoundManagementType.NONE)
+    _o, gpu, w = pair(x_size, d_size, mv_type=PNSD, out_noise=0.2, **base)
+    y = gpu.forward(torch.from_numpy(x).cuda()).cpu().numpy().astype(np.float64)
+    assert moments_ok((y - x.astype(np.float64) @ w.astype(np.float64).T) / (0.2 * np.sqrt(2.0)))
+
+
 def test_read_asymmetry_of_the_negative_pass(gpu_device):
     rng = np.random.default_rng(6)
     for x_size, d_size, batch in ((37, 23, 50), (300, 200, 96)):
@@ -264,4 +317,4 @@ def test_line_terms_are_refused_where_they_are_not_provided(gpu_device):
     with pytest.raises(Exception, match="not provided for the read of a transfer"):
         make_meta().create_array(8, 8, tr)
     with pytest.raises(Exception, match="AnalogMVType not implemented"):
-        pair(8, 8, mv_type=dv.AnalogMVType.PosNegSeparateDigitalSum)
+        pair(8, 8, mv_type=4)                                       # SplitMode

@@ -751,7 +751,7 @@ def one_periphery(seed):
     if rng.integers(3) == 0:
         io.update(ir_drop=float(rng.choice([0.5, 1.0])), ir_drop_g_ratio=lines * (0.3 * 0.5 * lines) / 0.4)
     if rng.integers(2):
-        io["mv_type"] = dv.AnalogMVType.PosNegSeparate
+        io["mv_type"] = dv.AnalogMVType.PosNegSeparate if rng.integers(3) else dv.AnalogMVType.PosNegSeparateDigitalSum
         if rng.integers(2):
             io["w_read_asymmetry_dtod"] = float(rng.choice([0.1, 0.4]))
     if not any(k in io for k in ("v_offset_std", "r_series", "out_nonlinearity", "mv_type")):
@@ -796,7 +796,7 @@ def one_periphery(seed):
 
 def test_random_periphery_cases_follow_the_oracle(gpu_device):
     """Voltage offsets (with and without a reference line), series resistance (capped or not), output non-linearity
-    with its calibration, asymmetries, IR drop and PosNegSeparate (with read asymmetry) in random combinations over shapes, layouts, bias
+    with its calibration, asymmetries, IR drop and PosNegSeparate / PosNegSeparateDigitalSum (with read asymmetry) in random combinations over shapes, layouts, bias
     column, noise and bound management: 5e-5 of the output range (the calibration factor of the non-linearity
     amplifies the rounding of the sums several times before the compression) and identical round counts."""
     failures = [desc for ok, desc in (one_periphery(seed) for seed in range(92000, 92200)) if not ok]

@@ -190,6 +190,46 @@ def test_pos_neg_separate_passes():
     assert abs(t.backward(np.array([[0.8, -0.3]], dtype=F))[0, 0] - (0.8 / 1.4 - 0.3 / 1.15)) < 1e-6
 
 
+def test_pos_neg_separate_digital_sum():
+    """Each pass through its own ADC stage, converted values added (R/rpu_forward_backward_pass.cpp:861-877): hand
+    values where the analog sum and the digital sum differ."""
+    pnsd = dv.AnalogMVType.PosNegSeparateDigitalSum
+    pns = dv.AnalogMVType.PosNegSeparate
+    # clipping per pass: 0.9 -> 0.4, -0.7 -> -0.4, sum 0 (the analog sum 0.2 fits the bound)
+    xs = np.array([[0.9, -0.7]], dtype=F)
+    assert oracle_tile(2, 1, [[1.0, 1.0]], mv_type=pnsd, out_bound=0.4).forward(xs)[0, 0] == 0.0
+    assert abs(oracle_tile(2, 1, [[1.0, 1.0]], mv_type=pns, out_bound=0.4).forward(xs)[0, 0] - 0.2) < 1e-6
+    # quantization per pass with step 0.25 (1 / 32 of the range of 8): 0.9 -> 1.0 and -0.3 -> -0.25 give 0.75; the analog sum 0.6 gives 0.5
+    xs = np.array([[0.9, -0.3]], dtype=F)
+    assert oracle_tile(2, 1, [[1.0, 1.0]], mv_type=pnsd, out_bound=4.0, out_res=1 / 32).forward(xs)[0, 0] == F(0.75)
+    assert oracle_tile(2, 1, [[1.0, 1.0]], mv_type=pns, out_bound=4.0, out_res=1 / 32).forward(xs)[0, 0] == F(0.5)
+    # the non-linearity acts on each pass: 0.9 / (1 + 0.4 * 0.9) - 0.7 / (1 + 0.4 * 0.7)
+    xs = np.array([[0.9, -0.7]], dtype=F)
+    t = oracle_tile(2, 1, [[1.0, 1.0]], mv_type=pnsd, out_bound=1.0, out_nonlinearity=0.4, slope_calibration=0.0)
+    np.testing.assert_allclose(t.forward(xs)[0, 0], 0.9 / 1.36 - 0.7 / 1.28, rtol=1e-6)
+    # bound management: a pass that saturates alone fails the test although the sum fits; with the upper bound only
+    # tested (bm_test_negative_bound off) a negative pass beyond the lower bound does not
+    bm = dict(out_bound=0.4, bound_management=dv.BoundManagementType.Iterative, noise_management=dv.NoiseManagementType.NONE)
+    t = oracle_tile(2, 1, [[1.0, 1.0]], mv_type=pnsd, **bm)
+    np.testing.assert_allclose(t.forward(np.array([[0.7, -0.6]], dtype=F))[0, 0], 0.1, atol=1e-6)   # 0.35 - 0.3 at half range, x 2
+    assert t.bm_rounds(1)[0] == 2
+    t = oracle_tile(2, 1, [[1.0, 1.0]], mv_type=pns, **bm)
+    np.testing.assert_allclose(t.forward(np.array([[0.7, -0.6]], dtype=F))[0, 0], 0.1, atol=1e-6)
+    assert t.bm_rounds(1)[0] == 1
+    t = oracle_tile(2, 1, [[1.0, 1.0]], mv_type=pnsd, **bm)
+    np.testing.assert_allclose(t.forward(np.array([[0.3, -0.7]], dtype=F))[0, 0], 2 * (0.15 - 0.35), atol=1e-6)
+    assert t.bm_rounds(1)[0] == 2                                  # the negative pass failed the lower bound
+    t = oracle_tile(2, 1, [[1.0, 1.0]], mv_type=pnsd, bm_test_negative_bound=False, **bm)
+    np.testing.assert_allclose(t.forward(np.array([[0.3, -0.7]], dtype=F))[0, 0], 0.3 - 0.4, atol=1e-6)   # lower bound not tested
+    assert t.bm_rounds(1)[0] == 1
+    # output noise is drawn for each pass
+    d = 4000
+    t = oracle_tile(3, d, np.zeros((d, 3)), mv_type=pnsd, out_noise=0.1)
+    t.use_gauss_table(False)
+    y = t.forward(np.array([[0.6, -0.8, 0.0]] * 10, dtype=F)).astype(np.float64) / (0.1 * np.sqrt(2.0))
+    assert abs(y.mean()) < 4 / np.sqrt(y.size) and abs(y.std() - 1) < 4 / np.sqrt(2 * y.size)
+
+
 def test_read_asymmetry_of_the_negative_pass():
     pns = dv.AnalogMVType.PosNegSeparate
     # w = [1, 1], factors [2, 3], x = [0.8, -0.3]: only the negative input reads its weight through the factor
