@@ -93,7 +93,7 @@ class TileConfig(C.Structure):
     _fields_ = [("f_io", IOParams), ("b_io", IOParams), ("up", UpdateParams), ("device", DeviceParams)]
 
 
-MAX_VECTOR_DEVICES = 4
+MAX_VECTOR_DEVICES = 16
 
 
 class TransferParams(C.Structure):

@@ -321,8 +321,8 @@ void launch_unit_vectors(float *out, int n_vec, int size, int start, hipStream_t
 
 // out = sum_k gamma[k] * w[k], k < n (VectorRPUDevice::reduceToWeights, rpu_vector_device.cpp:530-536)
 struct ReduceArgs {
-  const float *w[4];
-  float gamma[4];
+  const float *w[RPU_MAX_VECTOR_DEVICES];
+  float gamma[RPU_MAX_VECTOR_DEVICES];
   int n;
 };
 void launch_reduce_weights(float *out, const ReduceArgs &r, size_t size, hipStream_t s);

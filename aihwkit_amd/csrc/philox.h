@@ -73,7 +73,8 @@ enum RngPurpose : uint32_t {
   RNG_DEVICE_DRIFT = 13, // power-law drift of a training tile: nu variation and read noise
   RNG_MODIFIER = 14,     // weight modifier: noise, stochastic rounding, drop connections
   RNG_W_NOISE = 15,      // output-referred weight noise of the analog MVM
-  RNG_WRITE_NOISE = 16   // write noise on the shown weights (round 0: after an update, 1: refresh of all)
+  RNG_WRITE_NOISE = 16,  // write noise on the shown weights (round 0: after an update, 1: refresh of all)
+  RNG_TRANSFER = 17      // transfer compound, drawn on the host: word 0 random selection of the slice, word 1 reset lottery
 };
 
 // uniform in [0, 1) with 24 bits

@@ -352,9 +352,10 @@ void populate_from(const DevicePar &dev, ConstructionRng &rng, int x_size, int d
 void TransferPar::initialize(int x_size, int d_size) {
   const int n_dev = p.n_devices;
   if (n_dev < 2) throw RpuError("Need at least 2 devices");
-  if (n_dev > RPU_MAX_VECTOR_DEVICES) throw RpuError("At most 4 devices in a transfer chain.");
-  if (p.random_selection) throw RpuError("random_selection is not provided.");
-  if (p.with_reset_prob > 0.0f) throw RpuError("with_reset_prob > 0 is not provided.");
+  if (n_dev > RPU_MAX_VECTOR_DEVICES) throw RpuError("At most 16 devices in a transfer chain.");
+  if (p.with_reset_prob > 0.0f && !p.transfer_columns) {
+    throw RpuError("Reset prob is only implemented for column-transfer so far."); // rpu_transfer_device.cpp:198-200
+  }
   devs.clear();
   for (int k = 0; k < n_dev; ++k) {
     DevicePar d;

@@ -116,10 +116,10 @@ struct DeviceSlot {
   DevicePar par;
   DeviceArrays arr;
   std::vector<float> w_host; // weights while the tile is not resident on a GPU
-  DevBuf<float> d_w, d_wmax, d_wmin, d_sup, d_sdown, d_slup, d_sldown;
+  DevBuf<float> d_w, d_wmax, d_wmin, d_sup, d_sdown, d_slup, d_sldown, d_rbias;
   void release() {
     d_w.release(); d_wmax.release(); d_wmin.release(); d_sup.release(); d_sdown.release();
-    d_slup.release(); d_sldown.release();
+    d_slup.release(); d_sldown.release(); d_rbias.release();
   }
   void clip_host() {
     for (size_t i = 0; i < w_host.size(); ++i) {
@@ -129,6 +129,7 @@ struct DeviceSlot {
   }
   void upload(size_t n, bool with_weights) {
     const size_t bytes = n * sizeof(float);
+    d_rbias.release(); // uploaded again when a transfer resets columns of this device
     d_wmax.ensure(n); d_wmin.ensure(n); d_sup.ensure(n); d_sdown.ensure(n);
     RPU_HIP_CHECK(hipMemcpy(d_wmax.p, arr.w_max.data(), bytes, hipMemcpyHostToDevice));
     RPU_HIP_CHECK(hipMemcpy(d_wmin.p, arr.w_min.data(), bytes, hipMemcpyHostToDevice));
@@ -1377,21 +1378,39 @@ struct Tile {
   void do_transfer(int to, int from, float current_lr, hipStream_t s) {
     const TransferPar &tp = *tr;
     const int in_size = tp.in_size, out_size = tp.out_size;
-    const int start = slice_idx[from];
+    const bool cols = tp.p.transfer_columns != 0;
+    // the two host draws of a transfer (the reference's rw_rng_): one Philox call keyed by (device, update counter)
+    const PhiloxKey k = key();
+    const Philox4 draw = philox4x32_10((uint32_t)from, (uint32_t)update_idx, (uint32_t)(update_idx >> 32), RNG_TRANSFER, k.k0, k.k1);
+    int start = slice_idx[from];
+    if (tp.p.random_selection) { // rpu_transfer_device.cpp:486-488
+      start = std::max(std::min((int)floorf(u32_to_uniform(draw.v[0]) * (float)in_size), in_size - 1), 0);
+    }
     const int n_vec = std::min(tp.p.n_reads_per_transfer, in_size);
     slice_idx[from] = (start + n_vec) % in_size;
     const float lr_t = tp.transfer_lr(from, current_lr);
-    if (lr_t == 0.0f || to == from) return;
-    t_unit.ensure((size_t)n_vec * in_size);
-    t_read.ensure((size_t)n_vec * out_size);
-    launch_unit_vectors(t_unit.p, n_vec, in_size, start, s);
-    IOPar io = tp.io;
-    io.p.out_scale = -io.p.out_scale;
-    const bool cols = tp.p.transfer_columns != 0;
-    mvm(t_unit.p, t_read.p, n_vec, false, false, false, !cols, s, slots[from]->d_w.p, &io);
-    DeviceView dv = view_of(*slots[to], slots[to]->par.weight_granularity());
-    if (cols) pulsed_update_on(dv, tp.up, lr_t, t_unit.p, X, 1, t_read.p, D, 1, n_vec, s);
-    else pulsed_update_on(dv, tp.up, lr_t, t_read.p, X, 1, t_unit.p, D, 1, n_vec, s);
+    if (lr_t != 0.0f && to != from) {
+      t_unit.ensure((size_t)n_vec * in_size);
+      t_read.ensure((size_t)n_vec * out_size);
+      launch_unit_vectors(t_unit.p, n_vec, in_size, start, s);
+      IOPar io = tp.io;
+      io.p.out_scale = -io.p.out_scale;
+      mvm(t_unit.p, t_read.p, n_vec, false, false, false, !cols, s, slots[from]->d_w.p, &io);
+      DeviceView dv = view_of(*slots[to], slots[to]->par.weight_granularity());
+      if (cols) pulsed_update_on(dv, tp.up, lr_t, t_unit.p, X, 1, t_read.p, D, 1, n_vec, s);
+      else pulsed_update_on(dv, tp.up, lr_t, t_read.p, X, 1, t_unit.p, D, 1, n_vec, s);
+    }
+    // the columns that were read start again from their reset values with probability with_reset_prob per transfer,
+    // after all of them were read and written (cuda/rpucuda_transfer_device.cu:320-324)
+    if (cols && tp.p.with_reset_prob > 0.0f && u32_to_uniform(draw.v[1]) < tp.p.with_reset_prob) {
+      DeviceSlot &src = *slots[from];
+      if (src.d_rbias.n < size()) {
+        src.d_rbias.ensure(size());
+        RPU_HIP_CHECK(hipMemcpy(src.d_rbias.p, src.arr.reset_bias.data(), size() * sizeof(float), hipMemcpyHostToDevice));
+      }
+      launch_reset_cols(src.d_w.p, src.d_rbias.p, src.d_wmin.p, src.d_wmax.p, src.par.p.reset_std, start, n_vec, 1.0f, X, D,
+                        k, call++, s);
+    }
   }
 
   // TransferRPUDevice::doSparseUpdate / finishUpdateCycle per update vector (rpu_transfer_device.cpp:520-557):

@@ -66,9 +66,10 @@ class _TileBase:
     def get_transfer_state(self):
         """(number of update vectors since the weights were set, next column per device) of a transfer compound."""
         count = C.c_uint64(0)
-        slices = (C.c_int32 * 4)()
+        from .._cabi import MAX_VECTOR_DEVICES
+        slices = (C.c_int32 * MAX_VECTOR_DEVICES)(*([-1] * MAX_VECTOR_DEVICES))
         check(lib().rpu_tile_get_transfer_state(self._h, C.byref(count), slices))
-        return int(count.value), list(slices)
+        return int(count.value), [v for v in slices if v >= 0]
 
     def _clone_handle(self):
         handle = C.c_void_p()

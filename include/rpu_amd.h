@@ -228,20 +228,21 @@ typedef struct rpu_tile_config {
  * sum_k gamma_vec[k] * w_k.  Device 0 is fast_device, all others rest_device (the reference allows only
  * the first to differ, R/rpu_transfer_device.cpp:136-144).  Empty vectors (n_* = 0) are filled as the
  * reference does (R/rpu_transfer_device.cpp:146-196). */
-#define RPU_MAX_VECTOR_DEVICES 4
+#define RPU_MAX_VECTOR_DEVICES 16
 typedef struct rpu_transfer_params {
   int32_t n_devices;            /* 2 */
   uint32_t construction_seed;   /* 0 = time based; one stream samples all devices in order */
   int32_t units_in_mbatch;      /* 0 */
   int32_t n_reads_per_transfer; /* 1 */
   int32_t no_self_transfer;     /* 1 */
-  int32_t random_selection;     /* 0 ; 1 is not provided */
+  int32_t random_selection;     /* 1: a transfer starts at column floor(u in_size), u uniform (R/rpu_transfer_device.cpp:486-488) */
   int32_t scale_transfer_lr;    /* 1 */
   int32_t scale_fast_lr;        /* 1 */
   int32_t transfer_columns;     /* 1 ; 0 = rows (read with the backward pass) */
   float gamma;                  /* 0 */
   float transfer_every;         /* 1 */
-  float with_reset_prob;        /* 0 ; > 0 is not provided */
+  float with_reset_prob;        /* probability per transfer that the columns just read are reset on the source device,
+                                   after the write (C/rpucuda_transfer_device.cu:320-324); columns only */
   float fast_lr;                /* 0 */
   float transfer_lr;            /* 1 */
   int32_t n_gamma_vec;          /* 0 or n_devices */

@@ -11,7 +11,13 @@ TransferRPUDevice::doSparseUpdate / finishUpdateCycle):
 * after every update vector the counter advances and each device j whose period divides it transfers:
   the next n_reads_per_transfer unit vectors are forwarded through device j (scaled by -1) and written onto
   device j + 1 with learning rate transfer_lr (x current lr) (rpu_transfer_device.cpp:428-516,536-557);
-* tile weights = sum_k gamma_k w_k, or the last device alone when gamma = 0 (rpu_transfer_device.cpp:596-602).
+* tile weights = sum_k gamma_k w_k, or the last device alone when gamma = 0 (rpu_transfer_device.cpp:596-602);
+* random_selection: the first column of a transfer is floor(u * in_size) for a uniform u (rpu_transfer_device.cpp:486-488);
+  with_reset_prob: with that probability per transfer the columns just read are reset on the source device, after all
+  of them were read and written -- the order of the reference's GPU code (cuda/rpucuda_transfer_device.cu:320-324;
+  its CPU code draws per vector inside the loop, rpu_transfer_device.cpp:464-470), because the tile under test
+  stands in for that one.  Both uniforms come from callbacks (`select`, `reset_lottery`), so that a test feeds the
+  draws of the tile under test.
 
 This oracle samples nothing itself: tests copy the device arrays from the library through the hidden-parameter
 interface, and the library's draw order for a chain (one generator walked device by device,
@@ -83,6 +89,8 @@ class TransferOracle:
         self.lr = 0.0
         self.update_idx = 0
         self.slice_idx = [0] * n
+        self.select = None         # (update_idx, from) -> uniform in [0, 1) for random_selection
+        self.reset_lottery = None  # (update_idx, from) -> uniform in [0, 1) for with_reset_prob
         self.set_weights(np.zeros((d_size, x_size), np.float32))
 
     @staticmethod
@@ -149,22 +157,33 @@ class TransferOracle:
 
     def _transfer(self, to, frm, m_batch):
         start = self.slice_idx[frm]
+        if self.tp.random_selection:  # rpu_transfer_device.cpp:486-488
+            u = np.float32(self.select(self.update_idx, frm))
+            start = max(min(int(math.floor(float(np.float32(u * np.float32(self.in_size))))), self.in_size - 1), 0)
         self.slice_idx[frm] = (start + self.n_reads) % self.in_size
         lr = self.lr_vec[frm] * self.lr if self.tp.scale_transfer_lr else self.lr_vec[frm]
         lr = float(np.float32(lr))
-        if lr == 0.0 or to == frm:
-            return
-        for v in range(self.n_reads):
-            unit = np.zeros((1, self.in_size), np.float32)
-            unit[0, (start + v) % self.in_size] = 1.0
-            src, dst = self.devices[frm], self.devices[to]
-            dst.set_learning_rate(lr)
-            if self.cols:
-                read = (-src.forward(unit)).astype(np.float32)
-                dst.update(unit, read)
-            else:
-                read = (-src.backward(unit)).astype(np.float32)
-                dst.update(read, unit)
+        src, dst = self.devices[frm], self.devices[to]
+        if lr != 0.0 and to != frm:
+            for v in range(self.n_reads):
+                unit = np.zeros((1, self.in_size), np.float32)
+                unit[0, (start + v) % self.in_size] = 1.0
+                dst.set_learning_rate(lr)
+                if self.cols:
+                    read = (-src.forward(unit)).astype(np.float32)
+                    dst.update(unit, read)
+                else:
+                    read = (-src.backward(unit)).astype(np.float32)
+                    dst.update(read, unit)
+        # cuda/rpucuda_transfer_device.cu:320-324 (every element of the columns: device-wise probability 1)
+        if self.cols and self.tp.with_reset_prob > 0.0 and \
+                np.float32(self.reset_lottery(self.update_idx, frm)) < np.float32(self.tp.with_reset_prob):
+            from state_oracle import reset_cols
+            if float(self.tp.fast_device.reset_std if frm == 0 else self.tp.rest_device.reset_std) > 0.0:
+                raise NotImplementedError("the transfer oracle resets without noise (reset_std = 0)")
+            hidden = src.get_hidden()
+            w = reset_cols(src.get_weights(), hidden[6], hidden[1], hidden[0], 0.0, start, self.n_reads, None)
+            src.set_weights(w)
 
     def update(self, x, d):
         """Row-major batches x [B, X], d [B, D]."""

@@ -9,6 +9,7 @@ import torch
 
 from aihwkit_amd.rpu_base import devices as dv
 from aihwkit_amd.rpu_base import tiles
+from aihwkit_amd import _cabi
 from helpers import (CONFIG3_SHAPES, build_transfer_pair, config3, constant_step, device_weights, io_params,
                      make_meta, noise_free_io, soft_bounds, transfer_param)
 from test_gpu_statistics import compare_moments
@@ -102,7 +103,7 @@ def test_configuration_3_tiles_noise_free(gpu_device, shape):
         gpu.update(cuda(x), cuda(d), False, False, False, False)
         orc.update(x, d)
         check_state(gpu, orc, 2, f"step {step}")
-    assert gpu.get_transfer_state() == (256, [2, 0, 0, 0])
+    assert gpu.get_transfer_state() == (256, [2, 0])
     assert np.abs(orc.device_weights(0)).max() > 1e-3   # the gradient reached the fast device
     if d_size > 10:  # with ten outputs the first two columns of A are still below one ADC step when they are read
         hidden = orc.devices[1].get_hidden()
@@ -124,6 +125,85 @@ def test_three_device_chain_with_layouts_and_bias(gpu_device):
         orc.update(np.concatenate([x, np.ones((batch, 1), np.float32)], 1), d)
         check_state(gpu, orc, 3, f"step {step}")
     assert np.abs(orc.device_weights(2)).max() > 1e-3
+
+
+def transfer_draws(seed, update_idx, frm):
+    """The two uniforms a tile with this seed draws on the host for the transfer of device `frm` after update vector
+    `update_idx`: Philox4x32-10, counter (device, counter low, counter high, 17), key = seed; 24-bit uniforms."""
+    import ctypes as C
+    out = (C.c_uint32 * 4)()
+    _cabi.check(_cabi.lib().rpu_philox4x32_10((C.c_uint32 * 4)(frm, update_idx & 0xFFFFFFFF, update_idx >> 32, 17),
+                                              (C.c_uint32 * 2)(seed & 0xFFFFFFFF, seed >> 32), out))
+    return [np.float32((v >> 8) * (1.0 / 16777216.0)) for v in out]
+
+
+@pytest.mark.parametrize("n_devices,kw", [
+    (2, dict(transfer_every=2.0, n_reads_per_transfer=3, random_selection=True)),
+    (2, dict(transfer_every=2.0, n_reads_per_transfer=3, with_reset_prob=0.5)),
+    (3, dict(transfer_every=1.0, n_reads_per_transfer=5, random_selection=True, with_reset_prob=0.4,
+             transfer_every_vec=[1.0, 3.0, 0.0], gamma_vec=[0.1, 0.3, 1.0])),
+])
+def test_random_selection_and_reset_follow_the_oracle(gpu_device, n_devices, kw):
+    """The tile draws the first column of a transfer and the reset lottery on the host from its seed; the oracle is fed
+    the same draws, so whole trajectories (every device, counters, next columns) are comparable to 1e-5.  The reset
+    values differ per cross-point (reset_dtod) and are not noisy (reset_std = 0)."""
+    rng = np.random.default_rng(12)
+    x_size, d_size, batch, seed = 23, 14, 6, 4242
+    f_io = noise_free_io(noise_management=dv.NoiseManagementType.AbsMax, bound_management=dv.BoundManagementType.Iterative)
+    meta = make_meta(f_io, noise_free_io(noise_management=dv.NoiseManagementType.AbsMax), pulse_type=PT.DeterministicImplicit,
+                     desired_bl=31)
+    devs = [soft_bounds(dw_min=0.002, dw_min_std=0.0, enforce_consistency=True, reset=0.02, reset_dtod=0.1, reset_std=0.0)
+            for _ in range(n_devices)]
+    tr = transfer_param(devs, construction_seed=31, **kw)
+    tr.transfer_forward = noise_free_io()
+    tr.transfer_update.pulse_type = PT.DeterministicImplicit
+    tr.transfer_update.desired_bl = 31
+    host, orc, gpu = build_transfer_pair(meta, tr, x_size, d_size)
+    gpu.set_seed(seed)
+    starts, lottery = [], []
+    orc.select = lambda idx, frm: starts.append(transfer_draws(seed, idx, frm)[0]) or starts[-1]
+    orc.reset_lottery = lambda idx, frm: lottery.append(transfer_draws(seed, idx, frm)[1]) or lottery[-1]
+    w = rng.uniform(-0.4, 0.4, (d_size, x_size)).astype(np.float32)
+    gpu.set_weights(torch.from_numpy(w))
+    orc.set_weights(w)
+    gpu.set_learning_rate(0.05)
+    orc.set_learning_rate(0.05)
+    for step in range(6):
+        x = rng.uniform(-1, 1, (batch, x_size)).astype(np.float32)
+        d = (0.5 * rng.standard_normal((batch, d_size))).astype(np.float32)
+        gpu.update(cuda(x), cuda(d), False, False, False, False)
+        orc.update(x, d)
+        check_state(gpu, orc, n_devices, f"step {step}")
+    if kw.get("random_selection"):
+        assert len(set(int(u * x_size) for u in starts)) > 4          # the transfers started all over the tile
+    if kw.get("with_reset_prob"):
+        wins = sum(u < kw["with_reset_prob"] for u in lottery)
+        assert 0 < wins < len(lottery)                                 # some transfers reset their columns, some did not
+    assert np.abs(orc.device_weights(n_devices - 1)).max() > 1e-3
+
+
+def test_chain_of_six_devices(gpu_device):
+    rng = np.random.default_rng(13)
+    x_size, d_size, batch, n = 10, 7, 5, 6
+    meta, tr = deterministic_setup("constant", n_devices=n, transfer_every=1.0, n_reads_per_transfer=4,
+                                   transfer_every_vec=[1.0, 2.0, 3.0, 4.0, 6.0, 0.0], gamma_vec=[0.0, 0.05, 0.1, 0.2, 0.4, 1.0],
+                                   transfer_lr=2.0)
+    host, orc, gpu = build_transfer_pair(meta, tr, x_size, d_size)
+    gpu.set_learning_rate(0.2)
+    orc.set_learning_rate(0.2)
+    for step in range(8):
+        x = rng.uniform(-1, 1, (batch, x_size)).astype(np.float32)
+        d = (0.5 * rng.standard_normal((batch, d_size))).astype(np.float32)
+        gpu.update(cuda(x), cuda(d), False, False, False, False)
+        orc.update(x, d)
+        check_state(gpu, orc, n, f"step {step}")
+    count, slices = gpu.get_transfer_state()
+    assert count == 40 and len(slices) == n
+    assert all(np.abs(orc.device_weights(k)).max() > 1e-4 for k in range(n))   # the gradient travelled down the whole chain
+    twin = copy.deepcopy(gpu)
+    assert twin.get_transfer_state() == (count, slices)
+    for k in range(n):
+        assert np.array_equal(device_weights(twin, k), device_weights(gpu, k))
 
 
 def test_state_surface_of_a_gpu_transfer_tile(gpu_device):

@@ -13,7 +13,7 @@ PT = dv.PulseType
 
 def quiet_device(**kw):
     base = dict(dw_min=0.01, dw_min_dtod=0.0, dw_min_std=0.0, up_down_dtod=0.0, w_max_dtod=0.0, w_min_dtod=0.0,
-                w_max=1.0, w_min=-1.0, construction_seed=1)
+                w_max=1.0, w_min=-1.0, reset_std=0.0, construction_seed=1)
     base.update(kw)
     return constant_step(**base)
 
@@ -116,3 +116,40 @@ def test_fast_learning_rate_options():
         orc.update(np.array([[1.0, 0, 0, 0]], np.float32), np.array([[1.0, 0, 0]], np.float32))
         # BL management off: A = B = sqrt(lr / (dw_min BL)), n = rint(BL A B) = lr / dw_min pulses of dw_min
         assert orc.device_weights(0)[0, 0] == pytest.approx(-expected, abs=1e-6)
+
+
+def test_random_selection_and_reset_after_a_transfer():
+    """random_selection: the transfer starts at column floor(u * in_size), clamped, and the running index follows it
+    (R/rpu_transfer_device.cpp:486-488, 515).  with_reset_prob: when the lottery wins, the columns that were read are
+    back at their reset values on the source device AFTER the destination took the values they had
+    (C/rpucuda_transfer_device.cu:320-324); the other columns and a lost lottery change nothing."""
+    a = np.array([[0.3, -0.2, 0.1, 0.0], [0.5, 0.4, -0.3, 0.2], [-0.1, 0.0, 0.2, -0.4]], np.float32)
+    zeros_x, zeros_d = np.zeros((1, 4), np.float32), np.zeros((1, 3), np.float32)
+    for u, start in ((0.0, 0), (0.5, 2), (0.74, 2), (0.75, 3), (0.99999994, 3)):
+        orc = exact_transfer(transfer_every=1.0, scale_transfer_lr=False, random_selection=True, n_reads_per_transfer=2)
+        orc.select = lambda idx, frm, u=u: u
+        orc.set_device_weights(0, a)
+        orc.set_learning_rate(0.1)
+        orc.lr_vec = [0.1, 0.1]
+        orc.update(zeros_x, zeros_d)
+        c = orc.device_weights(1)
+        cols = [start, (start + 1) % 4]
+        rest = [j for j in range(4) if j not in cols]
+        assert np.allclose(c[:, cols], 0.1 * a[:, cols], atol=1e-6) and np.all(c[:, rest] == 0), (u, c)
+        assert orc.slice_idx[0] == (start + 2) % 4
+    for lottery, wins in ((0.2, True), (0.3, False)):
+        orc = exact_transfer(transfer_every=1.0, scale_transfer_lr=False, with_reset_prob=0.3, n_reads_per_transfer=2)
+        asked = []
+        orc.reset_lottery = lambda idx, frm, v=lottery: asked.append((idx, frm)) or v
+        orc.set_device_weights(0, a)
+        orc.set_learning_rate(0.1)
+        orc.lr_vec = [0.1, 0.1]
+        orc.update(zeros_x, zeros_d)
+        assert asked == [(1, 0)]                                    # one draw per transfer, none for the last device
+        assert np.allclose(orc.device_weights(1)[:, :2], 0.1 * a[:, :2], atol=1e-6)   # read before the reset
+        want = a.copy()
+        if wins:
+            want[:, :2] = 0.0                                       # reset bias 0, no reset noise
+        assert np.array_equal(orc.device_weights(0), want)
+    with pytest.raises(RuntimeError, match="column-transfer"):
+        exact_transfer(transfer_every=1.0, with_reset_prob=0.3, transfer_columns=False)
