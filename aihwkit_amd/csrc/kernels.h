@@ -188,6 +188,10 @@ struct UpdateArgs {
   float *prob_b; // [B] probability scale of x
   uint32_t *x_words; // [B][X] packed pulse words
   uint32_t *d_words; // [B][D]
+  // bit lines beyond 31 pulses: a sample takes words_per_sample consecutive rows of words (and bit positions in the
+  // planes); m_batch then counts those rows, bl / prob_a / prob_b / x / d stay per sample (row r belongs to sample
+  // r / words_per_sample and holds its pulse slots 31 (r % words_per_sample) + 1 ..).  0 or 1: one row per sample.
+  int words_per_sample;
   // sample-transposed pulse bits: plane (chunk c, slot k) of line element e is the 32-bit word whose bit q
   // is pulse slot k of sample 32 c + q; element (c, k, e) at planes[(c * plane_slots + k) * size + e];
   // slot plane_slots - 1 holds the sign bits (bit 0 of the packed words)

@@ -112,13 +112,11 @@ __global__ __launch_bounds__(256) void k_update_prepare(UpdateArgs a) {
     if (!leader) return;
     calc_bl_ab(a.up, BL, A, B, lr, dw_min);
   }
-  // one 32-bit word holds the sign and at most 31 pulses; the host refuses calls whose BL could exceed that, so
-  // this never changes a value -- the implicit pulse types keep no words and take any BL
-  if (a.up.pulse_type == RPU_PULSE_STOCHASTIC_COMPRESSED && BL > 31) BL = 31;
   a.bl[b] = BL;
-  // largest BL of the batch: this call's slot was zeroed by the previous call, which used the other one
+  // largest number of pulse slots in a row of words (a longer bit line takes several rows of 31): this call's slot
+  // was zeroed by the previous call, which used the other one
   if (a.kmax) {
-    if (BL > 0) atomicMax(&a.kmax[a.kmax_slot], BL);
+    if (BL > 0) atomicMax(&a.kmax[a.kmax_slot], min(BL, 31));
     if (b == 0) a.kmax[a.kmax_slot ^ 1] = 0;
   }
   a.prob_a[b] = A;
@@ -132,8 +130,10 @@ __device__ __forceinline__ float discretize_prob(float pp, float res, int sto_ro
   return rintf(q) * res;
 }
 
-// packed pulse word of line element j (an x line or a d line) for sample b: bit 0 = sign, bits 1..K = pulses
-__device__ __forceinline__ uint32_t pulse_word(const UpdateArgs &a, bool is_x, int j, int b, float v, float P, int K) {
+// packed pulse word of line element j (an x line or a d line) for sample b: bit 0 = sign, bits 1..K = pulses;
+// `row` numbers the sample's rows of words (pulse slots 31 row + 1 ..), each with its own uniforms
+__device__ __forceinline__ uint32_t pulse_word(const UpdateArgs &a, bool is_x, int j, int b, float v, float P, int K,
+                                               int row = 0) {
   uint32_t sr = 0;
   if (a.up.res > 0.0f && a.up.sto_round) {
     sr = philox4x32_10((uint32_t)j, (uint32_t)b, a.call, RNG_UPDATE_SR | ((uint32_t)is_x << 8), a.key.k0, a.key.k1).v[0];
@@ -143,7 +143,7 @@ __device__ __forceinline__ uint32_t pulse_word(const UpdateArgs &a, bool is_x, i
   uint32_t word = 0;
   if (PP != 0.0f && K > 0) {
     for (int k0 = 0; k0 < K; k0 += 4) {
-      const Philox4 r = philox4x32_10((uint32_t)j, (uint32_t)b, a.call, purpose | ((uint32_t)(k0 >> 2) << 8), a.key.k0, a.key.k1);
+      const Philox4 r = philox4x32_10((uint32_t)j, (uint32_t)b, a.call, purpose | ((uint32_t)(8 * row + (k0 >> 2)) << 8), a.key.k0, a.key.k1);
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         if (k0 + q < K && PP > u32_to_uniform(r.v[q])) word |= (2u << (k0 + q));
@@ -172,25 +172,28 @@ __global__ __launch_bounds__(256) void k_update_lines(UpdateArgs a) {
   const long s_b = is_x ? a.x_sb : a.d_sb, s_e = is_x ? a.x_sj : a.d_si;
   constexpr int ROWS_PER_PASS = 256 / LINES_E;
   const int col = threadIdx.x % LINES_E, row0 = threadIdx.x / LINES_E;
+  const int wps = max(a.words_per_sample, 1);
 #pragma unroll
   for (int i = 0; i < 64 / ROWS_PER_PASS; ++i) {
     const int rb = row0 + ROWS_PER_PASS * i;
     const int b = b0 + rb, e = e0 + col;
-    vals[rb][col] = (b < a.m_batch && e < size) ? src[(long)b * s_b + (long)e * s_e] : 0.0f;
+    const int sample = wps > 1 ? b / wps : b;
+    vals[rb][col] = (b < a.m_batch && e < size) ? src[(long)sample * s_b + (long)e * s_e] : 0.0f;
   }
   __syncthreads();
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int b = b0 + lane;
+  const int b = b0 + lane; // row of words
   const bool b_ok = b < a.m_batch;
-  const float P = b_ok ? (is_x ? a.prob_b[b] : a.prob_a[b]) : 0.0f;
-  const int K = b_ok ? a.bl[b] : 0;
+  const int sample = wps > 1 ? b / wps : b, wrow = wps > 1 ? b - sample * wps : 0;
+  const float P = b_ok ? (is_x ? a.prob_b[sample] : a.prob_a[sample]) : 0.0f;
+  const int K = b_ok ? min(max(a.bl[sample] - 31 * wrow, 0), 31) : 0;
   const int kmax = a.kmax[a.kmax_slot];
   uint32_t *planes = is_x ? a.x_planes : a.d_planes;
   const int c0 = 2 * blockIdx.y;
   for (int el = wave; el < LINES_E; el += 4) {
     const int e = e0 + el;
     if (e >= size) break; // wave-uniform
-    const uint32_t word = b_ok ? pulse_word(a, is_x, e, b, vals[lane][el], P, K) : 0u;
+    const uint32_t word = b_ok ? pulse_word(a, is_x, e, sample, vals[lane][el], P, K, wrow) : 0u;
     wt[lane][el] = word;
     for (int k = 0; k < kmax; ++k) {
       const unsigned long long m = __ballot((word >> (k + 1)) & 1u);

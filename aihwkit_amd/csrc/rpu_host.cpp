@@ -159,8 +159,8 @@ void UpdatePar::initialize() {
   default:
     throw RpuError("PulseType not supported");
   }
-  if (p.pulse_type != RPU_PULSE_NONE && p.pulse_type != RPU_PULSE_NONE_WITH_DEVICE && (p.desired_bl < 1 || p.desired_bl > 31)) {
-    throw RpuError("desired_bl must be within 1..31 (one 32-bit pulse word per line).");
+  if (p.pulse_type != RPU_PULSE_NONE && p.pulse_type != RPU_PULSE_NONE_WITH_DEVICE && (p.desired_bl < 1 || p.desired_bl > RPU_MAX_BL)) {
+    throw RpuError("desired_bl must be within 1.." + std::to_string(RPU_MAX_BL) + ".");
   }
 }
 

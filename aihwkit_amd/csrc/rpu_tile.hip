@@ -185,6 +185,7 @@ struct Tile {
   int *last_bl = nullptr;
   float *last_a = nullptr, *last_b = nullptr;
   uint32_t *last_xw = nullptr, *last_dw = nullptr;
+  int last_words_per_sample = 1;
   // transfer compound (rpu_transfer_device.{h,cpp}): device 0 takes the gradient update, device j is read
   // column by column and written onto device j + 1; the tile's weights d_w are the weighted sum, or the
   // last device itself when that one alone is visible
@@ -1108,13 +1109,23 @@ struct Tile {
                         const float *d, long d_sb, long d_si, int B, hipStream_t s, unsigned char *ws = nullptr) {
     if (lr == 0.0f) return;
     const DevicePar &dev = *dv.par;
-    // calculateBlAB (rpu_pulsed_meta_parameter.cpp:152-181): without a fixed BL and without BL management a learning
-    // rate beyond dw_min * desired_BL lengthens the bit line to ceil(lr / dw_min); a packed word holds 31 pulses
-    if (up.p.pulse_type == RPU_PULSE_STOCHASTIC_COMPRESSED && !up.p.fixed_bl && !up.p.update_bl_management &&
-        dv.granularity * (float)up.p.desired_bl < fabsf(lr) && ceilf(fabsf(lr) / dv.granularity) > 31.0f) {
-      throw RpuError("This learning rate needs a bit line of " + std::to_string((long)ceilf(fabsf(lr) / dv.granularity)) +
-                     " pulses (fixed_BL and update_bl_management are off); stochastic pulse trains hold at most 31.");
+    // The longest bit line this call can choose (calculateBlAB, rpu_pulsed_meta_parameter.cpp:152-181): desired_BL,
+    // or ceil(lr / dw_min) when neither a fixed BL nor BL management holds it there.  A packed word holds 31 pulses;
+    // longer lines take several rows of words per sample.
+    int bl_max = up.p.desired_bl;
+    if (!up.p.fixed_bl && !up.p.update_bl_management && dv.granularity * (float)up.p.desired_bl < fabsf(lr)) {
+      const float need = ceilf(fabsf(lr) / dv.granularity);
+      if (up.p.pulse_type == RPU_PULSE_STOCHASTIC_COMPRESSED && !(need <= (float)RPU_MAX_BL)) {
+        throw RpuError("This learning rate needs a bit line of " + std::to_string((long)need) +
+                       " pulses (fixed_BL and update_bl_management are off); stochastic pulse trains hold at most " +
+                       std::to_string(RPU_MAX_BL) + ".");
+      }
+      bl_max = std::max((int)need, 1);
     }
+    const int wps = up.p.pulse_type == RPU_PULSE_STOCHASTIC_COMPRESSED ? std::max((bl_max + 30) / 31, 1) : 1;
+    if (wps > 1 && ws) throw RpuError("update_noalloc holds bit lines of at most 31 pulses.");
+    if (wps > 1 && (long)B * wps > 0x7fffffffL) throw RpuError("Too many rows of pulse words for this batch.");
+    const int rows = B * wps; // rows of pulse words
     UpdateArgs a{};
     a.w = dv.w; a.x_size = X; a.d_size = D; a.m_batch = B;
     a.x = xin; a.x_sb = x_sb; a.x_sj = x_sj; a.d = d; a.d_sb = d_sb; a.d_si = d_si;
@@ -1138,9 +1149,9 @@ struct Tile {
       u_bl.ensure(B); u_a.ensure(B); u_b.ensure(B);
       a.bl = u_bl.p; a.prob_a = u_a.p; a.prob_b = u_b.p;
       if (up.p.pulse_type == RPU_PULSE_STOCHASTIC_COMPRESSED) {
-        u_xw.ensure((size_t)B * X); u_dw.ensure((size_t)B * D);
+        u_xw.ensure((size_t)rows * X); u_dw.ensure((size_t)rows * D);
         a.x_words = u_xw.p; a.d_words = u_dw.p;
-        set_plane_args(a, B);
+        set_plane_args(a, rows);
         a.kmax_slot = (int)(update_calls++ & 1u);
       } else {
         u_xval.ensure((size_t)B * X); u_dval.ensure((size_t)B * D);
@@ -1152,6 +1163,9 @@ struct Tile {
     prof_mark(s, "update_prepare");
     const bool counting = dev.p.count_pulses && !is_transfer();
     if (up.p.pulse_type == RPU_PULSE_STOCHASTIC_COMPRESSED) {
+      // from here on the kernels walk rows of words; a longer bit line is several rows of one sample in a row
+      a.m_batch = rows;
+      a.words_per_sample = wps;
       launch_update_lines(a, s);
       prof_mark(s, "update_lines");
       if (counting) count_pulses(a, false, s);
@@ -1178,6 +1192,7 @@ struct Tile {
     RPU_HIP_CHECK(hipGetLastError());
     last_stream = s;
     last_update_batch = B;
+    last_words_per_sample = wps;
     last_update_pulse = up.p.pulse_type;
     last_bl = a.bl; last_a = a.prob_a; last_b = a.prob_b; last_xw = a.x_words; last_dw = a.d_words;
   }
@@ -2625,9 +2640,22 @@ int rpu_tile_get_update_words(rpu_tile_t *tile, uint32_t *x_words_host, uint32_t
     }
     DeviceGuard g(t.device_id);
     t.sync_last();
-    RPU_HIP_CHECK(hipMemcpy(x_words_host, t.last_xw, (size_t)m_batch * t.X * 4, hipMemcpyDeviceToHost));
-    RPU_HIP_CHECK(hipMemcpy(d_words_host, t.last_dw, (size_t)m_batch * t.D * 4, hipMemcpyDeviceToHost));
+    const size_t rows = (size_t)m_batch * t.last_words_per_sample;
+    RPU_HIP_CHECK(hipMemcpy(x_words_host, t.last_xw, rows * t.X * 4, hipMemcpyDeviceToHost));
+    RPU_HIP_CHECK(hipMemcpy(d_words_host, t.last_dw, rows * t.D * 4, hipMemcpyDeviceToHost));
     RPU_HIP_CHECK(hipMemcpy(bl_host, t.last_bl, (size_t)m_batch * 4, hipMemcpyDeviceToHost));
+  });
+}
+
+int rpu_tile_get_update_words_per_sample(rpu_tile_t *tile, int32_t *words_per_sample) {
+  return guarded([&] {
+    if (!tile || !words_per_sample) throw RpuError("null argument");
+    Tile &t = tile->t;
+    std::lock_guard<std::mutex> lock(t.mutex);
+    if (!t.resident() || t.last_update_pulse != RPU_PULSE_STOCHASTIC_COMPRESSED) {
+      throw RpuError("No stochastic update has run on this tile.");
+    }
+    *words_per_sample = t.last_words_per_sample;
   });
 }
 

@@ -500,12 +500,20 @@ class _CudaTileMixin:
         self._finish(x_input, non_blocking)
 
     def get_update_words(self, m_batch: int):
-        """Packed pulse words and per-sample BL of the last stochastic update (CPU tensors)."""
-        x_words = torch.empty(m_batch, self.get_x_size(), dtype=torch.int32)
-        d_words = torch.empty(m_batch, self.get_d_size(), dtype=torch.int32)
+        """Packed pulse words and per-sample BL of the last stochastic update (CPU tensors).  With bit lines beyond 31
+        pulses a sample takes ``get_update_words_per_sample()`` consecutive rows of words."""
+        rows = m_batch * self.get_update_words_per_sample()
+        x_words = torch.empty(rows, self.get_x_size(), dtype=torch.int32)
+        d_words = torch.empty(rows, self.get_d_size(), dtype=torch.int32)
         bl = torch.empty(m_batch, dtype=torch.int32)
         check(lib().rpu_tile_get_update_words(self._h, x_words.data_ptr(), d_words.data_ptr(), bl.data_ptr(), m_batch))
         return x_words, d_words, bl
+
+    def get_update_words_per_sample(self) -> int:
+        """Rows of pulse words per sample of the last stochastic update: ceil(longest possible BL / 31)."""
+        n = C.c_int32(0)
+        check(lib().rpu_tile_get_update_words_per_sample(self._h, C.byref(n)))
+        return int(n.value)
 
     def get_update_ab(self, m_batch: int):
         """Per-sample probability scales (A for d, B for x) of the last pulsed update (CPU tensors)."""

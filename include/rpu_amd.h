@@ -138,7 +138,7 @@ typedef struct rpu_io_params {
  * AnalogTileUpdateParameter (B/rpu_base_devices.cpp:469-483). */
 typedef struct rpu_update_params {
   int32_t pulse_type;           /* RPU_PULSE_STOCHASTIC_COMPRESSED */
-  int32_t desired_bl;           /* 31; at most 31 (one 32-bit pulse word per line and sample) */
+  int32_t desired_bl;           /* 31; up to RPU_MAX_BL (beyond 31 a sample takes several rows of pulse words) */
   int32_t fixed_bl;             /* 1 */
   int32_t update_management;    /* 1 */
   int32_t update_bl_management; /* 1 */
@@ -346,8 +346,8 @@ int rpu_tile_update(rpu_tile_t *tile, const float *x_dev, const float *d_dev, in
  * (about 8 * m_batch * (x_size + d_size) bytes, + 4 * m_batch * x_size with bias) fails with a message that names both
  * sizes and changes nothing.  All tiles on a GPU share that GPU's array: calls that overlap in time on one GPU (other
  * streams, other threads) race, calls on one stream do not.  Not provided for transfer compounds, write noise, delta
- * weights and pulse counters (error).  rpu_tile_get_update_words / get_update_ab read this call's words until the
- * next no-allocation call on the same GPU overwrites them. */
+ * weights, pulse counters and bit lines beyond 31 pulses (error).  rpu_tile_get_update_words / get_update_ab read this
+ * call's words until the next no-allocation call on the same GPU overwrites them. */
 #define RPU_NOALLOC_MAX_SCRATCH_BYTES (6u << 20)
 int rpu_tile_update_noalloc(rpu_tile_t *tile, const float *x_dev, const float *d_dev, int m_batch, int bias,
                             int x_trans, int d_trans, void *stream);
@@ -639,6 +639,16 @@ int rpu_tile_set_extra(rpu_tile_t *tile, const int64_t *values_host, int count);
  * management).  Mirrors BitLineMaker::getCountsDebug (C/bit_line_maker.cu:1884). */
 int rpu_tile_get_update_words(rpu_tile_t *tile, uint32_t *x_words_host, uint32_t *d_words_host,
                               int32_t *bl_host, int m_batch);
+
+/* Bit lines longer than 31 pulses (the reference packs them into nK32 = BL / 32 + 1 words per line element,
+ * R/rpu_pulsed_meta_parameter.h:278, word layout R/rpu_weight_updater.cpp:297-324): a sample whose call can need
+ * up to BL_max pulses takes n = ceil(BL_max / 31) consecutive rows of words, each in the one-word format above (its own
+ * copy of the sign bit, 31 pulse slots); row r of sample b holds slots 31 r + 1 .. min(BL_b, 31 r + 31) and is zero
+ * beyond BL_b.  The device loop walks them as n samples in a row, which is the reference's slot order.
+ * rpu_tile_get_update_words then returns [m_batch * n][x_size] and [m_batch * n][d_size] (bl_host stays [m_batch]);
+ * *words_per_sample receives n of the last stochastic update (1 unless BL_max > 31). */
+#define RPU_MAX_BL 992 /* 32 rows of 31 pulses */
+int rpu_tile_get_update_words_per_sample(rpu_tile_t *tile, int32_t *words_per_sample);
 
 /* After a pulsed rpu_tile_update: the per-sample probability scales of that call, A for the d line and B for the x
  * line (PulsedUpdateMetaParameter::calculateBlAB / performUpdateManagement, R/rpu_pulsed_meta_parameter.cpp:152-236),

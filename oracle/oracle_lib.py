@@ -161,7 +161,8 @@ class OracleTile:
         xw = np.ascontiguousarray(x_words).view(np.uint32)
         dw = np.ascontiguousarray(d_words).view(np.uint32)
         bl = np.ascontiguousarray(bl, dtype=np.int32)
-        self.lib.orc_update_with_words(self.h, xw.ctypes.data, dw.ctypes.data, bl.ctypes.data, len(bl))
+        if self.lib.orc_update_with_words(self.h, xw.ctypes.data, dw.ctypes.data, bl.ctypes.data, len(bl)):
+            raise RuntimeError(self.lib.orc_last_error().decode())
 
     def update_bl_ab(self, x, d):
         x, d = _f32(x), _f32(d)

@@ -943,8 +943,8 @@ void sparse_update(OrcTile &t, int BL, int lr_sign) {
   }
 }
 
-void ensure_sparse_containers(OrcTile &t) {
-  const int K = std::max(t.up.desired_bl, 1);
+void ensure_sparse_containers(OrcTile &t, int bl = 0) {
+  const int K = std::max(std::max(t.up.desired_bl, bl), 1);
   if ((int)t.x_idx.size() < K) {
     t.x_idx.assign(K, std::vector<int>(t.X));
     t.d_idx.assign(K, std::vector<int>(t.D));
@@ -1068,7 +1068,7 @@ bool update_vector(OrcTile &t, const float *x, int x_inc, const float *d, int d_
   if (t.up.pulse_type == RPU_PULSE_STOCHASTIC_COMPRESSED || t.up.pulse_type == RPU_PULSE_STOCHASTIC) {
     if (!sample_bl_ab(t, x, x_inc, d, d_inc, lr < 0.0f ? -lr : lr, BL, A, B)) return false;
     if (BL == 0) return true;
-    ensure_sparse_containers(t);
+    ensure_sparse_containers(t, BL); // without update management a large learning rate lengthens the bit line
     generate_counts(t, t.x_cnt, t.x_idx, x, x_inc, X, B, BL);
     generate_counts(t, t.d_cnt, t.d_idx, d, d_inc, D, A, BL);
     sparse_update(t, BL, lr < 0.0f ? -1 : 1);
@@ -1133,8 +1133,8 @@ void *orc_create(int x_size, int d_size, const rpu_tile_config *cfg) {
   if (!init_io(t->fio, false) || !init_io(t->bio, true)) return nullptr;
   // R/rpu_pulsed_meta_parameter.cpp:134-150 initialize: UBLM implies UM
   t->up.update_management = t->up.update_management || t->up.update_bl_management;
-  if (t->up.desired_bl > 31 || t->up.desired_bl < 1) {
-    g_err = "oracle: desired_bl must be in 1..31";
+  if (t->up.desired_bl < 1) {
+    g_err = "oracle: desired_bl must be positive";
     return nullptr;
   }
   if (t->dev.kind == RPU_DEVICE_SOFT_BOUNDS) { // R/rpu_linearstep_device.h:68-80
@@ -1339,6 +1339,10 @@ int orc_update_with_words(void *h, const uint32_t *x_words, const uint32_t *d_wo
   for (int b = 0; b < m_batch; ++b) {
     const int BL = bl[b];
     if (BL <= 0) continue;
+    if (BL > 31) {
+      g_err = "oracle: a packed word holds 31 pulses (longer bit lines come as several rows of words)";
+      return 1;
+    }
     words_to_sparse(t->x_idx, t->x_cnt, x_words + (size_t)b * t->X, BL, t->X);
     words_to_sparse(t->d_idx, t->d_cnt, d_words + (size_t)b * t->D, BL, t->D);
     sparse_update(*t, BL, lr_sign);

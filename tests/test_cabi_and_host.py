@@ -118,7 +118,7 @@ def test_unsupported_parameters_fail_loudly():
     assert not any(k.startswith("rpu.bwd.") for k in host.dump_extra())
     make_meta(io_params(ir_drop=1.0, w_noise_type=dv.WeightNoiseType.PCMRead, w_noise=0.1)).create_array(4, 4, dev)
     with pytest.raises(RuntimeError, match="desired_bl"):
-        make_meta(desired_bl=255).create_array(4, 4, dev)
+        make_meta(desired_bl=1000).create_array(4, 4, dev)
     with pytest.raises(RuntimeError, match="not supported"):
         make_meta(pulse_type=17).create_array(4, 4, dev)
     make_meta(pulse_type=dv.PulseType.Stochastic).create_array(4, 4, dev)

@@ -275,26 +275,52 @@ def test_full_size_configuration_1_update_through_the_pulse_words(gpu_device):
         assert np.abs(orc.get_weights() - w).max() > 1e-3
 
 
-def test_learning_rate_beyond_the_pulse_word_is_refused_or_exact(gpu_device):
+def virtual_rows(bl, words_per_sample):
+    """Pulse slots held by each row of words: row r of a sample with bit line BL holds min(max(BL - 31 r, 0), 31)."""
+    r = np.arange(words_per_sample)[None, :]
+    return np.clip(np.asarray(bl)[:, None] - 31 * r, 0, 31).reshape(-1).astype(np.int32)
+
+
+def test_learning_rate_beyond_one_pulse_word(gpu_device):
     """Without a fixed BL and BL management, lr > dw_min * desired_BL stretches the bit line to ceil(lr / dw_min)
-    (rpu_pulsed_meta_parameter.cpp:166-171).  Stochastic words hold 31 pulses: refused.  The implicit pulse types keep
-    no words: they follow the oracle with the long bit line."""
+    (rpu_pulsed_meta_parameter.cpp:166-171).  Stochastic pulse trains beyond 31 pulses take several rows of words per
+    sample; the implicit pulse types keep no words.  Both follow the oracle with the long bit line."""
     rng = np.random.default_rng(4)
     x = rng.uniform(-1, 1, (9, 40)).astype(F32)
     d = rng.uniform(-1, 1, (9, 30)).astype(F32)
     w = rng.uniform(-0.3, 0.3, (30, 40)).astype(F32)
     kw = dict(dw_min=0.001, dw_min_std=0.0, construction_seed=2, enforce_consistency=True)
     meta = make_meta(desired_bl=31, fixed_bl=False, update_management=False, update_bl_management=False)
-    _, _, gpu = build_pair(meta, constant_step(**kw), 40, 30)
+    _, orc, gpu = build_pair(meta, constant_step(**kw), 40, 30)
     gpu.set_weights(torch.from_numpy(w))
+    orc.set_weights(w)
+    gpu.set_learning_rate(0.05)                       # ceil(0.05 / 0.001) = 50 pulses: two rows of words
+    orc.set_learning_rate(0.05)
+    gpu.update(cuda(x), cuda(d), False, False, False, False)
+    assert gpu.get_update_words_per_sample() == 2
+    xw, dw, bl = gpu.get_update_words(9)
+    assert xw.shape == (18, 40) and (bl.numpy() == 50).all()
+    a, b_ = gpu.get_update_ab(9)
+    assert (a.numpy() == 1.0).all() and (b_.numpy() == 1.0).all()             # :168-170
+    rows = virtual_rows(bl.numpy(), 2)
+    assert list(rows[:2]) == [31, 19]
+    xb = xw.numpy().view(np.uint32)
+    assert not (xb[1::2] >> 20).any()                 # nothing beyond slot 19 in the second row
+    # probability |x| per slot: the pulses of a line element over both rows
+    n_x = np.array([[bin(int(v) >> 1).count("1") for v in row] for row in xb]).reshape(9, 2, 40).sum(1)
+    assert abs((n_x - 50 * np.abs(x)).mean()) < 4 * np.sqrt(50 * 0.25 / x.size)
+    assert np.array_equal((xb[0::2] & 1)[n_x > 0], (x < 0).astype(np.uint32)[n_x > 0])
+    orc.update_with_words(xb, dw.numpy().view(np.uint32), rows)
+    assert np.abs(gpu.get_weights().numpy() - orc.get_weights()).max() <= 2e-5
+    assert np.abs(orc.get_weights() - w).max() > 0.01
+    gpu.set_learning_rate(0.031)                      # exactly 31: one row
+    gpu.update(cuda(x), cuda(d), False, False, False, False)
+    assert gpu.get_update_words_per_sample() == 1 and gpu.get_update_words(9)[2].max() == 31
+    gpu.set_learning_rate(1.5)                        # 1500 pulses: beyond what the rows hold
     before = gpu.get_weights().numpy().copy()
-    gpu.set_learning_rate(0.05)                       # ceil(0.05 / 0.001) = 50 pulses
-    with pytest.raises(RuntimeError, match="bit line of 50 pulses"):
+    with pytest.raises(RuntimeError, match="bit line of 1500 pulses"):
         gpu.update(cuda(x), cuda(d), False, False, False, False)
     assert np.array_equal(gpu.get_weights().numpy(), before)
-    gpu.set_learning_rate(0.031)                      # exactly 31: allowed
-    gpu.update(cuda(x), cuda(d), False, False, False, False)
-    assert gpu.get_update_words(9)[2].max() == 31
     meta = make_meta(desired_bl=31, fixed_bl=False, update_management=False, update_bl_management=False,
                      pulse_type=dv.PulseType.DeterministicImplicit)
     _, orc, gpu = build_pair(meta, soft_bounds(**kw), 40, 30)
@@ -307,6 +333,80 @@ def test_learning_rate_beyond_the_pulse_word_is_refused_or_exact(gpu_device):
     assert np.array_equal(counts, orc.implicit_counts(x, d)) and np.abs(counts).max() > 31
     orc.update(x, d)
     assert np.abs(gpu.get_weights().numpy() - orc.get_weights()).max() <= 1e-5
+
+
+@pytest.mark.parametrize("device", ["constant", "soft"])
+@pytest.mark.parametrize("desired_bl,ublm", [(100, True), (64, False), (200, True)])
+def test_bit_lines_beyond_31_pulses(gpu_device, device, desired_bl, ublm):
+    """desired_BL > 31 (nK32 > 1 in the reference, rpu_pulsed_meta_parameter.h:278): BL, A, B per sample bit-equal to
+    the oracle's, every row of words clean beyond its slots, and the weights after the GPU's words drive the oracle's
+    device loop row by row -- the rows of a sample in a row are the reference's slot order."""
+    rng = np.random.default_rng(desired_bl)
+    x_size, d_size, batch = 130, 70, 37
+    meta = make_meta(desired_bl=desired_bl, fixed_bl=not ublm, update_management=ublm, update_bl_management=ublm)
+    make = constant_step if device == "constant" else soft_bounds
+    _, orc, gpu = build_pair(meta, make(dw_min=0.001, dw_min_std=0.0, construction_seed=3, enforce_consistency=True), x_size, d_size)
+    w = rng.uniform(-0.3, 0.3, (d_size, x_size)).astype(F32)
+    x = (rng.uniform(-1, 1, (batch, x_size)) * rng.uniform(0.05, 1, (batch, 1))).astype(F32)
+    d = (rng.uniform(-1, 1, (batch, d_size)) * rng.uniform(0.05, 1, (batch, 1))).astype(F32)
+    x[5] = 0.0                                                       # a sample without pulses
+    gpu.set_weights(torch.from_numpy(w))
+    orc.set_weights(w)
+    lr = 0.1
+    gpu.set_learning_rate(lr)
+    orc.set_learning_rate(lr)
+    gpu.set_seed(11)
+    gpu.update(cuda(x), cuda(d), False, False, False, False)
+    wps = gpu.get_update_words_per_sample()
+    assert wps == (desired_bl + 30) // 31
+    xw, dw, bl = gpu.get_update_words(batch)
+    bl_o, a_o, b_o = orc.update_bl_ab(x, d)
+    assert np.array_equal(bl.numpy(), bl_o) and bl_o.max() > 31
+    if ublm:
+        assert len(set(bl_o.tolist())) > 5 and bl_o[5] == 0          # BL management picked different lengths
+    a, b_ = gpu.get_update_ab(batch)
+    assert np.array_equal(a.numpy(), a_o) and np.array_equal(b_.numpy(), b_o)
+    rows = virtual_rows(bl_o, wps)
+    xb, db = xw.numpy().view(np.uint32), dw.numpy().view(np.uint32)
+    for words in (xb, db):
+        beyond = (words.astype(np.uint64) >> (rows[:, None].astype(np.uint64) + 1)) != 0
+        assert not beyond.any()                                      # no bit beyond a row's slots (the sign is bit 0)
+        assert not words[rows == 0].any()
+    # pulse probabilities: mean number of pulses of a line element = BL * min(|x| B, 1)
+    n_x = np.array([[bin(int(v) >> 1).count("1") for v in row] for row in xb]).reshape(batch, wps, x_size).sum(1)
+    p = np.minimum(np.abs(x) * b_o[:, None], 1.0)
+    z = (n_x - bl_o[:, None] * p).sum() / np.sqrt((bl_o[:, None] * p * (1 - p)).sum())
+    assert abs(z) < 4
+    orc.update_with_words(xb, db, rows)
+    assert np.abs(gpu.get_weights().numpy() - orc.get_weights()).max() <= 2e-5
+    assert np.abs(orc.get_weights() - w).max() > 0.01
+
+
+def test_long_bit_line_moments_over_64_seeds(gpu_device):
+    """The stated statistical protocol on a long bit line (fixed BL = 80, three rows of words): mean and variance of the
+    weight change over 64 seeds, GPU's own pulse trains against the oracle's."""
+    rng = np.random.default_rng(1)
+    x_size, d_size, batch, seeds = 96, 64, 16, 64
+    meta = make_meta(desired_bl=80, fixed_bl=True, update_management=False, update_bl_management=False)
+    host, orc, _ = build_pair(meta, soft_bounds(dw_min=0.001, construction_seed=5, enforce_consistency=True), x_size, d_size, gpu=False)
+    w = rng.uniform(-0.3, 0.3, (d_size, x_size)).astype(F32)
+    x = rng.uniform(-1, 1, (batch, x_size)).astype(F32)
+    d = rng.uniform(-1, 1, (batch, d_size)).astype(F32)
+    host.set_weights(torch.from_numpy(w))
+    gpu = tiles.CudaAnalogTile(host)
+    dwg, dwo = [], []
+    for seed in range(seeds):
+        gpu.set_weights(torch.from_numpy(w))
+        gpu.set_learning_rate(0.05)
+        gpu.set_seed(100 + seed)
+        gpu.update(cuda(x), cuda(d), False, False, False, False)
+        dwg.append(gpu.get_weights().numpy() - w)
+        orc.set_weights(w)
+        orc.set_learning_rate(0.05)
+        orc.set_seed(500 + seed)
+        orc.update(x, d)
+        dwo.append(orc.get_weights() - w)
+    compare_moments(np.stack(dwg), np.stack(dwo), "weight change with a bit line of 80 pulses")
 
 
 # ---- configuration 4: LeNet5-shaped stack as im2col tiles -------------------------------------------------------
