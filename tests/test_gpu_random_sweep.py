@@ -63,12 +63,16 @@ def one_mvm(seed):
     ok2 = np.array_equal(g_g, g_o)
     return ok, ok2, desc
 
-def one_update(seed):
+def one_update(seed, long_lines=False):
     rng = np.random.default_rng(seed)
     x_size = int(rng.choice([1, 2, 3, 31, 32, 33, 63, 64, 65, 100, 255, 256, 257, 300]))
     d_size = int(rng.choice([1, 2, 3, 5, 16, 17, 33, 64, 65, 96, 128, 129]))
     batch = int(rng.choice([1, 2, 7, 31, 32, 33, 64, 65, 100, 127, 128, 129, 300]))
-    bl = int(rng.choice([1, 2, 3, 4, 7, 8, 15, 31]))
+    if long_lines:  # more than one row of 31 pulse slots per sample, at the edges of the rows
+        bl = int(rng.choice([32, 33, 61, 62, 63, 92, 93, 94, 100, 250]))
+        batch = min(batch, 100)
+    else:
+        bl = int(rng.choice([1, 2, 3, 4, 7, 8, 15, 31]))
     um = bool(rng.integers(2))
     soft = bool(rng.integers(2))
     lr = float(rng.choice([0.01, 0.05, -0.02]))
@@ -90,16 +94,19 @@ def one_update(seed):
         d[2] = 0.0
     gpu.update(cuda(x), cuda(d), False)
     xw, dw, blv = gpu.get_update_words(batch)
+    wps = gpu.get_update_words_per_sample()                       # rows of words per sample
     bl_orc, a_orc, b_orc = orc.update_bl_ab(x, d)
-    words_ok = np.array_equal(blv.numpy(), bl_orc) and int(blv.max()) <= bl
+    words_ok = np.array_equal(blv.numpy(), bl_orc) and int(blv.max()) <= bl and wps == (bl + 30) // 31
     a_gpu, b_gpu = (t.numpy() for t in gpu.get_update_ab(batch))
     words_ok = words_ok and np.array_equal(a_gpu, a_orc) and np.array_equal(b_gpu, b_orc)
+    rows = np.clip(blv.numpy()[:, None] - 31 * np.arange(wps)[None, :], 0, 31).reshape(-1).astype(np.int32)
     for words, values in ((xw.numpy().view(np.uint32), x), (dw.numpy().view(np.uint32), d)):
-        # no pulse beyond a sample's bit line, none on a zero value, the sign bit where the value is negative
-        words_ok = words_ok and not (words >> (blv.numpy().astype(np.uint32)[:, None] + 1)).any()
+        values = np.repeat(values, wps, axis=0)
+        # no pulse beyond a row's slots, none on a zero value, the sign bit where the value is negative
+        words_ok = words_ok and not (words.astype(np.uint64) >> (rows.astype(np.uint64)[:, None] + 1)).any()
         words_ok = words_ok and not (words[values == 0] >> 1).any()
         words_ok = words_ok and np.array_equal((words & 1)[(words >> 1) != 0] == 1, (values < 0)[(words >> 1) != 0])
-    orc.update_with_words(xw.numpy(), dw.numpy(), blv.numpy())
+    orc.update_with_words(xw.numpy(), dw.numpy(), rows)
     diff = np.abs(gpu.get_weights().numpy() - orc.get_weights()).max()
     desc = dict(seed=seed, X=x_size, D=d_size, B=batch, bl=bl, um=um, soft=soft, lr=lr, diff=float(diff), words_ok=words_ok)
     return diff <= 2e-5 and words_ok, desc
@@ -120,6 +127,12 @@ def test_random_update_cases_follow_the_oracle(gpu_device):
         ok, desc = one_update(seed)
         if not ok:
             failures.append(desc)
+    assert not failures, failures[:3]
+
+
+def test_random_update_cases_with_long_bit_lines_follow_the_oracle(gpu_device):
+    """Bit lines of 32 .. 250 pulses (two to nine rows of words per sample) over the same shapes."""
+    failures = [desc for ok, desc in (one_update(seed, long_lines=True) for seed in range(5500, 5600)) if not ok]
     assert not failures, failures[:3]
 
 
