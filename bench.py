@@ -408,7 +408,7 @@ def main() -> int:
             "value": devices_per_call / cpu_upd / 1e9, "unit": "Gdevice-updates/s", "cores": 1, "kind": "port",
             "sample": f"{n_upd} full update calls, 1 forward and 1 backward call of the same workload on the CPU oracle "
                       "(1 thread).  The oracle draws its random numbers faster than the reference's CPU path: it takes about "
-                      "0.23 s per update call where the compiled reference took 1.2 s on the survey machine (BASELINE.md), "
+                      "0.23 s per update call where the compiled reference took 1.2 s when it was measured on another machine, "
                       "so this baseline is about five times faster than the reference itself would be",
             "update_ms": cpu_upd * 1e3, "forward_ms": cpu_fwd * 1e3, "forward_gflops": flops_per_call / cpu_fwd / 1e9,
             "backward_ms": cpu_bwd * 1e3, "backward_gflops": flops_per_call / cpu_bwd / 1e9,
