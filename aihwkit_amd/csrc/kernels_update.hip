@@ -154,12 +154,13 @@ __device__ __forceinline__ uint32_t pulse_word(const UpdateArgs &a, bool is_x, i
   return word;
 }
 
-// Pulse words and their sample-transposed bit planes in one pass.  A workgroup owns 64 samples x 16 line elements
-// (x lines first, then d lines): the values are read 64 bytes per sample row into LDS, then each wave takes every
+// Pulse words and their sample-transposed bit planes in one pass.  A workgroup owns 64 samples x LINES_E line elements
+// (x lines first, then d lines): the values are read 4 LINES_E bytes per sample row into LDS, then each wave takes every
 // fourth element with its lanes on the 64 samples, so that a ballot over the wave is a plane word; the packed words
-// go back through LDS and are written 64 bytes per sample row.
-constexpr int LINES_E = 16;
-
+// go back through LDS and are written 4 LINES_E bytes per sample row.
+// LINES_E = 16 moves whole 64-byte row segments; small launches take 4 elements per workgroup (one per wave) so that
+// there are four times as many workgroups.
+template <int LINES_E>
 __global__ __launch_bounds__(256) void k_update_lines(UpdateArgs a) {
   __shared__ float vals[64][LINES_E + 1];
   __shared__ uint32_t wt[64][LINES_E + 1];
@@ -1103,8 +1104,13 @@ void launch_update_prepare(const UpdateArgs &a, hipStream_t s) {
 }
 
 void launch_update_lines(const UpdateArgs &a, hipStream_t s) {
-  const dim3 grid((a.x_size + LINES_E - 1) / LINES_E + (a.d_size + LINES_E - 1) / LINES_E, (a.m_batch + 63) / 64);
-  hipLaunchKernelGGL(k_update_lines, grid, dim3(256), 0, s, a);
+  const unsigned sample_tiles = (a.m_batch + 63) / 64;
+  const unsigned wide = (a.x_size + 15) / 16 + (a.d_size + 15) / 16;
+  if (wide * sample_tiles >= 256) {
+    hipLaunchKernelGGL(k_update_lines<16>, dim3(wide, sample_tiles), dim3(256), 0, s, a);
+  } else {
+    hipLaunchKernelGGL(k_update_lines<4>, dim3((a.x_size + 3) / 4 + (a.d_size + 3) / 4, sample_tiles), dim3(256), 0, s, a);
+  }
 }
 
 void launch_update_implicit_lines(const UpdateArgs &a, hipStream_t s) {
