@@ -38,3 +38,17 @@ def device_weights(tile, k):
     """Weights of device k of a transfer tile (the hidden_weights_k entry of its hidden parameters)."""
     names = tile.get_hidden_parameter_names()
     return tile.get_hidden_parameters()[names.index(f"hidden_weights_{k}")].numpy()
+
+
+def transfer_draws(seed, update_idx, frm):
+    """The two uniforms a tile with this seed draws on the host for the transfer of device `frm` after update vector
+    `update_idx`: Philox4x32-10, counter (device, counter low, counter high, 17), key = seed; 24-bit uniforms."""
+    import ctypes as C
+
+    import numpy as np
+
+    from aihwkit_amd import _cabi
+    out = (C.c_uint32 * 4)()
+    _cabi.check(_cabi.lib().rpu_philox4x32_10((C.c_uint32 * 4)(frm, update_idx & 0xFFFFFFFF, update_idx >> 32, 17),
+                                              (C.c_uint32 * 2)(seed & 0xFFFFFFFF, seed >> 32), out))
+    return [np.float32((v >> 8) * (1.0 / 16777216.0)) for v in out]

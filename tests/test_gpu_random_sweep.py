@@ -341,13 +341,13 @@ def test_random_groups_are_bit_exact(gpu_device):
 
 
 def one_transfer(seed):
-    from helpers import build_transfer_pair, device_weights, transfer_param
+    from helpers import build_transfer_pair, device_weights, transfer_draws, transfer_param
 
     rng = np.random.default_rng(seed)
     x_size = int(rng.choice([2, 5, 31, 33, 37, 64, 65, 130]))
     d_size = int(rng.choice([1, 3, 21, 32, 33, 64, 70]))
     batch = int(rng.choice([1, 3, 8, 33]))
-    n_devices = int(rng.choice([2, 2, 3, 4]))
+    n_devices = int(rng.choice([2, 2, 3, 4, 6]))
     soft = bool(rng.integers(2))
     kw = dict(transfer_every=float(rng.choice([1.0, 2.0, 3.0, 5.0])), n_reads_per_transfer=int(rng.choice([1, 2, 3, 40])),
               units_in_mbatch=bool(rng.integers(2)), transfer_columns=bool(rng.integers(2)))
@@ -359,17 +359,25 @@ def one_transfer(seed):
         kw.update(fast_lr=0.02, scale_fast_lr=bool(rng.integers(2)))
     if rng.integers(3) == 0:
         kw["scale_transfer_lr"] = bool(rng.integers(2))
+    if rng.integers(3) == 0:
+        kw["random_selection"] = True
+    if kw["transfer_columns"] and rng.integers(3) == 0:
+        kw["with_reset_prob"] = float(rng.choice([0.3, 1.0]))
     f_io = noise_free_io(noise_management=NM.AbsMax, bound_management=BM.Iterative)
     b_io = noise_free_io(noise_management=NM.AbsMax)
     meta = make_meta(f_io, b_io, pulse_type=dv.PulseType.DeterministicImplicit, desired_bl=31)
     make = soft_bounds if soft else constant_step
-    devs = [make(dw_min=0.002, dw_min_std=0.0, enforce_consistency=True) for _ in range(n_devices)]
+    devs = [make(dw_min=0.002, dw_min_std=0.0, enforce_consistency=True, reset=0.01, reset_dtod=0.1, reset_std=0.0)
+            for _ in range(n_devices)]
     devs[0].dw_min = 0.004
     tr = transfer_param(devs, construction_seed=int(rng.integers(1, 99)), **kw)
     tr.transfer_forward = noise_free_io()
     tr.transfer_update.pulse_type = dv.PulseType.DeterministicImplicit
     tr.transfer_update.desired_bl = 31
     host, orc, gpu = build_transfer_pair(meta, tr, x_size, d_size)
+    gpu.set_seed(seed)                                  # the tile's host draws (first column, reset lottery) ...
+    orc.select = lambda idx, frm: transfer_draws(seed, idx, frm)[0]          # ... go to the oracle as well
+    orc.reset_lottery = lambda idx, frm: transfer_draws(seed, idx, frm)[1]
     w = rng.uniform(-0.4, 0.4, (d_size, x_size)).astype(np.float32)
     gpu.set_weights(torch.from_numpy(w))
     orc.set_weights(w)
@@ -395,8 +403,9 @@ def one_transfer(seed):
 
 
 def test_random_transfer_compounds_follow_the_oracle(gpu_device):
-    """Two to four devices, columns or rows, transfer periods in vectors or mini-batches, more reads than columns,
-    learning-rate scalings, visible fast device or fully hidden chain: five update calls each, all device matrices,
+    """Two to six devices, columns or rows, transfer periods in vectors or mini-batches, more reads than columns,
+    learning-rate scalings, visible fast device or fully hidden chain, random selection of the first column, reset of
+    the read columns: five update calls each, all device matrices,
     the reduced weights and the transfer counters against the oracle."""
     failures = [desc for ok, desc in (one_transfer(seed) for seed in range(50000, 50080)) if not ok]
     assert not failures, failures[:3]
