@@ -194,6 +194,7 @@ SYMBOLS = {
     "rpu_tile_update_noalloc": (C.c_int, [_P, _P, _P, C.c_int, C.c_int, C.c_int, C.c_int, _P]),
     "rpu_tile_get_update_words": (C.c_int, [_P, _P, _P, _P, C.c_int]),
     "rpu_tile_get_update_words_per_sample": (C.c_int, [_P, _P]),
+    "rpu_tile_set_fused_rounds": (C.c_int, [_P, C.c_int]),
     "rpu_tile_get_update_ab": (C.c_int, [_P, _P, _P, C.c_int]),
     "rpu_tile_update_with_words": (C.c_int, [_P, _P, _P, C.c_int, _P]),
     "rpu_tile_get_implicit_counts": (C.c_int, [_P, _P, C.c_int]),

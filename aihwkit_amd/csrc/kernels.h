@@ -34,6 +34,17 @@ struct MvmState {
   int *tile_done;  // tile_done[r * tiles_b + t] = workgroups of round r that have finished sample tile t
 };
 
+// Rounds 0 and 1 of a call in one launch (samples that need a second round are the rule on some workloads):
+// the state of that launch and of the selection that the following launch starts with.
+struct DualDev {
+  float *buf[2]; // buf[r]: [m_batch][O] outputs of round r of the fused launch
+  int *sel;      // [m_batch] which of them is the sample's output (0 / 1); 2: the sample is listed for round 2
+  int *hit1;     // [2][m_batch] saturation marks of round 1: upper, lower (as MvmState::hit_up / hit_lo)
+  float *xq2;    // quantized rows of round 2, written while round 0's rows are still read
+  int *seen;     // host-visible: [0] samples of the last call that needed round 1, [1] its batch; null: not kept
+  int on;        // 1: the fused launch; 2: this launch starts with the selection of the fused launch's results
+};
+
 struct MvmArgs {
   const float *w; // row-major [d_size][x_size]
   int x_size, d_size;
@@ -72,12 +83,17 @@ struct MvmArgs {
                             // largest absolute input in st.nm, 2 = it takes the scales from st.nm; 0 otherwise
   int small_tiles_only;     // 1: never the large-tile kernel (its row padding differs)
   const int *skip_if_zero;  // non-null: a round launch does nothing when this device value is zero
+  DualDev dual;
 };
 
 // noise management + per-sample state for round 0
 void launch_mvm_init(const MvmArgs &a, hipStream_t s);
 // one round of DAC -> MFMA contraction -> ADC
 void launch_mvm_round(const MvmArgs &a, hipStream_t s);
+// rounds 0 and 1 in one launch (a.dual filled in); the launches of rounds 2 .. follow with a.dual.on = 2 on the first
+// of them and a.xq[0] = a.dual.xq2
+bool mvm_can_fuse_rounds(const MvmArgs &a);
+void launch_mvm_dual(const MvmArgs &a, hipStream_t s);
 // AverageAbsMax noise management (rpu_forward_backward_pass.cpp:138-149): nm[b] holds the largest absolute input of
 // sample b and becomes the running average after that sample, in batch order; aux carries the value between calls
 // (negative: not started)

@@ -162,17 +162,22 @@ __device__ __forceinline__ void mvm_adc_values(const MvmArgs &a, int round, int 
 // up / lo return 1 + the largest output index that hit the upper / lower ADC bound (0: none).
 __device__ __forceinline__ void mvm_finish_outputs(const MvmArgs &a, int round, int b, float fin, int o0, float (&v)[4],
                                                    int &up, int &lo, const float *pre = nullptr,
-                                                   const float *post = nullptr) {
+                                                   const float *post = nullptr, float *out_rows = nullptr) {
   up = 0;
   lo = 0;
   float *out_p = a.out + (long)b * a.out_sb + (long)o0 * a.out_so;
+  long out_so = a.out_so;
+  if (out_rows) { // results kept aside, sample-major: [m_batch][O]
+    out_p = out_rows + (long)b * a.O + o0;
+    out_so = 1;
+  }
   if (a.io.perfect) {
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
       if (o0 + q < a.O) {
         float res = a.alpha * v[q];
-        if (a.beta != 0.0f) res += a.beta * out_p[(long)q * a.out_so];
-        out_p[(long)q * a.out_so] = res;
+        if (a.beta != 0.0f) res += a.beta * out_p[(long)q * out_so];
+        out_p[(long)q * out_so] = res;
       }
     }
     return;
@@ -181,342 +186,19 @@ __device__ __forceinline__ void mvm_finish_outputs(const MvmArgs &a, int round, 
   if (fin == 0.0f) { // zero input: the reference short-cuts to a zero output
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
-      if (o0 + q < a.O) out_p[(long)q * a.out_so] = 0.0f;
+      if (o0 + q < a.O) out_p[(long)q * out_so] = 0.0f;
     }
     return;
   }
 
   mvm_adc_values(a, round, b, fin, o0, v, up, lo, pre, post);
-  if (a.out_so == 1 && (o0 + 3) < a.O && ((((uintptr_t)out_p) & 15) == 0)) {
+  if (out_so == 1 && (o0 + 3) < a.O && ((((uintptr_t)out_p) & 15) == 0)) {
     *reinterpret_cast<float4 *>(out_p) = make_float4(v[0], v[1], v[2], v[3]);
   } else {
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
-      if (o0 + q < a.O) out_p[(long)q * a.out_so] = v[q];
+      if (o0 + q < a.O) out_p[(long)q * out_so] = v[q];
     }
-  }
-}
-
-// Instruction order of one pipelined step (a hint to the scheduler): the 16 MFMAs are spread over the step with
-// the LDS writes of the next step's tiles between the first ones and its global loads and LDS reads
-// between the others, so that the LDS and memory pipes work underneath the matrix pipe of the same wave.
-template <int WMODE>
-__device__ __forceinline__ void mvm_step_schedule() {
-#define RPU_SG(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)
-#define RPU_SG_MFMA 0x008
-#define RPU_SG_VMEM 0x020
-#define RPU_SG_DSR 0x100
-#define RPU_SG_DSW 0x200
-  if (WMODE != 1) { // per step: 8 LDS writes, 8 global loads, 8 LDS reads
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      RPU_SG(RPU_SG_MFMA, 1);
-      RPU_SG(RPU_SG_DSW, 1);
-    }
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      RPU_SG(RPU_SG_MFMA, 1);
-      RPU_SG(RPU_SG_VMEM, 1);
-      RPU_SG(RPU_SG_DSR, 1);
-    }
-  } else { // per step: 4 LDS writes, 20 global loads, 4 LDS reads
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      RPU_SG(RPU_SG_MFMA, 1);
-      RPU_SG(RPU_SG_DSW, 1);
-    }
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      RPU_SG(RPU_SG_MFMA, 1);
-      RPU_SG(RPU_SG_VMEM, 2);
-      RPU_SG(RPU_SG_DSR, 1);
-    }
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      RPU_SG(RPU_SG_MFMA, 1);
-      RPU_SG(RPU_SG_VMEM, 2);
-    }
-  }
-#undef RPU_SG
-#undef RPU_SG_MFMA
-#undef RPU_SG_VMEM
-#undef RPU_SG_DSR
-#undef RPU_SG_DSW
-  __builtin_amdgcn_sched_barrier(0);
-}
-
-// WMODE = how the weight operand is addressed:
-//   0  contraction index contiguous (forward), rows 16-byte aligned, K a multiple of 16
-//   1  output index contiguous (backward: W is read transposed in place)
-//   2  contraction index contiguous, any row length and alignment (a tile with a bias column has an odd row
-//      length): 16-byte loads from 4-byte aligned addresses, the last 1 .. 3 elements of a row one by one
-// Operand tiles with a contiguous contraction index (the quantized inputs always, the weights in modes 0, 2) are
-// fetched with unit-stride 16-byte loads, 8 lanes per 128-byte row segment, staged in a wave-private LDS
-// tile and read back in the MFMA operand layout (lane (r, h) holds row r, k = 16 h .. 16 h + 15).  Reading
-// them straight into that layout would make every lane of a load touch a different cache line, which is
-// address-bound in the vector L1.  Mode 1 reads the weights directly: 32 consecutive outputs per half-wave
-// and k are one line.  Out-of-range rows / k are clamped to valid addresses: their products meet the zero
-// padding of the quantized inputs or are never stored.
-// PD = 2, 4: software pipeline with the global loads of PD steps in flight, k_pad a multiple of
-// PD * KSTEP * WAVES; PD = 1: one register set, for short contractions, k_pad a multiple of KSTEP.
-template <int PD, int WMODE>
-__device__ __forceinline__ void mvm_round_tile(const MvmArgs &a, int round, int tile_o, int tile_b, int n_act,
-                                               float (*red)[16][64], float *stage) {
-  const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
-  const int r = lane & 31;
-  const int h = lane >> 5;
-
-  // operand rows owned by this lane in the MFMA layout
-  const int o_in = tile_o * TILE + r;
-  const bool o_ok = o_in < a.O;
-  const int slot_in = tile_b * TILE + r;
-  const bool b_ok = slot_in < n_act;
-
-  const long w_so = a.transposed ? 1 : a.x_size;
-  const long w_sk = a.transposed ? a.x_size : 1;
-  const int K = a.K;
-  // steps of 32 k-values, dealt to the waves in contiguous parts (equal parts, a multiple of PD, when PD >= 2;
-  // a short contraction may leave the last waves without a step)
-  const int steps = a.k_pad / KSTEP;
-  const int per_wave = (steps + WAVES - 1) / WAVES;
-  const int s_begin = min(wave * per_wave, steps);
-  const int s_end = min(s_begin + per_wave, steps);
-
-  float *stage_x = stage + wave * (2 * TILE * LDS_ROW);
-  float *stage_w = stage_x + TILE * LDS_ROW;
-
-  // staging layout of this lane: pass t covers rows 8 t .. 8 t + 7, lane = (row in pass) * 8 + 16-byte chunk
-  const int st_row = lane >> 3;
-  const int st_chunk = (lane & 7) * 4;
-  const float *xq = pick2(a.xq, round & 1);
-  const float *x_src[4];
-  const float *w_src[4];
-#pragma unroll
-  for (int t = 0; t < 4; ++t) {
-    const int row = t * 8 + st_row;
-    const int slot = min(tile_b * TILE + row, n_act - 1);
-    const int xrow = (round > 0) ? pick2(a.st.row, round & 1)[slot] : slot;
-    x_src[t] = xq + (long)xrow * a.k_pad + st_chunk;
-    const int o = min(tile_o * TILE + row, a.O - 1);
-    w_src[t] = a.w + (long)o * a.x_size;
-  }
-  const float *w_col = a.w + (long)(o_ok ? o_in : a.O - 1) * w_so; // mode 1: this lane's output column
-
-  floatx16 acc;
-#pragma unroll
-  for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
-
-  // sample of this lane's output column and its output factor: fetched now, used by the ADC stage
-  int b_out = slot_in;
-  float fin_out = 1.0f;
-  if (!a.io.perfect && b_ok) {
-    if (round > 0) b_out = pick2(a.st.list, round & 1)[slot_in];
-    fin_out = a.st.fin[b_out];
-  }
-
-  auto gload = [&](int s, f32x4 (&gx)[4], f32x4 (&gw)[4], float (&wd)[16]) {
-    const int k0 = s * KSTEP;
-#pragma unroll
-    for (int t = 0; t < 4; ++t) gx[t] = *reinterpret_cast<const f32x4 *>(x_src[t] + k0);
-    if (WMODE == 0) {
-      const int kc = min(k0 + st_chunk, K - 4); // K % 16 == 0: past K the inputs are zero padding
-#pragma unroll
-      for (int t = 0; t < 4; ++t) gw[t] = *reinterpret_cast<const f32x4 *>(w_src[t] + kc);
-    } else if (WMODE == 1) {
-#pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const int kc = min(k0 + h * 16 + i, K - 1);
-        wd[i] = w_col[(long)kc * w_sk];
-      }
-    } else {
-      const int kc = k0 + st_chunk;
-      if (kc + 4 <= K) {
-#pragma unroll
-        for (int t = 0; t < 4; ++t) gw[t] = *reinterpret_cast<const f32x4_unaligned *>(w_src[t] + kc);
-      } else { // the end of a row: nothing is read past it
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {
-          f32x4 z;
-          z.x = (kc < K) ? w_src[t][kc] : 0.0f;
-          z.y = (kc + 1 < K) ? w_src[t][kc + 1] : 0.0f;
-          z.z = (kc + 2 < K) ? w_src[t][kc + 2] : 0.0f;
-          z.w = 0.0f;
-          gw[t] = z;
-        }
-      }
-    }
-  };
-  auto lds_store = [&](const f32x4 (&gx)[4], const f32x4 (&gw)[4]) {
-#pragma unroll
-    for (int t = 0; t < 4; ++t) {
-      const int off = (t * 8 + st_row) * LDS_ROW + st_chunk;
-      *reinterpret_cast<f32x4 *>(stage_x + off) = gx[t];
-      if (WMODE != 1) *reinterpret_cast<f32x4 *>(stage_w + off) = gw[t];
-    }
-  };
-  auto lds_read = [&](float (&xd)[16], float (&wd)[16]) {
-#pragma unroll
-    for (int v4 = 0; v4 < 4; ++v4) {
-      const int off = r * LDS_ROW + h * 16 + v4 * 4;
-      const f32x4 tx = *reinterpret_cast<const f32x4 *>(stage_x + off);
-      xd[v4 * 4 + 0] = tx.x; xd[v4 * 4 + 1] = tx.y; xd[v4 * 4 + 2] = tx.z; xd[v4 * 4 + 3] = tx.w;
-      if (WMODE != 1) {
-        const f32x4 tw = *reinterpret_cast<const f32x4 *>(stage_w + off);
-        wd[v4 * 4 + 0] = tw.x; wd[v4 * 4 + 1] = tw.y; wd[v4 * 4 + 2] = tw.z; wd[v4 * 4 + 3] = tw.w;
-      }
-    }
-  };
-  auto mfma16 = [&](const float (&wd)[16], const float (&xd)[16]) {
-#pragma unroll
-    for (int i = 0; i < 16; ++i) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(wd[i], xd[i], acc, 0, 0, 0);
-  };
-
-  if constexpr (PD >= 2) {
-    // PD register sets hold the global loads of the next PD steps; the operand registers are double
-    // buffered, so the LDS round trip of step t + 1 and the loads of step t + 1 + PD are issued ahead
-    // of the 16 MFMAs of step t and complete underneath them.
-    f32x4 gx0[4], gw0[4], gx1[4], gw1[4], gx2[4], gw2[4], gx3[4], gw3[4];
-    float wr0[16], wr1[16], wr2[16], wr3[16];
-    float xc0[16], wc0[16], xc1[16], wc1[16];
-    // step T runs from the operand registers (XC, WC); step T + 1 moves from register set (GX, GW, WR)
-    // through LDS into (XN, WN) and the set is refilled with step T + 1 + PD
-#define RPU_MVM_STEP(T, GX, GW, WR, XC, WC, XN, WN)                      \
-  {                                                                      \
-    lds_store(GX, GW);                                                   \
-    if (WMODE == 1) {                                                    \
-      _Pragma("unroll") for (int i = 0; i < 16; ++i) WN[i] = WR[i];      \
-    }                                                                    \
-    gload(min((T) + 1 + PD, s_end - 1), GX, GW, WR);                     \
-    lds_read(XN, WN);                                                    \
-    mfma16(WC, XC);                                                      \
-    mvm_step_schedule<WMODE>();                                          \
-  }
-    gload(s_begin, gx0, gw0, wr0);
-    gload(min(s_begin + 1, s_end - 1), gx1, gw1, wr1);
-    if constexpr (PD == 4) {
-      gload(min(s_begin + 2, s_end - 1), gx2, gw2, wr2);
-      gload(min(s_begin + 3, s_end - 1), gx3, gw3, wr3);
-    }
-    lds_store(gx0, gw0);
-    lds_read(xc0, wc0);
-    if (WMODE == 1) {
-#pragma unroll
-      for (int i = 0; i < 16; ++i) wc0[i] = wr0[i];
-    }
-    gload(min(s_begin + PD, s_end - 1), gx0, gw0, wr0);
-    for (int s = s_begin; s < s_end; s += PD) {
-      if constexpr (PD == 4) {
-        RPU_MVM_STEP(s, gx1, gw1, wr1, xc0, wc0, xc1, wc1)
-        RPU_MVM_STEP(s + 1, gx2, gw2, wr2, xc1, wc1, xc0, wc0)
-        RPU_MVM_STEP(s + 2, gx3, gw3, wr3, xc0, wc0, xc1, wc1)
-        RPU_MVM_STEP(s + 3, gx0, gw0, wr0, xc1, wc1, xc0, wc0)
-      } else {
-        RPU_MVM_STEP(s, gx1, gw1, wr1, xc0, wc0, xc1, wc1)
-        RPU_MVM_STEP(s + 1, gx0, gw0, wr0, xc1, wc1, xc0, wc0)
-      }
-    }
-#undef RPU_MVM_STEP
-  } else {
-    f32x4 gx[4], gw[4];
-    float wn[16], xc[16], wc[16];
-    if (s_begin < s_end) gload(s_begin, gx, gw, wn);
-    for (int s = s_begin; s < s_end; ++s) {
-      lds_store(gx, gw);
-      lds_read(xc, wc);
-      if (WMODE == 1) {
-#pragma unroll
-        for (int i = 0; i < 16; ++i) wc[i] = wn[i];
-      }
-      gload(min(s + 1, s_end - 1), gx, gw, wn);
-      mfma16(wc, xc);
-    }
-  }
-
-  // sum the four parts of the contraction in a fixed order
-#pragma unroll
-  for (int i = 0; i < 16; ++i) red[wave][i][lane] = acc[i];
-  __syncthreads();
-
-  // this wave finishes accumulator group `wave`: rows wave*8 + h*4 + m, column r
-  float v[4];
-#pragma unroll
-  for (int q = 0; q < 4; ++q) {
-    const int i = wave * 4 + q;
-    v[q] = ((red[0][i][lane] + red[1][i][lane]) + red[2][i][lane]) + red[3][i][lane];
-  }
-  const int o0 = tile_o * TILE + wave * 8 + h * 4;
-  int up = 0, lo = 0;
-  if (b_ok && o0 < a.O) {
-    const float *pre = nullptr, *post = nullptr;
-    if (a.pre_add) {
-      const int xrow = (round > 0) ? pick2(a.st.row, round & 1)[slot_in] : slot_in;
-      pre = a.pre_add + (long)xrow * a.O;
-      if (a.post_add) post = a.post_add + (long)xrow * a.O;
-    }
-    mvm_finish_outputs(a, round, b_out, fin_out, o0, v, up, lo, pre, post);
-  }
-  if (!a.io.perfect && a.io.bound_management != RPU_BM_NONE) {
-    // saturation flags of the tile's 32 samples: combined in LDS, then one device-scope atomic per sample
-    // and bound.  The returned values are consumed so that the wave waits until the atomics have been
-    // performed before the workgroup signals its tile as finished (mvm_tile_finished).
-    int *hits = reinterpret_cast<int *>(&red[0][0][0]); // the partial sums have been consumed ...
-    __syncthreads();                                      // ... by every wave
-    if (threadIdx.x < 2 * TILE) hits[threadIdx.x] = 0;
-    __syncthreads();
-    if (up) atomicMax(&hits[r], up);
-    if (lo) atomicMax(&hits[TILE + r], lo);
-    __syncthreads();
-    if (threadIdx.x < 2 * TILE) {
-      const int t = threadIdx.x & (TILE - 1);
-      const int hit = hits[threadIdx.x];
-      const int slot = tile_b * TILE + t;
-      if (hit && slot < n_act) {
-        const int bs = (round > 0) ? pick2(a.st.list, round & 1)[slot] : slot;
-        const int old = atomicMax(threadIdx.x < TILE ? &a.st.hit_up[bs] : &a.st.hit_lo[bs], hit);
-        asm volatile("" ::"v"(old));
-      }
-    }
-  }
-}
-
-// ---------------------------------------------------------------------------------------------
-// per-sample noise management and state of round 0.  One workgroup per sample.
-// rpu_forward_backward_pass.cpp:112-178 (scales), :919-969 (forward), :1003-1022 (backward)
-
-// Reductions over the SUB threads that share a sample: SUB = 256 is the whole workgroup (through LDS), smaller
-// values are aligned lane groups of a wave (shuffles).  Every thread of the group gets the result.
-template <int SUB>
-__device__ __forceinline__ float group_max(float v, float *sh) {
-  if constexpr (SUB == 256) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off));
-    if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = v;
-    __syncthreads();
-    const float r = fmaxf(fmaxf(sh[0], sh[1]), fmaxf(sh[2], sh[3]));
-    __syncthreads();
-    return r;
-  } else {
-#pragma unroll
-    for (int off = SUB / 2; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off));
-    return v;
-  }
-}
-
-template <int SUB>
-__device__ __forceinline__ float group_sum(float v, float *sh) {
-  if constexpr (SUB == 256) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
-    if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = v;
-    __syncthreads();
-    const float r = ((sh[0] + sh[1]) + sh[2]) + sh[3];
-    __syncthreads();
-    return r;
-  } else {
-#pragma unroll
-    for (int off = SUB / 2; off > 0; off >>= 1) v += __shfl_xor(v, off);
-    return v;
   }
 }
 
@@ -576,6 +258,404 @@ __device__ __forceinline__ float next_round_scale(const MvmArgs &a, int round, i
   if (!next_round_params(a, round, b, fin, nm, red)) return 0.0f;
   float fin_next;
   return round_scales(a, nm, red, fin_next);
+}
+
+// Instruction order of one pipelined step (a hint to the scheduler): the 16 MFMAs are spread over the step with
+// the LDS writes of the next step's tiles between the first ones and its global loads and LDS reads
+// between the others, so that the LDS and memory pipes work underneath the matrix pipe of the same wave.
+template <int WMODE, bool DUAL = false>
+__device__ __forceinline__ void mvm_step_schedule() {
+#define RPU_SG(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)
+#define RPU_SG_MFMA 0x008
+#define RPU_SG_VMEM 0x020
+#define RPU_SG_DSR 0x100
+#define RPU_SG_DSW 0x200
+  if (DUAL) { // per step: 32 MFMAs, 12 LDS writes, 12 global loads, 12 LDS reads
+#pragma unroll
+    for (int i = 0; i < 12; ++i) {
+      RPU_SG(RPU_SG_MFMA, 1);
+      RPU_SG(RPU_SG_DSW, 1);
+    }
+#pragma unroll
+    for (int i = 0; i < 12; ++i) {
+      RPU_SG(RPU_SG_MFMA, 1);
+      RPU_SG(RPU_SG_VMEM, 1);
+      RPU_SG(RPU_SG_DSR, 1);
+    }
+    RPU_SG(RPU_SG_MFMA, 8);
+  } else if (WMODE != 1) { // per step: 8 LDS writes, 8 global loads, 8 LDS reads
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      RPU_SG(RPU_SG_MFMA, 1);
+      RPU_SG(RPU_SG_DSW, 1);
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      RPU_SG(RPU_SG_MFMA, 1);
+      RPU_SG(RPU_SG_VMEM, 1);
+      RPU_SG(RPU_SG_DSR, 1);
+    }
+  } else { // per step: 4 LDS writes, 20 global loads, 4 LDS reads
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      RPU_SG(RPU_SG_MFMA, 1);
+      RPU_SG(RPU_SG_DSW, 1);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      RPU_SG(RPU_SG_MFMA, 1);
+      RPU_SG(RPU_SG_VMEM, 2);
+      RPU_SG(RPU_SG_DSR, 1);
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      RPU_SG(RPU_SG_MFMA, 1);
+      RPU_SG(RPU_SG_VMEM, 2);
+    }
+  }
+#undef RPU_SG
+#undef RPU_SG_MFMA
+#undef RPU_SG_VMEM
+#undef RPU_SG_DSR
+#undef RPU_SG_DSW
+  __builtin_amdgcn_sched_barrier(0);
+}
+
+// WMODE = how the weight operand is addressed:
+//   0  contraction index contiguous (forward), rows 16-byte aligned, K a multiple of 16
+//   1  output index contiguous (backward: W is read transposed in place)
+//   2  contraction index contiguous, any row length and alignment (a tile with a bias column has an odd row
+//      length): 16-byte loads from 4-byte aligned addresses, the last 1 .. 3 elements of a row one by one
+// Operand tiles with a contiguous contraction index (the quantized inputs always, the weights in modes 0, 2) are
+// fetched with unit-stride 16-byte loads, 8 lanes per 128-byte row segment, staged in a wave-private LDS
+// tile and read back in the MFMA operand layout (lane (r, h) holds row r, k = 16 h .. 16 h + 15).  Reading
+// them straight into that layout would make every lane of a load touch a different cache line, which is
+// address-bound in the vector L1.  Mode 1 reads the weights directly: 32 consecutive outputs per half-wave
+// and k are one line.  Out-of-range rows / k are clamped to valid addresses: their products meet the zero
+// padding of the quantized inputs or are never stored.
+// PD = 2, 4: software pipeline with the global loads of PD steps in flight, k_pad a multiple of
+// PD * KSTEP * WAVES; PD = 1: one register set, for short contractions, k_pad a multiple of KSTEP.
+// DUAL (round 0 only, PD = 2): the same weights also multiply the rows that round 1 would use (written by the init
+// kernel into the other scratch matrix), into a second accumulator; both rounds go through the ADC stage, round r
+// into a.dual.buf[r], with their own saturation marks.  Which of the two is a sample's output is decided when its
+// tile is finished (mvm_tile_finished_dual) and copied out at the start of the next launch.
+template <int PD, int WMODE, bool DUAL = false>
+__device__ __forceinline__ void mvm_round_tile(const MvmArgs &a, int round, int tile_o, int tile_b, int n_act,
+                                               float (*red)[16][64], float *stage) {
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int r = lane & 31;
+  const int h = lane >> 5;
+
+  // operand rows owned by this lane in the MFMA layout
+  const int o_in = tile_o * TILE + r;
+  const bool o_ok = o_in < a.O;
+  const int slot_in = tile_b * TILE + r;
+  const bool b_ok = slot_in < n_act;
+
+  const long w_so = a.transposed ? 1 : a.x_size;
+  const long w_sk = a.transposed ? a.x_size : 1;
+  const int K = a.K;
+  // steps of 32 k-values, dealt to the waves in contiguous parts (equal parts, a multiple of PD, when PD >= 2;
+  // a short contraction may leave the last waves without a step)
+  const int steps = a.k_pad / KSTEP;
+  const int per_wave = (steps + WAVES - 1) / WAVES;
+  const int s_begin = min(wave * per_wave, steps);
+  const int s_end = min(s_begin + per_wave, steps);
+
+  float *stage_x = stage + wave * ((DUAL ? 3 : 2) * TILE * LDS_ROW);
+  float *stage_w = stage_x + TILE * LDS_ROW;
+  float *stage_x1 = stage_w + TILE * LDS_ROW; // DUAL only
+
+  // staging layout of this lane: pass t covers rows 8 t .. 8 t + 7, lane = (row in pass) * 8 + 16-byte chunk
+  const int st_row = lane >> 3;
+  const int st_chunk = (lane & 7) * 4;
+  const float *xq = pick2(a.xq, round & 1);
+  const float *x_src[4];
+  const float *x1_src[4];
+  const float *w_src[4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    const int row = t * 8 + st_row;
+    const int slot = min(tile_b * TILE + row, n_act - 1);
+    const int xrow = (round > 0) ? pick2(a.st.row, round & 1)[slot] : slot;
+    x_src[t] = xq + (long)xrow * a.k_pad + st_chunk;
+    x1_src[t] = DUAL ? a.xq[1] + (long)xrow * a.k_pad + st_chunk : nullptr;
+    const int o = min(tile_o * TILE + row, a.O - 1);
+    w_src[t] = a.w + (long)o * a.x_size;
+  }
+  const float *w_col = a.w + (long)(o_ok ? o_in : a.O - 1) * w_so; // mode 1: this lane's output column
+
+  floatx16 acc, acc1;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    acc[i] = 0.0f;
+    acc1[i] = 0.0f;
+  }
+
+  // sample of this lane's output column and its output factor: fetched now, used by the ADC stage
+  int b_out = slot_in;
+  float fin_out = 1.0f;
+  if (!a.io.perfect && b_ok) {
+    if (round > 0) b_out = pick2(a.st.list, round & 1)[slot_in];
+    fin_out = a.st.fin[b_out];
+  }
+
+  auto gload = [&](int s, f32x4 (&gx)[4], f32x4 (&gw)[4], float (&wd)[16], f32x4 (&gx1)[4]) {
+    const int k0 = s * KSTEP;
+#pragma unroll
+    for (int t = 0; t < 4; ++t) gx[t] = *reinterpret_cast<const f32x4 *>(x_src[t] + k0);
+    if constexpr (DUAL) {
+#pragma unroll
+      for (int t = 0; t < 4; ++t) gx1[t] = *reinterpret_cast<const f32x4 *>(x1_src[t] + k0);
+    }
+    if (WMODE == 0) {
+      const int kc = min(k0 + st_chunk, K - 4); // K % 16 == 0: past K the inputs are zero padding
+#pragma unroll
+      for (int t = 0; t < 4; ++t) gw[t] = *reinterpret_cast<const f32x4 *>(w_src[t] + kc);
+    } else if (WMODE == 1) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int kc = min(k0 + h * 16 + i, K - 1);
+        wd[i] = w_col[(long)kc * w_sk];
+      }
+    } else {
+      const int kc = k0 + st_chunk;
+      if (kc + 4 <= K) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) gw[t] = *reinterpret_cast<const f32x4_unaligned *>(w_src[t] + kc);
+      } else { // the end of a row: nothing is read past it
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          f32x4 z;
+          z.x = (kc < K) ? w_src[t][kc] : 0.0f;
+          z.y = (kc + 1 < K) ? w_src[t][kc + 1] : 0.0f;
+          z.z = (kc + 2 < K) ? w_src[t][kc + 2] : 0.0f;
+          z.w = 0.0f;
+          gw[t] = z;
+        }
+      }
+    }
+  };
+  auto lds_store = [&](const f32x4 (&gx)[4], const f32x4 (&gw)[4], const f32x4 (&gx1)[4]) {
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      const int off = (t * 8 + st_row) * LDS_ROW + st_chunk;
+      *reinterpret_cast<f32x4 *>(stage_x + off) = gx[t];
+      if (WMODE != 1) *reinterpret_cast<f32x4 *>(stage_w + off) = gw[t];
+      if constexpr (DUAL) *reinterpret_cast<f32x4 *>(stage_x1 + off) = gx1[t];
+    }
+  };
+  auto lds_read = [&](float (&xd)[16], float (&wd)[16], float (&xd1)[16]) {
+#pragma unroll
+    for (int v4 = 0; v4 < 4; ++v4) {
+      const int off = r * LDS_ROW + h * 16 + v4 * 4;
+      const f32x4 tx = *reinterpret_cast<const f32x4 *>(stage_x + off);
+      xd[v4 * 4 + 0] = tx.x; xd[v4 * 4 + 1] = tx.y; xd[v4 * 4 + 2] = tx.z; xd[v4 * 4 + 3] = tx.w;
+      if constexpr (DUAL) {
+        const f32x4 t1 = *reinterpret_cast<const f32x4 *>(stage_x1 + off);
+        xd1[v4 * 4 + 0] = t1.x; xd1[v4 * 4 + 1] = t1.y; xd1[v4 * 4 + 2] = t1.z; xd1[v4 * 4 + 3] = t1.w;
+      }
+      if (WMODE != 1) {
+        const f32x4 tw = *reinterpret_cast<const f32x4 *>(stage_w + off);
+        wd[v4 * 4 + 0] = tw.x; wd[v4 * 4 + 1] = tw.y; wd[v4 * 4 + 2] = tw.z; wd[v4 * 4 + 3] = tw.w;
+      }
+    }
+  };
+  auto mfma16 = [&](const float (&wd)[16], const float (&xd)[16], const float (&xd1)[16]) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(wd[i], xd[i], acc, 0, 0, 0);
+      if constexpr (DUAL) acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(wd[i], xd1[i], acc1, 0, 0, 0);
+    }
+  };
+
+  if constexpr (PD >= 2) {
+    // PD register sets hold the global loads of the next PD steps; the operand registers are double
+    // buffered, so the LDS round trip of step t + 1 and the loads of step t + 1 + PD are issued ahead
+    // of the 16 MFMAs of step t and complete underneath them.
+    f32x4 gx0[4], gw0[4], gx1[4], gw1[4], gx2[4], gw2[4], gx3[4], gw3[4];
+    f32x4 hx0[4], hx1[4], hx2[4], hx3[4]; // DUAL: the rows of round 1
+    float wr0[16], wr1[16], wr2[16], wr3[16];
+    float xc0[16], wc0[16], xc1[16], wc1[16];
+    float yc0[16], yc1[16]; // DUAL: operands of round 1
+    // step T runs from the operand registers (XC, WC); step T + 1 moves from register set (GX, GW, WR)
+    // through LDS into (XN, WN) and the set is refilled with step T + 1 + PD
+#define RPU_MVM_STEP(T, GX, GW, WR, HX, XC, WC, YC, XN, WN, YN)          \
+  {                                                                      \
+    lds_store(GX, GW, HX);                                               \
+    if (WMODE == 1) {                                                    \
+      _Pragma("unroll") for (int i = 0; i < 16; ++i) WN[i] = WR[i];      \
+    }                                                                    \
+    gload(min((T) + 1 + PD, s_end - 1), GX, GW, WR, HX);                 \
+    lds_read(XN, WN, YN);                                                \
+    mfma16(WC, XC, YC);                                                  \
+    mvm_step_schedule<WMODE, DUAL>();                                    \
+  }
+    gload(s_begin, gx0, gw0, wr0, hx0);
+    gload(min(s_begin + 1, s_end - 1), gx1, gw1, wr1, hx1);
+    if constexpr (PD == 4) {
+      gload(min(s_begin + 2, s_end - 1), gx2, gw2, wr2, hx2);
+      gload(min(s_begin + 3, s_end - 1), gx3, gw3, wr3, hx3);
+    }
+    lds_store(gx0, gw0, hx0);
+    lds_read(xc0, wc0, yc0);
+    if (WMODE == 1) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) wc0[i] = wr0[i];
+    }
+    gload(min(s_begin + PD, s_end - 1), gx0, gw0, wr0, hx0);
+    for (int s = s_begin; s < s_end; s += PD) {
+      if constexpr (PD == 4) {
+        RPU_MVM_STEP(s, gx1, gw1, wr1, hx1, xc0, wc0, yc0, xc1, wc1, yc1)
+        RPU_MVM_STEP(s + 1, gx2, gw2, wr2, hx2, xc1, wc1, yc1, xc0, wc0, yc0)
+        RPU_MVM_STEP(s + 2, gx3, gw3, wr3, hx3, xc0, wc0, yc0, xc1, wc1, yc1)
+        RPU_MVM_STEP(s + 3, gx0, gw0, wr0, hx0, xc1, wc1, yc1, xc0, wc0, yc0)
+      } else {
+        RPU_MVM_STEP(s, gx1, gw1, wr1, hx1, xc0, wc0, yc0, xc1, wc1, yc1)
+        RPU_MVM_STEP(s + 1, gx0, gw0, wr0, hx0, xc1, wc1, yc1, xc0, wc0, yc0)
+      }
+    }
+#undef RPU_MVM_STEP
+  } else {
+    f32x4 gx[4], gw[4], hx[4];
+    float wn[16], xc[16], wc[16], yc[16];
+    if (s_begin < s_end) gload(s_begin, gx, gw, wn, hx);
+    for (int s = s_begin; s < s_end; ++s) {
+      lds_store(gx, gw, hx);
+      lds_read(xc, wc, yc);
+      if (WMODE == 1) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) wc[i] = wn[i];
+      }
+      gload(min(s + 1, s_end - 1), gx, gw, wn, hx);
+      mfma16(wc, xc, yc);
+    }
+  }
+
+  // sum the four parts of the contraction in a fixed order
+#pragma unroll
+  for (int i = 0; i < 16; ++i) red[wave][i][lane] = acc[i];
+  __syncthreads();
+
+  // this wave finishes accumulator group `wave`: rows wave*8 + h*4 + m, column r
+  float v[4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const int i = wave * 4 + q;
+    v[q] = ((red[0][i][lane] + red[1][i][lane]) + red[2][i][lane]) + red[3][i][lane];
+  }
+  const int o0 = tile_o * TILE + wave * 8 + h * 4;
+  int up = 0, lo = 0;
+  if (b_ok && o0 < a.O) {
+    const float *pre = nullptr, *post = nullptr;
+    if (a.pre_add) {
+      const int xrow = (round > 0) ? pick2(a.st.row, round & 1)[slot_in] : slot_in;
+      pre = a.pre_add + (long)xrow * a.O;
+      if (a.post_add) post = a.post_add + (long)xrow * a.O;
+    }
+    mvm_finish_outputs(a, round, b_out, fin_out, o0, v, up, lo, pre, post, DUAL ? a.dual.buf[0] : nullptr);
+  }
+  int up1 = 0, lo1 = 0;
+  if constexpr (DUAL) {
+    __syncthreads(); // the partial sums of round 0 have been read
+#pragma unroll
+    for (int i = 0; i < 16; ++i) red[wave][i][lane] = acc1[i];
+    __syncthreads();
+    float v1[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int i = wave * 4 + q;
+      v1[q] = ((red[0][i][lane] + red[1][i][lane]) + red[2][i][lane]) + red[3][i][lane];
+    }
+    if (b_ok && o0 < a.O) {
+      // scale and output factor of round 1, as the sample's state will hold them if it gets there
+      float nm = a.st.nm[b_out], rd = a.st.red[b_out], fin1;
+      if (next_round_params(a, 0, b_out, fin_out, nm, rd)) {
+        round_scales(a, nm, rd, fin1);
+        mvm_finish_outputs(a, 1, b_out, fin1, o0, v1, up1, lo1, nullptr, nullptr, a.dual.buf[1]);
+      }
+    }
+  }
+  if (!a.io.perfect && a.io.bound_management != RPU_BM_NONE) {
+    // saturation flags of the tile's 32 samples: combined in LDS, then one device-scope atomic per sample
+    // and bound.  The returned values are consumed so that the wave waits until the atomics have been
+    // performed before the workgroup signals its tile as finished (mvm_tile_finished).
+    int *hits = reinterpret_cast<int *>(&red[0][0][0]); // the partial sums have been consumed ...
+    __syncthreads();                                      // ... by every wave
+    if (threadIdx.x < 2 * TILE) hits[threadIdx.x] = 0;
+    __syncthreads();
+    if (up) atomicMax(&hits[r], up);
+    if (lo) atomicMax(&hits[TILE + r], lo);
+    __syncthreads();
+    if (threadIdx.x < 2 * TILE) {
+      const int t = threadIdx.x & (TILE - 1);
+      const int hit = hits[threadIdx.x];
+      const int slot = tile_b * TILE + t;
+      if (hit && slot < n_act) {
+        const int bs = (round > 0) ? pick2(a.st.list, round & 1)[slot] : slot;
+        const int old = atomicMax(threadIdx.x < TILE ? &a.st.hit_up[bs] : &a.st.hit_lo[bs], hit);
+        asm volatile("" ::"v"(old));
+      }
+    }
+    if constexpr (DUAL) { // the marks of round 1 (round 0 of a fused launch lists sample b at position b)
+      __syncthreads();
+      if (threadIdx.x < 2 * TILE) hits[threadIdx.x] = 0;
+      __syncthreads();
+      if (up1) atomicMax(&hits[r], up1);
+      if (lo1) atomicMax(&hits[TILE + r], lo1);
+      __syncthreads();
+      if (threadIdx.x < 2 * TILE) {
+        const int t = threadIdx.x & (TILE - 1);
+        const int hit = hits[threadIdx.x];
+        const int slot = tile_b * TILE + t;
+        if (hit && slot < n_act) {
+          const int old = atomicMax(&a.dual.hit1[(threadIdx.x < TILE ? 0 : a.m_batch) + slot], hit);
+          asm volatile("" ::"v"(old));
+        }
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// per-sample noise management and state of round 0.  One workgroup per sample.
+// rpu_forward_backward_pass.cpp:112-178 (scales), :919-969 (forward), :1003-1022 (backward)
+
+// Reductions over the SUB threads that share a sample: SUB = 256 is the whole workgroup (through LDS), smaller
+// values are aligned lane groups of a wave (shuffles).  Every thread of the group gets the result.
+template <int SUB>
+__device__ __forceinline__ float group_max(float v, float *sh) {
+  if constexpr (SUB == 256) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off));
+    if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = v;
+    __syncthreads();
+    const float r = fmaxf(fmaxf(sh[0], sh[1]), fmaxf(sh[2], sh[3]));
+    __syncthreads();
+    return r;
+  } else {
+#pragma unroll
+    for (int off = SUB / 2; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off));
+    return v;
+  }
+}
+
+template <int SUB>
+__device__ __forceinline__ float group_sum(float v, float *sh) {
+  if constexpr (SUB == 256) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
+    if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = v;
+    __syncthreads();
+    const float r = ((sh[0] + sh[1]) + sh[2]) + sh[3];
+    __syncthreads();
+    return r;
+  } else {
+#pragma unroll
+    for (int off = SUB / 2; off > 0; off >>= 1) v += __shfl_xor(v, off);
+    return v;
+  }
 }
 
 // State of round 0 and quantized input row of sample b, by the SUB threads that share the sample (this one is
@@ -707,6 +787,9 @@ __global__ __launch_bounds__(256) void k_mvm_init(MvmArgs a) {
 // into the other scratch matrix at the rows of this round's list positions.  Whether a sample needs that
 // round is only known when all of its outputs are done; writing the rows ahead costs a few elements per
 // thread and takes the re-quantization off the path between two rounds.
+// FUSED: called by the fused launch of rounds 0 and 1 for the rows of round 2 (as `round` = 1 with every sample
+// listed at its own number); the scale is derived from the sample's state of round 0 and the rows go to a.dual.xq2.
+template <bool FUSED = false>
 __device__ __forceinline__ void mvm_prepare_next_rows(const MvmArgs &a, int round, int tile_o, int tile_b, int n_act) {
   __shared__ float sh_next_scale[TILE];
   __shared__ int sh_next_b[TILE];
@@ -715,8 +798,17 @@ __device__ __forceinline__ void mvm_prepare_next_rows(const MvmArgs &a, int roun
     int b = 0;
     float scale = 0.0f; // 0: the sample can have no further round
     if (slot < n_act) {
-      b = (round > 0) ? pick2(a.st.list, round & 1)[slot] : slot;
-      scale = pick2(a.st.next_scale, round & 1)[slot];
+      if constexpr (FUSED) {
+        b = slot;
+        float nm = a.st.nm[b], red = a.st.red[b], fin = a.st.fin[b];
+        if (next_round_params(a, 0, b, fin, nm, red)) {
+          round_scales(a, nm, red, fin);
+          scale = next_round_scale(a, 1, b, fin, nm, red);
+        }
+      } else {
+        b = (round > 0) ? pick2(a.st.list, round & 1)[slot] : slot;
+        scale = pick2(a.st.next_scale, round & 1)[slot];
+      }
     }
     sh_next_b[threadIdx.x] = b;
     sh_next_scale[threadIdx.x] = scale;
@@ -726,7 +818,7 @@ __device__ __forceinline__ void mvm_prepare_next_rows(const MvmArgs &a, int roun
   const int chunk = (a.k_pad + tiles_o - 1) / tiles_o;
   const int k_lo = tile_o * chunk;
   const int k_hi = min(k_lo + chunk, a.k_pad);
-  float *__restrict__ dst = pick2(a.xq, (round + 1) & 1);
+  float *__restrict__ dst = FUSED ? a.dual.xq2 : pick2(a.xq, (round + 1) & 1);
   const float *__restrict__ in = a.in;
   // a trip covers 32 k-values of all 32 rows: 8 thread-rows x 4 rows each.  The loads of four trips are issued
   // together: a narrow tile has few workgroups per sample tile and each walks a long piece of the rows.
@@ -840,6 +932,79 @@ __device__ __forceinline__ void mvm_tile_finished(const MvmArgs &a, int round, i
   }
 }
 
+// The fused launch of rounds 0 and 1: the last workgroup of a sample tile decides for its 32 samples which result
+// stands (rpu_forward_backward_pass.cpp:944-983 walked twice): round 0 unless its ADC saturated and the reduction may
+// still grow, else round 1, unless that saturated too and may go on -- then the sample is listed for round 2, whose
+// rows the workgroups of this launch have written ahead (into a.dual.xq2: round 0's rows are still being read).
+__device__ __forceinline__ void mvm_tile_finished_dual(const MvmArgs &a, int tile_b) {
+  __shared__ int sh_last;
+  const int tiles_o = (a.O + TILE - 1) / TILE;
+  __syncthreads(); // all flag atomics of this workgroup have been performed
+  if (threadIdx.x == 0) {
+    const int prev = atomicAdd(&a.st.tile_done[tile_b], 1);
+    sh_last = (prev == tiles_o - 1) ? 1 : 0;
+  }
+  __syncthreads();
+  if (!sh_last) return;
+  const IoDev &io = a.io;
+  if (threadIdx.x < TILE) {
+    const int b = tile_b * TILE + threadIdx.x;
+    if (b < a.m_batch) {
+      const int up0 = atomicExch(&a.st.hit_up[b], 0), lo0 = atomicExch(&a.st.hit_lo[b], 0);
+      const int up1 = atomicExch(&a.dual.hit1[b], 0), lo1 = atomicExch(&a.dual.hit1[a.m_batch + b], 0);
+      int sel = 0;
+      const bool failed0 = io.bm_test_negative_bound ? (up0 > 0 || lo0 > 0) : (up0 > lo0);
+      float nm = a.st.nm[b], red = a.st.red[b];
+      if (failed0 && next_round_params(a, 0, b, a.st.fin[b], nm, red)) {
+        // the sample has run round 1
+        sel = 1;
+        atomicAdd(&a.st.count[1], 1); // how many did: read by the host for its choice of launches
+        a.st.rounds[b] += 1;
+        set_round_scales(a, b, nm, red);
+        const bool failed1 = io.bm_test_negative_bound ? (up1 > 0 || lo1 > 0) : (up1 > lo1);
+        if (failed1 && next_round_params(a, 1, b, a.st.fin[b], nm, red)) {
+          sel = 2;
+          a.st.rounds[b] += 1;
+          set_round_scales(a, b, nm, red);
+          const int pos = atomicAdd(&a.st.count[2], 1);
+          a.st.list[0][pos] = b;
+          a.st.row[0][pos] = b; // written ahead at the sample's own row
+          a.st.next_scale[0][pos] = next_round_scale(a, 2, b, a.st.fin[b], nm, red);
+        }
+        a.st.nm[b] = nm;
+        a.st.red[b] = red;
+      }
+      a.dual.sel[b] = sel;
+    }
+  }
+}
+
+// At the start of the launch after the fused one: workgroup n copies the 32 x 32 block of outputs it would own in a
+// round over all samples from the kept results to the caller's output, per sample by a.dual.sel (samples listed for
+// this round are written by it).
+__device__ __forceinline__ void mvm_dual_select(const MvmArgs &a, int n) {
+  int tile_o, tile_b;
+  if (!tile_of(a, n, a.m_batch, tile_o, tile_b)) return;
+  for (int idx = threadIdx.x; idx < TILE * TILE; idx += blockDim.x) {
+    const int b = tile_b * TILE + (idx >> 5), o = tile_o * TILE + (idx & 31);
+    if (b < a.m_batch && o < a.O) {
+      const int sel = a.dual.sel[b];
+      if (sel < 2) a.out[(long)b * a.out_sb + (long)o * a.out_so] = pick2(a.dual.buf, sel)[(long)b * a.O + o];
+    }
+  }
+}
+
+template <int WMODE>
+__global__ __launch_bounds__(256) void k_mvm_dual(MvmArgs a) {
+  __shared__ float red[WAVES][16][64];
+  __shared__ __attribute__((aligned(16))) float stage[WAVES * 3 * TILE * LDS_ROW];
+  int tile_o, tile_b;
+  if (!tile_of(a, blockIdx.x, a.m_batch, tile_o, tile_b)) return;
+  mvm_prepare_next_rows<true>(a, 1, tile_o, tile_b, a.m_batch);
+  mvm_round_tile<2, WMODE, true>(a, 0, tile_o, tile_b, a.m_batch, red, stage);
+  mvm_tile_finished_dual(a, tile_b);
+}
+
 // work of workgroup number n of a round launch of one tile
 template <int PD, int WMODE>
 __device__ __forceinline__ void mvm_round_workgroup(const MvmArgs &a, int round, int n, int n_act, float (*red)[16][64],
@@ -919,7 +1084,13 @@ __global__ __launch_bounds__(256) void k_mvm_round(MvmArgs a) {
   __shared__ float red[WAVES][16][64];
   __shared__ __attribute__((aligned(16))) float stage[WAVES * 2 * TILE * LDS_ROW];
   if (a.skip_if_zero && *a.skip_if_zero == 0) return;
+  if (a.dual.on == 2) mvm_dual_select(a, blockIdx.x);
   const int n_act = (a.round > 0) ? a.st.count[a.round] : a.m_batch;
+  // how many samples needed a second round: the host reads it (whenever it next looks) to choose its launches
+  if (a.dual.seen && blockIdx.x == 0 && threadIdx.x == 0 && (a.round == 1 || a.dual.on == 2)) {
+    a.dual.seen[0] = a.st.count[1];
+    a.dual.seen[1] = a.m_batch;
+  }
   if (runs_on_large_tiles(a, a.round, n_act)) return;
   mvm_round_workgroup<PD, WMODE>(a, a.round, blockIdx.x, n_act, red, stage);
 }
@@ -1771,6 +1942,25 @@ void launch_mvm_round_group(const MvmGroup &g, int depth, int mode, int total_wo
     else RPU_LAUNCH_ROUND(1, 2);
   }
 #undef RPU_LAUNCH_ROUND
+}
+
+// whether rounds 0 and 1 of this call can run as one launch (the caller decides whether they should)
+bool mvm_can_fuse_rounds(const MvmArgs &a) {
+  if (a.io.perfect || a.io.bound_management == RPU_BM_NONE || a.max_rounds < 3 || a.transposed) return false;
+  if (a.pre_add || a.skip_if_zero || a.nm_phase || !a.speculate || !a.rows_ahead_in_init) return false;
+  if (!a.small_tiles_only && big_threshold(a.m_batch, a.O) > 0) return false;
+  if (mvm_round_workgroups(a) > TAIL_GRID) return false;
+  return mvm_prefetch_depth(a.K, a.k_pad) >= 2 && weight_mode(a) != 1;
+}
+
+void launch_mvm_dual(const MvmArgs &a_in, hipStream_t s) {
+  MvmArgs a = a_in;
+  a.big_from = 0;
+  a.round = 0;
+  a.dual.on = 1;
+  const dim3 grid(mvm_round_workgroups(a));
+  if (weight_mode(a) == 0) hipLaunchKernelGGL(k_mvm_dual<0>, grid, dim3(256), 0, s, a);
+  else hipLaunchKernelGGL(k_mvm_dual<2>, grid, dim3(256), 0, s, a);
 }
 
 void launch_mvm_round(const MvmArgs &a_in, hipStream_t s) {

@@ -173,6 +173,13 @@ struct Tile {
   DevBuf<float> d_w, d_wmax, d_wmin, d_sup, d_sdown, d_slup, d_sldown;
   // MVM scratch
   DevBuf<float> s_nsc0, s_nsc1, s_nm, s_nmnp, s_red, s_scale, s_fin, s_bias, s_xq0, s_xq1;
+  // rounds 0 and 1 of a forward call in one launch: kept outputs of both, choice per sample, marks of round 1, rows of
+  // round 2; the host-visible pair (samples of the last call that needed round 1, its batch) that the choice between
+  // the fused and the separate launches is made from (fused_rounds: -1 by that pair, 0 never, 1 whenever possible)
+  DevBuf<float> s_dual0, s_dual1, s_xq2;
+  DevBuf<int> s_dsel, s_dhit1;
+  int *seen_host = nullptr, *seen_dev = nullptr;
+  int fused_rounds = -1;
   DevBuf<int> s_rounds, s_hitup, s_hitlo, s_list0, s_list1, s_row0, s_row1, s_count, s_tiledone;
   // update scratch
   DevBuf<int> u_bl;
@@ -304,6 +311,11 @@ struct Tile {
   void release_all() {
     d_w.release(); d_wmax.release(); d_wmin.release(); d_sup.release(); d_sdown.release();
     d_slup.release(); d_sldown.release();
+    s_dual0.release(); s_dual1.release(); s_xq2.release(); s_dsel.release(); s_dhit1.release();
+    if (seen_host) {
+      (void)hipHostFree(seen_host);
+      seen_host = seen_dev = nullptr;
+    }
     s_nsc0.release(); s_nsc1.release(); s_nm.release(); s_nmnp.release(); s_red.release(); s_scale.release(); s_fin.release(); s_bias.release(); s_xq0.release(); s_xq1.release();
     s_rounds.release(); s_hitup.release(); s_hitlo.release(); s_list0.release(); s_list1.release(); s_row0.release(); s_row1.release(); s_count.release(); s_tiledone.release();
     u_bl.release(); u_a.release(); u_b.release(); u_xval.release(); u_dval.release(); u_xw.release(); u_dw.release();
@@ -689,15 +701,50 @@ struct Tile {
         launch_nm_running_average(a.st.nm, B, io.p.nm_decay, nm_aux.p, s);
         a.nm_phase = 2;
       }
+      // Where most samples need a second round (as the last call on this tile showed), rounds 0 and 1 run as one
+      // launch: one chain of latencies instead of two.  Results are the same either way.
+      bool fuse = false;
+      if (!transposed && !w_other && !side && io.p.bound_management != RPU_BM_NONE && fused_rounds != 0) {
+        if (!seen_host) {
+          RPU_HIP_CHECK(hipHostMalloc((void **)&seen_host, 2 * sizeof(int), hipHostMallocMapped));
+          seen_host[0] = seen_host[1] = 0;
+          RPU_HIP_CHECK(hipHostGetDevicePointer((void **)&seen_dev, seen_host, 0));
+        }
+        a.dual.seen = seen_dev;
+        const int needed = *(volatile int *)&seen_host[0], of = *(volatile int *)&seen_host[1];
+        fuse = mvm_can_fuse_rounds(a) && (fused_rounds == 1 || (of > 0 && 2 * (long)needed > of));
+      }
+      if (fuse) {
+        s_dual0.ensure((size_t)B * a.O); s_dual1.ensure((size_t)B * a.O); s_xq2.ensure((size_t)B * a.k_pad);
+        s_dsel.ensure((size_t)B);
+        if (s_dhit1.n < 2 * (size_t)B) {
+          s_dhit1.ensure(2 * (size_t)B);
+          RPU_HIP_CHECK(hipMemset(s_dhit1.p, 0, s_dhit1.n * sizeof(int))); // cleared by every call after use
+        }
+        a.dual.buf[0] = s_dual0.p; a.dual.buf[1] = s_dual1.p; a.dual.sel = s_dsel.p; a.dual.hit1 = s_dhit1.p;
+        a.dual.xq2 = s_xq2.p;
+      }
       launch_mvm_init(a, s);
       prof_mark(s, "mvm_init");
       // every round after the first works on the samples whose ADC saturated in the one before; the
       // last workgroup to finish a sample tile sets up the next round for that tile
-      for (int r = 0; r < a.max_rounds; ++r) {
-        a.round = r;
-        if (side) pre_adc_terms(a, io, s);
-        launch_mvm_round(a, s);
+      if (fuse) {
+        launch_mvm_dual(a, s);
         prof_mark(s, "mvm_round");
+        a.xq[0] = s_xq2.p; // the fused launch wrote the rows of round 2 there, at each sample's own row
+        for (int r = 2; r < a.max_rounds; ++r) {
+          a.round = r;
+          a.dual.on = r == 2 ? 2 : 0;
+          launch_mvm_round(a, s);
+          prof_mark(s, "mvm_round");
+        }
+      } else {
+        for (int r = 0; r < a.max_rounds; ++r) {
+          a.round = r;
+          if (side) pre_adc_terms(a, io, s);
+          launch_mvm_round(a, s);
+          prof_mark(s, "mvm_round");
+        }
       }
     }
     if (transposed && bias) launch_drop_bias(s_bias.p, final_out, B, X, out_trans ? 1 : 0, s);
@@ -2214,6 +2261,7 @@ int rpu_tile_clone(rpu_tile_t **out, const rpu_tile_t *src_c) {
     t.update_calls = s.update_calls;
     t.update_variant = s.update_variant;
     t.update_variant_samples = s.update_variant_samples;
+    t.fused_rounds = s.fused_rounds;
     if (s.is_transfer()) {
       t.tr = std::make_unique<TransferPar>(*s.tr);
       t.update_idx = s.update_idx;
@@ -2644,6 +2692,15 @@ int rpu_tile_get_update_words(rpu_tile_t *tile, uint32_t *x_words_host, uint32_t
     RPU_HIP_CHECK(hipMemcpy(x_words_host, t.last_xw, rows * t.X * 4, hipMemcpyDeviceToHost));
     RPU_HIP_CHECK(hipMemcpy(d_words_host, t.last_dw, rows * t.D * 4, hipMemcpyDeviceToHost));
     RPU_HIP_CHECK(hipMemcpy(bl_host, t.last_bl, (size_t)m_batch * 4, hipMemcpyDeviceToHost));
+  });
+}
+
+int rpu_tile_set_fused_rounds(rpu_tile_t *tile, int mode) {
+  return guarded([&] {
+    if (!tile) throw RpuError("null tile");
+    if (mode < -1 || mode > 1) throw RpuError("fused rounds: mode must be -1 (by the last call), 0 (never) or 1 (whenever possible).");
+    std::lock_guard<std::mutex> lock(tile->t.mutex);
+    tile->t.fused_rounds = mode;
   });
 }
 

@@ -509,6 +509,11 @@ class _CudaTileMixin:
         check(lib().rpu_tile_get_update_words(self._h, x_words.data_ptr(), d_words.data_ptr(), bl.data_ptr(), m_batch))
         return x_words, d_words, bl
 
+    def set_fused_rounds(self, mode: int = -1) -> None:
+        """Rounds 0 and 1 of the forward pass with iterative bound management in one launch: -1 the tile decides by
+        what its last call needed, 0 never, 1 whenever the shape allows.  Outputs and round counts do not depend on it."""
+        check(lib().rpu_tile_set_fused_rounds(self._h, int(mode)))
+
     def get_update_words_per_sample(self) -> int:
         """Rows of pulse words per sample of the last stochastic update: ceil(longest possible BL / 31)."""
         n = C.c_int32(0)

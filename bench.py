@@ -309,6 +309,7 @@ def main() -> int:
     update_bytes = bytes_per_device * x_size * d_size + 4.0 * (x_size + d_size) * batch
     k_update_ms = prof_update["update_pulsed"][0]
     k_fwd_ms = prof_forward["mvm_round"][0]   # all round launches of one forward call
+    fused_forward = prof_forward["mvm_round"][1] < 5 and args.config == 2  # rounds 0 and 1 ran as one launch
     k_bwd_ms = prof_backward["mvm_round"][0]
 
     out = {
@@ -328,7 +329,10 @@ def main() -> int:
                    "step": "forward + backward + update"},
         "update": {"ms_per_call": ms_update, "kernels_ms": {k: v[0] for k, v in prof_update.items()}},
         "forward": {"ms_per_call": ms_forward, "gflops": flops_per_call / (ms_forward * 1e-3) / 1e9,
-                    "mean_bm_rounds": float(rounds.mean()), "kernels_ms": {k: v[0] for k, v in prof_forward.items()}},
+                    "mean_bm_rounds": float(rounds.mean()), "kernels_ms": {k: v[0] for k, v in prof_forward.items()},
+                    "round_launches": prof_forward["mvm_round"][1],
+                    "note": "with most samples in a second round the tile runs rounds 0 and 1 as one launch "
+                            "(rpu_tile_set_fused_rounds, default: by what its last call needed); same outputs"},
         "backward": {"ms_per_call": ms_backward, "gflops": flops_per_call / (ms_backward * 1e-3) / 1e9,
                      "kernels_ms": {k: v[0] for k, v in prof_backward.items()}},
         "roofline": {"kernel": "k_update_pulsed", "bound": "hbm", "achieved": update_bytes / (k_update_ms * 1e-3) / 1e9,
@@ -338,12 +342,13 @@ def main() -> int:
                      "traffic_source": ("constant from " + PMC_SOURCE["k_update_pulsed"] + " (rocprofv3 --pmc FETCH_SIZE / "
                                         "WRITE_SIZE), not measured in this run") if args.config == 2 else None,
                      "algorithmic_bytes": update_bytes, "kernel_ms": k_update_ms},
-        "roofline_forward": {"kernel": "k_mvm_round (all rounds of a call)", "bound": "mfma",
+        "roofline_forward": {"kernel": "k_mvm_dual + k_mvm_round (all rounds of a call)" if fused_forward
+                             else "k_mvm_round (all rounds of a call)", "bound": "mfma",
                              "achieved": flops_per_call / (k_fwd_ms * 1e-3) / 1e12, "peak": FP32_MFMA_PEAK_TFLOPS,
                              "unit": "TFLOP/s", "frac": flops_per_call / (k_fwd_ms * 1e-3) / 1e12 / FP32_MFMA_PEAK_TFLOPS,
-                             "traffic": PMC_TRAFFIC_BYTES["k_mvm_round"] if args.config == 2 else None,
+                             "traffic": PMC_TRAFFIC_BYTES["k_mvm_round"] if args.config == 2 and not fused_forward else None,
                              "traffic_source": ("constant from " + PMC_SOURCE["k_mvm_round"] + ", not measured in this run")
-                             if args.config == 2 else None,
+                             if args.config == 2 and not fused_forward else None,
                              "algorithmic_flops": flops_per_call, "kernel_ms": k_fwd_ms},
         "roofline_backward": {"kernel": "k_mvm_round", "bound": "mfma",
                               "achieved": flops_per_call / (k_bwd_ms * 1e-3) / 1e12, "peak": FP32_MFMA_PEAK_TFLOPS,

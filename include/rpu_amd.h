@@ -630,6 +630,15 @@ const char *rpu_tile_extra_name(const rpu_tile_t *tile, int idx);
 int rpu_tile_get_extra(rpu_tile_t *tile, int64_t *values_host);
 int rpu_tile_set_extra(rpu_tile_t *tile, const int64_t *values_host, int count);
 
+/* No counterpart in the reference.  With iterative bound management the forward pass of a batch runs round after
+ * round; where most samples need a second round (the rule when the outputs of a tile are large against out_bound),
+ * rounds 0 and 1 can run as ONE launch that computes both from the same weights and keeps, per sample, the one the
+ * reference's loop would have ended with -- the same outputs, bit for bit, and the same round counts.  By default
+ * (mode -1) a tile chooses by what its last forward call needed (more than half of the samples in a second round:
+ * fused); 0: never, 1: whenever the shape allows it (single tile, batch-first rounds on the 32 x 32 kernel, no
+ * per-line periphery terms). */
+int rpu_tile_set_fused_rounds(rpu_tile_t *tile, int mode);
+
 /* ---- inspection hooks (mirror the reference's debug hooks) ------------------------------ */
 
 /* After rpu_tile_update with a stochastic pulse type: copies the packed pulse words of that call

@@ -1,0 +1,98 @@
+"""Rounds 0 and 1 of the forward pass in one launch (rpu_tile_set_fused_rounds): outputs and round counts must be bit for
+bit those of the separate launches, which the other GPU tests hold against the oracle."""
+import numpy as np
+import pytest
+import torch
+
+from aihwkit_amd.rpu_base import devices as dv
+from aihwkit_amd.rpu_base import tiles
+from helpers import build_pair, config2, config2_data, io_params, make_meta, noise_free_io, soft_bounds
+
+pytestmark = pytest.mark.gpu
+F = np.float32
+NM, BM = dv.NoiseManagementType, dv.BoundManagementType
+
+
+def both_ways(meta, dev, x_size, d_size, w, x, seed=5, bias=False, x_trans=False, d_trans=False, calls=2):
+    host, _orc, _ = build_pair(meta, dev, x_size, d_size, gpu=False)
+    host.set_weights(torch.from_numpy(w))
+    results = []
+    xin = torch.from_numpy(np.ascontiguousarray(x.T if x_trans else x)).cuda()
+    for mode in (0, 1):
+        gpu = tiles.CudaAnalogTile(host)
+        gpu.set_fused_rounds(mode)
+        gpu.set_seed(seed)
+        outs = []
+        for _ in range(calls):                       # the second call reuses every buffer of the first
+            y = gpu.forward(xin, bias, x_trans, d_trans).cpu().numpy()
+            outs.append((y, gpu.get_bm_rounds(x.shape[0]).numpy().copy()))
+        results.append(outs)
+    for (y0, r0), (y1, r1) in zip(*results):
+        assert np.array_equal(r0, r1)
+        assert np.array_equal(y0, y1)
+    return results[0][0]
+
+
+def test_benchmark_configuration_with_noise_is_bit_equal(gpu_device):
+    meta, dev = config2()
+    w, x, _d = config2_data(1024, 1024, 256)
+    y, rounds = both_ways(meta, dev, 1024, 1024, w, x)
+    assert rounds.mean() > 1.9 and np.abs(y).max() > 1.0
+
+
+@pytest.mark.parametrize("bound_management", [BM.Iterative, BM.IterativeWorstCase])
+@pytest.mark.parametrize("shape,bias,trans", [((512, 300, 100), False, False), ((257, 96, 33), True, False),
+                                              ((1024, 256, 64), False, True), ((768, 1000, 256), False, False)])
+def test_shapes_layouts_and_many_rounds(gpu_device, shape, bias, trans, bound_management):
+    """Samples that stop after round 0, after round 1 and later (a small out_bound sends many to rounds 2 .. 4), a zero
+    sample, a bias column (rows that are not 16-byte aligned), transposed layouts, the worst-case switch of the scale."""
+    x_size, d_size, batch = shape
+    rng = np.random.default_rng(x_size)
+    io = io_params(out_noise=0.1, out_bound=3.0, noise_management=NM.AbsMax, bound_management=bound_management)
+    meta = make_meta(io, noise_free_io())
+    dev = soft_bounds(construction_seed=3)
+    w = rng.uniform(-0.3, 0.3, (d_size, x_size)).astype(F)
+    x = rng.uniform(-1, 1, (batch, x_size - (1 if bias else 0))).astype(F)
+    x *= rng.choice([0.02, 0.2, 1.0], (batch, 1)).astype(F)       # with abs-max scaling the rounds follow the weights ...
+    x[:, : x.shape[1] // 2] *= rng.choice([0.05, 1.0], (batch, 1)).astype(F)   # ... and how the input mass is spread
+    x[3] = 0.0
+    y, rounds = both_ways(meta, dev, x_size, d_size, w, x, bias=bias, x_trans=trans, d_trans=trans)
+    if not bias:                                                  # (the bias column keeps a zero sample alive)
+        assert rounds[3] == 0 and not (y.T if trans else y)[3].any()
+    if bound_management == BM.Iterative:
+        assert len(set(rounds.tolist())) >= 2 and (x_size < 512 or rounds.max() >= 3)
+    else:                                                         # the worst-case scale of round 1 always fits
+        assert set(rounds.tolist()) <= {0, 1, 2} and (rounds == 2).any()
+
+
+def test_the_tile_chooses_by_its_last_call(gpu_device):
+    """Default mode: the first call runs the separate launches, later ones the fused launch when most samples needed a
+    second round -- seen here only through equal results and through the kernel that the profile of a call names."""
+    meta, dev = config2()
+    w, x, _d = config2_data(1024, 1024, 256)
+    host, _orc, _ = build_pair(meta, dev, 1024, 1024, gpu=False)
+    host.set_weights(torch.from_numpy(w))
+    ref = tiles.CudaAnalogTile(host)
+    ref.set_fused_rounds(0)
+    auto = tiles.CudaAnalogTile(host)
+    xin = torch.from_numpy(x).cuda()
+    launches = []
+    for call in range(4):
+        for t in (ref, auto):
+            t.set_seed(100 + call)
+        auto.set_profiling(True)
+        y = auto.forward(xin).cpu().numpy()
+        launches.append(sum(1 for name, _ms in auto.get_profile() if name == "mvm_round"))
+        auto.set_profiling(False)
+        assert np.array_equal(y, ref.forward(xin).cpu().numpy())
+    assert launches[0] == 5 and launches[-1] == 4            # one launch less once the tile has seen its rounds
+    quiet = x * np.float32(0.01) + 0                          # nothing saturates ...
+    w_small = (w * 0.05).astype(F)
+    auto.set_weights(torch.from_numpy(w_small))
+    ref.set_weights(torch.from_numpy(w_small))
+    for call in range(3):
+        auto.set_profiling(True)
+        y = auto.forward(torch.from_numpy(quiet).cuda()).cpu().numpy()
+        n = sum(1 for name, _ms in auto.get_profile() if name == "mvm_round")
+        auto.set_profiling(False)
+    assert n == 5                                             # ... and the tile is back on the separate launches
