@@ -80,3 +80,11 @@ def test_update_without_allocation_refuses_what_does_not_fit():
     det.set_update_without_allocation(True)
     with pytest.raises(RuntimeError, match="stochastic pulses"):
         det.update(xg[:8, :40].contiguous(), dg[:8, :30].contiguous(), False, False, False, False)
+    # a bit line beyond 31 pulses needs several rows of words per sample: not in the static array
+    from helpers import make_meta, soft_bounds
+    long_meta = make_meta(desired_bl=64, fixed_bl=True, update_management=False, update_bl_management=False)
+    long_tile = tiles.CudaAnalogTile(long_meta.create_array(40, 30, soft_bounds(construction_seed=1)))
+    long_tile.set_learning_rate(0.01)
+    long_tile.set_update_without_allocation(True)
+    with pytest.raises(RuntimeError, match="at most 31 pulses"):
+        long_tile.update(xg[:8, :40].contiguous(), dg[:8, :30].contiguous(), False, False, False, False)
