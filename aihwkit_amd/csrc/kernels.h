@@ -84,6 +84,7 @@ struct MvmArgs {
   int small_tiles_only;     // 1: never the large-tile kernel (its row padding differs)
   const int *skip_if_zero;  // non-null: a round launch does nothing when this device value is zero
   DualDev dual;
+  int rest_in_one;          // 1: this launch runs round `round` and every round after it (k_mvm_rounds_rest)
 };
 
 // noise management + per-sample state for round 0
@@ -93,6 +94,8 @@ void launch_mvm_round(const MvmArgs &a, hipStream_t s);
 // rounds 0 and 1 in one launch (a.dual filled in); the launches of rounds 2 .. follow with a.dual.on = 2 on the first
 // of them and a.xq[0] = a.dual.xq2
 bool mvm_can_fuse_rounds(const MvmArgs &a);
+// the rounds from a.round on in one launch (a.rest_in_one = 1 for launch_mvm_round): for calls that expect them empty
+bool mvm_can_merge_rest(const MvmArgs &a, int n_cus);
 void launch_mvm_dual(const MvmArgs &a, hipStream_t s);
 // AverageAbsMax noise management (rpu_forward_backward_pass.cpp:138-149): nm[b] holds the largest absolute input of
 // sample b and becomes the running average after that sample, in batch order; aux carries the value between calls

@@ -747,7 +747,7 @@ __device__ __forceinline__ void mvm_init_sample(const MvmArgs &a, int b, int t, 
     a.st.rounds[b] = (fin == 0.0f) ? 0 : 1;
     if (io.bound_management != RPU_BM_NONE) a.st.next_scale[0][b] = next_round_scale(a, 0, b, fin, nm, 1.0f);
   }
-  if (gid < 40) a.st.count[gid] = 0;
+  if (gid < 64) a.st.count[gid] = 0; // count[0 .. 39] per round, count[48 ..] the arrival counters of k_mvm_rounds_rest
   {
     const long n_done = 32L * ((a.m_batch + TILE - 1) / TILE);
     for (long idx = gid; idx < n_done; idx += gstride) a.st.tile_done[idx] = 0;
@@ -1019,6 +1019,24 @@ __device__ __forceinline__ void mvm_round_workgroup(const MvmArgs &a, int round,
   if (more_rounds) mvm_tile_finished(a, round, tile_b, n_act);
 }
 
+// All workgroups of a launch wait for each other, and what they wrote before is visible to all of them after (the
+// launch must fit on the GPU at once).  The wait is bounded: if it ever ran out, the rounds after it would read
+// stale lists.
+constexpr int REST_SPIN_LIMIT = 1 << 28;
+__device__ __forceinline__ void mvm_device_barrier(int *counter, int total) {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    int spins = 0;
+    while (__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < total && ++spins < REST_SPIN_LIMIT) {
+      __builtin_amdgcn_s_sleep(8);
+    }
+  }
+  __syncthreads();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+}
+
 // big_from > 0: the large-tile kernel runs the rounds that list at least that many samples; < 0: it runs round 0
 __device__ __forceinline__ bool runs_on_large_tiles(const MvmArgs &a, int round, int n_act) {
   return (a.big_from > 0 && n_act >= a.big_from) || (a.big_from < 0 && round == 0);
@@ -1076,6 +1094,28 @@ __global__ __launch_bounds__(256) void k_mvm_round_tail_group(MvmGroup g, int ro
     const int n_act = (round > 0) ? a.st.count[round] : a.m_batch;
     mvm_round_workgroup<1, WMODE>(a, round, n - sh_first[t], n_act, red, stage);
     __syncthreads();
+  }
+}
+
+// Every round from a.round on in ONE launch, for calls whose samples are expected to be done by then (as the tile's
+// last call was): the workgroups find the round's list empty and leave, where the separate launches would cost a few
+// microseconds each for nothing.  Where the expectation fails the rounds still run, one after the other with all
+// workgroups waiting for each other in between (mvm_device_barrier: tens of microseconds per round, which is why
+// this launch is only chosen by expectation).
+template <int PD, int WMODE>
+__global__ __launch_bounds__(256) void k_mvm_rounds_rest(MvmArgs a) {
+  __shared__ float red[WAVES][16][64];
+  __shared__ __attribute__((aligned(16))) float stage[WAVES * 2 * TILE * LDS_ROW];
+  for (int r = a.round; r < a.max_rounds; ++r) {
+    const int n_act = __hip_atomic_load(&a.st.count[r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (a.dual.seen && r == 1 && blockIdx.x == 0 && threadIdx.x == 0) {
+      a.dual.seen[0] = n_act;
+      a.dual.seen[1] = a.m_batch;
+    }
+    if (n_act == 0) return; // the same for every workgroup: the count is final since the launch or barrier before
+    mvm_round_workgroup<PD, WMODE>(a, r, blockIdx.x, n_act, red, stage);
+    if (r + 1 == a.max_rounds) return;
+    mvm_device_barrier(&a.st.count[48 + r], (int)gridDim.x);
   }
 }
 
@@ -1953,6 +1993,15 @@ bool mvm_can_fuse_rounds(const MvmArgs &a) {
   return mvm_prefetch_depth(a.K, a.k_pad) >= 2 && weight_mode(a) != 1;
 }
 
+// whether the rounds after round 0 of this call can share one launch (mvm_can_fuse_rounds without the conditions of
+// the two-accumulator kernel; all workgroups must be resident at once: at most one per CU is assumed)
+bool mvm_can_merge_rest(const MvmArgs &a, int n_cus) {
+  if (a.io.perfect || a.io.bound_management == RPU_BM_NONE || a.max_rounds < 3 || a.transposed) return false;
+  if (a.pre_add || a.skip_if_zero || a.nm_phase) return false;
+  if (!a.small_tiles_only && big_threshold(a.m_batch, a.O) > 0) return false;
+  return mvm_round_workgroups(a) <= n_cus && weight_mode(a) != 1;
+}
+
 void launch_mvm_dual(const MvmArgs &a_in, hipStream_t s) {
   MvmArgs a = a_in;
   a.big_from = 0;
@@ -1984,6 +2033,20 @@ void launch_mvm_round(const MvmArgs &a_in, hipStream_t s) {
   }
   const dim3 grid(all);
   const int depth = mvm_prefetch_depth(a.K, a.k_pad);
+  if (a.rest_in_one) {
+#define RPU_LAUNCH_REST(PD, WMODE) hipLaunchKernelGGL((k_mvm_rounds_rest<PD, WMODE>), grid, dim3(256), 0, s, a)
+    if (mode == 0) {
+      if (depth == 4) RPU_LAUNCH_REST(4, 0);
+      else if (depth == 2) RPU_LAUNCH_REST(2, 0);
+      else RPU_LAUNCH_REST(1, 0);
+    } else {
+      if (depth == 4) RPU_LAUNCH_REST(4, 2);
+      else if (depth == 2) RPU_LAUNCH_REST(2, 2);
+      else RPU_LAUNCH_REST(1, 2);
+    }
+#undef RPU_LAUNCH_REST
+    return;
+  }
 #define RPU_LAUNCH_ROUND(PD, WMODE) hipLaunchKernelGGL((k_mvm_round<PD, WMODE>), grid, dim3(256), 0, s, a)
   if (mode == 0) {
     if (depth == 4) RPU_LAUNCH_ROUND(4, 0);

@@ -180,6 +180,15 @@ struct Tile {
   DevBuf<int> s_dsel, s_dhit1;
   int *seen_host = nullptr, *seen_dev = nullptr;
   int fused_rounds = -1;
+  int cu_count = 0;
+  int n_cus() {
+    if (!cu_count) {
+      hipDeviceProp_t prop;
+      RPU_HIP_CHECK(hipGetDeviceProperties(&prop, device_id));
+      cu_count = prop.multiProcessorCount;
+    }
+    return cu_count;
+  }
   DevBuf<int> s_rounds, s_hitup, s_hitlo, s_list0, s_list1, s_row0, s_row1, s_count, s_tiledone;
   // update scratch
   DevBuf<int> u_bl;
@@ -407,6 +416,7 @@ struct Tile {
     if (target >= count) throw RpuError("Invalid HIP device id.");
     DeviceGuard g(target);
     device_id = target;
+    cu_count = 0;
     try {
       if (is_transfer()) {
         for (auto &sl : slots) sl->upload(size(), true);
@@ -703,7 +713,7 @@ struct Tile {
       }
       // Where most samples need a second round (as the last call on this tile showed), rounds 0 and 1 run as one
       // launch: one chain of latencies instead of two.  Results are the same either way.
-      bool fuse = false;
+      bool fuse = false, merge_rest = false;
       if (!transposed && !w_other && !side && io.p.bound_management != RPU_BM_NONE && fused_rounds != 0) {
         if (!seen_host) {
           RPU_HIP_CHECK(hipHostMalloc((void **)&seen_host, 2 * sizeof(int), hipHostMallocMapped));
@@ -712,7 +722,9 @@ struct Tile {
         }
         a.dual.seen = seen_dev;
         const int needed = *(volatile int *)&seen_host[0], of = *(volatile int *)&seen_host[1];
-        fuse = mvm_can_fuse_rounds(a) && (fused_rounds == 1 || (of > 0 && 2 * (long)needed > of));
+        fuse = mvm_can_fuse_rounds(a) && (fused_rounds == 1 || (fused_rounds < 0 && of > 0 && 2 * (long)needed > of));
+        // no sample of the last call needed a second round: the launches after round 0 are expected to find nothing
+        merge_rest = !fuse && mvm_can_merge_rest(a, n_cus()) && (fused_rounds == 2 || (fused_rounds < 0 && of > 0 && needed == 0));
       }
       if (fuse) {
         s_dual0.ensure((size_t)B * a.O); s_dual1.ensure((size_t)B * a.O); s_xq2.ensure((size_t)B * a.k_pad);
@@ -742,8 +754,10 @@ struct Tile {
         for (int r = 0; r < a.max_rounds; ++r) {
           a.round = r;
           if (side) pre_adc_terms(a, io, s);
+          a.rest_in_one = (merge_rest && r == 1) ? 1 : 0;
           launch_mvm_round(a, s);
           prof_mark(s, "mvm_round");
+          if (a.rest_in_one) break;
         }
       }
     }
@@ -2698,7 +2712,10 @@ int rpu_tile_get_update_words(rpu_tile_t *tile, uint32_t *x_words_host, uint32_t
 int rpu_tile_set_fused_rounds(rpu_tile_t *tile, int mode) {
   return guarded([&] {
     if (!tile) throw RpuError("null tile");
-    if (mode < -1 || mode > 1) throw RpuError("fused rounds: mode must be -1 (by the last call), 0 (never) or 1 (whenever possible).");
+    if (mode < -1 || mode > 2) {
+      throw RpuError("fused rounds: mode must be -1 (by the last call), 0 (never), 1 (rounds 0 and 1 in one launch whenever "
+                     "possible) or 2 (the rounds after round 0 in one launch whenever possible).");
+    }
     std::lock_guard<std::mutex> lock(tile->t.mutex);
     tile->t.fused_rounds = mode;
   });

@@ -510,8 +510,9 @@ class _CudaTileMixin:
         return x_words, d_words, bl
 
     def set_fused_rounds(self, mode: int = -1) -> None:
-        """Rounds 0 and 1 of the forward pass with iterative bound management in one launch: -1 the tile decides by
-        what its last call needed, 0 never, 1 whenever the shape allows.  Outputs and round counts do not depend on it."""
+        """Fewer launches for the bound-management rounds of the forward pass: 1 = rounds 0 and 1 in one launch, 2 = all
+        rounds after round 0 in one launch, 0 = one launch per round, -1 (default) = the tile decides by what its last
+        call needed.  Outputs and round counts do not depend on it."""
         check(lib().rpu_tile_set_fused_rounds(self._h, int(mode)))
 
     def get_update_words_per_sample(self) -> int:

@@ -336,8 +336,9 @@ def main() -> int:
         "forward": {"ms_per_call": ms_forward, "gflops": flops_per_call / (ms_forward * 1e-3) / 1e9,
                     "mean_bm_rounds": float(rounds.mean()), "kernels_ms": {k: v[0] for k, v in prof_forward.items()},
                     "round_launches": prof_forward["mvm_round"][1],
-                    "note": "with most samples in a second round the tile runs rounds 0 and 1 as one launch "
-                            "(rpu_tile_set_fused_rounds, default: by what its last call needed); same outputs"},
+                    "note": "with most samples in a second round the tile runs rounds 0 and 1 as one launch, with none "
+                            "the rounds after round 0 as one launch (rpu_tile_set_fused_rounds, default: by what its "
+                            "last call needed); same outputs"},
         "backward": {"ms_per_call": ms_backward, "gflops": flops_per_call / (ms_backward * 1e-3) / 1e9,
                      "kernels_ms": {k: v[0] for k, v in prof_backward.items()}},
         "roofline": {"kernel": "k_update_pulsed", "bound": "hbm", "achieved": update_bytes / (k_update_ms * 1e-3) / 1e9,

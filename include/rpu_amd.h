@@ -631,12 +631,17 @@ int rpu_tile_get_extra(rpu_tile_t *tile, int64_t *values_host);
 int rpu_tile_set_extra(rpu_tile_t *tile, const int64_t *values_host, int count);
 
 /* No counterpart in the reference.  With iterative bound management the forward pass of a batch runs round after
- * round; where most samples need a second round (the rule when the outputs of a tile are large against out_bound),
- * rounds 0 and 1 can run as ONE launch that computes both from the same weights and keeps, per sample, the one the
- * reference's loop would have ended with -- the same outputs, bit for bit, and the same round counts.  By default
- * (mode -1) a tile chooses by what its last forward call needed (more than half of the samples in a second round:
- * fused); 0: never, 1: whenever the shape allows it (single tile, batch-first rounds on the 32 x 32 kernel, no
- * per-line periphery terms). */
+ * round, one launch each, and a launch costs a few microseconds even when its round lists no sample.  Two shortcuts,
+ * both with the same outputs, bit for bit, and the same round counts as the separate launches:
+ *   1  rounds 0 and 1 as ONE launch that computes both from the same weights and keeps, per sample, the one the
+ *      reference's loop would have ended with (pays where most samples need a second round: the outputs of the tile are
+ *      large against out_bound);
+ *   2  every round after round 0 as ONE launch whose workgroups leave when they find the round's list empty (pays where
+ *      no sample needs a second round; where some do, the rounds still run in that launch, with a wait of all
+ *      workgroups between them that costs more than a launch).
+ * Mode -1 (default): the tile chooses by what its last forward call needed -- more than half of the samples in a second
+ * round: 1; none: 2; else the separate launches.  0: always the separate launches.  1 / 2: that shortcut whenever the
+ * shape allows it (single tile, rounds on the 32 x 32 kernel, no per-line periphery terms). */
 int rpu_tile_set_fused_rounds(rpu_tile_t *tile, int mode);
 
 /* ---- inspection hooks (mirror the reference's debug hooks) ------------------------------ */

@@ -1,5 +1,6 @@
-"""Rounds 0 and 1 of the forward pass in one launch (rpu_tile_set_fused_rounds): outputs and round counts must be bit for
-bit those of the separate launches, which the other GPU tests hold against the oracle."""
+"""Fewer launches for the bound-management rounds of the forward pass (rpu_tile_set_fused_rounds): rounds 0 and 1 in one
+launch (mode 1), the rounds after round 0 in one launch (mode 2).  Outputs and round counts must be bit for bit those of
+the separate launches (mode 0), which the other GPU tests hold against the oracle."""
 import numpy as np
 import pytest
 import torch
@@ -18,7 +19,7 @@ def both_ways(meta, dev, x_size, d_size, w, x, seed=5, bias=False, x_trans=False
     host.set_weights(torch.from_numpy(w))
     results = []
     xin = torch.from_numpy(np.ascontiguousarray(x.T if x_trans else x)).cuda()
-    for mode in (0, 1):
+    for mode in (0, 1, 2):
         gpu = tiles.CudaAnalogTile(host)
         gpu.set_fused_rounds(mode)
         gpu.set_seed(seed)
@@ -27,9 +28,10 @@ def both_ways(meta, dev, x_size, d_size, w, x, seed=5, bias=False, x_trans=False
             y = gpu.forward(xin, bias, x_trans, d_trans).cpu().numpy()
             outs.append((y, gpu.get_bm_rounds(x.shape[0]).numpy().copy()))
         results.append(outs)
-    for (y0, r0), (y1, r1) in zip(*results):
-        assert np.array_equal(r0, r1)
-        assert np.array_equal(y0, y1)
+    for other in results[1:]:
+        for (y0, r0), (y1, r1) in zip(results[0], other):
+            assert np.array_equal(r0, r1)
+            assert np.array_equal(y0, y1)
     return results[0][0]
 
 
@@ -67,7 +69,8 @@ def test_shapes_layouts_and_many_rounds(gpu_device, shape, bias, trans, bound_ma
 
 def test_the_tile_chooses_by_its_last_call(gpu_device):
     """Default mode: the first call runs the separate launches, later ones the fused launch when most samples needed a
-    second round -- seen here only through equal results and through the kernel that the profile of a call names."""
+    second round, or round 0 and one launch for the rest when none did -- seen here only through equal results and
+    through the number of round launches in the profile of a call."""
     meta, dev = config2()
     w, x, _d = config2_data(1024, 1024, 256)
     host, _orc, _ = build_pair(meta, dev, 1024, 1024, gpu=False)
@@ -91,8 +94,18 @@ def test_the_tile_chooses_by_its_last_call(gpu_device):
     auto.set_weights(torch.from_numpy(w_small))
     ref.set_weights(torch.from_numpy(w_small))
     for call in range(3):
+        for t in (ref, auto):
+            t.set_seed(200 + call)
         auto.set_profiling(True)
         y = auto.forward(torch.from_numpy(quiet).cuda()).cpu().numpy()
         n = sum(1 for name, _ms in auto.get_profile() if name == "mvm_round")
         auto.set_profiling(False)
-    assert n == 5                                             # ... and the tile is back on the separate launches
+        assert np.array_equal(y, ref.forward(torch.from_numpy(quiet).cuda()).cpu().numpy())
+    assert n == 2                                             # ... and round 0 is followed by one launch for whatever is left
+    auto.set_weights(torch.from_numpy(w))                     # saturation again: that launch runs the rounds it finds
+    ref.set_weights(torch.from_numpy(w))
+    for t in (ref, auto):
+        t.set_seed(77)
+    y = auto.forward(xin).cpu().numpy()
+    assert np.array_equal(y, ref.forward(xin).cpu().numpy())
+    assert np.array_equal(auto.get_bm_rounds(256).numpy(), ref.get_bm_rounds(256).numpy())
