@@ -110,8 +110,13 @@ struct MvmGroup {
   int m_batch;
 };
 void launch_mvm_init_group(const MvmGroup &g, int max_k, hipStream_t s);
+// seen: host-visible pair (any tile lists a sample for round 1, batch) written by the launch of round 1; may be null
 void launch_mvm_round_group(const MvmGroup &g, int prefetch_depth, int weight_mode, int total_workgroups, int round,
-                            hipStream_t s);
+                            hipStream_t s, int *seen = nullptr);
+// the rounds from round_first on in one launch, for calls that expect them to list nothing (see k_mvm_rounds_rest)
+bool mvm_group_can_merge_rest(const MvmGroup &g, int weight_mode);
+void launch_mvm_rest_group(const MvmGroup &g, int weight_mode, int round_first, int rounds, int workgroups, int *seen,
+                           hipStream_t s);
 int mvm_round_workgroups(const MvmArgs &a);            // workgroups of a round launch for this tile
 // Large-tile (128 x 128) variant for round 0 of a group: args[t].big_from < 0 marks the tiles it runs, start[]
 // counts its workgroups (mvm_big_workgroups; 0 for the other tiles).

@@ -1058,15 +1058,33 @@ __global__ __launch_bounds__(256) void k_mvm_round_tail(MvmArgs a) {
   }
 }
 
+// Whether any tile of the group lists a sample for round 1: written to host-visible memory for the host's choice of
+// launches at its next call (seen[0]: 1 / 0, seen[1]: the batch).  Called by the first workgroup of a round-1 launch.
+__device__ __forceinline__ void group_seen_update(const MvmGroup &g, int *seen) {
+  __shared__ int sh_any;
+  if (threadIdx.x == 0) sh_any = 0;
+  __syncthreads();
+  for (int t = threadIdx.x; t < g.n; t += blockDim.x) {
+    const MvmArgs &a = g.args[t];
+    if (a.max_rounds > 1 && __hip_atomic_load(&a.st.count[1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) > 0) sh_any = 1;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    seen[0] = sh_any;
+    seen[1] = g.m_batch;
+  }
+}
+
 // The same for a group: the workgroups first find out, one thread per tile, how many 32 x 32 tiles each member has
 // listed for this round (usually none), then walk the concatenation of those.
 constexpr int MAX_GROUP = 1024;
 
 template <int WMODE>
-__global__ __launch_bounds__(256) void k_mvm_round_tail_group(MvmGroup g, int round) {
+__global__ __launch_bounds__(256) void k_mvm_round_tail_group(MvmGroup g, int round, int *seen) {
   __shared__ float red[WAVES][16][64];
   __shared__ __attribute__((aligned(16))) float stage[WAVES * 2 * TILE * LDS_ROW];
   __shared__ int sh_first[MAX_GROUP + 1]; // first workgroup number of member t; [g.n] = total
+  if (seen && round == 1 && blockIdx.x == 0) group_seen_update(g, seen);
   for (int t = threadIdx.x; t < g.n; t += blockDim.x) {
     const MvmArgs &a = g.args[t];
     int wg = 0;
@@ -1094,6 +1112,50 @@ __global__ __launch_bounds__(256) void k_mvm_round_tail_group(MvmGroup g, int ro
     const int n_act = (round > 0) ? a.st.count[round] : a.m_batch;
     mvm_round_workgroup<1, WMODE>(a, round, n - sh_first[t], n_act, red, stage);
     __syncthreads();
+  }
+}
+
+// The rounds from round_first on of all tiles of a group in one launch (see k_mvm_rounds_rest): a fixed number of
+// workgroups, all resident at once, walk the tiles that the members list for a round; they leave at the first round that
+// lists none.  The arrival counters are those of the group's first tile.
+template <int WMODE>
+__global__ __launch_bounds__(256) void k_mvm_rest_group(MvmGroup g, int round_first, int rounds, int *seen) {
+  __shared__ float red[WAVES][16][64];
+  __shared__ __attribute__((aligned(16))) float stage[WAVES * 2 * TILE * LDS_ROW];
+  __shared__ int sh_first[MAX_GROUP + 1]; // first workgroup number of member t; [g.n] = total
+  for (int round = round_first; round < rounds; ++round) {
+    for (int t = threadIdx.x; t < g.n; t += blockDim.x) {
+      const MvmArgs &a = g.args[t];
+      int wg = 0;
+      if (round < a.max_rounds) {
+        const int n_act = __hip_atomic_load(&a.st.count[round], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (!runs_on_large_tiles(a, round, n_act) && n_act > 0) wg = workgroups_for(a.O, n_act);
+      }
+      sh_first[t + 1] = wg;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      int sum = 0;
+      sh_first[0] = 0;
+      for (int t = 0; t < g.n; ++t) {
+        sum += sh_first[t + 1];
+        sh_first[t + 1] = sum;
+      }
+    }
+    __syncthreads();
+    const int total = sh_first[g.n];
+    if (seen && round == 1 && blockIdx.x == 0) group_seen_update(g, seen);
+    if (total == 0) return; // the same for every workgroup
+    int t = 0;
+    for (int n = blockIdx.x; n < total; n += gridDim.x) {
+      while (n >= sh_first[t + 1]) ++t;
+      const MvmArgs &a = g.args[t];
+      const int n_act = __hip_atomic_load(&a.st.count[round], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      mvm_round_workgroup<1, WMODE>(a, round, n - sh_first[t], n_act, red, stage);
+      __syncthreads();
+    }
+    if (round + 1 == rounds) return;
+    mvm_device_barrier(&g.args[0].st.count[48 + round], (int)gridDim.x);
   }
 }
 
@@ -1802,9 +1864,10 @@ __global__ __launch_bounds__(256) void k_conv_forward_split(MvmArgs a, ConvArgs 
 // The same for several tiles in one launch: a workgroup finds its tile in the table of first workgroup numbers
 // (a multiple of 8 per tile, so the XCD of a workgroup is the one its tile-local number implies).
 template <int PD, int WMODE>
-__global__ __launch_bounds__(256) void k_mvm_round_group(MvmGroup g, int round) {
+__global__ __launch_bounds__(256) void k_mvm_round_group(MvmGroup g, int round, int *seen) {
   __shared__ float red[WAVES][16][64];
   __shared__ __attribute__((aligned(16))) float stage[WAVES * 2 * TILE * LDS_ROW];
+  if (seen && round == 1 && blockIdx.x == 0) group_seen_update(g, seen);
   int t = 0;
   while (t + 1 < g.n && (int)blockIdx.x >= g.start[t + 1]) ++t;
   const MvmArgs &a = g.args[t];
@@ -1958,16 +2021,17 @@ static int big_threshold(int m_batch, int O) {
 
 bool mvm_uses_large_tiles(int m_batch, int O) { return big_threshold(m_batch, O) > 0; }
 
-void launch_mvm_round_group(const MvmGroup &g, int depth, int mode, int total_workgroups, int round, hipStream_t s) {
+void launch_mvm_round_group(const MvmGroup &g, int depth, int mode, int total_workgroups, int round, hipStream_t s,
+                            int *seen) {
   if (round > 0 && total_workgroups > TAIL_GRID && g.n <= MAX_GROUP) {
     const dim3 tail(TAIL_GRID);
-    if (mode == 0) hipLaunchKernelGGL(k_mvm_round_tail_group<0>, tail, dim3(256), 0, s, g, round);
-    else if (mode == 1) hipLaunchKernelGGL(k_mvm_round_tail_group<1>, tail, dim3(256), 0, s, g, round);
-    else hipLaunchKernelGGL(k_mvm_round_tail_group<2>, tail, dim3(256), 0, s, g, round);
+    if (mode == 0) hipLaunchKernelGGL(k_mvm_round_tail_group<0>, tail, dim3(256), 0, s, g, round, seen);
+    else if (mode == 1) hipLaunchKernelGGL(k_mvm_round_tail_group<1>, tail, dim3(256), 0, s, g, round, seen);
+    else hipLaunchKernelGGL(k_mvm_round_tail_group<2>, tail, dim3(256), 0, s, g, round, seen);
     return;
   }
   const dim3 grid(total_workgroups);
-#define RPU_LAUNCH_ROUND(PD, WMODE) hipLaunchKernelGGL((k_mvm_round_group<PD, WMODE>), grid, dim3(256), 0, s, g, round)
+#define RPU_LAUNCH_ROUND(PD, WMODE) hipLaunchKernelGGL((k_mvm_round_group<PD, WMODE>), grid, dim3(256), 0, s, g, round, seen)
   if (mode == 0) {
     if (depth == 4) RPU_LAUNCH_ROUND(4, 0);
     else if (depth == 2) RPU_LAUNCH_ROUND(2, 0);
@@ -1982,6 +2046,17 @@ void launch_mvm_round_group(const MvmGroup &g, int depth, int mode, int total_wo
     else RPU_LAUNCH_ROUND(1, 2);
   }
 #undef RPU_LAUNCH_ROUND
+}
+
+// all rounds from round_first on in one launch of `workgroups` workgroups (at most one per CU: they wait for each other
+// between rounds); for groups of at most MAX_GROUP tiles whose weights are not read transposed
+bool mvm_group_can_merge_rest(const MvmGroup &g, int mode) { return g.n <= MAX_GROUP && mode != 1; }
+
+void launch_mvm_rest_group(const MvmGroup &g, int mode, int round_first, int rounds, int workgroups, int *seen,
+                           hipStream_t s) {
+  const dim3 grid(workgroups);
+  if (mode == 0) hipLaunchKernelGGL(k_mvm_rest_group<0>, grid, dim3(256), 0, s, g, round_first, rounds, seen);
+  else hipLaunchKernelGGL(k_mvm_rest_group<2>, grid, dim3(256), 0, s, g, round_first, rounds, seen);
 }
 
 // whether rounds 0 and 1 of this call can run as one launch (the caller decides whether they should)

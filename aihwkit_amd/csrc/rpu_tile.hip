@@ -1993,6 +1993,10 @@ struct rpu_group {
   MvmArgs *h_args = nullptr; // pinned staging
   int *h_start = nullptr;
   hipEvent_t copied = nullptr;
+  // host-visible pairs (any tile listed a sample for round 1, batch), one per kernel variant of the group's last call:
+  // the next call runs the rounds after round 0 in one launch where nothing was listed
+  int *seen_host = nullptr, *seen_dev = nullptr;
+  int cu_count = 0;
   std::mutex mutex;
   ~rpu_group() {
     if (device_id >= 0) {
@@ -2004,6 +2008,7 @@ struct rpu_group {
         }
         if (h_args) (void)hipHostFree(h_args);
         if (h_start) (void)hipHostFree(h_start);
+        if (seen_host) (void)hipHostFree(seen_host);
         d_args.release();
         d_start.release();
       } catch (...) {
@@ -2160,15 +2165,35 @@ static int group_mvm(rpu_group_t *group, const float *const *x_dev, const long *
     int max_k = 0;
     for (int i = 0; i < n; ++i) max_k = std::max(max_k, args[i].K);
     launch_mvm_init_group(all, max_k, s);
+    constexpr int kSeenPairs = 16;
+    if (!group->seen_host) {
+      RPU_HIP_CHECK(hipHostMalloc((void **)&group->seen_host, 2 * kSeenPairs * sizeof(int), hipHostMallocMapped));
+      for (int i = 0; i < 2 * kSeenPairs; ++i) group->seen_host[i] = 0;
+      RPU_HIP_CHECK(hipHostGetDevicePointer((void **)&group->seen_dev, group->seen_host, 0));
+      hipDeviceProp_t prop;
+      RPU_HIP_CHECK(hipGetDeviceProperties(&prop, group->device_id));
+      group->cu_count = prop.multiProcessorCount;
+    }
+    std::vector<bool> merged(segments.size(), false);
     for (int r = 0; r < rounds; ++r) {
       if (use_big && r == 0) {
         MvmGroup g{group->d_args.p, group->d_start.p + big_offset, n, m_batch};
         launch_mvm_big_group(g, big_total, transposed, s);
         if (all_big) continue;
       }
-      for (const Segment &seg : segments) {
+      for (size_t k = 0; k < segments.size(); ++k) {
+        const Segment &seg = segments[k];
+        if (merged[k]) continue;
         MvmGroup g{group->d_args.p + seg.first, group->d_start.p + seg.start_offset, seg.count, m_batch};
-        launch_mvm_round_group(g, seg.depth, seg.mode, seg.workgroups, r, s);
+        int *seen = k < (size_t)kSeenPairs ? group->seen_dev + 2 * k : nullptr;
+        // the last call of this group listed nothing for round 1: one launch for all rounds after round 0
+        if (r == 1 && rounds >= 3 && seen && !transposed && mvm_group_can_merge_rest(g, seg.mode) &&
+            *(volatile int *)&group->seen_host[2 * k + 1] == m_batch && *(volatile int *)&group->seen_host[2 * k] == 0) {
+          launch_mvm_rest_group(g, seg.mode, 1, rounds, std::min(256, group->cu_count), seen, s);
+          merged[k] = true;
+          continue;
+        }
+        launch_mvm_round_group(g, seg.depth, seg.mode, seg.workgroups, r, s, seen);
       }
     }
     RPU_HIP_CHECK(hipGetLastError());

@@ -109,3 +109,41 @@ def test_the_tile_chooses_by_its_last_call(gpu_device):
     y = auto.forward(xin).cpu().numpy()
     assert np.array_equal(y, ref.forward(xin).cpu().numpy())
     assert np.array_equal(auto.get_bm_rounds(256).numpy(), ref.get_bm_rounds(256).numpy())
+
+
+def test_groups_share_one_launch_for_the_later_rounds_and_recover(gpu_device):
+    """A tile group whose last call listed no sample for round 1 runs all later rounds as one launch; when its inputs
+    then do saturate, that launch runs the rounds itself (waiting between them).  Exact-arithmetic setting: every call
+    must equal the oracle bit for bit, through quiet -> saturating -> quiet sequences, for groups on either side of the
+    size at which the later rounds take the walking kernel."""
+    from helpers import constant_step
+    rng = np.random.default_rng(21)
+    for n_tiles, batch, d_size in ((3, 96, 64), (9, 1100, 300)):
+        grouped, oracles = [], []
+        for k in range(n_tiles):
+            x_size = int(rng.choice([64, 96, 130]))
+            f_io = noise_free_io(inp_res=1 / 128.0, out_res=1 / 512.0, noise_management=NM.AbsMax,
+                                 bound_management=BM.Iterative, out_bound=2.0)
+            dev = constant_step(w_max_dtod=0.0, w_min_dtod=0.0, w_max=1.0, w_min=-1.0, construction_seed=k + 1)
+            host, orc, _ = build_pair(make_meta(f_io, noise_free_io()), dev, x_size, d_size, gpu=False)
+            w = (rng.integers(-60, 61, (d_size, x_size)) / 64.0).astype(F)
+            host.set_weights(torch.from_numpy(w))
+            orc.set_weights(w)
+            grouped.append(tiles.CudaAnalogTile(host))
+            oracles.append(orc)
+        group = tiles.TileGroup(grouped)
+        sizes = [t.get_x_size() for t in grouped]
+        loud = [(rng.integers(-64, 65, (batch, n)) / 64.0).astype(F) for n in sizes]     # several rounds per sample
+        quiet = []
+        for n in sizes:                                                                # one input line: nothing saturates
+            x = np.zeros((batch, n), F)
+            x[np.arange(batch), rng.integers(0, n, batch)] = 0.5
+            quiet.append(x)
+        seen_rounds = []
+        for xs in (quiet, quiet, loud, loud, quiet, quiet, loud):
+            got = group.forward([torch.from_numpy(x).cuda() for x in xs])
+            for y, orc, x, t in zip(got, oracles, xs, grouped):
+                assert np.array_equal(y.cpu().numpy(), orc.forward(x))
+                assert np.array_equal(t.get_bm_rounds(batch).numpy(), orc.bm_rounds(batch))
+            seen_rounds.append(max(int(t.get_bm_rounds(batch).max()) for t in grouped))
+        assert seen_rounds[0] == 1 and seen_rounds[2] >= 3
