@@ -84,7 +84,12 @@ struct MvmArgs {
   int small_tiles_only;     // 1: never the large-tile kernel (its row padding differs)
   const int *skip_if_zero;  // non-null: a round launch does nothing when this device value is zero
   DualDev dual;
-  int rest_in_one;          // 1: this launch runs round `round` and every round after it (k_mvm_rounds_rest)
+  int rest_in_one;          // 1: this launch runs round `round` and every round after it (k_mvm_rounds_rest)  // Tiles of a group call that quantize the same input the same way (the column blocks of a layer split over several
+  // tiles) share the rows of rounds 0 and 1: with xq_first[0] set, those rounds read xq_first[round] instead of
+  // xq[round & 1] (every later round uses the tile's own xq as usual), and the init kernel writes the shared rows
+  // for the one tile that has xq_first_writer = 1.  Requires rows_ahead_in_init (or a single round).
+  float *xq_first[2];
+  int xq_first_writer;
 };
 
 // noise management + per-sample state for round 0

@@ -47,6 +47,11 @@ template <typename T> __device__ __forceinline__ T *pick2(T *const (&p)[2], int 
   return (T *)(p0 ^ ((p0 ^ p1) & (uintptr_t)(-(intptr_t)(i & 1))));
 }
 
+// quantized input rows read by round `round`: the rows shared within a group for rounds 0 and 1, else the tile's own
+__device__ __forceinline__ const float *round_rows(const MvmArgs &a, int round) {
+  return (a.xq_first[0] && round < 2) ? a.xq_first[round] : pick2(a.xq, round & 1);
+}
+
 constexpr int TILE = 32;
 constexpr int WAVES = 4;
 constexpr int KSTEP = 32; // k-values per wave step: 128 bytes per operand row
@@ -370,7 +375,7 @@ __device__ __forceinline__ void mvm_round_tile(const MvmArgs &a, int round, int 
   // staging layout of this lane: pass t covers rows 8 t .. 8 t + 7, lane = (row in pass) * 8 + 16-byte chunk
   const int st_row = lane >> 3;
   const int st_chunk = (lane & 7) * 4;
-  const float *xq = pick2(a.xq, round & 1);
+  const float *xq = round_rows(a, round);
   const float *x_src[4];
   const float *x1_src[4];
   const float *w_src[4];
@@ -663,8 +668,12 @@ __device__ __forceinline__ float group_sum(float v, float *sh) {
 template <int SUB>
 __device__ __forceinline__ void mvm_init_sample(const MvmArgs &a, int b, int t, long gid, long gstride, float *sh) {
   const IoDev &io = a.io;
+  // rows shared with other tiles of a group are written by one of them
+  float *const rows0 = a.xq_first[0] ? a.xq_first[0] : a.xq[0];
+  float *const rows1 = a.xq_first[0] ? a.xq_first[1] : a.xq[1];
+  const bool writes = !a.xq_first[0] || a.xq_first_writer;
   if (io.perfect) { // plain copy into the k-contiguous scratch
-    write_dac_row(a, b, b, 1.0f, 0, a.xq[0], t, SUB);
+    if (writes) write_dac_row(a, b, b, 1.0f, 0, rows0, t, SUB);
     return;
   }
   const float *row = a.in + (long)b * a.in_sb;
@@ -756,9 +765,10 @@ __device__ __forceinline__ void mvm_init_sample(const MvmArgs &a, int b, int t, 
   // so that the first round has nothing to prepare
   float next = 0.0f;
   if (a.rows_ahead_in_init && io.bound_management != RPU_BM_NONE) next = next_round_scale(a, 0, b, fin, nm, 1.0f);
+  if (!writes) return;
   if (kept) {
-    float *out0 = a.xq[0] + (long)b * a.k_pad;
-    float *out1 = a.xq[1] + (long)b * a.k_pad;
+    float *out0 = rows0 + (long)b * a.k_pad;
+    float *out1 = rows1 + (long)b * a.k_pad;
 #pragma unroll
     for (int i = 0; i < KEEP; ++i) {
       const int k = t + i * SUB;
@@ -768,8 +778,8 @@ __device__ __forceinline__ void mvm_init_sample(const MvmArgs &a, int b, int t, 
       }
     }
   } else {
-    write_dac_row(a, b, b, scale, 0, a.xq[0], t, SUB);
-    if (next != 0.0f) write_dac_row(a, b, b, next, 1, a.xq[1], t, SUB);
+    write_dac_row(a, b, b, scale, 0, rows0, t, SUB);
+    if (next != 0.0f) write_dac_row(a, b, b, next, 1, rows1, t, SUB);
   }
 }
 
@@ -1295,7 +1305,7 @@ __device__ __forceinline__ void mvm_big_workgroup(const MvmArgs &a, const int ro
 
   // global -> LDS assignment.  k-contiguous operand: chunk c = t + 256 j covers row c / 8, floats 4 (c % 8) ..;
   // output-contiguous weights: chunk c covers k-row c / 32, outputs 4 (c % 32) ..
-  const float *xq = pick2(a.xq, round & 1);
+  const float *xq = round_rows(a, round);
   const float *x_src[4];
   const float *w_src[4];
   const int st_col = (t & 7) * 4;
@@ -1880,12 +1890,16 @@ __global__ __launch_bounds__(256) void k_mvm_round_group(MvmGroup g, int round, 
 template <int SUB>
 __global__ __launch_bounds__(256) void k_mvm_init_group(MvmGroup g) {
   __shared__ float sh[8];
+  static_assert(SUB % 64 == 0, "a wave works on one sample");
   const long sample = blockIdx.x * (long)(256 / SUB) + threadIdx.x / SUB; // m_batch is a multiple of 256 / SUB
-  const int t = (int)(sample / g.m_batch);
+  // the tile is the same for the whole wave: its arguments are fetched once, by scalar loads, into a copy that the
+  // stores of the per-sample state cannot alias (through the pointer, every store would be followed by reloads)
+  const int t = __builtin_amdgcn_readfirstlane((int)(sample / g.m_batch));
   if (t >= g.n) return;
   const int b = (int)(sample - (long)t * g.m_batch);
   const int lane = threadIdx.x % SUB;
-  mvm_init_sample<SUB>(g.args[t], b, lane, (long)b * SUB + lane, (long)g.m_batch * SUB, sh);
+  const MvmArgs a = g.args[t];
+  mvm_init_sample<SUB>(a, b, lane, (long)b * SUB + lane, (long)g.m_batch * SUB, sh);
 }
 
 __global__ void k_make_bias(const float *in, float *out, int m_batch, int x_size, int in_trans) {

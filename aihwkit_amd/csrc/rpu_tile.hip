@@ -1997,6 +1997,9 @@ struct rpu_group {
   // the next call runs the rounds after round 0 in one launch where nothing was listed
   int *seen_host = nullptr, *seen_dev = nullptr;
   int cu_count = 0;
+  // quantized rows of rounds 0 and 1 shared by tiles that read the same input with the same DAC (two buffers per set)
+  std::vector<DevBuf<float>> first_rows;
+  int shared_sets = 0, shared_tiles = 0; // of the last call
   std::mutex mutex;
   ~rpu_group() {
     if (device_id >= 0) {
@@ -2011,6 +2014,7 @@ struct rpu_group {
         if (seen_host) (void)hipHostFree(seen_host);
         d_args.release();
         d_start.release();
+        for (auto &b : first_rows) b.release();
       } catch (...) {
       }
     }
@@ -2041,6 +2045,15 @@ int rpu_group_create(rpu_group_t **out, rpu_tile_t *const *tiles, int n_tiles) {
     RPU_HIP_CHECK(hipHostMalloc((void **)&g->h_start, (3 * n + 4) * sizeof(int), hipHostMallocDefault));
     RPU_HIP_CHECK(hipEventCreateWithFlags(&g->copied, hipEventDisableTiming));
     *out = g.release();
+  });
+}
+
+int rpu_group_get_shared_input_sets(rpu_group_t *group, int *n_sets, int *n_tiles) {
+  return guarded([&] {
+    if (!group) throw RpuError("null argument");
+    std::lock_guard<std::mutex> glock(group->mutex);
+    if (n_sets) *n_sets = group->shared_sets;
+    if (n_tiles) *n_tiles = group->shared_tiles;
   });
 }
 
@@ -2124,6 +2137,64 @@ static int group_mvm(rpu_group_t *group, const float *const *x_dev, const long *
       args[i] = a;
       t.last_stream = s;
       if (!transposed) t.last_forward_batch = m_batch;
+    }
+    // Tiles that quantize the same input the same way (the column blocks of a layer that was split over several
+    // tiles) share the rows of rounds 0 and 1: one of them writes the rows, all of them read them.  Rows of later
+    // rounds sit at list positions that differ from tile to tile and stay in each tile's own scratch.
+    {
+      auto shares = [](const MvmArgs &a) {
+        if (a.io.perfect) return true;
+        if (a.io.inp_noise > 0.0f || a.io.inp_sto_round) return false; // random streams are the tile's own
+        return a.max_rounds <= 1 || (a.rows_ahead_in_init && (a.speculate || a.big_from < 0));
+      };
+      auto same_rows = [](const MvmArgs &a, const MvmArgs &b) {
+        const IoDev &p = a.io, &q = b.io;
+        return a.in == b.in && a.in_sb == b.in_sb && a.in_sk == b.in_sk && a.K == b.K && a.k_pad == b.k_pad &&
+               a.max_rounds == b.max_rounds && a.rows_ahead_in_init == b.rows_ahead_in_init && p.perfect == q.perfect &&
+               (p.perfect || (p.inp_res == q.inp_res && p.inp_bound == q.inp_bound && p.inp_asym == q.inp_asym &&
+                              p.nm_thres == q.nm_thres && p.max_bm_res == q.max_bm_res &&
+                              p.max_bm_factor == q.max_bm_factor && p.noise_management == q.noise_management &&
+                              p.bound_management == q.bound_management &&
+                              (p.out_scale != 0.0f) == (q.out_scale != 0.0f) &&
+                              // the output range enters the input scale only through the worst-case estimate
+                              (!(p.noise_management == RPU_NM_ABS_MAX_NP_SUM ||
+                                 p.bound_management == RPU_BM_ITERATIVE_WORST_CASE) ||
+                               (p.nm_assumed_wmax == q.nm_assumed_wmax &&
+                                ((std::isinf(p.out_bound) && std::isinf(q.out_bound)) || p.out_bound == q.out_bound)))));
+      };
+      std::vector<int> first_of; // first tile of each set
+      std::vector<int> set_of(n, -1), members;
+      for (int i = 0; i < n; ++i) {
+        if (!shares(args[i])) continue;
+        for (size_t c = 0; c < first_of.size() && set_of[i] < 0; ++c) {
+          if (same_rows(args[i], args[first_of[c]])) set_of[i] = (int)c;
+        }
+        if (set_of[i] < 0) {
+          set_of[i] = (int)first_of.size();
+          first_of.push_back(i);
+          members.push_back(0);
+        }
+        ++members[set_of[i]];
+      }
+      if (group->first_rows.size() < 2 * first_of.size()) group->first_rows.resize(2 * first_of.size());
+      group->shared_sets = group->shared_tiles = 0;
+      for (size_t c = 0; c < members.size(); ++c) {
+        if (members[c] >= 2) {
+          ++group->shared_sets;
+          group->shared_tiles += members[c];
+        }
+      }
+      for (int i = 0; i < n; ++i) {
+        const int c = set_of[i];
+        if (c < 0 || members[c] < 2) continue;
+        MvmArgs &a = args[i];
+        DevBuf<float> &r0 = group->first_rows[2 * c], &r1 = group->first_rows[2 * c + 1];
+        r0.ensure((size_t)m_batch * a.k_pad);
+        if (a.max_rounds > 1) r1.ensure((size_t)m_batch * a.k_pad);
+        a.xq_first[0] = r0.p;
+        a.xq_first[1] = a.max_rounds > 1 ? r1.p : nullptr;
+        a.xq_first_writer = first_of[c] == i ? 1 : 0;
+      }
     }
     // tiles that share a kernel variant sit next to each other
     std::vector<int> order(n);

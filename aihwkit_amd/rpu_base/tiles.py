@@ -619,6 +619,13 @@ class TileGroup:
             raise RuntimeError(what + " must be a matrix with unit column stride")
         return tensor
 
+    def get_shared_input_sets(self):
+        """(sets, tiles) of the last call: sets of at least two tiles that were handed the same input and convert it the
+        same way, so that its quantized rows were written once for the set, and the number of tiles in such sets."""
+        n_sets, n_tiles = C.c_int(0), C.c_int(0)
+        check(lib().rpu_group_get_shared_input_sets(self._g, C.byref(n_sets), C.byref(n_tiles)))
+        return n_sets.value, n_tiles.value
+
     def backward(self, d_inputs, non_blocking: bool = False, outs=None):
         """d_inputs[i]: CUDA tensor [m_batch, d_size_i]; returns the input gradients [m_batch, x_size_i] of every tile
         (``outs``: tensors to fill, e.g. column slices), each what the tile's own ``backward`` gives."""

@@ -444,6 +444,12 @@ int rpu_group_forward_strided(rpu_group_t *group, const float *const *x_dev, con
  * gives it. */
 int rpu_group_backward_strided(rpu_group_t *group, const float *const *d_dev, const long *d_ld, float *const *x_dev,
                                const long *x_ld, int m_batch, void *stream);
+/* Tiles of a group that are handed the same input (pointer, stride, length) and convert it with the same DAC, noise
+ * and bound management and without random numbers (the column blocks of a split layer, array.py:155-182, which the
+ * reference quantizes once per tile) share the quantized rows of rounds 0 and 1: one of them writes the rows, all read
+ * them; results are unchanged.  This reports what the last call of the group did: the number of such sets of at
+ * least two tiles, and the number of tiles in them. */
+int rpu_group_get_shared_input_sets(rpu_group_t *group, int *n_sets, int *n_tiles);
 int rpu_group_destroy(rpu_group_t *group);
 
 /* ---- inference weight pipeline ------------------------------------------------------------- */

@@ -147,3 +147,87 @@ def test_groups_share_one_launch_for_the_later_rounds_and_recover(gpu_device):
                 assert np.array_equal(t.get_bm_rounds(batch).numpy(), orc.bm_rounds(batch))
             seen_rounds.append(max(int(t.get_bm_rounds(batch).max()) for t in grouped))
         assert seen_rounds[0] == 1 and seen_rounds[2] >= 3
+
+
+@pytest.mark.parametrize("batch,out_blocks", [(96, (64, 130, 40)), (1100, (300,) * 6)])
+def test_tiles_of_a_split_layer_share_their_quantized_input(gpu_device, batch, out_blocks):
+    """A layer split into column and row blocks: the tiles of one input block are handed the same column slice of the
+    layer input, and the group quantizes it once for all of them (rounds 0 and 1; the rows of later rounds are each
+    tile's own, since the tiles saturate on different samples).  Exact-arithmetic setting against the oracle, through
+    quiet and saturating calls; one tile of each input block has a DAC of its own and must not take part."""
+    from helpers import constant_step
+    rng = np.random.default_rng(batch)
+    in_blocks = (96, 104)
+    grouped, oracles, where = [], [], []
+    i0 = 0
+    for bi, n_in in enumerate(in_blocks):
+        o0 = 0
+        for bo, n_out in enumerate(out_blocks):
+            own_dac = bo == len(out_blocks) - 1
+            f_io = noise_free_io(inp_res=1 / 64.0 if own_dac else 1 / 128.0, out_res=1 / 512.0, noise_management=NM.AbsMax,
+                                 bound_management=BM.Iterative, out_bound=1.0 + bo)
+            dev = constant_step(w_max_dtod=0.0, w_min_dtod=0.0, w_max=1.0, w_min=-1.0, construction_seed=7 * bi + bo + 1)
+            host, orc, _ = build_pair(make_meta(f_io, noise_free_io()), dev, n_in, n_out, gpu=False)
+            w = (rng.integers(-60, 61, (n_out, n_in)) / 64.0).astype(F) * F(0.25 if bo % 2 else 1.0)
+            host.set_weights(torch.from_numpy(w))
+            orc.set_weights(w)
+            grouped.append(tiles.CudaAnalogTile(host))
+            oracles.append(orc)
+            where.append((bi, i0, n_in, o0, n_out))
+            o0 += n_out
+        i0 += n_in
+    group = tiles.TileGroup(grouped)
+    loud = (rng.integers(-64, 65, (batch, sum(in_blocks))) / 64.0).astype(F)
+    loud *= rng.choice([1 / 64.0, 0.25, 1.0], (batch, 1)).astype(F)
+    loud[5] = 0.0
+    quiet = np.zeros_like(loud)
+    quiet[np.arange(batch), rng.integers(0, 96, batch)] = 0.5
+    quiet[np.arange(batch), 96 + rng.integers(0, 104, batch)] = -0.25
+    most = 0
+    for x in (loud, quiet, quiet, loud, loud):
+        x_layer = torch.from_numpy(x).cuda()
+        partial = torch.full((len(in_blocks), batch, sum(out_blocks)), float("nan"), device="cuda")
+        xs = [x_layer[:, i:i + n] for _bi, i, n, _o, _m in where]
+        ys = [partial[bi][:, o:o + m] for bi, _i, _n, o, m in where]
+        group.forward(xs, outs=ys)
+        assert group.get_shared_input_sets() == (len(in_blocks), len(in_blocks) * (len(out_blocks) - 1))
+        got = partial.cpu().numpy()
+        for (bi, i, n, o, m), orc, t in zip(where, oracles, grouped):
+            assert np.array_equal(got[bi][:, o:o + m], orc.forward(np.ascontiguousarray(x[:, i:i + n])))
+            rounds = t.get_bm_rounds(batch).numpy()
+            assert np.array_equal(rounds, orc.bm_rounds(batch))
+            most = max(most, int(rounds.max()))
+    assert most >= 3                                   # rows of rounds after round 1 were needed, and differ by tile
+
+
+def test_shared_input_rows_leave_noisy_results_unchanged(gpu_device):
+    """The same with the benchmark's analog noise on the outputs: a group call on column slices of one input equals the
+    tiles called one by one with the same seeds, bit for bit; tiles whose DAC draws random numbers (input noise,
+    stochastic rounding) keep rows of their own."""
+    rng = np.random.default_rng(3)
+    batch, n_in = 200, 160
+    ios = [io_params(out_noise=0.06, out_bound=4.0, noise_management=NM.AbsMax, bound_management=BM.Iterative),
+           io_params(out_noise=0.06, out_bound=4.0, noise_management=NM.AbsMax, bound_management=BM.Iterative),
+           io_params(out_noise=0.06, out_bound=4.0, inp_noise=0.01, noise_management=NM.AbsMax, bound_management=BM.Iterative),
+           io_params(out_noise=0.06, out_bound=4.0, inp_sto_round=True, noise_management=NM.AbsMax,
+                     bound_management=BM.Iterative),
+           io_params(out_noise=0.06, out_bound=12.0, noise_management=NM.AbsMaxNPSum, bound_management=BM.IterativeWorstCase),
+           io_params(out_noise=0.06, out_bound=12.0, noise_management=NM.AbsMaxNPSum, bound_management=BM.IterativeWorstCase)]
+    alone, grouped = [], []
+    for k, io in enumerate(ios):
+        host, _orc, _ = build_pair(make_meta(io, noise_free_io()), soft_bounds(construction_seed=k + 1), n_in, 70 + 10 * k,
+                                   gpu=False)
+        host.set_weights(torch.from_numpy(rng.uniform(-0.4, 0.4, (70 + 10 * k, n_in)).astype(F)))
+        alone.append(tiles.CudaAnalogTile(host))
+        grouped.append(tiles.CudaAnalogTile(host))
+    group = tiles.TileGroup(grouped)
+    for call in range(3):
+        x = torch.from_numpy((rng.uniform(-1, 1, (batch, n_in)) * rng.choice([0.05, 1.0], (batch, 1))).astype(F)).cuda()
+        for k, (a, g) in enumerate(zip(alone, grouped)):
+            a.set_seed(50 * call + k)
+            g.set_seed(50 * call + k)
+        got = group.forward([x] * len(grouped))
+        assert group.get_shared_input_sets() == (2, 4)
+        for a, g, y in zip(alone, grouped, got):
+            assert np.array_equal(y.cpu().numpy(), a.forward(x).cpu().numpy())
+            assert np.array_equal(g.get_bm_rounds(batch).numpy(), a.get_bm_rounds(batch).numpy())
