@@ -18,6 +18,10 @@ struct IoDev {
 };
 
 // Per-sample bookkeeping of the noisy MVM, all arrays of length >= m_batch.
+constexpr int MVM_COUNT_WORDS = 256; // MvmState::count: [0, 40) per round; [MVM_ARRIVE_BASE + 4 r, + 4): counter and flag of the
+                                     // arrivals after round r, counter and flag of the wait before round r
+constexpr int MVM_ARRIVE_BASE = 64;
+
 struct MvmState {
   float *nm;       // noise-management scale
   float *nm_np;    // AbsMaxNPSum scale (IterativeWorstCase only)
@@ -30,7 +34,8 @@ struct MvmState {
   int *list[2];    // ping-pong lists of samples that need another round
   int *row[2];     // row[i][pos]: row of xq[i] that holds the quantized input of the sample at list[i][pos]
   float *next_scale[2]; // next_scale[i][pos]: input scale that sample would use one round later (0: no such round)
-  int *count;      // count[r] = number of samples in the list read by round r (r >= 1)
+  int *count;      // count[r] = number of samples in the list read by round r (r >= 1); MVM_COUNT_WORDS words, the
+                   // upper half the arrival counters of the launches that run several rounds
   int *tile_done;  // tile_done[r * tiles_b + t] = workgroups of round r that have finished sample tile t
 };
 
@@ -41,7 +46,8 @@ struct DualDev {
   int *sel;      // [m_batch] which of them is the sample's output (0 / 1); 2: the sample is listed for round 2
   int *hit1;     // [2][m_batch] saturation marks of round 1: upper, lower (as MvmState::hit_up / hit_lo)
   float *xq2;    // quantized rows of round 2, written while round 0's rows are still read
-  int *seen;     // host-visible: [0] samples of the last call that needed round 1, [1] its batch; null: not kept
+  int *seen;     // host-visible: [0] samples of the last call that needed round 1, [1] its batch, [2] the last round
+                 // that listed a sample (0: none after round 0); null: not kept
   int on;        // 1: the fused launch; 2: this launch starts with the selection of the fused launch's results
 };
 

@@ -756,7 +756,7 @@ __device__ __forceinline__ void mvm_init_sample(const MvmArgs &a, int b, int t, 
     a.st.rounds[b] = (fin == 0.0f) ? 0 : 1;
     if (io.bound_management != RPU_BM_NONE) a.st.next_scale[0][b] = next_round_scale(a, 0, b, fin, nm, 1.0f);
   }
-  if (gid < 64) a.st.count[gid] = 0; // count[0 .. 39] per round, count[48 ..] the arrival counters of k_mvm_rounds_rest
+  if (gid < MVM_COUNT_WORDS) a.st.count[gid] = 0; // per-round counts and the arrival counters of k_mvm_rounds_rest
   {
     const long n_done = 32L * ((a.m_batch + TILE - 1) / TILE);
     for (long idx = gid; idx < n_done; idx += gstride) a.st.tile_done[idx] = 0;
@@ -1047,6 +1047,43 @@ __device__ __forceinline__ void mvm_device_barrier(int *counter, int total) {
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
 }
 
+// All workgroups of a launch wait until each has arrived, which it does once the atomics of its threads have been
+// performed (their results were consumed before the barrier): after the wait, what those atomics built up -- the number
+// of samples listed for the next round -- is final and can be read with a device-scope load.  Nothing else the
+// workgroups wrote is made visible: a launch that goes on to read such data calls mvm_device_barrier as well.  A few
+// microseconds, against tens for that one; bounded in the same way.
+// counter[0] counts the arrivals; the last one raises counter[1], which the others poll (so that the polls do not
+// queue up in front of the arrivals at the one address).
+__device__ __forceinline__ void mvm_arrive(int *counter, int total) {
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const int before = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (before == total - 1) {
+      __hip_atomic_store(counter + 1, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    } else {
+      int spins = 0;
+      while (__hip_atomic_load(counter + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0 && ++spins < REST_SPIN_LIMIT) {
+        __builtin_amdgcn_s_sleep(8);
+      }
+    }
+  }
+  __syncthreads();
+}
+
+// Host-visible summary of a call for the choice of the next call's launches (a.dual.seen), kept by the first thread of
+// a launch of round r that lists n_act samples; first_after_fused: the launch that follows the fused one.
+__device__ __forceinline__ void mvm_note_round(const MvmArgs &a, int r, int n_act, bool first_after_fused) {
+  if (!a.dual.seen || blockIdx.x != 0 || threadIdx.x != 0) return;
+  if (r == 1 || first_after_fused) {
+    const int needed = (r == 1) ? n_act : a.st.count[1];
+    a.dual.seen[0] = needed;
+    a.dual.seen[1] = a.m_batch;
+    a.dual.seen[2] = n_act > 0 ? r : (needed > 0 ? 1 : 0);
+  } else if (n_act > 0) {
+    a.dual.seen[2] = r;
+  }
+}
+
 // big_from > 0: the large-tile kernel runs the rounds that list at least that many samples; < 0: it runs round 0
 __device__ __forceinline__ bool runs_on_large_tiles(const MvmArgs &a, int round, int n_act) {
   return (a.big_from > 0 && n_act >= a.big_from) || (a.big_from < 0 && round == 0);
@@ -1126,8 +1163,9 @@ __global__ __launch_bounds__(256) void k_mvm_round_tail_group(MvmGroup g, int ro
 }
 
 // The rounds from round_first on of all tiles of a group in one launch (see k_mvm_rounds_rest): a fixed number of
-// workgroups, all resident at once, walk the tiles that the members list for a round; they leave at the first round that
-// lists none.  The arrival counters are those of the group's first tile.
+// workgroups, all resident at once, walk the tiles that the members list for a round; after a round they wait for each
+// other's arrival and leave if the next round lists nothing (else a full device-wide wait comes first).  The arrival
+// counters are those of the group's first tile.
 template <int WMODE>
 __global__ __launch_bounds__(256) void k_mvm_rest_group(MvmGroup g, int round_first, int rounds, int *seen) {
   __shared__ float red[WAVES][16][64];
@@ -1156,6 +1194,8 @@ __global__ __launch_bounds__(256) void k_mvm_rest_group(MvmGroup g, int round_fi
     const int total = sh_first[g.n];
     if (seen && round == 1 && blockIdx.x == 0) group_seen_update(g, seen);
     if (total == 0) return; // the same for every workgroup
+    // the rows and lists that the round before left must be visible on every XCD
+    if (round > round_first) mvm_device_barrier(&g.args[0].st.count[MVM_ARRIVE_BASE + 4 * round + 2], (int)gridDim.x);
     int t = 0;
     for (int n = blockIdx.x; n < total; n += gridDim.x) {
       while (n >= sh_first[t + 1]) ++t;
@@ -1165,29 +1205,31 @@ __global__ __launch_bounds__(256) void k_mvm_rest_group(MvmGroup g, int round_fi
       __syncthreads();
     }
     if (round + 1 == rounds) return;
-    mvm_device_barrier(&g.args[0].st.count[48 + round], (int)gridDim.x);
+    // the counts of the next round are final once every workgroup has arrived
+    mvm_arrive(&g.args[0].st.count[MVM_ARRIVE_BASE + 4 * round], (int)gridDim.x);
   }
 }
 
-// Every round from a.round on in ONE launch, for calls whose samples are expected to be done by then (as the tile's
-// last call was): the workgroups find the round's list empty and leave, where the separate launches would cost a few
-// microseconds each for nothing.  Where the expectation fails the rounds still run, one after the other with all
-// workgroups waiting for each other in between (mvm_device_barrier: tens of microseconds per round, which is why
-// this launch is only chosen by expectation).
+// Every round from a.round on in ONE launch, for calls whose samples are expected to be done by the end of round
+// a.round (as in the tile's last calls): after that round the workgroups wait for each other's arrival, find the next
+// list empty and leave, where separate launches would cost a few microseconds each for nothing.  Where the expectation
+// fails the rounds still run, one after the other, each behind a wait that also makes the rows and lists of the round
+// before visible on every XCD (mvm_device_barrier: tens of microseconds, which is why this launch is only chosen by
+// expectation).  With a.dual.on = 2 it is the launch after the fused one and starts with that launch's selection.
 template <int PD, int WMODE>
 __global__ __launch_bounds__(256) void k_mvm_rounds_rest(MvmArgs a) {
   __shared__ float red[WAVES][16][64];
   __shared__ __attribute__((aligned(16))) float stage[WAVES * 2 * TILE * LDS_ROW];
+  if (a.dual.on == 2) mvm_dual_select(a, blockIdx.x);
   for (int r = a.round; r < a.max_rounds; ++r) {
+    // final since the launch before (first round) or since every workgroup arrived after the round before
     const int n_act = __hip_atomic_load(&a.st.count[r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if (a.dual.seen && r == 1 && blockIdx.x == 0 && threadIdx.x == 0) {
-      a.dual.seen[0] = n_act;
-      a.dual.seen[1] = a.m_batch;
-    }
-    if (n_act == 0) return; // the same for every workgroup: the count is final since the launch or barrier before
+    mvm_note_round(a, r, n_act, r == a.round && a.dual.on == 2);
+    if (n_act == 0) return; // the same for every workgroup
+    if (r > a.round) mvm_device_barrier(&a.st.count[MVM_ARRIVE_BASE + 4 * r + 2], (int)gridDim.x);
     mvm_round_workgroup<PD, WMODE>(a, r, blockIdx.x, n_act, red, stage);
     if (r + 1 == a.max_rounds) return;
-    mvm_device_barrier(&a.st.count[48 + r], (int)gridDim.x);
+    mvm_arrive(&a.st.count[MVM_ARRIVE_BASE + 4 * r], (int)gridDim.x);
   }
 }
 
@@ -1198,11 +1240,9 @@ __global__ __launch_bounds__(256) void k_mvm_round(MvmArgs a) {
   if (a.skip_if_zero && *a.skip_if_zero == 0) return;
   if (a.dual.on == 2) mvm_dual_select(a, blockIdx.x);
   const int n_act = (a.round > 0) ? a.st.count[a.round] : a.m_batch;
-  // how many samples needed a second round: the host reads it (whenever it next looks) to choose its launches
-  if (a.dual.seen && blockIdx.x == 0 && threadIdx.x == 0 && (a.round == 1 || a.dual.on == 2)) {
-    a.dual.seen[0] = a.st.count[1];
-    a.dual.seen[1] = a.m_batch;
-  }
+  // how many samples needed a second round, and the last round that listed any: the host reads it (whenever it next
+  // looks) to choose its launches
+  if (a.round > 0) mvm_note_round(a, a.round, n_act, a.dual.on == 2);
   if (runs_on_large_tiles(a, a.round, n_act)) return;
   mvm_round_workgroup<PD, WMODE>(a, a.round, blockIdx.x, n_act, red, stage);
 }

@@ -175,10 +175,11 @@ struct Tile {
   DevBuf<float> s_nsc0, s_nsc1, s_nm, s_nmnp, s_red, s_scale, s_fin, s_bias, s_xq0, s_xq1;
   // rounds 0 and 1 of a forward call in one launch: kept outputs of both, choice per sample, marks of round 1, rows of
   // round 2; the host-visible pair (samples of the last call that needed round 1, its batch) that the choice between
-  // the fused and the separate launches is made from (fused_rounds: -1 by that pair, 0 never, 1 whenever possible)
+  // the fused and the separate launches is made from (fused_rounds: -1 by those values, 0 never, 1 .. 3 as forced)
   DevBuf<float> s_dual0, s_dual1, s_xq2;
   DevBuf<int> s_dsel, s_dhit1;
   int *seen_host = nullptr, *seen_dev = nullptr;
+  int rest_from = 0, rest_quiet = 0; // the last round that listed samples in the recent calls, and calls since it did
   int fused_rounds = -1;
   int cu_count = 0;
   int n_cus() {
@@ -434,7 +435,7 @@ struct Tile {
         }
         upload_params();
       }
-      s_count.ensure(64);
+      s_count.ensure(MVM_COUNT_WORDS);
       ensure_update_tables();
     } catch (...) {
       release_all();
@@ -451,7 +452,7 @@ struct Tile {
     const size_t n = (size_t)B;
     s_nsc0.ensure(n); s_nsc1.ensure(n); s_nm.ensure(n); s_nmnp.ensure(n); s_red.ensure(n); s_scale.ensure(n); s_fin.ensure(n);
     s_rounds.ensure(n); s_hitup.ensure(n); s_hitlo.ensure(n); s_list0.ensure(n); s_list1.ensure(n); s_row0.ensure(n); s_row1.ensure(n);
-    s_count.ensure(64);
+    s_count.ensure(MVM_COUNT_WORDS);
     s_tiledone.ensure((size_t)32 * ((n + 31) / 32));
   }
 
@@ -713,18 +714,39 @@ struct Tile {
       }
       // Where most samples need a second round (as the last call on this tile showed), rounds 0 and 1 run as one
       // launch: one chain of latencies instead of two.  Results are the same either way.
-      bool fuse = false, merge_rest = false;
+      bool fuse = false;
+      int merge_from = 0; // > 0: the rounds from this one on run as one launch
       if (!transposed && !w_other && !side && io.p.bound_management != RPU_BM_NONE && fused_rounds != 0) {
         if (!seen_host) {
-          RPU_HIP_CHECK(hipHostMalloc((void **)&seen_host, 2 * sizeof(int), hipHostMallocMapped));
-          seen_host[0] = seen_host[1] = 0;
+          RPU_HIP_CHECK(hipHostMalloc((void **)&seen_host, 4 * sizeof(int), hipHostMallocMapped));
+          seen_host[0] = seen_host[1] = seen_host[2] = seen_host[3] = 0;
           RPU_HIP_CHECK(hipHostGetDevicePointer((void **)&seen_dev, seen_host, 0));
         }
         a.dual.seen = seen_dev;
         const int needed = *(volatile int *)&seen_host[0], of = *(volatile int *)&seen_host[1];
-        fuse = mvm_can_fuse_rounds(a) && (fused_rounds == 1 || (fused_rounds < 0 && of > 0 && 2 * (long)needed > of));
-        // no sample of the last call needed a second round: the launches after round 0 are expected to find nothing
-        merge_rest = !fuse && mvm_can_merge_rest(a, n_cus()) && (fused_rounds == 2 || (fused_rounds < 0 && of > 0 && needed == 0));
+        const int last_listed = *(volatile int *)&seen_host[2];
+        fuse = mvm_can_fuse_rounds(a) &&
+               (fused_rounds == 1 || fused_rounds == 3 || (fused_rounds < 0 && of > 0 && 2 * (long)needed > of));
+        // The last round that listed samples in the recent calls is expected to be the last one of this call too: the
+        // rounds after it share a launch, whose workgroups find the first of their lists empty and leave.  The
+        // estimate rises at once and falls only after eight calls below it: a round that does run inside that launch
+        // costs a wait of all its workgroups for each other (about 8 us, tens if yet another round follows), an extra
+        // launch only a few microseconds.
+        if (of > 0) {
+          if (last_listed >= rest_from) {
+            rest_from = last_listed;
+            rest_quiet = 0;
+          } else if (++rest_quiet >= 8) {
+            rest_from = last_listed;
+            rest_quiet = 0;
+          }
+        }
+        const int first_mergeable = fuse ? 2 : 1;
+        if (mvm_can_merge_rest(a, n_cus())) {
+          if (fused_rounds == 2 || fused_rounds == 3) merge_from = first_mergeable;
+          else if (fused_rounds < 0 && of > 0) merge_from = std::max(first_mergeable, rest_from + 1);
+          if (merge_from + 1 >= a.max_rounds) merge_from = 0; // the last round alone: a plain launch
+        }
       }
       if (fuse) {
         s_dual0.ensure((size_t)B * a.O); s_dual1.ensure((size_t)B * a.O); s_xq2.ensure((size_t)B * a.k_pad);
@@ -747,14 +769,16 @@ struct Tile {
         for (int r = 2; r < a.max_rounds; ++r) {
           a.round = r;
           a.dual.on = r == 2 ? 2 : 0;
+          a.rest_in_one = (merge_from > 0 && r == merge_from) ? 1 : 0;
           launch_mvm_round(a, s);
           prof_mark(s, "mvm_round");
+          if (a.rest_in_one) break;
         }
       } else {
         for (int r = 0; r < a.max_rounds; ++r) {
           a.round = r;
           if (side) pre_adc_terms(a, io, s);
-          a.rest_in_one = (merge_rest && r == 1) ? 1 : 0;
+          a.rest_in_one = (merge_from > 0 && r == merge_from) ? 1 : 0;
           launch_mvm_round(a, s);
           prof_mark(s, "mvm_round");
           if (a.rest_in_one) break;
@@ -2808,9 +2832,10 @@ int rpu_tile_get_update_words(rpu_tile_t *tile, uint32_t *x_words_host, uint32_t
 int rpu_tile_set_fused_rounds(rpu_tile_t *tile, int mode) {
   return guarded([&] {
     if (!tile) throw RpuError("null tile");
-    if (mode < -1 || mode > 2) {
-      throw RpuError("fused rounds: mode must be -1 (by the last call), 0 (never), 1 (rounds 0 and 1 in one launch whenever "
-                     "possible) or 2 (the rounds after round 0 in one launch whenever possible).");
+    if (mode < -1 || mode > 3) {
+      throw RpuError("fused rounds: mode must be -1 (by the last calls), 0 (never), 1 (rounds 0 and 1 in one launch whenever "
+                     "possible), 2 (the rounds after round 0 in one launch whenever possible) or 3 (rounds 0 and 1 in one "
+                     "launch and the rounds after them in another).");
     }
     std::lock_guard<std::mutex> lock(tile->t.mutex);
     tile->t.fused_rounds = mode;

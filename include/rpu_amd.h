@@ -642,12 +642,16 @@ int rpu_tile_set_extra(rpu_tile_t *tile, const int64_t *values_host, int count);
  *   1  rounds 0 and 1 as ONE launch that computes both from the same weights and keeps, per sample, the one the
  *      reference's loop would have ended with (pays where most samples need a second round: the outputs of the tile are
  *      large against out_bound);
- *   2  every round after round 0 as ONE launch whose workgroups leave when they find the round's list empty (pays where
- *      no sample needs a second round; where some do, the rounds still run in that launch, with a wait of all
- *      workgroups between them that costs more than a launch).
- * Mode -1 (default): the tile chooses by what its last forward call needed -- more than half of the samples in a second
- * round: 1; none: 2; else the separate launches.  0: always the separate launches.  1 / 2: that shortcut whenever the
- * shape allows it (single tile, rounds on the 32 x 32 kernel, no per-line periphery terms). */
+ *   2  every round after round 0 as ONE launch: after a round its workgroups wait for each other's arrival (a few
+ *      microseconds) and leave when the next round lists no sample; a round that does follow inside that launch waits for
+ *      all workgroups once more, with the rows and lists of the round before made visible device-wide, which costs more
+ *      than a launch;
+ *   3  both: rounds 0 and 1 as one launch, the rounds after them as another.
+ * Mode -1 (default): the tile chooses by what its recent forward calls needed -- more than half of the samples in a
+ * second round: rounds 0 and 1 in one launch; and the rounds after the last one that listed any sample in those calls
+ * (the estimate rises at once and falls after eight calls below it), which are expected to be empty, share one
+ * launch.  0: always the separate launches.  1 / 2 / 3: that shortcut whenever the shape allows it
+ * (single tile, rounds on the 32 x 32 kernel, at most one workgroup per CU for 2 and 3, no per-line periphery terms). */
 int rpu_tile_set_fused_rounds(rpu_tile_t *tile, int mode);
 
 /* ---- inspection hooks (mirror the reference's debug hooks) ------------------------------ */
