@@ -234,3 +234,22 @@ def test_shared_input_rows_leave_noisy_results_unchanged(gpu_device):
         for a, g, y in zip(alone, grouped, got):
             assert np.array_equal(y.cpu().numpy(), a.forward(x).cpu().numpy())
             assert np.array_equal(g.get_bm_rounds(batch).numpy(), a.get_bm_rounds(batch).numpy())
+
+
+def test_more_than_sixteen_rounds_in_one_launch(gpu_device):
+    """No input quantization and a large max_bm_factor: samples whose outputs exceed a tiny out_bound by five orders of
+    magnitude halve their input seventeen to twenty times.  The single launch for the later rounds walks all of them
+    (its arrival words are per round) and must agree with the separate launches."""
+    rng = np.random.default_rng(17)
+    x_size, d_size, batch = 96, 64, 40
+    io = io_params(inp_res=-1.0, out_res=-1.0, out_noise=0.0, out_bound=2e-5, max_bm_factor=1 << 22,
+                   noise_management=NM.AbsMax, bound_management=BM.Iterative)
+    meta = make_meta(io, noise_free_io())
+    dev = soft_bounds(construction_seed=9)
+    w = rng.uniform(-0.3, 0.3, (d_size, x_size)).astype(F)
+    x = rng.uniform(-1, 1, (batch, x_size)).astype(F)
+    x[::3] *= F(1 / 64.0)                                        # abs-max scaling: the spread of a row decides, ...
+    x[::3, 0] = 1.0                                              # ... so these rows are one large and many small inputs
+    y, rounds = both_ways(meta, dev, x_size, d_size, w, x)
+    assert rounds.max() >= 18 and len(set(rounds.tolist())) >= 3
+    assert np.abs(y).max() > 0.0
