@@ -49,7 +49,7 @@ template <typename T> __device__ __forceinline__ T *pick2(T *const (&p)[2], int 
 
 // quantized input rows read by round `round`: the rows shared within a group for rounds 0 and 1, else the tile's own
 __device__ __forceinline__ const float *round_rows(const MvmArgs &a, int round) {
-  return (a.xq_first[0] && round < 2) ? a.xq_first[round] : pick2(a.xq, round & 1);
+  return (a.xq_first[0] && round < 2) ? (round ? a.xq_first[1] : a.xq_first[0]) : pick2(a.xq, round & 1);
 }
 
 constexpr int TILE = 32;
@@ -1584,7 +1584,7 @@ typedef int i32x4_unaligned __attribute__((ext_vector_type(4), aligned(4)));
 // ONE_STEP: the patch row fits one contraction step (K <= 32, a first convolution layer): the gathered values stay
 // in registers between noise management and the rounds.
 template <bool ONE_STEP>
-__global__ __launch_bounds__(256, 3) void k_conv_forward(MvmArgs a, ConvArgs c) {
+__global__ __launch_bounds__(256, 2) void k_conv_forward(MvmArgs a, ConvArgs c) {
   const int lane = threadIdx.x & 63;
   const int r = lane & 31, h = lane >> 5;
   const long tile = blockIdx.x * 4L + (threadIdx.x >> 6);
