@@ -131,8 +131,10 @@ void launch_mvm_rest_group(const MvmGroup &g, int weight_mode, int round_first, 
 int mvm_round_workgroups(const MvmArgs &a);            // workgroups of a round launch for this tile
 // Large-tile (128 x 128) variant for round 0 of a group: args[t].big_from < 0 marks the tiles it runs, start[]
 // counts its workgroups (mvm_big_workgroups; 0 for the other tiles).
-int mvm_big_workgroups(const MvmArgs &a);
-void launch_mvm_big_group(const MvmGroup &g, int total_workgroups, bool transposed, hipStream_t s);
+int mvm_big_workgroups(const MvmArgs &a, int bb);
+// bb: samples of a workgroup tile, 128 or 64 (mvm_big_sample_tile: by the workgroups the launch would have with 128)
+int mvm_big_sample_tile(int workgroups_128, int n_cus);
+void launch_mvm_big_group(const MvmGroup &g, int total_workgroups, int bb, bool transposed, hipStream_t s);
 void mvm_round_variant(const MvmArgs &a, int &prefetch_depth, int &weight_mode);
 
 // Fused convolution forward (unfold + noisy MVM with its bound-management rounds) for tiles of at most 32 outputs:

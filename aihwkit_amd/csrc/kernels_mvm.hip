@@ -1256,15 +1256,23 @@ __global__ __launch_bounds__(256) void k_mvm_round(MvmArgs a) {
 // may be run by either (the launcher picks by the number of samples in the round).
 // WT = 0: weights contiguous along k (forward), 1: contiguous along the outputs (backward, W read in place).
 
-constexpr int BT = 128;        // tile edge
+constexpr int BT = 128;        // outputs of a workgroup tile; its samples: BB = 128, or 64 (each wave 64 x 32: twice the
+                               // workgroups, for launches that would put fewer than about three of the square tiles on a CU)
 constexpr int BKS = 32;        // k-values per stage
-constexpr int BPITCH = 36;     // floats per staged row of a k-contiguous operand
+constexpr int BROW = 32;       // floats per staged row of a k-contiguous operand, no padding.  LDS has 64 banks: two rows
+                               // fill the 16 chunk slots (of 16 bytes) of a 256-byte line, and chunk c of row `row` sits in
+                               // slot (8 (row % 2) + c + row / 2) % 16 of its line: 16 rows that read the same chunk, and the 16
+                               // threads that store two rows, each touch all 64 banks once
+__device__ __forceinline__ int big_lds_offset(int row, int chunk) {
+  return (row >> 1) * (2 * BROW) + ((((row & 1) << 3) + chunk + (row >> 1)) & 15) * 4;
+}
 constexpr int BPITCH_T = 132;  // floats per staged k-row of an output-contiguous weight tile
 
+template <int BB>
 __device__ __forceinline__ void big_prepare_next_rows(const MvmArgs &a, int round, int tile_o, int tile_b, int n_act,
                                                       int *sh_b, float *sh_scale) {
-  if (threadIdx.x < BT) {
-    const int slot = tile_b * BT + threadIdx.x;
+  if (threadIdx.x < BB) {
+    const int slot = tile_b * BB + threadIdx.x;
     int b = 0;
     float scale = 0.0f;
     if (slot < n_act) {
@@ -1281,22 +1289,23 @@ __device__ __forceinline__ void big_prepare_next_rows(const MvmArgs &a, int roun
   const int k_hi = min(k_lo + chunk, a.k_pad);
   float *__restrict__ dst = pick2(a.xq, (round + 1) & 1);
   const float *__restrict__ in = a.in;
-  const int kq = threadIdx.x & 31, rq = threadIdx.x >> 5; // 8 thread-rows of 16 rows each
+  constexpr int RPT = BB / 8; // 8 thread-rows of RPT rows each
+  const int kq = threadIdx.x & 31, rq = threadIdx.x >> 5;
   for (int k0 = k_lo; k0 < k_hi; k0 += 32) {
     const int k = k0 + kq;
-    float xv[16]; // all 16 loads of a trip are in flight together
+    float xv[RPT]; // all loads of a trip are in flight together
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const int row = rq * 16 + i;
+    for (int i = 0; i < RPT; ++i) {
+      const int row = rq * RPT + i;
       xv[i] = (sh_scale[row] != 0.0f && k < a.K) ? in[(long)sh_b[row] * a.in_sb + (long)k * a.in_sk] : 0.0f;
     }
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const int row = rq * 16 + i;
+    for (int i = 0; i < RPT; ++i) {
+      const int row = rq * RPT + i;
       const float sc = sh_scale[row];
       if (sc != 0.0f) {
         const float v = (k < a.K) ? dac_value(xv[i], sc, a.io, a.key, a.call, round + 1, sh_b[row], k) : 0.0f;
-        dst[(long)(tile_b * BT + row) * a.k_pad + k] = v;
+        dst[(long)(tile_b * BB + row) * a.k_pad + k] = v;
       }
     }
   }
@@ -1304,25 +1313,37 @@ __device__ __forceinline__ void big_prepare_next_rows(const MvmArgs &a, int roun
 
 // Instruction order of 16 MFMAs and the LDS reads of the operands that follow them (a hint to the scheduler): the
 // reads are spread behind the first MFMAs so that they complete underneath the rest.
-template <int WT>
+template <int WT, int NB>
 __device__ __forceinline__ void mvm_big_schedule() {
-  // WT = 0: 4 wide LDS reads; WT = 1: 2 wide reads and the 8 single reads of the transposed weight tile
+  // NB sample blocks per wave: 8 NB MFMAs.  WT = 0: 2 + NB wide LDS reads; WT = 1: NB wide reads and the 8 single
+  // reads of the transposed weight tile
+  constexpr int mfmas = 8 * NB;
+  constexpr int paired = WT == 0 ? 2 + NB : (NB == 2 ? 6 : 5);
+  constexpr int doubled = (WT == 1 && NB == 1) ? 4 : 0; // pairs that carry two LDS reads
 #pragma unroll
-  for (int i = 0; i < (WT == 0 ? 4 : 6); ++i) {
+  for (int i = 0; i < doubled; ++i) {
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); // one MFMA
+    __builtin_amdgcn_sched_group_barrier(0x100, 2, 0); // two LDS reads
+  }
+#pragma unroll
+  for (int i = doubled; i < paired; ++i) {
     __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); // one MFMA
     __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); // one LDS read
   }
-  __builtin_amdgcn_sched_group_barrier(0x008, WT == 0 ? 12 : 10, 0);
+  __builtin_amdgcn_sched_group_barrier(0x008, mfmas - paired, 0);
 }
 
-// work of workgroup number n of a large-tile round launch of one tile
-template <int WT>
+// work of workgroup number n of a large-tile round launch of one tile; BB: samples of a workgroup tile (128 or 64)
+template <int WT, int BB>
 __device__ __forceinline__ void mvm_big_workgroup(const MvmArgs &a, const int round, const int n, const int min_active) {
-  __shared__ __attribute__((aligned(16))) float lds_x[2][BT * BPITCH];
-  __shared__ __attribute__((aligned(16))) float lds_w[2][WT ? BKS * BPITCH_T : BT * BPITCH];
-  __shared__ int sh_hits[2 * BT];
-  __shared__ int sh_b[BT];
-  __shared__ float sh_scale[BT];
+  static_assert(BB == 128 || BB == 64, "sample tile of 128 or 64");
+  constexpr int NB = BB / 64; // 32-sample blocks per wave
+  constexpr int XJ = BB / 32; // staged sample rows per thread
+  __shared__ __attribute__((aligned(16))) float lds_x[2][BB * BROW];
+  __shared__ __attribute__((aligned(16))) float lds_w[2][WT ? BKS * BPITCH_T : BT * BROW];
+  __shared__ int sh_hits[2 * BB];
+  __shared__ int sh_b[BB];
+  __shared__ float sh_scale[BB];
   __shared__ int sh_last;
 
   const int n_act = (round > 0) ? a.st.count[round] : a.m_batch;
@@ -1331,10 +1352,10 @@ __device__ __forceinline__ void mvm_big_workgroup(const MvmArgs &a, const int ro
   // quantized inputs (the large operand) enters one L2 only and the small weight matrix is what every XCD streams
   const int tile_o = (n >> 3) % ((a.O + BT - 1) / BT);
   const int tile_b = ((n >> 3) / ((a.O + BT - 1) / BT)) * 8 + (n & 7);
-  if (tile_b * BT >= n_act) return;
+  if (tile_b * BB >= n_act) return;
   const bool more_rounds = round + 1 < a.max_rounds;
   if (more_rounds && !(round == 0 && a.rows_ahead_in_init)) {
-    big_prepare_next_rows(a, round, tile_o, tile_b, n_act, sh_b, sh_scale);
+    big_prepare_next_rows<BB>(a, round, tile_o, tile_b, n_act, sh_b, sh_scale);
   }
 
   const int t = threadIdx.x;
@@ -1346,23 +1367,25 @@ __device__ __forceinline__ void mvm_big_workgroup(const MvmArgs &a, const int ro
   // global -> LDS assignment.  k-contiguous operand: chunk c = t + 256 j covers row c / 8, floats 4 (c % 8) ..;
   // output-contiguous weights: chunk c covers k-row c / 32, outputs 4 (c % 32) ..
   const float *xq = round_rows(a, round);
-  const float *x_src[4];
+  const float *x_src[XJ];
   const float *w_src[4];
   const int st_col = (t & 7) * 4;
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     const int row = (t >> 3) + 32 * j;
-    const int slot = min(tile_b * BT + row, n_act - 1);
-    const int xrow = (round > 0) ? pick2(a.st.row, round & 1)[slot] : slot;
-    x_src[j] = xq + (long)xrow * a.k_pad + st_col;
+    if (j < XJ) {
+      const int slot = min(tile_b * BB + row, n_act - 1);
+      const int xrow = (round > 0) ? pick2(a.st.row, round & 1)[slot] : slot;
+      x_src[j] = xq + (long)xrow * a.k_pad + st_col;
+    }
     if (WT == 0) w_src[j] = a.w + (long)min(tile_o * BT + row, a.O - 1) * a.x_size;
   }
   const int wt_o = tile_o * BT + (t & 31) * 4; // WT = 1: first of this thread's four outputs
 
-  auto gload = [&](int s, f32x4 (&gx)[4], f32x4 (&gw)[4]) {
+  auto gload = [&](int s, f32x4 (&gx)[XJ], f32x4 (&gw)[4]) {
     const int k0 = s * BKS;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) gx[j] = *reinterpret_cast<const f32x4 *>(x_src[j] + k0);
+    for (int j = 0; j < XJ; ++j) gx[j] = *reinterpret_cast<const f32x4 *>(x_src[j] + k0);
     if (WT == 0) {
       const int kc = k0 + st_col;
       if (kc + 4 <= K) {
@@ -1397,13 +1420,13 @@ __device__ __forceinline__ void mvm_big_workgroup(const MvmArgs &a, const int ro
       }
     }
   };
-  auto lds_store = [&](int buf, const f32x4 (&gx)[4], const f32x4 (&gw)[4]) {
+  auto lds_store = [&](int buf, const f32x4 (&gx)[XJ], const f32x4 (&gw)[4]) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int row = (t >> 3) + 32 * j;
-      *reinterpret_cast<f32x4 *>(&lds_x[buf][row * BPITCH + st_col]) = gx[j];
+      if (j < XJ) *reinterpret_cast<f32x4 *>(&lds_x[buf][big_lds_offset(row, t & 7)]) = gx[j < XJ ? j : 0];
       if (WT == 0) {
-        *reinterpret_cast<f32x4 *>(&lds_w[buf][row * BPITCH + st_col]) = gw[j];
+        *reinterpret_cast<f32x4 *>(&lds_w[buf][big_lds_offset(row, t & 7)]) = gw[j];
       } else {
         const int krow = (t >> 5) + 8 * j;
         *reinterpret_cast<f32x4 *>(&lds_w[buf][krow * BPITCH_T + (t & 31) * 4]) = gw[j];
@@ -1427,13 +1450,20 @@ __device__ __forceinline__ void mvm_big_workgroup(const MvmArgs &a, const int ro
   struct Operands {
     f32x4 xb0, xb1, wa0, wa1;
   };
+  // staged offsets of this lane's four operand chunks (rows 32 further on: 32 * BROW floats further on)
+  int x_off[4], w_off[4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    x_off[q] = big_lds_offset(wx * (BB / 2) + r, h * 4 + q);
+    w_off[q] = big_lds_offset(wy * 64 + r, h * 4 + q);
+  }
   auto read_operands = [&](int buf, int q, Operands &o) __attribute__((always_inline)) {
     const int kk = h * 16 + q * 4;
-    o.xb0 = *reinterpret_cast<const f32x4 *>(&lds_x[buf][(wx * 64 + r) * BPITCH + kk]);
-    o.xb1 = *reinterpret_cast<const f32x4 *>(&lds_x[buf][(wx * 64 + 32 + r) * BPITCH + kk]);
+    o.xb0 = *reinterpret_cast<const f32x4 *>(&lds_x[buf][x_off[q]]);
+    if (NB == 2) o.xb1 = *reinterpret_cast<const f32x4 *>(&lds_x[buf][x_off[q] + 32 * BROW]);
     if (WT == 0) {
-      o.wa0 = *reinterpret_cast<const f32x4 *>(&lds_w[buf][(wy * 64 + r) * BPITCH + kk]);
-      o.wa1 = *reinterpret_cast<const f32x4 *>(&lds_w[buf][(wy * 64 + 32 + r) * BPITCH + kk]);
+      o.wa0 = *reinterpret_cast<const f32x4 *>(&lds_w[buf][w_off[q]]);
+      o.wa1 = *reinterpret_cast<const f32x4 *>(&lds_w[buf][w_off[q] + 32 * BROW]);
     } else {
       const float *col = &lds_w[buf][kk * BPITCH_T + wy * 64 + r];
       o.wa0.x = col[0];
@@ -1450,9 +1480,9 @@ __device__ __forceinline__ void mvm_big_workgroup(const MvmArgs &a, const int ro
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       acc00 = __builtin_amdgcn_mfma_f32_32x32x2f32(o.wa0[e], o.xb0[e], acc00, 0, 0, 0);
-      acc01 = __builtin_amdgcn_mfma_f32_32x32x2f32(o.wa0[e], o.xb1[e], acc01, 0, 0, 0);
+      if (NB == 2) acc01 = __builtin_amdgcn_mfma_f32_32x32x2f32(o.wa0[e], o.xb1[e], acc01, 0, 0, 0);
       acc10 = __builtin_amdgcn_mfma_f32_32x32x2f32(o.wa1[e], o.xb0[e], acc10, 0, 0, 0);
-      acc11 = __builtin_amdgcn_mfma_f32_32x32x2f32(o.wa1[e], o.xb1[e], acc11, 0, 0, 0);
+      if (NB == 2) acc11 = __builtin_amdgcn_mfma_f32_32x32x2f32(o.wa1[e], o.xb1[e], acc11, 0, 0, 0);
     }
   };
   auto compute = [&](int buf) __attribute__((always_inline)) {
@@ -1460,19 +1490,19 @@ __device__ __forceinline__ void mvm_big_workgroup(const MvmArgs &a, const int ro
     read_operands(buf, 0, even);
     read_operands(buf, 1, odd);
     multiply(even);
-    mvm_big_schedule<WT>();
+    mvm_big_schedule<WT, NB>();
     read_operands(buf, 2, even);
     multiply(odd);
-    mvm_big_schedule<WT>();
+    mvm_big_schedule<WT, NB>();
     read_operands(buf, 3, odd);
     multiply(even);
-    mvm_big_schedule<WT>();
+    mvm_big_schedule<WT, NB>();
     multiply(odd);
   };
 
   const int stages = a.k_pad / BKS;
   {
-    f32x4 gx[4], gw[4];
+    f32x4 gx[XJ], gw[4];
     gload(0, gx, gw);
     lds_store(0, gx, gw);
     __syncthreads();
@@ -1487,13 +1517,13 @@ __device__ __forceinline__ void mvm_big_workgroup(const MvmArgs &a, const int ro
 
   // ADC stage: lane (r, h) of wave (wy, wx) holds, for its 2 x 2 tiles, sample column r and output rows
   // g * 8 + h * 4 + q of each tile
-  if (t < 2 * BT) sh_hits[t] = 0;
+  if (t < 2 * BB) sh_hits[t] = 0;
   __syncthreads();
   const bool flags = !a.io.perfect && a.io.bound_management != RPU_BM_NONE;
   // sample block bi of this wave: its two output blocks
   auto finish_block = [&](const int bi, const floatx16 &acc_o0, const floatx16 &acc_o1) __attribute__((always_inline)) {
-    const int local_b = wx * 64 + bi * 32 + r;
-    const int slot = tile_b * BT + local_b;
+    const int local_b = wx * (BB / 2) + bi * 32 + r;
+    const int slot = tile_b * BB + local_b;
     if (slot >= n_act) return;
     int b_out = slot;
     float fin_out = 1.0f;
@@ -1518,20 +1548,20 @@ __device__ __forceinline__ void mvm_big_workgroup(const MvmArgs &a, const int ro
     }
     if (flags) {
       if (up_max) atomicMax(&sh_hits[local_b], up_max);
-      if (lo_max) atomicMax(&sh_hits[BT + local_b], lo_max);
+      if (lo_max) atomicMax(&sh_hits[BB + local_b], lo_max);
     }
   };
   finish_block(0, acc00, acc10);
-  finish_block(1, acc01, acc11);
+  if (NB == 2) finish_block(1, acc01, acc11);
   if (!flags) return;
   __syncthreads();
-  {
-    const int local_b = t & (BT - 1);
+  if (t < 2 * BB) {
+    const int local_b = t & (BB - 1);
     const int hit = sh_hits[t];
-    const int slot = tile_b * BT + local_b;
+    const int slot = tile_b * BB + local_b;
     if (hit && slot < n_act) {
       const int bs = (round > 0) ? pick2(a.st.list, round & 1)[slot] : slot;
-      const int old = atomicMax(t < BT ? &a.st.hit_up[bs] : &a.st.hit_lo[bs], hit);
+      const int old = atomicMax(t < BB ? &a.st.hit_up[bs] : &a.st.hit_lo[bs], hit);
       asm volatile("" ::"v"(old));
     }
   }
@@ -1540,14 +1570,14 @@ __device__ __forceinline__ void mvm_big_workgroup(const MvmArgs &a, const int ro
   __syncthreads();
   if (t == 0) {
     const int tiles_o = (a.O + BT - 1) / BT;
-    const int tiles_b = (a.m_batch + BT - 1) / BT;
+    const int tiles_b = (a.m_batch + BB - 1) / BB;
     const int prev = atomicAdd(&a.st.tile_done[round * tiles_b + tile_b], 1);
     sh_last = (prev == tiles_o - 1) ? 1 : 0;
   }
   __syncthreads();
   if (!sh_last) return;
-  if (t < BT) {
-    const int slot = tile_b * BT + t;
+  if (t < BB) {
+    const int slot = tile_b * BB + t;
     if (slot < n_act) {
       float scale;
       mvm_advance_sample(a, round, (round > 0) ? pick2(a.st.list, round & 1)[slot] : slot, slot, true, scale);
@@ -1555,19 +1585,19 @@ __device__ __forceinline__ void mvm_big_workgroup(const MvmArgs &a, const int ro
   }
 }
 
-template <int WT>
+template <int WT, int BB>
 __global__ __launch_bounds__(256, 2) void k_mvm_big(MvmArgs a, int min_active) {
-  mvm_big_workgroup<WT>(a, a.round, (int)blockIdx.x, min_active);
+  mvm_big_workgroup<WT, BB>(a, a.round, (int)blockIdx.x, min_active);
 }
 
 // several tiles in one launch (round 0): a tile that is not run by this kernel has no workgroups in the table
-template <int WT>
+template <int WT, int BB>
 __global__ __launch_bounds__(256, 2) void k_mvm_big_group(MvmGroup g, int round) {
   int t = 0;
   while (t + 1 < g.n && (int)blockIdx.x >= g.start[t + 1]) ++t;
   const MvmArgs &a = g.args[t];
   if (round > 0 && round >= a.max_rounds) return;
-  mvm_big_workgroup<WT>(a, round, (int)blockIdx.x - g.start[t], 0);
+  mvm_big_workgroup<WT, BB>(a, round, (int)blockIdx.x - g.start[t], 0);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -2052,16 +2082,28 @@ void launch_mvm_init_group(const MvmGroup &g, int max_k, hipStream_t s) {
 
 constexpr int TAIL_GRID = 1024; // workgroups of a later-round launch when the full grid would be larger
 
-static int big_workgroups(const MvmArgs &a) {
-  const int tiles_o = (a.O + 127) / 128, tiles_b = (a.m_batch + 127) / 128;
+// workgroups of a large-tile launch with sample tiles of `bb` samples
+static int big_workgroups(const MvmArgs &a, int bb) {
+  const int tiles_o = (a.O + 127) / 128, tiles_b = (a.m_batch + bb - 1) / bb;
   return 8 * tiles_o * ((tiles_b + 7) / 8);
 }
 
-int mvm_big_workgroups(const MvmArgs &a) { return a.O >= 128 ? big_workgroups(a) : 0; }
+int mvm_big_workgroups(const MvmArgs &a, int bb) { return a.O >= 128 ? big_workgroups(a, bb) : 0; }
 
-void launch_mvm_big_group(const MvmGroup &g, int total_workgroups, bool transposed, hipStream_t s) {
-  if (transposed) hipLaunchKernelGGL(k_mvm_big_group<1>, dim3(total_workgroups), dim3(256), 0, s, g, 0);
-  else hipLaunchKernelGGL(k_mvm_big_group<0>, dim3(total_workgroups), dim3(256), 0, s, g, 0);
+// Sample-tile edge for a launch that would have `workgroups_128` workgroups with square tiles: a CU holds two
+// workgroups, and fewer than about three per CU leave the chip unevenly filled (384 of them occupy half of the CUs
+// twice as long as the other half); tiles of 64 samples give twice as many workgroups of half the work
+int mvm_big_sample_tile(int workgroups_128, int n_cus) { return 2 * workgroups_128 >= 5 * n_cus ? 128 : 64; }
+
+void launch_mvm_big_group(const MvmGroup &g, int total_workgroups, int bb, bool transposed, hipStream_t s) {
+  const dim3 grid(total_workgroups);
+  if (bb == 128) {
+    if (transposed) hipLaunchKernelGGL((k_mvm_big_group<1, 128>), grid, dim3(256), 0, s, g, 0);
+    else hipLaunchKernelGGL((k_mvm_big_group<0, 128>), grid, dim3(256), 0, s, g, 0);
+  } else {
+    if (transposed) hipLaunchKernelGGL((k_mvm_big_group<1, 64>), grid, dim3(256), 0, s, g, 0);
+    else hipLaunchKernelGGL((k_mvm_big_group<0, 64>), grid, dim3(256), 0, s, g, 0);
+  }
 }
 
 // samples of a round from which the large-tile kernel takes over, 0 when a call of this shape never uses it: it
@@ -2071,6 +2113,18 @@ static int big_threshold(int m_batch, int O) {
   const int tiles_o = (O + 127) / 128, tiles_b = (m_batch + 127) / 128;
   if (8 * tiles_o * ((tiles_b + 7) / 8) < 128) return 0;
   return 2048;
+}
+
+static int current_device_cus() {
+  static int cus[64] = {0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (cus[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cus[dev] = n;
+  }
+  return cus[dev];
 }
 
 bool mvm_uses_large_tiles(int m_batch, int O) { return big_threshold(m_batch, O) > 0; }
@@ -2145,10 +2199,16 @@ void launch_mvm_round(const MvmArgs &a_in, hipStream_t s) {
   MvmArgs a = a_in;
   a.big_from = a.small_tiles_only ? 0 : big_threshold(a.m_batch, a.O);
   if (a.big_from > 0) {
-    const dim3 big_grid(big_workgroups(a));
+    const int bb = mvm_big_sample_tile(big_workgroups(a, 128), current_device_cus());
+    const dim3 big_grid(big_workgroups(a, bb));
     const int min_active = a.round > 0 ? a.big_from : 0;
-    if (a.transposed) hipLaunchKernelGGL(k_mvm_big<1>, big_grid, dim3(256), 0, s, a, min_active);
-    else hipLaunchKernelGGL(k_mvm_big<0>, big_grid, dim3(256), 0, s, a, min_active);
+    if (bb == 128) {
+      if (a.transposed) hipLaunchKernelGGL((k_mvm_big<1, 128>), big_grid, dim3(256), 0, s, a, min_active);
+      else hipLaunchKernelGGL((k_mvm_big<0, 128>), big_grid, dim3(256), 0, s, a, min_active);
+    } else {
+      if (a.transposed) hipLaunchKernelGGL((k_mvm_big<1, 64>), big_grid, dim3(256), 0, s, a, min_active);
+      else hipLaunchKernelGGL((k_mvm_big<0, 64>), big_grid, dim3(256), 0, s, a, min_active);
+    }
     if (a.round == 0) return; // later rounds: whichever kernel the number of listed samples calls for
   }
   const int all = mvm_round_workgroups(a);

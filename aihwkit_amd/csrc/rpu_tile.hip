@@ -2119,16 +2119,26 @@ static int group_mvm(rpu_group_t *group, const float *const *x_dev, const long *
 
     // a batch of 1024 or more on tiles at least 128 outputs wide: the large-tile kernel runs round 0 of those tiles,
     // if the group has enough of its workgroups to fill the chip
-    int big_total = 0;
+    int big_total = 0, big_bb = 128;
     if (m_batch >= 1024) {
+      if (group->cu_count == 0) {
+        hipDeviceProp_t prop;
+        RPU_HIP_CHECK(hipGetDeviceProperties(&prop, group->device_id));
+        group->cu_count = prop.multiProcessorCount;
+      }
+      int total_128 = 0, total_64 = 0;
       for (int i = 0; i < n; ++i) {
         MvmArgs shape{};
         shape.O = transposed ? group->tiles[i]->t.X : group->tiles[i]->t.D;
         shape.m_batch = m_batch;
-        big_total += mvm_big_workgroups(shape);
+        total_128 += mvm_big_workgroups(shape, 128);
+        total_64 += mvm_big_workgroups(shape, 64);
       }
+      big_bb = mvm_big_sample_tile(total_128, group->cu_count);
+      big_total = big_bb == 128 ? total_128 : total_64;
     }
-    const bool use_big = big_total >= 256;
+    // with the half tiles, one workgroup on every second CU already beats the 32 x 32 kernel
+    const bool use_big = big_total >= (big_bb == 128 ? 256 : 128);
     bool all_big = use_big;
     // per tile: arguments of a plain forward call (row-major x [m_batch][x_size], y [m_batch][d_size])
     std::vector<MvmArgs> args(n);
@@ -2247,7 +2257,7 @@ static int group_mvm(rpu_group_t *group, const float *const *x_dev, const long *
       int wg = 0;
       for (int i = 0; i < n; ++i) {
         group->h_start[cursor++] = wg;
-        if (args[order[i]].big_from != 0) wg += mvm_big_workgroups(args[order[i]]);
+        if (args[order[i]].big_from != 0) wg += mvm_big_workgroups(args[order[i]], big_bb);
       }
       group->h_start[cursor++] = wg;
     }
@@ -2273,7 +2283,7 @@ static int group_mvm(rpu_group_t *group, const float *const *x_dev, const long *
     for (int r = 0; r < rounds; ++r) {
       if (use_big && r == 0) {
         MvmGroup g{group->d_args.p, group->d_start.p + big_offset, n, m_batch};
-        launch_mvm_big_group(g, big_total, transposed, s);
+        launch_mvm_big_group(g, big_total, big_bb, transposed, s);
         if (all_big) continue;
       }
       for (size_t k = 0; k < segments.size(); ++k) {
