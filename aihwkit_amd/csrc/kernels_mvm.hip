@@ -1776,7 +1776,7 @@ __global__ __launch_bounds__(256, 2) void k_conv_forward(MvmArgs a, ConvArgs c) 
 // Long patch rows (more than two contraction steps): one workgroup per 32 patches, its four waves share the patches
 // and deal the contraction steps among themselves (partial sums added through LDS in a fixed order, each wave then
 // finishes 8 of the 32 output rows).  Every wave keeps the per-patch state, so the round loop is workgroup-uniform.
-__global__ __launch_bounds__(256) void k_conv_forward_split(MvmArgs a, ConvArgs c) {
+__global__ __launch_bounds__(256, 4) void k_conv_forward_split(MvmArgs a, ConvArgs c) {
   __shared__ float red[WAVES][16][64];
   __shared__ float sh_max[2][WAVES][32];
   __shared__ int sh_hits[2][32];
