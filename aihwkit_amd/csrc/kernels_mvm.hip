@@ -56,13 +56,16 @@ constexpr int TILE = 32;
 constexpr int WAVES = 4;
 constexpr int KSTEP = 32; // k-values per wave step: 128 bytes per operand row
 
+// STOCH = false: for callers that have checked that the DAC draws no random numbers (no stochastic rounding, no input
+// noise): the draws are then not even compiled in, which the fully unrolled callers pay for in registers
+template <bool STOCH = true>
 __device__ __forceinline__ float dac_value(float x, float scale, const IoDev &io, PhiloxKey key,
                                            uint32_t call, int round, int b, int k) {
   // value *= scale; discretize; clip; (+ noise); (asymmetry)      rpu_forward_backward_pass.cpp:583-602
   float v = x * scale;
   if (io.inp_res > 0.0f) {
     float q = v / io.inp_res;
-    if (io.inp_sto_round) {
+    if (STOCH && io.inp_sto_round) {
       const Philox4 r = philox4x32_10((uint32_t)k, (uint32_t)b, call, RNG_INP_SR | ((uint32_t)round << 8), key.k0, key.k1);
       q = q + (u32_to_uniform(r.v[0]) - 0.5f);
     }
@@ -70,7 +73,7 @@ __device__ __forceinline__ float dac_value(float x, float scale, const IoDev &io
   }
   v = (v > io.inp_bound) ? io.inp_bound : v;
   v = (v < -io.inp_bound) ? -io.inp_bound : v;
-  if (io.inp_noise > 0.0f) {
+  if (STOCH && io.inp_noise > 0.0f) {
     float n[4];
     philox_normal4((uint32_t)k, (uint32_t)b, call, RNG_INP_NOISE | ((uint32_t)round << 8), key, n);
     v += io.inp_noise * n[0];
@@ -128,6 +131,8 @@ __host__ __device__ __forceinline__ int workgroups_for(int O, int n_act, int edg
 
 // ADC of the four analog sums v of outputs o0 .. o0 + 3 of sample b: asymmetry, noise, quantization, clipping, output
 // factor; up / lo return 1 + the largest output index that hit the upper / lower bound (0: none)
+// STOCH = false: for callers that have checked that the ADC does not round stochastically
+template <bool STOCH = true>
 __device__ __forceinline__ void mvm_adc_values(const MvmArgs &a, int round, int b, float fin, int o0, float (&v)[4],
                                                int &up, int &lo, const float *pre = nullptr, const float *post = nullptr) {
   float nz[4] = {0.f, 0.f, 0.f, 0.f};
@@ -145,7 +150,7 @@ __device__ __forceinline__ void mvm_adc_values(const MvmArgs &a, int round, int 
     if (a.io.out_noise > 0.0f) y += a.io.out_noise * nz[q];
     if (a.io.out_res > 0.0f) {
       float qq = y / a.io.out_res;
-      if (a.io.out_sto_round) {
+      if (STOCH && a.io.out_sto_round) {
         const Philox4 rr = philox4x32_10((uint32_t)(o0 + q), (uint32_t)b, a.call, RNG_OUT_SR | ((uint32_t)round << 8), a.key.k0, a.key.k1);
         qq = qq + (u32_to_uniform(rr.v[0]) - 0.5f);
       }
@@ -1613,8 +1618,9 @@ typedef int i32x4_unaligned __attribute__((ext_vector_type(4), aligned(4)));
 
 // ONE_STEP: the patch row fits one contraction step (K <= 32, a first convolution layer): the gathered values stay
 // in registers between noise management and the rounds.
-template <bool ONE_STEP>
-__global__ __launch_bounds__(256, 2) void k_conv_forward(MvmArgs a, ConvArgs c) {
+// STOCH: the DAC or the ADC draws random numbers beyond the output noise (see dac_value, mvm_adc_values).
+template <bool ONE_STEP, bool STOCH>
+__global__ __launch_bounds__(256, STOCH ? 2 : 3) void k_conv_forward(MvmArgs a, ConvArgs c) {
   const int lane = threadIdx.x & 63;
   const int r = lane & 31, h = lane >> 5;
   const long tile = blockIdx.x * 4L + (threadIdx.x >> 6);
@@ -1716,7 +1722,7 @@ __global__ __launch_bounds__(256, 2) void k_conv_forward(MvmArgs a, ConvArgs c) 
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
           float x = ONE_STEP ? x_keep[i] : xd[i];
-          if (!io.perfect && k0 + i < K) x = dac_value(x, scale, io, a.key, a.call, round, b, k0 + i);
+          if (!io.perfect && k0 + i < K) x = dac_value<STOCH>(x, scale, io, a.key, a.call, round, b, k0 + i);
           xd[i] = x;
         }
 #pragma unroll
@@ -1740,7 +1746,7 @@ __global__ __launch_bounds__(256, 2) void k_conv_forward(MvmArgs a, ConvArgs c) 
 #pragma unroll
         for (int q = 0; q < 4; ++q) v[q] = 0.0f;
       } else {
-        mvm_adc_values(a, round, b, fin, o0, v, up, lo);
+        mvm_adc_values<STOCH>(a, round, b, fin, o0, v, up, lo);
       }
       if (active) {
 #pragma unroll
@@ -1776,6 +1782,7 @@ __global__ __launch_bounds__(256, 2) void k_conv_forward(MvmArgs a, ConvArgs c) 
 // Long patch rows (more than two contraction steps): one workgroup per 32 patches, its four waves share the patches
 // and deal the contraction steps among themselves (partial sums added through LDS in a fixed order, each wave then
 // finishes 8 of the 32 output rows).  Every wave keeps the per-patch state, so the round loop is workgroup-uniform.
+template <bool STOCH>
 __global__ __launch_bounds__(256, 4) void k_conv_forward_split(MvmArgs a, ConvArgs c) {
   __shared__ float red[WAVES][16][64];
   __shared__ float sh_max[2][WAVES][32];
@@ -1880,7 +1887,7 @@ __global__ __launch_bounds__(256, 4) void k_conv_forward_split(MvmArgs a, ConvAr
         weights16(k0, wd);
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-          if (!io.perfect && k0 + i < K) xd[i] = dac_value(xd[i], scale, io, a.key, a.call, round, b, k0 + i);
+          if (!io.perfect && k0 + i < K) xd[i] = dac_value<STOCH>(xd[i], scale, io, a.key, a.call, round, b, k0 + i);
         }
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(wd[i], xd[i], acc, 0, 0, 0);
@@ -1908,7 +1915,7 @@ __global__ __launch_bounds__(256, 4) void k_conv_forward_split(MvmArgs a, ConvAr
 #pragma unroll
           for (int q = 0; q < 4; ++q) v[q] = 0.0f;
         } else {
-          mvm_adc_values(a, round, b, fin, o0, v, up, lo);
+          mvm_adc_values<STOCH>(a, round, b, fin, o0, v, up, lo);
         }
         if (active) {
 #pragma unroll
@@ -2264,9 +2271,16 @@ bool conv_forward_supported(const MvmArgs &a) {
 void launch_conv_forward(const MvmArgs &a, const ConvArgs &c, hipStream_t s) {
   const long tiles = ((long)c.n_images * c.patches + 31) / 32;
   const dim3 grid((unsigned)((tiles + 3) / 4));
-  if (a.K <= 32) hipLaunchKernelGGL(k_conv_forward<true>, grid, dim3(256), 0, s, a, c);
-  else if (a.K <= 64) hipLaunchKernelGGL(k_conv_forward<false>, grid, dim3(256), 0, s, a, c);
-  else hipLaunchKernelGGL(k_conv_forward_split, dim3((unsigned)tiles), dim3(256), 0, s, a, c);
+  const bool stoch = !a.io.perfect && (a.io.inp_sto_round || a.io.out_sto_round || a.io.inp_noise > 0.0f);
+  if (stoch) {
+    if (a.K <= 32) hipLaunchKernelGGL((k_conv_forward<true, true>), grid, dim3(256), 0, s, a, c);
+    else if (a.K <= 64) hipLaunchKernelGGL((k_conv_forward<false, true>), grid, dim3(256), 0, s, a, c);
+    else hipLaunchKernelGGL(k_conv_forward_split<true>, dim3((unsigned)tiles), dim3(256), 0, s, a, c);
+  } else {
+    if (a.K <= 32) hipLaunchKernelGGL((k_conv_forward<true, false>), grid, dim3(256), 0, s, a, c);
+    else if (a.K <= 64) hipLaunchKernelGGL((k_conv_forward<false, false>), grid, dim3(256), 0, s, a, c);
+    else hipLaunchKernelGGL(k_conv_forward_split<false>, dim3((unsigned)tiles), dim3(256), 0, s, a, c);
+  }
 }
 
 void launch_make_bias(const float *in, float *out, int m_batch, int x_size, int in_trans, hipStream_t s) {

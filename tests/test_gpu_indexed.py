@@ -146,3 +146,46 @@ def test_zero_patches_beside_others_without_a_bias_column(gpu_device, c_in, kern
     assert (rounds == 0).sum() >= patches and (rounds[:patches] == 0).any() and (rounds[:patches] > 0).any()
     assert np.array_equal(y, want)
     assert np.array_equal(gpu.get_bm_rounds(n * patches).numpy(), rounds)
+
+
+@pytest.mark.parametrize("c_in,kernel", [(2, 3), (5, 3), (16, 5)])   # patch rows of 19, 46 and 401 elements: the three kernels
+@pytest.mark.parametrize("stochastic", [False, True])
+def test_fused_convolution_forward_draws_what_the_unfolded_pass_draws(gpu_device, c_in, kernel, stochastic):
+    """The fused convolution kernels key their random draws by (patch row element, patch number) like the ordinary
+    forward pass on the unfolded patch matrix: with output noise, and with DAC / ADC stochastic rounding and input noise
+    (the kernel variants that compile those draws in), a tile gives on the images what a twin with the same seed gives on
+    the explicitly unfolded matrix -- up to the summation order of the contraction, which can move a value across one ADC
+    rounding edge."""
+    from indexed_oracle import copy_indexed_input
+    from helpers import io_params, soft_bounds
+    rng = np.random.default_rng(31 + c_in)
+    c_out, height, width, n = 24, 10, 9, 7
+    indices, patches = conv_indices((c_in, height, width), (kernel, kernel), (1, 1), (1, 1), (1, 1), True)
+    x_size = c_in * kernel * kernel + 1
+    out_res, out_bound = 1 / 4096.0, 16.0
+    io = io_params(inp_res=1 / 256.0, out_res=out_res, out_bound=out_bound, out_noise=0.05,
+                   inp_noise=0.01 if stochastic else 0.0, inp_sto_round=stochastic, out_sto_round=stochastic,
+                   noise_management=dv.NoiseManagementType.AbsMax, bound_management=dv.BoundManagementType.Iterative)
+    meta = make_meta(io, noise_free_io())
+    host, _orc, _ = build_pair(meta, soft_bounds(construction_seed=4), x_size, c_out, gpu=False)
+    host.set_weights(torch.from_numpy(rng.uniform(-0.3, 0.3, (c_out, x_size)).astype(np.float32)))
+    conv, plain = tiles.CudaAnalogTile(host), tiles.CudaAnalogTile(host)
+    conv.set_matrix_indices(indices)
+    x = rng.uniform(-1, 1, (n, c_in, height, width)).astype(np.float32)
+    x[1] = 0.0
+    unfolded = copy_indexed_input(x.reshape(n, -1), indices.numpy().reshape(-1).astype(np.int64), x_size, patches)  # [X, N P]
+    for call in range(2):
+        conv.set_seed(900 + call)
+        plain.set_seed(900 + call)
+        y = conv.forward_indexed(cuda(x), torch.empty(n, c_out, 1, patches).cuda()).cpu().numpy().reshape(n, c_out, patches)
+        y_rows = plain.forward(cuda(unfolded.T)).cpu().numpy()                                  # [N P, D]
+        want = y_rows.reshape(n, patches, c_out).transpose(0, 2, 1)
+        assert np.array_equal(conv.get_bm_rounds(n * patches).numpy(), plain.get_bm_rounds(n * patches).numpy())
+        diff = np.abs(y - want)
+        # one ADC step (the range 2 out_bound in 1 / out_res steps) in output units: the abs-max scale of a patch is below
+        # 1.2, and each further round doubles it
+        rounds = plain.get_bm_rounds(n * patches).numpy().reshape(n, 1, patches)
+        step = 2 * out_res * out_bound * 1.2 * np.exp2(np.maximum(rounds, 1) - 1)
+        assert (diff <= step * 1.01).all()
+        assert (diff > 1e-5).mean() < 0.002
+        assert np.abs(want).max() > 0.5
