@@ -100,10 +100,32 @@ __global__ __launch_bounds__(256) void k_pcm_drift(const float *w_prog, const fl
   }
 }
 
+// One workgroup, so that the order of the sum is fixed; eight 16-byte loads per thread are in flight at a time (one
+// load per trip made the kernel a chain of 256 memory latencies for a 512 x 512 tile).
 __global__ __launch_bounds__(1024) void k_mean_abs(const float *v, size_t n, float *out) {
   __shared__ float sh[16];
   float acc = 0.0f;
-  for (size_t i = threadIdx.x; i < n; i += blockDim.x) acc += fabsf(v[i]);
+  size_t done = 0;
+  if ((((uintptr_t)v) & 15) == 0) {
+    const size_t n4 = n >> 2;
+    const float4 *v4 = reinterpret_cast<const float4 *>(v);
+    float part[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) part[u] = 0.0f;
+    for (size_t q0 = 0; q0 < n4; q0 += 8 * (size_t)blockDim.x) {
+      float4 t[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const size_t q = q0 + (size_t)u * blockDim.x + threadIdx.x;
+        t[u] = q < n4 ? v4[q] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) part[u] += (fabsf(t[u].x) + fabsf(t[u].y)) + (fabsf(t[u].z) + fabsf(t[u].w));
+    }
+    acc = ((part[0] + part[1]) + (part[2] + part[3])) + ((part[4] + part[5]) + (part[6] + part[7]));
+    done = 4 * n4;
+  }
+  for (size_t i = done + threadIdx.x; i < n; i += blockDim.x) acc += fabsf(v[i]);
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off);
   if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = acc;
