@@ -50,40 +50,50 @@ __device__ __forceinline__ void calc_bl_ab(const UpdateDev &up, int &BL, float &
   }
 }
 
-// largest absolute value of a line of n elements (element j at v[j * stride]) over the lanes of a wave; rows that are
-// contiguous and 16-byte aligned are read four elements at a time
-__device__ __forceinline__ float wave_abs_max(const float *v, int n, long stride) {
-  const int lane = threadIdx.x & 63;
+// largest absolute value of a line of n elements (element j at v[j * stride]) over the part that thread `t` of `width`
+// takes; rows that are contiguous and 16-byte aligned are read four elements at a time
+__device__ __forceinline__ float part_abs_max(const float *v, int n, long stride, int t, int width) {
   float m = 0.0f;
   if (stride == 1 && ((((uintptr_t)v) & 15) == 0)) {
     const int n4 = n >> 2;
     const float4 *v4 = reinterpret_cast<const float4 *>(v);
-    for (int q = lane; q < n4; q += 64) {
-      const float4 t = v4[q];
-      m = fmaxf(fmaxf(m, fmaxf(fabsf(t.x), fabsf(t.y))), fmaxf(fabsf(t.z), fabsf(t.w)));
+    for (int q = t; q < n4; q += width) {
+      const float4 x = v4[q];
+      m = fmaxf(fmaxf(m, fmaxf(fabsf(x.x), fabsf(x.y))), fmaxf(fabsf(x.z), fabsf(x.w)));
     }
-    for (int j = 4 * n4 + lane; j < n; j += 64) m = fmaxf(m, fabsf(v[j]));
+    for (int j = 4 * n4 + t; j < n; j += width) m = fmaxf(m, fabsf(v[j]));
   } else {
-    for (int j = lane; j < n; j += 64) m = fmaxf(m, fabsf(v[(long)j * stride]));
+    for (int j = t; j < n; j += width) m = fmaxf(m, fabsf(v[(long)j * stride]));
   }
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off));
   return m;
 }
 
-// one wave per sample: no barrier between the two line maxima and the sample's BL, A, B
+// One workgroup per sample: the loads of both lines are in flight together (a line of 1024 elements is one 16-byte load
+// per thread), then one exchange through LDS gives the first thread both maxima and it sets the sample's BL, A, B.
 __global__ __launch_bounds__(256) void k_update_prepare(UpdateArgs a) {
-  const int b = blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (b >= a.m_batch) return;
-  const bool leader = (threadIdx.x & 63) == 0;
+  __shared__ float sh[2][4];
+  const int b = blockIdx.x;
+  const bool leader = threadIdx.x == 0;
   const float lr = fabsf(a.lr);
   const float dw_min = a.dev.dw_min;
   int BL;
   float A, B;
   if (a.up.update_management || a.up.update_bl_management) {
-    const float xm = wave_abs_max(a.x + (long)b * a.x_sb, a.x_size, a.x_sj);
-    const float dm = wave_abs_max(a.d + (long)b * a.d_sb, a.d_size, a.d_si);
+    float xm = part_abs_max(a.x + (long)b * a.x_sb, a.x_size, a.x_sj, threadIdx.x, 256);
+    float dm = part_abs_max(a.d + (long)b * a.d_sb, a.d_size, a.d_si, threadIdx.x, 256);
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+      xm = fmaxf(xm, __shfl_xor(xm, off));
+      dm = fmaxf(dm, __shfl_xor(dm, off));
+    }
+    if ((threadIdx.x & 63) == 0) {
+      sh[0][threadIdx.x >> 6] = xm;
+      sh[1][threadIdx.x >> 6] = dm;
+    }
+    __syncthreads();
     if (!leader) return;
+    xm = fmaxf(fmaxf(sh[0][0], sh[0][1]), fmaxf(sh[0][2], sh[0][3]));
+    dm = fmaxf(fmaxf(sh[1][0], sh[1][1]), fmaxf(sh[1][2], sh[1][3]));
     // rpu_pulsed_meta_parameter.cpp:183-236
     calc_bl_ab(a.up, BL, A, B, lr, dw_min);
     if (lr > 0.0f) {
@@ -1100,7 +1110,7 @@ int grid_for(long total) {
 } // namespace
 
 void launch_update_prepare(const UpdateArgs &a, hipStream_t s) {
-  hipLaunchKernelGGL(k_update_prepare, dim3((a.m_batch + 3) / 4), dim3(256), 0, s, a);
+  hipLaunchKernelGGL(k_update_prepare, dim3(a.m_batch), dim3(256), 0, s, a);
 }
 
 void launch_update_lines(const UpdateArgs &a, hipStream_t s) {
