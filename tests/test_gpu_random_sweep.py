@@ -279,10 +279,14 @@ def one_group(seed):
     n_tiles = int(rng.choice([1, 2, 3, 5, 9, 17]))
     batch = int(rng.choice([1, 7, 33, 96, 257, 1024, 1100, 2048]))
     strided = bool(rng.integers(2))
+    # one in three: the tiles of a split layer, all handed the same input (those with equal DAC settings then share its
+    # quantized rows)
+    shared_input = n_tiles > 1 and rng.integers(3) == 0
+    common_x = int(rng.choice([3, 33, 64, 96, 130, 257]))
     grouped, oracles, xs, ds, shapes = [], [], [], [], []
     budget = 40_000_000
     for k in range(n_tiles):
-        x_size = int(rng.choice([1, 3, 31, 33, 64, 70, 96, 129, 130, 257]))
+        x_size = common_x if shared_input else int(rng.choice([1, 3, 31, 33, 64, 70, 96, 129, 130, 257]))
         d_size = int(rng.choice([1, 5, 32, 40, 127, 128, 129, 256, 300, 512]))
         if x_size * d_size * batch > budget // n_tiles:
             d_size = max(1, (budget // n_tiles) // (x_size * batch))
@@ -301,11 +305,17 @@ def one_group(seed):
         grouped.append(tiles.CudaAnalogTile(host))
         oracles.append(orc)
         shapes.append((x_size, d_size))
-        xs.append((rng.integers(-64, 65, (batch, x_size)) / 64.0).astype(np.float32))
+        x_new = (rng.integers(-64, 65, (batch, x_size)) / 64.0).astype(np.float32)
+        xs.append(xs[0] if shared_input and k > 0 else x_new)
         ds.append((rng.integers(-64, 65, (batch, d_size)) / 64.0).astype(np.float32))
     group = tiles.TileGroup(grouped)
-    desc = dict(seed=seed, n=n_tiles, B=batch, strided=strided, shapes=shapes)
-    if strided:
+    desc = dict(seed=seed, n=n_tiles, B=batch, strided=strided, shapes=shapes, shared_input=shared_input)
+    if shared_input:
+        one_x = torch.cat([cuda(xs[0]), torch.zeros(batch, 3, device="cuda")], dim=1)       # a column slice, rows 12 bytes longer
+        outs = [torch.full((batch, d), 7.0, device="cuda") for _, d in shapes]
+        got = group.forward([one_x[:, :common_x]] * n_tiles, outs=outs)
+        got = group.forward([one_x[:, :common_x]] * n_tiles, outs=outs)                      # again, on the buffers of the first call
+    elif strided:
         all_x = torch.cat([cuda(x) for x in xs], dim=1)
         x_in, i0 = [], 0
         for x_size, _ in shapes:
