@@ -663,6 +663,7 @@ def bench_config4(args) -> int:
         if indices is not None:
             tile.set_matrix_indices(indices)
         tile.drift_weights(86400.0)
+        tile.compensate_in_tile(True)      # the drift-compensation factor rides on the ADC stage: no multiply of the output
         stack.append((kind, tile, patches, out_size))
         host_weights.append(w)
         flops += 2.0 * batch * patches * in_size * out_size

@@ -297,6 +297,32 @@ def test_group_reads_and_writes_column_slices_and_compensation_in_the_tile(gpu_d
         group.forward([s.t() for s in x_slices])
 
 
+@pytest.mark.parametrize("c_in,c_out", [(1, 16), (16, 32), (4, 48)])     # the two fused kernels and the unfolded path
+def test_compensation_in_the_tile_for_a_convolution(gpu_device, c_in, c_out):
+    """The drift-compensation factor on the ADC stage of the indexed forward equals the multiply of its output."""
+    from aihwkit_amd.benchmark_configs import conv_index_matrix
+
+    rng = np.random.default_rng(c_out)
+    f_io = io_params(inp_res=1 / 254.0, out_res=1 / 254.0, out_noise=0.04, noise_management=dv.NoiseManagementType.AbsMax,
+                     bound_management=dv.BoundManagementType.Iterative)
+    indices, patches = conv_index_matrix((c_in, 12, 12), (5, 5))
+    in_size = c_in * 25 + 1
+    t = InferenceTile(c_out, in_size, forward_io=f_io)
+    t.set_weights(torch.from_numpy((rng.uniform(-1, 1, (c_out, in_size)) / np.sqrt(in_size)).astype(np.float32)))
+    t.cuda()
+    t.set_matrix_indices(indices)
+    t.drift_weights(86400.0)
+    assert abs(t.alpha - 1.0) > 1e-3
+    x = torch.from_numpy(rng.uniform(0, 1, (6, c_in, 12, 12)).astype(np.float32)).cuda()
+    t.tile.set_seed(9)
+    y_mul = t.forward_indexed(x, torch.empty(6, c_out, 8, 8, device="cuda"), is_test=True).clone()
+    t.compensate_in_tile(True)
+    t.tile.set_seed(9)
+    y_tile = t.forward_indexed(x, torch.empty(6, c_out, 8, 8, device="cuda"), is_test=True)
+    assert patches == 64 and y_mul.abs().max() > 0.1
+    assert torch.allclose(y_tile, y_mul, rtol=1e-6, atol=1e-7)
+
+
 def test_grouped_backward_equals_the_tiles_own_backward(gpu_device):
     """Noisy backward pass (abs-max noise management) of tiles of different shapes: the group call gives every tile bit
     for bit what its own backward call gives for the same seed and call counter; strided gradients are filled in place."""
