@@ -164,9 +164,11 @@ class InferenceTile:
             out.mul_(self.alpha)
         return out
 
-    def forward(self, x_input: torch.Tensor, is_test: bool = False) -> torch.Tensor:
-        """Analog forward; in evaluation mode the output is scaled by the drift compensation (inference.py:264-282)."""
-        out = self._gpu().forward(x_input, False, False, False, is_test, False)
+    def forward(self, x_input: torch.Tensor, is_test: bool = False, bias: bool = False) -> torch.Tensor:
+        """Analog forward; in evaluation mode the output is scaled by the drift compensation (inference.py:264-282).
+        ``bias``: the tile's last input column is the bias column and ``x_input`` comes without it (the tile adds the
+        column of ones, as the reference's ``forward(x_input, bias=True)`` does)."""
+        out = self._gpu().forward(x_input, bias, False, False, is_test, False)
         if is_test and self.drift_compensation is not None and self.alpha != 1.0 and not self._alpha_in_tile:
             out = out * self.alpha
         return out

@@ -668,7 +668,6 @@ def bench_config4(args) -> int:
         host_weights.append(w)
         flops += 2.0 * batch * patches * in_size * out_size
     x = torch.from_numpy(rng.uniform(0, 1, (batch, 1, 28, 28)).astype(np.float32)).cuda()
-    ones = torch.ones(batch, 1, device="cuda")
 
     def step():
         h = x
@@ -678,7 +677,7 @@ def bench_config4(args) -> int:
                 y = tile.forward_indexed(h, torch.empty(h.size(0), out_size, side, side, device="cuda"), is_test=True)
                 h = F.max_pool2d(torch.tanh(y), 2)
             else:
-                h = tile.forward(torch.cat([h.reshape(h.size(0), -1), ones], dim=1), is_test=True)
+                h = tile.forward(h.reshape(h.size(0), -1), is_test=True, bias=True)     # the tile adds the bias column
                 if out_size != 10:
                     h = torch.tanh(h)
         return h
