@@ -283,12 +283,14 @@ def one_group(seed):
     # quantized rows)
     shared_input = n_tiles > 1 and rng.integers(3) == 0
     common_x = int(rng.choice([3, 33, 64, 96, 130, 257]))
+    shared_grad = n_tiles > 1 and rng.integers(3) == 0           # likewise for the backward pass: one output gradient
+    common_d = int(rng.choice([5, 32, 40, 128, 129, 300]))
     grouped, oracles, xs, ds, shapes = [], [], [], [], []
     budget = 40_000_000
     for k in range(n_tiles):
         x_size = common_x if shared_input else int(rng.choice([1, 3, 31, 33, 64, 70, 96, 129, 130, 257]))
-        d_size = int(rng.choice([1, 5, 32, 40, 127, 128, 129, 256, 300, 512]))
-        if x_size * d_size * batch > budget // n_tiles:
+        d_size = common_d if shared_grad else int(rng.choice([1, 5, 32, 40, 127, 128, 129, 256, 300, 512]))
+        if x_size * d_size * batch > budget // n_tiles and not shared_grad:
             d_size = max(1, (budget // n_tiles) // (x_size * batch))
         nm = [NM.NONE, NM.AbsMax, NM.Max][rng.integers(3)]
         bm = [BM.NONE, BM.Iterative][rng.integers(2)]
@@ -307,9 +309,10 @@ def one_group(seed):
         shapes.append((x_size, d_size))
         x_new = (rng.integers(-64, 65, (batch, x_size)) / 64.0).astype(np.float32)
         xs.append(xs[0] if shared_input and k > 0 else x_new)
-        ds.append((rng.integers(-64, 65, (batch, d_size)) / 64.0).astype(np.float32))
+        d_new = (rng.integers(-64, 65, (batch, d_size)) / 64.0).astype(np.float32)
+        ds.append(ds[0] if shared_grad and k > 0 else d_new)
     group = tiles.TileGroup(grouped)
-    desc = dict(seed=seed, n=n_tiles, B=batch, strided=strided, shapes=shapes, shared_input=shared_input)
+    desc = dict(seed=seed, n=n_tiles, B=batch, strided=strided, shapes=shapes, shared_input=shared_input, shared_grad=shared_grad)
     if shared_input:
         one_x = torch.cat([cuda(xs[0]), torch.zeros(batch, 3, device="cuda")], dim=1)       # a column slice, rows 12 bytes longer
         outs = [torch.full((batch, d), 7.0, device="cuda") for _, d in shapes]
@@ -334,7 +337,13 @@ def one_group(seed):
         if not np.array_equal(y.cpu().numpy(), orc.forward(x)):
             ok = False
             desc.setdefault("fwd_bad", []).append(k)
-    gb = group.backward([cuda(d) for d in ds])
+    if shared_grad:
+        one_d = cuda(ds[0])
+        gb = group.backward([one_d] * n_tiles)
+        gb = group.backward([one_d] * n_tiles)                     # again, on the buffers of the first call
+        desc["bwd_sets"] = group.get_shared_input_sets()
+    else:
+        gb = group.backward([cuda(d) for d in ds])
     for k, (g, orc, d) in enumerate(zip(gb, oracles, ds)):
         if not np.array_equal(g.cpu().numpy(), orc.backward(d)):
             ok = False
