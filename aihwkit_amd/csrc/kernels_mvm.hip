@@ -2097,10 +2097,18 @@ static int big_workgroups(const MvmArgs &a, int bb) {
 
 int mvm_big_workgroups(const MvmArgs &a, int bb) { return a.O >= 128 ? big_workgroups(a, bb) : 0; }
 
-// Sample-tile edge for a launch that would have `workgroups_128` workgroups with square tiles: a CU holds two
-// workgroups, and fewer than about three per CU leave the chip unevenly filled (384 of them occupy half of the CUs
-// twice as long as the other half); tiles of 64 samples give twice as many workgroups of half the work
-int mvm_big_sample_tile(int workgroups_128, int n_cus) { return 2 * workgroups_128 >= 5 * n_cus ? 128 : 64; }
+// Sample-tile edge for a launch that would have `workgroups_128` workgroups with square tiles.  A CU holds two of
+// those, so they run in rounds of 2 n_cus: where the last round is (nearly) full they are the better choice (more
+// multiply-adds per byte staged), otherwise its idle CUs cost more than that (384 workgroups occupy half of the CUs
+// twice as long as the other half) and tiles of 64 samples, three to a CU, fill the chip more evenly.  Measured on
+// the 1024 x 1024 tile: batch 8192 and 16384 (exactly one and two rounds) are 7 .. 12 % faster with 128, every other
+// batch between 2048 and 20480 with 64 (up to 35 % at 2048, 18 % at 10240).
+int mvm_big_sample_tile(int workgroups_128, int n_cus) {
+  const int slots = 2 * n_cus;
+  const int rounds = (workgroups_128 + slots - 1) / slots;
+  const int idle = rounds * slots - workgroups_128;
+  return 10 * idle <= rounds * slots ? 128 : 64;
+}
 
 void launch_mvm_big_group(const MvmGroup &g, int total_workgroups, int bb, bool transposed, hipStream_t s) {
   const dim3 grid(total_workgroups);

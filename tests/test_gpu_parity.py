@@ -41,8 +41,8 @@ def test_philox_known_answers_on_device(gpu_device):
 @pytest.mark.parametrize("x_size,d_size,batch", [(64, 32, 32), (100, 70, 33), (512, 512, 100), (1024, 1024, 256),
                                                  # large workgroup tiles: 128 outputs x 64 samples ...
                                                  (1024, 1024, 4096), (777, 1000, 4700),
-                                                 # ... and x 128 samples (640 of them), forward / backward
-                                                 (96, 1024, 10240), (1024, 96, 10240)])
+                                                 # ... and x 128 samples (512 of them: two on every CU), forward / backward
+                                                 (96, 1024, 8192), (1024, 96, 8192)])
 @pytest.mark.parametrize("bm", [dv.BoundManagementType.NONE, dv.BoundManagementType.Iterative])
 def test_forward_exact_arithmetic_is_bit_exact(gpu_device, x_size, d_size, batch, bm):
     """With a power-of-two DAC step and weights on a 1/64 grid every product and partial sum is exact in
