@@ -2122,12 +2122,15 @@ void launch_mvm_big_group(const MvmGroup &g, int total_workgroups, int bb, bool 
 }
 
 // samples of a round from which the large-tile kernel takes over, 0 when a call of this shape never uses it: it
-// needs outputs for a whole 128-wide tile and enough tiles to fill half the chip
+// needs outputs for a whole 128-wide tile and enough half tiles for every second CU
 static int big_threshold(int m_batch, int O) {
-  if (m_batch < 2048 || O < 128) return 0;
-  const int tiles_o = (O + 127) / 128, tiles_b = (m_batch + 127) / 128;
+  // measured on the 1024 x 1024 tile: the half tiles overtake the 32 x 32 kernel at about 1500 samples (backward 70
+  // against 88 us at 1536, 74 against 113 us at 2000; at 1024 the 32 x 32 kernel still leads, 63 against 68 us)
+  constexpr int big_min = 1536;
+  if (m_batch < big_min || O < 128) return 0;
+  const int tiles_o = (O + 127) / 128, tiles_b = (m_batch + 63) / 64;
   if (8 * tiles_o * ((tiles_b + 7) / 8) < 128) return 0;
-  return 2048;
+  return big_min;
 }
 
 static int current_device_cus() {
