@@ -2157,6 +2157,7 @@ void launch_mvm_round_group(const MvmGroup &g, int depth, int mode, int total_wo
     return;
   }
   const dim3 grid(total_workgroups);
+  if (mode == 1 && depth == 4 && total_workgroups > current_device_cus()) depth = 2; // as in launch_mvm_round
 #define RPU_LAUNCH_ROUND(PD, WMODE) hipLaunchKernelGGL((k_mvm_round_group<PD, WMODE>), grid, dim3(256), 0, s, g, round, seen)
   if (mode == 0) {
     if (depth == 4) RPU_LAUNCH_ROUND(4, 0);
@@ -2239,7 +2240,11 @@ void launch_mvm_round(const MvmArgs &a_in, hipStream_t s) {
     return;
   }
   const dim3 grid(all);
-  const int depth = mvm_prefetch_depth(a.K, a.k_pad);
+  int depth = mvm_prefetch_depth(a.K, a.k_pad);
+  // The deepest prefetch of the transposed-weight variant takes more than half of a SIMD's registers: one workgroup per
+  // CU at a time.  With more workgroups than CUs the variant with two stages in flight, two workgroups per CU, is faster
+  // (backward at batch 1024 on the 1024 x 1024 tile 63 -> 52 us; same sums, the waves split K the same way).
+  if (mode == 1 && depth == 4 && all > current_device_cus()) depth = 2;
   if (a.rest_in_one) {
 #define RPU_LAUNCH_REST(PD, WMODE) hipLaunchKernelGGL((k_mvm_rounds_rest<PD, WMODE>), grid, dim3(256), 0, s, a)
     if (mode == 0) {
