@@ -1101,7 +1101,12 @@ template <int WMODE>
 __global__ __launch_bounds__(256) void k_mvm_round_tail(MvmArgs a) {
   __shared__ float red[WAVES][16][64];
   __shared__ __attribute__((aligned(16))) float stage[WAVES * 2 * TILE * LDS_ROW];
+  if (a.dual.on == 2) { // the launch after the fused one: the kept results of every tile go to the caller's output
+    const int all = workgroups_for(a.O, a.m_batch);
+    for (int n = blockIdx.x; n < all; n += gridDim.x) mvm_dual_select(a, n);
+  }
   const int n_act = (a.round > 0) ? a.st.count[a.round] : a.m_batch;
+  if (a.round > 0) mvm_note_round(a, a.round, n_act, a.dual.on == 2);
   if (runs_on_large_tiles(a, a.round, n_act)) return;
   const int total = workgroups_for(a.O, n_act);
   for (int n = blockIdx.x; n < total; n += gridDim.x) {
@@ -2191,7 +2196,6 @@ bool mvm_can_fuse_rounds(const MvmArgs &a) {
   if (a.io.perfect || a.io.bound_management == RPU_BM_NONE || a.max_rounds < 3 || a.transposed) return false;
   if (a.pre_add || a.skip_if_zero || a.nm_phase || !a.speculate || !a.rows_ahead_in_init) return false;
   if (!a.small_tiles_only && big_threshold(a.m_batch, a.O) > 0) return false;
-  if (mvm_round_workgroups(a) > TAIL_GRID) return false;
   return mvm_prefetch_depth(a.K, a.k_pad) >= 2 && weight_mode(a) != 1;
 }
 

@@ -44,7 +44,8 @@ def test_benchmark_configuration_with_noise_is_bit_equal(gpu_device):
 
 @pytest.mark.parametrize("bound_management", [BM.Iterative, BM.IterativeWorstCase])
 @pytest.mark.parametrize("shape,bias,trans", [((512, 300, 100), False, False), ((257, 96, 33), True, False),
-                                              ((1024, 256, 64), False, True), ((768, 1000, 256), False, False)])
+                                              ((1024, 256, 64), False, True), ((768, 1000, 256), False, False),
+                                              ((256, 1024, 1100), False, False)])     # 1120 workgroups: the later rounds walk
 def test_shapes_layouts_and_many_rounds(gpu_device, shape, bias, trans, bound_management):
     """Samples that stop after round 0, after round 1 and later (a small out_bound sends many to rounds 2 .. 4), a zero
     sample, a bias column (rows that are not 16-byte aligned), transposed layouts, the worst-case switch of the scale."""
