@@ -164,6 +164,8 @@ SYMBOLS = {
                                             C.c_int, C.c_int, _P]),
     "rpu_group_backward_strided": (C.c_int, [_P, C.POINTER(_P), C.POINTER(C.c_long), C.POINTER(_P), C.POINTER(C.c_long),
                                              C.c_int, _P]),
+    "rpu_group_update_strided": (C.c_int, [_P, C.POINTER(_P), C.POINTER(C.c_long), C.POINTER(_P), C.POINTER(C.c_long),
+                                           C.c_int, _P]),
     "rpu_group_get_shared_input_sets": (C.c_int, [_P, C.POINTER(C.c_int), C.POINTER(C.c_int)]),
     "rpu_group_destroy": (C.c_int, [_P]),
     "rpu_tile_set_forward_out_scale": (C.c_int, [_P, C.c_float]),

@@ -244,6 +244,23 @@ struct UpdateArgs {
   uint32_t call;
 };
 
+// Several tiles in one launch of an update kernel: args[t] in HBM, start[t] .. start[t + 1] the workgroups (blockIdx.x)
+// of tile t in the launch at hand (each kernel has its own table); all tiles share m_batch.
+struct UpdateGroup {
+  const UpdateArgs *args;
+  const int *start; // [n + 1]; unused by the set-up kernel
+  int n;
+  int m_batch;
+};
+void launch_update_prepare_group(const UpdateGroup &g, hipStream_t s);
+// wide: 16 line elements per workgroup (else 4); total_blocks: sum of the tiles' element blocks; rows of words = m_batch
+void launch_update_lines_group(const UpdateGroup &g, bool wide, int total_blocks, hipStream_t s);
+int update_lines_blocks(const UpdateArgs &a, bool wide);
+// the tiles must agree in what update_pulsed_variant returns; total_workgroups: sum of update_pulsed_workgroups
+int update_pulsed_variant(const UpdateArgs &a);
+int update_pulsed_workgroups(const UpdateArgs &a);
+void launch_update_pulsed_group(const UpdateGroup &g, int variant, int total_workgroups, hipStream_t s);
+
 // tables of the update kernels on the current device (once per GPU; blocking copy, no allocation)
 void ensure_update_tables();
 void launch_update_prepare(const UpdateArgs &a, hipStream_t s);       // BL, A, B per sample

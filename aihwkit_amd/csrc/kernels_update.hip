@@ -70,9 +70,7 @@ __device__ __forceinline__ float part_abs_max(const float *v, int n, long stride
 
 // One workgroup per sample: the loads of both lines are in flight together (a line of 1024 elements is one 16-byte load
 // per thread), then one exchange through LDS gives the first thread both maxima and it sets the sample's BL, A, B.
-__global__ __launch_bounds__(256) void k_update_prepare(UpdateArgs a) {
-  __shared__ float sh[2][4];
-  const int b = blockIdx.x;
+__device__ __forceinline__ void update_prepare_sample(const UpdateArgs &a, const int b, float (*sh)[4]) {
   const bool leader = threadIdx.x == 0;
   const float lr = fabsf(a.lr);
   const float dw_min = a.dev.dw_min;
@@ -133,6 +131,20 @@ __global__ __launch_bounds__(256) void k_update_prepare(UpdateArgs a) {
   a.prob_b[b] = B;
 }
 
+__global__ __launch_bounds__(256) void k_update_prepare(UpdateArgs a) {
+  __shared__ float sh[2][4];
+  update_prepare_sample(a, (int)blockIdx.x, sh);
+}
+
+// The same for several tiles in one launch (all with the same batch): workgroup n works on sample n % m_batch of tile
+// n / m_batch.  A tile's arguments are copied out of HBM once, by scalar loads (the tile index is uniform).
+__global__ __launch_bounds__(256) void k_update_prepare_group(UpdateGroup g) {
+  __shared__ float sh[2][4];
+  const int t = (int)blockIdx.x / g.m_batch;
+  const UpdateArgs a = g.args[t];
+  update_prepare_sample(a, (int)blockIdx.x - t * g.m_batch, sh);
+}
+
 __device__ __forceinline__ float discretize_prob(float pp, float res, int sto_round, uint32_t rnd) {
   if (res <= 0.0f) return pp;
   float q = pp / res;
@@ -170,15 +182,15 @@ __device__ __forceinline__ uint32_t pulse_word(const UpdateArgs &a, bool is_x, i
 // go back through LDS and are written 4 LINES_E bytes per sample row.
 // LINES_E = 16 moves whole 64-byte row segments; small launches take 4 elements per workgroup (one per wave) so that
 // there are four times as many workgroups.
+// bx: number of the workgroup's block of line elements (x blocks first, then d blocks), by: its block of 64 rows of words
 template <int LINES_E>
-__global__ __launch_bounds__(256) void k_update_lines(UpdateArgs a) {
-  __shared__ float vals[64][LINES_E + 1];
-  __shared__ uint32_t wt[64][LINES_E + 1];
+__device__ __forceinline__ void update_lines_block(const UpdateArgs &a, const int bx, const int by,
+                                                   float (*vals)[LINES_E + 1], uint32_t (*wt)[LINES_E + 1]) {
   const int tiles_x = (a.x_size + LINES_E - 1) / LINES_E;
-  const bool is_x = (int)blockIdx.x < tiles_x;
-  const int e0 = (is_x ? (int)blockIdx.x : (int)blockIdx.x - tiles_x) * LINES_E;
+  const bool is_x = bx < tiles_x;
+  const int e0 = (is_x ? bx : bx - tiles_x) * LINES_E;
   const int size = is_x ? a.x_size : a.d_size;
-  const int b0 = blockIdx.y * 64;
+  const int b0 = by * 64;
   const float *src = is_x ? a.x : a.d;
   const long s_b = is_x ? a.x_sb : a.d_sb, s_e = is_x ? a.x_sj : a.d_si;
   constexpr int ROWS_PER_PASS = 256 / LINES_E;
@@ -200,7 +212,7 @@ __global__ __launch_bounds__(256) void k_update_lines(UpdateArgs a) {
   const int K = b_ok ? min(max(a.bl[sample] - 31 * wrow, 0), 31) : 0;
   const int kmax = a.kmax[a.kmax_slot];
   uint32_t *planes = is_x ? a.x_planes : a.d_planes;
-  const int c0 = 2 * blockIdx.y;
+  const int c0 = 2 * by;
   for (int el = wave; el < LINES_E; el += 4) {
     const int e = e0 + el;
     if (e >= size) break; // wave-uniform
@@ -228,6 +240,24 @@ __global__ __launch_bounds__(256) void k_update_lines(UpdateArgs a) {
     const int bb = b0 + rb, ee = e0 + col;
     if (bb < a.m_batch && ee < size) words[(long)bb * size + ee] = wt[rb][col];
   }
+}
+
+template <int LINES_E>
+__global__ __launch_bounds__(256) void k_update_lines(UpdateArgs a) {
+  __shared__ float vals[64][LINES_E + 1];
+  __shared__ uint32_t wt[64][LINES_E + 1];
+  update_lines_block<LINES_E>(a, (int)blockIdx.x, (int)blockIdx.y, vals, wt);
+}
+
+// Several tiles in one launch: start[t] .. start[t + 1] are the element blocks of tile t.
+template <int LINES_E>
+__global__ __launch_bounds__(256) void k_update_lines_group(UpdateGroup g) {
+  __shared__ float vals[64][LINES_E + 1];
+  __shared__ uint32_t wt[64][LINES_E + 1];
+  int t = 0;
+  while (t + 1 < g.n && (int)blockIdx.x >= g.start[t + 1]) ++t;
+  const UpdateArgs a = g.args[t];
+  update_lines_block<LINES_E>(a, (int)blockIdx.x - g.start[t], (int)blockIdx.y, vals, wt);
 }
 
 // deterministic implicit line values (src/rpucuda/dense_bit_line_maker.cpp:209-235)
@@ -684,15 +714,14 @@ __device__ __forceinline__ float pulsed_gather(const UpdateArgs &a, float w, con
 // wave covers 64 consecutive x per column group, so everything that belongs to the d line is wave-uniform and the x
 // planes, weights and parameters are read with unit stride.  The pulse loop is chosen by the longest bit line of
 // the batch.
+// bx: the workgroup's block of 256 C columns, i: its row; tbl: the noise factors 1 + std * quantile in LDS
 template <int KIND, bool MULT, bool NOISE, int C>
-__global__ __launch_bounds__(256, (C > 1 ? 4 : 8)) void k_update_pulsed(UpdateArgs a) {
-  __shared__ float tbl[CTOC_LEVELS]; // noise factors 1 + std * quantile
+__device__ __forceinline__ void update_pulsed_row(const UpdateArgs &a, const int bx, const int i, float *tbl) {
   if (NOISE) {
     static_assert(CTOC_LEVELS == 256, "one table entry per thread");
     tbl[threadIdx.x] = __builtin_fmaf(a.dev.dw_min_std, g_ctoc_xi[threadIdx.x], 1.0f);
     __syncthreads();
   }
-  const int i = blockIdx.y;
   int j[C];
   bool valid[C];
   unsigned cell[C];
@@ -700,7 +729,7 @@ __global__ __launch_bounds__(256, (C > 1 ? 4 : 8)) void k_update_pulsed(UpdateAr
   float w[C];
 #pragma unroll
   for (int c = 0; c < C; ++c) {
-    const int jt = (blockIdx.x * C + c) * 256 + threadIdx.x;
+    const int jt = (bx * C + c) * 256 + threadIdx.x;
     valid[c] = jt < a.x_size;
     j[c] = valid[c] ? jt : a.x_size - 1;
     cell[c] = (unsigned)i * (unsigned)a.x_size + (unsigned)j[c];
@@ -720,6 +749,25 @@ __global__ __launch_bounds__(256, (C > 1 ? 4 : 8)) void k_update_pulsed(UpdateAr
   for (int c = 0; c < C; ++c) {
     if (valid[c]) a.w[cell[c]] = w[c];
   }
+}
+
+template <int KIND, bool MULT, bool NOISE, int C>
+__global__ __launch_bounds__(256, (C > 1 ? 4 : 8)) void k_update_pulsed(UpdateArgs a) {
+  __shared__ float tbl[CTOC_LEVELS];
+  update_pulsed_row<KIND, MULT, NOISE, C>(a, (int)blockIdx.x, (int)blockIdx.y, tbl);
+}
+
+// Several tiles in one launch (same device kind, noise and columns per lane): start[t] .. start[t + 1] are the
+// workgroups of tile t, column blocks of a row next to each other.
+template <int KIND, bool MULT, bool NOISE, int C>
+__global__ __launch_bounds__(256, (C > 1 ? 4 : 8)) void k_update_pulsed_group(UpdateGroup g) {
+  __shared__ float tbl[CTOC_LEVELS];
+  int t = 0;
+  while (t + 1 < g.n && (int)blockIdx.x >= g.start[t + 1]) ++t;
+  const UpdateArgs a = g.args[t];
+  const int blocks = (a.x_size + 256 * C - 1) / (256 * C);
+  const int local = (int)blockIdx.x - g.start[t];
+  update_pulsed_row<KIND, MULT, NOISE, C>(a, local % blocks, local / blocks, tbl);
 }
 
 // ---- opt-in variant: aggregated steps -----------------------------------------------------------------------
@@ -1165,6 +1213,57 @@ void launch_update_pulsed(const UpdateArgs &a, hipStream_t s) {
     if (wide) launch_update_pulsed_t<false, 4>(a, s);
     else launch_update_pulsed_t<false, 1>(a, s);
   }
+}
+
+// 3 bits: device step (0 ConstantStep, 1 LinearStep with multiplicative noise, 2 with additive noise), cycle-to-cycle
+// noise on, four columns per lane
+int update_pulsed_variant(const UpdateArgs &a) {
+  const int step = a.dev.kind == RPU_DEVICE_CONSTANT_STEP ? 0 : (a.dev.ls_mult_noise ? 1 : 2);
+  const bool wide = a.x_size >= 1024 && (long)a.x_size * a.d_size >= (1L << 19);
+  return (step * 2 + (a.dev.dw_min_std > 0.0f ? 1 : 0)) * 2 + (wide ? 1 : 0);
+}
+
+int update_pulsed_workgroups(const UpdateArgs &a) {
+  const int c = (update_pulsed_variant(a) & 1) ? 4 : 1;
+  return ((a.x_size + 256 * c - 1) / (256 * c)) * a.d_size;
+}
+
+template <bool NOISE, int C> static void launch_update_pulsed_group_t(const UpdateGroup &g, int step, dim3 grid, hipStream_t s) {
+  if (step == 0) {
+    hipLaunchKernelGGL((k_update_pulsed_group<RPU_DEVICE_CONSTANT_STEP, true, NOISE, C>), grid, dim3(256), 0, s, g);
+  } else if (step == 1) {
+    hipLaunchKernelGGL((k_update_pulsed_group<RPU_DEVICE_LINEAR_STEP, true, NOISE, C>), grid, dim3(256), 0, s, g);
+  } else {
+    hipLaunchKernelGGL((k_update_pulsed_group<RPU_DEVICE_LINEAR_STEP, false, NOISE, C>), grid, dim3(256), 0, s, g);
+  }
+}
+
+void launch_update_pulsed_group(const UpdateGroup &g, int variant, int total_workgroups, hipStream_t s) {
+  const dim3 grid(total_workgroups);
+  const int step = variant >> 2;
+  const bool noise = (variant >> 1) & 1, wide = variant & 1;
+  if (noise) {
+    if (wide) launch_update_pulsed_group_t<true, 4>(g, step, grid, s);
+    else launch_update_pulsed_group_t<true, 1>(g, step, grid, s);
+  } else {
+    if (wide) launch_update_pulsed_group_t<false, 4>(g, step, grid, s);
+    else launch_update_pulsed_group_t<false, 1>(g, step, grid, s);
+  }
+}
+
+void launch_update_prepare_group(const UpdateGroup &g, hipStream_t s) {
+  hipLaunchKernelGGL(k_update_prepare_group, dim3((unsigned)g.n * (unsigned)g.m_batch), dim3(256), 0, s, g);
+}
+
+int update_lines_blocks(const UpdateArgs &a, bool wide) {
+  const int e = wide ? 16 : 4;
+  return (a.x_size + e - 1) / e + (a.d_size + e - 1) / e;
+}
+
+void launch_update_lines_group(const UpdateGroup &g, bool wide, int total_blocks, hipStream_t s) {
+  const dim3 grid(total_blocks, (g.m_batch + 63) / 64);
+  if (wide) hipLaunchKernelGGL(k_update_lines_group<16>, grid, dim3(256), 0, s, g);
+  else hipLaunchKernelGGL(k_update_lines_group<4>, grid, dim3(256), 0, s, g);
 }
 
 void launch_update_aggregated(const UpdateArgs &a, int samples_per_step, hipStream_t s) {

@@ -1190,16 +1190,13 @@ struct Tile {
 
   // pulsed update of one device matrix (rpu_weight_updater.cpp:197-294)
   // ws != nullptr: the per-call scratch is carved out of that block and nothing is allocated (stochastic pulses only)
-  void pulsed_update_on(const DeviceView &dv, const UpdatePar &up, float lr, const float *xin, long x_sb, long x_sj,
-                        const float *d, long d_sb, long d_si, int B, hipStream_t s, unsigned char *ws = nullptr) {
-    if (lr == 0.0f) return;
-    const DevicePar &dev = *dv.par;
-    // The longest bit line this call can choose (calculateBlAB, rpu_pulsed_meta_parameter.cpp:152-181): desired_BL,
-    // or ceil(lr / dw_min) when neither a fixed BL nor BL management holds it there.  A packed word holds 31 pulses;
-    // longer lines take several rows of words per sample.
+  // Rows of pulse words per sample.  The longest bit line a call can choose (calculateBlAB,
+  // rpu_pulsed_meta_parameter.cpp:152-181) is desired_BL, or ceil(lr / dw_min) when neither a fixed BL nor BL
+  // management holds it there.  A packed word holds 31 pulses; longer lines take several rows of words per sample.
+  static int words_per_sample_for(const UpdatePar &up, float lr, float granularity) {
     int bl_max = up.p.desired_bl;
-    if (!up.p.fixed_bl && !up.p.update_bl_management && dv.granularity * (float)up.p.desired_bl < fabsf(lr)) {
-      const float need = ceilf(fabsf(lr) / dv.granularity);
+    if (!up.p.fixed_bl && !up.p.update_bl_management && granularity * (float)up.p.desired_bl < fabsf(lr)) {
+      const float need = ceilf(fabsf(lr) / granularity);
       if (up.p.pulse_type == RPU_PULSE_STOCHASTIC_COMPRESSED && !(need <= (float)RPU_MAX_BL)) {
         throw RpuError("This learning rate needs a bit line of " + std::to_string((long)need) +
                        " pulses (fixed_BL and update_bl_management are off); stochastic pulse trains hold at most " +
@@ -1207,7 +1204,15 @@ struct Tile {
       }
       bl_max = std::max((int)need, 1);
     }
-    const int wps = up.p.pulse_type == RPU_PULSE_STOCHASTIC_COMPRESSED ? std::max((bl_max + 30) / 31, 1) : 1;
+    return up.p.pulse_type == RPU_PULSE_STOCHASTIC_COMPRESSED ? std::max((bl_max + 30) / 31, 1) : 1;
+  }
+
+  // Arguments of the update kernels for one call (lr != 0): scratch sized for B samples (or carved out of ws), the
+  // call's random-stream index taken; wps returns the rows of pulse words per sample.
+  UpdateArgs pulsed_update_args(const DeviceView &dv, const UpdatePar &up, float lr, const float *xin, long x_sb, long x_sj,
+                                const float *d, long d_sb, long d_si, int B, hipStream_t s, unsigned char *ws, int &wps_out) {
+    const DevicePar &dev = *dv.par;
+    const int wps = words_per_sample_for(up, lr, dv.granularity);
     if (wps > 1 && ws) throw RpuError("update_noalloc holds bit lines of at most 31 pulses.");
     if (wps > 1 && (long)B * wps > 0x7fffffffL) throw RpuError("Too many rows of pulse words for this batch.");
     const int rows = B * wps; // rows of pulse words
@@ -1243,6 +1248,26 @@ struct Tile {
         a.x_val = u_xval.p; a.d_val = u_dval.p;
       }
     }
+    wps_out = wps;
+    return a;
+  }
+
+  // what the debug hooks read after a pulsed update
+  void note_pulsed_update(const UpdateArgs &a, int B, int wps, int pulse_type, hipStream_t s) {
+    last_stream = s;
+    last_update_batch = B;
+    last_words_per_sample = wps;
+    last_update_pulse = pulse_type;
+    last_bl = a.bl; last_a = a.prob_a; last_b = a.prob_b; last_xw = a.x_words; last_dw = a.d_words;
+  }
+
+  void pulsed_update_on(const DeviceView &dv, const UpdatePar &up, float lr, const float *xin, long x_sb, long x_sj,
+                        const float *d, long d_sb, long d_si, int B, hipStream_t s, unsigned char *ws = nullptr) {
+    if (lr == 0.0f) return;
+    const DevicePar &dev = *dv.par;
+    int wps = 1;
+    UpdateArgs a = pulsed_update_args(dv, up, lr, xin, x_sb, x_sj, d, d_sb, d_si, B, s, ws, wps);
+    const int rows = B * wps;
     prof_begin(s);
     launch_update_prepare(a, s);
     prof_mark(s, "update_prepare");
@@ -1275,11 +1300,26 @@ struct Tile {
       prof_mark(s, "write_noise");
     }
     RPU_HIP_CHECK(hipGetLastError());
-    last_stream = s;
-    last_update_batch = B;
-    last_words_per_sample = wps;
-    last_update_pulse = up.p.pulse_type;
-    last_bl = a.bl; last_a = a.prob_a; last_b = a.prob_b; last_xw = a.x_words; last_dw = a.d_words;
+    note_pulsed_update(a, B, wps, up.p.pulse_type, s);
+  }
+
+  // Whether this tile's update is the plain stochastic pulsed one that a group launch provides; else why not.
+  const char *group_update_obstacle() const {
+    if (!dev.pulsed() || up.p.pulse_type != RPU_PULSE_STOCHASTIC_COMPRESSED) return "only stochastic pulses on a pulsed device";
+    if (is_transfer()) return "no transfer compounds";
+    if (persistent()) return "no write noise";
+    if (delta_w) return "no delta weights";
+    if (dev.p.count_pulses) return "no pulse counters";
+    if (update_variant == RPU_UPDATE_VARIANT_AGGREGATED) return "no update variants";
+    if (shared_xd) return "no column-major shared weights";
+    if (lr != 0.0f && words_per_sample_for(up, lr, dev.p.dw_min) > 1) return "bit lines of at most 31 pulses";
+    return nullptr;
+  }
+
+  // arguments of the plain pulsed update on this tile's own weights (see group_update_obstacle)
+  UpdateArgs group_update_args(const float *x, long x_ld, const float *d, long d_ld, int B, hipStream_t s, int &wps) {
+    DeviceView dv{wp_dev(), d_wmax.p, d_wmin.p, d_sup.p, d_sdown.p, d_slup.p, d_sldown.p, &dev, dev.p.dw_min};
+    return pulsed_update_args(dv, up, lr, x, x_ld, 1, d, d_ld, 1, B, s, nullptr, wps);
   }
 
   // The stochastic pulsed update without any allocation: every buffer beyond inputs and weights lives in the
@@ -2024,6 +2064,11 @@ struct rpu_group {
   // quantized rows of rounds 0 and 1 shared by tiles that read the same input with the same DAC (two buffers per set)
   std::vector<DevBuf<float>> first_rows;
   int shared_sets = 0, shared_tiles = 0; // of the last call
+  // grouped update: the tiles' argument blocks and the workgroup tables of its launches
+  DevBuf<UpdateArgs> d_uargs;
+  DevBuf<int> d_ustart;
+  UpdateArgs *h_uargs = nullptr; // pinned staging
+  int *h_ustart = nullptr;
   std::mutex mutex;
   ~rpu_group() {
     if (device_id >= 0) {
@@ -2036,6 +2081,10 @@ struct rpu_group {
         if (h_args) (void)hipHostFree(h_args);
         if (h_start) (void)hipHostFree(h_start);
         if (seen_host) (void)hipHostFree(seen_host);
+        if (h_uargs) (void)hipHostFree(h_uargs);
+        if (h_ustart) (void)hipHostFree(h_ustart);
+        d_uargs.release();
+        d_ustart.release();
         d_args.release();
         d_start.release();
         for (auto &b : first_rows) b.release();
@@ -2069,6 +2118,100 @@ int rpu_group_create(rpu_group_t **out, rpu_tile_t *const *tiles, int n_tiles) {
     RPU_HIP_CHECK(hipHostMalloc((void **)&g->h_start, (3 * n + 4) * sizeof(int), hipHostMallocDefault));
     RPU_HIP_CHECK(hipEventCreateWithFlags(&g->copied, hipEventDisableTiming));
     *out = g.release();
+  });
+}
+
+// Stochastic pulsed update of all tiles of a group: one set-up launch, one launch for the pulse trains and one update
+// launch per kernel variant among the tiles (device step, noise, columns per lane), instead of three launches per tile
+int rpu_group_update_strided(rpu_group_t *group, const float *const *x_dev, const long *x_ld, const float *const *d_dev,
+                             const long *d_ld, int m_batch, void *stream) {
+  return guarded([&] {
+    if (!group || !x_dev || !d_dev) throw RpuError("null argument");
+    if (m_batch < 0) throw RpuError("m_batch must not be negative.");
+    if (m_batch == 0) return;
+    std::lock_guard<std::mutex> glock(group->mutex);
+    DeviceGuard dg(group->device_id);
+    hipStream_t s = (hipStream_t)stream;
+    const int n = (int)group->tiles.size();
+    if (!group->h_uargs) {
+      group->d_uargs.ensure((size_t)n);
+      group->d_ustart.ensure(2 * (size_t)n + 16);
+      RPU_HIP_CHECK(hipHostMalloc((void **)&group->h_uargs, (size_t)n * sizeof(UpdateArgs), hipHostMallocDefault));
+      RPU_HIP_CHECK(hipHostMalloc((void **)&group->h_ustart, (2 * (size_t)n + 16) * sizeof(int), hipHostMallocDefault));
+    }
+    // the staging buffers may still feed the copy of the previous call
+    RPU_HIP_CHECK(hipEventSynchronize(group->copied));
+    ensure_update_tables();
+
+    // every tile is checked before any tile's call counter moves
+    for (int i = 0; i < n; ++i) {
+      Tile &t = group->tiles[i]->t;
+      std::lock_guard<std::mutex> lock(t.mutex);
+      (void)t.check_compute(m_batch, x_dev[i], d_dev[i]);
+      if (const char *why = t.group_update_obstacle()) {
+        throw RpuError(std::string("The grouped update runs the plain stochastic pulsed update (") + why +
+                       "): call this tile's own update.");
+      }
+      if ((x_ld && x_ld[i] < t.X) || (d_ld && d_ld[i] < t.D)) throw RpuError("A row stride is shorter than the row.");
+    }
+    std::vector<UpdateArgs> args;
+    std::vector<int> variant;
+    for (int i = 0; i < n; ++i) {
+      Tile &t = group->tiles[i]->t;
+      std::lock_guard<std::mutex> lock(t.mutex);
+      const long xl = x_ld ? x_ld[i] : t.X, dl = d_ld ? d_ld[i] : t.D;
+      if (t.lr == 0.0f) continue; // as the tile's own update: nothing happens, no random-stream index is used
+      int wps = 1;
+      UpdateArgs a = t.group_update_args(x_dev[i], xl, d_dev[i], dl, m_batch, s, wps);
+      a.words_per_sample = 1;
+      t.note_pulsed_update(a, m_batch, 1, RPU_PULSE_STOCHASTIC_COMPRESSED, s);
+      args.push_back(a);
+      variant.push_back(update_pulsed_variant(a));
+    }
+    const int m = (int)args.size();
+    if (m == 0) return;
+    // tiles that share a kernel variant sit next to each other
+    std::vector<int> order(m);
+    for (int i = 0; i < m; ++i) order[i] = i;
+    std::stable_sort(order.begin(), order.end(), [&](int a, int b) { return variant[a] < variant[b]; });
+    long lines_blocks_16 = 0;
+    for (int i = 0; i < m; ++i) lines_blocks_16 += update_lines_blocks(args[i], true);
+    const bool wide_lines = lines_blocks_16 * ((m_batch + 63) / 64) >= 256;
+    int cursor = 0, blocks = 0;
+    const int lines_offset = cursor;
+    for (int i = 0; i < m; ++i) {
+      group->h_ustart[cursor++] = blocks;
+      blocks += update_lines_blocks(args[order[i]], wide_lines);
+    }
+    group->h_ustart[cursor++] = blocks;
+    struct Segment { int first, count, variant, start_offset, workgroups; };
+    std::vector<Segment> segments;
+    for (int i = 0; i < m;) {
+      Segment seg{i, 0, variant[order[i]], cursor, 0};
+      int wg = 0, j = i;
+      for (; j < m && variant[order[j]] == seg.variant; ++j) {
+        group->h_ustart[cursor++] = wg;
+        wg += update_pulsed_workgroups(args[order[j]]);
+      }
+      group->h_ustart[cursor++] = wg;
+      seg.count = j - i;
+      seg.workgroups = wg;
+      segments.push_back(seg);
+      i = j;
+    }
+    for (int i = 0; i < m; ++i) group->h_uargs[i] = args[order[i]];
+    RPU_HIP_CHECK(hipMemcpyAsync(group->d_uargs.p, group->h_uargs, (size_t)m * sizeof(UpdateArgs), hipMemcpyHostToDevice, s));
+    RPU_HIP_CHECK(hipMemcpyAsync(group->d_ustart.p, group->h_ustart, (size_t)cursor * sizeof(int), hipMemcpyHostToDevice, s));
+    RPU_HIP_CHECK(hipEventRecord(group->copied, s));
+
+    UpdateGroup all{group->d_uargs.p, group->d_ustart.p + lines_offset, m, m_batch};
+    launch_update_prepare_group(all, s);
+    launch_update_lines_group(all, wide_lines, blocks, s);
+    for (const Segment &seg : segments) {
+      UpdateGroup g{group->d_uargs.p + seg.first, group->d_ustart.p + seg.start_offset, seg.count, m_batch};
+      launch_update_pulsed_group(g, seg.variant, seg.workgroups, s);
+    }
+    RPU_HIP_CHECK(hipGetLastError());
   });
 }
 

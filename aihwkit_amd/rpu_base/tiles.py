@@ -619,6 +619,30 @@ class TileGroup:
             raise RuntimeError(what + " must be a matrix with unit column stride")
         return tensor
 
+    def update(self, x_inputs, d_inputs, non_blocking: bool = False) -> None:
+        """Stochastic pulsed update of every tile with its own ``x_inputs[i]`` [m_batch, x_size_i] and ``d_inputs[i]``
+        [m_batch, d_size_i] (column slices of larger matrices are read in place): what each tile's own ``update`` does,
+        in three launches for the whole group."""
+        if len(x_inputs) != len(self._tiles) or len(d_inputs) != len(self._tiles):
+            raise RuntimeError("one input and one output gradient per tile expected")
+        xs = [self._rows(x, "x_input") for x in x_inputs]
+        ds = [self._rows(d, "d_input") for d in d_inputs]
+        m_batch = xs[0].shape[0]
+        for x, d, tile in zip(xs, ds, self._tiles):
+            if x.shape[0] != m_batch or x.shape[1] != tile.get_x_size():
+                raise RuntimeError("Invalid x_input dimensions")
+            if d.shape[0] != m_batch or d.shape[1] != tile.get_d_size():
+                raise RuntimeError("Invalid d_input dimensions")
+        n = len(xs)
+        x_ptrs = (C.c_void_p * n)(*[x.data_ptr() for x in xs])
+        d_ptrs = (C.c_void_p * n)(*[d.data_ptr() for d in ds])
+        x_ld = (C.c_long * n)(*[x.stride(0) if x.shape[0] > 1 else x.shape[1] for x in xs])
+        d_ld = (C.c_long * n)(*[d.stride(0) if d.shape[0] > 1 else d.shape[1] for d in ds])
+        stream = torch.cuda.current_stream(xs[0].device)
+        check(lib().rpu_group_update_strided(self._g, x_ptrs, x_ld, d_ptrs, d_ld, m_batch, C.c_void_p(stream.cuda_stream)))
+        if not non_blocking:
+            stream.synchronize()
+
     def get_shared_input_sets(self):
         """(sets, tiles) of the last call: sets of at least two tiles that were handed the same input and convert it the
         same way, so that its quantized rows were written once for the set, and the number of tiles in such sets."""

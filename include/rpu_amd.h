@@ -444,6 +444,15 @@ int rpu_group_forward_strided(rpu_group_t *group, const float *const *x_dev, con
  * gives it. */
 int rpu_group_backward_strided(rpu_group_t *group, const float *const *d_dev, const long *d_ld, float *const *x_dev,
                                const long *x_ld, int m_batch, void *stream);
+/* Stochastic pulsed update of all tiles of the group (the reference updates the tiles of an array one after the other
+ * through autograd, tiles/array.py; three launches per tile): x_dev[i] is [m_batch][x_size_i] with row stride x_ld[i],
+ * d_dev[i] is [m_batch][d_size_i] with row stride d_ld[i] (null strides: dense rows; no bias column, no transposed
+ * layouts).  Every tile gets exactly what rpu_tile_update with the same arguments gives it (same seed and call
+ * counter: same pulse trains, same weights).  Provided for the plain case -- stochastic compressed pulses on a pulsed
+ * device, bit lines of at most 31 pulses, no transfer compound, write noise, delta weights, pulse counters or update
+ * variant: any other tile in the group makes the call fail with a message that says so, before anything is launched. */
+int rpu_group_update_strided(rpu_group_t *group, const float *const *x_dev, const long *x_ld, const float *const *d_dev,
+                             const long *d_ld, int m_batch, void *stream);
 /* Tiles of a group that are handed the same input (pointer, stride, length) and convert it with the same DAC, noise
  * and bound management and without random numbers (the column blocks of a split layer, array.py:155-182, which the
  * reference quantizes once per tile) share the quantized rows of rounds 0 and 1: one of them writes the rows, all read
