@@ -70,28 +70,36 @@ __device__ __forceinline__ float part_abs_max(const float *v, int n, long stride
 
 // One workgroup per sample: the loads of both lines are in flight together (a line of 1024 elements is one 16-byte load
 // per thread), then one exchange through LDS gives the first thread both maxima and it sets the sample's BL, A, B.
+// SUB threads share a sample: the whole workgroup (long lines), a wave, or 16 lanes (the short patch rows of a
+// convolution come by the hundred thousand: a workgroup per sample would spend its time being launched)
+template <int SUB>
 __device__ __forceinline__ void update_prepare_sample(const UpdateArgs &a, const int b, float (*sh)[4]) {
-  const bool leader = threadIdx.x == 0;
+  const int t = threadIdx.x % SUB;
+  const bool leader = t == 0;
   const float lr = fabsf(a.lr);
   const float dw_min = a.dev.dw_min;
   int BL;
   float A, B;
   if (a.up.update_management || a.up.update_bl_management) {
-    float xm = part_abs_max(a.x + (long)b * a.x_sb, a.x_size, a.x_sj, threadIdx.x, 256);
-    float dm = part_abs_max(a.d + (long)b * a.d_sb, a.d_size, a.d_si, threadIdx.x, 256);
+    float xm = part_abs_max(a.x + (long)b * a.x_sb, a.x_size, a.x_sj, t, SUB);
+    float dm = part_abs_max(a.d + (long)b * a.d_sb, a.d_size, a.d_si, t, SUB);
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {
+    for (int off = (SUB < 64 ? SUB : 64) / 2; off > 0; off >>= 1) {
       xm = fmaxf(xm, __shfl_xor(xm, off));
       dm = fmaxf(dm, __shfl_xor(dm, off));
     }
-    if ((threadIdx.x & 63) == 0) {
-      sh[0][threadIdx.x >> 6] = xm;
-      sh[1][threadIdx.x >> 6] = dm;
+    if constexpr (SUB == 256) {
+      if ((threadIdx.x & 63) == 0) {
+        sh[0][threadIdx.x >> 6] = xm;
+        sh[1][threadIdx.x >> 6] = dm;
+      }
+      __syncthreads();
+      if (!leader) return;
+      xm = fmaxf(fmaxf(sh[0][0], sh[0][1]), fmaxf(sh[0][2], sh[0][3]));
+      dm = fmaxf(fmaxf(sh[1][0], sh[1][1]), fmaxf(sh[1][2], sh[1][3]));
+    } else {
+      if (!leader) return;
     }
-    __syncthreads();
-    if (!leader) return;
-    xm = fmaxf(fmaxf(sh[0][0], sh[0][1]), fmaxf(sh[0][2], sh[0][3]));
-    dm = fmaxf(fmaxf(sh[1][0], sh[1][1]), fmaxf(sh[1][2], sh[1][3]));
     // rpu_pulsed_meta_parameter.cpp:183-236
     calc_bl_ab(a.up, BL, A, B, lr, dw_min);
     if (lr > 0.0f) {
@@ -124,16 +132,24 @@ __device__ __forceinline__ void update_prepare_sample(const UpdateArgs &a, const
   // largest number of pulse slots in a row of words (a longer bit line takes several rows of 31): this call's slot
   // was zeroed by the previous call, which used the other one
   if (a.kmax) {
-    if (BL > 0) atomicMax(&a.kmax[a.kmax_slot], min(BL, 31));
+    // a running maximum of at most 31: a sample only sends its value when what it reads is still smaller (with
+    // hundreds of thousands of samples the atomics on the one word were most of this kernel's time)
+    const int mine = min(BL, 31);
+    if (mine > 0 && __hip_atomic_load(&a.kmax[a.kmax_slot], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < mine) {
+      atomicMax(&a.kmax[a.kmax_slot], mine);
+    }
     if (b == 0) a.kmax[a.kmax_slot ^ 1] = 0;
   }
   a.prob_a[b] = A;
   a.prob_b[b] = B;
 }
 
+template <int SUB>
 __global__ __launch_bounds__(256) void k_update_prepare(UpdateArgs a) {
   __shared__ float sh[2][4];
-  update_prepare_sample(a, (int)blockIdx.x, sh);
+  const int b = (int)blockIdx.x * (256 / SUB) + (int)threadIdx.x / SUB;
+  if (b >= a.m_batch) return; // all SUB threads of a sample leave together
+  update_prepare_sample<SUB>(a, b, sh);
 }
 
 // The same for several tiles in one launch (all with the same batch): workgroup n works on sample n % m_batch of tile
@@ -142,7 +158,7 @@ __global__ __launch_bounds__(256) void k_update_prepare_group(UpdateGroup g) {
   __shared__ float sh[2][4];
   const int t = (int)blockIdx.x / g.m_batch;
   const UpdateArgs a = g.args[t];
-  update_prepare_sample(a, (int)blockIdx.x - t * g.m_batch, sh);
+  update_prepare_sample<256>(a, (int)blockIdx.x - t * g.m_batch, sh);
 }
 
 __device__ __forceinline__ float discretize_prob(float pp, float res, int sto_round, uint32_t rnd) {
@@ -567,7 +583,11 @@ template <int KIND, bool MULT, int NK, bool NOISE, int C> struct PulsedRows {
     }
     if (!any) return;
     // bit set: x and d have the same sign, which steps down when lr > 0
-    const uint32_t dflip = ~dpl[(base + slots - 1u) * ds] ^ lr_mask;
+    walk(x, dk, any, ~dpl[(base + slots - 1u) * ds] ^ lr_mask);
+  }
+
+  // the passes of one chunk: dk the row's d pulses per slot (wave-uniform), any their union, dflip the direction bits
+  __device__ __forceinline__ void walk(const ChunkPlanes<NK, C> &x, const uint32_t (&dk)[NK], uint32_t any, const uint32_t dflip) {
     uint32_t same[C];
 #pragma unroll
     for (int c = 0; c < C; ++c) same[c] = x.sg[c] ^ dflip;
@@ -599,6 +619,55 @@ template <int KIND, bool MULT, int NK, bool NOISE, int C> struct PulsedRows {
     }
   }
 
+  // Long batches on small tiles (the patches of a convolution): a chunk with few d pulses is walked in a fraction of a
+  // memory latency, so fetching one chunk ahead leaves the wave waiting on every chunk.  Here the planes of PB chunks
+  // are fetched at a time, two such blocks in turn: the x planes per lane, the row's d planes with lane l fetching those
+  // of the block's chunk l (read back with v_readlane, which also keeps them out of the scalar cache's latency).
+  static constexpr int PB = 8;
+  struct Block {
+    ChunkPlanes<NK, C> x[PB];
+    uint32_t dk[NK], dsg; // of chunk (first chunk of the block + lane)
+  };
+  __device__ __forceinline__ void load_block(Block &b, const int (&j)[C], unsigned ch0, int i, int kmax) {
+    const unsigned n_chunks = (unsigned)a.n_chunks, ds = (unsigned)a.d_size, slots = (unsigned)a.plane_slots;
+#pragma unroll
+    for (int p = 0; p < PB; ++p) b.x[p].load(a, j, min(ch0 + (unsigned)p, n_chunks - 1u));
+    const unsigned chl = min(ch0 + (threadIdx.x & 63u), n_chunks - 1u);
+    const uint32_t *dpl = a.d_planes + i;
+#pragma unroll
+    for (int k = 0; k < NK; ++k) b.dk[k] = (k < kmax) ? dpl[(chl * slots + (unsigned)k) * ds] : 0u;
+    b.dsg = dpl[(chl * slots + slots - 1u) * ds];
+  }
+  __device__ __forceinline__ void walk_block(const Block &b, unsigned ch0, uint32_t lr_mask) {
+    const unsigned n_chunks = (unsigned)a.n_chunks;
+#pragma unroll
+    for (int p = 0; p < PB; ++p) {
+      if (ch0 + (unsigned)p >= n_chunks) break; // wave-uniform
+      uint32_t dk[NK], any = 0u;
+#pragma unroll
+      for (int k = 0; k < NK; ++k) {
+        dk[k] = (uint32_t)__builtin_amdgcn_readlane((int)b.dk[k], p);
+        any |= dk[k];
+      }
+      if (!any) continue;
+      walk(b.x[p], dk, any, ~(uint32_t)__builtin_amdgcn_readlane((int)b.dsg, p) ^ lr_mask);
+    }
+  }
+  __device__ __forceinline__ void run_blocks(int i, const int (&j)[C], int kmax, uint32_t lr_mask) {
+    const unsigned n_chunks = (unsigned)a.n_chunks;
+    Block ba, bb;
+    load_block(ba, j, 0u, i, kmax);
+    for (unsigned ch = 0; ch < n_chunks; ch += 2u * PB) {
+      if (ch + PB < n_chunks) load_block(bb, j, ch + PB, i, kmax);
+      walk_block(ba, ch, lr_mask);
+      if (ch + PB < n_chunks) {
+        if (ch + 2u * PB < n_chunks) load_block(ba, j, ch + 2u * PB, i, kmax);
+        walk_block(bb, ch + PB, lr_mask);
+      }
+    }
+  }
+
+  template <bool DEEP = false>
   __device__ __forceinline__ void run(unsigned cell, int i, const int (&j)[C], int kmax) {
     const uint32_t lr_mask = a.lr < 0.0f ? 0xffffffffu : 0u;
     const unsigned n_chunks = (unsigned)a.n_chunks;
@@ -607,6 +676,10 @@ template <int KIND, bool MULT, int NK, bool NOISE, int C> struct PulsedRows {
       s0 = r.v[0] | 1u; // the all-zero state is the one fixed point of the generator
       s1 = r.v[1];
       draw();
+    }
+    if constexpr (DEEP) {
+      run_blocks(i, j, kmax, lr_mask);
+      return;
     }
     if (NK > 3) { // one register set: the longer lines are the rarer case, and two sets would not fit
       ChunkPlanes<NK, C> p;
@@ -715,7 +788,8 @@ __device__ __forceinline__ float pulsed_gather(const UpdateArgs &a, float w, con
 // planes, weights and parameters are read with unit stride.  The pulse loop is chosen by the longest bit line of
 // the batch.
 // bx: the workgroup's block of 256 C columns, i: its row; tbl: the noise factors 1 + std * quantile in LDS
-template <int KIND, bool MULT, bool NOISE, int C>
+// DEEP: the planes of eight chunks are fetched at a time (PulsedRows::run_blocks; short bit lines, one column per lane)
+template <int KIND, bool MULT, bool NOISE, int C, bool DEEP>
 __device__ __forceinline__ void update_pulsed_row(const UpdateArgs &a, const int bx, const int i, float *tbl) {
   if (NOISE) {
     static_assert(CTOC_LEVELS == 256, "one table entry per thread");
@@ -738,7 +812,7 @@ __device__ __forceinline__ void update_pulsed_row(const UpdateArgs &a, const int
   }
   const int kmax = a.kmax[a.kmax_slot];
   if (kmax <= 3) {
-    PulsedRows<KIND, MULT, 3, NOISE, C>(a, w, cp, tbl).run(cell[0], i, j, kmax);
+    PulsedRows<KIND, MULT, 3, NOISE, C>(a, w, cp, tbl).template run<DEEP>(cell[0], i, j, kmax);
   } else if (kmax <= 7) {
     PulsedRows<KIND, MULT, 7, NOISE, C>(a, w, cp, tbl).run(cell[0], i, j, kmax);
   } else {
@@ -751,23 +825,23 @@ __device__ __forceinline__ void update_pulsed_row(const UpdateArgs &a, const int
   }
 }
 
-template <int KIND, bool MULT, bool NOISE, int C>
-__global__ __launch_bounds__(256, (C > 1 ? 4 : 8)) void k_update_pulsed(UpdateArgs a) {
+template <int KIND, bool MULT, bool NOISE, int C, bool DEEP = false>
+__global__ __launch_bounds__(256, ((C > 1 || DEEP) ? 4 : 8)) void k_update_pulsed(UpdateArgs a) {
   __shared__ float tbl[CTOC_LEVELS];
-  update_pulsed_row<KIND, MULT, NOISE, C>(a, (int)blockIdx.x, (int)blockIdx.y, tbl);
+  update_pulsed_row<KIND, MULT, NOISE, C, DEEP>(a, (int)blockIdx.x, (int)blockIdx.y, tbl);
 }
 
 // Several tiles in one launch (same device kind, noise and columns per lane): start[t] .. start[t + 1] are the
 // workgroups of tile t, column blocks of a row next to each other.
-template <int KIND, bool MULT, bool NOISE, int C>
-__global__ __launch_bounds__(256, (C > 1 ? 4 : 8)) void k_update_pulsed_group(UpdateGroup g) {
+template <int KIND, bool MULT, bool NOISE, int C, bool DEEP = false>
+__global__ __launch_bounds__(256, ((C > 1 || DEEP) ? 4 : 8)) void k_update_pulsed_group(UpdateGroup g) {
   __shared__ float tbl[CTOC_LEVELS];
   int t = 0;
   while (t + 1 < g.n && (int)blockIdx.x >= g.start[t + 1]) ++t;
   const UpdateArgs a = g.args[t];
   const int blocks = (a.x_size + 256 * C - 1) / (256 * C);
   const int local = (int)blockIdx.x - g.start[t];
-  update_pulsed_row<KIND, MULT, NOISE, C>(a, local % blocks, local / blocks, tbl);
+  update_pulsed_row<KIND, MULT, NOISE, C, DEEP>(a, local % blocks, local / blocks, tbl);
 }
 
 // ---- opt-in variant: aggregated steps -----------------------------------------------------------------------
@@ -1158,7 +1232,14 @@ int grid_for(long total) {
 } // namespace
 
 void launch_update_prepare(const UpdateArgs &a, hipStream_t s) {
-  hipLaunchKernelGGL(k_update_prepare, dim3(a.m_batch), dim3(256), 0, s, a);
+  const int longest = a.x_size > a.d_size ? a.x_size : a.d_size;
+  if (longest > 256 || a.m_batch <= 1024) {
+    hipLaunchKernelGGL(k_update_prepare<256>, dim3(a.m_batch), dim3(256), 0, s, a);
+  } else if (longest > 64) {
+    hipLaunchKernelGGL(k_update_prepare<64>, dim3((a.m_batch + 3) / 4), dim3(256), 0, s, a);
+  } else {
+    hipLaunchKernelGGL(k_update_prepare<16>, dim3((a.m_batch + 15) / 16), dim3(256), 0, s, a);
+  }
 }
 
 void launch_update_lines(const UpdateArgs &a, hipStream_t s) {
@@ -1192,16 +1273,19 @@ void launch_update_planes(const UpdateArgs &a, hipStream_t s) {
   hipLaunchKernelGGL(k_update_planes, grid, dim3(256), 0, s, a);
 }
 
-template <bool NOISE, int C> static void launch_update_pulsed_t(const UpdateArgs &a, hipStream_t s) {
+template <bool NOISE, int C, bool DEEP = false> static void launch_update_pulsed_t(const UpdateArgs &a, hipStream_t s) {
   dim3 grid((a.x_size + 256 * C - 1) / (256 * C), a.d_size);
   if (a.dev.kind == RPU_DEVICE_CONSTANT_STEP) {
-    hipLaunchKernelGGL((k_update_pulsed<RPU_DEVICE_CONSTANT_STEP, true, NOISE, C>), grid, dim3(256), 0, s, a);
+    hipLaunchKernelGGL((k_update_pulsed<RPU_DEVICE_CONSTANT_STEP, true, NOISE, C, DEEP>), grid, dim3(256), 0, s, a);
   } else if (a.dev.ls_mult_noise) {
-    hipLaunchKernelGGL((k_update_pulsed<RPU_DEVICE_LINEAR_STEP, true, NOISE, C>), grid, dim3(256), 0, s, a);
+    hipLaunchKernelGGL((k_update_pulsed<RPU_DEVICE_LINEAR_STEP, true, NOISE, C, DEEP>), grid, dim3(256), 0, s, a);
   } else {
-    hipLaunchKernelGGL((k_update_pulsed<RPU_DEVICE_LINEAR_STEP, false, NOISE, C>), grid, dim3(256), 0, s, a);
+    hipLaunchKernelGGL((k_update_pulsed<RPU_DEVICE_LINEAR_STEP, false, NOISE, C, DEEP>), grid, dim3(256), 0, s, a);
   }
 }
+
+// many chunks on one column per lane: the block-wise fetch of the planes (same results)
+static bool update_pulsed_deep(const UpdateArgs &a) { return a.n_chunks >= 32; }
 
 // Columns per lane: several once a row is long enough to keep every lane busy with them (they share the scalar work of a
 // pass) and the tile has enough rows to fill the chip with such workgroups.  A function of the tile alone: the noise
@@ -1218,10 +1302,12 @@ void launch_update_pulsed(const UpdateArgs &a, hipStream_t s) {
   if (a.dev.dw_min_std > 0.0f) {
     if (cols == 4) launch_update_pulsed_t<true, 4>(a, s);
     else if (cols == 2) launch_update_pulsed_t<true, 2>(a, s);
+    else if (update_pulsed_deep(a)) launch_update_pulsed_t<true, 1, true>(a, s);
     else launch_update_pulsed_t<true, 1>(a, s);
   } else {
     if (cols == 4) launch_update_pulsed_t<false, 4>(a, s);
     else if (cols == 2) launch_update_pulsed_t<false, 2>(a, s);
+    else if (update_pulsed_deep(a)) launch_update_pulsed_t<false, 1, true>(a, s);
     else launch_update_pulsed_t<false, 1>(a, s);
   }
 }
