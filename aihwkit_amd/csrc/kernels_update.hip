@@ -811,7 +811,11 @@ __device__ __forceinline__ void update_pulsed_row(const UpdateArgs &a, const int
     w[c] = a.w[cell[c]];
   }
   const int kmax = a.kmax[a.kmax_slot];
-  if (kmax <= 3) {
+  if (DEEP && kmax <= 1) {
+    // bit lines of one pulse (small gradients under update-BL management, the rule for the patches of a convolution):
+    // every sample with a d pulse is one pass, no slots to test
+    PulsedRows<KIND, MULT, 1, NOISE, C>(a, w, cp, tbl).template run<DEEP>(cell[0], i, j, kmax);
+  } else if (kmax <= 3) {
     PulsedRows<KIND, MULT, 3, NOISE, C>(a, w, cp, tbl).template run<DEEP>(cell[0], i, j, kmax);
   } else if (kmax <= 7) {
     PulsedRows<KIND, MULT, 7, NOISE, C>(a, w, cp, tbl).run(cell[0], i, j, kmax);
