@@ -366,9 +366,10 @@ void launch_mean_abs(const float *v, size_t n, float *out, hipStream_t s);
 // x_mat[(n * patches + p) * x_size + k] = value of patch p of image n
 void launch_gather_indexed(float *x_mat, const float *images, const int *indices, int x_size, int patches, int n_images,
                            long image_size, hipStream_t s);
-// images[(j - 2) + n * image_size] += x_mat[...] (images must be zeroed before)
-void launch_scatter_indexed(float *images, const float *x_mat, const int *indices, int x_size, int patches, int n_images,
-                            long image_size, hipStream_t s);
+// images[(j - 2) + n * image_size] = sum of the x_mat entries gathered from that element, without atomics and in the reference's order: ptr [image_size + 1] and off list, per image element, the
+// offsets p * x_size + k of the patch entries gathered from it (every image element is written; no zeroing before)
+void launch_fold_indexed(float *images, const float *x_mat, const int *ptr, const int *off, int x_size, int patches,
+                         int n_images, long image_size, hipStream_t s);
 // [n][d][p] <-> [(n, p)][d]
 void launch_ndp_to_bd(float *bd, const float *ndp, int n_images, int d_size, int patches, hipStream_t s);
 void launch_bd_to_ndp(float *ndp, const float *bd, int n_images, int d_size, int patches, hipStream_t s);

@@ -3,7 +3,7 @@
 // of its bindings: src/aihwkit/inference/noise/pcm.py:100-158 over
 // src/aihwkit/inference/converter/conductance.py:51-82).  Element-wise kernels, one read and one write of each
 // array: HBM-bound.  Every normal is a Philox draw keyed by (element, call), so a seed reproduces a run.
-// The file also holds the gather / scatter / permute kernels of the indexed (convolution) interface.
+// The file also holds the gather / fold / permute kernels of the indexed (convolution) interface.
 #include "kernels.h"
 
 namespace rpu_amd {
@@ -150,19 +150,6 @@ __global__ __launch_bounds__(256) void k_gather_indexed(float *x_mat, const floa
   }
 }
 
-__global__ __launch_bounds__(256) void k_scatter_indexed(float *images, const float *x_mat, const int *indices, int x_size,
-                                                          int patches, int n_images, long image_size) {
-  const size_t total = (size_t)n_images * patches * x_size;
-  for (size_t idx = blockIdx.x * (size_t)blockDim.x + threadIdx.x; idx < total; idx += (size_t)gridDim.x * blockDim.x) {
-    const int k = (int)(idx % x_size);
-    const size_t b = idx / x_size;
-    const int p = (int)(b % patches);
-    const size_t n = b / patches;
-    const int j = indices[(size_t)k * patches + p];
-    if (j > 1) atomicAdd(&images[(size_t)(j - 2) + n * image_size], x_mat[idx]);
-  }
-}
-
 // ndp index (n, d, p) <-> bd index ((n, p), d)
 __global__ __launch_bounds__(256) void k_ndp_bd(float *dst, const float *src, int n_images, int d_size, int patches,
                                                  int to_bd) {
@@ -222,10 +209,27 @@ void launch_gather_indexed(float *x_mat, const float *images, const int *indices
                      n_images, image_size);
 }
 
-void launch_scatter_indexed(float *images, const float *x_mat, const int *indices, int x_size, int patches, int n_images,
-                            long image_size, hipStream_t s) {
-  const size_t total = (size_t)n_images * patches * x_size;
-  hipLaunchKernelGGL(k_scatter_indexed, dim3(grid_of(total)), dim3(256), 0, s, images, x_mat, indices, x_size, patches,
+// Fold of the patch matrix back into the images without atomics: image element e of image n is the sum of the patch
+// entries that were gathered from it, listed per element (ptr[e] .. ptr[e + 1] into off: offsets p * x_size + k into an
+// image's block of x_mat) in the order of the reference's loop (math_util / rpu.cpp:1130-1141 walks k, then p), added
+// one after the other from zero: the same bits on every run, and the reference's.
+__global__ __launch_bounds__(256) void k_fold_indexed(float *images, const float *x_mat, const int *ptr, const int *off,
+                                                      long block, int n_images, long image_size) {
+  const size_t total = (size_t)n_images * image_size;
+  for (size_t idx = blockIdx.x * (size_t)blockDim.x + threadIdx.x; idx < total; idx += (size_t)gridDim.x * blockDim.x) {
+    const size_t n = idx / image_size;
+    const long e = (long)(idx - n * image_size);
+    const float *src = x_mat + n * block;
+    float acc = 0.0f;
+    for (int t = ptr[e]; t < ptr[e + 1]; ++t) acc += src[off[t]];
+    images[idx] = acc;
+  }
+}
+
+void launch_fold_indexed(float *images, const float *x_mat, const int *ptr, const int *off, int x_size, int patches,
+                         int n_images, long image_size, hipStream_t s) {
+  const size_t total = (size_t)n_images * image_size;
+  hipLaunchKernelGGL(k_fold_indexed, dim3(grid_of(total)), dim3(256), 0, s, images, x_mat, ptr, off, (long)patches * x_size,
                      n_images, image_size);
 }
 

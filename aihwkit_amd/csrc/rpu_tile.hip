@@ -220,6 +220,8 @@ struct Tile {
   int idx_patches = 0;
   int32_t idx_max = 0; // largest entry of the index matrix
   DevBuf<int> x_idx, x_idx_t; // [X][patches] as set, and its transpose [patches][X] for the fused forward
+  DevBuf<int> x_fold_ptr, x_fold_off; // per image element the patch entries gathered from it (backward_indexed)
+  long fold_image_size = -1;
   DevBuf<float> x_mat, d_mat;
   int last_update_batch = 0;
   int last_update_pulse = -1;
@@ -334,7 +336,8 @@ struct Tile {
     t_unit.release(); t_read.release();
     i_ref.release(); i_prog.release(); i_nu_plus.release(); i_nu_minus.release(); i_scalar.release(); i_absmax.release();
     has_reference = programmed = false;
-    x_idx.release(); x_idx_t.release(); x_mat.release(); d_mat.release();
+    x_idx.release(); x_idx_t.release(); x_fold_ptr.release(); x_fold_off.release(); fold_image_size = -1;
+    x_mat.release(); d_mat.release();
     d_decay.release(); d_diff.release(); d_rbias.release(); s_clip.release();
     state_params_valid = false;
     delta_w = nullptr;
@@ -1418,8 +1421,30 @@ struct Tile {
     const int B = n_images * idx_patches;
     launch_ndp_to_bd(d_mat.p, d, n_images, D, idx_patches, s);
     mvm(d_mat.p, x_mat.p, B, false, false, false, true, s);
-    launch_fill(x, 0.0f, (size_t)n_images * image_size, s);
-    launch_scatter_indexed(x, x_mat.p, x_idx.p, X, idx_patches, n_images, image_size, s);
+    if (fold_image_size != image_size) {
+      // per image element, the entries of the patch matrix that were gathered from it, in the order in which the
+      // reference's loop adds them up (k, then p)
+      if (image_size <= 0 || (long)idx_max - 2 >= image_size) throw RpuError("The index matrix points beyond the image.");
+      std::vector<int> ptr((size_t)image_size + 1, 0);
+      for (int32_t j : idx_host) {
+        if (j > 1) ++ptr[(size_t)(j - 2) + 1];
+      }
+      for (long e = 0; e < image_size; ++e) ptr[(size_t)e + 1] += ptr[(size_t)e];
+      std::vector<int> off((size_t)ptr[(size_t)image_size]), cursor(ptr.begin(), ptr.end() - 1);
+      for (int k = 0; k < X; ++k) {
+        for (int p = 0; p < idx_patches; ++p) {
+          const int32_t j = idx_host[(size_t)k * idx_patches + p];
+          if (j > 1) off[(size_t)cursor[(size_t)(j - 2)]++] = p * X + k;
+        }
+      }
+      sync_last(); // the lists of another image size may still be read
+      x_fold_ptr.ensure(ptr.size());
+      x_fold_off.ensure(std::max<size_t>(off.size(), 1));
+      RPU_HIP_CHECK(hipMemcpy(x_fold_ptr.p, ptr.data(), ptr.size() * sizeof(int), hipMemcpyHostToDevice));
+      if (!off.empty()) RPU_HIP_CHECK(hipMemcpy(x_fold_off.p, off.data(), off.size() * sizeof(int), hipMemcpyHostToDevice));
+      fold_image_size = image_size;
+    }
+    launch_fold_indexed(x, x_mat.p, x_fold_ptr.p, x_fold_off.p, X, idx_patches, n_images, image_size, s);
     RPU_HIP_CHECK(hipGetLastError());
   }
 
@@ -1747,7 +1772,10 @@ int rpu_tile_set_matrix_indices(rpu_tile_t *tile, const int32_t *indices_host, i
       t.sync_last();
       t.x_idx.release();
       t.x_idx_t.release();
+      t.x_fold_ptr.release();
+      t.x_fold_off.release();
     }
+    t.fold_image_size = -1;
     t.idx_host.assign(indices_host, indices_host + (size_t)x_size * patches);
     t.idx_max = 0;
     for (int32_t j : t.idx_host) {

@@ -189,3 +189,30 @@ def test_fused_convolution_forward_draws_what_the_unfolded_pass_draws(gpu_device
         assert (diff <= step * 1.01).all()
         assert (diff > 1e-5).mean() < 0.002
         assert np.abs(want).max() > 0.5
+
+
+def test_indexed_backward_adds_overlapping_patches_in_a_fixed_order(gpu_device):
+    """Input gradients of overlapping patches are summed per image element in a fixed order (no atomics): repeated calls
+    give the same bits, and a perfect tile on values of a binary grid, where no rounding happens, is exact."""
+    rng = np.random.default_rng(4)
+    c_in, c_out, height, width, n = 6, 40, 11, 10, 9
+    indices, patches = conv_indices((c_in, height, width), (3, 3), (1, 1), (1, 1), (1, 1), True)
+    x_size = c_in * 9 + 1
+    host = dv.FloatingPointTileParameter().create_array(x_size, c_out)
+    w = rng.normal(0, 0.1, (c_out, x_size)).astype(np.float32)
+    host.set_weights(torch.from_numpy(w))
+    gpu = tiles.CudaFloatingPointTile(host)
+    gpu.set_matrix_indices(indices)
+    grad = rng.normal(0, 1, (n, c_out, height, width)).astype(np.float32)
+    runs = [gpu.backward_indexed(cuda(grad), torch.empty(n, c_in, height, width).cuda()).clone() for _ in range(3)]
+    assert torch.equal(runs[0], runs[1]) and torch.equal(runs[0], runs[2])
+    weight = torch.from_numpy(w[:, :-1].reshape(c_out, c_in, 3, 3).copy())
+    assert torch.allclose(runs[0].cpu(), F.conv_transpose2d(torch.from_numpy(grad), weight, padding=1), atol=1e-4)
+    # exact arithmetic: integers / 8 times integers / 8, sums far below 2^24 / 64
+    w_grid = (rng.integers(-8, 9, (c_out, x_size)) / 8.0).astype(np.float32)
+    g_grid = (rng.integers(-8, 9, (n, c_out, height, width)) / 8.0).astype(np.float32)
+    gpu.set_weights(torch.from_numpy(w_grid))
+    got = gpu.backward_indexed(cuda(g_grid), torch.empty(n, c_in, height, width).cuda()).cpu()
+    want = F.conv_transpose2d(torch.from_numpy(g_grid).double(),
+                              torch.from_numpy(w_grid[:, :-1].reshape(c_out, c_in, 3, 3).copy()).double(), padding=1)
+    assert torch.equal(got.double(), want)
