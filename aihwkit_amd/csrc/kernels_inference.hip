@@ -221,7 +221,16 @@ __global__ __launch_bounds__(256) void k_fold_indexed(float *images, const float
     const long e = (long)(idx - n * image_size);
     const float *src = x_mat + n * block;
     float acc = 0.0f;
-    for (int t = ptr[e]; t < ptr[e + 1]; ++t) acc += src[off[t]];
+    const int t_end = ptr[e + 1];
+    for (int t0 = ptr[e]; t0 < t_end; t0 += 8) { // eight loads in flight, added in list order
+      float v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) v[u] = (t0 + u < t_end) ? src[off[t0 + u]] : 0.0f;
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        if (t0 + u < t_end) acc += v[u];
+      }
+    }
     images[idx] = acc;
   }
 }
