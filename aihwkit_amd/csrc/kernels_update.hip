@@ -1320,7 +1320,9 @@ void launch_update_pulsed(const UpdateArgs &a, hipStream_t s) {
 // columns per lane (two bits: 1, 2 or 4)
 int update_pulsed_variant(const UpdateArgs &a) {
   const int step = a.dev.kind == RPU_DEVICE_CONSTANT_STEP ? 0 : (a.dev.ls_mult_noise ? 1 : 2);
-  return (step * 2 + (a.dev.dw_min_std > 0.0f ? 1 : 0)) * 4 + update_pulsed_columns(a) / 2;
+  const int cols = update_pulsed_columns(a);
+  const int deep = (cols == 1 && update_pulsed_deep(a)) ? 1 : 0; // block-wise fetch of the planes (long batches)
+  return ((step * 2 + (a.dev.dw_min_std > 0.0f ? 1 : 0)) * 2 + deep) * 4 + cols / 2;
 }
 
 int update_pulsed_workgroups(const UpdateArgs &a) {
@@ -1328,27 +1330,30 @@ int update_pulsed_workgroups(const UpdateArgs &a) {
   return ((a.x_size + 256 * c - 1) / (256 * c)) * a.d_size;
 }
 
-template <bool NOISE, int C> static void launch_update_pulsed_group_t(const UpdateGroup &g, int step, dim3 grid, hipStream_t s) {
+template <bool NOISE, int C, bool DEEP = false>
+static void launch_update_pulsed_group_t(const UpdateGroup &g, int step, dim3 grid, hipStream_t s) {
   if (step == 0) {
-    hipLaunchKernelGGL((k_update_pulsed_group<RPU_DEVICE_CONSTANT_STEP, true, NOISE, C>), grid, dim3(256), 0, s, g);
+    hipLaunchKernelGGL((k_update_pulsed_group<RPU_DEVICE_CONSTANT_STEP, true, NOISE, C, DEEP>), grid, dim3(256), 0, s, g);
   } else if (step == 1) {
-    hipLaunchKernelGGL((k_update_pulsed_group<RPU_DEVICE_LINEAR_STEP, true, NOISE, C>), grid, dim3(256), 0, s, g);
+    hipLaunchKernelGGL((k_update_pulsed_group<RPU_DEVICE_LINEAR_STEP, true, NOISE, C, DEEP>), grid, dim3(256), 0, s, g);
   } else {
-    hipLaunchKernelGGL((k_update_pulsed_group<RPU_DEVICE_LINEAR_STEP, false, NOISE, C>), grid, dim3(256), 0, s, g);
+    hipLaunchKernelGGL((k_update_pulsed_group<RPU_DEVICE_LINEAR_STEP, false, NOISE, C, DEEP>), grid, dim3(256), 0, s, g);
   }
 }
 
 void launch_update_pulsed_group(const UpdateGroup &g, int variant, int total_workgroups, hipStream_t s) {
   const dim3 grid(total_workgroups);
-  const int step = variant >> 3, cols = 1 << (variant & 3); // 1, 2, 4 columns per lane were stored as 0, 1, 2
-  const bool noise = (variant >> 2) & 1;
+  const int step = variant >> 4, cols = 1 << (variant & 3); // 1, 2, 4 columns per lane were stored as 0, 1, 2
+  const bool deep = (variant >> 2) & 1, noise = (variant >> 3) & 1;
   if (noise) {
     if (cols == 4) launch_update_pulsed_group_t<true, 4>(g, step, grid, s);
     else if (cols == 2) launch_update_pulsed_group_t<true, 2>(g, step, grid, s);
+    else if (deep) launch_update_pulsed_group_t<true, 1, true>(g, step, grid, s);
     else launch_update_pulsed_group_t<true, 1>(g, step, grid, s);
   } else {
     if (cols == 4) launch_update_pulsed_group_t<false, 4>(g, step, grid, s);
     else if (cols == 2) launch_update_pulsed_group_t<false, 2>(g, step, grid, s);
+    else if (deep) launch_update_pulsed_group_t<false, 1, true>(g, step, grid, s);
     else launch_update_pulsed_group_t<false, 1>(g, step, grid, s);
   }
 }

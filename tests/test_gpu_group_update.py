@@ -37,7 +37,7 @@ def make_tiles(rng, shapes, devices, lr=0.01, **up_kw):
     return alone, grouped, oracles
 
 
-@pytest.mark.parametrize("batch", [1, 33, 100, 257])
+@pytest.mark.parametrize("batch", [1, 33, 100, 257, 1100])     # 1100: the long-batch variant of the narrow tiles
 def test_grouped_update_equals_the_tiles_own_update(gpu_device, batch):
     """Tiles of different shapes and three kernel variants (ConstantStep, SoftBounds with and without cycle-to-cycle
     noise, a 1024-wide tile that takes four columns per lane), dense inputs and column slices, two calls in a row."""
