@@ -96,7 +96,25 @@ struct MvmArgs {
   // for the one tile that has xq_first_writer = 1.  Requires rows_ahead_in_init (or a single round).
   float *xq_first[2];
   int xq_first_writer;
+  // Image layouts of the indexed (convolution) interface, where sample b is patch b % group of image b / group and an
+  // image holds its lines one after the other ([image][line][patch]): with in_group / out_group > 0 the element
+  // (b, k) sits a further (b / group) * gs away, so that in_sb = 1, in_sk = group, in_gs = (K - 1) * group
+  // addresses such a tensor directly.  0: plain strides.
+  int in_group, out_group;
+  long in_gs, out_gs;
 };
+
+// offset of sample b's first element in the input / output of a call (see in_group / out_group)
+__host__ __device__ inline long mvm_in_row(const MvmArgs &a, int b) {
+  long off = (long)b * a.in_sb;
+  if (a.in_group) off += (long)(b / a.in_group) * a.in_gs;
+  return off;
+}
+__host__ __device__ inline long mvm_out_row(const MvmArgs &a, int b) {
+  long off = (long)b * a.out_sb;
+  if (a.out_group) off += (long)(b / a.out_group) * a.out_gs;
+  return off;
+}
 
 // noise management + per-sample state for round 0
 void launch_mvm_init(const MvmArgs &a, hipStream_t s);
@@ -361,14 +379,16 @@ void launch_pcm_drift(const float *w_prog, const float *nu_plus, const float *nu
 void launch_mean_abs(const float *v, size_t n, float *out, hipStream_t s);
 
 // ---- indexed (convolution) interface: RPUSimple::copyIndexedInput / copyIndexedOutput / permute132 with
-// trans = true (rpu.cpp:1017-1115, math_util.cpp:319-346).  indices is [x_size][patches]: 0 = padding zero,
-// 1 = bias one, j >= 2 = element j - 2 of the image; images are `image_size` apart.
+// trans = true (rpu.cpp:1017-1115, math_util.cpp:319-346).  The caller's index is [x_size][patches]: 0 = padding
+// zero, 1 = bias one, j >= 2 = element j - 2 of the image; images are `image_size` apart.  The kernels take it
+// patch-major, indices_pk [patches][x_size], the order of the rows they write.
 // x_mat[(n * patches + p) * x_size + k] = value of patch p of image n
-void launch_gather_indexed(float *x_mat, const float *images, const int *indices, int x_size, int patches, int n_images,
+void launch_gather_indexed(float *x_mat, const float *images, const int *indices_pk, int x_size, int patches, int n_images,
                            long image_size, hipStream_t s);
-// images[(j - 2) + n * image_size] = sum of the x_mat entries gathered from that element, without atomics and in the reference's order: ptr [image_size + 1] and off list, per image element, the
-// offsets p * x_size + k of the patch entries gathered from it (every image element is written; no zeroing before)
-void launch_fold_indexed(float *images, const float *x_mat, const int *ptr, const int *off, int x_size, int patches,
+// images[(j - 2) + n * image_size] = sum of the patch entries gathered from that element, without atomics and in the
+// reference's order.  Here x_mat is line-major, [x_size][n_images * patches]; ptr [image_size + 1] and kp list, per
+// image element, the pairs (k, p) of the entries gathered from it (every image element is written; no zeroing before)
+void launch_fold_indexed(float *images, const float *x_mat, const int *ptr, const int *kp, int x_size, int patches,
                          int n_images, long image_size, hipStream_t s);
 // [n][d][p] <-> [(n, p)][d]
 void launch_ndp_to_bd(float *bd, const float *ndp, int n_images, int d_size, int patches, hipStream_t s);

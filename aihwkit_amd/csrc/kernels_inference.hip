@@ -6,6 +6,8 @@
 // The file also holds the gather / fold / permute kernels of the indexed (convolution) interface.
 #include "kernels.h"
 
+#include <algorithm>
+
 namespace rpu_amd {
 
 namespace {
@@ -137,16 +139,26 @@ __global__ __launch_bounds__(1024) void k_mean_abs(const float *v, size_t n, flo
   }
 }
 
-__global__ __launch_bounds__(256) void k_gather_indexed(float *x_mat, const float *images, const int *indices, int x_size,
-                                                         int patches, int n_images, long image_size) {
-  const size_t total = (size_t)n_images * patches * x_size;
-  for (size_t idx = blockIdx.x * (size_t)blockDim.x + threadIdx.x; idx < total; idx += (size_t)gridDim.x * blockDim.x) {
-    const int k = (int)(idx % x_size);
-    const size_t b = idx / x_size;
-    const int p = (int)(b % patches);
-    const size_t n = b / patches;
-    const int j = indices[(size_t)k * patches + p];
-    x_mat[idx] = (j <= 1) ? (float)j : images[(size_t)(j - 2) + n * image_size];
+// Patch matrix of the images: entry (p, k) of image n is the image element that the index names, 0 or 1 (bias row).
+// The index is held patch-major here ([p][k], the order of the rows written), so index reads and stores are unit
+// stride and only the image reads are gathers (neighbouring patches overlap: they hit the caches).
+__global__ __launch_bounds__(256) void k_gather_indexed(float *x_mat, const float *images, const int *indices_pk, long block,
+                                                         int n_images, long image_size) {
+  const long stride = (long)gridDim.x * 1024;
+  for (int n = blockIdx.y; n < n_images; n += gridDim.y)
+  for (long i0 = blockIdx.x * 1024L + threadIdx.x; i0 < block; i0 += stride) {
+    const float *image = images + (size_t)n * image_size;
+    float *dst = x_mat + (size_t)n * block;
+    int j[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) j[u] = (i0 + 256 * u < block) ? indices_pk[i0 + 256 * u] : 0;
+    float v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) v[u] = (j[u] <= 1) ? (float)j[u] : image[j[u] - 2];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      if (i0 + 256 * u < block) dst[i0 + 256 * u] = v[u];
+    }
   }
 }
 
@@ -202,30 +214,41 @@ void launch_pcm_drift(const float *w_prog, const float *nu_plus, const float *nu
                      key, call);
 }
 
-void launch_gather_indexed(float *x_mat, const float *images, const int *indices, int x_size, int patches, int n_images,
+void launch_gather_indexed(float *x_mat, const float *images, const int *indices_pk, int x_size, int patches, int n_images,
                            long image_size, hipStream_t s) {
-  const size_t total = (size_t)n_images * patches * x_size;
-  hipLaunchKernelGGL(k_gather_indexed, dim3(grid_of(total)), dim3(256), 0, s, x_mat, images, indices, x_size, patches,
-                     n_images, image_size);
+  const long block = (long)patches * x_size;
+  long per_image = (block + 1023) / 1024;
+  const long want = std::max(1L, 8192L / n_images); // enough workgroups for the chip, a few passes each at most
+  if (per_image > want) per_image = want;
+  hipLaunchKernelGGL(k_gather_indexed, dim3((unsigned)per_image, (unsigned)std::min(n_images, 65535)), dim3(256), 0, s, x_mat,
+                     images, indices_pk, block, n_images, image_size);
 }
 
 // Fold of the patch matrix back into the images without atomics: image element e of image n is the sum of the patch
-// entries that were gathered from it, listed per element (ptr[e] .. ptr[e + 1] into off: offsets p * x_size + k into an
-// image's block of x_mat) in the order of the reference's loop (math_util / rpu.cpp:1130-1141 walks k, then p), added
-// one after the other from zero: the same bits on every run, and the reference's.
-__global__ __launch_bounds__(256) void k_fold_indexed(float *images, const float *x_mat, const int *ptr, const int *off,
-                                                      long block, int n_images, long image_size) {
+// entries that were gathered from it, listed per element (ptr[e] .. ptr[e + 1] into kp: pairs (k, p) of line and
+// patch) in the order of the reference's loop (math_util / rpu.cpp:1130-1141 walks k, then p), added one after the
+// other from zero: the same bits on every run, and the reference's.  x_mat is line-major, [x_size][n_images * patches]:
+// neighbouring image elements meet the same lines at neighbouring patches, so a wave reads runs of a row.
+__global__ __launch_bounds__(256) void k_fold_indexed(float *images, const float *x_mat, const int *ptr, const int2 *kp,
+                                                      int patches, int n_images, long image_size) {
   const size_t total = (size_t)n_images * image_size;
+  const long row = (long)n_images * patches;
   for (size_t idx = blockIdx.x * (size_t)blockDim.x + threadIdx.x; idx < total; idx += (size_t)gridDim.x * blockDim.x) {
     const size_t n = idx / image_size;
     const long e = (long)(idx - n * image_size);
-    const float *src = x_mat + n * block;
+    const float *src = x_mat + n * patches;
     float acc = 0.0f;
     const int t_end = ptr[e + 1];
     for (int t0 = ptr[e]; t0 < t_end; t0 += 8) { // eight loads in flight, added in list order
       float v[8];
 #pragma unroll
-      for (int u = 0; u < 8; ++u) v[u] = (t0 + u < t_end) ? src[off[t0 + u]] : 0.0f;
+      for (int u = 0; u < 8; ++u) {
+        v[u] = 0.0f;
+        if (t0 + u < t_end) {
+          const int2 at = kp[t0 + u];
+          v[u] = src[(long)at.x * row + at.y];
+        }
+      }
 #pragma unroll
       for (int u = 0; u < 8; ++u) {
         if (t0 + u < t_end) acc += v[u];
@@ -235,11 +258,12 @@ __global__ __launch_bounds__(256) void k_fold_indexed(float *images, const float
   }
 }
 
-void launch_fold_indexed(float *images, const float *x_mat, const int *ptr, const int *off, int x_size, int patches,
+void launch_fold_indexed(float *images, const float *x_mat, const int *ptr, const int *kp, int x_size, int patches,
                          int n_images, long image_size, hipStream_t s) {
+  (void)x_size;
   const size_t total = (size_t)n_images * image_size;
-  hipLaunchKernelGGL(k_fold_indexed, dim3(grid_of(total)), dim3(256), 0, s, images, x_mat, ptr, off, (long)patches * x_size,
-                     n_images, image_size);
+  hipLaunchKernelGGL(k_fold_indexed, dim3(grid_of(total)), dim3(256), 0, s, images, x_mat, ptr,
+                     reinterpret_cast<const int2 *>(kp), patches, n_images, image_size);
 }
 
 void launch_ndp_to_bd(float *bd, const float *ndp, int n_images, int d_size, int patches, hipStream_t s) {

@@ -88,7 +88,7 @@ __device__ __forceinline__ float dac_value(float x, float scale, const IoDev &io
 // this one is number t
 __device__ __forceinline__ void write_dac_row(const MvmArgs &a, int b, int slot, float scale, int round, float *dst,
                                               int t, int width) {
-  const float *row = a.in + (long)b * a.in_sb;
+  const float *row = a.in + mvm_in_row(a, b);
   float *out = dst + (long)slot * a.k_pad;
   for (int k = t; k < a.k_pad; k += width) {
     float v = 0.0f;
@@ -175,7 +175,7 @@ __device__ __forceinline__ void mvm_finish_outputs(const MvmArgs &a, int round, 
                                                    const float *post = nullptr, float *out_rows = nullptr) {
   up = 0;
   lo = 0;
-  float *out_p = a.out + (long)b * a.out_sb + (long)o0 * a.out_so;
+  float *out_p = a.out + mvm_out_row(a, b) + (long)o0 * a.out_so;
   long out_so = a.out_so;
   if (out_rows) { // results kept aside, sample-major: [m_batch][O]
     out_p = out_rows + (long)b * a.O + o0;
@@ -681,7 +681,7 @@ __device__ __forceinline__ void mvm_init_sample(const MvmArgs &a, int b, int t, 
     if (writes) write_dac_row(a, b, b, 1.0f, 0, rows0, t, SUB);
     return;
   }
-  const float *row = a.in + (long)b * a.in_sb;
+  const float *row = a.in + mvm_in_row(a, b);
   // a row of up to 8 elements per thread is read once and kept for the statistics and the quantized rows
   constexpr int KEEP = 8;
   const bool kept = a.k_pad <= KEEP * SUB;
@@ -840,10 +840,12 @@ __device__ __forceinline__ void mvm_prepare_next_rows(const MvmArgs &a, int roun
   const int kq = threadIdx.x & 31, rq = threadIdx.x >> 5;
   float sc[4];
   int bt[4];
+  long ro[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     bt[i] = sh_next_b[4 * rq + i];
     sc[i] = sh_next_scale[4 * rq + i];
+    ro[i] = mvm_in_row(a, bt[i]);
   }
   for (int k0 = k_lo; k0 < k_hi; k0 += 128) {
     float xv[4][4];
@@ -852,7 +854,7 @@ __device__ __forceinline__ void mvm_prepare_next_rows(const MvmArgs &a, int roun
       const int k = k0 + 32 * u + kq;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        xv[u][i] = (k < k_hi && sc[i] != 0.0f && k < a.K) ? in[(long)bt[i] * a.in_sb + (long)k * a.in_sk] : 0.0f;
+        xv[u][i] = (k < k_hi && sc[i] != 0.0f && k < a.K) ? in[ro[i] + (long)k * a.in_sk] : 0.0f;
       }
     }
 #pragma unroll
@@ -1004,7 +1006,7 @@ __device__ __forceinline__ void mvm_dual_select(const MvmArgs &a, int n) {
     const int b = tile_b * TILE + (idx >> 5), o = tile_o * TILE + (idx & 31);
     if (b < a.m_batch && o < a.O) {
       const int sel = a.dual.sel[b];
-      if (sel < 2) a.out[(long)b * a.out_sb + (long)o * a.out_so] = pick2(a.dual.buf, sel)[(long)b * a.O + o];
+      if (sel < 2) a.out[mvm_out_row(a, b) + (long)o * a.out_so] = pick2(a.dual.buf, sel)[(long)b * a.O + o];
     }
   }
 }
@@ -1307,7 +1309,7 @@ __device__ __forceinline__ void big_prepare_next_rows(const MvmArgs &a, int roun
 #pragma unroll
     for (int i = 0; i < RPT; ++i) {
       const int row = rq * RPT + i;
-      xv[i] = (sh_scale[row] != 0.0f && k < a.K) ? in[(long)sh_b[row] * a.in_sb + (long)k * a.in_sk] : 0.0f;
+      xv[i] = (sh_scale[row] != 0.0f && k < a.K) ? in[mvm_in_row(a, sh_b[row]) + (long)k * a.in_sk] : 0.0f;
     }
 #pragma unroll
     for (int i = 0; i < RPT; ++i) {

@@ -219,7 +219,7 @@ struct Tile {
   std::vector<int32_t> idx_host;
   int idx_patches = 0;
   int32_t idx_max = 0; // largest entry of the index matrix
-  DevBuf<int> x_idx, x_idx_t; // [X][patches] as set, and its transpose [patches][X] for the fused forward
+  DevBuf<int> x_idx_t; // the index matrix patch-major, [patches][X] (set as [X][patches])
   DevBuf<int> x_fold_ptr, x_fold_off; // per image element the patch entries gathered from it (backward_indexed)
   long fold_image_size = -1;
   DevBuf<float> x_mat, d_mat;
@@ -336,7 +336,7 @@ struct Tile {
     t_unit.release(); t_read.release();
     i_ref.release(); i_prog.release(); i_nu_plus.release(); i_nu_minus.release(); i_scalar.release(); i_absmax.release();
     has_reference = programmed = false;
-    x_idx.release(); x_idx_t.release(); x_fold_ptr.release(); x_fold_off.release(); fold_image_size = -1;
+    x_idx_t.release(); x_fold_ptr.release(); x_fold_off.release(); fold_image_size = -1;
     x_mat.release(); d_mat.release();
     d_decay.release(); d_diff.release(); d_rbias.release(); s_clip.release();
     state_params_valid = false;
@@ -668,8 +668,11 @@ struct Tile {
     prof_mark(s, "pre_adc_terms");
   }
 
+  // in_images / out_images > 0: that side is an image tensor [image][line][patch] with so many patches per image and
+  // sample b = patch b % patches of image b / patches (no bias column then)
   void mvm(const float *in, float *out, int B, bool bias, bool in_trans, bool out_trans, bool transposed, hipStream_t s,
-           const float *w_other = nullptr, const IOPar *io_other = nullptr, bool is_test = false) {
+           const float *w_other = nullptr, const IOPar *io_other = nullptr, bool is_test = false, int in_images = 0,
+           int out_images = 0) {
     const IOPar &io = io_other ? *io_other : (transposed ? bio : fio);
     const bool side = has_pre_adc_terms(io);
     MvmArgs a = mvm_args(B, transposed, w_other ? w_other : mvm_weights(is_test), io, side ? 0 : -1);
@@ -694,6 +697,14 @@ struct Tile {
       } else {
         a.out = out; a.out_sb = out_trans ? 1 : X; a.out_so = out_trans ? B : 1;
       }
+    }
+
+    if ((in_images || out_images) && bias) throw RpuError("Image layouts carry no bias column.");
+    if (in_images) {
+      a.in_sb = 1; a.in_sk = in_images; a.in_group = in_images; a.in_gs = (long)(a.K - 1) * in_images;
+    }
+    if (out_images) {
+      a.out_sb = 1; a.out_so = out_images; a.out_group = out_images; a.out_gs = (long)(a.O - 1) * out_images;
     }
 
     prof_begin(s);
@@ -1364,16 +1375,23 @@ struct Tile {
 
   // ---- indexed (convolution) interface ---------------------------------------------------------------
 
-  void ensure_indexed(int n_images) {
+  // the index matrix as the kernels read it: [patches][X], the order of the rows of the patch matrix
+  void ensure_patch_major_index() {
+    if (x_idx_t.p) return;
+    std::vector<int32_t> tr((size_t)X * idx_patches);
+    for (int k = 0; k < X; ++k)
+      for (int p = 0; p < idx_patches; ++p) tr[(size_t)p * X + k] = idx_host[(size_t)k * idx_patches + p];
+    x_idx_t.ensure(tr.size());
+    RPU_HIP_CHECK(hipMemcpy(x_idx_t.p, tr.data(), tr.size() * sizeof(int32_t), hipMemcpyHostToDevice));
+  }
+
+  void ensure_indexed(int n_images, bool with_d_mat = true) {
     if (idx_patches <= 0) throw RpuError("The index matrix has not been set (set_matrix_indices).");
     if (n_images <= 0) throw RpuError("n_images must be positive.");
-    if (!x_idx.p) {
-      x_idx.ensure(idx_host.size());
-      RPU_HIP_CHECK(hipMemcpy(x_idx.p, idx_host.data(), idx_host.size() * sizeof(int32_t), hipMemcpyHostToDevice));
-    }
+    ensure_patch_major_index();
     const size_t B = (size_t)n_images * idx_patches;
     x_mat.ensure(B * X);
-    d_mat.ensure(B * D);
+    if (with_d_mat) d_mat.ensure(B * D);
   }
 
   void forward_indexed(const float *x, float *d, int n_images, long image_size, bool is_test, hipStream_t s) {
@@ -1390,13 +1408,7 @@ struct Tile {
       a.max_rounds = fio.perfect ? 0 : mvm_max_rounds(a.io);
       a.st.rounds = s_rounds.p;
       if (conv_forward_supported(a)) {
-        if (!x_idx_t.p) {
-          std::vector<int32_t> tr((size_t)X * idx_patches);
-          for (int k = 0; k < X; ++k)
-            for (int p = 0; p < idx_patches; ++p) tr[(size_t)p * X + k] = idx_host[(size_t)k * idx_patches + p];
-          x_idx_t.ensure(tr.size());
-          RPU_HIP_CHECK(hipMemcpy(x_idx_t.p, tr.data(), tr.size() * sizeof(int32_t), hipMemcpyHostToDevice));
-        }
+        ensure_patch_major_index();
         a.key = key(); a.call = call++;
         ConvArgs c{x, x_idx_t.p, d, idx_patches, n_images, image_size};
         prof_begin(s);
@@ -1408,19 +1420,21 @@ struct Tile {
         return;
       }
     }
-    ensure_indexed(n_images);
+    ensure_indexed(n_images, false);
     const int B = n_images * idx_patches;
-    launch_gather_indexed(x_mat.p, x, x_idx.p, X, idx_patches, n_images, image_size, s);
-    mvm(x_mat.p, d_mat.p, B, false, false, false, false, s, nullptr, nullptr, is_test);
-    launch_bd_to_ndp(d, d_mat.p, n_images, D, idx_patches, s);
+    launch_gather_indexed(x_mat.p, x, x_idx_t.p, X, idx_patches, n_images, image_size, s);
+    // the outputs go straight into the caller's [image][output][patch] tensor
+    mvm(x_mat.p, d, B, false, false, false, false, s, nullptr, nullptr, is_test, 0, idx_patches);
     RPU_HIP_CHECK(hipGetLastError());
   }
 
   void backward_indexed(const float *d, float *x, int n_images, long image_size, hipStream_t s) {
-    ensure_indexed(n_images);
+    ensure_indexed(n_images, false);
     const int B = n_images * idx_patches;
-    launch_ndp_to_bd(d_mat.p, d, n_images, D, idx_patches, s);
-    mvm(d_mat.p, x_mat.p, B, false, false, false, true, s);
+    // the caller's [image][output][patch] tensor is read in place; the patch matrix comes out line-major, [X][B]:
+    // stores of a wave (one sample per lane) and the reads of the fold (neighbouring image elements meet neighbouring
+    // patches) are then unit stride
+    mvm(d, x_mat.p, B, false, false, true, true, s, nullptr, nullptr, false, idx_patches, 0);
     if (fold_image_size != image_size) {
       // per image element, the entries of the patch matrix that were gathered from it, in the order in which the
       // reference's loop adds them up (k, then p)
@@ -1430,11 +1444,15 @@ struct Tile {
         if (j > 1) ++ptr[(size_t)(j - 2) + 1];
       }
       for (long e = 0; e < image_size; ++e) ptr[(size_t)e + 1] += ptr[(size_t)e];
-      std::vector<int> off((size_t)ptr[(size_t)image_size]), cursor(ptr.begin(), ptr.end() - 1);
+      std::vector<int> off(2 * (size_t)ptr[(size_t)image_size]), cursor(ptr.begin(), ptr.end() - 1);
       for (int k = 0; k < X; ++k) {
         for (int p = 0; p < idx_patches; ++p) {
           const int32_t j = idx_host[(size_t)k * idx_patches + p];
-          if (j > 1) off[(size_t)cursor[(size_t)(j - 2)]++] = p * X + k;
+          if (j > 1) {
+            const size_t at = 2 * (size_t)cursor[(size_t)(j - 2)]++;
+            off[at] = k;
+            off[at + 1] = p;
+          }
         }
       }
       sync_last(); // the lists of another image size may still be read
@@ -1451,7 +1469,7 @@ struct Tile {
   void update_indexed(const float *x, const float *d, int n_images, long image_size, hipStream_t s) {
     ensure_indexed(n_images);
     const int B = n_images * idx_patches;
-    launch_gather_indexed(x_mat.p, x, x_idx.p, X, idx_patches, n_images, image_size, s);
+    launch_gather_indexed(x_mat.p, x, x_idx_t.p, X, idx_patches, n_images, image_size, s);
     launch_ndp_to_bd(d_mat.p, d, n_images, D, idx_patches, s);
     update(x_mat.p, d_mat.p, B, false, false, false, s);
     RPU_HIP_CHECK(hipGetLastError());
@@ -1770,7 +1788,6 @@ int rpu_tile_set_matrix_indices(rpu_tile_t *tile, const int32_t *indices_host, i
     if (t.resident()) {
       DeviceGuard g(t.device_id);
       t.sync_last();
-      t.x_idx.release();
       t.x_idx_t.release();
       t.x_fold_ptr.release();
       t.x_fold_off.release();

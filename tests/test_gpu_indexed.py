@@ -216,3 +216,36 @@ def test_indexed_backward_adds_overlapping_patches_in_a_fixed_order(gpu_device):
     want = F.conv_transpose2d(torch.from_numpy(g_grid).double(),
                               torch.from_numpy(w_grid[:, :-1].reshape(c_out, c_in, 3, 3).copy()).double(), padding=1)
     assert torch.equal(got.double(), want)
+
+
+@pytest.mark.parametrize("c_out", [40, 136])      # outputs below and above the width from which forward takes large tiles
+def test_wide_convolution_on_many_patches_equals_the_pass_over_the_unfolded_images(gpu_device, c_out):
+    """2048 patches of 145 elements: the contraction kernels (the large-tile one for the backward pass, and for the
+    forward pass of the wider tile) read the gradient tensor [image][output][patch] and write the output tensor in place;
+    same bits as the pass over the patch matrix that torch unfolds, and the fold of that pass's input gradients."""
+    rng = np.random.default_rng(12)
+    c_in, side, n = 16, 16, 8
+    indices, patches = conv_indices((c_in, side, side), (3, 3), (1, 1), (1, 1), (1, 1), True)
+    x_size = c_in * 9 + 1
+    f_io = noise_free_io(inp_res=1 / 128.0, out_res=1 / 512.0, out_bound=2.0, noise_management=dv.NoiseManagementType.AbsMax,
+                         bound_management=dv.BoundManagementType.Iterative)
+    b_io = noise_free_io(inp_res=1 / 128.0, out_res=1 / 512.0, noise_management=dv.NoiseManagementType.AbsMax)
+    dev = constant_step(dw_min=0.002, dw_min_std=0.0, construction_seed=4, w_max_dtod=0.0, w_min_dtod=0.0, w_max=1.0, w_min=-1.0)
+    _host, _orc, gpu = build_pair(make_meta(f_io, b_io), dev, x_size, c_out)
+    gpu.set_weights(torch.from_numpy(rng.normal(0, 0.25, (c_out, x_size)).astype(np.float32)))
+    gpu.set_matrix_indices(indices)
+    x = torch.from_numpy(rng.normal(0, 1, (n, c_in, side, side)).astype(np.float32)).cuda()
+    y = gpu.forward_indexed(x, torch.empty(n, c_out, side, side).cuda())
+    rounds = gpu.get_bm_rounds(n * patches)
+    assert rounds.max() > 1 and (rounds == 1).any()                  # some patches saturate the ADC, others do not
+    unfolded = torch.cat([F.unfold(x, 3, padding=1), torch.ones(n, 1, patches).cuda()], dim=1)      # [n, x_size, patches]
+    x_mat = unfolded.permute(0, 2, 1).reshape(n * patches, x_size).contiguous()
+    y_mat = gpu.forward(x_mat)
+    assert torch.equal(y, y_mat.reshape(n, patches, c_out).permute(0, 2, 1).reshape(n, c_out, side, side))
+    grad = torch.from_numpy((0.3 * rng.normal(0, 1, (n, c_out, side, side))).astype(np.float32)).cuda()
+    dx = gpu.backward_indexed(grad, torch.empty(n, c_in, side, side).cuda())
+    d_mat = grad.reshape(n, c_out, patches).permute(0, 2, 1).reshape(n * patches, c_out).contiguous()
+    back = gpu.backward(d_mat).reshape(n, patches, x_size)[:, :, :-1].permute(0, 2, 1)                # bias column dropped
+    want = F.fold(back.double(), (side, side), 3, padding=1)
+    assert (dx.double() - want).abs().max() <= 1e-5 * want.abs().max()
+    assert dx.abs().max() > 0.1
