@@ -380,11 +380,11 @@ void launch_mean_abs(const float *v, size_t n, float *out, hipStream_t s);
 
 // ---- indexed (convolution) interface: RPUSimple::copyIndexedInput / copyIndexedOutput / permute132 with
 // trans = true (rpu.cpp:1017-1115, math_util.cpp:319-346).  The caller's index is [x_size][patches]: 0 = padding
-// zero, 1 = bias one, j >= 2 = element j - 2 of the image; images are `image_size` apart.  The kernels take it
-// patch-major, indices_pk [patches][x_size], the order of the rows they write.
-// x_mat[(n * patches + p) * x_size + k] = value of patch p of image n
-void launch_gather_indexed(float *x_mat, const float *images, const int *indices_pk, int x_size, int patches, int n_images,
-                           long image_size, hipStream_t s);
+// zero, 1 = bias one, j >= 2 = element j - 2 of the image; images are `image_size` apart.
+// x_mat[(n * patches + p) * x_ld + k] = value of patch p of image n (x_ld >= x_size: rows may be padded so that they
+// start on cache lines)
+void launch_gather_indexed(float *x_mat, const float *images, const int *indices, int x_size, int x_ld, int patches,
+                           int n_images, long image_size, hipStream_t s);
 // images[(j - 2) + n * image_size] = sum of the patch entries gathered from that element, without atomics and in the
 // reference's order.  Here x_mat is line-major, [x_size][n_images * patches]; ptr [image_size + 1] and kp list, per
 // image element, the pairs (k, p) of the entries gathered from it (every image element is written; no zeroing before)

@@ -140,25 +140,33 @@ __global__ __launch_bounds__(1024) void k_mean_abs(const float *v, size_t n, flo
 }
 
 // Patch matrix of the images: entry (p, k) of image n is the image element that the index names, 0 or 1 (bias row).
-// The index is held patch-major here ([p][k], the order of the rows written), so index reads and stores are unit
-// stride and only the image reads are gathers (neighbouring patches overlap: they hit the caches).
-__global__ __launch_bounds__(256) void k_gather_indexed(float *x_mat, const float *images, const int *indices_pk, long block,
-                                                         int n_images, long image_size) {
-  const long stride = (long)gridDim.x * 1024;
-  for (int n = blockIdx.y; n < n_images; n += gridDim.y)
-  for (long i0 = blockIdx.x * 1024L + threadIdx.x; i0 < block; i0 += stride) {
+// A workgroup moves a block of 64 patches x 64 lines through LDS: it reads with lanes along the patches, the order
+// of the index matrix [x_size][patches] and, for a convolution, of the image rows (neighbouring patches read
+// neighbouring elements), and writes with lanes along the lines, the order of the rows of x_mat.
+__global__ __launch_bounds__(256) void k_gather_indexed(float *x_mat, const float *images, const int *indices, int x_size,
+                                                         int x_ld, int patches, int n_images, long image_size) {
+  __shared__ float tile[64][65];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int blocks_p = (patches + 63) / 64;
+  const int p0 = (int)(blockIdx.x % blocks_p) * 64, k0 = (int)(blockIdx.x / blocks_p) * 64;
+  for (int n = blockIdx.y; n < n_images; n += gridDim.y) {
     const float *image = images + (size_t)n * image_size;
-    float *dst = x_mat + (size_t)n * block;
-    int j[4];
+    int j[16];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) j[u] = (i0 + 256 * u < block) ? indices_pk[i0 + 256 * u] : 0;
-    float v[4];
-#pragma unroll
-    for (int u = 0; u < 4; ++u) v[u] = (j[u] <= 1) ? (float)j[u] : image[j[u] - 2];
-#pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      if (i0 + 256 * u < block) dst[i0 + 256 * u] = v[u];
+    for (int i = 0; i < 16; ++i) {
+      const int k = k0 + wave * 16 + i, p = p0 + lane;
+      j[i] = (k < x_size && p < patches) ? indices[(size_t)k * patches + p] : 0;
     }
+#pragma unroll
+    for (int i = 0; i < 16; ++i) tile[lane][wave * 16 + i] = (j[i] <= 1) ? (float)j[i] : image[j[i] - 2];
+    __syncthreads();
+    float *dst = x_mat + ((size_t)n * patches + p0) * x_ld + k0;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int row = i * 4 + wave;
+      if (p0 + row < patches && k0 + lane < x_size) dst[(size_t)row * x_ld + lane] = tile[row][lane];
+    }
+    __syncthreads();
   }
 }
 
@@ -214,14 +222,11 @@ void launch_pcm_drift(const float *w_prog, const float *nu_plus, const float *nu
                      key, call);
 }
 
-void launch_gather_indexed(float *x_mat, const float *images, const int *indices_pk, int x_size, int patches, int n_images,
-                           long image_size, hipStream_t s) {
-  const long block = (long)patches * x_size;
-  long per_image = (block + 1023) / 1024;
-  const long want = std::max(1L, 8192L / n_images); // enough workgroups for the chip, a few passes each at most
-  if (per_image > want) per_image = want;
-  hipLaunchKernelGGL(k_gather_indexed, dim3((unsigned)per_image, (unsigned)std::min(n_images, 65535)), dim3(256), 0, s, x_mat,
-                     images, indices_pk, block, n_images, image_size);
+void launch_gather_indexed(float *x_mat, const float *images, const int *indices, int x_size, int x_ld, int patches,
+                           int n_images, long image_size, hipStream_t s) {
+  const unsigned blocks = (unsigned)(((patches + 63) / 64) * ((x_size + 63) / 64));
+  hipLaunchKernelGGL(k_gather_indexed, dim3(blocks, (unsigned)std::min(n_images, 65535)), dim3(256), 0, s, x_mat, images,
+                     indices, x_size, x_ld, patches, n_images, image_size);
 }
 
 // Fold of the patch matrix back into the images without atomics: image element e of image n is the sum of the patch

@@ -1366,7 +1366,7 @@ __device__ __forceinline__ void mvm_big_workgroup(const MvmArgs &a, const int ro
   const int tile_b = ((n >> 3) / ((a.O + BT - 1) / BT)) * 8 + (n & 7);
   if (tile_b * BB >= n_act) return;
   const bool more_rounds = round + 1 < a.max_rounds;
-  if (more_rounds && !(round == 0 && a.rows_ahead_in_init)) {
+  if (more_rounds && a.speculate && !(round == 0 && a.rows_ahead_in_init)) {
     big_prepare_next_rows<BB>(a, round, tile_o, tile_b, n_act, sh_b, sh_scale);
   }
 
@@ -1588,12 +1588,32 @@ __device__ __forceinline__ void mvm_big_workgroup(const MvmArgs &a, const int ro
   }
   __syncthreads();
   if (!sh_last) return;
+  const bool ahead = a.speculate != 0;
+  if (!ahead) { // sh_last becomes the number of samples of this tile that go on
+    __syncthreads();
+    if (t == 0) sh_last = 0;
+    __syncthreads();
+  }
   if (t < BB) {
     const int slot = tile_b * BB + t;
     if (slot < n_act) {
-      float scale;
-      mvm_advance_sample(a, round, (round > 0) ? pick2(a.st.list, round & 1)[slot] : slot, slot, true, scale);
+      float scale = 0.0f;
+      const int b = (round > 0) ? pick2(a.st.list, round & 1)[slot] : slot;
+      const int pos = mvm_advance_sample(a, round, b, slot, ahead, scale);
+      if (pos >= 0 && !ahead) {
+        const int i = atomicAdd(&sh_last, 1);
+        sh_b[i] = b;
+        sh_hits[i] = pos;
+        sh_scale[i] = scale;
+      }
     }
+  }
+  if (ahead) return;
+  // nothing was quantized ahead (a long batch on a narrow tile: few samples go on, and every row written ahead
+  // would be paid for): the rows of the samples that do go on are written now
+  __syncthreads();
+  for (int i = 0; i < sh_last; ++i) {
+    write_dac_row(a, sh_b[i], sh_hits[i], sh_scale[i], round + 1, pick2(a.xq, (round + 1) & 1), t, 256);
   }
 }
 
@@ -2134,7 +2154,10 @@ static int big_threshold(int m_batch, int O) {
   // measured on the 1024 x 1024 tile: the half tiles overtake the 32 x 32 kernel at about 1500 samples (backward 70
   // against 88 us at 1536, 74 against 113 us at 2000; at 1024 the 32 x 32 kernel still leads, 63 against 68 us)
   constexpr int big_min = 1536;
-  if (m_batch < big_min || O < 128) return 0;
+  // narrower tiles (the patches of a convolution): part of the 128 outputs of a tile are idle, but a staged operand
+  // byte still meets four times the multiply-adds of the 32 x 32 kernel
+  constexpr int narrow_min_batch = 16384, narrow_min_outputs = 33;
+  if (m_batch < big_min || O < narrow_min_outputs || (O < 128 && m_batch < narrow_min_batch)) return 0;
   const int tiles_o = (O + 127) / 128, tiles_b = (m_batch + 63) / 64;
   if (8 * tiles_o * ((tiles_b + 7) / 8) < 128) return 0;
   return big_min;

@@ -219,7 +219,7 @@ struct Tile {
   std::vector<int32_t> idx_host;
   int idx_patches = 0;
   int32_t idx_max = 0; // largest entry of the index matrix
-  DevBuf<int> x_idx_t; // the index matrix patch-major, [patches][X] (set as [X][patches])
+  DevBuf<int> x_idx, x_idx_t; // the index matrix as set, [X][patches], and patch-major, [patches][X] (fused forward)
   DevBuf<int> x_fold_ptr, x_fold_off; // per image element the patch entries gathered from it (backward_indexed)
   long fold_image_size = -1;
   DevBuf<float> x_mat, d_mat;
@@ -336,7 +336,7 @@ struct Tile {
     t_unit.release(); t_read.release();
     i_ref.release(); i_prog.release(); i_nu_plus.release(); i_nu_minus.release(); i_scalar.release(); i_absmax.release();
     has_reference = programmed = false;
-    x_idx_t.release(); x_fold_ptr.release(); x_fold_off.release(); fold_image_size = -1;
+    x_idx.release(); x_idx_t.release(); x_fold_ptr.release(); x_fold_off.release(); fold_image_size = -1;
     x_mat.release(); d_mat.release();
     d_decay.release(); d_diff.release(); d_rbias.release(); s_clip.release();
     state_params_valid = false;
@@ -510,7 +510,7 @@ struct Tile {
     // rounds) or when at least four workgroups per sample tile share that work; a large batch on a narrow tile
     // quantizes only the rows of the samples that saturated
     a.speculate = (B <= 1024 || O > 96) ? 1 : 0;
-    a.rows_ahead_in_init = (a.speculate || tight) ? 1 : 0;
+    a.rows_ahead_in_init = a.speculate;
     return a;
   }
 
@@ -672,7 +672,7 @@ struct Tile {
   // sample b = patch b % patches of image b / patches (no bias column then)
   void mvm(const float *in, float *out, int B, bool bias, bool in_trans, bool out_trans, bool transposed, hipStream_t s,
            const float *w_other = nullptr, const IOPar *io_other = nullptr, bool is_test = false, int in_images = 0,
-           int out_images = 0) {
+           int out_images = 0, long in_ld = 0) {
     const IOPar &io = io_other ? *io_other : (transposed ? bio : fio);
     const bool side = has_pre_adc_terms(io);
     MvmArgs a = mvm_args(B, transposed, w_other ? w_other : mvm_weights(is_test), io, side ? 0 : -1);
@@ -700,6 +700,10 @@ struct Tile {
     }
 
     if ((in_images || out_images) && bias) throw RpuError("Image layouts carry no bias column.");
+    if (in_ld) { // padded rows of a plain row-major input
+      if (in_trans || bias || in_images) throw RpuError("A row stride goes with a plain row-major input only.");
+      a.in_sb = in_ld;
+    }
     if (in_images) {
       a.in_sb = 1; a.in_sk = in_images; a.in_group = in_images; a.in_gs = (long)(a.K - 1) * in_images;
     }
@@ -1375,7 +1379,7 @@ struct Tile {
 
   // ---- indexed (convolution) interface ---------------------------------------------------------------
 
-  // the index matrix as the kernels read it: [patches][X], the order of the rows of the patch matrix
+  // the index matrix as the fused forward kernels read it: [patches][X], the order of the rows of the patch matrix
   void ensure_patch_major_index() {
     if (x_idx_t.p) return;
     std::vector<int32_t> tr((size_t)X * idx_patches);
@@ -1385,12 +1389,18 @@ struct Tile {
     RPU_HIP_CHECK(hipMemcpy(x_idx_t.p, tr.data(), tr.size() * sizeof(int32_t), hipMemcpyHostToDevice));
   }
 
+  // rows of the patch matrix start on 128-byte lines: a workgroup's stores then fill whole lines
+  int x_mat_ld() const { return (X + 31) & ~31; }
+
   void ensure_indexed(int n_images, bool with_d_mat = true) {
     if (idx_patches <= 0) throw RpuError("The index matrix has not been set (set_matrix_indices).");
     if (n_images <= 0) throw RpuError("n_images must be positive.");
-    ensure_patch_major_index();
+    if (!x_idx.p) {
+      x_idx.ensure(idx_host.size());
+      RPU_HIP_CHECK(hipMemcpy(x_idx.p, idx_host.data(), idx_host.size() * sizeof(int32_t), hipMemcpyHostToDevice));
+    }
     const size_t B = (size_t)n_images * idx_patches;
-    x_mat.ensure(B * X);
+    x_mat.ensure(B * (size_t)x_mat_ld());
     if (with_d_mat) d_mat.ensure(B * D);
   }
 
@@ -1422,9 +1432,9 @@ struct Tile {
     }
     ensure_indexed(n_images, false);
     const int B = n_images * idx_patches;
-    launch_gather_indexed(x_mat.p, x, x_idx_t.p, X, idx_patches, n_images, image_size, s);
+    launch_gather_indexed(x_mat.p, x, x_idx.p, X, x_mat_ld(), idx_patches, n_images, image_size, s);
     // the outputs go straight into the caller's [image][output][patch] tensor
-    mvm(x_mat.p, d, B, false, false, false, false, s, nullptr, nullptr, is_test, 0, idx_patches);
+    mvm(x_mat.p, d, B, false, false, false, false, s, nullptr, nullptr, is_test, 0, idx_patches, x_mat_ld());
     RPU_HIP_CHECK(hipGetLastError());
   }
 
@@ -1469,7 +1479,7 @@ struct Tile {
   void update_indexed(const float *x, const float *d, int n_images, long image_size, hipStream_t s) {
     ensure_indexed(n_images);
     const int B = n_images * idx_patches;
-    launch_gather_indexed(x_mat.p, x, x_idx_t.p, X, idx_patches, n_images, image_size, s);
+    launch_gather_indexed(x_mat.p, x, x_idx.p, X, X, idx_patches, n_images, image_size, s);
     launch_ndp_to_bd(d_mat.p, d, n_images, D, idx_patches, s);
     update(x_mat.p, d_mat.p, B, false, false, false, s);
     RPU_HIP_CHECK(hipGetLastError());
@@ -1788,6 +1798,7 @@ int rpu_tile_set_matrix_indices(rpu_tile_t *tile, const int32_t *indices_host, i
     if (t.resident()) {
       DeviceGuard g(t.device_id);
       t.sync_last();
+      t.x_idx.release();
       t.x_idx_t.release();
       t.x_fold_ptr.release();
       t.x_fold_off.release();
