@@ -96,25 +96,17 @@ struct MvmArgs {
   // for the one tile that has xq_first_writer = 1.  Requires rows_ahead_in_init (or a single round).
   float *xq_first[2];
   int xq_first_writer;
-  // Image layouts of the indexed (convolution) interface, where sample b is patch b % group of image b / group and an
-  // image holds its lines one after the other ([image][line][patch]): with in_group / out_group > 0 the element
-  // (b, k) sits a further (b / group) * gs away, so that in_sb = 1, in_sk = group, in_gs = (K - 1) * group
-  // addresses such a tensor directly.  0: plain strides.
-  int in_group, out_group;
-  long in_gs, out_gs;
+  // Input gathered through an index (the patches of a convolution, never materialized) when in_index is set:
+  // sample b is patch b % in_group of image b / in_group, images are in_gs apart in `in`, and element k of the sample
+  // is what in_index[(b % in_group) * K + k] names: 0, 1 (bias) or, from 2 on, element j - 2 of the image.
+  // in_index_lines is the same index line-major, [K][in_group] (the init kernels read it with lanes along the
+  // patches).  Only for calls that read their input row by row (the gathering init kernels, rows of a further round
+  // written once it is known who goes on: speculate = 0, or a single round).
+  const int *in_index;
+  const int *in_index_lines;
+  int in_group;
+  long in_gs;
 };
-
-// offset of sample b's first element in the input / output of a call (see in_group / out_group)
-__host__ __device__ inline long mvm_in_row(const MvmArgs &a, int b) {
-  long off = (long)b * a.in_sb;
-  if (a.in_group) off += (long)(b / a.in_group) * a.in_gs;
-  return off;
-}
-__host__ __device__ inline long mvm_out_row(const MvmArgs &a, int b) {
-  long off = (long)b * a.out_sb;
-  if (a.out_group) off += (long)(b / a.out_group) * a.out_gs;
-  return off;
-}
 
 // noise management + per-sample state for round 0
 void launch_mvm_init(const MvmArgs &a, hipStream_t s);
@@ -390,6 +382,9 @@ void launch_gather_indexed(float *x_mat, const float *images, const int *indices
 // image element, the pairs (k, p) of the entries gathered from it (every image element is written; no zeroing before)
 void launch_fold_indexed(float *images, const float *x_mat, const int *ptr, const int *kp, int x_size, int patches,
                          int n_images, long image_size, hipStream_t s);
+// [n][line][p] <-> [line][(n, p)]: what a contraction call reads or writes with its transposed layouts
+void launch_images_to_lines(float *lines_major, const float *images, int n_images, int lines, int patches, hipStream_t s);
+void launch_lines_to_images(float *images, const float *lines_major, int n_images, int lines, int patches, hipStream_t s);
 // [n][d][p] <-> [(n, p)][d]
 void launch_ndp_to_bd(float *bd, const float *ndp, int n_images, int d_size, int patches, hipStream_t s);
 void launch_bd_to_ndp(float *ndp, const float *bd, int n_images, int d_size, int patches, hipStream_t s);

@@ -192,6 +192,24 @@ __global__ __launch_bounds__(256) void k_ndp_bd(float *dst, const float *src, in
   }
 }
 
+// [image][line][patch] <-> [line][image][patch]: runs of `patches` elements move as they are
+__global__ __launch_bounds__(256) void k_images_lines(float *dst, const float *src, int n_images, int lines, int patches,
+                                                       int to_lines) {
+  const size_t total = (size_t)n_images * lines * patches;
+  for (size_t idx = blockIdx.x * (size_t)blockDim.x + threadIdx.x; idx < total; idx += (size_t)gridDim.x * blockDim.x) {
+    const int p = (int)(idx % patches);
+    const size_t r = idx / patches;
+    // idx walks the destination with unit stride
+    if (to_lines) {
+      const int n = (int)(r % n_images), l = (int)(r / n_images);
+      dst[idx] = src[((size_t)n * lines + l) * patches + p];
+    } else {
+      const int l = (int)(r % lines), n = (int)(r / lines);
+      dst[idx] = src[((size_t)l * n_images + n) * patches + p];
+    }
+  }
+}
+
 __global__ void k_fill(float *p, float value, size_t n) {
   for (size_t idx = blockIdx.x * (size_t)blockDim.x + threadIdx.x; idx < n; idx += (size_t)gridDim.x * blockDim.x) p[idx] = value;
 }
@@ -269,6 +287,16 @@ void launch_fold_indexed(float *images, const float *x_mat, const int *ptr, cons
   const size_t total = (size_t)n_images * image_size;
   hipLaunchKernelGGL(k_fold_indexed, dim3(grid_of(total)), dim3(256), 0, s, images, x_mat, ptr,
                      reinterpret_cast<const int2 *>(kp), patches, n_images, image_size);
+}
+
+void launch_images_to_lines(float *lines_major, const float *images, int n_images, int lines, int patches, hipStream_t s) {
+  const size_t total = (size_t)n_images * lines * patches;
+  hipLaunchKernelGGL(k_images_lines, dim3(grid_of(total)), dim3(256), 0, s, lines_major, images, n_images, lines, patches, 1);
+}
+
+void launch_lines_to_images(float *images, const float *lines_major, int n_images, int lines, int patches, hipStream_t s) {
+  const size_t total = (size_t)n_images * lines * patches;
+  hipLaunchKernelGGL(k_images_lines, dim3(grid_of(total)), dim3(256), 0, s, images, lines_major, n_images, lines, patches, 0);
 }
 
 void launch_ndp_to_bd(float *bd, const float *ndp, int n_images, int d_size, int patches, hipStream_t s) {

@@ -84,12 +84,38 @@ __device__ __forceinline__ float dac_value(float x, float scale, const IoDev &io
   return v;
 }
 
+// a sample's input row when the call gathers its input through an index (a.in_index)
+struct MvmGatherRow {
+  const float *image; // element j - 2 at image[j]
+  const int *idx;
+  __device__ __forceinline__ float at(int k) const {
+    const int j = idx[k];
+    return j <= 1 ? (float)j : image[j];
+  }
+};
+__device__ __forceinline__ MvmGatherRow mvm_gather_row(const MvmArgs &a, int b) {
+  const int n = b / a.in_group;
+  return MvmGatherRow{a.in + (long)n * a.in_gs - 2, a.in_index + (long)(b - n * a.in_group) * a.K};
+}
+
 // quantized copy of sample b's input row into row `slot` of a scratch matrix, by `width` threads of which
 // this one is number t
 __device__ __forceinline__ void write_dac_row(const MvmArgs &a, int b, int slot, float scale, int round, float *dst,
                                               int t, int width) {
-  const float *row = a.in + mvm_in_row(a, b);
   float *out = dst + (long)slot * a.k_pad;
+  if (a.in_index) {
+    const MvmGatherRow row = mvm_gather_row(a, b);
+    for (int k = t; k < a.k_pad; k += width) {
+      float v = 0.0f;
+      if (k < a.K) {
+        v = row.at(k);
+        if (!a.io.perfect) v = dac_value(v, scale, a.io, a.key, a.call, round, b, k);
+      }
+      out[k] = v;
+    }
+    return;
+  }
+  const float *row = a.in + (long)b * a.in_sb;
   for (int k = t; k < a.k_pad; k += width) {
     float v = 0.0f;
     if (k < a.K) {
@@ -175,7 +201,7 @@ __device__ __forceinline__ void mvm_finish_outputs(const MvmArgs &a, int round, 
                                                    const float *post = nullptr, float *out_rows = nullptr) {
   up = 0;
   lo = 0;
-  float *out_p = a.out + mvm_out_row(a, b) + (long)o0 * a.out_so;
+  float *out_p = a.out + (long)b * a.out_sb + (long)o0 * a.out_so;
   long out_so = a.out_so;
   if (out_rows) { // results kept aside, sample-major: [m_batch][O]
     out_p = out_rows + (long)b * a.O + o0;
@@ -681,7 +707,7 @@ __device__ __forceinline__ void mvm_init_sample(const MvmArgs &a, int b, int t, 
     if (writes) write_dac_row(a, b, b, 1.0f, 0, rows0, t, SUB);
     return;
   }
-  const float *row = a.in + mvm_in_row(a, b);
+  const float *row = a.in + (long)b * a.in_sb;
   // a row of up to 8 elements per thread is read once and kept for the statistics and the quantized rows
   constexpr int KEEP = 8;
   const bool kept = a.k_pad <= KEEP * SUB;
@@ -797,6 +823,119 @@ __global__ __launch_bounds__(256) void k_mvm_init(MvmArgs a) {
   mvm_init_sample<SUB>(a, b, threadIdx.x % SUB, blockIdx.x * 256L + threadIdx.x, gridDim.x * 256L, sh);
 }
 
+// Init kernels of a call whose samples are patches gathered from images (MvmArgs::in_index).  Both read with lanes
+// along the patches: that follows the index matrix as it is set ([K][patches]) and, for a convolution, the image rows
+// (neighbouring patches read neighbouring elements).  Same per-sample state and the same DAC draws (keyed by sample
+// and element) as mvm_init_sample on the materialized patch matrix.  For noise management none / constant / abs-max /
+// max; the other kinds run mvm_init_sample, which gathers row by row.
+//
+// First kernel (abs-max / max only): a workgroup of 16 waves owns 64 patches of one image, one per lane; wave w takes
+// the elements k = w (mod 16), so a patch's largest input is a running maximum of its lane and the waves meet in LDS.
+// The noise-management value goes to st.nm.
+__global__ __launch_bounds__(1024) void k_mvm_gather_max(MvmArgs a) {
+  __shared__ float sh_max[2][16][64];
+  const IoDev &io = a.io;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int P = a.in_group;
+  const int blocks_p = (P + 63) / 64;
+  const int n = (int)(blockIdx.x / blocks_p), p0 = (int)(blockIdx.x % blocks_p) * 64;
+  const bool live = p0 + lane < P;
+  const float *image = a.in + (long)n * a.in_gs - 2;
+  const int *idx = a.in_index_lines + p0 + lane; // + k * P
+  float amax = 0.0f, vmax = -INFINITY;
+  for (int k0 = wave; k0 < a.K; k0 += 128) { // eight loads in flight
+    int j[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int k = k0 + 16 * u;
+      j[u] = (live && k < a.K) ? idx[(long)k * P] : -1;
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      if (j[u] >= 0) {
+        const float x = (j[u] <= 1) ? (float)j[u] : image[j[u]];
+        amax = fmaxf(amax, fabsf(x));
+        vmax = fmaxf(vmax, x);
+      }
+    }
+  }
+  sh_max[0][wave][lane] = amax;
+  sh_max[1][wave][lane] = vmax;
+  __syncthreads();
+  if (wave != 0 || !live) return;
+#pragma unroll
+  for (int w = 1; w < 16; ++w) {
+    amax = fmaxf(amax, sh_max[0][w][lane]);
+    vmax = fmaxf(vmax, sh_max[1][w][lane]);
+  }
+  float nm;
+  if (io.noise_management == RPU_NM_MAX) nm = io.nm_thres > 0.0f ? fminf(vmax, io.nm_thres) : vmax;
+  else nm = io.nm_thres > 0.0f ? fminf(amax, io.nm_thres) : amax;
+  a.st.nm[n * P + p0 + lane] = nm;
+}
+
+// Second kernel: a workgroup quantizes a block of 64 patches x 64 elements with each patch's input scale and stores it
+// through LDS with lanes along a row; the workgroups of the first 64 elements also set up the per-sample state.
+__global__ __launch_bounds__(256) void k_mvm_init_gather(MvmArgs a) {
+  __shared__ float tile[64][65];
+  const IoDev &io = a.io;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int P = a.in_group;
+  const int blocks_p = (P + 63) / 64, blocks_k = a.k_pad / 64 + ((a.k_pad & 63) ? 1 : 0);
+  const int k0 = (int)(blockIdx.x % blocks_k) * 64;
+  const int pb = (int)(blockIdx.x / blocks_k);
+  const int n = pb / blocks_p, p0 = (pb % blocks_p) * 64;
+  const bool live = p0 + lane < P;
+  const int b = n * P + p0 + lane;
+  const float *image = a.in + (long)n * a.in_gs - 2;
+  const int *idx = a.in_index_lines + p0 + lane; // + k * P
+  int j[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int k = k0 + wave * 16 + i;
+    j[i] = (live && k < a.K) ? idx[(long)k * P] : -1;
+  }
+  float scale = 1.0f;
+  if (!io.perfect) {
+    float nm = 1.0f;
+    if (io.noise_management == RPU_NM_ABS_MAX || io.noise_management == RPU_NM_MAX) nm = live ? a.st.nm[b] : 1.0f;
+    else if (io.noise_management == RPU_NM_CONSTANT) nm = io.nm_thres > 0.0f ? io.nm_thres : 1.0f;
+    float fin;
+    scale = round_scales(a, nm, 1.0f, fin);
+    if (k0 == 0 && wave == 0 && live) {
+      a.st.nm[b] = nm;
+      a.st.red[b] = 1.0f;
+      a.st.hit_up[b] = 0;
+      a.st.hit_lo[b] = 0;
+      a.st.scale[b] = scale;
+      a.st.fin[b] = fin;
+      a.st.rounds[b] = (fin == 0.0f) ? 0 : 1;
+      if (io.bound_management != RPU_BM_NONE) a.st.next_scale[0][b] = next_round_scale(a, 0, b, fin, nm, 1.0f);
+    }
+    const long gid = blockIdx.x * 256L + threadIdx.x, gstride = gridDim.x * 256L;
+    if (gid < MVM_COUNT_WORDS) a.st.count[gid] = 0;
+    const long n_done = 32L * ((a.m_batch + TILE - 1) / TILE);
+    for (long i = gid; i < n_done; i += gstride) a.st.tile_done[i] = 0;
+  }
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int k = k0 + wave * 16 + i;
+    float v = 0.0f;
+    if (j[i] >= 0) {
+      v = (j[i] <= 1) ? (float)j[i] : image[j[i]];
+      if (!io.perfect) v = dac_value(v, scale, io, a.key, a.call, 0, b, k);
+    }
+    tile[lane][wave * 16 + i] = v;
+  }
+  __syncthreads();
+  float *rows = a.xq[0] + ((long)n * P + p0) * a.k_pad + k0;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int row = i * 4 + wave;
+    if (p0 + row < P && k0 + lane < a.k_pad) rows[(long)row * a.k_pad + lane] = tile[row][lane];
+  }
+}
+
 // At the start of round `round`, the workgroups of a sample tile (one per output tile) each quantize a
 // 1 / tiles_o share of the tile's input rows with the input range the *next* round would use (next_scale),
 // into the other scratch matrix at the rows of this round's list positions.  Whether a sample needs that
@@ -840,12 +979,10 @@ __device__ __forceinline__ void mvm_prepare_next_rows(const MvmArgs &a, int roun
   const int kq = threadIdx.x & 31, rq = threadIdx.x >> 5;
   float sc[4];
   int bt[4];
-  long ro[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     bt[i] = sh_next_b[4 * rq + i];
     sc[i] = sh_next_scale[4 * rq + i];
-    ro[i] = mvm_in_row(a, bt[i]);
   }
   for (int k0 = k_lo; k0 < k_hi; k0 += 128) {
     float xv[4][4];
@@ -854,7 +991,7 @@ __device__ __forceinline__ void mvm_prepare_next_rows(const MvmArgs &a, int roun
       const int k = k0 + 32 * u + kq;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        xv[u][i] = (k < k_hi && sc[i] != 0.0f && k < a.K) ? in[ro[i] + (long)k * a.in_sk] : 0.0f;
+        xv[u][i] = (k < k_hi && sc[i] != 0.0f && k < a.K) ? in[(long)bt[i] * a.in_sb + (long)k * a.in_sk] : 0.0f;
       }
     }
 #pragma unroll
@@ -1006,7 +1143,7 @@ __device__ __forceinline__ void mvm_dual_select(const MvmArgs &a, int n) {
     const int b = tile_b * TILE + (idx >> 5), o = tile_o * TILE + (idx & 31);
     if (b < a.m_batch && o < a.O) {
       const int sel = a.dual.sel[b];
-      if (sel < 2) a.out[mvm_out_row(a, b) + (long)o * a.out_so] = pick2(a.dual.buf, sel)[(long)b * a.O + o];
+      if (sel < 2) a.out[(long)b * a.out_sb + (long)o * a.out_so] = pick2(a.dual.buf, sel)[(long)b * a.O + o];
     }
   }
 }
@@ -1309,7 +1446,7 @@ __device__ __forceinline__ void big_prepare_next_rows(const MvmArgs &a, int roun
 #pragma unroll
     for (int i = 0; i < RPT; ++i) {
       const int row = rq * RPT + i;
-      xv[i] = (sh_scale[row] != 0.0f && k < a.K) ? in[mvm_in_row(a, sh_b[row]) + (long)k * a.in_sk] : 0.0f;
+      xv[i] = (sh_scale[row] != 0.0f && k < a.K) ? in[(long)sh_b[row] * a.in_sb + (long)k * a.in_sk] : 0.0f;
     }
 #pragma unroll
     for (int i = 0; i < RPT; ++i) {
@@ -2072,6 +2209,14 @@ static int weight_mode(const MvmArgs &a) {
 // A small batch gets a workgroup per sample (most workgroups in flight, shortest latency); a large one gets as
 // many threads per sample as its rows can keep busy.
 void launch_mvm_init(const MvmArgs &a, hipStream_t s) {
+  if (a.in_index_lines) { // gathered input; the caller has checked that the noise management is one of these kernels'
+    const long blocks = (long)(a.m_batch / a.in_group) * ((a.in_group + 63) / 64);
+    if (!a.io.perfect && (a.io.noise_management == RPU_NM_ABS_MAX || a.io.noise_management == RPU_NM_MAX)) {
+      hipLaunchKernelGGL(k_mvm_gather_max, dim3((unsigned)blocks), dim3(1024), 0, s, a);
+    }
+    hipLaunchKernelGGL(k_mvm_init_gather, dim3((unsigned)(blocks * ((a.k_pad + 63) / 64))), dim3(256), 0, s, a);
+    return;
+  }
   if (a.m_batch <= 1024 || a.K > 512) {
     hipLaunchKernelGGL(k_mvm_init<256>, dim3(a.m_batch), dim3(256), 0, s, a);
   } else if (a.K > 64) {

@@ -509,10 +509,11 @@ struct Tile {
     // rows for the next bound-management round are quantized ahead when the batch is small (shortest path between
     // rounds) or when at least four workgroups per sample tile share that work; a large batch on a narrow tile
     // quantizes only the rows of the samples that saturated
-    a.speculate = (B <= 1024 || O > 96) ? 1 : 0;
+    a.speculate = mvm_speculates(B, O) ? 1 : 0;
     a.rows_ahead_in_init = a.speculate;
     return a;
   }
+  static bool mvm_speculates(int B, int O) { return B <= 1024 || O > 96; }
 
   // whether a pass with these IO parameters has non-idealities that add to the sums before the ADC
   static bool has_pre_adc_terms(const IOPar &io) {
@@ -671,8 +672,8 @@ struct Tile {
   // in_images / out_images > 0: that side is an image tensor [image][line][patch] with so many patches per image and
   // sample b = patch b % patches of image b / patches (no bias column then)
   void mvm(const float *in, float *out, int B, bool bias, bool in_trans, bool out_trans, bool transposed, hipStream_t s,
-           const float *w_other = nullptr, const IOPar *io_other = nullptr, bool is_test = false, int in_images = 0,
-           int out_images = 0, long in_ld = 0) {
+           const float *w_other = nullptr, const IOPar *io_other = nullptr, bool is_test = false, long in_ld = 0,
+           const int *in_index = nullptr, const int *in_index_lines = nullptr, int in_patches = 0, long image_size = 0) {
     const IOPar &io = io_other ? *io_other : (transposed ? bio : fio);
     const bool side = has_pre_adc_terms(io);
     MvmArgs a = mvm_args(B, transposed, w_other ? w_other : mvm_weights(is_test), io, side ? 0 : -1);
@@ -699,16 +700,20 @@ struct Tile {
       }
     }
 
-    if ((in_images || out_images) && bias) throw RpuError("Image layouts carry no bias column.");
     if (in_ld) { // padded rows of a plain row-major input
-      if (in_trans || bias || in_images) throw RpuError("A row stride goes with a plain row-major input only.");
+      if (in_trans || bias || in_index) throw RpuError("A row stride goes with a plain row-major input only.");
       a.in_sb = in_ld;
     }
-    if (in_images) {
-      a.in_sb = 1; a.in_sk = in_images; a.in_group = in_images; a.in_gs = (long)(a.K - 1) * in_images;
-    }
-    if (out_images) {
-      a.out_sb = 1; a.out_so = out_images; a.out_group = out_images; a.out_gs = (long)(a.O - 1) * out_images;
+    if (in_index) { // the samples are patches gathered from the images `in` (see MvmArgs::in_index)
+      if (in_trans || bias || transposed || side || in_patches <= 0) throw RpuError("Gathered input: plain forward calls only.");
+      if (a.speculate && a.max_rounds > 1) throw RpuError("Gathered input: not with rows quantized ahead.");
+      const int nm = io.p.noise_management;
+      if (!io.perfect && ((nm != RPU_NM_NONE && nm != RPU_NM_CONSTANT && nm != RPU_NM_ABS_MAX && nm != RPU_NM_MAX) ||
+                          io.p.bound_management == RPU_BM_ITERATIVE_WORST_CASE)) {
+        throw RpuError("Gathered input: not with this noise or bound management.");
+      }
+      a.in_index = in_index; a.in_index_lines = in_index_lines; a.in_group = in_patches; a.in_gs = image_size;
+      a.in_sb = 0; a.in_sk = 0;
     }
 
     prof_begin(s);
@@ -1389,16 +1394,19 @@ struct Tile {
     RPU_HIP_CHECK(hipMemcpy(x_idx_t.p, tr.data(), tr.size() * sizeof(int32_t), hipMemcpyHostToDevice));
   }
 
+  void ensure_line_major_index() {
+    if (x_idx.p) return;
+    x_idx.ensure(idx_host.size());
+    RPU_HIP_CHECK(hipMemcpy(x_idx.p, idx_host.data(), idx_host.size() * sizeof(int32_t), hipMemcpyHostToDevice));
+  }
+
   // rows of the patch matrix start on 128-byte lines: a workgroup's stores then fill whole lines
   int x_mat_ld() const { return (X + 31) & ~31; }
 
   void ensure_indexed(int n_images, bool with_d_mat = true) {
     if (idx_patches <= 0) throw RpuError("The index matrix has not been set (set_matrix_indices).");
     if (n_images <= 0) throw RpuError("n_images must be positive.");
-    if (!x_idx.p) {
-      x_idx.ensure(idx_host.size());
-      RPU_HIP_CHECK(hipMemcpy(x_idx.p, idx_host.data(), idx_host.size() * sizeof(int32_t), hipMemcpyHostToDevice));
-    }
+    ensure_line_major_index();
     const size_t B = (size_t)n_images * idx_patches;
     x_mat.ensure(B * (size_t)x_mat_ld());
     if (with_d_mat) d_mat.ensure(B * D);
@@ -1430,21 +1438,44 @@ struct Tile {
         return;
       }
     }
-    ensure_indexed(n_images, false);
     const int B = n_images * idx_patches;
+    {
+      // a call that reads its input row by row only (one round, or the rows of a further round written once it is
+      // known who goes on) gathers the patches in the init kernel: the patch matrix is never written
+      MvmArgs probe{};
+      probe.io = io_dev(fio);
+      const bool one_round = fio.perfect || mvm_max_rounds(probe.io) <= 1;
+      const int nm = fio.p.noise_management;
+      const bool nm_ok = fio.perfect || ((nm == RPU_NM_NONE || nm == RPU_NM_CONSTANT || nm == RPU_NM_ABS_MAX || nm == RPU_NM_MAX) &&
+                                         fio.p.bound_management != RPU_BM_ITERATIVE_WORST_CASE);
+      if ((one_round || !mvm_speculates(B, D)) && !has_pre_adc_terms(fio) && nm_ok) {
+        ensure_patch_major_index();
+        ensure_line_major_index();
+        d_mat.ensure((size_t)B * D);
+        mvm(x, d_mat.p, B, false, false, true, false, s, nullptr, nullptr, is_test, 0, x_idx_t.p, x_idx.p, idx_patches,
+            image_size);
+        launch_lines_to_images(d, d_mat.p, n_images, D, idx_patches, s);
+        RPU_HIP_CHECK(hipGetLastError());
+        return;
+      }
+    }
+    ensure_indexed(n_images);
     launch_gather_indexed(x_mat.p, x, x_idx.p, X, x_mat_ld(), idx_patches, n_images, image_size, s);
-    // the outputs go straight into the caller's [image][output][patch] tensor
-    mvm(x_mat.p, d, B, false, false, false, false, s, nullptr, nullptr, is_test, 0, idx_patches, x_mat_ld());
+    // the outputs come out line-major, [D][N P] (stores of a wave, one sample per lane, are unit stride), and move to
+    // the caller's [image][output][patch] tensor in runs of a patch row
+    mvm(x_mat.p, d_mat.p, B, false, false, true, false, s, nullptr, nullptr, is_test, x_mat_ld());
+    launch_lines_to_images(d, d_mat.p, n_images, D, idx_patches, s);
     RPU_HIP_CHECK(hipGetLastError());
   }
 
   void backward_indexed(const float *d, float *x, int n_images, long image_size, hipStream_t s) {
-    ensure_indexed(n_images, false);
+    ensure_indexed(n_images);
     const int B = n_images * idx_patches;
-    // the caller's [image][output][patch] tensor is read in place; the patch matrix comes out line-major, [X][B]:
-    // stores of a wave (one sample per lane) and the reads of the fold (neighbouring image elements meet neighbouring
-    // patches) are then unit stride
-    mvm(d, x_mat.p, B, false, false, true, true, s, nullptr, nullptr, false, idx_patches, 0);
+    // the caller's [image][output][patch] tensor moves to line-major [D][N P] in runs of a patch row and is read
+    // transposed; the patch matrix comes out line-major too, [X][N P]: stores of a wave (one sample per lane) and the
+    // reads of the fold (neighbouring image elements meet neighbouring patches) are then unit stride
+    launch_images_to_lines(d_mat.p, d, n_images, D, idx_patches, s);
+    mvm(d_mat.p, x_mat.p, B, false, true, true, true, s);
     if (fold_image_size != image_size) {
       // per image element, the entries of the patch matrix that were gathered from it, in the order in which the
       // reference's loop adds them up (k, then p)

@@ -218,13 +218,16 @@ def test_indexed_backward_adds_overlapping_patches_in_a_fixed_order(gpu_device):
     assert torch.equal(got.double(), want)
 
 
-@pytest.mark.parametrize("c_out", [40, 136])      # outputs below and above the width from which forward takes large tiles
-def test_wide_convolution_on_many_patches_equals_the_pass_over_the_unfolded_images(gpu_device, c_out):
-    """2048 patches of 145 elements: the contraction kernels (the large-tile one for the backward pass, and for the
-    forward pass of the wider tile) read the gradient tensor [image][output][patch] and write the output tensor in place;
-    same bits as the pass over the patch matrix that torch unfolds, and the fold of that pass's input gradients."""
+@pytest.mark.parametrize("c_in,side,n,c_out", [
+    (16, 16, 8, 40),      # 2048 patches of 145 elements: patches gathered by the init kernels, 32 x 32 tiles
+    (16, 16, 8, 136),     # rows quantized ahead: the patch matrix is written; large tiles in both directions
+    (3, 64, 5, 40),       # 20480 patches of 28 elements: gathered patches and large tiles with idle outputs
+])
+def test_wide_convolution_on_many_patches_equals_the_pass_over_the_unfolded_images(gpu_device, c_in, side, n, c_out):
+    """Forward and backward of convolutions too wide for the fused kernel: same bits as the pass over the patch matrix
+    that torch unfolds (the samples that saturate the ADC go through further rounds either way), and the fold of that
+    pass's input gradients."""
     rng = np.random.default_rng(12)
-    c_in, side, n = 16, 16, 8
     indices, patches = conv_indices((c_in, side, side), (3, 3), (1, 1), (1, 1), (1, 1), True)
     x_size = c_in * 9 + 1
     f_io = noise_free_io(inp_res=1 / 128.0, out_res=1 / 512.0, out_bound=2.0, noise_management=dv.NoiseManagementType.AbsMax,
