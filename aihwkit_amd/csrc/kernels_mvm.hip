@@ -2391,6 +2391,9 @@ void launch_mvm_dual(const MvmArgs &a_in, hipStream_t s) {
 void launch_mvm_round(const MvmArgs &a_in, hipStream_t s) {
   MvmArgs a = a_in;
   a.big_from = a.small_tiles_only ? 0 : big_threshold(a.m_batch, a.O);
+  // calls that quantize nothing ahead expect few samples in a further round: the 32 x 32 kernels take them all, and
+  // the round is one launch
+  if (a.round > 0 && !a.speculate) a.big_from = 0;
   if (a.big_from > 0) {
     const int bb = mvm_big_sample_tile(big_workgroups(a, 128), current_device_cus());
     const dim3 big_grid(big_workgroups(a, bb));
