@@ -1237,7 +1237,7 @@ int grid_for(long total) {
 
 void launch_update_prepare(const UpdateArgs &a, hipStream_t s) {
   const int longest = a.x_size > a.d_size ? a.x_size : a.d_size;
-  if (longest > 256 || a.m_batch <= 1024) {
+  if (longest > 1024 || a.m_batch <= 1024) {
     hipLaunchKernelGGL(k_update_prepare<256>, dim3(a.m_batch), dim3(256), 0, s, a);
   } else if (longest > 64) {
     hipLaunchKernelGGL(k_update_prepare<64>, dim3((a.m_batch + 3) / 4), dim3(256), 0, s, a);
