@@ -93,9 +93,10 @@ def main() -> int:
     ap.add_argument("--batch-sweep", action="store_true",
                     help="instead of the benchmark line: forward and backward call times of the configuration-2 tile "
                          "at batches 32 .. 2000 (HIP events over 200 calls each), one JSON line")
-    ap.add_argument("--config", type=int, default=2, choices=(1, 2, 3, 4, 5),
+    ap.add_argument("--config", type=int, default=2, choices=(1, 2, 3, 4, 5, 6),
                     help="benchmark configuration: 2 is the graded one; 3 is the Tiki-Taka MLP of transfer tiles; "
-                         "5 is the forward pass of the GPT-2-small linear layers as PCM inference tiles")
+                         "5 is the forward pass of the GPT-2-small linear layers as PCM inference tiles; 6 "
+                         "(supplementary) is one wide convolution layer through the indexed interface")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; an analog tile is an independent unit and the path "
@@ -123,6 +124,8 @@ def main() -> int:
         return bench_config4(args)
     if args.config == 5:
         return bench_config5(args)
+    if args.config == 6:
+        return bench_config6(args)
 
     if args.config == 2:
         x_size, d_size, batch = 1024, 1024, 256
@@ -730,6 +733,78 @@ def bench_config4(args) -> int:
                    "batch": batch},
         "useful_tflops": flops / (ms_per_step * 1e-3) / 1e12,
         "cpu_baseline": cpu,
+    }
+    print(json.dumps(out))
+    return 0
+
+
+def bench_config6(args) -> int:
+    """Supplementary configuration 6: one 3 x 3 convolution 48 -> 48 on 128 images of 34 x 34 (1024 patches per image,
+    131072 in all) as an analog training tile of 433 x 48 (SoftBounds, IO of configuration 2) through the indexed
+    interface: too wide for the fused convolution kernel, so the patches are gathered by the init kernels and the
+    contraction runs on the large-tile kernel.  A step = forward + backward + update of the 128 images; the calls are
+    also timed one by one, with their kernels (HIP events on the tile's stream)."""
+    import numpy as np
+    import torch
+
+    from aihwkit_amd.benchmark_configs import config2, conv_index_matrix
+    from aihwkit_amd.rpu_base import tiles
+
+    torch.cuda.set_device(0)
+    c_in, c_out, side, n = 48, 48, 34, 128
+    rng = np.random.default_rng(0)
+    indices, patches = conv_index_matrix((c_in, side, side), (3, 3))
+    out_side = side - 2
+    x_size = c_in * 9 + 1
+    meta, dev = config2(noise=True)
+    host = meta.create_array(x_size, c_out, dev)
+    host.set_weights(torch.from_numpy(rng.uniform(-0.1, 0.1, (c_out, x_size)).astype(np.float32)))
+    tile = tiles.CudaAnalogTile(host)
+    tile.set_learning_rate(0.01)
+    tile.set_matrix_indices(indices)
+    x = torch.from_numpy(rng.uniform(0, 1, (n, c_in, side, side)).astype(np.float32)).cuda()
+    g = torch.from_numpy(rng.normal(0, 0.01, (n, c_out, out_side, out_side)).astype(np.float32)).cuda()
+    y = torch.empty(n, c_out, out_side, out_side, device="cuda")
+    dx = torch.empty_like(x)
+    calls = (("forward", lambda: tile.forward_indexed(x, y)), ("backward", lambda: tile.backward_indexed(g, dx)),
+             ("update", lambda: tile.update_indexed(x, g)))
+
+    def step():
+        for _name, fn in calls:
+            fn()
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    per_call = {}
+    for name, fn in calls:
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            fn()
+        torch.cuda.synchronize()
+        tile.set_profiling(True)
+        fn()
+        kernels = [(k, round(ms, 5)) for k, ms in tile.get_profile()]
+        tile.set_profiling(False)
+        per_call[name] = {"ms_per_call": (time.perf_counter() - t0) * 1e3 / (args.steps + 1), "kernels_ms": kernels}
+    flops = 2.0 * n * patches * x_size * c_out
+    out = {
+        "metric": "patches/s through forward + backward + update of one wide convolution tile, 1 MI355X (supplementary)",
+        "value": n * patches / (ms_per_step * 1e-3), "unit": "patches/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "config6 (supplementary): conv 48->48 3x3 on 128 images 34 x 34 = 131072 patches, tile "
+                               "433 x 48 SoftBounds (dtod + ctoc), BL 31, UM+UBLM, 7/9-bit IO, iterative BM, indexed "
+                               "interface", "patches": n * patches},
+        "calls": per_call,
+        "forward_useful_tflops": flops / (per_call["forward"]["ms_per_call"] * 1e-3) / 1e12,
+        "cpu_baseline": None,
     }
     print(json.dumps(out))
     return 0
