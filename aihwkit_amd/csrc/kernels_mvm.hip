@@ -829,49 +829,69 @@ __global__ __launch_bounds__(256) void k_mvm_init(MvmArgs a) {
 // and element) as mvm_init_sample on the materialized patch matrix.  For noise management none / constant / abs-max /
 // max; the other kinds run mvm_init_sample, which gathers row by row.
 //
-// First kernel (abs-max / max only): a workgroup of 16 waves owns 64 patches of one image, one per lane; wave w takes
-// the elements k = w (mod 16), so a patch's largest input is a running maximum of its lane and the waves meet in LDS.
-// The noise-management value goes to st.nm.
+// First kernel (abs-max / max only): a workgroup of 16 waves owns 64 patches, one per lane, of four images; wave w
+// takes the elements k = w (mod 16), so a patch's largest input is a running maximum of its lane and the waves meet in
+// LDS.  The noise-management value goes to st.nm.
 __global__ __launch_bounds__(1024) void k_mvm_gather_max(MvmArgs a) {
-  __shared__ float sh_max[2][16][64];
+  constexpr int NI = 4; // images per workgroup: an index entry is read once for the four
+  __shared__ float sh_max[2][NI][16][64];
   const IoDev &io = a.io;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int P = a.in_group;
   const int blocks_p = (P + 63) / 64;
-  const int n = (int)(blockIdx.x / blocks_p), p0 = (int)(blockIdx.x % blocks_p) * 64;
+  const int n_images = a.m_batch / P;
+  const int n0 = (int)(blockIdx.x / blocks_p) * NI, p0 = (int)(blockIdx.x % blocks_p) * 64;
   const bool live = p0 + lane < P;
-  const float *image = a.in + (long)n * a.in_gs - 2;
+  const int images = min(NI, n_images - n0);
+  const float *image = a.in + (long)n0 * a.in_gs - 2;
   const int *idx = a.in_index_lines + p0 + lane; // + k * P
-  float amax = 0.0f, vmax = -INFINITY;
-  for (int k0 = wave; k0 < a.K; k0 += 128) { // eight loads in flight
-    int j[8];
+  float amax[NI], vmax[NI];
 #pragma unroll
-    for (int u = 0; u < 8; ++u) {
+  for (int i = 0; i < NI; ++i) {
+    amax[i] = 0.0f;
+    vmax[i] = -INFINITY;
+  }
+  for (int k0 = wave; k0 < a.K; k0 += 64) { // sixteen loads in flight
+    int j[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
       const int k = k0 + 16 * u;
       j[u] = (live && k < a.K) ? idx[(long)k * P] : -1;
     }
+    float x[4][NI];
 #pragma unroll
-    for (int u = 0; u < 8; ++u) {
+    for (int u = 0; u < 4; ++u) {
+#pragma unroll
+      for (int i = 0; i < NI; ++i) x[u][i] = (j[u] > 1 && i < images) ? image[j[u] + (long)i * a.in_gs] : (float)j[u];
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
       if (j[u] >= 0) {
-        const float x = (j[u] <= 1) ? (float)j[u] : image[j[u]];
-        amax = fmaxf(amax, fabsf(x));
-        vmax = fmaxf(vmax, x);
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+          amax[i] = fmaxf(amax[i], fabsf(x[u][i]));
+          vmax[i] = fmaxf(vmax[i], x[u][i]);
+        }
       }
     }
   }
-  sh_max[0][wave][lane] = amax;
-  sh_max[1][wave][lane] = vmax;
-  __syncthreads();
-  if (wave != 0 || !live) return;
 #pragma unroll
-  for (int w = 1; w < 16; ++w) {
-    amax = fmaxf(amax, sh_max[0][w][lane]);
-    vmax = fmaxf(vmax, sh_max[1][w][lane]);
+  for (int i = 0; i < NI; ++i) {
+    sh_max[0][i][wave][lane] = amax[i];
+    sh_max[1][i][wave][lane] = vmax[i];
+  }
+  __syncthreads();
+  if (wave >= images || !live) return; // wave i finishes image n0 + i
+  float am = 0.0f, vm = -INFINITY;
+#pragma unroll
+  for (int w = 0; w < 16; ++w) {
+    am = fmaxf(am, sh_max[0][wave][w][lane]);
+    vm = fmaxf(vm, sh_max[1][wave][w][lane]);
   }
   float nm;
-  if (io.noise_management == RPU_NM_MAX) nm = io.nm_thres > 0.0f ? fminf(vmax, io.nm_thres) : vmax;
-  else nm = io.nm_thres > 0.0f ? fminf(amax, io.nm_thres) : amax;
-  a.st.nm[n * P + p0 + lane] = nm;
+  if (io.noise_management == RPU_NM_MAX) nm = io.nm_thres > 0.0f ? fminf(vm, io.nm_thres) : vm;
+  else nm = io.nm_thres > 0.0f ? fminf(am, io.nm_thres) : am;
+  a.st.nm[(n0 + wave) * P + p0 + lane] = nm;
 }
 
 // Second kernel: a workgroup quantizes a block of 64 patches x 64 elements with each patch's input scale and stores it
@@ -2212,7 +2232,8 @@ void launch_mvm_init(const MvmArgs &a, hipStream_t s) {
   if (a.in_index_lines) { // gathered input; the caller has checked that the noise management is one of these kernels'
     const long blocks = (long)(a.m_batch / a.in_group) * ((a.in_group + 63) / 64);
     if (!a.io.perfect && (a.io.noise_management == RPU_NM_ABS_MAX || a.io.noise_management == RPU_NM_MAX)) {
-      hipLaunchKernelGGL(k_mvm_gather_max, dim3((unsigned)blocks), dim3(1024), 0, s, a);
+      const long max_blocks = (long)((a.m_batch / a.in_group + 3) / 4) * ((a.in_group + 63) / 64);
+      hipLaunchKernelGGL(k_mvm_gather_max, dim3((unsigned)max_blocks), dim3(1024), 0, s, a);
     }
     hipLaunchKernelGGL(k_mvm_init_gather, dim3((unsigned)(blocks * ((a.k_pad + 63) / 64))), dim3(256), 0, s, a);
     return;
