@@ -385,9 +385,8 @@ void launch_fold_indexed(float *images, const float *x_mat, const int *ptr, cons
 // [n][line][p] <-> [line][(n, p)]: what a contraction call reads or writes with its transposed layouts
 void launch_images_to_lines(float *lines_major, const float *images, int n_images, int lines, int patches, hipStream_t s);
 void launch_lines_to_images(float *images, const float *lines_major, int n_images, int lines, int patches, hipStream_t s);
-// [n][d][p] <-> [(n, p)][d]
+// [n][d][p] -> [(n, p)][d]
 void launch_ndp_to_bd(float *bd, const float *ndp, int n_images, int d_size, int patches, hipStream_t s);
-void launch_bd_to_ndp(float *ndp, const float *bd, int n_images, int d_size, int patches, hipStream_t s);
 void launch_fill(float *p, float value, size_t n, hipStream_t s);
 
 // n_vec unit vectors of length `size`: row v is e_((start + v) % size)

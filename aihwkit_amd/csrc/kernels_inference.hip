@@ -170,25 +170,16 @@ __global__ __launch_bounds__(256) void k_gather_indexed(float *x_mat, const floa
   }
 }
 
-// ndp index (n, d, p) <-> bd index ((n, p), d)
-__global__ __launch_bounds__(256) void k_ndp_bd(float *dst, const float *src, int n_images, int d_size, int patches,
-                                                 int to_bd) {
+// [image][line][patch] -> [(image, patch)][line]: the gradient rows of the samples of an indexed update
+__global__ __launch_bounds__(256) void k_ndp_bd(float *dst, const float *src, int n_images, int d_size, int patches) {
   const size_t total = (size_t)n_images * d_size * patches;
   for (size_t idx = blockIdx.x * (size_t)blockDim.x + threadIdx.x; idx < total; idx += (size_t)gridDim.x * blockDim.x) {
     // idx walks the destination with unit stride
-    if (to_bd) {
-      const int d = (int)(idx % d_size);
-      const size_t b = idx / d_size;
-      const int p = (int)(b % patches);
-      const size_t n = b / patches;
-      dst[idx] = src[(n * d_size + d) * patches + p];
-    } else {
-      const int p = (int)(idx % patches);
-      const size_t nd = idx / patches;
-      const int d = (int)(nd % d_size);
-      const size_t n = nd / d_size;
-      dst[idx] = src[(n * patches + p) * d_size + d];
-    }
+    const int d = (int)(idx % d_size);
+    const size_t b = idx / d_size;
+    const int p = (int)(b % patches);
+    const size_t n = b / patches;
+    dst[idx] = src[(n * d_size + d) * patches + p];
   }
 }
 
@@ -315,12 +306,7 @@ void launch_lines_to_images(float *images, const float *lines_major, int n_image
 
 void launch_ndp_to_bd(float *bd, const float *ndp, int n_images, int d_size, int patches, hipStream_t s) {
   const size_t total = (size_t)n_images * d_size * patches;
-  hipLaunchKernelGGL(k_ndp_bd, dim3(grid_of(total)), dim3(256), 0, s, bd, ndp, n_images, d_size, patches, 1);
-}
-
-void launch_bd_to_ndp(float *ndp, const float *bd, int n_images, int d_size, int patches, hipStream_t s) {
-  const size_t total = (size_t)n_images * d_size * patches;
-  hipLaunchKernelGGL(k_ndp_bd, dim3(grid_of(total)), dim3(256), 0, s, ndp, bd, n_images, d_size, patches, 0);
+  hipLaunchKernelGGL(k_ndp_bd, dim3(grid_of(total)), dim3(256), 0, s, bd, ndp, n_images, d_size, patches);
 }
 
 void launch_fill(float *p, float value, size_t n, hipStream_t s) {

@@ -1403,13 +1403,13 @@ struct Tile {
   // rows of the patch matrix start on 128-byte lines: a workgroup's stores then fill whole lines
   int x_mat_ld() const { return (X + 31) & ~31; }
 
-  void ensure_indexed(int n_images, bool with_d_mat = true) {
+  void ensure_indexed(int n_images) {
     if (idx_patches <= 0) throw RpuError("The index matrix has not been set (set_matrix_indices).");
     if (n_images <= 0) throw RpuError("n_images must be positive.");
     ensure_line_major_index();
     const size_t B = (size_t)n_images * idx_patches;
     x_mat.ensure(B * (size_t)x_mat_ld());
-    if (with_d_mat) d_mat.ensure(B * D);
+    d_mat.ensure(B * D);
   }
 
   void forward_indexed(const float *x, float *d, int n_images, long image_size, bool is_test, hipStream_t s) {

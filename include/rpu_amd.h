@@ -412,8 +412,9 @@ int rpu_tile_has_matrix_indices(const rpu_tile_t *tile); /* patches per image of
  * B/rpu_base_tiles.cpp:621-720 (always with trans = true, dim3 = images, m_batch = patches per image):
  * x_dev holds n_images input images of image_size floats (N, C, H, W), d_dev is [n_images][d_size][patches]
  * (N, C_out, H_out * W_out).  Forward gathers the patches through the index matrix and runs the tile's forward
- * pass over n_images * patches samples; backward runs the tile's backward pass and adds the patch gradients
- * into the (zeroed) images; update gathers the patches and runs the tile's update. */
+ * pass over n_images * patches samples; backward runs the tile's backward pass and adds the patch gradients up
+ * per image element (every element of x_dev is written, in a fixed order: nothing to zero, same bits on every
+ * call); update gathers the patches and runs the tile's update. */
 int rpu_tile_forward_indexed(rpu_tile_t *tile, const float *x_dev, float *d_dev, int n_images, long image_size,
                              int is_test, void *stream);
 int rpu_tile_backward_indexed(rpu_tile_t *tile, const float *d_dev, float *x_dev, int n_images, long image_size,
