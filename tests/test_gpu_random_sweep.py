@@ -494,11 +494,11 @@ def noise_check(z, desc):
         probs.append(("std", z.std()))
     if z.shape[1] > 1:
         c = np.corrcoef(z[:, :-1].ravel(), z[:, 1:].ravel())[0, 1]
-        if abs(c) > 4.5 / np.sqrt(n):
+        if abs(c) > 4.5 / np.sqrt(z[:, 1:].size):                   # 1 / sqrt(pairs) is the spread of the estimate
             probs.append(("corr_out", c))
     if z.shape[0] > 1:
         c = np.corrcoef(z[:-1].ravel(), z[1:].ravel())[0, 1]
-        if abs(c) > 4.5 / np.sqrt(n):
+        if abs(c) > 4.5 / np.sqrt(z[1:].size):
             probs.append(("corr_sample", c))
     # shared streams show up as repeated values
     r = np.round(z.ravel() * 2 ** 12).astype(np.int64)
