@@ -1503,10 +1503,14 @@ __device__ __forceinline__ void mvm_big_schedule() {
 }
 
 // work of workgroup number n of a large-tile round launch of one tile; BB: samples of a workgroup tile (128 or 64)
-template <int WT, int BB>
+// NARROW (tiles of at most 64 outputs, BB = 128): every wave takes outputs 0 .. 63 and one of the four 32-sample
+// blocks, instead of two waves on outputs that do not exist: half of the MFMAs, spread over all four SIMDs; the
+// k order of every sum is the same.
+template <int WT, int BB, bool NARROW = false>
 __device__ __forceinline__ void mvm_big_workgroup(const MvmArgs &a, const int round, const int n, const int min_active) {
   static_assert(BB == 128 || BB == 64, "sample tile of 128 or 64");
-  constexpr int NB = BB / 64; // 32-sample blocks per wave
+  static_assert(!NARROW || BB == 128, "the narrow wave layout covers four sample blocks");
+  constexpr int NB = NARROW ? 1 : BB / 64; // 32-sample blocks per wave
   constexpr int XJ = BB / 32; // staged sample rows per thread
   __shared__ __attribute__((aligned(16))) float lds_x[2][BB * BROW];
   __shared__ __attribute__((aligned(16))) float lds_w[2][WT ? BKS * BPITCH_T : BT * BROW];
@@ -1530,7 +1534,8 @@ __device__ __forceinline__ void mvm_big_workgroup(const MvmArgs &a, const int ro
   const int t = threadIdx.x;
   const int lane = t & 63, wave = t >> 6;
   const int r = lane & 31, h = lane >> 5;
-  const int wy = wave >> 1, wx = wave & 1;
+  const int wy = NARROW ? 0 : wave >> 1, wx = wave & 1;
+  const int blk = NARROW ? wave >> 1 : 0; // NARROW: this wave's sample block within its half
   const int K = a.K;
 
   // global -> LDS assignment.  k-contiguous operand: chunk c = t + 256 j covers row c / 8, floats 4 (c % 8) ..;
@@ -1623,7 +1628,7 @@ __device__ __forceinline__ void mvm_big_workgroup(const MvmArgs &a, const int ro
   int x_off[4], w_off[4];
 #pragma unroll
   for (int q = 0; q < 4; ++q) {
-    x_off[q] = big_lds_offset(wx * (BB / 2) + r, h * 4 + q);
+    x_off[q] = big_lds_offset(wx * (BB / 2) + blk * 32 + r, h * 4 + q);
     w_off[q] = big_lds_offset(wy * 64 + r, h * 4 + q);
   }
   auto read_operands = [&](int buf, int q, Operands &o) __attribute__((always_inline)) {
@@ -1720,7 +1725,7 @@ __device__ __forceinline__ void mvm_big_workgroup(const MvmArgs &a, const int ro
       if (lo_max) atomicMax(&sh_hits[BB + local_b], lo_max);
     }
   };
-  finish_block(0, acc00, acc10);
+  finish_block(blk, acc00, acc10);
   if (NB == 2) finish_block(1, acc01, acc11);
   if (!flags) return;
   __syncthreads();
@@ -1777,6 +1782,9 @@ __device__ __forceinline__ void mvm_big_workgroup(const MvmArgs &a, const int ro
 template <int WT, int BB>
 __global__ __launch_bounds__(256, 2) void k_mvm_big(MvmArgs a, int min_active) {
   mvm_big_workgroup<WT, BB>(a, a.round, (int)blockIdx.x, min_active);
+}
+__global__ __launch_bounds__(256, 2) void k_mvm_big_narrow(MvmArgs a, int min_active) {
+  mvm_big_workgroup<0, 128, true>(a, a.round, (int)blockIdx.x, min_active);
 }
 
 // several tiles in one launch (round 0): a tile that is not run by this kernel has no workgroups in the table
@@ -2416,10 +2424,13 @@ void launch_mvm_round(const MvmArgs &a_in, hipStream_t s) {
   // the round is one launch
   if (a.round > 0 && !a.speculate) a.big_from = 0;
   if (a.big_from > 0) {
-    const int bb = mvm_big_sample_tile(big_workgroups(a, 128), current_device_cus());
+    const bool narrow = !a.transposed && a.O <= 64; // see mvm_big_workgroup
+    const int bb = narrow ? 128 : mvm_big_sample_tile(big_workgroups(a, 128), current_device_cus());
     const dim3 big_grid(big_workgroups(a, bb));
     const int min_active = a.round > 0 ? a.big_from : 0;
-    if (bb == 128) {
+    if (narrow) {
+      hipLaunchKernelGGL(k_mvm_big_narrow, big_grid, dim3(256), 0, s, a, min_active);
+    } else if (bb == 128) {
       if (a.transposed) hipLaunchKernelGGL((k_mvm_big<1, 128>), big_grid, dim3(256), 0, s, a, min_active);
       else hipLaunchKernelGGL((k_mvm_big<0, 128>), big_grid, dim3(256), 0, s, a, min_active);
     } else {
