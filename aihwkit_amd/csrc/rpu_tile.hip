@@ -1394,6 +1394,13 @@ struct Tile {
     RPU_HIP_CHECK(hipMemcpy(x_idx_t.p, tr.data(), tr.size() * sizeof(int32_t), hipMemcpyHostToDevice));
   }
 
+  // samples of an indexed call: the kernels count them in 32 bits
+  int indexed_samples(int n_images) const {
+    const long B = (long)n_images * idx_patches;
+    if (B >= (1L << 31) || B * std::max(X, D) >= (1L << 40)) throw RpuError("Too many patches for one call: split the images.");
+    return (int)B;
+  }
+
   void ensure_line_major_index() {
     if (x_idx.p) return;
     x_idx.ensure(idx_host.size());
@@ -1406,6 +1413,7 @@ struct Tile {
   void ensure_indexed(int n_images) {
     if (idx_patches <= 0) throw RpuError("The index matrix has not been set (set_matrix_indices).");
     if (n_images <= 0) throw RpuError("n_images must be positive.");
+    (void)indexed_samples(n_images);
     ensure_line_major_index();
     const size_t B = (size_t)n_images * idx_patches;
     x_mat.ensure(B * (size_t)x_mat_ld());
@@ -1438,7 +1446,7 @@ struct Tile {
         return;
       }
     }
-    const int B = n_images * idx_patches;
+    const int B = indexed_samples(n_images);
     {
       // a call that reads its input row by row only (one round, or the rows of a further round written once it is
       // known who goes on) gathers the patches in the init kernel: the patch matrix is never written
@@ -1470,7 +1478,7 @@ struct Tile {
 
   void backward_indexed(const float *d, float *x, int n_images, long image_size, hipStream_t s) {
     ensure_indexed(n_images);
-    const int B = n_images * idx_patches;
+    const int B = indexed_samples(n_images);
     // the caller's [image][output][patch] tensor moves to line-major [D][N P] in runs of a patch row and is read
     // transposed; the patch matrix comes out line-major too, [X][N P]: stores of a wave (one sample per lane) and the
     // reads of the fold (neighbouring image elements meet neighbouring patches) are then unit stride
@@ -1509,7 +1517,7 @@ struct Tile {
 
   void update_indexed(const float *x, const float *d, int n_images, long image_size, hipStream_t s) {
     ensure_indexed(n_images);
-    const int B = n_images * idx_patches;
+    const int B = indexed_samples(n_images);
     launch_gather_indexed(x_mat.p, x, x_idx.p, X, X, idx_patches, n_images, image_size, s);
     launch_ndp_to_bd(d_mat.p, d, n_images, D, idx_patches, s);
     update(x_mat.p, d_mat.p, B, false, false, false, s);
