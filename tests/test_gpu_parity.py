@@ -144,9 +144,11 @@ def test_forward_backward_layouts(gpu_device, x_trans, d_trans, bias):
     assert np.array_equal(x_gpu, orc.backward(d, bias, d_trans, x_trans))
 
 
-def test_floating_point_tile(gpu_device):
+@pytest.mark.parametrize("x_size,d_size,batch", [(200, 150, 64),
+                                                 (100, 48, 20000),     # large tiles with idle outputs, both directions
+                                                 (60, 130, 4000)])
+def test_floating_point_tile(gpu_device, x_size, d_size, batch):
     rng = np.random.default_rng(3)
-    x_size, d_size, batch = 200, 150, 64
     host = dv.FloatingPointTileParameter().create_array(x_size, d_size)
     w = rng.standard_normal((d_size, x_size)).astype(np.float32)
     host.set_weights(torch.from_numpy(w))
@@ -160,7 +162,7 @@ def test_floating_point_tile(gpu_device):
     gpu.set_learning_rate(0.1)
     gpu.update(cuda(x), cuda(d), False)
     want = w.astype(np.float64) - 0.1 * d.T.astype(np.float64) @ x.astype(np.float64)
-    assert np.allclose(gpu.get_weights().numpy(), want, atol=1e-4)
+    assert np.allclose(gpu.get_weights().numpy(), want, atol=1e-4 * max(1.0, batch / 64.0))
 
 
 def _word_invariants(words, values, bl):
