@@ -1506,14 +1506,16 @@ __device__ __forceinline__ void mvm_big_schedule() {
 // NARROW (tiles of at most 64 outputs, BB = 128): every wave takes outputs 0 .. 63 and one of the four 32-sample
 // blocks, instead of two waves on outputs that do not exist: half of the MFMAs, spread over all four SIMDs; the
 // k order of every sum is the same.
-template <int WT, int BB, bool NARROW = false>
+// NBUF = 1 (contractions of one or two stages): a single staging buffer, half of the LDS, so that a third workgroup
+// fits a CU and covers the ADC stage of the other two, which is all such a call consists of.
+template <int WT, int BB, bool NARROW = false, int NBUF = 2>
 __device__ __forceinline__ void mvm_big_workgroup(const MvmArgs &a, const int round, const int n, const int min_active) {
   static_assert(BB == 128 || BB == 64, "sample tile of 128 or 64");
   static_assert(!NARROW || BB == 128, "the narrow wave layout covers four sample blocks");
   constexpr int NB = NARROW ? 1 : BB / 64; // 32-sample blocks per wave
   constexpr int XJ = BB / 32; // staged sample rows per thread
-  __shared__ __attribute__((aligned(16))) float lds_x[2][BB * BROW];
-  __shared__ __attribute__((aligned(16))) float lds_w[2][WT ? BKS * BPITCH_T : BT * BROW];
+  __shared__ __attribute__((aligned(16))) float lds_x[NBUF][BB * BROW];
+  __shared__ __attribute__((aligned(16))) float lds_w[NBUF][WT ? BKS * BPITCH_T : BT * BROW];
   __shared__ int sh_hits[2 * BB];
   __shared__ int sh_b[BB];
   __shared__ float sh_scale[BB];
@@ -1683,8 +1685,9 @@ __device__ __forceinline__ void mvm_big_workgroup(const MvmArgs &a, const int ro
     for (int s = 0; s < stages; ++s) {
       const bool next = s + 1 < stages;
       if (next) gload(s + 1, gx, gw);
-      compute(s & 1);
-      if (next) lds_store((s + 1) & 1, gx, gw);
+      compute(NBUF == 1 ? 0 : s & 1);
+      if (NBUF == 1 && next) __syncthreads(); // every wave is done with the one buffer
+      if (next) lds_store(NBUF == 1 ? 0 : (s + 1) & 1, gx, gw);
       __syncthreads();
     }
   }
@@ -1782,6 +1785,10 @@ __device__ __forceinline__ void mvm_big_workgroup(const MvmArgs &a, const int ro
 template <int WT, int BB>
 __global__ __launch_bounds__(256, 2) void k_mvm_big(MvmArgs a, int min_active) {
   mvm_big_workgroup<WT, BB>(a, a.round, (int)blockIdx.x, min_active);
+}
+template <int BB>
+__global__ __launch_bounds__(256, 3) void k_mvm_big_short(MvmArgs a, int min_active) {
+  mvm_big_workgroup<1, BB, false, 1>(a, a.round, (int)blockIdx.x, min_active);
 }
 __global__ __launch_bounds__(256, 2) void k_mvm_big_narrow(MvmArgs a, int min_active) {
   mvm_big_workgroup<0, 128, true>(a, a.round, (int)blockIdx.x, min_active);
@@ -2430,6 +2437,9 @@ void launch_mvm_round(const MvmArgs &a_in, hipStream_t s) {
     const int min_active = a.round > 0 ? a.big_from : 0;
     if (narrow) {
       hipLaunchKernelGGL(k_mvm_big_narrow, big_grid, dim3(256), 0, s, a, min_active);
+    } else if (a.transposed && a.k_pad <= 2 * BKS) { // see mvm_big_workgroup, NBUF
+      if (bb == 128) hipLaunchKernelGGL((k_mvm_big_short<128>), big_grid, dim3(256), 0, s, a, min_active);
+      else hipLaunchKernelGGL((k_mvm_big_short<64>), big_grid, dim3(256), 0, s, a, min_active);
     } else if (bb == 128) {
       if (a.transposed) hipLaunchKernelGGL((k_mvm_big<1, 128>), big_grid, dim3(256), 0, s, a, min_active);
       else hipLaunchKernelGGL((k_mvm_big<0, 128>), big_grid, dim3(256), 0, s, a, min_active);
