@@ -103,18 +103,7 @@ __device__ __forceinline__ MvmGatherRow mvm_gather_row(const MvmArgs &a, int b) 
 __device__ __forceinline__ void write_dac_row(const MvmArgs &a, int b, int slot, float scale, int round, float *dst,
                                               int t, int width) {
   float *out = dst + (long)slot * a.k_pad;
-  if (a.in_index) {
-    const MvmGatherRow row = mvm_gather_row(a, b);
-    for (int k = t; k < a.k_pad; k += width) {
-      float v = 0.0f;
-      if (k < a.K) {
-        v = row.at(k);
-        if (!a.io.perfect) v = dac_value(v, scale, a.io, a.key, a.call, round, b, k);
-      }
-      out[k] = v;
-    }
-    return;
-  }
+  if (a.in_sk == 0) return; // gathered input: the round that reads the rows writes them (mvm_gather_tile_rows)
   const float *row = a.in + (long)b * a.in_sb;
   for (int k = t; k < a.k_pad; k += width) {
     float v = 0.0f;
@@ -1256,6 +1245,27 @@ __device__ __forceinline__ bool runs_on_large_tiles(const MvmArgs &a, int round,
 // Rounds after the first usually list few samples, but their launch is sized before that is known.  When the
 // full grid would be large, this variant runs them instead: a fixed number of workgroups walk the tiles of the
 // listed samples, with one register set (k_pad only needs to be a multiple of 32).
+// Calls on gathered patches (MvmArgs::in_index) write no rows for the samples that go on to a further round
+// (write_dac_row has no patch matrix to read): the workgroup that is about to run sample tile tile_b of round `round`
+// gathers the quantized rows of that tile's listed samples itself, through the patch-major index and with the scale
+// that the round before has set.  The workgroups of the other output tiles of the same samples write the same values.
+__device__ __forceinline__ void mvm_gather_tile_rows(const MvmArgs &a, int round, int tile_b, int n_act) {
+  float *rows = pick2(a.xq, round & 1);
+  const int *list = pick2(a.st.list, round & 1);
+  const int first = tile_b * TILE, count = min(TILE, n_act - first);
+  for (int i = threadIdx.x >> 3; i < count; i += 32) { // eight threads per row
+    const int b = list[first + i];
+    const float scale = a.st.scale[b];
+    const MvmGatherRow row = mvm_gather_row(a, b);
+    float *out = rows + (long)(first + i) * a.k_pad;
+    for (int k = threadIdx.x & 7; k < a.k_pad; k += 8) {
+      out[k] = (k < a.K) ? dac_value(row.at(k), scale, a.io, a.key, a.call, round, b, k) : 0.0f;
+    }
+  }
+  __threadfence_block();
+  __syncthreads();
+}
+
 template <int WMODE>
 __global__ __launch_bounds__(256) void k_mvm_round_tail(MvmArgs a) {
   __shared__ float red[WAVES][16][64];
@@ -1269,6 +1279,10 @@ __global__ __launch_bounds__(256) void k_mvm_round_tail(MvmArgs a) {
   if (runs_on_large_tiles(a, a.round, n_act)) return;
   const int total = workgroups_for(a.O, n_act);
   for (int n = blockIdx.x; n < total; n += gridDim.x) {
+    if (a.in_index && a.round > 0) {
+      int tile_o, tile_b;
+      if (tile_of(a, n, n_act, tile_o, tile_b)) mvm_gather_tile_rows(a, a.round, tile_b, n_act);
+    }
     mvm_round_workgroup<1, WMODE>(a, a.round, n, n_act, red, stage);
     __syncthreads(); // LDS is reused by the next tile
   }
@@ -2451,7 +2465,7 @@ void launch_mvm_round(const MvmArgs &a_in, hipStream_t s) {
   }
   const int all = mvm_round_workgroups(a);
   const int mode = weight_mode(a);
-  if (a.round > 0 && all > TAIL_GRID) {
+  if (a.round > 0 && (all > TAIL_GRID || a.in_index)) { // gathered input: only this kernel writes the rows it reads
     const dim3 grid(TAIL_GRID);
     if (mode == 0) hipLaunchKernelGGL(k_mvm_round_tail<0>, grid, dim3(256), 0, s, a);
     else if (mode == 1) hipLaunchKernelGGL(k_mvm_round_tail<1>, grid, dim3(256), 0, s, a);
