@@ -218,21 +218,26 @@ def test_indexed_backward_adds_overlapping_patches_in_a_fixed_order(gpu_device):
     assert torch.equal(got.double(), want)
 
 
-@pytest.mark.parametrize("c_in,side,n,c_out,bm", [
-    (16, 16, 8, 40, True),     # 2048 patches of 145 elements: patches gathered by the init kernels, 32 x 32 tiles
-    (16, 16, 8, 136, True),    # rows quantized ahead: the patch matrix is written; large tiles in both directions
-    (16, 16, 8, 136, False),   # a single round: gathered patches on the wide tile too, large tiles in both directions
-    (3, 64, 5, 40, True),      # 20480 patches of 28 elements: gathered patches and large tiles with idle outputs
-    (8, 48, 8, 40, True),      # 18432 patches of 73 elements: the same with rows of two blocks of the gathering kernel
+@pytest.mark.parametrize("c_in,side,n,c_out,bm,nm", [
+    (16, 16, 8, 40, True, "AbsMax"),     # 2048 patches of 145 elements: patches gathered by the init kernels, 32 x 32 tiles
+    (16, 16, 8, 40, True, "Max"),        # ... with the other noise managements of the gathering kernels
+    (16, 16, 8, 40, True, "Constant"),
+    (16, 16, 8, 136, True, "AbsMax"),    # rows quantized ahead: the patch matrix is written; large tiles in both directions
+    (16, 16, 8, 136, False, "AbsMax"),   # a single round: gathered patches on the wide tile too, large tiles in both directions
+    (3, 64, 5, 40, True, "AbsMax"),      # 20480 patches of 28 elements: gathered patches and large tiles with idle outputs
+    (3, 64, 5, 40, True, "Max"),
+    (3, 64, 5, 40, True, "Constant"),
+    (8, 48, 8, 40, True, "AbsMax"),      # 18432 patches of 73 elements: the same with rows of two blocks of the gathering kernel
 ])
-def test_wide_convolution_on_many_patches_equals_the_pass_over_the_unfolded_images(gpu_device, c_in, side, n, c_out, bm):
+def test_wide_convolution_on_many_patches_equals_the_pass_over_the_unfolded_images(gpu_device, c_in, side, n, c_out, bm, nm):
     """Forward and backward of convolutions too wide for the fused kernel: same bits as the pass over the patch matrix
     that torch unfolds (the samples that saturate the ADC go through further rounds either way), and the fold of that
     pass's input gradients."""
     rng = np.random.default_rng(12)
     indices, patches = conv_indices((c_in, side, side), (3, 3), (1, 1), (1, 1), (1, 1), True)
     x_size = c_in * 9 + 1
-    f_io = noise_free_io(inp_res=1 / 128.0, out_res=1 / 512.0, out_bound=2.0, noise_management=dv.NoiseManagementType.AbsMax,
+    f_io = noise_free_io(inp_res=1 / 128.0, out_res=1 / 512.0, out_bound=2.0, noise_management=getattr(dv.NoiseManagementType, nm),
+                         nm_thres=3.0 if nm == "Constant" else 0.0,
                          bound_management=dv.BoundManagementType.Iterative if bm else dv.BoundManagementType.NONE)
     b_io = noise_free_io(inp_res=1 / 128.0, out_res=1 / 512.0, noise_management=dv.NoiseManagementType.AbsMax)
     dev = constant_step(dw_min=0.002, dw_min_std=0.0, construction_seed=4, w_max_dtod=0.0, w_min_dtod=0.0, w_max=1.0, w_min=-1.0)
