@@ -669,11 +669,19 @@ struct Tile {
     prof_mark(s, "pre_adc_terms");
   }
 
-  // in_images / out_images > 0: that side is an image tensor [image][line][patch] with so many patches per image and
-  // sample b = patch b % patches of image b / patches (no bias column then)
+  // Input of a forward call whose samples are the patches of images, read through the index matrix (MvmArgs::in_index):
+  // `in` then points to the images
+  struct GatherSource {
+    const int *index_patch_major; // [patches][X]
+    const int *index_line_major;  // [X][patches]
+    int patches;                  // per image
+    long image_size;
+  };
+
+  // in_ld: row stride of a plain row-major input with padded rows (0: the rows are dense)
   void mvm(const float *in, float *out, int B, bool bias, bool in_trans, bool out_trans, bool transposed, hipStream_t s,
            const float *w_other = nullptr, const IOPar *io_other = nullptr, bool is_test = false, long in_ld = 0,
-           const int *in_index = nullptr, const int *in_index_lines = nullptr, int in_patches = 0, long image_size = 0) {
+           const GatherSource *gather = nullptr) {
     const IOPar &io = io_other ? *io_other : (transposed ? bio : fio);
     const bool side = has_pre_adc_terms(io);
     MvmArgs a = mvm_args(B, transposed, w_other ? w_other : mvm_weights(is_test), io, side ? 0 : -1);
@@ -701,18 +709,19 @@ struct Tile {
     }
 
     if (in_ld) { // padded rows of a plain row-major input
-      if (in_trans || bias || in_index) throw RpuError("A row stride goes with a plain row-major input only.");
+      if (in_trans || bias || gather) throw RpuError("A row stride goes with a plain row-major input only.");
       a.in_sb = in_ld;
     }
-    if (in_index) { // the samples are patches gathered from the images `in` (see MvmArgs::in_index)
-      if (in_trans || bias || transposed || side || in_patches <= 0) throw RpuError("Gathered input: plain forward calls only.");
+    if (gather) { // the samples are patches gathered from the images `in` (see MvmArgs::in_index)
+      if (in_trans || bias || transposed || side || gather->patches <= 0) throw RpuError("Gathered input: plain forward calls only.");
       if (a.speculate && a.max_rounds > 1) throw RpuError("Gathered input: not with rows quantized ahead.");
       const int nm = io.p.noise_management;
       if (!io.perfect && ((nm != RPU_NM_NONE && nm != RPU_NM_CONSTANT && nm != RPU_NM_ABS_MAX && nm != RPU_NM_MAX) ||
                           io.p.bound_management == RPU_BM_ITERATIVE_WORST_CASE)) {
         throw RpuError("Gathered input: not with this noise or bound management.");
       }
-      a.in_index = in_index; a.in_index_lines = in_index_lines; a.in_group = in_patches; a.in_gs = image_size;
+      a.in_index = gather->index_patch_major; a.in_index_lines = gather->index_line_major; a.in_group = gather->patches;
+      a.in_gs = gather->image_size;
       a.in_sb = 0; a.in_sk = 0;
     }
 
@@ -1460,8 +1469,8 @@ struct Tile {
         ensure_patch_major_index();
         ensure_line_major_index();
         d_mat.ensure((size_t)B * D);
-        mvm(x, d_mat.p, B, false, false, true, false, s, nullptr, nullptr, is_test, 0, x_idx_t.p, x_idx.p, idx_patches,
-            image_size);
+        const GatherSource patches_of{x_idx_t.p, x_idx.p, idx_patches, image_size};
+        mvm(x, d_mat.p, B, false, false, true, false, s, nullptr, nullptr, is_test, 0, &patches_of);
         launch_lines_to_images(d, d_mat.p, n_images, D, idx_patches, s);
         RPU_HIP_CHECK(hipGetLastError());
         return;
