@@ -1522,7 +1522,9 @@ __device__ __forceinline__ void mvm_big_schedule() {
 // k order of every sum is the same.
 // NBUF = 1 (contractions of one or two stages): a single staging buffer, half of the LDS, so that a third workgroup
 // fits a CU and covers the ADC stage of the other two, which is all such a call consists of.
-template <int WT, int BB, bool NARROW = false, int NBUF = 2>
+// LAZY (calls with speculate = 0): nothing is quantized ahead; the last workgroup of a sample tile writes the rows of
+// the samples that go on.  The other instantiations always quantize ahead, as their callers ask for.
+template <int WT, int BB, bool NARROW = false, int NBUF = 2, bool LAZY = false>
 __device__ __forceinline__ void mvm_big_workgroup(const MvmArgs &a, const int round, const int n, const int min_active) {
   static_assert(BB == 128 || BB == 64, "sample tile of 128 or 64");
   static_assert(!NARROW || BB == 128, "the narrow wave layout covers four sample blocks");
@@ -1543,7 +1545,7 @@ __device__ __forceinline__ void mvm_big_workgroup(const MvmArgs &a, const int ro
   const int tile_b = ((n >> 3) / ((a.O + BT - 1) / BT)) * 8 + (n & 7);
   if (tile_b * BB >= n_act) return;
   const bool more_rounds = round + 1 < a.max_rounds;
-  if (more_rounds && a.speculate && !(round == 0 && a.rows_ahead_in_init)) {
+  if (more_rounds && !LAZY && !(round == 0 && a.rows_ahead_in_init)) {
     big_prepare_next_rows<BB>(a, round, tile_o, tile_b, n_act, sh_b, sh_scale);
   }
 
@@ -1767,7 +1769,7 @@ __device__ __forceinline__ void mvm_big_workgroup(const MvmArgs &a, const int ro
   }
   __syncthreads();
   if (!sh_last) return;
-  const bool ahead = a.speculate != 0;
+  constexpr bool ahead = !LAZY;
   if (!ahead) { // sh_last becomes the number of samples of this tile that go on
     __syncthreads();
     if (t == 0) sh_last = 0;
@@ -1805,7 +1807,11 @@ __global__ __launch_bounds__(256, 3) void k_mvm_big_short(MvmArgs a, int min_act
   mvm_big_workgroup<1, BB, false, 1>(a, a.round, (int)blockIdx.x, min_active);
 }
 __global__ __launch_bounds__(256, 2) void k_mvm_big_narrow(MvmArgs a, int min_active) {
-  mvm_big_workgroup<0, 128, true>(a, a.round, (int)blockIdx.x, min_active);
+  mvm_big_workgroup<0, 128, true, 2, true>(a, a.round, (int)blockIdx.x, min_active);
+}
+template <int BB>
+__global__ __launch_bounds__(256, 2) void k_mvm_big_lazy(MvmArgs a, int min_active) {
+  mvm_big_workgroup<0, BB, false, 2, true>(a, a.round, (int)blockIdx.x, min_active);
 }
 
 // several tiles in one launch (round 0): a tile that is not run by this kernel has no workgroups in the table
@@ -2451,6 +2457,9 @@ void launch_mvm_round(const MvmArgs &a_in, hipStream_t s) {
     const int min_active = a.round > 0 ? a.big_from : 0;
     if (narrow) {
       hipLaunchKernelGGL(k_mvm_big_narrow, big_grid, dim3(256), 0, s, a, min_active);
+    } else if (!a.transposed && !a.speculate && a.max_rounds > 1) {
+      if (bb == 128) hipLaunchKernelGGL((k_mvm_big_lazy<128>), big_grid, dim3(256), 0, s, a, min_active);
+      else hipLaunchKernelGGL((k_mvm_big_lazy<64>), big_grid, dim3(256), 0, s, a, min_active);
     } else if (a.transposed && a.k_pad <= 2 * BKS) { // see mvm_big_workgroup, NBUF
       if (bb == 128) hipLaunchKernelGGL((k_mvm_big_short<128>), big_grid, dim3(256), 0, s, a, min_active);
       else hipLaunchKernelGGL((k_mvm_big_short<64>), big_grid, dim3(256), 0, s, a, min_active);
