@@ -198,6 +198,8 @@ SYMBOLS = {
     "rpu_tile_get_update_words": (C.c_int, [_P, _P, _P, _P, C.c_int]),
     "rpu_tile_get_update_words_per_sample": (C.c_int, [_P, _P]),
     "rpu_tile_set_fused_rounds": (C.c_int, [_P, C.c_int]),
+    "rpu_tile_set_round_wait_test_hook": (C.c_int, [_P, C.c_int, C.c_int]),
+    "rpu_group_set_round_wait_test_hook": (C.c_int, [_P, C.c_int, C.c_int]),
     "rpu_tile_get_update_ab": (C.c_int, [_P, _P, _P, C.c_int]),
     "rpu_tile_update_with_words": (C.c_int, [_P, _P, _P, C.c_int, _P]),
     "rpu_tile_get_implicit_counts": (C.c_int, [_P, _P, C.c_int]),
@@ -207,6 +209,7 @@ SYMBOLS = {
     "rpu_tile_profile_name": (C.c_char_p, [_P, C.c_int]),
     "rpu_philox4x32_10": (C.c_int, [C.POINTER(C.c_uint32), C.POINTER(C.c_uint32), C.POINTER(C.c_uint32)]),
     "rpu_philox4x32_10_device": (C.c_int, [C.POINTER(C.c_uint32), C.POINTER(C.c_uint32), C.POINTER(C.c_uint32), C.c_int]),
+    "rpu_device_allocation_count": (C.c_long, []),
     "rpu_last_error": (C.c_char_p, []),
     "rpu_abi_version": (C.c_int, []),
 }

@@ -21,6 +21,7 @@ struct IoDev {
 constexpr int MVM_COUNT_WORDS = 256; // MvmState::count: [0, 40) per round; [MVM_ARRIVE_BASE + 4 r, + 4): counter and flag of the
                                      // arrivals after round r, counter and flag of the wait before round r
 constexpr int MVM_ARRIVE_BASE = 64;
+constexpr int MVM_ABORT_WORD = 255;  // MvmState::count[MVM_ABORT_WORD]: raised by a workgroup whose wait for the others ran out
 
 struct MvmState {
   float *nm;       // noise-management scale
@@ -47,7 +48,8 @@ struct DualDev {
   int *hit1;     // [2][m_batch] saturation marks of round 1: upper, lower (as MvmState::hit_up / hit_lo)
   float *xq2;    // quantized rows of round 2, written while round 0's rows are still read
   int *seen;     // host-visible: [0] samples of the last call that needed round 1, [1] its batch, [2] the last round
-                 // that listed a sample (0: none after round 0); null: not kept
+                 // that listed a sample (0: none after round 0), [3] 1 + the round at which a wait between the
+                 // workgroups of a launch gave up (0: none); null: not kept
   int on;        // 1: the fused launch; 2: this launch starts with the selection of the fused launch's results
 };
 
@@ -90,7 +92,10 @@ struct MvmArgs {
   int small_tiles_only;     // 1: never the large-tile kernel (its row padding differs)
   const int *skip_if_zero;  // non-null: a round launch does nothing when this device value is zero
   DualDev dual;
-  int rest_in_one;          // 1: this launch runs round `round` and every round after it (k_mvm_rounds_rest)  // Tiles of a group call that quantize the same input the same way (the column blocks of a layer split over several
+  int rest_in_one;          // 1: this launch runs round `round` and every round after it (k_mvm_rounds_rest)
+  int wait_spins;           // polls after which a wait between the workgroups of such a launch gives up (0: the default)
+  int wait_extra;           // arrivals such a wait expects beyond the launch's workgroups (0; tests of the give-up path: 1)
+  // Tiles of a group call that quantize the same input the same way (the column blocks of a layer split over several
   // tiles) share the rows of rounds 0 and 1: with xq_first[0] set, those rounds read xq_first[round] instead of
   // xq[round & 1] (every later round uses the tile's own xq as usual), and the init kernel writes the shared rows
   // for the one tile that has xq_first_writer = 1.  Requires rows_ahead_in_init (or a single round).
@@ -116,7 +121,9 @@ void launch_mvm_round(const MvmArgs &a, hipStream_t s);
 // of them and a.xq[0] = a.dual.xq2
 bool mvm_can_fuse_rounds(const MvmArgs &a);
 // the rounds from a.round on in one launch (a.rest_in_one = 1 for launch_mvm_round): for calls that expect them empty
-bool mvm_can_merge_rest(const MvmArgs &a, int n_cus);
+// resident_limit: workgroups of that launch that the GPU holds at once (mvm_rest_resident_limit)
+bool mvm_can_merge_rest(const MvmArgs &a, int resident_limit);
+int mvm_rest_resident_limit(const MvmArgs &a);
 void launch_mvm_dual(const MvmArgs &a, hipStream_t s);
 // AverageAbsMax noise management (rpu_forward_backward_pass.cpp:138-149): nm[b] holds the largest absolute input of
 // sample b and becomes the running average after that sample, in batch order; aux carries the value between calls
@@ -129,6 +136,10 @@ struct MvmGroup {
   const int *start; // [n + 1]
   int n;
   int m_batch;
+  // waits between the workgroups of k_mvm_rest_group (see MvmArgs::wait_spins / wait_extra); wait_failed: host-visible
+  // word that takes 1 + the round at which a wait gave up
+  int wait_spins = 0, wait_extra = 0;
+  int *wait_failed = nullptr;
 };
 void launch_mvm_init_group(const MvmGroup &g, int max_k, hipStream_t s);
 // seen: host-visible pair (any tile lists a sample for round 1, batch) written by the launch of round 1; may be null
@@ -136,6 +147,7 @@ void launch_mvm_round_group(const MvmGroup &g, int prefetch_depth, int weight_mo
                             hipStream_t s, int *seen = nullptr);
 // the rounds from round_first on in one launch, for calls that expect them to list nothing (see k_mvm_rounds_rest)
 bool mvm_group_can_merge_rest(const MvmGroup &g, int weight_mode);
+int mvm_group_rest_resident_limit(int weight_mode); // workgroups of k_mvm_rest_group that the GPU holds at once
 void launch_mvm_rest_group(const MvmGroup &g, int weight_mode, int round_first, int rounds, int workgroups, int *seen,
                            hipStream_t s);
 int mvm_round_workgroups(const MvmArgs &a);            // workgroups of a round launch for this tile
@@ -246,7 +258,8 @@ struct UpdateArgs {
   uint32_t *d_planes;
   int plane_slots; // slots per chunk the plane buffers are laid out for
   int n_chunks;    // ceil(m_batch / 32)
-  int *kmax;       // kmax[0..1]: largest BL of a batch (ping-pong by call), kmax[2]: constant 31
+  int *kmax;       // kmax[0..1]: largest BL of a batch (ping-pong by call), kmax[2]: constant 31, kmax[3]: longest line
+                   // among pulse words made elsewhere (launch_words_kmax)
   int kmax_slot;   // which entry this call uses
   float *x_val;  // [B][X] implicit line values
   float *d_val;  // [B][D]
@@ -277,6 +290,7 @@ void launch_update_prepare(const UpdateArgs &a, hipStream_t s);       // BL, A, 
 void launch_update_lines(const UpdateArgs &a, hipStream_t s);         // stochastic pulse words and their bit planes
 void launch_update_implicit_lines(const UpdateArgs &a, hipStream_t s); // deterministic line values
 void launch_update_planes(const UpdateArgs &a, hipStream_t s);        // bit planes of pulse words made elsewhere
+void launch_words_kmax(const UpdateArgs &a, hipStream_t s);           // a.kmax[a.kmax_slot] = longest bit line among such words
 void launch_update_pulsed(const UpdateArgs &a, hipStream_t s);        // coincidences + device steps
 // opt-in variant for LinearStep devices with multiplicative noise: per group of samples_per_step samples the
 // coincidences are counted and applied in closed form with one normal draw for their summed noise

@@ -31,6 +31,8 @@
 //   *_group        the same kernels over the tiles of a group in one launch.
 #include "kernels.h"
 
+#include <mutex>
+
 namespace rpu_amd {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
@@ -1182,45 +1184,76 @@ __device__ __forceinline__ void mvm_round_workgroup(const MvmArgs &a, int round,
   if (more_rounds) mvm_tile_finished(a, round, tile_b, n_act);
 }
 
+// Waits between the workgroups of one launch.  They are bounded, and a wait that runs out is reported, not passed
+// over: the thread that gives up raises the launch's abort word (every other waiting workgroup sees it and gives up
+// too), writes 1 + the round into the host-visible word `failed`, and every workgroup leaves the kernel -- the rounds
+// that were still to run would read stale lists.  The host finds the word at its next call on the tile, reports that
+// call's results as invalid and goes back to one launch per round.
+struct RoundWait {
+  int *abort;   // device memory, zero at the start of the call
+  int *failed;  // host-visible, may be null
+  int limit;    // polls before giving up
+  int extra;    // arrivals expected beyond the launch's own workgroups (0; a test of the give-up path asks for one more)
+};
+constexpr int REST_SPIN_LIMIT = 1 << 15; // about 1 us per poll: some tens of milliseconds
+
+__device__ __forceinline__ RoundWait round_wait_of(int *count, int *seen, int spins, int extra) {
+  return RoundWait{count + MVM_ABORT_WORD, seen ? seen + 3 : nullptr, spins > 0 ? spins : REST_SPIN_LIMIT, extra};
+}
+
+// thread 0: polls until *word reaches `target`; false when the wait ran out or another workgroup gave up
+__device__ __forceinline__ bool round_wait_poll(const RoundWait &wt, int *word, int target, int round) {
+  int spins = 0;
+  while (__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < target) {
+    const bool gave_up = ++spins >= wt.limit;
+    if (gave_up || ((spins & 15) == 0 && __hip_atomic_load(wt.abort, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0)) {
+      if (gave_up) {
+        __hip_atomic_store(wt.abort, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (wt.failed) __hip_atomic_store(wt.failed, round + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+      }
+      return false;
+    }
+    __builtin_amdgcn_s_sleep(8);
+  }
+  return true;
+}
+
 // All workgroups of a launch wait for each other, and what they wrote before is visible to all of them after (the
-// launch must fit on the GPU at once).  The wait is bounded: if it ever ran out, the rounds after it would read
-// stale lists.
-constexpr int REST_SPIN_LIMIT = 1 << 28;
-__device__ __forceinline__ void mvm_device_barrier(int *counter, int total) {
+// launch must fit on the GPU at once).  Returns false when the wait gave up: the caller leaves the kernel.
+__device__ __forceinline__ bool mvm_device_barrier(int *counter, int total, const RoundWait &wt, int round) {
+  __shared__ int sh_ok;
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
   __syncthreads();
   if (threadIdx.x == 0) {
     __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    int spins = 0;
-    while (__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < total && ++spins < REST_SPIN_LIMIT) {
-      __builtin_amdgcn_s_sleep(8);
-    }
+    sh_ok = round_wait_poll(wt, counter, total + wt.extra, round) ? 1 : 0;
   }
   __syncthreads();
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+  return sh_ok != 0;
 }
 
 // All workgroups of a launch wait until each has arrived, which it does once the atomics of its threads have been
 // performed (their results were consumed before the barrier): after the wait, what those atomics built up -- the number
 // of samples listed for the next round -- is final and can be read with a device-scope load.  Nothing else the
 // workgroups wrote is made visible: a launch that goes on to read such data calls mvm_device_barrier as well.  A few
-// microseconds, against tens for that one; bounded in the same way.
+// microseconds, against tens for that one; bounded and reported in the same way.
 // counter[0] counts the arrivals; the last one raises counter[1], which the others poll (so that the polls do not
 // queue up in front of the arrivals at the one address).
-__device__ __forceinline__ void mvm_arrive(int *counter, int total) {
+__device__ __forceinline__ bool mvm_arrive(int *counter, int total, const RoundWait &wt, int round) {
+  __shared__ int sh_ok;
   __syncthreads();
   if (threadIdx.x == 0) {
     const int before = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if (before == total - 1) {
+    if (before == total + wt.extra - 1) {
       __hip_atomic_store(counter + 1, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      sh_ok = 1;
     } else {
-      int spins = 0;
-      while (__hip_atomic_load(counter + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0 && ++spins < REST_SPIN_LIMIT) {
-        __builtin_amdgcn_s_sleep(8);
-      }
+      sh_ok = round_wait_poll(wt, counter + 1, 1, round) ? 1 : 0;
     }
   }
   __syncthreads();
+  return sh_ok != 0;
 }
 
 // Host-visible summary of a call for the choice of the next call's launches (a.dual.seen), kept by the first thread of
@@ -1354,6 +1387,8 @@ __global__ __launch_bounds__(256) void k_mvm_rest_group(MvmGroup g, int round_fi
   __shared__ float red[WAVES][16][64];
   __shared__ __attribute__((aligned(16))) float stage[WAVES * 2 * TILE * LDS_ROW];
   __shared__ int sh_first[MAX_GROUP + 1]; // first workgroup number of member t; [g.n] = total
+  const RoundWait wt{g.args[0].st.count + MVM_ABORT_WORD, g.wait_failed, g.wait_spins > 0 ? g.wait_spins : REST_SPIN_LIMIT,
+                     g.wait_extra};
   for (int round = round_first; round < rounds; ++round) {
     for (int t = threadIdx.x; t < g.n; t += blockDim.x) {
       const MvmArgs &a = g.args[t];
@@ -1378,7 +1413,10 @@ __global__ __launch_bounds__(256) void k_mvm_rest_group(MvmGroup g, int round_fi
     if (seen && round == 1 && blockIdx.x == 0) group_seen_update(g, seen);
     if (total == 0) return; // the same for every workgroup
     // the rows and lists that the round before left must be visible on every XCD
-    if (round > round_first) mvm_device_barrier(&g.args[0].st.count[MVM_ARRIVE_BASE + 4 * round + 2], (int)gridDim.x);
+    if (round > round_first &&
+        !mvm_device_barrier(&g.args[0].st.count[MVM_ARRIVE_BASE + 4 * round + 2], (int)gridDim.x, wt, round)) {
+      return;
+    }
     int t = 0;
     for (int n = blockIdx.x; n < total; n += gridDim.x) {
       while (n >= sh_first[t + 1]) ++t;
@@ -1389,7 +1427,7 @@ __global__ __launch_bounds__(256) void k_mvm_rest_group(MvmGroup g, int round_fi
     }
     if (round + 1 == rounds) return;
     // the counts of the next round are final once every workgroup has arrived
-    mvm_arrive(&g.args[0].st.count[MVM_ARRIVE_BASE + 4 * round], (int)gridDim.x);
+    if (!mvm_arrive(&g.args[0].st.count[MVM_ARRIVE_BASE + 4 * round], (int)gridDim.x, wt, round)) return;
   }
 }
 
@@ -1404,15 +1442,16 @@ __global__ __launch_bounds__(256) void k_mvm_rounds_rest(MvmArgs a) {
   __shared__ float red[WAVES][16][64];
   __shared__ __attribute__((aligned(16))) float stage[WAVES * 2 * TILE * LDS_ROW];
   if (a.dual.on == 2) mvm_dual_select(a, blockIdx.x);
+  const RoundWait wt = round_wait_of(a.st.count, a.dual.seen, a.wait_spins, a.wait_extra);
   for (int r = a.round; r < a.max_rounds; ++r) {
     // final since the launch before (first round) or since every workgroup arrived after the round before
     const int n_act = __hip_atomic_load(&a.st.count[r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     mvm_note_round(a, r, n_act, r == a.round && a.dual.on == 2);
     if (n_act == 0) return; // the same for every workgroup
-    if (r > a.round) mvm_device_barrier(&a.st.count[MVM_ARRIVE_BASE + 4 * r + 2], (int)gridDim.x);
+    if (r > a.round && !mvm_device_barrier(&a.st.count[MVM_ARRIVE_BASE + 4 * r + 2], (int)gridDim.x, wt, r)) return;
     mvm_round_workgroup<PD, WMODE>(a, r, blockIdx.x, n_act, red, stage);
     if (r + 1 == a.max_rounds) return;
-    mvm_arrive(&a.st.count[MVM_ARRIVE_BASE + 4 * r], (int)gridDim.x);
+    if (!mvm_arrive(&a.st.count[MVM_ARRIVE_BASE + 4 * r], (int)gridDim.x, wt, r)) return;
   }
 }
 
@@ -2420,18 +2459,67 @@ void launch_mvm_rest_group(const MvmGroup &g, int mode, int round_first, int rou
 // whether rounds 0 and 1 of this call can run as one launch (the caller decides whether they should)
 bool mvm_can_fuse_rounds(const MvmArgs &a) {
   if (a.io.perfect || a.io.bound_management == RPU_BM_NONE || a.max_rounds < 3 || a.transposed) return false;
-  if (a.pre_add || a.skip_if_zero || a.nm_phase || !a.speculate || !a.rows_ahead_in_init) return false;
+  if (a.pre_add || a.skip_if_zero || a.nm_phase || !a.speculate || !a.rows_ahead_in_init || a.in_index) return false;
   if (!a.small_tiles_only && big_threshold(a.m_batch, a.O) > 0) return false;
   return mvm_prefetch_depth(a.K, a.k_pad) >= 2 && weight_mode(a) != 1;
 }
 
+// Workgroups of `kernel` (256 threads, static LDS only) that the current GPU holds at once: what the occupancy query
+// reports per CU times the number of CUs.  The launches whose workgroups wait for each other are sized by it.
+template <typename K> static int resident_workgroups(K kernel) {
+  int per_cu = 0;
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, 256, 0) != hipSuccess || per_cu < 1) return 0;
+  return per_cu * current_device_cus();
+}
+
+int mvm_rest_resident_limit(const MvmArgs &a) {
+  static std::mutex m;
+  static int limit[64][3][3] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
+  const int mode = weight_mode(a);
+  if (mode == 1) return 0; // not instantiated
+  const int depth = mvm_prefetch_depth(a.K, a.k_pad);
+  const int di = depth == 4 ? 2 : (depth == 2 ? 1 : 0);
+  std::lock_guard<std::mutex> lock(m);
+  int &v = limit[dev][di][mode];
+  if (v == 0) {
+    if (mode == 0) {
+      v = depth == 4 ? resident_workgroups(k_mvm_rounds_rest<4, 0>)
+                     : (depth == 2 ? resident_workgroups(k_mvm_rounds_rest<2, 0>) : resident_workgroups(k_mvm_rounds_rest<1, 0>));
+    } else {
+      v = depth == 4 ? resident_workgroups(k_mvm_rounds_rest<4, 2>)
+                     : (depth == 2 ? resident_workgroups(k_mvm_rounds_rest<2, 2>) : resident_workgroups(k_mvm_rounds_rest<1, 2>));
+    }
+    if (v == 0) v = -1; // the query failed: never merge
+  }
+  return v > 0 ? v : 0;
+}
+
+int mvm_group_rest_resident_limit(int mode) {
+  static std::mutex m;
+  static int limit[64][3] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64 || mode == 1) return 0;
+  std::lock_guard<std::mutex> lock(m);
+  int &v = limit[dev][mode];
+  if (v == 0) {
+    v = mode == 0 ? resident_workgroups(k_mvm_rest_group<0>) : resident_workgroups(k_mvm_rest_group<2>);
+    if (v == 0) v = -1;
+  }
+  return v > 0 ? v : 0;
+}
+
 // whether the rounds after round 0 of this call can share one launch (mvm_can_fuse_rounds without the conditions of
-// the two-accumulator kernel; all workgroups must be resident at once: at most one per CU is assumed)
-bool mvm_can_merge_rest(const MvmArgs &a, int n_cus) {
+// the two-accumulator kernel).  Its workgroups wait for each other between rounds, so all of them must be resident at
+// once: resident_limit is what the GPU holds of that kernel when nothing else runs on it.  Another launch that holds
+// CUs at that moment (a second stream) can make a wait run out; that is reported (see RoundWait), never passed over.
+bool mvm_can_merge_rest(const MvmArgs &a, int resident_limit) {
   if (a.io.perfect || a.io.bound_management == RPU_BM_NONE || a.max_rounds < 3 || a.transposed) return false;
-  if (a.pre_add || a.skip_if_zero || a.nm_phase) return false;
+  // gathered input: the rows of a further round are written by k_mvm_round_tail alone, one launch per round
+  if (a.pre_add || a.skip_if_zero || a.nm_phase || a.in_index) return false;
   if (!a.small_tiles_only && big_threshold(a.m_batch, a.O) > 0) return false;
-  return mvm_round_workgroups(a) <= n_cus && weight_mode(a) != 1;
+  return mvm_round_workgroups(a) <= resident_limit && weight_mode(a) != 1;
 }
 
 void launch_mvm_dual(const MvmArgs &a_in, hipStream_t s) {

@@ -457,6 +457,28 @@ __global__ __launch_bounds__(256) void k_update_planes(UpdateArgs a) {
   }
 }
 
+// Longest bit line among packed pulse words made elsewhere: the highest pulse slot set in any word of the batch
+// (bit 0 is the sign).  out[0] must be zero before; every workgroup sends its own maximum.
+__global__ __launch_bounds__(256) void k_words_kmax(const uint32_t *xw, size_t nx, const uint32_t *dw, size_t nd, int *out) {
+  __shared__ uint32_t sh[4];
+  uint32_t acc = 0u;
+  const size_t stride = (size_t)gridDim.x * 256u, first = (size_t)blockIdx.x * 256u + threadIdx.x;
+  for (size_t i = first; i < nx; i += stride) acc |= xw[i];
+  for (size_t i = first; i < nd; i += stride) acc |= dw[i];
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) acc |= (uint32_t)__shfl_xor((int)acc, off);
+  if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = acc;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const uint32_t pulses = (sh[0] | sh[1] | sh[2] | sh[3]) >> 1;
+    if (pulses) atomicMax(out, 32 - __clz((int)pulses));
+  }
+}
+
+__global__ void k_zero_word(int *p) {
+  if (threadIdx.x == 0) *p = 0;
+}
+
 // Cross-point parameters of the pulse loop.  A step down subtracts (slope_down * w + scale_down) * f; with
 // the down parameters negated every pulse is the same "w += (slope * w + scale) * f", and negation is
 // exact in floating point.  The two clips of the reference (rpu_constantstep_device.cpp:48-53:
@@ -1271,6 +1293,14 @@ void launch_update_implicit_lines(const UpdateArgs &a, hipStream_t s) {
       hipLaunchKernelGGL((KERNEL<RPU_DEVICE_LINEAR_STEP, false>), grid, dim3(256), 0, s, a);        \
     }                                                                                               \
   } while (0)
+
+void launch_words_kmax(const UpdateArgs &a, hipStream_t s) {
+  const size_t nx = (size_t)a.m_batch * a.x_size, nd = (size_t)a.m_batch * a.d_size;
+  const size_t blocks = std::min<size_t>(256, (nx + nd + 4095) / 4096);
+  hipLaunchKernelGGL(k_zero_word, dim3(1), dim3(64), 0, s, a.kmax + a.kmax_slot);
+  hipLaunchKernelGGL(k_words_kmax, dim3((unsigned)std::max<size_t>(blocks, 1)), dim3(256), 0, s, a.x_words, nx, a.d_words, nd,
+                     a.kmax + a.kmax_slot);
+}
 
 void launch_update_planes(const UpdateArgs &a, hipStream_t s) {
   dim3 grid((a.x_size + a.d_size + 3) / 4, (a.m_batch + 63) / 64);

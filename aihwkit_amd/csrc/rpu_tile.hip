@@ -9,6 +9,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <atomic>
 #include <cmath>
 #include <cstring>
 #include <memory>
@@ -34,6 +35,9 @@ namespace rpu_amd {
 
 namespace {
 
+// device allocations made by the library's buffers so far (rpu_device_allocation_count)
+std::atomic<long> g_device_allocations{0};
+
 template <typename T> struct DevBuf {
   T *p = nullptr;
   size_t n = 0;
@@ -43,6 +47,7 @@ template <typename T> struct DevBuf {
     if (!owned) throw RpuError("A buffer that belongs to the caller cannot grow.");
     release();
     RPU_HIP_CHECK(hipMalloc((void **)&p, count * sizeof(T)));
+    g_device_allocations.fetch_add(1, std::memory_order_relaxed);
     n = count;
   }
   // use memory of the caller from now on (never freed here)
@@ -96,6 +101,10 @@ unsigned char *noalloc_scratch(int device) {
   static std::mutex m;
   static unsigned char *ptr[64] = {};
   if (device < 0 || device >= 64) throw RpuError("Device number out of range for the static scratch array.");
+  // every GPU holds its own copy of the array at its own address, and the lookup answers for the current device
+  int current = -1;
+  RPU_HIP_CHECK(hipGetDevice(&current));
+  if (current != device) throw RpuError("The static scratch array is looked up with its device current.");
   std::lock_guard<std::mutex> lock(m);
   if (!ptr[device]) {
     unsigned char *p = nullptr;
@@ -181,6 +190,22 @@ struct Tile {
   int *seen_host = nullptr, *seen_dev = nullptr;
   int rest_from = 0, rest_quiet = 0; // the last round that listed samples in the recent calls, and calls since it did
   int fused_rounds = -1;
+  // A launch that runs several rounds makes its workgroups wait for each other; a wait that runs out is written to
+  // seen_host[3] by the kernel.  The next compute call on the tile reports it (the results of that forward call are
+  // invalid) and from then on the tile runs one launch per round.  The hook values shorten the wait and make it expect
+  // one arrival too many, for the test of that path.
+  bool merged_off = false;
+  uint32_t merged_call = 0; // random-stream index of the last forward call that used such a launch
+  int wait_spins_hook = 0, wait_extra_hook = 0;
+  void check_round_waits() {
+    if (!seen_host) return;
+    const int failed = *(volatile int *)&seen_host[3];
+    if (!failed) return;
+    *(volatile int *)&seen_host[3] = 0;
+    merged_off = true;
+    throw RpuError("forward round barrier timed out in round " + std::to_string(failed - 1) + "; results of call " +
+                   std::to_string(merged_call) + " are invalid (the tile now runs one launch per round).");
+  }
   int cu_count = 0;
   int n_cus() {
     if (!cu_count) {
@@ -475,6 +500,7 @@ struct Tile {
   // tensor may be null)
   bool check_compute(int m_batch, const void *p0, const void *p1) {
     if (!resident()) throw RpuError("Tile is not resident on a GPU: forward / backward / update need rpu_tile_to_device first.");
+    check_round_waits();
     if (m_batch < 0) throw RpuError("m_batch must not be negative.");
     if (m_batch == 0) return false;
     if (!p0 || !p1) throw RpuError("Null device pointer.");
@@ -774,10 +800,15 @@ struct Tile {
           }
         }
         const int first_mergeable = fuse ? 2 : 1;
-        if (mvm_can_merge_rest(a, n_cus())) {
+        if (!merged_off && mvm_can_merge_rest(a, mvm_rest_resident_limit(a))) {
           if (fused_rounds == 2 || fused_rounds == 3) merge_from = first_mergeable;
           else if (fused_rounds < 0 && of > 0) merge_from = std::max(first_mergeable, rest_from + 1);
           if (merge_from + 1 >= a.max_rounds) merge_from = 0; // the last round alone: a plain launch
+          if (merge_from > 0) {
+            a.wait_spins = wait_spins_hook;
+            a.wait_extra = wait_extra_hook;
+            merged_call = a.call;
+          }
         }
       }
       if (fuse) {
@@ -875,8 +906,11 @@ struct Tile {
     a.x_words = const_cast<uint32_t *>(x_words); a.d_words = const_cast<uint32_t *>(d_words);
     a.key = key(); a.call = call++;
     set_plane_args(a, B);
-    a.kmax_slot = 2; // words from outside: all 31 slots may be in use
+    // words from outside: the longest bit line among them picks the pulse loop, as the batch's largest BL does for the
+    // tile's own words (short lines then take the same loop, and the same noise stream, as in rpu_tile_update)
+    a.kmax_slot = 3;
     prof_begin(s);
+    launch_words_kmax(a, s);
     launch_update_planes(a, s);
     prof_mark(s, "update_planes");
     if (dev.p.count_pulses) count_pulses(a, false, s);
@@ -1370,6 +1404,8 @@ struct Tile {
                      std::to_string((size_t)RPU_NOALLOC_MAX_SCRATCH_BYTES) + ".");
     }
     if (lr == 0.0f) return;
+    // refused before anything is written to the shared array
+    if (words_per_sample_for(up, lr, dev.p.dw_min) > 1) throw RpuError("update_noalloc holds bit lines of at most 31 pulses.");
     unsigned char *ws = noalloc_scratch(device_id);
     carve_update_scratch(ws, X, D, B, bias, nullptr, &rows);
     const float *xin = x;
@@ -2164,6 +2200,10 @@ struct rpu_group {
   // host-visible pairs (any tile listed a sample for round 1, batch), one per kernel variant of the group's last call:
   // the next call runs the rounds after round 0 in one launch where nothing was listed
   int *seen_host = nullptr, *seen_dev = nullptr;
+  // the word after the pairs: 1 + the round at which a wait between the workgroups of a merged-round launch gave up;
+  // reported by the next call, after which the group runs one launch per round
+  bool merged_off = false;
+  int wait_spins_hook = 0, wait_extra_hook = 0;
   int cu_count = 0;
   // quantized rows of rounds 0 and 1 shared by tiles that read the same input with the same DAC (two buffers per set)
   std::vector<DevBuf<float>> first_rows;
@@ -2361,6 +2401,14 @@ static int group_mvm(rpu_group_t *group, const float *const *x_dev, const long *
     DeviceGuard dg(group->device_id);
     hipStream_t s = (hipStream_t)stream;
     const int n = (int)group->tiles.size();
+    constexpr int kSeenPairs = 16;
+    if (group->seen_host && *(volatile int *)&group->seen_host[2 * kSeenPairs]) {
+      const int failed = *(volatile int *)&group->seen_host[2 * kSeenPairs];
+      *(volatile int *)&group->seen_host[2 * kSeenPairs] = 0;
+      group->merged_off = true;
+      throw RpuError("forward round barrier timed out in round " + std::to_string(failed - 1) +
+                     "; results of the group's last forward call are invalid (the group now runs one launch per round).");
+    }
     // the staging buffers may still feed the copy of the previous call
     RPU_HIP_CHECK(hipEventSynchronize(group->copied));
 
@@ -2517,10 +2565,9 @@ static int group_mvm(rpu_group_t *group, const float *const *x_dev, const long *
     int max_k = 0;
     for (int i = 0; i < n; ++i) max_k = std::max(max_k, args[i].K);
     launch_mvm_init_group(all, max_k, s);
-    constexpr int kSeenPairs = 16;
     if (!group->seen_host) {
-      RPU_HIP_CHECK(hipHostMalloc((void **)&group->seen_host, 2 * kSeenPairs * sizeof(int), hipHostMallocMapped));
-      for (int i = 0; i < 2 * kSeenPairs; ++i) group->seen_host[i] = 0;
+      RPU_HIP_CHECK(hipHostMalloc((void **)&group->seen_host, (2 * kSeenPairs + 1) * sizeof(int), hipHostMallocMapped));
+      for (int i = 0; i < 2 * kSeenPairs + 1; ++i) group->seen_host[i] = 0;
       RPU_HIP_CHECK(hipHostGetDevicePointer((void **)&group->seen_dev, group->seen_host, 0));
       hipDeviceProp_t prop;
       RPU_HIP_CHECK(hipGetDeviceProperties(&prop, group->device_id));
@@ -2539,9 +2586,13 @@ static int group_mvm(rpu_group_t *group, const float *const *x_dev, const long *
         MvmGroup g{group->d_args.p + seg.first, group->d_start.p + seg.start_offset, seg.count, m_batch};
         int *seen = k < (size_t)kSeenPairs ? group->seen_dev + 2 * k : nullptr;
         // the last call of this group listed nothing for round 1: one launch for all rounds after round 0
-        if (r == 1 && rounds >= 3 && seen && !transposed && mvm_group_can_merge_rest(g, seg.mode) &&
+        const int rest_wgs = (r == 1 && rounds >= 3) ? std::min(256, mvm_group_rest_resident_limit(seg.mode)) : 0;
+        if (rest_wgs > 0 && seen && !transposed && !group->merged_off && mvm_group_can_merge_rest(g, seg.mode) &&
             *(volatile int *)&group->seen_host[2 * k + 1] == m_batch && *(volatile int *)&group->seen_host[2 * k] == 0) {
-          launch_mvm_rest_group(g, seg.mode, 1, rounds, std::min(256, group->cu_count), seen, s);
+          g.wait_spins = group->wait_spins_hook;
+          g.wait_extra = group->wait_extra_hook;
+          g.wait_failed = group->seen_dev + 2 * kSeenPairs;
+          launch_mvm_rest_group(g, seg.mode, 1, rounds, rest_wgs, seen, s);
           merged[k] = true;
           continue;
         }
@@ -3096,6 +3147,29 @@ int rpu_tile_set_fused_rounds(rpu_tile_t *tile, int mode) {
     }
     std::lock_guard<std::mutex> lock(tile->t.mutex);
     tile->t.fused_rounds = mode;
+    tile->t.merged_off = false; // an explicit choice re-arms the merged launches after a reported time-out
+  });
+}
+
+long rpu_device_allocation_count(void) { return g_device_allocations.load(std::memory_order_relaxed); }
+
+int rpu_tile_set_round_wait_test_hook(rpu_tile_t *tile, int spin_limit, int extra_arrivals) {
+  return guarded([&] {
+    if (!tile) throw RpuError("null tile");
+    if (spin_limit < 0 || extra_arrivals < 0 || extra_arrivals > 1) throw RpuError("round wait hook: spin_limit >= 0, extra_arrivals 0 or 1");
+    std::lock_guard<std::mutex> lock(tile->t.mutex);
+    tile->t.wait_spins_hook = spin_limit;
+    tile->t.wait_extra_hook = extra_arrivals;
+  });
+}
+
+int rpu_group_set_round_wait_test_hook(rpu_group_t *group, int spin_limit, int extra_arrivals) {
+  return guarded([&] {
+    if (!group) throw RpuError("null group");
+    if (spin_limit < 0 || extra_arrivals < 0 || extra_arrivals > 1) throw RpuError("round wait hook: spin_limit >= 0, extra_arrivals 0 or 1");
+    std::lock_guard<std::mutex> lock(group->mutex);
+    group->wait_spins_hook = spin_limit;
+    group->wait_extra_hook = extra_arrivals;
   });
 }
 

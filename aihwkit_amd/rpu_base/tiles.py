@@ -515,6 +515,11 @@ class _CudaTileMixin:
         -1 (default) = the tile decides by what its recent calls needed.  Outputs and round counts do not depend on it."""
         check(lib().rpu_tile_set_fused_rounds(self._h, int(mode)))
 
+    def set_round_wait_test_hook(self, spin_limit: int = 0, extra_arrivals: int = 0) -> None:
+        """For the test of the time-out path of the merged-round launches only: shorten their bounded waits to
+        ``spin_limit`` polls and make them expect ``extra_arrivals`` workgroups more than the launch has."""
+        check(lib().rpu_tile_set_round_wait_test_hook(self._h, int(spin_limit), int(extra_arrivals)))
+
     def get_update_words_per_sample(self) -> int:
         """Rows of pulse words per sample of the last stochastic update: ceil(longest possible BL / 31)."""
         n = C.c_int32(0)
@@ -609,6 +614,10 @@ class TileGroup:
                 lib().rpu_group_destroy(handle)
             except Exception:  # pylint: disable=broad-except
                 pass
+
+    def set_round_wait_test_hook(self, spin_limit: int = 0, extra_arrivals: int = 0) -> None:
+        """For the test of the time-out path of the group's merged-round launch only (see the tiles' method)."""
+        check(lib().rpu_group_set_round_wait_test_hook(self._g, int(spin_limit), int(extra_arrivals)))
 
     @staticmethod
     def _rows(tensor: torch.Tensor, what: str) -> torch.Tensor:

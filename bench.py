@@ -180,10 +180,28 @@ def main() -> int:
               "variant, then (unless --no-other-batches) 2 forward and 2 backward calls at batch 16384", file=sys.stderr)
         return 0
 
+    # The contract loop works on the configuration as stated: repeated updates with the same inputs let the weights of
+    # a SoftBounds tile shrink until no sample saturates the ADC any more (1.0 bound-management rounds instead of the
+    # stated 2.1), so every step starts from the initial weights (a 4 MB device copy into the tile's weight matrix, on
+    # the same stream and inside the timed region) and takes the next of POOL pre-uploaded (x, d) batches.
+    POOL = 8
+    rng_pool = np.random.default_rng(77)
+    x_pool = [xg] + [torch.from_numpy(rng_pool.uniform(-1, 1, x.shape).astype(np.float32)).cuda() for _ in range(POOL - 1)]
+    d_pool = [dg] + [torch.from_numpy((d.std() * rng_pool.standard_normal(d.shape)).astype(np.float32)).cuda()
+                     for _ in range(POOL - 1)]
+    w_live = torch.empty(d_size, x_size, dtype=torch.float32, device="cuda")
+    tile.set_shared_weights_row_major(w_live)   # the tile's weight matrix is this tensor from now on (zero copy)
+    torch.cuda.synchronize()
+    w_init = w_live.clone()                     # the initial weights as the tile holds them (clipped to the device bounds)
+    step_no = [0]
+
     def step():
-        tile.forward(xg, False, False, False, False, True)
-        tile.backward(dg, False, False, False, True)
-        tile.update(xg, dg, False, False, False, True)
+        k = step_no[0] % POOL
+        step_no[0] += 1
+        w_live.copy_(w_init, non_blocking=True)
+        tile.forward(x_pool[k], False, False, False, False, True)
+        tile.backward(d_pool[k], False, False, False, True)
+        tile.update(x_pool[k], d_pool[k], False, False, False, True)
 
     def time_calls(fn, n):
         start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -230,6 +248,11 @@ def main() -> int:
         step()
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    # bound-management rounds the forward calls of that loop ran: the next step's forward call, read back
+    w_live.copy_(w_init)
+    tile.forward(x_pool[step_no[0] % POOL], False, False, False, False, True)
+    loop_rounds = float(tile.get_bm_rounds(batch).numpy().mean())
+    w_live.copy_(w_init)
 
     # update alone
     ms_update = time_calls(lambda: tile.update(xg, dg, False, False, False, True), n)
@@ -334,7 +357,9 @@ def main() -> int:
         "dtype": "f32",
         "data": "synthetic",
         "config": {"workload": workload, "x_size": x_size, "d_size": d_size, "batch": batch, "lr": lr,
-                   "step": "forward + backward + update"},
+                   "step": "initial weights restored (4 MB device copy, timed) + forward + backward + update on the next "
+                           "of %d pre-uploaded input batches" % POOL,
+                   "mean_bm_rounds_in_step_loop": loop_rounds},
         "update": {"ms_per_call": ms_update, "kernels_ms": {k: v[0] for k, v in prof_update.items()}},
         "forward": {"ms_per_call": ms_forward, "gflops": flops_per_call / (ms_forward * 1e-3) / 1e9,
                     "mean_bm_rounds": float(rounds.mean()), "kernels_ms": {k: v[0] for k, v in prof_forward.items()},

@@ -661,8 +661,21 @@ int rpu_tile_set_extra(rpu_tile_t *tile, const int64_t *values_host, int count);
  * second round: rounds 0 and 1 in one launch; and the rounds after the last one that listed any sample in those calls
  * (the estimate rises at once and falls after eight calls below it), which are expected to be empty, share one
  * launch.  0: always the separate launches.  1 / 2 / 3: that shortcut whenever the shape allows it
- * (single tile, rounds on the 32 x 32 kernel, at most one workgroup per CU for 2 and 3, no per-line periphery terms). */
+ * (single tile, rounds on the 32 x 32 kernel, for 2 and 3 no more workgroups than the GPU holds of that kernel at once
+ * -- what the occupancy query reports per CU times the CUs --, no per-line periphery terms).
+ * The waits of shortcut 2 are bounded (some tens of milliseconds).  They assume that the launch has the GPU's CUs to
+ * itself; work on another stream that holds CUs at that moment can make a wait run out.  That is never passed over: the
+ * launch stops, and the next forward / backward / update call on the tile fails with "forward round barrier timed out
+ * ...; results of call N are invalid", after which the tile runs one launch per round (setting a mode again re-arms
+ * the shortcut).  Tile groups report the same way at their next call. */
 int rpu_tile_set_fused_rounds(rpu_tile_t *tile, int mode);
+
+/* No counterpart in the reference; for the test of the time-out path above only.  spin_limit > 0 shortens the bounded
+ * waits of the tile's (or group's) merged-round launches to that many polls, extra_arrivals = 1 makes every wait expect
+ * one workgroup more than the launch has, so that it runs out while every workgroup still leaves its kernel normally.
+ * 0, 0 restores the defaults. */
+int rpu_tile_set_round_wait_test_hook(rpu_tile_t *tile, int spin_limit, int extra_arrivals);
+int rpu_group_set_round_wait_test_hook(rpu_group_t *group, int spin_limit, int extra_arrivals);
 
 /* ---- inspection hooks (mirror the reference's debug hooks) ------------------------------ */
 
@@ -721,6 +734,11 @@ int rpu_philox4x32_10_device(const uint32_t counter[4], const uint32_t key[2], u
                              int device_id);
 
 /* ---- errors / info ------------------------------------------------------------------------ */
+
+/* No counterpart in the reference.  Number of device allocations (hipMalloc) that the buffers of this library's tiles
+ * and groups have made in this process so far; a caller, or a test, can hold it against the claim that a call allocates
+ * nothing. */
+long rpu_device_allocation_count(void);
 
 const char *rpu_last_error(void);
 int rpu_abi_version(void);

@@ -254,3 +254,80 @@ def test_more_than_sixteen_rounds_in_one_launch(gpu_device):
     y, rounds = both_ways(meta, dev, x_size, d_size, w, x)
     assert rounds.max() >= 18 and len(set(rounds.tolist())) >= 3
     assert np.abs(y).max() > 0.0
+
+
+def test_a_wait_that_runs_out_is_reported_and_the_tile_recovers(gpu_device):
+    """The launch that runs several rounds makes its workgroups wait for each other.  The test hook shortens that wait and
+    makes it expect one arrival too many, so that it runs out while every workgroup still leaves its kernel: the next
+    call on the tile must fail with the time-out message, and the calls after it (one launch per round again) must give
+    the results of the separate launches."""
+    meta, dev = config2()
+    for io in (meta.forward_io, meta.backward_io):
+        io.out_noise = 0.0
+    w, x, _d = config2_data(1024, 1024, 256)
+    host, _orc, _ = build_pair(meta, dev, 1024, 1024, gpu=False)
+    host.set_weights(torch.from_numpy(w))
+    ref, tile = tiles.CudaAnalogTile(host), tiles.CudaAnalogTile(host)
+    ref.set_fused_rounds(0)
+    xin = torch.from_numpy(x).cuda()
+    want = ref.forward(xin).cpu().numpy()
+    assert ref.get_bm_rounds(256).max() >= 3                     # rounds beyond the first merged one have work
+    tile.set_fused_rounds(2)
+    assert np.array_equal(tile.forward(xin).cpu().numpy(), want)  # the merged launch, waits intact
+    tile.set_round_wait_test_hook(2000, 1)
+    tile.forward(xin)                                             # stops after its first round
+    torch.cuda.synchronize()
+    with pytest.raises(RuntimeError, match="forward round barrier timed out in round 1; results of call"):
+        tile.forward(xin)
+    tile.set_round_wait_test_hook(0, 0)
+    tile.set_profiling(True)
+    assert np.array_equal(tile.forward(xin).cpu().numpy(), want)  # recovered: separate launches although mode 2 stands
+    assert sum(1 for name, _ms in tile.get_profile() if name == "mvm_round") == 5
+    tile.set_profiling(False)
+    assert np.array_equal(tile.get_bm_rounds(256).numpy(), ref.get_bm_rounds(256).numpy())
+    tile.set_fused_rounds(2)                                      # an explicit choice arms the merged launch again
+    tile.set_profiling(True)
+    assert np.array_equal(tile.forward(xin).cpu().numpy(), want)
+    assert sum(1 for name, _ms in tile.get_profile() if name == "mvm_round") == 2
+    tile.set_profiling(False)
+
+
+def test_a_group_reports_a_wait_that_runs_out(gpu_device):
+    """The same for the launch that runs the later rounds of a whole group."""
+    from helpers import constant_step
+    rng = np.random.default_rng(5)
+    batch, d_size = 96, 64
+    grouped, oracles = [], []
+    for k in range(3):
+        x_size = (64, 96, 130)[k]
+        f_io = noise_free_io(inp_res=1 / 128.0, out_res=1 / 512.0, noise_management=NM.AbsMax,
+                             bound_management=BM.Iterative, out_bound=2.0)
+        dev = constant_step(w_max_dtod=0.0, w_min_dtod=0.0, w_max=1.0, w_min=-1.0, construction_seed=k + 1)
+        host, orc, _ = build_pair(make_meta(f_io, noise_free_io()), dev, x_size, d_size, gpu=False)
+        w = (rng.integers(-60, 61, (d_size, x_size)) / 64.0).astype(F)
+        host.set_weights(torch.from_numpy(w))
+        orc.set_weights(w)
+        grouped.append(tiles.CudaAnalogTile(host))
+        oracles.append(orc)
+    group = tiles.TileGroup(grouped)
+    sizes = [t.get_x_size() for t in grouped]
+    loud = [(rng.integers(-64, 65, (batch, n)) / 64.0).astype(F) for n in sizes]
+    quiet = []
+    for n in sizes:
+        x = np.zeros((batch, n), F)
+        x[np.arange(batch), rng.integers(0, n, batch)] = 0.5
+        quiet.append(x)
+
+    def run(xs):
+        return [y.cpu().numpy() for y in group.forward([torch.from_numpy(x).cuda() for x in xs])]
+
+    run(quiet)                                                    # nothing listed: the next call merges its later rounds
+    group.set_round_wait_test_hook(2000, 1)
+    run(loud)                                                     # the merged launch runs round 1 and gives up after it
+    torch.cuda.synchronize()
+    with pytest.raises(RuntimeError, match="forward round barrier timed out"):
+        run(loud)
+    group.set_round_wait_test_hook(0, 0)
+    for xs in (loud, quiet, quiet, loud):                         # one launch per round from now on: exact again
+        for y, orc, x in zip(run(xs), oracles, xs):
+            assert np.array_equal(y, orc.forward(x))

@@ -260,3 +260,37 @@ def test_wide_convolution_on_many_patches_equals_the_pass_over_the_unfolded_imag
     want = F.fold(back.double(), (side, side), 3, padding=1)
     assert (dx.double() - want).abs().max() <= 1e-5 * want.abs().max()
     assert dx.abs().max() > 0.1
+
+
+@pytest.mark.parametrize("mode", [2, -1, 3])
+def test_gathered_forward_runs_every_round_whatever_the_launch_mode(gpu_device, mode):
+    """A wide convolution whose patches are gathered by the init kernels (2048 patches, 40 outputs: few enough workgroups
+    for the launch that merges the later rounds): two calls in a row, quiet inputs and then saturating ones, give the
+    outputs and round counts of the separate launches (mode 0) in every launch mode."""
+    rng = np.random.default_rng(21)
+    c_in, side, n, c_out = 16, 16, 8, 40
+    indices, patches = conv_indices((c_in, side, side), (3, 3), (1, 1), (1, 1), (1, 1), True)
+    x_size = c_in * 9 + 1
+    f_io = noise_free_io(inp_res=1 / 128.0, out_res=1 / 512.0, out_bound=1.0, noise_management=dv.NoiseManagementType.AbsMax,
+                         bound_management=dv.BoundManagementType.Iterative)
+    dev = constant_step(dw_min=0.002, dw_min_std=0.0, construction_seed=4, w_max_dtod=0.0, w_min_dtod=0.0, w_max=1.0, w_min=-1.0)
+    w = torch.from_numpy(rng.normal(0, 0.25, (c_out, x_size)).astype(np.float32))
+    quiet = torch.from_numpy(rng.normal(0, 1, (n, c_in, side, side)).astype(np.float32)).cuda()
+    loud = quiet.clone()
+    quiet_w = w * 0.02          # no patch saturates the ADC with these weights
+    results = {}
+    for m in (0, mode):
+        _host, _orc, gpu = build_pair(make_meta(f_io, noise_free_io()), dev, x_size, c_out)
+        gpu.set_matrix_indices(indices)
+        gpu.set_fused_rounds(m)
+        out = []
+        for weights, x in ((quiet_w, quiet), (quiet_w, quiet), (w, loud), (w, loud)):
+            gpu.set_weights(weights)
+            y = gpu.forward_indexed(x, torch.empty(n, c_out, side, side).cuda())
+            out.append((y.clone(), gpu.get_bm_rounds(n * patches).clone()))
+        results[m] = out
+    assert results[0][0][1].max() == 1                       # the quiet calls stop after one round
+    assert results[0][2][1].max() >= 3                       # the loud ones need at least two further rounds
+    for (y0, r0), (y1, r1) in zip(results[0], results[mode]):
+        assert torch.equal(r0, r1)
+        assert torch.equal(y0, y1)

@@ -48,6 +48,28 @@ def test_update_without_allocation_equals_update(bias, layout):
             assert torch.equal(u, v)
 
 
+def test_first_call_without_allocation_on_a_fresh_tile_allocates_nothing():
+    """The defining property: across the first such call on a tile that has never run an update, the library's buffers
+    make no device allocation and the free device memory does not change (the kernels' code is loaded beforehand by an
+    ordinary update on another tile)."""
+    from aihwkit_amd._cabi import lib
+    meta, dev = config2()
+    ref, noa = pair(meta, dev, 300, 200)
+    rng = np.random.default_rng(2)
+    for bias in (False, True):
+        batch = 96
+        xg = torch.from_numpy(rng.uniform(-1, 1, (batch, 300 - int(bias))).astype(np.float32)).cuda()
+        dg = torch.from_numpy((0.05 * rng.standard_normal((batch, 200))).astype(np.float32)).cuda()
+        ref.update(xg, dg, bias, False, False, False)
+        torch.cuda.synchronize()
+        allocations, free = lib().rpu_device_allocation_count(), torch.cuda.mem_get_info()[0]
+        noa.update(xg, dg, bias, False, False, True)
+        torch.cuda.synchronize()
+        assert lib().rpu_device_allocation_count() == allocations
+        assert torch.cuda.mem_get_info()[0] == free
+        assert np.array_equal(ref.get_weights().numpy(), noa.get_weights().numpy())
+
+
 def test_update_without_allocation_on_another_device_kind_and_long_bit_lines():
     meta = make_meta(desired_bl=31, update_management=False, update_bl_management=False)
     dev = constant_step(dw_min=0.001, dw_min_std=0.3, construction_seed=9, enforce_consistency=True)
