@@ -54,7 +54,13 @@ struct DualDev {
 };
 
 struct MvmArgs {
-  const float *w; // row-major [d_size][x_size]
+  // The weight matrix as it is stored: rows of w_ld elements.  w_oc = 0: a row holds the contraction index of one
+  // output (out[o] = sum_k w[o * w_ld + k] in[k]); w_oc = 1: a row holds the outputs of one contraction index
+  // (out[o] = sum_k w[k * w_ld + o] in[k]).  A tile that stores [d_size][x_size] runs forward with w_oc = 0 and
+  // backward with w_oc = 1; one that stores [x_size][d_size] (the layout of the reference's CUDA tiles) the other way
+  // round.  Set by mvm_set_weights.
+  const float *w;
+  int w_oc, w_ld;
   int x_size, d_size;
   const float *in;
   long in_sb, in_sk; // input element (b, k) at in[b * in_sb + k * in_sk]
@@ -64,7 +70,8 @@ struct MvmArgs {
   int K, O;       // contraction length and number of outputs
   int k_pad;      // K rounded up to the step of the contraction kernel (mvm_k_pad)
   float *xq[2];   // ping-pong scratch [rows][k_pad]: DAC-quantized inputs, zero padded (rows: see MvmState::row)
-  int transposed; // 0: out[o] = sum_k W[o][k] in[k] (forward); 1: out[o] = sum_k W[k][o] in[k] (backward)
+  int transposed; // 0: forward pass (out = W in), 1: backward pass (out = W^T in); decides the scales of a round, not
+                  // how the weights are addressed (w_oc)
   int round;      // bound-management round, 0-based
   int max_rounds; // rounds launched for this call (mvm_max_rounds)
   int speculate;  // 1: each round also quantizes every row for the round after it (short path between rounds, for
@@ -113,6 +120,13 @@ struct MvmArgs {
   long in_gs;
 };
 
+// weight operand of a call: the matrix at w with rows of `ld` elements, stored [d_size][x_size] (xd_storage = false) or
+// [x_size][d_size]; a.transposed must be set
+inline void mvm_set_weights(MvmArgs &a, const float *w, int ld, bool xd_storage) {
+  a.w = w;
+  a.w_ld = ld;
+  a.w_oc = (a.transposed != 0) != xd_storage ? 1 : 0;
+}
 // noise management + per-sample state for round 0
 void launch_mvm_init(const MvmArgs &a, hipStream_t s);
 // one round of DAC -> MFMA contraction -> ADC
@@ -156,7 +170,8 @@ int mvm_round_workgroups(const MvmArgs &a);            // workgroups of a round 
 int mvm_big_workgroups(const MvmArgs &a, int bb);
 // bb: samples of a workgroup tile, 128 or 64 (mvm_big_sample_tile: by the workgroups the launch would have with 128)
 int mvm_big_sample_tile(int workgroups_128, int n_cus);
-void launch_mvm_big_group(const MvmGroup &g, int total_workgroups, int bb, bool transposed, hipStream_t s);
+// w_oc: how the tiles of the launch address their weights (MvmArgs::w_oc; the same for all of them)
+void launch_mvm_big_group(const MvmGroup &g, int total_workgroups, int bb, bool w_oc, hipStream_t s);
 void mvm_round_variant(const MvmArgs &a, int &prefetch_depth, int &weight_mode);
 
 // Fused convolution forward (unfold + noisy MVM with its bound-management rounds) for tiles of at most 32 outputs:
@@ -233,6 +248,10 @@ struct DeviceDev {
 
 struct UpdateArgs {
   float *w; // [d_size][x_size]
+  // swapped = 1: the view of a tile that stores [x_size][d_size], for the kernels that work cross-point by cross-point:
+  // everything named x here belongs to the tile's d lines and the other way round (sizes, words, planes, line values,
+  // inputs), so that "rows" are again what is contiguous in memory.  The kernels that make the lines never see it.
+  int swapped;
   int x_size, d_size, m_batch;
   const float *x;
   long x_sb, x_sj; // x element (b, j) at x[b * x_sb + j * x_sj]
@@ -296,6 +315,8 @@ void launch_update_pulsed(const UpdateArgs &a, hipStream_t s);        // coincid
 // coincidences are counted and applied in closed form with one normal draw for their summed noise
 void launch_update_aggregated(const UpdateArgs &a, int samples_per_step, hipStream_t s);
 void launch_update_implicit(const UpdateArgs &a, hipStream_t s);
+// the swapped view of a call's arguments (UpdateArgs::swapped)
+UpdateArgs update_swapped_view(const UpdateArgs &a);
 void launch_implicit_counts(const UpdateArgs &a, int32_t *counts, hipStream_t s);
 // after an update of the persistent weights: w_apparent = w_persistent + noise_std * N(0, 1) at every cross-point that
 // took a pulse (from the planes / line values of that update)
@@ -306,10 +327,22 @@ void launch_write_noise_all(float *w_apparent, const float *w_persistent, float 
                             size_t n, hipStream_t s);
 // floating-point update with the device bounds applied after every sample (x, d, strides, lr, w, dev.w_min / w_max)
 void launch_update_fp_clipped(const UpdateArgs &a, hipStream_t s);
+// How the cross-point arrays of a tile are stored: element (row i of d, column j of x) at i * x_size + j (xd = 0) or at
+// j * d_size + i (xd = 1, the layout of the reference's CUDA tiles).  Kernels that work element by element do not
+// care; those with rows or columns in their meaning take this.
+struct MatLayout {
+  int x_size, d_size, xd;
+  __host__ __device__ size_t size() const { return (size_t)x_size * (size_t)d_size; }
+  __host__ __device__ size_t at(int i, int j) const {
+    return xd ? (size_t)j * (size_t)d_size + (size_t)i : (size_t)i * (size_t)x_size + (size_t)j;
+  }
+  __host__ __device__ int col_of(size_t idx) const { return xd ? (int)(idx / (size_t)d_size) : (int)(idx % (size_t)x_size); }
+  __host__ __device__ int row_of(size_t idx) const { return xd ? (int)(idx % (size_t)d_size) : (int)(idx / (size_t)x_size); }
+};
 // ----- weight maintenance between steps (kernels_state.hip); w_min / w_max may be null (no device bounds)
 void launch_decay_device(float *w, const float *decay_scale, const float *reset_bias, const float *w_min,
-                         const float *w_max, float alpha, int bias_no_decay, int x_size, size_t n, hipStream_t s);
-void launch_decay_scalar(float *w, float scale, int bias_no_decay, int x_size, size_t n, hipStream_t s);
+                         const float *w_max, float alpha, int bias_no_decay, const MatLayout &lay, hipStream_t s);
+void launch_decay_scalar(float *w, float scale, int bias_no_decay, const MatLayout &lay, hipStream_t s);
 // rates == null: the same rate for every element
 void launch_diffuse(float *w, const float *rates, float rate, const float *w_min, const float *w_max, PhiloxKey key,
                     uint32_t call, size_t n, hipStream_t s);
@@ -318,10 +351,10 @@ void launch_diffuse(float *w, const float *rates, float rate, const float *w_min
 void launch_clip_value(float *w, const float *w_min, const float *w_max, float clip, const float *clip_dev, size_t n,
                        hipStream_t s);
 void launch_clip_value_gaussian(const float *w, size_t n, float sigma, float fixed_value, float *clip_out, hipStream_t s);
-void launch_clip_value_channel(const float *w, int x_size, int d_size, float fixed_value, float *row_max, float *clip_out,
+void launch_clip_value_channel(const float *w, const MatLayout &lay, float fixed_value, float *row_max, float *clip_out,
                                hipStream_t s);
 void launch_reset_cols(float *w, const float *reset_bias, const float *w_min, const float *w_max, float reset_std,
-                       int start_col, int n_cols, float reset_prob, int x_size, int d_size, PhiloxKey key, uint32_t call,
+                       int start_col, int n_cols, float reset_prob, const MatLayout &lay, PhiloxKey key, uint32_t call,
                        hipStream_t s);
 // prev_w_and_delta holds the weights from before an update: it becomes scale * (w - previous), w gets them back
 void launch_delta_finish(float *w, float *prev_w_and_delta, float scale, size_t n, hipStream_t s);
@@ -339,7 +372,7 @@ void launch_device_drift(float *w, float *prev, float *w0, float *t, const float
                          hipStream_t s);
 
 // per-row statistic of the first n_cols columns: largest absolute value, or sum of squares
-void launch_row_stat(const float *w, int x_size, int d_size, int n_cols, int sum_squares, float *row_out, hipStream_t s);
+void launch_row_stat(const float *w, const MatLayout &lay, int n_cols, int sum_squares, float *row_out, hipStream_t s);
 // out[0] = largest of v[0..n-1] when positive, else 1
 void launch_max_or_one(const float *v, int n, float *out, hipStream_t s);
 // WeightRemapper::apply (weight_remapper.cpp:19-190): from the row statistic in row_stat the per-row factors
@@ -348,7 +381,7 @@ struct RemapDev {
   int type, clip_if;
   float max_scale_range, max_scale_ref, row_norm, remapped_wmax;
 };
-void launch_remap(float *w, float *scales, float *row_stat, float *mul, float *div, int x_size, int d_size,
+void launch_remap(float *w, float *scales, float *row_stat, float *mul, float *div, const MatLayout &lay,
                   const RemapDev &p, hipStream_t s);
 
 // WeightModifier::apply (weight_modifier.cpp:28-224): out = modified copy of w; amax_dev == null: assumed_wmax
@@ -358,7 +391,7 @@ struct ModifierDev {
   float coeffs[8];
 };
 void launch_modify(float *out, const float *w, const ModifierDev &p, const float *amax_dev, PhiloxKey key, uint32_t call,
-                   int x_size, size_t n, hipStream_t s);
+                   const MatLayout &lay, hipStream_t s);
 
 // adds the coincidences of the batch to the per-cross-point counters: pos where the signs of x and d agree,
 // neg where they differ (kernelPulseCounter, cuda/pwu_kernel.h:1523-1627); implicit: from the line values

@@ -297,7 +297,25 @@ __device__ __forceinline__ void mvm_step_schedule() {
 #define RPU_SG_VMEM 0x020
 #define RPU_SG_DSR 0x100
 #define RPU_SG_DSW 0x200
-  if (DUAL) { // per step: 32 MFMAs, 12 LDS writes, 12 global loads, 12 LDS reads
+  if (DUAL && WMODE == 1) { // per step: 32 MFMAs, 8 LDS writes, 24 global loads, 8 LDS reads
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      RPU_SG(RPU_SG_MFMA, 1);
+      RPU_SG(RPU_SG_DSW, 1);
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      RPU_SG(RPU_SG_MFMA, 1);
+      RPU_SG(RPU_SG_VMEM, 2);
+      RPU_SG(RPU_SG_DSR, 1);
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      RPU_SG(RPU_SG_MFMA, 1);
+      RPU_SG(RPU_SG_VMEM, 1);
+    }
+    RPU_SG(RPU_SG_MFMA, 8);
+  } else if (DUAL) { // per step: 32 MFMAs, 12 LDS writes, 12 global loads, 12 LDS reads
 #pragma unroll
     for (int i = 0; i < 12; ++i) {
       RPU_SG(RPU_SG_MFMA, 1);
@@ -380,8 +398,8 @@ __device__ __forceinline__ void mvm_round_tile(const MvmArgs &a, int round, int 
   const int slot_in = tile_b * TILE + r;
   const bool b_ok = slot_in < n_act;
 
-  const long w_so = a.transposed ? 1 : a.x_size;
-  const long w_sk = a.transposed ? a.x_size : 1;
+  const long w_so = a.w_oc ? 1 : a.w_ld;
+  const long w_sk = a.w_oc ? a.w_ld : 1;
   const int K = a.K;
   // steps of 32 k-values, dealt to the waves in contiguous parts (equal parts, a multiple of PD, when PD >= 2;
   // a short contraction may leave the last waves without a step)
@@ -409,7 +427,7 @@ __device__ __forceinline__ void mvm_round_tile(const MvmArgs &a, int round, int 
     x_src[t] = xq + (long)xrow * a.k_pad + st_chunk;
     x1_src[t] = DUAL ? a.xq[1] + (long)xrow * a.k_pad + st_chunk : nullptr;
     const int o = min(tile_o * TILE + row, a.O - 1);
-    w_src[t] = a.w + (long)o * a.x_size;
+    w_src[t] = a.w + (long)o * a.w_ld;
   }
   const float *w_col = a.w + (long)(o_ok ? o_in : a.O - 1) * w_so; // mode 1: this lane's output column
 
@@ -1609,7 +1627,7 @@ __device__ __forceinline__ void mvm_big_workgroup(const MvmArgs &a, const int ro
       const int xrow = (round > 0) ? pick2(a.st.row, round & 1)[slot] : slot;
       x_src[j] = xq + (long)xrow * a.k_pad + st_col;
     }
-    if (WT == 0) w_src[j] = a.w + (long)min(tile_o * BT + row, a.O - 1) * a.x_size;
+    if (WT == 0) w_src[j] = a.w + (long)min(tile_o * BT + row, a.O - 1) * a.w_ld;
   }
   const int wt_o = tile_o * BT + (t & 31) * 4; // WT = 1: first of this thread's four outputs
 
@@ -1637,7 +1655,7 @@ __device__ __forceinline__ void mvm_big_workgroup(const MvmArgs &a, const int ro
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const int k = min(k0 + (t >> 5) + 8 * j, K - 1); // rows past K meet the zero padding of the inputs
-        const float *row = a.w + (long)k * a.x_size;
+        const float *row = a.w + (long)k * a.w_ld;
         if (wt_o + 4 <= a.O) {
           gw[j] = *reinterpret_cast<const f32x4_unaligned *>(row + wt_o);
         } else {
@@ -1848,9 +1866,9 @@ __global__ __launch_bounds__(256, 3) void k_mvm_big_short(MvmArgs a, int min_act
 __global__ __launch_bounds__(256, 2) void k_mvm_big_narrow(MvmArgs a, int min_active) {
   mvm_big_workgroup<0, 128, true, 2, true>(a, a.round, (int)blockIdx.x, min_active);
 }
-template <int BB>
+template <int WT, int BB>
 __global__ __launch_bounds__(256, 2) void k_mvm_big_lazy(MvmArgs a, int min_active) {
-  mvm_big_workgroup<0, BB, false, 2, true>(a, a.round, (int)blockIdx.x, min_active);
+  mvm_big_workgroup<WT, BB, false, 2, true>(a, a.round, (int)blockIdx.x, min_active);
 }
 
 // several tiles in one launch (round 0): a tile that is not run by this kernel has no workgroups in the table
@@ -1891,7 +1909,7 @@ __global__ __launch_bounds__(256, STOCH ? 2 : 3) void k_conv_forward(MvmArgs a, 
   const int p = (int)(sample - (long)n * c.patches);
   const float *image = c.images + (long)n * c.image_size;
   const int *idx_row = c.idx_t + (long)p * a.K;
-  const float *w_row = a.w + (long)min(r, a.O - 1) * a.x_size;
+  const float *w_row = a.w + (long)min(r, a.O - 1) * (a.w_oc ? 1 : a.w_ld); // w_oc: the lane's output column
   const int K = a.K, O = a.O;
   const int steps = ONE_STEP ? 1 : (K + 31) / 32;
   const IoDev &io = a.io;
@@ -1915,6 +1933,10 @@ __global__ __launch_bounds__(256, STOCH ? 2 : 3) void k_conv_forward(MvmArgs a, 
     }
   };
   auto weights16 = [&](int k0, float (&w)[16]) __attribute__((always_inline)) {
+    if (a.w_oc) { // rows of the stored matrix hold the outputs of one k (wave-uniform choice)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) w[i] = (k0 + i < K) ? w_row[(long)(k0 + i) * a.w_ld] : 0.0f;
+    } else
 #pragma unroll
     for (int v4 = 0; v4 < 4; ++v4) {
       const int k = k0 + 4 * v4;
@@ -2056,7 +2078,7 @@ __global__ __launch_bounds__(256, 4) void k_conv_forward_split(MvmArgs a, ConvAr
   const int p = (int)(sample - (long)n * c.patches);
   const float *image = c.images + (long)n * c.image_size;
   const int *idx_row = c.idx_t + (long)p * a.K;
-  const float *w_row = a.w + (long)min(r, a.O - 1) * a.x_size;
+  const float *w_row = a.w + (long)min(r, a.O - 1) * (a.w_oc ? 1 : a.w_ld); // w_oc: the lane's output column
   const int K = a.K, O = a.O;
   const int steps = (K + 31) / 32;
   const IoDev &io = a.io;
@@ -2079,6 +2101,10 @@ __global__ __launch_bounds__(256, 4) void k_conv_forward_split(MvmArgs a, ConvAr
     }
   };
   auto weights16 = [&](int k0, float (&w)[16]) __attribute__((always_inline)) {
+    if (a.w_oc) { // rows of the stored matrix hold the outputs of one k (wave-uniform choice)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) w[i] = (k0 + i < K) ? w_row[(long)(k0 + i) * a.w_ld] : 0.0f;
+    } else
 #pragma unroll
     for (int v4 = 0; v4 < 4; ++v4) {
       const int k = k0 + 4 * v4;
@@ -2295,8 +2321,8 @@ int mvm_k_pad(int K, bool tight) {
 
 // addressing mode of the weight operand (see k_mvm_round)
 static int weight_mode(const MvmArgs &a) {
-  if (!a.transposed && (a.x_size & 3) == 0 && (a.K & 15) == 0 && a.K >= 16 && ((((uintptr_t)a.w) & 15) == 0)) return 0;
-  if (a.transposed) return 1;
+  if (!a.w_oc && (a.w_ld & 3) == 0 && (a.K & 15) == 0 && a.K >= 16 && ((((uintptr_t)a.w) & 15) == 0)) return 0;
+  if (a.w_oc) return 1;
   return 2;
 }
 
@@ -2377,13 +2403,13 @@ int mvm_big_sample_tile(int workgroups_128, int n_cus) {
   return 10 * idle <= rounds * slots ? 128 : 64;
 }
 
-void launch_mvm_big_group(const MvmGroup &g, int total_workgroups, int bb, bool transposed, hipStream_t s) {
+void launch_mvm_big_group(const MvmGroup &g, int total_workgroups, int bb, bool w_oc, hipStream_t s) {
   const dim3 grid(total_workgroups);
   if (bb == 128) {
-    if (transposed) hipLaunchKernelGGL((k_mvm_big_group<1, 128>), grid, dim3(256), 0, s, g, 0);
+    if (w_oc) hipLaunchKernelGGL((k_mvm_big_group<1, 128>), grid, dim3(256), 0, s, g, 0);
     else hipLaunchKernelGGL((k_mvm_big_group<0, 128>), grid, dim3(256), 0, s, g, 0);
   } else {
-    if (transposed) hipLaunchKernelGGL((k_mvm_big_group<1, 64>), grid, dim3(256), 0, s, g, 0);
+    if (w_oc) hipLaunchKernelGGL((k_mvm_big_group<1, 64>), grid, dim3(256), 0, s, g, 0);
     else hipLaunchKernelGGL((k_mvm_big_group<0, 64>), grid, dim3(256), 0, s, g, 0);
   }
 }
@@ -2447,12 +2473,13 @@ void launch_mvm_round_group(const MvmGroup &g, int depth, int mode, int total_wo
 
 // all rounds from round_first on in one launch of `workgroups` workgroups (at most one per CU: they wait for each other
 // between rounds); for groups of at most MAX_GROUP tiles whose weights are not read transposed
-bool mvm_group_can_merge_rest(const MvmGroup &g, int mode) { return g.n <= MAX_GROUP && mode != 1; }
+bool mvm_group_can_merge_rest(const MvmGroup &g, int) { return g.n <= MAX_GROUP; }
 
 void launch_mvm_rest_group(const MvmGroup &g, int mode, int round_first, int rounds, int workgroups, int *seen,
                            hipStream_t s) {
   const dim3 grid(workgroups);
   if (mode == 0) hipLaunchKernelGGL(k_mvm_rest_group<0>, grid, dim3(256), 0, s, g, round_first, rounds, seen);
+  else if (mode == 1) hipLaunchKernelGGL(k_mvm_rest_group<1>, grid, dim3(256), 0, s, g, round_first, rounds, seen);
   else hipLaunchKernelGGL(k_mvm_rest_group<2>, grid, dim3(256), 0, s, g, round_first, rounds, seen);
 }
 
@@ -2461,7 +2488,7 @@ bool mvm_can_fuse_rounds(const MvmArgs &a) {
   if (a.io.perfect || a.io.bound_management == RPU_BM_NONE || a.max_rounds < 3 || a.transposed) return false;
   if (a.pre_add || a.skip_if_zero || a.nm_phase || !a.speculate || !a.rows_ahead_in_init || a.in_index) return false;
   if (!a.small_tiles_only && big_threshold(a.m_batch, a.O) > 0) return false;
-  return mvm_prefetch_depth(a.K, a.k_pad) >= 2 && weight_mode(a) != 1;
+  return mvm_prefetch_depth(a.K, a.k_pad) >= 2;
 }
 
 // Workgroups of `kernel` (256 threads, static LDS only) that the current GPU holds at once: what the occupancy query
@@ -2472,14 +2499,20 @@ template <typename K> static int resident_workgroups(K kernel) {
   return per_cu * current_device_cus();
 }
 
+// prefetch depth of the launch that runs several rounds: with the weights addressed along the outputs the deepest
+// variant takes more than half of a SIMD's registers, and these launches mostly walk empty rounds
+static int mvm_rest_depth(const MvmArgs &a) {
+  const int depth = mvm_prefetch_depth(a.K, a.k_pad);
+  return (weight_mode(a) == 1 && depth == 4) ? 2 : depth;
+}
+
 int mvm_rest_resident_limit(const MvmArgs &a) {
   static std::mutex m;
   static int limit[64][3][3] = {};
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
   const int mode = weight_mode(a);
-  if (mode == 1) return 0; // not instantiated
-  const int depth = mvm_prefetch_depth(a.K, a.k_pad);
+  const int depth = mvm_rest_depth(a);
   const int di = depth == 4 ? 2 : (depth == 2 ? 1 : 0);
   std::lock_guard<std::mutex> lock(m);
   int &v = limit[dev][di][mode];
@@ -2487,6 +2520,8 @@ int mvm_rest_resident_limit(const MvmArgs &a) {
     if (mode == 0) {
       v = depth == 4 ? resident_workgroups(k_mvm_rounds_rest<4, 0>)
                      : (depth == 2 ? resident_workgroups(k_mvm_rounds_rest<2, 0>) : resident_workgroups(k_mvm_rounds_rest<1, 0>));
+    } else if (mode == 1) { // the deepest prefetch is not built for this addressing (mvm_rest_depth)
+      v = depth == 2 ? resident_workgroups(k_mvm_rounds_rest<2, 1>) : resident_workgroups(k_mvm_rounds_rest<1, 1>);
     } else {
       v = depth == 4 ? resident_workgroups(k_mvm_rounds_rest<4, 2>)
                      : (depth == 2 ? resident_workgroups(k_mvm_rounds_rest<2, 2>) : resident_workgroups(k_mvm_rounds_rest<1, 2>));
@@ -2500,11 +2535,12 @@ int mvm_group_rest_resident_limit(int mode) {
   static std::mutex m;
   static int limit[64][3] = {};
   int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64 || mode == 1) return 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
   std::lock_guard<std::mutex> lock(m);
   int &v = limit[dev][mode];
   if (v == 0) {
-    v = mode == 0 ? resident_workgroups(k_mvm_rest_group<0>) : resident_workgroups(k_mvm_rest_group<2>);
+    v = mode == 0 ? resident_workgroups(k_mvm_rest_group<0>)
+                  : (mode == 1 ? resident_workgroups(k_mvm_rest_group<1>) : resident_workgroups(k_mvm_rest_group<2>));
     if (v == 0) v = -1;
   }
   return v > 0 ? v : 0;
@@ -2519,7 +2555,7 @@ bool mvm_can_merge_rest(const MvmArgs &a, int resident_limit) {
   // gathered input: the rows of a further round are written by k_mvm_round_tail alone, one launch per round
   if (a.pre_add || a.skip_if_zero || a.nm_phase || a.in_index) return false;
   if (!a.small_tiles_only && big_threshold(a.m_batch, a.O) > 0) return false;
-  return mvm_round_workgroups(a) <= resident_limit && weight_mode(a) != 1;
+  return mvm_round_workgroups(a) <= resident_limit;
 }
 
 void launch_mvm_dual(const MvmArgs &a_in, hipStream_t s) {
@@ -2528,7 +2564,9 @@ void launch_mvm_dual(const MvmArgs &a_in, hipStream_t s) {
   a.round = 0;
   a.dual.on = 1;
   const dim3 grid(mvm_round_workgroups(a));
-  if (weight_mode(a) == 0) hipLaunchKernelGGL(k_mvm_dual<0>, grid, dim3(256), 0, s, a);
+  const int mode = weight_mode(a);
+  if (mode == 0) hipLaunchKernelGGL(k_mvm_dual<0>, grid, dim3(256), 0, s, a);
+  else if (mode == 1) hipLaunchKernelGGL(k_mvm_dual<1>, grid, dim3(256), 0, s, a);
   else hipLaunchKernelGGL(k_mvm_dual<2>, grid, dim3(256), 0, s, a);
 }
 
@@ -2539,23 +2577,29 @@ void launch_mvm_round(const MvmArgs &a_in, hipStream_t s) {
   // the round is one launch
   if (a.round > 0 && !a.speculate) a.big_from = 0;
   if (a.big_from > 0) {
-    const bool narrow = !a.transposed && a.O <= 64; // see mvm_big_workgroup
+    // the variants below exist for the way a tile that stores [d_size][x_size] addresses its weights (forward: rows
+    // along k, backward: rows along the outputs); the other storage takes the general kernels where its case has none
+    const bool lazy = !a.transposed && !a.speculate && a.max_rounds > 1;
+    const bool narrow = !a.transposed && !a.w_oc && a.O <= 64; // see mvm_big_workgroup
     const int bb = narrow ? 128 : mvm_big_sample_tile(big_workgroups(a, 128), current_device_cus());
     const dim3 big_grid(big_workgroups(a, bb));
     const int min_active = a.round > 0 ? a.big_from : 0;
     if (narrow) {
       hipLaunchKernelGGL(k_mvm_big_narrow, big_grid, dim3(256), 0, s, a, min_active);
-    } else if (!a.transposed && !a.speculate && a.max_rounds > 1) {
-      if (bb == 128) hipLaunchKernelGGL((k_mvm_big_lazy<128>), big_grid, dim3(256), 0, s, a, min_active);
-      else hipLaunchKernelGGL((k_mvm_big_lazy<64>), big_grid, dim3(256), 0, s, a, min_active);
-    } else if (a.transposed && a.k_pad <= 2 * BKS) { // see mvm_big_workgroup, NBUF
+    } else if (lazy && !a.w_oc) {
+      if (bb == 128) hipLaunchKernelGGL((k_mvm_big_lazy<0, 128>), big_grid, dim3(256), 0, s, a, min_active);
+      else hipLaunchKernelGGL((k_mvm_big_lazy<0, 64>), big_grid, dim3(256), 0, s, a, min_active);
+    } else if (lazy) {
+      if (bb == 128) hipLaunchKernelGGL((k_mvm_big_lazy<1, 128>), big_grid, dim3(256), 0, s, a, min_active);
+      else hipLaunchKernelGGL((k_mvm_big_lazy<1, 64>), big_grid, dim3(256), 0, s, a, min_active);
+    } else if (a.transposed && a.w_oc && a.k_pad <= 2 * BKS) { // see mvm_big_workgroup, NBUF
       if (bb == 128) hipLaunchKernelGGL((k_mvm_big_short<128>), big_grid, dim3(256), 0, s, a, min_active);
       else hipLaunchKernelGGL((k_mvm_big_short<64>), big_grid, dim3(256), 0, s, a, min_active);
     } else if (bb == 128) {
-      if (a.transposed) hipLaunchKernelGGL((k_mvm_big<1, 128>), big_grid, dim3(256), 0, s, a, min_active);
+      if (a.w_oc) hipLaunchKernelGGL((k_mvm_big<1, 128>), big_grid, dim3(256), 0, s, a, min_active);
       else hipLaunchKernelGGL((k_mvm_big<0, 128>), big_grid, dim3(256), 0, s, a, min_active);
     } else {
-      if (a.transposed) hipLaunchKernelGGL((k_mvm_big<1, 64>), big_grid, dim3(256), 0, s, a, min_active);
+      if (a.w_oc) hipLaunchKernelGGL((k_mvm_big<1, 64>), big_grid, dim3(256), 0, s, a, min_active);
       else hipLaunchKernelGGL((k_mvm_big<0, 64>), big_grid, dim3(256), 0, s, a, min_active);
     }
     if (a.round == 0) return; // later rounds: whichever kernel the number of listed samples calls for
@@ -2581,6 +2625,9 @@ void launch_mvm_round(const MvmArgs &a_in, hipStream_t s) {
       if (depth == 4) RPU_LAUNCH_REST(4, 0);
       else if (depth == 2) RPU_LAUNCH_REST(2, 0);
       else RPU_LAUNCH_REST(1, 0);
+    } else if (mode == 1) {
+      if (mvm_rest_depth(a) == 2) RPU_LAUNCH_REST(2, 1);
+      else RPU_LAUNCH_REST(1, 1);
     } else {
       if (depth == 4) RPU_LAUNCH_REST(4, 2);
       else if (depth == 2) RPU_LAUNCH_REST(2, 2);

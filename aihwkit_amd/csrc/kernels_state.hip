@@ -16,19 +16,19 @@ __device__ __forceinline__ float clip_to(float w, const float *w_min, const floa
 // PulsedRPUDevice::decayWeights (rpu_pulsed_device.cpp:392-420): towards the reset bias, then the device bounds
 __global__ __launch_bounds__(256) void k_decay_device(float *w, const float *decay_scale, const float *reset_bias,
                                                        const float *w_min, const float *w_max, float alpha,
-                                                       int bias_no_decay, int x_size, size_t n) {
+                                                       int bias_no_decay, MatLayout lay, size_t n) {
   for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
     float s = 1.0f + alpha * (decay_scale[i] - 1.0f);
-    if (bias_no_decay && (int)(i % x_size) == x_size - 1) s = 1.0f;
+    if (bias_no_decay && lay.col_of(i) == lay.x_size - 1) s = 1.0f;
     const float b = reset_bias[i];
     w[i] = clip_to((w[i] - b) * s + b, w_min, w_max, i);
   }
 }
 
 // RPUSimple::decayWeights (rpu.cpp:1556-1575)
-__global__ __launch_bounds__(256) void k_decay_scalar(float *w, float scale, int bias_no_decay, int x_size, size_t n) {
+__global__ __launch_bounds__(256) void k_decay_scalar(float *w, float scale, int bias_no_decay, MatLayout lay, size_t n) {
   for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
-    if (!(bias_no_decay && (int)(i % x_size) == x_size - 1)) w[i] *= scale;
+    if (!(bias_no_decay && lay.col_of(i) == lay.x_size - 1)) w[i] *= scale;
   }
 }
 
@@ -112,11 +112,10 @@ __global__ __launch_bounds__(1024) void k_clip_value_gaussian(const float *w, si
 }
 
 // AverageChannelMax (weight_clipper.cpp:38-66): mean over the rows of the largest absolute weight of a row
-__global__ __launch_bounds__(256) void k_row_abs_max(const float *w, int x_size, float *row_max) {
+__global__ __launch_bounds__(256) void k_row_abs_max(const float *w, MatLayout lay, float *row_max) {
   __shared__ float sh[4];
-  const float *row = w + (size_t)blockIdx.x * x_size;
   float m = 0.0f;
-  for (int j = threadIdx.x; j < x_size; j += blockDim.x) m = fmaxf(m, fabsf(row[j]));
+  for (int j = threadIdx.x; j < lay.x_size; j += blockDim.x) m = fmaxf(m, fabsf(w[lay.at((int)blockIdx.x, j)]));
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off));
   if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = m;
@@ -141,13 +140,13 @@ __global__ __launch_bounds__(256) void k_clip_value_channel(const float *row_max
 // (wrapping around) are set to the reset bias plus noise, each element with probability reset_prob
 __global__ __launch_bounds__(256) void k_reset_cols(float *w, const float *reset_bias, const float *w_min,
                                                      const float *w_max, float reset_std, int start_col, int n_cols,
-                                                     float reset_prob, int x_size, int d_size, PhiloxKey key,
-                                                     uint32_t call) {
-  const size_t total = (size_t)d_size * n_cols;
+                                                     float reset_prob, MatLayout lay, PhiloxKey key, uint32_t call) {
+  const int x_size = lay.x_size;
+  const size_t total = (size_t)lay.d_size * n_cols;
   for (size_t idx = blockIdx.x * (size_t)blockDim.x + threadIdx.x; idx < total; idx += (size_t)gridDim.x * blockDim.x) {
     const int i = (int)(idx / n_cols);
     const int j = (start_col + (int)(idx % n_cols)) % x_size;
-    const size_t k = (size_t)i * x_size + j;
+    const size_t k = lay.at(i, j);
     float z[4];
     philox_normal4((uint32_t)j, (uint32_t)i, call, RNG_RESET, key, z);
     if (reset_prob < 1.0f) {
@@ -218,19 +217,20 @@ __global__ __launch_bounds__(256) void k_device_drift(float *w, float *prev, flo
 }
 
 // one workgroup per row: largest absolute value (0), sum of squares (1) or sum (2) of the first n_cols columns
-__global__ __launch_bounds__(256) void k_row_stat(const float *w, int x_size, int n_cols, int sum_squares,
+__global__ __launch_bounds__(256) void k_row_stat(const float *w, MatLayout lay, int n_cols, int sum_squares,
                                                    float *row_out) {
   __shared__ float sh[4];
-  const float *row = w + (size_t)blockIdx.x * x_size;
+  const float *row = w + lay.at((int)blockIdx.x, 0);
+  const size_t sj = lay.xd ? (size_t)lay.d_size : 1; // distance between the columns of a row
   float m = 0.0f;
   if (sum_squares == 2) {
-    for (int j = threadIdx.x; j < n_cols; j += blockDim.x) m += row[j];
+    for (int j = threadIdx.x; j < n_cols; j += blockDim.x) m += row[j * sj];
     m = block_sum(m, sh);
   } else if (sum_squares) {
-    for (int j = threadIdx.x; j < n_cols; j += blockDim.x) m = __builtin_fmaf(row[j], row[j], m);
+    for (int j = threadIdx.x; j < n_cols; j += blockDim.x) m = __builtin_fmaf(row[j * sj], row[j * sj], m);
     m = block_sum(m, sh);
   } else {
-    for (int j = threadIdx.x; j < n_cols; j += blockDim.x) m = fmaxf(m, fabsf(row[j]));
+    for (int j = threadIdx.x; j < n_cols; j += blockDim.x) m = fmaxf(m, fabsf(row[j * sj]));
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off));
     if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = m;
@@ -311,9 +311,9 @@ __global__ __launch_bounds__(256) void k_remap_factors(float *scales, const floa
   }
 }
 
-__global__ __launch_bounds__(256) void k_remap_apply(float *w, const float *mul, const float *div, int x_size, size_t n) {
+__global__ __launch_bounds__(256) void k_remap_apply(float *w, const float *mul, const float *div, MatLayout lay, size_t n) {
   for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
-    const size_t r = i / x_size;
+    const int r = lay.row_of(i);
     w[i] = w[i] * mul[r] / div[r];
   }
 }
@@ -327,11 +327,11 @@ __device__ __forceinline__ float discretize(float v, float res, int sto_round, f
 // WeightModifier::apply (weight_modifier.cpp:28-224).  One Philox call per element: words 0, 1 give the normal
 // draw, word 2 the stochastic rounding, word 3 the dropped connections.
 __global__ __launch_bounds__(256) void k_modify(float *out, const float *w, ModifierDev p, const float *amax_dev,
-                                                 PhiloxKey key, uint32_t call, int x_size, size_t n) {
+                                                 PhiloxKey key, uint32_t call, MatLayout lay, size_t n) {
   const float amax = amax_dev ? *amax_dev : p.assumed_wmax;
   for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
     float v = w[i];
-    if (p.copy_last_column && (int)(i % x_size) == x_size - 1) {
+    if (p.copy_last_column && lay.col_of(i) == lay.x_size - 1) {
       out[i] = v;
       continue;
     }
@@ -397,13 +397,15 @@ int grid_for(size_t n) {
 } // namespace
 
 void launch_decay_device(float *w, const float *decay_scale, const float *reset_bias, const float *w_min,
-                         const float *w_max, float alpha, int bias_no_decay, int x_size, size_t n, hipStream_t s) {
+                         const float *w_max, float alpha, int bias_no_decay, const MatLayout &lay, hipStream_t s) {
+  const size_t n = lay.size();
   hipLaunchKernelGGL(k_decay_device, dim3(grid_for(n)), dim3(256), 0, s, w, decay_scale, reset_bias, w_min, w_max, alpha,
-                     bias_no_decay, x_size, n);
+                     bias_no_decay, lay, n);
 }
 
-void launch_decay_scalar(float *w, float scale, int bias_no_decay, int x_size, size_t n, hipStream_t s) {
-  hipLaunchKernelGGL(k_decay_scalar, dim3(grid_for(n)), dim3(256), 0, s, w, scale, bias_no_decay, x_size, n);
+void launch_decay_scalar(float *w, float scale, int bias_no_decay, const MatLayout &lay, hipStream_t s) {
+  const size_t n = lay.size();
+  hipLaunchKernelGGL(k_decay_scalar, dim3(grid_for(n)), dim3(256), 0, s, w, scale, bias_no_decay, lay, n);
 }
 
 void launch_diffuse(float *w, const float *rates, float rate, const float *w_min, const float *w_max, PhiloxKey key,
@@ -420,17 +422,17 @@ void launch_clip_value_gaussian(const float *w, size_t n, float sigma, float fix
   hipLaunchKernelGGL(k_clip_value_gaussian, dim3(1), dim3(1024), 0, s, w, n, sigma, fixed_value, clip_out);
 }
 
-void launch_clip_value_channel(const float *w, int x_size, int d_size, float fixed_value, float *row_max, float *clip_out,
+void launch_clip_value_channel(const float *w, const MatLayout &lay, float fixed_value, float *row_max, float *clip_out,
                                hipStream_t s) {
-  hipLaunchKernelGGL(k_row_abs_max, dim3(d_size), dim3(256), 0, s, w, x_size, row_max);
-  hipLaunchKernelGGL(k_clip_value_channel, dim3(1), dim3(256), 0, s, row_max, d_size, fixed_value, clip_out);
+  hipLaunchKernelGGL(k_row_abs_max, dim3(lay.d_size), dim3(256), 0, s, w, lay, row_max);
+  hipLaunchKernelGGL(k_clip_value_channel, dim3(1), dim3(256), 0, s, row_max, lay.d_size, fixed_value, clip_out);
 }
 
 void launch_reset_cols(float *w, const float *reset_bias, const float *w_min, const float *w_max, float reset_std,
-                       int start_col, int n_cols, float reset_prob, int x_size, int d_size, PhiloxKey key, uint32_t call,
+                       int start_col, int n_cols, float reset_prob, const MatLayout &lay, PhiloxKey key, uint32_t call,
                        hipStream_t s) {
-  hipLaunchKernelGGL(k_reset_cols, dim3(grid_for((size_t)d_size * n_cols)), dim3(256), 0, s, w, reset_bias, w_min, w_max,
-                     reset_std, start_col, n_cols, reset_prob, x_size, d_size, key, call);
+  hipLaunchKernelGGL(k_reset_cols, dim3(grid_for((size_t)lay.d_size * n_cols)), dim3(256), 0, s, w, reset_bias, w_min, w_max,
+                     reset_std, start_col, n_cols, reset_prob, lay, key, call);
 }
 
 void launch_device_drift(float *w, float *prev, float *w0, float *t, const float *nu, const float *w_min,
@@ -440,25 +442,26 @@ void launch_device_drift(float *w, float *prev, float *w0, float *t, const float
                      key, call, n);
 }
 
-void launch_row_stat(const float *w, int x_size, int d_size, int n_cols, int sum_squares, float *row_out, hipStream_t s) {
-  hipLaunchKernelGGL(k_row_stat, dim3(d_size), dim3(256), 0, s, w, x_size, n_cols, sum_squares, row_out);
+void launch_row_stat(const float *w, const MatLayout &lay, int n_cols, int sum_squares, float *row_out, hipStream_t s) {
+  hipLaunchKernelGGL(k_row_stat, dim3(lay.d_size), dim3(256), 0, s, w, lay, n_cols, sum_squares, row_out);
 }
 
 void launch_max_or_one(const float *v, int n, float *out, hipStream_t s) {
   hipLaunchKernelGGL(k_max_or_one, dim3(1), dim3(256), 0, s, v, n, out);
 }
 
-void launch_remap(float *w, float *scales, float *row_stat, float *mul, float *div, int x_size, int d_size,
+void launch_remap(float *w, float *scales, float *row_stat, float *mul, float *div, const MatLayout &lay,
                   const RemapDev &p, hipStream_t s) {
-  launch_row_stat(w, x_size, d_size, x_size, p.type == RPU_REMAP_CHANNELWISE_NORM ? 1 : 0, row_stat, s);
-  hipLaunchKernelGGL(k_remap_factors, dim3(1), dim3(256), 0, s, scales, row_stat, mul, div, d_size, p);
-  const size_t n = (size_t)x_size * d_size;
-  hipLaunchKernelGGL(k_remap_apply, dim3(grid_for(n)), dim3(256), 0, s, w, mul, div, x_size, n);
+  launch_row_stat(w, lay, lay.x_size, p.type == RPU_REMAP_CHANNELWISE_NORM ? 1 : 0, row_stat, s);
+  hipLaunchKernelGGL(k_remap_factors, dim3(1), dim3(256), 0, s, scales, row_stat, mul, div, lay.d_size, p);
+  const size_t n = lay.size();
+  hipLaunchKernelGGL(k_remap_apply, dim3(grid_for(n)), dim3(256), 0, s, w, mul, div, lay, n);
 }
 
 void launch_modify(float *out, const float *w, const ModifierDev &p, const float *amax_dev, PhiloxKey key, uint32_t call,
-                   int x_size, size_t n, hipStream_t s) {
-  hipLaunchKernelGGL(k_modify, dim3(grid_for(n)), dim3(256), 0, s, out, w, p, amax_dev, key, call, x_size, n);
+                   const MatLayout &lay, hipStream_t s) {
+  const size_t n = lay.size();
+  hipLaunchKernelGGL(k_modify, dim3(grid_for(n)), dim3(256), 0, s, out, w, p, amax_dev, key, call, lay, n);
 }
 
 void launch_write_noise_all(float *w_apparent, const float *w_persistent, float noise_std, PhiloxKey key, uint32_t call,

@@ -315,11 +315,14 @@ __global__ __launch_bounds__(256) void k_update_implicit_lines(UpdateArgs a) {
 // signed coincidence count of cross-point (i, j) for sample b from the stored line values:
 // rintf((dv * BL) * xv) (generateCoincidencesDetI, dense_bit_line_maker.cpp:237-264), or with mean counts
 // rintf((d_count / BL) * x_count) (generateCoincidences, :176-201)
+// (i, j) are the row and column of the stored matrix: with the swapped view, row i is an x line of the tile and the
+// arrays named d hold the x values, and the product keeps the reference's operand order
 __device__ __forceinline__ int implicit_count(const UpdateArgs &a, int b, int i, int j) {
-  float dc = a.d_val[(long)b * a.d_size + i];
+  const float row_val = a.d_val[(long)b * a.d_size + i], col_val = a.x_val[(long)b * a.x_size + j];
+  float dc = a.swapped ? col_val : row_val;
   if (dc == 0.0f) return 0;
   if (a.up.pulse_type != RPU_PULSE_MEAN_COUNT) dc *= (float)a.bl[b];
-  return (int)rintf(dc * a.x_val[(long)b * a.x_size + j]);
+  return (int)rintf(dc * (a.swapped ? row_val : col_val));
 }
 
 // ---- device steps ------------------------------------------------------------------------------
@@ -1215,8 +1218,10 @@ __global__ __launch_bounds__(256) void k_update_fp_clipped(UpdateArgs a) {
   float w = a.w[cell];
   const float lo = a.dev.w_min[cell], hi = a.dev.w_max[cell];
   for (int b = 0; b < a.m_batch; ++b) {
-    const float di = -a.lr * a.d[(long)b * a.d_sb + (long)i * a.d_si]; // wave-uniform
-    w = w + di * a.x[(long)b * a.x_sb + (long)j * a.x_sj];
+    const float row_val = a.d[(long)b * a.d_sb + (long)i * a.d_si]; // wave-uniform
+    const float col_val = a.x[(long)b * a.x_sb + (long)j * a.x_sj];
+    const float di = -a.lr * (a.swapped ? col_val : row_val); // the tile's d value, whichever side holds it
+    w = w + di * (a.swapped ? row_val : col_val);
     w = fmaxf(fminf(w, hi), lo);
   }
   a.w[cell] = w;
@@ -1441,6 +1446,19 @@ void ensure_update_tables() {
     throw RpuError("Upload of the noise quantile table failed.");
   }
   done[device] = true;
+}
+
+UpdateArgs update_swapped_view(const UpdateArgs &a) {
+  UpdateArgs v = a;
+  v.swapped = a.swapped ? 0 : 1;
+  std::swap(v.x_size, v.d_size);
+  std::swap(v.x, v.d);
+  std::swap(v.x_sb, v.d_sb);
+  std::swap(v.x_sj, v.d_si);
+  std::swap(v.x_words, v.d_words);
+  std::swap(v.x_planes, v.d_planes);
+  std::swap(v.x_val, v.d_val);
+  return v;
 }
 
 void launch_update_implicit(const UpdateArgs &a, hipStream_t s) {

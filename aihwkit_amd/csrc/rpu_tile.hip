@@ -263,6 +263,49 @@ struct Tile {
   float *shared_xd = nullptr;
   float *delta_xd = nullptr;
   DevBuf<float> d_delta_own;
+  // Zero-copy form of the same binding (RPUCudaSimple::setSharedWeights, cuda/rpucuda.cu:322-334): the caller's
+  // [x_size][d_size] tensor IS the weight matrix, and every other cross-point array of the tile (device parameters,
+  // drift clocks, modified weights, inference arrays) is kept in that layout too, transposed once when the tensor is
+  // bound.  The kernels then read the weights with the roles of rows and columns exchanged: forward addresses them as
+  // backward does on a row-major tile and the other way round (MvmArgs::w_oc), the update kernels see x and d swapped.
+  // Plain tiles take this form; transfer compounds, write noise, pulse counters and the analog terms before the ADC
+  // keep the mirror above.
+  bool xd = false;
+  int w_ld() const { return xd ? D : X; } // row length of the stored matrices
+  MatLayout layout() const { return MatLayout{X, D, xd ? 1 : 0}; }
+  // Host matrices are row-major [D][X] on every interface; the device copies follow the tile's storage.
+  void upload_mat(float *dst_dev, const float *src_host) {
+    const size_t bytes = size() * sizeof(float);
+    if (!xd) {
+      RPU_HIP_CHECK(hipMemcpy(dst_dev, src_host, bytes, hipMemcpyHostToDevice));
+      return;
+    }
+    std::vector<float> t(size());
+    for (int i = 0; i < D; ++i)
+      for (int j = 0; j < X; ++j) t[(size_t)j * D + i] = src_host[(size_t)i * X + j];
+    RPU_HIP_CHECK(hipMemcpy(dst_dev, t.data(), bytes, hipMemcpyHostToDevice));
+  }
+  void download_mat(float *dst_host, const float *src_dev) const {
+    const size_t bytes = size() * sizeof(float);
+    if (!xd) {
+      RPU_HIP_CHECK(hipMemcpy(dst_host, src_dev, bytes, hipMemcpyDeviceToHost));
+      return;
+    }
+    std::vector<float> t(size());
+    RPU_HIP_CHECK(hipMemcpy(t.data(), src_dev, bytes, hipMemcpyDeviceToHost));
+    for (int i = 0; i < D; ++i)
+      for (int j = 0; j < X; ++j) dst_host[(size_t)i * X + j] = t[(size_t)j * D + i];
+  }
+  // row-major [D][X] device matrix -> [X][D] in place (through a temporary), on the last stream, waited for
+  void to_xd_in_place(DevBuf<float> &b) {
+    if (!b.p || b.n < size()) return;
+    DevBuf<float> tmp;
+    tmp.ensure(size());
+    launch_transpose(b.p, tmp.p, D, X, last_stream);
+    RPU_HIP_CHECK(hipMemcpyAsync(b.p, tmp.p, size() * sizeof(float), hipMemcpyDeviceToDevice, last_stream));
+    RPU_HIP_CHECK(hipStreamSynchronize(last_stream));
+    tmp.release();
+  }
   // hardware-aware training: the modified copy of the weights that forward / backward contract with, scratch of
   // the remapper ([3 D + 1]: row statistic, multiplier, divisor, one scalar), the drift clock per weight and the
   // pulse counters [2][size]
@@ -368,6 +411,7 @@ struct Tile {
     delta_w = nullptr;
     shared_xd = nullptr;
     delta_xd = nullptr;
+    xd = false;
     d_delta_own.release();
     n_pre.release(); n_s1.release(); n_s2.release(); n_s3.release(); n_rows.release(); n_absw.release();
     n_sumsq.release();
@@ -422,15 +466,16 @@ struct Tile {
     nu_valid = false;
     if (!dev.pulsed()) return;
     const size_t n = size(), bytes = n * sizeof(float);
+    (void)bytes;
     d_wmax.ensure(n); d_wmin.ensure(n); d_sup.ensure(n); d_sdown.ensure(n);
-    RPU_HIP_CHECK(hipMemcpy(d_wmax.p, arr.w_max.data(), bytes, hipMemcpyHostToDevice));
-    RPU_HIP_CHECK(hipMemcpy(d_wmin.p, arr.w_min.data(), bytes, hipMemcpyHostToDevice));
-    RPU_HIP_CHECK(hipMemcpy(d_sup.p, arr.scale_up.data(), bytes, hipMemcpyHostToDevice));
-    RPU_HIP_CHECK(hipMemcpy(d_sdown.p, arr.scale_down.data(), bytes, hipMemcpyHostToDevice));
+    upload_mat(d_wmax.p, arr.w_max.data());
+    upload_mat(d_wmin.p, arr.w_min.data());
+    upload_mat(d_sup.p, arr.scale_up.data());
+    upload_mat(d_sdown.p, arr.scale_down.data());
     if (dev.linear()) {
       d_slup.ensure(n); d_sldown.ensure(n);
-      RPU_HIP_CHECK(hipMemcpy(d_slup.p, arr.slope_up.data(), bytes, hipMemcpyHostToDevice));
-      RPU_HIP_CHECK(hipMemcpy(d_sldown.p, arr.slope_down.data(), bytes, hipMemcpyHostToDevice));
+      upload_mat(d_slup.p, arr.slope_up.data());
+      upload_mat(d_sldown.p, arr.slope_down.data());
     }
   }
 
@@ -514,8 +559,9 @@ struct Tile {
     const int O = transposed ? X : D;
     ensure_mvm_scratch(B);
     MvmArgs a{};
-    a.w = w_other ? w_other : wdev(); a.x_size = X; a.d_size = D; a.m_batch = B; a.K = K; a.O = O;
+    a.x_size = X; a.d_size = D; a.m_batch = B; a.K = K; a.O = O;
     a.transposed = transposed ? 1 : 0;
+    mvm_set_weights(a, w_other ? w_other : wdev(), w_ld(), xd);
     a.io = io_dev(io);
     a.alpha = io.p.out_scale; a.beta = 0.0f;
     a.key = key(); a.call = call++;
@@ -610,8 +656,9 @@ struct Tile {
       const auto contract = [&](const float *w, int mode, float *dst) {
         if (mode != 3) launch_side_rows(xin, n_rows.p, B, a.k_pad, a.K, mode, 0, skip, s);
         MvmArgs g{};
-        g.w = w; g.x_size = X; g.d_size = D; g.m_batch = B; g.K = a.K; g.O = a.O; g.k_pad = a.k_pad;
+        g.x_size = X; g.d_size = D; g.m_batch = B; g.K = a.K; g.O = a.O; g.k_pad = a.k_pad;
         g.transposed = a.transposed;
+        mvm_set_weights(g, w, w_ld(), xd);
         g.xq[0] = mode != 3 ? n_rows.p : const_cast<float *>(xin); g.xq[1] = nullptr;
         g.out = dst; g.out_sb = a.O; g.out_so = 1;
         g.io = a.io; g.io.perfect = 1;
@@ -623,7 +670,7 @@ struct Tile {
       };
       if (noisy && io.p.w_noise_type == 1) {
         n_sumsq.ensure((size_t)B);
-        launch_row_stat(xin, a.k_pad, B, a.K, 1, n_sumsq.p, s);
+        launch_row_stat(xin, MatLayout{a.k_pad, B, 0}, a.K, 1, n_sumsq.p, s);
       } else if (noisy) {
         n_s1.ensure(out_n);
         contract(absw_pass, 0, n_s1.p);
@@ -647,7 +694,7 @@ struct Tile {
           p.v_offset = line_values(dir, 0, io.v_offset);
           if (io.p.v_offset_w_min != 0.0f) {
             n_xsum.ensure((size_t)B);
-            launch_row_stat(xin, a.k_pad, B, a.K, 2, n_xsum.p, s);
+            launch_row_stat(xin, MatLayout{a.k_pad, B, 0}, a.K, 2, n_xsum.p, s);
             p.x_accum = n_xsum.p;
           }
         }
@@ -914,7 +961,7 @@ struct Tile {
     launch_update_planes(a, s);
     prof_mark(s, "update_planes");
     if (dev.p.count_pulses) count_pulses(a, false, s);
-    launch_update_pulsed(a, s);
+    launch_update_pulsed(cross_point_view(a), s);
     prof_mark(s, "update_pulsed");
     if (persistent()) launch_write_noise_touched(a, d_w.p, d_wp.p, dev.scaled_write_noise(), false, s);
     RPU_HIP_CHECK(hipGetLastError());
@@ -961,7 +1008,7 @@ struct Tile {
       a.x = xin; a.x_sb = x_sb; a.x_sj = x_sj; a.d = d; a.d_sb = d_sb; a.d_si = d_si;
       a.dev.w_max = d_wmax.p; a.dev.w_min = d_wmin.p;
       prof_begin(s);
-      launch_update_fp_clipped(a, s);
+      launch_update_fp_clipped(cross_point_view(a), s);
       prof_mark(s, "update_fp_clipped");
       refresh_shown_weights(s); // clipWeights ends with applyUpdateWriteNoise (rpu_pulsed_device.cpp:448-467)
       RPU_HIP_CHECK(hipGetLastError());
@@ -973,11 +1020,13 @@ struct Tile {
     if (fp_update) {
       // W += -lr * d^T x as a contraction over the batch (rpu.cpp:624-634): "weights" = d, K = batch
       MvmArgs a{};
-      a.w = d; a.transposed = d_trans ? 0 : 1; // element (o = i, k = b): d[b * D + i] or d[i * B + b]
+      a.transposed = d_trans ? 0 : 1; // element (o = i, k = b): d[b * D + i] or d[i * B + b]
       a.x_size = d_trans ? B : D; a.d_size = d_trans ? D : B;
+      mvm_set_weights(a, d, a.x_size, false);
       a.K = B; a.O = D; a.m_batch = X;
       a.in = xin; a.in_sb = x_sj; a.in_sk = x_sb; // "sample" = column j of x, contraction over b
-      a.out = delta_w ? delta_w : d_w.p; a.out_sb = 1; a.out_so = X;
+      a.out = delta_w ? delta_w : d_w.p; // W[i][j] of sample j, output i
+      a.out_sb = xd ? D : 1; a.out_so = xd ? 1 : X;
       a.io = io_dev(fio); a.io.perfect = 1;
       a.alpha = delta_w ? 1.0f : -lr; a.beta = delta_w ? 0.0f : 1.0f; a.round = 0;
       a.key = key(); a.call = call++;
@@ -1010,10 +1059,11 @@ struct Tile {
   void ensure_state_params() {
     if (!dev.pulsed() || state_params_valid) return;
     const size_t n = size(), bytes = n * sizeof(float);
+    (void)bytes;
     d_decay.ensure(n); d_diff.ensure(n); d_rbias.ensure(n);
-    RPU_HIP_CHECK(hipMemcpy(d_decay.p, arr.decay_scale.data(), bytes, hipMemcpyHostToDevice));
-    RPU_HIP_CHECK(hipMemcpy(d_diff.p, arr.diffusion_rate.data(), bytes, hipMemcpyHostToDevice));
-    RPU_HIP_CHECK(hipMemcpy(d_rbias.p, arr.reset_bias.data(), bytes, hipMemcpyHostToDevice));
+    upload_mat(d_decay.p, arr.decay_scale.data());
+    upload_mat(d_diff.p, arr.diffusion_rate.data());
+    upload_mat(d_rbias.p, arr.reset_bias.data());
     state_params_valid = true;
   }
 
@@ -1028,12 +1078,12 @@ struct Tile {
     check_maintenance("decay_weights");
     if (dev.pulsed()) {
       ensure_state_params();
-      launch_decay_device(wp_dev(), d_decay.p, d_rbias.p, d_wmin.p, d_wmax.p, alpha, bias_no_decay ? 1 : 0, X, size(), s);
+      launch_decay_device(wp_dev(), d_decay.p, d_rbias.p, d_wmin.p, d_wmax.p, alpha, bias_no_decay ? 1 : 0, layout(), s);
       refresh_shown_weights(s);
     } else {
       const float rate = dev.p.lifetime > 1.0f ? 1.0f / dev.p.lifetime : 0.0f;
       const float scale = 1.0f - alpha * rate;
-      if (scale > 0.0f && scale < 1.0f) launch_decay_scalar(d_w.p, scale, bias_no_decay ? 1 : 0, X, size(), s);
+      if (scale > 0.0f && scale < 1.0f) launch_decay_scalar(d_w.p, scale, bias_no_decay ? 1 : 0, layout(), s);
     }
     RPU_HIP_CHECK(hipGetLastError());
     last_stream = s;
@@ -1067,7 +1117,7 @@ struct Tile {
       if (dev.pulsed()) throw RpuError("Sophisticated clipping is NOT implemented for most training devices");
       s_clip.ensure(1 + (size_t)D);
       if (type == RPU_CLIP_LAYER_GAUSSIAN) launch_clip_value_gaussian(d_w.p, size(), sigma, fixed_value, s_clip.p, s);
-      else launch_clip_value_channel(d_w.p, X, D, fixed_value, s_clip.p + 1, s_clip.p, s);
+      else launch_clip_value_channel(d_w.p, layout(), fixed_value, s_clip.p + 1, s_clip.p, s);
       launch_clip_value(d_w.p, nullptr, nullptr, 0.0f, s_clip.p, size(), s);
     } else {
       throw RpuError("Clipping type not implemented.");
@@ -1085,11 +1135,11 @@ struct Tile {
     if (n == 0) return;
     if (dev.pulsed()) {
       ensure_state_params();
-      launch_reset_cols(wp_dev(), d_rbias.p, d_wmin.p, d_wmax.p, dev.p.reset_std, start_col, n, reset_prob, X, D, key(),
+      launch_reset_cols(wp_dev(), d_rbias.p, d_wmin.p, d_wmax.p, dev.p.reset_std, start_col, n, reset_prob, layout(), key(),
                         call++, s);
       refresh_shown_weights(s);
     } else {
-      launch_reset_cols(d_w.p, nullptr, nullptr, nullptr, dev.p.reset_std, start_col, n, reset_prob, X, D, key(), call++, s);
+      launch_reset_cols(d_w.p, nullptr, nullptr, nullptr, dev.p.reset_std, start_col, n, reset_prob, layout(), key(), call++, s);
     }
     RPU_HIP_CHECK(hipGetLastError());
     last_stream = s;
@@ -1107,7 +1157,7 @@ struct Tile {
     const bool per_device = arr.drift_nu.size() == n;
     if (per_device && !nu_valid) {
       d_nu.ensure(n);
-      RPU_HIP_CHECK(hipMemcpy(d_nu.p, arr.drift_nu.data(), n * sizeof(float), hipMemcpyHostToDevice));
+      upload_mat(d_nu.p, arr.drift_nu.data());
       nu_valid = true;
     }
     if (!dr_prev.p) {
@@ -1157,7 +1207,7 @@ struct Tile {
     RemapDev p{};
     p.type = q.type; p.clip_if = q.clip_if; p.max_scale_range = q.max_scale_range; p.max_scale_ref = q.max_scale_ref;
     p.row_norm = q.row_norm; p.remapped_wmax = q.remapped_wmax;
-    launch_remap(d_w.p, scales_dev, s_rowstat.p, s_rowstat.p + D, s_rowstat.p + 2 * (size_t)D, X, D, p, s);
+    launch_remap(d_w.p, scales_dev, s_rowstat.p, s_rowstat.p + D, s_rowstat.p + 2 * (size_t)D, layout(), p, s);
     RPU_HIP_CHECK(hipGetLastError());
     last_stream = s;
   }
@@ -1182,11 +1232,11 @@ struct Tile {
     const float *amax_dev = nullptr;
     if (q.rel_to_actual_wmax && q.type != RPU_MODIFIER_COPY) {
       s_rowstat.ensure(3 * (size_t)D + 1);
-      launch_row_stat(d_w.p, X, D, q.copy_last_column ? X - 1 : X, 0, s_rowstat.p, s);
+      launch_row_stat(d_w.p, layout(), q.copy_last_column ? X - 1 : X, 0, s_rowstat.p, s);
       launch_max_or_one(s_rowstat.p, D, s_rowstat.p + 3 * (size_t)D, s);
       amax_dev = s_rowstat.p + 3 * (size_t)D;
     }
-    launch_modify(d_fbw.p, d_w.p, p, amax_dev, key(), call++, X, n, s);
+    launch_modify(d_fbw.p, d_w.p, p, amax_dev, key(), call++, layout(), s);
     RPU_HIP_CHECK(hipGetLastError());
     last_stream = s;
   }
@@ -1205,6 +1255,7 @@ struct Tile {
   void set_shared_weights(float *w_dev) {
     check_maintenance("set_shared_weights");
     if (!w_dev) throw RpuError("Null device pointer.");
+    if (xd || shared_xd) throw RpuError("The tile already uses an [x_size, d_size] shared weight tensor.");
     if (w_dev == d_w.p) return;
     sync_last();
     RPU_HIP_CHECK(hipMemcpy(w_dev, d_w.p, size() * sizeof(float), hipMemcpyDeviceToDevice));
@@ -1214,21 +1265,46 @@ struct Tile {
   // RPUSimple::setDeltaWeights (rpu.cpp:1459-1481): null ends the mode
   void set_delta_weights(float *dw_dev) {
     if (dw_dev) check_maintenance("set_delta_weights");
+    if (dw_dev && xd) throw RpuError("A tile with [x_size, d_size] weights takes its delta weights in that layout.");
     delta_w = dw_dev;
     delta_xd = nullptr;
   }
 
-  // RPUCudaSimple::setSharedWeights (cuda/rpucuda.cu:322-334) with the CUDA tiles' [x_size][d_size] layout: the
-  // tile's weights are copied into the tensor, which mirrors them from then on
+  // RPUCudaSimple::setSharedWeights (cuda/rpucuda.cu:322-334) with the CUDA tiles' [x_size][d_size] layout.  A plain
+  // tile takes the tensor as its weight matrix (see `xd`); the kinds of tile named there keep their row-major matrix
+  // and mirror it into the tensor around every call.
+  bool takes_xd_storage() const {
+    return !is_transfer() && !persistent() && !dev.p.count_pulses && !has_pre_adc_terms(fio) && !has_pre_adc_terms(bio) &&
+           !d_cnt.p && !delta_w;
+  }
   void set_shared_weights_xd(float *w_xd_dev) {
     check_maintenance("set_shared_weights");
     if (!w_xd_dev) throw RpuError("Null device pointer.");
+    if (xd) { // bound already: the weights move to the new tensor
+      if (w_xd_dev == d_w.p) return;
+      sync_last();
+      RPU_HIP_CHECK(hipMemcpy(w_xd_dev, d_w.p, size() * sizeof(float), hipMemcpyDeviceToDevice));
+      d_w.adopt(w_xd_dev, size());
+      return;
+    }
     if (!d_w.owned) throw RpuError("The tile already uses a row-major shared weight buffer.");
     sync_last();
     launch_transpose(d_w.p, w_xd_dev, D, X, last_stream);
     RPU_HIP_CHECK(hipGetLastError());
     RPU_HIP_CHECK(hipStreamSynchronize(last_stream));
-    shared_xd = w_xd_dev;
+    if (shared_xd || !takes_xd_storage()) {
+      shared_xd = w_xd_dev;
+      return;
+    }
+    d_w.adopt(w_xd_dev, size());
+    for (DevBuf<float> *b : {&d_wmax, &d_wmin, &d_sup, &d_sdown, &d_slup, &d_sldown, &d_nu, &dr_prev, &dr_w0, &dr_t, &d_fbw,
+                             &i_ref, &i_prog, &i_nu_plus, &i_nu_minus}) {
+      to_xd_in_place(*b);
+    }
+    if (state_params_valid) {
+      for (DevBuf<float> *b : {&d_decay, &d_diff, &d_rbias}) to_xd_in_place(*b);
+    }
+    xd = true;
   }
   void set_delta_weights_xd(float *dw_xd_dev) {
     if (!dw_xd_dev) {
@@ -1236,6 +1312,11 @@ struct Tile {
       return;
     }
     check_maintenance("set_delta_weights");
+    if (xd) { // the tile's own layout: the buffer is written in place
+      delta_w = dw_xd_dev;
+      delta_xd = nullptr;
+      return;
+    }
     d_delta_own.ensure(size());
     delta_w = d_delta_own.p;
     delta_xd = dw_xd_dev;
@@ -1318,6 +1399,10 @@ struct Tile {
     return a;
   }
 
+  // the arguments of a pulsed update as the kernels that work cross-point by cross-point take them: as they are on a
+  // row-major tile, with x and d exchanged on one that stores [x_size][d_size] (UpdateArgs::swapped)
+  UpdateArgs cross_point_view(const UpdateArgs &a) const { return xd ? update_swapped_view(a) : a; }
+
   // what the debug hooks read after a pulsed update
   void note_pulsed_update(const UpdateArgs &a, int B, int wps, int pulse_type, hipStream_t s) {
     last_stream = s;
@@ -1346,17 +1431,17 @@ struct Tile {
       prof_mark(s, "update_lines");
       if (counting) count_pulses(a, false, s);
       if (update_variant == RPU_UPDATE_VARIANT_AGGREGATED && dev.linear() && dev.p.ls_mult_noise && !is_transfer()) {
-        launch_update_aggregated(a, update_variant_samples, s);
+        launch_update_aggregated(cross_point_view(a), update_variant_samples, s);
         prof_mark(s, "update_aggregated");
       } else {
-        launch_update_pulsed(a, s);
+        launch_update_pulsed(cross_point_view(a), s);
         prof_mark(s, "update_pulsed");
       }
     } else {
       launch_update_implicit_lines(a, s);
       prof_mark(s, "update_implicit_lines");
       if (counting) count_pulses(a, true, s);
-      launch_update_implicit(a, s);
+      launch_update_implicit(cross_point_view(a), s);
       prof_mark(s, "update_implicit");
     }
     // write noise: cross-points that took a pulse show their new persistent weight with fresh noise
@@ -1377,7 +1462,7 @@ struct Tile {
     if (delta_w) return "no delta weights";
     if (dev.p.count_pulses) return "no pulse counters";
     if (update_variant == RPU_UPDATE_VARIANT_AGGREGATED) return "no update variants";
-    if (shared_xd) return "no column-major shared weights";
+    if (shared_xd) return "no mirrored shared weights";
     if (lr != 0.0f && words_per_sample_for(up, lr, dev.p.dw_min) > 1) return "bit lines of at most 31 pulses";
     return nullptr;
   }
@@ -1473,7 +1558,8 @@ struct Tile {
       const int B = n_images * idx_patches;
       s_rounds.ensure((size_t)B); // the only per-patch state that leaves the kernel: rounds run (get_bm_rounds)
       MvmArgs a{};
-      a.w = mvm_weights(is_test); a.x_size = X; a.d_size = D; a.m_batch = B; a.K = X; a.O = D;
+      a.x_size = X; a.d_size = D; a.m_batch = B; a.K = X; a.O = D;
+      mvm_set_weights(a, mvm_weights(is_test), w_ld(), xd);
       a.io = io_dev(fio);
       a.alpha = fio.p.out_scale;
       a.max_rounds = fio.perfect ? 0 : mvm_max_rounds(a.io);
@@ -1685,7 +1771,7 @@ struct Tile {
         src.d_rbias.ensure(size());
         RPU_HIP_CHECK(hipMemcpy(src.d_rbias.p, src.arr.reset_bias.data(), size() * sizeof(float), hipMemcpyHostToDevice));
       }
-      launch_reset_cols(src.d_w.p, src.d_rbias.p, src.d_wmin.p, src.d_wmax.p, src.par.p.reset_std, start, n_vec, 1.0f, X, D,
+      launch_reset_cols(src.d_w.p, src.d_rbias.p, src.d_wmin.p, src.d_wmax.p, src.par.p.reset_std, start, n_vec, 1.0f, layout(),
                         k, call++, s);
     }
   }
@@ -1998,7 +2084,7 @@ int rpu_tile_get_modified_weights(rpu_tile_t *tile, float *w_host) {
     if (!t.resident() || !t.d_fbw.p) throw RpuError("No modified weights: modify_weights has not been called.");
     DeviceGuard g(t.device_id);
     t.sync_last();
-    RPU_HIP_CHECK(hipMemcpy(w_host, t.d_fbw.p, t.size() * sizeof(float), hipMemcpyDeviceToHost));
+    t.download_mat(w_host, t.d_fbw.p);
   });
 }
 
@@ -2249,7 +2335,7 @@ int rpu_group_create(rpu_group_t **out, rpu_tile_t *const *tiles, int n_tiles) {
       }
       Tile &t = tiles[i]->t;
       if (!t.resident()) throw RpuError("All tiles of a group must be resident on a GPU.");
-      if (t.shared_xd) throw RpuError("A tile with column-major shared weights cannot be in a group.");
+      if (t.shared_xd) throw RpuError("A tile that mirrors its weights into a shared tensor cannot be in a group.");
       if (g->device_id < 0) g->device_id = t.device_id;
       if (t.device_id != g->device_id) throw RpuError("All tiles of a group must be on the same GPU.");
       g->tiles.push_back(tiles[i]);
@@ -2278,9 +2364,11 @@ int rpu_group_update_strided(rpu_group_t *group, const float *const *x_dev, cons
     hipStream_t s = (hipStream_t)stream;
     const int n = (int)group->tiles.size();
     if (!group->h_uargs) {
-      group->d_uargs.ensure((size_t)n);
+      // per tile the arguments of the kernels that make the lines and, after those of all tiles, the view that the
+      // cross-point kernels take (the same, or with x and d exchanged for a tile that stores [x_size][d_size])
+      group->d_uargs.ensure(2 * (size_t)n);
       group->d_ustart.ensure(2 * (size_t)n + 16);
-      RPU_HIP_CHECK(hipHostMalloc((void **)&group->h_uargs, (size_t)n * sizeof(UpdateArgs), hipHostMallocDefault));
+      RPU_HIP_CHECK(hipHostMalloc((void **)&group->h_uargs, 2 * (size_t)n * sizeof(UpdateArgs), hipHostMallocDefault));
       RPU_HIP_CHECK(hipHostMalloc((void **)&group->h_ustart, (2 * (size_t)n + 16) * sizeof(int), hipHostMallocDefault));
     }
     // the staging buffers may still feed the copy of the previous call
@@ -2298,7 +2386,7 @@ int rpu_group_update_strided(rpu_group_t *group, const float *const *x_dev, cons
       }
       if ((x_ld && x_ld[i] < t.X) || (d_ld && d_ld[i] < t.D)) throw RpuError("A row stride is shorter than the row.");
     }
-    std::vector<UpdateArgs> args;
+    std::vector<UpdateArgs> args, views;
     std::vector<int> variant;
     for (int i = 0; i < n; ++i) {
       Tile &t = group->tiles[i]->t;
@@ -2310,7 +2398,8 @@ int rpu_group_update_strided(rpu_group_t *group, const float *const *x_dev, cons
       a.words_per_sample = 1;
       t.note_pulsed_update(a, m_batch, 1, RPU_PULSE_STOCHASTIC_COMPRESSED, s);
       args.push_back(a);
-      variant.push_back(update_pulsed_variant(a));
+      views.push_back(t.cross_point_view(a));
+      variant.push_back(update_pulsed_variant(views.back()));
     }
     const int m = (int)args.size();
     if (m == 0) return;
@@ -2335,7 +2424,7 @@ int rpu_group_update_strided(rpu_group_t *group, const float *const *x_dev, cons
       int wg = 0, j = i;
       for (; j < m && variant[order[j]] == seg.variant; ++j) {
         group->h_ustart[cursor++] = wg;
-        wg += update_pulsed_workgroups(args[order[j]]);
+        wg += update_pulsed_workgroups(views[order[j]]);
       }
       group->h_ustart[cursor++] = wg;
       seg.count = j - i;
@@ -2343,8 +2432,11 @@ int rpu_group_update_strided(rpu_group_t *group, const float *const *x_dev, cons
       segments.push_back(seg);
       i = j;
     }
-    for (int i = 0; i < m; ++i) group->h_uargs[i] = args[order[i]];
-    RPU_HIP_CHECK(hipMemcpyAsync(group->d_uargs.p, group->h_uargs, (size_t)m * sizeof(UpdateArgs), hipMemcpyHostToDevice, s));
+    for (int i = 0; i < m; ++i) {
+      group->h_uargs[i] = args[order[i]];
+      group->h_uargs[m + i] = views[order[i]];
+    }
+    RPU_HIP_CHECK(hipMemcpyAsync(group->d_uargs.p, group->h_uargs, 2 * (size_t)m * sizeof(UpdateArgs), hipMemcpyHostToDevice, s));
     RPU_HIP_CHECK(hipMemcpyAsync(group->d_ustart.p, group->h_ustart, (size_t)cursor * sizeof(int), hipMemcpyHostToDevice, s));
     RPU_HIP_CHECK(hipEventRecord(group->copied, s));
 
@@ -2352,7 +2444,7 @@ int rpu_group_update_strided(rpu_group_t *group, const float *const *x_dev, cons
     launch_update_prepare_group(all, s);
     launch_update_lines_group(all, wide_lines, blocks, s);
     for (const Segment &seg : segments) {
-      UpdateGroup g{group->d_uargs.p + seg.first, group->d_ustart.p + seg.start_offset, seg.count, m_batch};
+      UpdateGroup g{group->d_uargs.p + m + seg.first, group->d_ustart.p + seg.start_offset, seg.count, m_batch};
       launch_update_pulsed_group(g, seg.variant, seg.workgroups, s);
     }
     RPU_HIP_CHECK(hipGetLastError());
@@ -2439,6 +2531,7 @@ static int group_mvm(rpu_group_t *group, const float *const *x_dev, const long *
     std::vector<MvmArgs> args(n);
     std::vector<int> depth(n), mode(n);
     int rounds = 1;
+    bool storage_xd = false;
     for (int i = 0; i < n; ++i) {
       Tile &t = group->tiles[i]->t;
       std::lock_guard<std::mutex> lock(t.mutex);
@@ -2453,6 +2546,9 @@ static int group_mvm(rpu_group_t *group, const float *const *x_dev, const long *
           throw RpuError("Running-average noise management is not provided for a group: call the tiles one by one.");
         }
       }
+      if (t.shared_xd) throw RpuError("A tile that mirrors its weights into a shared tensor cannot be in a group.");
+      if (i == 0) storage_xd = t.xd;
+      if (t.xd != storage_xd) throw RpuError("The tiles of a group must store their weights the same way (all bound to [x_size, d_size] tensors, or none).");
       const int in_size = transposed ? t.D : t.X, out_size = transposed ? t.X : t.D;
       const bool big = use_big && out_size >= 128;
       MvmArgs a = t.mvm_args(m_batch, transposed, t.mvm_weights(is_test), transposed ? t.bio : t.fio, big ? 1 : 0);
@@ -2577,7 +2673,7 @@ static int group_mvm(rpu_group_t *group, const float *const *x_dev, const long *
     for (int r = 0; r < rounds; ++r) {
       if (use_big && r == 0) {
         MvmGroup g{group->d_args.p, group->d_start.p + big_offset, n, m_batch};
-        launch_mvm_big_group(g, big_total, big_bb, transposed, s);
+        launch_mvm_big_group(g, big_total, big_bb, transposed != storage_xd, s);
         if (all_big) continue;
       }
       for (size_t k = 0; k < segments.size(); ++k) {
@@ -2650,9 +2746,10 @@ int rpu_tile_get_drift_state(rpu_tile_t *tile, float *programmed_host, float *nu
     DeviceGuard g(t.device_id);
     t.sync_last();
     const size_t bytes = t.size() * sizeof(float);
-    if (programmed_host) RPU_HIP_CHECK(hipMemcpy(programmed_host, t.i_prog.p, bytes, hipMemcpyDeviceToHost));
-    if (nu_plus_host) RPU_HIP_CHECK(hipMemcpy(nu_plus_host, t.i_nu_plus.p, bytes, hipMemcpyDeviceToHost));
-    if (nu_minus_host) RPU_HIP_CHECK(hipMemcpy(nu_minus_host, t.i_nu_minus.p, bytes, hipMemcpyDeviceToHost));
+    (void)bytes;
+    if (programmed_host) t.download_mat(programmed_host, t.i_prog.p);
+    if (nu_plus_host) t.download_mat(nu_plus_host, t.i_nu_plus.p);
+    if (nu_minus_host) t.download_mat(nu_minus_host, t.i_nu_minus.p);
   });
 }
 
@@ -2726,14 +2823,20 @@ int rpu_tile_clone(rpu_tile_t **out, const rpu_tile_t *src_c) {
       DeviceGuard g(s.device_id);
       RPU_HIP_CHECK(hipStreamSynchronize(s.last_stream));
       t.w_host.resize(s.size());
-      RPU_HIP_CHECK(hipMemcpy(t.w_host.data(), s.d_w.p, s.size() * sizeof(float), hipMemcpyDeviceToHost));
+      s.download_mat(t.w_host.data(), s.d_w.p);
       t.to_device(s.device_id);
       // modified weights, drift clocks and pulse counters travel with the copy
       const size_t n = s.size();
+      // the copy owns its weights and stores them row-major, whatever the source is bound to
       const auto dup = [&](DevBuf<float> &dst, const DevBuf<float> &from) {
         if (!from.p) return;
         dst.ensure(n);
-        RPU_HIP_CHECK(hipMemcpy(dst.p, from.p, n * sizeof(float), hipMemcpyDeviceToDevice));
+        if (s.xd) {
+          launch_transpose(from.p, dst.p, s.X, s.D, s.last_stream);
+          RPU_HIP_CHECK(hipStreamSynchronize(s.last_stream));
+        } else {
+          RPU_HIP_CHECK(hipMemcpy(dst.p, from.p, n * sizeof(float), hipMemcpyDeviceToDevice));
+        }
       };
       dup(t.d_fbw, s.d_fbw);
       dup(t.d_wp, s.d_wp);
@@ -2870,7 +2973,7 @@ int rpu_tile_set_weights(rpu_tile_t *tile, const float *w_host) {
     if (t.resident()) {
       DeviceGuard g(t.device_id);
       t.sync_last();
-      RPU_HIP_CHECK(hipMemcpy(t.d_w.p, w.data(), t.size() * sizeof(float), hipMemcpyHostToDevice));
+      t.upload_mat(t.d_w.p, w.data());
       if (t.persistent()) {
         RPU_HIP_CHECK(hipMemcpy(t.d_wp.p, w.data(), t.size() * sizeof(float), hipMemcpyHostToDevice));
         if (t.dev.p.apply_write_noise_on_set) {
@@ -2907,7 +3010,7 @@ int rpu_tile_get_weights(rpu_tile_t *tile, float *w_host) {
       DeviceGuard g(t.device_id);
       t.shared_in(t.last_stream);
       t.sync_last();
-      RPU_HIP_CHECK(hipMemcpy(w_host, t.wdev(), t.size() * sizeof(float), hipMemcpyDeviceToHost));
+      t.download_mat(w_host, t.wdev());
     } else {
       std::memcpy(w_host, t.w_host.data(), t.size() * sizeof(float));
     }

@@ -581,7 +581,15 @@ class CudaFloatingPointTile(_CudaTileMixin, _TileBase):
 
 
 class CudaAnalogTile(_CudaTileMixin, _TileBase):
-    """GPU analog tile (rpu_base_tiles_cuda.cpp:524-543): built from a host tile."""
+    """GPU analog tile (rpu_base_tiles_cuda.cpp:524-543): built from a host tile.
+
+    ``bind_shared_weights`` (class attribute, default off): allocate an ``[x_size, d_size]`` CUDA tensor for every new
+    tile and bind it with ``set_shared_weights``, which is what the reference's Python does for every CUDA tile when a
+    module is moved to the GPU (src/aihwkit/simulator/tiles/base.py:386-446).  Tiles that the library cannot bind
+    (transfer compounds) stay as they are.
+    """
+
+    bind_shared_weights = False
 
     def __init__(self, tile):  # pylint: disable=super-init-not-called
         if isinstance(tile, int):
@@ -589,6 +597,13 @@ class CudaAnalogTile(_CudaTileMixin, _TileBase):
             self._device = torch.device("cuda", torch.cuda.current_device())
         else:
             self._init_cuda(tile)
+        if type(self).bind_shared_weights:
+            shared = torch.empty(self.get_x_size(), self.get_d_size(), dtype=_DTYPE, device=self._device)
+            try:
+                self.set_shared_weights(shared)
+            except RuntimeError as err:
+                if "transfer compound" not in str(err):
+                    raise
 
 
 class TileGroup:

@@ -93,6 +93,10 @@ def main() -> int:
     ap.add_argument("--batch-sweep", action="store_true",
                     help="instead of the benchmark line: forward and backward call times of the configuration-2 tile "
                          "at batches 32 .. 2000 (HIP events over 200 calls each), one JSON line")
+    ap.add_argument("--storage", default="row_major", choices=("row_major", "xd_shared"),
+                    help="xd_shared: every GPU tile is bound to an [x_size, d_size] shared weight tensor, as the reference's "
+                         "Python binds its CUDA tiles (the library then works on that layout in place); configuration 2 "
+                         "reports that mode as a second block in any case")
     ap.add_argument("--config", type=int, default=2, choices=(1, 2, 3, 4, 5, 6),
                     help="benchmark configuration: 2 is the graded one; 3 is the Tiki-Taka MLP of transfer tiles; "
                          "5 is the forward pass of the GPT-2-small linear layers as PCM inference tiles; 6 "
@@ -116,6 +120,8 @@ def main() -> int:
         return 1
     torch.cuda.set_device(0)
 
+    if args.storage == "xd_shared":
+        tiles.CudaAnalogTile.bind_shared_weights = True
     if args.batch_sweep:
         return batch_sweep()
     if args.config == 3:
@@ -189,8 +195,11 @@ def main() -> int:
     x_pool = [xg] + [torch.from_numpy(rng_pool.uniform(-1, 1, x.shape).astype(np.float32)).cuda() for _ in range(POOL - 1)]
     d_pool = [dg] + [torch.from_numpy((d.std() * rng_pool.standard_normal(d.shape)).astype(np.float32)).cuda()
                      for _ in range(POOL - 1)]
-    w_live = torch.empty(d_size, x_size, dtype=torch.float32, device="cuda")
-    tile.set_shared_weights_row_major(w_live)   # the tile's weight matrix is this tensor from now on (zero copy)
+    if args.storage == "xd_shared":
+        w_live = tile._shared_weights           # the [x_size, d_size] tensor the tile was bound to when it was made
+    else:
+        w_live = torch.empty(d_size, x_size, dtype=torch.float32, device="cuda")
+        tile.set_shared_weights_row_major(w_live)   # the tile's weight matrix is this tensor from now on (zero copy)
     torch.cuda.synchronize()
     w_init = w_live.clone()                     # the initial weights as the tile holds them (clipped to the device bounds)
     step_no = [0]
@@ -259,6 +268,74 @@ def main() -> int:
     tile.set_profiling(True)
     prof_update = kernel_ms(lambda: tile.update(xg, dg, False, False, False, True), n)
     tile.set_profiling(False)
+
+    # The same tile bound to an [x_size, d_size] shared weight tensor, which is how the reference's Python holds every
+    # CUDA tile: the library works on that layout in place (forward addresses the weights as backward does on the
+    # row-major tile and the other way round, the update walks the cross-points with x and d exchanged).
+    xd_block = None
+    if args.storage != "xd_shared":
+        w_xd = torch.empty(x_size, d_size, dtype=torch.float32, device="cuda")
+        tile_x = tiles.CudaAnalogTile(host)
+        tile_x.set_learning_rate(lr)
+        tile_x.set_seed(1234)
+        tile_x.set_shared_weights(w_xd)
+        torch.cuda.synchronize()
+        w_xd_init = w_xd.clone()
+        msx_f = time_calls(lambda: tile_x.forward(xg, False, False, False, False, True), n)
+        msx_b = time_calls(lambda: tile_x.backward(dg, False, False, False, True), n)
+        tile_x.set_profiling(True)
+        px_f = kernel_ms(lambda: tile_x.forward(xg, False, False, False, False, True), n, tile_x)
+        rounds_x = float(tile_x.get_bm_rounds(batch).numpy().mean())
+        px_b = kernel_ms(lambda: tile_x.backward(dg, False, False, False, True), n, tile_x)
+        tile_x.set_profiling(False)
+        sx = [0]
+
+        def step_x():
+            k = sx[0] % POOL
+            sx[0] += 1
+            w_xd.copy_(w_xd_init, non_blocking=True)
+            tile_x.forward(x_pool[k], False, False, False, False, True)
+            tile_x.backward(d_pool[k], False, False, False, True)
+            tile_x.update(x_pool[k], d_pool[k], False, False, False, True)
+
+        for _ in range(args.warmup):
+            step_x()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            step_x()
+        torch.cuda.synchronize()
+        msx_step = (time.perf_counter() - t0) * 1e3 / args.steps
+        w_xd.copy_(w_xd_init)
+        msx_u = time_calls(lambda: tile_x.update(xg, dg, False, False, False, True), n)
+        tile_x.set_profiling(True)
+        px_u = kernel_ms(lambda: tile_x.update(xg, dg, False, False, False, True), n, tile_x)
+        tile_x.set_profiling(False)
+        ubytes = bytes_per_device * x_size * d_size + 4.0 * (x_size + d_size) * batch
+        fl = 2.0 * x_size * d_size * batch
+        xd_block = {
+            "storage": "xd_shared",
+            "what": "the same workload on a tile bound to an [x_size, d_size] shared weight tensor (zero copy)",
+            "value": float(x_size) * d_size * batch / (msx_u * 1e-3) / 1e9, "unit": "Gdevice-updates/s",
+            "ms_per_step": msx_step,
+            "update": {"ms_per_call": msx_u, "kernels_ms": {k: v[0] for k, v in px_u.items()}},
+            "forward": {"ms_per_call": msx_f, "gflops": fl / (msx_f * 1e-3) / 1e9, "mean_bm_rounds": rounds_x,
+                        "kernels_ms": {k: v[0] for k, v in px_f.items()}, "round_launches": px_f["mvm_round"][1]},
+            "backward": {"ms_per_call": msx_b, "gflops": fl / (msx_b * 1e-3) / 1e9,
+                         "kernels_ms": {k: v[0] for k, v in px_b.items()}},
+            "roofline": {"kernel": "k_update_pulsed", "bound": "hbm", "achieved": ubytes / (px_u["update_pulsed"][0] * 1e-3) / 1e9,
+                         "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": ubytes / (px_u["update_pulsed"][0] * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                         "traffic": None, "algorithmic_bytes": ubytes, "kernel_ms": px_u["update_pulsed"][0]},
+            "roofline_forward": {"kernel": "all round launches of a call", "bound": "mfma",
+                                 "achieved": fl / (px_f["mvm_round"][0] * 1e-3) / 1e12, "peak": FP32_MFMA_PEAK_TFLOPS,
+                                 "unit": "TFLOP/s", "frac": fl / (px_f["mvm_round"][0] * 1e-3) / 1e12 / FP32_MFMA_PEAK_TFLOPS,
+                                 "kernel_ms": px_f["mvm_round"][0]},
+            "roofline_backward": {"kernel": "k_mvm_round", "bound": "mfma",
+                                  "achieved": fl / (px_b["mvm_round"][0] * 1e-3) / 1e12, "peak": FP32_MFMA_PEAK_TFLOPS,
+                                  "unit": "TFLOP/s", "frac": fl / (px_b["mvm_round"][0] * 1e-3) / 1e12 / FP32_MFMA_PEAK_TFLOPS,
+                                  "kernel_ms": px_b["mvm_round"][0]},
+        }
+        del tile_x
 
     # coincidences (device pulses) of one update call, from the packed words of the last call: the pulses of sample b
     # in slot k are (x lines that fired) x (d lines that fired)
@@ -399,6 +476,9 @@ def main() -> int:
             " (rocprofv3 --pmc SQ_INSTS_VALU), not measured in this run",
             "pulses_per_call": pulses, "pulses_per_cross_point": pulses / (x_size * d_size),
             "wave_instructions_per_pulse": insts / pulses, "lane_instructions_per_pulse": 64.0 * insts / pulses}
+    out["config"]["storage"] = args.storage
+    if xd_block is not None:
+        out["storage_xd_shared"] = xd_block
     if variants is not None:
         out["update_variants"] = variants
     if other is not None:
@@ -507,7 +587,7 @@ def bench_config3(args) -> int:
         "value": 1e3 / ms_per_step, "unit": "steps/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
         "data": "synthetic",
-        "config": {"workload": "config3: transfer compound of two SoftBounds devices per tile, tiles 785x256, 257x128, "
+        "config": {"storage": args.storage, "workload": "config3: transfer compound of two SoftBounds devices per tile, tiles 785x256, 257x128, "
                                "129x10, batch 64, one column transferred every 2 mini-batches, stochastic pulses, 7/9-bit IO",
                    "batch": batch, "lr": lr, "step": "forward + backward + update of the three tiles"},
         "gdevice_updates_per_s": devices / (ms_per_step * 1e-3) / 1e9,
@@ -647,7 +727,7 @@ def bench_config5(args) -> int:
         "value": tokens / (ms_per_step * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "config5: 768->2304, 768->768, 768->3072, 3072->768 split into 38 tiles of at most 512 x 512, "
+        "config": {"storage": args.storage, "workload": "config5: 768->2304, 768->768, 768->3072, 3072->768 split into 38 tiles of at most 512 x 512, "
                                "1024 tokens, PCM programming noise + drift to 1 day + global drift compensation, 8-bit IO, "
                                "out_noise 0.04, abs-max noise management", "tokens": tokens, "tiles": n_tiles},
         "useful_tflops": flops / (ms_per_step * 1e-3) / 1e12,
@@ -752,7 +832,7 @@ def bench_config4(args) -> int:
         "value": batch / (ms_per_step * 1e-3), "unit": "images/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "config4: conv 1->16 5x5 (tile 26 x 16, 576 patches), conv 16->32 5x5 (tile 401 x 32, 64 "
+        "config": {"storage": args.storage, "workload": "config4: conv 1->16 5x5 (tile 26 x 16, 576 patches), conv 16->32 5x5 (tile 401 x 32, 64 "
                                "patches), fc 513 x 128, fc 129 x 10, batch 512 images 28 x 28, PCM programming noise + "
                                "drift to 1 day + global drift compensation, 8-bit IO, abs-max noise management",
                    "batch": batch},
@@ -824,7 +904,7 @@ def bench_config6(args) -> int:
         "value": n * patches / (ms_per_step * 1e-3), "unit": "patches/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "config6 (supplementary): conv 48->48 3x3 on 128 images 34 x 34 = 131072 patches, tile "
+        "config": {"storage": args.storage, "workload": "config6 (supplementary): conv 48->48 3x3 on 128 images 34 x 34 = 131072 patches, tile "
                                "433 x 48 SoftBounds (dtod + ctoc), BL 31, UM+UBLM, 7/9-bit IO, iterative BM, indexed "
                                "interface", "patches": n * patches},
         "calls": per_call,

@@ -368,8 +368,8 @@ float rpu_tile_get_learning_rate(const rpu_tile_t *tile);
 int rpu_tile_set_weights(rpu_tile_t *tile, const float *w_host);
 int rpu_tile_get_weights(rpu_tile_t *tile, float *w_host);
 
-/* Device pointer of the row-major [d_size][x_size] weight matrix in HBM (NULL if not resident).
- * Stands in for the shared-weights aliasing of RPUCudaSimple::setSharedWeights (C/rpucuda.cu:322-334). */
+/* Device pointer of the weight matrix in HBM (NULL if not resident): row-major [d_size][x_size], or the bound
+ * [x_size][d_size] tensor of a tile with the zero-copy binding of rpu_tile_set_shared_weights_xd. */
 int rpu_tile_weights_device_ptr(rpu_tile_t *tile, float **w_dev);
 
 /* Hidden per-device parameters: RPUPulsed::getDeviceParameterNames / getDeviceParameter /
@@ -621,15 +621,24 @@ int rpu_tile_set_shared_weights(rpu_tile_t *tile, float *weights_dev);
 int rpu_tile_get_shared_weights_if(const rpu_tile_t *tile);
 
 /* set_shared_weights / set_delta_weights as the reference's CUDA tiles bind them (rpu_base_tiles_cuda.cpp:88-130,
- * RPUCudaSimple::setSharedWeights, C/rpucuda.cu:322-334): the device tensor is [x_size][d_size] (column-major W), which
- * is what the reference's Python allocates for a tile whose class name contains "Cuda" and reads back through .t()
- * (src/aihwkit/simulator/tiles/base.py:392-446).  The matrices of this library stay row-major, so the tensor is kept
- * in step by a transposition kernel: it takes the tile's weights when it is set, is read into the tile before every
- * call that uses the weights (the caller may have written to it) and written back after every call that may change
- * them -- one or two passes over the matrix per call (about 3 us each for 1024 x 1024) on top of the call itself;
- * the row-major entry points above have no such cost.  With delta weights the update lands in a buffer of the tile
- * and is transposed into the caller's tensor after the call; null ends the mode.  Not provided for transfer compounds
- * and for members of a group. */
+ * RPUCudaSimple::setSharedWeights, cuda/rpucuda.cu:322-334): a device tensor [x_size][d_size].  That is what the
+ * reference's Python allocates for every tile whose class name contains "Cuda" and reads back through .t()
+ * (src/aihwkit/simulator/tiles/base.py:392-446, tiles/rpucuda.py:166-183).
+ * A plain tile (no transfer compound, no write noise, no pulse counters, no analog terms before the ADC beyond output
+ * noise) takes the tensor as its weight matrix itself, zero copy: its weights are transposed into the tensor once,
+ * every per-cross-point array of the tile (device parameters, drift clocks, modified weights, inference arrays) is
+ * transposed once as well, and from then on the kernels address that layout in place -- forward reads the weights
+ * the way backward does on a row-major tile and the other way round, the update kernels walk the cross-points with x
+ * and d exchanged.  Results are those of the row-major tile (the same pulse trains and ADC draws; the cycle-to-cycle
+ * noise of the update is keyed by the position in memory and so is a different draw of the same law).  Host-side
+ * interfaces (get / set weights, hidden parameters, ...) stay [d_size][x_size]; rpu_tile_weights_device_ptr returns
+ * the tensor.  Such tiles can be members of a group when all members are bound that way.
+ * The other kinds of tile keep their row-major matrix and mirror it: the tensor takes the tile's weights when it is
+ * set, is read into the tile before every call that uses the weights and written back after every call that may
+ * change them (one or two transposition passes per call); they cannot be members of a group.
+ * Delta weights: with the zero-copy binding the caller's [x_size][d_size] tensor is written in place, otherwise the
+ * update lands in a buffer of the tile and is transposed into the tensor after the call; null ends the mode.  Not
+ * provided for transfer compounds. */
 int rpu_tile_set_shared_weights_xd(rpu_tile_t *tile, float *weights_xd_dev);
 int rpu_tile_set_delta_weights_xd(rpu_tile_t *tile, float *delta_weights_xd_dev);
 

@@ -154,8 +154,10 @@ def test_reset_columns(gpu_device):
     assert np.abs(got[:, 1:4]).max() < 0.06 and abs(got[:, 1:4].std() - 0.01) < 0.002     # reset_std 0.01, no bias
 
 
-def test_shared_weights(gpu_device):
+def test_shared_weights(gpu_device, storage_mode):
     """The reference's CUDA tiles take a [x_size, d_size] tensor (rpu_base_tiles_cuda.cpp:88-109)."""
+    if storage_mode != "row_major":
+        pytest.skip("binds a tile that is not bound yet")
     tile = pulsed_tile()
     w = tile.get_weights()
     shared = torch.zeros(37, 23, device="cuda")
@@ -220,8 +222,10 @@ def test_shared_weights_binding_sequence_of_the_reference(gpu_device, x_size, d_
     assert torch.equal(view.cpu(), w_cpu)
 
 
-def test_shared_weights_row_major(gpu_device):
+def test_shared_weights_row_major(gpu_device, storage_mode):
     """The library's own zero-copy form: a [d_size, x_size] tensor becomes the weight matrix itself."""
+    if storage_mode != "row_major":
+        pytest.skip("a tile bound to an [x_size, d_size] tensor refuses the row-major form")
     tile = pulsed_tile()
     w = tile.get_weights()
     shared = torch.zeros(23, 37, device="cuda")
