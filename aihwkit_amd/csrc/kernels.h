@@ -253,6 +253,13 @@ struct UpdateArgs {
   // inputs), so that "rows" are again what is contiguous in memory.  The kernels that make the lines never see it.
   int swapped;
   int x_size, d_size, m_batch;
+  // The stochastic pulse loop on a tile that stores [x_size][d_size]: it walks a row-major copy of the weights (w) with
+  // the tile's row-major parameter copies and stores cross-point (i, j) to w_out[i * wo_si + j * wo_sj], the tile's own
+  // matrix.  The copy is made from wt_src ([x_size][d_size]) by extra workgroups of the kernel that makes the pulse
+  // trains, or by launch_transpose.  All null / zero on a row-major tile: the loop then stores to w in place.
+  float *w_out;
+  long wo_si, wo_sj;
+  const float *wt_src;
   const float *x;
   long x_sb, x_sj; // x element (b, j) at x[b * x_sb + j * x_sj]
   const float *d;

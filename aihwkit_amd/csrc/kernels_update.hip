@@ -258,10 +258,41 @@ __device__ __forceinline__ void update_lines_block(const UpdateArgs &a, const in
   }
 }
 
+// Row-major copy a.w of the [x_size][d_size] matrix a.wt_src for the pulse loop, 32 x 32 tiles through LDS: made by
+// workgroups that the launch of the pulse trains carries beyond its own (`first` .. of blockIdx.x), so that it costs no
+// launch of its own and runs beside that kernel's work.
+__device__ __forceinline__ void update_copy_weights(const UpdateArgs &a, int first, float (*tile)[33]) {
+  const int tiles_j = (a.x_size + 31) / 32, tiles_i = (a.d_size + 31) / 32;
+  const int workers = ((int)gridDim.x - first) * (int)gridDim.y;
+  const int me = ((int)blockIdx.x - first) * (int)gridDim.y + (int)blockIdx.y;
+  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5; // 8 rows of 32 per pass
+  for (int t = me; t < tiles_j * tiles_i; t += workers) {
+    const int j0 = (t / tiles_i) * 32, i0 = (t % tiles_i) * 32;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int j = j0 + ty + 8 * r, i = i0 + tx;
+      tile[ty + 8 * r][tx] = (j < a.x_size && i < a.d_size) ? a.wt_src[(size_t)j * a.d_size + i] : 0.0f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int i = i0 + ty + 8 * r, j = j0 + tx;
+      if (i < a.d_size && j < a.x_size) a.w[(size_t)i * a.x_size + j] = tile[tx][ty + 8 * r];
+    }
+    __syncthreads();
+  }
+}
+
 template <int LINES_E>
 __global__ __launch_bounds__(256) void k_update_lines(UpdateArgs a) {
   __shared__ float vals[64][LINES_E + 1];
   __shared__ uint32_t wt[64][LINES_E + 1];
+  const int own = (a.x_size + LINES_E - 1) / LINES_E + (a.d_size + LINES_E - 1) / LINES_E;
+  if ((int)blockIdx.x >= own) { // only launched with a.wt_src set
+    __shared__ float tile[32][33];
+    update_copy_weights(a, own, tile);
+    return;
+  }
   update_lines_block<LINES_E>(a, (int)blockIdx.x, (int)blockIdx.y, vals, wt);
 }
 
@@ -848,6 +879,13 @@ __device__ __forceinline__ void update_pulsed_row(const UpdateArgs &a, const int
 #pragma unroll
     for (int c = 0; c < C; ++c) w[c] = pulsed_gather<KIND, MULT>(a, w[c], cp[c], cell[c], i, j[c], valid[c], kmax);
   }
+  if (a.w_out) { // the tile's own matrix is laid out another way (UpdateArgs::w_out)
+#pragma unroll
+    for (int c = 0; c < C; ++c) {
+      if (valid[c]) a.w_out[(long)i * a.wo_si + (long)j[c] * a.wo_sj] = w[c];
+    }
+    return;
+  }
 #pragma unroll
   for (int c = 0; c < C; ++c) {
     if (valid[c]) a.w[cell[c]] = w[c];
@@ -857,7 +895,14 @@ __device__ __forceinline__ void update_pulsed_row(const UpdateArgs &a, const int
 template <int KIND, bool MULT, bool NOISE, int C, bool DEEP = false>
 __global__ __launch_bounds__(256, ((C > 1 || DEEP) ? 4 : 8)) void k_update_pulsed(UpdateArgs a) {
   __shared__ float tbl[CTOC_LEVELS];
-  update_pulsed_row<KIND, MULT, NOISE, C, DEEP>(a, (int)blockIdx.x, (int)blockIdx.y, tbl);
+  int row = (int)blockIdx.y;
+  if (a.w_out && (a.d_size & 7) == 0 && gridDim.x == 1) {
+    // Stores along a column of a matrix whose rows run the other way: consecutive workgroups go to different XCDs, so
+    // each XCD is given a band of consecutive rows and the cache lines of the target are put together in one L2.
+    const int band = a.d_size >> 3;
+    row = (row & 7) * band + (row >> 3);
+  }
+  update_pulsed_row<KIND, MULT, NOISE, C, DEEP>(a, (int)blockIdx.x, row, tbl);
 }
 
 // Several tiles in one launch (same device kind, noise and columns per lane): start[t] .. start[t + 1] are the
@@ -1276,10 +1321,18 @@ void launch_update_prepare(const UpdateArgs &a, hipStream_t s) {
 void launch_update_lines(const UpdateArgs &a, hipStream_t s) {
   const unsigned sample_tiles = (a.m_batch + 63) / 64;
   const unsigned wide = (a.x_size + 15) / 16 + (a.d_size + 15) / 16;
+  // workgroups beyond the kernel's own make the row-major copy of the weights (update_copy_weights): about four
+  // 32 x 32 tiles each, at most 256 of them
+  unsigned extra = 0;
+  if (a.wt_src) {
+    const unsigned tiles = ((a.x_size + 31) / 32) * ((a.d_size + 31) / 32);
+    extra = std::min(256u, (tiles + 3) / 4);
+    extra = (extra + sample_tiles - 1) / sample_tiles;
+  }
   if (wide * sample_tiles >= 256) {
-    hipLaunchKernelGGL(k_update_lines<16>, dim3(wide, sample_tiles), dim3(256), 0, s, a);
+    hipLaunchKernelGGL(k_update_lines<16>, dim3(wide + extra, sample_tiles), dim3(256), 0, s, a);
   } else {
-    hipLaunchKernelGGL(k_update_lines<4>, dim3((a.x_size + 3) / 4 + (a.d_size + 3) / 4, sample_tiles), dim3(256), 0, s, a);
+    hipLaunchKernelGGL(k_update_lines<4>, dim3((a.x_size + 3) / 4 + (a.d_size + 3) / 4 + extra, sample_tiles), dim3(256), 0, s, a);
   }
 }
 

@@ -271,6 +271,12 @@ struct Tile {
   // Plain tiles take this form; transfer compounds, write noise, pulse counters and the analog terms before the ADC
   // keep the mirror above.
   bool xd = false;
+  // The stochastic pulse loop is the exception: it walks the d pulses of a row of W with its lanes along x, which on
+  // the usual workloads (inputs denser than errors) takes half the passes of the walk the other way round.  For it
+  // the tile keeps the device parameters row-major as well (r_*) and a row-major scratch copy of the weights (u_wrm),
+  // filled by workgroups that the launch of the pulse trains carries along; the loop stores its results into the
+  // bound tensor directly.
+  DevBuf<float> r_wmax, r_wmin, r_sup, r_sdown, r_slup, r_sldown, u_wrm;
   int w_ld() const { return xd ? D : X; } // row length of the stored matrices
   MatLayout layout() const { return MatLayout{X, D, xd ? 1 : 0}; }
   // Host matrices are row-major [D][X] on every interface; the device copies follow the tile's storage.
@@ -400,6 +406,7 @@ struct Tile {
     s_rounds.release(); s_hitup.release(); s_hitlo.release(); s_list0.release(); s_list1.release(); s_row0.release(); s_row1.release(); s_count.release(); s_tiledone.release();
     u_bl.release(); u_a.release(); u_b.release(); u_xval.release(); u_dval.release(); u_xw.release(); u_dw.release();
     u_xpl.release(); u_dpl.release(); u_kmax.release();
+    r_wmax.release(); r_wmin.release(); r_sup.release(); r_sdown.release(); r_slup.release(); r_sldown.release(); u_wrm.release();
     last_bl = nullptr; last_a = last_b = nullptr; last_xw = last_dw = nullptr;
     t_unit.release(); t_read.release();
     i_ref.release(); i_prog.release(); i_nu_plus.release(); i_nu_minus.release(); i_scalar.release(); i_absmax.release();
@@ -466,7 +473,6 @@ struct Tile {
     nu_valid = false;
     if (!dev.pulsed()) return;
     const size_t n = size(), bytes = n * sizeof(float);
-    (void)bytes;
     d_wmax.ensure(n); d_wmin.ensure(n); d_sup.ensure(n); d_sdown.ensure(n);
     upload_mat(d_wmax.p, arr.w_max.data());
     upload_mat(d_wmin.p, arr.w_min.data());
@@ -476,6 +482,18 @@ struct Tile {
       d_slup.ensure(n); d_sldown.ensure(n);
       upload_mat(d_slup.p, arr.slope_up.data());
       upload_mat(d_sldown.p, arr.slope_down.data());
+    }
+    if (xd) { // the row-major copies of the pulse loop
+      r_wmax.ensure(n); r_wmin.ensure(n); r_sup.ensure(n); r_sdown.ensure(n);
+      RPU_HIP_CHECK(hipMemcpy(r_wmax.p, arr.w_max.data(), bytes, hipMemcpyHostToDevice));
+      RPU_HIP_CHECK(hipMemcpy(r_wmin.p, arr.w_min.data(), bytes, hipMemcpyHostToDevice));
+      RPU_HIP_CHECK(hipMemcpy(r_sup.p, arr.scale_up.data(), bytes, hipMemcpyHostToDevice));
+      RPU_HIP_CHECK(hipMemcpy(r_sdown.p, arr.scale_down.data(), bytes, hipMemcpyHostToDevice));
+      if (dev.linear()) {
+        r_slup.ensure(n); r_sldown.ensure(n);
+        RPU_HIP_CHECK(hipMemcpy(r_slup.p, arr.slope_up.data(), bytes, hipMemcpyHostToDevice));
+        RPU_HIP_CHECK(hipMemcpy(r_sldown.p, arr.slope_down.data(), bytes, hipMemcpyHostToDevice));
+      }
     }
   }
 
@@ -953,6 +971,10 @@ struct Tile {
     a.x_words = const_cast<uint32_t *>(x_words); a.d_words = const_cast<uint32_t *>(d_words);
     a.key = key(); a.call = call++;
     set_plane_args(a, B);
+    if (xd) { // see r_wmax
+      row_major_pulse_loop(a);
+      launch_transpose(d_w.p, u_wrm.p, X, D, s);
+    }
     // words from outside: the longest bit line among them picks the pulse loop, as the batch's largest BL does for the
     // tile's own words (short lines then take the same loop, and the same noise stream, as in rpu_tile_update)
     a.kmax_slot = 3;
@@ -961,7 +983,7 @@ struct Tile {
     launch_update_planes(a, s);
     prof_mark(s, "update_planes");
     if (dev.p.count_pulses) count_pulses(a, false, s);
-    launch_update_pulsed(cross_point_view(a), s);
+    launch_update_pulsed(a, s);
     prof_mark(s, "update_pulsed");
     if (persistent()) launch_write_noise_touched(a, d_w.p, d_wp.p, dev.scaled_write_noise(), false, s);
     RPU_HIP_CHECK(hipGetLastError());
@@ -1297,8 +1319,20 @@ struct Tile {
       return;
     }
     d_w.adopt(w_xd_dev, size());
-    for (DevBuf<float> *b : {&d_wmax, &d_wmin, &d_sup, &d_sdown, &d_slup, &d_sldown, &d_nu, &dr_prev, &dr_w0, &dr_t, &d_fbw,
-                             &i_ref, &i_prog, &i_nu_plus, &i_nu_minus}) {
+    // the device parameters: the row-major arrays stay for the pulse loop, copies in the tensor's layout serve the rest
+    {
+      DevBuf<float> *own[6] = {&d_wmax, &d_wmin, &d_sup, &d_sdown, &d_slup, &d_sldown};
+      DevBuf<float> *kept[6] = {&r_wmax, &r_wmin, &r_sup, &r_sdown, &r_slup, &r_sldown};
+      for (int k = 0; k < 6; ++k) {
+        if (!own[k]->p) continue;
+        std::swap(*own[k], *kept[k]);
+        own[k]->ensure(size());
+        launch_transpose(kept[k]->p, own[k]->p, D, X, last_stream);
+      }
+      RPU_HIP_CHECK(hipStreamSynchronize(last_stream));
+    }
+    if (dev.pulsed()) u_wrm.ensure(size()); // here, so that no update call has to allocate it
+    for (DevBuf<float> *b : {&d_nu, &dr_prev, &dr_w0, &dr_t, &d_fbw, &i_ref, &i_prog, &i_nu_plus, &i_nu_minus}) {
       to_xd_in_place(*b);
     }
     if (state_params_valid) {
@@ -1399,6 +1433,15 @@ struct Tile {
     return a;
   }
 
+  // the pulse loop of a tile that stores [x_size][d_size]: on the row-major copies, results into the tile's matrix
+  void row_major_pulse_loop(UpdateArgs &a) {
+    u_wrm.ensure(size());
+    a.w = u_wrm.p;
+    a.w_out = d_w.p; a.wo_si = 1; a.wo_sj = D;
+    a.dev.w_max = r_wmax.p; a.dev.w_min = r_wmin.p; a.dev.scale_up = r_sup.p; a.dev.scale_down = r_sdown.p;
+    a.dev.slope_up = r_slup.p; a.dev.slope_down = r_sldown.p;
+  }
+
   // the arguments of a pulsed update as the kernels that work cross-point by cross-point take them: as they are on a
   // row-major tile, with x and d exchanged on one that stores [x_size][d_size] (UpdateArgs::swapped)
   UpdateArgs cross_point_view(const UpdateArgs &a) const { return xd ? update_swapped_view(a) : a; }
@@ -1427,14 +1470,19 @@ struct Tile {
       // from here on the kernels walk rows of words; a longer bit line is several rows of one sample in a row
       a.m_batch = rows;
       a.words_per_sample = wps;
+      const bool aggregated = update_variant == RPU_UPDATE_VARIANT_AGGREGATED && dev.linear() && dev.p.ls_mult_noise && !is_transfer();
+      if (xd && !aggregated && dv.w == d_w.p) {
+        row_major_pulse_loop(a);
+        a.wt_src = d_w.p; // the launch of the pulse trains makes the row-major copy
+      }
       launch_update_lines(a, s);
       prof_mark(s, "update_lines");
       if (counting) count_pulses(a, false, s);
-      if (update_variant == RPU_UPDATE_VARIANT_AGGREGATED && dev.linear() && dev.p.ls_mult_noise && !is_transfer()) {
+      if (aggregated) {
         launch_update_aggregated(cross_point_view(a), update_variant_samples, s);
         prof_mark(s, "update_aggregated");
       } else {
-        launch_update_pulsed(cross_point_view(a), s);
+        launch_update_pulsed(a, s);
         prof_mark(s, "update_pulsed");
       }
     } else {
@@ -2398,7 +2446,12 @@ int rpu_group_update_strided(rpu_group_t *group, const float *const *x_dev, cons
       a.words_per_sample = 1;
       t.note_pulsed_update(a, m_batch, 1, RPU_PULSE_STOCHASTIC_COMPRESSED, s);
       args.push_back(a);
-      views.push_back(t.cross_point_view(a));
+      UpdateArgs v = a;
+      if (t.xd) { // the pulse loop runs on row-major copies (Tile::r_wmax); here the copy of the weights is a launch of its own
+        t.row_major_pulse_loop(v);
+        launch_transpose(t.d_w.p, t.u_wrm.p, t.X, t.D, s);
+      }
+      views.push_back(v);
       variant.push_back(update_pulsed_variant(views.back()));
     }
     const int m = (int)args.size();

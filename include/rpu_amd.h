@@ -627,12 +627,16 @@ int rpu_tile_get_shared_weights_if(const rpu_tile_t *tile);
  * A plain tile (no transfer compound, no write noise, no pulse counters, no analog terms before the ADC beyond output
  * noise) takes the tensor as its weight matrix itself, zero copy: its weights are transposed into the tensor once,
  * every per-cross-point array of the tile (device parameters, drift clocks, modified weights, inference arrays) is
- * transposed once as well, and from then on the kernels address that layout in place -- forward reads the weights
- * the way backward does on a row-major tile and the other way round, the update kernels walk the cross-points with x
- * and d exchanged.  Results are those of the row-major tile (the same pulse trains and ADC draws; the cycle-to-cycle
- * noise of the update is keyed by the position in memory and so is a different draw of the same law).  Host-side
- * interfaces (get / set weights, hidden parameters, ...) stay [d_size][x_size]; rpu_tile_weights_device_ptr returns
- * the tensor.  Such tiles can be members of a group when all members are bound that way.
+ * transposed once as well, and from then on the kernels address that layout in place: forward reads the weights
+ * the way backward does on a row-major tile and the other way round, maintenance kernels know both layouts, the
+ * deterministic and floating-point updates walk the cross-points with x and d exchanged.  The stochastic pulse loop
+ * alone keeps its row-major form (lanes along x, walking the d pulses of a row: half the passes of the walk the other
+ * way round where inputs are denser than errors): the tile keeps row-major copies of the device parameters for it, the
+ * launch that makes the pulse trains also makes a row-major scratch copy of the weights, and the loop stores its
+ * results straight into the tensor.  Results are bit for bit those of the row-major tile (same pulse trains, same noise
+ * draws per cross-point, same ADC draws).  Host-side interfaces (get / set weights, hidden parameters, ...) stay
+ * [d_size][x_size]; rpu_tile_weights_device_ptr returns the tensor.  Such tiles can be members of a group when all
+ * members are bound that way.
  * The other kinds of tile keep their row-major matrix and mirror it: the tensor takes the tile's weights when it is
  * set, is read into the tile before every call that uses the weights and written back after every call that may
  * change them (one or two transposition passes per call); they cannot be members of a group.
