@@ -128,3 +128,81 @@ def conv_index_matrix(image_shape, kernel, with_bias=True):
     if with_bias:
         unfolded = torch.cat([unfolded, torch.ones(1, unfolded.shape[1])], dim=0)
     return unfolded.to(torch.int32).contiguous().reshape(-1), unfolded.shape[1]
+
+
+# ---- configuration 5: the GPT-2-small linear layers as PCM inference tiles ---------------------------------------
+
+# split into tiles of at most 512 x 512 the way the reference's tile array does
+# (src/aihwkit/simulator/tiles/array.py:82-97): (in, out, input splits, output splits)
+CONFIG5_LAYERS = (
+    (768, 2304, (384, 384), (461, 461, 461, 461, 460)),
+    (768, 768, (384, 384), (384, 384)),
+    (768, 3072, (384, 384), (512,) * 6),
+    (3072, 768, (512,) * 6, (384, 384)),
+)
+
+
+def config5_io(out_noise=0.04):
+    return io_params(inp_res=1 / 254.0, out_res=1 / 254.0, out_noise=out_noise,
+                     noise_management=dv.NoiseManagementType.AbsMax,
+                     bound_management=dv.BoundManagementType.Iterative)
+
+
+def config5_layers(tokens=1024, io=None, noise_model=None, t_inference=86400.0, seed=0):
+    """The 38 tiles, on the GPU: weights N(0, 0.02), programmed with ``noise_model`` (default: the PCM model) and
+    drifted to ``t_inference`` seconds.  Returns per layer a list of (x_part [tokens, n_in], row of tiles), one entry
+    per input split; the inputs are N(0, 1)."""
+    from aihwkit_amd.inference import InferenceTile
+    rng = np.random.default_rng(seed)
+    io = io or config5_io()
+    layers, n_tiles = [], 0
+    for in_size, out_size, in_split, out_split in CONFIG5_LAYERS:
+        x = torch.from_numpy(rng.standard_normal((tokens, in_size)).astype(np.float32)).cuda()
+        grid, i0 = [], 0
+        for n_in in in_split:
+            row = []
+            for n_out in out_split:
+                tile = InferenceTile(n_out, n_in, forward_io=io, noise_model=noise_model)
+                tile.set_weights(torch.from_numpy((0.02 * rng.standard_normal((n_out, n_in))).astype(np.float32)))
+                tile.cuda()
+                tile.tile.set_seed(1000 + n_tiles)
+                tile.drift_weights(t_inference)
+                row.append(tile)
+                n_tiles += 1
+            grid.append((x[:, i0:i0 + n_in].contiguous(), row))
+            i0 += n_in
+        layers.append(grid)
+    return layers
+
+
+def config5_groups(layers, tokens=1024):
+    """One tile group per layer: all tiles of the layer in a few launches.  The tiles read column slices of the layer
+    input and write column slices of one partial-output matrix per input split in place; the drift-compensation
+    factor of a tile rides on its ADC stage.  Returns per layer (group, tiles, inputs, outputs, partial [splits,
+    tokens, out_size])."""
+    from aihwkit_amd.rpu_base.tiles import TileGroup
+    groups = []
+    for (in_size, out_size, in_split, out_split), grid in zip(CONFIG5_LAYERS, layers):
+        x_layer = torch.cat([x_part for x_part, _ in grid], dim=1)                       # [tokens, in_size]
+        partial = torch.empty(len(in_split), tokens, out_size, device="cuda")
+        flat_tiles, flat_x, flat_y, i0 = [], [], [], 0
+        for i, (n_in, (_, row)) in enumerate(zip(in_split, grid)):
+            o0 = 0
+            for tile, n_out in zip(row, out_split):
+                tile.compensate_in_tile(True)
+                flat_tiles.append(tile)
+                flat_x.append(x_layer[:, i0:i0 + n_in])
+                flat_y.append(partial[i][:, o0:o0 + n_out])
+                o0 += n_out
+            i0 += n_in
+        groups.append((TileGroup([t.tile for t in flat_tiles]), flat_tiles, flat_x, flat_y, partial))
+    return groups
+
+
+def config5_step(groups):
+    """Forward pass of all tiles; the partial outputs of the input splits are summed digitally."""
+    outs = []
+    for group, _, flat_x, flat_y, partial in groups:
+        group.forward(flat_x, is_test=True, non_blocking=True, outs=flat_y)
+        outs.append(partial.sum(dim=0) if partial.shape[0] > 1 else partial[0])
+    return outs

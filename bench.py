@@ -621,52 +621,20 @@ def bench_config3(args) -> int:
     return 0
 
 
-# GPT-2-small linear layers split into tiles of at most 512 x 512 the way the reference's tile array does
-# (src/aihwkit/simulator/tiles/array.py:82-97): (in, out) -> input splits x output splits
-CONFIG5_LAYERS = (
-    (768, 2304, (384, 384), (461, 461, 461, 461, 460)),
-    (768, 768, (384, 384), (384, 384)),
-    (768, 3072, (384, 384), (512,) * 6),
-    (3072, 768, (512,) * 6, (384, 384)),
-)
-
-
 def bench_config5(args) -> int:
     """Configuration 5: forward pass of the four GPT-2-small linear shapes for 1024 tokens through PCM inference
     tiles (weights N(0, 0.02) programmed with PCM noise and drifted to one day, global drift compensation, 8-bit
     DAC / ADC, out_noise 0.04, abs-max noise management); the partial outputs of the input splits are summed
     digitally.  A step = the forward pass of all 38 tiles."""
-    import numpy as np
     import torch
 
-    from aihwkit_amd.inference import InferenceTile
-    from aihwkit_amd.rpu_base import devices as dv
-    from aihwkit_amd.rpu_base.tiles import TileGroup
-    from aihwkit_amd.benchmark_configs import io_params
+    from aihwkit_amd.benchmark_configs import CONFIG5_LAYERS, config5_groups, config5_layers, config5_step
 
     torch.cuda.set_device(0)
     tokens = 1024
-    rng = np.random.default_rng(0)
-    io = io_params(inp_res=1 / 254.0, out_res=1 / 254.0, out_noise=0.04, noise_management=dv.NoiseManagementType.AbsMax,
-                   bound_management=dv.BoundManagementType.Iterative)
-    layers, flops, n_tiles = [], 0.0, 0
-    for in_size, out_size, in_split, out_split in CONFIG5_LAYERS:
-        x = torch.from_numpy(rng.standard_normal((tokens, in_size)).astype(np.float32)).cuda()
-        grid, i0 = [], 0
-        for n_in in in_split:
-            row = []
-            for n_out in out_split:
-                tile = InferenceTile(n_out, n_in, forward_io=io)
-                tile.set_weights(torch.from_numpy((0.02 * rng.standard_normal((n_out, n_in))).astype(np.float32)))
-                tile.cuda()
-                tile.tile.set_seed(1000 + n_tiles)
-                tile.drift_weights(86400.0)
-                row.append(tile)
-                n_tiles += 1
-            grid.append((x[:, i0:i0 + n_in].contiguous(), row))
-            i0 += n_in
-        layers.append(grid)
-        flops += 2.0 * tokens * in_size * out_size
+    layers = config5_layers(tokens)
+    n_tiles = sum(len(row) for grid in layers for _, row in grid)
+    flops = sum(2.0 * tokens * in_size * out_size for in_size, out_size, _, _ in CONFIG5_LAYERS)
 
     def step_per_tile():
         outs = []
@@ -687,32 +655,10 @@ def bench_config5(args) -> int:
     torch.cuda.synchronize()
     ms_per_tile_loop = (time.perf_counter() - t0) * 1e3 / max(args.steps // 4, 3)
 
-    # one group per layer: all tiles of the layer in a few launches.  The tiles read column slices of the layer input
-    # and write column slices of one partial-output matrix per input split in place; the drift-compensation factor of
-    # a tile rides on its ADC stage; the partial outputs of the input splits are summed digitally.
-    groups = []
-    for li, grid in enumerate(layers):
-        in_size, out_size, in_split, out_split = CONFIG5_LAYERS[li]
-        x_layer = torch.cat([x_part for x_part, _ in grid], dim=1)                       # [tokens, in_size]
-        partial = torch.empty(len(in_split), tokens, out_size, device="cuda")
-        flat_tiles, flat_x, flat_y, i0 = [], [], [], 0
-        for i, (n_in, (_, row)) in enumerate(zip(in_split, grid)):
-            o0 = 0
-            for tile, n_out in zip(row, out_split):
-                tile.compensate_in_tile(True)
-                flat_tiles.append(tile)
-                flat_x.append(x_layer[:, i0:i0 + n_in])
-                flat_y.append(partial[i][:, o0:o0 + n_out])
-                o0 += n_out
-            i0 += n_in
-        groups.append((TileGroup([t.tile for t in flat_tiles]), flat_x, flat_y, partial))
+    groups = config5_groups(layers, tokens)
 
     def step():
-        outs = []
-        for group, flat_x, flat_y, partial in groups:
-            group.forward(flat_x, is_test=True, non_blocking=True, outs=flat_y)
-            outs.append(partial.sum(dim=0) if partial.shape[0] > 1 else partial[0])
-        return outs
+        return config5_step(groups)
 
     for _ in range(args.warmup):
         step()

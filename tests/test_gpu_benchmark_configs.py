@@ -6,13 +6,15 @@
 * the 64-seed mean / variance protocol (src/rpucuda/cuda/rpucuda_pulsed_test.cpp:1048-1131) at 1024 x 1024 x 256 for
   forward, backward and the weight change;
 * a full-size configuration-1 update through the pulse words;
-* configuration 4: the four LeNet5 tiles at their real shapes, 8-bit converters, batch 512.
+* configuration 4: the four LeNet5 tiles at their real shapes, 8-bit converters, batch 512;
+* configuration 5: the 38 tiles of the GPT-2-small linear shapes through one tile group per layer, 1024 tokens.
 """
 import numpy as np
 import pytest
 import torch
 import torch.nn.functional as F
 
+from aihwkit_amd.benchmark_configs import CONFIG5_LAYERS, config5_groups, config5_io, config5_layers, config5_step
 from aihwkit_amd.inference import InferenceTile, PCMLikeNoiseModel
 from aihwkit_amd.rpu_base import devices as dv
 from aihwkit_amd.rpu_base import tiles
@@ -520,3 +522,119 @@ def test_configuration_4_full_batch_with_pcm_noise_drift_and_compensation(gpu_de
         assert float(comp.abs().max()) <= bound * 1.001
         h = F.max_pool2d(torch.tanh(comp), 2) if kind == "conv" else torch.tanh(comp)
     assert h.shape == (batch, 10)
+
+
+# ---- configuration 5: the GPT-2-small linear shapes as 38 tiles, one tile group per layer -------------------------
+
+@pytest.mark.parametrize("out_bound", [12.0, 0.2])
+def test_configuration_5_tiles_without_noise_match_the_oracle(gpu_device, out_bound):
+    """The whole workload the way the benchmark drives it: 1024 tokens, the tiles of a layer in one group that reads
+    column slices of the layer input and writes column slices of the partial-output matrices, the drift-compensation
+    factor on each tile's ADC stage.  All noise scales zero: every partial output against an oracle tile that holds
+    the tile's weights and its factor as out_scale; round counts equal.  With the benchmark's ADC range (12) no sample
+    of these weights needs a second round; the range 0.2 sends most of them through two or three."""
+    tokens = 1024
+    io = config5_io(out_noise=0.0)
+    io.out_bound = out_bound
+    quiet = PCMLikeNoiseModel(prog_noise_scale=0.0, read_noise_scale=0.0, drift_scale=0.0)
+    layers = config5_layers(tokens, io=io, noise_model=quiet)
+    groups = config5_groups(layers, tokens)
+    assert sum(len(g[1]) for g in groups) == 38
+    totals = config5_step(groups)
+    torch.cuda.synchronize()
+    most_rounds = 0
+    for (in_size, out_size, in_split, out_split), (_, flat_tiles, flat_x, flat_y, partial), total in zip(
+            CONFIG5_LAYERS, groups, totals):
+        assert total.shape == (tokens, out_size)
+        assert torch.equal(total, partial.sum(dim=0) if len(in_split) > 1 else partial[0])
+        for tile, x_part, y_part in zip(flat_tiles, flat_x, flat_y):
+            n_out, n_in = y_part.shape[1], x_part.shape[1]
+            assert abs(tile.alpha - 1.0) < 1e-4          # nothing drifted
+            o_io = config5_io(out_noise=0.0)
+            o_io.out_bound = out_bound
+            o_io.out_scale = float(F32(tile.alpha))
+            meta = make_meta(o_io, noise_free_io())
+            meta.backward_io.is_perfect = True
+            meta.update.pulse_type = dv.PulseType.NONE
+            orc = OracleTile(n_in, n_out, meta._config(dv.IdealResistiveDeviceParameter()))
+            orc.set_weights(tile.get_weights().numpy())
+            x = np.ascontiguousarray(x_part.cpu().numpy())
+            want = orc.forward(x)
+            got = y_part.cpu().numpy()
+            r_gpu, r_orc = tile.tile.get_bm_rounds(tokens).numpy(), orc.bm_rounds(tokens)
+            same = r_gpu == r_orc                        # a sample exactly on the ADC's edge may be read either way
+            assert same.mean() > 0.995, (n_in, n_out, same.mean())
+            if out_bound == 12.0:
+                assert same.all() and (r_gpu == 1).all()
+            most_rounds = max(most_rounds, int(r_gpu.max()))
+            diff = np.abs(got - want)[same]
+            off = diff > 1e-5
+            assert off.mean() < 5e-3, (n_in, n_out, off.mean())
+            # a flip is one ADC code of that sample: 2 * out_bound / 254 * largest input of the row * 2^(rounds - 1)
+            code = 2.0 * out_bound / 254.0 * np.abs(x).max(axis=1) * 2.0 ** (r_gpu - 1.0) * tile.alpha
+            assert (diff.max(axis=1) <= code[same] * 1.001 + 1e-5).all()
+    assert most_rounds == 1 if out_bound == 12.0 else most_rounds >= 3
+
+
+def test_configuration_5_with_pcm_noise_drift_and_compensation(gpu_device):
+    """The benchmark's own settings (PCM programming noise, drift to one day, read noise, out_noise 0.04, global drift
+    compensation inside the tiles), 1024 tokens through the groups: size-independent properties per tile and per
+    layer -- the compensation factor follows from the expected read-outs, the uncompensated partial output carries
+    the drifted share of the signal and the compensated one that share times the factor, the layer output correlates
+    with the exact product, outputs stay within the ADC range, a re-seeded
+    run repeats bit for bit, and the group's outputs are those of one call per tile up to single ADC codes."""
+    tokens = 1024
+    layers = config5_layers(tokens)
+    groups = config5_groups(layers, tokens)
+    seeds = lambda: [t.tile.set_seed(4000 + k) for k, t in enumerate(t for g in groups for t in g[1])]
+    seeds()
+    first = [t.clone() for t in config5_step(groups)]
+    seeds()
+    again = config5_step(groups)
+    for a, b in zip(first, again):
+        assert torch.equal(a, b) and torch.isfinite(a).all()
+    seeds()
+    # one call per tile draws the same noise; at this batch the group sums in another order (128 x 128 workgroup tiles),
+    # so a value on an ADC edge may land on the neighbouring code
+    for _, flat_tiles, flat_x, flat_y, _ in groups:
+        for tile, x_part, y_part in zip(flat_tiles, flat_x, flat_y):
+            single = tile.forward(x_part.contiguous(), is_test=True)
+            diff = (single - y_part).abs()
+            assert float((diff > 0).float().mean()) < 2e-3, (x_part.shape, y_part.shape)
+            code = 24.0 / 254.0 * x_part.abs().amax(dim=1, keepdim=True) * tile.alpha
+            assert bool((diff <= code * 1.001 + 1e-6).all())
+    # These weights (N(0, 0.02), not mapped to the conductance range) sit below the converter's step (24 / 254) and the
+    # output noise (0.04): the read-out behind the compensation factor sees mostly noise, so the factor is NOT the
+    # inverse of the weights' shrinkage.  It is checked against the expected read-out (mean |ADC(w + 0.04 N)| over the
+    # identity's outputs) before and after the drift.
+    noise = np.random.default_rng(5)
+
+    def expected_readout(w):
+        v = w.numpy().astype(np.float64) + 0.04 * noise.standard_normal(tuple(w.shape))
+        step = 24.0 / 254.0
+        return np.abs(np.clip(np.rint(v / step) * step, -12.0, 12.0)).mean()
+
+    for (in_size, out_size, in_split, out_split), (_, flat_tiles, flat_x, flat_y, partial), total in zip(
+            CONFIG5_LAYERS, groups, first):
+        exact = torch.zeros(tokens, out_size, device="cuda", dtype=torch.float64)
+        for k, (tile, x_part, y_part) in enumerate(zip(flat_tiles, flat_x, flat_y)):
+            programmed, _nu_p, _nu_m = tile.drift_state()
+            drifted = tile.get_weights()
+            shrink = float(drifted.abs().mean() / programmed.abs().mean())
+            assert 0.4 < shrink < 0.9
+            assert tile.alpha == pytest.approx(expected_readout(programmed) / expected_readout(drifted), rel=0.02)
+            assert 1.0 < tile.alpha < 1.0 / shrink
+            ideal = x_part.double() @ programmed.double().cuda().T        # the undrifted tile without converters
+            slope = lambda y: float((y.double() * ideal).sum() / (ideal * ideal).sum())
+            kept = float((drifted.double() * programmed.double()).sum() / (programmed.double() ** 2).sum())
+            tile.compensate_in_tile(False)
+            raw = tile.forward(x_part.contiguous(), is_test=False)        # (evaluation mode would multiply by the factor)
+            tile.compensate_in_tile(True)
+            assert slope(raw) == pytest.approx(kept, rel=0.08)            # the drifted signal passes the converters unbiased
+            assert slope(y_part) == pytest.approx(tile.alpha * kept, rel=0.08)
+            bound = 12.0 * float(x_part.abs().max()) * 16.0 * tile.alpha
+            assert float(y_part.abs().max()) <= bound * 1.001
+            o0 = sum(out_split[:k % len(out_split)])
+            exact[:, o0:o0 + y_part.shape[1]] += ideal
+        c = np.corrcoef(total.cpu().numpy().ravel(), exact.cpu().numpy().ravel())[0, 1]
+        assert c > 0.7, (in_size, out_size, c)
