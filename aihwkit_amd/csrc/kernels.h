@@ -43,10 +43,14 @@ struct MvmState {
 // Rounds 0 and 1 of a call in one launch (samples that need a second round are the rule on some workloads):
 // the state of that launch and of the selection that the following launch starts with.
 struct DualDev {
-  float *buf[2]; // buf[r]: [m_batch][O] outputs of round r of the fused launch
-  int *sel;      // [m_batch] which of them is the sample's output (0 / 1); 2: the sample is listed for round 2
+  float *buf[3]; // buf[r]: [m_batch][O] outputs of round r of the fused launch
+  int *sel;      // [m_batch] which of them is the sample's output (0 .. rounds - 1); rounds: the sample is listed
+                 // for the round after the fused launch
   int *hit1;     // [2][m_batch] saturation marks of round 1: upper, lower (as MvmState::hit_up / hit_lo)
-  float *xq2;    // quantized rows of round 2, written while round 0's rows are still read
+  int *hit2;     // the same of round 2 (three fused rounds)
+  float *xq2;    // quantized rows of round 2: written by the fused launch of two rounds while round 0's rows are still
+                 // read, by the init kernel for a fused launch of three
+  int rounds;    // rounds of the fused launch: 2 or 3 (0: the call has none)
   int *seen;     // host-visible: [0] samples of the last call that needed round 1, [1] its batch, [2] the last round
                  // that listed a sample (0: none after round 0), [3] 1 + the round at which a wait between the
                  // workgroups of a launch gave up (0: none); null: not kept

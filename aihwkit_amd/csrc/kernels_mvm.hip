@@ -290,14 +290,46 @@ __device__ __forceinline__ float next_round_scale(const MvmArgs &a, int round, i
 // Instruction order of one pipelined step (a hint to the scheduler): the 16 MFMAs are spread over the step with
 // the LDS writes of the next step's tiles between the first ones and its global loads and LDS reads
 // between the others, so that the LDS and memory pipes work underneath the matrix pipe of the same wave.
-template <int WMODE, bool DUAL = false>
+template <int WMODE, int NACC = 1>
 __device__ __forceinline__ void mvm_step_schedule() {
+  constexpr bool DUAL = NACC == 2;
 #define RPU_SG(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)
 #define RPU_SG_MFMA 0x008
 #define RPU_SG_VMEM 0x020
 #define RPU_SG_DSR 0x100
 #define RPU_SG_DSW 0x200
-  if (DUAL && WMODE == 1) { // per step: 32 MFMAs, 8 LDS writes, 24 global loads, 8 LDS reads
+  if (NACC == 3 && WMODE == 1) { // per step: 48 MFMAs, 12 LDS writes, 28 global loads, 12 LDS reads
+#pragma unroll
+    for (int i = 0; i < 12; ++i) {
+      RPU_SG(RPU_SG_MFMA, 1);
+      RPU_SG(RPU_SG_DSW, 1);
+    }
+#pragma unroll
+    for (int i = 0; i < 12; ++i) {
+      RPU_SG(RPU_SG_MFMA, 1);
+      RPU_SG(RPU_SG_VMEM, 2);
+      RPU_SG(RPU_SG_DSR, 1);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      RPU_SG(RPU_SG_MFMA, 1);
+      RPU_SG(RPU_SG_VMEM, 1);
+    }
+    RPU_SG(RPU_SG_MFMA, 20);
+  } else if (NACC == 3) { // per step: 48 MFMAs, 16 LDS writes, 16 global loads, 16 LDS reads
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      RPU_SG(RPU_SG_MFMA, 1);
+      RPU_SG(RPU_SG_DSW, 1);
+    }
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      RPU_SG(RPU_SG_MFMA, 1);
+      RPU_SG(RPU_SG_VMEM, 1);
+      RPU_SG(RPU_SG_DSR, 1);
+    }
+    RPU_SG(RPU_SG_MFMA, 16);
+  } else if (DUAL && WMODE == 1) { // per step: 32 MFMAs, 8 LDS writes, 24 global loads, 8 LDS reads
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       RPU_SG(RPU_SG_MFMA, 1);
@@ -380,13 +412,16 @@ __device__ __forceinline__ void mvm_step_schedule() {
 // padding of the quantized inputs or are never stored.
 // PD = 2, 4: software pipeline with the global loads of PD steps in flight, k_pad a multiple of
 // PD * KSTEP * WAVES; PD = 1: one register set, for short contractions, k_pad a multiple of KSTEP.
-// DUAL (round 0 only, PD = 2): the same weights also multiply the rows that round 1 would use (written by the init
+// NACC = 2 (round 0 only, PD = 2): the same weights also multiply the rows that round 1 would use (written by the init
 // kernel into the other scratch matrix), into a second accumulator; both rounds go through the ADC stage, round r
 // into a.dual.buf[r], with their own saturation marks.  Which of the two is a sample's output is decided when its
-// tile is finished (mvm_tile_finished_dual) and copied out at the start of the next launch.
-template <int PD, int WMODE, bool DUAL = false>
+// tile is finished (mvm_tile_finished_dual) and copied out at the start of the next launch.  NACC = 3: the rows of
+// round 2 as well (a.dual.xq2, also written by the init kernel), into a third accumulator.
+template <int PD, int WMODE, int NACC = 1>
 __device__ __forceinline__ void mvm_round_tile(const MvmArgs &a, int round, int tile_o, int tile_b, int n_act,
                                                float (*red)[16][64], float *stage) {
+  constexpr bool DUAL = NACC >= 2;
+  constexpr bool TRI = NACC == 3;
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int r = lane & 31;
@@ -408,9 +443,10 @@ __device__ __forceinline__ void mvm_round_tile(const MvmArgs &a, int round, int 
   const int s_begin = min(wave * per_wave, steps);
   const int s_end = min(s_begin + per_wave, steps);
 
-  float *stage_x = stage + wave * ((DUAL ? 3 : 2) * TILE * LDS_ROW);
+  float *stage_x = stage + wave * ((NACC + 1) * TILE * LDS_ROW);
   float *stage_w = stage_x + TILE * LDS_ROW;
-  float *stage_x1 = stage_w + TILE * LDS_ROW; // DUAL only
+  float *stage_x1 = stage_w + TILE * LDS_ROW;  // DUAL only
+  float *stage_x2 = stage_x1 + TILE * LDS_ROW; // TRI only
 
   // staging layout of this lane: pass t covers rows 8 t .. 8 t + 7, lane = (row in pass) * 8 + 16-byte chunk
   const int st_row = lane >> 3;
@@ -418,6 +454,7 @@ __device__ __forceinline__ void mvm_round_tile(const MvmArgs &a, int round, int 
   const float *xq = round_rows(a, round);
   const float *x_src[4];
   const float *x1_src[4];
+  const float *x2_src[4];
   const float *w_src[4];
 #pragma unroll
   for (int t = 0; t < 4; ++t) {
@@ -426,16 +463,18 @@ __device__ __forceinline__ void mvm_round_tile(const MvmArgs &a, int round, int 
     const int xrow = (round > 0) ? pick2(a.st.row, round & 1)[slot] : slot;
     x_src[t] = xq + (long)xrow * a.k_pad + st_chunk;
     x1_src[t] = DUAL ? a.xq[1] + (long)xrow * a.k_pad + st_chunk : nullptr;
+    x2_src[t] = TRI ? a.dual.xq2 + (long)xrow * a.k_pad + st_chunk : nullptr;
     const int o = min(tile_o * TILE + row, a.O - 1);
     w_src[t] = a.w + (long)o * a.w_ld;
   }
   const float *w_col = a.w + (long)(o_ok ? o_in : a.O - 1) * w_so; // mode 1: this lane's output column
 
-  floatx16 acc, acc1;
+  floatx16 acc, acc1, acc2;
 #pragma unroll
   for (int i = 0; i < 16; ++i) {
     acc[i] = 0.0f;
     acc1[i] = 0.0f;
+    acc2[i] = 0.0f;
   }
 
   // sample of this lane's output column and its output factor: fetched now, used by the ADC stage
@@ -446,13 +485,17 @@ __device__ __forceinline__ void mvm_round_tile(const MvmArgs &a, int round, int 
     fin_out = a.st.fin[b_out];
   }
 
-  auto gload = [&](int s, f32x4 (&gx)[4], f32x4 (&gw)[4], float (&wd)[16], f32x4 (&gx1)[4]) {
+  auto gload = [&](int s, f32x4 (&gx)[4], f32x4 (&gw)[4], float (&wd)[16], f32x4 (&gx1)[4], f32x4 (&gx2)[4]) {
     const int k0 = s * KSTEP;
 #pragma unroll
     for (int t = 0; t < 4; ++t) gx[t] = *reinterpret_cast<const f32x4 *>(x_src[t] + k0);
     if constexpr (DUAL) {
 #pragma unroll
       for (int t = 0; t < 4; ++t) gx1[t] = *reinterpret_cast<const f32x4 *>(x1_src[t] + k0);
+    }
+    if constexpr (TRI) {
+#pragma unroll
+      for (int t = 0; t < 4; ++t) gx2[t] = *reinterpret_cast<const f32x4 *>(x2_src[t] + k0);
     }
     if (WMODE == 0) {
       const int kc = min(k0 + st_chunk, K - 4); // K % 16 == 0: past K the inputs are zero padding
@@ -482,16 +525,17 @@ __device__ __forceinline__ void mvm_round_tile(const MvmArgs &a, int round, int 
       }
     }
   };
-  auto lds_store = [&](const f32x4 (&gx)[4], const f32x4 (&gw)[4], const f32x4 (&gx1)[4]) {
+  auto lds_store = [&](const f32x4 (&gx)[4], const f32x4 (&gw)[4], const f32x4 (&gx1)[4], const f32x4 (&gx2)[4]) {
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
       const int off = (t * 8 + st_row) * LDS_ROW + st_chunk;
       *reinterpret_cast<f32x4 *>(stage_x + off) = gx[t];
       if (WMODE != 1) *reinterpret_cast<f32x4 *>(stage_w + off) = gw[t];
       if constexpr (DUAL) *reinterpret_cast<f32x4 *>(stage_x1 + off) = gx1[t];
+      if constexpr (TRI) *reinterpret_cast<f32x4 *>(stage_x2 + off) = gx2[t];
     }
   };
-  auto lds_read = [&](float (&xd)[16], float (&wd)[16], float (&xd1)[16]) {
+  auto lds_read = [&](float (&xd)[16], float (&wd)[16], float (&xd1)[16], float (&xd2)[16]) {
 #pragma unroll
     for (int v4 = 0; v4 < 4; ++v4) {
       const int off = r * LDS_ROW + h * 16 + v4 * 4;
@@ -501,17 +545,22 @@ __device__ __forceinline__ void mvm_round_tile(const MvmArgs &a, int round, int 
         const f32x4 t1 = *reinterpret_cast<const f32x4 *>(stage_x1 + off);
         xd1[v4 * 4 + 0] = t1.x; xd1[v4 * 4 + 1] = t1.y; xd1[v4 * 4 + 2] = t1.z; xd1[v4 * 4 + 3] = t1.w;
       }
+      if constexpr (TRI) {
+        const f32x4 t2 = *reinterpret_cast<const f32x4 *>(stage_x2 + off);
+        xd2[v4 * 4 + 0] = t2.x; xd2[v4 * 4 + 1] = t2.y; xd2[v4 * 4 + 2] = t2.z; xd2[v4 * 4 + 3] = t2.w;
+      }
       if (WMODE != 1) {
         const f32x4 tw = *reinterpret_cast<const f32x4 *>(stage_w + off);
         wd[v4 * 4 + 0] = tw.x; wd[v4 * 4 + 1] = tw.y; wd[v4 * 4 + 2] = tw.z; wd[v4 * 4 + 3] = tw.w;
       }
     }
   };
-  auto mfma16 = [&](const float (&wd)[16], const float (&xd)[16], const float (&xd1)[16]) {
+  auto mfma16 = [&](const float (&wd)[16], const float (&xd)[16], const float (&xd1)[16], const float (&xd2)[16]) {
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
       acc = __builtin_amdgcn_mfma_f32_32x32x2f32(wd[i], xd[i], acc, 0, 0, 0);
       if constexpr (DUAL) acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(wd[i], xd1[i], acc1, 0, 0, 0);
+      if constexpr (TRI) acc2 = __builtin_amdgcn_mfma_f32_32x32x2f32(wd[i], xd2[i], acc2, 0, 0, 0);
     }
   };
 
@@ -521,60 +570,62 @@ __device__ __forceinline__ void mvm_round_tile(const MvmArgs &a, int round, int 
     // of the 16 MFMAs of step t and complete underneath them.
     f32x4 gx0[4], gw0[4], gx1[4], gw1[4], gx2[4], gw2[4], gx3[4], gw3[4];
     f32x4 hx0[4], hx1[4], hx2[4], hx3[4]; // DUAL: the rows of round 1
+    f32x4 ix0[4], ix1[4], ix2[4], ix3[4]; // TRI: the rows of round 2
     float wr0[16], wr1[16], wr2[16], wr3[16];
     float xc0[16], wc0[16], xc1[16], wc1[16];
     float yc0[16], yc1[16]; // DUAL: operands of round 1
+    float zc0[16], zc1[16]; // TRI: operands of round 2
     // step T runs from the operand registers (XC, WC); step T + 1 moves from register set (GX, GW, WR)
     // through LDS into (XN, WN) and the set is refilled with step T + 1 + PD
-#define RPU_MVM_STEP(T, GX, GW, WR, HX, XC, WC, YC, XN, WN, YN)          \
-  {                                                                      \
-    lds_store(GX, GW, HX);                                               \
-    if (WMODE == 1) {                                                    \
-      _Pragma("unroll") for (int i = 0; i < 16; ++i) WN[i] = WR[i];      \
-    }                                                                    \
-    gload(min((T) + 1 + PD, s_end - 1), GX, GW, WR, HX);                 \
-    lds_read(XN, WN, YN);                                                \
-    mfma16(WC, XC, YC);                                                  \
-    mvm_step_schedule<WMODE, DUAL>();                                    \
+#define RPU_MVM_STEP(T, GX, GW, WR, HX, IX, XC, WC, YC, ZC, XN, WN, YN, ZN) \
+  {                                                                         \
+    lds_store(GX, GW, HX, IX);                                              \
+    if (WMODE == 1) {                                                       \
+      _Pragma("unroll") for (int i = 0; i < 16; ++i) WN[i] = WR[i];         \
+    }                                                                       \
+    gload(min((T) + 1 + PD, s_end - 1), GX, GW, WR, HX, IX);                \
+    lds_read(XN, WN, YN, ZN);                                               \
+    mfma16(WC, XC, YC, ZC);                                                 \
+    mvm_step_schedule<WMODE, NACC>();                                       \
   }
-    gload(s_begin, gx0, gw0, wr0, hx0);
-    gload(min(s_begin + 1, s_end - 1), gx1, gw1, wr1, hx1);
+    gload(s_begin, gx0, gw0, wr0, hx0, ix0);
+    gload(min(s_begin + 1, s_end - 1), gx1, gw1, wr1, hx1, ix1);
     if constexpr (PD == 4) {
-      gload(min(s_begin + 2, s_end - 1), gx2, gw2, wr2, hx2);
-      gload(min(s_begin + 3, s_end - 1), gx3, gw3, wr3, hx3);
+      gload(min(s_begin + 2, s_end - 1), gx2, gw2, wr2, hx2, ix2);
+      gload(min(s_begin + 3, s_end - 1), gx3, gw3, wr3, hx3, ix3);
     }
-    lds_store(gx0, gw0, hx0);
-    lds_read(xc0, wc0, yc0);
+    lds_store(gx0, gw0, hx0, ix0);
+    lds_read(xc0, wc0, yc0, zc0);
     if (WMODE == 1) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) wc0[i] = wr0[i];
     }
-    gload(min(s_begin + PD, s_end - 1), gx0, gw0, wr0, hx0);
+    gload(min(s_begin + PD, s_end - 1), gx0, gw0, wr0, hx0, ix0);
     for (int s = s_begin; s < s_end; s += PD) {
       if constexpr (PD == 4) {
-        RPU_MVM_STEP(s, gx1, gw1, wr1, hx1, xc0, wc0, yc0, xc1, wc1, yc1)
-        RPU_MVM_STEP(s + 1, gx2, gw2, wr2, hx2, xc1, wc1, yc1, xc0, wc0, yc0)
-        RPU_MVM_STEP(s + 2, gx3, gw3, wr3, hx3, xc0, wc0, yc0, xc1, wc1, yc1)
-        RPU_MVM_STEP(s + 3, gx0, gw0, wr0, hx0, xc1, wc1, yc1, xc0, wc0, yc0)
+        RPU_MVM_STEP(s, gx1, gw1, wr1, hx1, ix1, xc0, wc0, yc0, zc0, xc1, wc1, yc1, zc1)
+        RPU_MVM_STEP(s + 1, gx2, gw2, wr2, hx2, ix2, xc1, wc1, yc1, zc1, xc0, wc0, yc0, zc0)
+        RPU_MVM_STEP(s + 2, gx3, gw3, wr3, hx3, ix3, xc0, wc0, yc0, zc0, xc1, wc1, yc1, zc1)
+        RPU_MVM_STEP(s + 3, gx0, gw0, wr0, hx0, ix0, xc1, wc1, yc1, zc1, xc0, wc0, yc0, zc0)
       } else {
-        RPU_MVM_STEP(s, gx1, gw1, wr1, hx1, xc0, wc0, yc0, xc1, wc1, yc1)
-        RPU_MVM_STEP(s + 1, gx0, gw0, wr0, hx0, xc1, wc1, yc1, xc0, wc0, yc0)
+        RPU_MVM_STEP(s, gx1, gw1, wr1, hx1, ix1, xc0, wc0, yc0, zc0, xc1, wc1, yc1, zc1)
+        RPU_MVM_STEP(s + 1, gx0, gw0, wr0, hx0, ix0, xc1, wc1, yc1, zc1, xc0, wc0, yc0, zc0)
       }
     }
 #undef RPU_MVM_STEP
   } else {
-    f32x4 gx[4], gw[4], hx[4];
-    float wn[16], xc[16], wc[16], yc[16];
-    if (s_begin < s_end) gload(s_begin, gx, gw, wn, hx);
+    f32x4 gx[4], gw[4], hx[4], ix[4];
+    float wn[16], xc[16], wc[16], yc[16], zc[16];
+    if (s_begin < s_end) gload(s_begin, gx, gw, wn, hx, ix);
     for (int s = s_begin; s < s_end; ++s) {
-      lds_store(gx, gw, hx);
-      lds_read(xc, wc, yc);
+      lds_store(gx, gw, hx, ix);
+      lds_read(xc, wc, yc, zc);
       if (WMODE == 1) {
 #pragma unroll
         for (int i = 0; i < 16; ++i) wc[i] = wn[i];
       }
-      gload(min(s + 1, s_end - 1), gx, gw, wn, hx);
-      mfma16(wc, xc, yc);
+      gload(min(s + 1, s_end - 1), gx, gw, wn, hx, ix);
+      mfma16(wc, xc, yc, zc);
     }
   }
 
@@ -601,26 +652,34 @@ __device__ __forceinline__ void mvm_round_tile(const MvmArgs &a, int round, int 
     }
     mvm_finish_outputs(a, round, b_out, fin_out, o0, v, up, lo, pre, post, DUAL ? a.dual.buf[0] : nullptr);
   }
-  int up1 = 0, lo1 = 0;
+  int up1 = 0, lo1 = 0, up2 = 0, lo2 = 0;
   if constexpr (DUAL) {
-    __syncthreads(); // the partial sums of round 0 have been read
-#pragma unroll
-    for (int i = 0; i < 16; ++i) red[wave][i][lane] = acc1[i];
-    __syncthreads();
-    float v1[4];
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const int i = wave * 4 + q;
-      v1[q] = ((red[0][i][lane] + red[1][i][lane]) + red[2][i][lane]) + red[3][i][lane];
+    // scale and output factor of the later rounds, as the sample's state will hold them if it gets there
+    bool goes_on = b_ok && o0 < a.O;
+    float nm = 0.0f, rd = 0.0f, fin_r = fin_out;
+    if (goes_on) {
+      nm = a.st.nm[b_out];
+      rd = a.st.red[b_out];
     }
-    if (b_ok && o0 < a.O) {
-      // scale and output factor of round 1, as the sample's state will hold them if it gets there
-      float nm = a.st.nm[b_out], rd = a.st.red[b_out], fin1;
-      if (next_round_params(a, 0, b_out, fin_out, nm, rd)) {
-        round_scales(a, nm, rd, fin1);
-        mvm_finish_outputs(a, 1, b_out, fin1, o0, v1, up1, lo1, nullptr, nullptr, a.dual.buf[1]);
+    auto later_round = [&](const floatx16 &acc_r, int r, float *rows, int &up_r, int &lo_r) {
+      __syncthreads(); // the partial sums of the round before have been read
+#pragma unroll
+      for (int i = 0; i < 16; ++i) red[wave][i][lane] = acc_r[i];
+      __syncthreads();
+      float vr[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int i = wave * 4 + q;
+        vr[q] = ((red[0][i][lane] + red[1][i][lane]) + red[2][i][lane]) + red[3][i][lane];
       }
-    }
+      if (goes_on) goes_on = next_round_params(a, r - 1, b_out, fin_r, nm, rd);
+      if (goes_on) {
+        round_scales(a, nm, rd, fin_r);
+        mvm_finish_outputs(a, r, b_out, fin_r, o0, vr, up_r, lo_r, nullptr, nullptr, rows);
+      }
+    };
+    later_round(acc1, 1, a.dual.buf[1], up1, lo1);
+    if constexpr (TRI) later_round(acc2, 2, a.dual.buf[2], up2, lo2);
   }
   if (!a.io.perfect && a.io.bound_management != RPU_BM_NONE) {
     // saturation flags of the tile's 32 samples: combined in LDS, then one device-scope atomic per sample
@@ -643,22 +702,26 @@ __device__ __forceinline__ void mvm_round_tile(const MvmArgs &a, int round, int 
         asm volatile("" ::"v"(old));
       }
     }
-    if constexpr (DUAL) { // the marks of round 1 (round 0 of a fused launch lists sample b at position b)
-      __syncthreads();
-      if (threadIdx.x < 2 * TILE) hits[threadIdx.x] = 0;
-      __syncthreads();
-      if (up1) atomicMax(&hits[r], up1);
-      if (lo1) atomicMax(&hits[TILE + r], lo1);
-      __syncthreads();
-      if (threadIdx.x < 2 * TILE) {
-        const int t = threadIdx.x & (TILE - 1);
-        const int hit = hits[threadIdx.x];
-        const int slot = tile_b * TILE + t;
-        if (hit && slot < n_act) {
-          const int old = atomicMax(&a.dual.hit1[(threadIdx.x < TILE ? 0 : a.m_batch) + slot], hit);
-          asm volatile("" ::"v"(old));
+    if constexpr (DUAL) { // the marks of the later rounds (round 0 of a fused launch lists sample b at position b)
+      auto later_marks = [&](int up_r, int lo_r, int *marks) {
+        __syncthreads();
+        if (threadIdx.x < 2 * TILE) hits[threadIdx.x] = 0;
+        __syncthreads();
+        if (up_r) atomicMax(&hits[r], up_r);
+        if (lo_r) atomicMax(&hits[TILE + r], lo_r);
+        __syncthreads();
+        if (threadIdx.x < 2 * TILE) {
+          const int t = threadIdx.x & (TILE - 1);
+          const int hit = hits[threadIdx.x];
+          const int slot = tile_b * TILE + t;
+          if (hit && slot < n_act) {
+            const int old = atomicMax(&marks[(threadIdx.x < TILE ? 0 : a.m_batch) + slot], hit);
+            asm volatile("" ::"v"(old));
+          }
         }
-      }
+      };
+      later_marks(up1, lo1, a.dual.hit1);
+      if constexpr (TRI) later_marks(up2, lo2, a.dual.hit2);
     }
   }
 }
@@ -803,23 +866,33 @@ __device__ __forceinline__ void mvm_init_sample(const MvmArgs &a, int b, int t, 
   }
   // the input range of a second round is known as well: its row is quantized now, while the input is at hand,
   // so that the first round has nothing to prepare
-  float next = 0.0f;
+  float next = 0.0f, next2 = 0.0f;
   if (a.rows_ahead_in_init && io.bound_management != RPU_BM_NONE) next = next_round_scale(a, 0, b, fin, nm, 1.0f);
+  if (a.dual.rounds == 3 && next != 0.0f) { // the fused launch of three rounds reads the rows of round 2 as well
+    float nm1 = nm, red1 = 1.0f, fin1 = fin;
+    if (next_round_params(a, 0, b, fin1, nm1, red1)) {
+      round_scales(a, nm1, red1, fin1);
+      next2 = next_round_scale(a, 1, b, fin1, nm1, red1);
+    }
+  }
   if (!writes) return;
   if (kept) {
     float *out0 = rows0 + (long)b * a.k_pad;
     float *out1 = rows1 + (long)b * a.k_pad;
+    float *out2 = a.dual.xq2 + (long)b * a.k_pad;
 #pragma unroll
     for (int i = 0; i < KEEP; ++i) {
       const int k = t + i * SUB;
       if (k < a.k_pad) {
         out0[k] = (k < a.K) ? dac_value(xk[i], scale, io, a.key, a.call, 0, b, k) : 0.0f;
         if (next != 0.0f) out1[k] = (k < a.K) ? dac_value(xk[i], next, io, a.key, a.call, 1, b, k) : 0.0f;
+        if (next2 != 0.0f) out2[k] = (k < a.K) ? dac_value(xk[i], next2, io, a.key, a.call, 2, b, k) : 0.0f;
       }
     }
   } else {
     write_dac_row(a, b, b, scale, 0, rows0, t, SUB);
     if (next != 0.0f) write_dac_row(a, b, b, next, 1, rows1, t, SUB);
+    if (next2 != 0.0f) write_dac_row(a, b, b, next2, 2, a.dual.xq2, t, SUB);
   }
 }
 
@@ -1115,10 +1188,14 @@ __device__ __forceinline__ void mvm_tile_finished(const MvmArgs &a, int round, i
   }
 }
 
-// The fused launch of rounds 0 and 1: the last workgroup of a sample tile decides for its 32 samples which result
-// stands (rpu_forward_backward_pass.cpp:944-983 walked twice): round 0 unless its ADC saturated and the reduction may
-// still grow, else round 1, unless that saturated too and may go on -- then the sample is listed for round 2, whose
-// rows the workgroups of this launch have written ahead (into a.dual.xq2: round 0's rows are still being read).
+// The fused launch of rounds 0 and 1 (and 2): the last workgroup of a sample tile decides for its 32 samples which
+// result stands (rpu_forward_backward_pass.cpp:944-983 walked once per fused round): round 0 unless its ADC saturated
+// and the reduction may still grow, else round 1, unless that saturated too and may go on, and so on; a sample whose
+// last fused round saturated as well is listed for the round after the launch.  With two fused rounds the workgroups of
+// the launch have written the rows of round 2 ahead (into a.dual.xq2: round 0's rows are still being read); with three
+// (the init kernel wrote those rows) a sample listed for round 3 is rare, and this workgroup writes its row now, over
+// the sample's row of round 1, which every workgroup of the sample tile has finished reading.
+template <int NACC>
 __device__ __forceinline__ void mvm_tile_finished_dual(const MvmArgs &a, int tile_b) {
   __shared__ int sh_last;
   const int tiles_o = (a.O + TILE - 1) / TILE;
@@ -1129,36 +1206,64 @@ __device__ __forceinline__ void mvm_tile_finished_dual(const MvmArgs &a, int til
   }
   __syncthreads();
   if (!sh_last) return;
+  __shared__ int sh_more, sh_more_b[TILE];
+  __shared__ float sh_more_scale[TILE];
+  if (threadIdx.x == 0) sh_more = 0;
+  __syncthreads();
   const IoDev &io = a.io;
+  constexpr int next_launch = NACC; // the first round after the fused ones
   if (threadIdx.x < TILE) {
     const int b = tile_b * TILE + threadIdx.x;
     if (b < a.m_batch) {
       const int up0 = atomicExch(&a.st.hit_up[b], 0), lo0 = atomicExch(&a.st.hit_lo[b], 0);
       const int up1 = atomicExch(&a.dual.hit1[b], 0), lo1 = atomicExch(&a.dual.hit1[a.m_batch + b], 0);
+      int up2 = 0, lo2 = 0;
+      if (NACC == 3) {
+        up2 = atomicExch(&a.dual.hit2[b], 0);
+        lo2 = atomicExch(&a.dual.hit2[a.m_batch + b], 0);
+      }
+      auto failed = [&](int up, int lo) { return io.bm_test_negative_bound ? (up > 0 || lo > 0) : (up > lo); };
       int sel = 0;
-      const bool failed0 = io.bm_test_negative_bound ? (up0 > 0 || lo0 > 0) : (up0 > lo0);
       float nm = a.st.nm[b], red = a.st.red[b];
-      if (failed0 && next_round_params(a, 0, b, a.st.fin[b], nm, red)) {
+      bool more = failed(up0, lo0) && next_round_params(a, 0, b, a.st.fin[b], nm, red);
+      if (more) {
         // the sample has run round 1
         sel = 1;
         atomicAdd(&a.st.count[1], 1); // how many did: read by the host for its choice of launches
         a.st.rounds[b] += 1;
         set_round_scales(a, b, nm, red);
-        const bool failed1 = io.bm_test_negative_bound ? (up1 > 0 || lo1 > 0) : (up1 > lo1);
-        if (failed1 && next_round_params(a, 1, b, a.st.fin[b], nm, red)) {
+        more = failed(up1, lo1) && next_round_params(a, 1, b, a.st.fin[b], nm, red);
+        if (NACC == 3 && more) { // and round 2
           sel = 2;
+          atomicAdd(&a.st.count[2], 1);
           a.st.rounds[b] += 1;
           set_round_scales(a, b, nm, red);
-          const int pos = atomicAdd(&a.st.count[2], 1);
-          a.st.list[0][pos] = b;
-          a.st.row[0][pos] = b; // written ahead at the sample's own row
-          a.st.next_scale[0][pos] = next_round_scale(a, 2, b, a.st.fin[b], nm, red);
+          more = failed(up2, lo2) && next_round_params(a, 2, b, a.st.fin[b], nm, red);
+        }
+        if (more) {
+          sel = next_launch;
+          a.st.rounds[b] += 1;
+          const float scale = set_round_scales(a, b, nm, red);
+          const int pos = atomicAdd(&a.st.count[next_launch], 1);
+          pick2(a.st.list, next_launch & 1)[pos] = b;
+          pick2(a.st.row, next_launch & 1)[pos] = b; // at the sample's own row
+          pick2(a.st.next_scale, next_launch & 1)[pos] = next_round_scale(a, next_launch, b, a.st.fin[b], nm, red);
+          if (NACC == 3) {
+            const int i = atomicAdd(&sh_more, 1);
+            sh_more_b[i] = b;
+            sh_more_scale[i] = scale;
+          }
         }
         a.st.nm[b] = nm;
         a.st.red[b] = red;
       }
       a.dual.sel[b] = sel;
     }
+  }
+  if (NACC != 3) return;
+  __syncthreads();
+  for (int i = 0; i < sh_more; ++i) {
+    write_dac_row(a, sh_more_b[i], sh_more_b[i], sh_more_scale[i], next_launch, pick2(a.xq, next_launch & 1), threadIdx.x, 256);
   }
 }
 
@@ -1172,20 +1277,24 @@ __device__ __forceinline__ void mvm_dual_select(const MvmArgs &a, int n) {
     const int b = tile_b * TILE + (idx >> 5), o = tile_o * TILE + (idx & 31);
     if (b < a.m_batch && o < a.O) {
       const int sel = a.dual.sel[b];
-      if (sel < 2) a.out[(long)b * a.out_sb + (long)o * a.out_so] = pick2(a.dual.buf, sel)[(long)b * a.O + o];
+      if (sel < a.dual.rounds) {
+        const float *kept = sel == 2 ? a.dual.buf[2] : (sel == 1 ? a.dual.buf[1] : a.dual.buf[0]);
+        a.out[(long)b * a.out_sb + (long)o * a.out_so] = kept[(long)b * a.O + o];
+      }
     }
   }
 }
 
-template <int WMODE>
+// NACC rounds in one launch, from round 0
+template <int WMODE, int NACC>
 __global__ __launch_bounds__(256) void k_mvm_dual(MvmArgs a) {
   __shared__ float red[WAVES][16][64];
-  __shared__ __attribute__((aligned(16))) float stage[WAVES * 3 * TILE * LDS_ROW];
+  __shared__ __attribute__((aligned(16))) float stage[WAVES * (NACC + 1) * TILE * LDS_ROW];
   int tile_o, tile_b;
   if (!tile_of(a, blockIdx.x, a.m_batch, tile_o, tile_b)) return;
-  mvm_prepare_next_rows<true>(a, 1, tile_o, tile_b, a.m_batch);
-  mvm_round_tile<2, WMODE, true>(a, 0, tile_o, tile_b, a.m_batch, red, stage);
-  mvm_tile_finished_dual(a, tile_b);
+  if (NACC == 2) mvm_prepare_next_rows<true>(a, 1, tile_o, tile_b, a.m_batch);
+  mvm_round_tile<2, WMODE, NACC>(a, 0, tile_o, tile_b, a.m_batch, red, stage);
+  mvm_tile_finished_dual<NACC>(a, tile_b);
 }
 
 // work of workgroup number n of a round launch of one tile
@@ -1282,7 +1391,8 @@ __device__ __forceinline__ void mvm_note_round(const MvmArgs &a, int r, int n_ac
     const int needed = (r == 1) ? n_act : a.st.count[1];
     a.dual.seen[0] = needed;
     a.dual.seen[1] = a.m_batch;
-    a.dual.seen[2] = n_act > 0 ? r : (needed > 0 ? 1 : 0);
+    // (after three fused rounds count[2] is the number of samples whose round 2 was used)
+    a.dual.seen[2] = n_act > 0 ? r : ((r == 3 && a.st.count[2] > 0) ? 2 : (needed > 0 ? 1 : 0));
   } else if (n_act > 0) {
     a.dual.seen[2] = r;
   }
@@ -2565,9 +2675,15 @@ void launch_mvm_dual(const MvmArgs &a_in, hipStream_t s) {
   a.dual.on = 1;
   const dim3 grid(mvm_round_workgroups(a));
   const int mode = weight_mode(a);
-  if (mode == 0) hipLaunchKernelGGL(k_mvm_dual<0>, grid, dim3(256), 0, s, a);
-  else if (mode == 1) hipLaunchKernelGGL(k_mvm_dual<1>, grid, dim3(256), 0, s, a);
-  else hipLaunchKernelGGL(k_mvm_dual<2>, grid, dim3(256), 0, s, a);
+  if (a.dual.rounds == 3) {
+    if (mode == 0) hipLaunchKernelGGL((k_mvm_dual<0, 3>), grid, dim3(256), 0, s, a);
+    else if (mode == 1) hipLaunchKernelGGL((k_mvm_dual<1, 3>), grid, dim3(256), 0, s, a);
+    else hipLaunchKernelGGL((k_mvm_dual<2, 3>), grid, dim3(256), 0, s, a);
+    return;
+  }
+  if (mode == 0) hipLaunchKernelGGL((k_mvm_dual<0, 2>), grid, dim3(256), 0, s, a);
+  else if (mode == 1) hipLaunchKernelGGL((k_mvm_dual<1, 2>), grid, dim3(256), 0, s, a);
+  else hipLaunchKernelGGL((k_mvm_dual<2, 2>), grid, dim3(256), 0, s, a);
 }
 
 void launch_mvm_round(const MvmArgs &a_in, hipStream_t s) {

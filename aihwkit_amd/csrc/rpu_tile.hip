@@ -185,8 +185,8 @@ struct Tile {
   // rounds 0 and 1 of a forward call in one launch: kept outputs of both, choice per sample, marks of round 1, rows of
   // round 2; the host-visible pair (samples of the last call that needed round 1, its batch) that the choice between
   // the fused and the separate launches is made from (fused_rounds: -1 by those values, 0 never, 1 .. 3 as forced)
-  DevBuf<float> s_dual0, s_dual1, s_xq2;
-  DevBuf<int> s_dsel, s_dhit1;
+  DevBuf<float> s_dual0, s_dual1, s_dual2, s_xq2;
+  DevBuf<int> s_dsel, s_dhit1, s_dhit2;
   int *seen_host = nullptr, *seen_dev = nullptr;
   int rest_from = 0, rest_quiet = 0; // the last round that listed samples in the recent calls, and calls since it did
   int fused_rounds = -1;
@@ -397,7 +397,8 @@ struct Tile {
   void release_all() {
     d_w.release(); d_wmax.release(); d_wmin.release(); d_sup.release(); d_sdown.release();
     d_slup.release(); d_sldown.release();
-    s_dual0.release(); s_dual1.release(); s_xq2.release(); s_dsel.release(); s_dhit1.release();
+    s_dual0.release(); s_dual1.release(); s_dual2.release(); s_xq2.release(); s_dsel.release(); s_dhit1.release();
+    s_dhit2.release();
     if (seen_host) {
       (void)hipHostFree(seen_host);
       seen_host = seen_dev = nullptr;
@@ -838,6 +839,7 @@ struct Tile {
       // Where most samples need a second round (as the last call on this tile showed), rounds 0 and 1 run as one
       // launch: one chain of latencies instead of two.  Results are the same either way.
       bool fuse = false;
+      int fused = 0;      // rounds of the fused launch: 2, or 3 where the recent calls listed samples for round 2
       int merge_from = 0; // > 0: the rounds from this one on run as one launch
       if (!transposed && !w_other && !side && io.p.bound_management != RPU_BM_NONE && fused_rounds != 0) {
         if (!seen_host) {
@@ -849,7 +851,7 @@ struct Tile {
         const int needed = *(volatile int *)&seen_host[0], of = *(volatile int *)&seen_host[1];
         const int last_listed = *(volatile int *)&seen_host[2];
         fuse = mvm_can_fuse_rounds(a) &&
-               (fused_rounds == 1 || fused_rounds == 3 || (fused_rounds < 0 && of > 0 && 2 * (long)needed > of));
+               ((fused_rounds > 0 && (fused_rounds & 1)) || (fused_rounds < 0 && of > 0 && 2 * (long)needed > of));
         // The last round that listed samples in the recent calls is expected to be the last one of this call too: the
         // rounds after it share a launch, whose workgroups find the first of their lists empty and leave.  The
         // estimate rises at once and falls only after eight calls below it: a round that does run inside that launch
@@ -864,9 +866,11 @@ struct Tile {
             rest_quiet = 0;
           }
         }
-        const int first_mergeable = fuse ? 2 : 1;
+        // a third round in the fused launch costs half of what its own launch does, even for a few samples
+        if (fuse) fused = (a.max_rounds >= 4 && ((fused_rounds > 0 && (fused_rounds & 4)) || (fused_rounds < 0 && rest_from >= 2))) ? 3 : 2;
+        const int first_mergeable = fuse ? fused : 1;
         if (!merged_off && mvm_can_merge_rest(a, mvm_rest_resident_limit(a))) {
-          if (fused_rounds == 2 || fused_rounds == 3) merge_from = first_mergeable;
+          if (fused_rounds > 0 && (fused_rounds & 2)) merge_from = first_mergeable;
           else if (fused_rounds < 0 && of > 0) merge_from = std::max(first_mergeable, rest_from + 1);
           if (merge_from + 1 >= a.max_rounds) merge_from = 0; // the last round alone: a plain launch
           if (merge_from > 0) {
@@ -885,6 +889,15 @@ struct Tile {
         }
         a.dual.buf[0] = s_dual0.p; a.dual.buf[1] = s_dual1.p; a.dual.sel = s_dsel.p; a.dual.hit1 = s_dhit1.p;
         a.dual.xq2 = s_xq2.p;
+        a.dual.rounds = fused;
+        if (fused == 3) {
+          s_dual2.ensure((size_t)B * a.O);
+          if (s_dhit2.n < 2 * (size_t)B) {
+            s_dhit2.ensure(2 * (size_t)B);
+            RPU_HIP_CHECK(hipMemset(s_dhit2.p, 0, s_dhit2.n * sizeof(int)));
+          }
+          a.dual.buf[2] = s_dual2.p; a.dual.hit2 = s_dhit2.p;
+        }
       }
       launch_mvm_init(a, s);
       prof_mark(s, "mvm_init");
@@ -893,10 +906,12 @@ struct Tile {
       if (fuse) {
         launch_mvm_dual(a, s);
         prof_mark(s, "mvm_round");
-        a.xq[0] = s_xq2.p; // the fused launch wrote the rows of round 2 there, at each sample's own row
-        for (int r = 2; r < a.max_rounds; ++r) {
+        // two fused rounds: the launch wrote the rows of round 2 into the third buffer, at each sample's own row; three:
+        // the row of a sample listed for round 3 replaced its row of round 1
+        if (fused == 2) a.xq[0] = s_xq2.p;
+        for (int r = fused; r < a.max_rounds; ++r) {
           a.round = r;
-          a.dual.on = r == 2 ? 2 : 0;
+          a.dual.on = r == fused ? 2 : 0;
           a.rest_in_one = (merge_from > 0 && r == merge_from) ? 1 : 0;
           launch_mvm_round(a, s);
           prof_mark(s, "mvm_round");
@@ -3296,10 +3311,10 @@ int rpu_tile_get_update_words(rpu_tile_t *tile, uint32_t *x_words_host, uint32_t
 int rpu_tile_set_fused_rounds(rpu_tile_t *tile, int mode) {
   return guarded([&] {
     if (!tile) throw RpuError("null tile");
-    if (mode < -1 || mode > 3) {
+    if (mode < -1 || mode > 7 || mode == 4 || mode == 6) {
       throw RpuError("fused rounds: mode must be -1 (by the last calls), 0 (never), 1 (rounds 0 and 1 in one launch whenever "
-                     "possible), 2 (the rounds after round 0 in one launch whenever possible) or 3 (rounds 0 and 1 in one "
-                     "launch and the rounds after them in another).");
+                     "possible), 2 (the rounds after round 0 in one launch whenever possible), 3 (rounds 0 and 1 in one "
+                     "launch and the rounds after them in another), or 5 / 7 (as 1 / 3 with round 2 in the first launch too).");
     }
     std::lock_guard<std::mutex> lock(tile->t.mutex);
     tile->t.fused_rounds = mode;

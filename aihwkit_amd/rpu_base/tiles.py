@@ -511,8 +511,8 @@ class _CudaTileMixin:
 
     def set_fused_rounds(self, mode: int = -1) -> None:
         """Fewer launches for the bound-management rounds of the forward pass: 1 = rounds 0 and 1 in one launch, 2 = all
-        rounds after round 0 in one launch, 3 = both (rounds 0 and 1, then all others), 0 = one launch per round,
-        -1 (default) = the tile decides by what its recent calls needed.  Outputs and round counts do not depend on it."""
+        rounds after round 0 in one launch, 3 = both (rounds 0 and 1, then all others), 5 / 7 = as 1 / 3 with round 2 in the
+        first launch as well, 0 = one launch per round, -1 (default) = the tile decides by what its recent calls needed.  Outputs and round counts do not depend on it."""
         check(lib().rpu_tile_set_fused_rounds(self._h, int(mode)))
 
     def set_round_wait_test_hook(self, spin_limit: int = 0, extra_arrivals: int = 0) -> None:

@@ -1,5 +1,6 @@
 """Fewer launches for the bound-management rounds of the forward pass (rpu_tile_set_fused_rounds): rounds 0 and 1 in one
-launch (mode 1), the rounds after round 0 in one launch (mode 2), both (mode 3).  Outputs and round counts must be bit
+launch (mode 1), the rounds after round 0 in one launch (mode 2), both (mode 3), rounds 0 to 2 in one launch (modes 5
+and 7).  Outputs and round counts must be bit
 for bit those of the separate launches (mode 0), which the other GPU tests hold against the oracle."""
 import numpy as np
 import pytest
@@ -19,7 +20,7 @@ def both_ways(meta, dev, x_size, d_size, w, x, seed=5, bias=False, x_trans=False
     host.set_weights(torch.from_numpy(w))
     results = []
     xin = torch.from_numpy(np.ascontiguousarray(x.T if x_trans else x)).cuda()
-    for mode in (0, 1, 2, 3):
+    for mode in (0, 1, 2, 3, 5, 7):
         gpu = tiles.CudaAnalogTile(host)
         gpu.set_fused_rounds(mode)
         gpu.set_seed(seed)
@@ -89,7 +90,7 @@ def test_the_tile_chooses_by_its_last_call(gpu_device):
         launches.append(sum(1 for name, _ms in auto.get_profile() if name == "mvm_round"))
         auto.set_profiling(False)
         assert np.array_equal(y, ref.forward(xin).cpu().numpy())
-    assert launches[0] == 5 and launches[-1] == 3            # rounds 0 + 1, round 2, and one launch for rounds 3 and 4
+    assert launches[0] == 5 and launches[-1] == 2            # rounds 0 to 2 (round 2 listed samples), and one launch for rounds 3 and 4
     quiet = x * np.float32(0.01) + 0                          # nothing saturates ...
     w_small = (w * 0.05).astype(F)
     auto.set_weights(torch.from_numpy(w_small))
