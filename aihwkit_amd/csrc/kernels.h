@@ -288,6 +288,8 @@ struct UpdateArgs {
   uint32_t *d_planes;
   int plane_slots; // slots per chunk the plane buffers are laid out for
   int n_chunks;    // ceil(m_batch / 32)
+  int *row_cost;   // [d_size] work of the pulse loop on each d row of this call (zeroed by the prepare kernel, summed by
+                   // the kernel that makes the d pulse trains); null: not kept
   int *kmax;       // kmax[0..1]: largest BL of a batch (ping-pong by call), kmax[2]: constant 31, kmax[3]: longest line
                    // among pulse words made elsewhere (launch_words_kmax)
   int kmax_slot;   // which entry this call uses

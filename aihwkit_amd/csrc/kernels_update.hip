@@ -147,6 +147,9 @@ __device__ __forceinline__ void update_prepare_sample(const UpdateArgs &a, const
 template <int SUB>
 __global__ __launch_bounds__(256) void k_update_prepare(UpdateArgs a) {
   __shared__ float sh[2][4];
+  if (a.row_cost) {
+    for (int i = (int)(blockIdx.x * 256u + threadIdx.x); i < a.d_size; i += (int)(gridDim.x * 256u)) a.row_cost[i] = 0;
+  }
   const int b = (int)blockIdx.x * (256 / SUB) + (int)threadIdx.x / SUB;
   if (b >= a.m_batch) return; // all SUB threads of a sample leave together
   update_prepare_sample<SUB>(a, b, sh);
@@ -234,13 +237,19 @@ __device__ __forceinline__ void update_lines_block(const UpdateArgs &a, const in
     if (e >= size) break; // wave-uniform
     const uint32_t word = b_ok ? pulse_word(a, is_x, e, sample, vals[lane][el], P, K, wrow) : 0u;
     wt[lane][el] = word;
+    unsigned long long any = 0ull;
+    int passes = 0;
     for (int k = 0; k < kmax; ++k) {
       const unsigned long long m = __ballot((word >> (k + 1)) & 1u);
+      any |= m;
+      passes += __popcll(m);
       if (lane == 0) {
         planes[((long)c0 * a.plane_slots + k) * size + e] = (uint32_t)m;
         if (c0 + 1 < a.n_chunks) planes[((long)(c0 + 1) * a.plane_slots + k) * size + e] = (uint32_t)(m >> 32);
       }
     }
+    // what the pulse loop will spend on this d row for these samples: a pass per pulse, a set-up per sample with pulses
+    if (!is_x && a.row_cost && lane == 0 && passes) atomicAdd(&a.row_cost[e], 9 * passes + 4 * __popcll(any));
     const unsigned long long sg = __ballot(word & 1u); // the last slot of a chunk holds the sign bits
     if (lane == 0) {
       const int ks = a.plane_slots - 1;
@@ -845,11 +854,13 @@ __device__ __forceinline__ float pulsed_gather(const UpdateArgs &a, float w, con
 // the batch.
 // bx: the workgroup's block of 256 C columns, i: its row; tbl: the noise factors 1 + std * quantile in LDS
 // DEEP: the planes of eight chunks are fetched at a time (PulsedRows::run_blocks; short bit lines, one column per lane)
+// tid: number of the thread among the 256 that share the row
 template <int KIND, bool MULT, bool NOISE, int C, bool DEEP>
-__device__ __forceinline__ void update_pulsed_row(const UpdateArgs &a, const int bx, const int i, float *tbl) {
+__device__ __forceinline__ void update_pulsed_row(const UpdateArgs &a, const int bx, const int i, float *tbl,
+                                                  const int tid = (int)threadIdx.x) {
   if (NOISE) {
     static_assert(CTOC_LEVELS == 256, "one table entry per thread");
-    tbl[threadIdx.x] = __builtin_fmaf(a.dev.dw_min_std, g_ctoc_xi[threadIdx.x], 1.0f);
+    if (threadIdx.x < CTOC_LEVELS) tbl[threadIdx.x] = __builtin_fmaf(a.dev.dw_min_std, g_ctoc_xi[threadIdx.x], 1.0f);
     __syncthreads();
   }
   int j[C];
@@ -859,7 +870,7 @@ __device__ __forceinline__ void update_pulsed_row(const UpdateArgs &a, const int
   float w[C];
 #pragma unroll
   for (int c = 0; c < C; ++c) {
-    const int jt = (bx * C + c) * 256 + threadIdx.x;
+    const int jt = (bx * C + c) * 256 + tid;
     valid[c] = jt < a.x_size;
     j[c] = valid[c] ? jt : a.x_size - 1;
     cell[c] = (unsigned)i * (unsigned)a.x_size + (unsigned)j[c];
@@ -903,6 +914,62 @@ __global__ __launch_bounds__(256, ((C > 1 || DEEP) ? 4 : 8)) void k_update_pulse
     row = (row & 7) * band + (row >> 3);
   }
   update_pulsed_row<KIND, MULT, NOISE, C, DEEP>(a, (int)blockIdx.x, row, tbl);
+}
+
+// The same pulse loop with the rows dealt out by their work.  The time a row takes follows its number of d pulses, which
+// varies by several percent between rows, and a CU holds four rows at a time: whichever CU draws four long ones sets
+// the kernel's time.  Here a workgroup of 1024 threads fills a CU and takes four rows, one per 256 threads, chosen so
+// that every workgroup has the same work: workgroup n (on XCD n % 8) belongs to the band of d_size / 8 consecutive rows
+// of its XCD, ranks the band's rows by a.row_cost (ties by row number: every workgroup of the band finds the same
+// order) and takes, as number s of the band's S = d_size / 32 workgroups, the ranks s, 2 S - 1 - s, 2 S + s and
+// 4 S - 1 - s.  Rows of a band in one L2 also keep the strided stores of UpdateArgs::w_out together.
+// For four columns per lane, rows of at most 1024 columns, d_size a multiple of 256 (bands of whole groups of 32 rows).  Which row a group of threads works
+// on changes nothing in the result of the row.
+constexpr int BALANCED_MAX_BAND = 1024;
+template <int KIND, bool MULT, bool NOISE>
+__global__ __launch_bounds__(1024) void k_update_pulsed_balanced(UpdateArgs a) {
+  __shared__ float tbl[CTOC_LEVELS];
+  __shared__ int cost[BALANCED_MAX_BAND];
+  __shared__ int order[BALANCED_MAX_BAND];
+  const int band = a.d_size >> 3, per_band = band >> 2;
+  const int xcd = (int)blockIdx.x & 7, s = (int)blockIdx.x >> 3;
+  const int row0 = xcd * band;
+  for (int t = (int)threadIdx.x; t < band; t += 1024) {
+    cost[t] = a.row_cost[row0 + t];
+    order[t] = 0; // first the rank of row t, summed from the parts below
+  }
+  __syncthreads();
+  // rank of a row = rows of the band that come before it; the threads split the comparisons, 32 rows each
+  for (int idx = (int)threadIdx.x; idx < band * (band >> 5); idx += 1024) {
+    const int t = idx % band, u0 = (idx / band) << 5;
+    const int mine = cost[t];
+    int before = 0;
+#pragma unroll 8
+    for (int u = u0; u < u0 + 32; ++u) {
+      const int c = cost[u];
+      before += (c < mine || (c == mine && u < t)) ? 1 : 0;
+    }
+    atomicAdd(&order[t], before);
+  }
+  __syncthreads();
+  int rank_of[BALANCED_MAX_BAND / 1024];
+#pragma unroll
+  for (int q = 0; q < BALANCED_MAX_BAND / 1024; ++q) {
+    const int t = (int)threadIdx.x + 1024 * q;
+    rank_of[q] = t < band ? order[t] : 0;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int q = 0; q < BALANCED_MAX_BAND / 1024; ++q) {
+    const int t = (int)threadIdx.x + 1024 * q;
+    if (t < band) order[rank_of[q]] = t;
+  }
+  __syncthreads();
+  const int g = (int)threadIdx.x >> 8;
+  const int rank = (g & 1) ? (g + 1) * per_band - 1 - s : g * per_band + s;
+  // the same for the 256 threads of a row: kept in a scalar register, like a row number taken from the grid
+  const int row = __builtin_amdgcn_readfirstlane(row0 + order[rank]);
+  update_pulsed_row<KIND, MULT, NOISE, 4, false>(a, 0, row, tbl, (int)threadIdx.x & 255);
 }
 
 // Several tiles in one launch (same device kind, noise and columns per lane): start[t] .. start[t + 1] are the
@@ -1365,7 +1432,25 @@ void launch_update_planes(const UpdateArgs &a, hipStream_t s) {
   hipLaunchKernelGGL(k_update_planes, grid, dim3(256), 0, s, a);
 }
 
+// whether the launch that deals the rows out by their work serves this call (see k_update_pulsed_balanced): only
+// where its workgroups, a quarter as many as rows, still fill the chip
+bool update_pulsed_balanced(const UpdateArgs &a, int columns) {
+  return columns == 4 && a.row_cost && a.x_size <= 1024 && a.d_size >= 1024 && a.d_size % 256 == 0 &&
+         a.d_size / 8 <= BALANCED_MAX_BAND;
+}
+
 template <bool NOISE, int C, bool DEEP = false> static void launch_update_pulsed_t(const UpdateArgs &a, hipStream_t s) {
+  if (C == 4 && !DEEP && update_pulsed_balanced(a, C)) {
+    const dim3 grid(a.d_size / 4);
+    if (a.dev.kind == RPU_DEVICE_CONSTANT_STEP) {
+      hipLaunchKernelGGL((k_update_pulsed_balanced<RPU_DEVICE_CONSTANT_STEP, true, NOISE>), grid, dim3(1024), 0, s, a);
+    } else if (a.dev.ls_mult_noise) {
+      hipLaunchKernelGGL((k_update_pulsed_balanced<RPU_DEVICE_LINEAR_STEP, true, NOISE>), grid, dim3(1024), 0, s, a);
+    } else {
+      hipLaunchKernelGGL((k_update_pulsed_balanced<RPU_DEVICE_LINEAR_STEP, false, NOISE>), grid, dim3(1024), 0, s, a);
+    }
+    return;
+  }
   dim3 grid((a.x_size + 256 * C - 1) / (256 * C), a.d_size);
   if (a.dev.kind == RPU_DEVICE_CONSTANT_STEP) {
     hipLaunchKernelGGL((k_update_pulsed<RPU_DEVICE_CONSTANT_STEP, true, NOISE, C, DEEP>), grid, dim3(256), 0, s, a);

@@ -217,7 +217,7 @@ struct Tile {
   }
   DevBuf<int> s_rounds, s_hitup, s_hitlo, s_list0, s_list1, s_row0, s_row1, s_count, s_tiledone;
   // update scratch
-  DevBuf<int> u_bl;
+  DevBuf<int> u_bl, u_rowcost;
   DevBuf<float> u_a, u_b, u_xval, u_dval;
   DevBuf<uint32_t> u_xw, u_dw, u_xpl, u_dpl;
   DevBuf<int> u_kmax;
@@ -405,6 +405,7 @@ struct Tile {
     }
     s_nsc0.release(); s_nsc1.release(); s_nm.release(); s_nmnp.release(); s_red.release(); s_scale.release(); s_fin.release(); s_bias.release(); s_xq0.release(); s_xq1.release();
     s_rounds.release(); s_hitup.release(); s_hitlo.release(); s_list0.release(); s_list1.release(); s_row0.release(); s_row1.release(); s_count.release(); s_tiledone.release();
+    u_rowcost.release();
     u_bl.release(); u_a.release(); u_b.release(); u_xval.release(); u_dval.release(); u_xw.release(); u_dw.release();
     u_xpl.release(); u_dpl.release(); u_kmax.release();
     r_wmax.release(); r_wmin.release(); r_sup.release(); r_sdown.release(); r_slup.release(); r_sldown.release(); u_wrm.release();
@@ -945,13 +946,14 @@ struct Tile {
     };
     const size_t chunks = ((size_t)B + 31) / 32, slots = 32;
     int *kmax = (int *)take(4 * sizeof(int));
+    int *row_cost = (int *)take((size_t)D * 4);
     int *bl = (int *)take((size_t)B * 4);
     float *pa = (float *)take((size_t)B * 4), *pb = (float *)take((size_t)B * 4);
     uint32_t *xw = (uint32_t *)take((size_t)B * X * 4), *dw = (uint32_t *)take((size_t)B * D * 4);
     uint32_t *xpl = (uint32_t *)take(chunks * slots * X * 4), *dpl = (uint32_t *)take(chunks * slots * D * 4);
     float *rows = bias ? (float *)take((size_t)B * X * 4) : nullptr;
     if (a) {
-      a->kmax = kmax; a->bl = bl; a->prob_a = pa; a->prob_b = pb; a->x_words = xw; a->d_words = dw;
+      a->kmax = kmax; a->row_cost = row_cost; a->bl = bl; a->prob_a = pa; a->prob_b = pb; a->x_words = xw; a->d_words = dw;
       a->x_planes = xpl; a->d_planes = dpl; a->plane_slots = (int)slots; a->n_chunks = (int)chunks;
     }
     if (bias_rows) *bias_rows = rows;
@@ -1439,6 +1441,8 @@ struct Tile {
         a.x_words = u_xw.p; a.d_words = u_dw.p;
         set_plane_args(a, rows);
         a.kmax_slot = (int)(update_calls++ & 1u);
+        u_rowcost.ensure((size_t)D);
+        a.row_cost = u_rowcost.p;
       } else {
         u_xval.ensure((size_t)B * X); u_dval.ensure((size_t)B * D);
         a.x_val = u_xval.p; a.d_val = u_dval.p;
@@ -1533,7 +1537,9 @@ struct Tile {
   // arguments of the plain pulsed update on this tile's own weights (see group_update_obstacle)
   UpdateArgs group_update_args(const float *x, long x_ld, const float *d, long d_ld, int B, hipStream_t s, int &wps) {
     DeviceView dv{wp_dev(), d_wmax.p, d_wmin.p, d_sup.p, d_sdown.p, d_slup.p, d_sldown.p, &dev, dev.p.dw_min};
-    return pulsed_update_args(dv, up, lr, x, x_ld, 1, d, d_ld, 1, B, s, nullptr, wps);
+    UpdateArgs a = pulsed_update_args(dv, up, lr, x, x_ld, 1, d, d_ld, 1, B, s, nullptr, wps);
+    a.row_cost = nullptr; // the group launches deal the rows out in their order
+    return a;
   }
 
   // The stochastic pulsed update without any allocation: every buffer beyond inputs and weights lives in the
