@@ -30,17 +30,17 @@ FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix
 
 # Counter values at configuration 2 from rocprofv3 runs of `bench.py --pmc` (one run per counter group; the summaries,
 # with the commands, are under profiles/).  They are constants of this file, not measured in a benchmark run, and
-# the JSON line says so ("traffic_source", "instructions_source").
+# the JSON line says so ("traffic_source").
 # FETCH_SIZE / WRITE_SIZE are KiB per dispatch; a device copy of 64 MiB in the same runs reads FETCH_SIZE = 32782 and
 # WRITE_SIZE = 65536, so FETCH_SIZE is scaled by 2.0 and WRITE_SIZE by 1.0.
 PMC_TRAFFIC_BYTES = {
-    "k_update_pulsed": (15936 * 2.0 + 4096 * 1.0) * 1024,
+    "k_update_pulsed": (15063 * 2.0 + 4096 * 1.0) * 1024,
     "k_mvm_round": (6851 * 2.0 + 2115 * 1.0) * 1024,  # a round over all 256 samples
+    # the launches of a forward call whose rounds 0 to 2 share one launch: k_mvm_dual<0, 3>, then k_mvm_rounds_rest
+    "forward_fused_3": ((14557 + 586) * 2.0 + (3157 + 1024) * 1.0) * 1024,
 }
-PMC_SOURCE = {"k_update_pulsed": "profiles/k_update_pulsed_config2.txt", "k_mvm_round": "profiles/k_mvm_round_config2.txt"}
-# vector-ALU instructions of one k_update_pulsed launch at configuration 2 (SQ_INSTS_VALU summed over its 4096 waves)
-PMC_VALU_INSTS = {"k_update_pulsed": 21947648}
-VALU_PEAK_GINST = 256 * 4 * 2.4 / 4.0  # wave-instructions per ns: 1024 SIMDs, one wave64 instruction per 4 cycles at 2.4 GHz
+PMC_SOURCE = {"k_update_pulsed": "profiles/k_update_pulsed_config2.txt", "k_mvm_round": "profiles/k_mvm_round_config2.txt",
+              "forward_fused_3": "profiles/k_mvm_dual_config2.txt"}
 
 
 def batch_sweep() -> int:
@@ -160,12 +160,13 @@ def main() -> int:
         torch.cuda.synchronize()
         dst.copy_(src)
         torch.cuda.synchronize()
-        for _ in range(3):
-            tile.update(xg, dg, False, False, False, False)
+        # forward first, on the stated weights (updates change them, and with them the rounds a forward call needs)
         for _ in range(3):
             tile.forward(xg, False, False, False, False, False)
         for _ in range(3):
             tile.backward(dg, False, False, False, False)
+        for _ in range(3):
+            tile.update(xg, dg, False, False, False, False)
         if args.config == 2:
             tile_v = tiles.CudaAnalogTile(host)
             tile_v.set_learning_rate(lr)
@@ -182,7 +183,7 @@ def main() -> int:
                 tile.forward(xb, False, False, False, False, False)
             for _ in range(2):
                 tile.backward(db, False, False, False, False)
-        print("pmc run done: 1 copy of 64 MiB, 3 update, 3 forward, 3 backward calls, 3 update calls of the aggregated "
+        print("pmc run done: 1 copy of 64 MiB, 3 forward, 3 backward, 3 update calls, 3 update calls of the aggregated "
               "variant, then (unless --no-other-batches) 2 forward and 2 backward calls at batch 16384", file=sys.stderr)
         return 0
 
@@ -418,6 +419,8 @@ def main() -> int:
     k_update_ms = prof_update["update_pulsed"][0]
     k_fwd_ms = prof_forward["mvm_round"][0]   # all round launches of one forward call
     fused_forward = prof_forward["mvm_round"][1] < 5 and args.config == 2  # rounds 0 and 1 ran as one launch
+    fused_3 = fused_forward and prof_forward["mvm_round"][1] == 2           # rounds 0 to 2, then one launch for the rest
+    fwd_traffic = "forward_fused_3" if fused_3 else ("k_mvm_round" if args.config == 2 and not fused_forward else None)
     k_bwd_ms = prof_backward["mvm_round"][0]
 
     out = {
@@ -437,13 +440,14 @@ def main() -> int:
                    "step": "initial weights restored (4 MB device copy, timed) + forward + backward + update on the next "
                            "of %d pre-uploaded input batches" % POOL,
                    "mean_bm_rounds_in_step_loop": loop_rounds},
-        "update": {"ms_per_call": ms_update, "kernels_ms": {k: v[0] for k, v in prof_update.items()}},
+        "update": {"ms_per_call": ms_update, "kernels_ms": {k: v[0] for k, v in prof_update.items()},
+                   "pulses_per_call": pulses, "pulses_per_cross_point": pulses / (x_size * d_size)},
         "forward": {"ms_per_call": ms_forward, "gflops": flops_per_call / (ms_forward * 1e-3) / 1e9,
                     "mean_bm_rounds": float(rounds.mean()), "kernels_ms": {k: v[0] for k, v in prof_forward.items()},
                     "round_launches": prof_forward["mvm_round"][1],
-                    "note": "with most samples in a second round the tile runs rounds 0 and 1 as one launch, with none "
-                            "the rounds after round 0 as one launch (rpu_tile_set_fused_rounds, default: by what its "
-                            "last call needed); same outputs"},
+                    "note": "with most samples in a second round the tile runs rounds 0 and 1 as one launch (round 2 as well "
+                            "when its recent calls listed samples for it), with none the rounds after round 0 as one "
+                            "launch (rpu_tile_set_fused_rounds, default: by what its last calls needed); same outputs"},
         "backward": {"ms_per_call": ms_backward, "gflops": flops_per_call / (ms_backward * 1e-3) / 1e9,
                      "kernels_ms": {k: v[0] for k, v in prof_backward.items()}},
         "roofline": {"kernel": "k_update_pulsed", "bound": "hbm", "achieved": update_bytes / (k_update_ms * 1e-3) / 1e9,
@@ -453,29 +457,19 @@ def main() -> int:
                      "traffic_source": ("constant from " + PMC_SOURCE["k_update_pulsed"] + " (rocprofv3 --pmc FETCH_SIZE / "
                                         "WRITE_SIZE), not measured in this run") if args.config == 2 else None,
                      "algorithmic_bytes": update_bytes, "kernel_ms": k_update_ms},
-        "roofline_forward": {"kernel": "k_mvm_dual + k_mvm_round (all rounds of a call)" if fused_forward
+        "roofline_forward": {"kernel": "k_mvm_dual + k_mvm_rounds_rest (all rounds of a call)" if fused_forward
                              else "k_mvm_round (all rounds of a call)", "bound": "mfma",
                              "achieved": flops_per_call / (k_fwd_ms * 1e-3) / 1e12, "peak": FP32_MFMA_PEAK_TFLOPS,
                              "unit": "TFLOP/s", "frac": flops_per_call / (k_fwd_ms * 1e-3) / 1e12 / FP32_MFMA_PEAK_TFLOPS,
-                             "traffic": PMC_TRAFFIC_BYTES["k_mvm_round"] if args.config == 2 and not fused_forward else None,
-                             "traffic_source": ("constant from " + PMC_SOURCE["k_mvm_round"] + ", not measured in this run")
-                             if args.config == 2 and not fused_forward else None,
+                             "traffic": PMC_TRAFFIC_BYTES[fwd_traffic] if fwd_traffic else None,
+                             "traffic_source": ("constant from " + PMC_SOURCE[fwd_traffic] + ", not measured in this run")
+                             if fwd_traffic else None,
                              "algorithmic_flops": flops_per_call, "kernel_ms": k_fwd_ms},
         "roofline_backward": {"kernel": "k_mvm_round", "bound": "mfma",
                               "achieved": flops_per_call / (k_bwd_ms * 1e-3) / 1e12, "peak": FP32_MFMA_PEAK_TFLOPS,
                               "unit": "TFLOP/s", "frac": flops_per_call / (k_bwd_ms * 1e-3) / 1e12 / FP32_MFMA_PEAK_TFLOPS,
                               "kernel_ms": k_bwd_ms},
     }
-    if args.config == 2:
-        # what actually bounds the per-pulse kernel: vector-ALU issue (one wave64 instruction per SIMD and 4 cycles)
-        insts = float(PMC_VALU_INSTS["k_update_pulsed"])
-        out["roofline_valu"] = {
-            "kernel": "k_update_pulsed", "bound": "valu issue", "achieved": insts / (k_update_ms * 1e6), "peak": VALU_PEAK_GINST,
-            "unit": "wave-instructions/ns", "frac": insts / (k_update_ms * 1e6) / VALU_PEAK_GINST,
-            "instructions": insts, "instructions_source": "constant from " + PMC_SOURCE["k_update_pulsed"] +
-            " (rocprofv3 --pmc SQ_INSTS_VALU), not measured in this run",
-            "pulses_per_call": pulses, "pulses_per_cross_point": pulses / (x_size * d_size),
-            "wave_instructions_per_pulse": insts / pulses, "lane_instructions_per_pulse": 64.0 * insts / pulses}
     out["config"]["storage"] = args.storage
     if xd_block is not None:
         out["storage_xd_shared"] = xd_block
