@@ -2005,7 +2005,9 @@ typedef int i32x4_unaligned __attribute__((ext_vector_type(4), aligned(4)));
 // ONE_STEP: the patch row fits one contraction step (K <= 32, a first convolution layer): the gathered values stay
 // in registers between noise management and the rounds.
 // STOCH: the DAC or the ADC draws random numbers beyond the output noise (see dac_value, mvm_adc_values).
-template <bool ONE_STEP, bool STOCH>
+// WOC: the stored matrix holds the outputs of one k per row (MvmArgs::w_oc); a kernel instance per addressing, so that
+// neither carries the other's registers.
+template <bool ONE_STEP, bool STOCH, bool WOC = false>
 __global__ __launch_bounds__(256, STOCH ? 2 : 3) void k_conv_forward(MvmArgs a, ConvArgs c) {
   const int lane = threadIdx.x & 63;
   const int r = lane & 31, h = lane >> 5;
@@ -2019,7 +2021,7 @@ __global__ __launch_bounds__(256, STOCH ? 2 : 3) void k_conv_forward(MvmArgs a, 
   const int p = (int)(sample - (long)n * c.patches);
   const float *image = c.images + (long)n * c.image_size;
   const int *idx_row = c.idx_t + (long)p * a.K;
-  const float *w_row = a.w + (long)min(r, a.O - 1) * (a.w_oc ? 1 : a.w_ld); // w_oc: the lane's output column
+  const float *w_row = a.w + (long)min(r, a.O - 1) * (WOC ? 1 : a.w_ld); // WOC: the lane's output column
   const int K = a.K, O = a.O;
   const int steps = ONE_STEP ? 1 : (K + 31) / 32;
   const IoDev &io = a.io;
@@ -2043,9 +2045,14 @@ __global__ __launch_bounds__(256, STOCH ? 2 : 3) void k_conv_forward(MvmArgs a, 
     }
   };
   auto weights16 = [&](int k0, float (&w)[16]) __attribute__((always_inline)) {
-    if (a.w_oc) { // rows of the stored matrix hold the outputs of one k (wave-uniform choice)
+    if constexpr (WOC) { // rows of the stored matrix hold the outputs of one k: a uniform row address + the lane's column
+      const unsigned col = (unsigned)min(r, O - 1);
 #pragma unroll
-      for (int i = 0; i < 16; ++i) w[i] = (k0 + i < K) ? w_row[(long)(k0 + i) * a.w_ld] : 0.0f;
+      for (int i = 0; i < 16; ++i) w[i] = (a.w + (long)min(k0 + i, K - 1) * a.w_ld)[col];
+      if (k0 + 16 > K) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) w[i] = (k0 + i < K) ? w[i] : 0.0f;
+      }
     } else
 #pragma unroll
     for (int v4 = 0; v4 < 4; ++v4) {
@@ -2172,7 +2179,7 @@ __global__ __launch_bounds__(256, STOCH ? 2 : 3) void k_conv_forward(MvmArgs a, 
 // Long patch rows (more than two contraction steps): one workgroup per 32 patches, its four waves share the patches
 // and deal the contraction steps among themselves (partial sums added through LDS in a fixed order, each wave then
 // finishes 8 of the 32 output rows).  Every wave keeps the per-patch state, so the round loop is workgroup-uniform.
-template <bool STOCH>
+template <bool STOCH, bool WOC = false>
 __global__ __launch_bounds__(256, 4) void k_conv_forward_split(MvmArgs a, ConvArgs c) {
   __shared__ float red[WAVES][16][64];
   __shared__ float sh_max[2][WAVES][32];
@@ -2188,7 +2195,7 @@ __global__ __launch_bounds__(256, 4) void k_conv_forward_split(MvmArgs a, ConvAr
   const int p = (int)(sample - (long)n * c.patches);
   const float *image = c.images + (long)n * c.image_size;
   const int *idx_row = c.idx_t + (long)p * a.K;
-  const float *w_row = a.w + (long)min(r, a.O - 1) * (a.w_oc ? 1 : a.w_ld); // w_oc: the lane's output column
+  const float *w_row = a.w + (long)min(r, a.O - 1) * (WOC ? 1 : a.w_ld); // WOC: the lane's output column
   const int K = a.K, O = a.O;
   const int steps = (K + 31) / 32;
   const IoDev &io = a.io;
@@ -2211,9 +2218,14 @@ __global__ __launch_bounds__(256, 4) void k_conv_forward_split(MvmArgs a, ConvAr
     }
   };
   auto weights16 = [&](int k0, float (&w)[16]) __attribute__((always_inline)) {
-    if (a.w_oc) { // rows of the stored matrix hold the outputs of one k (wave-uniform choice)
+    if constexpr (WOC) { // rows of the stored matrix hold the outputs of one k: a uniform row address + the lane's column
+      const unsigned col = (unsigned)min(r, O - 1);
 #pragma unroll
-      for (int i = 0; i < 16; ++i) w[i] = (k0 + i < K) ? w_row[(long)(k0 + i) * a.w_ld] : 0.0f;
+      for (int i = 0; i < 16; ++i) w[i] = (a.w + (long)min(k0 + i, K - 1) * a.w_ld)[col];
+      if (k0 + 16 > K) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) w[i] = (k0 + i < K) ? w[i] : 0.0f;
+      }
     } else
 #pragma unroll
     for (int v4 = 0; v4 < 4; ++v4) {
@@ -2781,15 +2793,18 @@ void launch_conv_forward(const MvmArgs &a, const ConvArgs &c, hipStream_t s) {
   const long tiles = ((long)c.n_images * c.patches + 31) / 32;
   const dim3 grid((unsigned)((tiles + 3) / 4));
   const bool stoch = !a.io.perfect && (a.io.inp_sto_round || a.io.out_sto_round || a.io.inp_noise > 0.0f);
-  if (stoch) {
-    if (a.K <= 32) hipLaunchKernelGGL((k_conv_forward<true, true>), grid, dim3(256), 0, s, a, c);
-    else if (a.K <= 64) hipLaunchKernelGGL((k_conv_forward<false, true>), grid, dim3(256), 0, s, a, c);
-    else hipLaunchKernelGGL(k_conv_forward_split<true>, dim3((unsigned)tiles), dim3(256), 0, s, a, c);
-  } else {
-    if (a.K <= 32) hipLaunchKernelGGL((k_conv_forward<true, false>), grid, dim3(256), 0, s, a, c);
-    else if (a.K <= 64) hipLaunchKernelGGL((k_conv_forward<false, false>), grid, dim3(256), 0, s, a, c);
-    else hipLaunchKernelGGL(k_conv_forward_split<false>, dim3((unsigned)tiles), dim3(256), 0, s, a, c);
+#define RPU_LAUNCH_CONV(STOCH, WOC)                                                                                  \
+  {                                                                                                                   \
+    if (a.K <= 32) hipLaunchKernelGGL((k_conv_forward<true, STOCH, WOC>), grid, dim3(256), 0, s, a, c);              \
+    else if (a.K <= 64) hipLaunchKernelGGL((k_conv_forward<false, STOCH, WOC>), grid, dim3(256), 0, s, a, c);        \
+    else hipLaunchKernelGGL((k_conv_forward_split<STOCH, WOC>), dim3((unsigned)tiles), dim3(256), 0, s, a, c);       \
   }
+  if (stoch) {
+    if (a.w_oc) RPU_LAUNCH_CONV(true, true) else RPU_LAUNCH_CONV(true, false)
+  } else {
+    if (a.w_oc) RPU_LAUNCH_CONV(false, true) else RPU_LAUNCH_CONV(false, false)
+  }
+#undef RPU_LAUNCH_CONV
 }
 
 void launch_make_bias(const float *in, float *out, int m_batch, int x_size, int in_trans, hipStream_t s) {
