@@ -634,7 +634,8 @@ int rpu_tile_get_shared_weights_if(const rpu_tile_t *tile);
  * way round where inputs are denser than errors): the tile keeps row-major copies of the device parameters for it, the
  * launch that makes the pulse trains also makes a row-major scratch copy of the weights, and the loop stores its
  * results straight into the tensor.  Results are bit for bit those of the row-major tile (same pulse trains, same noise
- * draws per cross-point, same ADC draws).  Host-side interfaces (get / set weights, hidden parameters, ...) stay
+ * draws per cross-point, same ADC draws) for forward, backward and the stochastic pulse loop; the deterministic-implicit
+ * update keys its cycle-to-cycle noise by storage position, so with that noise on its weights agree statistically.  Host-side interfaces (get / set weights, hidden parameters, ...) stay
  * [d_size][x_size]; rpu_tile_weights_device_ptr returns the tensor.  Such tiles can be members of a group when all
  * members are bound that way.
  * The other kinds of tile keep their row-major matrix and mirror it: the tensor takes the tile's weights when it is
@@ -669,11 +670,15 @@ int rpu_tile_set_extra(rpu_tile_t *tile, const int64_t *values_host, int count);
  *      microseconds) and leave when the next round lists no sample; a round that does follow inside that launch waits for
  *      all workgroups once more, with the rows and lists of the round before made visible device-wide, which costs more
  *      than a launch;
- *   3  both: rounds 0 and 1 as one launch, the rounds after them as another.
+ *   3  both: rounds 0 and 1 as one launch, the rounds after them as another;
+ *   5, 7  as 1 and 3 with round 2 in the first launch as well (a third result from the same weights; needs at least
+ *      four rounds to be possible): pays as soon as a call lists any sample for round 2, whose own launch costs more
+ *      than the extra matrix work.
  * Mode -1 (default): the tile chooses by what its recent forward calls needed -- more than half of the samples in a
- * second round: rounds 0 and 1 in one launch; and the rounds after the last one that listed any sample in those calls
+ * second round: rounds 0 and 1 in one launch, and round 2 with them when those calls listed samples for it; and the
+ * rounds after the last one that listed any sample in those calls
  * (the estimate rises at once and falls after eight calls below it), which are expected to be empty, share one
- * launch.  0: always the separate launches.  1 / 2 / 3: that shortcut whenever the shape allows it
+ * launch.  0: always the separate launches.  1 / 2 / 3 / 5 / 7: that shortcut whenever the shape allows it
  * (single tile, rounds on the 32 x 32 kernel, for 2 and 3 no more workgroups than the GPU holds of that kernel at once
  * -- what the occupancy query reports per CU times the CUs --, no per-line periphery terms).
  * The waits of shortcut 2 are bounded (some tens of milliseconds).  They assume that the launch has the GPU's CUs to
