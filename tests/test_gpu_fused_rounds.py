@@ -15,12 +15,12 @@ F = np.float32
 NM, BM = dv.NoiseManagementType, dv.BoundManagementType
 
 
-def both_ways(meta, dev, x_size, d_size, w, x, seed=5, bias=False, x_trans=False, d_trans=False, calls=2):
+def both_ways(meta, dev, x_size, d_size, w, x, seed=5, bias=False, x_trans=False, d_trans=False, calls=3):
     host, _orc, _ = build_pair(meta, dev, x_size, d_size, gpu=False)
     host.set_weights(torch.from_numpy(w))
     results = []
     xin = torch.from_numpy(np.ascontiguousarray(x.T if x_trans else x)).cuda()
-    for mode in (0, 1, 2, 3, 5, 7):
+    for mode in (0, 1, 2, 3, 5, 7, -1):              # -1: the tile's own choice, which changes from call to call
         gpu = tiles.CudaAnalogTile(host)
         gpu.set_fused_rounds(mode)
         gpu.set_seed(seed)
