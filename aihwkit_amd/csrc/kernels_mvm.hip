@@ -684,44 +684,41 @@ __device__ __forceinline__ void mvm_round_tile(const MvmArgs &a, int round, int 
   if (!a.io.perfect && a.io.bound_management != RPU_BM_NONE) {
     // saturation flags of the tile's 32 samples: combined in LDS, then one device-scope atomic per sample
     // and bound.  The returned values are consumed so that the wave waits until the atomics have been
-    // performed before the workgroup signals its tile as finished (mvm_tile_finished).
+    // performed before the workgroup signals its tile as finished (mvm_tile_finished).  A fused launch sends the
+    // marks of all its rounds together (thread 64 rr + t: round rr), so that it waits for one round trip, not one
+    // per round; round 0 of a fused launch lists sample b at position b.
     int *hits = reinterpret_cast<int *>(&red[0][0][0]); // the partial sums have been consumed ...
     __syncthreads();                                      // ... by every wave
-    if (threadIdx.x < 2 * TILE) hits[threadIdx.x] = 0;
+    if (threadIdx.x < NACC * 2 * TILE) hits[threadIdx.x] = 0;
     __syncthreads();
     if (up) atomicMax(&hits[r], up);
     if (lo) atomicMax(&hits[TILE + r], lo);
+    if constexpr (DUAL) {
+      if (up1) atomicMax(&hits[2 * TILE + r], up1);
+      if (lo1) atomicMax(&hits[3 * TILE + r], lo1);
+    }
+    if constexpr (TRI) {
+      if (up2) atomicMax(&hits[4 * TILE + r], up2);
+      if (lo2) atomicMax(&hits[5 * TILE + r], lo2);
+    }
     __syncthreads();
-    if (threadIdx.x < 2 * TILE) {
+    if (threadIdx.x < NACC * 2 * TILE) {
+      const int rr = (int)threadIdx.x / (2 * TILE);       // round of the fused launch (0 otherwise)
+      const bool upper = ((int)threadIdx.x & (2 * TILE - 1)) < TILE;
       const int t = threadIdx.x & (TILE - 1);
       const int hit = hits[threadIdx.x];
       const int slot = tile_b * TILE + t;
       if (hit && slot < n_act) {
-        const int bs = (round > 0) ? pick2(a.st.list, round & 1)[slot] : slot;
-        const int old = atomicMax(threadIdx.x < TILE ? &a.st.hit_up[bs] : &a.st.hit_lo[bs], hit);
+        int *target;
+        if (rr == 0) {
+          const int bs = (round > 0) ? pick2(a.st.list, round & 1)[slot] : slot;
+          target = upper ? &a.st.hit_up[bs] : &a.st.hit_lo[bs];
+        } else {
+          target = (rr == 1 ? a.dual.hit1 : a.dual.hit2) + (upper ? 0 : a.m_batch) + slot;
+        }
+        const int old = atomicMax(target, hit);
         asm volatile("" ::"v"(old));
       }
-    }
-    if constexpr (DUAL) { // the marks of the later rounds (round 0 of a fused launch lists sample b at position b)
-      auto later_marks = [&](int up_r, int lo_r, int *marks) {
-        __syncthreads();
-        if (threadIdx.x < 2 * TILE) hits[threadIdx.x] = 0;
-        __syncthreads();
-        if (up_r) atomicMax(&hits[r], up_r);
-        if (lo_r) atomicMax(&hits[TILE + r], lo_r);
-        __syncthreads();
-        if (threadIdx.x < 2 * TILE) {
-          const int t = threadIdx.x & (TILE - 1);
-          const int hit = hits[threadIdx.x];
-          const int slot = tile_b * TILE + t;
-          if (hit && slot < n_act) {
-            const int old = atomicMax(&marks[(threadIdx.x < TILE ? 0 : a.m_batch) + slot], hit);
-            asm volatile("" ::"v"(old));
-          }
-        }
-      };
-      later_marks(up1, lo1, a.dual.hit1);
-      if constexpr (TRI) later_marks(up2, lo2, a.dual.hit2);
     }
   }
 }
@@ -1273,15 +1270,31 @@ __device__ __forceinline__ void mvm_tile_finished_dual(const MvmArgs &a, int til
 __device__ __forceinline__ void mvm_dual_select(const MvmArgs &a, int n) {
   int tile_o, tile_b;
   if (!tile_of(a, n, a.m_batch, tile_o, tile_b)) return;
-  for (int idx = threadIdx.x; idx < TILE * TILE; idx += blockDim.x) {
+  // four elements per thread (workgroups of 256): the choices first, then the kept values, then the stores, so that
+  // the loads of a step are in flight together
+  int sel[4];
+  float v[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int idx = (int)threadIdx.x + 256 * i;
     const int b = tile_b * TILE + (idx >> 5), o = tile_o * TILE + (idx & 31);
-    if (b < a.m_batch && o < a.O) {
-      const int sel = a.dual.sel[b];
-      if (sel < a.dual.rounds) {
-        const float *kept = sel == 2 ? a.dual.buf[2] : (sel == 1 ? a.dual.buf[1] : a.dual.buf[0]);
-        a.out[(long)b * a.out_sb + (long)o * a.out_so] = kept[(long)b * a.O + o];
-      }
+    sel[i] = (b < a.m_batch && o < a.O) ? a.dual.sel[b] : a.dual.rounds;
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int idx = (int)threadIdx.x + 256 * i;
+    const int b = tile_b * TILE + (idx >> 5), o = tile_o * TILE + (idx & 31);
+    v[i] = 0.0f;
+    if (sel[i] < a.dual.rounds) {
+      const float *kept = sel[i] == 2 ? a.dual.buf[2] : (sel[i] == 1 ? a.dual.buf[1] : a.dual.buf[0]);
+      v[i] = kept[(long)b * a.O + o];
     }
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int idx = (int)threadIdx.x + 256 * i;
+    const int b = tile_b * TILE + (idx >> 5), o = tile_o * TILE + (idx & 31);
+    if (sel[i] < a.dual.rounds) a.out[(long)b * a.out_sb + (long)o * a.out_so] = v[i];
   }
 }
 
