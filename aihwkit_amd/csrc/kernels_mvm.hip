@@ -267,22 +267,26 @@ __device__ __forceinline__ float set_round_scales(const MvmArgs &a, int b, float
 // Noise-management value and reduction that sample b, now at (nm, red) with output factor fin, would use in
 // the round after `round`; false when the reduction limit is reached or the sample is short-cut to zero
 // (rpu_forward_backward_pass.cpp:944-983).
-__device__ __forceinline__ bool next_round_params(const MvmArgs &a, int round, int b, float fin, float &nm, float &red) {
+// np_known: the sample's AbsMaxNPSum scale where the caller has just computed it (the init kernel, whose other
+// threads must not read back what its first thread is storing); null: read from the per-sample state.
+__device__ __forceinline__ bool next_round_params(const MvmArgs &a, int round, int b, float fin, float &nm, float &red,
+                                                  const float *np_known = nullptr) {
   const IoDev &io = a.io;
   if (fin == 0.0f) return false;
   const bool stop = ((int)red > io.max_bm_factor) || ((io.inp_res > 0.0f) && (red > io.max_bm_res / io.inp_res));
   if (stop) return false;
   red *= 2.0f;
   if (round == 0 && io.bound_management == RPU_BM_ITERATIVE_WORST_CASE && io.noise_management != RPU_NM_ABS_MAX_NP_SUM) {
-    nm = a.st.nm_np[b];
+    nm = np_known ? *np_known : a.st.nm_np[b];
     red = 1.0f;
   }
   return true;
 }
 
 // input scale of the round after `round` for such a sample, 0 when there is none
-__device__ __forceinline__ float next_round_scale(const MvmArgs &a, int round, int b, float fin, float nm, float red) {
-  if (!next_round_params(a, round, b, fin, nm, red)) return 0.0f;
+__device__ __forceinline__ float next_round_scale(const MvmArgs &a, int round, int b, float fin, float nm, float red,
+                                                  const float *np_known = nullptr) {
+  if (!next_round_params(a, round, b, fin, nm, red, np_known)) return 0.0f;
   float fin_next;
   return round_scales(a, nm, red, fin_next);
 }
@@ -789,6 +793,7 @@ __device__ __forceinline__ void mvm_init_sample(const MvmArgs &a, int b, int t, 
     }
   }
   float nm = 1.0f;
+  float np_scale = 0.0f; // the AbsMaxNPSum scale, known to every thread of the group once it is computed
   const bool worst_case = io.bound_management == RPU_BM_ITERATIVE_WORST_CASE;
   const bool need_np = io.noise_management == RPU_NM_ABS_MAX_NP_SUM || worst_case;
   const bool running = io.noise_management == RPU_NM_AVERAGE_ABS_MAX ||
@@ -837,6 +842,7 @@ __device__ __forceinline__ void mvm_init_sample(const MvmArgs &a, int b, int t, 
       np = fmaxf(am, np);
       if (io.noise_management == RPU_NM_ABS_MAX_NP_SUM) nm = np;
       if (t == 0) a.st.nm_np[b] = np;
+      np_scale = np;
     }
   }
   if (io.noise_management == RPU_NM_CONSTANT) {
@@ -854,7 +860,7 @@ __device__ __forceinline__ void mvm_init_sample(const MvmArgs &a, int b, int t, 
     a.st.scale[b] = scale;
     a.st.fin[b] = fin;
     a.st.rounds[b] = (fin == 0.0f) ? 0 : 1;
-    if (io.bound_management != RPU_BM_NONE) a.st.next_scale[0][b] = next_round_scale(a, 0, b, fin, nm, 1.0f);
+    if (io.bound_management != RPU_BM_NONE) a.st.next_scale[0][b] = next_round_scale(a, 0, b, fin, nm, 1.0f, &np_scale);
   }
   if (gid < MVM_COUNT_WORDS) a.st.count[gid] = 0; // per-round counts and the arrival counters of k_mvm_rounds_rest
   {
@@ -864,10 +870,12 @@ __device__ __forceinline__ void mvm_init_sample(const MvmArgs &a, int b, int t, 
   // the input range of a second round is known as well: its row is quantized now, while the input is at hand,
   // so that the first round has nothing to prepare
   float next = 0.0f, next2 = 0.0f;
-  if (a.rows_ahead_in_init && io.bound_management != RPU_BM_NONE) next = next_round_scale(a, 0, b, fin, nm, 1.0f);
+  // (the scale of a worst-case second round is the one just computed: the threads of the other waves must not read it
+  // back from memory, where the group's first thread may not have stored it yet)
+  if (a.rows_ahead_in_init && io.bound_management != RPU_BM_NONE) next = next_round_scale(a, 0, b, fin, nm, 1.0f, &np_scale);
   if (a.dual.rounds == 3 && next != 0.0f) { // the fused launch of three rounds reads the rows of round 2 as well
     float nm1 = nm, red1 = 1.0f, fin1 = fin;
-    if (next_round_params(a, 0, b, fin1, nm1, red1)) {
+    if (next_round_params(a, 0, b, fin1, nm1, red1, &np_scale)) {
       round_scales(a, nm1, red1, fin1);
       next2 = next_round_scale(a, 1, b, fin1, nm1, red1);
     }
@@ -2626,12 +2634,15 @@ bool mvm_can_fuse_rounds(const MvmArgs &a) {
   return mvm_prefetch_depth(a.K, a.k_pad) >= 2;
 }
 
-// Workgroups of `kernel` (256 threads, static LDS only) that the current GPU holds at once: what the occupancy query
-// reports per CU times the number of CUs.  The launches whose workgroups wait for each other are sized by it.
+// Workgroups of `kernel` (256 threads, static LDS only) that a launch may count on being resident together: one per CU,
+// and none where the occupancy query finds no room for the kernel at all.  What the query reports beyond one per CU is
+// not relied on: for k_mvm_rounds_rest<1, 0> (54 KB of LDS) it reports three, and a launch of 560 workgroups, 70 per
+// XCD of 32 CUs, then ran into the limit of its wait -- not all of them had been placed.  The launches whose workgroups
+// wait for each other are sized by this.
 template <typename K> static int resident_workgroups(K kernel) {
   int per_cu = 0;
   if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, 256, 0) != hipSuccess || per_cu < 1) return 0;
-  return per_cu * current_device_cus();
+  return current_device_cus();
 }
 
 // prefetch depth of the launch that runs several rounds: with the weights addressed along the outputs the deepest

@@ -13,6 +13,7 @@
 #include <cmath>
 #include <cstring>
 #include <memory>
+#include <cstdlib>
 #include <mutex>
 #include <random>
 #include <string>
@@ -38,6 +39,14 @@ namespace {
 // device allocations made by the library's buffers so far (rpu_device_allocation_count)
 std::atomic<long> g_device_allocations{0};
 
+// Test switch: with RPU_AMD_POISON_NEW_BUFFERS set in the environment every new device buffer of the library is filled
+// with 0xff bytes (NaN as a float, -1 as an integer), so that a kernel that reads scratch memory nothing has written
+// shows up in the results instead of finding plausible values that an earlier call left there.
+static bool poison_new_buffers() {
+  static const bool on = std::getenv("RPU_AMD_POISON_NEW_BUFFERS") != nullptr;
+  return on;
+}
+
 template <typename T> struct DevBuf {
   T *p = nullptr;
   size_t n = 0;
@@ -49,6 +58,7 @@ template <typename T> struct DevBuf {
     RPU_HIP_CHECK(hipMalloc((void **)&p, count * sizeof(T)));
     g_device_allocations.fetch_add(1, std::memory_order_relaxed);
     n = count;
+    if (poison_new_buffers()) RPU_HIP_CHECK(hipMemset(p, 0xff, count * sizeof(T)));
   }
   // use memory of the caller from now on (never freed here)
   void adopt(T *external, size_t count) {

@@ -332,3 +332,31 @@ def test_a_group_reports_a_wait_that_runs_out(gpu_device):
     for xs in (loud, quiet, quiet, loud):                         # one launch per round from now on: exact again
         for y, orc, x in zip(run(xs), oracles, xs):
             assert np.array_equal(y, orc.forward(x))
+
+
+def test_worst_case_second_round_on_a_fresh_tile_matches_the_oracle(gpu_device):
+    """IterativeWorstCase: round 1 runs at the AbsMaxNPSum scale.  The init kernel quantizes the rows of that round ahead
+    and must use the scale its threads have just computed, not one read back from the per-sample state that the group's
+    first thread is still storing (on a fresh tile that state holds anything).  Exact-arithmetic setting, first call of
+    fresh tiles in every launch mode against the oracle, at a batch that takes the walking kernel for the later rounds."""
+    from helpers import constant_step
+    rng = np.random.default_rng(31)
+    x_size, d_size, batch = 512, 256, 1100
+    f_io = noise_free_io(inp_res=1 / 128.0, out_res=1 / 512.0, out_bound=2.0, noise_management=NM.AbsMax,
+                         bound_management=BM.IterativeWorstCase)
+    dev = constant_step(w_max_dtod=0.0, w_min_dtod=0.0, w_max=1.0, w_min=-1.0, construction_seed=2)
+    host, orc, _ = build_pair(make_meta(f_io, noise_free_io()), dev, x_size, d_size, gpu=False)
+    w = (rng.integers(-60, 61, (d_size, x_size)) / 64.0).astype(F)
+    host.set_weights(torch.from_numpy(w))
+    orc.set_weights(w)
+    x = rng.uniform(-1, 1, (batch, x_size)).astype(F)
+    x *= rng.choice([0.02, 0.2, 1.0], (batch, 1)).astype(F)
+    want, rounds = orc.forward(x), orc.bm_rounds(batch)
+    assert (rounds >= 2).mean() > 0.3
+    xin = torch.from_numpy(x).cuda()
+    for mode in (0, 1, 3, 5, 7, -1):
+        gpu = tiles.CudaAnalogTile(host)
+        gpu.set_fused_rounds(mode)
+        y = gpu.forward(xin).cpu().numpy()
+        assert np.array_equal(gpu.get_bm_rounds(batch).numpy(), rounds), mode
+        assert np.array_equal(y, want), mode
