@@ -1219,7 +1219,8 @@ __global__ __launch_bounds__(256) void k_update_implicit(UpdateArgs a) {
   CtocStream rng;
   rng.left = 0;
   rng.refill = 0;
-  rng.cell = (uint32_t)k;
+  // the noise stream of a cross-point is keyed by its row-major number in the tile, however the matrix is stored
+  rng.cell = a.swapped ? (uint32_t)((long)j * a.d_size + i) : (uint32_t)k;
   rng.n0 = rng.n1 = rng.n2 = rng.n3 = 0.0f;
   const float std_ = a.dev.dw_min_std;
   for (int b = 0; b < a.m_batch; ++b) {

@@ -634,8 +634,9 @@ int rpu_tile_get_shared_weights_if(const rpu_tile_t *tile);
  * way round where inputs are denser than errors): the tile keeps row-major copies of the device parameters for it, the
  * launch that makes the pulse trains also makes a row-major scratch copy of the weights, and the loop stores its
  * results straight into the tensor.  Results are bit for bit those of the row-major tile (same pulse trains, same noise
- * draws per cross-point, same ADC draws) for forward, backward and the stochastic pulse loop; the deterministic-implicit
- * update keys its cycle-to-cycle noise by storage position, so with that noise on its weights agree statistically.  Host-side interfaces (get / set weights, hidden parameters, ...) stay
+ * draws per cross-point, same ADC draws) for forward, backward, the stochastic pulse loop and the deterministic-implicit
+ * update; the opt-in aggregated update deals its noise streams to lanes, which hold other cross-points in the other
+ * layout, so its weights agree statistically.  Host-side interfaces (get / set weights, hidden parameters, ...) stay
  * [d_size][x_size]; rpu_tile_weights_device_ptr returns the tensor.  Such tiles can be members of a group when all
  * members are bound that way.
  * The other kinds of tile keep their row-major matrix and mirror it: the tensor takes the tile's weights when it is

@@ -34,6 +34,9 @@ def pytest_generate_tests(metafunc):
     if "storage_mode" in metafunc.fixturenames:
         module = metafunc.module.__name__.split(".")[-1]
         modes = ["row_major", "xd_shared"] if module in BOTH_STORAGES else ["row_major"]
+        # RPU_TEST_STORAGE=xd_shared runs every module on bound tiles only (the sweeps too: a longer, occasional run)
+        if os.environ.get("RPU_TEST_STORAGE") in ("row_major", "xd_shared"):
+            modes = [os.environ["RPU_TEST_STORAGE"]]
         metafunc.parametrize("storage_mode", modes, indirect=True)
 
 

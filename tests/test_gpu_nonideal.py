@@ -139,9 +139,9 @@ def test_weight_noise_under_bound_management_and_other_paths(gpu_device):
     resid = (got - want)[same]
     # the noise rides on the drifted sums of whichever round was the last one: small against the signal, not zero
     assert 0.01 < resid.std() < 0.15 and abs(resid.mean()) < 4 * resid.std() / np.sqrt(resid.size)
-    # a group does not take these tiles
-    group = tiles.TileGroup([gpu, quiet_gpu])
-    with pytest.raises(RuntimeError, match="not provided for a group"):
+    # a group does not take these tiles (bound to a shared tensor they mirror it, and the group refuses them at once)
+    with pytest.raises(RuntimeError, match="not provided for a group|cannot be in a group"):
+        group = tiles.TileGroup([gpu, quiet_gpu])
         group.forward([torch.from_numpy(x).cuda(), torch.from_numpy(x).cuda()])
 
 
