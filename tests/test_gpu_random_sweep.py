@@ -901,3 +901,112 @@ def test_random_write_noise_cases(gpu_device):
     every cross-point that stepped shows a new value, none without pulses does, residuals are N(0, (std dw_min)^2)."""
     failures = [desc for ok, desc in (one_write_noise(seed) for seed in range(93000, 93080)) if not ok]
     assert not failures, failures[:3]
+
+
+# ---- launch modes of the forward pass: every mode must give what one launch per round gives ---------------------
+
+def one_launch_mode_case(seed):
+    """Random shape, batch, layout, iterative scheme, ADC range (small ranges force up to five rounds) and storage mode;
+    noise on.  Three calls on a fresh tile per launch mode (the tile's own choice changes from call to call): outputs
+    and round counts bit for bit those of one launch per round."""
+    F = np.float32
+    rng = np.random.default_rng(seed)
+    x_size = int(rng.choice([33, 64, 96, 128, 200, 256, 257, 384, 512, 513, 768, 1024]))
+    d_size = int(rng.choice([10, 32, 33, 64, 100, 128, 256, 300, 512, 1024]))
+    batch = int(rng.choice([1, 5, 31, 32, 33, 64, 100, 256, 300, 600, 1100]))
+    if x_size * d_size * batch > 300_000_000:
+        batch = 256
+    bias, trans = bool(rng.integers(2)), bool(rng.integers(2))
+    bm = BM.Iterative if rng.random() < 0.8 else BM.IterativeWorstCase
+    bound = float(rng.choice([1.5, 3.0, 6.0, 12.0]))
+    bound_tensor = bool(rng.integers(2))
+    io = io_params(out_noise=float(rng.choice([0.0, 0.06, 0.2])), out_bound=bound, noise_management=NM.AbsMax, bound_management=bm,
+                   inp_res=float(rng.choice([1 / 126.0, 1 / 254.0, -1.0])), out_res=float(rng.choice([1 / 510.0, 1 / 254.0])))
+    desc = dict(seed=seed, X=x_size, D=d_size, B=batch, bias=bias, trans=trans, bm=str(bm), bound=bound, bound_tensor=bound_tensor)
+    before = tiles.CudaAnalogTile.bind_shared_weights
+    tiles.CudaAnalogTile.bind_shared_weights = bound_tensor
+    try:
+        host, _orc, _ = build_pair(make_meta(io, noise_free_io()), soft_bounds(construction_seed=3), x_size, d_size, gpu=False)
+        host.set_weights(torch.from_numpy(rng.uniform(-0.4, 0.4, (d_size, x_size)).astype(F)))
+        x = rng.uniform(-1, 1, (batch, x_size - int(bias))).astype(F)
+        x *= rng.choice([0.02, 0.2, 1.0], (batch, 1)).astype(F)
+        x[:, : x.shape[1] // 2] *= rng.choice([0.05, 1.0], (batch, 1)).astype(F)
+        if batch > 3:
+            x[3] = 0.0
+        xin = cuda(x.T if trans else x)
+        results = []
+        for mode in (0, 3, 5, 7, -1):
+            gpu = tiles.CudaAnalogTile(host)
+            gpu.set_fused_rounds(mode)
+            gpu.set_seed(5)
+            outs = []
+            for _ in range(3):
+                y = gpu.forward(xin, bias, trans, trans).cpu().numpy()
+                outs.append((y, gpu.get_bm_rounds(batch).numpy().copy()))
+            results.append(outs)
+    finally:
+        tiles.CudaAnalogTile.bind_shared_weights = before
+    ok = all(np.array_equal(a[0], b[0]) and np.array_equal(a[1], b[1]) for other in results[1:] for a, b in zip(results[0], other))
+    desc["most_rounds"] = max(int(o[1].max()) for o in results[0])
+    return ok, desc
+
+
+def test_random_launch_mode_cases_are_bit_equal(gpu_device):
+    results = [one_launch_mode_case(seed) for seed in range(95000, 95120)]
+    failures = [desc for ok, desc in results if not ok]
+    assert not failures, failures[:3]
+    assert sum(desc["most_rounds"] >= 3 for _, desc in results) >= 20      # the later rounds had work in many cases
+
+
+def one_call_sequence(seed):
+    """Ten calls with changing batches and input scales on one tile per launch mode, some followed by a backward pass
+    and an update: the tile's choice of launches follows its history, the scratch buffers grow and are reused."""
+    F = np.float32
+    rng = np.random.default_rng(seed)
+    x_size = int(rng.choice([64, 128, 256, 257, 512, 1024]))
+    d_size = int(rng.choice([32, 64, 100, 256, 300, 1024]))
+    bias, bound_tensor = bool(rng.integers(2)), bool(rng.integers(2))
+    bm = BM.Iterative if rng.random() < 0.8 else BM.IterativeWorstCase
+    io = io_params(out_noise=float(rng.choice([0.0, 0.06])), out_bound=float(rng.choice([1.5, 3.0, 12.0])), noise_management=NM.AbsMax,
+                   bound_management=bm, inp_res=float(rng.choice([1 / 126.0, -1.0])), out_res=1 / 510.0)
+    desc = dict(seed=seed, X=x_size, D=d_size, bias=bias, bm=str(bm), bound_tensor=bound_tensor)
+    before = tiles.CudaAnalogTile.bind_shared_weights
+    tiles.CudaAnalogTile.bind_shared_weights = bound_tensor
+    try:
+        meta = make_meta(io, io_params(out_noise=0.06, noise_management=NM.AbsMax))
+        host, _orc, _ = build_pair(meta, soft_bounds(construction_seed=3), x_size, d_size, gpu=False)
+        host.set_weights(torch.from_numpy(rng.uniform(-0.4, 0.4, (d_size, x_size)).astype(F)))
+        group = []
+        for mode in (0, 3, 7, -1):
+            t = tiles.CudaAnalogTile(host)
+            t.set_fused_rounds(mode)
+            t.set_seed(5)
+            t.set_learning_rate(0.01)
+            group.append(t)
+        for call in range(10):
+            batch = int(rng.choice([1, 31, 33, 64, 256, 300, 700, 1100]))
+            x = (rng.uniform(-1, 1, (batch, x_size - int(bias))) * float(rng.choice([0.01, 0.1, 1.0]))).astype(F)
+            x[:, : x.shape[1] // 2] *= rng.choice([0.05, 1.0], (batch, 1)).astype(F)
+            xg = cuda(x)
+            train = rng.integers(4) == 1
+            dg = cuda((0.05 * rng.standard_normal((batch, d_size))).astype(F))
+            outs = []
+            for t in group:
+                got = [t.forward(xg, bias, False, False), t.get_bm_rounds(batch).clone()]
+                if train:
+                    got.append(t.backward(dg, bias, False, False))
+                    t.update(xg, dg, bias, False, False, False)
+                    got.append(t.get_weights())
+                outs.append(got)
+            for other in outs[1:]:
+                if not all(torch.equal(u, v) for u, v in zip(outs[0], other)):
+                    desc.update(call=call, batch=batch)
+                    return False, desc
+    finally:
+        tiles.CudaAnalogTile.bind_shared_weights = before
+    return True, desc
+
+
+def test_random_call_sequences_are_bit_equal_across_launch_modes(gpu_device):
+    failures = [desc for ok, desc in (one_call_sequence(seed) for seed in range(96000, 96040)) if not ok]
+    assert not failures, failures[:3]
