@@ -296,104 +296,29 @@ __device__ __forceinline__ float next_round_scale(const MvmArgs &a, int round, i
 // between the others, so that the LDS and memory pipes work underneath the matrix pipe of the same wave.
 template <int WMODE, int NACC = 1>
 __device__ __forceinline__ void mvm_step_schedule() {
-  constexpr bool DUAL = NACC == 2;
 #define RPU_SG(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)
 #define RPU_SG_MFMA 0x008
 #define RPU_SG_VMEM 0x020
 #define RPU_SG_DSR 0x100
 #define RPU_SG_DSW 0x200
-  if (NACC == 3 && WMODE == 1) { // per step: 48 MFMAs, 12 LDS writes, 28 global loads, 12 LDS reads
+  // per step: 16 NACC MFMAs; 4 (NACC + 1) LDS writes and as many global loads (a tile of the weights and NACC tiles of
+  // quantized rows); LDS reads: 4 per tile of rows, 4 for the weights staged along k or 16 (one per k) for the weights
+  // staged along the outputs
+  constexpr int mfmas = 16 * NACC, tiles = NACC + 1;
+  constexpr int reads = 4 * NACC + (WMODE == 1 ? 16 : 4);
+  constexpr int reads_per_slot = (reads + 4 * tiles - 1) / (4 * tiles);
 #pragma unroll
-    for (int i = 0; i < 12; ++i) {
-      RPU_SG(RPU_SG_MFMA, 1);
-      RPU_SG(RPU_SG_DSW, 1);
-    }
-#pragma unroll
-    for (int i = 0; i < 12; ++i) {
-      RPU_SG(RPU_SG_MFMA, 1);
-      RPU_SG(RPU_SG_VMEM, 2);
-      RPU_SG(RPU_SG_DSR, 1);
-    }
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      RPU_SG(RPU_SG_MFMA, 1);
-      RPU_SG(RPU_SG_VMEM, 1);
-    }
-    RPU_SG(RPU_SG_MFMA, 20);
-  } else if (NACC == 3) { // per step: 48 MFMAs, 16 LDS writes, 16 global loads, 16 LDS reads
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      RPU_SG(RPU_SG_MFMA, 1);
-      RPU_SG(RPU_SG_DSW, 1);
-    }
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      RPU_SG(RPU_SG_MFMA, 1);
-      RPU_SG(RPU_SG_VMEM, 1);
-      RPU_SG(RPU_SG_DSR, 1);
-    }
-    RPU_SG(RPU_SG_MFMA, 16);
-  } else if (DUAL && WMODE == 1) { // per step: 32 MFMAs, 8 LDS writes, 24 global loads, 8 LDS reads
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      RPU_SG(RPU_SG_MFMA, 1);
-      RPU_SG(RPU_SG_DSW, 1);
-    }
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      RPU_SG(RPU_SG_MFMA, 1);
-      RPU_SG(RPU_SG_VMEM, 2);
-      RPU_SG(RPU_SG_DSR, 1);
-    }
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      RPU_SG(RPU_SG_MFMA, 1);
-      RPU_SG(RPU_SG_VMEM, 1);
-    }
-    RPU_SG(RPU_SG_MFMA, 8);
-  } else if (DUAL) { // per step: 32 MFMAs, 12 LDS writes, 12 global loads, 12 LDS reads
-#pragma unroll
-    for (int i = 0; i < 12; ++i) {
-      RPU_SG(RPU_SG_MFMA, 1);
-      RPU_SG(RPU_SG_DSW, 1);
-    }
-#pragma unroll
-    for (int i = 0; i < 12; ++i) {
-      RPU_SG(RPU_SG_MFMA, 1);
-      RPU_SG(RPU_SG_VMEM, 1);
-      RPU_SG(RPU_SG_DSR, 1);
-    }
-    RPU_SG(RPU_SG_MFMA, 8);
-  } else if (WMODE != 1) { // per step: 8 LDS writes, 8 global loads, 8 LDS reads
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      RPU_SG(RPU_SG_MFMA, 1);
-      RPU_SG(RPU_SG_DSW, 1);
-    }
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      RPU_SG(RPU_SG_MFMA, 1);
-      RPU_SG(RPU_SG_VMEM, 1);
-      RPU_SG(RPU_SG_DSR, 1);
-    }
-  } else { // per step: 4 LDS writes, 20 global loads, 4 LDS reads
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      RPU_SG(RPU_SG_MFMA, 1);
-      RPU_SG(RPU_SG_DSW, 1);
-    }
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      RPU_SG(RPU_SG_MFMA, 1);
-      RPU_SG(RPU_SG_VMEM, 2);
-      RPU_SG(RPU_SG_DSR, 1);
-    }
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      RPU_SG(RPU_SG_MFMA, 1);
-      RPU_SG(RPU_SG_VMEM, 2);
-    }
+  for (int i = 0; i < 4 * tiles; ++i) {
+    RPU_SG(RPU_SG_MFMA, 1);
+    RPU_SG(RPU_SG_DSW, 1);
   }
+#pragma unroll
+  for (int i = 0; i < 4 * tiles; ++i) {
+    RPU_SG(RPU_SG_MFMA, 1);
+    RPU_SG(RPU_SG_VMEM, 1);
+    RPU_SG(RPU_SG_DSR, reads_per_slot);
+  }
+  if (mfmas > 8 * tiles) RPU_SG(RPU_SG_MFMA, mfmas - 8 * tiles);
 #undef RPU_SG
 #undef RPU_SG_MFMA
 #undef RPU_SG_VMEM
@@ -411,9 +336,13 @@ __device__ __forceinline__ void mvm_step_schedule() {
 // fetched with unit-stride 16-byte loads, 8 lanes per 128-byte row segment, staged in a wave-private LDS
 // tile and read back in the MFMA operand layout (lane (r, h) holds row r, k = 16 h .. 16 h + 15).  Reading
 // them straight into that layout would make every lane of a load touch a different cache line, which is
-// address-bound in the vector L1.  Mode 1 reads the weights directly: 32 consecutive outputs per half-wave
-// and k are one line.  Out-of-range rows / k are clamped to valid addresses: their products meet the zero
-// padding of the quantized inputs or are never stored.
+// address-bound in the vector L1.  Mode 1 fetches its weight tile the same way, along the outputs (a tile row is the
+// 32 outputs of one k: 16-byte loads from 4-byte aligned addresses, nothing read past a row's end), and transposes it
+// on the way through LDS: staged as [k][o], read back with one 4-byte read per k (sixteen instead of four 16-byte
+// reads; the two half-waves meet in the same banks, which costs little beside a step's matrix work).  Loading the
+// sixteen values straight into the operand layout, one 4-byte load each, was the slower way (backward round at
+// configuration 2: 11.9 -> 10.8 us, at batch 1024 51.6 -> 43.5 us).  Out-of-range rows / k are clamped to valid
+// addresses: their products meet the zero padding of the quantized inputs or are never stored.
 // PD = 2, 4: software pipeline with the global loads of PD steps in flight, k_pad a multiple of
 // PD * KSTEP * WAVES; PD = 1: one register set, for short contractions, k_pad a multiple of KSTEP.
 // NACC = 2 (round 0 only, PD = 2): the same weights also multiply the rows that round 1 would use (written by the init
@@ -432,13 +361,9 @@ __device__ __forceinline__ void mvm_round_tile(const MvmArgs &a, int round, int 
   const int h = lane >> 5;
 
   // operand rows owned by this lane in the MFMA layout
-  const int o_in = tile_o * TILE + r;
-  const bool o_ok = o_in < a.O;
   const int slot_in = tile_b * TILE + r;
   const bool b_ok = slot_in < n_act;
 
-  const long w_so = a.w_oc ? 1 : a.w_ld;
-  const long w_sk = a.w_oc ? a.w_ld : 1;
   const int K = a.K;
   // steps of 32 k-values, dealt to the waves in contiguous parts (equal parts, a multiple of PD, when PD >= 2;
   // a short contraction may leave the last waves without a step)
@@ -471,7 +396,6 @@ __device__ __forceinline__ void mvm_round_tile(const MvmArgs &a, int round, int 
     const int o = min(tile_o * TILE + row, a.O - 1);
     w_src[t] = a.w + (long)o * a.w_ld;
   }
-  const float *w_col = a.w + (long)(o_ok ? o_in : a.O - 1) * w_so; // mode 1: this lane's output column
 
   floatx16 acc, acc1, acc2;
 #pragma unroll
@@ -506,10 +430,23 @@ __device__ __forceinline__ void mvm_round_tile(const MvmArgs &a, int round, int 
 #pragma unroll
       for (int t = 0; t < 4; ++t) gw[t] = *reinterpret_cast<const f32x4 *>(w_src[t] + kc);
     } else if (WMODE == 1) {
+      // rows of the stored matrix run along the outputs: 16-byte loads along o (eight lanes per 128-byte row of the
+      // tile), transposed on the way through LDS
+      const int o_base = tile_o * TILE + st_chunk;
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const int kc = min(k0 + h * 16 + i, K - 1);
-        wd[i] = w_col[(long)kc * w_sk];
+      for (int t = 0; t < 4; ++t) {
+        const int kc = min(k0 + t * 8 + st_row, K - 1);
+        const float *p = a.w + (long)kc * a.w_ld + o_base;
+        if (o_base + 4 <= a.O) {
+          gw[t] = *reinterpret_cast<const f32x4_unaligned *>(p);
+        } else { // the end of a row: nothing is read past it
+          f32x4 z;
+          z.x = (o_base < a.O) ? p[0] : 0.0f;
+          z.y = (o_base + 1 < a.O) ? p[1] : 0.0f;
+          z.z = (o_base + 2 < a.O) ? p[2] : 0.0f;
+          z.w = 0.0f;
+          gw[t] = z;
+        }
       }
     } else {
       const int kc = k0 + st_chunk;
@@ -534,7 +471,7 @@ __device__ __forceinline__ void mvm_round_tile(const MvmArgs &a, int round, int 
     for (int t = 0; t < 4; ++t) {
       const int off = (t * 8 + st_row) * LDS_ROW + st_chunk;
       *reinterpret_cast<f32x4 *>(stage_x + off) = gx[t];
-      if (WMODE != 1) *reinterpret_cast<f32x4 *>(stage_w + off) = gw[t];
+      *reinterpret_cast<f32x4 *>(stage_w + off) = gw[t];
       if constexpr (DUAL) *reinterpret_cast<f32x4 *>(stage_x1 + off) = gx1[t];
       if constexpr (TRI) *reinterpret_cast<f32x4 *>(stage_x2 + off) = gx2[t];
     }
@@ -557,6 +494,10 @@ __device__ __forceinline__ void mvm_round_tile(const MvmArgs &a, int round, int 
         const f32x4 tw = *reinterpret_cast<const f32x4 *>(stage_w + off);
         wd[v4 * 4 + 0] = tw.x; wd[v4 * 4 + 1] = tw.y; wd[v4 * 4 + 2] = tw.z; wd[v4 * 4 + 3] = tw.w;
       }
+    }
+    if (WMODE == 1) { // the staged tile is [k][o]: this lane's output column, k = 16 h .. 16 h + 15
+#pragma unroll
+      for (int i = 0; i < 16; ++i) wd[i] = stage_w[(h * 16 + i) * LDS_ROW + r];
     }
   };
   auto mfma16 = [&](const float (&wd)[16], const float (&xd)[16], const float (&xd1)[16], const float (&xd2)[16]) {
@@ -584,9 +525,6 @@ __device__ __forceinline__ void mvm_round_tile(const MvmArgs &a, int round, int 
 #define RPU_MVM_STEP(T, GX, GW, WR, HX, IX, XC, WC, YC, ZC, XN, WN, YN, ZN) \
   {                                                                         \
     lds_store(GX, GW, HX, IX);                                              \
-    if (WMODE == 1) {                                                       \
-      _Pragma("unroll") for (int i = 0; i < 16; ++i) WN[i] = WR[i];         \
-    }                                                                       \
     gload(min((T) + 1 + PD, s_end - 1), GX, GW, WR, HX, IX);                \
     lds_read(XN, WN, YN, ZN);                                               \
     mfma16(WC, XC, YC, ZC);                                                 \
@@ -600,10 +538,6 @@ __device__ __forceinline__ void mvm_round_tile(const MvmArgs &a, int round, int 
     }
     lds_store(gx0, gw0, hx0, ix0);
     lds_read(xc0, wc0, yc0, zc0);
-    if (WMODE == 1) {
-#pragma unroll
-      for (int i = 0; i < 16; ++i) wc0[i] = wr0[i];
-    }
     gload(min(s_begin + PD, s_end - 1), gx0, gw0, wr0, hx0, ix0);
     for (int s = s_begin; s < s_end; s += PD) {
       if constexpr (PD == 4) {
@@ -624,10 +558,6 @@ __device__ __forceinline__ void mvm_round_tile(const MvmArgs &a, int round, int 
     for (int s = s_begin; s < s_end; ++s) {
       lds_store(gx, gw, hx, ix);
       lds_read(xc, wc, yc, zc);
-      if (WMODE == 1) {
-#pragma unroll
-        for (int i = 0; i < 16; ++i) wc[i] = wn[i];
-      }
       gload(min(s + 1, s_end - 1), gx, gw, wn, hx, ix);
       mfma16(wc, xc, yc, zc);
     }
@@ -2767,9 +2697,9 @@ void launch_mvm_round(const MvmArgs &a_in, hipStream_t s) {
   }
   const dim3 grid(all);
   int depth = mvm_prefetch_depth(a.K, a.k_pad);
-  // The deepest prefetch of the transposed-weight variant takes more than half of a SIMD's registers: one workgroup per
-  // CU at a time.  With more workgroups than CUs the variant with two stages in flight, two workgroups per CU, is faster
-  // (backward at batch 1024 on the 1024 x 1024 tile 63 -> 52 us; same sums, the waves split K the same way).
+  // With more workgroups than CUs the output-contiguous variant is a little faster with two stages of loads in flight
+  // than with four (backward on the 1024 x 1024 tile at batch 512 / 1024: 25.9 / 43.5 us against 26.7 / 44.9; same sums,
+  // the waves split K the same way).
   if (mode == 1 && depth == 4 && all > current_device_cus()) depth = 2;
   if (a.rest_in_one) {
 #define RPU_LAUNCH_REST(PD, WMODE) hipLaunchKernelGGL((k_mvm_rounds_rest<PD, WMODE>), grid, dim3(256), 0, s, a)
