@@ -268,6 +268,17 @@ struct UpdateArgs {
   long x_sb, x_sj; // x element (b, j) at x[b * x_sb + j * x_sj]
   const float *d;
   long d_sb, d_si;
+  // Lines read in place from the image tensors of the indexed interface (all zero / null otherwise; only the kernels
+  // that make the lines look at these).  x_index set: sample b is patch b % x_group of image b / x_group, the images
+  // are x_gs apart in x, and element j of the sample is what x_index[(b % x_group) * x_size + j] names: 0, 1 (bias)
+  // or, from 2 on, element idx - 2 of the image.  d_group > 0: element (b, i) of d is at
+  // d[(b / d_group) * d_gs + (b % d_group) * d_sb + i * d_si] (the [image][output][patch] tensor of a convolution).
+  const int *x_index;
+  const int *x_index_lines; // the same index line-major, [x_size][x_group], for kernels with their lanes along the samples
+  int x_group;
+  long x_gs;
+  int d_group;
+  long d_gs;
   float lr;
   UpdateDev up;
   DeviceDev dev;
@@ -313,6 +324,7 @@ void launch_update_lines_group(const UpdateGroup &g, bool wide, int total_blocks
 int update_lines_blocks(const UpdateArgs &a, bool wide);
 // the tiles must agree in what update_pulsed_variant returns; total_workgroups: sum of update_pulsed_workgroups
 int update_pulsed_variant(const UpdateArgs &a);
+bool update_reads_row_cost(const UpdateArgs &a); // by its shape: whether the pulse loop of this call looks at row_cost
 int update_pulsed_workgroups(const UpdateArgs &a);
 void launch_update_pulsed_group(const UpdateGroup &g, int variant, int total_workgroups, hipStream_t s);
 

@@ -50,6 +50,24 @@ __device__ __forceinline__ void calc_bl_ab(const UpdateDev &up, int &BL, float &
   }
 }
 
+// x and d values of a sample wherever the call keeps them: plain strided matrices, or the image tensors of the indexed
+// interface read in place (UpdateArgs::x_index, d_group)
+__device__ __forceinline__ float update_x_value(const UpdateArgs &a, int b, int j) {
+  if (a.x_index) {
+    const int n = b / a.x_group;
+    const int idx = a.x_index[(long)(b - n * a.x_group) * a.x_size + j];
+    return idx <= 1 ? (float)idx : a.x[(long)n * a.x_gs + (idx - 2)];
+  }
+  return a.x[(long)b * a.x_sb + (long)j * a.x_sj];
+}
+__device__ __forceinline__ const float *update_d_row(const UpdateArgs &a, int b) {
+  if (a.d_group) {
+    const int n = b / a.d_group;
+    return a.d + (long)n * a.d_gs + (long)(b - n * a.d_group) * a.d_sb;
+  }
+  return a.d + (long)b * a.d_sb;
+}
+
 // largest absolute value of a line of n elements (element j at v[j * stride]) over the part that thread `t` of `width`
 // takes; rows that are contiguous and 16-byte aligned are read four elements at a time
 __device__ __forceinline__ float part_abs_max(const float *v, int n, long stride, int t, int width) {
@@ -81,8 +99,13 @@ __device__ __forceinline__ void update_prepare_sample(const UpdateArgs &a, const
   int BL;
   float A, B;
   if (a.up.update_management || a.up.update_bl_management) {
-    float xm = part_abs_max(a.x + (long)b * a.x_sb, a.x_size, a.x_sj, t, SUB);
-    float dm = part_abs_max(a.d + (long)b * a.d_sb, a.d_size, a.d_si, t, SUB);
+    float xm = 0.0f;
+    if (a.x_index) {
+      for (int j = t; j < a.x_size; j += SUB) xm = fmaxf(xm, fabsf(update_x_value(a, b, j)));
+    } else {
+      xm = part_abs_max(a.x + (long)b * a.x_sb, a.x_size, a.x_sj, t, SUB);
+    }
+    float dm = part_abs_max(update_d_row(a, b), a.d_size, a.d_si, t, SUB);
 #pragma unroll
     for (int off = (SUB < 64 ? SUB : 64) / 2; off > 0; off >>= 1) {
       xm = fmaxf(xm, __shfl_xor(xm, off));
@@ -202,7 +225,8 @@ __device__ __forceinline__ uint32_t pulse_word(const UpdateArgs &a, bool is_x, i
 // LINES_E = 16 moves whole 64-byte row segments; small launches take 4 elements per workgroup (one per wave) so that
 // there are four times as many workgroups.
 // bx: number of the workgroup's block of line elements (x blocks first, then d blocks), by: its block of 64 rows of words
-template <int LINES_E>
+// IN_PLACE: the call may read its lines from the tensors of the indexed interface (UpdateArgs::x_index, d_group)
+template <int LINES_E, bool IN_PLACE = false>
 __device__ __forceinline__ void update_lines_block(const UpdateArgs &a, const int bx, const int by,
                                                    float (*vals)[LINES_E + 1], uint32_t (*wt)[LINES_E + 1]) {
   const int tiles_x = (a.x_size + LINES_E - 1) / LINES_E;
@@ -215,12 +239,46 @@ __device__ __forceinline__ void update_lines_block(const UpdateArgs &a, const in
   constexpr int ROWS_PER_PASS = 256 / LINES_E;
   const int col = threadIdx.x % LINES_E, row0 = threadIdx.x / LINES_E;
   const int wps = max(a.words_per_sample, 1);
-#pragma unroll
-  for (int i = 0; i < 64 / ROWS_PER_PASS; ++i) {
-    const int rb = row0 + ROWS_PER_PASS * i;
-    const int b = b0 + rb, e = e0 + col;
+  if (IN_PLACE && is_x && a.x_index) {
+    // patches read in place, a wave on one element of 64 samples: the entries of the line-major index are one run, and
+    // so are the image elements they name wherever neighbouring patches are neighbours in the image
+    const int rb = threadIdx.x & 63;
+    const int b = b0 + rb;
     const int sample = wps > 1 ? b / wps : b;
-    vals[rb][col] = (b < a.m_batch && e < size) ? src[(long)sample * s_b + (long)e * s_e] : 0.0f;
+    const int n = sample / a.x_group;
+    const int *idx = a.x_index_lines + (sample - n * a.x_group);
+    const float *image = a.x + (long)n * a.x_gs - 2;
+    int at[LINES_E / 4];
+#pragma unroll
+    for (int i = 0; i < LINES_E / 4; ++i) {
+      const int e = e0 + (threadIdx.x >> 6) + 4 * i;
+      at[i] = (b < a.m_batch && e < size) ? idx[(long)e * a.x_group] : 0;
+    }
+#pragma unroll
+    for (int i = 0; i < LINES_E / 4; ++i) {
+      vals[rb][(threadIdx.x >> 6) + 4 * i] = at[i] <= 1 ? (float)at[i] : image[at[i]];
+    }
+  } else if (IN_PLACE && !is_x && a.d_group) {
+    // the [image][output][patch] tensor in place: neighbouring samples are neighbours in memory, so a wave takes one
+    // element of 64 samples
+    const int rb = threadIdx.x & 63;
+    const int b = b0 + rb;
+    const int sample = wps > 1 ? b / wps : b;
+    const float *row = b < a.m_batch ? update_d_row(a, sample) : a.d;
+#pragma unroll
+    for (int i = 0; i < LINES_E / 4; ++i) {
+      const int c = (threadIdx.x >> 6) + 4 * i;
+      const int e = e0 + c;
+      vals[rb][c] = (b < a.m_batch && e < size) ? row[(long)e * s_e] : 0.0f;
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 64 / ROWS_PER_PASS; ++i) {
+      const int rb = row0 + ROWS_PER_PASS * i;
+      const int b = b0 + rb, e = e0 + col;
+      const int sample = wps > 1 ? b / wps : b;
+      vals[rb][col] = (b < a.m_batch && e < size) ? src[(long)sample * s_b + (long)e * s_e] : 0.0f;
+    }
   }
   __syncthreads();
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -292,7 +350,7 @@ __device__ __forceinline__ void update_copy_weights(const UpdateArgs &a, int fir
   }
 }
 
-template <int LINES_E>
+template <int LINES_E, bool IN_PLACE = false>
 __global__ __launch_bounds__(256) void k_update_lines(UpdateArgs a) {
   __shared__ float vals[64][LINES_E + 1];
   __shared__ uint32_t wt[64][LINES_E + 1];
@@ -302,7 +360,7 @@ __global__ __launch_bounds__(256) void k_update_lines(UpdateArgs a) {
     update_copy_weights(a, own, tile);
     return;
   }
-  update_lines_block<LINES_E>(a, (int)blockIdx.x, (int)blockIdx.y, vals, wt);
+  update_lines_block<LINES_E, IN_PLACE>(a, (int)blockIdx.x, (int)blockIdx.y, vals, wt);
 }
 
 // Several tiles in one launch: start[t] .. start[t + 1] are the element blocks of tile t.
@@ -325,7 +383,7 @@ __global__ __launch_bounds__(256) void k_update_implicit_lines(UpdateArgs a) {
     const int e = (int)(idx % per_sample);
     const bool is_x = e < a.x_size;
     const int j = is_x ? e : e - a.x_size;
-    float v = is_x ? a.x[(long)b * a.x_sb + (long)j * a.x_sj] : a.d[(long)b * a.d_sb + (long)j * a.d_si];
+    float v = is_x ? update_x_value(a, b, j) : update_d_row(a, b)[(long)j * a.d_si];
     if (a.lr < 0.0f) v = -v;
     const float P = is_x ? a.prob_b[b] : a.prob_a[b];
     const bool mean_count = a.up.pulse_type == RPU_PULSE_MEAN_COUNT;
@@ -1397,10 +1455,14 @@ void launch_update_lines(const UpdateArgs &a, hipStream_t s) {
     extra = std::min(256u, (tiles + 3) / 4);
     extra = (extra + sample_tiles - 1) / sample_tiles;
   }
+  const bool in_place = a.x_index || a.d_group;
+  const dim3 narrow((a.x_size + 3) / 4 + (a.d_size + 3) / 4 + extra, sample_tiles);
   if (wide * sample_tiles >= 256) {
-    hipLaunchKernelGGL(k_update_lines<16>, dim3(wide + extra, sample_tiles), dim3(256), 0, s, a);
+    if (in_place) hipLaunchKernelGGL((k_update_lines<16, true>), dim3(wide + extra, sample_tiles), dim3(256), 0, s, a);
+    else hipLaunchKernelGGL(k_update_lines<16>, dim3(wide + extra, sample_tiles), dim3(256), 0, s, a);
   } else {
-    hipLaunchKernelGGL(k_update_lines<4>, dim3((a.x_size + 3) / 4 + (a.d_size + 3) / 4 + extra, sample_tiles), dim3(256), 0, s, a);
+    if (in_place) hipLaunchKernelGGL((k_update_lines<4, true>), narrow, dim3(256), 0, s, a);
+    else hipLaunchKernelGGL(k_update_lines<4>, narrow, dim3(256), 0, s, a);
   }
 }
 
@@ -1438,6 +1500,17 @@ void launch_update_planes(const UpdateArgs &a, hipStream_t s) {
 bool update_pulsed_balanced(const UpdateArgs &a, int columns) {
   return columns == 4 && a.row_cost && a.x_size <= 1024 && a.d_size >= 1024 && a.d_size % 256 == 0 &&
          a.d_size / 8 <= BALANCED_MAX_BAND;
+}
+
+static int update_pulsed_columns(const UpdateArgs &a);
+
+// whether a call of this shape reads UpdateArgs::row_cost at all: elsewhere the tile leaves it null, and the kernel that
+// makes the pulse trains sends no sums (on a tile of few rows and very many samples those were thousands of atomics per
+// address)
+bool update_reads_row_cost(const UpdateArgs &a) {
+  UpdateArgs probe = a;
+  probe.row_cost = reinterpret_cast<int *>(sizeof(int)); // any non-null value: only the shape is looked at
+  return update_pulsed_balanced(probe, update_pulsed_columns(a));
 }
 
 template <bool NOISE, int C, bool DEEP = false> static void launch_update_pulsed_t(const UpdateArgs &a, hipStream_t s) {

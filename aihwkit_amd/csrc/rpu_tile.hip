@@ -781,6 +781,8 @@ struct Tile {
     long image_size;
   };
 
+  const GatherSource *lines_in_place = nullptr; // set while update_indexed runs a pulsed update (pulsed_update_args)
+
   // in_ld: row stride of a plain row-major input with padded rows (0: the rows are dense)
   void mvm(const float *in, float *out, int B, bool bias, bool in_trans, bool out_trans, bool transposed, hipStream_t s,
            const float *w_other = nullptr, const IOPar *io_other = nullptr, bool is_test = false, long in_ld = 0,
@@ -1427,6 +1429,11 @@ struct Tile {
     UpdateArgs a{};
     a.w = dv.w; a.x_size = X; a.d_size = D; a.m_batch = B;
     a.x = xin; a.x_sb = x_sb; a.x_sj = x_sj; a.d = d; a.d_sb = d_sb; a.d_si = d_si;
+    if (lines_in_place) { // update_indexed: xin and d are the caller's image tensors
+      a.x_index = lines_in_place->index_patch_major; a.x_index_lines = lines_in_place->index_line_major; a.x_group = lines_in_place->patches; a.x_gs = lines_in_place->image_size;
+      a.x_sb = 0; a.x_sj = 0;
+      a.d_group = lines_in_place->patches; a.d_gs = (long)D * lines_in_place->patches; a.d_sb = 1; a.d_si = lines_in_place->patches;
+    }
     a.lr = lr;
     a.up.pulse_type = up.p.pulse_type; a.up.desired_bl = up.p.desired_bl; a.up.fixed_bl = up.p.fixed_bl;
     a.up.update_management = up.p.update_management; a.up.update_bl_management = up.p.update_bl_management;
@@ -1451,8 +1458,10 @@ struct Tile {
         a.x_words = u_xw.p; a.d_words = u_dw.p;
         set_plane_args(a, rows);
         a.kmax_slot = (int)(update_calls++ & 1u);
-        u_rowcost.ensure((size_t)D);
-        a.row_cost = u_rowcost.p;
+        if (update_reads_row_cost(a)) {
+          u_rowcost.ensure((size_t)D);
+          a.row_cost = u_rowcost.p;
+        }
       } else {
         u_xval.ensure((size_t)B * X); u_dval.ensure((size_t)B * D);
         a.x_val = u_xval.p; a.d_val = u_dval.p;
@@ -1726,8 +1735,29 @@ struct Tile {
   }
 
   void update_indexed(const float *x, const float *d, int n_images, long image_size, hipStream_t s) {
-    ensure_indexed(n_images);
+    if (idx_patches <= 0) throw RpuError("The index matrix has not been set (set_matrix_indices).");
+    if (n_images <= 0) throw RpuError("n_images must be positive.");
     const int B = indexed_samples(n_images);
+    const int pt = up.p.pulse_type;
+    if (dev.pulsed() && !is_transfer() && pt != RPU_PULSE_NONE && pt != RPU_PULSE_NONE_WITH_DEVICE) {
+      // pulsed update: the kernels that make the pulse trains read the patches through the index matrix and the
+      // gradients where the caller keeps them; neither the patch matrix nor a patch-major copy of d is written
+      // (the reference walks both tensors through iterators, cuda/io_iterator.h:160-696, cuda/rpucuda_pulsed.cu:575-604)
+      ensure_patch_major_index();
+      ensure_line_major_index();
+      const GatherSource patches_of{x_idx_t.p, x_idx.p, idx_patches, image_size};
+      lines_in_place = &patches_of;
+      try {
+        update(x, d, B, false, false, false, s);
+      } catch (...) {
+        lines_in_place = nullptr;
+        throw;
+      }
+      lines_in_place = nullptr;
+      RPU_HIP_CHECK(hipGetLastError());
+      return;
+    }
+    ensure_indexed(n_images);
     launch_gather_indexed(x_mat.p, x, x_idx.p, X, X, idx_patches, n_images, image_size, s);
     launch_ndp_to_bd(d_mat.p, d, n_images, D, idx_patches, s);
     update(x_mat.p, d_mat.p, B, false, false, false, s);

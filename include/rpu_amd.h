@@ -414,7 +414,10 @@ int rpu_tile_has_matrix_indices(const rpu_tile_t *tile); /* patches per image of
  * (N, C_out, H_out * W_out).  Forward gathers the patches through the index matrix and runs the tile's forward
  * pass over n_images * patches samples; backward runs the tile's backward pass and adds the patch gradients up
  * per image element (every element of x_dev is written, in a fixed order: nothing to zero, same bits on every
- * call); update gathers the patches and runs the tile's update. */
+ * call); update runs the tile's update over the same samples: a pulsed update reads the patches through the index
+ * matrix and the gradients from d_dev where they are (as the reference's iterators do, C/io_iterator.h:160-696; no
+ * patch matrix is written, same weights as the update on the unfolded matrices bit for bit), the floating-point
+ * update and a transfer compound unfold them first. */
 int rpu_tile_forward_indexed(rpu_tile_t *tile, const float *x_dev, float *d_dev, int n_images, long image_size,
                              int is_test, void *stream);
 int rpu_tile_backward_indexed(rpu_tile_t *tile, const float *d_dev, float *x_dev, int n_images, long image_size,

@@ -7,7 +7,7 @@ import torch.nn.functional as F
 
 from aihwkit_amd.rpu_base import devices as dv
 from aihwkit_amd.rpu_base import tiles
-from helpers import build_pair, constant_step, make_meta, noise_free_io
+from helpers import build_pair, constant_step, make_meta, noise_free_io, soft_bounds
 from indexed_oracle import IndexedOracle
 from test_oracle_indexed_pins import conv_indices
 
@@ -294,3 +294,53 @@ def test_gathered_forward_runs_every_round_whatever_the_launch_mode(gpu_device, 
     for (y0, r0), (y1, r1) in zip(results[0], results[mode]):
         assert torch.equal(r0, r1)
         assert torch.equal(y0, y1)
+
+
+@pytest.mark.parametrize("case", [
+    # 110 patches per image, 28 elements per patch with zero padding and a bias entry, 20 outputs (one block of 16 and a
+    # tail), ConstantStep with update-BL management: short bit lines
+    dict(c_in=3, hw=(11, 10), kernel=(3, 3), stride=(1, 1), padding=(1, 1), n=5, c_out=20, device="constant", bl=31,
+         pulse="StochasticCompressed"),
+    # 196 patches of 73 elements, 40 outputs, SoftBounds with cycle-to-cycle noise
+    dict(c_in=8, hw=(14, 14), kernel=(3, 3), stride=(1, 1), padding=(1, 1), n=3, c_out=40, device="soft", bl=31,
+         pulse="StochasticCompressed"),
+    # 9 patches per image (a block of 64 samples spans seven images), bit lines of 80 pulses: three rows of words per sample
+    dict(c_in=2, hw=(9, 9), kernel=(5, 5), stride=(2, 2), padding=(0, 0), n=23, c_out=33, device="constant", bl=80,
+         pulse="StochasticCompressed"),
+    dict(c_in=3, hw=(11, 10), kernel=(3, 3), stride=(1, 1), padding=(1, 1), n=5, c_out=20, device="constant", bl=31,
+         pulse="DeterministicImplicit"),
+])
+def test_pulsed_update_reads_patches_and_gradients_in_place(gpu_device, case):
+    """update_indexed of a pulsed tile reads the images through the index matrix and the gradient tensor where the caller
+    keeps it; neither the patch matrix nor a patch-major copy of the gradients is made.  Same weights, bit for bit, as
+    update() of a twin tile on the patch matrix that torch unfolds and the patch-major gradients."""
+    rng = np.random.default_rng(31)
+    c_in, (height, width), kernel, n, c_out = case["c_in"], case["hw"], case["kernel"], case["n"], case["c_out"]
+    indices, patches = conv_indices((c_in, height, width), kernel, case["stride"], case["padding"], (1, 1), True)
+    x_size = c_in * kernel[0] * kernel[1] + 1
+    meta = make_meta(noise_free_io(), noise_free_io(), pulse_type=getattr(dv.PulseType, case["pulse"]), desired_bl=case["bl"],
+                     update_bl_management=case["bl"] == 31, update_management=True)
+    if case["device"] == "soft":
+        dev = soft_bounds(dw_min=0.002, dw_min_std=0.3, construction_seed=9)
+    else:
+        dev = constant_step(dw_min=0.002, dw_min_std=0.0, construction_seed=4)
+    w = torch.from_numpy(rng.normal(0, 0.2, (c_out, x_size)).astype(np.float32))
+    x = torch.from_numpy(rng.normal(0, 1, (n, c_in, height, width)).astype(np.float32)).cuda()
+    grad = torch.from_numpy((0.3 * rng.normal(0, 1, (n, c_out, patches))).astype(np.float32)).cuda()
+    unfolded = torch.cat([F.unfold(x, kernel, padding=case["padding"], stride=case["stride"]), torch.ones(n, 1, patches).cuda()], dim=1)
+    x_mat = unfolded.permute(0, 2, 1).reshape(n * patches, x_size).contiguous()
+    d_mat = grad.permute(0, 2, 1).reshape(n * patches, c_out).contiguous()
+    got = []
+    for in_place in (True, False):
+        _host, _orc, gpu = build_pair(meta, dev, x_size, c_out)
+        gpu.set_weights(w)
+        gpu.set_learning_rate(0.05)
+        gpu.set_matrix_indices(indices)
+        for _ in range(2):
+            if in_place:
+                gpu.update_indexed(x, grad)
+            else:
+                gpu.update(x_mat, d_mat, False)
+        got.append(gpu.get_weights().clone())
+    assert torch.equal(got[0], got[1])
+    assert (got[0] - torch.from_numpy(np.clip(w.numpy(), -0.6, 0.6))).abs().max() > 1e-3
