@@ -217,7 +217,13 @@ struct SideDev {
   int adc_here, adc_sto_round;
   float adc_res, adc_bound;
   int *hit_up, *hit_lo; // [rows], null: no bound management
+  // rounds after the first: row_sample[row] = the sample whose quantized input the row holds (made by
+  // launch_side_row_samples); null: row r holds sample r.  The random draws are keyed by the sample, not by the row:
+  // which row a sample gets in a later round depends on the order in which workgroups finished the round before.
+  const int *row_sample;
 };
+// row_sample[row[pos]] = list[pos] for pos < *count (the list of a bound-management round and its rows)
+void launch_side_row_samples(int *row_sample, const int *list, const int *row, const int *count, int rows, hipStream_t s);
 // addend mode: pre[row][o] = w_noise term * N(0, 1) - IR-drop term; s_cur / s_ir are null without IR drop.
 // total mode: pre[row][o] = asymmetry(nonlinearity(offsets(s_y - IR drop) + w_noise term)) + output noise
 void launch_side_combine(float *pre, const float *s_noise, const float *row_sumsq, const float *s_cur, const float *s_ir,

@@ -61,13 +61,14 @@ __global__ __launch_bounds__(256) void k_side_combine(float *pre, const float *s
   for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
     const int row = (int)(i / quads);
     const int o0 = (int)(i % quads) * 4;
+    const uint32_t sample = p.row_sample ? (uint32_t)p.row_sample[row] : (uint32_t)row; // keys the random draws
     float z[4] = {0.f, 0.f, 0.f, 0.f}, zo[4] = {0.f, 0.f, 0.f, 0.f};
     int hit_u = 0, hit_l = 0;
     const bool noisy = p.w_noise_type != 0 && p.w_noise > 0.0f;
-    if (noisy) philox_normal4((uint32_t)(o0 >> 2), (uint32_t)row, call, RNG_W_NOISE | ((uint32_t)round << 8), key, z);
+    if (noisy) philox_normal4((uint32_t)(o0 >> 2), sample, call, RNG_W_NOISE | ((uint32_t)round << 8), key, z);
     const bool total = p.s_y != nullptr;
     const bool out_noisy = total && (p.out_noise != nullptr || p.out_noise_all > 0.0f);
-    if (out_noisy) philox_normal4((uint32_t)(o0 >> 2), (uint32_t)row, call, RNG_OUT_NOISE | ((uint32_t)round << 8), key, zo);
+    if (out_noisy) philox_normal4((uint32_t)(o0 >> 2), sample, call, RNG_OUT_NOISE | ((uint32_t)round << 8), key, zo);
     const float x_norm = (noisy && p.w_noise_type == 1) ? sqrtf(row_sumsq[row]) : 0.0f;
     const float y_ref = (total && p.v_offset && p.v_offset_w_min != 0.0f) ? -p.v_offset_w_min * p.x_accum[row] : 0.0f;
 #pragma unroll
@@ -112,7 +113,7 @@ __global__ __launch_bounds__(256) void k_side_combine(float *pre, const float *s
         if (p.adc_res > 0.0f) {
           float qq = v / p.adc_res;
           if (p.adc_sto_round) {
-            const Philox4 rr = philox4x32_10((uint32_t)o, (uint32_t)row, call, RNG_OUT_SR | ((uint32_t)round << 8), key.k0, key.k1);
+            const Philox4 rr = philox4x32_10((uint32_t)o, sample, call, RNG_OUT_SR | ((uint32_t)round << 8), key.k0, key.k1);
             qq = qq + (u32_to_uniform(rr.v[0]) - 0.5f);
           }
           v = rintf(qq) * p.adc_res;
@@ -131,7 +132,20 @@ __global__ __launch_bounds__(256) void k_side_combine(float *pre, const float *s
   }
 }
 
+__global__ __launch_bounds__(256) void k_side_row_samples(int *row_sample, const int *list, const int *row, const int *count,
+                                                           int rows) {
+  const int n = min(*count, rows);
+  for (int pos = blockIdx.x * blockDim.x + threadIdx.x; pos < n; pos += gridDim.x * blockDim.x) {
+    const int r = row[pos];
+    if (r >= 0 && r < rows) row_sample[r] = list[pos];
+  }
+}
+
 } // namespace
+
+void launch_side_row_samples(int *row_sample, const int *list, const int *row, const int *count, int rows, hipStream_t s) {
+  hipLaunchKernelGGL(k_side_row_samples, dim3(grid_for((size_t)rows)), dim3(256), 0, s, row_sample, list, row, count, rows);
+}
 
 void launch_side_rows(const float *xq, float *out, int rows, int k_pad, int K, int mode, int part, const int *skip_if_zero,
                       hipStream_t s) {

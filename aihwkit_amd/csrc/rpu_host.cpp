@@ -409,9 +409,8 @@ void TransferPar::initialize(int x_size, int d_size) {
   io.p.bound_management = RPU_BM_NONE;
   io.p.noise_management = RPU_NM_NONE;
   io.initialize(!p.transfer_columns);
-  if (io.has_line_terms()) {
-    throw RpuError("Per-line terms (voltage offsets, series resistance, output non-linearity, out_noise_std) and "
-                   "PosNegSeparate are not provided for the read of a transfer.");
+  if (io.p.w_read_asymmetry_dtod != 0.0f) {
+    throw RpuError("Read asymmetry of the negative pass (w_read_asymmetry_dtod) is not provided for the read of a transfer.");
   }
   up.p = p.transfer_up;
   up.initialize();

@@ -333,9 +333,12 @@ struct Tile {
   // input rows, |W| and the squared row norms
   DevBuf<float> n_pre, n_s1, n_s2, n_s3, n_s4, n_rows, n_absw, n_sumsq, n_xsum, n_part, n_neg;
   DevBuf<int> n_neghit; // [2][B] saturation marks of the negative pass (PosNegSeparateDigitalSum)
+  DevBuf<int> n_rowsample; // [B] sample of every row of a later round (SideDev::row_sample)
   // per direction: voltage offsets, non-linearity coefficients, output noise levels, read-asymmetry factors
-  DevBuf<float> d_line[2][4];
-  bool line_valid[2][4] = {{false, false, false, false}, {false, false, false, false}};
+  // per-line values on the device: of the forward IO, the backward IO and the IO of a transfer compound's read
+  DevBuf<float> d_line[3][4];
+  bool line_valid[3][4] = {{false, false, false, false}, {false, false, false, false}, {false, false, false, false}};
+  int line_set = -1; // 2 while the read of a transfer runs (pre_adc_terms then takes that IO's lines), else by direction
   DevBuf<float> n_wneg, n_absneg; // weights of the negative pass with read asymmetry, and their absolute values
   // running AverageAbsMax noise-management scale, one value shared by forward and backward as in the reference
   // (rpu_forward_backward_pass.h:241); negative: not started
@@ -439,6 +442,7 @@ struct Tile {
     n_part.release();
     n_neg.release();
     n_neghit.release();
+    n_rowsample.release();
     n_wneg.release();
     n_absneg.release();
     for (auto &dir : d_line) for (auto &b : dir) b.release();
@@ -628,7 +632,7 @@ struct Tile {
     bio.populate_lines(X, construction_seed ? construction_seed * 2654435761u + 2u : 0u, size());
   }
 
-  // device copies of the per-line values of a direction (0 forward, 1 backward)
+  // device copies of the per-line values of a direction (0 forward, 1 backward, 2 the read of a transfer)
   const float *line_values(int dir, int which, const std::vector<float> &host) {
     if (host.empty()) return nullptr;
     DevBuf<float> &buf = d_line[dir][which];
@@ -660,6 +664,16 @@ struct Tile {
     }
     // PosNegSeparate: the negative and the positive inputs see the array one after the other, each pass with its
     // own IR drop, offsets and weight noise; the sums of both go through the ADC (rpu_forward_backward_pass.cpp:832-893)
+    // a later round keeps its samples in rows handed out in the order in which the round before finished them
+    const int *row_sample = nullptr;
+    if (r > 0) {
+      if (n_rowsample.n < (size_t)B) {
+        n_rowsample.ensure((size_t)B);
+        launch_fill(reinterpret_cast<float *>(n_rowsample.p), 0.0f, (size_t)B, s); // rows without a sample: any valid key
+      }
+      launch_side_row_samples(n_rowsample.p, a.st.list[r & 1], a.st.row[r & 1], a.st.count + r, B, s);
+      row_sample = n_rowsample.p;
+    }
     const bool separate = io.separate_passes();
     for (int pass = 0; pass < (separate ? 2 : 1); ++pass) {
       const int part = separate ? (pass == 0 ? -1 : 1) : 0;
@@ -668,7 +682,7 @@ struct Tile {
       if (part < 0 && io.p.w_read_asymmetry_dtod > 0.0f && !io.w_asymmetry.empty()) {
         if (r == 0) {
           n_wneg.ensure(size());
-          launch_mul_copy(a.w, line_values(a.transposed ? 1 : 0, 3, io.w_asymmetry), n_wneg.p, size(), s);
+          launch_mul_copy(a.w, line_values(line_set >= 0 ? line_set : (a.transposed ? 1 : 0), 3, io.w_asymmetry), n_wneg.p, size(), s);
           if (need_abs) {
             n_absneg.ensure(size());
             launch_abs_copy(n_wneg.p, n_absneg.p, size(), s);
@@ -711,12 +725,13 @@ struct Tile {
         contract(w_pass, 2, n_s3.p);
       }
       SideDev p{};
+      p.row_sample = row_sample;
       p.w_noise_type = noisy ? io.p.w_noise_type : 0;
       p.w_noise = io.p.w_noise; p.ir_drop = ir ? io.p.ir_drop : 0.0f;
       p.a_scale = (float)a.K / io.p.ir_drop_g_ratio;
       if (total) {
         // the value itself is made beside the round kernel, whose ADC stage then only quantizes and clips
-        const int dir = a.transposed ? 1 : 0;
+        const int dir = line_set >= 0 ? line_set : (a.transposed ? 1 : 0);
         n_s4.ensure(out_n);
         contract(w_pass, 3, n_s4.p);
         p.s_y = n_s4.p;
@@ -786,7 +801,7 @@ struct Tile {
   // in_ld: row stride of a plain row-major input with padded rows (0: the rows are dense)
   void mvm(const float *in, float *out, int B, bool bias, bool in_trans, bool out_trans, bool transposed, hipStream_t s,
            const float *w_other = nullptr, const IOPar *io_other = nullptr, bool is_test = false, long in_ld = 0,
-           const GatherSource *gather = nullptr) {
+           const GatherSource *gather = nullptr, long out_ld = 0) {
     const IOPar &io = io_other ? *io_other : (transposed ? bio : fio);
     const bool side = has_pre_adc_terms(io);
     MvmArgs a = mvm_args(B, transposed, w_other ? w_other : mvm_weights(is_test), io, side ? 0 : -1);
@@ -816,6 +831,10 @@ struct Tile {
     if (in_ld) { // padded rows of a plain row-major input
       if (in_trans || bias || gather) throw RpuError("A row stride goes with a plain row-major input only.");
       a.in_sb = in_ld;
+    }
+    if (out_ld) { // padded rows of a plain row-major output
+      if (out_trans || bias) throw RpuError("A row stride goes with a plain row-major output only.");
+      a.out_sb = out_ld;
     }
     if (gather) { // the samples are patches gathered from the images `in` (see MvmArgs::in_index)
       if (in_trans || bias || transposed || side || gather->patches <= 0) throw RpuError("Gathered input: plain forward calls only.");
@@ -1867,7 +1886,14 @@ struct Tile {
       launch_unit_vectors(t_unit.p, n_vec, in_size, start, s);
       IOPar io = tp.io;
       io.p.out_scale = -io.p.out_scale;
-      mvm(t_unit.p, t_read.p, n_vec, false, false, false, !cols, s, slots[from]->d_w.p, &io);
+      line_set = 2; // the periphery of the read has its own per-line values (rpu_transfer_device.cpp:198-213)
+      try {
+        mvm(t_unit.p, t_read.p, n_vec, false, false, false, !cols, s, slots[from]->d_w.p, &io);
+      } catch (...) {
+        line_set = -1;
+        throw;
+      }
+      line_set = -1;
       DeviceView dv = view_of(*slots[to], slots[to]->par.weight_granularity());
       if (cols) pulsed_update_on(dv, tp.up, lr_t, t_unit.p, X, 1, t_read.p, D, 1, n_vec, s);
       else pulsed_update_on(dv, tp.up, lr_t, t_read.p, X, 1, t_unit.p, D, 1, n_vec, s);
@@ -2051,6 +2077,7 @@ int rpu_tile_create_transfer(rpu_tile_t **out, int x_size, int d_size, const rpu
     t.tr = std::make_unique<TransferPar>();
     t.tr->p = *tp;
     t.tr->initialize(x_size, d_size);
+    t.tr->io.populate_lines(t.tr->out_size, tp->construction_seed ? tp->construction_seed * 2654435761u + 3u : 0u, 0);
     t.dev = t.tr->devs[0]; // the device the gradient update sees
     std::vector<DeviceArrays> arrays;
     populate_chain(t.tr->devs, tp->construction_seed, x_size, d_size, arrays);
@@ -2310,17 +2337,20 @@ static void extra_fields(const Tile &t, std::vector<std::string> &names, std::ve
       values.push_back(float_bits(v[k]));
     }
   };
-  const IOPar *ios[2] = {&t.fio, &t.bio};
-  for (int dir = 0; dir < 2; ++dir) {
-    const char *prefix = dir ? "bwd." : "fwd.";
-    lines(prefix, "v_offset", ios[dir]->v_offset);
-    lines(prefix, "out_nonlinearity", ios[dir]->out_nl);
-    lines(prefix, "out_noise_values", ios[dir]->out_noise_values);
+  const IOPar *ios[3] = {&t.fio, &t.bio, t.tr ? &t.tr->io : nullptr};
+  const char *prefixes[3] = {"fwd.", "bwd.", "transfer.io."};
+  for (int dir = 0; dir < 3; ++dir) {
+    if (!ios[dir]) continue;
+    lines(prefixes[dir], "v_offset", ios[dir]->v_offset);
+    lines(prefixes[dir], "out_nonlinearity", ios[dir]->out_nl);
+    lines(prefixes[dir], "out_noise_values", ios[dir]->out_noise_values);
   }
 }
 static size_t line_entries(const Tile &t) {
-  return t.fio.v_offset.size() + t.fio.out_nl.size() + t.fio.out_noise_values.size() + t.bio.v_offset.size() +
-         t.bio.out_nl.size() + t.bio.out_noise_values.size();
+  size_t n = t.fio.v_offset.size() + t.fio.out_nl.size() + t.fio.out_noise_values.size() + t.bio.v_offset.size() +
+             t.bio.out_nl.size() + t.bio.out_noise_values.size();
+  if (t.tr) n += t.tr->io.v_offset.size() + t.tr->io.out_nl.size() + t.tr->io.out_noise_values.size();
+  return n;
 }
 static thread_local std::string g_extra_name;
 
@@ -2371,8 +2401,9 @@ int rpu_tile_set_extra(rpu_tile_t *tile, const int64_t *values_host, int count) 
     }
     for (size_t k = 0; k < t.slice_idx.size(); ++k) t.slice_idx[k] = (int)values_host[kFixedExtras + k];
     size_t at = kFixedExtras + t.slice_idx.size();
-    IOPar *ios[2] = {&t.fio, &t.bio};
-    for (int dir = 0; dir < 2; ++dir) {
+    IOPar *ios[3] = {&t.fio, &t.bio, t.tr ? &t.tr->io : nullptr};
+    for (int dir = 0; dir < 3; ++dir) {
+      if (!ios[dir]) continue;
       for (std::vector<float> *v : {&ios[dir]->v_offset, &ios[dir]->out_nl, &ios[dir]->out_noise_values}) {
         for (float &x : *v) x = bits_float(values_host[at++]);
       }
@@ -2615,6 +2646,37 @@ static int group_mvm(rpu_group_t *group, const float *const *x_dev, const long *
       throw RpuError("forward round barrier timed out in round " + std::to_string(failed - 1) +
                      "; results of the group's last forward call are invalid (the group now runs one launch per round).");
     }
+    // Tiles whose pass has terms that the group launches do not carry (the periphery terms before the ADC: weight noise
+    // referred to the output, IR drop, per-line offsets and non-linearities, separate passes for the two input signs;
+    // running-average noise management, a recurrence over the batch): the call runs the tiles one after the other on
+    // the stream, each with its own launches -- same results as rpu_tile_forward / rpu_tile_backward on each tile.
+    {
+      bool one_by_one = false;
+      for (int i = 0; i < n && !one_by_one; ++i) {
+        const Tile &t = group->tiles[i]->t;
+        const IOPar &gio = transposed ? t.bio : t.fio;
+        one_by_one = Tile::has_pre_adc_terms(gio) ||
+                     (!gio.perfect && (gio.p.noise_management == RPU_NM_AVERAGE_ABS_MAX ||
+                                       gio.p.noise_management == RPU_NM_AVERAGE_ABS_MAX_SINGLE_VALUE));
+      }
+      if (one_by_one) {
+        for (int i = 0; i < n; ++i) {
+          Tile &t = group->tiles[i]->t;
+          std::lock_guard<std::mutex> lock(t.mutex);
+          (void)t.check_compute(m_batch, x_dev[i], y_dev[i]);
+          if (t.shared_xd) throw RpuError("A tile that mirrors its weights into a shared tensor cannot be in a group.");
+          const int in_size = transposed ? t.D : t.X, out_size = transposed ? t.X : t.D;
+          const long in_ld = x_ld ? x_ld[i] : in_size, out_ld = y_ld ? y_ld[i] : out_size;
+          if (in_ld < in_size || out_ld < out_size) throw RpuError("A row stride is shorter than the row.");
+          t.mvm(x_dev[i], y_dev[i], m_batch, false, false, false, transposed, s, nullptr, nullptr, is_test,
+                in_ld == in_size ? 0 : in_ld, nullptr, out_ld == out_size ? 0 : out_ld);
+          t.last_stream = s;
+          if (!transposed) t.last_forward_batch = m_batch;
+        }
+        group->shared_sets = group->shared_tiles = 0;
+        return;
+      }
+    }
     // the staging buffers may still feed the copy of the previous call
     RPU_HIP_CHECK(hipEventSynchronize(group->copied));
 
@@ -2650,16 +2712,6 @@ static int group_mvm(rpu_group_t *group, const float *const *x_dev, const long *
       Tile &t = group->tiles[i]->t;
       std::lock_guard<std::mutex> lock(t.mutex);
       (void)t.check_compute(m_batch, x_dev[i], y_dev[i]);
-      if (Tile::has_pre_adc_terms(transposed ? t.bio : t.fio)) {
-        throw RpuError("Output-referred weight noise and IR drop are not provided for a group: call the tiles one by one.");
-      }
-      {
-        const IOPar &gio = transposed ? t.bio : t.fio;
-        if (!gio.perfect && (gio.p.noise_management == RPU_NM_AVERAGE_ABS_MAX ||
-                             gio.p.noise_management == RPU_NM_AVERAGE_ABS_MAX_SINGLE_VALUE)) {
-          throw RpuError("Running-average noise management is not provided for a group: call the tiles one by one.");
-        }
-      }
       if (t.shared_xd) throw RpuError("A tile that mirrors its weights into a shared tensor cannot be in a group.");
       if (i == 0) storage_xd = t.xd;
       if (t.xd != storage_xd) throw RpuError("The tiles of a group must store their weights the same way (all bound to [x_size, d_size] tensors, or none).");

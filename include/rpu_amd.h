@@ -433,7 +433,10 @@ int rpu_tile_update_indexed(rpu_tile_t *tile, const float *x_dev, const float *d
  * several per tile.  The tiles must be resident on the same GPU; each keeps its own state, seed and call
  * counter, and a grouped call gives every tile exactly what rpu_tile_forward with the same arguments would.
  * x_dev[i] is [m_batch][x_size_i], y_dev[i] is [m_batch][d_size_i] (no bias column, no transposed layouts).
- * The tiles must outlive the group. */
+ * A group that holds a tile whose pass has periphery terms before the ADC (output-referred weight noise, IR drop,
+ * per-line offsets and non-linearities, separate passes per input sign) or running-average noise management runs
+ * its tiles one after the other on the stream, each with the launches of rpu_tile_forward / rpu_tile_backward:
+ * same results, no shared launches.  The tiles must outlive the group. */
 typedef struct rpu_group rpu_group_t; /* opaque */
 int rpu_group_create(rpu_group_t **out, rpu_tile_t *const *tiles, int n_tiles);
 int rpu_group_forward(rpu_group_t *group, const float *const *x_dev, float *const *y_dev, int m_batch,

@@ -139,10 +139,27 @@ def test_weight_noise_under_bound_management_and_other_paths(gpu_device):
     resid = (got - want)[same]
     # the noise rides on the drifted sums of whichever round was the last one: small against the signal, not zero
     assert 0.01 < resid.std() < 0.15 and abs(resid.mean()) < 4 * resid.std() / np.sqrt(resid.size)
-    # a group does not take these tiles (bound to a shared tensor they mirror it, and the group refuses them at once)
-    with pytest.raises(RuntimeError, match="not provided for a group|cannot be in a group"):
-        group = tiles.TileGroup([gpu, quiet_gpu])
-        group.forward([torch.from_numpy(x).cuda(), torch.from_numpy(x).cuda()])
+    # a group takes these tiles and runs them one after the other, each with the launches of its own call (bound to a
+    # shared tensor they mirror it, and the group refuses them at once)
+    if tiles.CudaAnalogTile.bind_shared_weights:
+        with pytest.raises(RuntimeError, match="cannot be in a group"):
+            tiles.TileGroup([gpu, quiet_gpu])
+        return
+    _orc, twin, _w = pair(x_size, d_size, **io)
+    gpu.set_seed(77)
+    twin.set_seed(77)                                                          # same seed, same call numbers: same draws
+    d = rng.normal(0, 0.5, (batch, d_size)).astype(F)
+    group = tiles.TileGroup([gpu, quiet_gpu])
+    wide = torch.zeros(batch, x_size + 24).cuda()                              # inputs and outputs as column slices
+    wide[:, 8:8 + x_size] = torch.from_numpy(x).cuda()
+    outs = [torch.zeros(batch, d_size + 8).cuda()[:, 3:3 + d_size], torch.empty(batch, d_size).cuda()]
+    ys = group.forward([wide[:, 8:8 + x_size], torch.from_numpy(x).cuda()], outs=outs)
+    assert torch.equal(ys[0], twin.forward(torch.from_numpy(x).cuda()))
+    assert torch.equal(ys[1], quiet_gpu.forward(torch.from_numpy(x).cuda()))
+    assert torch.equal(outs[0], ys[0])                                          # written through the column slice
+    gs = group.backward([torch.from_numpy(d).cuda(), torch.from_numpy(d).cuda()])
+    assert torch.equal(gs[0], twin.backward(torch.from_numpy(d).cuda()))
+    assert torch.equal(gs[1], quiet_gpu.backward(torch.from_numpy(d).cuda()))
 
 
 @pytest.mark.parametrize("bm", [dv.BoundManagementType.NONE, dv.BoundManagementType.Iterative,
@@ -186,5 +203,31 @@ def test_running_average_noise_management_is_bit_exact_and_shared(gpu_device, bm
     twin = copy.deepcopy(gpu)                                     # a copy carries the value
     x2 = (rng.integers(-64, 65, (5, x_size)) / 128.0).astype(F)
     assert np.array_equal(twin.forward(torch.from_numpy(x2).cuda()).cpu().numpy(), orc.forward(x2))
-    with pytest.raises(RuntimeError, match="not provided for a group"):
-        tiles.TileGroup([gpu, twin]).forward([torch.from_numpy(x2).cuda(), torch.from_numpy(x2).cuda()])
+    # a group runs such tiles one after the other: the recurrence goes on from each tile's own running value
+    if not tiles.CudaAnalogTile.bind_shared_weights:
+        x3 = (rng.integers(-64, 65, (7, x_size)) / 128.0).astype(F)
+        gpu.forward(torch.from_numpy(x2).cuda())                   # now both tiles have seen x2 last
+        ys = tiles.TileGroup([gpu, twin]).forward([torch.from_numpy(x3).cuda(), torch.from_numpy(x3).cuda()])
+        want3 = orc.forward(x3)
+        assert np.array_equal(ys[0].cpu().numpy(), want3) and np.array_equal(ys[1].cpu().numpy(), want3)
+
+
+@pytest.mark.parametrize("noise_type", ["AdditiveConstant", "PCMRead"])
+def test_weight_noise_under_bound_management_is_a_function_of_the_seed(gpu_device, noise_type):
+    """Output-referred weight noise in the later rounds of bound management: a sample's row in such a round depends on
+    the order in which workgroups finished the round before, its draws do not (they are keyed by the sample).  The same
+    seed gives the same outputs and round counts, on the same tile and on another one."""
+    rng = np.random.default_rng(6)
+    x_size, d_size, batch = 64, 48, 256
+    x = torch.from_numpy(rng.uniform(-1, 1, (batch, x_size)).astype(F)).cuda()
+    io = dict(w_noise=0.02, w_noise_type=getattr(dv.WeightNoiseType, noise_type), out_bound=0.9,
+              noise_management=dv.NoiseManagementType.AbsMax, bound_management=dv.BoundManagementType.Iterative)
+    got = []
+    for _tile in range(2):
+        _orc, gpu, _w = pair(x_size, d_size, **io)
+        for _call in range(2):
+            gpu.set_seed(77)
+            got.append((gpu.forward(x).clone(), gpu.get_bm_rounds(batch).clone()))
+    assert got[0][1].max() >= 3 and got[0][1].min() < got[0][1].max()      # rows change hands between the rounds
+    for y, rounds in got[1:]:
+        assert torch.equal(rounds, got[0][1]) and torch.equal(y, got[0][0])

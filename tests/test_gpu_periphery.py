@@ -313,7 +313,8 @@ def test_line_values_are_state(gpu_device):
 def test_line_terms_are_refused_where_they_are_not_provided(gpu_device):
     from helpers import soft_bounds, transfer_param
     tr = transfer_param([soft_bounds(), soft_bounds()])
-    tr.transfer_forward.v_offset_std = 0.1
+    tr.transfer_forward.mv_type = PNS
+    tr.transfer_forward.w_read_asymmetry_dtod = 0.1
     with pytest.raises(Exception, match="not provided for the read of a transfer"):
         make_meta().create_array(8, 8, tr)
     with pytest.raises(Exception, match="AnalogMVType not implemented"):

@@ -253,3 +253,54 @@ def test_stochastic_transfer_moments_over_64_seeds(gpu_device):
     assert np.abs(want[:, 1].mean(0) - w0).max() > 5e-3  # the transfers did move the slow device
     compare_moments(got[:, 0], want[:, 0], "fast device weights")
     compare_moments(got[:, 1], want[:, 1], "slow device weights")
+
+
+@pytest.mark.parametrize("columns,terms", [
+    (True, dict(v_offset_std=0.1, out_nonlinearity=0.4, out_nonlinearity_std=0.2, r_series=0.01)),
+    (False, dict(v_offset_std=0.1, out_nonlinearity=0.4, out_nonlinearity_std=0.2)),       # rows: read by the backward pass
+    (True, dict(mv_type=dv.AnalogMVType.PosNegSeparate, v_offset_std=0.05, ir_drop=1.0)),
+])
+def test_transfer_read_with_per_line_periphery_terms(gpu_device, columns, terms):
+    """The read of a transfer with voltage offsets, output non-linearity, series resistance, IR drop and separate passes
+    (ForwardBackwardPassIOManaged with the transfer's own per-line values, rpu_transfer_device.cpp:198-213): the values
+    are part of the tile's state; given to the oracle's devices, whole trajectories agree."""
+    rng = np.random.default_rng(19)
+    x_size, d_size, batch = 37, 21, 8
+    meta, tr = deterministic_setup("soft", transfer_every=3.0, n_reads_per_transfer=2, transfer_columns=columns)
+    for k, v in terms.items():
+        setattr(tr.transfer_forward, k, v)
+    host, orc, gpu = build_transfer_pair(meta, tr, x_size, d_size)
+    state = gpu.dump_extra()
+    direction = 0 if columns else 1
+    found = 0
+    for which, kind in enumerate(("v_offset", "out_nonlinearity", "out_noise_values")):
+        prefix = f"rpu.transfer.io.{kind}_"
+        n = sum(1 for k in state if k.startswith(prefix))
+        values = np.array([state[f"{prefix}{i}.bits"] for i in range(n)], dtype=np.uint32).view(np.float32)
+        assert n in (0, d_size if columns else x_size)
+        found += n
+        for dev_tile in orc.devices:
+            assert dev_tile.get_lines(direction, which).size == n
+            if n:
+                dev_tile.set_lines(direction, which, values)
+    assert found > 0
+    w = rng.uniform(-0.4, 0.4, (d_size, x_size)).astype(np.float32)
+    gpu.set_weights(torch.from_numpy(w))
+    orc.set_weights(w)
+    gpu.set_learning_rate(0.05)
+    orc.set_learning_rate(0.05)
+    plain_meta, plain_tr = deterministic_setup("soft", transfer_every=3.0, n_reads_per_transfer=2, transfer_columns=columns)
+    _h, plain_orc, _g = build_transfer_pair(plain_meta, plain_tr, x_size, d_size, gpu=False)
+    plain_orc.set_weights(w)
+    plain_orc.set_learning_rate(0.05)
+    for step in range(6):
+        x = rng.uniform(-1, 1, (batch, x_size)).astype(np.float32)
+        d = (0.5 * rng.standard_normal((batch, d_size))).astype(np.float32)
+        gpu.update(cuda(x), cuda(d), False, False, False, False)
+        orc.update(x, d)
+        plain_orc.update(x, d)
+        check_state(gpu, orc, 2, f"step {step}")
+    # the terms matter: the slow device ends elsewhere than with an ideal periphery
+    assert np.abs(orc.device_weights(1) - plain_orc.device_weights(1)).max() > 10 * TOL
+    twin = copy.deepcopy(gpu)                                   # the lines travel with the tile
+    assert twin.dump_extra() == gpu.dump_extra()
