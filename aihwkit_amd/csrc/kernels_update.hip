@@ -86,70 +86,34 @@ __device__ __forceinline__ float part_abs_max(const float *v, int n, long stride
   return m;
 }
 
-// One workgroup per sample: the loads of both lines are in flight together (a line of 1024 elements is one 16-byte load
-// per thread), then one exchange through LDS gives the first thread both maxima and it sets the sample's BL, A, B.
-// SUB threads share a sample: the whole workgroup (long lines), a wave, or 16 lanes (the short patch rows of a
-// convolution come by the hundred thousand: a workgroup per sample would spend its time being launched)
-template <int SUB>
-__device__ __forceinline__ void update_prepare_sample(const UpdateArgs &a, const int b, float (*sh)[4]) {
-  const int t = threadIdx.x % SUB;
-  const bool leader = t == 0;
+// BL, A and B of sample b from the largest |x| and |d| of its lines (rpu_pulsed_meta_parameter.cpp:183-236), by one thread
+__device__ __forceinline__ void update_prepare_finish(const UpdateArgs &a, const int b, const float xm, const float dm) {
   const float lr = fabsf(a.lr);
   const float dw_min = a.dev.dw_min;
   int BL;
   float A, B;
-  if (a.up.update_management || a.up.update_bl_management) {
-    float xm = 0.0f;
-    if (a.x_index) {
-      for (int j = t; j < a.x_size; j += SUB) xm = fmaxf(xm, fabsf(update_x_value(a, b, j)));
+  calc_bl_ab(a.up, BL, A, B, lr, dw_min);
+  if ((a.up.update_management || a.up.update_bl_management) && lr > 0.0f) {
+    if (dm == 0.0f || xm == 0.0f) {
+      A = 1.0f;
+      B = 1.0f;
+      BL = 0;
     } else {
-      xm = part_abs_max(a.x + (long)b * a.x_sb, a.x_size, a.x_sj, t, SUB);
-    }
-    float dm = part_abs_max(update_d_row(a, b), a.d_size, a.d_si, t, SUB);
-#pragma unroll
-    for (int off = (SUB < 64 ? SUB : 64) / 2; off > 0; off >>= 1) {
-      xm = fmaxf(xm, __shfl_xor(xm, off));
-      dm = fmaxf(dm, __shfl_xor(dm, off));
-    }
-    if constexpr (SUB == 256) {
-      if ((threadIdx.x & 63) == 0) {
-        sh[0][threadIdx.x >> 6] = xm;
-        sh[1][threadIdx.x >> 6] = dm;
+      const float x_val = xm;
+      float d_val = a.up.um_grad_scale * dm;
+      const float k_val = lr * x_val * d_val / dw_min;
+      if (a.up.update_bl_management) {
+        BL = (int)ceilf(k_val);
+        if (BL > a.up.desired_bl) BL = a.up.desired_bl;
+        A = sqrtf(lr / (dw_min * (float)BL));
+        B = A;
       }
-      __syncthreads();
-      if (!leader) return;
-      xm = fmaxf(fmaxf(sh[0][0], sh[0][1]), fmaxf(sh[0][2], sh[0][3]));
-      dm = fmaxf(fmaxf(sh[1][0], sh[1][1]), fmaxf(sh[1][2], sh[1][3]));
-    } else {
-      if (!leader) return;
-    }
-    // rpu_pulsed_meta_parameter.cpp:183-236
-    calc_bl_ab(a.up, BL, A, B, lr, dw_min);
-    if (lr > 0.0f) {
-      if (dm == 0.0f || xm == 0.0f) {
-        A = 1.0f;
-        B = 1.0f;
-        BL = 0;
-      } else {
-        const float x_val = xm;
-        float d_val = a.up.um_grad_scale * dm;
-        const float k_val = lr * x_val * d_val / dw_min;
-        if (a.up.update_bl_management) {
-          BL = (int)ceilf(k_val);
-          if (BL > a.up.desired_bl) BL = a.up.desired_bl;
-          A = sqrtf(lr / (dw_min * (float)BL));
-          B = A;
-        }
-        if (a.up.update_management) {
-          if (k_val > (float)a.up.desired_bl) d_val *= (float)a.up.desired_bl / k_val;
-          A *= sqrtf(x_val / d_val);
-          B *= sqrtf(d_val / x_val);
-        }
+      if (a.up.update_management) {
+        if (k_val > (float)a.up.desired_bl) d_val *= (float)a.up.desired_bl / k_val;
+        A *= sqrtf(x_val / d_val);
+        B *= sqrtf(d_val / x_val);
       }
     }
-  } else {
-    if (!leader) return;
-    calc_bl_ab(a.up, BL, A, B, lr, dw_min);
   }
   a.bl[b] = BL;
   // largest number of pulse slots in a row of words (a longer bit line takes several rows of 31): this call's slot
@@ -165,6 +129,79 @@ __device__ __forceinline__ void update_prepare_sample(const UpdateArgs &a, const
   }
   a.prob_a[b] = A;
   a.prob_b[b] = B;
+}
+
+// One workgroup per sample: the loads of both lines are in flight together (a line of 1024 elements is one 16-byte load
+// per thread), then one exchange through LDS gives the first thread both maxima and it sets the sample's BL, A, B.
+// SUB threads share a sample: the whole workgroup (long lines), a wave, or 16 lanes (the short patch rows of a
+// convolution come by the hundred thousand: a workgroup per sample would spend its time being launched)
+template <int SUB>
+__device__ __forceinline__ void update_prepare_sample(const UpdateArgs &a, const int b, float (*sh)[4]) {
+  const int t = threadIdx.x % SUB;
+  const bool leader = t == 0;
+  float xm = 0.0f, dm = 0.0f;
+  if (a.up.update_management || a.up.update_bl_management) {
+    if (a.x_index) {
+      for (int j = t; j < a.x_size; j += SUB) xm = fmaxf(xm, fabsf(update_x_value(a, b, j)));
+    } else {
+      xm = part_abs_max(a.x + (long)b * a.x_sb, a.x_size, a.x_sj, t, SUB);
+    }
+    dm = part_abs_max(update_d_row(a, b), a.d_size, a.d_si, t, SUB);
+#pragma unroll
+    for (int off = (SUB < 64 ? SUB : 64) / 2; off > 0; off >>= 1) {
+      xm = fmaxf(xm, __shfl_xor(xm, off));
+      dm = fmaxf(dm, __shfl_xor(dm, off));
+    }
+    if constexpr (SUB == 256) {
+      if ((threadIdx.x & 63) == 0) {
+        sh[0][threadIdx.x >> 6] = xm;
+        sh[1][threadIdx.x >> 6] = dm;
+      }
+      __syncthreads();
+      if (!leader) return;
+      xm = fmaxf(fmaxf(sh[0][0], sh[0][1]), fmaxf(sh[0][2], sh[0][3]));
+      dm = fmaxf(fmaxf(sh[1][0], sh[1][1]), fmaxf(sh[1][2], sh[1][3]));
+    }
+  }
+  if (!leader) return;
+  update_prepare_finish(a, b, xm, dm);
+}
+
+// The lines of the indexed interface read in place, for long batches: one thread per sample, so that neighbouring
+// lanes read neighbouring patches -- the line-major index, the gradient tensor and (mostly) the image elements are
+// then runs of a row for every load of a wave.
+__global__ __launch_bounds__(64) void k_update_prepare_in_place(UpdateArgs a) {
+  if (a.row_cost) {
+    for (int i = (int)(blockIdx.x * 64u + threadIdx.x); i < a.d_size; i += (int)(gridDim.x * 64u)) a.row_cost[i] = 0;
+  }
+  const int b = (int)blockIdx.x * 64 + (int)threadIdx.x;
+  if (b >= a.m_batch) return;
+  float xm = 0.0f, dm = 0.0f;
+  if (a.up.update_management || a.up.update_bl_management) {
+    const int n = b / a.x_group;
+    const int *idx = a.x_index_lines + (b - n * a.x_group);
+    const float *image = a.x + (long)n * a.x_gs - 2;
+    // eight entries of the index, then the eight elements they name, in flight together
+    for (int j0 = 0; j0 < a.x_size; j0 += 8) {
+      int at[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) at[u] = (j0 + u < a.x_size) ? idx[(long)(j0 + u) * a.x_group] : 0;
+      float v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) v[u] = at[u] <= 1 ? (float)at[u] : image[at[u]];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) xm = fmaxf(xm, fabsf(v[u]));
+    }
+    const float *row = update_d_row(a, b);
+    for (int i0 = 0; i0 < a.d_size; i0 += 8) {
+      float v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) v[u] = (i0 + u < a.d_size) ? row[(long)(i0 + u) * a.d_si] : 0.0f;
+#pragma unroll
+      for (int u = 0; u < 8; ++u) dm = fmaxf(dm, fabsf(v[u]));
+    }
+  }
+  update_prepare_finish(a, b, xm, dm);
 }
 
 template <int SUB>
@@ -1435,6 +1472,10 @@ int grid_for(long total) {
 
 void launch_update_prepare(const UpdateArgs &a, hipStream_t s) {
   const int longest = a.x_size > a.d_size ? a.x_size : a.d_size;
+  if (a.x_index_lines && a.d_group && a.m_batch >= 4096) {
+    hipLaunchKernelGGL(k_update_prepare_in_place, dim3((a.m_batch + 63) / 64), dim3(64), 0, s, a);
+    return;
+  }
   if (longest > 1024 || a.m_batch <= 1024) {
     hipLaunchKernelGGL(k_update_prepare<256>, dim3(a.m_batch), dim3(256), 0, s, a);
   } else if (longest > 64) {

@@ -309,6 +309,9 @@ def test_gathered_forward_runs_every_round_whatever_the_launch_mode(gpu_device, 
          pulse="StochasticCompressed"),
     dict(c_in=3, hw=(11, 10), kernel=(3, 3), stride=(1, 1), padding=(1, 1), n=5, c_out=20, device="constant", bl=31,
          pulse="DeterministicImplicit"),
+    # 4800 samples: the per-sample maxima come from the kernel with one thread per sample
+    dict(c_in=3, hw=(40, 40), kernel=(3, 3), stride=(1, 1), padding=(1, 1), n=3, c_out=20, device="soft", bl=31,
+         pulse="StochasticCompressed"),
 ])
 def test_pulsed_update_reads_patches_and_gradients_in_place(gpu_device, case):
     """update_indexed of a pulsed tile reads the images through the index matrix and the gradient tensor where the caller
