@@ -1538,21 +1538,17 @@ void launch_update_planes(const UpdateArgs &a, hipStream_t s) {
 
 // whether the launch that deals the rows out by their work serves this call (see k_update_pulsed_balanced): only
 // where its workgroups, a quarter as many as rows, still fill the chip
-bool update_pulsed_balanced(const UpdateArgs &a, int columns) {
-  return columns == 4 && a.row_cost && a.x_size <= 1024 && a.d_size >= 1024 && a.d_size % 256 == 0 &&
-         a.d_size / 8 <= BALANCED_MAX_BAND;
+static bool balanced_shape(const UpdateArgs &a, int columns) {
+  return columns == 4 && a.x_size <= 1024 && a.d_size >= 1024 && a.d_size % 256 == 0 && a.d_size / 8 <= BALANCED_MAX_BAND;
 }
+bool update_pulsed_balanced(const UpdateArgs &a, int columns) { return a.row_cost && balanced_shape(a, columns); }
 
 static int update_pulsed_columns(const UpdateArgs &a);
 
 // whether a call of this shape reads UpdateArgs::row_cost at all: elsewhere the tile leaves it null, and the kernel that
 // makes the pulse trains sends no sums (on a tile of few rows and very many samples those were thousands of atomics per
 // address)
-bool update_reads_row_cost(const UpdateArgs &a) {
-  UpdateArgs probe = a;
-  probe.row_cost = reinterpret_cast<int *>(sizeof(int)); // any non-null value: only the shape is looked at
-  return update_pulsed_balanced(probe, update_pulsed_columns(a));
-}
+bool update_reads_row_cost(const UpdateArgs &a) { return balanced_shape(a, update_pulsed_columns(a)); }
 
 template <bool NOISE, int C, bool DEEP = false> static void launch_update_pulsed_t(const UpdateArgs &a, hipStream_t s) {
   if (C == 4 && !DEEP && update_pulsed_balanced(a, C)) {
