@@ -883,7 +883,9 @@ def one_write_noise(seed):
         shown = noisy.get_weights().numpy()
         changed = shown != before_shown
         stepped = after_plain != before_plain                      # a step was taken (hard bounds are far away)
-        if (stepped & ~changed).any():
+        # (a redrawn value equals the old one bit for bit about once in 10^7 cross-points, measured on 3 x 10^7 of them:
+        # a float has that many neighbours within the noise; a cross-point that is skipped shows up by the thousand)
+        if (stepped & ~changed).sum() > 2 + 1e-5 * stepped.sum():
             bad.append(("not redrawn", call, int((stepped & ~changed).sum())))
         # a cross-point that saw pulses which cancelled is redrawn too, one that saw none never is
         silent = (np.abs(x).sum(axis=0) == 0)[None, :] | (np.abs(d).sum(axis=0) == 0)[:, None]
